@@ -1,0 +1,119 @@
+// Shared device/host helpers for the gfx950 kernels of libbamboo_hip.so.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <stdio.h>
+#include <string.h>
+
+#include "../../include/bamboo_hip.h"
+
+typedef __bf16 bf16;
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+typedef __attribute__((ext_vector_type(4))) float f32x4;
+typedef __attribute__((ext_vector_type(16))) float f32x16;
+typedef __attribute__((ext_vector_type(4))) uint32_t u32x4;
+typedef __attribute__((ext_vector_type(2))) uint32_t u32x2;
+
+#define BB_WAVE 64
+
+// ---- error plumbing -------------------------------------------------------------------
+void bb_set_error(const char* fmt, ...);
+
+#define BB_REQUIRE(cond, ...)          \
+    do {                               \
+        if (!(cond)) {                 \
+            bb_set_error(__VA_ARGS__); \
+            return BB_EINVAL;          \
+        }                              \
+    } while (0)
+
+#define BB_HIP_CHECK(expr)                                                              \
+    do {                                                                                \
+        hipError_t e_ = (expr);                                                         \
+        if (e_ != hipSuccess) {                                                         \
+            bb_set_error("%s failed: %s (%s:%d)", #expr, hipGetErrorString(e_), __FILE__, \
+                         __LINE__);                                                     \
+            return BB_EHIP;                                                             \
+        }                                                                               \
+    } while (0)
+
+#define BB_LAUNCH_CHECK() BB_HIP_CHECK(hipGetLastError())
+
+// ---- scalar conversions -----------------------------------------------------------------
+__device__ __forceinline__ float bf2f(uint16_t b) { return __uint_as_float(((uint32_t)b) << 16); }
+__device__ __forceinline__ uint16_t f2bf(float f) {
+    return __builtin_bit_cast(uint16_t, (__bf16)f);  // round-to-nearest-even (v_cvt_pk_bf16_f32)
+}
+__device__ __forceinline__ uint32_t pack2bf(float lo, float hi) {
+    return (uint32_t)f2bf(lo) | ((uint32_t)f2bf(hi) << 16);
+}
+
+template <typename T> struct Elem;
+template <> struct Elem<float> {
+    static constexpr int VEC = 4;  // elements per 16-byte vector
+    __device__ static __forceinline__ float load(const float* p) { return *p; }
+    __device__ static __forceinline__ void store(float* p, float v) { *p = v; }
+};
+template <> struct Elem<bf16> {
+    static constexpr int VEC = 8;
+    __device__ static __forceinline__ float load(const bf16* p) { return bf2f(*(const uint16_t*)p); }
+    __device__ static __forceinline__ void store(bf16* p, float v) { *(uint16_t*)p = f2bf(v); }
+};
+
+// 16-byte vector load/store of VEC elements <-> float registers
+__device__ __forceinline__ void load_vec(const float* p, float (&v)[4]) {
+    f32x4 t = *(const f32x4*)p;
+    v[0] = t.x; v[1] = t.y; v[2] = t.z; v[3] = t.w;
+}
+__device__ __forceinline__ void store_vec(float* p, const float (&v)[4]) {
+    f32x4 t = {v[0], v[1], v[2], v[3]};
+    *(f32x4*)p = t;
+}
+__device__ __forceinline__ void load_vec(const bf16* p, float (&v)[8]) {
+    u32x4 t = *(const u32x4*)p;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        v[2 * i] = __uint_as_float(t[i] << 16);
+        v[2 * i + 1] = __uint_as_float(t[i] & 0xffff0000u);
+    }
+}
+__device__ __forceinline__ void store_vec(bf16* p, const float (&v)[8]) {
+    u32x4 t;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) t[i] = pack2bf(v[2 * i], v[2 * i + 1]);
+    *(u32x4*)p = t;
+}
+
+// ---- wavefront reductions (64 lanes, butterfly: every lane gets the result, fixed order) --
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+    return v;
+}
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, 64));
+    return v;
+}
+
+// ---- activations ------------------------------------------------------------------------
+__device__ __forceinline__ float gelu_tanh_f(float x) {
+    const float k0 = 0.7978845608028654f, k1 = 0.044715f;
+    float u = k0 * (x + k1 * x * x * x);
+    return 0.5f * x * (1.0f + tanhf(u));
+}
+__device__ __forceinline__ float dgelu_tanh_f(float x) {
+    const float k0 = 0.7978845608028654f, k1 = 0.044715f;
+    float u = k0 * (x + k1 * x * x * x);
+    float t = tanhf(u);
+    float du = k0 * (1.0f + 3.0f * k1 * x * x);
+    return 0.5f * (1.0f + t) + 0.5f * x * (1.0f - t * t) * du;
+}
+__device__ __forceinline__ float act_f(float x, int kind) {
+    return kind == BB_ACT_RELU ? fmaxf(x, 0.0f) : gelu_tanh_f(x);
+}
+__device__ __forceinline__ float dact_f(float x, int kind) {
+    return kind == BB_ACT_RELU ? (x > 0.0f ? 1.0f : 0.0f) : dgelu_tanh_f(x);
+}
+
+static inline int64_t ceil_div64(int64_t a, int64_t b) { return (a + b - 1) / b; }

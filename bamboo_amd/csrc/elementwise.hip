@@ -1,0 +1,633 @@
+// Bandwidth-bound kernels of the stage: LayerNorm fwd/bwd, bias-gradient column sums, masked
+// softmax fwd/bwd, residual add, MSE head, casts.  One 64-lane wavefront owns one row; lanes
+// read 16-byte vectors (lane l takes vector l, l+64, ...) so a wave load covers 1 KiB of
+// contiguous memory, rows are kept in registers between the passes of a kernel, and all
+// reductions are butterfly shuffles or fixed-order partial sums (no atomics: results are
+// reproducible bit for bit).
+#include "common.h"
+
+#include <stdarg.h>
+
+// ---- error string ------------------------------------------------------------------------
+static thread_local char g_err[512] = "";
+void bb_set_error(const char* fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_err, sizeof(g_err), fmt, ap);
+    va_end(ap);
+}
+extern "C" const char* bb_last_error(void) { return g_err; }
+extern "C" int bb_version(void) { return 1; }
+extern "C" int bb_init(void) {
+    int dev = 0;
+    BB_HIP_CHECK(hipGetDevice(&dev));
+    hipDeviceProp_t prop;
+    BB_HIP_CHECK(hipGetDeviceProperties(&prop, dev));
+    if (strncmp(prop.gcnArchName, "gfx950", 6) != 0) {
+        bb_set_error("bb_init: device %d is %s, this library is built for gfx950 only", dev, prop.gcnArchName);
+        return BB_EHIP;
+    }
+    return BB_OK;
+}
+
+// =========================================================================================
+// LayerNorm
+// =========================================================================================
+// Row held in registers: lane owns vectors lane, lane+64, ... (IT of them, VEC elements each).
+template <typename T, int IT>
+__global__ __launch_bounds__(256) void layernorm_fwd_kernel(int kind, int rows, int cols, float eps,
+                                                            const T* __restrict__ x, const T* __restrict__ gain,
+                                                            const T* __restrict__ shift, T* __restrict__ y,
+                                                            float* __restrict__ mean_out, float* __restrict__ rinv_out) {
+    constexpr int VEC = Elem<T>::VEC;
+    const int lane = threadIdx.x & 63;
+    const int row = blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (row >= rows) return;
+    const int nvec = cols / VEC;
+    const T* xr = x + (int64_t)row * cols;
+    float v[IT][VEC];
+    float s = 0.f;
+#pragma unroll
+    for (int i = 0; i < IT; ++i) {
+        const int c = lane + i * 64;
+        if (c < nvec) {
+            load_vec(xr + c * VEC, v[i]);
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) s += v[i][e];
+        } else {
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) v[i][e] = 0.f;
+        }
+    }
+    const float mean = wave_sum(s) / (float)cols;
+    float q = 0.f;
+#pragma unroll
+    for (int i = 0; i < IT; ++i) {
+        const int c = lane + i * 64;
+        if (c < nvec) {
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) {
+                const float d = v[i][e] - mean;
+                q += d * d;
+            }
+        }
+    }
+    q = wave_sum(q);
+    float rinv;
+    if (kind == BB_LN_ANNOTATED)
+        rinv = 1.0f / (sqrtf(q / (float)(cols - 1)) + eps);
+    else
+        rinv = 1.0f / sqrtf(q / (float)cols + eps);
+    if (lane == 0) {
+        mean_out[row] = mean;
+        rinv_out[row] = rinv;
+    }
+    T* yr = y + (int64_t)row * cols;
+#pragma unroll
+    for (int i = 0; i < IT; ++i) {
+        const int c = lane + i * 64;
+        if (c < nvec) {
+            float gv[VEC], bv[VEC], o[VEC];
+            load_vec(gain + c * VEC, gv);
+            load_vec(shift + c * VEC, bv);
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) o[e] = gv[e] * ((v[i][e] - mean) * rinv) + bv[e];
+            store_vec(yr + c * VEC, o);
+        }
+    }
+}
+
+constexpr int LN_BWD_BLOCKS = 256;
+
+// dx per row, dgain/dshift partial sums per block (fixed row->block assignment).
+template <typename T, int IT>
+__global__ __launch_bounds__(256) void layernorm_bwd_kernel(int kind, int rows, int cols, float eps,
+                                                            const T* __restrict__ x, const T* __restrict__ gain,
+                                                            const float* __restrict__ mean_in,
+                                                            const float* __restrict__ rinv_in, const T* __restrict__ dy,
+                                                            const T* __restrict__ dres, T* __restrict__ dx,
+                                                            float* __restrict__ partial) {
+    constexpr int VEC = Elem<T>::VEC;
+    extern __shared__ float red[];  // [3 waves][2][cols] for the cross-wave sum
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int nvec = cols / VEC;
+    float gv[IT][VEC], dg[IT][VEC], db[IT][VEC];
+#pragma unroll
+    for (int i = 0; i < IT; ++i) {
+        const int c = lane + i * 64;
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) dg[i][e] = db[i][e] = gv[i][e] = 0.f;
+        if (c < nvec) load_vec(gain + c * VEC, gv[i]);
+    }
+    for (int row = blockIdx.x * 4 + wave; row < rows; row += gridDim.x * 4) {
+        const float mean = mean_in[row], rinv = rinv_in[row];
+        const T* xr = x + (int64_t)row * cols;
+        const T* dyr = dy + (int64_t)row * cols;
+        float xh[IT][VEC], dyh[IT][VEC];
+        float s1 = 0.f, s2 = 0.f;
+#pragma unroll
+        for (int i = 0; i < IT; ++i) {
+            const int c = lane + i * 64;
+            if (c < nvec) {
+                float xv[VEC], dv[VEC];
+                load_vec(xr + c * VEC, xv);
+                load_vec(dyr + c * VEC, dv);
+#pragma unroll
+                for (int e = 0; e < VEC; ++e) {
+                    xh[i][e] = (xv[e] - mean) * rinv;
+                    dyh[i][e] = dv[e] * gv[i][e];
+                    dg[i][e] += dv[e] * xh[i][e];
+                    db[i][e] += dv[e];
+                    s1 += dyh[i][e];
+                    s2 += dyh[i][e] * xh[i][e];
+                }
+            } else {
+#pragma unroll
+                for (int e = 0; e < VEC; ++e) xh[i][e] = dyh[i][e] = 0.f;
+            }
+        }
+        s1 = wave_sum(s1) / (float)cols;
+        s2 = wave_sum(s2);
+        float c2;  // coefficient of xh in dx
+        if (kind == BB_LN_ANNOTATED) {
+            const float sigma = 1.0f / rinv - eps;
+            c2 = sigma > 0.f ? s2 / ((float)(cols - 1) * sigma) : 0.f;
+        } else {
+            c2 = rinv * s2 / (float)cols;
+        }
+        T* dxr = dx + (int64_t)row * cols;
+#pragma unroll
+        for (int i = 0; i < IT; ++i) {
+            const int c = lane + i * 64;
+            if (c < nvec) {
+                float o[VEC];
+#pragma unroll
+                for (int e = 0; e < VEC; ++e) o[e] = rinv * (dyh[i][e] - s1) - xh[i][e] * c2;
+                if (dres) {
+                    float rv[VEC];
+                    load_vec(dres + (int64_t)row * cols + c * VEC, rv);
+#pragma unroll
+                    for (int e = 0; e < VEC; ++e) o[e] += rv[e];
+                }
+                store_vec(dxr + c * VEC, o);
+            }
+        }
+    }
+    // cross-wave sum in fixed order (wave 0 + 1 + 2 + 3), then one partial row per block
+    if (wave > 0) {
+        float* r = red + (int64_t)(wave - 1) * 2 * cols;
+#pragma unroll
+        for (int i = 0; i < IT; ++i) {
+            const int c = lane + i * 64;
+            if (c < nvec) {
+#pragma unroll
+                for (int e = 0; e < VEC; ++e) {
+                    r[c * VEC + e] = dg[i][e];
+                    r[cols + c * VEC + e] = db[i][e];
+                }
+            }
+        }
+    }
+    __syncthreads();
+    if (wave == 0) {
+        float* out = partial + (int64_t)blockIdx.x * 2 * cols;
+#pragma unroll
+        for (int i = 0; i < IT; ++i) {
+            const int c = lane + i * 64;
+            if (c < nvec) {
+#pragma unroll
+                for (int e = 0; e < VEC; ++e) {
+                    float a = dg[i][e], b = db[i][e];
+                    for (int w = 0; w < 3; ++w) {
+                        a += red[(int64_t)w * 2 * cols + c * VEC + e];
+                        b += red[(int64_t)w * 2 * cols + cols + c * VEC + e];
+                    }
+                    out[c * VEC + e] = a;
+                    out[cols + c * VEC + e] = b;
+                }
+            }
+        }
+    }
+}
+
+// out[i] += sum_p partial[p * stride + i], p ascending (fixed order)
+__global__ __launch_bounds__(256) void reduce_partials_acc_kernel(const float* __restrict__ partial, int nparts,
+                                                                  int64_t stride, int n, float* __restrict__ out) {
+    const int i = blockIdx.x * 256 + threadIdx.x;
+    if (i >= n) return;
+    float s = 0.f;
+    for (int p = 0; p < nparts; ++p) s += partial[p * stride + i];
+    out[i] += s;
+}
+
+template <typename T, int IT>
+static int ln_fwd_launch(int kind, int rows, int cols, float eps, const void* x, const void* gain, const void* shift,
+                         void* y, float* mean, float* rinv, hipStream_t st) {
+    hipLaunchKernelGGL((layernorm_fwd_kernel<T, IT>), dim3((rows + 3) / 4), dim3(256), 0, st, kind, rows, cols, eps,
+                       (const T*)x, (const T*)gain, (const T*)shift, (T*)y, mean, rinv);
+    BB_LAUNCH_CHECK();
+    return BB_OK;
+}
+template <typename T, int IT>
+static int ln_bwd_launch(int kind, int rows, int cols, float eps, const void* x, const void* gain, const float* mean,
+                         const float* rinv, const void* dy, const void* dres, void* dx, float* ws, hipStream_t st) {
+    const size_t smem = (size_t)3 * 2 * cols * sizeof(float);
+    auto kern = layernorm_bwd_kernel<T, IT>;
+    if (smem > 64 * 1024) BB_HIP_CHECK(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
+    hipLaunchKernelGGL(kern, dim3(LN_BWD_BLOCKS), dim3(256), smem, st, kind, rows, cols, eps, (const T*)x,
+                       (const T*)gain, mean, rinv, (const T*)dy, (const T*)dres, (T*)dx, ws);
+    BB_LAUNCH_CHECK();
+    return BB_OK;
+}
+
+#define BB_DISPATCH_IT(T, nvec, CALL)                       \
+    do {                                                    \
+        const int it_ = ((nvec) + 63) / 64;                 \
+        if (it_ <= 2) { constexpr int IT = 2; return CALL; }  \
+        if (it_ <= 4) { constexpr int IT = 4; return CALL; }  \
+        if (it_ <= 8) { constexpr int IT = 8; return CALL; }  \
+        if (it_ <= 16) { constexpr int IT = 16; return CALL; } \
+    } while (0)
+
+static int check_rowop(const char* name, int dtype, int rows, int cols) {
+    BB_REQUIRE(dtype == BB_F32 || dtype == BB_BF16, "%s: bad dtype %d", name, dtype);
+    const int vec = dtype == BB_BF16 ? 8 : 4;
+    BB_REQUIRE(rows >= 0 && cols > 0, "%s: bad shape %d x %d", name, rows, cols);
+    BB_REQUIRE(cols % vec == 0, "%s: cols (%d) must be a multiple of %d", name, cols, vec);
+    BB_REQUIRE(cols / vec <= 64 * 16, "%s: cols (%d) too large (max %d)", name, cols, 64 * 16 * vec);
+    return BB_OK;
+}
+
+extern "C" int bb_layernorm_fwd(int dtype, int kind, int rows, int cols, float eps, const void* x, const void* gain,
+                                const void* shift, void* y, float* mean, float* rinv, void* stream) {
+    int rc = check_rowop("bb_layernorm_fwd", dtype, rows, cols);
+    if (rc) return rc;
+    BB_REQUIRE(kind == BB_LN_STANDARD || kind == BB_LN_ANNOTATED, "bb_layernorm_fwd: bad kind %d", kind);
+    BB_REQUIRE(x && gain && shift && y && mean && rinv, "bb_layernorm_fwd: null pointer");
+    BB_REQUIRE(kind != BB_LN_ANNOTATED || cols > 1, "bb_layernorm_fwd: annotated LayerNorm needs cols > 1");
+    if (rows == 0) return BB_OK;
+    hipStream_t st = (hipStream_t)stream;
+    if (dtype == BB_BF16)
+        BB_DISPATCH_IT(bf16, cols / 8, (ln_fwd_launch<bf16, IT>(kind, rows, cols, eps, x, gain, shift, y, mean, rinv, st)));
+    else
+        BB_DISPATCH_IT(float, cols / 4, (ln_fwd_launch<float, IT>(kind, rows, cols, eps, x, gain, shift, y, mean, rinv, st)));
+    return BB_EINVAL;
+}
+
+extern "C" int64_t bb_layernorm_bwd_workspace(int cols) { return (int64_t)LN_BWD_BLOCKS * 2 * cols; }
+
+extern "C" int bb_layernorm_bwd(int dtype, int kind, int rows, int cols, float eps, const void* x, const void* gain,
+                                const float* mean, const float* rinv, const void* dy, const void* dres, void* dx,
+                                float* dgain, float* dshift, float* workspace, void* stream) {
+    int rc = check_rowop("bb_layernorm_bwd", dtype, rows, cols);
+    if (rc) return rc;
+    BB_REQUIRE(kind == BB_LN_STANDARD || kind == BB_LN_ANNOTATED, "bb_layernorm_bwd: bad kind %d", kind);
+    BB_REQUIRE(x && gain && mean && rinv && dy && dx && dgain && dshift && workspace, "bb_layernorm_bwd: null pointer");
+    BB_REQUIRE((size_t)3 * 2 * cols * sizeof(float) <= 160 * 1024, "bb_layernorm_bwd: cols (%d) too large (max 6826)", cols);
+    if (rows == 0) return BB_OK;
+    hipStream_t st = (hipStream_t)stream;
+    auto finish = [&]() -> int {
+        const int nb = (cols + 255) / 256;
+        hipLaunchKernelGGL(reduce_partials_acc_kernel, dim3(nb), dim3(256), 0, st, workspace, LN_BWD_BLOCKS,
+                           (int64_t)2 * cols, cols, dgain);
+        hipLaunchKernelGGL(reduce_partials_acc_kernel, dim3(nb), dim3(256), 0, st, workspace + cols, LN_BWD_BLOCKS,
+                           (int64_t)2 * cols, cols, dshift);
+        BB_LAUNCH_CHECK();
+        return BB_OK;
+    };
+    auto run = [&](auto launch) -> int {
+        int r = launch;
+        return r ? r : finish();
+    };
+    if (dtype == BB_BF16)
+        BB_DISPATCH_IT(bf16, cols / 8, run(ln_bwd_launch<bf16, IT>(kind, rows, cols, eps, x, gain, mean, rinv, dy, dres, dx, workspace, st)));
+    else
+        BB_DISPATCH_IT(float, cols / 4, run(ln_bwd_launch<float, IT>(kind, rows, cols, eps, x, gain, mean, rinv, dy, dres, dx, workspace, st)));
+    return BB_EINVAL;
+}
+
+// =========================================================================================
+// column sums (bias gradient)
+// =========================================================================================
+constexpr int COLSUM_SPLITS = 64;
+
+template <typename T>
+__global__ __launch_bounds__(256) void colsum_partial_kernel(int rows, int cols, const T* __restrict__ x, int64_t ldx,
+                                                             float* __restrict__ partial) {
+    constexpr int VEC = Elem<T>::VEC;
+    __shared__ float red[3][64 * VEC];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int c0 = (blockIdx.x * 64 + lane) * VEC;
+    float acc[VEC];
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) acc[e] = 0.f;
+    if (c0 < cols) {
+        for (int r = blockIdx.y * 4 + wave; r < rows; r += gridDim.y * 4) {
+            float v[VEC];
+            load_vec(x + (int64_t)r * ldx + c0, v);
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) acc[e] += v[e];
+        }
+    }
+    if (wave > 0) {
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) red[wave - 1][lane * VEC + e] = acc[e];
+    }
+    __syncthreads();
+    if (wave == 0 && c0 < cols) {
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) {
+            float a = acc[e];
+            for (int w = 0; w < 3; ++w) a += red[w][lane * VEC + e];
+            partial[(int64_t)blockIdx.y * cols + c0 + e] = a;
+        }
+    }
+}
+
+extern "C" int64_t bb_colsum_workspace(int cols) { return (int64_t)COLSUM_SPLITS * cols; }
+
+extern "C" int bb_colsum_acc(int dtype, int rows, int cols, const void* x, int64_t ldx, float* out, float* workspace,
+                             void* stream) {
+    BB_REQUIRE(dtype == BB_F32 || dtype == BB_BF16, "bb_colsum_acc: bad dtype %d", dtype);
+    const int vec = dtype == BB_BF16 ? 8 : 4;
+    BB_REQUIRE(rows >= 0 && cols > 0 && cols % vec == 0 && ldx % vec == 0 && ldx >= cols,
+               "bb_colsum_acc: bad shape rows=%d cols=%d ldx=%lld", rows, cols, (long long)ldx);
+    BB_REQUIRE(x && out && workspace, "bb_colsum_acc: null pointer");
+    if (rows == 0) return BB_OK;
+    hipStream_t st = (hipStream_t)stream;
+    dim3 grid((cols + 64 * vec - 1) / (64 * vec), COLSUM_SPLITS);
+    if (dtype == BB_BF16)
+        hipLaunchKernelGGL(colsum_partial_kernel<bf16>, grid, dim3(256), 0, st, rows, cols, (const bf16*)x, ldx, workspace);
+    else
+        hipLaunchKernelGGL(colsum_partial_kernel<float>, grid, dim3(256), 0, st, rows, cols, (const float*)x, ldx, workspace);
+    hipLaunchKernelGGL(reduce_partials_acc_kernel, dim3((cols + 255) / 256), dim3(256), 0, st, workspace, COLSUM_SPLITS,
+                       (int64_t)cols, cols, out);
+    BB_LAUNCH_CHECK();
+    return BB_OK;
+}
+
+// =========================================================================================
+// masked softmax (in place)
+// =========================================================================================
+template <typename T, int IT>
+__global__ __launch_bounds__(256) void softmax_fwd_kernel(int mask, int heads, int sq, int sk, int64_t rows,
+                                                          T* __restrict__ s, const int32_t* __restrict__ key_len) {
+    constexpr int VEC = Elem<T>::VEC;
+    const int lane = threadIdx.x & 63;
+    const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (row >= rows) return;
+    const int q = (int)(row % sq);
+    const int b = (int)(row / ((int64_t)heads * sq));
+    int limit = sk;  // keep columns < limit
+    if (mask == BB_MASK_CAUSAL) limit = min(sk, q + 1);
+    else if (mask == BB_MASK_KEY_PADDING) limit = min(sk, key_len[b]);
+    const int nvec = sk / VEC;
+    T* sr = s + row * sk;
+    float v[IT][VEC];
+    float mx = -INFINITY;
+#pragma unroll
+    for (int i = 0; i < IT; ++i) {
+        const int c = lane + i * 64;
+        if (c < nvec) {
+            load_vec(sr + c * VEC, v[i]);
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) {
+                if (c * VEC + e >= limit) v[i][e] = -1e9f;
+                mx = fmaxf(mx, v[i][e]);
+            }
+        }
+    }
+    mx = wave_max(mx);
+    float sum = 0.f;
+#pragma unroll
+    for (int i = 0; i < IT; ++i) {
+        const int c = lane + i * 64;
+        if (c < nvec) {
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) {
+                v[i][e] = expf(v[i][e] - mx);
+                sum += v[i][e];
+            }
+        }
+    }
+    const float inv = 1.0f / wave_sum(sum);
+#pragma unroll
+    for (int i = 0; i < IT; ++i) {
+        const int c = lane + i * 64;
+        if (c < nvec) {
+            float o[VEC];
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) o[e] = v[i][e] * inv;
+            store_vec(sr + c * VEC, o);
+        }
+    }
+}
+
+template <typename T, int IT>
+__global__ __launch_bounds__(256) void softmax_bwd_kernel(int sk, int64_t rows, const T* __restrict__ p,
+                                                          T* __restrict__ dp) {
+    constexpr int VEC = Elem<T>::VEC;
+    const int lane = threadIdx.x & 63;
+    const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (row >= rows) return;
+    const int nvec = sk / VEC;
+    const T* pr = p + row * sk;
+    T* dr = dp + row * sk;
+    float pv[IT][VEC], dv[IT][VEC];
+    float t = 0.f;
+#pragma unroll
+    for (int i = 0; i < IT; ++i) {
+        const int c = lane + i * 64;
+        if (c < nvec) {
+            load_vec(pr + c * VEC, pv[i]);
+            load_vec(dr + c * VEC, dv[i]);
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) t += pv[i][e] * dv[i][e];
+        }
+    }
+    t = wave_sum(t);
+#pragma unroll
+    for (int i = 0; i < IT; ++i) {
+        const int c = lane + i * 64;
+        if (c < nvec) {
+            float o[VEC];
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) o[e] = pv[i][e] * (dv[i][e] - t);
+            store_vec(dr + c * VEC, o);
+        }
+    }
+}
+
+template <typename T, int IT>
+static int softmax_fwd_launch(int mask, int heads, int sq, int sk, int64_t rows, void* s, const int32_t* kl, hipStream_t st) {
+    hipLaunchKernelGGL((softmax_fwd_kernel<T, IT>), dim3((unsigned)((rows + 3) / 4)), dim3(256), 0, st, mask, heads, sq, sk,
+                       rows, (T*)s, kl);
+    BB_LAUNCH_CHECK();
+    return BB_OK;
+}
+template <typename T, int IT>
+static int softmax_bwd_launch(int sk, int64_t rows, const void* p, void* dp, hipStream_t st) {
+    hipLaunchKernelGGL((softmax_bwd_kernel<T, IT>), dim3((unsigned)((rows + 3) / 4)), dim3(256), 0, st, sk, rows,
+                       (const T*)p, (T*)dp);
+    BB_LAUNCH_CHECK();
+    return BB_OK;
+}
+
+extern "C" int bb_softmax_fwd(int dtype, int mask, int batch, int heads, int sq, int sk, void* s, const int32_t* key_len,
+                              void* stream) {
+    int rc = check_rowop("bb_softmax_fwd", dtype, 1, sk);
+    if (rc) return rc;
+    BB_REQUIRE(mask >= BB_MASK_NONE && mask <= BB_MASK_KEY_PADDING, "bb_softmax_fwd: bad mask %d", mask);
+    BB_REQUIRE(mask != BB_MASK_KEY_PADDING || key_len, "bb_softmax_fwd: key_padding mask needs key_len");
+    BB_REQUIRE(batch >= 0 && heads >= 0 && sq >= 0 && s, "bb_softmax_fwd: bad arguments");
+    const int64_t rows = (int64_t)batch * heads * sq;
+    if (rows == 0) return BB_OK;
+    BB_REQUIRE((rows + 3) / 4 < (1ll << 31), "bb_softmax_fwd: too many rows");
+    hipStream_t st = (hipStream_t)stream;
+    if (dtype == BB_BF16)
+        BB_DISPATCH_IT(bf16, sk / 8, (softmax_fwd_launch<bf16, IT>(mask, heads, sq, sk, rows, s, key_len, st)));
+    else
+        BB_DISPATCH_IT(float, sk / 4, (softmax_fwd_launch<float, IT>(mask, heads, sq, sk, rows, s, key_len, st)));
+    return BB_EINVAL;
+}
+
+extern "C" int bb_softmax_bwd(int dtype, int batch, int heads, int sq, int sk, const void* p, void* dp, void* stream) {
+    int rc = check_rowop("bb_softmax_bwd", dtype, 1, sk);
+    if (rc) return rc;
+    BB_REQUIRE(batch >= 0 && heads >= 0 && sq >= 0 && p && dp, "bb_softmax_bwd: bad arguments");
+    const int64_t rows = (int64_t)batch * heads * sq;
+    if (rows == 0) return BB_OK;
+    BB_REQUIRE((rows + 3) / 4 < (1ll << 31), "bb_softmax_bwd: too many rows");
+    hipStream_t st = (hipStream_t)stream;
+    if (dtype == BB_BF16)
+        BB_DISPATCH_IT(bf16, sk / 8, (softmax_bwd_launch<bf16, IT>(sk, rows, p, dp, st)));
+    else
+        BB_DISPATCH_IT(float, sk / 4, (softmax_bwd_launch<float, IT>(sk, rows, p, dp, st)));
+    return BB_EINVAL;
+}
+
+// =========================================================================================
+// residual add, cast, fill
+// =========================================================================================
+template <typename T>
+__global__ __launch_bounds__(256) void add_kernel(int64_t nvec, const T* __restrict__ a, const T* __restrict__ b,
+                                                  T* __restrict__ out) {
+    constexpr int VEC = Elem<T>::VEC;
+    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < nvec; i += (int64_t)gridDim.x * 256) {
+        float x[VEC], y[VEC];
+        load_vec(a + i * VEC, x);
+        load_vec(b + i * VEC, y);
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) x[e] += y[e];
+        store_vec(out + i * VEC, x);
+    }
+}
+
+static unsigned grid_for(int64_t work_items) {
+    int64_t b = (work_items + 255) / 256;
+    if (b > 256 * 16) b = 256 * 16;  // 16 blocks per CU, grid-stride beyond
+    if (b < 1) b = 1;
+    return (unsigned)b;
+}
+
+extern "C" int bb_residual_add(int dtype, int64_t n, const void* a, const void* b, void* out, void* stream) {
+    BB_REQUIRE(dtype == BB_F32 || dtype == BB_BF16, "bb_residual_add: bad dtype %d", dtype);
+    const int vec = dtype == BB_BF16 ? 8 : 4;
+    BB_REQUIRE(n >= 0 && n % vec == 0, "bb_residual_add: n (%lld) must be a multiple of %d", (long long)n, vec);
+    BB_REQUIRE(a && b && out, "bb_residual_add: null pointer");
+    if (n == 0) return BB_OK;
+    hipStream_t st = (hipStream_t)stream;
+    const int64_t nvec = n / vec;
+    if (dtype == BB_BF16)
+        hipLaunchKernelGGL(add_kernel<bf16>, dim3(grid_for(nvec)), dim3(256), 0, st, nvec, (const bf16*)a, (const bf16*)b, (bf16*)out);
+    else
+        hipLaunchKernelGGL(add_kernel<float>, dim3(grid_for(nvec)), dim3(256), 0, st, nvec, (const float*)a, (const float*)b, (float*)out);
+    BB_LAUNCH_CHECK();
+    return BB_OK;
+}
+
+template <typename S, typename D>
+__global__ __launch_bounds__(256) void cast_kernel(int64_t n, const S* __restrict__ src, D* __restrict__ dst) {
+    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (int64_t)gridDim.x * 256)
+        Elem<D>::store(dst + i, Elem<S>::load(src + i));
+}
+
+extern "C" int bb_cast(int src_dtype, int dst_dtype, int64_t n, const void* src, void* dst, void* stream) {
+    BB_REQUIRE((src_dtype == BB_F32 || src_dtype == BB_BF16) && (dst_dtype == BB_F32 || dst_dtype == BB_BF16),
+               "bb_cast: bad dtype");
+    BB_REQUIRE(n >= 0 && src && dst, "bb_cast: bad arguments");
+    if (n == 0) return BB_OK;
+    hipStream_t st = (hipStream_t)stream;
+    dim3 grid(grid_for(n)), block(256);
+    if (src_dtype == BB_F32 && dst_dtype == BB_BF16)
+        hipLaunchKernelGGL((cast_kernel<float, bf16>), grid, block, 0, st, n, (const float*)src, (bf16*)dst);
+    else if (src_dtype == BB_BF16 && dst_dtype == BB_F32)
+        hipLaunchKernelGGL((cast_kernel<bf16, float>), grid, block, 0, st, n, (const bf16*)src, (float*)dst);
+    else if (src_dtype == BB_F32)
+        hipLaunchKernelGGL((cast_kernel<float, float>), grid, block, 0, st, n, (const float*)src, (float*)dst);
+    else
+        hipLaunchKernelGGL((cast_kernel<bf16, bf16>), grid, block, 0, st, n, (const bf16*)src, (bf16*)dst);
+    BB_LAUNCH_CHECK();
+    return BB_OK;
+}
+
+__global__ __launch_bounds__(256) void fill_kernel(float* dst, int64_t n, float value) {
+    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (int64_t)gridDim.x * 256) dst[i] = value;
+}
+extern "C" int bb_fill_f32(float* dst, int64_t n, float value, void* stream) {
+    BB_REQUIRE(n >= 0 && (dst || n == 0), "bb_fill_f32: bad arguments");
+    if (n == 0) return BB_OK;
+    hipLaunchKernelGGL(fill_kernel, dim3(grid_for(n)), dim3(256), 0, (hipStream_t)stream, dst, n, value);
+    BB_LAUNCH_CHECK();
+    return BB_OK;
+}
+
+// =========================================================================================
+// MSE head: loss and its gradient in one pass over y
+// =========================================================================================
+constexpr int MSE_BLOCKS = 1024;
+
+template <typename T>
+__global__ __launch_bounds__(256) void mse_partial_kernel(int64_t n, const T* __restrict__ y, const T* __restrict__ t,
+                                                          T* __restrict__ dy, float gscale, float* __restrict__ partial) {
+    __shared__ float red[4];
+    // contiguous slice per block so the summation order is fixed by n alone
+    const int64_t per = (n + MSE_BLOCKS - 1) / MSE_BLOCKS;
+    const int64_t lo = (int64_t)blockIdx.x * per;
+    const int64_t hi = lo + per < n ? lo + per : n;
+    float s = 0.f;
+    for (int64_t i = lo + threadIdx.x; i < hi; i += 256) {
+        const float d = Elem<T>::load(y + i) - Elem<T>::load(t + i);
+        s += d * d;
+        if (dy) Elem<T>::store(dy + i, gscale * d);
+    }
+    s = wave_sum(s);
+    if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = s;
+    __syncthreads();
+    if (threadIdx.x == 0) partial[blockIdx.x] = (red[0] + red[1]) + (red[2] + red[3]);
+}
+
+__global__ __launch_bounds__(64) void mse_final_kernel(const float* __restrict__ partial, float inv_n, int accumulate,
+                                                       float* __restrict__ loss) {
+    float s = 0.f;
+    for (int i = threadIdx.x; i < MSE_BLOCKS; i += 64) s += partial[i];
+    s = wave_sum(s);
+    if (threadIdx.x == 0) loss[0] = (accumulate ? loss[0] : 0.f) + s * inv_n;
+}
+
+extern "C" int64_t bb_mse_workspace(void) { return MSE_BLOCKS; }
+
+extern "C" int bb_mse_fwd_bwd(int dtype, int64_t n, const void* y, const void* target, void* dy, float grad_scale,
+                              float* loss_out, int accumulate_loss, float* workspace, void* stream) {
+    BB_REQUIRE(dtype == BB_F32 || dtype == BB_BF16, "bb_mse_fwd_bwd: bad dtype %d", dtype);
+    BB_REQUIRE(n > 0 && y && target && loss_out && workspace, "bb_mse_fwd_bwd: bad arguments");
+    hipStream_t st = (hipStream_t)stream;
+    const float gs = grad_scale * 2.0f / (float)n;
+    if (dtype == BB_BF16)
+        hipLaunchKernelGGL(mse_partial_kernel<bf16>, dim3(MSE_BLOCKS), dim3(256), 0, st, n, (const bf16*)y, (const bf16*)target, (bf16*)dy, gs, workspace);
+    else
+        hipLaunchKernelGGL(mse_partial_kernel<float>, dim3(MSE_BLOCKS), dim3(256), 0, st, n, (const float*)y, (const float*)target, (float*)dy, gs, workspace);
+    hipLaunchKernelGGL(mse_final_kernel, dim3(1), dim3(64), 0, st, workspace, 1.0f / (float)n, accumulate_loss, loss_out);
+    BB_LAUNCH_CHECK();
+    return BB_OK;
+}

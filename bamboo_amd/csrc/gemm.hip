@@ -1,0 +1,453 @@
+// MFMA GEMM for gfx950: bf16 (v_mfma_f32_32x32x16_bf16) and fp32 (v_mfma_f32_32x32x2_f32),
+// LDS-tiled, double-buffered, batched with two-level strides, fused epilogues.
+//
+// Stands in for F.linear / torch.matmul and their autograd backward in the reference layer
+// (DeepSpeedExamples/pipeline_parallelism/transformer.py:121,127,136-146,158).
+//
+// bf16 data path.  Both operand tiles are kept in LDS "k-contiguous": tile row r (an m- or
+// n-index) owns 64 consecutive k values = 8 chunks of 16 bytes, chunk c stored at chunk slot
+// c ^ swz(r) so that the 16-byte fragment reads of 16 consecutive rows hit distinct banks.
+// An operand whose memory layout is k-major (the transposed operand of NN / TN) is loaded as
+// 16-byte vectors along its contiguous dimension and transposed in registers before the LDS
+// store, so the MFMA side never changes.
+#include "common.h"
+
+struct GemmArgs {
+    const void* A; const void* B; void* C;
+    const void* bias; const void* aux_in; void* aux_out; const void* resid;
+    int64_t lda, ldb, ldc, ldaux;
+    int64_t sA1, sA2, sB1, sB2, sC1, sC2;
+    int M, N, K, nb2;
+    float alpha;
+    int epilogue, act, accumulate, c_f32;
+    int tiles_m, tiles_n;
+};
+
+// ---- tile order: consecutive logical tiles land on the same XCD (workgroups are dealt
+// round-robin over the 8 XCDs, each with a private L2), and walk the output in column
+// panels of GROUP_M row-tiles so that an XCD's resident tiles share A rows and B columns.
+__device__ __forceinline__ void tile_coords(int bid, int tiles_m, int tiles_n, int& tm, int& tn) {
+    const int total = tiles_m * tiles_n;
+    int lid = bid;
+    const int per = total / 8;
+    if (per > 0 && bid < per * 8) lid = (bid % 8) * per + bid / 8;
+    constexpr int GROUP_M = 8;
+    const int width = GROUP_M * tiles_n;
+    const int group = lid / width;
+    const int first_m = group * GROUP_M;
+    const int gsize = min(tiles_m - first_m, GROUP_M);
+    tm = first_m + (lid % width) % gsize;
+    tn = (lid % width) / gsize;
+}
+
+// Generic scalar epilogue.  T = operand dtype (bias/aux/resid), output fp32 or T.
+template <typename T>
+__device__ __forceinline__ void epilogue_elem(const GemmArgs& g, int64_t coff, int64_t xoff, int m,
+                                              int n, float acc) {
+    float v = acc * g.alpha;
+    if (g.bias) v += Elem<T>::load((const T*)g.bias + n);
+    const int64_t ci = coff + (int64_t)m * g.ldc + n;
+    const int64_t xi = xoff + (int64_t)m * g.ldaux + n;
+    if (g.epilogue == BB_EPI_ACT) {
+        if (g.aux_out) Elem<T>::store((T*)g.aux_out + xi, v);
+        v = act_f(v, g.act);
+    } else if (g.epilogue == BB_EPI_DACT) {
+        v *= dact_f(Elem<T>::load((const T*)g.aux_in + xi), g.act);
+    } else if (g.epilogue == BB_EPI_RESIDUAL) {
+        v += Elem<T>::load((const T*)g.resid + xi);
+    }
+    if (g.c_f32) {
+        float* c = (float*)g.C + ci;
+        *c = g.accumulate ? (*c + v) : v;
+    } else {
+        Elem<T>::store((T*)g.C + ci, v);
+    }
+}
+
+// =========================================================================================
+// bf16 kernel
+// =========================================================================================
+__device__ __forceinline__ int swz(int row) {
+    return ((row >> 1) & 7) ^ ((row & 1) << 2) ^ ((row >> 4) & 7);
+}
+
+// Loader of one operand tile: R tile rows (m or n index) x 64 k.  TR = operand memory is
+// k-major ([K, rows], rows contiguous).
+template <int R, int NT, bool TR> struct TileLoader;
+
+template <int R, int NT> struct TileLoader<R, NT, false> {
+    static constexpr int NCH = R * 8 / NT;  // 16-byte chunks per thread
+    static_assert(NCH >= 1, "tile too small for the block");
+    u32x4 regs[NCH];
+    __device__ __forceinline__ void gload(const bf16* base, int64_t ld, int row0, int rows, int k0,
+                                          int K, int tid) {
+#pragma unroll
+        for (int i = 0; i < NCH; ++i) {
+            const int c = tid + i * NT;
+            const int r = c >> 3, kc = c & 7;
+            const int gr = row0 + r, gk = k0 + kc * 8;
+            u32x4 v = {0u, 0u, 0u, 0u};
+            if (gr < rows && gk < K) v = *(const u32x4*)(base + (int64_t)gr * ld + gk);
+            regs[i] = v;
+        }
+    }
+    __device__ __forceinline__ void sstore(bf16* lds, int tid) const {
+#pragma unroll
+        for (int i = 0; i < NCH; ++i) {
+            const int c = tid + i * NT;
+            const int r = c >> 3, kc = c & 7;
+            *(u32x4*)(lds + r * 64 + ((kc ^ swz(r)) << 3)) = regs[i];
+        }
+    }
+};
+
+template <int R, int NT> struct TileLoader<R, NT, true> {
+    // each thread owns an 8-row x KB-k block: KB 16-byte loads, each 8 rows at one k
+    static constexpr int KB = 8 * R / NT;
+    static_assert(KB == 2 || KB == 4 || KB == 8, "unsupported tile/block combination");
+    static constexpr int NRB = R / 8;
+    u32x4 regs[KB];
+    __device__ __forceinline__ void gload(const bf16* base, int64_t ld, int row0, int rows, int k0,
+                                          int K, int tid) {
+        const int rb = tid % NRB, kb = tid / NRB;
+        const int gr = row0 + rb * 8;
+#pragma unroll
+        for (int j = 0; j < KB; ++j) {
+            const int gk = k0 + kb * KB + j;
+            u32x4 v = {0u, 0u, 0u, 0u};
+            if (gr < rows && gk < K) v = *(const u32x4*)(base + (int64_t)gk * ld + gr);
+            regs[j] = v;
+        }
+    }
+    __device__ __forceinline__ void sstore(bf16* lds, int tid) const {
+        const int rb = tid % NRB, kb = tid / NRB;
+        const int ko = kb * KB;  // k offset inside the 64-wide tile
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            // row i of the block: element i of every loaded vector
+            uint32_t w[KB / 2];
+#pragma unroll
+            for (int j = 0; j < KB / 2; ++j) {
+                const uint32_t lo = regs[2 * j][i >> 1], hi = regs[2 * j + 1][i >> 1];
+                w[j] = (i & 1) ? ((lo >> 16) | (hi & 0xffff0000u)) : ((lo & 0xffffu) | (hi << 16));
+            }
+            const int r = rb * 8 + i;
+            bf16* dst = lds + r * 64 + ((((ko >> 3) ^ swz(r))) << 3) + (ko & 7);
+            if constexpr (KB == 8) {
+                u32x4 t = {w[0], w[1], w[2], w[3]};
+                *(u32x4*)dst = t;
+            } else if constexpr (KB == 4) {
+                u32x2 t = {w[0], w[1]};
+                *(u32x2*)dst = t;
+            } else {
+                *(uint32_t*)dst = w[0];
+            }
+        }
+    }
+};
+
+template <int BM, int BN, int WM, int WN, bool TA, bool TB>
+__global__ __launch_bounds__(WM* WN * 64) void gemm_bf16_kernel(const GemmArgs g) {
+    constexpr int NT = WM * WN * 64, BK = 64;
+    constexpr int WTM = BM / WM, WTN = BN / WN, TM = WTM / 32, TN = WTN / 32;
+    static_assert(TM >= 1 && TN >= 1, "wave tile must hold a 32x32 MFMA tile");
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+    bf16* As = (bf16*)smem;            // [2][BM*BK]
+    bf16* Bs = As + 2 * BM * BK;       // [2][BN*BK]
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wm = wave / WN, wn = wave % WN;
+    int tile_m, tile_n;
+    tile_coords(blockIdx.x, g.tiles_m, g.tiles_n, tile_m, tile_n);
+    const int m0 = tile_m * BM, n0 = tile_n * BN;
+    const int b1 = blockIdx.z / g.nb2, b2 = blockIdx.z % g.nb2;
+    const bf16* A = (const bf16*)g.A + b1 * g.sA1 + b2 * g.sA2;
+    const bf16* B = (const bf16*)g.B + b1 * g.sB1 + b2 * g.sB2;
+    const int64_t coff = b1 * g.sC1 + b2 * g.sC2;
+
+    TileLoader<BM, NT, TA> la;
+    TileLoader<BN, NT, TB> lb;
+
+    f32x16 acc[TM][TN];
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+
+    const int KT = (g.K + BK - 1) / BK;
+    la.gload(A, g.lda, m0, g.M, 0, g.K, tid);
+    lb.gload(B, g.ldb, n0, g.N, 0, g.K, tid);
+    la.sstore(As, tid);
+    lb.sstore(Bs, tid);
+    __syncthreads();
+
+    const int frow = lane & 31, fk = lane >> 5;
+    for (int kt = 0; kt < KT; ++kt) {
+        const int cur = kt & 1;
+        const bool more = kt + 1 < KT;
+        if (more) {
+            la.gload(A, g.lda, m0, g.M, (kt + 1) * BK, g.K, tid);
+            lb.gload(B, g.ldb, n0, g.N, (kt + 1) * BK, g.K, tid);
+        }
+        const bf16* as = As + cur * BM * BK;
+        const bf16* bs = Bs + cur * BN * BK;
+#pragma unroll
+        for (int ks = 0; ks < BK / 16; ++ks) {
+            bf16x8 af[TM], bfr[TN];
+#pragma unroll
+            for (int i = 0; i < TM; ++i) {
+                const int r = wm * WTM + i * 32 + frow;
+                af[i] = *(const bf16x8*)(as + r * 64 + (((ks * 2 + fk) ^ swz(r)) << 3));
+            }
+#pragma unroll
+            for (int j = 0; j < TN; ++j) {
+                const int r = wn * WTN + j * 32 + frow;
+                bfr[j] = *(const bf16x8*)(bs + r * 64 + (((ks * 2 + fk) ^ swz(r)) << 3));
+            }
+#pragma unroll
+            for (int i = 0; i < TM; ++i)
+#pragma unroll
+                for (int j = 0; j < TN; ++j)
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[i], bfr[j], acc[i][j], 0, 0, 0);
+        }
+        if (more) {
+            la.sstore(As + (cur ^ 1) * BM * BK, tid);
+            lb.sstore(Bs + (cur ^ 1) * BN * BK, tid);
+        }
+        __syncthreads();
+    }
+
+    // epilogue: lane holds column (lane & 31); register r is row 8*(r/4) + 4*(lane/32) + r%4
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j) {
+            const int n = n0 + wn * WTN + j * 32 + (lane & 31);
+            if (n >= g.N) continue;
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int m = m0 + wm * WTM + i * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
+                if (m < g.M) epilogue_elem<bf16>(g, coff, coff, m, n, acc[i][j][r]);
+            }
+        }
+}
+
+// =========================================================================================
+// fp32 kernel: 128x128x16 tiles, 4 waves (2x2), LDS k-major with padded rows.
+// =========================================================================================
+template <bool TA, bool TB>
+__global__ __launch_bounds__(256) void gemm_f32_kernel(const GemmArgs g) {
+    constexpr int BM = 128, BN = 128, BK = 16, LDS_LD = 132, NT = 256;
+    __shared__ __attribute__((aligned(16))) float As[2][BK * LDS_LD];
+    __shared__ __attribute__((aligned(16))) float Bs[2][BK * LDS_LD];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wm = wave >> 1, wn = wave & 1;
+    int tile_m, tile_n;
+    tile_coords(blockIdx.x, g.tiles_m, g.tiles_n, tile_m, tile_n);
+    const int m0 = tile_m * BM, n0 = tile_n * BN;
+    const int b1 = blockIdx.z / g.nb2, b2 = blockIdx.z % g.nb2;
+    const float* A = (const float*)g.A + b1 * g.sA1 + b2 * g.sA2;
+    const float* B = (const float*)g.B + b1 * g.sB1 + b2 * g.sB2;
+    const int64_t coff = b1 * g.sC1 + b2 * g.sC2;
+
+    f32x4 ra[2], rb[2];
+    auto gload = [&](const float* base, int64_t ld, int row0, int rows, int k0, bool tr, f32x4 (&r)[2]) {
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+            const int c = tid + i * NT;
+            f32x4 v = {0.f, 0.f, 0.f, 0.f};
+            if (!tr) {
+                const int row = c >> 2, kq = c & 3;
+                if (row0 + row < rows && k0 + kq * 4 < g.K)
+                    v = *(const f32x4*)(base + (int64_t)(row0 + row) * ld + k0 + kq * 4);
+            } else {
+                const int k = c >> 5, rq = c & 31;
+                if (row0 + rq * 4 < rows && k0 + k < g.K)
+                    v = *(const f32x4*)(base + (int64_t)(k0 + k) * ld + row0 + rq * 4);
+            }
+            r[i] = v;
+        }
+    };
+    auto sstore = [&](float* lds, bool tr, const f32x4 (&r)[2]) {
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+            const int c = tid + i * NT;
+            if (!tr) {
+                const int row = c >> 2, kq = c & 3;
+#pragma unroll
+                for (int e = 0; e < 4; ++e) lds[(kq * 4 + e) * LDS_LD + row] = r[i][e];
+            } else {
+                const int k = c >> 5, rq = c & 31;
+                *(f32x4*)(lds + k * LDS_LD + rq * 4) = r[i];
+            }
+        }
+    };
+
+    f32x16 acc[2][2];
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+
+    const int KT = (g.K + BK - 1) / BK;
+    gload(A, g.lda, m0, g.M, 0, TA, ra);
+    gload(B, g.ldb, n0, g.N, 0, TB, rb);
+    sstore(As[0], TA, ra);
+    sstore(Bs[0], TB, rb);
+    __syncthreads();
+    for (int kt = 0; kt < KT; ++kt) {
+        const int cur = kt & 1;
+        const bool more = kt + 1 < KT;
+        if (more) {
+            gload(A, g.lda, m0, g.M, (kt + 1) * BK, TA, ra);
+            gload(B, g.ldb, n0, g.N, (kt + 1) * BK, TB, rb);
+        }
+#pragma unroll
+        for (int ks = 0; ks < BK / 2; ++ks) {
+            float af[2], bfr[2];
+            const int kk = ks * 2 + (lane >> 5);
+#pragma unroll
+            for (int i = 0; i < 2; ++i) af[i] = As[cur][kk * LDS_LD + wm * 64 + i * 32 + (lane & 31)];
+#pragma unroll
+            for (int j = 0; j < 2; ++j) bfr[j] = Bs[cur][kk * LDS_LD + wn * 64 + j * 32 + (lane & 31)];
+#pragma unroll
+            for (int i = 0; i < 2; ++i)
+#pragma unroll
+                for (int j = 0; j < 2; ++j)
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(af[i], bfr[j], acc[i][j], 0, 0, 0);
+        }
+        if (more) {
+            sstore(As[cur ^ 1], TA, ra);
+            sstore(Bs[cur ^ 1], TB, rb);
+        }
+        __syncthreads();
+    }
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+            const int n = n0 + wn * 64 + j * 32 + (lane & 31);
+            if (n >= g.N) continue;
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int m = m0 + wm * 64 + i * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
+                if (m < g.M) epilogue_elem<float>(g, coff, coff, m, n, acc[i][j][r]);
+            }
+        }
+}
+
+// =========================================================================================
+// host dispatch
+// =========================================================================================
+template <int BM, int BN, int WM, int WN, bool TA, bool TB>
+static int launch_bf16(GemmArgs& g, int batches, hipStream_t st) {
+    constexpr int smem = 2 * (BM + BN) * 64 * 2;
+    auto kern = gemm_bf16_kernel<BM, BN, WM, WN, TA, TB>;
+    static bool configured = false;
+    if (!configured) {
+        BB_HIP_CHECK(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, smem));
+        configured = true;
+    }
+    g.tiles_m = (g.M + BM - 1) / BM;
+    g.tiles_n = (g.N + BN - 1) / BN;
+    dim3 grid(g.tiles_m * g.tiles_n, 1, batches);
+    hipLaunchKernelGGL(kern, grid, dim3(WM * WN * 64), smem, st, g);
+    BB_LAUNCH_CHECK();
+    return BB_OK;
+}
+
+// Tile choice: the largest tile that still gives every CU work; small problems (attention
+// heads: 64-wide operands) take the 128x64 / 64x128 tiles.
+enum Bf16Tile { T128x64 = 0, T64x128, T256x256, T256x128, T128x128 };
+static const char* const kBf16TileNames[] = {"128x64", "64x128", "256x256", "256x128", "128x128"};
+
+static Bf16Tile pick_bf16_tile(int M, int N, int64_t batches) {
+    const int64_t t256 = (int64_t)((M + 255) / 256) * ((N + 255) / 256) * batches;
+    const int64_t t2128 = (int64_t)((M + 255) / 256) * ((N + 127) / 128) * batches;
+    if (N <= 64) return T128x64;
+    if (M <= 64) return T64x128;
+    if (M >= 256 && N >= 256 && t256 >= 256) return T256x256;
+    if (M >= 256 && N >= 128 && t2128 >= 200) return T256x128;
+    return T128x128;
+}
+
+template <bool TA, bool TB> static int dispatch_bf16(GemmArgs& g, int batches, hipStream_t st) {
+    switch (pick_bf16_tile(g.M, g.N, batches)) {
+        case T128x64: return launch_bf16<128, 64, 4, 1, TA, TB>(g, batches, st);
+        case T64x128: return launch_bf16<64, 128, 1, 4, TA, TB>(g, batches, st);
+        case T256x256: return launch_bf16<256, 256, 2, 4, TA, TB>(g, batches, st);
+        case T256x128: return launch_bf16<256, 128, 4, 2, TA, TB>(g, batches, st);
+        default: return launch_bf16<128, 128, 2, 2, TA, TB>(g, batches, st);
+    }
+}
+
+template <bool TA, bool TB> static int dispatch_f32(GemmArgs& g, int batches, hipStream_t st) {
+    g.tiles_m = (g.M + 127) / 128;
+    g.tiles_n = (g.N + 127) / 128;
+    dim3 grid(g.tiles_m * g.tiles_n, 1, batches);
+    hipLaunchKernelGGL((gemm_f32_kernel<TA, TB>), grid, dim3(256), 0, st, g);
+    BB_LAUNCH_CHECK();
+    return BB_OK;
+}
+
+extern "C" int bb_gemm_variant(const bb_gemm_desc* d, char* out, int out_len) {
+    BB_REQUIRE(d && out && out_len > 0, "bb_gemm_variant: bad arguments");
+    static const char* const layouts[] = {"nt", "nn", "tn"};
+    BB_REQUIRE(d->layout >= BB_NT && d->layout <= BB_TN, "bb_gemm_variant: bad layout %d", d->layout);
+    const int64_t batches = (int64_t)(d->nb1 > 0 ? d->nb1 : 1) * (d->nb2 > 0 ? d->nb2 : 1);
+    if (d->dtype == BB_BF16)
+        snprintf(out, out_len, "bf16_%s_%s", layouts[d->layout], kBf16TileNames[pick_bf16_tile(d->M, d->N, batches)]);
+    else
+        snprintf(out, out_len, "f32_%s_128x128", layouts[d->layout]);
+    return BB_OK;
+}
+
+extern "C" int bb_gemm(const bb_gemm_desc* d, void* stream) {
+    BB_REQUIRE(d != nullptr, "bb_gemm: null descriptor");
+    BB_REQUIRE(d->dtype == BB_F32 || d->dtype == BB_BF16, "bb_gemm: bad dtype %d", d->dtype);
+    BB_REQUIRE(d->c_dtype == d->dtype || d->c_dtype == BB_F32, "bb_gemm: bad c_dtype %d", d->c_dtype);
+    BB_REQUIRE(d->layout >= BB_NT && d->layout <= BB_TN, "bb_gemm: bad layout %d", d->layout);
+    BB_REQUIRE(d->M >= 0 && d->N >= 0 && d->K >= 0, "bb_gemm: negative dimension");
+    BB_REQUIRE(d->A && d->B && d->C, "bb_gemm: null operand");
+    BB_REQUIRE(!d->accumulate || d->c_dtype == BB_F32, "bb_gemm: accumulate needs an fp32 C");
+    BB_REQUIRE(d->epilogue >= BB_EPI_NONE && d->epilogue <= BB_EPI_RESIDUAL, "bb_gemm: bad epilogue");
+    BB_REQUIRE(d->epilogue != BB_EPI_DACT || d->aux_in, "bb_gemm: DACT epilogue needs aux_in");
+    BB_REQUIRE(d->epilogue != BB_EPI_RESIDUAL || d->resid, "bb_gemm: RESIDUAL epilogue needs resid");
+    const int nb1 = d->nb1 > 0 ? d->nb1 : 1, nb2 = d->nb2 > 0 ? d->nb2 : 1;
+    const int64_t batches = (int64_t)nb1 * nb2;
+    BB_REQUIRE(batches <= 65535, "bb_gemm: too many batches (%lld)", (long long)batches);
+    const int vec = d->dtype == BB_BF16 ? 8 : 4;
+    const bool ta = d->layout == BB_TN, tb = d->layout != BB_NT;
+    // the contiguous dimension of every operand is read in 16-byte vectors
+    const int a_contig = ta ? d->M : d->K, b_contig = tb ? d->N : d->K;
+    BB_REQUIRE(a_contig % vec == 0 && d->lda % vec == 0, "bb_gemm: A contiguous dim/lda must be a multiple of %d", vec);
+    BB_REQUIRE(b_contig % vec == 0 && d->ldb % vec == 0, "bb_gemm: B contiguous dim/ldb must be a multiple of %d", vec);
+    BB_REQUIRE(((uintptr_t)d->A % 16) == 0 && ((uintptr_t)d->B % 16) == 0, "bb_gemm: operands must be 16-byte aligned");
+    BB_REQUIRE(d->sA1 % vec == 0 && d->sA2 % vec == 0 && d->sB1 % vec == 0 && d->sB2 % vec == 0,
+               "bb_gemm: batch strides of A/B must be multiples of %d", vec);
+    BB_REQUIRE(d->lda >= a_contig && d->ldb >= b_contig && d->ldc >= d->N, "bb_gemm: leading dimension too small");
+    if (d->M == 0 || d->N == 0) return BB_OK;
+
+    GemmArgs g;
+    g.A = d->A; g.B = d->B; g.C = d->C;
+    g.bias = d->bias; g.aux_in = d->aux_in; g.aux_out = d->aux_out; g.resid = d->resid;
+    g.lda = d->lda; g.ldb = d->ldb; g.ldc = d->ldc; g.ldaux = d->ldaux > 0 ? d->ldaux : d->ldc;
+    g.sA1 = d->sA1; g.sA2 = d->sA2; g.sB1 = d->sB1; g.sB2 = d->sB2; g.sC1 = d->sC1; g.sC2 = d->sC2;
+    g.M = d->M; g.N = d->N; g.K = d->K; g.nb2 = nb2;
+    g.alpha = d->alpha;
+    g.epilogue = d->epilogue; g.act = d->act; g.accumulate = d->accumulate;
+    g.c_f32 = (d->c_dtype == BB_F32);
+    hipStream_t st = (hipStream_t)stream;
+    if (d->dtype == BB_BF16) {
+        if (!ta && !tb) return dispatch_bf16<false, false>(g, (int)batches, st);
+        if (!ta && tb) return dispatch_bf16<false, true>(g, (int)batches, st);
+        return dispatch_bf16<true, true>(g, (int)batches, st);
+    }
+    if (!ta && !tb) return dispatch_f32<false, false>(g, (int)batches, st);
+    if (!ta && tb) return dispatch_f32<false, true>(g, (int)batches, st);
+    return dispatch_f32<true, true>(g, (int)batches, st);
+}

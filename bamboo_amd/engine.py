@@ -1,0 +1,465 @@
+"""``PipelineEngine``: executes the instruction stream of one pipeline stage on one MI355X.
+
+Surface of the reference engine (deepspeed/runtime/pipe/engine.py): constructor keywords
+``redundancy_level, sync_save, eager_recovery`` (:104-105), ``train_batch(data_iter, debug,
+mem_status, mem_log)`` (:1068-1423), attributes ``micro_batches, micro_batch_size, stage_id,
+num_stages, stage_ids, r_stage_ids, pipe_buffers, global_steps``, the ``_exec_*`` handlers
+and ``_INSTRUCTION_MAP`` (:1626-2147, :2324-2394), and the ``NextStageException`` failover
+branch (:1190-1264).
+
+What is different underneath:
+  * layer arithmetic runs on the HIP kernels of ``libbamboo_hip.so`` with explicit backward
+    passes; activations needed by a backward live in a per-stage HBM stash indexed by
+    micro-batch (``buffer_id == micro_batch_id`` as in schedule.py:299-301);
+  * stage-to-stage transfers are served by an in-process :class:`SeededActivationQueue`;
+  * redundant forwards of the shadow stage can be issued to a second HIP stream so that the
+    GPU overlaps them with the stage's own kernels (``rc_stream=True``); with either setting
+    the shadow forward uses the same kernels, tiles and reduction order as a normal forward,
+    so its output is bit-identical;
+  * the Adam state of the shadow parameters is allocated up front, so promotion after a
+    failure extends the optimizer without allocating (reference rebuilds FusedAdam,
+    deepspeed/runtime/engine.py:306-333).
+"""
+import signal
+import time
+
+import torch
+
+from . import hip, schedule
+from .config import BambooConfig
+from .module import PipelineError, PipelineModule
+from .optim import FusedAdam
+from .p2p import AllReduceException, NextStageException, PrevStageException, SeededActivationQueue
+from .utils import get_redundant_stage_ids, get_redundant_user_stage_ids
+
+should_stop = False
+
+
+def sig_handler(signum, frame):
+    global should_stop
+    print("[Engine] Signal handler called with signal", signum)
+    should_stop = True
+
+
+class PipelineEngine:
+    def __init__(self, args=None, model=None, optimizer=None, model_parameters=None, training_data=None,
+                 lr_scheduler=None, mpu=None, dist_init_required=None, collate_fn=None, config=None,
+                 config_params=None, redundancy_level=0, sync_save=False, eager_recovery=False, prev_state={},
+                 activation_queue=None, rc_stream=False, install_signal_handler=True):
+        if not isinstance(model, PipelineModule):
+            raise PipelineError("model must base PipelineModule")
+        hip.init()
+        self.module = model
+        cfg = config if config is not None else config_params
+        if cfg is None and args is not None and getattr(args, "deepspeed_config", None):
+            cfg = args.deepspeed_config
+        self.config = cfg if isinstance(cfg, BambooConfig) else BambooConfig(cfg)
+        if self.config.compute_dtype != model.dtype:
+            raise PipelineError(f"config asks for {self.config.compute_dtype} but the module was built for {model.dtype}")
+        if install_signal_handler:
+            signal.signal(signal.SIGTERM, sig_handler)
+
+        self.device = model.device
+        self.micro_batch_size = self.config.train_micro_batch_size_per_gpu
+        self.micro_batches = self.config.gradient_accumulation_steps
+        self.num_stages = model.num_stages
+        self.stage_id = model.stage_id
+        self.stage_ids = [self.stage_id]
+        self.prev_stage = self.stage_id - 1
+        self.next_stage = self.stage_id + 1
+        self.dp_world_size = 1
+        self.global_rank = 0
+        self.global_steps = 0
+        self.global_samples = 0
+        self.training_data = training_data
+        self.data_iterator = None
+        self.lr_scheduler = lr_scheduler
+
+        if redundancy_level > 1:
+            raise NotImplementedError(f"R level {redundancy_level} > 1 is not supported now.")
+        if eager_recovery and redundancy_level == 0:
+            raise Exception("Must set redundancy level to enable eager recovery")
+        self.redundancy_level = redundancy_level
+        self.eager_recovery = eager_recovery
+        self.sync_save = sync_save
+        self.init_redundancy()
+
+        self.queue = activation_queue
+        if self.queue is None:
+            raise PipelineError("activation_queue is required: it stands in for the neighbouring stages "
+                                "(bamboo_amd.SeededActivationQueue)")
+        if self.queue.shape[0] != self.micro_batch_size:
+            raise PipelineError("activation queue micro-batch size differs from the config")
+        self.batch, self.seq = self.queue.shape[0], self.queue.shape[1]
+
+        # execution lanes: the stage's own work on the current stream, redundant forwards
+        # optionally on a second stream of the same (default) priority
+        self.main_stream = torch.cuda.current_stream(self.device)
+        self.rc_stream = torch.cuda.Stream(self.device) if (rc_stream and self.r_stage_ids and eager_recovery) else None
+        built = list(self.stage_ids) + (list(self.r_stage_ids) if self.eager_recovery else [])
+        self.ctx = model.prepare_context(built, self.batch, self.seq, stream=self.main_stream)
+        self.rc_ctx = self.ctx
+        if self.rc_stream is not None:
+            self.rc_ctx = model.prepare_context([], self.batch, self.seq, stream=self.rc_stream)
+        self.stash_bytes = 0
+        for sid in built:
+            self.stash_bytes += model.allocate_stash(sid, self.ctx, self.micro_batches)
+        self._fwd_done = [torch.cuda.Event() for _ in range(self.micro_batches)]
+
+        act_shape = (self.batch * self.seq, self.queue.shape[2])
+        self._input_grad_store = {
+            sid: [torch.empty(act_shape, dtype=model.dtype, device=self.device) for _ in range(self.micro_batches)]
+            for sid in built}
+        self._loss_grad = None
+        if model.loss_fn is not None:
+            self._loss_grad = torch.empty(act_shape, dtype=model.dtype, device=self.device)
+            self._loss_ws = torch.empty(hip.mse_workspace(), dtype=torch.float32, device=self.device)
+        self.total_loss = torch.zeros(1, dtype=torch.float32, device=self.device)
+
+        self.optimizer = optimizer if optimizer is not None else FusedAdam(
+            lr=self.config.lr, betas=self.config.betas, eps=self.config.eps, weight_decay=self.config.weight_decay,
+            adam_w_mode=self.config.adam_w_mode, bias_correction=self.config.bias_correction)
+        self.optimizer.add_stage(self.stage_id, model.stage_params[self.stage_id])
+
+        self.init_pipe_buffers()
+        self._failover = None          # (failed_step, curr_step) once the successor is absorbed
+        self.last_failover = None      # timing record of the most recent promotion
+        self._install_sched_generator()
+        self.tput_t0 = None
+        self.timers = {}
+
+    # ------------------------------------------------------------------ redundancy
+    def _inc(self, stage_id):
+        return (stage_id + 1) % self.num_stages
+
+    def _dec(self, stage_id):
+        return (stage_id - 1 + self.num_stages) % self.num_stages
+
+    def init_redundancy(self):
+        """Decide which stage is shadowed and materialise its layers (eager mode) or zero CPU
+        mirrors of its parameters and Adam state (lazy mode); reference engine.py:317-350."""
+        self.r_stage_ids = get_redundant_stage_ids(self.redundancy_level, self.stage_id, self.num_stages)
+        self.r_user_stage_ids = get_redundant_user_stage_ids(self.redundancy_level, self.stage_id, self.num_stages)
+        self.param_buffers, self.state_buffers = {}, {}
+        for sid in self.r_stage_ids:
+            self.param_buffers[sid], self.state_buffers[sid] = {}, {}
+            if self.eager_recovery:
+                self.module.build_layers(sid)
+                for name, p in self.module.get_named_param(sid):
+                    self.param_buffers[sid][name] = p
+                sp = self.module.stage_params[sid]
+                for i, name in enumerate(sp.index):
+                    self.state_buffers[sid][f"{i}.exp_avg"] = sp.view(sp.exp_avg, name)
+                    self.state_buffers[sid][f"{i}.exp_avg_sq"] = sp.view(sp.exp_avg_sq, name)
+            else:
+                names = self.module.allocate_param(sid, self.param_buffers[sid], "cpu")
+                for i, name in enumerate(names):
+                    z = self.param_buffers[sid][name]
+                    self.state_buffers[sid][f"{i}.exp_avg"] = torch.zeros_like(z)
+                    self.state_buffers[sid][f"{i}.exp_avg_sq"] = torch.zeros_like(z)
+
+    def init_pipe_buffers(self):
+        """Per-micro-batch buffer lists keyed like the reference's (engine.py:352-387)."""
+        self.num_pipe_buffers = 0
+        self.pipe_buffers = {"data": [], "label": [], f"input_{self.stage_id}": [], f"output_{self.stage_id}": []}
+        if self.stage_id != 0:
+            self.pipe_buffers[f"input_grad_{self.stage_id}"] = []
+        if self.eager_recovery:
+            for sid in self.r_stage_ids:
+                self.pipe_buffers[f"input_{sid}"] = []
+                self.pipe_buffers[f"output_{sid}"] = []
+                self.pipe_buffers[f"input_grad_{sid}"] = []
+        self.grad_layer = {}
+
+    def _reserve_pipe_buffers(self, num_buffers):
+        for key in self.pipe_buffers:
+            cur = self.pipe_buffers[key]
+            cur.extend([None] * (num_buffers - len(cur)))
+        self.num_pipe_buffers = max(self.num_pipe_buffers, num_buffers)
+
+    def _clean_pipe_buffers(self):
+        for key in self.pipe_buffers:
+            self.pipe_buffers[key] = [None] * len(self.pipe_buffers[key])
+
+    # ------------------------------------------------------------------ schedules
+    def _train_sched(self, stage_id):
+        return schedule.TrainSchedule(micro_batches=self.micro_batches, stages=self.num_stages, stage_id=stage_id)
+
+    def _install_sched_generator(self):
+        if self._failover is not None:
+            own, absorbed = self.stage_ids[0], self.stage_ids[1]
+            fs, cs = self._failover
+            self._generate_sched = lambda: schedule.NextStageFailoverSchedule(
+                self._train_sched(own), self._train_sched(absorbed), failed_step=fs, curr_step=cs)
+        elif self.r_stage_ids:
+            cls = schedule.EagerRecoverySchedule if self.eager_recovery else schedule.LazyRecoverySchedule
+            nxt = self.r_stage_ids[0]
+            self._generate_sched = lambda: cls(self._train_sched(self.stage_id), self._train_sched(nxt))
+        else:
+            self._generate_sched = lambda: self._train_sched(self.stage_id)
+
+    # ------------------------------------------------------------------ properties
+    def is_first_stage(self):
+        return self.stage_id == 0
+
+    def is_last_stage(self):
+        return self.stage_id == self.num_stages - 1
+
+    def train_batch_size(self):
+        return self.config.train_batch_size
+
+    def train_micro_batch_size_per_gpu(self):
+        return self.micro_batch_size
+
+    def gradient_accumulation_steps(self):
+        return self.micro_batches
+
+    def steps_per_print(self):
+        return self.config.steps_per_print
+
+    def wall_clock_breakdown(self):
+        return self.config.wall_clock_breakdown
+
+    def set_dataiterator(self, iterator):
+        self.data_iterator = iterator
+
+    def forward(self, *args, **kwargs):
+        raise PipelineError("Only train_batch() is accessible in pipeline mode.")
+
+    def backward(self, *args, **kwargs):
+        raise PipelineError("Only train_batch() is accessible in pipeline mode.")
+
+    def step(self, *args, **kwargs):
+        raise PipelineError("Only train_batch() is accessible in pipeline mode.")
+
+    def log(self, msg):
+        print(f"[ {self.global_rank:02d}|{self.global_steps:02d} ] {msg}", flush=True)
+
+    def mem_status(self, msg, print_rank=-1, reset_max=False):
+        alloc = torch.cuda.memory_allocated(self.device) / 2 ** 30
+        peak = torch.cuda.max_memory_allocated(self.device) / 2 ** 30
+        self.log(f"MEMSTATS {msg} current alloc={alloc:.2f}GB (peak {peak:.2f}GB) stash={self.stash_bytes / 2 ** 30:.2f}GB")
+        if reset_max:
+            torch.cuda.reset_peak_memory_stats(self.device)
+
+    # ------------------------------------------------------------------ train_batch
+    def train_batch(self, data_iter=None, debug=False, mem_status=False, mem_log=False):
+        """Run one batch (``micro_batches`` micro-batches) through the stage's schedule, including
+        the redundant forwards and, if the successor is lost, the failover; returns the mean
+        micro-batch loss where this process sees one (loss-head peer or last stage), else 0."""
+        global should_stop
+        if should_stop:
+            raise SystemExit(13)
+        if data_iter is not None:
+            self.set_dataiterator(data_iter)
+        elif self.data_iterator is None and self.training_data is not None:
+            self.data_iterator = iter(self.training_data)
+        self._reserve_pipe_buffers(self.micro_batches)
+        self.queue.start_batch()
+        self.total_loss.zero_()
+        self._debug = debug
+        t0 = time.perf_counter()
+
+        self.check_preemptions()
+        status = self._exec_schedule(self._generate_sched())
+        if status is not None:
+            step_i, exc = status
+            if isinstance(exc, NextStageException) and self.r_stage_ids:
+                self._handle_next_stage_failure(step_i)
+                status = self._exec_schedule(self._generate_sched())
+                if status is not None:
+                    raise status[1]
+                # later batches run the merged stream from its first step
+                self._failover = (0, 0)
+                self._install_sched_generator()
+            else:
+                raise exc
+        if self.rc_stream is not None:
+            self.main_stream.wait_stream(self.rc_stream)
+
+        if self.queue.grad_mode == "mse":
+            loss = self.queue.loss / self.micro_batches
+        else:
+            loss = self.total_loss / self.micro_batches
+        self.agg_train_loss = loss
+
+        if self.global_steps % self.steps_per_print() == 0 and (debug or self.wall_clock_breakdown()):
+            torch.cuda.synchronize(self.device)
+            elapsed = time.perf_counter() - t0
+            self.log(f"steps: {self.global_steps} loss: {float(loss):0.4f} iter time (s): {elapsed:0.3f} "
+                     f"samples/sec: {self.train_batch_size() / elapsed:0.3f}")
+        if mem_status or mem_log:
+            self.mem_status("AFTER BATCH")
+        self._clean_pipe_buffers()
+        return loss
+
+    def check_preemptions(self):
+        """Announced preemption (reference engine.py:731-809): if the successor is already known to
+        be gone before the batch starts, absorb it now and run the merged stream from step 0."""
+        q = self.queue
+        if (self._failover is None and self.r_stage_ids and q.dead_from is not None and q.dead_from <= 0
+                and q.dead_stage == self.stage_id):
+            self._promote(self.r_stage_ids[0], failed_step=0, curr_step=0)
+
+    def _handle_next_stage_failure(self, step_i):
+        t0 = time.perf_counter()
+        nxt = self.r_stage_ids[0]
+        # failed_step = 0: the in-process queue has seen nothing of the dead successor's traffic
+        # with the stage after it, so the replay keeps the successor's sends (the second replay
+        # case of the reference, schedule.py:349-353)
+        self._promote(nxt, failed_step=0, curr_step=step_i)
+        self.last_failover = {"step": step_i, "host_promote_s": time.perf_counter() - t0}
+
+    def _promote(self, absorbed, failed_step, curr_step):
+        """Turn the shadow layers of ``absorbed`` into active layers of this process
+        (reference engine.py:1190-1264)."""
+        if not self.eager_recovery:
+            # lazy mode keeps CPU mirrors only: materialise the layers from them now
+            self.module.build_layers(absorbed, self.param_buffers[absorbed])
+            self.ctx = self.module.prepare_context(self.stage_ids + [absorbed], self.batch, self.seq, stream=self.main_stream)
+            self.stash_bytes += self.module.allocate_stash(absorbed, self.ctx, self.micro_batches)
+            act_shape = (self.batch * self.seq, self.queue.shape[2])
+            self._input_grad_store[absorbed] = [torch.empty(act_shape, dtype=self.module.dtype, device=self.device)
+                                                for _ in range(self.micro_batches)]
+            for key in (f"input_{absorbed}", f"output_{absorbed}", f"input_grad_{absorbed}"):
+                self.pipe_buffers[key] = [None] * self.micro_batches
+        if self.rc_stream is not None:
+            self.main_stream.wait_stream(self.rc_stream)
+        self.rc_ctx = self.ctx
+        self.optimizer.add_stage(absorbed, self.module.stage_params[absorbed])
+        self.stage_ids.append(absorbed)
+        self.r_stage_ids = []
+        self.next_stage = self._inc(absorbed)
+        self._failover = (failed_step, curr_step)
+        self._install_sched_generator()
+
+    # ------------------------------------------------------------------ instruction handlers
+    def _exec_load_micro_batch(self, buffer_id):
+        if self.pipe_buffers["label"][buffer_id] is not None or self.pipe_buffers["data"][buffer_id] is not None:
+            return
+        if self.data_iterator is None:
+            raise PipelineError("LoadMicroBatch needs training_data or a data_iter")
+        batch = next(self.data_iterator)
+        hosted = self.stage_ids + self.r_stage_ids
+        if 0 in hosted:
+            x = batch[0].to(self.device).to(self.module.dtype)
+            self.pipe_buffers["data"][buffer_id] = x.reshape(-1, x.shape[-1]).contiguous()
+        if self.num_stages - 1 in hosted:
+            y = batch[1].to(self.device).to(self.module.dtype)
+            self.pipe_buffers["label"][buffer_id] = y.reshape(-1, y.shape[-1]).contiguous()
+
+    def _exec_recv_activations(self, buffer_id, stage_id):
+        if buffer_id == -1:
+            self.queue.ping(self._dec(stage_id))
+            return
+        key = f"input_{stage_id}"
+        if self.pipe_buffers[key][buffer_id] is not None:
+            return
+        producer = stage_id - 1
+        if producer in self.stage_ids:
+            # local hand-off: the producer's output buffer stays valid until the end of the batch
+            self.pipe_buffers[key][buffer_id] = self.pipe_buffers[f"output_{producer}"][buffer_id]
+        else:
+            x = self.queue.recv_activation(buffer_id)
+            self.pipe_buffers[key][buffer_id] = x.view(-1, x.shape[-1])
+
+    def _exec_send_activations(self, buffer_id, stage_id):
+        if buffer_id == -1:
+            self.queue.ping(stage_id)
+            return
+        if stage_id + 1 in self.stage_ids:
+            return
+        out = self.pipe_buffers[f"output_{stage_id}"][buffer_id]
+        self.queue.send_activation(buffer_id, out, stage_id, stream=self.main_stream)
+
+    def _exec_recv_grads(self, buffer_id, stage_id):
+        if stage_id + 1 in self.stage_ids:
+            self.grad_layer[stage_id] = self.pipe_buffers[f"input_grad_{stage_id + 1}"][buffer_id]
+        else:
+            g = self.queue.recv_grad(buffer_id, stage_id)
+            self.grad_layer[stage_id] = g.view(-1, g.shape[-1])
+
+    def _exec_send_grads(self, buffer_id, stage_id):
+        if stage_id - 1 in self.stage_ids:
+            return
+        self.queue.send_grad(buffer_id, self.pipe_buffers[f"input_grad_{stage_id}"][buffer_id], stage_id)
+
+    def _exec_forward_pass(self, buffer_id, stage_id):
+        out_key = f"output_{stage_id}"
+        if self.pipe_buffers[out_key][buffer_id] is not None:
+            return
+        inputs = self.pipe_buffers["data" if stage_id == 0 else f"input_{stage_id}"][buffer_id]
+        redundant = stage_id in self.r_stage_ids
+        ctx = self.rc_ctx if redundant else self.ctx
+        ctx.key_len = self.queue.key_len(buffer_id)
+        if redundant and self.rc_stream is not None:
+            self.rc_stream.wait_event(self._fwd_done[buffer_id])
+        out = self.module.forward(inputs, stage_id, slot=buffer_id, ctx=ctx)
+        self.pipe_buffers[out_key][buffer_id] = out
+        if not redundant and self.rc_stream is not None:
+            self._fwd_done[buffer_id].record(self.main_stream)
+        if stage_id == self.num_stages - 1 and not redundant and self.module.loss_fn is not None:
+            labels = self.pipe_buffers["label"][buffer_id]
+            self.module.loss_fn(out, labels, self._loss_grad, 1.0 / self.micro_batches, self.total_loss, True,
+                                self._loss_ws, stream=self.main_stream)
+            self.grad_layer[stage_id] = self._loss_grad
+
+    def _exec_backward_pass(self, buffer_id, stage_id):
+        grad = self.grad_layer.get(stage_id)
+        if grad is None:
+            raise PipelineError(f"BackwardPass({buffer_id}, {stage_id}) without a received gradient")
+        self.ctx.key_len = self.queue.key_len(buffer_id)
+        dst = self._input_grad_store[stage_id][buffer_id]
+        self.module.backward(grad, dst, stage_id, slot=buffer_id, ctx=self.ctx)
+        key = f"input_grad_{stage_id}"
+        if key in self.pipe_buffers:
+            self.pipe_buffers[key][buffer_id] = dst
+        self.grad_layer[stage_id] = None
+
+    def _exec_reduce_grads(self, stage_id):
+        # data-parallel world of one: the all-reduce of deepspeed/runtime/engine.py:1773-1802 is the identity
+        return
+
+    def _exec_optimizer_step(self):
+        self.optimizer.step(stream=self.main_stream)
+        if self.lr_scheduler is not None:
+            self.lr_scheduler.step()
+        self.global_steps += 1
+        self.global_samples += self.train_batch_size()
+
+    def _exec_send_weights(self, stage_id):
+        return
+
+    def _exec_recv_weights(self, stage_id):
+        return
+
+    _INSTRUCTION_MAP = {
+        schedule.OptimizerStep: _exec_optimizer_step,
+        schedule.ReduceGrads: _exec_reduce_grads,
+        schedule.LoadMicroBatch: _exec_load_micro_batch,
+        schedule.ForwardPass: _exec_forward_pass,
+        schedule.BackwardPass: _exec_backward_pass,
+        schedule.SendActivation: _exec_send_activations,
+        schedule.RecvActivation: _exec_recv_activations,
+        schedule.SendGrad: _exec_send_grads,
+        schedule.RecvGrad: _exec_recv_grads,
+        schedule.SendWeights: _exec_send_weights,
+        schedule.RecvWeights: _exec_recv_weights,
+    }
+
+    def _exec_schedule(self, pipe_schedule):
+        """Interpreter loop (reference engine.py:2339-2394): returns None, or ``(step, exception)``
+        when a neighbour failed."""
+        self._reserve_pipe_buffers(pipe_schedule.num_pipe_buffers())
+        for step_i, step_cmds in enumerate(pipe_schedule):
+            if self._debug:
+                self.log(f"step {step_i}: {step_cmds}")
+            try:
+                for cmd in step_cmds:
+                    handler = self._INSTRUCTION_MAP.get(type(cmd))
+                    if handler is None:
+                        raise RuntimeError(f"{self.__class__.__name__} does not understand instruction {cmd!r}")
+                    handler(self, **cmd.kwargs)
+            except (NextStageException, PrevStageException, AllReduceException) as e:
+                return step_i, e
+        return None

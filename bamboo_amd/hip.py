@@ -1,0 +1,293 @@
+"""ctypes binding of ``libbamboo_hip.so`` (the C ABI declared in ``include/bamboo_hip.h``).
+
+The library is the only compute path of this package: if it is missing, loading raises,
+and every wrapper raises :class:`HipKernelError` when the library reports a failure.
+Tensors are passed as raw device pointers (``tensor.data_ptr()``); torch is used only to
+own device memory and streams.
+"""
+import ctypes
+import os
+from ctypes import POINTER, Structure, byref, c_char_p, c_float, c_int, c_int32, c_int64, c_void_p
+
+import torch
+
+F32, BF16 = 0, 1
+NT, NN, TN = 0, 1, 2
+EPI_NONE, EPI_ACT, EPI_DACT, EPI_RESIDUAL = 0, 1, 2, 3
+ACT_RELU, ACT_GELU_TANH = 0, 1
+MASK_NONE, MASK_CAUSAL, MASK_KEY_PADDING = 0, 1, 2
+LN_STANDARD, LN_ANNOTATED = 0, 1
+
+ACT_CODES = {"relu": ACT_RELU, "gelu_tanh": ACT_GELU_TANH}
+MASK_CODES = {"none": MASK_NONE, "causal": MASK_CAUSAL, "key_padding": MASK_KEY_PADDING}
+LN_CODES = {"standard": LN_STANDARD, "annotated": LN_ANNOTATED}
+
+EXPORTS = (
+    "bb_version", "bb_last_error", "bb_init", "bb_gemm", "bb_gemm_variant", "bb_layernorm_fwd",
+    "bb_layernorm_bwd_workspace", "bb_layernorm_bwd", "bb_colsum_workspace", "bb_colsum_acc",
+    "bb_softmax_fwd", "bb_softmax_bwd", "bb_residual_add", "bb_mse_workspace", "bb_mse_fwd_bwd",
+    "bb_adam_multi", "bb_cast", "bb_fill_f32",
+)
+
+
+class HipKernelError(RuntimeError):
+    pass
+
+
+class GemmDesc(Structure):
+    _fields_ = [
+        ("layout", c_int32), ("dtype", c_int32), ("c_dtype", c_int32),
+        ("M", c_int32), ("N", c_int32), ("K", c_int32),
+        ("A", c_void_p), ("lda", c_int64),
+        ("B", c_void_p), ("ldb", c_int64),
+        ("C", c_void_p), ("ldc", c_int64),
+        ("nb1", c_int32), ("nb2", c_int32),
+        ("sA1", c_int64), ("sA2", c_int64), ("sB1", c_int64), ("sB2", c_int64),
+        ("sC1", c_int64), ("sC2", c_int64),
+        ("alpha", c_float), ("epilogue", c_int32), ("act", c_int32), ("accumulate", c_int32),
+        ("bias", c_void_p), ("aux_in", c_void_p), ("aux_out", c_void_p), ("resid", c_void_p),
+        ("ldaux", c_int64),
+    ]
+
+
+def library_path():
+    return os.path.join(os.path.dirname(os.path.abspath(__file__)), "lib", "libbamboo_hip.so")
+
+
+_lib = None
+
+
+def lib():
+    """Load (once) and return the shared library; raises if it has not been built."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    path = library_path()
+    if not os.path.exists(path):
+        raise HipKernelError(
+            f"{path} is missing: build it with `make -C bamboo_amd/csrc` (or __graft_entry__.build()); "
+            "there is no fallback compute path")
+    L = ctypes.CDLL(path)
+    L.bb_last_error.restype = c_char_p
+    L.bb_version.restype = c_int
+    L.bb_init.restype = c_int
+    L.bb_gemm.argtypes = [POINTER(GemmDesc), c_void_p]
+    L.bb_gemm_variant.argtypes = [POINTER(GemmDesc), c_char_p, c_int]
+    L.bb_layernorm_fwd.argtypes = [c_int, c_int, c_int, c_int, c_float, c_void_p, c_void_p, c_void_p,
+                                   c_void_p, c_void_p, c_void_p, c_void_p]
+    L.bb_layernorm_bwd_workspace.argtypes = [c_int]
+    L.bb_layernorm_bwd_workspace.restype = c_int64
+    L.bb_layernorm_bwd.argtypes = [c_int, c_int, c_int, c_int, c_float] + [c_void_p] * 11
+    L.bb_colsum_workspace.argtypes = [c_int]
+    L.bb_colsum_workspace.restype = c_int64
+    L.bb_colsum_acc.argtypes = [c_int, c_int, c_int, c_void_p, c_int64, c_void_p, c_void_p, c_void_p]
+    L.bb_softmax_fwd.argtypes = [c_int, c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p]
+    L.bb_softmax_bwd.argtypes = [c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p]
+    L.bb_residual_add.argtypes = [c_int, c_int64, c_void_p, c_void_p, c_void_p, c_void_p]
+    L.bb_mse_workspace.restype = c_int64
+    L.bb_mse_fwd_bwd.argtypes = [c_int, c_int64, c_void_p, c_void_p, c_void_p, c_float, c_void_p, c_int,
+                                 c_void_p, c_void_p]
+    L.bb_adam_multi.argtypes = [c_int, POINTER(c_void_p), POINTER(c_void_p), POINTER(c_void_p),
+                                POINTER(c_void_p), POINTER(c_void_p), POINTER(c_int64), c_float, c_float,
+                                c_float, c_float, c_int, c_int, c_int, c_float, c_int, c_void_p]
+    L.bb_cast.argtypes = [c_int, c_int, c_int64, c_void_p, c_void_p, c_void_p]
+    L.bb_fill_f32.argtypes = [c_void_p, c_int64, c_float, c_void_p]
+    _lib = L
+    return L
+
+
+def check(rc, what):
+    if rc != 0:
+        raise HipKernelError(f"{what} failed ({rc}): {lib().bb_last_error().decode()}")
+
+
+def init():
+    """Verify the current device is a gfx950 part."""
+    check(lib().bb_init(), "bb_init")
+
+
+def dtype_code(dt):
+    if dt == torch.float32:
+        return F32
+    if dt == torch.bfloat16:
+        return BF16
+    raise HipKernelError(f"unsupported dtype {dt}: the kernels take float32 or bfloat16")
+
+
+def stream_ptr(stream=None):
+    if stream is None:
+        stream = torch.cuda.current_stream()
+    return c_void_p(stream.cuda_stream)
+
+
+def _ptr(t):
+    return None if t is None else c_void_p(t.data_ptr())
+
+
+def _row_major(t, name):
+    if t.dim() != 2 or t.stride(1) != 1:
+        raise HipKernelError(f"{name}: expected a 2-D tensor with unit inner stride, got {tuple(t.shape)}/{t.stride()}")
+    return t.stride(0)
+
+
+# ------------------------------------------------------------------------------------- GEMM
+def gemm(layout, A, B, C, *, alpha=1.0, bias=None, epilogue=EPI_NONE, act=ACT_RELU, accumulate=False,
+         aux_in=None, aux_out=None, resid=None, stream=None):
+    """C = epilogue(alpha * op(A) op(B) [+ bias]) on 2-D row-major views (inner stride 1)."""
+    lda, ldb, ldc = _row_major(A, "A"), _row_major(B, "B"), _row_major(C, "C")
+    if layout == NT:
+        M, K = A.shape; N, Kb = B.shape
+    elif layout == NN:
+        M, K = A.shape; Kb, N = B.shape
+    elif layout == TN:
+        K, M = A.shape; Kb, N = B.shape
+    else:
+        raise HipKernelError(f"bad layout {layout}")
+    if K != Kb or tuple(C.shape) != (M, N):
+        raise HipKernelError(f"gemm shape mismatch: A{tuple(A.shape)} B{tuple(B.shape)} C{tuple(C.shape)} layout {layout}")
+    if A.dtype != B.dtype:
+        raise HipKernelError("gemm: A and B dtypes differ")
+    d = GemmDesc()
+    d.layout, d.dtype, d.c_dtype = layout, dtype_code(A.dtype), dtype_code(C.dtype)
+    d.M, d.N, d.K = M, N, K
+    d.A, d.lda, d.B, d.ldb, d.C, d.ldc = A.data_ptr(), lda, B.data_ptr(), ldb, C.data_ptr(), ldc
+    d.nb1 = d.nb2 = 1
+    d.alpha, d.epilogue, d.act, d.accumulate = alpha, epilogue, act, int(accumulate)
+    ldaux = 0
+    for t in (aux_in, aux_out, resid):
+        if t is not None:
+            if t.dtype != A.dtype or tuple(t.shape) != (M, N):
+                raise HipKernelError("gemm: aux/resid tensors must be [M,N] of the operand dtype")
+            ld = _row_major(t, "aux")
+            if ldaux and ld != ldaux:
+                raise HipKernelError("gemm: aux tensors must share one leading dimension")
+            ldaux = ld
+    d.ldaux = ldaux
+    if bias is not None and (bias.dtype != A.dtype or bias.numel() != N):
+        raise HipKernelError("gemm: bias must be [N] of the operand dtype")
+    d.bias = None if bias is None else bias.data_ptr()
+    d.aux_in = None if aux_in is None else aux_in.data_ptr()
+    d.aux_out = None if aux_out is None else aux_out.data_ptr()
+    d.resid = None if resid is None else resid.data_ptr()
+    if gemm_hook is not None:
+        gemm_hook(d, lambda: check(lib().bb_gemm(byref(d), stream_ptr(stream)), "bb_gemm"))
+    else:
+        check(lib().bb_gemm(byref(d), stream_ptr(stream)), "bb_gemm")
+    return C
+
+
+def gemm_variant(desc):
+    buf = ctypes.create_string_buffer(64)
+    check(lib().bb_gemm_variant(byref(desc), buf, 64), "bb_gemm_variant")
+    return buf.value.decode()
+
+
+# Optional observer called as hook(desc, launch) around every dense GEMM; `launch()` performs
+# the call.  Used by the benchmark to bracket launches with events; None in normal operation.
+gemm_hook = None
+
+
+def gemm_batched(layout, dtype, M, N, K, A_ptr, lda, sA, B_ptr, ldb, sB, C_ptr, ldc, sC, nb1, nb2, *,
+                 c_dtype=None, alpha=1.0, stream=None):
+    """Strided two-level batched GEMM on raw pointers (attention heads inside [rows, 3h] buffers).
+    sA/sB/sC are (outer, inner) element strides."""
+    d = GemmDesc()
+    d.layout, d.dtype, d.c_dtype = layout, dtype, dtype if c_dtype is None else c_dtype
+    d.M, d.N, d.K = M, N, K
+    d.A, d.lda, d.B, d.ldb, d.C, d.ldc = A_ptr, lda, B_ptr, ldb, C_ptr, ldc
+    d.nb1, d.nb2 = nb1, nb2
+    d.sA1, d.sA2 = sA
+    d.sB1, d.sB2 = sB
+    d.sC1, d.sC2 = sC
+    d.alpha, d.epilogue = alpha, EPI_NONE
+    check(lib().bb_gemm(byref(d), stream_ptr(stream)), "bb_gemm(batched)")
+
+
+# ------------------------------------------------------------------------- row-wise kernels
+def layernorm_fwd(x, gain, shift, y, mean, rinv, kind, eps, stream=None):
+    rows, cols = x.shape
+    check(lib().bb_layernorm_fwd(dtype_code(x.dtype), kind, rows, cols, eps, _ptr(x), _ptr(gain), _ptr(shift),
+                                 _ptr(y), _ptr(mean), _ptr(rinv), stream_ptr(stream)), "bb_layernorm_fwd")
+
+
+def layernorm_bwd_workspace(cols):
+    return int(lib().bb_layernorm_bwd_workspace(cols))
+
+
+def layernorm_bwd(x, gain, mean, rinv, dy, dres, dx, dgain, dshift, workspace, kind, eps, stream=None):
+    rows, cols = x.shape
+    if workspace.numel() < layernorm_bwd_workspace(cols) or workspace.dtype != torch.float32:
+        raise HipKernelError("layernorm_bwd: workspace too small")
+    check(lib().bb_layernorm_bwd(dtype_code(x.dtype), kind, rows, cols, eps, _ptr(x), _ptr(gain), _ptr(mean),
+                                 _ptr(rinv), _ptr(dy), _ptr(dres), _ptr(dx), _ptr(dgain), _ptr(dshift),
+                                 _ptr(workspace), stream_ptr(stream)), "bb_layernorm_bwd")
+
+
+def colsum_workspace(cols):
+    return int(lib().bb_colsum_workspace(cols))
+
+
+def colsum_acc(x, out, workspace, stream=None):
+    rows, cols = x.shape
+    ldx = _row_major(x, "x")
+    if workspace.numel() < colsum_workspace(cols) or out.dtype != torch.float32 or out.numel() != cols:
+        raise HipKernelError("colsum_acc: bad workspace/out")
+    check(lib().bb_colsum_acc(dtype_code(x.dtype), rows, cols, _ptr(x), ldx, _ptr(out), _ptr(workspace),
+                              stream_ptr(stream)), "bb_colsum_acc")
+
+
+def softmax_fwd(s, mask, key_len=None, stream=None):
+    b, h, sq, sk = s.shape
+    if not s.is_contiguous():
+        raise HipKernelError("softmax_fwd: scores must be contiguous")
+    check(lib().bb_softmax_fwd(dtype_code(s.dtype), mask, b, h, sq, sk, _ptr(s), _ptr(key_len),
+                               stream_ptr(stream)), "bb_softmax_fwd")
+
+
+def softmax_bwd(p, dp, stream=None):
+    b, h, sq, sk = p.shape
+    if not (p.is_contiguous() and dp.is_contiguous()):
+        raise HipKernelError("softmax_bwd: tensors must be contiguous")
+    check(lib().bb_softmax_bwd(dtype_code(p.dtype), b, h, sq, sk, _ptr(p), _ptr(dp), stream_ptr(stream)),
+          "bb_softmax_bwd")
+
+
+def residual_add(a, b, out, stream=None):
+    check(lib().bb_residual_add(dtype_code(a.dtype), a.numel(), _ptr(a), _ptr(b), _ptr(out), stream_ptr(stream)),
+          "bb_residual_add")
+
+
+def mse_workspace():
+    return int(lib().bb_mse_workspace())
+
+
+def mse_fwd_bwd(y, target, dy, grad_scale, loss_out, accumulate, workspace, stream=None):
+    check(lib().bb_mse_fwd_bwd(dtype_code(y.dtype), y.numel(), _ptr(y), _ptr(target), _ptr(dy), grad_scale,
+                               _ptr(loss_out), int(accumulate), _ptr(workspace), stream_ptr(stream)),
+          "bb_mse_fwd_bwd")
+
+
+def adam_multi(g, p, m, v, lowp, *, lr, beta1, beta2, eps, step, adam_w_mode=True, bias_correction=True,
+               weight_decay=0.0, zero_grad=False, stream=None):
+    """Lists of fp32 tensors g/p/m/v (same lengths); lowp: list of bf16 tensors or None entries, or None."""
+    n = len(p)
+    arr = lambda ts: (c_void_p * n)(*[None if t is None else t.data_ptr() for t in ts])
+    sizes = (c_int64 * n)(*[t.numel() for t in p])
+    for a, b_, c, d in zip(g, p, m, v):
+        if not (a.dtype == b_.dtype == c.dtype == d.dtype == torch.float32):
+            raise HipKernelError("adam_multi: g, p, m, v must be float32")
+        if not (a.numel() == b_.numel() == c.numel() == d.numel()):
+            raise HipKernelError("adam_multi: size mismatch")
+    lp = arr(lowp) if lowp is not None else None
+    check(lib().bb_adam_multi(n, arr(g), arr(p), arr(m), arr(v), lp, sizes, lr, beta1, beta2, eps, step,
+                              1 if adam_w_mode else 0, 1 if bias_correction else 0, weight_decay,
+                              int(zero_grad), stream_ptr(stream)), "bb_adam_multi")
+
+
+def cast(src, dst, stream=None):
+    check(lib().bb_cast(dtype_code(src.dtype), dtype_code(dst.dtype), src.numel(), _ptr(src), _ptr(dst),
+                        stream_ptr(stream)), "bb_cast")
+
+
+def fill_f32(dst, value, stream=None):
+    check(lib().bb_fill_f32(_ptr(dst), dst.numel(), value, stream_ptr(stream)), "bb_fill_f32")

@@ -1,0 +1,262 @@
+"""Layers of a pipeline stage, executed by the gfx950 kernels of ``libbamboo_hip.so``.
+
+``TransformerLayer`` computes what the reference's ``EncoderLayer`` computes
+(DeepSpeedExamples/pipeline_parallelism/transformer.py:77-172: pre-LN residual blocks around
+multi-head self-attention and a position-wise feed-forward), with explicit forward and
+backward passes instead of autograd: every tensor the backward needs is written once, by the
+kernel that produces it, into a per-micro-batch *stash* slot in HBM.  Parameter names are
+the reference module's (``self_attn.linears.0.weight`` ...), so ``"{layer_idx}.{name}"`` keys
+of the reference's parameter buffers (module.py:229-246) carry over.
+
+Memory layout.  Activations are ``[rows, features]`` row-major with ``rows = batch * seq``.
+Heads are never split out: Q, K and V of head ``j`` are the column slices
+``[j*d, (j+1)*d)`` of the three thirds of the ``[rows, 3*hidden]`` QKV buffer, and the
+batched GEMMs walk them with (batch, head) strides.  The Q/K/V projection weights are three
+adjacent ``[hidden, hidden]`` blocks of one ``[3*hidden, hidden]`` allocation, so the three
+``nn.Linear`` calls of the reference become a single GEMM.
+"""
+import math
+from collections import OrderedDict
+
+import torch
+
+from . import hip
+
+
+class StageContext:
+    """Per-execution-lane state shared by the layers of a stage: shapes, dtype, the stream the
+    kernels go to, backward scratch and reduction workspaces."""
+
+    def __init__(self, batch, seq, dtype, device, stream=None):
+        self.batch, self.seq, self.dtype, self.device = batch, seq, dtype, device
+        self.stream = stream
+        self.scratch = {}
+        self.key_len = None
+        self.workspace = None
+
+    @property
+    def rows(self):
+        return self.batch * self.seq
+
+    def ensure_scratch(self, specs):
+        for name, shape, dtype in specs:
+            cur = self.scratch.get(name)
+            n = math.prod(shape)
+            if cur is None or cur.numel() < n or cur.dtype != dtype:
+                self.scratch[name] = torch.empty(n, dtype=dtype, device=self.device)
+
+    def ensure_workspace(self, n):
+        if self.workspace is None or self.workspace.numel() < n:
+            self.workspace = torch.empty(n, dtype=torch.float32, device=self.device)
+
+    def buf(self, name, shape):
+        return self.scratch[name][: math.prod(shape)].view(shape)
+
+
+class TransformerLayer:
+    """Pre-LN transformer layer: ``x + Attn(LN(x))`` then ``x + FFN(LN(x))``.
+
+    activation: ``relu`` (reference) or ``gelu_tanh``; ln: ``annotated`` (reference: unbiased
+    std, eps added to the std) or ``standard``; mask: ``none`` (reference scripts), ``causal``
+    or ``key_padding``.  Dropout is not implemented (p = 0): redundant and normal forward must
+    agree bit for bit.
+    """
+
+    def __init__(self, hidden, heads, ffn, activation="relu", ln="annotated", mask="none", ln_eps=None,
+                 init_std=0.02):
+        if hidden % heads:
+            raise ValueError("hidden must be divisible by heads")
+        self.hidden, self.heads, self.ffn = hidden, heads, ffn
+        self.head_dim = hidden // heads
+        if activation not in hip.ACT_CODES or ln not in hip.LN_CODES or mask not in hip.MASK_CODES:
+            raise ValueError(f"unsupported variant activation={activation} ln={ln} mask={mask}")
+        self.activation, self.ln, self.mask = activation, ln, mask
+        self.eps = ln_eps if ln_eps is not None else (1e-6 if ln == "annotated" else 1e-5)
+        self.init_std = init_std
+        self.w = self.g = None
+
+    # ------------------------------------------------------------------ parameters
+    def param_specs(self):
+        h, f = self.hidden, self.ffn
+        return OrderedDict([
+            ("sublayer.0.norm.a_2", (h,)), ("sublayer.0.norm.b_2", (h,)),
+            ("self_attn.linears.0.weight", (h, h)), ("self_attn.linears.1.weight", (h, h)),
+            ("self_attn.linears.2.weight", (h, h)),
+            ("self_attn.linears.0.bias", (h,)), ("self_attn.linears.1.bias", (h,)),
+            ("self_attn.linears.2.bias", (h,)),
+            ("self_attn.linears.3.weight", (h, h)), ("self_attn.linears.3.bias", (h,)),
+            ("sublayer.1.norm.a_2", (h,)), ("sublayer.1.norm.b_2", (h,)),
+            ("feed_forward.w_1.weight", (f, h)), ("feed_forward.w_1.bias", (f,)),
+            ("feed_forward.w_2.weight", (h, f)), ("feed_forward.w_2.bias", (h,)),
+        ])
+
+    def num_params(self):
+        return sum(math.prod(s) for s in self.param_specs().values())
+
+    def init_params(self, master, seed):
+        """Fill fp32 master views: weights N(0, init_std) from per-tensor seeded CPU generators
+        (index = position in the reference module's parameter order), biases 0, LN gain 1."""
+        order = ("sublayer.0.norm.a_2", "sublayer.0.norm.b_2",
+                 "self_attn.linears.0.weight", "self_attn.linears.0.bias",
+                 "self_attn.linears.1.weight", "self_attn.linears.1.bias",
+                 "self_attn.linears.2.weight", "self_attn.linears.2.bias",
+                 "self_attn.linears.3.weight", "self_attn.linears.3.bias",
+                 "sublayer.1.norm.a_2", "sublayer.1.norm.b_2",
+                 "feed_forward.w_1.weight", "feed_forward.w_1.bias",
+                 "feed_forward.w_2.weight", "feed_forward.w_2.bias")
+        for i, name in enumerate(order):
+            t = master[name]
+            if name.endswith("a_2"):
+                t.fill_(1.0)
+            elif name.endswith("weight"):
+                g = torch.Generator().manual_seed(seed * 1000 + i)
+                t.copy_(torch.randn(t.shape, generator=g, dtype=torch.float32) * self.init_std)
+            else:
+                t.zero_()
+
+    def bind(self, compute, grads):
+        """compute / grads: name -> view (compute dtype / fp32) inside the stage's flat arenas."""
+        h = self.hidden
+        w, g = dict(compute), dict(grads)
+        # fused QKV views over the three adjacent blocks
+        for d, src in ((w, compute), (g, grads)):
+            q = src["self_attn.linears.0.weight"]
+            d["qkv.weight"] = torch.as_strided(q, (3 * h, h), (h, 1))
+            b = src["self_attn.linears.0.bias"]
+            d["qkv.bias"] = torch.as_strided(b, (3 * h,), (1,))
+        self.w, self.g = w, g
+
+    # ------------------------------------------------------------------ memory plans
+    def out_shape(self, in_shape):
+        return in_shape
+
+    def stash_specs(self, ctx):
+        R, h, f = ctx.rows, self.hidden, self.ffn
+        dt, f32 = ctx.dtype, torch.float32
+        return [
+            ("n1", (R, h), dt), ("qkv", (R, 3 * h), dt),
+            ("prob", (ctx.batch, self.heads, ctx.seq, ctx.seq), dt),
+            ("ctx", (R, h), dt), ("x1", (R, h), dt), ("n2", (R, h), dt),
+            ("u", (R, f), dt), ("act", (R, f), dt), ("out", (R, h), dt),
+            ("mean1", (R,), f32), ("rinv1", (R,), f32), ("mean2", (R,), f32), ("rinv2", (R,), f32),
+        ]
+
+    def scratch_specs(self, ctx):
+        R, h, f = ctx.rows, self.hidden, self.ffn
+        dt = ctx.dtype
+        return [("d_ffn", (R, f), dt), ("d_h0", (R, h), dt), ("d_h1", (R, h), dt), ("d_qkv", (R, 3 * h), dt),
+                ("d_prob", (ctx.batch, self.heads, ctx.seq, ctx.seq), dt)]
+
+    def workspace_elems(self):
+        n = max(self.hidden * 3, self.ffn)
+        return max(hip.layernorm_bwd_workspace(self.hidden), hip.colsum_workspace(n))
+
+    def flops_fwd(self, batch, seq):
+        h, f = self.hidden, self.ffn
+        return batch * seq * (8 * h * h + 4 * h * f) + 4 * batch * seq * seq * h
+
+    # ------------------------------------------------------------------ attention core
+    def _heads_gemm(self, ctx, layout, M, N, K, A, lda, sA, B, ldb, sB, C, ldc, sC, alpha=1.0):
+        hip.gemm_batched(layout, hip.dtype_code(ctx.dtype), M, N, K, A, lda, sA, B, ldb, sB, C, ldc, sC,
+                         ctx.batch, self.heads, alpha=alpha, stream=ctx.stream)
+
+    def _attention_fwd(self, st, ctx):
+        h, d, s = self.hidden, self.head_dim, ctx.seq
+        es = st["qkv"].element_size()
+        q = st["qkv"].data_ptr()
+        k, v = q + h * es, q + 2 * h * es
+        head_in = (s * 3 * h, d)               # (batch, head) strides inside the QKV buffer
+        prob = st["prob"]
+        # scores = Q K^T / sqrt(d)
+        self._heads_gemm(ctx, hip.NT, s, s, d, q, 3 * h, head_in, k, 3 * h, head_in,
+                         prob.data_ptr(), s, (self.heads * s * s, s * s), alpha=1.0 / math.sqrt(d))
+        hip.softmax_fwd(prob, hip.MASK_CODES[self.mask], ctx.key_len, stream=ctx.stream)
+        # ctx = P V, written straight into the [rows, hidden] layout (head j -> columns j*d..)
+        self._heads_gemm(ctx, hip.NN, s, d, s, prob.data_ptr(), s, (self.heads * s * s, s * s), v, 3 * h, head_in,
+                         st["ctx"].data_ptr(), h, (s * h, d))
+
+    def _attention_bwd(self, d_ctx, d_qkv, st, ctx):
+        h, d, s = self.hidden, self.head_dim, ctx.seq
+        es = st["qkv"].element_size()
+        q = st["qkv"].data_ptr()
+        k, v = q + h * es, q + 2 * h * es
+        dq = d_qkv.data_ptr()
+        dk, dv = dq + h * es, dq + 2 * h * es
+        head_in, head_ctx, head_p = (s * 3 * h, d), (s * h, d), (self.heads * s * s, s * s)
+        prob = st["prob"]
+        d_prob = ctx.buf("d_prob", tuple(prob.shape))
+        scale = 1.0 / math.sqrt(d)
+        # dV = P^T dctx
+        self._heads_gemm(ctx, hip.TN, s, d, s, prob.data_ptr(), s, head_p, d_ctx.data_ptr(), h, head_ctx,
+                         dv, 3 * h, head_in)
+        # dP = dctx V^T ; dS = P * (dP - rowsum(dP * P))
+        self._heads_gemm(ctx, hip.NT, s, s, d, d_ctx.data_ptr(), h, head_ctx, v, 3 * h, head_in,
+                         d_prob.data_ptr(), s, head_p)
+        hip.softmax_bwd(prob, d_prob, stream=ctx.stream)
+        # dQ = dS K / sqrt(d) ; dK = dS^T Q / sqrt(d)
+        self._heads_gemm(ctx, hip.NN, s, d, s, d_prob.data_ptr(), s, head_p, k, 3 * h, head_in,
+                         dq, 3 * h, head_in, alpha=scale)
+        self._heads_gemm(ctx, hip.TN, s, d, s, d_prob.data_ptr(), s, head_p, q, 3 * h, head_in,
+                         dk, 3 * h, head_in, alpha=scale)
+
+    # ------------------------------------------------------------------ forward / backward
+    def forward(self, x, st, ctx):
+        """x: [rows, hidden] (kept by reference in the stash); returns st['out']."""
+        w, sm = self.w, ctx.stream
+        kind, act = hip.LN_CODES[self.ln], hip.ACT_CODES[self.activation]
+        st["x0"] = x
+        hip.layernorm_fwd(x, w["sublayer.0.norm.a_2"], w["sublayer.0.norm.b_2"], st["n1"], st["mean1"],
+                          st["rinv1"], kind, self.eps, stream=sm)
+        hip.gemm(hip.NT, st["n1"], w["qkv.weight"], st["qkv"], bias=w["qkv.bias"], stream=sm)
+        self._attention_fwd(st, ctx)
+        hip.gemm(hip.NT, st["ctx"], w["self_attn.linears.3.weight"], st["x1"], bias=w["self_attn.linears.3.bias"],
+                 epilogue=hip.EPI_RESIDUAL, resid=x, stream=sm)
+        hip.layernorm_fwd(st["x1"], w["sublayer.1.norm.a_2"], w["sublayer.1.norm.b_2"], st["n2"], st["mean2"],
+                          st["rinv2"], kind, self.eps, stream=sm)
+        hip.gemm(hip.NT, st["n2"], w["feed_forward.w_1.weight"], st["act"], bias=w["feed_forward.w_1.bias"],
+                 epilogue=hip.EPI_ACT, act=act, aux_out=st["u"], stream=sm)
+        hip.gemm(hip.NT, st["act"], w["feed_forward.w_2.weight"], st["out"], bias=w["feed_forward.w_2.bias"],
+                 epilogue=hip.EPI_RESIDUAL, resid=st["x1"], stream=sm)
+        return st["out"]
+
+    def backward(self, d_out, d_x, st, ctx):
+        """d_out: gradient of st['out']; writes the input gradient into d_x; parameter
+        gradients are accumulated (fp32)."""
+        w, g, sm, ws = self.w, self.g, ctx.stream, ctx.workspace
+        R, h, f = ctx.rows, self.hidden, self.ffn
+        kind, act = hip.LN_CODES[self.ln], hip.ACT_CODES[self.activation]
+        d_ffn, d_h0, d_h1 = ctx.buf("d_ffn", (R, f)), ctx.buf("d_h0", (R, h)), ctx.buf("d_h1", (R, h))
+        d_qkv = ctx.buf("d_qkv", (R, 3 * h))
+        # feed-forward
+        hip.gemm(hip.TN, d_out, st["act"], g["feed_forward.w_2.weight"], accumulate=True, stream=sm)
+        hip.colsum_acc(d_out, g["feed_forward.w_2.bias"], ws, stream=sm)
+        hip.gemm(hip.NN, d_out, w["feed_forward.w_2.weight"], d_ffn, epilogue=hip.EPI_DACT, act=act,
+                 aux_in=st["u"], stream=sm)
+        hip.gemm(hip.TN, d_ffn, st["n2"], g["feed_forward.w_1.weight"], accumulate=True, stream=sm)
+        hip.colsum_acc(d_ffn, g["feed_forward.w_1.bias"], ws, stream=sm)
+        hip.gemm(hip.NN, d_ffn, w["feed_forward.w_1.weight"], d_h0, stream=sm)
+        # d_x1 = d_out + LN2'(d_n2)
+        hip.layernorm_bwd(st["x1"], w["sublayer.1.norm.a_2"], st["mean2"], st["rinv2"], d_h0, d_out, d_h1,
+                          g["sublayer.1.norm.a_2"], g["sublayer.1.norm.b_2"], ws, kind, self.eps, stream=sm)
+        # attention output projection
+        hip.gemm(hip.TN, d_h1, st["ctx"], g["self_attn.linears.3.weight"], accumulate=True, stream=sm)
+        hip.colsum_acc(d_h1, g["self_attn.linears.3.bias"], ws, stream=sm)
+        hip.gemm(hip.NN, d_h1, w["self_attn.linears.3.weight"], d_h0, stream=sm)
+        self._attention_bwd(d_h0, d_qkv, st, ctx)
+        # QKV projection
+        hip.gemm(hip.TN, d_qkv, st["n1"], g["qkv.weight"], accumulate=True, stream=sm)
+        hip.colsum_acc(d_qkv, g["qkv.bias"], ws, stream=sm)
+        hip.gemm(hip.NN, d_qkv, w["qkv.weight"], d_h0, stream=sm)
+        # d_x0 = d_x1 + LN1'(d_n1)
+        hip.layernorm_bwd(st["x0"], w["sublayer.0.norm.a_2"], st["mean1"], st["rinv1"], d_h0, d_h1, d_x,
+                          g["sublayer.0.norm.a_2"], g["sublayer.0.norm.b_2"], ws, kind, self.eps, stream=sm)
+        return d_x
+
+
+class MSELoss:
+    """``nn.MSELoss()`` of the reference scripts (transformer.py:264) as a fused HIP kernel that
+    also yields the output gradient.  Used as ``loss_fn`` of a last stage, and by the in-process
+    peer that stands in for the downstream stages."""
+
+    def __call__(self, y, target, d_y, grad_scale, loss_out, accumulate, workspace, stream=None):
+        hip.mse_fwd_bwd(y, target, d_y, grad_scale, loss_out, accumulate, workspace, stream=stream)

@@ -1,0 +1,322 @@
+"""``PipelineModule`` / ``LayerSpec``: the layer list of a pipelined model and the layers this
+process has materialised (its own stage and the stages it shadows).
+
+Interface of ``deepspeed/runtime/pipe/module.py`` of the reference: constructor :95-106,
+``build_layers(stage_id, buffer)`` :262-332, ``allocate_param`` :229-260,
+``get_named_param`` :219-227, ``forward(x, stage_id)`` :516-574, ``_partition_layers``
+:576-635.  Differences that follow from running on hand-written kernels instead of autograd:
+layers are native layer objects (``bamboo_amd.layers``) with explicit forward/backward; the
+parameters of a stage live in flat HBM arenas (fp32 master, fp32 gradient, compute-dtype copy)
+and ``forward`` takes the stash slot that receives the activations of this micro-batch.
+"""
+import math
+import os
+import re
+from collections import OrderedDict
+
+import torch
+
+from . import hip
+from .layers import StageContext
+from .utils import partition_balanced, partition_uniform
+
+
+class PipelineError(Exception):
+    """Errors related to the use of pipeline parallelism."""
+
+
+class LayerSpec:
+    """Delayed construction of a layer: ``LayerSpec(TransformerLayer, hidden=..., ...)``
+    (reference module.py:25-69)."""
+
+    def __init__(self, typename, *module_args, **module_kwargs):
+        if not isinstance(typename, type):
+            raise RuntimeError("LayerSpec expects a class")
+        self.typename = typename
+        self.module_args = module_args
+        self.module_kwargs = module_kwargs
+
+    def __repr__(self):
+        from .schedule import call_to_str
+        return call_to_str(self.typename.__name__, *self.module_args, **self.module_kwargs)
+
+    def build(self, log=False):
+        return self.typename(*self.module_args, **self.module_kwargs)
+
+
+class TiedLayerSpec(LayerSpec):
+    """Accepted for interface compatibility; tied layers are outside the accelerated path
+    (the reference itself disables ReduceTiedGrads, schedule.py:283-285)."""
+
+    def __init__(self, key, typename, *module_args, forward_fn=None, tied_weight_attr="weight", **module_kwargs):
+        super().__init__(typename, *module_args, **module_kwargs)
+        self.key, self.forward_fn, self.tied_weight_attr = key, forward_fn, tied_weight_attr
+
+
+class StageParams:
+    """Flat parameter arenas of one stage and the per-layer named views into them."""
+
+    def __init__(self, layers, first_layer_idx, dtype, device):
+        self.layers, self.dtype, self.device = layers, dtype, device
+        self.index = OrderedDict()   # "{layer_idx}.{name}" -> (offset, shape)
+        off = 0
+        for li, layer in enumerate(layers):
+            for name, shape in layer.param_specs().items():
+                n = math.prod(shape)
+                if n % 8:
+                    raise PipelineError(f"parameter {name} of size {n} breaks the 16-byte arena alignment")
+                self.index[f"{first_layer_idx + li}.{name}"] = (off, tuple(shape))
+                off += n
+        self.numel = off
+        f32 = torch.float32
+        self.master = torch.zeros(off, dtype=f32, device=device)
+        self.grad = torch.zeros(off, dtype=f32, device=device)
+        self.exp_avg = torch.zeros(off, dtype=f32, device=device)
+        self.exp_avg_sq = torch.zeros(off, dtype=f32, device=device)
+        self.compute = self.master if dtype == f32 else torch.zeros(off, dtype=dtype, device=device)
+        self.first_layer_idx = first_layer_idx
+        for li, layer in enumerate(layers):
+            prefix = f"{first_layer_idx + li}."
+            names = [k[len(prefix):] for k in self.index if k.startswith(prefix)]
+            layer.bind({n: self.view(self.compute, prefix + n) for n in names},
+                       {n: self.view(self.grad, prefix + n) for n in names})
+
+    def view(self, arena, key):
+        off, shape = self.index[key]
+        return arena[off: off + math.prod(shape)].view(shape)
+
+    def named(self, arena):
+        return OrderedDict((k, self.view(arena, k)) for k in self.index)
+
+    def init(self, base_seed):
+        host = torch.zeros(self.numel, dtype=torch.float32)
+        for li, layer in enumerate(self.layers):
+            prefix = f"{self.first_layer_idx + li}."
+            views = {k[len(prefix):]: host[o: o + math.prod(s)].view(s)
+                     for k, (o, s) in self.index.items() if k.startswith(prefix)}
+            layer.init_params(views, base_seed + self.first_layer_idx + li)
+        self.master.copy_(host)
+        self.refresh_compute()
+
+    def refresh_compute(self):
+        if self.compute is not self.master:
+            hip.cast(self.master, self.compute)
+
+    def load(self, named_tensors):
+        """Copy ``{"{layer_idx}.{name}": tensor}`` into the master arena (missing keys are left)."""
+        for k, t in named_tensors.items():
+            if k in self.index:
+                self.view(self.master, k).copy_(t.to(torch.float32))
+        self.refresh_compute()
+
+
+class PipelineModule:
+    """Sequence of layers partitioned over ``num_stages`` pipeline stages.
+
+    ``stage_id`` (keyword, or the ``pipe`` coordinate of ``PROJECT_PACTUM_COORDINATES`` /
+    ``BAMBOO_STAGE_ID`` in the environment) says which stage this process executes; the
+    reference obtains it from its rendezvous (module.py:150-170)."""
+
+    def __init__(self, layers, num_stages=None, topology=None, loss_fn=None, seed_layers=False, seed_fn=None,
+                 base_seed=1234, partition_method="parameters", custom_partitions=[],
+                 activation_checkpoint_interval=0, activation_checkpoint_func=None, stage_id=None,
+                 dtype=torch.float32, device=None):
+        if num_stages is None and topology is None:
+            raise RuntimeError("must provide num_stages or topology")
+        if activation_checkpoint_interval != 0:
+            raise NotImplementedError("activation checkpointing is not part of the accelerated stage path")
+        self.num_stages = num_stages if num_stages is not None else topology.get_dim("pipe")
+        if stage_id is None:
+            stage_id = self._stage_from_env()
+        if not 0 <= stage_id < self.num_stages:
+            raise PipelineError(f"stage_id {stage_id} outside [0, {self.num_stages})")
+        self.stage_id = stage_id
+        self.loss_fn = loss_fn
+        self.seed_layers, self.seed_fn, self.base_seed = seed_layers, seed_fn, base_seed
+        self.micro_offset = 0
+        self._layer_specs = list(layers)
+        self._num_layers = len(self._layer_specs)
+        self.partition_method = partition_method
+        self.dtype = dtype
+        self.device = torch.device(device if device is not None else "cuda:0")
+        self.func_buckets = {}        # stage_id -> [layer objects]
+        self.param_name_buckets = {}  # stage_id -> ["{layer_idx}.{name}"]
+        self.stage_params = {}        # stage_id -> StageParams
+        self._stash = {}              # stage_id -> [slot][layer] -> dict of views
+        self._partition_layers(method=partition_method, partitions=custom_partitions)
+        self.build_layers(self.stage_id)
+
+    @staticmethod
+    def _stage_from_env():
+        if "BAMBOO_STAGE_ID" in os.environ:
+            return int(os.environ["BAMBOO_STAGE_ID"])
+        coords = os.environ.get("PROJECT_PACTUM_COORDINATES")
+        if coords:
+            import json
+            c = json.loads(coords)
+            first = c[0] if isinstance(c, list) and c and isinstance(c[0], (list, tuple)) else c
+            return int(first[1])  # (dp_id, stage_id)
+        return 0
+
+    # ------------------------------------------------------------------ partitioning
+    def _count_layer_params(self):
+        counts = []
+        for spec in self._layer_specs:
+            layer = spec.build() if isinstance(spec, LayerSpec) else spec
+            counts.append(layer.num_params() if hasattr(layer, "num_params") else 0)
+        return counts
+
+    def _find_layer_type(self, layername):
+        rx = re.compile(layername, re.IGNORECASE)
+        out = []
+        for i, spec in enumerate(self._layer_specs):
+            name = spec.typename.__name__ if isinstance(spec, LayerSpec) else type(spec).__name__
+            if rx.search(name):
+                out.append(i)
+        return out
+
+    def _partition_layers(self, method="uniform", partitions=[]):
+        method = method.lower()
+        if method == "custom":
+            assert partitions, "Required customized partitions"
+            self.parts = list(partitions)
+        elif method == "uniform":
+            self.parts = partition_uniform(self._num_layers, self.num_stages)
+        elif method == "parameters":
+            self.parts = partition_balanced(self._count_layer_params(), self.num_stages)
+        elif method.startswith("type:"):
+            weights = [0] * self._num_layers
+            for i in self._find_layer_type(method.split(":")[1]):
+                weights[i] = 1
+            self.parts = partition_balanced(weights, self.num_stages)
+        else:
+            raise NotImplementedError(f"Partitioning method {method} not implemented.")
+        if len(self.parts) != self.num_stages + 1 or self.parts[-1] != self._num_layers:
+            raise PipelineError(f"partition {self.parts} does not cover {self._num_layers} layers in {self.num_stages} stages")
+        self._local_start, self._local_stop = self.parts[self.stage_id], self.parts[self.stage_id + 1]
+
+    # ------------------------------------------------------------------ building
+    def _instantiate(self, stage_id):
+        built = []
+        for spec in self._layer_specs[self.parts[stage_id]: self.parts[stage_id + 1]]:
+            if isinstance(spec, TiedLayerSpec):
+                raise NotImplementedError("tied layers are not supported on the accelerated stage path")
+            layer = spec.build() if isinstance(spec, LayerSpec) else spec
+            if not (hasattr(layer, "forward") and hasattr(layer, "backward") and hasattr(layer, "param_specs")):
+                raise PipelineError(
+                    f"layer {layer!r} is not a native bamboo_amd layer: this engine runs hand-written HIP kernels "
+                    "only and has no autograd fallback")
+            built.append(layer)
+        return built
+
+    def build_layers(self, stage_id, buffer=None):
+        """Materialise the layers of ``stage_id`` on the GPU (own stage, or a stage this process
+        shadows).  ``buffer``: optional ``{"{layer_idx}.{name}": tensor}`` to copy weights from."""
+        if stage_id in self.func_buckets:
+            if buffer is not None:
+                self.stage_params[stage_id].load(buffer)
+            return self.param_name_buckets[stage_id]
+        layers = self._instantiate(stage_id)
+        sp = StageParams(layers, self.parts[stage_id], self.dtype, self.device)
+        sp.init(self.base_seed)
+        if buffer is not None:
+            sp.load(buffer)
+        self.func_buckets[stage_id] = layers
+        self.stage_params[stage_id] = sp
+        self.param_name_buckets[stage_id] = list(sp.index.keys())
+        return self.param_name_buckets[stage_id]
+
+    def allocate_param(self, stage_id, param_buffer, device="cpu"):
+        """Zero mirrors of the parameters of ``stage_id`` (reference module.py:229-260)."""
+        layers = self.func_buckets.get(stage_id) or self._instantiate(stage_id)
+        names = []
+        for li, layer in enumerate(layers):
+            for name, shape in layer.param_specs().items():
+                key = f"{self.parts[stage_id] + li}.{name}"
+                param_buffer[key] = torch.zeros(shape, dtype=torch.float32, device=device)
+                names.append(key)
+        self.param_name_buckets.setdefault(stage_id, names)
+        return names
+
+    def get_named_param(self, stage_id):
+        """(name, fp32 master view) pairs of a built stage."""
+        sp = self.stage_params[stage_id]
+        yield from sp.named(sp.master).items()
+
+    def get_named_grad(self, stage_id):
+        sp = self.stage_params[stage_id]
+        yield from sp.named(sp.grad).items()
+
+    def parameters(self):
+        for sid in sorted(self.stage_params):
+            for _, p in self.get_named_param(sid):
+                yield p
+
+    def num_layers(self, stage_id):
+        return self.parts[stage_id + 1] - self.parts[stage_id]
+
+    # ------------------------------------------------------------------ stash
+    def allocate_stash(self, stage_id, ctx, slots):
+        """One arena holding, for every (slot, layer), the activations its backward needs."""
+        layers = self.func_buckets[stage_id]
+        plans, total = [], 0
+        for layer in layers:
+            plan = []
+            for name, shape, dtype in layer.stash_specs(ctx):
+                nbytes = math.prod(shape) * torch.empty((), dtype=dtype).element_size()
+                plan.append((name, shape, dtype, total, nbytes))
+                total += (nbytes + 255) // 256 * 256
+            plans.append(plan)
+        arena = torch.empty(total * slots, dtype=torch.uint8, device=self.device)
+        table = []
+        for s in range(slots):
+            per_layer = []
+            for plan in plans:
+                views = {}
+                for name, shape, dtype, off, nbytes in plan:
+                    lo = s * total + off
+                    views[name] = arena[lo: lo + nbytes].view(dtype).view(shape)
+                per_layer.append(views)
+            table.append(per_layer)
+        self._stash[stage_id] = table
+        self._stash_arena = getattr(self, "_stash_arena", {})
+        self._stash_arena[stage_id] = arena
+        return total * slots
+
+    # ------------------------------------------------------------------ execution
+    def forward(self, forward_input, stage_id, slot=0, ctx=None):
+        layers = self.func_buckets.get(stage_id)
+        if layers is None:
+            raise Exception(f"Unregistered stage id {stage_id}")
+        self.micro_offset += 1
+        x = forward_input
+        for layer, st in zip(layers, self._stash[stage_id][slot]):
+            x = layer.forward(x, st, ctx)
+        return x
+
+    def backward(self, grad_output, grad_input, stage_id, slot=0, ctx=None):
+        """Back-propagate through the layers of ``stage_id`` from the stash of ``slot``; parameter
+        gradients accumulate in the stage's fp32 gradient arena, the input gradient is written to
+        ``grad_input``."""
+        layers = self.func_buckets[stage_id]
+        stash = self._stash[stage_id][slot]
+        n = len(layers)
+        d = grad_output
+        for i in range(n - 1, -1, -1):
+            dst = grad_input if i == 0 else ctx.buf(f"d_layer{i % 2}", tuple(grad_output.shape))
+            layers[i].backward(d, dst, stash[i], ctx)
+            d = dst
+        return grad_input
+
+    def prepare_context(self, stage_ids, batch, seq, stream=None):
+        """Execution context with scratch sized for the largest layer of the given stages."""
+        ctx = StageContext(batch, seq, self.dtype, self.device, stream)
+        ws = 0
+        for sid in stage_ids:
+            for layer in self.func_buckets[sid]:
+                ctx.ensure_scratch(layer.scratch_specs(ctx))
+                ws = max(ws, layer.workspace_elems())
+                h = layer.out_shape((ctx.rows, layer.hidden))
+                ctx.ensure_scratch([("d_layer0", h, self.dtype), ("d_layer1", h, self.dtype)])
+        ctx.ensure_workspace(ws)
+        return ctx

@@ -1,0 +1,171 @@
+/* bamboo_hip.h -- C ABI of libbamboo_hip.so, the gfx950 (MI355X) kernel library under
+ * one Bamboo pipeline stage.
+ *
+ * Conventions (every entry point):
+ *   - returns 0 on success, a negative BB_E* code otherwise; never throws, never exits.
+ *     bb_last_error() gives a thread-local human-readable message for the last failure.
+ *   - all data pointers are DEVICE pointers owned by the caller (any allocator), 16-byte
+ *     aligned, row-major; leading dimensions and strides are in ELEMENTS.
+ *   - `stream` is a hipStream_t passed as void*; work is stream-ordered, no hidden
+ *     synchronisation, no allocation (workspaces are caller-provided).
+ *   - results are deterministic: no atomics in reductions, no split-K, so running the same
+ *     call twice on the same inputs gives bit-identical outputs (this is what makes the
+ *     redundant forward of shadow layers bit-exact with the normal forward).
+ *   - dtype codes: BB_F32 = 0, BB_BF16 = 1.
+ *
+ * The reference has exactly one native entry point on this path, the torch extension
+ *   multi_tensor_adam(chunk_size, noop_flag, [[g],[p],[m],[v]], lr, b1, b2, eps, step, mode,
+ *                     bias_correction, wd)   (csrc/adam/fused_adam_frontend.cpp:3-20);
+ * bb_adam_multi replaces it.  All other layer arithmetic of the reference runs through
+ * ATen operators called from Python (DeepSpeedExamples/pipeline_parallelism/transformer.py:77-172,
+ * resnet.py:49-75); each entry point below names the call site it stands in for.
+ */
+#ifndef BAMBOO_HIP_H
+#define BAMBOO_HIP_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define BB_F32 0
+#define BB_BF16 1
+
+#define BB_OK 0
+#define BB_EINVAL (-1)  /* bad argument / unsupported shape */
+#define BB_EHIP (-2)    /* a HIP runtime call failed */
+#define BB_ENOSPC (-3)  /* caller workspace too small */
+
+/* GEMM operand layouts (row-major storage):
+ *   BB_NT  C[M,N] = A[M,K] * B[N,K]^T   y = x W^T        (nn.Linear forward, Q K^T, dctx V^T)
+ *   BB_NN  C[M,N] = A[M,K] * B[K,N]     dx = dy W        (linear dgrad, P V, dS K)
+ *   BB_TN  C[M,N] = A[K,M]^T * B[K,N]   dW = dy^T x      (linear wgrad, P^T dctx, dS^T Q)   */
+#define BB_NT 0
+#define BB_NN 1
+#define BB_TN 2
+
+/* GEMM epilogues, applied to v = alpha * acc (+ bias[n] if bias != NULL):
+ *   BB_EPI_NONE      C = v
+ *   BB_EPI_ACT       aux_out = v (if aux_out != NULL);  C = act(v)
+ *   BB_EPI_DACT      C = v * act'(aux_in[m,n])
+ *   BB_EPI_RESIDUAL  C = v + resid[m,n]
+ * `accumulate` != 0 adds the result to the existing contents of C (C must be fp32).       */
+#define BB_EPI_NONE 0
+#define BB_EPI_ACT 1
+#define BB_EPI_DACT 2
+#define BB_EPI_RESIDUAL 3
+
+#define BB_ACT_RELU 0
+#define BB_ACT_GELU_TANH 1
+
+/* attention / softmax mask kinds (reference hook: scores.masked_fill(mask == 0, -1e9),
+ * transformer.py:122-123) */
+#define BB_MASK_NONE 0
+#define BB_MASK_CAUSAL 1      /* keep col <= row */
+#define BB_MASK_KEY_PADDING 2 /* keep col < key_len[batch] */
+
+/* LayerNorm flavours */
+#define BB_LN_STANDARD 0  /* (x-mean) * rsqrt(var_biased + eps) */
+#define BB_LN_ANNOTATED 1 /* (x-mean) / (std_unbiased + eps), transformer.py:77-88 */
+
+typedef struct bb_gemm_desc {
+    int32_t layout;     /* BB_NT / BB_NN / BB_TN */
+    int32_t dtype;      /* dtype of A, B, bias, aux, resid (BB_F32 / BB_BF16) */
+    int32_t c_dtype;    /* dtype of C (same as dtype, or BB_F32) */
+    int32_t M, N, K;
+    const void* A; int64_t lda;
+    const void* B; int64_t ldb;
+    void* C; int64_t ldc;
+    /* batching: grid z = nb1 * nb2, operand offset = i1 * s?1 + i2 * s?2 (elements) */
+    int32_t nb1, nb2;
+    int64_t sA1, sA2, sB1, sB2, sC1, sC2;
+    float alpha;
+    int32_t epilogue;   /* BB_EPI_* */
+    int32_t act;        /* BB_ACT_* */
+    int32_t accumulate; /* C += ... (c_dtype must be BB_F32) */
+    const void* bias;   /* [N] or NULL */
+    const void* aux_in; /* [M,N], leading dim ldaux, batch strides as C */
+    void* aux_out;      /* [M,N], leading dim ldaux */
+    const void* resid;  /* [M,N], leading dim ldaux */
+    int64_t ldaux;
+} bb_gemm_desc;
+
+/* library ------------------------------------------------------------------------------ */
+int bb_version(void);
+const char* bb_last_error(void);
+/* Device name check: fails with BB_EHIP when the current device is not a gfx950 part.    */
+int bb_init(void);
+
+/* GEMM (MFMA, LDS-tiled).  Stands in for every F.linear / torch.matmul call of the reference
+ * layer (transformer.py:121,127,136-146,158) and for their autograd backward
+ * (engine.py:1701-1709 torch.autograd.backward).  bf16 needs K, lda, ldb, ldc % 8 == 0;
+ * fp32 needs them % 4 == 0.                                                               */
+int bb_gemm(const bb_gemm_desc* desc, void* stream);
+/* Name of the kernel variant bb_gemm would launch for this descriptor ("bf16_nt_256x256", ...),
+ * written NUL-terminated into out; for correlating launches with profiler output.        */
+int bb_gemm_variant(const bb_gemm_desc* desc, char* out, int out_len);
+
+/* LayerNorm over the last dimension (transformer.py:77-88 custom LayerNorm, or the standard
+ * one).  x, y: [rows, cols] of `dtype`; gain, shift: [cols] of `dtype`; mean, rinv: [rows]
+ * fp32 saved for backward (rinv = 1/(std+eps) or rsqrt(var+eps)).  cols <= 8192.          */
+int bb_layernorm_fwd(int dtype, int kind, int rows, int cols, float eps, const void* x,
+                     const void* gain, const void* shift, void* y, float* mean, float* rinv,
+                     void* stream);
+/* Backward: dx = dLN(dy) (+ dres if dres != NULL, the residual branch's gradient);
+ * dgain/dshift (fp32, [cols]) are ACCUMULATED.  workspace: fp32, at least
+ * bb_layernorm_bwd_workspace(cols) elements.                                              */
+int64_t bb_layernorm_bwd_workspace(int cols);
+int bb_layernorm_bwd(int dtype, int kind, int rows, int cols, float eps, const void* x,
+                     const void* gain, const float* mean, const float* rinv, const void* dy,
+                     const void* dres, void* dx, float* dgain, float* dshift,
+                     float* workspace, void* stream);
+
+/* Column sums of a [rows, cols] matrix accumulated into an fp32 vector: the bias gradient of
+ * nn.Linear (autograd of transformer.py:136-146,158).  workspace: fp32, at least
+ * bb_colsum_workspace(cols) elements.                                                     */
+int64_t bb_colsum_workspace(int cols);
+int bb_colsum_acc(int dtype, int rows, int cols, const void* x, int64_t ldx, float* out,
+                  float* workspace, void* stream);
+
+/* Masked softmax over the last dimension, in place (transformer.py:121-124).
+ * s: [batch, heads, sq, sk] contiguous of `dtype`; key_len: int32 [batch] for
+ * BB_MASK_KEY_PADDING.  Masked scores are replaced by -1e9 before the softmax.            */
+int bb_softmax_fwd(int dtype, int mask, int batch, int heads, int sq, int sk, void* s,
+                   const int32_t* key_len, void* stream);
+/* In place on dp: dp <- p * (dp - sum_j dp*p).                                            */
+int bb_softmax_bwd(int dtype, int batch, int heads, int sq, int sk, const void* p, void* dp,
+                   void* stream);
+
+/* out = a + b, elementwise (SublayerConnection residual, transformer.py:103).             */
+int bb_residual_add(int dtype, int64_t n, const void* a, const void* b, void* out,
+                    void* stream);
+
+/* Mean-squared-error head (nn.MSELoss, transformer.py:264) fused with its gradient:
+ * loss_out[0] (+)= mean((y-t)^2);  dy = grad_scale * 2 (y-t) / n.  Deterministic two-pass
+ * reduction; workspace: fp32, at least bb_mse_workspace() elements.                       */
+int64_t bb_mse_workspace(void);
+int bb_mse_fwd_bwd(int dtype, int64_t n, const void* y, const void* target, void* dy,
+                   float grad_scale, float* loss_out, int accumulate_loss, float* workspace,
+                   void* stream);
+
+/* Fused multi-tensor Adam / AdamW; replaces multi_tensor_adam
+ * (csrc/adam/fused_adam_frontend.cpp:3-20, kernel csrc/adam/multi_tensor_adam.cu:28-121).
+ * All of g, p, m, v are fp32; `lowp` (may be NULL, entries may be NULL) receives a bf16 copy
+ * of the updated parameter (the compute weights of the bf16 configurations).
+ * The pointer tables are HOST arrays of n_tensors device pointers; `sizes` are element counts.
+ * mode: 0 = L2 (g += wd*p), 1 = decoupled weight decay (AdamW).  step >= 1.
+ * zero_grad != 0 also clears g after use (the engine's zero_grad, fused).                 */
+int bb_adam_multi(int n_tensors, void* const* g, void* const* p, void* const* m,
+                  void* const* v, void* const* lowp, const int64_t* sizes, float lr,
+                  float beta1, float beta2, float eps, int step, int mode,
+                  int bias_correction, float weight_decay, int zero_grad, void* stream);
+
+/* dtype conversion / fill helpers used when (re)materialising compute weights.            */
+int bb_cast(int src_dtype, int dst_dtype, int64_t n, const void* src, void* dst, void* stream);
+int bb_fill_f32(float* dst, int64_t n, float value, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* BAMBOO_HIP_H */

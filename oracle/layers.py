@@ -1,0 +1,182 @@
+"""Layer mathematics of the reference models on torch CPU ops (TEST ORACLE).
+
+Follows DeepSpeedExamples/pipeline_parallelism/transformer.py of the reference:
+  layer_norm          transformer.py:77-88   (LayerNorm: unbiased std, eps outside sqrt)
+  attention           transformer.py:106-146 (MultiHeadedAttention, masked_fill(mask==0,-1e9))
+  feed_forward        transformer.py:149-158 (PositionwiseFeedForward)
+  transformer_layer   transformer.py:91-103,161-172 (SublayerConnection + EncoderLayer, pre-LN)
+  bottleneck          resnet.py:49-75        (BottleNeck, bias-free convs, train-mode BN)
+Dropout is fixed to 0 (the reference's own parity test disables it,
+tests/unit/test_pipe.py:144-145).  Switches beyond the reference's setting
+(`relu`, `annotated`, no mask) exist because the benchmark configurations ask
+for causal / key-padding masks, tanh-GELU and the standard LayerNorm.
+"""
+import math
+from dataclasses import dataclass
+
+import torch
+import torch.nn.functional as F
+
+PARAM_ORDER = (
+    "sublayer.0.norm.a_2", "sublayer.0.norm.b_2",
+    "self_attn.linears.0.weight", "self_attn.linears.0.bias",
+    "self_attn.linears.1.weight", "self_attn.linears.1.bias",
+    "self_attn.linears.2.weight", "self_attn.linears.2.bias",
+    "self_attn.linears.3.weight", "self_attn.linears.3.bias",
+    "sublayer.1.norm.a_2", "sublayer.1.norm.b_2",
+    "feed_forward.w_1.weight", "feed_forward.w_1.bias",
+    "feed_forward.w_2.weight", "feed_forward.w_2.bias",
+)
+
+
+@dataclass(frozen=True)
+class TransformerCfg:
+    hidden: int
+    heads: int
+    ffn: int
+    activation: str = "relu"      # relu | gelu_tanh
+    ln: str = "annotated"         # annotated (reference) | standard
+    mask: str = "none"            # none | causal | key_padding
+    ln_eps: float = None
+
+    @property
+    def eps(self):
+        if self.ln_eps is not None:
+            return self.ln_eps
+        return 1e-6 if self.ln == "annotated" else 1e-5
+
+
+def param_shapes(cfg):
+    h, f = cfg.hidden, cfg.ffn
+    return {
+        "sublayer.0.norm.a_2": (h,), "sublayer.0.norm.b_2": (h,),
+        "self_attn.linears.0.weight": (h, h), "self_attn.linears.0.bias": (h,),
+        "self_attn.linears.1.weight": (h, h), "self_attn.linears.1.bias": (h,),
+        "self_attn.linears.2.weight": (h, h), "self_attn.linears.2.bias": (h,),
+        "self_attn.linears.3.weight": (h, h), "self_attn.linears.3.bias": (h,),
+        "sublayer.1.norm.a_2": (h,), "sublayer.1.norm.b_2": (h,),
+        "feed_forward.w_1.weight": (f, h), "feed_forward.w_1.bias": (f,),
+        "feed_forward.w_2.weight": (h, f), "feed_forward.w_2.bias": (h,),
+    }
+
+
+def init_params(cfg, seed, dtype=torch.float32, std=0.02):
+    """Weights N(0, std) from a per-tensor seeded generator, biases 0, LN gain 1."""
+    out = {}
+    for i, (name, shape) in enumerate(param_shapes(cfg).items()):
+        if name.endswith("a_2"):
+            t = torch.ones(shape, dtype=dtype)
+        elif name.endswith("weight"):
+            g = torch.Generator().manual_seed(seed * 1000 + i)
+            t = (torch.randn(shape, generator=g, dtype=torch.float32) * std).to(dtype)
+        else:
+            t = torch.zeros(shape, dtype=dtype)
+        out[name] = t
+    return out
+
+
+def layer_norm(x, gain, shift, kind, eps):
+    if kind == "annotated":
+        mean = x.mean(-1, keepdim=True)
+        std = x.std(-1, keepdim=True)            # unbiased (n-1)
+        return gain * (x - mean) / (std + eps) + shift
+    return F.layer_norm(x, x.shape[-1:], gain, shift, eps)
+
+
+def activation(x, kind):
+    if kind == "relu":
+        return F.relu(x)
+    if kind == "gelu_tanh":
+        return F.gelu(x, approximate="tanh")
+    raise ValueError(kind)
+
+
+def build_mask(cfg, batch, seq, key_lens=None):
+    """Boolean [b,1,s,s] / [b,1,1,s] mask, True = keep (reference: mask == 0 is filled)."""
+    if cfg.mask == "none":
+        return None
+    if cfg.mask == "causal":
+        return torch.tril(torch.ones(seq, seq, dtype=torch.bool)).view(1, 1, seq, seq)
+    if cfg.mask == "key_padding":
+        ar = torch.arange(seq).view(1, 1, 1, seq)
+        return ar < key_lens.view(batch, 1, 1, 1)
+    raise ValueError(cfg.mask)
+
+
+def attention(x, p, cfg, key_lens=None):
+    b, s, h = x.shape
+    a, d = cfg.heads, cfg.hidden // cfg.heads
+    lin = lambda i, t: F.linear(t, p[f"self_attn.linears.{i}.weight"], p[f"self_attn.linears.{i}.bias"])
+    q, k, v = [lin(i, x).view(b, s, a, d).transpose(1, 2) for i in range(3)]
+    scores = torch.matmul(q, k.transpose(-2, -1)) / math.sqrt(d)
+    mask = build_mask(cfg, b, s, key_lens)
+    if mask is not None:
+        scores = scores.masked_fill(~mask, -1e9)
+    prob = F.softmax(scores, dim=-1)
+    ctx = torch.matmul(prob, v).transpose(1, 2).contiguous().view(b, s, h)
+    return lin(3, ctx)
+
+
+def feed_forward(x, p, cfg):
+    u = F.linear(x, p["feed_forward.w_1.weight"], p["feed_forward.w_1.bias"])
+    return F.linear(activation(u, cfg.activation), p["feed_forward.w_2.weight"], p["feed_forward.w_2.bias"])
+
+
+def transformer_layer(x, p, cfg, key_lens=None):
+    n1 = layer_norm(x, p["sublayer.0.norm.a_2"], p["sublayer.0.norm.b_2"], cfg.ln, cfg.eps)
+    x = x + attention(n1, p, cfg, key_lens)
+    n2 = layer_norm(x, p["sublayer.1.norm.a_2"], p["sublayer.1.norm.b_2"], cfg.ln, cfg.eps)
+    return x + feed_forward(n2, p, cfg)
+
+
+# ---------------------------------------------------------------- ResNet bottleneck
+
+@dataclass(frozen=True)
+class BottleneckCfg:
+    in_channels: int = 1024
+    mid_channels: int = 256
+    stride: int = 1
+    bn_eps: float = 1e-5
+
+    @property
+    def out_channels(self):
+        return 4 * self.mid_channels
+
+
+def bottleneck_param_shapes(cfg):
+    ci, cm, co = cfg.in_channels, cfg.mid_channels, cfg.out_channels
+    return {
+        "residual_function.0.weight": (cm, ci, 1, 1),
+        "residual_function.1.weight": (cm,), "residual_function.1.bias": (cm,),
+        "residual_function.3.weight": (cm, cm, 3, 3),
+        "residual_function.4.weight": (cm,), "residual_function.4.bias": (cm,),
+        "residual_function.6.weight": (co, cm, 1, 1),
+        "residual_function.7.weight": (co,), "residual_function.7.bias": (co,),
+    }
+
+
+def init_bottleneck_params(cfg, seed, dtype=torch.float32):
+    """He-normal conv weights (std = sqrt(2/fan_in)), BN gamma 1 / beta 0."""
+    out = {}
+    for i, (name, shape) in enumerate(bottleneck_param_shapes(cfg).items()):
+        if len(shape) == 4:
+            fan_in = shape[1] * shape[2] * shape[3]
+            g = torch.Generator().manual_seed(seed * 1000 + i)
+            t = torch.randn(shape, generator=g, dtype=torch.float32) * math.sqrt(2.0 / fan_in)
+        elif name.endswith("weight"):
+            t = torch.ones(shape)
+        else:
+            t = torch.zeros(shape)
+        out[name] = t.to(dtype)
+    return out
+
+
+def bottleneck(x, p, cfg):
+    """x is NCHW here (torch's convention); identity shortcut (stride 1, Cin == 4*Cmid)."""
+    assert cfg.stride == 1 and cfg.in_channels == cfg.out_channels
+    bn = lambda t, i: F.batch_norm(t, None, None, p[f"residual_function.{i}.weight"],
+                                   p[f"residual_function.{i}.bias"], training=True, eps=cfg.bn_eps)
+    y = F.relu(bn(F.conv2d(x, p["residual_function.0.weight"]), 1))
+    y = F.relu(bn(F.conv2d(y, p["residual_function.3.weight"], stride=cfg.stride, padding=1), 4))
+    y = bn(F.conv2d(y, p["residual_function.6.weight"]), 7)
+    return F.relu(y + x)

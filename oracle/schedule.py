@@ -1,0 +1,138 @@
+"""Instruction streams of one pipeline stage, restated in closed form (TEST ORACLE).
+
+An instruction is a tuple ``(name, buffer_id, stage_id)``; ``buffer_id`` /
+``stage_id`` are ``None`` where the reference instruction does not carry them
+(``OptimizerStep()``, ``ReduceGrads(stage_id)``, ``LoadMicroBatch(buffer_id)``).
+
+Follows deepspeed/runtime/pipe/schedule.py of the reference:
+  step_to_micro_batch   schedule.py:6-46
+  train_schedule        schedule.py:225-310  (TrainSchedule.steps)
+  eager_merge           schedule.py:504-524  (EagerRecoverySchedule._merge_cmds)
+  next_stage_failover   schedule.py:343-430  (NextStageFailoverSchedule._merge_cmds)
+"""
+
+RC_KINDS = ("RecvActivation", "LoadMicroBatch", "ForwardPass")
+
+
+def step_to_micro_batch(stages, stage_id, step_id):
+    """(micro_batch_id, is_forward) of a step.  A step is a forward step when its
+    parity equals the stage's parity; forward id = (t - s)/2, backward id =
+    (t + s + 1)/2 - S  (closed form of schedule.py:6-46)."""
+    if (step_id - stage_id) % 2 == 0:
+        return (step_id - stage_id) // 2, True
+    return (step_id + stage_id + 1) // 2 - stages, False
+
+
+def total_steps(micro_batches, stages):
+    return 2 * (micro_batches + stages - 1)
+
+
+def train_schedule(micro_batches, stages, stage_id):
+    """List (one entry per step) of instruction lists of a 1F1B stage."""
+    M, S, s = micro_batches, stages, stage_id
+    valid = lambda k: 0 <= k < M
+    has_prev, has_next = s > 0, s < S - 1
+    loads = (s == 0) or (s == S - 1)
+    out, prev = [], -1
+    T = total_steps(M, S)
+    for t in range(T):
+        k, fwd = step_to_micro_batch(S, s, t)
+        cmds = []
+        if loads and fwd and valid(k):
+            cmds.append(("LoadMicroBatch", k, None))
+        if fwd:
+            if valid(k) and has_prev:
+                cmds.append(("RecvActivation", k, s))
+            if valid(prev) and has_prev:
+                cmds.append(("SendGrad", prev, s))
+        else:
+            if valid(prev) and has_next:
+                cmds.append(("SendActivation", prev, s))
+            if valid(k) and has_next:
+                cmds.append(("RecvGrad", k, s))
+        if valid(k):
+            cmds.append(("ForwardPass" if fwd else "BackwardPass", k, s))
+        if t == T - 1:
+            cmds.append(("ReduceGrads", None, s))
+            cmds.append(("OptimizerStep", None, None))
+        prev = k
+        out.append(cmds)
+    return out
+
+
+def eager_merge(own_steps, next_steps):
+    """Eager redundant computation: the successor's Recv/Load/Forward commands of a
+    step are queued, and the oldest queued step is emitted in front of the first
+    later own step that holds a RecvGrad (schedule.py:504-524)."""
+    fifo, out = [], []
+    for own, nxt in zip(own_steps, next_steps):
+        cmds = []
+        if any(c[0] == "RecvGrad" for c in own) and fifo:
+            cmds += [c for c in fifo.pop(0) if c[0] in RC_KINDS]
+        if any(c[0] in RC_KINDS for c in nxt):
+            fifo.append(nxt)
+        out.append(cmds + list(own))
+    return out
+
+
+def next_stage_failover(own_steps, next_steps, failed_step, curr_step):
+    """Merged stream after the successor died (schedule.py:343-430).
+
+    Steps before ``curr_step`` replay only the successor's commands (without its
+    sends while ``< failed_step``); later steps interleave both streams by the
+    eleven first-match rules of the reference."""
+    out = []
+    for i, (own, nxt) in enumerate(zip(own_steps, next_steps)):
+        if i < curr_step:
+            if i < failed_step:
+                out.append([c for c in nxt if c[0] not in ("SendActivation", "SendGrad")])
+            else:
+                out.append(list(nxt))
+            continue
+        a, b, res = list(own), list(nxt), []
+        while a or b:
+            ha = a[0][0] if a else None
+            hb = b[0][0] if b else None
+            if ha == "LoadMicroBatch":
+                res.append(a.pop(0))
+            elif ha == "RecvWeights":
+                a.pop(0)
+            elif hb == "SendWeights":
+                b.pop(0)
+            elif hb == "LoadMicroBatch":
+                res.append(b.pop(0))
+            elif hb in ("SendActivation", "RecvGrad"):
+                res.append(b.pop(0))
+            elif hb == "SendGrad":
+                assert ha == "RecvGrad", (own, nxt)
+                b.pop(0)
+                res.append(a.pop(0))
+            elif hb == "RecvActivation":
+                assert ha == "SendActivation", (own, nxt)
+                a.pop(0)
+                res.append(b.pop(0))
+            elif ha == "BackwardPass":
+                res.append(a.pop(0))
+            elif hb == "BackwardPass":
+                res.append(b.pop(0))
+            elif ha is not None:
+                res.append(a.pop(0))
+            else:
+                if hb in ("ForwardPass", "BackwardPass", "RecvWeights", "ReduceGrads"):
+                    res.append(b.pop(0))
+                elif hb == "OptimizerStep":
+                    b.pop(0)
+                else:
+                    raise RuntimeError(f"cannot merge {own} and {nxt}")
+        out.append(res)
+    return out
+
+
+def redundant_stage_ids(level, stage_id, stages):
+    """Stages whose layers ``stage_id`` shadows (redundancy.py:7-19)."""
+    return [(stage_id + i) % stages for i in range(1, level + 1)]
+
+
+def redundant_user_stage_ids(level, stage_id, stages):
+    """Stages that shadow ``stage_id`` (redundancy.py:22-31)."""
+    return [i for i in range(stages) if stage_id in redundant_stage_ids(level, i, stages)]

@@ -1,0 +1,265 @@
+"""Kernel parity on the GPU, called through the C ABI: every kernel against the oracle / a plain
+torch fp32 statement of the same operation on the same seeded inputs.
+
+Tolerances: fp32 relative 1e-5 of the tensor's scale (accumulation order differs from the
+CPU's), bf16 relative 2e-2; Adam is compared bit for bit with the oracle formula."""
+import math
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import adam as oadam
+from oracle import layers as ol
+
+pytestmark = pytest.mark.gpu
+
+DEV = "cuda:0"
+DTYPES = [torch.float32, torch.bfloat16]
+
+
+def tol(dtype):
+    return 1e-5 if dtype == torch.float32 else 2e-2
+
+
+def rel_err(got, ref):
+    got, ref = got.double().cpu(), ref.double().cpu()
+    return float((got - ref).abs().max() / ref.abs().max().clamp_min(1e-30))
+
+
+def randn(*shape, dtype=torch.float32, seed=0, scale=1.0):
+    g = torch.Generator().manual_seed(seed)
+    return (torch.randn(*shape, generator=g) * scale).to(dtype).to(DEV)
+
+
+GEMM_SHAPES = [(256, 256, 64), (512, 384, 128), (304, 200, 96), (64, 1024, 256), (1024, 64, 512),
+               (136, 72, 40), (2048, 768, 768), (8, 8, 8)]
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("layout", [0, 1, 2])
+@pytest.mark.parametrize("M,N,K", GEMM_SHAPES)
+def test_gemm_layouts(hiplib, dtype, layout, M, N, K):
+    a_shape = (K, M) if layout == hiplib.TN else (M, K)
+    b_shape = (N, K) if layout == hiplib.NT else (K, N)
+    A, B = randn(*a_shape, dtype=dtype, seed=1), randn(*b_shape, dtype=dtype, seed=2)
+    C = torch.full((M, N), float("nan"), dtype=dtype, device=DEV)
+    hiplib.gemm(layout, A, B, C)
+    Af, Bf = A.double().cpu(), B.double().cpu()
+    ref = (Af.t() if layout == hiplib.TN else Af) @ (Bf.t() if layout == hiplib.NT else Bf)
+    assert rel_err(C, ref) < tol(dtype)
+    # determinism: a second run is bit-identical
+    C2 = torch.empty_like(C)
+    hiplib.gemm(layout, A, B, C2)
+    assert torch.equal(C, C2)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_gemm_epilogues(hiplib, dtype):
+    M, N, K = 384, 512, 256
+    A, W = randn(M, K, dtype=dtype, seed=3), randn(N, K, dtype=dtype, seed=4, scale=0.1)
+    bias, R = randn(N, dtype=dtype, seed=5), randn(M, N, dtype=dtype, seed=6)
+    Af, Wf, bf_, Rf = A.double().cpu(), W.double().cpu(), bias.double().cpu(), R.double().cpu()
+    lin = Af @ Wf.t() + bf_
+    C = torch.empty(M, N, dtype=dtype, device=DEV)
+    hiplib.gemm(hiplib.NT, A, W, C, bias=bias)
+    assert rel_err(C, lin) < tol(dtype)
+    hiplib.gemm(hiplib.NT, A, W, C, bias=bias, epilogue=hiplib.EPI_RESIDUAL, resid=R)
+    assert rel_err(C, lin + Rf) < tol(dtype)
+    for act, name in ((hiplib.ACT_RELU, "relu"), (hiplib.ACT_GELU_TANH, "gelu_tanh")):
+        U = torch.empty_like(C)
+        hiplib.gemm(hiplib.NT, A, W, C, bias=bias, epilogue=hiplib.EPI_ACT, act=act, aux_out=U)
+        assert rel_err(U, lin) < tol(dtype)
+        assert rel_err(C, ol.activation(lin, name)) < tol(dtype)
+        # dact: C = (A W^T) * act'(U)
+        Uf = U.double().cpu().requires_grad_(True)
+        ol.activation(Uf, name).sum().backward()
+        hiplib.gemm(hiplib.NT, A, W, C, epilogue=hiplib.EPI_DACT, act=act, aux_in=U)
+        assert rel_err(C, (Af @ Wf.t()) * Uf.grad) < tol(dtype)
+    # fp32 accumulate (weight-gradient form): G += A^T B
+    G0 = randn(K, N, dtype=torch.float32, seed=7)
+    G = G0.clone()
+    Bm = randn(M, N, dtype=dtype, seed=8)
+    hiplib.gemm(hiplib.TN, A, Bm, G, accumulate=True)
+    assert rel_err(G, G0.double().cpu() + Af.t() @ Bm.double().cpu()) < tol(dtype)
+    # alpha
+    hiplib.gemm(hiplib.NT, A, W, C, alpha=0.125)
+    assert rel_err(C, 0.125 * (Af @ Wf.t())) < tol(dtype)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_gemm_batched_heads(hiplib, dtype):
+    """Q K^T and P V over (batch, head) strides inside a [rows, 3h] buffer."""
+    b, a, s, d = 2, 3, 128, 64
+    h = a * d
+    qkv = randn(b * s, 3 * h, dtype=dtype, seed=9, scale=0.5)
+    P = torch.empty(b, a, s, s, dtype=dtype, device=DEV)
+    es = qkv.element_size()
+    hiplib.gemm_batched(hiplib.NT, hiplib.dtype_code(dtype), s, s, d, qkv.data_ptr(), 3 * h, (s * 3 * h, d),
+                        qkv.data_ptr() + h * es, 3 * h, (s * 3 * h, d), P.data_ptr(), s, (a * s * s, s * s), b, a,
+                        alpha=0.125)
+    q = qkv[:, :h].double().cpu().view(b, s, a, d).transpose(1, 2)
+    k = qkv[:, h:2 * h].double().cpu().view(b, s, a, d).transpose(1, 2)
+    v = qkv[:, 2 * h:].double().cpu().view(b, s, a, d).transpose(1, 2)
+    assert rel_err(P, 0.125 * q @ k.transpose(-1, -2)) < tol(dtype)
+    ctx = torch.empty(b * s, h, dtype=dtype, device=DEV)
+    hiplib.gemm_batched(hiplib.NN, hiplib.dtype_code(dtype), s, d, s, P.data_ptr(), s, (a * s * s, s * s),
+                        qkv.data_ptr() + 2 * h * es, 3 * h, (s * 3 * h, d), ctx.data_ptr(), h, (s * h, d), b, a)
+    ref = (P.double().cpu() @ v).transpose(1, 2).reshape(b * s, h)
+    assert rel_err(ctx, ref) < tol(dtype)
+    dV = torch.empty(b * s, h, dtype=dtype, device=DEV)
+    hiplib.gemm_batched(hiplib.TN, hiplib.dtype_code(dtype), s, d, s, P.data_ptr(), s, (a * s * s, s * s),
+                        ctx.data_ptr(), h, (s * h, d), dV.data_ptr(), h, (s * h, d), b, a)
+    c4 = ctx.double().cpu().view(b, s, a, d).transpose(1, 2)
+    ref = (P.double().cpu().transpose(-1, -2) @ c4).transpose(1, 2).reshape(b * s, h)
+    assert rel_err(dV, ref) < tol(dtype)
+
+
+def test_gemm_rejects_bad_arguments(hiplib):
+    A = torch.zeros(16, 12, dtype=torch.bfloat16, device=DEV)   # K = 12 is not a multiple of 8
+    B = torch.zeros(16, 12, dtype=torch.bfloat16, device=DEV)
+    C = torch.zeros(16, 16, dtype=torch.bfloat16, device=DEV)
+    with pytest.raises(hiplib.HipKernelError):
+        hiplib.gemm(hiplib.NT, A, B, C)
+    A8 = torch.zeros(16, 8, dtype=torch.bfloat16, device=DEV)
+    with pytest.raises(hiplib.HipKernelError):
+        hiplib.gemm(hiplib.NT, A8, A8, C, accumulate=True)  # accumulate needs fp32 C
+    # empty problem is a no-op
+    hiplib.gemm(hiplib.NT, A8[:0], A8, C[:0])
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("kind", ["standard", "annotated"])
+@pytest.mark.parametrize("rows,cols", [(64, 768), (37, 1024), (16, 1600), (5, 64), (3, 4096)])
+def test_layernorm_fwd_bwd(hiplib, dtype, kind, rows, cols):
+    eps = 1e-6 if kind == "annotated" else 1e-5
+    x, dy, dres = randn(rows, cols, dtype=dtype, seed=10), randn(rows, cols, dtype=dtype, seed=11), randn(rows, cols, dtype=dtype, seed=12)
+    g = (1 + 0.1 * randn(cols, seed=13)).to(dtype)
+    b = (0.1 * randn(cols, seed=14)).to(dtype)
+    y = torch.empty_like(x)
+    mean, rinv = torch.empty(rows, device=DEV), torch.empty(rows, device=DEV)
+    hiplib.layernorm_fwd(x, g, b, y, mean, rinv, hiplib.LN_CODES[kind], eps)
+    xr = x.double().cpu().requires_grad_(True)
+    gr, br = g.double().cpu().requires_grad_(True), b.double().cpu().requires_grad_(True)
+    yr = ol.layer_norm(xr, gr, br, kind, eps)
+    assert rel_err(y, yr.detach()) < tol(dtype)
+    yr.backward(dy.double().cpu())
+    dx = torch.empty_like(x)
+    dg0, db0 = randn(cols, seed=15), randn(cols, seed=16)
+    dg, db = dg0.clone(), db0.clone()
+    ws = torch.empty(hiplib.layernorm_bwd_workspace(cols), device=DEV)
+    hiplib.layernorm_bwd(x, g, mean, rinv, dy, dres, dx, dg, db, ws, hiplib.LN_CODES[kind], eps)
+    assert rel_err(dx, xr.grad + dres.double().cpu()) < tol(dtype)
+    assert rel_err(dg - dg0, gr.grad) < tol(dtype) * 2
+    assert rel_err(db - db0, br.grad) < tol(dtype) * 2
+    hiplib.layernorm_bwd(x, g, mean, rinv, dy, None, dx, dg, db, ws, hiplib.LN_CODES[kind], eps)
+    assert rel_err(dx, xr.grad) < tol(dtype)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("mask", ["none", "causal", "key_padding"])
+def test_softmax(hiplib, dtype, mask):
+    b, a, s = 3, 2, 256
+    sc = randn(b, a, s, s, dtype=dtype, seed=17, scale=2.0)
+    lens = torch.tensor([256, 1, 100], dtype=torch.int32, device=DEV) if mask == "key_padding" else None
+    ref_in = sc.double().cpu()
+    cfg = ol.TransformerCfg(hidden=8, heads=a, ffn=8, mask=mask)
+    m = ol.build_mask(cfg, b, s, None if lens is None else lens.cpu())
+    if m is not None:
+        ref_in = ref_in.masked_fill(~m, -1e9)
+    ref = torch.softmax(ref_in, -1)
+    p = sc.clone()
+    hiplib.softmax_fwd(p, hiplib.MASK_CODES[mask], lens)
+    assert float((p.double().cpu() - ref).abs().max()) < (1e-6 if dtype == torch.float32 else 4e-3)
+    if mask == "causal":
+        assert float(p[:, :, 0, 1:].abs().max()) == 0.0
+    dp = randn(b, a, s, s, dtype=dtype, seed=18)
+    pr = p.double().cpu()
+    dref = pr * (dp.double().cpu() - (dp.double().cpu() * pr).sum(-1, keepdim=True))
+    hiplib.softmax_bwd(p, dp)
+    assert rel_err(dp, dref) < tol(dtype)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("rows,cols", [(1000, 768), (8192, 3072), (7, 64), (513, 1600)])
+def test_colsum(hiplib, dtype, rows, cols):
+    x = randn(rows, cols, dtype=dtype, seed=19)
+    out0 = randn(cols, seed=20)
+    out = out0.clone()
+    ws = torch.empty(hiplib.colsum_workspace(cols), device=DEV)
+    hiplib.colsum_acc(x, out, ws)
+    ref = out0.double().cpu() + x.double().cpu().sum(0)
+    assert rel_err(out, ref) < 1e-5
+    out2 = out0.clone()
+    hiplib.colsum_acc(x, out2, ws)
+    assert torch.equal(out, out2)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_residual_add_cast_fill(hiplib, dtype):
+    a, b = randn(1000, 64, dtype=dtype, seed=21), randn(1000, 64, dtype=dtype, seed=22)
+    out = torch.empty_like(a)
+    hiplib.residual_add(a, b, out)
+    assert torch.equal(out, (a.float() + b.float()).to(dtype))
+    src = randn(12345, seed=23)
+    dst = torch.empty(12345, dtype=torch.bfloat16, device=DEV)
+    hiplib.cast(src, dst)
+    assert torch.equal(dst, src.to(torch.bfloat16))             # round-to-nearest-even both sides
+    back = torch.empty(12345, device=DEV)
+    hiplib.cast(dst, back)
+    assert torch.equal(back, dst.float())
+    f = torch.empty(777, device=DEV)
+    hiplib.fill_f32(f, 3.5)
+    assert float(f.min()) == float(f.max()) == 3.5
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_mse(hiplib, dtype):
+    n = 4 * 128 * 768
+    y, t = randn(n, dtype=dtype, seed=24), randn(n, dtype=dtype, seed=25)
+    dy = torch.empty_like(y)
+    loss = torch.full((1,), 5.0, device=DEV)
+    ws = torch.empty(hiplib.mse_workspace(), device=DEV)
+    hiplib.mse_fwd_bwd(y, t, dy, 0.125, loss, True, ws)
+    yr = y.double().cpu().requires_grad_(True)
+    lr = torch.nn.functional.mse_loss(yr, t.double().cpu())
+    (lr * 0.125).backward()
+    assert abs(float(loss) - 5.0 - float(lr)) < 1e-5 * float(lr)
+    assert rel_err(dy, yr.grad) < tol(dtype)
+    hiplib.mse_fwd_bwd(y, t, dy, 0.125, loss, False, ws)
+    assert abs(float(loss) - float(lr)) < 1e-5 * float(lr)
+
+
+@pytest.mark.parametrize("adam_w,wd", [(True, 0.0), (True, 0.01), (False, 0.01)])
+def test_adam_bit_exact_with_oracle(hiplib, adam_w, wd):
+    """Sizes of the reference's own Adam test (tests/unit/test_cpu_adam.py:25-27) plus ragged
+    ones; 10 steps; fp32 state compared bit for bit with the oracle formula, bf16 copy with
+    the rounded parameter."""
+    sizes = [22, 55, 64, 127, 1024, 1048576, 4097, 8192 + 3]
+    sizes = [(n + 3) // 4 * 4 for n in sizes]          # 16-byte aligned tensor starts
+    total = sum(sizes)
+    flat = lambda seed: randn(total, seed=seed)
+    P, M_, V = flat(30), torch.zeros(total, device=DEV), torch.zeros(total, device=DEV)
+    LP = torch.zeros(total, dtype=torch.bfloat16, device=DEV)
+    offs = np.cumsum([0] + sizes)
+    split = lambda t: [t[offs[i]: offs[i + 1]] for i in range(len(sizes))]
+    p_ref = P.cpu().numpy().copy()
+    m_ref, v_ref = np.zeros(total, np.float32), np.zeros(total, np.float32)
+    for step in range(1, 11):
+        G = flat(100 + step)
+        g_ref = G.cpu().numpy().copy()
+        hiplib.adam_multi(split(G), split(P), split(M_), split(V), split(LP), lr=1e-3, beta1=0.9, beta2=0.999,
+                          eps=1e-8, step=step, adam_w_mode=adam_w, weight_decay=wd, zero_grad=(step % 2 == 0))
+        oadam.adam_step(p_ref, g_ref, m_ref, v_ref, step, weight_decay=wd, adam_w_mode=adam_w)
+        assert np.array_equal(P.cpu().numpy(), p_ref), f"step {step}: parameters differ"
+        assert np.array_equal(M_.cpu().numpy(), m_ref) and np.array_equal(V.cpu().numpy(), v_ref)
+        assert torch.equal(LP, P.to(torch.bfloat16))
+        assert (float(G.abs().max()) == 0.0) == (step % 2 == 0)
+    # agreement with torch.optim (the reference's own check, atol 1e-2) follows from the oracle test
+
+
+def test_adam_rejects_bad_arguments(hiplib):
+    t = torch.zeros(16, device=DEV)
+    with pytest.raises(hiplib.HipKernelError):
+        hiplib.adam_multi([t], [t], [t], [t], None, lr=1e-3, beta1=0.9, beta2=0.999, eps=1e-8, step=0)
+    hiplib.adam_multi([], [], [], [], None, lr=1e-3, beta1=0.9, beta2=0.999, eps=1e-8, step=1)  # empty list is fine

@@ -1,0 +1,241 @@
+"""Stage-level parity on the GPU: the engine (HIP kernels through the C ABI) against the CPU
+oracle stage on the same seeded inputs -- loss, parameter gradients, input gradients, the
+bit-exactness of redundant forwards, failover promotion and the optimizer step.
+
+Tolerances (of the tensor's own scale): fp32 1e-5 on activations / 1e-4 on accumulated
+gradients (different summation order over 2048 rows x 8 micro-batches), bf16 2e-2."""
+import pytest
+import torch
+
+import bamboo_amd
+from bamboo_amd import LayerSpec, PipelineModule, SeededActivationQueue, TransformerLayer
+from oracle import layers as ol
+from oracle.stage import OraclePeer, OracleStage
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+def rel_err(got, ref):
+    got, ref = got.double().cpu(), ref.double().cpu()
+    return float((got - ref).abs().max() / ref.abs().max().clamp_min(1e-30))
+
+
+def build(hidden, heads, ffn, layers_per_stage, stages, stage_id, mb, M, seq, dtype, variant, rl, eager,
+          grad_mode="queue", rc_stream=False, key_len_range=None):
+    specs = [LayerSpec(TransformerLayer, hidden, heads, ffn, **variant) for _ in range(layers_per_stage * stages)]
+    model = PipelineModule(specs, num_stages=stages, partition_method="uniform", stage_id=stage_id, dtype=dtype, device=DEV)
+    q = SeededActivationQueue((mb, seq, hidden), dtype, M, stage_ids=[stage_id, (stage_id + 1) % stages], seed=7,
+                              grad_mode=grad_mode, device=DEV, key_len_range=key_len_range)
+    cfg = {"train_micro_batch_size_per_gpu": mb, "gradient_accumulation_steps": M,
+           "optimizer": {"type": "Adam", "params": {"lr": 1e-3}}, "bf16": {"enabled": dtype == torch.bfloat16}}
+    engine, _, _, _ = bamboo_amd.initialize(model=model, config=cfg, redundancy_level=rl, eager_recovery=eager,
+                                            activation_queue=q, rc_stream=rc_stream, install_signal_handler=False)
+    return engine, q
+
+
+def oracle_for(engine, q, variant, hidden, heads, ffn, layers_per_stage, stages, stage_id, M, rl, eager, dtype=torch.float64):
+    cfg = ol.TransformerCfg(hidden=hidden, heads=heads, ffn=ffn, **variant)
+    parts = [i * layers_per_stage for i in range(stages + 1)]
+    st = OracleStage(cfg, parts, stage_id, M, dtype=dtype, redundancy_level=rl, eager=eager)
+    # the oracle starts from exactly the engine's (possibly bf16-rounded) compute weights
+    for sid in list(st.params):
+        sp = engine.module.stage_params[sid]
+        named = sp.named(sp.compute)
+        for key, t in st.named_params(sid).items():
+            with torch.no_grad():
+                t.copy_(named[key].to(dtype).cpu())
+    acts = [a.to(dtype).cpu() for a in q.activations]
+    kl = None if q.key_lens is None else [k.cpu() for k in q.key_lens]
+    if q.grad_mode == "queue":
+        peer = OraclePeer(acts, M, grads={s: [g.to(dtype).cpu() for g in gs] for s, gs in q.grads.items()}, key_lens=kl)
+    else:
+        peer = OraclePeer(acts, M, targets={s: [t.to(dtype).cpu() for t in ts] for s, ts in q.targets.items()}, key_lens=kl)
+    return st, peer
+
+
+def snapshot_grads(engine, sid):
+    return {k: v.clone() for k, v in engine.module.get_named_grad(sid)}
+
+
+class NoStep:
+    """Keeps the optimizer from consuming the gradients so they can be inspected."""
+
+    def __init__(self, engine):
+        self.engine = engine
+
+    def __enter__(self):
+        self.saved = self.engine._exec_optimizer_step
+        self.engine._INSTRUCTION_MAP = dict(self.engine._INSTRUCTION_MAP)
+        from bamboo_amd import schedule
+        self.engine._INSTRUCTION_MAP[schedule.OptimizerStep] = lambda self_: None
+        return self
+
+    def __exit__(self, *a):
+        del self.engine._INSTRUCTION_MAP
+
+
+REFERENCE_VARIANT = dict(activation="relu", ln="annotated", mask="none")
+GPT_VARIANT = dict(activation="gelu_tanh", ln="standard", mask="causal")
+BERT_VARIANT = dict(activation="gelu_tanh", ln="standard", mask="key_padding")
+
+
+@pytest.mark.parametrize("variant,klr", [(REFERENCE_VARIANT, None), (GPT_VARIANT, None), (BERT_VARIANT, (5, 64))],
+                         ids=["reference", "gpt", "bert"])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["fp32", "bf16"])
+def test_stage_matches_oracle_with_rc(hiplib, variant, klr, dtype):
+    hid, heads, ffn, L, S, sid, mb, M, seq = 128, 2, 256, 2, 4, 1, 2, 4, 64
+    engine, q = build(hid, heads, ffn, L, S, sid, mb, M, seq, dtype, variant, 1, True, key_len_range=klr)
+    st, peer = oracle_for(engine, q, variant, hid, heads, ffn, L, S, sid, M, 1, True)
+    bufs, _ = st.run_batch(peer, optimizer_step=False)
+    with NoStep(engine):
+        engine._reserve_pipe_buffers(M)
+        keep = {}
+        orig_clean = engine._clean_pipe_buffers
+        engine._clean_pipe_buffers = lambda: keep.update({k: list(v) for k, v in engine.pipe_buffers.items()})
+        engine.train_batch()
+        engine._clean_pipe_buffers = orig_clean
+    t_act = 1e-5 if dtype == torch.float32 else 2e-2
+    t_grad = 1e-4 if dtype == torch.float32 else 2e-2
+    for k in range(M):
+        assert rel_err(keep[f"output_{sid}"][k], bufs["out"][(sid, k)].detach().view(mb * seq, hid)) < t_act
+        assert rel_err(keep[f"output_{sid + 1}"][k], bufs["out"][(sid + 1, k)].detach().view(mb * seq, hid)) < t_act
+        assert rel_err(keep[f"input_grad_{sid}"][k], bufs["sent_grad"][(sid, k)].view(mb * seq, hid)) < t_grad
+    ref_grads = st.named_grads(sid)
+    for name, g in engine.module.get_named_grad(sid):
+        assert rel_err(g, ref_grads[name]) < t_grad, name
+    # shadow parameters receive no gradient from redundant forwards
+    for name, g in engine.module.get_named_grad(sid + 1):
+        assert float(g.abs().max()) == 0.0
+
+
+@pytest.mark.parametrize("rc_stream", [False, True], ids=["one-stream", "rc-stream"])
+def test_rc_forward_bit_exact_and_rc_neutral(hiplib, rc_stream):
+    """(1) The redundant forward of the shadow layers is bit-identical to a normal forward of the
+    same layers on the same input; (2) switching RC on changes nothing in the own results."""
+    hid, heads, ffn, L, S, sid, mb, M, seq = 256, 4, 512, 2, 4, 1, 2, 6, 128
+    dtype = torch.bfloat16
+    outs = {}
+    for tag, (rl, eager) in {"off": (0, False), "on": (1, True)}.items():
+        engine, q = build(hid, heads, ffn, L, S, sid, mb, M, seq, dtype, GPT_VARIANT, rl, eager, rc_stream=rc_stream)
+        with NoStep(engine):
+            keep = {}
+            engine._clean_pipe_buffers = lambda: keep.update({k: [None if t is None else t.clone() for t in v]
+                                                              for k, v in engine.pipe_buffers.items()})
+            engine.train_batch()
+        torch.cuda.synchronize()
+        outs[tag] = (keep, snapshot_grads(engine, sid), engine)
+    for k in range(M):
+        assert torch.equal(outs["off"][0][f"output_{sid}"][k], outs["on"][0][f"output_{sid}"][k])
+        assert torch.equal(outs["off"][0][f"input_grad_{sid}"][k], outs["on"][0][f"input_grad_{sid}"][k])
+    for name in outs["off"][1]:
+        assert torch.equal(outs["off"][1][name], outs["on"][1][name]), name
+    # normal forward of the shadow stage's layers, as a stage of its own, on the own outputs
+    keep, _, engine = outs["on"]
+    specs = [LayerSpec(TransformerLayer, hid, heads, ffn, **GPT_VARIANT) for _ in range(L * S)]
+    model2 = PipelineModule(specs, num_stages=S, partition_method="uniform", stage_id=sid + 1, dtype=dtype, device=DEV)
+    ctx2 = model2.prepare_context([sid + 1], mb, seq)
+    model2.allocate_stash(sid + 1, ctx2, 1)
+    for k in range(M):
+        normal = model2.forward(keep[f"output_{sid}"][k], sid + 1, slot=0, ctx=ctx2)
+        torch.cuda.synchronize()
+        assert torch.equal(normal, keep[f"output_{sid + 1}"][k]), f"micro-batch {k}"
+
+
+@pytest.mark.parametrize("dead_from", [0, 2, 3])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["fp32", "bf16"])
+def test_failover_promotion_matches_oracle(hiplib, dead_from, dtype):
+    """The successor is preempted at micro-batch ``dead_from``: the engine promotes the shadow
+    layers, replays the successor's backward passes from the stashed redundant activations and
+    ends the batch with the gradients of both stages (oracle: same stream on CPU autograd)."""
+    hid, heads, ffn, L, S, sid, mb, M, seq = 128, 2, 256, 2, 4, 1, 2, 4, 64
+    engine, q = build(hid, heads, ffn, L, S, sid, mb, M, seq, dtype, GPT_VARIANT, 1, True, grad_mode="mse")
+    st, peer = oracle_for(engine, q, GPT_VARIANT, hid, heads, ffn, L, S, sid, M, 1, True)
+    # while alive, the successor returns the true gradients of the downstream loss
+    succ_cfg = ol.TransformerCfg(hidden=hid, heads=heads, ffn=ffn, **GPT_VARIANT)
+    true_grads = []
+    for k in range(M):
+        o1 = st.forward(peer.activations[k], sid).detach().requires_grad_(True)
+        o2 = st.forward(o1, sid + 1)
+        (torch.nn.functional.mse_loss(o2, peer.targets[sid + 1][k]) / M).backward()
+        true_grads.append(o1.grad)
+    for s_ in st.params.values():
+        for p in s_:
+            for t in p.values():
+                t.grad = None
+    peer.targets = {sid + 1: peer.targets[sid + 1]}
+    peer.grads = {sid: true_grads}
+    peer.dead_from, peer.dead_stage = dead_from, sid
+    st.run_batch(peer, optimizer_step=False)
+
+    q.grad_mode = "mse"
+    q.set_grads(sid, [g.view(mb, seq, hid) for g in true_grads])
+    q.targets.pop(sid)                      # own outputs go to a live successor, not to a loss head
+    orig_send = q.send_activation
+
+    def send(k, tensor, stage_id, stream=None):
+        if stage_id == sid:
+            q._check_alive(k, stage_id)
+            return
+        return orig_send(k, tensor, stage_id, stream=stream)
+    q.send_activation = send
+    q.preempt_successor(dead_from, sid)
+    with NoStep(engine):
+        loss = engine.train_batch()
+    assert engine.stage_ids == [sid, sid + 1] and engine.r_stage_ids == []
+    tg = 1e-4 if dtype == torch.float32 else 3e-2
+    for s_ in (sid, sid + 1):
+        ref = st.named_grads(s_)
+        for name, g in engine.module.get_named_grad(s_):
+            assert rel_err(g, ref[name]) < tg, (s_, name)
+    assert abs(float(loss) - float(peer.loss) / M) < tg * max(1.0, float(peer.loss) / M)
+    # next batch runs as a merged two-stage process from step 0
+    q.revive()
+    engine.train_batch()
+    assert engine.global_steps == 1 or engine.global_steps == 2
+
+
+def test_optimizer_step_matches_oracle(hiplib):
+    hid, heads, ffn, L, S, sid, mb, M, seq = 128, 2, 256, 2, 4, 1, 2, 4, 64
+    engine, q = build(hid, heads, ffn, L, S, sid, mb, M, seq, torch.float32, GPT_VARIANT, 0, False)
+    st, peer = oracle_for(engine, q, GPT_VARIANT, hid, heads, ffn, L, S, sid, M, 0, False, dtype=torch.float32)
+    before = {k: v.clone() for k, v in engine.module.get_named_param(sid)}
+    for _ in range(2):
+        engine.train_batch()
+        st.run_batch(peer)
+    assert engine.global_steps == 2
+    ref = st.named_params(sid)
+    for name, p in engine.module.get_named_param(sid):
+        # Adam's first steps move every weight by ~lr whatever the gradient scale, so compare the
+        # movement: |delta - delta_ref| small against lr
+        d, dr = (p - before[name]).cpu(), (ref[name].detach() - before[name].cpu())
+        assert float((d - dr).abs().max()) < 2e-4, name
+        assert float(d.abs().max()) > 1e-4
+    for name, g in engine.module.get_named_grad(sid):
+        assert float(g.abs().max()) == 0.0      # zero_grad fused into the optimizer kernel
+
+
+def test_engine_surface(hiplib):
+    hid, heads, ffn, L, S, sid, mb, M, seq = 128, 2, 256, 1, 4, 1, 2, 4, 64
+    engine, q = build(hid, heads, ffn, L, S, sid, mb, M, seq, torch.float32, GPT_VARIANT, 1, True)
+    assert (engine.micro_batches, engine.micro_batch_size, engine.stage_id, engine.num_stages) == (M, mb, sid, S)
+    assert engine.stage_ids == [sid] and engine.r_stage_ids == [sid + 1] and engine.r_user_stage_ids == [sid - 1]
+    assert not engine.is_first_stage() and not engine.is_last_stage()
+    for key in (f"input_{sid}", f"output_{sid}", f"input_{sid + 1}", f"output_{sid + 1}", f"input_grad_{sid}", "data", "label"):
+        assert key in engine.pipe_buffers
+    with pytest.raises(bamboo_amd.PipelineError):
+        engine.forward(None)
+    with pytest.raises(bamboo_amd.PipelineError):
+        engine.backward(None)
+    with pytest.raises(bamboo_amd.PipelineError):
+        engine.step()
+    names = [n for n, _ in engine.module.get_named_param(sid)]
+    assert names[0] == "1.sublayer.0.norm.a_2" and "1.self_attn.linears.3.weight" in names
+    assert set(engine.param_buffers[sid + 1]) == {n for n, _ in engine.module.get_named_param(sid + 1)}
+    with pytest.raises(Exception):
+        build(hid, heads, ffn, L, S, sid, mb, M, seq, torch.float32, GPT_VARIANT, 0, True)
+    with pytest.raises(NotImplementedError):
+        build(hid, heads, ffn, L, S, sid, mb, M, seq, torch.float32, GPT_VARIANT, 2, True)
+    loss = engine.train_batch()
+    assert loss.shape == (1,) and engine.global_steps == 1
+    assert all(b is None for b in engine.pipe_buffers[f"output_{sid}"])

@@ -1,0 +1,127 @@
+"""Pins of the layer oracle against torch library routines and closed forms."""
+import math
+
+import numpy as np
+import pytest
+import torch
+import torch.nn.functional as F
+
+from oracle import adam as oadam
+from oracle import layers as ol
+
+
+def test_annotated_layernorm_closed_form():
+    torch.manual_seed(0)
+    x = torch.randn(5, 7, 32, dtype=torch.float64)
+    g, b = torch.randn(32, dtype=torch.float64), torch.randn(32, dtype=torch.float64)
+    y = ol.layer_norm(x, g, b, "annotated", 1e-6)
+    xn = x.numpy()
+    mean = xn.mean(-1, keepdims=True)
+    std = np.sqrt(((xn - mean) ** 2).sum(-1, keepdims=True) / (32 - 1))      # unbiased
+    ref = g.numpy() * (xn - mean) / (std + 1e-6) + b.numpy()
+    np.testing.assert_allclose(y.numpy(), ref, rtol=1e-12, atol=1e-12)
+    # a biased estimator or eps inside the sqrt must NOT pass
+    bad = g.numpy() * (xn - mean) / (np.sqrt(((xn - mean) ** 2).mean(-1, keepdims=True)) + 1e-6) + b.numpy()
+    assert np.abs(bad - ref).max() > 1e-3
+
+
+@pytest.mark.parametrize("mask", ["none", "causal", "key_padding"])
+def test_attention_matches_sdpa(mask):
+    torch.manual_seed(1)
+    cfg = ol.TransformerCfg(hidden=64, heads=4, ffn=128, mask=mask)
+    p = ol.init_params(cfg, 3, dtype=torch.float64, std=0.3)
+    for k in p:
+        if k.endswith("bias"):
+            p[k] = torch.randn_like(p[k]) * 0.1
+    b, s = 3, 16
+    x = torch.randn(b, s, 64, dtype=torch.float64)
+    lens = torch.tensor([16, 5, 9]) if mask == "key_padding" else None
+    got = ol.attention(x, p, cfg, lens)
+    lin = lambda i, t: F.linear(t, p[f"self_attn.linears.{i}.weight"], p[f"self_attn.linears.{i}.bias"])
+    q, k, v = [lin(i, x).view(b, s, 4, 16).transpose(1, 2) for i in range(3)]
+    if mask == "none":
+        ctx = F.scaled_dot_product_attention(q, k, v)
+    elif mask == "causal":
+        ctx = F.scaled_dot_product_attention(q, k, v, is_causal=True)
+    else:
+        m = (torch.arange(s).view(1, 1, 1, s) < lens.view(b, 1, 1, 1))
+        ctx = F.scaled_dot_product_attention(q, k, v, attn_mask=m)
+    ref = lin(3, ctx.transpose(1, 2).reshape(b, s, 64))
+    torch.testing.assert_close(got, ref, rtol=1e-10, atol=1e-10)
+
+
+def test_layer_matches_torch_encoder_layer():
+    """Pre-LN, ReLU, standard LayerNorm, no mask == nn.TransformerEncoderLayer(norm_first=True)."""
+    torch.manual_seed(2)
+    h, a, f = 48, 4, 96
+    cfg = ol.TransformerCfg(hidden=h, heads=a, ffn=f, activation="relu", ln="standard", mask="none")
+    p = ol.init_params(cfg, 5, dtype=torch.float64, std=0.2)
+    for k in p:
+        if k.endswith("bias") or k.endswith("b_2"):
+            p[k] = torch.randn_like(p[k]) * 0.1
+        if k.endswith("a_2"):
+            p[k] = 1 + 0.1 * torch.randn_like(p[k])
+    ref = torch.nn.TransformerEncoderLayer(h, a, f, dropout=0.0, activation="relu", batch_first=True,
+                                           norm_first=True, dtype=torch.float64)
+    with torch.no_grad():
+        ref.self_attn.in_proj_weight.copy_(torch.cat([p[f"self_attn.linears.{i}.weight"] for i in range(3)]))
+        ref.self_attn.in_proj_bias.copy_(torch.cat([p[f"self_attn.linears.{i}.bias"] for i in range(3)]))
+        ref.self_attn.out_proj.weight.copy_(p["self_attn.linears.3.weight"])
+        ref.self_attn.out_proj.bias.copy_(p["self_attn.linears.3.bias"])
+        ref.linear1.weight.copy_(p["feed_forward.w_1.weight"]); ref.linear1.bias.copy_(p["feed_forward.w_1.bias"])
+        ref.linear2.weight.copy_(p["feed_forward.w_2.weight"]); ref.linear2.bias.copy_(p["feed_forward.w_2.bias"])
+        ref.norm1.weight.copy_(p["sublayer.0.norm.a_2"]); ref.norm1.bias.copy_(p["sublayer.0.norm.b_2"])
+        ref.norm2.weight.copy_(p["sublayer.1.norm.a_2"]); ref.norm2.bias.copy_(p["sublayer.1.norm.b_2"])
+    x = torch.randn(2, 10, h, dtype=torch.float64)
+    torch.testing.assert_close(ol.transformer_layer(x, p, cfg), ref(x), rtol=1e-9, atol=1e-9)
+    cfg_c = ol.TransformerCfg(hidden=h, heads=a, ffn=f, activation="relu", ln="standard", mask="causal")
+    cm = torch.nn.Transformer.generate_square_subsequent_mask(10, dtype=torch.float64)
+    torch.testing.assert_close(ol.transformer_layer(x, p, cfg_c), ref(x, src_mask=cm, is_causal=True), rtol=1e-9, atol=1e-9)
+
+
+def test_gelu_tanh_formula():
+    x = torch.linspace(-4, 4, 101, dtype=torch.float64)
+    ref = 0.5 * x * (1 + torch.tanh(0.7978845608028654 * (x + 0.044715 * x ** 3)))
+    torch.testing.assert_close(ol.activation(x, "gelu_tanh"), ref, rtol=1e-12, atol=1e-12)
+
+
+def test_param_count_matches_reference_known_answer():
+    # 12 596 224 parameters per layer at hidden 1024, ffn 4096 (tests/unit/test_partition.py:161)
+    cfg = ol.TransformerCfg(hidden=1024, heads=16, ffn=4096)
+    assert sum(math.prod(s) for s in ol.param_shapes(cfg).values()) == 12596224
+
+
+def test_bottleneck_identity_shapes_and_relu():
+    cfg = ol.BottleneckCfg(in_channels=64, mid_channels=16)
+    p = ol.init_bottleneck_params(cfg, 1)
+    x = torch.randn(4, 64, 6, 6)
+    y = ol.bottleneck(x, p, cfg)
+    assert y.shape == x.shape and (y >= 0).all()
+    # zero last BN gain => residual branch vanishes => relu(x)
+    p["residual_function.7.weight"].zero_()
+    torch.testing.assert_close(ol.bottleneck(x, p, cfg), F.relu(x))
+
+
+@pytest.mark.parametrize("adam_w,wd", [(True, 0.0), (True, 0.01), (False, 0.01)])
+def test_adam_matches_torch(adam_w, wd):
+    torch.manual_seed(3)
+    n = 1031
+    p0 = torch.randn(n)
+    p_t = p0.clone().requires_grad_(True)
+    opt = (torch.optim.AdamW if adam_w else torch.optim.Adam)([p_t], lr=1e-3, betas=(0.9, 0.999), eps=1e-8, weight_decay=wd)
+    p, m, v = p0.numpy().copy(), np.zeros(n, np.float32), np.zeros(n, np.float32)
+    for step in range(1, 11):
+        g = torch.randn(n)
+        p_t.grad = g.clone()
+        opt.step()
+        oadam.adam_step(p, g.numpy(), m, v, step, weight_decay=wd, adam_w_mode=adam_w)
+        np.testing.assert_allclose(p, p_t.detach().numpy(), rtol=2e-6, atol=2e-7)
+
+
+def test_adam_first_step_closed_form():
+    # step 1 with zero moments: update = g / (|g| + eps*sqrt(1-b2)) ~ sign(g): p1 = p0 - lr*sign(g)
+    p = np.array([1.0, -2.0, 3.0], np.float32)
+    g = np.array([0.5, -0.25, 4.0], np.float32)
+    m, v = np.zeros(3, np.float32), np.zeros(3, np.float32)
+    oadam.adam_step(p, g, m, v, 1, lr=0.1)
+    np.testing.assert_allclose(p, [0.9, -1.9, 2.9], rtol=1e-5)
