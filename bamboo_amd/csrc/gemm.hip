@@ -412,6 +412,7 @@ extern "C" int bb_gemm(const bb_gemm_desc* d, void* stream) {
     BB_REQUIRE(d->c_dtype == d->dtype || d->c_dtype == BB_F32, "bb_gemm: bad c_dtype %d", d->c_dtype);
     BB_REQUIRE(d->layout >= BB_NT && d->layout <= BB_TN, "bb_gemm: bad layout %d", d->layout);
     BB_REQUIRE(d->M >= 0 && d->N >= 0 && d->K >= 0, "bb_gemm: negative dimension");
+    if (d->M == 0 || d->N == 0) return BB_OK;
     BB_REQUIRE(d->A && d->B && d->C, "bb_gemm: null operand");
     BB_REQUIRE(!d->accumulate || d->c_dtype == BB_F32, "bb_gemm: accumulate needs an fp32 C");
     BB_REQUIRE(d->epilogue >= BB_EPI_NONE && d->epilogue <= BB_EPI_RESIDUAL, "bb_gemm: bad epilogue");
@@ -430,7 +431,6 @@ extern "C" int bb_gemm(const bb_gemm_desc* d, void* stream) {
     BB_REQUIRE(d->sA1 % vec == 0 && d->sA2 % vec == 0 && d->sB1 % vec == 0 && d->sB2 % vec == 0,
                "bb_gemm: batch strides of A/B must be multiples of %d", vec);
     BB_REQUIRE(d->lda >= a_contig && d->ldb >= b_contig && d->ldc >= d->N, "bb_gemm: leading dimension too small");
-    if (d->M == 0 || d->N == 0) return BB_OK;
 
     GemmArgs g;
     g.A = d->A; g.B = d->B; g.C = d->C;

@@ -16,9 +16,21 @@ pytestmark = pytest.mark.gpu
 DEV = "cuda:0"
 
 
-def rel_err(got, ref):
+def rel_err(got, ref, floor=1e-30):
+    """fp32 results: max-abs error over the tensor's max; bf16 results (every intermediate is
+    rounded to 8 bits of mantissa between kernels): relative L2 error, the 2e-2 of the spec."""
+    lowp = got.dtype == torch.bfloat16 or getattr(rel_err, "lowp", False)
     got, ref = got.double().cpu(), ref.double().cpu()
-    return float((got - ref).abs().max() / ref.abs().max().clamp_min(1e-30))
+    if lowp:
+        return float((got - ref).norm() / ref.norm().clamp_min(floor * ref.numel() ** 0.5))
+    return float((got - ref).abs().max() / ref.abs().max().clamp_min(floor))
+
+
+def grad_floor(ref_grads):
+    """Some gradients are zero by construction (the key bias: softmax is invariant to a constant
+    added to every key score), so errors are measured against at least 1e-3 of the largest
+    gradient of the stage."""
+    return 1e-3 * max(float(g.abs().max()) for g in ref_grads.values())
 
 
 def build(hidden, heads, ffn, layers_per_stage, stages, stage_id, mb, M, seq, dtype, variant, rl, eager,
@@ -97,13 +109,19 @@ def test_stage_matches_oracle_with_rc(hiplib, variant, klr, dtype):
         engine._clean_pipe_buffers = orig_clean
     t_act = 1e-5 if dtype == torch.float32 else 2e-2
     t_grad = 1e-4 if dtype == torch.float32 else 2e-2
+    if dtype == torch.bfloat16 and variant["activation"] == "relu":
+        # ReLU'(u) is discontinuous: the ~0.2 % of pre-activations closer to zero than their bf16
+        # rounding error take the other branch than in the fp64 oracle, and gradients built from
+        # random-sign terms then differ by sqrt(0.002) ~ 4 % whatever the kernel does
+        t_grad = 6e-2
+    rel_err.lowp = dtype == torch.bfloat16          # fp32 gradient arenas of a bf16 run
     for k in range(M):
         assert rel_err(keep[f"output_{sid}"][k], bufs["out"][(sid, k)].detach().view(mb * seq, hid)) < t_act
         assert rel_err(keep[f"output_{sid + 1}"][k], bufs["out"][(sid + 1, k)].detach().view(mb * seq, hid)) < t_act
         assert rel_err(keep[f"input_grad_{sid}"][k], bufs["sent_grad"][(sid, k)].view(mb * seq, hid)) < t_grad
     ref_grads = st.named_grads(sid)
     for name, g in engine.module.get_named_grad(sid):
-        assert rel_err(g, ref_grads[name]) < t_grad, name
+        assert rel_err(g, ref_grads[name], grad_floor(ref_grads)) < t_grad, name
     # shadow parameters receive no gradient from redundant forwards
     for name, g in engine.module.get_named_grad(sid + 1):
         assert float(g.abs().max()) == 0.0
@@ -183,11 +201,12 @@ def test_failover_promotion_matches_oracle(hiplib, dead_from, dtype):
     with NoStep(engine):
         loss = engine.train_batch()
     assert engine.stage_ids == [sid, sid + 1] and engine.r_stage_ids == []
-    tg = 1e-4 if dtype == torch.float32 else 3e-2
+    tg = 1e-4 if dtype == torch.float32 else 2e-2
+    rel_err.lowp = dtype == torch.bfloat16
     for s_ in (sid, sid + 1):
         ref = st.named_grads(s_)
         for name, g in engine.module.get_named_grad(s_):
-            assert rel_err(g, ref[name]) < tg, (s_, name)
+            assert rel_err(g, ref[name], grad_floor(ref)) < tg, (s_, name)
     assert abs(float(loss) - float(peer.loss) / M) < tg * max(1.0, float(peer.loss) / M)
     # next batch runs as a merged two-stage process from step 0
     q.revive()
@@ -196,6 +215,7 @@ def test_failover_promotion_matches_oracle(hiplib, dead_from, dtype):
 
 
 def test_optimizer_step_matches_oracle(hiplib):
+    rel_err.lowp = False
     hid, heads, ffn, L, S, sid, mb, M, seq = 128, 2, 256, 2, 4, 1, 2, 4, 64
     engine, q = build(hid, heads, ffn, L, S, sid, mb, M, seq, torch.float32, GPT_VARIANT, 0, False)
     st, peer = oracle_for(engine, q, GPT_VARIANT, hid, heads, ffn, L, S, sid, M, 0, False, dtype=torch.float32)
@@ -208,6 +228,8 @@ def test_optimizer_step_matches_oracle(hiplib):
     for name, p in engine.module.get_named_param(sid):
         # Adam's first steps move every weight by ~lr whatever the gradient scale, so compare the
         # movement: |delta - delta_ref| small against lr
+        if name.endswith("linears.1.bias"):
+            continue    # key bias: exact gradient is zero, Adam normalises pure rounding noise to +-lr
         d, dr = (p - before[name]).cpu(), (ref[name].detach() - before[name].cpu())
         assert float((d - dr).abs().max()) < 2e-4, name
         assert float(d.abs().max()) > 1e-4
