@@ -210,14 +210,20 @@ __global__ __launch_bounds__(256) void layernorm_bwd_kernel(int kind, int rows, 
     }
 }
 
-// out[i] += sum_p partial[p * stride + i], p ascending (fixed order)
+// out[i] += sum_p partial[p * stride + i].  One block owns 64 columns; its four waves sum
+// interleaved quarters of the partial rows (p = w, w+4, ...) and the four results are combined
+// in wave order, so the summation order is fixed by nparts alone.
 __global__ __launch_bounds__(256) void reduce_partials_acc_kernel(const float* __restrict__ partial, int nparts,
                                                                   int64_t stride, int n, float* __restrict__ out) {
-    const int i = blockIdx.x * 256 + threadIdx.x;
-    if (i >= n) return;
+    __shared__ float red[4][64];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int i = blockIdx.x * 64 + lane;
     float s = 0.f;
-    for (int p = 0; p < nparts; ++p) s += partial[p * stride + i];
-    out[i] += s;
+    if (i < n)
+        for (int p = wave; p < nparts; p += 4) s += partial[p * stride + i];
+    red[wave][lane] = s;
+    __syncthreads();
+    if (wave == 0 && i < n) out[i] += (red[0][lane] + red[1][lane]) + (red[2][lane] + red[3][lane]);
 }
 
 template <typename T, int IT>
@@ -287,7 +293,7 @@ extern "C" int bb_layernorm_bwd(int dtype, int kind, int rows, int cols, float e
     if (rows == 0) return BB_OK;
     hipStream_t st = (hipStream_t)stream;
     auto finish = [&]() -> int {
-        const int nb = (cols + 255) / 256;
+        const int nb = (cols + 63) / 64;
         hipLaunchKernelGGL(reduce_partials_acc_kernel, dim3(nb), dim3(256), 0, st, workspace, LN_BWD_BLOCKS,
                            (int64_t)2 * cols, cols, dgain);
         hipLaunchKernelGGL(reduce_partials_acc_kernel, dim3(nb), dim3(256), 0, st, workspace + cols, LN_BWD_BLOCKS,
@@ -360,7 +366,7 @@ extern "C" int bb_colsum_acc(int dtype, int rows, int cols, const void* x, int64
         hipLaunchKernelGGL(colsum_partial_kernel<bf16>, grid, dim3(256), 0, st, rows, cols, (const bf16*)x, ldx, workspace);
     else
         hipLaunchKernelGGL(colsum_partial_kernel<float>, grid, dim3(256), 0, st, rows, cols, (const float*)x, ldx, workspace);
-    hipLaunchKernelGGL(reduce_partials_acc_kernel, dim3((cols + 255) / 256), dim3(256), 0, st, workspace, COLSUM_SPLITS,
+    hipLaunchKernelGGL(reduce_partials_acc_kernel, dim3((cols + 63) / 64), dim3(256), 0, st, workspace, COLSUM_SPLITS,
                        (int64_t)cols, cols, out);
     BB_LAUNCH_CHECK();
     return BB_OK;

@@ -366,11 +366,9 @@ enum Bf16Tile { T128x64 = 0, T64x128, T256x256, T256x128, T128x128 };
 static const char* const kBf16TileNames[] = {"128x64", "64x128", "256x256", "256x128", "128x128"};
 
 static Bf16Tile pick_bf16_tile(int M, int N, int64_t batches) {
-    const int64_t t256 = (int64_t)((M + 255) / 256) * ((N + 255) / 256) * batches;
     const int64_t t2128 = (int64_t)((M + 255) / 256) * ((N + 127) / 128) * batches;
     if (N <= 64) return T128x64;
     if (M <= 64) return T64x128;
-    if (M >= 256 && N >= 256 && t256 >= 256) return T256x256;
     if (M >= 256 && N >= 128 && t2128 >= 200) return T256x128;
     return T128x128;
 }
@@ -379,7 +377,6 @@ template <bool TA, bool TB> static int dispatch_bf16(GemmArgs& g, int batches, h
     switch (pick_bf16_tile(g.M, g.N, batches)) {
         case T128x64: return launch_bf16<128, 64, 4, 1, TA, TB>(g, batches, st);
         case T64x128: return launch_bf16<64, 128, 1, 4, TA, TB>(g, batches, st);
-        case T256x256: return launch_bf16<256, 256, 2, 4, TA, TB>(g, batches, st);
         case T256x128: return launch_bf16<256, 128, 4, 2, TA, TB>(g, batches, st);
         default: return launch_bf16<128, 128, 2, 2, TA, TB>(g, batches, st);
     }

@@ -1,0 +1,219 @@
+"""Benchmark of one Bamboo pipeline stage on one MI355X.
+
+A step is one ``train_batch`` of the stage (M micro-batches of own forward+backward through
+the 1F1B instruction stream, the redundant forwards of the shadow layers, one fused Adam
+step) over synthetic inputs that are resident in HBM before the timed region starts.
+
+Prints ONE JSON line: ``value`` = samples/s with redundant computation ON (the configuration
+the metric is quoted on), plus the RC-off rate and the RC overhead, a ``roofline`` object for
+the dominant kernel (measured with HIP events around its launches inside the timed region)
+and a ``cpu_baseline`` object (the CPU oracle timed on a bounded sample of the same workload).
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+CONFIGS = {
+    # name: hidden, heads, ffn, layers per stage, seq, micro-batch, micro-batches, dtype, variant
+    "c1": dict(hidden=768, heads=12, ffn=3072, layers=2, seq=512, mb=4, M=8, dtype="fp32",
+               variant=dict(activation="gelu_tanh", ln="standard", mask="causal"), grad_mode="mse",
+               label="GPT-2-small stage 2+2 layers h768 s512 mb4 M8 fp32"),
+    "c2": dict(hidden=1024, heads=16, ffn=4096, layers=6, seq=1024, mb=8, M=16, dtype="bf16",
+               variant=dict(activation="gelu_tanh", ln="standard", mask="causal"), grad_mode="queue",
+               label="GPT-2-medium stage 6+6 layers h1024 s1024 mb8 M16 bf16"),
+    "c3": dict(hidden=1024, heads=16, ffn=4096, layers=4, seq=512, mb=16, M=12, dtype="bf16",
+               variant=dict(activation="gelu_tanh", ln="standard", mask="key_padding"), grad_mode="queue",
+               key_len_range=(128, 512), label="BERT-large stage 4+4 layers h1024 s512 mb16 M12 bf16"),
+    "c5": dict(hidden=1600, heads=25, ffn=6400, layers=8, seq=1024, mb=4, M=16, dtype="bf16",
+               variant=dict(activation="gelu_tanh", ln="standard", mask="causal"), grad_mode="queue",
+               label="GPT-2-1.5B stage 8+8 layers h1600 s1024 mb4 M16 bf16"),
+}
+STAGES, STAGE_ID = 4, 1
+PEAK_BF16_TFLOPS, PEAK_F32_TFLOPS = 2500.0, 157.3
+
+
+def build_engine(cfg, rc, rc_stream, seed=1138):
+    import torch
+
+    import bamboo_amd
+    from bamboo_amd import LayerSpec, PipelineModule, SeededActivationQueue, TransformerLayer
+    dtype = torch.bfloat16 if cfg["dtype"] == "bf16" else torch.float32
+    specs = [LayerSpec(TransformerLayer, cfg["hidden"], cfg["heads"], cfg["ffn"], **cfg["variant"])
+             for _ in range(cfg["layers"] * STAGES)]
+    model = PipelineModule(specs, num_stages=STAGES, partition_method="uniform", stage_id=STAGE_ID, dtype=dtype,
+                           device="cuda:0")
+    q = SeededActivationQueue((cfg["mb"], cfg["seq"], cfg["hidden"]), dtype, cfg["M"],
+                              stage_ids=[STAGE_ID, STAGE_ID + 1], seed=seed, grad_mode=cfg["grad_mode"],
+                              device="cuda:0", key_len_range=cfg.get("key_len_range"))
+    ds = {"train_micro_batch_size_per_gpu": cfg["mb"], "gradient_accumulation_steps": cfg["M"],
+          "optimizer": {"type": "Adam", "params": {"lr": 1e-3, "betas": [0.9, 0.999], "eps": 1e-8}},
+          "bf16": {"enabled": cfg["dtype"] == "bf16"}}
+    engine, _, _, _ = bamboo_amd.initialize(model=model, config=ds, redundancy_level=1 if rc else 0,
+                                            eager_recovery=rc, activation_queue=q, rc_stream=rc_stream,
+                                            install_signal_handler=False)
+    return engine, q
+
+
+def time_steps(engine, steps, warmup):
+    import torch
+    for _ in range(warmup):
+        engine.train_batch()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        engine.train_batch()
+    torch.cuda.synchronize()
+    return (time.perf_counter() - t0) / steps
+
+
+class GemmProbe:
+    """Brackets every dense GEMM launch with HIP events on the launch stream."""
+
+    def __init__(self):
+        self.records = []
+
+    def __call__(self, desc, launch):
+        import torch
+
+        from bamboo_amd import hip
+        name = hip.gemm_variant(desc)
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        launch()
+        e1.record()
+        self.records.append((name, 2.0 * desc.M * desc.N * desc.K, e0, e1))
+
+    def summary(self):
+        agg = {}
+        for name, flops, e0, e1 in self.records:
+            a = agg.setdefault(name, [0, 0.0, 0.0])
+            a[0] += 1
+            a[1] += flops
+            a[2] += e0.elapsed_time(e1) * 1e-3
+        return agg
+
+
+def cpu_baseline(cfg, threads):
+    """Oracle stage on the host: one micro-batch of own forward+backward and one redundant
+    forward at the benchmark's shapes (fp32), extrapolated to the batch."""
+    import torch
+
+    from oracle import layers as ol
+    from oracle.stage import OracleStage
+    torch.set_num_threads(threads)
+    ocfg = ol.TransformerCfg(hidden=cfg["hidden"], heads=cfg["heads"], ffn=cfg["ffn"], **cfg["variant"])
+    parts = [i * cfg["layers"] for i in range(STAGES + 1)]
+    st = OracleStage(ocfg, parts, STAGE_ID, cfg["M"], dtype=torch.float32, redundancy_level=1, eager=True)
+    g = torch.Generator().manual_seed(1)
+    x = torch.randn(cfg["mb"], cfg["seq"], cfg["hidden"], generator=g)
+    dy = torch.randn(cfg["mb"], cfg["seq"], cfg["hidden"], generator=g)
+    kl = None
+    if cfg["variant"]["mask"] == "key_padding":
+        kl = torch.randint(cfg["key_len_range"][0], cfg["key_len_range"][1] + 1, (cfg["mb"],), generator=g)
+    t0 = time.perf_counter()
+    xin = x.clone().requires_grad_(True)
+    out = st.forward(xin, STAGE_ID, kl)
+    torch.autograd.backward(out, dy)
+    t_own = time.perf_counter() - t0
+    t0 = time.perf_counter()
+    with torch.enable_grad():
+        st.forward(out.detach().requires_grad_(True), STAGE_ID + 1, kl)
+    t_rc = time.perf_counter() - t0
+    M = cfg["M"]
+    samples = cfg["mb"] * M
+    off, on = M * t_own, M * (t_own + t_rc)
+    return {"value": samples / on, "unit": "samples/s", "cores": threads, "kind": "port",
+            "rc_off_value": samples / off, "rc_overhead_pct": 100.0 * (on - off) / off,
+            "sample": f"1 micro-batch own fwd+bwd ({t_own:.2f}s) + 1 redundant fwd ({t_rc:.2f}s), fp32, "
+                      f"extrapolated x{M} micro-batches; optimizer step not included"}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=5)
+    ap.add_argument("--warmup", type=int, default=2)
+    ap.add_argument("--config", default="c2", choices=sorted(CONFIGS))
+    ap.add_argument("--rc-stream", type=int, default=1, help="issue redundant forwards on a second HIP stream")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-probe", action="store_true", help="do not bracket GEMM launches with events")
+    ap.add_argument("--skip-rc-off", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py measures ONE pipeline stage on ONE GPU; --gpus N>1 is not part of this build", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+
+    from bamboo_amd import hip
+    cfg = CONFIGS[args.config]
+    samples = cfg["mb"] * cfg["M"]
+
+    t_off = None
+    if not args.skip_rc_off:
+        engine, q = build_engine(cfg, rc=False, rc_stream=False)
+        t_off = time_steps(engine, args.steps, args.warmup)
+        del engine, q
+        torch.cuda.empty_cache()
+
+    engine, q = build_engine(cfg, rc=True, rc_stream=bool(args.rc_stream))
+    probe = None
+    for _ in range(args.warmup):
+        engine.train_batch()
+    torch.cuda.synchronize()
+    if not args.no_probe:
+        probe = GemmProbe()
+        hip.gemm_hook = probe
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        engine.train_batch()
+    torch.cuda.synchronize()
+    t_on = (time.perf_counter() - t0) / args.steps
+    hip.gemm_hook = None
+
+    layer = engine.module.func_buckets[STAGE_ID][0]
+    fwd_flops = layer.flops_fwd(cfg["mb"], cfg["seq"]) * cfg["layers"]
+    own_flops, rc_flops = 3 * fwd_flops * cfg["M"], fwd_flops * cfg["M"]
+
+    roofline = None
+    if probe is not None:
+        agg = probe.summary()
+        name, (count, flops, secs) = max(agg.items(), key=lambda kv: kv[1][2])
+        peak = PEAK_BF16_TFLOPS if cfg["dtype"] == "bf16" else PEAK_F32_TFLOPS
+        achieved = flops / secs / 1e12
+        roofline = {"bound": "mfma", "achieved": round(achieved, 2), "peak": peak, "unit": "TFLOP/s",
+                    "frac": round(achieved / peak, 4), "traffic": None, "kernel": f"gemm_{name}",
+                    "launches": count, "avg_launch_us": round(secs / count * 1e6, 2),
+                    "avg_launch_gflop": round(flops / count / 1e9, 3),
+                    "all_gemm_variants": {k: {"launches": v[0], "tflops": round(v[1] / v[2] / 1e12, 2),
+                                              "time_s": round(v[2], 4)} for k, v in agg.items()}}
+
+    out = {
+        "metric": "stage samples/s RC on vs off, RC overhead %, MFMA util % (GPT-2-med stage)",
+        "value": round(samples / t_on, 3), "unit": "samples/s", "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": round(t_on * 1e3, 3), "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": cfg["dtype"], "data": "synthetic",
+        "config": {"workload": cfg["label"], "stage": f"{STAGE_ID} of {STAGES}", "redundancy_level": 1,
+                   "eager_recovery": True, "rc_stream": bool(args.rc_stream), "samples_per_step": samples,
+                   "attention": "dense scores materialised (unfused), flops counted dense"},
+        "rc_on_samples_per_s": round(samples / t_on, 3),
+        "rc_off_samples_per_s": None if t_off is None else round(samples / t_off, 3),
+        "rc_overhead_pct": None if t_off is None else round(100.0 * (t_on - t_off) / t_off, 2),
+        "stage_tflops_rc_on": round((own_flops + rc_flops) / t_on / 1e12, 2),
+        "stage_tflops_rc_off": None if t_off is None else round(own_flops / t_off / 1e12, 2),
+        "roofline": roofline,
+    }
+    if not args.no_cpu_baseline:
+        threads = min(os.cpu_count() or 1, 16)
+        out["cpu_baseline"] = cpu_baseline(cfg, threads)
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()
