@@ -12,6 +12,8 @@
 // store, so the MFMA side never changes.
 #include "common.h"
 
+#include <utility>
+
 struct GemmArgs {
     const void* A; const void* B; void* C;
     const void* bias; const void* aux_in; void* aux_out; const void* resid;
@@ -62,6 +64,49 @@ __device__ __forceinline__ void epilogue_elem(const GemmArgs& g, int64_t coff, i
     } else {
         Elem<T>::store((T*)g.C + ci, v);
     }
+}
+
+// Vector epilogue for bf16 operands: 8 consecutive columns of one row (n % 8 == 0, n + 8 <= N).
+__device__ __forceinline__ void epilogue_vec8(const GemmArgs& g, int64_t coff, int m, int n, float (&v)[8]) {
+    const int64_t ci = coff + (int64_t)m * g.ldc + n;
+    const int64_t xi = coff + (int64_t)m * g.ldaux + n;
+    if (g.bias) {
+        float b[8];
+        load_vec((const bf16*)g.bias + n, b);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) v[e] += b[e];
+    }
+    if (g.epilogue == BB_EPI_ACT) {
+        if (g.aux_out) store_vec((bf16*)g.aux_out + xi, v);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) v[e] = act_f(v[e], g.act);
+    } else if (g.epilogue == BB_EPI_DACT) {
+        float u[8];
+        load_vec((const bf16*)g.aux_in + xi, u);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) v[e] *= dact_f(u[e], g.act);
+    } else if (g.epilogue == BB_EPI_RESIDUAL) {
+        float r[8];
+        load_vec((const bf16*)g.resid + xi, r);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) v[e] += r[e];
+    }
+    if (g.c_f32) {
+        float* c = (float*)g.C + ci;
+        f32x4 lo = {v[0], v[1], v[2], v[3]}, hi = {v[4], v[5], v[6], v[7]};
+        if (g.accumulate) {
+            lo += *(const f32x4*)c;
+            hi += *(const f32x4*)(c + 4);
+        }
+        *(f32x4*)c = lo;
+        *(f32x4*)(c + 4) = hi;
+    } else {
+        store_vec((bf16*)g.C + ci, v);
+    }
+}
+
+template <typename F, int... Is> __device__ __forceinline__ void static_for(F&& f, std::integer_sequence<int, Is...>) {
+    (f(std::integral_constant<int, Is>{}), ...);
 }
 
 // =========================================================================================
@@ -235,6 +280,237 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_bf16_kernel(const GemmArgs g
 }
 
 // =========================================================================================
+// bf16 kernel, DMA generation: tiles go global -> LDS directly (global_load_lds_dwordx4, no
+// VGPR staging) through a 4-stage ring of 32-wide k-tiles, MFMA fragments are double-buffered
+// in registers so LDS reads of tile t+1 overlap the MFMAs of tile t.
+//
+// LDS tile formats (one wave-instruction always fills 1024 contiguous bytes, 16 B per lane):
+//   KC operand (memory rows are k-contiguous): [rows][32 k], 64 B per row = 4 chunks of 16 B,
+//       chunk c of row r at slot c ^ ((r >> 2) & 3); fragments by ds_read_b128.
+//   KM operand (memory is k-major, rows contiguous): [32 k][rows], chunk c of k-row k at slot
+//       c ^ (4 * (k & 3)); fragments by two ds_read_b64_tr_b16 (the hardware transposes a
+//       4k x 16row block across 16 lanes: lane j reads row k0 + j/4, cols 4*(j%4)..+3 and
+//       receives column j, k0..k0+3).
+// Rows beyond M / N are clamped to the last valid row (their results are never stored);
+// K must be a multiple of 32.
+// =========================================================================================
+typedef __attribute__((address_space(3))) void lds_ptr_t;
+typedef const __attribute__((address_space(1))) void gbl_ptr_t;
+typedef __attribute__((ext_vector_type(4))) short s16x4;
+
+template <int N> __device__ __forceinline__ void wait_vmcnt_lgkm0() {
+    // s_waitcnt vmcnt(N) lgkmcnt(0): vmcnt[3:0] | expcnt(7) << 4 | lgkmcnt << 8 | vmcnt[5:4] << 14
+    __builtin_amdgcn_s_waitcnt((N & 15) | (7 << 4) | (0 << 8) | ((N >> 4) << 14));
+}
+
+template <int BR, bool KM> struct DmaOperand {
+    static constexpr int BYTES = BR * 32 * 2;
+    static constexpr int ROUNDS = BYTES / 4096;  // instructions per thread per k-tile (4 waves)
+    const bf16* src[ROUNDS];
+    int64_t step;  // elements to advance per k-tile
+
+    __device__ __forceinline__ void init(const bf16* base, int64_t ld, int row0, int rows, int tid) {
+        const int lane = tid & 63, wave = tid >> 6;
+#pragma unroll
+        for (int i = 0; i < ROUNDS; ++i) {
+            const int q = i * 4 + wave;
+            if constexpr (!KM) {
+                const int r = q * 16 + (lane >> 2);
+                const int c = (lane & 3) ^ ((r >> 2) & 3);
+                const int gr = min(row0 + r, rows - 1);
+                src[i] = base + (int64_t)gr * ld + c * 8;
+            } else {
+                constexpr int CPR = BR / 8, RPI = 64 / CPR;
+                const int k = q * RPI + lane / CPR;
+                const int c = (lane % CPR) ^ (4 * (k & 3));
+                const int gc = min(row0 + c * 8, rows - 8);
+                src[i] = base + (int64_t)k * ld + gc;
+            }
+        }
+        step = KM ? 32 * ld : 32;
+    }
+    __device__ __forceinline__ void issue(unsigned char* tile, int wave) {
+#pragma unroll
+        for (int i = 0; i < ROUNDS; ++i) {
+            __builtin_amdgcn_global_load_lds((gbl_ptr_t*)src[i], (lds_ptr_t*)(tile + (i * 4 + wave) * 1024), 16, 0, 0);
+            src[i] += step;
+        }
+    }
+};
+
+// per-lane fragment offsets (bytes inside an operand tile) and the fragment fetch
+template <int BR, int T, bool KM> struct FragReader {
+    int off[KM ? T : 1];
+    int sw, hi;
+    __device__ __forceinline__ void init(int wbase, int lane) {
+        hi = lane >> 5;
+        if constexpr (!KM) {
+            sw = ((lane & 31) >> 2) & 3;
+            off[0] = (wbase + (lane & 31)) * 64;
+        } else {
+            const int j4 = (lane & 15) >> 2;
+            const int lo = ((lane >> 4) & 1) * 2 + ((lane & 3) >> 1);
+            const int within = (lane & 1) * 4;  // element offset inside the 16-byte chunk
+            sw = 0;
+#pragma unroll
+            for (int t = 0; t < T; ++t) {
+                const int c4 = ((wbase >> 5) + t) ^ j4;  // chunk-of-four index after the swizzle
+                off[t] = (hi * 8 + j4) * (BR * 2) + ((c4 * 4 + lo) << 4) + within * 2;
+            }
+        }
+    }
+    __device__ __forceinline__ bf16x8 load(const unsigned char* tile, int t, int ks) const {
+        if constexpr (!KM) {
+            return *(const bf16x8*)(tile + off[0] + t * 2048 + (((ks * 2 + hi) ^ sw) << 4));
+        } else {
+            const unsigned char* p = tile + off[t] + ks * 16 * (BR * 2);
+            s16x4 lo4 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4*)(p));
+            s16x4 hi4 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4*)(p + 4 * (BR * 2)));
+            typedef __attribute__((ext_vector_type(8))) short s16x8;
+            s16x8 v = __builtin_shufflevector(lo4, hi4, 0, 1, 2, 3, 4, 5, 6, 7);
+            return __builtin_bit_cast(bf16x8, v);
+        }
+    }
+};
+
+template <int BM, int BN, int WM, int WN, bool AKM, bool BKM>
+__global__ __launch_bounds__(256) void gemm_bf16_dma_kernel(const GemmArgs g) {
+    static_assert(WM * WN == 4, "four waves per block");
+    constexpr int STAGES = 4;
+    constexpr int WTM = BM / WM, WTN = BN / WN, TM = WTM / 32, TN = WTN / 32;
+    using OpA = DmaOperand<BM, AKM>;
+    using OpB = DmaOperand<BN, BKM>;
+    constexpr int STAGE_BYTES = OpA::BYTES + OpB::BYTES;
+    constexpr int LOADS = OpA::ROUNDS + OpB::ROUNDS;
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wm = wave / WN, wn = wave % WN;
+    int tile_m, tile_n;
+    tile_coords(blockIdx.x, g.tiles_m, g.tiles_n, tile_m, tile_n);
+    const int m0 = tile_m * BM, n0 = tile_n * BN;
+    const int b1 = blockIdx.z / g.nb2, b2 = blockIdx.z % g.nb2;
+    const bf16* A = (const bf16*)g.A + b1 * g.sA1 + b2 * g.sA2;
+    const bf16* B = (const bf16*)g.B + b1 * g.sB1 + b2 * g.sB2;
+    const int64_t coff = b1 * g.sC1 + b2 * g.sC2;
+
+    OpA opa;
+    OpB opb;
+    opa.init(A, g.lda, m0, g.M, tid);
+    opb.init(B, g.ldb, n0, g.N, tid);
+    FragReader<BM, TM, AKM> fa;
+    FragReader<BN, TN, BKM> fb;
+    fa.init(wm * WTM, lane);
+    fb.init(wn * WTN, lane);
+
+    f32x16 acc[TM][TN];
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+
+    struct Frags {
+        bf16x8 a[2][TM], b[2][TN];
+    };
+    Frags f0, f1;
+    const int KT = g.K / 32;
+
+    auto issue_tile = [&](int kt) {
+        unsigned char* st = smem + (kt & (STAGES - 1)) * STAGE_BYTES;
+        opa.issue(st, wave);
+        opb.issue(st + OpA::BYTES, wave);
+    };
+    auto load_frags = [&](int kt, Frags& f) {
+        const unsigned char* st = smem + (kt & (STAGES - 1)) * STAGE_BYTES;
+#pragma unroll
+        for (int ks = 0; ks < 2; ++ks) {
+#pragma unroll
+            for (int i = 0; i < TM; ++i) f.a[ks][i] = fa.load(st, i, ks);
+#pragma unroll
+            for (int j = 0; j < TN; ++j) f.b[ks][j] = fb.load(st + OpA::BYTES, j, ks);
+        }
+    };
+    auto mfma_step = [&](const Frags& f, int ks) {
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+            for (int j = 0; j < TN; ++j)
+                acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(f.a[ks][i], f.b[ks][j], acc[i][j], 0, 0, 0);
+    };
+    // Steady state is branch-free: a tile is issued every iteration (past the end of K the
+    // sources stop advancing, so the last tile is fetched again into a stage nobody reads),
+    // hence exactly two newer tiles are in flight whenever a wave waits for tile kt + 1.
+    auto sync_tile = [&]() {
+        asm volatile("" ::: "memory");
+        wait_vmcnt_lgkm0<2 * LOADS>();
+        __builtin_amdgcn_s_barrier();
+        asm volatile("" ::: "memory");
+    };
+    auto body = [&](int kt, Frags& cur, Frags& nxt) {
+        if (kt + 4 >= KT) {
+            opa.step = 0;
+            opb.step = 0;
+        }
+        issue_tile(kt + 3);
+        mfma_step(cur, 0);
+        sync_tile();
+        load_frags(kt + 1, nxt);
+        mfma_step(cur, 1);
+    };
+
+    // prologue: tiles 0..2 (clamped to the last tile when K is short)
+#pragma unroll
+    for (int t = 0; t < 3; ++t) {
+        if (t + 1 >= KT) {
+            opa.step = 0;
+            opb.step = 0;
+        }
+        issue_tile(t);
+    }
+    sync_tile();
+    load_frags(0, f0);
+    int kt = 0;
+    for (; kt + 1 < KT; kt += 2) {
+        body(kt, f0, f1);
+        body(kt + 1, f1, f0);
+    }
+    if (kt < KT) body(kt, f0, f1);
+
+    // Epilogue through LDS: every wave parks one 32x32 accumulator tile at a time in a private
+    // [32][36] fp32 patch, then lane l takes 16 consecutive columns of row l/2 so that global
+    // loads and stores are 16-byte vectors along rows.
+    __syncthreads();
+    float* patch = (float*)smem + wave * (32 * 36);
+    const int prow = lane >> 1, pcol = (lane & 1) * 16;
+    static_for(
+        [&](auto idx) {
+            constexpr int i = decltype(idx)::value / TN, j = decltype(idx)::value % TN;
+#pragma unroll
+            for (int r = 0; r < 16; ++r)
+                patch[(8 * (r >> 2) + 4 * (lane >> 5) + (r & 3)) * 36 + (lane & 31)] = acc[i][j][r] * g.alpha;
+            asm volatile("" ::: "memory");
+            const int m = m0 + wm * WTM + i * 32 + prow;
+            const int n = n0 + wn * WTN + j * 32 + pcol;
+#pragma unroll
+            for (int h = 0; h < 2; ++h) {
+                float v[8];
+                const f32x4 lo = *(const f32x4*)(patch + prow * 36 + pcol + h * 8);
+                const f32x4 hi = *(const f32x4*)(patch + prow * 36 + pcol + h * 8 + 4);
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    v[e] = lo[e];
+                    v[4 + e] = hi[e];
+                }
+                if (m < g.M && n + h * 8 < g.N) epilogue_vec8(g, coff, m, n + h * 8, v);
+            }
+            asm volatile("" ::: "memory");
+        },
+        std::make_integer_sequence<int, TM * TN>{});
+}
+
+// =========================================================================================
 // fp32 kernel: 128x128x16 tiles, 4 waves (2x2), LDS k-major with padded rows.
 // =========================================================================================
 template <bool TA, bool TB>
@@ -373,7 +649,42 @@ static Bf16Tile pick_bf16_tile(int M, int N, int64_t batches) {
     return T128x128;
 }
 
+template <int BM, int BN, int WM, int WN, bool AKM, bool BKM>
+static int launch_bf16_dma(GemmArgs& g, int batches, hipStream_t st) {
+    constexpr int smem = 4 * (BM + BN) * 32 * 2;
+    auto kern = gemm_bf16_dma_kernel<BM, BN, WM, WN, AKM, BKM>;
+    static bool configured = false;
+    if (!configured) {
+        BB_HIP_CHECK(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, smem));
+        configured = true;
+    }
+    g.tiles_m = (g.M + BM - 1) / BM;
+    g.tiles_n = (g.N + BN - 1) / BN;
+    dim3 grid(g.tiles_m * g.tiles_n, 1, batches);
+    hipLaunchKernelGGL(kern, grid, dim3(256), smem, st, g);
+    BB_LAUNCH_CHECK();
+    return BB_OK;
+}
+
+// DMA kernels need K % 32 == 0 and at least one full vector of rows; tile by problem size
+enum DmaTile { D_NONE = 0, D256x256, D256x128, D128x128 };
+static const char* const kDmaTileNames[] = {"", "dma256x256", "dma256x128", "dma128x128"};
+static DmaTile pick_dma_tile(int M, int N, int K, int64_t batches) {
+    if (K % 32 != 0 || K < 64 || M < 128 || N < 128 || N % 8 != 0) return D_NONE;
+    const int64_t t256 = (int64_t)((M + 255) / 256) * ((N + 255) / 256) * batches;
+    const int64_t t2128 = (int64_t)((M + 255) / 256) * ((N + 127) / 128) * batches;
+    if (M >= 256 && N >= 256 && t256 >= 256) return D256x256;
+    if (M >= 256 && t2128 >= 256) return D256x128;
+    return D128x128;
+}
+
 template <bool TA, bool TB> static int dispatch_bf16(GemmArgs& g, int batches, hipStream_t st) {
+    switch (pick_dma_tile(g.M, g.N, g.K, batches)) {
+        case D256x256: return launch_bf16_dma<256, 256, 2, 2, TA, TB>(g, batches, st);
+        case D256x128: return launch_bf16_dma<256, 128, 2, 2, TA, TB>(g, batches, st);
+        case D128x128: return launch_bf16_dma<128, 128, 2, 2, TA, TB>(g, batches, st);
+        default: break;
+    }
     switch (pick_bf16_tile(g.M, g.N, batches)) {
         case T128x64: return launch_bf16<128, 64, 4, 1, TA, TB>(g, batches, st);
         case T64x128: return launch_bf16<64, 128, 1, 4, TA, TB>(g, batches, st);
@@ -396,8 +707,11 @@ extern "C" int bb_gemm_variant(const bb_gemm_desc* d, char* out, int out_len) {
     static const char* const layouts[] = {"nt", "nn", "tn"};
     BB_REQUIRE(d->layout >= BB_NT && d->layout <= BB_TN, "bb_gemm_variant: bad layout %d", d->layout);
     const int64_t batches = (int64_t)(d->nb1 > 0 ? d->nb1 : 1) * (d->nb2 > 0 ? d->nb2 : 1);
-    if (d->dtype == BB_BF16)
-        snprintf(out, out_len, "bf16_%s_%s", layouts[d->layout], kBf16TileNames[pick_bf16_tile(d->M, d->N, batches)]);
+    if (d->dtype == BB_BF16) {
+        const DmaTile dt = pick_dma_tile(d->M, d->N, d->K, batches);
+        snprintf(out, out_len, "bf16_%s_%s", layouts[d->layout],
+                 dt != D_NONE ? kDmaTileNames[dt] : kBf16TileNames[pick_bf16_tile(d->M, d->N, batches)]);
+    }
     else
         snprintf(out, out_len, "f32_%s_128x128", layouts[d->layout]);
     return BB_OK;
