@@ -12,6 +12,7 @@
 // store, so the MFMA side never changes.
 #include "common.h"
 
+#include <stdlib.h>
 #include <utility>
 
 struct GemmArgs {
@@ -303,9 +304,10 @@ template <int N> __device__ __forceinline__ void wait_vmcnt_lgkm0() {
     __builtin_amdgcn_s_waitcnt((N & 15) | (7 << 4) | (0 << 8) | ((N >> 4) << 14));
 }
 
-template <int BR, bool KM> struct DmaOperand {
+template <int BR, bool KM, int NW> struct DmaOperand {
     static constexpr int BYTES = BR * 32 * 2;
-    static constexpr int ROUNDS = BYTES / 4096;  // instructions per thread per k-tile (4 waves)
+    static constexpr int ROUNDS = BYTES / (1024 * NW);  // instructions per thread per k-tile
+    static_assert(ROUNDS >= 1, "tile too small for the block");
     const bf16* src[ROUNDS];
     int64_t step;  // elements to advance per k-tile
 
@@ -313,7 +315,7 @@ template <int BR, bool KM> struct DmaOperand {
         const int lane = tid & 63, wave = tid >> 6;
 #pragma unroll
         for (int i = 0; i < ROUNDS; ++i) {
-            const int q = i * 4 + wave;
+            const int q = i * NW + wave;
             if constexpr (!KM) {
                 const int r = q * 16 + (lane >> 2);
                 const int c = (lane & 3) ^ ((r >> 2) & 3);
@@ -332,7 +334,7 @@ template <int BR, bool KM> struct DmaOperand {
     __device__ __forceinline__ void issue(unsigned char* tile, int wave) {
 #pragma unroll
         for (int i = 0; i < ROUNDS; ++i) {
-            __builtin_amdgcn_global_load_lds((gbl_ptr_t*)src[i], (lds_ptr_t*)(tile + (i * 4 + wave) * 1024), 16, 0, 0);
+            __builtin_amdgcn_global_load_lds((gbl_ptr_t*)src[i], (lds_ptr_t*)(tile + (i * NW + wave) * 1024), 16, 0, 0);
             src[i] += step;
         }
     }
@@ -373,13 +375,13 @@ template <int BR, int T, bool KM> struct FragReader {
     }
 };
 
-template <int BM, int BN, int WM, int WN, bool AKM, bool BKM>
-__global__ __launch_bounds__(256) void gemm_bf16_dma_kernel(const GemmArgs g) {
-    static_assert(WM * WN == 4, "four waves per block");
-    constexpr int STAGES = 4;
+template <int BM, int BN, int WM, int WN, bool AKM, bool BKM, bool DB, int STAGES>
+__device__ __forceinline__ void gemm_bf16_dma_body(const GemmArgs& g, const int block_id, const int batch_id) {
+    constexpr int NW = WM * WN;
+    static_assert(STAGES >= 3, "the ring needs one stage being read, one landing, one in flight");
     constexpr int WTM = BM / WM, WTN = BN / WN, TM = WTM / 32, TN = WTN / 32;
-    using OpA = DmaOperand<BM, AKM>;
-    using OpB = DmaOperand<BN, BKM>;
+    using OpA = DmaOperand<BM, AKM, NW>;
+    using OpB = DmaOperand<BN, BKM, NW>;
     constexpr int STAGE_BYTES = OpA::BYTES + OpB::BYTES;
     constexpr int LOADS = OpA::ROUNDS + OpB::ROUNDS;
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
@@ -387,9 +389,9 @@ __global__ __launch_bounds__(256) void gemm_bf16_dma_kernel(const GemmArgs g) {
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wm = wave / WN, wn = wave % WN;
     int tile_m, tile_n;
-    tile_coords(blockIdx.x, g.tiles_m, g.tiles_n, tile_m, tile_n);
+    tile_coords(block_id, g.tiles_m, g.tiles_n, tile_m, tile_n);
     const int m0 = tile_m * BM, n0 = tile_n * BN;
-    const int b1 = blockIdx.z / g.nb2, b2 = blockIdx.z % g.nb2;
+    const int b1 = batch_id / g.nb2, b2 = batch_id % g.nb2;
     const bf16* A = (const bf16*)g.A + b1 * g.sA1 + b2 * g.sA2;
     const bf16* B = (const bf16*)g.B + b1 * g.sB1 + b2 * g.sB2;
     const int64_t coff = b1 * g.sC1 + b2 * g.sC2;
@@ -417,13 +419,16 @@ __global__ __launch_bounds__(256) void gemm_bf16_dma_kernel(const GemmArgs g) {
     Frags f0, f1;
     const int KT = g.K / 32;
 
-    auto issue_tile = [&](int kt) {
-        unsigned char* st = smem + (kt & (STAGES - 1)) * STAGE_BYTES;
+    // ring positions: tile t lives in stage t % STAGES
+    int issue_stage = 0, read_stage = 0;
+    auto issue_tile = [&]() {
+        unsigned char* st = smem + issue_stage * STAGE_BYTES;
         opa.issue(st, wave);
         opb.issue(st + OpA::BYTES, wave);
+        issue_stage = issue_stage + 1 == STAGES ? 0 : issue_stage + 1;
     };
-    auto load_frags = [&](int kt, Frags& f) {
-        const unsigned char* st = smem + (kt & (STAGES - 1)) * STAGE_BYTES;
+    auto load_frags = [&](Frags& f) {
+        const unsigned char* st = smem + read_stage * STAGE_BYTES;
 #pragma unroll
         for (int ks = 0; ks < 2; ++ks) {
 #pragma unroll
@@ -431,6 +436,7 @@ __global__ __launch_bounds__(256) void gemm_bf16_dma_kernel(const GemmArgs g) {
 #pragma unroll
             for (int j = 0; j < TN; ++j) f.b[ks][j] = fb.load(st + OpA::BYTES, j, ks);
         }
+        read_stage = read_stage + 1 == STAGES ? 0 : read_stage + 1;
     };
     auto mfma_step = [&](const Frags& f, int ks) {
 #pragma unroll
@@ -441,42 +447,56 @@ __global__ __launch_bounds__(256) void gemm_bf16_dma_kernel(const GemmArgs g) {
     };
     // Steady state is branch-free: a tile is issued every iteration (past the end of K the
     // sources stop advancing, so the last tile is fetched again into a stage nobody reads),
-    // hence exactly two newer tiles are in flight whenever a wave waits for tile kt + 1.
+    // hence exactly STAGES-2 newer tiles are in flight whenever a wave waits for the next tile.
     auto sync_tile = [&]() {
         asm volatile("" ::: "memory");
-        wait_vmcnt_lgkm0<2 * LOADS>();
+        wait_vmcnt_lgkm0<(STAGES - 2) * LOADS>();
         __builtin_amdgcn_s_barrier();
         asm volatile("" ::: "memory");
     };
-    auto body = [&](int kt, Frags& cur, Frags& nxt) {
-        if (kt + 4 >= KT) {
+    auto stop_at_end = [&](int next_tile) {
+        if (next_tile >= KT) {
             opa.step = 0;
             opb.step = 0;
         }
-        issue_tile(kt + 3);
-        mfma_step(cur, 0);
-        sync_tile();
-        load_frags(kt + 1, nxt);
-        mfma_step(cur, 1);
     };
 
-    // prologue: tiles 0..2 (clamped to the last tile when K is short)
+    // prologue: tiles 0..STAGES-2 (clamped to the last tile when K is short)
 #pragma unroll
-    for (int t = 0; t < 3; ++t) {
-        if (t + 1 >= KT) {
-            opa.step = 0;
-            opb.step = 0;
-        }
-        issue_tile(t);
+    for (int t = 0; t < STAGES - 1; ++t) {
+        stop_at_end(t + 1);
+        issue_tile();
     }
     sync_tile();
-    load_frags(0, f0);
-    int kt = 0;
-    for (; kt + 1 < KT; kt += 2) {
-        body(kt, f0, f1);
-        body(kt + 1, f1, f0);
+    if constexpr (DB) {
+        // fragments of tile kt+1 are fetched while the second half of tile kt is multiplied,
+        // into the other register set
+        auto body = [&](int kt, Frags& cur, Frags& nxt) {
+            stop_at_end(kt + STAGES);
+            issue_tile();
+            mfma_step(cur, 0);
+            sync_tile();
+            load_frags(nxt);
+            mfma_step(cur, 1);
+        };
+        load_frags(f0);
+        int kt = 0;
+        for (; kt + 1 < KT; kt += 2) {
+            body(kt, f0, f1);
+            body(kt + 1, f1, f0);
+        }
+        if (kt < KT) body(kt, f0, f1);
+    } else {
+        // single fragment set: other resident waves cover LDS latency and barrier waits
+        for (int kt = 0; kt < KT; ++kt) {
+            stop_at_end(kt + STAGES);
+            issue_tile();
+            load_frags(f0);
+            mfma_step(f0, 0);
+            mfma_step(f0, 1);
+            sync_tile();
+        }
     }
-    if (kt < KT) body(kt, f0, f1);
 
     // Epilogue through LDS: every wave parks one 32x32 accumulator tile at a time in a private
     // [32][36] fp32 patch, then lane l takes 16 consecutive columns of row l/2 so that global
@@ -508,6 +528,26 @@ __global__ __launch_bounds__(256) void gemm_bf16_dma_kernel(const GemmArgs g) {
             asm volatile("" ::: "memory");
         },
         std::make_integer_sequence<int, TM * TN>{});
+}
+
+template <int BM, int BN, int WM, int WN, bool AKM, bool BKM, bool DB, int STAGES>
+__global__ __launch_bounds__(WM* WN * 64) void gemm_bf16_dma_kernel(const GemmArgs g) {
+    gemm_bf16_dma_body<BM, BN, WM, WN, AKM, BKM, DB, STAGES>(g, blockIdx.x, blockIdx.z);
+}
+
+// Several independent problems of one kind in a single launch (the four weight-gradient GEMMs
+// of a transformer layer: each alone has too few output tiles to fill 256 CUs).
+constexpr int GROUP_MAX = 8;
+struct GroupedArgs {
+    GemmArgs p[GROUP_MAX];
+    int first_block[GROUP_MAX + 1];
+    int count;
+};
+template <int BM, int BN, int WM, int WN, bool AKM, bool BKM, bool DB, int STAGES>
+__global__ __launch_bounds__(WM* WN * 64) void gemm_bf16_dma_grouped_kernel(const GroupedArgs G) {
+    int pi = 0;
+    while (pi + 1 < G.count && (int)blockIdx.x >= G.first_block[pi + 1]) ++pi;
+    gemm_bf16_dma_body<BM, BN, WM, WN, AKM, BKM, DB, STAGES>(G.p[pi], blockIdx.x - G.first_block[pi], 0);
 }
 
 // =========================================================================================
@@ -649,10 +689,10 @@ static Bf16Tile pick_bf16_tile(int M, int N, int64_t batches) {
     return T128x128;
 }
 
-template <int BM, int BN, int WM, int WN, bool AKM, bool BKM>
+template <int BM, int BN, int WM, int WN, bool AKM, bool BKM, bool DB, int STAGES = 4>
 static int launch_bf16_dma(GemmArgs& g, int batches, hipStream_t st) {
-    constexpr int smem = 4 * (BM + BN) * 32 * 2;
-    auto kern = gemm_bf16_dma_kernel<BM, BN, WM, WN, AKM, BKM>;
+    constexpr int smem = STAGES * (BM + BN) * 32 * 2;
+    auto kern = gemm_bf16_dma_kernel<BM, BN, WM, WN, AKM, BKM, DB, STAGES>;
     static bool configured = false;
     if (!configured) {
         BB_HIP_CHECK(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, smem));
@@ -661,28 +701,49 @@ static int launch_bf16_dma(GemmArgs& g, int batches, hipStream_t st) {
     g.tiles_m = (g.M + BM - 1) / BM;
     g.tiles_n = (g.N + BN - 1) / BN;
     dim3 grid(g.tiles_m * g.tiles_n, 1, batches);
-    hipLaunchKernelGGL(kern, grid, dim3(256), smem, st, g);
+    hipLaunchKernelGGL(kern, grid, dim3(WM * WN * 64), smem, st, g);
     BB_LAUNCH_CHECK();
     return BB_OK;
 }
 
 // DMA kernels need K % 32 == 0 and at least one full vector of rows; tile by problem size
-enum DmaTile { D_NONE = 0, D256x256, D256x128, D128x128 };
-static const char* const kDmaTileNames[] = {"", "dma256x256", "dma256x128", "dma128x128"};
+enum DmaTile { D_NONE = 0, D256x256, D256x128, D128x128, D_OFF, D256x256w8, D256x128w8, D256x256w8db, D256x128w8db,
+               D256x128w8s3, D128x128s3 };
+static const char* const kDmaTileNames[] = {"", "dma256x256", "dma256x128", "dma128x128", "", "dma256x256w8", "dma256x128w8",
+                                            "dma256x256w8db", "dma256x128w8db", "dma256x128w8s3", "dma128x128s3"};
+// BB_DMA_TILE (tuning aid): 1..3 force a DMA tile where it is legal, 4 disables the DMA kernels.
+static int dma_tile_override() {
+    static const int v = [] {
+        const char* e = getenv("BB_DMA_TILE");
+        return e ? atoi(e) : 0;
+    }();
+    return v;
+}
 static DmaTile pick_dma_tile(int M, int N, int K, int64_t batches) {
     if (K % 32 != 0 || K < 64 || M < 128 || N < 128 || N % 8 != 0) return D_NONE;
+    const int ov = dma_tile_override();
+    if (ov == 4) return D_NONE;
+    if ((ov >= 1 && ov <= 3) || (ov >= 5 && ov <= 10)) return (DmaTile)ov;
+    // measured on MI355X (256 CUs): 256x256 tiles pay off from two full rounds of blocks on,
+    // 256x128 from one round, smaller problems take 128x128 tiles with two blocks per CU
     const int64_t t256 = (int64_t)((M + 255) / 256) * ((N + 255) / 256) * batches;
     const int64_t t2128 = (int64_t)((M + 255) / 256) * ((N + 127) / 128) * batches;
-    if (M >= 256 && N >= 256 && t256 >= 256) return D256x256;
-    if (M >= 256 && t2128 >= 256) return D256x128;
-    return D128x128;
+    if (M >= 256 && N >= 256 && t256 >= 512) return D256x256w8db;
+    if (M >= 256 && t2128 >= 256) return D256x128w8db;
+    return D128x128s3;
 }
 
 template <bool TA, bool TB> static int dispatch_bf16(GemmArgs& g, int batches, hipStream_t st) {
     switch (pick_dma_tile(g.M, g.N, g.K, batches)) {
-        case D256x256: return launch_bf16_dma<256, 256, 2, 2, TA, TB>(g, batches, st);
-        case D256x128: return launch_bf16_dma<256, 128, 2, 2, TA, TB>(g, batches, st);
-        case D128x128: return launch_bf16_dma<128, 128, 2, 2, TA, TB>(g, batches, st);
+        case D256x256: return launch_bf16_dma<256, 256, 2, 2, TA, TB, true>(g, batches, st);
+        case D256x128: return launch_bf16_dma<256, 128, 2, 2, TA, TB, true>(g, batches, st);
+        case D128x128: return launch_bf16_dma<128, 128, 2, 2, TA, TB, true>(g, batches, st);
+        case D256x256w8: return launch_bf16_dma<256, 256, 2, 4, TA, TB, false>(g, batches, st);
+        case D256x128w8: return launch_bf16_dma<256, 128, 4, 2, TA, TB, false>(g, batches, st);
+        case D256x256w8db: return launch_bf16_dma<256, 256, 2, 4, TA, TB, true>(g, batches, st);
+        case D256x128w8db: return launch_bf16_dma<256, 128, 4, 2, TA, TB, true>(g, batches, st);
+        case D256x128w8s3: return launch_bf16_dma<256, 128, 4, 2, TA, TB, true, 3>(g, batches, st);
+        case D128x128s3: return launch_bf16_dma<128, 128, 2, 2, TA, TB, true, 3>(g, batches, st);
         default: break;
     }
     switch (pick_bf16_tile(g.M, g.N, batches)) {
@@ -717,23 +778,25 @@ extern "C" int bb_gemm_variant(const bb_gemm_desc* d, char* out, int out_len) {
     return BB_OK;
 }
 
-extern "C" int bb_gemm(const bb_gemm_desc* d, void* stream) {
+static int fill_args(const bb_gemm_desc* d, GemmArgs& g, int64_t& batches, bool& ta, bool& tb) {
     BB_REQUIRE(d != nullptr, "bb_gemm: null descriptor");
     BB_REQUIRE(d->dtype == BB_F32 || d->dtype == BB_BF16, "bb_gemm: bad dtype %d", d->dtype);
     BB_REQUIRE(d->c_dtype == d->dtype || d->c_dtype == BB_F32, "bb_gemm: bad c_dtype %d", d->c_dtype);
     BB_REQUIRE(d->layout >= BB_NT && d->layout <= BB_TN, "bb_gemm: bad layout %d", d->layout);
     BB_REQUIRE(d->M >= 0 && d->N >= 0 && d->K >= 0, "bb_gemm: negative dimension");
-    if (d->M == 0 || d->N == 0) return BB_OK;
-    BB_REQUIRE(d->A && d->B && d->C, "bb_gemm: null operand");
     BB_REQUIRE(!d->accumulate || d->c_dtype == BB_F32, "bb_gemm: accumulate needs an fp32 C");
     BB_REQUIRE(d->epilogue >= BB_EPI_NONE && d->epilogue <= BB_EPI_RESIDUAL, "bb_gemm: bad epilogue");
+    const int nb1 = d->nb1 > 0 ? d->nb1 : 1, nb2 = d->nb2 > 0 ? d->nb2 : 1;
+    batches = (int64_t)nb1 * nb2;
+    ta = d->layout == BB_TN;
+    tb = d->layout != BB_NT;
+    g.M = d->M; g.N = d->N; g.K = d->K; g.nb2 = nb2;
+    if (d->M == 0 || d->N == 0) return BB_OK;
+    BB_REQUIRE(d->A && d->B && d->C, "bb_gemm: null operand");
     BB_REQUIRE(d->epilogue != BB_EPI_DACT || d->aux_in, "bb_gemm: DACT epilogue needs aux_in");
     BB_REQUIRE(d->epilogue != BB_EPI_RESIDUAL || d->resid, "bb_gemm: RESIDUAL epilogue needs resid");
-    const int nb1 = d->nb1 > 0 ? d->nb1 : 1, nb2 = d->nb2 > 0 ? d->nb2 : 1;
-    const int64_t batches = (int64_t)nb1 * nb2;
     BB_REQUIRE(batches <= 65535, "bb_gemm: too many batches (%lld)", (long long)batches);
     const int vec = d->dtype == BB_BF16 ? 8 : 4;
-    const bool ta = d->layout == BB_TN, tb = d->layout != BB_NT;
     // the contiguous dimension of every operand is read in 16-byte vectors
     const int a_contig = ta ? d->M : d->K, b_contig = tb ? d->N : d->K;
     BB_REQUIRE(a_contig % vec == 0 && d->lda % vec == 0, "bb_gemm: A contiguous dim/lda must be a multiple of %d", vec);
@@ -742,16 +805,24 @@ extern "C" int bb_gemm(const bb_gemm_desc* d, void* stream) {
     BB_REQUIRE(d->sA1 % vec == 0 && d->sA2 % vec == 0 && d->sB1 % vec == 0 && d->sB2 % vec == 0,
                "bb_gemm: batch strides of A/B must be multiples of %d", vec);
     BB_REQUIRE(d->lda >= a_contig && d->ldb >= b_contig && d->ldc >= d->N, "bb_gemm: leading dimension too small");
-
-    GemmArgs g;
     g.A = d->A; g.B = d->B; g.C = d->C;
     g.bias = d->bias; g.aux_in = d->aux_in; g.aux_out = d->aux_out; g.resid = d->resid;
     g.lda = d->lda; g.ldb = d->ldb; g.ldc = d->ldc; g.ldaux = d->ldaux > 0 ? d->ldaux : d->ldc;
     g.sA1 = d->sA1; g.sA2 = d->sA2; g.sB1 = d->sB1; g.sB2 = d->sB2; g.sC1 = d->sC1; g.sC2 = d->sC2;
-    g.M = d->M; g.N = d->N; g.K = d->K; g.nb2 = nb2;
     g.alpha = d->alpha;
     g.epilogue = d->epilogue; g.act = d->act; g.accumulate = d->accumulate;
     g.c_f32 = (d->c_dtype == BB_F32);
+    g.tiles_m = g.tiles_n = 0;
+    return BB_OK;
+}
+
+extern "C" int bb_gemm(const bb_gemm_desc* d, void* stream) {
+    GemmArgs g;
+    int64_t batches;
+    bool ta, tb;
+    int rc = fill_args(d, g, batches, ta, tb);
+    if (rc) return rc;
+    if (d->M == 0 || d->N == 0) return BB_OK;
     hipStream_t st = (hipStream_t)stream;
     if (d->dtype == BB_BF16) {
         if (!ta && !tb) return dispatch_bf16<false, false>(g, (int)batches, st);
@@ -761,4 +832,59 @@ extern "C" int bb_gemm(const bb_gemm_desc* d, void* stream) {
     if (!ta && !tb) return dispatch_f32<false, false>(g, (int)batches, st);
     if (!ta && tb) return dispatch_f32<false, true>(g, (int)batches, st);
     return dispatch_f32<true, true>(g, (int)batches, st);
+}
+
+template <bool TA, bool TB> static int launch_grouped(GroupedArgs& G, hipStream_t st) {
+    constexpr int BM = 128, BN = 128, STAGES = 3;
+    constexpr int smem = STAGES * (BM + BN) * 32 * 2;
+    auto kern = gemm_bf16_dma_grouped_kernel<BM, BN, 2, 2, TA, TB, true, STAGES>;
+    static bool configured = false;
+    if (!configured) {
+        BB_HIP_CHECK(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, smem));
+        configured = true;
+    }
+    int blocks = 0;
+    for (int i = 0; i < G.count; ++i) {
+        GemmArgs& g = G.p[i];
+        g.tiles_m = (g.M + BM - 1) / BM;
+        g.tiles_n = (g.N + BN - 1) / BN;
+        G.first_block[i] = blocks;
+        blocks += g.tiles_m * g.tiles_n;
+    }
+    G.first_block[G.count] = blocks;
+    hipLaunchKernelGGL(kern, dim3(blocks), dim3(256), smem, st, G);
+    BB_LAUNCH_CHECK();
+    return BB_OK;
+}
+
+extern "C" int bb_gemm_grouped(const bb_gemm_desc* descs, int count, void* stream) {
+    BB_REQUIRE(count >= 0 && (descs || count == 0), "bb_gemm_grouped: bad arguments");
+    hipStream_t st = (hipStream_t)stream;
+    // one launch when every problem is an unbatched bf16 problem of one layout that the DMA
+    // kernel accepts; otherwise the problems run one after the other (same results)
+    bool fuse = count >= 2 && count <= GROUP_MAX;
+    for (int i = 0; i < count && fuse; ++i) {
+        const bb_gemm_desc& d = descs[i];
+        fuse = d.dtype == BB_BF16 && d.layout == descs[0].layout && d.nb1 <= 1 && d.nb2 <= 1 && d.M > 0 && d.N > 0 &&
+               pick_dma_tile(d.M, d.N, d.K, 1) != D_NONE && dma_tile_override() != 4;
+    }
+    if (!fuse) {
+        for (int i = 0; i < count; ++i) {
+            int rc = bb_gemm(&descs[i], stream);
+            if (rc) return rc;
+        }
+        return BB_OK;
+    }
+    GroupedArgs G;
+    G.count = count;
+    for (int i = 0; i < count; ++i) {
+        int64_t batches;
+        bool ta, tb;
+        int rc = fill_args(&descs[i], G.p[i], batches, ta, tb);
+        if (rc) return rc;
+    }
+    const int layout = descs[0].layout;
+    if (layout == BB_NT) return launch_grouped<false, false>(G, st);
+    if (layout == BB_NN) return launch_grouped<false, true>(G, st);
+    return launch_grouped<true, true>(G, st);
 }

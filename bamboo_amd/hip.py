@@ -23,7 +23,7 @@ MASK_CODES = {"none": MASK_NONE, "causal": MASK_CAUSAL, "key_padding": MASK_KEY_
 LN_CODES = {"standard": LN_STANDARD, "annotated": LN_ANNOTATED}
 
 EXPORTS = (
-    "bb_version", "bb_last_error", "bb_init", "bb_gemm", "bb_gemm_variant", "bb_layernorm_fwd",
+    "bb_version", "bb_last_error", "bb_init", "bb_gemm", "bb_gemm_grouped", "bb_gemm_variant", "bb_layernorm_fwd",
     "bb_layernorm_bwd_workspace", "bb_layernorm_bwd", "bb_colsum_workspace", "bb_colsum_acc",
     "bb_softmax_fwd", "bb_softmax_bwd", "bb_residual_add", "bb_mse_workspace", "bb_mse_fwd_bwd",
     "bb_adam_multi", "bb_cast", "bb_fill_f32",
@@ -72,6 +72,7 @@ def lib():
     L.bb_version.restype = c_int
     L.bb_init.restype = c_int
     L.bb_gemm.argtypes = [POINTER(GemmDesc), c_void_p]
+    L.bb_gemm_grouped.argtypes = [POINTER(GemmDesc), c_int, c_void_p]
     L.bb_gemm_variant.argtypes = [POINTER(GemmDesc), c_char_p, c_int]
     L.bb_layernorm_fwd.argtypes = [c_int, c_int, c_int, c_int, c_float, c_void_p, c_void_p, c_void_p,
                                    c_void_p, c_void_p, c_void_p, c_void_p]
@@ -131,9 +132,9 @@ def _row_major(t, name):
 
 
 # ------------------------------------------------------------------------------------- GEMM
-def gemm(layout, A, B, C, *, alpha=1.0, bias=None, epilogue=EPI_NONE, act=ACT_RELU, accumulate=False,
-         aux_in=None, aux_out=None, resid=None, stream=None):
-    """C = epilogue(alpha * op(A) op(B) [+ bias]) on 2-D row-major views (inner stride 1)."""
+def gemm_desc(layout, A, B, C, *, alpha=1.0, bias=None, epilogue=EPI_NONE, act=ACT_RELU, accumulate=False,
+              aux_in=None, aux_out=None, resid=None):
+    """Descriptor of C = epilogue(alpha * op(A) op(B) [+ bias]) on 2-D row-major views."""
     lda, ldb, ldc = _row_major(A, "A"), _row_major(B, "B"), _row_major(C, "C")
     if layout == NT:
         M, K = A.shape; N, Kb = B.shape
@@ -169,11 +170,28 @@ def gemm(layout, A, B, C, *, alpha=1.0, bias=None, epilogue=EPI_NONE, act=ACT_RE
     d.aux_in = None if aux_in is None else aux_in.data_ptr()
     d.aux_out = None if aux_out is None else aux_out.data_ptr()
     d.resid = None if resid is None else resid.data_ptr()
+    return d
+
+
+def gemm(layout, A, B, C, *, stream=None, **kw):
+    """C = epilogue(alpha * op(A) op(B) [+ bias]) on 2-D row-major views (inner stride 1)."""
+    d = gemm_desc(layout, A, B, C, **kw)
     if gemm_hook is not None:
         gemm_hook(d, lambda: check(lib().bb_gemm(byref(d), stream_ptr(stream)), "bb_gemm"))
     else:
         check(lib().bb_gemm(byref(d), stream_ptr(stream)), "bb_gemm")
     return C
+
+
+def gemm_grouped(descs, stream=None):
+    """Independent GEMMs of one layout in one launch (falls back to one launch each inside the
+    library when they cannot share a kernel)."""
+    arr = (GemmDesc * len(descs))(*descs)
+    call = lambda: check(lib().bb_gemm_grouped(arr, len(descs), stream_ptr(stream)), "bb_gemm_grouped")
+    if gemm_hook is not None:
+        gemm_hook(descs, call)
+    else:
+        call()
 
 
 def gemm_variant(desc):

@@ -227,29 +227,35 @@ class TransformerLayer:
         kind, act = hip.LN_CODES[self.ln], hip.ACT_CODES[self.activation]
         d_ffn, d_h0, d_h1 = ctx.buf("d_ffn", (R, f)), ctx.buf("d_h0", (R, h)), ctx.buf("d_h1", (R, h))
         d_qkv = ctx.buf("d_qkv", (R, 3 * h))
+        # weight gradients dW += dy^T x are collected and issued as one grouped launch at the end:
+        # each alone has too few output tiles to fill the GPU
+        wgrads = []
+        wgrad = lambda dy, x, name: wgrads.append(hip.gemm_desc(hip.TN, dy, x, g[name], accumulate=True))
         # feed-forward
-        hip.gemm(hip.TN, d_out, st["act"], g["feed_forward.w_2.weight"], accumulate=True, stream=sm)
+        wgrad(d_out, st["act"], "feed_forward.w_2.weight")
         hip.colsum_acc(d_out, g["feed_forward.w_2.bias"], ws, stream=sm)
         hip.gemm(hip.NN, d_out, w["feed_forward.w_2.weight"], d_ffn, epilogue=hip.EPI_DACT, act=act,
                  aux_in=st["u"], stream=sm)
-        hip.gemm(hip.TN, d_ffn, st["n2"], g["feed_forward.w_1.weight"], accumulate=True, stream=sm)
+        wgrad(d_ffn, st["n2"], "feed_forward.w_1.weight")
         hip.colsum_acc(d_ffn, g["feed_forward.w_1.bias"], ws, stream=sm)
         hip.gemm(hip.NN, d_ffn, w["feed_forward.w_1.weight"], d_h0, stream=sm)
         # d_x1 = d_out + LN2'(d_n2)
         hip.layernorm_bwd(st["x1"], w["sublayer.1.norm.a_2"], st["mean2"], st["rinv2"], d_h0, d_out, d_h1,
                           g["sublayer.1.norm.a_2"], g["sublayer.1.norm.b_2"], ws, kind, self.eps, stream=sm)
         # attention output projection
-        hip.gemm(hip.TN, d_h1, st["ctx"], g["self_attn.linears.3.weight"], accumulate=True, stream=sm)
+        wgrad(d_h1, st["ctx"], "self_attn.linears.3.weight")
         hip.colsum_acc(d_h1, g["self_attn.linears.3.bias"], ws, stream=sm)
         hip.gemm(hip.NN, d_h1, w["self_attn.linears.3.weight"], d_h0, stream=sm)
         self._attention_bwd(d_h0, d_qkv, st, ctx)
         # QKV projection
-        hip.gemm(hip.TN, d_qkv, st["n1"], g["qkv.weight"], accumulate=True, stream=sm)
+        wgrad(d_qkv, st["n1"], "qkv.weight")
         hip.colsum_acc(d_qkv, g["qkv.bias"], ws, stream=sm)
         hip.gemm(hip.NN, d_qkv, w["qkv.weight"], d_h0, stream=sm)
         # d_x0 = d_x1 + LN1'(d_n1)
         hip.layernorm_bwd(st["x0"], w["sublayer.0.norm.a_2"], st["mean1"], st["rinv1"], d_h0, d_h1, d_x,
                           g["sublayer.0.norm.a_2"], g["sublayer.0.norm.b_2"], ws, kind, self.eps, stream=sm)
+        # d_out, d_ffn, d_h1 and d_qkv still hold the four output gradients here
+        hip.gemm_grouped(wgrads, stream=sm)
         return d_x
 
 

@@ -82,12 +82,16 @@ class GemmProbe:
         import torch
 
         from bamboo_amd import hip
-        name = hip.gemm_variant(desc)
+        if isinstance(desc, (list, tuple)):
+            name = "grouped_" + hip.gemm_variant(desc[0]).rsplit("_", 1)[0]
+            flops = sum(2.0 * d.M * d.N * d.K for d in desc)
+        else:
+            name, flops = hip.gemm_variant(desc), 2.0 * desc.M * desc.N * desc.K
         e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         e0.record()
         launch()
         e1.record()
-        self.records.append((name, 2.0 * desc.M * desc.N * desc.K, e0, e1))
+        self.records.append((name, flops, e0, e1))
 
     def summary(self):
         agg = {}

@@ -102,6 +102,11 @@ int bb_init(void);
  * (engine.py:1701-1709 torch.autograd.backward).  bf16 needs K, lda, ldb, ldc % 8 == 0;
  * fp32 needs them % 4 == 0.                                                               */
 int bb_gemm(const bb_gemm_desc* desc, void* stream);
+/* `count` independent GEMMs of one layout/dtype; results are identical to calling bb_gemm on
+ * each descriptor in turn.  When all are unbatched bf16 problems they share one launch, which
+ * is how the four weight-gradient products of a layer (autograd of transformer.py:136-146,158)
+ * fill the GPU although each has few output tiles.                                         */
+int bb_gemm_grouped(const bb_gemm_desc* descs, int count, void* stream);
 /* Name of the kernel variant bb_gemm would launch for this descriptor ("bf16_nt_256x256", ...),
  * written NUL-terminated into out; for correlating launches with profiler output.        */
 int bb_gemm_variant(const bb_gemm_desc* desc, char* out, int out_len);

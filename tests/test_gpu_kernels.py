@@ -115,6 +115,25 @@ def test_gemm_batched_heads(hiplib, dtype):
     assert rel_err(dV, ref) < tol(dtype)
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_gemm_grouped_weight_gradients(hiplib, dtype):
+    """Four dW += dy^T x products in one launch equal the four separate calls."""
+    rows = 512
+    shapes = [(256, 1024), (1024, 256), (256, 256), (768, 256)]      # (out_features, in_features)
+    dys = [randn(rows, o, dtype=dtype, seed=40 + i) for i, (o, _) in enumerate(shapes)]
+    xs = [randn(rows, k, dtype=dtype, seed=50 + i) for i, (_, k) in enumerate(shapes)]
+    g0 = [randn(o, k, seed=60 + i) for i, (o, k) in enumerate(shapes)]
+    one = [g.clone() for g in g0]
+    for dy, x, g in zip(dys, xs, one):
+        hiplib.gemm(hiplib.TN, dy, x, g, accumulate=True)
+    grp = [g.clone() for g in g0]
+    hiplib.gemm_grouped([hiplib.gemm_desc(hiplib.TN, dy, x, g, accumulate=True) for dy, x, g in zip(dys, xs, grp)])
+    for a, b, dy, x, g in zip(one, grp, dys, xs, g0):
+        ref = g.double().cpu() + dy.double().cpu().t() @ x.double().cpu()
+        assert rel_err(b, ref) < tol(dtype)
+        assert rel_err(a, b.double().cpu()) < 1e-6
+
+
 def test_gemm_rejects_bad_arguments(hiplib):
     A = torch.zeros(16, 12, dtype=torch.bfloat16, device=DEV)   # K = 12 is not a multiple of 8
     B = torch.zeros(16, 12, dtype=torch.bfloat16, device=DEV)
