@@ -97,17 +97,19 @@ __device__ __forceinline__ float wave_max(float v) {
 }
 
 // ---- activations ------------------------------------------------------------------------
-__device__ __forceinline__ float gelu_tanh_f(float x) {
+// tanh-GELU: 0.5 x (1 + tanh z) = x * sigmoid(2z), z = k0 (x + k1 x^3); one v_exp_f32 and one
+// v_rcp_f32 per element (both accurate to 1 ulp), so the epilogue stays far below the MFMA time.
+__device__ __forceinline__ float sigmoid2z_f(float x) {
     const float k0 = 0.7978845608028654f, k1 = 0.044715f;
-    float u = k0 * (x + k1 * x * x * x);
-    return 0.5f * x * (1.0f + tanhf(u));
+    const float z2 = 2.0f * k0 * (x + k1 * x * x * x);
+    return __frcp_rn(1.0f + __expf(-z2));
 }
+__device__ __forceinline__ float gelu_tanh_f(float x) { return x * sigmoid2z_f(x); }
 __device__ __forceinline__ float dgelu_tanh_f(float x) {
     const float k0 = 0.7978845608028654f, k1 = 0.044715f;
-    float u = k0 * (x + k1 * x * x * x);
-    float t = tanhf(u);
-    float du = k0 * (1.0f + 3.0f * k1 * x * x);
-    return 0.5f * (1.0f + t) + 0.5f * x * (1.0f - t * t) * du;
+    const float s = sigmoid2z_f(x);
+    const float dz2 = 2.0f * k0 * (1.0f + 3.0f * k1 * x * x);
+    return s + x * s * (1.0f - s) * dz2;
 }
 __device__ __forceinline__ float act_f(float x, int kind) {
     return kind == BB_ACT_RELU ? fmaxf(x, 0.0f) : gelu_tanh_f(x);

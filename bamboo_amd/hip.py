@@ -177,7 +177,7 @@ def gemm(layout, A, B, C, *, stream=None, **kw):
     """C = epilogue(alpha * op(A) op(B) [+ bias]) on 2-D row-major views (inner stride 1)."""
     d = gemm_desc(layout, A, B, C, **kw)
     if gemm_hook is not None:
-        gemm_hook(d, lambda: check(lib().bb_gemm(byref(d), stream_ptr(stream)), "bb_gemm"))
+        gemm_hook(d, lambda: check(lib().bb_gemm(byref(d), stream_ptr(stream)), "bb_gemm"), stream)
     else:
         check(lib().bb_gemm(byref(d), stream_ptr(stream)), "bb_gemm")
     return C
@@ -189,7 +189,7 @@ def gemm_grouped(descs, stream=None):
     arr = (GemmDesc * len(descs))(*descs)
     call = lambda: check(lib().bb_gemm_grouped(arr, len(descs), stream_ptr(stream)), "bb_gemm_grouped")
     if gemm_hook is not None:
-        gemm_hook(descs, call)
+        gemm_hook(descs, call, stream)
     else:
         call()
 
@@ -200,8 +200,8 @@ def gemm_variant(desc):
     return buf.value.decode()
 
 
-# Optional observer called as hook(desc, launch) around every dense GEMM; `launch()` performs
-# the call.  Used by the benchmark to bracket launches with events; None in normal operation.
+# Optional observer called as hook(desc, launch, stream) around every dense GEMM; `launch()`
+# performs the call on `stream` (None = the current stream).  Used by the benchmark to bracket launches with events; None in normal operation.
 gemm_hook = None
 
 

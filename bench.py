@@ -78,7 +78,7 @@ class GemmProbe:
     def __init__(self):
         self.records = []
 
-    def __call__(self, desc, launch):
+    def __call__(self, desc, launch, stream=None):
         import torch
 
         from bamboo_amd import hip
@@ -88,9 +88,10 @@ class GemmProbe:
         else:
             name, flops = hip.gemm_variant(desc), 2.0 * desc.M * desc.N * desc.K
         e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        e0.record()
+        stream = stream if stream is not None else torch.cuda.current_stream()
+        e0.record(stream)        # on the stream the kernel is launched on
         launch()
-        e1.record()
+        e1.record(stream)
         self.records.append((name, flops, e0, e1))
 
     def summary(self):
