@@ -1,0 +1,549 @@
+// Fused masked softmax-attention for gfx950, bf16, head dimension 64: forward and the two
+// backward kernels (dK/dV and dQ).  No [batch, heads, seq, seq] tensor ever reaches HBM; the
+// forward keeps one fp32 log-sum-exp per (batch, head, query) for the backward.
+//
+// Stands in for MultiHeadedAttention.attention of the reference
+// (DeepSpeedExamples/pipeline_parallelism/transformer.py:117-127: softmax(QK^T/sqrt(d) with
+// masked_fill(mask == 0, -1e9)) V) and for its autograd backward.
+//
+// Layout.  Q, K, V of head j are the 64-wide column slices at j*64 of the three thirds of the
+// [rows, 3*hidden] projection buffer; the context goes to columns j*64 of a [rows, hidden]
+// buffer.  Each wave owns 32 rows (queries in forward / dQ, keys in dK/dV) and keeps one score
+// COLUMN per lane: scores are produced transposed (S^T = K Q^T), so the softmax reductions over
+// keys are in-lane plus one cross-half shuffle, and P^T comes out of the accumulators already
+// in the register layout the next MFMA wants as its B operand.  Operands that are contracted
+// over their row index (V in O = PV, Q and dO in dK/dV, K in dQ) are read from LDS with
+// ds_read_b64_tr_b16.  Tiles travel global -> LDS by DMA (global_load_lds_dwordx4),
+// double-buffered.  All reductions have a fixed order: results are reproducible bit for bit.
+#include "common.h"
+
+typedef __attribute__((address_space(3))) void lds_ptr_t;
+typedef const __attribute__((address_space(1))) void gbl_ptr_t;
+typedef __attribute__((ext_vector_type(4))) short s16x4;
+typedef __attribute__((ext_vector_type(8))) short s16x8;
+
+struct AttnArgs {
+    const bf16* q; const bf16* k; const bf16* v;   // head 0 of batch 0; row stride ld_qkv
+    const bf16* o; const bf16* d_o;                // [rows, hidden] context and its gradient
+    bf16* out;                                     // forward: context
+    bf16* dq; bf16* dk; bf16* dv;                  // backward outputs, row stride ld_dqkv
+    float* lse;                                    // [batch, heads, seq], log2 domain
+    float* delta;                                  // [batch, heads, seq], rowsum(dO * O)
+    const int32_t* key_len;
+    int64_t ld_qkv, ld_o, ld_dqkv;
+    int batch, heads, seq, mask;
+    float scale_log2;                              // log2(e) / sqrt(d)
+    float scale;                                   // 1 / sqrt(d)
+};
+
+// ---- LDS tile format: [rows][64] bf16, 128 B per row, 16-byte chunk c of row r at slot c ^ fsw(r)
+__device__ __forceinline__ int fsw(int r) { return (((r >> 1) & 1) << 2) | (((r >> 2) & 1) << 1) | ((r >> 3) & 1); }
+
+// one wave-instruction moves 8 rows; instruction `idx` of a tile covers rows idx*8 .. idx*8+7
+__device__ __forceinline__ void dma_rows8(const bf16* gbase, int64_t ld, int row0, int last_row, unsigned char* tile,
+                                          int idx, int lane) {
+    const int r = idx * 8 + (lane >> 3);
+    const int c = (lane & 7) ^ fsw(r);
+    const int gr = min(row0 + r, last_row);
+    __builtin_amdgcn_global_load_lds((gbl_ptr_t*)(gbase + (int64_t)gr * ld + c * 8), (lds_ptr_t*)(tile + idx * 1024), 16, 0, 0);
+}
+// 4-byte variant for the per-row fp32 statistics: 64 consecutive floats
+__device__ __forceinline__ void dma_f32x64(const float* gbase, int idx0, int last, unsigned char* dst, int lane) {
+    const int i = min(idx0 + lane, last);
+    __builtin_amdgcn_global_load_lds((gbl_ptr_t*)(gbase + i), (lds_ptr_t*)dst, 4, 0, 0);
+}
+
+// A/B fragment along the contiguous (feature) dimension: lane (r = lane%32, kg = lane/32) gets
+// features ks*16 + kg*8 .. +8 of tile row row0 + r
+__device__ __forceinline__ bf16x8 frag_kc(const unsigned char* tile, int row0, int ks, int lane) {
+    const int r = row0 + (lane & 31);
+    const int chunk = ks * 2 + (lane >> 5);
+    return *(const bf16x8*)(tile + r * 128 + ((chunk ^ fsw(r)) << 4));
+}
+// A fragment contracted over tile ROWS: lane (c = lane%32, kg = lane/32) gets, for feature column
+// col0 + c, the rows rbase + 4kg + {0..3} and rbase + 8 + 4kg + {0..3}: the row order in which a
+// 32x32 accumulator column sits in registers 0..7 of a lane
+__device__ __forceinline__ bf16x8 frag_tr(const unsigned char* tile, int rbase, int col0, int lane) {
+    const int j = lane & 15;
+    const int col = col0 + ((lane >> 4) & 1) * 16 + 4 * (j & 3);
+    const int r0 = rbase + 4 * (lane >> 5) + (j >> 2);
+    const int r1 = r0 + 8;
+    const unsigned char* p0 = tile + r0 * 128 + (((col >> 3) ^ fsw(r0)) << 4) + (col & 7) * 2;
+    const unsigned char* p1 = tile + r1 * 128 + (((col >> 3) ^ fsw(r1)) << 4) + (col & 7) * 2;
+    s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4*)p0);
+    s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4*)p1);
+    s16x8 v = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+    return __builtin_bit_cast(bf16x8, v);
+}
+// registers 8*half .. 8*half+7 of a 32x32 accumulator as a bf16 B fragment
+__device__ __forceinline__ bf16x8 pack_acc(const f32x16& a, int half) {
+    bf16x8 v;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) v[e] = (__bf16)a[half * 8 + e];
+    return v;
+}
+// row index (0..31) that register r of a 32x32 accumulator holds in this lane
+__device__ __forceinline__ int acc_row(int r, int lane) { return 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3); }
+
+template <int N> __device__ __forceinline__ void wait_vm() {
+    __builtin_amdgcn_s_waitcnt((N & 15) | (7 << 4) | (0 << 8) | ((N >> 4) << 14));
+}
+__device__ __forceinline__ void block_sync() {
+    asm volatile("" ::: "memory");
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+}
+
+// number of leading keys a query may see (mask applied as in the reference: keep kv < limit)
+__device__ __forceinline__ int kv_limit(const AttnArgs& a, int b, int q) {
+    if (a.mask == BB_MASK_CAUSAL) return min(a.seq, q + 1);
+    if (a.mask == BB_MASK_KEY_PADDING) return min(a.seq, a.key_len[b]);
+    return a.seq;
+}
+
+// =========================================================================================
+// forward: block = 128 queries (4 waves x 32), loop over 64-key tiles
+// =========================================================================================
+__global__ __launch_bounds__(256) void attn_fwd_kernel(const AttnArgs a) {
+    __shared__ __attribute__((aligned(16))) unsigned char smem[2 * 2 * 8192];  // 2 stages x (K, V)
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int qb = gridDim.x - 1 - blockIdx.x;  // long (late) query blocks first
+    const int b = blockIdx.y / a.heads, head = blockIdx.y % a.heads;
+    const int64_t row_base = (int64_t)b * a.seq;
+    const bf16* Q = a.q + row_base * a.ld_qkv + head * 64;
+    const bf16* K = a.k + row_base * a.ld_qkv + head * 64;
+    const bf16* V = a.v + row_base * a.ld_qkv + head * 64;
+    const int q0 = qb * 128 + wave * 32;
+    const int myq = q0 + (lane & 31);
+    const int last = a.seq - 1;
+
+    // block-wide key range
+    int kv_end = a.seq;
+    if (a.mask == BB_MASK_CAUSAL) kv_end = min(a.seq, qb * 128 + 128);
+    else if (a.mask == BB_MASK_KEY_PADDING) kv_end = min(a.seq, a.key_len[b]);
+    const int ntiles = (kv_end + 63) / 64;
+    const int my_limit = kv_limit(a, b, myq);
+
+    bf16x8 qf[4];
+    {
+        const bf16* qp = Q + (int64_t)min(myq, last) * a.ld_qkv + (lane >> 5) * 8;
+#pragma unroll
+        for (int ks = 0; ks < 4; ++ks) qf[ks] = *(const bf16x8*)(qp + ks * 16);
+    }
+    f32x16 o[2];
+#pragma unroll
+    for (int t = 0; t < 2; ++t)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) o[t][r] = 0.f;
+    float m = -INFINITY, lsum = 0.f;
+
+    auto issue = [&](int t) {
+        unsigned char* st = smem + (t & 1) * 16384;
+        const int kv0 = t * 64;
+        dma_rows8(K, a.ld_qkv, kv0, last, st, wave, lane);
+        dma_rows8(K, a.ld_qkv, kv0, last, st, wave + 4, lane);
+        dma_rows8(V, a.ld_qkv, kv0, last, st + 8192, wave, lane);
+        dma_rows8(V, a.ld_qkv, kv0, last, st + 8192, wave + 4, lane);
+    };
+
+    if (ntiles > 0) issue(0);
+    for (int t = 0; t < ntiles; ++t) {
+        asm volatile("" ::: "memory");
+        if (t + 1 < ntiles) {
+            issue(t + 1);
+            wait_vm<4>();
+        } else {
+            wait_vm<0>();
+        }
+        block_sync();
+        const unsigned char* kt = smem + (t & 1) * 16384;
+        const unsigned char* vt = kt + 8192;
+        const int kv0 = t * 64;
+        // waves whose queries all precede this tile have nothing to add (causal)
+        const bool active = !(a.mask == BB_MASK_CAUSAL && kv0 > q0 + 31);
+        if (active) {
+            f32x16 s[2];
+#pragma unroll
+            for (int u = 0; u < 2; ++u) {
+#pragma unroll
+                for (int r = 0; r < 16; ++r) s[u][r] = 0.f;
+#pragma unroll
+                for (int ks = 0; ks < 4; ++ks)
+                    s[u] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frag_kc(kt, u * 32, ks, lane), qf[ks], s[u], 0, 0, 0);
+            }
+            // scale, mask, running max
+            float tmax = -INFINITY;
+#pragma unroll
+            for (int u = 0; u < 2; ++u)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    const int kv = kv0 + u * 32 + acc_row(r, lane);
+                    const float x = kv < my_limit ? s[u][r] * a.scale_log2 : -INFINITY;
+                    s[u][r] = x;
+                    tmax = fmaxf(tmax, x);
+                }
+            tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
+            const float mnew = fmaxf(m, tmax);
+            const float msafe = mnew == -INFINITY ? 0.f : mnew;
+            const float alpha = exp2f(m - msafe);  // m = -inf -> 0
+            float psum = 0.f;
+#pragma unroll
+            for (int u = 0; u < 2; ++u)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    const float p = exp2f(s[u][r] - msafe);
+                    s[u][r] = p;
+                    psum += p;
+                }
+            lsum = lsum * alpha + psum;
+            m = mnew;
+#pragma unroll
+            for (int t2 = 0; t2 < 2; ++t2)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) o[t2][r] *= alpha;
+            // O^T += V^T P^T
+#pragma unroll
+            for (int kk = 0; kk < 4; ++kk) {
+                const bf16x8 pf = pack_acc(s[kk >> 1], kk & 1);
+#pragma unroll
+                for (int dt = 0; dt < 2; ++dt)
+                    o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frag_tr(vt, kk * 16, dt * 32, lane), pf, o[dt], 0, 0, 0);
+            }
+        }
+        block_sync();
+    }
+    lsum += __shfl_xor(lsum, 32, 64);
+    const float inv = lsum > 0.f ? 1.0f / lsum : 0.f;
+    if (myq < a.seq) {
+        bf16* op = a.out + (row_base + myq) * a.ld_o + head * 64;
+#pragma unroll
+        for (int dt = 0; dt < 2; ++dt)
+#pragma unroll
+            for (int g4 = 0; g4 < 4; ++g4) {
+                const int d = dt * 32 + 8 * g4 + 4 * (lane >> 5);
+                u32x2 w = {pack2bf(o[dt][g4 * 4] * inv, o[dt][g4 * 4 + 1] * inv),
+                           pack2bf(o[dt][g4 * 4 + 2] * inv, o[dt][g4 * 4 + 3] * inv)};
+                *(u32x2*)(op + d) = w;
+            }
+        if (lane < 32) a.lse[((int64_t)b * a.heads + head) * a.seq + myq] = m + log2f(lsum);
+    }
+}
+
+// =========================================================================================
+// backward, preparation: delta[b, head, q] = sum_d dO[q, d] * O[q, d]
+// =========================================================================================
+__global__ __launch_bounds__(256) void attn_delta_kernel(const AttnArgs a) {
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;  // (row, head), head fastest
+    const int64_t rows = (int64_t)a.batch * a.seq;
+    if (i >= rows * a.heads) return;
+    const int head = (int)(i % a.heads);
+    const int64_t row = i / a.heads;
+    const bf16* op = a.o + row * a.ld_o + head * 64;
+    const bf16* gp = a.d_o + row * a.ld_o + head * 64;
+    float s = 0.f;
+#pragma unroll
+    for (int c = 0; c < 8; ++c) {
+        float x[8], y[8];
+        load_vec(op + c * 8, x);
+        load_vec(gp + c * 8, y);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) s += x[e] * y[e];
+    }
+    const int b = (int)(row / a.seq), q = (int)(row % a.seq);
+    a.delta[((int64_t)b * a.heads + head) * a.seq + q] = s;
+}
+
+// =========================================================================================
+// backward dK, dV: block = 128 keys (4 waves x 32), loop over 64-query tiles
+// =========================================================================================
+__global__ __launch_bounds__(256) void attn_bwd_dkv_kernel(const AttnArgs a) {
+    // 2 stages x (Q tile 8 KiB, dO tile 8 KiB, lse 256 B, delta 256 B)
+    constexpr int STAGE = 2 * 8192 + 512;
+    __shared__ __attribute__((aligned(16))) unsigned char smem[2 * STAGE];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int kb = blockIdx.x;
+    const int b = blockIdx.y / a.heads, head = blockIdx.y % a.heads;
+    const int64_t row_base = (int64_t)b * a.seq;
+    const bf16* Q = a.q + row_base * a.ld_qkv + head * 64;
+    const bf16* K = a.k + row_base * a.ld_qkv + head * 64;
+    const bf16* V = a.v + row_base * a.ld_qkv + head * 64;
+    const bf16* DO = a.d_o + row_base * a.ld_o + head * 64;
+    const float* LSE = a.lse + ((int64_t)b * a.heads + head) * a.seq;
+    const float* DELTA = a.delta + ((int64_t)b * a.heads + head) * a.seq;
+    const int kv0 = kb * 128 + wave * 32;
+    const int mykv = kv0 + (lane & 31);
+    const int last = a.seq - 1;
+    const int pad_limit = a.mask == BB_MASK_KEY_PADDING ? min(a.seq, a.key_len[b]) : a.seq;
+
+    // query range that can see keys of this block
+    const int q_begin = a.mask == BB_MASK_CAUSAL ? (kb * 128) / 64 : 0;  // first 64-query tile
+    const int ntiles = (a.seq + 63) / 64;
+
+    bf16x8 kf[4], vf[4];
+    {
+        const int64_t off = (int64_t)min(mykv, last) * a.ld_qkv + (lane >> 5) * 8;
+#pragma unroll
+        for (int ks = 0; ks < 4; ++ks) {
+            kf[ks] = *(const bf16x8*)(K + off + ks * 16);
+            vf[ks] = *(const bf16x8*)(V + off + ks * 16);
+        }
+    }
+    f32x16 dk[2], dv[2];
+#pragma unroll
+    for (int t = 0; t < 2; ++t)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) dk[t][r] = dv[t][r] = 0.f;
+
+    auto issue = [&](int t, int slot) {
+        unsigned char* st = smem + slot * STAGE;
+        const int qs = t * 64;
+        dma_rows8(Q, a.ld_qkv, qs, last, st, wave, lane);
+        dma_rows8(Q, a.ld_qkv, qs, last, st, wave + 4, lane);
+        dma_rows8(DO, a.ld_o, qs, last, st + 8192, wave, lane);
+        dma_rows8(DO, a.ld_o, qs, last, st + 8192, wave + 4, lane);
+        if (wave == 0) dma_f32x64(LSE, qs, last, st + 16384, lane);
+        if (wave == 1) dma_f32x64(DELTA, qs, last, st + 16384 + 256, lane);
+    };
+
+    if (q_begin < ntiles) issue(q_begin, 0);
+    for (int t = q_begin; t < ntiles; ++t) {
+        const int slot = (t - q_begin) & 1;
+        asm volatile("" ::: "memory");
+        if (t + 1 < ntiles) {
+            issue(t + 1, slot ^ 1);
+            // waves 0 and 1 carry one extra load each; waiting for <= 5 newer loads covers both cases
+            if (wave < 2) wait_vm<5>(); else wait_vm<4>();
+        } else {
+            wait_vm<0>();
+        }
+        block_sync();
+        const unsigned char* qt = smem + slot * STAGE;
+        const unsigned char* dot = qt + 8192;
+        const float* lse_t = (const float*)(qt + 16384);
+        const float* del_t = lse_t + 64;
+#pragma unroll
+        for (int u = 0; u < 2; ++u) {
+            const int qs = t * 64 + u * 32;
+            if (a.mask == BB_MASK_CAUSAL && qs + 31 < kv0) continue;  // all queries precede this wave's keys
+            if (qs >= a.seq) continue;
+            // S[q][kv] and dP[q][kv]
+            f32x16 s, dp;
+#pragma unroll
+            for (int r = 0; r < 16; ++r) s[r] = dp[r] = 0.f;
+#pragma unroll
+            for (int ks = 0; ks < 4; ++ks) {
+                s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frag_kc(qt, u * 32, ks, lane), kf[ks], s, 0, 0, 0);
+                dp = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frag_kc(dot, u * 32, ks, lane), vf[ks], dp, 0, 0, 0);
+            }
+            // P = exp2(S * c - lse[q]); dS = P * (dP - delta[q]); rows q = acc_row(r), column kv = lane
+#pragma unroll
+            for (int g4 = 0; g4 < 4; ++g4) {
+                const int ql = u * 32 + 8 * g4 + 4 * (lane >> 5);
+                const f32x4 l4 = *(const f32x4*)(lse_t + ql);
+                const f32x4 d4 = *(const f32x4*)(del_t + ql);
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    const int r = g4 * 4 + e;
+                    const int q = t * 64 + ql + e;
+                    bool keep = mykv < pad_limit && q < a.seq;
+                    if (a.mask == BB_MASK_CAUSAL) keep = keep && mykv <= q;
+                    const float p = keep ? exp2f(s[r] * a.scale_log2 - l4[e]) : 0.f;
+                    s[r] = p;
+                    dp[r] = p * (dp[r] - d4[e]);
+                }
+            }
+            // dV^T += dO^T P ; dK^T += Q^T dS   (contraction over the 32 queries of this sub-tile)
+#pragma unroll
+            for (int kk = 0; kk < 2; ++kk) {
+                const bf16x8 pf = pack_acc(s, kk), dsf = pack_acc(dp, kk);
+#pragma unroll
+                for (int dt = 0; dt < 2; ++dt) {
+                    dv[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frag_tr(dot, u * 32 + kk * 16, dt * 32, lane), pf, dv[dt], 0, 0, 0);
+                    dk[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frag_tr(qt, u * 32 + kk * 16, dt * 32, lane), dsf, dk[dt], 0, 0, 0);
+                }
+            }
+        }
+        block_sync();
+    }
+    if (mykv < a.seq) {
+        bf16* dkp = a.dk + (row_base + mykv) * a.ld_dqkv + head * 64;
+        bf16* dvp = a.dv + (row_base + mykv) * a.ld_dqkv + head * 64;
+#pragma unroll
+        for (int dt = 0; dt < 2; ++dt)
+#pragma unroll
+            for (int g4 = 0; g4 < 4; ++g4) {
+                const int d = dt * 32 + 8 * g4 + 4 * (lane >> 5);
+                u32x2 wk = {pack2bf(dk[dt][g4 * 4] * a.scale, dk[dt][g4 * 4 + 1] * a.scale),
+                            pack2bf(dk[dt][g4 * 4 + 2] * a.scale, dk[dt][g4 * 4 + 3] * a.scale)};
+                u32x2 wv = {pack2bf(dv[dt][g4 * 4], dv[dt][g4 * 4 + 1]), pack2bf(dv[dt][g4 * 4 + 2], dv[dt][g4 * 4 + 3])};
+                *(u32x2*)(dkp + d) = wk;
+                *(u32x2*)(dvp + d) = wv;
+            }
+    }
+}
+
+// =========================================================================================
+// backward dQ: block = 128 queries (4 waves x 32), loop over 64-key tiles
+// =========================================================================================
+__global__ __launch_bounds__(256) void attn_bwd_dq_kernel(const AttnArgs a) {
+    __shared__ __attribute__((aligned(16))) unsigned char smem[2 * 2 * 8192];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int qb = gridDim.x - 1 - blockIdx.x;
+    const int b = blockIdx.y / a.heads, head = blockIdx.y % a.heads;
+    const int64_t row_base = (int64_t)b * a.seq;
+    const bf16* Q = a.q + row_base * a.ld_qkv + head * 64;
+    const bf16* K = a.k + row_base * a.ld_qkv + head * 64;
+    const bf16* V = a.v + row_base * a.ld_qkv + head * 64;
+    const bf16* DO = a.d_o + row_base * a.ld_o + head * 64;
+    const int q0 = qb * 128 + wave * 32;
+    const int myq = q0 + (lane & 31);
+    const int last = a.seq - 1;
+    int kv_end = a.seq;
+    if (a.mask == BB_MASK_CAUSAL) kv_end = min(a.seq, qb * 128 + 128);
+    else if (a.mask == BB_MASK_KEY_PADDING) kv_end = min(a.seq, a.key_len[b]);
+    const int ntiles = (kv_end + 63) / 64;
+    const int my_limit = myq < a.seq ? kv_limit(a, b, myq) : 0;
+
+    bf16x8 qf[4], dof[4];
+    {
+        const int64_t r = min(myq, last);
+#pragma unroll
+        for (int ks = 0; ks < 4; ++ks) {
+            qf[ks] = *(const bf16x8*)(Q + r * a.ld_qkv + (lane >> 5) * 8 + ks * 16);
+            dof[ks] = *(const bf16x8*)(DO + r * a.ld_o + (lane >> 5) * 8 + ks * 16);
+        }
+    }
+    const int64_t stat = ((int64_t)b * a.heads + head) * a.seq + min(myq, last);
+    const float my_lse = a.lse[stat], my_delta = a.delta[stat];
+    f32x16 dq[2];
+#pragma unroll
+    for (int t = 0; t < 2; ++t)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) dq[t][r] = 0.f;
+
+    auto issue = [&](int t) {
+        unsigned char* st = smem + (t & 1) * 16384;
+        const int kv0 = t * 64;
+        dma_rows8(K, a.ld_qkv, kv0, last, st, wave, lane);
+        dma_rows8(K, a.ld_qkv, kv0, last, st, wave + 4, lane);
+        dma_rows8(V, a.ld_qkv, kv0, last, st + 8192, wave, lane);
+        dma_rows8(V, a.ld_qkv, kv0, last, st + 8192, wave + 4, lane);
+    };
+    if (ntiles > 0) issue(0);
+    for (int t = 0; t < ntiles; ++t) {
+        asm volatile("" ::: "memory");
+        if (t + 1 < ntiles) {
+            issue(t + 1);
+            wait_vm<4>();
+        } else {
+            wait_vm<0>();
+        }
+        block_sync();
+        const unsigned char* kt = smem + (t & 1) * 16384;
+        const unsigned char* vt = kt + 8192;
+        const int kv0 = t * 64;
+        const bool active = !(a.mask == BB_MASK_CAUSAL && kv0 > q0 + 31);
+        if (active) {
+#pragma unroll
+            for (int u = 0; u < 2; ++u) {
+                f32x16 s, dp;
+#pragma unroll
+                for (int r = 0; r < 16; ++r) s[r] = dp[r] = 0.f;
+#pragma unroll
+                for (int ks = 0; ks < 4; ++ks) {
+                    s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frag_kc(kt, u * 32, ks, lane), qf[ks], s, 0, 0, 0);
+                    dp = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frag_kc(vt, u * 32, ks, lane), dof[ks], dp, 0, 0, 0);
+                }
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    const int kv = kv0 + u * 32 + acc_row(r, lane);
+                    const float p = kv < my_limit ? exp2f(s[r] * a.scale_log2 - my_lse) : 0.f;
+                    dp[r] = p * (dp[r] - my_delta);
+                }
+                // dQ^T += K^T dS^T (contraction over the 32 keys of this sub-tile)
+#pragma unroll
+                for (int kk = 0; kk < 2; ++kk) {
+                    const bf16x8 dsf = pack_acc(dp, kk);
+#pragma unroll
+                    for (int dt = 0; dt < 2; ++dt)
+                        dq[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frag_tr(kt, u * 32 + kk * 16, dt * 32, lane), dsf, dq[dt], 0, 0, 0);
+                }
+            }
+        }
+        block_sync();
+    }
+    if (myq < a.seq) {
+        bf16* dqp = a.dq + (row_base + myq) * a.ld_dqkv + head * 64;
+#pragma unroll
+        for (int dt = 0; dt < 2; ++dt)
+#pragma unroll
+            for (int g4 = 0; g4 < 4; ++g4) {
+                const int d = dt * 32 + 8 * g4 + 4 * (lane >> 5);
+                u32x2 w = {pack2bf(dq[dt][g4 * 4] * a.scale, dq[dt][g4 * 4 + 1] * a.scale),
+                           pack2bf(dq[dt][g4 * 4 + 2] * a.scale, dq[dt][g4 * 4 + 3] * a.scale)};
+                *(u32x2*)(dqp + d) = w;
+            }
+    }
+}
+
+// =========================================================================================
+// host entry points
+// =========================================================================================
+static int check_attn(const char* name, int dtype, int mask, int batch, int heads, int seq, int head_dim, int64_t ld_qkv,
+                      int64_t ld_o, const int32_t* key_len) {
+    BB_REQUIRE(dtype == BB_BF16, "%s: the fused attention kernels are bf16 only (got dtype %d)", name, dtype);
+    BB_REQUIRE(head_dim == 64, "%s: head dimension must be 64 (got %d)", name, head_dim);
+    BB_REQUIRE(mask >= BB_MASK_NONE && mask <= BB_MASK_KEY_PADDING, "%s: bad mask %d", name, mask);
+    BB_REQUIRE(mask != BB_MASK_KEY_PADDING || key_len, "%s: key_padding mask needs key_len", name);
+    BB_REQUIRE(batch >= 0 && heads > 0 && seq >= 0, "%s: bad shape", name);
+    BB_REQUIRE(ld_qkv % 8 == 0 && ld_o % 8 == 0 && ld_qkv >= heads * 64 && ld_o >= heads * 64, "%s: bad leading dimension", name);
+    BB_REQUIRE((int64_t)batch * heads <= 65535, "%s: batch * heads exceeds the grid limit", name);
+    return BB_OK;
+}
+
+extern "C" int bb_attention_fwd(int dtype, int mask, int batch, int heads, int seq, int head_dim, const void* q,
+                                const void* k, const void* v, int64_t ld_qkv, void* out, int64_t ld_out, float* lse,
+                                const int32_t* key_len, void* stream) {
+    int rc = check_attn("bb_attention_fwd", dtype, mask, batch, heads, seq, head_dim, ld_qkv, ld_out, key_len);
+    if (rc) return rc;
+    if (batch == 0 || seq == 0) return BB_OK;
+    BB_REQUIRE(q && k && v && out && lse, "bb_attention_fwd: null pointer");
+    AttnArgs a = {};
+    a.q = (const bf16*)q; a.k = (const bf16*)k; a.v = (const bf16*)v;
+    a.out = (bf16*)out; a.lse = lse; a.key_len = key_len;
+    a.ld_qkv = ld_qkv; a.ld_o = ld_out;
+    a.batch = batch; a.heads = heads; a.seq = seq; a.mask = mask;
+    a.scale = 1.0f / sqrtf((float)head_dim);
+    a.scale_log2 = a.scale * 1.4426950408889634f;
+    hipLaunchKernelGGL(attn_fwd_kernel, dim3((seq + 127) / 128, batch * heads), dim3(256), 0, (hipStream_t)stream, a);
+    BB_LAUNCH_CHECK();
+    return BB_OK;
+}
+
+extern "C" int bb_attention_bwd(int dtype, int mask, int batch, int heads, int seq, int head_dim, const void* q,
+                                const void* k, const void* v, int64_t ld_qkv, const void* out, const void* d_out,
+                                int64_t ld_out, const float* lse, float* delta, void* dq, void* dk, void* dv,
+                                int64_t ld_dqkv, const int32_t* key_len, void* stream) {
+    int rc = check_attn("bb_attention_bwd", dtype, mask, batch, heads, seq, head_dim, ld_qkv, ld_out, key_len);
+    if (rc) return rc;
+    if (batch == 0 || seq == 0) return BB_OK;
+    BB_REQUIRE(q && k && v && out && d_out && lse && delta && dq && dk && dv, "bb_attention_bwd: null pointer");
+    BB_REQUIRE(ld_dqkv % 4 == 0 && ld_dqkv >= heads * 64, "bb_attention_bwd: bad gradient leading dimension");
+    AttnArgs a = {};
+    a.q = (const bf16*)q; a.k = (const bf16*)k; a.v = (const bf16*)v;
+    a.o = (const bf16*)out; a.d_o = (const bf16*)d_out;
+    a.dq = (bf16*)dq; a.dk = (bf16*)dk; a.dv = (bf16*)dv;
+    a.lse = (float*)lse; a.delta = delta; a.key_len = key_len;
+    a.ld_qkv = ld_qkv; a.ld_o = ld_out; a.ld_dqkv = ld_dqkv;
+    a.batch = batch; a.heads = heads; a.seq = seq; a.mask = mask;
+    a.scale = 1.0f / sqrtf((float)head_dim);
+    a.scale_log2 = a.scale * 1.4426950408889634f;
+    hipStream_t st = (hipStream_t)stream;
+    const int64_t n = (int64_t)batch * seq * heads;
+    hipLaunchKernelGGL(attn_delta_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st, a);
+    dim3 grid((seq + 127) / 128, batch * heads);
+    hipLaunchKernelGGL(attn_bwd_dkv_kernel, grid, dim3(256), 0, st, a);
+    hipLaunchKernelGGL(attn_bwd_dq_kernel, grid, dim3(256), 0, st, a);
+    BB_LAUNCH_CHECK();
+    return BB_OK;
+}

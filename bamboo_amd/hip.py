@@ -25,7 +25,7 @@ LN_CODES = {"standard": LN_STANDARD, "annotated": LN_ANNOTATED}
 EXPORTS = (
     "bb_version", "bb_last_error", "bb_init", "bb_gemm", "bb_gemm_grouped", "bb_gemm_variant", "bb_layernorm_fwd",
     "bb_layernorm_bwd_workspace", "bb_layernorm_bwd", "bb_colsum_workspace", "bb_colsum_acc",
-    "bb_softmax_fwd", "bb_softmax_bwd", "bb_residual_add", "bb_mse_workspace", "bb_mse_fwd_bwd",
+    "bb_softmax_fwd", "bb_softmax_bwd", "bb_attention_fwd", "bb_attention_bwd", "bb_residual_add", "bb_mse_workspace", "bb_mse_fwd_bwd",
     "bb_adam_multi", "bb_cast", "bb_fill_f32",
 )
 
@@ -84,6 +84,10 @@ def lib():
     L.bb_colsum_acc.argtypes = [c_int, c_int, c_int, c_void_p, c_int64, c_void_p, c_void_p, c_void_p]
     L.bb_softmax_fwd.argtypes = [c_int, c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p]
     L.bb_softmax_bwd.argtypes = [c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p]
+    L.bb_attention_fwd.argtypes = [c_int] * 6 + [c_void_p, c_void_p, c_void_p, c_int64, c_void_p, c_int64, c_void_p,
+                                   c_void_p, c_void_p]
+    L.bb_attention_bwd.argtypes = [c_int] * 6 + [c_void_p, c_void_p, c_void_p, c_int64, c_void_p, c_void_p, c_int64,
+                                   c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_void_p, c_void_p]
     L.bb_residual_add.argtypes = [c_int, c_int64, c_void_p, c_void_p, c_void_p, c_void_p]
     L.bb_mse_workspace.restype = c_int64
     L.bb_mse_fwd_bwd.argtypes = [c_int, c_int64, c_void_p, c_void_p, c_void_p, c_float, c_void_p, c_int,
@@ -268,6 +272,27 @@ def softmax_bwd(p, dp, stream=None):
         raise HipKernelError("softmax_bwd: tensors must be contiguous")
     check(lib().bb_softmax_bwd(dtype_code(p.dtype), b, h, sq, sk, _ptr(p), _ptr(dp), stream_ptr(stream)),
           "bb_softmax_bwd")
+
+
+def attention_fwd(qkv, out, lse, batch, heads, seq, mask, key_len=None, stream=None):
+    """qkv: [batch*seq, 3*heads*64] (Q | K | V thirds), out: [batch*seq, heads*64], lse: fp32 [batch, heads, seq]."""
+    h = heads * 64
+    es = qkv.element_size()
+    q = qkv.data_ptr()
+    check(lib().bb_attention_fwd(dtype_code(qkv.dtype), mask, batch, heads, seq, qkv.shape[1] // (3 * heads),
+                                 c_void_p(q), c_void_p(q + h * es), c_void_p(q + 2 * h * es), qkv.stride(0), _ptr(out),
+                                 out.stride(0), _ptr(lse), _ptr(key_len), stream_ptr(stream)), "bb_attention_fwd")
+
+
+def attention_bwd(qkv, out, d_out, lse, delta, d_qkv, batch, heads, seq, mask, key_len=None, stream=None):
+    h = heads * 64
+    es = qkv.element_size()
+    q, dq = qkv.data_ptr(), d_qkv.data_ptr()
+    check(lib().bb_attention_bwd(dtype_code(qkv.dtype), mask, batch, heads, seq, qkv.shape[1] // (3 * heads),
+                                 c_void_p(q), c_void_p(q + h * es), c_void_p(q + 2 * h * es), qkv.stride(0), _ptr(out),
+                                 _ptr(d_out), out.stride(0), _ptr(lse), _ptr(delta), c_void_p(dq),
+                                 c_void_p(dq + h * es), c_void_p(dq + 2 * h * es), d_qkv.stride(0), _ptr(key_len),
+                                 stream_ptr(stream)), "bb_attention_bwd")
 
 
 def residual_add(a, b, out, stream=None):

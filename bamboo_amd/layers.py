@@ -130,12 +130,22 @@ class TransformerLayer:
     def out_shape(self, in_shape):
         return in_shape
 
+    def fused_attention(self, ctx):
+        """bf16 runs the fused attention kernels (no score matrix in HBM); fp32, the correctness
+        configuration, materialises the probabilities like the reference does."""
+        if ctx.dtype == torch.bfloat16:
+            if self.head_dim != 64:
+                raise hip.HipKernelError(f"bf16 attention kernels need head_dim 64, got {self.head_dim}")
+            return True
+        return False
+
     def stash_specs(self, ctx):
         R, h, f = ctx.rows, self.hidden, self.ffn
         dt, f32 = ctx.dtype, torch.float32
+        attn = ("lse", (ctx.batch, self.heads, ctx.seq), f32) if self.fused_attention(ctx) else \
+            ("prob", (ctx.batch, self.heads, ctx.seq, ctx.seq), dt)
         return [
-            ("n1", (R, h), dt), ("qkv", (R, 3 * h), dt),
-            ("prob", (ctx.batch, self.heads, ctx.seq, ctx.seq), dt),
+            ("n1", (R, h), dt), ("qkv", (R, 3 * h), dt), attn,
             ("ctx", (R, h), dt), ("x1", (R, h), dt), ("n2", (R, h), dt),
             ("u", (R, f), dt), ("act", (R, f), dt), ("out", (R, h), dt),
             ("mean1", (R,), f32), ("rinv1", (R,), f32), ("mean2", (R,), f32), ("rinv2", (R,), f32),
@@ -144,8 +154,9 @@ class TransformerLayer:
     def scratch_specs(self, ctx):
         R, h, f = ctx.rows, self.hidden, self.ffn
         dt = ctx.dtype
-        return [("d_ffn", (R, f), dt), ("d_h0", (R, h), dt), ("d_h1", (R, h), dt), ("d_qkv", (R, 3 * h), dt),
-                ("d_prob", (ctx.batch, self.heads, ctx.seq, ctx.seq), dt)]
+        attn = ("attn_delta", (ctx.batch, self.heads, ctx.seq), torch.float32) if self.fused_attention(ctx) else \
+            ("d_prob", (ctx.batch, self.heads, ctx.seq, ctx.seq), dt)
+        return [("d_ffn", (R, f), dt), ("d_h0", (R, h), dt), ("d_h1", (R, h), dt), ("d_qkv", (R, 3 * h), dt), attn]
 
     def workspace_elems(self):
         n = max(self.hidden * 3, self.ffn)
@@ -162,6 +173,10 @@ class TransformerLayer:
 
     def _attention_fwd(self, st, ctx):
         h, d, s = self.hidden, self.head_dim, ctx.seq
+        if self.fused_attention(ctx):
+            hip.attention_fwd(st["qkv"], st["ctx"], st["lse"], ctx.batch, self.heads, s, hip.MASK_CODES[self.mask],
+                              ctx.key_len, stream=ctx.stream)
+            return
         es = st["qkv"].element_size()
         q = st["qkv"].data_ptr()
         k, v = q + h * es, q + 2 * h * es
@@ -177,6 +192,11 @@ class TransformerLayer:
 
     def _attention_bwd(self, d_ctx, d_qkv, st, ctx):
         h, d, s = self.hidden, self.head_dim, ctx.seq
+        if self.fused_attention(ctx):
+            delta = ctx.buf("attn_delta", (ctx.batch, self.heads, s))
+            hip.attention_bwd(st["qkv"], st["ctx"], d_ctx, st["lse"], delta, d_qkv, ctx.batch, self.heads, s,
+                              hip.MASK_CODES[self.mask], ctx.key_len, stream=ctx.stream)
+            return
         es = st["qkv"].element_size()
         q = st["qkv"].data_ptr()
         k, v = q + h * es, q + 2 * h * es

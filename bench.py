@@ -219,7 +219,7 @@ def main():
         "vs_baseline": None, "dtype": cfg["dtype"], "data": "synthetic",
         "config": {"workload": cfg["label"], "stage": f"{STAGE_ID} of {STAGES}", "redundancy_level": 1,
                    "eager_recovery": True, "rc_stream": bool(args.rc_stream), "samples_per_step": samples,
-                   "attention": "dense scores materialised (unfused), flops counted dense"},
+                   "attention": "fused (no score matrix in HBM); flops counted dense, the causal kernel skips masked tiles"},
         "rc_on_samples_per_s": round(samples / t_on, 3),
         "rc_off_samples_per_s": None if t_off is None else round(samples / t_off, 3),
         "rc_overhead_pct": None if t_off is None else round(100.0 * (t_on - t_off) / t_off, 2),

@@ -142,6 +142,23 @@ int bb_softmax_fwd(int dtype, int mask, int batch, int heads, int sq, int sk, vo
 int bb_softmax_bwd(int dtype, int batch, int heads, int sq, int sk, const void* p, void* dp,
                    void* stream);
 
+/* Fused masked softmax-attention (bf16, head_dim 64): out = softmax(Q K^T / sqrt(d), mask) V for
+ * every (batch, head), without materialising the score matrix (transformer.py:117-127).
+ * q, k, v point at head 0 of batch 0; rows are tokens (batch-major), head j occupies columns
+ * j*64.. of each pointer, row stride ld_qkv (the three pointers may alias one [rows, 3h] buffer).
+ * out: [rows, heads*64] with row stride ld_out.  lse: fp32 [batch, heads, seq] log-sum-exp (base 2,
+ * scaled scores) kept for the backward.                                                     */
+int bb_attention_fwd(int dtype, int mask, int batch, int heads, int seq, int head_dim, const void* q,
+                     const void* k, const void* v, int64_t ld_qkv, void* out, int64_t ld_out, float* lse,
+                     const int32_t* key_len, void* stream);
+/* Backward of bb_attention_fwd: dq, dk, dv (same addressing as q, k, v with row stride ld_dqkv)
+ * from d_out, the forward's out and lse.  delta: fp32 workspace [batch, heads, seq].
+ * Deterministic (no atomics): dK/dV and dQ are produced by two passes over the score tiles. */
+int bb_attention_bwd(int dtype, int mask, int batch, int heads, int seq, int head_dim, const void* q,
+                     const void* k, const void* v, int64_t ld_qkv, const void* out, const void* d_out,
+                     int64_t ld_out, const float* lse, float* delta, void* dq, void* dk, void* dv,
+                     int64_t ld_dqkv, const int32_t* key_len, void* stream);
+
 /* out = a + b, elementwise (SublayerConnection residual, transformer.py:103).             */
 int bb_residual_add(int dtype, int64_t n, const void* a, const void* b, void* out,
                     void* stream);

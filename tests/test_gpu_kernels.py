@@ -199,6 +199,55 @@ def test_softmax(hiplib, dtype, mask):
     assert rel_err(dp, dref) < tol(dtype)
 
 
+@pytest.mark.parametrize("mask", ["none", "causal", "key_padding"])
+@pytest.mark.parametrize("b,a,s", [(2, 3, 128), (1, 2, 64), (2, 2, 96), (1, 4, 384), (3, 1, 32), (1, 16, 1024)])
+def test_fused_attention_fwd_bwd(hiplib, mask, b, a, s):
+    """Fused attention (bf16, d = 64) against softmax(QK^T/sqrt(d), mask) V and its autograd gradients,
+    computed in fp64 from the same bf16 inputs."""
+    d, h = 64, a * 64
+    qkv = randn(b * s, 3 * h, dtype=torch.bfloat16, seed=70, scale=1.0)
+    d_out = randn(b * s, h, dtype=torch.bfloat16, seed=71)
+    lens = None
+    if mask == "key_padding":
+        g = torch.Generator().manual_seed(3)
+        lens = torch.randint(max(1, s // 4), s + 1, (b,), generator=g, dtype=torch.int32)
+        lens[0] = s
+    out = torch.full((b * s, h), float("nan"), dtype=torch.bfloat16, device=DEV)
+    lse = torch.empty(b, a, s, device=DEV)
+    kl = None if lens is None else lens.to(DEV)
+    hiplib.attention_fwd(qkv, out, lse, b, a, s, hiplib.MASK_CODES[mask], kl)
+    x = qkv.double().cpu().requires_grad_(True)
+    q, k, v = [x[:, i * h:(i + 1) * h].view(b, s, a, d).transpose(1, 2) for i in range(3)]
+    sc = q @ k.transpose(-1, -2) / math.sqrt(d)
+    m = ol.build_mask(ol.TransformerCfg(hidden=h, heads=a, ffn=8, mask=mask), b, s, lens)
+    if m is not None:
+        sc = sc.masked_fill(~m, -1e9)
+    ref = (torch.softmax(sc, -1) @ v).transpose(1, 2).reshape(b * s, h)
+    l2 = lambda t, r: float((t.double().cpu() - r).norm() / r.norm())
+    assert l2(out, ref.detach()) < 1e-2
+    ref_lse = torch.logsumexp(sc, -1) / math.log(2.0)
+    assert float((lse.double().cpu() - ref_lse.detach()).abs().max()) < 2e-2
+    ref.backward(d_out.double().cpu())
+    d_qkv = torch.full((b * s, 3 * h), float("nan"), dtype=torch.bfloat16, device=DEV)
+    delta = torch.empty(b, a, s, device=DEV)
+    hiplib.attention_bwd(qkv, out, d_out, lse, delta, d_qkv, b, a, s, hiplib.MASK_CODES[mask], kl)
+    for i, name in enumerate("qkv"):
+        got, want = d_qkv[:, i * h:(i + 1) * h], x.grad[:, i * h:(i + 1) * h]
+        assert torch.isfinite(got.float()).all(), name
+        assert l2(got, want) < 2e-2, (name, l2(got, want))
+    # determinism
+    out2, d2 = torch.empty_like(out), torch.empty_like(d_qkv)
+    hiplib.attention_fwd(qkv, out2, lse, b, a, s, hiplib.MASK_CODES[mask], kl)
+    hiplib.attention_bwd(qkv, out2, d_out, lse, delta, d2, b, a, s, hiplib.MASK_CODES[mask], kl)
+    assert torch.equal(out, out2) and torch.equal(d_qkv, d2)
+
+
+def test_fused_attention_rejects(hiplib):
+    qkv = torch.zeros(64, 3 * 64, device=DEV)
+    with pytest.raises(hiplib.HipKernelError):
+        hiplib.attention_fwd(qkv, torch.zeros(64, 64, device=DEV), torch.zeros(1, 1, 64, device=DEV), 1, 1, 64, 0)  # fp32
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("rows,cols", [(1000, 768), (8192, 3072), (7, 64), (513, 1600)])
 def test_colsum(hiplib, dtype, rows, cols):
