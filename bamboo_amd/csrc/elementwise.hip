@@ -226,6 +226,24 @@ __global__ __launch_bounds__(256) void reduce_partials_acc_kernel(const float* _
     if (wave == 0 && i < n) out[i] += (red[0][lane] + red[1][lane]) + (red[2][lane] + red[3][lane]);
 }
 
+// two vectors at once (LayerNorm gain and shift gradients): blockIdx.y picks the half of every
+// partial row and the output
+__global__ __launch_bounds__(256) void reduce_partials_acc2_kernel(const float* __restrict__ partial, int nparts,
+                                                                   int64_t stride, int n, float* __restrict__ out0,
+                                                                   float* __restrict__ out1) {
+    __shared__ float red[4][64];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int i = blockIdx.x * 64 + lane;
+    const float* src = partial + (int64_t)blockIdx.y * n;
+    float* out = blockIdx.y == 0 ? out0 : out1;
+    float s = 0.f;
+    if (i < n)
+        for (int p = wave; p < nparts; p += 4) s += src[p * stride + i];
+    red[wave][lane] = s;
+    __syncthreads();
+    if (wave == 0 && i < n) out[i] += (red[0][lane] + red[1][lane]) + (red[2][lane] + red[3][lane]);
+}
+
 template <typename T, int IT>
 static int ln_fwd_launch(int kind, int rows, int cols, float eps, const void* x, const void* gain, const void* shift,
                          void* y, float* mean, float* rinv, hipStream_t st) {
@@ -294,10 +312,8 @@ extern "C" int bb_layernorm_bwd(int dtype, int kind, int rows, int cols, float e
     hipStream_t st = (hipStream_t)stream;
     auto finish = [&]() -> int {
         const int nb = (cols + 63) / 64;
-        hipLaunchKernelGGL(reduce_partials_acc_kernel, dim3(nb), dim3(256), 0, st, workspace, LN_BWD_BLOCKS,
-                           (int64_t)2 * cols, cols, dgain);
-        hipLaunchKernelGGL(reduce_partials_acc_kernel, dim3(nb), dim3(256), 0, st, workspace + cols, LN_BWD_BLOCKS,
-                           (int64_t)2 * cols, cols, dshift);
+        hipLaunchKernelGGL(reduce_partials_acc2_kernel, dim3(nb, 2), dim3(256), 0, st, workspace, LN_BWD_BLOCKS,
+                           (int64_t)2 * cols, cols, dgain, dshift);
         BB_LAUNCH_CHECK();
         return BB_OK;
     };
@@ -548,6 +564,35 @@ extern "C" int bb_residual_add(int dtype, int64_t n, const void* a, const void* 
         hipLaunchKernelGGL(add_kernel<bf16>, dim3(grid_for(nvec)), dim3(256), 0, st, nvec, (const bf16*)a, (const bf16*)b, (bf16*)out);
     else
         hipLaunchKernelGGL(add_kernel<float>, dim3(grid_for(nvec)), dim3(256), 0, st, nvec, (const float*)a, (const float*)b, (float*)out);
+    BB_LAUNCH_CHECK();
+    return BB_OK;
+}
+
+// out = act(x), elementwise (the activation between the two feed-forward GEMMs)
+template <typename T>
+__global__ __launch_bounds__(256) void act_kernel(int64_t nvec, int act, const T* __restrict__ x, T* __restrict__ out) {
+    constexpr int VEC = Elem<T>::VEC;
+    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < nvec; i += (int64_t)gridDim.x * 256) {
+        float v[VEC];
+        load_vec(x + i * VEC, v);
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) v[e] = act_f(v[e], act);
+        store_vec(out + i * VEC, v);
+    }
+}
+
+extern "C" int bb_act_fwd(int dtype, int act, int64_t n, const void* x, void* out, void* stream) {
+    BB_REQUIRE(dtype == BB_F32 || dtype == BB_BF16, "bb_act_fwd: bad dtype %d", dtype);
+    BB_REQUIRE(act == BB_ACT_RELU || act == BB_ACT_GELU_TANH, "bb_act_fwd: bad activation %d", act);
+    const int vec = dtype == BB_BF16 ? 8 : 4;
+    BB_REQUIRE(n >= 0 && n % vec == 0 && (n == 0 || (x && out)), "bb_act_fwd: n (%lld) must be a multiple of %d", (long long)n, vec);
+    if (n == 0) return BB_OK;
+    hipStream_t st = (hipStream_t)stream;
+    const int64_t nvec = n / vec;
+    if (dtype == BB_BF16)
+        hipLaunchKernelGGL(act_kernel<bf16>, dim3(grid_for(nvec)), dim3(256), 0, st, nvec, act, (const bf16*)x, (bf16*)out);
+    else
+        hipLaunchKernelGGL(act_kernel<float>, dim3(grid_for(nvec)), dim3(256), 0, st, nvec, act, (const float*)x, (float*)out);
     BB_LAUNCH_CHECK();
     return BB_OK;
 }

@@ -18,6 +18,7 @@
 struct GemmArgs {
     const void* A; const void* B; void* C;
     const void* bias; const void* aux_in; void* aux_out; const void* resid;
+    float* colsum;  // TN only: += column sums of A over K (the bias gradient of a linear layer)
     int64_t lda, ldb, ldc, ldaux;
     int64_t sA1, sA2, sB1, sB2, sC1, sC2;
     int M, N, K, nb2;
@@ -438,12 +439,29 @@ __device__ __forceinline__ void gemm_bf16_dma_body(const GemmArgs& g, const int 
         }
         read_stage = read_stage + 1 == STAGES ? 0 : read_stage + 1;
     };
+    // bias gradient riding along: the waves of the first block column (and first wave column)
+    // add up the A fragments they hold anyway: lane (m, kg) sees 8 of the 16 k values per step
+    const bool do_colsum = AKM && g.colsum != nullptr && tile_n == 0 && wn == 0;
+    float csum[TM];
+#pragma unroll
+    for (int i = 0; i < TM; ++i) csum[i] = 0.f;
     auto mfma_step = [&](const Frags& f, int ks) {
 #pragma unroll
         for (int i = 0; i < TM; ++i)
 #pragma unroll
             for (int j = 0; j < TN; ++j)
                 acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(f.a[ks][i], f.b[ks][j], acc[i][j], 0, 0, 0);
+        if constexpr (AKM) {
+            if (do_colsum) {
+#pragma unroll
+                for (int i = 0; i < TM; ++i) {
+                    float t = 0.f;
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) t += (float)f.a[ks][i][e];
+                    csum[i] += t;
+                }
+            }
+        }
     };
     // Steady state is branch-free: a tile is issued every iteration (past the end of K the
     // sources stop advancing, so the last tile is fetched again into a stage nobody reads),
@@ -495,6 +513,17 @@ __device__ __forceinline__ void gemm_bf16_dma_body(const GemmArgs& g, const int 
             mfma_step(f0, 0);
             mfma_step(f0, 1);
             sync_tile();
+        }
+    }
+
+    if constexpr (AKM) {
+        if (do_colsum) {
+#pragma unroll
+            for (int i = 0; i < TM; ++i) {
+                const float t = csum[i] + __shfl_xor(csum[i], 32, 64);
+                const int m = m0 + wm * WTM + i * 32 + (lane & 31);
+                if (lane < 32 && m < g.M) g.colsum[m] += t;
+            }
         }
     }
 
@@ -807,6 +836,8 @@ static int fill_args(const bb_gemm_desc* d, GemmArgs& g, int64_t& batches, bool&
     BB_REQUIRE(d->lda >= a_contig && d->ldb >= b_contig && d->ldc >= d->N, "bb_gemm: leading dimension too small");
     g.A = d->A; g.B = d->B; g.C = d->C;
     g.bias = d->bias; g.aux_in = d->aux_in; g.aux_out = d->aux_out; g.resid = d->resid;
+    g.colsum = nullptr;
+    BB_REQUIRE(!d->colsum_out || d->layout == BB_TN, "bb_gemm: colsum_out needs the BB_TN layout");
     g.lda = d->lda; g.ldb = d->ldb; g.ldc = d->ldc; g.ldaux = d->ldaux > 0 ? d->ldaux : d->ldc;
     g.sA1 = d->sA1; g.sA2 = d->sA2; g.sB1 = d->sB1; g.sB2 = d->sB2; g.sC1 = d->sC1; g.sC2 = d->sC2;
     g.alpha = d->alpha;
@@ -814,6 +845,16 @@ static int fill_args(const bb_gemm_desc* d, GemmArgs& g, int64_t& batches, bool&
     g.c_f32 = (d->c_dtype == BB_F32);
     g.tiles_m = g.tiles_n = 0;
     return BB_OK;
+}
+
+// The bias-gradient column sums ride inside the DMA kernel when it runs the problem; otherwise
+// the stand-alone reduction computes them.
+static bool colsum_fusable(const bb_gemm_desc* d, int64_t batches) {
+    return d->colsum_out && d->dtype == BB_BF16 && batches == 1 && pick_dma_tile(d->M, d->N, d->K, 1) != D_NONE;
+}
+static int colsum_standalone(const bb_gemm_desc* d, void* stream) {
+    BB_REQUIRE(d->colsum_ws, "bb_gemm: colsum_out on this problem needs colsum_ws");
+    return bb_colsum_acc(d->dtype, d->K, d->M, d->A, d->lda, d->colsum_out, d->colsum_ws, stream);
 }
 
 extern "C" int bb_gemm(const bb_gemm_desc* d, void* stream) {
@@ -824,6 +865,10 @@ extern "C" int bb_gemm(const bb_gemm_desc* d, void* stream) {
     if (rc) return rc;
     if (d->M == 0 || d->N == 0) return BB_OK;
     hipStream_t st = (hipStream_t)stream;
+    if (d->colsum_out) {
+        if (colsum_fusable(d, batches)) g.colsum = d->colsum_out;
+        else if ((rc = colsum_standalone(d, stream)) != BB_OK) return rc;
+    }
     if (d->dtype == BB_BF16) {
         if (!ta && !tb) return dispatch_bf16<false, false>(g, (int)batches, st);
         if (!ta && tb) return dispatch_bf16<false, true>(g, (int)batches, st);
@@ -882,6 +927,7 @@ extern "C" int bb_gemm_grouped(const bb_gemm_desc* descs, int count, void* strea
         bool ta, tb;
         int rc = fill_args(&descs[i], G.p[i], batches, ta, tb);
         if (rc) return rc;
+        if (descs[i].colsum_out) G.p[i].colsum = descs[i].colsum_out;  // every grouped problem runs the DMA kernel
     }
     const int layout = descs[0].layout;
     if (layout == BB_NT) return launch_grouped<false, false>(G, st);

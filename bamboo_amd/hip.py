@@ -25,7 +25,7 @@ LN_CODES = {"standard": LN_STANDARD, "annotated": LN_ANNOTATED}
 EXPORTS = (
     "bb_version", "bb_last_error", "bb_init", "bb_gemm", "bb_gemm_grouped", "bb_gemm_variant", "bb_layernorm_fwd",
     "bb_layernorm_bwd_workspace", "bb_layernorm_bwd", "bb_colsum_workspace", "bb_colsum_acc",
-    "bb_softmax_fwd", "bb_softmax_bwd", "bb_attention_fwd", "bb_attention_bwd", "bb_residual_add", "bb_mse_workspace", "bb_mse_fwd_bwd",
+    "bb_softmax_fwd", "bb_softmax_bwd", "bb_attention_fwd", "bb_attention_bwd", "bb_residual_add", "bb_act_fwd", "bb_mse_workspace", "bb_mse_fwd_bwd",
     "bb_adam_multi", "bb_cast", "bb_fill_f32",
 )
 
@@ -46,7 +46,7 @@ class GemmDesc(Structure):
         ("sC1", c_int64), ("sC2", c_int64),
         ("alpha", c_float), ("epilogue", c_int32), ("act", c_int32), ("accumulate", c_int32),
         ("bias", c_void_p), ("aux_in", c_void_p), ("aux_out", c_void_p), ("resid", c_void_p),
-        ("ldaux", c_int64),
+        ("ldaux", c_int64), ("colsum_out", c_void_p), ("colsum_ws", c_void_p),
     ]
 
 
@@ -89,6 +89,7 @@ def lib():
     L.bb_attention_bwd.argtypes = [c_int] * 6 + [c_void_p, c_void_p, c_void_p, c_int64, c_void_p, c_void_p, c_int64,
                                    c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_void_p, c_void_p]
     L.bb_residual_add.argtypes = [c_int, c_int64, c_void_p, c_void_p, c_void_p, c_void_p]
+    L.bb_act_fwd.argtypes = [c_int, c_int, c_int64, c_void_p, c_void_p, c_void_p]
     L.bb_mse_workspace.restype = c_int64
     L.bb_mse_fwd_bwd.argtypes = [c_int, c_int64, c_void_p, c_void_p, c_void_p, c_float, c_void_p, c_int,
                                  c_void_p, c_void_p]
@@ -137,7 +138,7 @@ def _row_major(t, name):
 
 # ------------------------------------------------------------------------------------- GEMM
 def gemm_desc(layout, A, B, C, *, alpha=1.0, bias=None, epilogue=EPI_NONE, act=ACT_RELU, accumulate=False,
-              aux_in=None, aux_out=None, resid=None):
+              aux_in=None, aux_out=None, resid=None, colsum_out=None, colsum_ws=None):
     """Descriptor of C = epilogue(alpha * op(A) op(B) [+ bias]) on 2-D row-major views."""
     lda, ldb, ldc = _row_major(A, "A"), _row_major(B, "B"), _row_major(C, "C")
     if layout == NT:
@@ -174,6 +175,13 @@ def gemm_desc(layout, A, B, C, *, alpha=1.0, bias=None, epilogue=EPI_NONE, act=A
     d.aux_in = None if aux_in is None else aux_in.data_ptr()
     d.aux_out = None if aux_out is None else aux_out.data_ptr()
     d.resid = None if resid is None else resid.data_ptr()
+    if colsum_out is not None:
+        if layout != TN or colsum_out.dtype != torch.float32 or colsum_out.numel() != M:
+            raise HipKernelError("gemm: colsum_out needs the TN layout and an fp32 [M] vector")
+        if colsum_ws is not None and (colsum_ws.dtype != torch.float32 or colsum_ws.numel() < colsum_workspace(M)):
+            raise HipKernelError("gemm: colsum_ws too small")
+        d.colsum_out = colsum_out.data_ptr()
+        d.colsum_ws = None if colsum_ws is None else colsum_ws.data_ptr()
     return d
 
 
@@ -298,6 +306,10 @@ def attention_bwd(qkv, out, d_out, lse, delta, d_qkv, batch, heads, seq, mask, k
 def residual_add(a, b, out, stream=None):
     check(lib().bb_residual_add(dtype_code(a.dtype), a.numel(), _ptr(a), _ptr(b), _ptr(out), stream_ptr(stream)),
           "bb_residual_add")
+
+
+def act_fwd(x, out, act, stream=None):
+    check(lib().bb_act_fwd(dtype_code(x.dtype), act, x.numel(), _ptr(x), _ptr(out), stream_ptr(stream)), "bb_act_fwd")
 
 
 def mse_workspace():

@@ -233,8 +233,10 @@ class TransformerLayer:
                  epilogue=hip.EPI_RESIDUAL, resid=x, stream=sm)
         hip.layernorm_fwd(st["x1"], w["sublayer.1.norm.a_2"], w["sublayer.1.norm.b_2"], st["n2"], st["mean2"],
                           st["rinv2"], kind, self.eps, stream=sm)
-        hip.gemm(hip.NT, st["n2"], w["feed_forward.w_1.weight"], st["act"], bias=w["feed_forward.w_1.bias"],
-                 epilogue=hip.EPI_ACT, act=act, aux_out=st["u"], stream=sm)
+        # the activation runs as its own bandwidth-bound pass: inside the GEMM epilogue its
+        # transcendental work would sit on the critical path of every tile while the MFMA pipe idles
+        hip.gemm(hip.NT, st["n2"], w["feed_forward.w_1.weight"], st["u"], bias=w["feed_forward.w_1.bias"], stream=sm)
+        hip.act_fwd(st["u"], st["act"], act, stream=sm)
         hip.gemm(hip.NT, st["act"], w["feed_forward.w_2.weight"], st["out"], bias=w["feed_forward.w_2.bias"],
                  epilogue=hip.EPI_RESIDUAL, resid=st["x1"], stream=sm)
         return st["out"]
@@ -250,26 +252,24 @@ class TransformerLayer:
         # weight gradients dW += dy^T x are collected and issued as one grouped launch at the end:
         # each alone has too few output tiles to fill the GPU
         wgrads = []
-        wgrad = lambda dy, x, name: wgrads.append(hip.gemm_desc(hip.TN, dy, x, g[name], accumulate=True))
+        # ... and each carries its bias gradient (column sums of dy) in the same kernel
+        wgrad = lambda dy, x, name: wgrads.append(hip.gemm_desc(
+            hip.TN, dy, x, g[name], accumulate=True, colsum_out=g[name[:-len("weight")] + "bias"], colsum_ws=ws))
         # feed-forward
         wgrad(d_out, st["act"], "feed_forward.w_2.weight")
-        hip.colsum_acc(d_out, g["feed_forward.w_2.bias"], ws, stream=sm)
         hip.gemm(hip.NN, d_out, w["feed_forward.w_2.weight"], d_ffn, epilogue=hip.EPI_DACT, act=act,
                  aux_in=st["u"], stream=sm)
         wgrad(d_ffn, st["n2"], "feed_forward.w_1.weight")
-        hip.colsum_acc(d_ffn, g["feed_forward.w_1.bias"], ws, stream=sm)
         hip.gemm(hip.NN, d_ffn, w["feed_forward.w_1.weight"], d_h0, stream=sm)
         # d_x1 = d_out + LN2'(d_n2)
         hip.layernorm_bwd(st["x1"], w["sublayer.1.norm.a_2"], st["mean2"], st["rinv2"], d_h0, d_out, d_h1,
                           g["sublayer.1.norm.a_2"], g["sublayer.1.norm.b_2"], ws, kind, self.eps, stream=sm)
         # attention output projection
         wgrad(d_h1, st["ctx"], "self_attn.linears.3.weight")
-        hip.colsum_acc(d_h1, g["self_attn.linears.3.bias"], ws, stream=sm)
         hip.gemm(hip.NN, d_h1, w["self_attn.linears.3.weight"], d_h0, stream=sm)
         self._attention_bwd(d_h0, d_qkv, st, ctx)
         # QKV projection
         wgrad(d_qkv, st["n1"], "qkv.weight")
-        hip.colsum_acc(d_qkv, g["qkv.bias"], ws, stream=sm)
         hip.gemm(hip.NN, d_qkv, w["qkv.weight"], d_h0, stream=sm)
         # d_x0 = d_x1 + LN1'(d_n1)
         hip.layernorm_bwd(st["x0"], w["sublayer.0.norm.a_2"], st["mean1"], st["rinv1"], d_h0, d_h1, d_x,

@@ -89,6 +89,13 @@ typedef struct bb_gemm_desc {
     void* aux_out;      /* [M,N], leading dim ldaux */
     const void* resid;  /* [M,N], leading dim ldaux */
     int64_t ldaux;
+    /* BB_TN only: colsum_out[m] += sum_k A[k,m] (fp32, [M]) -- with A = dy this is the bias gradient
+     * of the linear layer whose weight gradient the GEMM computes.  Fused into the GEMM where the
+     * kernel allows; otherwise computed by bb_colsum_acc with colsum_ws (>= bb_colsum_workspace(M)
+     * floats, may be NULL only if the fused path is certain).  Same result either way up to the
+     * fp32 summation order.                                                                */
+    float* colsum_out;
+    float* colsum_ws;
 } bb_gemm_desc;
 
 /* library ------------------------------------------------------------------------------ */
@@ -162,6 +169,10 @@ int bb_attention_bwd(int dtype, int mask, int batch, int heads, int seq, int hea
 /* out = a + b, elementwise (SublayerConnection residual, transformer.py:103).             */
 int bb_residual_add(int dtype, int64_t n, const void* a, const void* b, void* out,
                     void* stream);
+
+/* out = act(x), elementwise: the activation of PositionwiseFeedForward (transformer.py:158) as a
+ * bandwidth-bound pass of its own (2 * n * sizeof(dtype) bytes).                             */
+int bb_act_fwd(int dtype, int act, int64_t n, const void* x, void* out, void* stream);
 
 /* Mean-squared-error head (nn.MSELoss, transformer.py:264) fused with its gradient:
  * loss_out[0] (+)= mean((y-t)^2);  dy = grad_scale * 2 (y-t) / n.  Deterministic two-pass

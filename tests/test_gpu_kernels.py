@@ -282,6 +282,29 @@ def test_residual_add_cast_fill(hiplib, dtype):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name", ["relu", "gelu_tanh"])
+def test_act_fwd(hiplib, dtype, name):
+    x = randn(4096, 96, dtype=dtype, seed=26, scale=3.0)
+    out = torch.empty_like(x)
+    hiplib.act_fwd(x, out, hiplib.ACT_CODES[name])
+    assert rel_err(out, ol.activation(x.double().cpu(), name)) < tol(dtype)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_gemm_fused_bias_gradient(hiplib, dtype):
+    """dW += dy^T x with db += colsum(dy) riding in the same call, fused (bf16, large) or not."""
+    for rows, out_f, in_f in [(512, 256, 384), (96, 40, 72)]:
+        dy, x = randn(rows, out_f, dtype=dtype, seed=27), randn(rows, in_f, dtype=dtype, seed=28)
+        g0, b0 = randn(out_f, in_f, seed=29), randn(out_f, seed=30)
+        g, bgrad = g0.clone(), b0.clone()
+        ws = torch.empty(hiplib.colsum_workspace(out_f), device=DEV)
+        d = hiplib.gemm_desc(hiplib.TN, dy, x, g, accumulate=True, colsum_out=bgrad, colsum_ws=ws)
+        hiplib.gemm_grouped([d])
+        assert rel_err(g, g0.double().cpu() + dy.double().cpu().t() @ x.double().cpu()) < tol(dtype)
+        assert rel_err(bgrad, b0.double().cpu() + dy.double().cpu().sum(0)) < 1e-5
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
 def test_mse(hiplib, dtype):
     n = 4 * 128 * 768
     y, t = randn(n, dtype=dtype, seed=24), randn(n, dtype=dtype, seed=25)
