@@ -302,13 +302,15 @@ class PipelineEngine:
             self._promote(self.r_stage_ids[0], failed_step=0, curr_step=0)
 
     def _handle_next_stage_failure(self, step_i):
+        torch.cuda.synchronize(self.device)   # the pause starts when the work issued before the failure has drained
         t0 = time.perf_counter()
         nxt = self.r_stage_ids[0]
         # failed_step = 0: the in-process queue has seen nothing of the dead successor's traffic
         # with the stage after it, so the replay keeps the successor's sends (the second replay
         # case of the reference, schedule.py:349-353)
         self._promote(nxt, failed_step=0, curr_step=step_i)
-        self.last_failover = {"step": step_i, "host_promote_s": time.perf_counter() - t0}
+        self.last_failover = {"step": step_i, "t_detect": t0, "promote_s": time.perf_counter() - t0}
+        self._replay_until = step_i
 
     def _promote(self, absorbed, failed_step, curr_step):
         """Turn the shadow layers of ``absorbed`` into active layers of this process
@@ -452,6 +454,12 @@ class PipelineEngine:
         when a neighbour failed."""
         self._reserve_pipe_buffers(pipe_schedule.num_pipe_buffers())
         for step_i, step_cmds in enumerate(pipe_schedule):
+            if getattr(self, "_replay_until", None) == step_i:
+                # the successor's lost work has been redone: the stage is back where it was when the
+                # failure was detected (pause = detection -> here, GPU drained)
+                torch.cuda.synchronize(self.device)
+                self.last_failover["pause_s"] = time.perf_counter() - self.last_failover["t_detect"]
+                self._replay_until = None
             if self._debug:
                 self.log(f"step {step_i}: {step_cmds}")
             try:

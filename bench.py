@@ -149,6 +149,8 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-probe", action="store_true", help="do not bracket GEMM launches with events")
     ap.add_argument("--skip-rc-off", action="store_true")
+    ap.add_argument("--failover-at", type=int, default=None,
+                    help="also measure a failover: the successor is preempted at this micro-batch (config c5: 7)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures ONE pipeline stage on ONE GPU; --gpus N>1 is not part of this build", file=sys.stderr)
@@ -194,6 +196,26 @@ def main():
         engine, q = build_engine(cfg, rc=True, rc_stream=True)
         t_on = time_steps(engine, args.steps, args.warmup)
 
+    failover = None
+    if args.failover_at is not None:
+        # the engine of the last leg has run warm-up + timed batches with RC; now lose the successor
+        q.preempt_successor(args.failover_at, STAGE_ID)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        engine.train_batch()
+        torch.cuda.synchronize()
+        t_fail_batch = time.perf_counter() - t0
+        q.revive()
+        t_post = time_steps(engine, args.steps, 1)       # merged own+promoted stream from step 0
+        fo = engine.last_failover
+        failover = {"preempted_at_micro_batch": args.failover_at, "detected_at_step": fo["step"],
+                    "promote_ms": round(fo["promote_s"] * 1e3, 3), "pause_ms": round(fo["pause_s"] * 1e3, 3),
+                    "failover_batch_ms": round(t_fail_batch * 1e3, 3),
+                    "post_failover_samples_per_s": round(samples / t_post, 3),
+                    "post_failover_ms_per_step": round(t_post * 1e3, 3),
+                    "note": "pause = failure detected (GPU drained) -> successor's lost work replayed from the RC stash; "
+                            "post-failover = own + promoted layers as two local stages"}
+
     layer = engine.module.func_buckets[STAGE_ID][0]
     fwd_flops = layer.flops_fwd(cfg["mb"], cfg["seq"]) * cfg["layers"]
     own_flops, rc_flops = 3 * fwd_flops * cfg["M"], fwd_flops * cfg["M"]
@@ -229,6 +251,8 @@ def main():
         "stage_tflops_rc_off": None if t_off is None else round(own_flops / t_off / 1e12, 2),
         "roofline": roofline,
     }
+    if failover is not None:
+        out["failover"] = failover
     if not args.no_cpu_baseline:
         threads = min(os.cpu_count() or 1, 16)
         out["cpu_baseline"] = cpu_baseline(cfg, threads)
