@@ -682,3 +682,299 @@ extern "C" int bb_mse_fwd_bwd(int dtype, int64_t n, const void* y, const void* t
     BB_LAUNCH_CHECK();
     return BB_OK;
 }
+
+// =========================================================================================
+// BatchNorm (training mode, per-channel statistics over all rows of an NHWC activation viewed
+// as [rows = N*H*W, channels]) and the 3x3 patch gather / scatter of the bottleneck block
+// (DeepSpeedExamples/pipeline_parallelism/resnet.py:49-75).
+// =========================================================================================
+constexpr int BN_SPLITS = 64;
+
+// column partial sums of f(x): MODE 0: x ; MODE 1: (x - mean[c])^2 ;
+// MODE 2 (backward): two sums, g and g * xhat, with g = dy * (out > 0 if relu_out given)
+template <typename T, int MODE>
+__global__ __launch_bounds__(256) void bn_colred_kernel(int rows, int cols, const T* __restrict__ x,
+                                                        const float* __restrict__ mean, const float* __restrict__ rstd,
+                                                        const T* __restrict__ dy, const T* __restrict__ relu_out,
+                                                        float* __restrict__ partial) {
+    constexpr int VEC = Elem<T>::VEC;
+    __shared__ float red[3][2][64 * VEC];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int c0 = (blockIdx.x * 64 + lane) * VEC;
+    float a0[VEC], a1[VEC], mu[VEC], rs[VEC];
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) a0[e] = a1[e] = mu[e] = rs[e] = 0.f;
+    if (c0 < cols) {
+        if (MODE >= 1) {
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) mu[e] = mean[c0 + e];
+        }
+        if (MODE == 2) {
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) rs[e] = rstd[c0 + e];
+        }
+        for (int r = blockIdx.y * 4 + wave; r < rows; r += gridDim.y * 4) {
+            float v[VEC];
+            load_vec(x + (int64_t)r * cols + c0, v);
+            if (MODE == 0) {
+#pragma unroll
+                for (int e = 0; e < VEC; ++e) a0[e] += v[e];
+            } else if (MODE == 1) {
+#pragma unroll
+                for (int e = 0; e < VEC; ++e) {
+                    const float d = v[e] - mu[e];
+                    a0[e] += d * d;
+                }
+            } else {
+                float g[VEC];
+                load_vec(dy + (int64_t)r * cols + c0, g);
+                if (relu_out) {
+                    float o[VEC];
+                    load_vec(relu_out + (int64_t)r * cols + c0, o);
+#pragma unroll
+                    for (int e = 0; e < VEC; ++e) g[e] = o[e] > 0.f ? g[e] : 0.f;
+                }
+#pragma unroll
+                for (int e = 0; e < VEC; ++e) {
+                    a0[e] += g[e];
+                    a1[e] += g[e] * (v[e] - mu[e]) * rs[e];
+                }
+            }
+        }
+    }
+    if (wave > 0) {
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) {
+            red[wave - 1][0][lane * VEC + e] = a0[e];
+            red[wave - 1][1][lane * VEC + e] = a1[e];
+        }
+    }
+    __syncthreads();
+    if (wave == 0 && c0 < cols) {
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) {
+            float s0 = a0[e], s1 = a1[e];
+            for (int w = 0; w < 3; ++w) {
+                s0 += red[w][0][lane * VEC + e];
+                s1 += red[w][1][lane * VEC + e];
+            }
+            partial[((int64_t)blockIdx.y * 2) * cols + c0 + e] = s0;
+            partial[((int64_t)blockIdx.y * 2 + 1) * cols + c0 + e] = s1;
+        }
+    }
+}
+
+// finish: sums over the BN_SPLITS partial rows in fixed order.
+// what 0: mean = s0/rows ; 1: rstd = 1/sqrt(s0/rows + eps) (+ running stats) ; 2: dbeta += s0, dgamma += s1,
+// and keep the batch means of g and g*xhat for the apply pass
+__global__ __launch_bounds__(256) void bn_finish_kernel(int what, int rows, int cols, float eps, float momentum,
+                                                        const float* __restrict__ partial, float* __restrict__ mean,
+                                                        float* __restrict__ rstd, float* __restrict__ run_mean,
+                                                        float* __restrict__ run_var, float* __restrict__ dgamma,
+                                                        float* __restrict__ dbeta, float* __restrict__ sums) {
+    const int c = blockIdx.x * 256 + threadIdx.x;
+    if (c >= cols) return;
+    float s0 = 0.f, s1 = 0.f;
+    for (int p = 0; p < BN_SPLITS; ++p) {
+        s0 += partial[((int64_t)p * 2) * cols + c];
+        s1 += partial[((int64_t)p * 2 + 1) * cols + c];
+    }
+    if (what == 0) {
+        mean[c] = s0 / (float)rows;
+    } else if (what == 1) {
+        const float var = s0 / (float)rows;
+        rstd[c] = 1.0f / sqrtf(var + eps);
+        if (run_mean) {  // nn.BatchNorm2d: running_var uses the unbiased estimate
+            run_mean[c] = (1.f - momentum) * run_mean[c] + momentum * mean[c];
+            run_var[c] = (1.f - momentum) * run_var[c] + momentum * var * (float)rows / (float)(rows - 1);
+        }
+    } else {
+        dbeta[c] += s0;
+        dgamma[c] += s1;
+        sums[c] = s0 / (float)rows;
+        sums[cols + c] = s1 / (float)rows;
+    }
+}
+
+// forward apply: y = gamma * (x - mean) * rstd + beta (+ resid), optional ReLU
+template <typename T>
+__global__ __launch_bounds__(256) void bn_apply_kernel(int64_t nvec, int cols, int relu, const T* __restrict__ x,
+                                                       const float* __restrict__ mean, const float* __restrict__ rstd,
+                                                       const T* __restrict__ gamma, const T* __restrict__ beta,
+                                                       const T* __restrict__ resid, T* __restrict__ y) {
+    constexpr int VEC = Elem<T>::VEC;
+    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < nvec; i += (int64_t)gridDim.x * 256) {
+        const int c0 = (int)((i * VEC) % cols);
+        float v[VEC], g[VEC], b[VEC];
+        load_vec(x + i * VEC, v);
+        load_vec(gamma + c0, g);
+        load_vec(beta + c0, b);
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) v[e] = g[e] * ((v[e] - mean[c0 + e]) * rstd[c0 + e]) + b[e];
+        if (resid) {
+            float r[VEC];
+            load_vec(resid + i * VEC, r);
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) v[e] += r[e];
+        }
+        if (relu) {
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) v[e] = fmaxf(v[e], 0.f);
+        }
+        store_vec(y + i * VEC, v);
+    }
+}
+
+// backward apply: g = dy * (relu_out > 0); dx = gamma * rstd * (g - mean(g) - xhat * mean(g * xhat));
+// optionally also writes g itself (the gradient that flows into the residual branch)
+template <typename T>
+__global__ __launch_bounds__(256) void bn_bwd_apply_kernel(int64_t nvec, int cols, const T* __restrict__ x,
+                                                           const float* __restrict__ mean, const float* __restrict__ rstd,
+                                                           const T* __restrict__ gamma, const float* __restrict__ sums,
+                                                           const T* __restrict__ dy, const T* __restrict__ relu_out,
+                                                           T* __restrict__ dx, T* __restrict__ g_out) {
+    constexpr int VEC = Elem<T>::VEC;
+    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < nvec; i += (int64_t)gridDim.x * 256) {
+        const int c0 = (int)((i * VEC) % cols);
+        float v[VEC], g[VEC], gm[VEC], o[VEC];
+        load_vec(x + i * VEC, v);
+        load_vec(dy + i * VEC, g);
+        load_vec(gamma + c0, gm);
+        if (relu_out) {
+            float ro[VEC];
+            load_vec(relu_out + i * VEC, ro);
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) g[e] = ro[e] > 0.f ? g[e] : 0.f;
+        }
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) {
+            const float xh = (v[e] - mean[c0 + e]) * rstd[c0 + e];
+            o[e] = gm[e] * rstd[c0 + e] * (g[e] - sums[c0 + e] - xh * sums[cols + c0 + e]);
+        }
+        store_vec(dx + i * VEC, o);
+        if (g_out) store_vec(g_out + i * VEC, g);
+    }
+}
+
+extern "C" int64_t bb_bn_workspace(int cols) { return (int64_t)BN_SPLITS * 2 * cols + 2 * cols; }
+
+static int check_bn(const char* name, int dtype, int rows, int cols) {
+    BB_REQUIRE(dtype == BB_F32 || dtype == BB_BF16, "%s: bad dtype %d", name, dtype);
+    const int vec = dtype == BB_BF16 ? 8 : 4;
+    BB_REQUIRE(rows > 1 && cols > 0 && cols % vec == 0, "%s: bad shape %d x %d", name, rows, cols);
+    return BB_OK;
+}
+
+extern "C" int bb_batchnorm_fwd(int dtype, int rows, int cols, float eps, float momentum, int relu, const void* x,
+                                const void* gamma, const void* beta, const void* resid, void* y, float* mean,
+                                float* rstd, float* running_mean, float* running_var, float* workspace, void* stream) {
+    int rc = check_bn("bb_batchnorm_fwd", dtype, rows, cols);
+    if (rc) return rc;
+    BB_REQUIRE(x && gamma && beta && y && mean && rstd && workspace, "bb_batchnorm_fwd: null pointer");
+    BB_REQUIRE((running_mean == nullptr) == (running_var == nullptr), "bb_batchnorm_fwd: give both running buffers or none");
+    hipStream_t st = (hipStream_t)stream;
+    const int vec = dtype == BB_BF16 ? 8 : 4;
+    dim3 grid((cols + 64 * vec - 1) / (64 * vec), BN_SPLITS), fgrid((cols + 255) / 256);
+    const int64_t nvec = (int64_t)rows * cols / vec;
+    if (dtype == BB_BF16) {
+        hipLaunchKernelGGL((bn_colred_kernel<bf16, 0>), grid, dim3(256), 0, st, rows, cols, (const bf16*)x, nullptr, nullptr, nullptr, nullptr, workspace);
+        hipLaunchKernelGGL(bn_finish_kernel, fgrid, dim3(256), 0, st, 0, rows, cols, eps, momentum, workspace, mean, rstd, nullptr, nullptr, nullptr, nullptr, nullptr);
+        hipLaunchKernelGGL((bn_colred_kernel<bf16, 1>), grid, dim3(256), 0, st, rows, cols, (const bf16*)x, mean, nullptr, nullptr, nullptr, workspace);
+        hipLaunchKernelGGL(bn_finish_kernel, fgrid, dim3(256), 0, st, 1, rows, cols, eps, momentum, workspace, mean, rstd, running_mean, running_var, nullptr, nullptr, nullptr);
+        hipLaunchKernelGGL(bn_apply_kernel<bf16>, dim3(grid_for(nvec)), dim3(256), 0, st, nvec, cols, relu, (const bf16*)x, mean, rstd, (const bf16*)gamma, (const bf16*)beta, (const bf16*)resid, (bf16*)y);
+    } else {
+        hipLaunchKernelGGL((bn_colred_kernel<float, 0>), grid, dim3(256), 0, st, rows, cols, (const float*)x, nullptr, nullptr, nullptr, nullptr, workspace);
+        hipLaunchKernelGGL(bn_finish_kernel, fgrid, dim3(256), 0, st, 0, rows, cols, eps, momentum, workspace, mean, rstd, nullptr, nullptr, nullptr, nullptr, nullptr);
+        hipLaunchKernelGGL((bn_colred_kernel<float, 1>), grid, dim3(256), 0, st, rows, cols, (const float*)x, mean, nullptr, nullptr, nullptr, workspace);
+        hipLaunchKernelGGL(bn_finish_kernel, fgrid, dim3(256), 0, st, 1, rows, cols, eps, momentum, workspace, mean, rstd, running_mean, running_var, nullptr, nullptr, nullptr);
+        hipLaunchKernelGGL(bn_apply_kernel<float>, dim3(grid_for(nvec)), dim3(256), 0, st, nvec, cols, relu, (const float*)x, mean, rstd, (const float*)gamma, (const float*)beta, (const float*)resid, (float*)y);
+    }
+    BB_LAUNCH_CHECK();
+    return BB_OK;
+}
+
+extern "C" int bb_batchnorm_bwd(int dtype, int rows, int cols, const void* x, const void* gamma, const float* mean,
+                                const float* rstd, const void* dy, const void* relu_out, void* dx, void* g_out,
+                                float* dgamma, float* dbeta, float* workspace, void* stream) {
+    int rc = check_bn("bb_batchnorm_bwd", dtype, rows, cols);
+    if (rc) return rc;
+    BB_REQUIRE(x && gamma && mean && rstd && dy && dx && dgamma && dbeta && workspace, "bb_batchnorm_bwd: null pointer");
+    hipStream_t st = (hipStream_t)stream;
+    const int vec = dtype == BB_BF16 ? 8 : 4;
+    dim3 grid((cols + 64 * vec - 1) / (64 * vec), BN_SPLITS), fgrid((cols + 255) / 256);
+    const int64_t nvec = (int64_t)rows * cols / vec;
+    float* sums = workspace + (int64_t)BN_SPLITS * 2 * cols;
+    if (dtype == BB_BF16) {
+        hipLaunchKernelGGL((bn_colred_kernel<bf16, 2>), grid, dim3(256), 0, st, rows, cols, (const bf16*)x, mean, rstd, (const bf16*)dy, (const bf16*)relu_out, workspace);
+        hipLaunchKernelGGL(bn_finish_kernel, fgrid, dim3(256), 0, st, 2, rows, cols, 0.f, 0.f, workspace, nullptr, nullptr, nullptr, nullptr, dgamma, dbeta, sums);
+        hipLaunchKernelGGL(bn_bwd_apply_kernel<bf16>, dim3(grid_for(nvec)), dim3(256), 0, st, nvec, cols, (const bf16*)x, mean, rstd, (const bf16*)gamma, sums, (const bf16*)dy, (const bf16*)relu_out, (bf16*)dx, (bf16*)g_out);
+    } else {
+        hipLaunchKernelGGL((bn_colred_kernel<float, 2>), grid, dim3(256), 0, st, rows, cols, (const float*)x, mean, rstd, (const float*)dy, (const float*)relu_out, workspace);
+        hipLaunchKernelGGL(bn_finish_kernel, fgrid, dim3(256), 0, st, 2, rows, cols, 0.f, 0.f, workspace, nullptr, nullptr, nullptr, nullptr, dgamma, dbeta, sums);
+        hipLaunchKernelGGL(bn_bwd_apply_kernel<float>, dim3(grid_for(nvec)), dim3(256), 0, st, nvec, cols, (const float*)x, mean, rstd, (const float*)gamma, sums, (const float*)dy, (const float*)relu_out, (float*)dx, (float*)g_out);
+    }
+    BB_LAUNCH_CHECK();
+    return BB_OK;
+}
+
+// 3x3, stride 1, pad 1 patch gather on NHWC: col[p][tap*C + c] = x[n, y+dy, x+dx, c] (0 outside), and its
+// adjoint as a gather (every input pixel sums the nine patch entries that referenced it: no atomics)
+template <typename T, bool ADJOINT>
+__global__ __launch_bounds__(256) void patch3x3_kernel(int n, int h, int w, int c, const T* __restrict__ src,
+                                                       T* __restrict__ dst) {
+    constexpr int VEC = Elem<T>::VEC;
+    const int cv = c / VEC;
+    const int64_t pixels = (int64_t)n * h * w;
+    const int64_t total = ADJOINT ? pixels * cv : pixels * 9 * cv;
+    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < total; i += (int64_t)gridDim.x * 256) {
+        if (!ADJOINT) {
+            const int ch = (int)(i % cv) * VEC;
+            const int tap = (int)((i / cv) % 9);
+            const int64_t p = i / (cv * 9);
+            const int px = (int)(p % w), py = (int)((p / w) % h);
+            const int sy = py + tap / 3 - 1, sx = px + tap % 3 - 1;
+            float v[VEC];
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) v[e] = 0.f;
+            if (sy >= 0 && sy < h && sx >= 0 && sx < w) load_vec(src + (p + (int64_t)(sy - py) * w + (sx - px)) * c + ch, v);
+            store_vec(dst + (p * 9 + tap) * c + ch, v);
+        } else {
+            const int ch = (int)(i % cv) * VEC;
+            const int64_t p = i / cv;
+            const int px = (int)(p % w), py = (int)((p / w) % h);
+            float acc[VEC];
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) acc[e] = 0.f;
+#pragma unroll
+            for (int tap = 0; tap < 9; ++tap) {
+                // patch of pixel q = p - shift(tap) holds x[p] at position tap
+                const int qy = py - (tap / 3 - 1), qx = px - (tap % 3 - 1);
+                if (qy >= 0 && qy < h && qx >= 0 && qx < w) {
+                    float v[VEC];
+                    load_vec(src + ((p + (int64_t)(qy - py) * w + (qx - px)) * 9 + tap) * c + ch, v);
+#pragma unroll
+                    for (int e = 0; e < VEC; ++e) acc[e] += v[e];
+                }
+            }
+            store_vec(dst + p * c + ch, acc);
+        }
+    }
+}
+
+extern "C" int bb_patch3x3(int dtype, int adjoint, int n, int h, int w, int c, const void* src, void* dst, void* stream) {
+    BB_REQUIRE(dtype == BB_F32 || dtype == BB_BF16, "bb_patch3x3: bad dtype %d", dtype);
+    const int vec = dtype == BB_BF16 ? 8 : 4;
+    BB_REQUIRE(n > 0 && h > 0 && w > 0 && c > 0 && c % vec == 0 && src && dst, "bb_patch3x3: bad arguments");
+    hipStream_t st = (hipStream_t)stream;
+    const int64_t items = (int64_t)n * h * w * (adjoint ? 1 : 9) * (c / vec);
+    dim3 grid(grid_for(items));
+    if (dtype == BB_BF16) {
+        if (adjoint) hipLaunchKernelGGL((patch3x3_kernel<bf16, true>), grid, dim3(256), 0, st, n, h, w, c, (const bf16*)src, (bf16*)dst);
+        else hipLaunchKernelGGL((patch3x3_kernel<bf16, false>), grid, dim3(256), 0, st, n, h, w, c, (const bf16*)src, (bf16*)dst);
+    } else {
+        if (adjoint) hipLaunchKernelGGL((patch3x3_kernel<float, true>), grid, dim3(256), 0, st, n, h, w, c, (const float*)src, (float*)dst);
+        else hipLaunchKernelGGL((patch3x3_kernel<float, false>), grid, dim3(256), 0, st, n, h, w, c, (const float*)src, (float*)dst);
+    }
+    BB_LAUNCH_CHECK();
+    return BB_OK;
+}

@@ -100,7 +100,8 @@ class PipelineEngine:
         self.ctx = model.prepare_context(built, self.batch, self.seq, stream=self.main_stream)
         self.rc_ctx = self.ctx
         if self.rc_stream is not None:
-            self.rc_ctx = model.prepare_context([], self.batch, self.seq, stream=self.rc_stream)
+            self.rc_ctx = model.prepare_context(self.r_stage_ids, self.batch, self.seq, stream=self.rc_stream,
+                                                forward_only=True)
         self.stash_bytes = 0
         for sid in built:
             self.stash_bytes += model.allocate_stash(sid, self.ctx, self.micro_batches)
@@ -394,6 +395,7 @@ class PipelineEngine:
         redundant = stage_id in self.r_stage_ids
         ctx = self.rc_ctx if redundant else self.ctx
         ctx.key_len = self.queue.key_len(buffer_id)
+        ctx.redundant = redundant
         if redundant and self.rc_stream is not None:
             self.rc_stream.wait_event(self._fwd_done[buffer_id])
         out = self.module.forward(inputs, stage_id, slot=buffer_id, ctx=ctx)

@@ -25,7 +25,7 @@ LN_CODES = {"standard": LN_STANDARD, "annotated": LN_ANNOTATED}
 EXPORTS = (
     "bb_version", "bb_last_error", "bb_init", "bb_gemm", "bb_gemm_grouped", "bb_gemm_variant", "bb_layernorm_fwd",
     "bb_layernorm_bwd_workspace", "bb_layernorm_bwd", "bb_colsum_workspace", "bb_colsum_acc",
-    "bb_softmax_fwd", "bb_softmax_bwd", "bb_attention_fwd", "bb_attention_bwd", "bb_residual_add", "bb_act_fwd", "bb_mse_workspace", "bb_mse_fwd_bwd",
+    "bb_softmax_fwd", "bb_softmax_bwd", "bb_attention_fwd", "bb_attention_bwd", "bb_residual_add", "bb_act_fwd", "bb_bn_workspace", "bb_batchnorm_fwd", "bb_batchnorm_bwd", "bb_patch3x3", "bb_mse_workspace", "bb_mse_fwd_bwd",
     "bb_adam_multi", "bb_cast", "bb_fill_f32",
 )
 
@@ -90,6 +90,11 @@ def lib():
                                    c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_void_p, c_void_p]
     L.bb_residual_add.argtypes = [c_int, c_int64, c_void_p, c_void_p, c_void_p, c_void_p]
     L.bb_act_fwd.argtypes = [c_int, c_int, c_int64, c_void_p, c_void_p, c_void_p]
+    L.bb_bn_workspace.argtypes = [c_int]
+    L.bb_bn_workspace.restype = c_int64
+    L.bb_batchnorm_fwd.argtypes = [c_int, c_int, c_int, c_float, c_float, c_int] + [c_void_p] * 11
+    L.bb_batchnorm_bwd.argtypes = [c_int, c_int, c_int] + [c_void_p] * 12
+    L.bb_patch3x3.argtypes = [c_int, c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p]
     L.bb_mse_workspace.restype = c_int64
     L.bb_mse_fwd_bwd.argtypes = [c_int, c_int64, c_void_p, c_void_p, c_void_p, c_float, c_void_p, c_int,
                                  c_void_p, c_void_p]
@@ -310,6 +315,33 @@ def residual_add(a, b, out, stream=None):
 
 def act_fwd(x, out, act, stream=None):
     check(lib().bb_act_fwd(dtype_code(x.dtype), act, x.numel(), _ptr(x), _ptr(out), stream_ptr(stream)), "bb_act_fwd")
+
+
+def bn_workspace(cols):
+    return int(lib().bb_bn_workspace(cols))
+
+
+def batchnorm_fwd(x, gamma, beta, resid, y, mean, rstd, run_mean, run_var, workspace, eps, momentum, relu, stream=None):
+    rows, cols = x.shape
+    if workspace.numel() < bn_workspace(cols):
+        raise HipKernelError("batchnorm_fwd: workspace too small")
+    check(lib().bb_batchnorm_fwd(dtype_code(x.dtype), rows, cols, eps, momentum, int(relu), _ptr(x), _ptr(gamma),
+                                 _ptr(beta), _ptr(resid), _ptr(y), _ptr(mean), _ptr(rstd), _ptr(run_mean),
+                                 _ptr(run_var), _ptr(workspace), stream_ptr(stream)), "bb_batchnorm_fwd")
+
+
+def batchnorm_bwd(x, gamma, mean, rstd, dy, relu_out, dx, g_out, dgamma, dbeta, workspace, stream=None):
+    rows, cols = x.shape
+    if workspace.numel() < bn_workspace(cols):
+        raise HipKernelError("batchnorm_bwd: workspace too small")
+    check(lib().bb_batchnorm_bwd(dtype_code(x.dtype), rows, cols, _ptr(x), _ptr(gamma), _ptr(mean), _ptr(rstd),
+                                 _ptr(dy), _ptr(relu_out), _ptr(dx), _ptr(g_out), _ptr(dgamma), _ptr(dbeta),
+                                 _ptr(workspace), stream_ptr(stream)), "bb_batchnorm_bwd")
+
+
+def patch3x3(src, dst, n, h, w, c, adjoint=False, stream=None):
+    check(lib().bb_patch3x3(dtype_code(src.dtype), int(adjoint), n, h, w, c, _ptr(src), _ptr(dst), stream_ptr(stream)),
+          "bb_patch3x3")
 
 
 def mse_workspace():

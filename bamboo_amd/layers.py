@@ -33,6 +33,7 @@ class StageContext:
         self.scratch = {}
         self.key_len = None
         self.workspace = None
+        self.redundant = False   # set per forward call: a redundant forward must not touch running statistics
 
     @property
     def rows(self):
@@ -127,8 +128,9 @@ class TransformerLayer:
         self.w, self.g = w, g
 
     # ------------------------------------------------------------------ memory plans
-    def out_shape(self, in_shape):
-        return in_shape
+    @property
+    def feature_dim(self):
+        return self.hidden
 
     def fused_attention(self, ctx):
         """bf16 runs the fused attention kernels (no score matrix in HBM); fp32, the correctness
@@ -276,6 +278,147 @@ class TransformerLayer:
                           g["sublayer.0.norm.a_2"], g["sublayer.0.norm.b_2"], ws, kind, self.eps, stream=sm)
         # d_out, d_ffn, d_h1 and d_qkv still hold the four output gradients here
         hip.gemm_grouped(wgrads, stream=sm)
+        return d_x
+
+
+class BottleNeck:
+    """ResNet bottleneck block ``ReLU(BN(conv1x1(ReLU(BN(conv3x3(ReLU(BN(conv1x1 x)))))) + x)`` with the
+    identity shortcut (reference ``BottleNeck``, DeepSpeedExamples/pipeline_parallelism/resnet.py:49-75:
+    stride 1 and ``in_channels == 4 * out_channels``), on NHWC activations viewed as
+    ``[rows = N*H*W, channels]``.  The 1x1 convolutions are plain GEMMs on that view; the 3x3
+    convolution is a GEMM over the gathered patch matrix ``[rows, 9*C]``.  Parameter names are the
+    reference's; the 3x3 weight is kept as ``[out, 3, 3, in]`` (tap-major, channel-minor) so that it is the
+    ``[out, 9*in]`` GEMM operand as it lies in memory (the reference holds ``[out, in, 3, 3]``)."""
+
+    def __init__(self, in_channels, out_channels, stride=1, height=14, width=14, bn_eps=1e-5, bn_momentum=0.1):
+        if stride != 1 or in_channels != 4 * out_channels:
+            raise NotImplementedError("only the identity-shortcut bottleneck (stride 1, in = 4 * out) is built")
+        self.cin, self.cmid, self.h, self.w = in_channels, out_channels, height, width
+        self.eps, self.momentum = bn_eps, bn_momentum
+        self.w_ = self.g_ = None
+        self.running = None
+
+    @property
+    def feature_dim(self):
+        return self.cin
+
+    def param_specs(self):
+        ci, cm = self.cin, self.cmid
+        return OrderedDict([
+            ("residual_function.0.weight", (cm, ci)),
+            ("residual_function.1.weight", (cm,)), ("residual_function.1.bias", (cm,)),
+            ("residual_function.3.weight", (cm, 3, 3, cm)),
+            ("residual_function.4.weight", (cm,)), ("residual_function.4.bias", (cm,)),
+            ("residual_function.6.weight", (ci, cm)),
+            ("residual_function.7.weight", (ci,)), ("residual_function.7.bias", (ci,)),
+        ])
+
+    def num_params(self):
+        return sum(math.prod(s) for s in self.param_specs().values())
+
+    @staticmethod
+    def to_native(name, tensor):
+        """Reference layout -> arena layout: conv weights [O, I, kh, kw] -> [O, kh, kw, I]."""
+        if tensor.dim() == 4:
+            t = tensor.permute(0, 2, 3, 1).contiguous()
+            return t.view(t.shape[0], -1) if t.shape[1] == 1 else t
+        return tensor
+
+    def init_params(self, master, seed):
+        """He-normal convolution weights (std = sqrt(2 / fan_in)) from per-tensor seeded generators drawn in
+        the reference's [O, I, kh, kw] layout, BN gain 1 / shift 0."""
+        ref_shapes = {"residual_function.0.weight": (self.cmid, self.cin, 1, 1),
+                      "residual_function.3.weight": (self.cmid, self.cmid, 3, 3),
+                      "residual_function.6.weight": (self.cin, self.cmid, 1, 1)}
+        for i, name in enumerate(self.param_specs()):
+            t = master[name]
+            if name in ref_shapes:
+                shape = ref_shapes[name]
+                g = torch.Generator().manual_seed(seed * 1000 + i)
+                wt = torch.randn(shape, generator=g, dtype=torch.float32) * math.sqrt(2.0 / (shape[1] * shape[2] * shape[3]))
+                t.copy_(self.to_native(name, wt).view(t.shape))
+            elif name.endswith("weight"):
+                t.fill_(1.0)
+            else:
+                t.zero_()
+
+    def bind(self, compute, grads):
+        self.w_, self.g_ = dict(compute), dict(grads)
+        for d in (self.w_, self.g_):
+            d["conv2"] = d["residual_function.3.weight"].view(self.cmid, 9 * self.cmid)
+
+    def stash_specs(self, ctx):
+        R, ci, cm = ctx.rows, self.cin, self.cmid
+        dt, f32 = ctx.dtype, torch.float32
+        return [("y1", (R, cm), dt), ("a1", (R, cm), dt), ("y2", (R, cm), dt), ("a2", (R, cm), dt),
+                ("y3", (R, ci), dt), ("out", (R, ci), dt),
+                ("mean1", (cm,), f32), ("rstd1", (cm,), f32), ("mean2", (cm,), f32), ("rstd2", (cm,), f32),
+                ("mean3", (ci,), f32), ("rstd3", (ci,), f32)]
+
+    def scratch_specs(self, ctx):
+        R, ci, cm = ctx.rows, self.cin, self.cmid
+        dt = ctx.dtype
+        return [("col", (R, 9 * cm), dt), ("d_col", (R, 9 * cm), dt), ("d_y3", (R, ci), dt), ("d_res", (R, ci), dt),
+                ("d_m0", (R, cm), dt), ("d_m1", (R, cm), dt)]
+
+    def forward_scratch_specs(self, ctx):
+        return [("col", (ctx.rows, 9 * self.cmid), ctx.dtype)]
+
+    def workspace_elems(self):
+        return max(hip.bn_workspace(self.cin), hip.colsum_workspace(self.cin))
+
+    def flops_fwd(self, batch, seq):
+        return 2 * batch * seq * (self.cin * self.cmid + 9 * self.cmid * self.cmid + self.cmid * self.cin)
+
+    def _running(self, device):
+        if self.running is None:
+            z = lambda n, v: torch.full((n,), v, dtype=torch.float32, device=device)
+            self.running = {i: (z(n, 0.0), z(n, 1.0)) for i, n in ((1, self.cmid), (4, self.cmid), (7, self.cin))}
+        return self.running
+
+    def _bn_fwd(self, idx, x, resid, y, mean, rstd, relu, ctx):
+        run = (None, None) if ctx.redundant else self._running(x.device)[idx]
+        hip.batchnorm_fwd(x, self.w_[f"residual_function.{idx}.weight"], self.w_[f"residual_function.{idx}.bias"],
+                          resid, y, mean, rstd, run[0], run[1], ctx.workspace, self.eps, self.momentum, relu,
+                          stream=ctx.stream)
+
+    def forward(self, x, st, ctx):
+        if ctx.seq != self.h * self.w:
+            raise hip.HipKernelError(f"activation has {ctx.seq} positions, the block expects {self.h}x{self.w}")
+        w, sm = self.w_, ctx.stream
+        st["x0"] = x
+        col = ctx.buf("col", (ctx.rows, 9 * self.cmid))
+        hip.gemm(hip.NT, x, w["residual_function.0.weight"], st["y1"], stream=sm)
+        self._bn_fwd(1, st["y1"], None, st["a1"], st["mean1"], st["rstd1"], True, ctx)
+        hip.patch3x3(st["a1"], col, ctx.batch, self.h, self.w, self.cmid, stream=sm)
+        hip.gemm(hip.NT, col, w["conv2"], st["y2"], stream=sm)
+        self._bn_fwd(4, st["y2"], None, st["a2"], st["mean2"], st["rstd2"], True, ctx)
+        hip.gemm(hip.NT, st["a2"], w["residual_function.6.weight"], st["y3"], stream=sm)
+        self._bn_fwd(7, st["y3"], x, st["out"], st["mean3"], st["rstd3"], True, ctx)
+        return st["out"]
+
+    def backward(self, d_out, d_x, st, ctx):
+        w, g, sm, ws = self.w_, self.g_, ctx.stream, ctx.workspace
+        R, ci, cm = ctx.rows, self.cin, self.cmid
+        col, d_col = ctx.buf("col", (R, 9 * cm)), ctx.buf("d_col", (R, 9 * cm))
+        d_y3, d_res = ctx.buf("d_y3", (R, ci)), ctx.buf("d_res", (R, ci))
+        d_m0, d_m1 = ctx.buf("d_m0", (R, cm)), ctx.buf("d_m1", (R, cm))
+        bn = lambda idx, xk, mk, rk, dy, relu_out, dx, g_out: hip.batchnorm_bwd(
+            st[xk], w[f"residual_function.{idx}.weight"], st[mk], st[rk], dy, relu_out, dx, g_out,
+            g[f"residual_function.{idx}.weight"], g[f"residual_function.{idx}.bias"], ws, stream=sm)
+        # final ReLU + BN3; d_res keeps the masked gradient for the identity shortcut
+        bn(7, "y3", "mean3", "rstd3", d_out, st["out"], d_y3, d_res)
+        hip.gemm(hip.NN, d_y3, w["residual_function.6.weight"], d_m0, stream=sm)          # d_a2
+        bn(4, "y2", "mean2", "rstd2", d_m0, st["a2"], d_m1, None)                          # d_y2
+        hip.patch3x3(st["a1"], col, ctx.batch, self.h, self.w, cm, stream=sm)              # patches again: cheaper than stashing
+        hip.gemm(hip.NN, d_m1, w["conv2"], d_col, stream=sm)
+        d_a1 = ctx.buf("d_m0", (R, cm))
+        hip.gemm_grouped([hip.gemm_desc(hip.TN, d_y3, st["a2"], g["residual_function.6.weight"], accumulate=True),
+                          hip.gemm_desc(hip.TN, d_m1, col, g["conv2"], accumulate=True)], stream=sm)
+        hip.patch3x3(d_col, d_a1, ctx.batch, self.h, self.w, cm, adjoint=True, stream=sm)
+        bn(1, "y1", "mean1", "rstd1", d_a1, st["a1"], d_m1, None)                          # d_y1
+        hip.gemm(hip.TN, d_m1, st["x0"], g["residual_function.0.weight"], accumulate=True, stream=sm)
+        hip.gemm(hip.NN, d_m1, w["residual_function.0.weight"], d_x, epilogue=hip.EPI_RESIDUAL, resid=d_res, stream=sm)
         return d_x
 
 

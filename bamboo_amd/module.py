@@ -103,10 +103,15 @@ class StageParams:
             hip.cast(self.master, self.compute)
 
     def load(self, named_tensors):
-        """Copy ``{"{layer_idx}.{name}": tensor}`` into the master arena (missing keys are left)."""
+        """Copy ``{"{layer_idx}.{name}": tensor}`` into the master arena (missing keys are left).  Tensors in
+        the reference's layout (4-D convolution weights) are converted by the layer's ``to_native``."""
         for k, t in named_tensors.items():
             if k in self.index:
-                self.view(self.master, k).copy_(t.to(torch.float32))
+                dst = self.view(self.master, k)
+                layer = self.layers[int(k.split(".", 1)[0]) - self.first_layer_idx]
+                if tuple(t.shape) != tuple(dst.shape) and hasattr(layer, "to_native"):
+                    t = layer.to_native(k.split(".", 1)[1], t)
+                dst.copy_(t.to(torch.float32).reshape(dst.shape))
         self.refresh_compute()
 
 
@@ -308,15 +313,20 @@ class PipelineModule:
             d = dst
         return grad_input
 
-    def prepare_context(self, stage_ids, batch, seq, stream=None):
-        """Execution context with scratch sized for the largest layer of the given stages."""
+    def prepare_context(self, stage_ids, batch, seq, stream=None, forward_only=False):
+        """Execution context with scratch sized for the largest layer of the given stages
+        (``forward_only``: a lane that only runs redundant forwards needs no backward scratch)."""
         ctx = StageContext(batch, seq, self.dtype, self.device, stream)
         ws = 0
         for sid in stage_ids:
             for layer in self.func_buckets[sid]:
-                ctx.ensure_scratch(layer.scratch_specs(ctx))
+                if hasattr(layer, "forward_scratch_specs"):
+                    ctx.ensure_scratch(layer.forward_scratch_specs(ctx))
                 ws = max(ws, layer.workspace_elems())
-                h = layer.out_shape((ctx.rows, layer.hidden))
+                if forward_only:
+                    continue
+                ctx.ensure_scratch(layer.scratch_specs(ctx))
+                h = (ctx.rows, layer.feature_dim)
                 ctx.ensure_scratch([("d_layer0", h, self.dtype), ("d_layer1", h, self.dtype)])
         ctx.ensure_workspace(ws)
         return ctx

@@ -30,6 +30,8 @@ CONFIGS = {
     "c3": dict(hidden=1024, heads=16, ffn=4096, layers=4, seq=512, mb=16, M=12, dtype="bf16",
                variant=dict(activation="gelu_tanh", ln="standard", mask="key_padding"), grad_mode="queue",
                key_len_range=(128, 512), label="BERT-large stage 4+4 layers h1024 s512 mb16 M12 bf16"),
+    "c4": dict(kind="resnet", hidden=1024, mid=256, side=14, layers=12, seq=196, mb=32, M=8, dtype="bf16",
+               grad_mode="queue", label="ResNet-152 conv4_x stage 12+12 bottleneck blocks 1024-256-256-1024 @14x14 mb32 M8 bf16 NHWC"),
     "c5": dict(hidden=1600, heads=25, ffn=6400, layers=8, seq=1024, mb=4, M=16, dtype="bf16",
                variant=dict(activation="gelu_tanh", ln="standard", mask="causal"), grad_mode="queue",
                label="GPT-2-1.5B stage 8+8 layers h1600 s1024 mb4 M16 bf16"),
@@ -42,10 +44,14 @@ def build_engine(cfg, rc, rc_stream, seed=1138):
     import torch
 
     import bamboo_amd
-    from bamboo_amd import LayerSpec, PipelineModule, SeededActivationQueue, TransformerLayer
+    from bamboo_amd import BottleNeck, LayerSpec, PipelineModule, SeededActivationQueue, TransformerLayer
     dtype = torch.bfloat16 if cfg["dtype"] == "bf16" else torch.float32
-    specs = [LayerSpec(TransformerLayer, cfg["hidden"], cfg["heads"], cfg["ffn"], **cfg["variant"])
-             for _ in range(cfg["layers"] * STAGES)]
+    if cfg.get("kind") == "resnet":
+        specs = [LayerSpec(BottleNeck, cfg["hidden"], cfg["mid"], height=cfg["side"], width=cfg["side"])
+                 for _ in range(cfg["layers"] * STAGES)]
+    else:
+        specs = [LayerSpec(TransformerLayer, cfg["hidden"], cfg["heads"], cfg["ffn"], **cfg["variant"])
+                 for _ in range(cfg["layers"] * STAGES)]
     model = PipelineModule(specs, num_stages=STAGES, partition_method="uniform", stage_id=STAGE_ID, dtype=dtype,
                            device="cuda:0")
     q = SeededActivationQueue((cfg["mb"], cfg["seq"], cfg["hidden"]), dtype, cfg["M"],
@@ -112,7 +118,11 @@ def cpu_baseline(cfg, threads):
     from oracle import layers as ol
     from oracle.stage import OracleStage
     torch.set_num_threads(threads)
-    ocfg = ol.TransformerCfg(hidden=cfg["hidden"], heads=cfg["heads"], ffn=cfg["ffn"], **cfg["variant"])
+    if cfg.get("kind") == "resnet":
+        ocfg = ol.BottleneckCfg(in_channels=cfg["hidden"], mid_channels=cfg["mid"])
+        cfg = dict(cfg, variant={"mask": "none"})
+    else:
+        ocfg = ol.TransformerCfg(hidden=cfg["hidden"], heads=cfg["heads"], ffn=cfg["ffn"], **cfg["variant"])
     parts = [i * cfg["layers"] for i in range(STAGES + 1)]
     st = OracleStage(ocfg, parts, STAGE_ID, cfg["M"], dtype=torch.float32, redundancy_level=1, eager=True)
     g = torch.Generator().manual_seed(1)
@@ -149,6 +159,9 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-probe", action="store_true", help="do not bracket GEMM launches with events")
     ap.add_argument("--skip-rc-off", action="store_true")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="first run three 256 MiB fp32 copies (cast_kernel<float,float>): the known-size kernel that "
+                         "FETCH_SIZE / WRITE_SIZE counters of a --pmc run are scaled by")
     ap.add_argument("--failover-at", type=int, default=None,
                     help="also measure a failover: the successor is preempted at this micro-batch (config c5: 7)")
     args = ap.parse_args()
@@ -161,6 +174,13 @@ def main():
     from bamboo_amd import hip
     cfg = CONFIGS[args.config]
     samples = cfg["mb"] * cfg["M"]
+    if args.calibrate_copy:
+        src = torch.ones(64 * 1024 * 1024, dtype=torch.float32, device="cuda:0")
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            hip.cast(src, dst)
+        torch.cuda.synchronize()
+        del src, dst
 
     # leg 1: RC off (plain 1F1B stream of the stage)
     t_off = None
@@ -241,7 +261,8 @@ def main():
         "vs_baseline": None, "dtype": cfg["dtype"], "data": "synthetic",
         "config": {"workload": cfg["label"], "stage": f"{STAGE_ID} of {STAGES}", "redundancy_level": 1,
                    "eager_recovery": True, "rc_stream": bool(args.rc_stream), "samples_per_step": samples,
-                   "attention": "fused (no score matrix in HBM); flops counted dense, the causal kernel skips masked tiles"},
+                   "attention": "n/a (convolutions as GEMMs over NHWC rows, 3x3 via patch matrix)" if cfg.get("kind") == "resnet"
+                   else "fused (no score matrix in HBM); flops counted dense, the causal kernel skips masked tiles"},
         "rc_on_samples_per_s": round(samples / t_on, 3),
         "rc_off_samples_per_s": None if t_off is None else round(samples / t_off, 3),
         "rc_overhead_pct": None if t_off is None else round(100.0 * (t_on - t_off) / t_off, 2),

@@ -174,6 +174,28 @@ int bb_residual_add(int dtype, int64_t n, const void* a, const void* b, void* ou
  * bandwidth-bound pass of its own (2 * n * sizeof(dtype) bytes).                             */
 int bb_act_fwd(int dtype, int act, int64_t n, const void* x, void* out, void* stream);
 
+/* BatchNorm2d in training mode on an NHWC activation viewed as [rows = N*H*W, cols = channels]
+ * (resnet.py:56,59,62): per-channel batch mean and biased variance (two passes), then
+ * y = gamma * (x - mean) * rstd + beta (+ resid) with optional ReLU (the block's final
+ * ReLU(residual_function(x) + shortcut(x)), resnet.py:75).  mean / rstd: fp32 [cols], kept for the
+ * backward.  running_mean / running_var (both or neither; may be NULL for a redundant forward,
+ * which must not update them) follow nn.BatchNorm2d (momentum, unbiased running variance).
+ * workspace: fp32, >= bb_bn_workspace(cols).                                                  */
+int64_t bb_bn_workspace(int cols);
+int bb_batchnorm_fwd(int dtype, int rows, int cols, float eps, float momentum, int relu, const void* x,
+                     const void* gamma, const void* beta, const void* resid, void* y, float* mean,
+                     float* rstd, float* running_mean, float* running_var, float* workspace, void* stream);
+/* Backward through (optional ReLU given by its output relu_out) and the batch normalisation:
+ * g = dy * (relu_out > 0); dgamma += sum g*xhat; dbeta += sum g;
+ * dx = gamma * rstd * (g - mean(g) - xhat * mean(g*xhat)); g_out (optional) receives g.       */
+int bb_batchnorm_bwd(int dtype, int rows, int cols, const void* x, const void* gamma, const float* mean,
+                     const float* rstd, const void* dy, const void* relu_out, void* dx, void* g_out,
+                     float* dgamma, float* dbeta, float* workspace, void* stream);
+/* 3x3 / stride 1 / pad 1 patch matrix of an NHWC tensor: col[p, tap*C + c] = x[n, y+dy, x+dx, c]
+ * (adjoint = 0), or its adjoint dx[p, c] = sum of the patch entries that read x[p, c]
+ * (adjoint = 1); turns nn.Conv2d(k=3, padding=1) (resnet.py:58) and its input gradient into GEMMs. */
+int bb_patch3x3(int dtype, int adjoint, int n, int h, int w, int c, const void* src, void* dst, void* stream);
+
 /* Mean-squared-error head (nn.MSELoss, transformer.py:264) fused with its gradient:
  * loss_out[0] (+)= mean((y-t)^2);  dy = grad_scale * 2 (y-t) / n.  Deterministic two-pass
  * reduction; workspace: fp32, at least bb_mse_workspace() elements.                       */

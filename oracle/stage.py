@@ -78,13 +78,25 @@ class OracleStage:
         self.step_count = 0
 
     def build(self, stage):
+        conv = isinstance(self.cfg, olayers.BottleneckCfg)
         layers = []
         for li in range(self.parts[stage], self.parts[stage + 1]):
-            p = olayers.init_params(self.cfg, self.base_seed + li, dtype=self.dtype)
+            if conv:
+                p = olayers.init_bottleneck_params(self.cfg, self.base_seed + li, dtype=self.dtype)
+            else:
+                p = olayers.init_params(self.cfg, self.base_seed + li, dtype=self.dtype)
             layers.append({k: v.requires_grad_(True) for k, v in p.items()})
         self.params[stage] = layers
 
     def forward(self, x, stage, key_lens=None):
+        if isinstance(self.cfg, olayers.BottleneckCfg):
+            # activations travel as [batch, H*W, C] (NHWC); torch convolutions want NCHW
+            b, hw, c = x.shape
+            side = int(round(hw ** 0.5))
+            y = x.view(b, side, side, c).permute(0, 3, 1, 2)
+            for p in self.params[stage]:
+                y = olayers.bottleneck(y, p, self.cfg)
+            return y.permute(0, 2, 3, 1).reshape(b, hw, c)
         for p in self.params[stage]:
             x = olayers.transformer_layer(x, p, self.cfg, key_lens)
         return x

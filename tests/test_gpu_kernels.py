@@ -305,6 +305,68 @@ def test_gemm_fused_bias_gradient(hiplib, dtype):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("rows,cols,relu,with_resid", [(144, 16, True, False), (6272, 256, True, False), (500, 64, True, True), (144, 64, False, False)])
+def test_batchnorm_fwd_bwd(hiplib, dtype, rows, cols, relu, with_resid):
+    x = randn(rows, cols, dtype=dtype, seed=31, scale=2.0) + 0.5
+    gamma = (1 + 0.1 * randn(cols, seed=32)).to(dtype)
+    beta = (0.1 * randn(cols, seed=33)).to(dtype)
+    resid = randn(rows, cols, dtype=dtype, seed=34) if with_resid else None
+    dy = randn(rows, cols, dtype=dtype, seed=35)
+    y = torch.empty_like(x)
+    mean, rstd = torch.empty(cols, device=DEV), torch.empty(cols, device=DEV)
+    rm, rv = torch.zeros(cols, device=DEV), torch.ones(cols, device=DEV)
+    ws = torch.empty(hiplib.bn_workspace(cols), device=DEV)
+    hiplib.batchnorm_fwd(x, gamma, beta, resid, y, mean, rstd, rm, rv, ws, 1e-5, 0.1, relu)
+    xr = x.double().cpu().requires_grad_(True)
+    gr, br = gamma.double().cpu().requires_grad_(True), beta.double().cpu().requires_grad_(True)
+    rm_ref, rv_ref = torch.zeros(cols, dtype=torch.float64), torch.ones(cols, dtype=torch.float64)
+    z = torch.nn.functional.batch_norm(xr, rm_ref, rv_ref, gr, br, training=True, momentum=0.1, eps=1e-5)
+    if with_resid:
+        z = z + resid.double().cpu()
+    yr = torch.relu(z) if relu else z
+    assert rel_err(y, yr.detach()) < tol(dtype)
+    assert rel_err(rm, rm_ref) < 1e-5 and rel_err(rv, rv_ref) < 1e-4
+    yr.backward(dy.double().cpu())
+    dx, g_out = torch.empty_like(x), torch.empty_like(x)
+    dg0, db0 = randn(cols, seed=36), randn(cols, seed=37)
+    dg, db = dg0.clone(), db0.clone()
+    hiplib.batchnorm_bwd(x, gamma, mean, rstd, dy, y if relu else None, dx, g_out, dg, db, ws)
+    t = tol(dtype) * (1 if dtype == torch.float32 else 1.5)
+    assert rel_err(dx, xr.grad) < max(t, 1e-4)
+    assert rel_err(dg - dg0, gr.grad) < max(t, 1e-4) and rel_err(db - db0, br.grad) < max(t, 1e-4)
+    mask = (yr.detach() > 0) if relu else torch.ones_like(yr, dtype=torch.bool)
+    assert rel_err(g_out, dy.double().cpu() * mask) < tol(dtype)
+    # a redundant forward (no running buffers) leaves the statistics untouched and gives the same output
+    y2 = torch.empty_like(y)
+    rm2 = rm.clone()
+    hiplib.batchnorm_fwd(x, gamma, beta, resid, y2, mean, rstd, None, None, ws, 1e-5, 0.1, relu)
+    assert torch.equal(y, y2) and torch.equal(rm, rm2)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_patch3x3_and_adjoint(hiplib, dtype):
+    n, h, w, c = 3, 5, 7, 16
+    x = randn(n * h * w, c, dtype=dtype, seed=38)
+    col = torch.empty(n * h * w, 9 * c, dtype=dtype, device=DEV)
+    hiplib.patch3x3(x, col, n, h, w, c)
+    xn = x.float().cpu().view(n, h, w, c).permute(0, 3, 1, 2)
+    ref = torch.nn.functional.unfold(xn, 3, padding=1)                      # [n, c*9, h*w], (c, tap) order
+    ref = ref.view(n, c, 9, h * w).permute(0, 3, 2, 1).reshape(n * h * w, 9 * c)
+    assert torch.equal(col.float().cpu(), ref)
+    # conv3x3 == patches @ W^T with W in [out, tap, in] order
+    wt = randn(8, c, 3, 3, seed=39).cpu()
+    conv = torch.nn.functional.conv2d(xn, wt, padding=1).permute(0, 2, 3, 1).reshape(n * h * w, 8)
+    assert rel_err(col.float().cpu() @ wt.permute(0, 2, 3, 1).reshape(8, 9 * c).t(), conv) < 1e-5
+    # adjoint: <patch(x), d> == <x, adjoint(d)>
+    d = randn(n * h * w, 9 * c, dtype=dtype, seed=40)
+    back = torch.empty_like(x)
+    hiplib.patch3x3(d, back, n, h, w, c, adjoint=True)
+    dn = d.float().cpu().view(n, h * w, 9, c).permute(0, 3, 2, 1).reshape(n, c * 9, h * w)
+    fold = torch.nn.functional.fold(dn, (h, w), 3, padding=1).permute(0, 2, 3, 1).reshape(n * h * w, c)
+    assert rel_err(back, fold) < (1e-6 if dtype == torch.float32 else 1e-2)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
 def test_mse(hiplib, dtype):
     n = 4 * 128 * 768
     y, t = randn(n, dtype=dtype, seed=24), randn(n, dtype=dtype, seed=25)
