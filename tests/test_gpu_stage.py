@@ -266,6 +266,53 @@ def test_resnet_stage_matches_oracle_with_rc(hiplib, dtype):
         assert float(layer.running[1][0].abs().max()) > 0
 
 
+@pytest.mark.parametrize("dead_from", [0, 2])
+def test_lazy_recovery_failover(hiplib, dead_from):
+    """redundancy_level=1 without eager recovery: no redundant forwards (only pings); the shadow stage exists
+    as CPU parameter mirrors and is materialised at the failover, its forwards are recomputed in the replay."""
+    rel_err.lowp = False
+    hid, heads, ffn, L, S, sid, mb, M, seq = 128, 2, 256, 2, 4, 1, 2, 4, 64
+    dtype = torch.float32
+    engine, q = build(hid, heads, ffn, L, S, sid, mb, M, seq, dtype, GPT_VARIANT, 1, False, grad_mode="mse")
+    assert engine.r_stage_ids == [sid + 1] and (sid + 1) not in engine.module.func_buckets
+    assert all(t.device.type == "cpu" and float(t.abs().max()) == 0 for t in engine.param_buffers[sid + 1].values())
+    # what a weight synchronisation would have put into the mirrors: the successor's parameters
+    specs = [LayerSpec(TransformerLayer, hid, heads, ffn, **GPT_VARIANT) for _ in range(L * S)]
+    succ = PipelineModule(specs, num_stages=S, partition_method="uniform", stage_id=sid + 1, dtype=dtype, device=DEV)
+    for name, p in succ.get_named_param(sid + 1):
+        engine.param_buffers[sid + 1][name].copy_(p.cpu())
+    st, peer = oracle_for(engine, q, GPT_VARIANT, hid, heads, ffn, L, S, sid, M, 1, False)
+    true_grads = []
+    st.build(sid + 1)
+    for k in range(M):
+        o1 = st.forward(peer.activations[k], sid).detach().requires_grad_(True)
+        (torch.nn.functional.mse_loss(st.forward(o1, sid + 1), peer.targets[sid + 1][k]) / M).backward()
+        true_grads.append(o1.grad)
+    for s_ in st.params.values():
+        for p in s_:
+            for t in p.values():
+                t.grad = None
+    peer.targets = {sid + 1: peer.targets[sid + 1]}
+    peer.grads = {sid: true_grads}
+    peer.dead_from, peer.dead_stage = dead_from, sid
+    st.run_batch(peer, optimizer_step=False)
+
+    q.set_grads(sid, [g.view(mb, seq, hid) for g in true_grads])
+    q.targets.pop(sid)
+    orig_send = q.send_activation
+    q.send_activation = lambda k, t, stage_id, stream=None: (q._check_alive(k, stage_id) if stage_id == sid
+                                                              else orig_send(k, t, stage_id, stream=stream))
+    q.preempt_successor(dead_from, sid)
+    with NoStep(engine):
+        loss = engine.train_batch()
+    assert engine.stage_ids == [sid, sid + 1]
+    for s_ in (sid, sid + 1):
+        ref = st.named_grads(s_)
+        for name, g in engine.module.get_named_grad(s_):
+            assert rel_err(g, ref[name], grad_floor(ref)) < 1e-4, (s_, name)
+    assert abs(float(loss) - float(peer.loss) / M) < 1e-4 * max(1.0, float(peer.loss) / M)
+
+
 def test_optimizer_step_matches_oracle(hiplib):
     rel_err.lowp = False
     hid, heads, ffn, L, S, sid, mb, M, seq = 128, 2, 256, 2, 4, 1, 2, 4, 64
