@@ -300,6 +300,20 @@ typedef __attribute__((address_space(3))) void lds_ptr_t;
 typedef const __attribute__((address_space(1))) void gbl_ptr_t;
 typedef __attribute__((ext_vector_type(4))) short s16x4;
 
+// Ask the machine scheduler for "one MFMA, then its share of NMEM memory instructions" NMFMA times:
+// the memory instructions of a region (LDS fragment reads or DMA issues) are spread between the
+// MFMAs instead of being bunched in front of a full wait.
+template <int NMFMA, int NMEM, int MEM_MASK> __device__ __forceinline__ void interleave_mfma_with() {
+    static_for(
+        [&](auto idx) {
+            constexpr int i = decltype(idx)::value;
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+            constexpr int n = (NMEM * (i + 1)) / NMFMA - (NMEM * i) / NMFMA;
+            if constexpr (n > 0) __builtin_amdgcn_sched_group_barrier(MEM_MASK, n, 0);
+        },
+        std::make_integer_sequence<int, NMFMA>{});
+}
+
 template <int N> __device__ __forceinline__ void wait_vmcnt_lgkm0() {
     // s_waitcnt vmcnt(N) lgkmcnt(0): vmcnt[3:0] | expcnt(7) << 4 | lgkmcnt << 8 | vmcnt[5:4] << 14
     __builtin_amdgcn_s_waitcnt((N & 15) | (7 << 4) | (0 << 8) | ((N >> 4) << 14));
@@ -490,12 +504,15 @@ __device__ __forceinline__ void gemm_bf16_dma_body(const GemmArgs& g, const int 
         // fragments of tile kt+1 are fetched while the second half of tile kt is multiplied,
         // into the other register set
         auto body = [&](int kt, Frags& cur, Frags& nxt) {
+            constexpr int FRAG_READS = 2 * (TM * (AKM ? 2 : 1) + TN * (BKM ? 2 : 1));
             stop_at_end(kt + STAGES);
             issue_tile();
             mfma_step(cur, 0);
+            interleave_mfma_with<TM * TN, LOADS, 0x020>();   // DMA issues between the first-half MFMAs
             sync_tile();
             load_frags(nxt);
             mfma_step(cur, 1);
+            interleave_mfma_with<TM * TN, FRAG_READS, 0x100>();  // next tile's fragment reads between the rest
         };
         load_frags(f0);
         int kt = 0;
@@ -737,9 +754,10 @@ static int launch_bf16_dma(GemmArgs& g, int batches, hipStream_t st) {
 
 // DMA kernels need K % 32 == 0 and at least one full vector of rows; tile by problem size
 enum DmaTile { D_NONE = 0, D256x256, D256x128, D128x128, D_OFF, D256x256w8, D256x128w8, D256x256w8db, D256x128w8db,
-               D256x128w8s3, D128x128s3 };
+               D256x128w8s3, D128x128s3, D256x256w8s5, D256x128w8s6, D256x256w8s3, D256x128w4s3 };
 static const char* const kDmaTileNames[] = {"", "dma256x256", "dma256x128", "dma128x128", "", "dma256x256w8", "dma256x128w8",
-                                            "dma256x256w8db", "dma256x128w8db", "dma256x128w8s3", "dma128x128s3"};
+                                            "dma256x256w8db", "dma256x128w8db", "dma256x128w8s3", "dma128x128s3",
+                                            "dma256x256w8s5", "dma256x128w8s6", "dma256x256w8s3", "dma256x128w4s3"};
 // BB_DMA_TILE (tuning aid): 1..3 force a DMA tile where it is legal, 4 disables the DMA kernels.
 static int dma_tile_override() {
     static const int v = [] {
@@ -752,7 +770,7 @@ static DmaTile pick_dma_tile(int M, int N, int K, int64_t batches) {
     if (K % 32 != 0 || K < 64 || M < 128 || N < 128 || N % 8 != 0) return D_NONE;
     const int ov = dma_tile_override();
     if (ov == 4) return D_NONE;
-    if ((ov >= 1 && ov <= 3) || (ov >= 5 && ov <= 10)) return (DmaTile)ov;
+    if ((ov >= 1 && ov <= 3) || (ov >= 5 && ov <= 14)) return (DmaTile)ov;
     // measured on MI355X (256 CUs): 256x256 tiles pay off from two full rounds of blocks on,
     // 256x128 from one round, smaller problems take 128x128 tiles with two blocks per CU
     const int64_t t256 = (int64_t)((M + 255) / 256) * ((N + 255) / 256) * batches;
@@ -773,6 +791,10 @@ template <bool TA, bool TB> static int dispatch_bf16(GemmArgs& g, int batches, h
         case D256x128w8db: return launch_bf16_dma<256, 128, 4, 2, TA, TB, true>(g, batches, st);
         case D256x128w8s3: return launch_bf16_dma<256, 128, 4, 2, TA, TB, true, 3>(g, batches, st);
         case D128x128s3: return launch_bf16_dma<128, 128, 2, 2, TA, TB, true, 3>(g, batches, st);
+        case D256x256w8s5: return launch_bf16_dma<256, 256, 2, 4, TA, TB, true, 5>(g, batches, st);
+        case D256x128w8s6: return launch_bf16_dma<256, 128, 4, 2, TA, TB, true, 6>(g, batches, st);
+        case D256x256w8s3: return launch_bf16_dma<256, 256, 2, 4, TA, TB, true, 3>(g, batches, st);
+        case D256x128w4s3: return launch_bf16_dma<256, 128, 2, 2, TA, TB, true, 3>(g, batches, st);
         default: break;
     }
     switch (pick_bf16_tile(g.M, g.N, batches)) {

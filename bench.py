@@ -272,6 +272,16 @@ def main():
         "stage_tflops_rc_off": None if t_off is None else round(own_flops / t_off / 1e12, 2),
         "roofline": roofline,
     }
+    if t_off is not None:
+        # What the same work costs inside a real S-stage 1F1B pipeline, where each stage idles for
+        # (S-1) forward+backward slots per batch and the redundant forwards fall into that idle time
+        # (lock-step model; slot = t_off / M): only the part of the RC time that exceeds the bubbles delays
+        # the batch.  Modelled from the measured times above, not measured itself.
+        slot = t_off / cfg["M"]
+        idle = (STAGES - 1) * slot
+        model = lambda t_with_rc: round(100.0 * max(0.0, (t_with_rc - t_off) - idle) / (t_off + idle), 2)
+        out["rc_overhead_bubble_model_pct"] = {"stages": STAGES, "single_stream": model(t_on_serial),
+                                               "second_stream": model(t_on)}
     if failover is not None:
         out["failover"] = failover
     if not args.no_cpu_baseline:
