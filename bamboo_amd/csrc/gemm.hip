@@ -544,36 +544,41 @@ __device__ __forceinline__ void gemm_bf16_dma_body(const GemmArgs& g, const int 
         }
     }
 
-    // Epilogue through LDS: every wave parks one 32x32 accumulator tile at a time in a private
-    // [32][36] fp32 patch, then lane l takes 16 consecutive columns of row l/2 so that global
-    // loads and stores are 16-byte vectors along rows.
+    // Epilogue through LDS: every wave parks two horizontally adjacent 32x32 accumulator tiles in a
+    // private [32][64 (+4 pad)] fp32 patch; then one wave instruction covers 8 rows x 64 columns, lane l
+    // taking 8 consecutive columns of row l/8, so every global load / store of the epilogue moves whole
+    // 128-byte row segments (256 bytes for fp32 outputs).
+    static_assert(TN % 2 == 0, "the epilogue walks the accumulator tiles in pairs");
     __syncthreads();
-    float* patch = (float*)smem + wave * (32 * 36);
-    const int prow = lane >> 1, pcol = (lane & 1) * 16;
+    constexpr int PLD = 68;
+    float* patch = (float*)smem + wave * (32 * PLD);
+    const int prow = lane >> 3, pcol = (lane & 7) * 8;
     static_for(
         [&](auto idx) {
-            constexpr int i = decltype(idx)::value / TN, j = decltype(idx)::value % TN;
+            constexpr int i = decltype(idx)::value / (TN / 2), jp = decltype(idx)::value % (TN / 2);
 #pragma unroll
-            for (int r = 0; r < 16; ++r)
-                patch[(8 * (r >> 2) + 4 * (lane >> 5) + (r & 3)) * 36 + (lane & 31)] = acc[i][j][r] * g.alpha;
+            for (int h = 0; h < 2; ++h)
+#pragma unroll
+                for (int r = 0; r < 16; ++r)
+                    patch[(8 * (r >> 2) + 4 * (lane >> 5) + (r & 3)) * PLD + h * 32 + (lane & 31)] = acc[i][jp * 2 + h][r] * g.alpha;
             asm volatile("" ::: "memory");
-            const int m = m0 + wm * WTM + i * 32 + prow;
-            const int n = n0 + wn * WTN + j * 32 + pcol;
+            const int n = n0 + wn * WTN + jp * 64 + pcol;
 #pragma unroll
-            for (int h = 0; h < 2; ++h) {
+            for (int it = 0; it < 4; ++it) {
+                const int m = m0 + wm * WTM + i * 32 + it * 8 + prow;
                 float v[8];
-                const f32x4 lo = *(const f32x4*)(patch + prow * 36 + pcol + h * 8);
-                const f32x4 hi = *(const f32x4*)(patch + prow * 36 + pcol + h * 8 + 4);
+                const f32x4 lo = *(const f32x4*)(patch + (it * 8 + prow) * PLD + pcol);
+                const f32x4 hi = *(const f32x4*)(patch + (it * 8 + prow) * PLD + pcol + 4);
 #pragma unroll
                 for (int e = 0; e < 4; ++e) {
                     v[e] = lo[e];
                     v[4 + e] = hi[e];
                 }
-                if (m < g.M && n + h * 8 < g.N) epilogue_vec8(g, coff, m, n + h * 8, v);
+                if (m < g.M && n < g.N) epilogue_vec8(g, coff, m, n, v);
             }
             asm volatile("" ::: "memory");
         },
-        std::make_integer_sequence<int, TM * TN>{});
+        std::make_integer_sequence<int, TM * TN / 2>{});
 }
 
 template <int BM, int BN, int WM, int WN, bool AKM, bool BKM, bool DB, int STAGES>
