@@ -123,6 +123,7 @@ __global__ __launch_bounds__(256) void attn_fwd_kernel(const AttnArgs a) {
     else if (a.mask == BB_MASK_KEY_PADDING) kv_end = min(a.seq, a.key_len[b]);
     const int ntiles = (kv_end + 63) / 64;
     const int my_limit = kv_limit(a, b, myq);
+    const int wave_min_limit = kv_limit(a, b, q0);  // limits grow with the query index
 
     bf16x8 qf[4];
     {
@@ -171,36 +172,44 @@ __global__ __launch_bounds__(256) void attn_fwd_kernel(const AttnArgs a) {
                 for (int ks = 0; ks < 4; ++ks)
                     s[u] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frag_kc(kt, u * 32, ks, lane), qf[ks], s[u], 0, 0, 0);
             }
-            // scale, mask, running max
+            // running max on the raw scores (the scale is positive), masking only on tiles that
+            // reach past the first key some query of this wave may not see
+            const bool need_mask = kv0 + 64 > wave_min_limit;
             float tmax = -INFINITY;
+            if (need_mask) {
+#pragma unroll
+                for (int u = 0; u < 2; ++u)
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) {
+                        const int kv = kv0 + u * 32 + acc_row(r, lane);
+                        s[u][r] = kv < my_limit ? s[u][r] : -INFINITY;
+                    }
+            }
 #pragma unroll
             for (int u = 0; u < 2; ++u)
 #pragma unroll
-                for (int r = 0; r < 16; ++r) {
-                    const int kv = kv0 + u * 32 + acc_row(r, lane);
-                    const float x = kv < my_limit ? s[u][r] * a.scale_log2 : -INFINITY;
-                    s[u][r] = x;
-                    tmax = fmaxf(tmax, x);
-                }
-            tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
+                for (int r = 0; r < 16; ++r) tmax = fmaxf(tmax, s[u][r]);
+            tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64)) * a.scale_log2;
             const float mnew = fmaxf(m, tmax);
             const float msafe = mnew == -INFINITY ? 0.f : mnew;
-            const float alpha = exp2f(m - msafe);  // m = -inf -> 0
+            const float alpha = __builtin_amdgcn_exp2f(m - msafe);  // m = -inf -> 0
             float psum = 0.f;
 #pragma unroll
             for (int u = 0; u < 2; ++u)
 #pragma unroll
                 for (int r = 0; r < 16; ++r) {
-                    const float p = exp2f(s[u][r] - msafe);
+                    const float p = __builtin_amdgcn_exp2f(fmaf(s[u][r], a.scale_log2, -msafe));
                     s[u][r] = p;
                     psum += p;
                 }
             lsum = lsum * alpha + psum;
             m = mnew;
+            if (__any(alpha != 1.0f)) {  // wave-uniform: once the maxima have settled nothing is rescaled
 #pragma unroll
-            for (int t2 = 0; t2 < 2; ++t2)
+                for (int t2 = 0; t2 < 2; ++t2)
 #pragma unroll
-                for (int r = 0; r < 16; ++r) o[t2][r] *= alpha;
+                    for (int r = 0; r < 16; ++r) o[t2][r] *= alpha;
+            }
             // O^T += V^T P^T
 #pragma unroll
             for (int kk = 0; kk < 4; ++kk) {
@@ -347,7 +356,7 @@ __global__ __launch_bounds__(256) void attn_bwd_dkv_kernel(const AttnArgs a) {
                     const int q = t * 64 + ql + e;
                     bool keep = mykv < pad_limit && q < a.seq;
                     if (a.mask == BB_MASK_CAUSAL) keep = keep && mykv <= q;
-                    const float p = keep ? exp2f(s[r] * a.scale_log2 - l4[e]) : 0.f;
+                    const float p = keep ? __builtin_amdgcn_exp2f(fmaf(s[r], a.scale_log2, -l4[e])) : 0.f;
                     s[r] = p;
                     dp[r] = p * (dp[r] - d4[e]);
                 }
@@ -457,7 +466,7 @@ __global__ __launch_bounds__(256) void attn_bwd_dq_kernel(const AttnArgs a) {
 #pragma unroll
                 for (int r = 0; r < 16; ++r) {
                     const int kv = kv0 + u * 32 + acc_row(r, lane);
-                    const float p = kv < my_limit ? exp2f(s[r] * a.scale_log2 - my_lse) : 0.f;
+                    const float p = kv < my_limit ? __builtin_amdgcn_exp2f(fmaf(s[r], a.scale_log2, -my_lse)) : 0.f;
                     dp[r] = p * (dp[r] - my_delta);
                 }
                 // dQ^T += K^T dS^T (contraction over the 32 keys of this sub-tile)
