@@ -47,6 +47,25 @@ __device__ __forceinline__ void dma_rows8(const bf16* gbase, int64_t ld, int row
     const int gr = min(row0 + r, last_row);
     __builtin_amdgcn_global_load_lds((gbl_ptr_t*)(gbase + (int64_t)gr * ld + c * 8), (lds_ptr_t*)(tile + idx * 1024), 16, 0, 0);
 }
+// Whole 64-row tile: this wave's two instructions (row groups wave and wave + 4).  Full tiles
+// take a wave-uniform base plus the lane's fixed offset; only a tile that reaches past the last
+// row pays for per-lane clamping.
+struct LaneOff { uint32_t o0, o1; };
+__device__ __forceinline__ LaneOff lane_off(int64_t ld, int wave, int lane) {
+    const int r0 = wave * 8 + (lane >> 3), r1 = r0 + 32;
+    return {(uint32_t)(r0 * ld + (((lane & 7) ^ fsw(r0)) << 3)), (uint32_t)(r1 * ld + (((lane & 7) ^ fsw(r1)) << 3))};
+}
+__device__ __forceinline__ void dma_tile64(const bf16* gbase, int64_t ld, int row0, int last_row, unsigned char* tile,
+                                           int wave, int lane, LaneOff lo) {
+    if (row0 + 63 <= last_row) {
+        const bf16* g = gbase + (int64_t)row0 * ld;
+        __builtin_amdgcn_global_load_lds((gbl_ptr_t*)(g + lo.o0), (lds_ptr_t*)(tile + wave * 1024), 16, 0, 0);
+        __builtin_amdgcn_global_load_lds((gbl_ptr_t*)(g + lo.o1), (lds_ptr_t*)(tile + (wave + 4) * 1024), 16, 0, 0);
+    } else {
+        dma_rows8(gbase, ld, row0, last_row, tile, wave, lane);
+        dma_rows8(gbase, ld, row0, last_row, tile, wave + 4, lane);
+    }
+}
 // 4-byte variant for the per-row fp32 statistics: 64 consecutive floats
 __device__ __forceinline__ void dma_f32x64(const float* gbase, int idx0, int last, unsigned char* dst, int lane) {
     const int i = min(idx0 + lane, last);
@@ -101,14 +120,29 @@ __device__ __forceinline__ int kv_limit(const AttnArgs& a, int b, int q) {
     return a.seq;
 }
 
+// Block -> (row block, batch*head) map for a 1-D grid of 8 * ceil(nbh / 8) * nblk blocks.  The
+// hardware deals consecutive block ids round-robin over the 8 XCDs, so the low three bits of
+// the id pick the XCD.  Each XCD is given whole (batch, head) pairs - all their row blocks, so
+// the pair's K and V stay in that XCD's L2 - and, under a causal mask, the same mix of long and
+// short blocks as every other XCD, longest first (rank 0 = most work).
+struct BlockMap { int rank, bh; };
+__device__ __forceinline__ BlockMap map_block(int nbh) {
+    const int per_xcd = (nbh + 7) >> 3;
+    const int xcd = blockIdx.x & 7, j = blockIdx.x >> 3;
+    return {j / per_xcd, (j % per_xcd) * 8 + xcd};
+}
+static unsigned attn_grid(int seq, int nbh) { return (unsigned)(8 * ((nbh + 7) / 8) * ((seq + 127) / 128)); }
+
 // =========================================================================================
 // forward: block = 128 queries (4 waves x 32), loop over 64-key tiles
 // =========================================================================================
-__global__ __launch_bounds__(256) void attn_fwd_kernel(const AttnArgs a) {
+__global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const AttnArgs a) {
     __shared__ __attribute__((aligned(16))) unsigned char smem[2 * 2 * 8192];  // 2 stages x (K, V)
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int qb = gridDim.x - 1 - blockIdx.x;  // long (late) query blocks first
-    const int b = blockIdx.y / a.heads, head = blockIdx.y % a.heads;
+    const BlockMap bm = map_block(a.batch * a.heads);
+    if (bm.bh >= a.batch * a.heads) return;
+    const int qb = (a.seq + 127) / 128 - 1 - bm.rank;  // long (late) query blocks first
+    const int b = bm.bh / a.heads, head = bm.bh % a.heads;
     const int64_t row_base = (int64_t)b * a.seq;
     const bf16* Q = a.q + row_base * a.ld_qkv + head * 64;
     const bf16* K = a.k + row_base * a.ld_qkv + head * 64;
@@ -138,13 +172,12 @@ __global__ __launch_bounds__(256) void attn_fwd_kernel(const AttnArgs a) {
         for (int r = 0; r < 16; ++r) o[t][r] = 0.f;
     float m = -INFINITY, lsum = 0.f;
 
+    const LaneOff lo = lane_off(a.ld_qkv, wave, lane);
     auto issue = [&](int t) {
         unsigned char* st = smem + (t & 1) * 16384;
         const int kv0 = t * 64;
-        dma_rows8(K, a.ld_qkv, kv0, last, st, wave, lane);
-        dma_rows8(K, a.ld_qkv, kv0, last, st, wave + 4, lane);
-        dma_rows8(V, a.ld_qkv, kv0, last, st + 8192, wave, lane);
-        dma_rows8(V, a.ld_qkv, kv0, last, st + 8192, wave + 4, lane);
+        dma_tile64(K, a.ld_qkv, kv0, last, st, wave, lane, lo);
+        dma_tile64(V, a.ld_qkv, kv0, last, st + 8192, wave, lane, lo);
     };
 
     if (ntiles > 0) issue(0);
@@ -265,13 +298,15 @@ __global__ __launch_bounds__(256) void attn_delta_kernel(const AttnArgs a) {
 // =========================================================================================
 // backward dK, dV: block = 128 keys (4 waves x 32), loop over 64-query tiles
 // =========================================================================================
-__global__ __launch_bounds__(256) void attn_bwd_dkv_kernel(const AttnArgs a) {
+__global__ __launch_bounds__(256, 2) void attn_bwd_dkv_kernel(const AttnArgs a) {
     // 2 stages x (Q tile 8 KiB, dO tile 8 KiB, lse 256 B, delta 256 B)
     constexpr int STAGE = 2 * 8192 + 512;
     __shared__ __attribute__((aligned(16))) unsigned char smem[2 * STAGE];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int kb = blockIdx.x;
-    const int b = blockIdx.y / a.heads, head = blockIdx.y % a.heads;
+    const BlockMap bm = map_block(a.batch * a.heads);
+    if (bm.bh >= a.batch * a.heads) return;
+    const int kb = bm.rank;  // early key blocks are seen by the most queries
+    const int b = bm.bh / a.heads, head = bm.bh % a.heads;
     const int64_t row_base = (int64_t)b * a.seq;
     const bf16* Q = a.q + row_base * a.ld_qkv + head * 64;
     const bf16* K = a.k + row_base * a.ld_qkv + head * 64;
@@ -303,13 +338,12 @@ __global__ __launch_bounds__(256) void attn_bwd_dkv_kernel(const AttnArgs a) {
 #pragma unroll
         for (int r = 0; r < 16; ++r) dk[t][r] = dv[t][r] = 0.f;
 
+    const LaneOff lo = lane_off(a.ld_qkv, wave, lane), lo_o = lane_off(a.ld_o, wave, lane);
     auto issue = [&](int t, int slot) {
         unsigned char* st = smem + slot * STAGE;
         const int qs = t * 64;
-        dma_rows8(Q, a.ld_qkv, qs, last, st, wave, lane);
-        dma_rows8(Q, a.ld_qkv, qs, last, st, wave + 4, lane);
-        dma_rows8(DO, a.ld_o, qs, last, st + 8192, wave, lane);
-        dma_rows8(DO, a.ld_o, qs, last, st + 8192, wave + 4, lane);
+        dma_tile64(Q, a.ld_qkv, qs, last, st, wave, lane, lo);
+        dma_tile64(DO, a.ld_o, qs, last, st + 8192, wave, lane, lo_o);
         if (wave == 0) dma_f32x64(LSE, qs, last, st + 16384, lane);
         if (wave == 1) dma_f32x64(DELTA, qs, last, st + 16384 + 256, lane);
     };
@@ -394,11 +428,13 @@ __global__ __launch_bounds__(256) void attn_bwd_dkv_kernel(const AttnArgs a) {
 // =========================================================================================
 // backward dQ: block = 128 queries (4 waves x 32), loop over 64-key tiles
 // =========================================================================================
-__global__ __launch_bounds__(256) void attn_bwd_dq_kernel(const AttnArgs a) {
+__global__ __launch_bounds__(256, 2) void attn_bwd_dq_kernel(const AttnArgs a) {
     __shared__ __attribute__((aligned(16))) unsigned char smem[2 * 2 * 8192];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int qb = gridDim.x - 1 - blockIdx.x;
-    const int b = blockIdx.y / a.heads, head = blockIdx.y % a.heads;
+    const BlockMap bm = map_block(a.batch * a.heads);
+    if (bm.bh >= a.batch * a.heads) return;
+    const int qb = (a.seq + 127) / 128 - 1 - bm.rank;
+    const int b = bm.bh / a.heads, head = bm.bh % a.heads;
     const int64_t row_base = (int64_t)b * a.seq;
     const bf16* Q = a.q + row_base * a.ld_qkv + head * 64;
     const bf16* K = a.k + row_base * a.ld_qkv + head * 64;
@@ -430,13 +466,12 @@ __global__ __launch_bounds__(256) void attn_bwd_dq_kernel(const AttnArgs a) {
 #pragma unroll
         for (int r = 0; r < 16; ++r) dq[t][r] = 0.f;
 
+    const LaneOff lo = lane_off(a.ld_qkv, wave, lane);
     auto issue = [&](int t) {
         unsigned char* st = smem + (t & 1) * 16384;
         const int kv0 = t * 64;
-        dma_rows8(K, a.ld_qkv, kv0, last, st, wave, lane);
-        dma_rows8(K, a.ld_qkv, kv0, last, st, wave + 4, lane);
-        dma_rows8(V, a.ld_qkv, kv0, last, st + 8192, wave, lane);
-        dma_rows8(V, a.ld_qkv, kv0, last, st + 8192, wave + 4, lane);
+        dma_tile64(K, a.ld_qkv, kv0, last, st, wave, lane, lo);
+        dma_tile64(V, a.ld_qkv, kv0, last, st + 8192, wave, lane, lo);
     };
     if (ntiles > 0) issue(0);
     for (int t = 0; t < ntiles; ++t) {
@@ -506,7 +541,8 @@ static int check_attn(const char* name, int dtype, int mask, int batch, int head
     BB_REQUIRE(mask != BB_MASK_KEY_PADDING || key_len, "%s: key_padding mask needs key_len", name);
     BB_REQUIRE(batch >= 0 && heads > 0 && seq >= 0, "%s: bad shape", name);
     BB_REQUIRE(ld_qkv % 8 == 0 && ld_o % 8 == 0 && ld_qkv >= heads * 64 && ld_o >= heads * 64, "%s: bad leading dimension", name);
-    BB_REQUIRE((int64_t)batch * heads <= 65535, "%s: batch * heads exceeds the grid limit", name);
+    BB_REQUIRE(ld_qkv < (1 << 24) && ld_o < (1 << 24), "%s: leading dimension too large", name);
+    BB_REQUIRE(((int64_t)batch * heads + 8) * ((seq + 127) / 128) < (1ll << 31), "%s: batch * heads * seq exceeds the grid limit", name);
     return BB_OK;
 }
 
@@ -524,7 +560,7 @@ extern "C" int bb_attention_fwd(int dtype, int mask, int batch, int heads, int s
     a.batch = batch; a.heads = heads; a.seq = seq; a.mask = mask;
     a.scale = 1.0f / sqrtf((float)head_dim);
     a.scale_log2 = a.scale * 1.4426950408889634f;
-    hipLaunchKernelGGL(attn_fwd_kernel, dim3((seq + 127) / 128, batch * heads), dim3(256), 0, (hipStream_t)stream, a);
+    hipLaunchKernelGGL(attn_fwd_kernel, dim3(attn_grid(seq, batch * heads)), dim3(256), 0, (hipStream_t)stream, a);
     BB_LAUNCH_CHECK();
     return BB_OK;
 }
@@ -550,7 +586,7 @@ extern "C" int bb_attention_bwd(int dtype, int mask, int batch, int heads, int s
     hipStream_t st = (hipStream_t)stream;
     const int64_t n = (int64_t)batch * seq * heads;
     hipLaunchKernelGGL(attn_delta_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st, a);
-    dim3 grid((seq + 127) / 128, batch * heads);
+    dim3 grid(attn_grid(seq, batch * heads));
     hipLaunchKernelGGL(attn_bwd_dkv_kernel, grid, dim3(256), 0, st, a);
     hipLaunchKernelGGL(attn_bwd_dq_kernel, grid, dim3(256), 0, st, a);
     BB_LAUNCH_CHECK();
