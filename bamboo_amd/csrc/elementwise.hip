@@ -97,11 +97,18 @@ __global__ __launch_bounds__(256) void layernorm_fwd_kernel(int kind, int rows, 
     }
 }
 
+// N contiguous floats (N a multiple of 4, 16-byte aligned destination)
+template <int N> __device__ __forceinline__ void store_f32s(float* dst, const float* v) {
+#pragma unroll
+    for (int e = 0; e < N; e += 4) *(f32x4*)(dst + e) = f32x4{v[e], v[e + 1], v[e + 2], v[e + 3]};
+}
+
 constexpr int LN_BWD_BLOCKS = 256;
+constexpr int LN_BWD_WAVES = 16;  // one block per CU, four waves per SIMD to cover the load latency
 
 // dx per row, dgain/dshift partial sums per block (fixed row->block assignment).
 template <typename T, int IT>
-__global__ __launch_bounds__(256) void layernorm_bwd_kernel(int kind, int rows, int cols, float eps,
+__global__ __launch_bounds__(LN_BWD_WAVES * 64) void layernorm_bwd_kernel(int kind, int rows, int cols, float eps,
                                                             const T* __restrict__ x, const T* __restrict__ gain,
                                                             const float* __restrict__ mean_in,
                                                             const float* __restrict__ rinv_in, const T* __restrict__ dy,
@@ -119,7 +126,7 @@ __global__ __launch_bounds__(256) void layernorm_bwd_kernel(int kind, int rows, 
         for (int e = 0; e < VEC; ++e) dg[i][e] = db[i][e] = gv[i][e] = 0.f;
         if (c < nvec) load_vec(gain + c * VEC, gv[i]);
     }
-    for (int row = blockIdx.x * 4 + wave; row < rows; row += gridDim.x * 4) {
+    for (int row = blockIdx.x * LN_BWD_WAVES + wave; row < rows; row += gridDim.x * LN_BWD_WAVES) {
         const float mean = mean_in[row], rinv = rinv_in[row];
         const T* xr = x + (int64_t)row * cols;
         const T* dyr = dy + (int64_t)row * cols;
@@ -173,75 +180,105 @@ __global__ __launch_bounds__(256) void layernorm_bwd_kernel(int kind, int rows, 
             }
         }
     }
-    // cross-wave sum in fixed order (wave 0 + 1 + 2 + 3), then one partial row per block
-    if (wave > 0) {
-        float* r = red + (int64_t)(wave - 1) * 2 * cols;
+    // cross-wave sum in fixed order (wave 0 + 1 + 2 + ... ), three waves per round through the
+    // three LDS slots, then one partial row per block
+    for (int w0 = 1; w0 < LN_BWD_WAVES; w0 += 3) {
+        if (wave >= w0 && wave < w0 + 3) {
+            float* r = red + (int64_t)(wave - w0) * 2 * cols;
 #pragma unroll
-        for (int i = 0; i < IT; ++i) {
-            const int c = lane + i * 64;
-            if (c < nvec) {
-#pragma unroll
-                for (int e = 0; e < VEC; ++e) {
-                    r[c * VEC + e] = dg[i][e];
-                    r[cols + c * VEC + e] = db[i][e];
+            for (int i = 0; i < IT; ++i) {
+                const int c = lane + i * 64;
+                if (c < nvec) {
+                    store_f32s<VEC>(r + c * VEC, dg[i]);
+                    store_f32s<VEC>(r + cols + c * VEC, db[i]);
                 }
             }
         }
+        __syncthreads();
+        if (wave == 0) {
+            const int nslot = min(3, LN_BWD_WAVES - w0);
+            for (int w = 0; w < nslot; ++w) {
+                const float* r = red + (int64_t)w * 2 * cols;
+#pragma unroll
+                for (int i = 0; i < IT; ++i) {
+                    const int c = lane + i * 64;
+                    if (c < nvec) {
+#pragma unroll
+                        for (int e = 0; e < VEC; ++e) {
+                            dg[i][e] += r[c * VEC + e];
+                            db[i][e] += r[cols + c * VEC + e];
+                        }
+                    }
+                }
+            }
+        }
+        __syncthreads();
     }
-    __syncthreads();
     if (wave == 0) {
         float* out = partial + (int64_t)blockIdx.x * 2 * cols;
 #pragma unroll
         for (int i = 0; i < IT; ++i) {
             const int c = lane + i * 64;
             if (c < nvec) {
-#pragma unroll
-                for (int e = 0; e < VEC; ++e) {
-                    float a = dg[i][e], b = db[i][e];
-                    for (int w = 0; w < 3; ++w) {
-                        a += red[(int64_t)w * 2 * cols + c * VEC + e];
-                        b += red[(int64_t)w * 2 * cols + cols + c * VEC + e];
-                    }
-                    out[c * VEC + e] = a;
-                    out[cols + c * VEC + e] = b;
-                }
+                store_f32s<VEC>(out + c * VEC, dg[i]);
+                store_f32s<VEC>(out + cols + c * VEC, db[i]);
             }
         }
     }
 }
 
-// out[i] += sum_p partial[p * stride + i].  One block owns 64 columns; its four waves sum
-// interleaved quarters of the partial rows (p = w, w+4, ...) and the four results are combined
+// Sum of partial rows p = first, first + step, ... in that order, eight loads in flight at a time.
+__device__ __forceinline__ float sum_partials(const float* __restrict__ src, int first, int step, int nparts, int64_t stride) {
+    float s = 0.f;
+    int p = first;
+    for (; p + 7 * step < nparts; p += 8 * step) {
+        float v[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) v[j] = src[(int64_t)(p + j * step) * stride];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) s += v[j];
+    }
+    for (; p < nparts; p += step) s += src[(int64_t)p * stride];
+    return s;
+}
+constexpr int RED_WAVES = 16;
+
+// out[i] += sum_p partial[p * stride + i].  One block owns 64 columns; its sixteen waves sum
+// interleaved shares of the partial rows (p = w, w+16, ...) and the sixteen results are combined
 // in wave order, so the summation order is fixed by nparts alone.
-__global__ __launch_bounds__(256) void reduce_partials_acc_kernel(const float* __restrict__ partial, int nparts,
-                                                                  int64_t stride, int n, float* __restrict__ out) {
-    __shared__ float red[4][64];
+__global__ __launch_bounds__(RED_WAVES * 64) void reduce_partials_acc_kernel(const float* __restrict__ partial, int nparts,
+                                                                             int64_t stride, int n, float* __restrict__ out) {
+    __shared__ float red[RED_WAVES][64];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int i = blockIdx.x * 64 + lane;
-    float s = 0.f;
-    if (i < n)
-        for (int p = wave; p < nparts; p += 4) s += partial[p * stride + i];
-    red[wave][lane] = s;
+    red[wave][lane] = i < n ? sum_partials(partial + i, wave, RED_WAVES, nparts, stride) : 0.f;
     __syncthreads();
-    if (wave == 0 && i < n) out[i] += (red[0][lane] + red[1][lane]) + (red[2][lane] + red[3][lane]);
+    if (wave == 0 && i < n) {
+        float s = red[0][lane];
+#pragma unroll
+        for (int w = 1; w < RED_WAVES; ++w) s += red[w][lane];
+        out[i] += s;
+    }
 }
 
 // two vectors at once (LayerNorm gain and shift gradients): blockIdx.y picks the half of every
 // partial row and the output
-__global__ __launch_bounds__(256) void reduce_partials_acc2_kernel(const float* __restrict__ partial, int nparts,
-                                                                   int64_t stride, int n, float* __restrict__ out0,
-                                                                   float* __restrict__ out1) {
-    __shared__ float red[4][64];
+__global__ __launch_bounds__(RED_WAVES * 64) void reduce_partials_acc2_kernel(const float* __restrict__ partial, int nparts,
+                                                                              int64_t stride, int n, float* __restrict__ out0,
+                                                                              float* __restrict__ out1) {
+    __shared__ float red[RED_WAVES][64];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int i = blockIdx.x * 64 + lane;
     const float* src = partial + (int64_t)blockIdx.y * n;
     float* out = blockIdx.y == 0 ? out0 : out1;
-    float s = 0.f;
-    if (i < n)
-        for (int p = wave; p < nparts; p += 4) s += src[p * stride + i];
-    red[wave][lane] = s;
+    red[wave][lane] = i < n ? sum_partials(src + i, wave, RED_WAVES, nparts, stride) : 0.f;
     __syncthreads();
-    if (wave == 0 && i < n) out[i] += (red[0][lane] + red[1][lane]) + (red[2][lane] + red[3][lane]);
+    if (wave == 0 && i < n) {
+        float s = red[0][lane];
+#pragma unroll
+        for (int w = 1; w < RED_WAVES; ++w) s += red[w][lane];
+        out[i] += s;
+    }
 }
 
 template <typename T, int IT>
@@ -258,7 +295,7 @@ static int ln_bwd_launch(int kind, int rows, int cols, float eps, const void* x,
     const size_t smem = (size_t)3 * 2 * cols * sizeof(float);
     auto kern = layernorm_bwd_kernel<T, IT>;
     if (smem > 64 * 1024) BB_HIP_CHECK(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
-    hipLaunchKernelGGL(kern, dim3(LN_BWD_BLOCKS), dim3(256), smem, st, kind, rows, cols, eps, (const T*)x,
+    hipLaunchKernelGGL(kern, dim3(LN_BWD_BLOCKS), dim3(LN_BWD_WAVES * 64), smem, st, kind, rows, cols, eps, (const T*)x,
                        (const T*)gain, mean, rinv, (const T*)dy, (const T*)dres, (T*)dx, ws);
     BB_LAUNCH_CHECK();
     return BB_OK;
@@ -312,7 +349,7 @@ extern "C" int bb_layernorm_bwd(int dtype, int kind, int rows, int cols, float e
     hipStream_t st = (hipStream_t)stream;
     auto finish = [&]() -> int {
         const int nb = (cols + 63) / 64;
-        hipLaunchKernelGGL(reduce_partials_acc2_kernel, dim3(nb, 2), dim3(256), 0, st, workspace, LN_BWD_BLOCKS,
+        hipLaunchKernelGGL(reduce_partials_acc2_kernel, dim3(nb, 2), dim3(RED_WAVES * 64), 0, st, workspace, LN_BWD_BLOCKS,
                            (int64_t)2 * cols, cols, dgain, dshift);
         BB_LAUNCH_CHECK();
         return BB_OK;
@@ -382,7 +419,7 @@ extern "C" int bb_colsum_acc(int dtype, int rows, int cols, const void* x, int64
         hipLaunchKernelGGL(colsum_partial_kernel<bf16>, grid, dim3(256), 0, st, rows, cols, (const bf16*)x, ldx, workspace);
     else
         hipLaunchKernelGGL(colsum_partial_kernel<float>, grid, dim3(256), 0, st, rows, cols, (const float*)x, ldx, workspace);
-    hipLaunchKernelGGL(reduce_partials_acc_kernel, dim3((cols + 63) / 64), dim3(256), 0, st, workspace, COLSUM_SPLITS,
+    hipLaunchKernelGGL(reduce_partials_acc_kernel, dim3((cols + 63) / 64), dim3(RED_WAVES * 64), 0, st, workspace, COLSUM_SPLITS,
                        (int64_t)cols, cols, out);
     BB_LAUNCH_CHECK();
     return BB_OK;
