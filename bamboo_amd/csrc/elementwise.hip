@@ -605,31 +605,42 @@ extern "C" int bb_residual_add(int dtype, int64_t n, const void* a, const void* 
     return BB_OK;
 }
 
-// out = act(x), elementwise (the activation between the two feed-forward GEMMs)
-template <typename T>
-__global__ __launch_bounds__(256) void act_kernel(int64_t nvec, int act, const T* __restrict__ x, T* __restrict__ out) {
+// out = act(x) and, if wanted, dact = act'(x), elementwise (the activation between the two
+// feed-forward GEMMs).  dact may alias x: a thread reads its elements before it writes them.
+template <typename T, bool DACT>
+__global__ __launch_bounds__(256) void act_kernel(int64_t nvec, int act, const T* x, T* __restrict__ out, T* dact) {
     constexpr int VEC = Elem<T>::VEC;
     for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < nvec; i += (int64_t)gridDim.x * 256) {
-        float v[VEC];
+        float v[VEC], a[VEC];
         load_vec(x + i * VEC, v);
 #pragma unroll
-        for (int e = 0; e < VEC; ++e) v[e] = act_f(v[e], act);
-        store_vec(out + i * VEC, v);
+        for (int e = 0; e < VEC; ++e) a[e] = act_f(v[e], act);
+        store_vec(out + i * VEC, a);
+        if (DACT) {
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) a[e] = dact_f(v[e], act);
+            store_vec(dact + i * VEC, a);
+        }
     }
 }
 
-extern "C" int bb_act_fwd(int dtype, int act, int64_t n, const void* x, void* out, void* stream) {
+extern "C" int bb_act_fwd(int dtype, int act, int64_t n, const void* x, void* out, void* dact, void* stream) {
     BB_REQUIRE(dtype == BB_F32 || dtype == BB_BF16, "bb_act_fwd: bad dtype %d", dtype);
     BB_REQUIRE(act == BB_ACT_RELU || act == BB_ACT_GELU_TANH, "bb_act_fwd: bad activation %d", act);
     const int vec = dtype == BB_BF16 ? 8 : 4;
     BB_REQUIRE(n >= 0 && n % vec == 0 && (n == 0 || (x && out)), "bb_act_fwd: n (%lld) must be a multiple of %d", (long long)n, vec);
+    BB_REQUIRE(out != x && out != dact, "bb_act_fwd: out must not alias x or dact");
     if (n == 0) return BB_OK;
     hipStream_t st = (hipStream_t)stream;
     const int64_t nvec = n / vec;
-    if (dtype == BB_BF16)
-        hipLaunchKernelGGL(act_kernel<bf16>, dim3(grid_for(nvec)), dim3(256), 0, st, nvec, act, (const bf16*)x, (bf16*)out);
-    else
-        hipLaunchKernelGGL(act_kernel<float>, dim3(grid_for(nvec)), dim3(256), 0, st, nvec, act, (const float*)x, (float*)out);
+    dim3 grid(grid_for(nvec)), block(256);
+    if (dtype == BB_BF16) {
+        if (dact) hipLaunchKernelGGL((act_kernel<bf16, true>), grid, block, 0, st, nvec, act, (const bf16*)x, (bf16*)out, (bf16*)dact);
+        else hipLaunchKernelGGL((act_kernel<bf16, false>), grid, block, 0, st, nvec, act, (const bf16*)x, (bf16*)out, (bf16*)nullptr);
+    } else {
+        if (dact) hipLaunchKernelGGL((act_kernel<float, true>), grid, block, 0, st, nvec, act, (const float*)x, (float*)out, (float*)dact);
+        else hipLaunchKernelGGL((act_kernel<float, false>), grid, block, 0, st, nvec, act, (const float*)x, (float*)out, (float*)nullptr);
+    }
     BB_LAUNCH_CHECK();
     return BB_OK;
 }

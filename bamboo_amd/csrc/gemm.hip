@@ -59,6 +59,8 @@ __device__ __forceinline__ void epilogue_elem(const GemmArgs& g, int64_t coff, i
         v *= dact_f(Elem<T>::load((const T*)g.aux_in + xi), g.act);
     } else if (g.epilogue == BB_EPI_RESIDUAL) {
         v += Elem<T>::load((const T*)g.resid + xi);
+    } else if (g.epilogue == BB_EPI_MUL) {
+        v *= Elem<T>::load((const T*)g.aux_in + xi);
     }
     if (g.c_f32) {
         float* c = (float*)g.C + ci;
@@ -92,6 +94,11 @@ __device__ __forceinline__ void epilogue_vec8(const GemmArgs& g, int64_t coff, i
         load_vec((const bf16*)g.resid + xi, r);
 #pragma unroll
         for (int e = 0; e < 8; ++e) v[e] += r[e];
+    } else if (g.epilogue == BB_EPI_MUL) {
+        float d[8];
+        load_vec((const bf16*)g.aux_in + xi, d);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) v[e] *= d[e];
     }
     if (g.c_f32) {
         float* c = (float*)g.C + ci;
@@ -776,11 +783,11 @@ static DmaTile pick_dma_tile(int M, int N, int K, int64_t batches) {
     const int ov = dma_tile_override();
     if (ov == 4) return D_NONE;
     if ((ov >= 1 && ov <= 3) || (ov >= 5 && ov <= 14)) return (DmaTile)ov;
-    // measured on MI355X (256 CUs): 256x256 tiles pay off from two full rounds of blocks on,
+    // measured on MI355X (256 CUs): 256x256 tiles pay off from one and a half rounds of blocks on,
     // 256x128 from one round, smaller problems take 128x128 tiles with two blocks per CU
     const int64_t t256 = (int64_t)((M + 255) / 256) * ((N + 255) / 256) * batches;
     const int64_t t2128 = (int64_t)((M + 255) / 256) * ((N + 127) / 128) * batches;
-    if (M >= 256 && N >= 256 && t256 >= 512) return D256x256w8db;
+    if (M >= 256 && N >= 256 && t256 >= 384) return D256x256w8db;
     if (M >= 256 && t2128 >= 256) return D256x128w8db;
     return D128x128s3;
 }
@@ -841,7 +848,7 @@ static int fill_args(const bb_gemm_desc* d, GemmArgs& g, int64_t& batches, bool&
     BB_REQUIRE(d->layout >= BB_NT && d->layout <= BB_TN, "bb_gemm: bad layout %d", d->layout);
     BB_REQUIRE(d->M >= 0 && d->N >= 0 && d->K >= 0, "bb_gemm: negative dimension");
     BB_REQUIRE(!d->accumulate || d->c_dtype == BB_F32, "bb_gemm: accumulate needs an fp32 C");
-    BB_REQUIRE(d->epilogue >= BB_EPI_NONE && d->epilogue <= BB_EPI_RESIDUAL, "bb_gemm: bad epilogue");
+    BB_REQUIRE(d->epilogue >= BB_EPI_NONE && d->epilogue <= BB_EPI_MUL, "bb_gemm: bad epilogue");
     const int nb1 = d->nb1 > 0 ? d->nb1 : 1, nb2 = d->nb2 > 0 ? d->nb2 : 1;
     batches = (int64_t)nb1 * nb2;
     ta = d->layout == BB_TN;
@@ -849,7 +856,7 @@ static int fill_args(const bb_gemm_desc* d, GemmArgs& g, int64_t& batches, bool&
     g.M = d->M; g.N = d->N; g.K = d->K; g.nb2 = nb2;
     if (d->M == 0 || d->N == 0) return BB_OK;
     BB_REQUIRE(d->A && d->B && d->C, "bb_gemm: null operand");
-    BB_REQUIRE(d->epilogue != BB_EPI_DACT || d->aux_in, "bb_gemm: DACT epilogue needs aux_in");
+    BB_REQUIRE((d->epilogue != BB_EPI_DACT && d->epilogue != BB_EPI_MUL) || d->aux_in, "bb_gemm: DACT/MUL epilogue needs aux_in");
     BB_REQUIRE(d->epilogue != BB_EPI_RESIDUAL || d->resid, "bb_gemm: RESIDUAL epilogue needs resid");
     BB_REQUIRE(batches <= 65535, "bb_gemm: too many batches (%lld)", (long long)batches);
     const int vec = d->dtype == BB_BF16 ? 8 : 4;

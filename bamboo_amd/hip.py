@@ -13,7 +13,7 @@ import torch
 
 F32, BF16 = 0, 1
 NT, NN, TN = 0, 1, 2
-EPI_NONE, EPI_ACT, EPI_DACT, EPI_RESIDUAL = 0, 1, 2, 3
+EPI_NONE, EPI_ACT, EPI_DACT, EPI_RESIDUAL, EPI_MUL = 0, 1, 2, 3, 4
 ACT_RELU, ACT_GELU_TANH = 0, 1
 MASK_NONE, MASK_CAUSAL, MASK_KEY_PADDING = 0, 1, 2
 LN_STANDARD, LN_ANNOTATED = 0, 1
@@ -89,7 +89,7 @@ def lib():
     L.bb_attention_bwd.argtypes = [c_int] * 6 + [c_void_p, c_void_p, c_void_p, c_int64, c_void_p, c_void_p, c_int64,
                                    c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_void_p, c_void_p]
     L.bb_residual_add.argtypes = [c_int, c_int64, c_void_p, c_void_p, c_void_p, c_void_p]
-    L.bb_act_fwd.argtypes = [c_int, c_int, c_int64, c_void_p, c_void_p, c_void_p]
+    L.bb_act_fwd.argtypes = [c_int, c_int, c_int64, c_void_p, c_void_p, c_void_p, c_void_p]
     L.bb_bn_workspace.argtypes = [c_int]
     L.bb_bn_workspace.restype = c_int64
     L.bb_batchnorm_fwd.argtypes = [c_int, c_int, c_int, c_float, c_float, c_int] + [c_void_p] * 11
@@ -313,8 +313,10 @@ def residual_add(a, b, out, stream=None):
           "bb_residual_add")
 
 
-def act_fwd(x, out, act, stream=None):
-    check(lib().bb_act_fwd(dtype_code(x.dtype), act, x.numel(), _ptr(x), _ptr(out), stream_ptr(stream)), "bb_act_fwd")
+def act_fwd(x, out, act, dact=None, stream=None):
+    """out = act(x); dact (optional, may be x itself) receives act'(x)."""
+    check(lib().bb_act_fwd(dtype_code(x.dtype), act, x.numel(), _ptr(x), _ptr(out), _ptr(dact), stream_ptr(stream)),
+          "bb_act_fwd")
 
 
 def bn_workspace(cols):

@@ -91,18 +91,30 @@ class GemmProbe:
         if isinstance(desc, (list, tuple)):
             name = "grouped_" + hip.gemm_variant(desc[0]).rsplit("_", 1)[0]
             flops = sum(2.0 * d.M * d.N * d.K for d in desc)
+            shape = "+".join(f"{d.M}x{d.N}x{d.K}" for d in desc)
         else:
             name, flops = hip.gemm_variant(desc), 2.0 * desc.M * desc.N * desc.K
+            shape = f"{desc.M}x{desc.N}x{desc.K}"
         e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         stream = stream if stream is not None else torch.cuda.current_stream()
         e0.record(stream)        # on the stream the kernel is launched on
         launch()
         e1.record(stream)
-        self.records.append((name, flops, e0, e1))
+        self.records.append((name, flops, e0, e1, shape))
+
+    def by_shape(self):
+        """{(variant, shape): [launches, flops, seconds]} for the --gemm-shapes table."""
+        agg = {}
+        for name, flops, e0, e1, shape in self.records:
+            a = agg.setdefault((name, shape), [0, 0.0, 0.0])
+            a[0] += 1
+            a[1] += flops
+            a[2] += e0.elapsed_time(e1) * 1e-3
+        return agg
 
     def summary(self):
         agg = {}
-        for name, flops, e0, e1 in self.records:
+        for name, flops, e0, e1, _ in self.records:
             a = agg.setdefault(name, [0, 0.0, 0.0])
             a[0] += 1
             a[1] += flops
@@ -158,6 +170,7 @@ def main():
     ap.add_argument("--rc-stream", type=int, default=1, help="issue redundant forwards on a second HIP stream")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-probe", action="store_true", help="do not bracket GEMM launches with events")
+    ap.add_argument("--gemm-shapes", action="store_true", help="print a per-shape GEMM table on stderr")
     ap.add_argument("--skip-rc-off", action="store_true")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="first run three 256 MiB fp32 copies (cast_kernel<float,float>): the known-size kernel that "
@@ -243,6 +256,10 @@ def main():
     roofline = None
     if probe is not None:
         agg = probe.summary()
+        if args.gemm_shapes:
+            for (name, shape), (n, fl, sec) in sorted(probe.by_shape().items(), key=lambda kv: -kv[1][2]):
+                print(f"{name:34s} {shape:40s} n={n:5d} {sec / n * 1e6:8.1f} us {fl / sec / 1e12:7.1f} TF {sec * 1e3:8.2f} ms",
+                      file=sys.stderr)
         name, (count, flops, secs) = max(agg.items(), key=lambda kv: kv[1][2])
         peak = PEAK_BF16_TFLOPS if cfg["dtype"] == "bf16" else PEAK_F32_TFLOPS
         achieved = flops / secs / 1e12

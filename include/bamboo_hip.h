@@ -50,11 +50,14 @@ extern "C" {
  *   BB_EPI_ACT       aux_out = v (if aux_out != NULL);  C = act(v)
  *   BB_EPI_DACT      C = v * act'(aux_in[m,n])
  *   BB_EPI_RESIDUAL  C = v + resid[m,n]
+ *   BB_EPI_MUL       C = v * aux_in[m,n]  (aux_in = act'(u) kept by bb_act_fwd: the backward of
+ *                    the activation costs one multiply in the epilogue)
  * `accumulate` != 0 adds the result to the existing contents of C (C must be fp32).       */
 #define BB_EPI_NONE 0
 #define BB_EPI_ACT 1
 #define BB_EPI_DACT 2
 #define BB_EPI_RESIDUAL 3
+#define BB_EPI_MUL 4
 
 #define BB_ACT_RELU 0
 #define BB_ACT_GELU_TANH 1
@@ -171,8 +174,10 @@ int bb_residual_add(int dtype, int64_t n, const void* a, const void* b, void* ou
                     void* stream);
 
 /* out = act(x), elementwise: the activation of PositionwiseFeedForward (transformer.py:158) as a
- * bandwidth-bound pass of its own (2 * n * sizeof(dtype) bytes).                             */
-int bb_act_fwd(int dtype, int act, int64_t n, const void* x, void* out, void* stream);
+ * bandwidth-bound pass of its own.  If dact != NULL it also receives act'(x), the factor autograd
+ * applies in the backward pass; dact may be x itself (each element is read before it is
+ * replaced), so keeping the derivative instead of the pre-activation costs no memory.         */
+int bb_act_fwd(int dtype, int act, int64_t n, const void* x, void* out, void* dact, void* stream);
 
 /* BatchNorm2d in training mode on an NHWC activation viewed as [rows = N*H*W, cols = channels]
  * (resnet.py:56,59,62): per-channel batch mean and biased variance (two passes), then

@@ -76,6 +76,9 @@ def test_gemm_epilogues(hiplib, dtype):
         ol.activation(Uf, name).sum().backward()
         hiplib.gemm(hiplib.NT, A, W, C, epilogue=hiplib.EPI_DACT, act=act, aux_in=U)
         assert rel_err(C, (Af @ Wf.t()) * Uf.grad) < tol(dtype)
+    # mul: C = (A W^T) * R
+    hiplib.gemm(hiplib.NT, A, W, C, epilogue=hiplib.EPI_MUL, aux_in=R)
+    assert rel_err(C, (Af @ Wf.t()) * Rf) < tol(dtype)
     # fp32 accumulate (weight-gradient form): G += A^T B
     G0 = randn(K, N, dtype=torch.float32, seed=7)
     G = G0.clone()
@@ -287,7 +290,15 @@ def test_act_fwd(hiplib, dtype, name):
     x = randn(4096, 96, dtype=dtype, seed=26, scale=3.0)
     out = torch.empty_like(x)
     hiplib.act_fwd(x, out, hiplib.ACT_CODES[name])
-    assert rel_err(out, ol.activation(x.double().cpu(), name)) < tol(dtype)
+    ref = ol.activation(x.double().cpu(), name)
+    assert rel_err(out, ref) < tol(dtype)
+    # with the derivative, written over the input
+    xf = x.double().cpu().requires_grad_(True)
+    ol.activation(xf, name).sum().backward()
+    out2, x2 = torch.empty_like(x), x.clone()
+    hiplib.act_fwd(x2, out2, hiplib.ACT_CODES[name], dact=x2)
+    assert torch.equal(out2, out)
+    assert rel_err(x2, xf.grad) < tol(dtype)
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
