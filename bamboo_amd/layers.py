@@ -238,8 +238,7 @@ class TransformerLayer:
         # the activation runs as its own bandwidth-bound pass: inside the GEMM epilogue its
         # transcendental work would sit on the critical path of every tile while the MFMA pipe idles
         hip.gemm(hip.NT, st["n2"], w["feed_forward.w_1.weight"], st["u"], bias=w["feed_forward.w_1.bias"], stream=sm)
-        # the pre-activation is needed again only through act'(u): keep that in its place
-        hip.act_fwd(st["u"], st["act"], act, dact=st["u"], stream=sm)
+        hip.act_fwd(st["u"], st["act"], act, stream=sm)
         hip.gemm(hip.NT, st["act"], w["feed_forward.w_2.weight"], st["out"], bias=w["feed_forward.w_2.bias"],
                  epilogue=hip.EPI_RESIDUAL, resid=st["x1"], stream=sm)
         return st["out"]
@@ -260,7 +259,7 @@ class TransformerLayer:
             hip.TN, dy, x, g[name], accumulate=True, colsum_out=g[name[:-len("weight")] + "bias"], colsum_ws=ws))
         # feed-forward
         wgrad(d_out, st["act"], "feed_forward.w_2.weight")
-        hip.gemm(hip.NN, d_out, w["feed_forward.w_2.weight"], d_ffn, epilogue=hip.EPI_MUL,
+        hip.gemm(hip.NN, d_out, w["feed_forward.w_2.weight"], d_ffn, epilogue=hip.EPI_DACT, act=act,
                  aux_in=st["u"], stream=sm)
         wgrad(d_ffn, st["n2"], "feed_forward.w_1.weight")
         hip.gemm(hip.NN, d_ffn, w["feed_forward.w_1.weight"], d_h0, stream=sm)

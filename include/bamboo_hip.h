@@ -50,8 +50,7 @@ extern "C" {
  *   BB_EPI_ACT       aux_out = v (if aux_out != NULL);  C = act(v)
  *   BB_EPI_DACT      C = v * act'(aux_in[m,n])
  *   BB_EPI_RESIDUAL  C = v + resid[m,n]
- *   BB_EPI_MUL       C = v * aux_in[m,n]  (aux_in = act'(u) kept by bb_act_fwd: the backward of
- *                    the activation costs one multiply in the epilogue)
+ *   BB_EPI_MUL       C = v * aux_in[m,n]  (e.g. aux_in = act'(u) kept by bb_act_fwd)
  * `accumulate` != 0 adds the result to the existing contents of C (C must be fp32).       */
 #define BB_EPI_NONE 0
 #define BB_EPI_ACT 1
