@@ -39,6 +39,14 @@ CONFIGS = {
 STAGES, STAGE_ID = 4, 1
 PEAK_BF16_TFLOPS, PEAK_F32_TFLOPS = 2500.0, 157.3
 
+# HBM bytes per launch of the dominant kernel, from the two rocprofv3 --pmc runs summarised in
+# profiles/ (FETCH_SIZE x 2.0 and WRITE_SIZE x 1.0, the factors a 256 MiB copy kernel gives);
+# counters cannot be read from inside this process, so the figure is carried here per
+# (config, kernel) and is null for anything that was not profiled.
+MEASURED_TRAFFIC_BYTES = {
+    ("c2", "gemm_bf16_nt_dma256x256w8db"): int((47515.1 * 2.0 + 57344.0) * 1024),
+}
+
 
 def build_engine(cfg, rc, rc_stream, seed=1138):
     import torch
@@ -102,6 +110,22 @@ class GemmProbe:
         e1.record(stream)
         self.records.append((name, flops, e0, e1, shape))
 
+    @staticmethod
+    def bracket_overhead(n=200):
+        """Seconds that an empty event bracket reads on an idle stream: what each bracket adds to
+        the kernel it encloses (marker processing + dispatch), subtracted per launch in summary()."""
+        import torch
+        torch.cuda.synchronize()
+        pairs = []
+        for _ in range(n):
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            e1.record()
+            pairs.append((e0, e1))
+        torch.cuda.synchronize()
+        ts = sorted(a.elapsed_time(b) for a, b in pairs)
+        return ts[len(ts) // 2] * 1e-3
+
     def by_shape(self):
         """{(variant, shape): [launches, flops, seconds]} for the --gemm-shapes table."""
         agg = {}
@@ -112,13 +136,15 @@ class GemmProbe:
             a[2] += e0.elapsed_time(e1) * 1e-3
         return agg
 
-    def summary(self):
+    def summary(self, overhead_s=0.0):
+        """{variant: [launches, flops, seconds]}; ``overhead_s`` (an empty bracket's reading) is
+        taken off every launch so that the durations are the kernels' own, as a kernel trace shows them."""
         agg = {}
         for name, flops, e0, e1, _ in self.records:
             a = agg.setdefault(name, [0, 0.0, 0.0])
             a[0] += 1
             a[1] += flops
-            a[2] += e0.elapsed_time(e1) * 1e-3
+            a[2] += max(e0.elapsed_time(e1) * 1e-3 - overhead_s, 1e-9)
         return agg
 
 
@@ -143,22 +169,25 @@ def cpu_baseline(cfg, threads):
     kl = None
     if cfg["variant"]["mask"] == "key_padding":
         kl = torch.randint(cfg["key_len_range"][0], cfg["key_len_range"][1] + 1, (cfg["mb"],), generator=g)
-    t0 = time.perf_counter()
-    xin = x.clone().requires_grad_(True)
-    out = st.forward(xin, STAGE_ID, kl)
-    torch.autograd.backward(out, dy)
-    t_own = time.perf_counter() - t0
-    t0 = time.perf_counter()
-    with torch.enable_grad():
-        st.forward(out.detach().requires_grad_(True), STAGE_ID + 1, kl)
-    t_rc = time.perf_counter() - t0
+    reps = 2  # two micro-batches: about 10-15 s on 16 host cores at the c2 shapes
+    t_own = t_rc = 0.0
+    for _ in range(reps):
+        t0 = time.perf_counter()
+        xin = x.clone().requires_grad_(True)
+        out = st.forward(xin, STAGE_ID, kl)
+        torch.autograd.backward(out, dy)
+        t_own += (time.perf_counter() - t0) / reps
+        t0 = time.perf_counter()
+        with torch.enable_grad():
+            st.forward(out.detach().requires_grad_(True), STAGE_ID + 1, kl)
+        t_rc += (time.perf_counter() - t0) / reps
     M = cfg["M"]
     samples = cfg["mb"] * M
     off, on = M * t_own, M * (t_own + t_rc)
     return {"value": samples / on, "unit": "samples/s", "cores": threads, "kind": "port",
             "rc_off_value": samples / off, "rc_overhead_pct": 100.0 * (on - off) / off,
-            "sample": f"1 micro-batch own fwd+bwd ({t_own:.2f}s) + 1 redundant fwd ({t_rc:.2f}s), fp32, "
-                      f"extrapolated x{M} micro-batches; optimizer step not included"}
+            "sample": f"{reps} micro-batches, each own fwd+bwd ({t_own:.2f}s) + redundant fwd ({t_rc:.2f}s), fp32, "
+                      f"mean extrapolated x{M} micro-batches; optimizer step not included"}
 
 
 def main():
@@ -255,7 +284,8 @@ def main():
 
     roofline = None
     if probe is not None:
-        agg = probe.summary()
+        overhead_s = probe.bracket_overhead()
+        agg = probe.summary(overhead_s)
         if args.gemm_shapes:
             for (name, shape), (n, fl, sec) in sorted(probe.by_shape().items(), key=lambda kv: -kv[1][2]):
                 print(f"{name:34s} {shape:40s} n={n:5d} {sec / n * 1e6:8.1f} us {fl / sec / 1e12:7.1f} TF {sec * 1e3:8.2f} ms",
@@ -264,8 +294,11 @@ def main():
         peak = PEAK_BF16_TFLOPS if cfg["dtype"] == "bf16" else PEAK_F32_TFLOPS
         achieved = flops / secs / 1e12
         roofline = {"bound": "mfma", "achieved": round(achieved, 2), "peak": peak, "unit": "TFLOP/s",
-                    "frac": round(achieved / peak, 4), "traffic": None, "kernel": f"gemm_{name}",
-                    "measured_in": "timed steps of the RC-on single-stream leg, HIP events around each launch",
+                    "frac": round(achieved / peak, 4),
+                    "traffic": MEASURED_TRAFFIC_BYTES.get((args.config, f"gemm_{name}")), "kernel": f"gemm_{name}",
+                    "measured_in": "timed steps of the RC-on single-stream leg, HIP events around each launch on its "
+                                   "stream, minus the reading of an empty event bracket",
+                    "event_bracket_overhead_us": round(overhead_s * 1e6, 2),
                     "launches": count, "avg_launch_us": round(secs / count * 1e6, 2),
                     "avg_launch_gflop": round(flops / count / 1e9, 3),
                     "all_gemm_variants": {k: {"launches": v[0], "tflops": round(v[1] / v[2] / 1e12, 2),
