@@ -378,22 +378,33 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dkv_kernel(const AttnArgs a) 
                 s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frag_kc(qt, u * 32, ks, lane), kf[ks], s, 0, 0, 0);
                 dp = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frag_kc(dot, u * 32, ks, lane), vf[ks], dp, 0, 0, 0);
             }
-            // P = exp2(S * c - lse[q]); dS = P * (dP - delta[q]); rows q = acc_row(r), column kv = lane
+            // P = exp2(S * c - lse[q]); dS = P * (dP - delta[q]); rows q = acc_row(r), column kv = lane.
+            // Only sub-tiles on the causal diagonal or past the last query mask per element; keys
+            // beyond the padding limit are whole lanes and are cleared once, after the loop.
+            const bool need_mask = (a.mask == BB_MASK_CAUSAL && qs < kv0 + 31) || qs + 32 > a.seq;
 #pragma unroll
             for (int g4 = 0; g4 < 4; ++g4) {
                 const int ql = u * 32 + 8 * g4 + 4 * (lane >> 5);
                 const f32x4 l4 = *(const f32x4*)(lse_t + ql);
+#pragma unroll
+                for (int e = 0; e < 4; ++e) s[g4 * 4 + e] = __builtin_amdgcn_exp2f(fmaf(s[g4 * 4 + e], a.scale_log2, -l4[e]));
+            }
+            if (need_mask) {
+                asm volatile("" ::: "memory");  // a real branch: most sub-tiles skip it
+                const int qlane = t * 64 + u * 32 + 4 * (lane >> 5);  // register r holds query qlane + 8*(r/4) + r%4
+                const int qmin = a.mask == BB_MASK_CAUSAL ? mykv : 0;
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    const int q = qlane + 8 * (r >> 2) + (r & 3);
+                    s[r] = q >= qmin && q < a.seq ? s[r] : 0.f;
+                }
+            }
+#pragma unroll
+            for (int g4 = 0; g4 < 4; ++g4) {
+                const int ql = u * 32 + 8 * g4 + 4 * (lane >> 5);
                 const f32x4 d4 = *(const f32x4*)(del_t + ql);
 #pragma unroll
-                for (int e = 0; e < 4; ++e) {
-                    const int r = g4 * 4 + e;
-                    const int q = t * 64 + ql + e;
-                    bool keep = mykv < pad_limit && q < a.seq;
-                    if (a.mask == BB_MASK_CAUSAL) keep = keep && mykv <= q;
-                    const float p = keep ? __builtin_amdgcn_exp2f(fmaf(s[r], a.scale_log2, -l4[e])) : 0.f;
-                    s[r] = p;
-                    dp[r] = p * (dp[r] - d4[e]);
-                }
+                for (int e = 0; e < 4; ++e) dp[g4 * 4 + e] = s[g4 * 4 + e] * (dp[g4 * 4 + e] - d4[e]);
             }
             // dV^T += dO^T P ; dK^T += Q^T dS   (contraction over the 32 queries of this sub-tile)
 #pragma unroll
@@ -407,6 +418,12 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dkv_kernel(const AttnArgs a) 
             }
         }
         block_sync();
+    }
+    if (mykv >= pad_limit) {  // a padded key takes no probability mass: its gradients are zero
+#pragma unroll
+        for (int t = 0; t < 2; ++t)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) dk[t][r] = dv[t][r] = 0.f;
     }
     if (mykv < a.seq) {
         bf16* dkp = a.dk + (row_base + mykv) * a.ld_dqkv + head * 64;
@@ -447,7 +464,9 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dq_kernel(const AttnArgs a) {
     if (a.mask == BB_MASK_CAUSAL) kv_end = min(a.seq, qb * 128 + 128);
     else if (a.mask == BB_MASK_KEY_PADDING) kv_end = min(a.seq, a.key_len[b]);
     const int ntiles = (kv_end + 63) / 64;
-    const int my_limit = myq < a.seq ? kv_limit(a, b, myq) : 0;
+    // rows past the end compute on clamped inputs and are not stored
+    const int my_limit = kv_limit(a, b, myq);
+    const int wave_min_limit = kv_limit(a, b, q0);  // limits grow with the query index
 
     bf16x8 qf[4], dof[4];
     {
@@ -499,11 +518,15 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dq_kernel(const AttnArgs a) {
                     dp = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frag_kc(vt, u * 32, ks, lane), dof[ks], dp, 0, 0, 0);
                 }
 #pragma unroll
-                for (int r = 0; r < 16; ++r) {
-                    const int kv = kv0 + u * 32 + acc_row(r, lane);
-                    const float p = kv < my_limit ? __builtin_amdgcn_exp2f(fmaf(s[r], a.scale_log2, -my_lse)) : 0.f;
-                    dp[r] = p * (dp[r] - my_delta);
+                for (int r = 0; r < 16; ++r) s[r] = __builtin_amdgcn_exp2f(fmaf(s[r], a.scale_log2, -my_lse));
+                if (kv0 + u * 32 + 32 > wave_min_limit) {
+                    asm volatile("" ::: "memory");  // a real branch: only tiles on the mask boundary pay for it
+                    const int lim = my_limit - kv0 - u * 32 - 4 * (lane >> 5);
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) s[r] = 8 * (r >> 2) + (r & 3) < lim ? s[r] : 0.f;
                 }
+#pragma unroll
+                for (int r = 0; r < 16; ++r) dp[r] = s[r] * (dp[r] - my_delta);
                 // dQ^T += K^T dS^T (contraction over the 32 keys of this sub-tile)
 #pragma unroll
                 for (int kk = 0; kk < 2; ++kk) {
