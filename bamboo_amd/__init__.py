@@ -10,7 +10,8 @@ from .config import BambooConfig
 from .layers import BottleNeck, MSELoss, TransformerLayer
 from .module import LayerSpec, PipelineError, PipelineModule, TiedLayerSpec
 from .optim import FusedAdam
-from .p2p import AllReduceException, NextStageException, PrevStageException, SeededActivationQueue
+from .p2p import (AllReduceException, LocalFabric, NextStageException, PrevStageException, SeededActivationQueue,
+                  StageKilled)
 
 __version__ = "0.1.0"
 

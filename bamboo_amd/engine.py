@@ -29,7 +29,7 @@ from . import hip, schedule
 from .config import BambooConfig
 from .module import PipelineError, PipelineModule
 from .optim import FusedAdam
-from .p2p import AllReduceException, NextStageException, PrevStageException, SeededActivationQueue
+from .p2p import AllReduceException, NextStageException, PrevStageException, SeededActivationQueue  # noqa: F401
 from .utils import get_redundant_stage_ids, get_redundant_user_stage_ids
 
 should_stop = False
@@ -124,6 +124,7 @@ class PipelineEngine:
 
         self.init_pipe_buffers()
         self._failover = None          # (failed_step, curr_step) once the successor is absorbed
+        self._prev_failover = None     # (failed_step, curr_step) once the predecessor has been replaced
         self.last_failover = None      # timing record of the most recent promotion
         self._install_sched_generator()
         self.tput_t0 = None
@@ -190,14 +191,22 @@ class PipelineEngine:
         if self._failover is not None:
             own, absorbed = self.stage_ids[0], self.stage_ids[1]
             fs, cs = self._failover
-            self._generate_sched = lambda: schedule.NextStageFailoverSchedule(
+            base = lambda: schedule.NextStageFailoverSchedule(
                 self._train_sched(own), self._train_sched(absorbed), failed_step=fs, curr_step=cs)
         elif self.r_stage_ids:
             cls = schedule.EagerRecoverySchedule if self.eager_recovery else schedule.LazyRecoverySchedule
             nxt = self.r_stage_ids[0]
-            self._generate_sched = lambda: cls(self._train_sched(self.stage_id), self._train_sched(nxt))
+            base = lambda: cls(self._train_sched(self.stage_id), self._train_sched(nxt))
         else:
-            self._generate_sched = lambda: self._train_sched(self.stage_id)
+            base = lambda: self._train_sched(self.stage_id)
+        if self._prev_failover is not None:
+            # the stage in front of this one was lost and is now run by ITS predecessor
+            # (reference engine.py:1266-1303): re-send what the lost stage had been given, then carry on
+            fs, cs = self._prev_failover
+            self._generate_sched = lambda: schedule.PrevStageFailoverSchedule(
+                self._train_sched(self.prev_stage), base(), failed_step=fs, curr_step=cs)
+        else:
+            self._generate_sched = base
 
     # ------------------------------------------------------------------ properties
     def is_first_stage(self):
@@ -273,8 +282,17 @@ class PipelineEngine:
                 # later batches run the merged stream from its first step
                 self._failover = (0, 0)
                 self._install_sched_generator()
+            elif isinstance(exc, PrevStageException) and hasattr(self.queue, "coordinate_fail_step"):
+                self._handle_prev_stage_failure(step_i)
+                status = self._exec_schedule(self._generate_sched())
+                if status is not None:
+                    raise status[1]
+                self._prev_failover = (0, 0)
+                self._install_sched_generator()
             else:
                 raise exc
+        if hasattr(self.queue, "end_batch"):
+            self.queue.end_batch(self.stage_ids)
         if self.rc_stream is not None:
             self.main_stream.wait_stream(self.rc_stream)
 
@@ -306,12 +324,30 @@ class PipelineEngine:
         torch.cuda.synchronize(self.device)   # the pause starts when the work issued before the failure has drained
         t0 = time.perf_counter()
         nxt = self.r_stage_ids[0]
-        # failed_step = 0: the in-process queue has seen nothing of the dead successor's traffic
-        # with the stage after it, so the replay keeps the successor's sends (the second replay
-        # case of the reference, schedule.py:349-353)
-        self._promote(nxt, failed_step=0, curr_step=step_i)
-        self.last_failover = {"step": step_i, "t_detect": t0, "promote_s": time.perf_counter() - t0}
+        if hasattr(self.queue, "coordinate_fail_step"):
+            # both neighbours of the lost stage agree on the earlier of the two steps at which they
+            # noticed (reference engine.py:1207-1222)
+            failed_step = self.queue.coordinate_fail_step(nxt, step_i)
+        else:
+            # the seeded queue has seen nothing of the dead successor's traffic with the stage after
+            # it, so the replay keeps the successor's sends (the second replay case of the
+            # reference, schedule.py:349-353)
+            failed_step = 0
+        self._promote(nxt, failed_step=failed_step, curr_step=step_i)
+        if hasattr(self.queue, "adopt"):
+            self.queue.adopt(nxt)
+        self.last_failover = {"step": step_i, "failed_step": failed_step, "t_detect": t0,
+                              "promote_s": time.perf_counter() - t0}
         self._replay_until = step_i
+
+    def _handle_prev_stage_failure(self, step_i):
+        """The stage in front of this one is gone (reference engine.py:1266-1303): agree on the
+        failed step with the stage that takes its place and switch to the stream that re-sends the
+        gradients of the steps before it."""
+        failed_step = self.queue.coordinate_fail_step(self.prev_stage, step_i)
+        self._prev_failover = (failed_step, step_i)
+        self._install_sched_generator()
+        self.last_failover = {"step": step_i, "failed_step": failed_step, "role": "successor of the lost stage"}
 
     def _promote(self, absorbed, failed_step, curr_step):
         """Turn the shadow layers of ``absorbed`` into active layers of this process
@@ -319,6 +355,10 @@ class PipelineEngine:
         if not self.eager_recovery:
             # lazy mode keeps CPU mirrors only: materialise the layers from them now
             self.module.build_layers(absorbed, self.param_buffers[absorbed])
+            sp = self.module.stage_params[absorbed]
+            for i, name in enumerate(sp.index):
+                sp.view(sp.exp_avg, name).copy_(self.state_buffers[absorbed][f"{i}.exp_avg"])
+                sp.view(sp.exp_avg_sq, name).copy_(self.state_buffers[absorbed][f"{i}.exp_avg_sq"])
             self.ctx = self.module.prepare_context(self.stage_ids + [absorbed], self.batch, self.seq, stream=self.main_stream)
             self.stash_bytes += self.module.allocate_stash(absorbed, self.ctx, self.micro_batches)
             act_shape = (self.batch * self.seq, self.queue.shape[2])
@@ -432,10 +472,44 @@ class PipelineEngine:
         self.global_samples += self.train_batch_size()
 
     def _exec_send_weights(self, stage_id):
-        return
+        """Publish the parameters and Adam moments of ``stage_id`` for the stage that shadows it
+        (reference engine.py:2084-2108, never wired there).  A stage is one flat arena per kind, so
+        the message is four tensors; on one GPU the link hands over references."""
+        if not hasattr(self.queue, "send_weights"):
+            return
+        sp = self.module.stage_params[stage_id]
+        self.queue.send_weights(stage_id, {"master": sp.master, "exp_avg": sp.exp_avg, "exp_avg_sq": sp.exp_avg_sq,
+                                           "step": self.optimizer.step_count(stage_id)})
 
     def _exec_recv_weights(self, stage_id):
-        return
+        """Refresh the shadow copy of ``stage_id`` (reference engine.py:2110-2137): device-to-device
+        copies into the arenas that were allocated when the shadow stage was built."""
+        if not hasattr(self.queue, "recv_weights") or stage_id not in self.r_stage_ids:
+            return
+        msg = self.queue.recv_weights(stage_id)
+        if msg is None:
+            return
+        if not self.eager_recovery:
+            # lazy mode keeps host mirrors only (engine.py:336-350): parameters and both moments come
+            # down as three flat copies and are scattered into the named buffers
+            names = self.module.param_name_buckets[stage_id]
+            host = {k: msg[k].cpu() for k in ("master", "exp_avg", "exp_avg_sq")}
+            off = 0
+            for i, name in enumerate(names):
+                buf = self.param_buffers[stage_id][name]
+                n = buf.numel()
+                buf.copy_(host["master"][off: off + n].view_as(buf))
+                self.state_buffers[stage_id][f"{i}.exp_avg"].copy_(host["exp_avg"][off: off + n].view_as(buf))
+                self.state_buffers[stage_id][f"{i}.exp_avg_sq"].copy_(host["exp_avg_sq"][off: off + n].view_as(buf))
+                off += n
+            self._shadow_step = msg["step"]
+            return
+        sp = self.module.stage_params[stage_id]
+        sp.master.copy_(msg["master"])
+        sp.exp_avg.copy_(msg["exp_avg"])
+        sp.exp_avg_sq.copy_(msg["exp_avg_sq"])
+        sp.refresh_compute()
+        self._shadow_step = msg["step"]
 
     _INSTRUCTION_MAP = {
         schedule.OptimizerStep: _exec_optimizer_step,
@@ -456,7 +530,7 @@ class PipelineEngine:
         when a neighbour failed."""
         self._reserve_pipe_buffers(pipe_schedule.num_pipe_buffers())
         for step_i, step_cmds in enumerate(pipe_schedule):
-            if getattr(self, "_replay_until", None) == step_i:
+            if getattr(self, "_replay_until", None) == step_i and self.last_failover and "t_detect" in self.last_failover:
                 # the successor's lost work has been redone: the stage is back where it was when the
                 # failure was detected (pause = detection -> here, GPU drained)
                 torch.cuda.synchronize(self.device)

@@ -34,6 +34,11 @@ class FusedAdam:
     def state(self):
         return {sid: {"exp_avg": sp.exp_avg, "exp_avg_sq": sp.exp_avg_sq} for sid, sp in self.stages.items()}
 
+    def step_count(self, stage_id=None):
+        """Steps taken so far (one counter for the group, as in the reference: every stage of a
+        pipeline steps once per batch, so an absorbed stage continues with the same count)."""
+        return self.param_groups[0].get("step", 0)
+
     def zero_grad(self):
         for sp in self.stages.values():
             sp.grad.zero_()

@@ -128,3 +128,186 @@ class SeededActivationQueue:
     def ping(self, stage_id):
         if self.dead_from is not None and stage_id == self.dead_stage and self.dead_from <= 0:
             raise NextStageException(f"successor of stage {stage_id} does not answer")
+
+
+# =============================================================================================
+# Several stages in one process: a mailbox fabric between engines that run in threads
+# =============================================================================================
+import threading  # noqa: E402
+
+
+class StageKilled(BaseException):
+    """Raised inside the thread of a stage that the fabric preempts (the analogue of the spot
+    instance disappearing): it unwinds ``train_batch`` of that engine and nothing else."""
+
+
+class FabricTimeout(RuntimeError):
+    ...
+
+
+class LocalFabric:
+    """Stage-to-stage transfers between engines of ONE process that share one GPU.
+
+    Each engine runs ``train_batch`` in its own thread and blocks in ``recv_*`` until the
+    neighbour has produced the tensor, as with ``dist.recv`` (p2p_direct.py:11-17).  All
+    engines issue their kernels to the same HIP stream, so a tensor handed over here is ordered
+    before its consumer's kernels without any further synchronisation.
+
+    Messages are keyed by (batch, kind, producing stage, consuming stage, micro-batch), are not
+    removed when read and are idempotent to re-send: after a stage is lost, its predecessor
+    replays the lost stage's stream (``NextStageFailoverSchedule``) and finds everything the
+    stage after it has sent, whether or not the dead stage had consumed it.
+
+    Failure protocol of the reference (engine.py:1190-1303): both neighbours of the dead stage
+    report the step at which they noticed (``fail-step-<rank>`` in the etcd store there,
+    :meth:`FabricEndpoint.coordinate_fail_step` here) and continue from the smaller one.
+    """
+
+    def __init__(self, num_stages, shape, dtype, micro_batches, device="cuda:0", timeout=120.0):
+        self.num_stages, self.shape, self.dtype, self.M = num_stages, tuple(shape), dtype, micro_batches
+        self.device, self.timeout = torch.device(device), timeout
+        self.cv = threading.Condition()
+        self.box = {}
+        self.dead = set()          # stages whose engine is gone and whose layers nobody has adopted yet
+        self.kill_at = {}          # stage -> micro-batch at which its engine stops
+        self.fail_steps = {}       # dead stage -> {reporting stage: step}
+        self.finished = {}         # stage -> last batch it completed
+
+    def endpoint(self, stage_id):
+        return FabricEndpoint(self, stage_id)
+
+    def kill(self, stage_id, at_micro_batch=0):
+        """The engine of ``stage_id`` stops at its next transfer that concerns a micro-batch
+        >= ``at_micro_batch`` (of the batch it is in)."""
+        if stage_id in (0, self.num_stages - 1):
+            raise ValueError("the first and the last stage have no two neighbours to recover them "
+                             "(reference engine.py:1313-1315)")
+        with self.cv:
+            self.kill_at[stage_id] = at_micro_batch
+
+
+class FabricEndpoint:
+    """What one engine sees of the fabric: the ``activation_queue`` interface of
+    :class:`SeededActivationQueue` for the stage(s) it hosts."""
+
+    grad_mode = "queue"
+    key_lens = None
+    dead_from = dead_stage = None
+
+    def __init__(self, fabric, stage_id):
+        self.f, self.stage = fabric, stage_id
+        self.shape, self.dtype, self.M, self.device = fabric.shape, fabric.dtype, fabric.M, fabric.device
+        self.batch = -1
+        self.acknowledged = set()  # dead stages whose loss this endpoint has already reported
+        self.loss = torch.zeros(1, dtype=torch.float32, device=self.device)
+
+    # ---------------------------------------------------------------- helpers
+    def _check_kill(self, k):
+        f = self.f
+        with f.cv:
+            at = f.kill_at.get(self.stage)
+            if at is not None and k >= at:
+                del f.kill_at[self.stage]
+                f.dead.add(self.stage)
+                f.cv.notify_all()
+                raise StageKilled(f"stage {self.stage} preempted at micro-batch {k}")
+
+    def _put(self, kind, src, dst, k, tensor, exc):
+        f = self.f
+        with f.cv:
+            if dst in f.dead and dst not in self.acknowledged:
+                raise exc(f"stage {dst} is gone ({kind} of micro-batch {k} from stage {src})")
+            f.box[(self.batch, kind, src, dst, k)] = tensor
+            f.cv.notify_all()
+
+    def _get(self, kind, src, dst, k, exc):
+        f = self.f
+        key = (self.batch, kind, src, dst, k)
+        waited = 0.0
+        with f.cv:
+            while key not in f.box:
+                if src in f.dead and src not in self.acknowledged:
+                    raise exc(f"stage {src} is gone ({kind} of micro-batch {k} for stage {dst})")
+                if waited >= f.timeout:
+                    raise FabricTimeout(f"stage {dst} waited {waited:.0f}s for {kind} {k} of stage {src}")
+                f.cv.wait(0.5)
+                waited += 0.5
+            return f.box[key]
+
+    # ---------------------------------------------------------------- queue interface
+    def start_batch(self):
+        self.batch += 1
+        self.loss.zero_()
+        f = self.f
+        with f.cv:   # neighbours are never more than one batch apart
+            for key in [key for key in f.box if isinstance(key[0], int) and key[0] < self.batch - 1]:
+                del f.box[key]
+
+    def end_batch(self, stage_ids):
+        f = self.f
+        with f.cv:
+            for s in stage_ids:
+                f.finished[s] = self.batch
+            f.cv.notify_all()
+
+    def key_len(self, k):
+        return None
+
+    def recv_activation(self, k):
+        self._check_kill(k)
+        return self._get("act", self.stage - 1, self.stage, k, PrevStageException)
+
+    def send_activation(self, k, tensor, stage_id, stream=None):
+        self._check_kill(k)
+        self._put("act", stage_id, stage_id + 1, k, tensor, NextStageException)
+
+    def recv_grad(self, k, stage_id):
+        self._check_kill(k)
+        return self._get("grad", stage_id + 1, stage_id, k, NextStageException)
+
+    def send_grad(self, k, tensor, stage_id):
+        self._check_kill(k)
+        self._put("grad", stage_id, stage_id - 1, k, tensor, PrevStageException)
+
+    def ping(self, stage_id):
+        with self.f.cv:
+            if stage_id in self.f.dead and stage_id not in self.acknowledged:
+                raise NextStageException(f"stage {stage_id} does not answer")
+
+    # ---------------------------------------------------------------- weights of a stage for its shadow
+    def send_weights(self, stage_id, arenas):
+        f = self.f
+        with f.cv:
+            f.box[("weights", stage_id)] = arenas
+            f.cv.notify_all()
+
+    def recv_weights(self, stage_id):
+        with self.f.cv:
+            return self.f.box.get(("weights", stage_id))
+
+    # ---------------------------------------------------------------- failure protocol
+    def coordinate_fail_step(self, dead_stage, step):
+        """Report the step at which this engine noticed that ``dead_stage`` is gone and return the
+        smallest step reported by its neighbours (both of them unless the other one has already
+        finished the batch without needing the dead stage any more)."""
+        f = self.f
+        other = dead_stage + 1 if self.stage < dead_stage else dead_stage - 1
+        waited = 0.0
+        with f.cv:
+            self.acknowledged.add(dead_stage)
+            reports = f.fail_steps.setdefault(dead_stage, {})
+            reports[self.stage] = step
+            f.cv.notify_all()
+            while other not in reports and f.finished.get(other, -1) < self.batch:
+                if waited >= f.timeout:
+                    raise FabricTimeout(f"stage {self.stage}: no failure report from stage {other}")
+                f.cv.wait(0.5)
+                waited += 0.5
+            return min(reports.values())
+
+    def adopt(self, dead_stage):
+        """The caller now runs the layers of ``dead_stage``: its transfers flow again."""
+        f = self.f
+        with f.cv:
+            f.dead.discard(dead_stage)
+            f.cv.notify_all()

@@ -7,8 +7,9 @@ against.  Only ``tests/``, ``__graft_entry__.smoke()`` and the ``cpu_baseline``
 leg of ``bench.py`` may import it; ``bamboo_amd`` never does.
 
 Modules
-  schedule  instruction streams (1F1B TrainSchedule, eager-RC merge, next-stage
-            failover merge) -- follows deepspeed/runtime/pipe/schedule.py
+  schedule  instruction streams (1F1B TrainSchedule, eager-RC merge, next-stage,
+            previous-stage and data-parallel failover merges)
+            -- follows deepspeed/runtime/pipe/schedule.py
   layers    transformer layer / bottleneck block maths on torch CPU ops
             -- follows DeepSpeedExamples/pipeline_parallelism/{transformer,resnet}.py
   adam      the fused-Adam update formula -- follows csrc/adam/multi_tensor_adam.cu
@@ -24,6 +25,12 @@ Pin status (what each function was checked against, see tests/test_oracle_*.py):
   schedule.eager_merge           hand trace + "RC F(k) directly before RecvGrad(k)"
   schedule.next_stage_failover   semantic pin: gradients of the merged stream equal
                                  those of own+shadow run as one stage
+  schedule.prev_stage_failover   what its definition fixes: before curr_step only the
+                                 own SendGrad of steps < failed_step, each once, then the
+                                 own stream unchanged; end to end: a pipeline that loses
+                                 a stage mid-batch ends with the gradients and weights of
+                                 the run in which nothing fails (tests/test_gpu_pipeline.py)
+  schedule.allreduce_failover    its definition (empty before failed_step, own after)
   layers.*                       reduce to torch library routines (linear, softmax,
                                  conv2d, batch_norm); custom LayerNorm checked against
                                  the closed form with torch.std (unbiased)

@@ -128,6 +128,26 @@ def next_stage_failover(own_steps, next_steps, failed_step, curr_step):
     return out
 
 
+def prev_stage_failover(own_steps, failed_step, curr_step):
+    """Stream of the stage AFTER a lost one (schedule.py:433-454): steps it has already run are
+    not run again, except that the gradients sent before ``failed_step`` are sent once more (the
+    stage that replays the lost work has never received them); from ``curr_step`` on the own
+    stream continues, without weight sends and without the lazy-mode pings."""
+    out = []
+    for i, own in enumerate(own_steps):
+        if i < curr_step:
+            out.append([c for c in own if c[0] == "SendGrad"] if i < failed_step else [])
+        else:
+            out.append([c for c in own if c[0] != "SendWeights" and not (c[0] == "RecvActivation" and c[1] == -1)])
+    return out
+
+
+def allreduce_failover(own_steps, failed_step):
+    """Stream of a data-parallel peer of a lost rank (schedule.py:457-466): nothing before the
+    failed step, the own stream from it on."""
+    return [[] if i < failed_step else list(own) for i, own in enumerate(own_steps)]
+
+
 def redundant_stage_ids(level, stage_id, stages):
     """Stages whose layers ``stage_id`` shadows (redundancy.py:7-19)."""
     return [(stage_id + i) % stages for i in range(1, level + 1)]

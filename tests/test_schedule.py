@@ -36,6 +36,32 @@ def test_eager_and_failover_equal_oracle(stages, mbs):
             assert got == osched.next_stage_failover(own, nxt, fs, cs)
 
 
+@pytest.mark.parametrize("stages,mbs", [(3, 3), (4, 4), (4, 8), (5, 7)])
+def test_prev_stage_and_allreduce_failover_equal_oracle(stages, mbs):
+    mk = lambda s: S.TrainSchedule(micro_batches=mbs, stages=stages, stage_id=s)
+    for sid in range(2, stages):                  # the stage after a lost middle stage
+        own = osched.train_schedule(mbs, stages, sid)
+        eager_own = osched.eager_merge(own, osched.train_schedule(mbs, stages, (sid + 1) % stages))
+        T = len(own)
+        for fs, cs in [(0, 0), (T // 3, T // 3), (T // 3, T // 2), (T // 2, T - 1)]:
+            got = as_tuples(S.PrevStageFailoverSchedule(mk(sid - 1), mk(sid), failed_step=fs, curr_step=cs))
+            want = osched.prev_stage_failover(own, fs, cs)
+            assert got == want
+            # what the definition fixes: before curr_step nothing but gradient re-sends, every own
+            # gradient send of the steps before failed_step exactly once, afterwards the own stream
+            resent = [c for i, cmds in enumerate(want) if i < cs for c in cmds]
+            assert all(c[0] == "SendGrad" for c in resent)
+            assert resent == [c for i, cmds in enumerate(own) if i < min(fs, cs) for c in cmds if c[0] == "SendGrad"]
+            assert want[cs:] == own[cs:]
+            # wrapped around the stage's own RC stream, as the engine builds it
+            wrapped = as_tuples(S.PrevStageFailoverSchedule(
+                mk(sid - 1), S.EagerRecoverySchedule(mk(sid), mk((sid + 1) % stages)), failed_step=fs, curr_step=cs))
+            assert wrapped == osched.prev_stage_failover(eager_own, fs, cs)
+        for fs in (0, T // 2, T):
+            got = as_tuples(S.AllReduceFailoverSchedule(mk(sid), [[] for _ in range(T)], failed_step=fs))
+            assert got == osched.allreduce_failover(own, fs)
+
+
 def test_upstream_invariants():
     """tests/unit/test_pipe_schedule.py:126-157 of the reference tree, on this implementation."""
     sched = S.TrainSchedule(stages=3, micro_batches=4, stage_id=0)
