@@ -22,6 +22,7 @@ What is different underneath:
 """
 import signal
 import time
+from collections import OrderedDict
 
 import torch
 
@@ -510,6 +511,57 @@ class PipelineEngine:
         sp.exp_avg_sq.copy_(msg["exp_avg_sq"])
         sp.refresh_compute()
         self._shadow_step = msg["step"]
+
+    # ------------------------------------------------------------------ moving layers (reconfiguration)
+    def _stage_of_layer(self, layer_idx):
+        prefix = f"{layer_idx}."
+        for sid, sp in self.module.stage_params.items():
+            if any(k.startswith(prefix) for k in sp.index):
+                return sid
+        raise PipelineError(f"layer {layer_idx} is not built in this process")
+
+    def get_layer_state(self, layer_idxs):
+        """``{idx: [state_dict, [ {exp_avg, exp_avg_sq} per parameter ]]}``: the ``state`` argument of
+        ``send_layers`` (reference engine.py:893-901, ``get_optimizer_state`` :1005-1014)."""
+        out = {}
+        for idx in layer_idxs:
+            sp = self.module.stage_params[self._stage_of_layer(idx)]
+            sd = self.module.layer_state_dict(idx)
+            opt = [{"exp_avg": sp.view(sp.exp_avg, f"{idx}.{name}"), "exp_avg_sq": sp.view(sp.exp_avg_sq, f"{idx}.{name}")}
+                   for name in sd]
+            out[idx] = [sd, opt]
+        return out
+
+    def send_layers(self, dst_rank, layer_idxs, state):
+        """Layers and their Adam moments as the reference's two flat tensors (engine.py:893-927).
+        Returns them; a fabric that can carry them also gets them handed over."""
+        from .wire import pack_layers
+        layer_tensor, optim_tensor = pack_layers(layer_idxs, state)
+        if hasattr(self.queue, "send_layer_tensors"):
+            self.queue.send_layer_tensors(dst_rank, layer_tensor, optim_tensor)
+        return layer_tensor, optim_tensor
+
+    def recv_layers(self, src_rank, layer_idxs, tensors=None):
+        """Inverse of :meth:`send_layers` (engine.py:929-1003): ``recvd_state`` keyed by layer index.
+        Shapes come from this process's own layer specs, as in the reference."""
+        from .wire import unpack_layers
+        if tensors is None:
+            tensors = self.queue.recv_layer_tensors(src_rank)
+        shapes = {}
+        for idx in layer_idxs:
+            sd = self.module.layer_state_dict(idx)
+            shapes[idx] = OrderedDict((k, tuple(v.shape)) for k, v in sd.items())
+        return unpack_layers(layer_idxs, shapes, tensors[0], tensors[1])
+
+    def load_layer_state(self, recvd_state):
+        """Put received layers (parameters and moments) into this process's arenas."""
+        for idx, (sd, opt) in recvd_state.items():
+            sp = self.module.stage_params[self._stage_of_layer(idx)]
+            for (name, t), moments in zip(sd.items(), opt):
+                sp.view(sp.master, f"{idx}.{name}").copy_(t)
+                sp.view(sp.exp_avg, f"{idx}.{name}").copy_(moments["exp_avg"])
+                sp.view(sp.exp_avg_sq, f"{idx}.{name}").copy_(moments["exp_avg_sq"])
+            sp.refresh_compute()
 
     _INSTRUCTION_MAP = {
         schedule.OptimizerStep: _exec_optimizer_step,

@@ -243,6 +243,46 @@ class PipelineModule:
         self.param_name_buckets.setdefault(stage_id, names)
         return names
 
+    # ------------------------------------------------------------------ layer state and checkpoints
+    def layer_state_dict(self, layer_idx):
+        """``state_dict`` of one layer (global index): ordered ``{name: fp32 master view}``."""
+        for sid, sp in self.stage_params.items():
+            prefix = f"{layer_idx}."
+            keys = [k for k in sp.index if k.startswith(prefix)]
+            if keys:
+                return OrderedDict((k[len(prefix):], sp.view(sp.master, k)) for k in keys)
+        raise PipelineError(f"layer {layer_idx} is not built in this process")
+
+    def save_state_dict(self, save_dir, stage_id=None):
+        """One ``layer_XX-model_states.pt`` per layer of the stage (reference module.py:804-826)."""
+        import os
+
+        from .wire import ckpt_layer_path
+        os.makedirs(save_dir, exist_ok=True)
+        sid = self.stage_id if stage_id is None else stage_id
+        for idx in range(self.parts[sid], self.parts[sid + 1]):
+            sd = OrderedDict((k, v.detach().clone().cpu()) for k, v in self.layer_state_dict(idx).items())
+            torch.save(sd, ckpt_layer_path(save_dir, idx))
+
+    def load_state_dir(self, load_dir, strict=True, stage_id=None):
+        """Read the per-layer files back into the master arena (reference module.py:828-850)."""
+        import os
+
+        from .wire import ckpt_layer_path
+        sid = self.stage_id if stage_id is None else stage_id
+        sp = self.stage_params[sid]
+        for idx in range(self.parts[sid], self.parts[sid + 1]):
+            path = ckpt_layer_path(load_dir, idx)
+            if not os.path.exists(path):
+                if strict:
+                    raise FileNotFoundError(path)
+                continue
+            sd = torch.load(path, map_location="cpu", weights_only=True)
+            want = self.layer_state_dict(idx)
+            if strict and set(sd) != set(want):
+                raise PipelineError(f"{path}: keys {sorted(sd)} do not match the layer's {sorted(want)}")
+            sp.load({f"{idx}.{k}": v for k, v in sd.items()})
+
     def get_named_param(self, stage_id):
         """(name, fp32 master view) pairs of a built stage."""
         sp = self.stage_params[stage_id]

@@ -285,6 +285,25 @@ class FabricEndpoint:
         with self.f.cv:
             return self.f.box.get(("weights", stage_id))
 
+    # ---------------------------------------------------------------- whole layers (reconfiguration)
+    def send_layer_tensors(self, dst_stage, layer_tensor, optim_tensor):
+        f = self.f
+        with f.cv:
+            f.box[("layers", self.stage, dst_stage)] = (layer_tensor, optim_tensor)
+            f.cv.notify_all()
+
+    def recv_layer_tensors(self, src_stage):
+        f = self.f
+        key = ("layers", src_stage, self.stage)
+        waited = 0.0
+        with f.cv:
+            while key not in f.box:
+                if waited >= f.timeout:
+                    raise FabricTimeout(f"stage {self.stage} waited {waited:.0f}s for layers of stage {src_stage}")
+                f.cv.wait(0.5)
+                waited += 0.5
+            return f.box.pop(key)
+
     # ---------------------------------------------------------------- failure protocol
     def coordinate_fail_step(self, dead_stage, step):
         """Report the step at which this engine noticed that ``dead_stage`` is gone and return the

@@ -13,6 +13,8 @@ Modules
   layers    transformer layer / bottleneck block maths on torch CPU ops
             -- follows DeepSpeedExamples/pipeline_parallelism/{transformer,resnet}.py
   adam      the fused-Adam update formula -- follows csrc/adam/multi_tensor_adam.cu
+  wire      flat wire format of whole layers with their Adam moments
+            -- follows deepspeed/runtime/pipe/engine.py send_layers / recv_layers
   stage     interpreter that runs an instruction stream over the oracle layers
             with torch.autograd -- follows deepspeed/runtime/pipe/engine.py _exec_*
 
@@ -31,6 +33,8 @@ Pin status (what each function was checked against, see tests/test_oracle_*.py):
                                  a stage mid-batch ends with the gradients and weights of
                                  the run in which nothing fails (tests/test_gpu_pipeline.py)
   schedule.allreduce_failover    its definition (empty before failed_step, own after)
+  wire.pack_layers/unpack_layers hand-written known answer with distinct elements (order of
+                                 layers, parameters and moments), round trip
   layers.*                       reduce to torch library routines (linear, softmax,
                                  conv2d, batch_norm); custom LayerNorm checked against
                                  the closed form with torch.std (unbiased)

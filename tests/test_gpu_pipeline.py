@@ -172,3 +172,31 @@ def test_without_refresh_the_shadow_goes_stale(hiplib):
     assert not torch.equal(e0.module.stage_params[1].master, pipe.engines[1].module.stage_params[1].master)
     pipe.sync_shadow_weights()
     assert torch.equal(e0.module.stage_params[1].master, pipe.engines[1].module.stage_params[1].master)
+
+
+def test_layers_travel_between_engines_and_through_checkpoints(hiplib, tmp_path):
+    """send_layers / recv_layers (two flat tensors) and layer_XX-model_states.pt files."""
+    dtype = torch.bfloat16
+    a = make_pipeline(dtype, layers_per_stage=2)
+    a.train_batch()                                        # moments and weights away from their initial values
+    src, dst = a.engines[1], a.engines[0]                  # engine 0 holds shadow copies of layers 2 and 3
+    idxs = [2, 3]
+    state = src.get_layer_state(idxs)
+    lt, ot = src.send_layers(0, idxs, state)
+    n = sum(v.numel() for v in state[2][0].values()) + sum(v.numel() for v in state[3][0].values())
+    assert lt.numel() == n and ot.numel() == 2 * n and lt.dtype == torch.float32
+    sp_dst, sp_src = dst.module.stage_params[1], src.module.stage_params[1]
+    sp_dst.master.zero_(); sp_dst.exp_avg.zero_(); sp_dst.exp_avg_sq.zero_()
+    dst.load_layer_state(dst.recv_layers(1, idxs))         # through the fabric mailbox
+    assert torch.equal(sp_dst.master, sp_src.master) and torch.equal(sp_dst.exp_avg, sp_src.exp_avg)
+    assert torch.equal(sp_dst.exp_avg_sq, sp_src.exp_avg_sq) and torch.equal(sp_dst.compute, sp_src.compute)
+    # checkpoint files, one per layer, loadable with weights_only
+    src.module.save_state_dict(str(tmp_path))
+    assert sorted(p.name for p in tmp_path.iterdir()) == ["layer_02-model_states.pt", "layer_03-model_states.pt"]
+    sd = torch.load(str(tmp_path / "layer_02-model_states.pt"), weights_only=True)
+    assert list(sd) == list(src.module.layer_state_dict(2))
+    sp_dst.master.zero_()
+    dst.module.load_state_dir(str(tmp_path), stage_id=1)
+    assert torch.equal(sp_dst.master, sp_src.master) and torch.equal(sp_dst.compute, sp_src.compute)
+    with pytest.raises(FileNotFoundError):
+        dst.module.load_state_dir(str(tmp_path))           # stage 0's own layers were not saved
