@@ -30,11 +30,8 @@ struct GemmArgs {
 // ---- tile order: consecutive logical tiles land on the same XCD (workgroups are dealt
 // round-robin over the 8 XCDs, each with a private L2), and walk the output in column
 // panels of GROUP_M row-tiles so that an XCD's resident tiles share A rows and B columns.
-__device__ __forceinline__ void tile_coords(int bid, int tiles_m, int tiles_n, int& tm, int& tn) {
-    const int total = tiles_m * tiles_n;
-    int lid = bid;
-    const int per = total / 8;
-    if (per > 0 && bid < per * 8) lid = (bid % 8) * per + bid / 8;
+// logical tile -> (row tile, column tile): column panels of GROUP_M row-tiles
+__device__ __forceinline__ void panel_coords(int lid, int tiles_m, int tiles_n, int& tm, int& tn) {
     constexpr int GROUP_M = 8;
     const int width = GROUP_M * tiles_n;
     const int group = lid / width;
@@ -42,6 +39,15 @@ __device__ __forceinline__ void tile_coords(int bid, int tiles_m, int tiles_n, i
     const int gsize = min(tiles_m - first_m, GROUP_M);
     tm = first_m + (lid % width) % gsize;
     tn = (lid % width) / gsize;
+}
+// block id -> logical tile such that XCD x (which receives the block ids = x mod 8) owns the
+// contiguous range [x * total / 8, (x + 1) * total / 8) of logical tiles
+__device__ __forceinline__ int xcd_contiguous(int bid, int total) {
+    const int per = total / 8;
+    return (per > 0 && bid < per * 8) ? (bid % 8) * per + bid / 8 : bid;
+}
+__device__ __forceinline__ void tile_coords(int bid, int tiles_m, int tiles_n, int& tm, int& tn) {
+    panel_coords(xcd_contiguous(bid, tiles_m * tiles_n), tiles_m, tiles_n, tm, tn);
 }
 
 // Generic scalar epilogue.  T = operand dtype (bias/aux/resid), output fp32 or T.
@@ -398,7 +404,8 @@ template <int BR, int T, bool KM> struct FragReader {
 };
 
 template <int BM, int BN, int WM, int WN, bool AKM, bool BKM, bool DB, int STAGES>
-__device__ __forceinline__ void gemm_bf16_dma_body(const GemmArgs& g, const int block_id, const int batch_id) {
+__device__ __forceinline__ void gemm_bf16_dma_body(const GemmArgs& g, const int block_id, const int batch_id,
+                                                   const bool logical_id = false) {
     constexpr int NW = WM * WN;
     static_assert(STAGES >= 3, "the ring needs one stage being read, one landing, one in flight");
     constexpr int WTM = BM / WM, WTN = BN / WN, TM = WTM / 32, TN = WTN / 32;
@@ -411,7 +418,8 @@ __device__ __forceinline__ void gemm_bf16_dma_body(const GemmArgs& g, const int 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wm = wave / WN, wn = wave % WN;
     int tile_m, tile_n;
-    tile_coords(block_id, g.tiles_m, g.tiles_n, tile_m, tile_n);
+    if (logical_id) panel_coords(block_id, g.tiles_m, g.tiles_n, tile_m, tile_n);
+    else tile_coords(block_id, g.tiles_m, g.tiles_n, tile_m, tile_n);
     const int m0 = tile_m * BM, n0 = tile_n * BN;
     const int b1 = batch_id / g.nb2, b2 = batch_id % g.nb2;
     const bf16* A = (const bf16*)g.A + b1 * g.sA1 + b2 * g.sA2;
@@ -603,9 +611,13 @@ struct GroupedArgs {
 };
 template <int BM, int BN, int WM, int WN, bool AKM, bool BKM, bool DB, int STAGES>
 __global__ __launch_bounds__(WM* WN * 64) void gemm_bf16_dma_grouped_kernel(const GroupedArgs G) {
+    // The tiles of all problems form one list; an XCD takes a contiguous stretch of it, so its
+    // resident blocks are a few wide rectangles of one or two problems (few distinct operand
+    // panels in its L2) rather than a narrow slice of every problem.
+    const int lid = xcd_contiguous(blockIdx.x, G.first_block[G.count]);
     int pi = 0;
-    while (pi + 1 < G.count && (int)blockIdx.x >= G.first_block[pi + 1]) ++pi;
-    gemm_bf16_dma_body<BM, BN, WM, WN, AKM, BKM, DB, STAGES>(G.p[pi], blockIdx.x - G.first_block[pi], 0);
+    while (pi + 1 < G.count && lid >= G.first_block[pi + 1]) ++pi;
+    gemm_bf16_dma_body<BM, BN, WM, WN, AKM, BKM, DB, STAGES>(G.p[pi], lid - G.first_block[pi], 0, true);
 }
 
 // =========================================================================================
