@@ -46,7 +46,7 @@ class PipelineEngine:
     def __init__(self, args=None, model=None, optimizer=None, model_parameters=None, training_data=None,
                  lr_scheduler=None, mpu=None, dist_init_required=None, collate_fn=None, config=None,
                  config_params=None, redundancy_level=0, sync_save=False, eager_recovery=False, prev_state={},
-                 activation_queue=None, rc_stream=False, install_signal_handler=True):
+                 activation_queue=None, rc_stream=False, install_signal_handler=True, use_graphs=False):
         if not isinstance(model, PipelineModule):
             raise PipelineError("model must base PipelineModule")
         hip.init()
@@ -96,6 +96,14 @@ class PipelineEngine:
         # execution lanes: the stage's own work on the current stream, redundant forwards
         # optionally on a second stream of the same (default) priority
         self.main_stream = torch.cuda.current_stream(self.device)
+        # Replay of the per-micro-batch launch sequences as HIP graphs: every forward or backward
+        # of (stage, micro-batch) touches the same static buffers in every batch, so its ~100
+        # launches are captured the second time they occur and launched as one graph afterwards.
+        self.use_graphs = bool(use_graphs)
+        if self.use_graphs and self.main_stream.cuda_stream == 0:
+            raise PipelineError("use_graphs needs the engine built and run under a created stream "
+                                "(torch.cuda.stream(...)): the default stream cannot be captured")
+        self._graphs = {}
         self.rc_stream = torch.cuda.Stream(self.device) if (rc_stream and self.r_stage_ids and eager_recovery) else None
         built = list(self.stage_ids) + (list(self.r_stage_ids) if self.eager_recovery else [])
         self.ctx = model.prepare_context(built, self.batch, self.seq, stream=self.main_stream)
@@ -377,6 +385,25 @@ class PipelineEngine:
         self._failover = (failed_step, curr_step)
         self._install_sched_generator()
 
+    # ------------------------------------------------------------------ graph replay
+    def _graphed(self, key, stream, issue):
+        """Run ``issue()`` (which only launches kernels of this library on ``stream`` and returns a
+        value that does not change between batches): eagerly the first time ``key`` occurs, captured
+        and launched the second time, replayed from then on."""
+        if not self.use_graphs or hip.gemm_hook is not None:
+            return issue()
+        state = self._graphs.get(key)
+        if state is None:
+            self._graphs[key] = "seen"
+            return issue()
+        if state == "seen":
+            with hip.Graph.capture(stream) as graph:
+                out = issue()
+            self._graphs[key] = (graph, out)
+        graph, out = self._graphs[key]
+        graph.launch(stream)
+        return out
+
     # ------------------------------------------------------------------ instruction handlers
     def _exec_load_micro_batch(self, buffer_id):
         if self.pipe_buffers["label"][buffer_id] is not None or self.pipe_buffers["data"][buffer_id] is not None:
@@ -439,7 +466,9 @@ class PipelineEngine:
         ctx.redundant = redundant
         if redundant and self.rc_stream is not None:
             self.rc_stream.wait_event(self._fwd_done[buffer_id])
-        out = self.module.forward(inputs, stage_id, slot=buffer_id, ctx=ctx)
+        kl = ctx.key_len
+        key = ("F", stage_id, buffer_id, id(ctx), inputs.data_ptr(), None if kl is None else kl.data_ptr())
+        out = self._graphed(key, ctx.stream, lambda: self.module.forward(inputs, stage_id, slot=buffer_id, ctx=ctx))
         self.pipe_buffers[out_key][buffer_id] = out
         if not redundant and self.rc_stream is not None:
             self._fwd_done[buffer_id].record(self.main_stream)
@@ -455,7 +484,9 @@ class PipelineEngine:
             raise PipelineError(f"BackwardPass({buffer_id}, {stage_id}) without a received gradient")
         self.ctx.key_len = self.queue.key_len(buffer_id)
         dst = self._input_grad_store[stage_id][buffer_id]
-        self.module.backward(grad, dst, stage_id, slot=buffer_id, ctx=self.ctx)
+        kl = self.ctx.key_len
+        key = ("B", stage_id, buffer_id, id(self.ctx), grad.data_ptr(), dst.data_ptr(), None if kl is None else kl.data_ptr())
+        self._graphed(key, self.ctx.stream, lambda: self.module.backward(grad, dst, stage_id, slot=buffer_id, ctx=self.ctx))
         key = f"input_grad_{stage_id}"
         if key in self.pipe_buffers:
             self.pipe_buffers[key][buffer_id] = dst

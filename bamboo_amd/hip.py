@@ -25,7 +25,7 @@ LN_CODES = {"standard": LN_STANDARD, "annotated": LN_ANNOTATED}
 EXPORTS = (
     "bb_version", "bb_last_error", "bb_init", "bb_gemm", "bb_gemm_grouped", "bb_gemm_variant", "bb_layernorm_fwd",
     "bb_layernorm_bwd_workspace", "bb_layernorm_bwd", "bb_colsum_workspace", "bb_colsum_acc",
-    "bb_softmax_fwd", "bb_softmax_bwd", "bb_attention_fwd", "bb_attention_bwd", "bb_residual_add", "bb_act_fwd", "bb_bn_workspace", "bb_batchnorm_fwd", "bb_batchnorm_bwd", "bb_patch3x3", "bb_mse_workspace", "bb_mse_fwd_bwd",
+    "bb_softmax_fwd", "bb_softmax_bwd", "bb_attention_fwd", "bb_attention_bwd", "bb_residual_add", "bb_act_fwd", "bb_bn_workspace", "bb_batchnorm_fwd", "bb_batchnorm_bwd", "bb_patch3x3", "bb_mse_workspace", "bb_mse_fwd_bwd", "bb_graph_begin", "bb_graph_end", "bb_graph_launch", "bb_graph_destroy",
     "bb_adam_multi", "bb_cast", "bb_fill_f32",
 )
 
@@ -89,6 +89,10 @@ def lib():
     L.bb_attention_bwd.argtypes = [c_int] * 6 + [c_void_p, c_void_p, c_void_p, c_int64, c_void_p, c_void_p, c_int64,
                                    c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_void_p, c_void_p]
     L.bb_residual_add.argtypes = [c_int, c_int64, c_void_p, c_void_p, c_void_p, c_void_p]
+    L.bb_graph_begin.argtypes = [c_void_p]
+    L.bb_graph_end.argtypes = [c_void_p, POINTER(c_void_p)]
+    L.bb_graph_launch.argtypes = [c_void_p, c_void_p]
+    L.bb_graph_destroy.argtypes = [c_void_p]
     L.bb_act_fwd.argtypes = [c_int, c_int, c_int64, c_void_p, c_void_p, c_void_p, c_void_p]
     L.bb_bn_workspace.argtypes = [c_int]
     L.bb_bn_workspace.restype = c_int64
@@ -317,6 +321,45 @@ def act_fwd(x, out, act, dact=None, stream=None):
     """out = act(x); dact (optional, may be x itself) receives act'(x)."""
     check(lib().bb_act_fwd(dtype_code(x.dtype), act, x.numel(), _ptr(x), _ptr(out), _ptr(dact), stream_ptr(stream)),
           "bb_act_fwd")
+
+
+class Graph:
+    """An executable HIP graph captured from a stream (``with Graph.capture(stream) as g: ...``)."""
+
+    def __init__(self):
+        self.exec = None
+
+    class _Capture:
+        def __init__(self, graph, stream):
+            self.graph, self.stream = graph, stream
+
+        def __enter__(self):
+            check(lib().bb_graph_begin(stream_ptr(self.stream)), "bb_graph_begin")
+            return self.graph
+
+        def __exit__(self, exc_type, exc, tb):
+            out = c_void_p()
+            rc = lib().bb_graph_end(stream_ptr(self.stream), ctypes.byref(out))
+            if exc_type is None:
+                check(rc, "bb_graph_end")
+                self.graph.exec = out
+            elif rc == 0 and out:
+                lib().bb_graph_destroy(out)
+            return False
+
+    @classmethod
+    def capture(cls, stream):
+        return cls._Capture(cls(), stream)
+
+    def launch(self, stream):
+        check(lib().bb_graph_launch(self.exec, stream_ptr(stream)), "bb_graph_launch")
+
+    def __del__(self):
+        try:
+            if self.exec:
+                lib().bb_graph_destroy(self.exec)
+        except Exception:
+            pass
 
 
 def bn_workspace(cols):

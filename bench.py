@@ -48,7 +48,7 @@ MEASURED_TRAFFIC_BYTES = {
 }
 
 
-def build_engine(cfg, rc, rc_stream, seed=1138):
+def build_engine(cfg, rc, rc_stream, seed=1138, use_graphs=False):
     import torch
 
     import bamboo_amd
@@ -70,7 +70,7 @@ def build_engine(cfg, rc, rc_stream, seed=1138):
           "bf16": {"enabled": cfg["dtype"] == "bf16"}}
     engine, _, _, _ = bamboo_amd.initialize(model=model, config=ds, redundancy_level=1 if rc else 0,
                                             eager_recovery=rc, activation_queue=q, rc_stream=rc_stream,
-                                            install_signal_handler=False)
+                                            install_signal_handler=False, use_graphs=use_graphs)
     return engine, q
 
 
@@ -201,6 +201,10 @@ def main():
     ap.add_argument("--no-probe", action="store_true", help="do not bracket GEMM launches with events")
     ap.add_argument("--gemm-shapes", action="store_true", help="print a per-shape GEMM table on stderr")
     ap.add_argument("--skip-rc-off", action="store_true")
+    ap.add_argument("--graphs", type=int, default=0,
+                    help="replay each micro-batch's forward/backward launch sequence as a HIP graph in the RC-off leg and "
+                         "in the leg `value` is quoted on (captured during warm-up; the probed leg always launches eagerly); "
+                         "off by default: at these shapes the GPU is never waiting for the host, so it measures the same")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="first run three 256 MiB fp32 copies (cast_kernel<float,float>): the known-size kernel that "
                          "FETCH_SIZE / WRITE_SIZE counters of a --pmc run are scaled by")
@@ -216,6 +220,14 @@ def main():
     from bamboo_amd import hip
     cfg = CONFIGS[args.config]
     samples = cfg["mb"] * cfg["M"]
+    graphs = bool(args.graphs)
+    if graphs:
+        # graphs are captured from a created stream (the default stream cannot be captured), in the
+        # second warm-up batch: the first one launches every kernel eagerly
+        args.warmup = max(args.warmup, 2)
+        work_stream = torch.cuda.Stream()
+        work_stream.wait_stream(torch.cuda.current_stream())
+        torch.cuda.set_stream(work_stream)
     if args.calibrate_copy:
         src = torch.ones(64 * 1024 * 1024, dtype=torch.float32, device="cuda:0")
         dst = torch.empty_like(src)
@@ -227,7 +239,7 @@ def main():
     # leg 1: RC off (plain 1F1B stream of the stage)
     t_off = None
     if not args.skip_rc_off:
-        engine, q = build_engine(cfg, rc=False, rc_stream=False)
+        engine, q = build_engine(cfg, rc=False, rc_stream=False, use_graphs=graphs)
         t_off = time_steps(engine, args.steps, args.warmup)
         del engine, q
         torch.cuda.empty_cache()
@@ -255,7 +267,7 @@ def main():
     if args.rc_stream:
         del engine, q
         torch.cuda.empty_cache()
-        engine, q = build_engine(cfg, rc=True, rc_stream=True)
+        engine, q = build_engine(cfg, rc=True, rc_stream=True, use_graphs=graphs)
         t_on = time_steps(engine, args.steps, args.warmup)
 
     failover = None
@@ -278,6 +290,7 @@ def main():
                     "note": "pause = failure detected (GPU drained) -> successor's lost work replayed from the RC stash; "
                             "post-failover = own + promoted layers as two local stages"}
 
+    n_graphs = sum(1 for v in engine._graphs.values() if isinstance(v, tuple))
     layer = engine.module.func_buckets[STAGE_ID][0]
     fwd_flops = layer.flops_fwd(cfg["mb"], cfg["seq"]) * cfg["layers"]
     own_flops, rc_flops = 3 * fwd_flops * cfg["M"], fwd_flops * cfg["M"]
@@ -310,7 +323,8 @@ def main():
         "warmup": args.warmup, "ms_per_step": round(t_on * 1e3, 3), "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": cfg["dtype"], "data": "synthetic",
         "config": {"workload": cfg["label"], "stage": f"{STAGE_ID} of {STAGES}", "redundancy_level": 1,
-                   "eager_recovery": True, "rc_stream": bool(args.rc_stream), "samples_per_step": samples,
+                   "eager_recovery": True, "rc_stream": bool(args.rc_stream), "hip_graphs": n_graphs if graphs else 0,
+                   "samples_per_step": samples,
                    "attention": "n/a (convolutions as GEMMs over NHWC rows, 3x3 via patch matrix)" if cfg.get("kind") == "resnet"
                    else "fused (no score matrix in HBM); flops counted dense, the causal kernel skips masked tiles"},
         "rc_on_samples_per_s": round(samples / t_on, 3),

@@ -224,6 +224,19 @@ int bb_adam_multi(int n_tensors, void* const* g, void* const* p, void* const* m,
 int bb_cast(int src_dtype, int dst_dtype, int64_t n, const void* src, void* dst, void* stream);
 int bb_fill_f32(float* dst, int64_t n, float value, void* stream);
 
+/* Replay of a fixed launch sequence as a HIP graph.  The reference replays nothing: its engine
+ * issues every ATen kernel of a micro-batch from Python on each step (engine.py:1626-1727); on
+ * static buffers the same sequence is captured once and launched as one graph.
+ *   bb_graph_begin   starts capturing `stream` (not the default stream; thread-local mode).  Calls
+ *                    of this library on that stream are recorded, not run, until bb_graph_end.
+ *   bb_graph_end     ends the capture and returns an executable graph in *exec_out.
+ *   bb_graph_launch  runs it on a stream.   bb_graph_destroy  releases it.
+ * Every kernel of the sequence must have been launched once before it is captured.            */
+int bb_graph_begin(void* stream);
+int bb_graph_end(void* stream, void** exec_out);
+int bb_graph_launch(void* exec, void* stream);
+int bb_graph_destroy(void* exec);
+
 #ifdef __cplusplus
 }
 #endif

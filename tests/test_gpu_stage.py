@@ -34,7 +34,7 @@ def grad_floor(ref_grads):
 
 
 def build(hidden, heads, ffn, layers_per_stage, stages, stage_id, mb, M, seq, dtype, variant, rl, eager,
-          grad_mode="queue", rc_stream=False, key_len_range=None):
+          grad_mode="queue", rc_stream=False, key_len_range=None, **engine_kwargs):
     specs = [LayerSpec(TransformerLayer, hidden, heads, ffn, **variant) for _ in range(layers_per_stage * stages)]
     model = PipelineModule(specs, num_stages=stages, partition_method="uniform", stage_id=stage_id, dtype=dtype, device=DEV)
     q = SeededActivationQueue((mb, seq, hidden), dtype, M, stage_ids=[stage_id, (stage_id + 1) % stages], seed=7,
@@ -42,7 +42,8 @@ def build(hidden, heads, ffn, layers_per_stage, stages, stage_id, mb, M, seq, dt
     cfg = {"train_micro_batch_size_per_gpu": mb, "gradient_accumulation_steps": M,
            "optimizer": {"type": "Adam", "params": {"lr": 1e-3}}, "bf16": {"enabled": dtype == torch.bfloat16}}
     engine, _, _, _ = bamboo_amd.initialize(model=model, config=cfg, redundancy_level=rl, eager_recovery=eager,
-                                            activation_queue=q, rc_stream=rc_stream, install_signal_handler=False)
+                                            activation_queue=q, rc_stream=rc_stream, install_signal_handler=False,
+                                            **engine_kwargs)
     return engine, q
 
 
@@ -311,6 +312,42 @@ def test_lazy_recovery_failover(hiplib, dead_from):
         for name, g in engine.module.get_named_grad(s_):
             assert rel_err(g, ref[name], grad_floor(ref)) < 1e-4, (s_, name)
     assert abs(float(loss) - float(peer.loss) / M) < 1e-4 * max(1.0, float(peer.loss) / M)
+
+
+@pytest.mark.parametrize("rc_stream", [False, True], ids=["one-stream", "rc-stream"])
+@pytest.mark.parametrize("variant,klr", [(GPT_VARIANT, None), (BERT_VARIANT, (5, 64))], ids=["gpt", "bert"])
+def test_graph_replay_equals_eager(hiplib, variant, klr, rc_stream):
+    """Forward / backward launch sequences replayed as HIP graphs: five batches with optimizer steps
+    (eager work and synchronisation between the replays), loss after every batch and the weights at
+    the end bit-equal to an engine that launches every kernel itself.  Batch 1 runs eagerly, batch 2
+    captures, batches 3-5 replay."""
+    hid, heads, ffn, L, S, sid, mb, M, seq = 128, 2, 256, 2, 4, 1, 2, 4, 64
+    dtype = torch.bfloat16
+    eager_engine, _ = build(hid, heads, ffn, L, S, sid, mb, M, seq, dtype, variant, 1, True, grad_mode="mse",
+                            rc_stream=rc_stream, key_len_range=klr)
+    ref_losses = []
+    for _ in range(5):
+        ref_losses.append(float(eager_engine.train_batch()))
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream()
+    with torch.cuda.stream(side):
+        with pytest.raises(bamboo_amd.PipelineError):
+            pass_default = torch.cuda.default_stream()
+            with torch.cuda.stream(pass_default):
+                build(hid, heads, ffn, L, S, sid, mb, M, seq, dtype, variant, 1, True, grad_mode="mse", use_graphs=True)
+        engine, _ = build(hid, heads, ffn, L, S, sid, mb, M, seq, dtype, variant, 1, True, grad_mode="mse",
+                          rc_stream=rc_stream, key_len_range=klr, use_graphs=True)
+        torch.cuda.synchronize()
+        losses = []
+        for _ in range(5):
+            losses.append(float(engine.train_batch()))
+            torch.cuda.synchronize()
+    assert losses == ref_losses
+    assert len(engine._graphs) == 3 * M and all(isinstance(v, tuple) for v in engine._graphs.values())
+    for s_ in (sid, sid + 1):
+        a, b = engine.module.stage_params[s_], eager_engine.module.stage_params[s_]
+        assert torch.equal(a.master, b.master) and torch.equal(a.compute, b.compute)
+    assert losses[4] != losses[0]
 
 
 def test_optimizer_step_matches_oracle(hiplib):
