@@ -761,9 +761,8 @@ __global__ __launch_bounds__(256) void bn_colred_kernel(int rows, int cols, cons
 #pragma unroll
             for (int e = 0; e < VEC; ++e) rs[e] = rstd[c0 + e];
         }
-        for (int r = blockIdx.y * 4 + wave; r < rows; r += gridDim.y * 4) {
-            float v[VEC];
-            load_vec(x + (int64_t)r * cols + c0, v);
+        // rows r0, r0 + step, ... in that order; four rows' loads are issued before their sums
+        auto add_row = [&](const float (&v)[VEC], const float (&g)[VEC]) {
             if (MODE == 0) {
 #pragma unroll
                 for (int e = 0; e < VEC; ++e) a0[e] += v[e];
@@ -774,7 +773,16 @@ __global__ __launch_bounds__(256) void bn_colred_kernel(int rows, int cols, cons
                     a0[e] += d * d;
                 }
             } else {
-                float g[VEC];
+#pragma unroll
+                for (int e = 0; e < VEC; ++e) {
+                    a0[e] += g[e];
+                    a1[e] += g[e] * (v[e] - mu[e]) * rs[e];
+                }
+            }
+        };
+        auto load_row = [&](int r, float (&v)[VEC], float (&g)[VEC]) {
+            load_vec(x + (int64_t)r * cols + c0, v);
+            if (MODE == 2) {
                 load_vec(dy + (int64_t)r * cols + c0, g);
                 if (relu_out) {
                     float o[VEC];
@@ -782,12 +790,21 @@ __global__ __launch_bounds__(256) void bn_colred_kernel(int rows, int cols, cons
 #pragma unroll
                     for (int e = 0; e < VEC; ++e) g[e] = o[e] > 0.f ? g[e] : 0.f;
                 }
-#pragma unroll
-                for (int e = 0; e < VEC; ++e) {
-                    a0[e] += g[e];
-                    a1[e] += g[e] * (v[e] - mu[e]) * rs[e];
-                }
             }
+        };
+        const int step = gridDim.y * 4;
+        int r = blockIdx.y * 4 + wave;
+        for (; r + 3 * step < rows; r += 4 * step) {
+            float v[4][VEC], g[4][VEC];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) load_row(r + j * step, v[j], g[j]);
+#pragma unroll
+            for (int j = 0; j < 4; ++j) add_row(v[j], g[j]);
+        }
+        for (; r < rows; r += step) {
+            float v[VEC], g[VEC];
+            load_row(r, v, g);
+            add_row(v, g);
         }
     }
     if (wave > 0) {
@@ -815,17 +832,26 @@ __global__ __launch_bounds__(256) void bn_colred_kernel(int rows, int cols, cons
 // finish: sums over the BN_SPLITS partial rows in fixed order.
 // what 0: mean = s0/rows ; 1: rstd = 1/sqrt(s0/rows + eps) (+ running stats) ; 2: dbeta += s0, dgamma += s1,
 // and keep the batch means of g and g*xhat for the apply pass
-__global__ __launch_bounds__(256) void bn_finish_kernel(int what, int rows, int cols, float eps, float momentum,
+__global__ __launch_bounds__(64) void bn_finish_kernel(int what, int rows, int cols, float eps, float momentum,
                                                         const float* __restrict__ partial, float* __restrict__ mean,
                                                         float* __restrict__ rstd, float* __restrict__ run_mean,
                                                         float* __restrict__ run_var, float* __restrict__ dgamma,
                                                         float* __restrict__ dbeta, float* __restrict__ sums) {
-    const int c = blockIdx.x * 256 + threadIdx.x;
+    const int c = blockIdx.x * 64 + threadIdx.x;
     if (c >= cols) return;
     float s0 = 0.f, s1 = 0.f;
-    for (int p = 0; p < BN_SPLITS; ++p) {
-        s0 += partial[((int64_t)p * 2) * cols + c];
-        s1 += partial[((int64_t)p * 2 + 1) * cols + c];
+    for (int p0 = 0; p0 < BN_SPLITS; p0 += 8) {  // eight rows' loads in flight, summed in row order
+        float t0[8], t1[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            t0[j] = partial[((int64_t)(p0 + j) * 2) * cols + c];
+            t1[j] = what == 2 ? partial[((int64_t)(p0 + j) * 2 + 1) * cols + c] : 0.f;
+        }
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            s0 += t0[j];
+            s1 += t1[j];
+        }
     }
     if (what == 0) {
         mean[c] = s0 / (float)rows;
@@ -851,14 +877,29 @@ __global__ __launch_bounds__(256) void bn_apply_kernel(int64_t nvec, int cols, i
                                                        const T* __restrict__ gamma, const T* __restrict__ beta,
                                                        const T* __restrict__ resid, T* __restrict__ y) {
     constexpr int VEC = Elem<T>::VEC;
-    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < nvec; i += (int64_t)gridDim.x * 256) {
-        const int c0 = (int)((i * VEC) % cols);
-        float v[VEC], g[VEC], b[VEC];
-        load_vec(x + i * VEC, v);
+    // with a grid stride that is a multiple of the row length a thread stays on its channels:
+    // scale and shift are then folded once (y = x * sc + sh), outside the loop
+    const int64_t stride = (int64_t)gridDim.x * 256;
+    const bool fixed = stride % (cols / VEC) == 0;
+    float sc[VEC], sh[VEC];
+    auto fold = [&](int c0) {
+        float g[VEC], b[VEC];
         load_vec(gamma + c0, g);
         load_vec(beta + c0, b);
 #pragma unroll
-        for (int e = 0; e < VEC; ++e) v[e] = g[e] * ((v[e] - mean[c0 + e]) * rstd[c0 + e]) + b[e];
+        for (int e = 0; e < VEC; ++e) {
+            sc[e] = g[e] * rstd[c0 + e];
+            sh[e] = b[e] - mean[c0 + e] * sc[e];
+        }
+    };
+    const int64_t first = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (fixed && first < nvec) fold((int)((first * VEC) % cols));
+    for (int64_t i = first; i < nvec; i += stride) {
+        if (!fixed) fold((int)((i * VEC) % cols));
+        float v[VEC];
+        load_vec(x + i * VEC, v);
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) v[e] = fmaf(v[e], sc[e], sh[e]);
         if (resid) {
             float r[VEC];
             load_vec(resid + i * VEC, r);
@@ -882,12 +923,29 @@ __global__ __launch_bounds__(256) void bn_bwd_apply_kernel(int64_t nvec, int col
                                                            const T* __restrict__ dy, const T* __restrict__ relu_out,
                                                            T* __restrict__ dx, T* __restrict__ g_out) {
     constexpr int VEC = Elem<T>::VEC;
-    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < nvec; i += (int64_t)gridDim.x * 256) {
-        const int c0 = (int)((i * VEC) % cols);
-        float v[VEC], g[VEC], gm[VEC], o[VEC];
+    // dx = k (g - mean(g) - xhat mean(g xhat)), k = gamma rstd, folded per channel into
+    // dx = k g + a x + b; a thread keeps its channels when the grid stride is a multiple of a row
+    const int64_t stride = (int64_t)gridDim.x * 256;
+    const bool fixed = stride % (cols / VEC) == 0;
+    float k[VEC], ka[VEC], kb[VEC];
+    auto fold = [&](int c0) {
+        float gm[VEC];
+        load_vec(gamma + c0, gm);
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) {
+            const float rs = rstd[c0 + e];
+            k[e] = gm[e] * rs;
+            ka[e] = -k[e] * sums[cols + c0 + e] * rs;
+            kb[e] = -k[e] * sums[c0 + e] - ka[e] * mean[c0 + e];
+        }
+    };
+    const int64_t first = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (fixed && first < nvec) fold((int)((first * VEC) % cols));
+    for (int64_t i = first; i < nvec; i += stride) {
+        if (!fixed) fold((int)((i * VEC) % cols));
+        float v[VEC], g[VEC], o[VEC];
         load_vec(x + i * VEC, v);
         load_vec(dy + i * VEC, g);
-        load_vec(gamma + c0, gm);
         if (relu_out) {
             float ro[VEC];
             load_vec(relu_out + i * VEC, ro);
@@ -895,10 +953,7 @@ __global__ __launch_bounds__(256) void bn_bwd_apply_kernel(int64_t nvec, int col
             for (int e = 0; e < VEC; ++e) g[e] = ro[e] > 0.f ? g[e] : 0.f;
         }
 #pragma unroll
-        for (int e = 0; e < VEC; ++e) {
-            const float xh = (v[e] - mean[c0 + e]) * rstd[c0 + e];
-            o[e] = gm[e] * rstd[c0 + e] * (g[e] - sums[c0 + e] - xh * sums[cols + c0 + e]);
-        }
+        for (int e = 0; e < VEC; ++e) o[e] = fmaf(k[e], g[e], fmaf(ka[e], v[e], kb[e]));
         store_vec(dx + i * VEC, o);
         if (g_out) store_vec(g_out + i * VEC, g);
     }
@@ -922,19 +977,19 @@ extern "C" int bb_batchnorm_fwd(int dtype, int rows, int cols, float eps, float 
     BB_REQUIRE((running_mean == nullptr) == (running_var == nullptr), "bb_batchnorm_fwd: give both running buffers or none");
     hipStream_t st = (hipStream_t)stream;
     const int vec = dtype == BB_BF16 ? 8 : 4;
-    dim3 grid((cols + 64 * vec - 1) / (64 * vec), BN_SPLITS), fgrid((cols + 255) / 256);
+    dim3 grid((cols + 64 * vec - 1) / (64 * vec), BN_SPLITS), fgrid((cols + 63) / 64);
     const int64_t nvec = (int64_t)rows * cols / vec;
     if (dtype == BB_BF16) {
         hipLaunchKernelGGL((bn_colred_kernel<bf16, 0>), grid, dim3(256), 0, st, rows, cols, (const bf16*)x, nullptr, nullptr, nullptr, nullptr, workspace);
-        hipLaunchKernelGGL(bn_finish_kernel, fgrid, dim3(256), 0, st, 0, rows, cols, eps, momentum, workspace, mean, rstd, nullptr, nullptr, nullptr, nullptr, nullptr);
+        hipLaunchKernelGGL(bn_finish_kernel, fgrid, dim3(64), 0, st, 0, rows, cols, eps, momentum, workspace, mean, rstd, nullptr, nullptr, nullptr, nullptr, nullptr);
         hipLaunchKernelGGL((bn_colred_kernel<bf16, 1>), grid, dim3(256), 0, st, rows, cols, (const bf16*)x, mean, nullptr, nullptr, nullptr, workspace);
-        hipLaunchKernelGGL(bn_finish_kernel, fgrid, dim3(256), 0, st, 1, rows, cols, eps, momentum, workspace, mean, rstd, running_mean, running_var, nullptr, nullptr, nullptr);
+        hipLaunchKernelGGL(bn_finish_kernel, fgrid, dim3(64), 0, st, 1, rows, cols, eps, momentum, workspace, mean, rstd, running_mean, running_var, nullptr, nullptr, nullptr);
         hipLaunchKernelGGL(bn_apply_kernel<bf16>, dim3(grid_for(nvec)), dim3(256), 0, st, nvec, cols, relu, (const bf16*)x, mean, rstd, (const bf16*)gamma, (const bf16*)beta, (const bf16*)resid, (bf16*)y);
     } else {
         hipLaunchKernelGGL((bn_colred_kernel<float, 0>), grid, dim3(256), 0, st, rows, cols, (const float*)x, nullptr, nullptr, nullptr, nullptr, workspace);
-        hipLaunchKernelGGL(bn_finish_kernel, fgrid, dim3(256), 0, st, 0, rows, cols, eps, momentum, workspace, mean, rstd, nullptr, nullptr, nullptr, nullptr, nullptr);
+        hipLaunchKernelGGL(bn_finish_kernel, fgrid, dim3(64), 0, st, 0, rows, cols, eps, momentum, workspace, mean, rstd, nullptr, nullptr, nullptr, nullptr, nullptr);
         hipLaunchKernelGGL((bn_colred_kernel<float, 1>), grid, dim3(256), 0, st, rows, cols, (const float*)x, mean, nullptr, nullptr, nullptr, workspace);
-        hipLaunchKernelGGL(bn_finish_kernel, fgrid, dim3(256), 0, st, 1, rows, cols, eps, momentum, workspace, mean, rstd, running_mean, running_var, nullptr, nullptr, nullptr);
+        hipLaunchKernelGGL(bn_finish_kernel, fgrid, dim3(64), 0, st, 1, rows, cols, eps, momentum, workspace, mean, rstd, running_mean, running_var, nullptr, nullptr, nullptr);
         hipLaunchKernelGGL(bn_apply_kernel<float>, dim3(grid_for(nvec)), dim3(256), 0, st, nvec, cols, relu, (const float*)x, mean, rstd, (const float*)gamma, (const float*)beta, (const float*)resid, (float*)y);
     }
     BB_LAUNCH_CHECK();
@@ -949,16 +1004,16 @@ extern "C" int bb_batchnorm_bwd(int dtype, int rows, int cols, const void* x, co
     BB_REQUIRE(x && gamma && mean && rstd && dy && dx && dgamma && dbeta && workspace, "bb_batchnorm_bwd: null pointer");
     hipStream_t st = (hipStream_t)stream;
     const int vec = dtype == BB_BF16 ? 8 : 4;
-    dim3 grid((cols + 64 * vec - 1) / (64 * vec), BN_SPLITS), fgrid((cols + 255) / 256);
+    dim3 grid((cols + 64 * vec - 1) / (64 * vec), BN_SPLITS), fgrid((cols + 63) / 64);
     const int64_t nvec = (int64_t)rows * cols / vec;
     float* sums = workspace + (int64_t)BN_SPLITS * 2 * cols;
     if (dtype == BB_BF16) {
         hipLaunchKernelGGL((bn_colred_kernel<bf16, 2>), grid, dim3(256), 0, st, rows, cols, (const bf16*)x, mean, rstd, (const bf16*)dy, (const bf16*)relu_out, workspace);
-        hipLaunchKernelGGL(bn_finish_kernel, fgrid, dim3(256), 0, st, 2, rows, cols, 0.f, 0.f, workspace, nullptr, nullptr, nullptr, nullptr, dgamma, dbeta, sums);
+        hipLaunchKernelGGL(bn_finish_kernel, fgrid, dim3(64), 0, st, 2, rows, cols, 0.f, 0.f, workspace, nullptr, nullptr, nullptr, nullptr, dgamma, dbeta, sums);
         hipLaunchKernelGGL(bn_bwd_apply_kernel<bf16>, dim3(grid_for(nvec)), dim3(256), 0, st, nvec, cols, (const bf16*)x, mean, rstd, (const bf16*)gamma, sums, (const bf16*)dy, (const bf16*)relu_out, (bf16*)dx, (bf16*)g_out);
     } else {
         hipLaunchKernelGGL((bn_colred_kernel<float, 2>), grid, dim3(256), 0, st, rows, cols, (const float*)x, mean, rstd, (const float*)dy, (const float*)relu_out, workspace);
-        hipLaunchKernelGGL(bn_finish_kernel, fgrid, dim3(256), 0, st, 2, rows, cols, 0.f, 0.f, workspace, nullptr, nullptr, nullptr, nullptr, dgamma, dbeta, sums);
+        hipLaunchKernelGGL(bn_finish_kernel, fgrid, dim3(64), 0, st, 2, rows, cols, 0.f, 0.f, workspace, nullptr, nullptr, nullptr, nullptr, dgamma, dbeta, sums);
         hipLaunchKernelGGL(bn_bwd_apply_kernel<float>, dim3(grid_for(nvec)), dim3(256), 0, st, nvec, cols, (const float*)x, mean, rstd, (const float*)gamma, sums, (const float*)dy, (const float*)relu_out, (float*)dx, (float*)g_out);
     }
     BB_LAUNCH_CHECK();

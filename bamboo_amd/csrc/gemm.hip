@@ -603,7 +603,7 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_bf16_dma_kernel(const GemmAr
 
 // Several independent problems of one kind in a single launch (the four weight-gradient GEMMs
 // of a transformer layer: each alone has too few output tiles to fill 256 CUs).
-constexpr int GROUP_MAX = 8;
+constexpr int GROUP_MAX = 16;
 struct GroupedArgs {
     GemmArgs p[GROUP_MAX];
     int first_block[GROUP_MAX + 1];
@@ -979,4 +979,108 @@ extern "C" int bb_gemm_grouped(const bb_gemm_desc* descs, int count, void* strea
     if (layout == BB_NT) return launch_grouped<false, false>(G, st);
     if (layout == BB_NN) return launch_grouped<false, true>(G, st);
     return launch_grouped<true, true>(G, st);
+}
+
+// =========================================================================================
+// Grouped GEMMs with few output tiles and a long contraction (the weight gradients of a ResNet
+// bottleneck: 68 tiles of 128x128 over K = 6272 rows): the contraction is cut into `splits`
+// chunks, each chunk of each problem becomes a problem of its own that writes an fp32 partial
+// product into the caller's workspace, and a second kernel adds the partials to C in chunk order.
+// =========================================================================================
+constexpr int SPLITK_MAX = 8;
+
+__global__ __launch_bounds__(256) void splitk_reduce_kernel(const float* __restrict__ ws, int splits, int64_t part, int M,
+                                                            int N, float* __restrict__ C, int64_t ldc, int accumulate) {
+    const int64_t nvec = (int64_t)M * N / 4;
+    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < nvec; i += (int64_t)gridDim.x * 256) {
+        const int64_t e = i * 4;
+        const int m = (int)(e / N), n = (int)(e % N);
+        float* c = C + (int64_t)m * ldc + n;
+        f32x4 acc = accumulate ? *(const f32x4*)c : f32x4{0.f, 0.f, 0.f, 0.f};
+        f32x4 v[SPLITK_MAX];
+#pragma unroll
+        for (int p = 0; p < SPLITK_MAX; ++p)
+            if (p < splits) v[p] = *(const f32x4*)(ws + p * part + e);
+#pragma unroll
+        for (int p = 0; p < SPLITK_MAX; ++p)
+            if (p < splits) acc += v[p];
+        *(f32x4*)c = acc;
+    }
+}
+
+// chunks of the contraction: 0 or 1 = run the group whole
+static int pick_splits(const bb_gemm_desc* descs, int count) {
+    if (count < 1 || count > GROUP_MAX || dma_tile_override() != 0) return 0;
+    int64_t tiles = 0;
+    int kmin = 1 << 30;
+    for (int i = 0; i < count; ++i) {
+        const bb_gemm_desc& d = descs[i];
+        if (d.dtype != BB_BF16 || d.c_dtype != BB_F32 || d.layout != descs[0].layout || d.nb1 > 1 || d.nb2 > 1 || d.M <= 0 ||
+            d.N <= 0 || d.colsum_out || d.bias || d.epilogue != BB_EPI_NONE || d.alpha != 1.0f || d.N % 4 != 0 ||
+            pick_dma_tile(d.M, d.N, d.K, 1) == D_NONE)
+            return 0;
+        tiles += (int64_t)((d.M + 127) / 128) * ((d.N + 127) / 128);
+        kmin = d.K < kmin ? d.K : kmin;
+    }
+    int splits = (int)(256 / tiles);                 // fill the 256 CUs once
+    if (splits > SPLITK_MAX) splits = SPLITK_MAX;
+    if (splits > GROUP_MAX / count) splits = GROUP_MAX / count;
+    while (splits > 1 && kmin / splits < 512) --splits;  // keep the pipelines of the chunks long
+    return splits;
+}
+
+extern "C" int64_t bb_gemm_splitk_workspace(const bb_gemm_desc* descs, int count) {
+    int64_t n = 0;
+    for (int i = 0; descs && i < count; ++i) n += (int64_t)descs[i].M * descs[i].N;
+    return n * SPLITK_MAX * (int64_t)sizeof(float);
+}
+
+extern "C" int bb_gemm_grouped_splitk(const bb_gemm_desc* descs, int count, void* workspace, int64_t workspace_bytes,
+                                      void* stream) {
+    BB_REQUIRE(count >= 0 && (descs || count == 0), "bb_gemm_grouped_splitk: bad arguments");
+    const int splits = pick_splits(descs, count);
+    if (splits <= 1) return bb_gemm_grouped(descs, count, stream);
+    int64_t need = 0;
+    for (int i = 0; i < count; ++i) need += (int64_t)descs[i].M * descs[i].N * splits * (int64_t)sizeof(float);
+    BB_REQUIRE(workspace && workspace_bytes >= need && ((uintptr_t)workspace % 16) == 0,
+               "bb_gemm_grouped_splitk: workspace of %lld bytes needed (16-byte aligned), got %lld", (long long)need,
+               (long long)workspace_bytes);
+    bb_gemm_desc sub[GROUP_MAX];
+    float* ws = (float*)workspace;
+    int ns = 0;
+    for (int i = 0; i < count; ++i) {
+        const bb_gemm_desc& d = descs[i];
+        // chunk boundaries on multiples of 32 rows of the contraction
+        const int kt = d.K / 32, per = kt / splits, extra = kt % splits;
+        int k0 = 0;
+        for (int p = 0; p < splits; ++p) {
+            int kc = (per + (p < extra ? 1 : 0)) * 32;
+            if (p == splits - 1) kc = d.K - k0;
+            bb_gemm_desc& t = sub[ns++];
+            t = d;
+            t.K = kc;
+            // A advances along its contraction index: rows for TN ([K, M]), columns otherwise ([M, K])
+            t.A = (const char*)d.A + (d.layout == BB_TN ? (int64_t)k0 * d.lda : (int64_t)k0) * 2;
+            // B: [N, K] for NT, [K, N] for NN and TN
+            t.B = (const char*)d.B + (d.layout == BB_NT ? (int64_t)k0 : (int64_t)k0 * d.ldb) * 2;
+            t.C = ws + (int64_t)p * d.M * d.N;
+            t.ldc = d.N;
+            t.accumulate = 0;
+            k0 += kc;
+        }
+        ws += (int64_t)splits * d.M * d.N;
+    }
+    int rc = bb_gemm_grouped(sub, ns, stream);
+    if (rc) return rc;
+    ws = (float*)workspace;
+    for (int i = 0; i < count; ++i) {
+        const bb_gemm_desc& d = descs[i];
+        const int64_t part = (int64_t)d.M * d.N;
+        const int64_t nvec = part / 4;
+        hipLaunchKernelGGL(splitk_reduce_kernel, dim3((unsigned)((nvec + 255) / 256 > 1024 ? 1024 : (nvec + 255) / 256)),
+                           dim3(256), 0, (hipStream_t)stream, ws, splits, part, d.M, d.N, (float*)d.C, d.ldc, d.accumulate);
+        ws += (int64_t)splits * part;
+    }
+    BB_LAUNCH_CHECK();
+    return BB_OK;
 }

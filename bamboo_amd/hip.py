@@ -23,7 +23,7 @@ MASK_CODES = {"none": MASK_NONE, "causal": MASK_CAUSAL, "key_padding": MASK_KEY_
 LN_CODES = {"standard": LN_STANDARD, "annotated": LN_ANNOTATED}
 
 EXPORTS = (
-    "bb_version", "bb_last_error", "bb_init", "bb_gemm", "bb_gemm_grouped", "bb_gemm_variant", "bb_layernorm_fwd",
+    "bb_version", "bb_last_error", "bb_init", "bb_gemm", "bb_gemm_grouped", "bb_gemm_splitk_workspace", "bb_gemm_grouped_splitk", "bb_gemm_variant", "bb_layernorm_fwd",
     "bb_layernorm_bwd_workspace", "bb_layernorm_bwd", "bb_colsum_workspace", "bb_colsum_acc",
     "bb_softmax_fwd", "bb_softmax_bwd", "bb_attention_fwd", "bb_attention_bwd", "bb_residual_add", "bb_act_fwd", "bb_bn_workspace", "bb_batchnorm_fwd", "bb_batchnorm_bwd", "bb_patch3x3", "bb_mse_workspace", "bb_mse_fwd_bwd", "bb_graph_begin", "bb_graph_end", "bb_graph_launch", "bb_graph_destroy",
     "bb_adam_multi", "bb_cast", "bb_fill_f32",
@@ -73,6 +73,9 @@ def lib():
     L.bb_init.restype = c_int
     L.bb_gemm.argtypes = [POINTER(GemmDesc), c_void_p]
     L.bb_gemm_grouped.argtypes = [POINTER(GemmDesc), c_int, c_void_p]
+    L.bb_gemm_splitk_workspace.argtypes = [POINTER(GemmDesc), c_int]
+    L.bb_gemm_splitk_workspace.restype = c_int64
+    L.bb_gemm_grouped_splitk.argtypes = [POINTER(GemmDesc), c_int, c_void_p, c_int64, c_void_p]
     L.bb_gemm_variant.argtypes = [POINTER(GemmDesc), c_char_p, c_int]
     L.bb_layernorm_fwd.argtypes = [c_int, c_int, c_int, c_int, c_float, c_void_p, c_void_p, c_void_p,
                                    c_void_p, c_void_p, c_void_p, c_void_p]
@@ -204,11 +207,23 @@ def gemm(layout, A, B, C, *, stream=None, **kw):
     return C
 
 
-def gemm_grouped(descs, stream=None):
-    """Independent GEMMs of one layout in one launch (falls back to one launch each inside the
-    library when they cannot share a kernel)."""
+def gemm_splitk_workspace(descs):
     arr = (GemmDesc * len(descs))(*descs)
-    call = lambda: check(lib().bb_gemm_grouped(arr, len(descs), stream_ptr(stream)), "bb_gemm_grouped")
+    return int(lib().bb_gemm_splitk_workspace(arr, len(descs)))
+
+
+def gemm_grouped(descs, stream=None, splitk_ws=None):
+    """Independent GEMMs of one layout in one launch (falls back to one launch each inside the
+    library when they cannot share a kernel).  With ``splitk_ws`` (a tensor of at least
+    ``gemm_splitk_workspace(descs)`` bytes) problems with few output tiles and a long contraction
+    are cut along the contraction and reduced in fixed order."""
+    arr = (GemmDesc * len(descs))(*descs)
+    if splitk_ws is not None:
+        nbytes = splitk_ws.numel() * splitk_ws.element_size()
+        call = lambda: check(lib().bb_gemm_grouped_splitk(arr, len(descs), _ptr(splitk_ws), nbytes, stream_ptr(stream)),
+                             "bb_gemm_grouped_splitk")
+    else:
+        call = lambda: check(lib().bb_gemm_grouped(arr, len(descs), stream_ptr(stream)), "bb_gemm_grouped")
     if gemm_hook is not None:
         gemm_hook(descs, call, stream)
     else:

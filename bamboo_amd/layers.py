@@ -358,8 +358,10 @@ class BottleNeck:
     def scratch_specs(self, ctx):
         R, ci, cm = ctx.rows, self.cin, self.cmid
         dt = ctx.dtype
+        # split-K partial products of the three weight gradients (8 chunks of each, fp32)
+        nws = 8 * (ci * cm + 9 * cm * cm + cm * ci)
         return [("col", (R, 9 * cm), dt), ("d_col", (R, 9 * cm), dt), ("d_y3", (R, ci), dt), ("d_res", (R, ci), dt),
-                ("d_m0", (R, cm), dt), ("d_m1", (R, cm), dt)]
+                ("d_m0", (R, cm), dt), ("d_m1", (R, cm), dt), ("d_m2", (R, cm), dt), ("splitk", (nws,), torch.float32)]
 
     def forward_scratch_specs(self, ctx):
         return [("col", (ctx.rows, 9 * self.cmid), ctx.dtype)]
@@ -412,13 +414,15 @@ class BottleNeck:
         bn(4, "y2", "mean2", "rstd2", d_m0, st["a2"], d_m1, None)                          # d_y2
         hip.patch3x3(st["a1"], col, ctx.batch, self.h, self.w, cm, stream=sm)              # patches again: cheaper than stashing
         hip.gemm(hip.NN, d_m1, w["conv2"], d_col, stream=sm)
-        d_a1 = ctx.buf("d_m0", (R, cm))
-        hip.gemm_grouped([hip.gemm_desc(hip.TN, d_y3, st["a2"], g["residual_function.6.weight"], accumulate=True),
-                          hip.gemm_desc(hip.TN, d_m1, col, g["conv2"], accumulate=True)], stream=sm)
+        d_a1, d_m2 = ctx.buf("d_m0", (R, cm)), ctx.buf("d_m2", (R, cm))
         hip.patch3x3(d_col, d_a1, ctx.batch, self.h, self.w, cm, adjoint=True, stream=sm)
-        bn(1, "y1", "mean1", "rstd1", d_a1, st["a1"], d_m1, None)                          # d_y1
-        hip.gemm(hip.TN, d_m1, st["x0"], g["residual_function.0.weight"], accumulate=True, stream=sm)
-        hip.gemm(hip.NN, d_m1, w["residual_function.0.weight"], d_x, epilogue=hip.EPI_RESIDUAL, resid=d_res, stream=sm)
+        bn(1, "y1", "mean1", "rstd1", d_a1, st["a1"], d_m2, None)                          # d_y1
+        hip.gemm(hip.NN, d_m2, w["residual_function.0.weight"], d_x, epilogue=hip.EPI_RESIDUAL, resid=d_res, stream=sm)
+        # the three weight gradients in one launch: 68 output tiles over 6272 rows, cut along the rows
+        hip.gemm_grouped([hip.gemm_desc(hip.TN, d_y3, st["a2"], g["residual_function.6.weight"], accumulate=True),
+                          hip.gemm_desc(hip.TN, d_m1, col, g["conv2"], accumulate=True),
+                          hip.gemm_desc(hip.TN, d_m2, st["x0"], g["residual_function.0.weight"], accumulate=True)],
+                         stream=sm, splitk_ws=ctx.buf("splitk", (8 * (ci * cm + 9 * cm * cm + cm * ci),)))
         return d_x
 
 

@@ -116,6 +116,15 @@ int bb_gemm(const bb_gemm_desc* desc, void* stream);
  * is how the four weight-gradient products of a layer (autograd of transformer.py:136-146,158)
  * fill the GPU although each has few output tiles.                                         */
 int bb_gemm_grouped(const bb_gemm_desc* descs, int count, void* stream);
+/* bb_gemm_grouped for problems with an fp32 C, few output tiles and a long contraction (weight
+ * gradients dW += dy^T x of narrow layers, e.g. the three convolutions of resnet.py:49-75 over
+ * K = N*H*W rows): the contraction is cut into chunks that run as problems of their own into fp32
+ * partial products in `workspace` (>= bb_gemm_splitk_workspace(descs, count) bytes, 16-byte
+ * aligned), then added to C in chunk order -- deterministic, and equal to bb_gemm_grouped up to
+ * the fp32 summation order.  Falls back to bb_gemm_grouped when cutting does not pay.          */
+int64_t bb_gemm_splitk_workspace(const bb_gemm_desc* descs, int count);
+int bb_gemm_grouped_splitk(const bb_gemm_desc* descs, int count, void* workspace,
+                           int64_t workspace_bytes, void* stream);
 /* Name of the kernel variant bb_gemm would launch for this descriptor ("bf16_nt_256x256", ...),
  * written NUL-terminated into out; for correlating launches with profiler output.        */
 int bb_gemm_variant(const bb_gemm_desc* desc, char* out, int out_len);

@@ -90,6 +90,62 @@ def test_gemm_epilogues(hiplib, dtype):
     assert rel_err(C, 0.125 * (Af @ Wf.t())) < tol(dtype)
 
 
+@pytest.mark.parametrize("layout", ["tn", "nt"])
+def test_gemm_grouped_splitk(hiplib, layout):
+    """Few output tiles, long contraction: chunks of the contraction into fp32 partials, added to C
+    in chunk order.  Against fp64, against the unsplit grouped call, twice in a row (accumulate),
+    and with a C that is a strided view."""
+    torch.manual_seed(0)
+    dtype = torch.bfloat16
+    K = 6272
+    shapes = [(1024, 256), (256, 2304), (256, 1024)]
+    As, Bs, Cs, refs = [], [], [], []
+    for i, (M, N) in enumerate(shapes):
+        if layout == "tn":
+            A, B = randn(K, M, dtype=dtype, seed=50 + i, scale=0.1), randn(K, N, dtype=dtype, seed=60 + i, scale=0.1)
+            ref = A.double().cpu().t() @ B.double().cpu()
+        else:
+            A, B = randn(M, K, dtype=dtype, seed=50 + i, scale=0.1), randn(N, K, dtype=dtype, seed=60 + i, scale=0.1)
+            ref = A.double().cpu() @ B.double().cpu().t()
+        As.append(A); Bs.append(B); refs.append(ref)
+    C0 = [randn(M, N, dtype=torch.float32, seed=70 + i) for i, (M, N) in enumerate(shapes)]
+    lay = hiplib.TN if layout == "tn" else hiplib.NT
+    # last C is a view with a larger leading dimension
+    big = torch.zeros(shapes[2][0], shapes[2][1] + 64, device=DEV)
+    Cs = [C0[0].clone(), C0[1].clone(), big[:, :shapes[2][1]]]
+    Cs[2].copy_(C0[2])
+    descs = [hiplib.gemm_desc(lay, A, B, C, accumulate=True) for A, B, C in zip(As, Bs, Cs)]
+    ws = torch.empty(hiplib.gemm_splitk_workspace(descs) // 4, device=DEV)
+    hiplib.gemm_grouped(descs, splitk_ws=ws)
+    plain = [c.clone() for c in C0]
+    hiplib.gemm_grouped([hiplib.gemm_desc(lay, A, B, C, accumulate=True) for A, B, C in zip(As, Bs, plain)])
+    for C, c0, ref, pl in zip(Cs, C0, refs, plain):
+        assert rel_err(C, c0.double().cpu() + ref) < tol(dtype)
+        assert rel_err(C, pl) < 1e-5                     # same products, different fp32 summation order
+    assert float(big[:, shapes[2][1]:].abs().max()) == 0.0   # nothing written past the view
+    hiplib.gemm_grouped(descs, splitk_ws=ws)            # accumulates once more, reproducibly
+    again = [c.clone() for c in Cs]
+    for C, c0, ref in zip(Cs, C0, refs):
+        assert rel_err(C, c0.double().cpu() + 2 * ref) < tol(dtype)
+    Cs2 = [C0[0].clone(), C0[1].clone(), C0[2].clone()]
+    d2 = [hiplib.gemm_desc(lay, A, B, C, accumulate=True) for A, B, C in zip(As, Bs, Cs2)]
+    hiplib.gemm_grouped(d2, splitk_ws=ws); hiplib.gemm_grouped(d2, splitk_ws=ws)
+    for a, b in zip(again, Cs2):
+        assert torch.equal(a.contiguous(), b)
+    # too small a workspace is an error, not a silent fallback
+    with pytest.raises(hiplib.HipKernelError):
+        hiplib.gemm_grouped(descs, splitk_ws=ws[:1024])
+    # large groups are not cut: same call, same result as the plain grouped entry
+    M, N = 1024, 4096
+    A, B = randn(8192, M, dtype=dtype, seed=80, scale=0.1), randn(8192, N, dtype=dtype, seed=81, scale=0.1)
+    c1, c2 = torch.zeros(M, N, device=DEV), torch.zeros(M, N, device=DEV)
+    d_big = [hiplib.gemm_desc(hiplib.TN, A, B, c1, accumulate=True), hiplib.gemm_desc(hiplib.TN, A, B, c2, accumulate=True)]
+    hiplib.gemm_grouped(d_big, splitk_ws=ws)
+    ref_big = torch.zeros(M, N, device=DEV)
+    hiplib.gemm(hiplib.TN, A, B, ref_big, accumulate=True)
+    assert torch.equal(c1, ref_big) and torch.equal(c2, ref_big)
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 def test_gemm_batched_heads(hiplib, dtype):
     """Q K^T and P V over (batch, head) strides inside a [rows, 3h] buffer."""
