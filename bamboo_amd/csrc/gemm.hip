@@ -336,52 +336,34 @@ template <int BR, bool KM, int NW> struct DmaOperand {
     static constexpr int BYTES = BR * 32 * 2;
     static constexpr int ROUNDS = BYTES / (1024 * NW);  // instructions per thread per k-tile
     static_assert(ROUNDS >= 1, "tile too small for the block");
-    // Row-major operands (!KM) advance 64 bytes per k-tile: a lane keeps one pointer per instruction,
-    // the tiles of one turn of the ring are reached through the instruction's immediate offset and
-    // the pointers move once per turn.  K-major operands advance by 32 rows: the source is a base
-    // common to all lanes (scalar arithmetic per k-tile) plus the lane's fixed byte offset.
-    const char* ptr[KM ? 1 : ROUNDS];
-    const char* base;
-    uint32_t off[KM ? ROUNDS : 1];
-    int64_t step;  // bytes to advance per k-tile (set to 0 at the end of K)
+    const bf16* src[ROUNDS];
+    int64_t step;  // elements to advance per k-tile
 
-    __device__ __forceinline__ void init(const bf16* mat, int64_t ld, int row0, int rows, int lane, int wave) {
+    __device__ __forceinline__ void init(const bf16* base, int64_t ld, int row0, int rows, int tid) {
+        const int lane = tid & 63, wave = tid >> 6;
 #pragma unroll
         for (int i = 0; i < ROUNDS; ++i) {
             const int q = i * NW + wave;
             if constexpr (!KM) {
                 const int r = q * 16 + (lane >> 2);
                 const int c = (lane & 3) ^ ((r >> 2) & 3);
-                const int gr = min(row0 + r, rows - 1);  // rows past the end repeat the last one
-                ptr[i] = (const char*)(mat + (int64_t)gr * ld + c * 8);
+                const int gr = min(row0 + r, rows - 1);
+                src[i] = base + (int64_t)gr * ld + c * 8;
             } else {
                 constexpr int CPR = BR / 8, RPI = 64 / CPR;
                 const int k = q * RPI + lane / CPR;
                 const int c = (lane % CPR) ^ (4 * (k & 3));
                 const int gc = min(row0 + c * 8, rows - 8);
-                off[i] = (uint32_t)((k * ld + gc) * 2);
+                src[i] = base + (int64_t)k * ld + gc;
             }
         }
-        base = (const char*)mat;
-        step = (KM ? 32 * ld : 32) * 2;
+        step = KM ? 32 * ld : 32;
     }
-    // AHEAD: k-tiles beyond the operand's current position, a compile-time constant (row-major
-    // operands only; the caller guarantees those tiles exist)
-    template <int AHEAD> __device__ __forceinline__ void issue(unsigned char* tile, int wave) {
+    __device__ __forceinline__ void issue(unsigned char* tile, int wave) {
 #pragma unroll
         for (int i = 0; i < ROUNDS; ++i) {
-            const char* src;
-            if constexpr (KM) src = base + off[i];
-            else src = ptr[i] + AHEAD * 64;
-            __builtin_amdgcn_global_load_lds((gbl_ptr_t*)src, (lds_ptr_t*)(tile + (i * NW + wave) * 1024), 16, 0, 0);
-        }
-    }
-    __device__ __forceinline__ void advance(int tiles) {
-        if constexpr (KM) {
-            base += tiles * step;
-        } else {
-#pragma unroll
-            for (int i = 0; i < ROUNDS; ++i) ptr[i] += tiles * step;
+            __builtin_amdgcn_global_load_lds((gbl_ptr_t*)src[i], (lds_ptr_t*)(tile + (i * NW + wave) * 1024), 16, 0, 0);
+            src[i] += step;
         }
     }
 };
@@ -433,8 +415,7 @@ __device__ __forceinline__ void gemm_bf16_dma_body(const GemmArgs& g, const int 
     constexpr int LOADS = OpA::ROUNDS + OpB::ROUNDS;
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
 
-    const int tid = threadIdx.x, lane = tid & 63;
-    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // scalar: LDS targets and tile bases stay in SGPRs
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wm = wave / WN, wn = wave % WN;
     int tile_m, tile_n;
     if (logical_id) panel_coords(block_id, g.tiles_m, g.tiles_n, tile_m, tile_n);
@@ -447,8 +428,8 @@ __device__ __forceinline__ void gemm_bf16_dma_body(const GemmArgs& g, const int 
 
     OpA opa;
     OpB opb;
-    opa.init(A, g.lda, m0, g.M, lane, wave);
-    opb.init(B, g.ldb, n0, g.N, lane, wave);
+    opa.init(A, g.lda, m0, g.M, tid);
+    opb.init(B, g.ldb, n0, g.N, tid);
     FragReader<BM, TM, AKM> fa;
     FragReader<BN, TN, BKM> fb;
     fa.init(wm * WTM, lane);
@@ -469,23 +450,15 @@ __device__ __forceinline__ void gemm_bf16_dma_body(const GemmArgs& g, const int 
     const int KT = g.K / 32;
 
     // ring positions: tile t lives in stage t % STAGES
-    // Stage arguments are std::integral_constant<int, s>: s >= 0 names the ring stage at compile
-    // time (LDS addresses become instruction immediates), s < 0 takes the running counter.
     int issue_stage = 0, read_stage = 0;
-    auto issue_tile = [&](auto sc, auto ahead_c) {
-        constexpr int s = decltype(sc)::value, ahead = decltype(ahead_c)::value;
-        unsigned char* st = smem + (s >= 0 ? s : issue_stage) * STAGE_BYTES;
-        // inside an unrolled turn row-major operands stay put and reach tile `ahead` by immediate
-        // offset; k-major operands (and the running path, ahead < 0) advance after every tile
-        opa.template issue<(!AKM && ahead > 0) ? ahead : 0>(st, wave);
-        opb.template issue<(!BKM && ahead > 0) ? ahead : 0>(st + OpA::BYTES, wave);
-        if (AKM || ahead < 0) opa.advance(1);
-        if (BKM || ahead < 0) opb.advance(1);
-        if constexpr (s < 0) issue_stage = issue_stage + 1 == STAGES ? 0 : issue_stage + 1;
+    auto issue_tile = [&]() {
+        unsigned char* st = smem + issue_stage * STAGE_BYTES;
+        opa.issue(st, wave);
+        opb.issue(st + OpA::BYTES, wave);
+        issue_stage = issue_stage + 1 == STAGES ? 0 : issue_stage + 1;
     };
-    auto load_frags = [&](Frags& f, auto sc) {
-        constexpr int s = decltype(sc)::value;
-        const unsigned char* st = smem + (s >= 0 ? s : read_stage) * STAGE_BYTES;
+    auto load_frags = [&](Frags& f) {
+        const unsigned char* st = smem + read_stage * STAGE_BYTES;
 #pragma unroll
         for (int ks = 0; ks < 2; ++ks) {
 #pragma unroll
@@ -493,7 +466,7 @@ __device__ __forceinline__ void gemm_bf16_dma_body(const GemmArgs& g, const int 
 #pragma unroll
             for (int j = 0; j < TN; ++j) f.b[ks][j] = fb.load(st + OpA::BYTES, j, ks);
         }
-        if constexpr (s < 0) read_stage = read_stage + 1 == STAGES ? 0 : read_stage + 1;
+        read_stage = read_stage + 1 == STAGES ? 0 : read_stage + 1;
     };
     // bias gradient riding along: the waves of the first block column (and first wave column)
     // add up the A fragments they hold anyway: lane (m, kg) sees 8 of the 16 k values per step
@@ -535,59 +508,40 @@ __device__ __forceinline__ void gemm_bf16_dma_body(const GemmArgs& g, const int 
         }
     };
 
-    using Running = std::integral_constant<int, -1>;
     // prologue: tiles 0..STAGES-2 (clamped to the last tile when K is short)
 #pragma unroll
     for (int t = 0; t < STAGES - 1; ++t) {
         stop_at_end(t + 1);
-        issue_tile(Running{}, Running{});
+        issue_tile();
     }
     sync_tile();
     if constexpr (DB) {
         // fragments of tile kt+1 are fetched while the second half of tile kt is multiplied,
-        auto body = [&](int kt, Frags& cur, Frags& nxt, auto issue_sc, auto read_sc, auto ahead_c) {
+        // into the other register set
+        auto body = [&](int kt, Frags& cur, Frags& nxt) {
             constexpr int FRAG_READS = 2 * (TM * (AKM ? 2 : 1) + TN * (BKM ? 2 : 1));
-            if constexpr (decltype(ahead_c)::value < 0) stop_at_end(kt + STAGES);
-            issue_tile(issue_sc, ahead_c);
+            stop_at_end(kt + STAGES);
+            issue_tile();
             mfma_step(cur, 0);
             interleave_mfma_with<TM * TN, LOADS, 0x020>();   // DMA issues between the first-half MFMAs
             sync_tile();
-            load_frags(nxt, read_sc);
+            load_frags(nxt);
             mfma_step(cur, 1);
             interleave_mfma_with<TM * TN, FRAG_READS, 0x100>();  // next tile's fragment reads between the rest
         };
-        load_frags(f0, Running{});
+        load_frags(f0);
         int kt = 0;
-        // whole turns of the ring with the stage of every access fixed at compile time: tile t
-        // sits in stage t % STAGES, the loop advances by a multiple of STAGES (and of the two
-        // fragment sets), so the running counters stay where the prologue left them
-        constexpr int TURN = STAGES % 2 == 0 ? STAGES : 2 * STAGES;
-        // ... and only while every tile issued in the turn (up to kt + TURN + STAGES - 2) exists
-        for (; kt + TURN + STAGES - 1 <= KT; kt += TURN) {
-            static_for(
-                [&](auto uc) {
-                    constexpr int u = decltype(uc)::value;
-                    using IssueStage = std::integral_constant<int, (u + STAGES - 1) % STAGES>;
-                    using ReadStage = std::integral_constant<int, (u + 1) % STAGES>;
-                    using Ahead = std::integral_constant<int, u>;
-                    if constexpr (u % 2 == 0) body(kt + u, f0, f1, IssueStage{}, ReadStage{}, Ahead{});
-                    else body(kt + u, f1, f0, IssueStage{}, ReadStage{}, Ahead{});
-                },
-                std::make_integer_sequence<int, TURN>{});
-            if (!AKM) opa.advance(TURN);
-            if (!BKM) opb.advance(TURN);
-        }
         for (; kt + 1 < KT; kt += 2) {
-            body(kt, f0, f1, Running{}, Running{}, Running{});
-            body(kt + 1, f1, f0, Running{}, Running{}, Running{});
+            body(kt, f0, f1);
+            body(kt + 1, f1, f0);
         }
-        if (kt < KT) body(kt, f0, f1, Running{}, Running{}, Running{});
+        if (kt < KT) body(kt, f0, f1);
     } else {
         // single fragment set: other resident waves cover LDS latency and barrier waits
         for (int kt = 0; kt < KT; ++kt) {
             stop_at_end(kt + STAGES);
-            issue_tile(Running{}, Running{});
-            load_frags(f0, Running{});
+            issue_tile();
+            load_frags(f0);
             mfma_step(f0, 0);
             mfma_step(f0, 1);
             sync_tile();
