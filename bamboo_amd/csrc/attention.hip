@@ -36,6 +36,19 @@ struct AttnArgs {
     float scale;                                   // 1 / sqrt(d)
 };
 
+// Global -> LDS transfers (16 or 4 bytes per lane; the LDS target is M0 + lane * size), issued as
+// inline assembly: while the compiler sees such a load in flight it turns every wait for an LDS
+// read into lgkmcnt(0).  Unseen, fragment waits keep their exact counts; the kernels wait for
+// these loads explicitly (wait_vm) before each barrier, as they always did.
+__device__ __forceinline__ void dma16(const void* src, const unsigned char* lds_dst) {
+    const unsigned m0 = __builtin_amdgcn_readfirstlane((unsigned)(uintptr_t)(lds_ptr_t*)lds_dst);
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(m0), "v"(src) : "m0");
+}
+__device__ __forceinline__ void dma4(const void* src, const unsigned char* lds_dst) {
+    const unsigned m0 = __builtin_amdgcn_readfirstlane((unsigned)(uintptr_t)(lds_ptr_t*)lds_dst);
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, off" ::"s"(m0), "v"(src) : "m0");
+}
+
 // ---- LDS tile format: [rows][64] bf16, 128 B per row, 16-byte chunk c of row r at slot c ^ fsw(r)
 __device__ __forceinline__ int fsw(int r) { return (((r >> 1) & 1) << 2) | (((r >> 2) & 1) << 1) | ((r >> 3) & 1); }
 
@@ -45,7 +58,7 @@ __device__ __forceinline__ void dma_rows8(const bf16* gbase, int64_t ld, int row
     const int r = idx * 8 + (lane >> 3);
     const int c = (lane & 7) ^ fsw(r);
     const int gr = min(row0 + r, last_row);
-    __builtin_amdgcn_global_load_lds((gbl_ptr_t*)(gbase + (int64_t)gr * ld + c * 8), (lds_ptr_t*)(tile + idx * 1024), 16, 0, 0);
+    dma16(gbase + (int64_t)gr * ld + c * 8, tile + idx * 1024);
 }
 // Whole 64-row tile: this wave's two instructions (row groups wave and wave + 4).  Full tiles
 // take a wave-uniform base plus the lane's fixed offset; only a tile that reaches past the last
@@ -59,8 +72,8 @@ __device__ __forceinline__ void dma_tile64(const bf16* gbase, int64_t ld, int ro
                                            int wave, int lane, LaneOff lo) {
     if (row0 + 63 <= last_row) {
         const bf16* g = gbase + (int64_t)row0 * ld;
-        __builtin_amdgcn_global_load_lds((gbl_ptr_t*)(g + lo.o0), (lds_ptr_t*)(tile + wave * 1024), 16, 0, 0);
-        __builtin_amdgcn_global_load_lds((gbl_ptr_t*)(g + lo.o1), (lds_ptr_t*)(tile + (wave + 4) * 1024), 16, 0, 0);
+        dma16(g + lo.o0, tile + wave * 1024);
+        dma16(g + lo.o1, tile + (wave + 4) * 1024);
     } else {
         dma_rows8(gbase, ld, row0, last_row, tile, wave, lane);
         dma_rows8(gbase, ld, row0, last_row, tile, wave + 4, lane);
@@ -69,7 +82,7 @@ __device__ __forceinline__ void dma_tile64(const bf16* gbase, int64_t ld, int ro
 // 4-byte variant for the per-row fp32 statistics: 64 consecutive floats
 __device__ __forceinline__ void dma_f32x64(const float* gbase, int idx0, int last, unsigned char* dst, int lane) {
     const int i = min(idx0 + lane, last);
-    __builtin_amdgcn_global_load_lds((gbl_ptr_t*)(gbase + i), (lds_ptr_t*)dst, 4, 0, 0);
+    dma4(gbase + i, dst);
 }
 
 // A/B fragment along the contiguous (feature) dimension: lane (r = lane%32, kg = lane/32) gets

@@ -332,6 +332,18 @@ template <int N> __device__ __forceinline__ void wait_vmcnt_lgkm0() {
     __builtin_amdgcn_s_waitcnt((N & 15) | (7 << 4) | (0 << 8) | ((N >> 4) << 14));
 }
 
+// One wave-wide 16-byte-per-lane global -> LDS transfer (global_load_lds_dwordx4; the LDS target
+// is M0 + lane * 16).  Issued as inline assembly on purpose: while the compiler sees such a load in
+// flight it turns EVERY wait for an LDS read into lgkmcnt(0), i.e. each fragment wait would drain
+// all outstanding fragment reads.  Unseen, the fragment waits keep their exact counts.  The price:
+// the compiler does not count these loads in vmcnt either - the main loop waits for them explicitly
+// (it always did), and nothing else may touch the target stage or leave the kernel's main loop
+// without an explicit vmcnt wait.
+__device__ __forceinline__ void dma16(const void* src, const unsigned char* lds_dst) {
+    const unsigned m0 = __builtin_amdgcn_readfirstlane((unsigned)(uintptr_t)(lds_ptr_t*)lds_dst);
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(m0), "v"(src) : "m0");
+}
+
 template <int BR, bool KM, int NW> struct DmaOperand {
     static constexpr int BYTES = BR * 32 * 2;
     static constexpr int ROUNDS = BYTES / (1024 * NW);  // instructions per thread per k-tile
@@ -362,7 +374,7 @@ template <int BR, bool KM, int NW> struct DmaOperand {
     __device__ __forceinline__ void issue(unsigned char* tile, int wave) {
 #pragma unroll
         for (int i = 0; i < ROUNDS; ++i) {
-            __builtin_amdgcn_global_load_lds((gbl_ptr_t*)src[i], (lds_ptr_t*)(tile + (i * NW + wave) * 1024), 16, 0, 0);
+            dma16(src[i], tile + (i * NW + wave) * 1024);
             src[i] += step;
         }
     }
@@ -564,6 +576,7 @@ __device__ __forceinline__ void gemm_bf16_dma_body(const GemmArgs& g, const int 
     // taking 8 consecutive columns of row l/8, so every global load / store of the epilogue moves whole
     // 128-byte row segments (256 bytes for fp32 outputs).
     static_assert(TN % 2 == 0, "the epilogue walks the accumulator tiles in pairs");
+    wait_vmcnt_lgkm0<0>();  // the tiles issued past the end of K have to land before their stages become the patch
     __syncthreads();
     constexpr int PLD = 68;
     float* patch = (float*)smem + wave * (32 * PLD);
