@@ -808,12 +808,23 @@ static DmaTile pick_dma_tile(int M, int N, int K, int64_t batches) {
     const int ov = dma_tile_override();
     if (ov == 4) return D_NONE;
     if ((ov >= 1 && ov <= 3) || (ov >= 5 && ov <= 14)) return (DmaTile)ov;
-    // measured on MI355X (256 CUs): 256x256 tiles pay off from one and a half rounds of blocks on,
-    // 256x128 from one round, smaller problems take 128x128 tiles with two blocks per CU
+    // Rules read off a sweep of M 2048..16384 x N 768..6400 x K 1024/4096 on MI355X (256 CUs, one block
+    // of the 256-row tiles per CU):
+    //  - above one round of 256x256 tiles they win while the last round is at least ~70 % full;
+    //    a thinner last round goes to them only for long K (their main loop is the most efficient),
+    //    otherwise to 128x128 tiles, whose three blocks per CU smooth the tail
+    //  - within one round: 256x256 once 256x128 tiles would need a second round, 256x128 from about half
+    //    a round on, and 128x128 tiles for anything smaller
     const int64_t t256 = (int64_t)((M + 255) / 256) * ((N + 255) / 256) * batches;
     const int64_t t2128 = (int64_t)((M + 255) / 256) * ((N + 127) / 128) * batches;
-    if (M >= 256 && N >= 256 && t256 >= 384) return D256x256w8db;
-    if (M >= 256 && t2128 >= 256) return D256x128w8db;
+    const bool big_ok = M >= 256 && N >= 256;
+    if (t256 > 256) {
+        const int64_t rounds = (t256 + 255) / 256;
+        if (big_ok && (t256 * 10 >= rounds * 256 * 7 || K >= 1536)) return D256x256w8db;
+        return D128x128s3;
+    }
+    if (big_ok && t2128 > 256) return D256x256w8db;
+    if (M >= 256 && t2128 > 136) return D256x128w8db;
     return D128x128s3;
 }
 
