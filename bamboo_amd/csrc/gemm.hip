@@ -344,8 +344,8 @@ __device__ __forceinline__ void dma16(const void* src, const unsigned char* lds_
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(m0), "v"(src) : "m0");
 }
 
-template <int BR, bool KM, int NW> struct DmaOperand {
-    static constexpr int BYTES = BR * 32 * 2;
+template <int BR, bool KM, int NW, int BK = 32> struct DmaOperand {
+    static constexpr int BYTES = BR * BK * 2;
     static constexpr int ROUNDS = BYTES / (1024 * NW);  // instructions per thread per k-tile
     static_assert(ROUNDS >= 1, "tile too small for the block");
     const bf16* src[ROUNDS];
@@ -356,7 +356,13 @@ template <int BR, bool KM, int NW> struct DmaOperand {
 #pragma unroll
         for (int i = 0; i < ROUNDS; ++i) {
             const int q = i * NW + wave;
-            if constexpr (!KM) {
+            if constexpr (!KM && BK == 64) {
+                // 64-wide k-tiles: one instruction takes 8 rows x 128 B, whole cache lines
+                const int r = q * 8 + (lane >> 3);
+                const int c = (lane & 7) ^ ((r >> 1) & 7);
+                const int gr = min(row0 + r, rows - 1);
+                src[i] = base + (int64_t)gr * ld + c * 8;
+            } else if constexpr (!KM) {
                 const int r = q * 16 + (lane >> 2);
                 const int c = (lane & 3) ^ ((r >> 2) & 3);
                 const int gr = min(row0 + r, rows - 1);
@@ -369,7 +375,7 @@ template <int BR, bool KM, int NW> struct DmaOperand {
                 src[i] = base + (int64_t)k * ld + gc;
             }
         }
-        step = KM ? 32 * ld : 32;
+        step = KM ? BK * ld : BK;
     }
     __device__ __forceinline__ void issue(unsigned char* tile, int wave) {
 #pragma unroll
@@ -381,14 +387,14 @@ template <int BR, bool KM, int NW> struct DmaOperand {
 };
 
 // per-lane fragment offsets (bytes inside an operand tile) and the fragment fetch
-template <int BR, int T, bool KM> struct FragReader {
+template <int BR, int T, bool KM, int BK = 32> struct FragReader {
     int off[KM ? T : 1];
     int sw, hi;
     __device__ __forceinline__ void init(int wbase, int lane) {
         hi = lane >> 5;
         if constexpr (!KM) {
-            sw = ((lane & 31) >> 2) & 3;
-            off[0] = (wbase + (lane & 31)) * 64;
+            sw = BK == 64 ? ((lane & 31) >> 1) & 7 : ((lane & 31) >> 2) & 3;
+            off[0] = (wbase + (lane & 31)) * (BK * 2);
         } else {
             const int j4 = (lane & 15) >> 2;
             const int lo = ((lane >> 4) & 1) * 2 + ((lane & 3) >> 1);
@@ -403,7 +409,7 @@ template <int BR, int T, bool KM> struct FragReader {
     }
     __device__ __forceinline__ bf16x8 load(const unsigned char* tile, int t, int ks) const {
         if constexpr (!KM) {
-            return *(const bf16x8*)(tile + off[0] + t * 2048 + (((ks * 2 + hi) ^ sw) << 4));
+            return *(const bf16x8*)(tile + off[0] + t * (32 * BK * 2) + (((ks * 2 + hi) ^ sw) << 4));
         } else {
             const unsigned char* p = tile + off[t] + ks * 16 * (BR * 2);
             s16x4 lo4 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4*)(p));
@@ -415,14 +421,16 @@ template <int BR, int T, bool KM> struct FragReader {
     }
 };
 
-template <int BM, int BN, int WM, int WN, bool AKM, bool BKM, bool DB, int STAGES>
+template <int BM, int BN, int WM, int WN, bool AKM, bool BKM, bool DB, int STAGES, int BK = 32>
 __device__ __forceinline__ void gemm_bf16_dma_body(const GemmArgs& g, const int block_id, const int batch_id,
                                                    const bool logical_id = false) {
     constexpr int NW = WM * WN;
-    static_assert(STAGES >= 3, "the ring needs one stage being read, one landing, one in flight");
+    static_assert(BK == 64 ? ((STAGES == 2 || STAGES == 3) && DB) : STAGES >= 3,
+                  "32-wide k-tiles: the ring needs one stage being read, one landing, one in flight; "
+                  "64-wide k-tiles alternate between two stages or rotate through three");
     constexpr int WTM = BM / WM, WTN = BN / WN, TM = WTM / 32, TN = WTN / 32;
-    using OpA = DmaOperand<BM, AKM, NW>;
-    using OpB = DmaOperand<BN, BKM, NW>;
+    using OpA = DmaOperand<BM, AKM, NW, BK>;
+    using OpB = DmaOperand<BN, BKM, NW, BK>;
     constexpr int STAGE_BYTES = OpA::BYTES + OpB::BYTES;
     constexpr int LOADS = OpA::ROUNDS + OpB::ROUNDS;
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
@@ -442,8 +450,8 @@ __device__ __forceinline__ void gemm_bf16_dma_body(const GemmArgs& g, const int 
     OpB opb;
     opa.init(A, g.lda, m0, g.M, tid);
     opb.init(B, g.ldb, n0, g.N, tid);
-    FragReader<BM, TM, AKM> fa;
-    FragReader<BN, TN, BKM> fb;
+    FragReader<BM, TM, AKM, BK> fa;
+    FragReader<BN, TN, BKM, BK> fb;
     fa.init(wm * WTM, lane);
     fb.init(wn * WTN, lane);
 
@@ -459,7 +467,7 @@ __device__ __forceinline__ void gemm_bf16_dma_body(const GemmArgs& g, const int 
         bf16x8 a[2][TM], b[2][TN];
     };
     Frags f0, f1;
-    const int KT = g.K / 32;
+    const int KT = g.K / BK;
 
     // ring positions: tile t lives in stage t % STAGES
     int issue_stage = 0, read_stage = 0;
@@ -520,6 +528,58 @@ __device__ __forceinline__ void gemm_bf16_dma_body(const GemmArgs& g, const int 
         }
     };
 
+    if constexpr (BK == 64) {
+        // Two stages of 64-wide k-tiles, each multiplied as two 32-wide halves from the two fragment
+        // sets.  Per tile one barrier, in the middle of its second half: by then every wave has read
+        // the tile's last fragments (so its stage can take tile kt+2) and tile kt+1, issued one whole
+        // tile earlier, has to have landed (its first fragments are read right after).
+        auto load_half = [&](Frags& f, const unsigned char* st, int h) {
+#pragma unroll
+            for (int ks = 0; ks < 2; ++ks) {
+#pragma unroll
+                for (int i = 0; i < TM; ++i) f.a[ks][i] = fa.load(st, i, h * 2 + ks);
+#pragma unroll
+                for (int j = 0; j < TN; ++j) f.b[ks][j] = fb.load(st + OpA::BYTES, j, h * 2 + ks);
+            }
+        };
+        constexpr int FRAG_READS = 2 * (TM * (AKM ? 2 : 1) + TN * (BKM ? 2 : 1));
+        stop_at_end(1);
+        issue_tile();
+        stop_at_end(2);
+        issue_tile();
+        asm volatile("" ::: "memory");
+        wait_vmcnt_lgkm0<LOADS>();
+        __builtin_amdgcn_s_barrier();
+        asm volatile("" ::: "memory");
+        load_half(f0, smem, 0);
+        int rs = 0;
+        for (int kt = 0; kt < KT; ++kt) {
+            const unsigned char* cur = smem + rs * STAGE_BYTES;
+            rs = rs + 1 == STAGES ? 0 : rs + 1;
+            const unsigned char* nxt = smem + rs * STAGE_BYTES;
+            if constexpr (STAGES == 3) {
+                // a third stage lets tile kt+2 start a whole tile earlier: its stage held tile kt-1
+                stop_at_end(kt + 3);
+                issue_tile();
+            }
+            load_half(f1, cur, 1);
+            mfma_step(f0, 0);
+            mfma_step(f0, 1);
+            interleave_mfma_with<2 * TM * TN, FRAG_READS, 0x100>();
+            mfma_step(f1, 0);
+            asm volatile("" ::: "memory");
+            wait_vmcnt_lgkm0<(STAGES - 2) * LOADS>();
+            __builtin_amdgcn_s_barrier();
+            asm volatile("" ::: "memory");
+            if constexpr (STAGES == 2) {
+                stop_at_end(kt + 3);
+                issue_tile();  // tile kt+2 into the stage of tile kt
+            }
+            load_half(f0, nxt, 0);
+            mfma_step(f1, 1);
+            interleave_mfma_with<TM * TN, FRAG_READS, 0x100>();
+        }
+    } else {
     // prologue: tiles 0..STAGES-2 (clamped to the last tile when K is short)
 #pragma unroll
     for (int t = 0; t < STAGES - 1; ++t) {
@@ -558,6 +618,7 @@ __device__ __forceinline__ void gemm_bf16_dma_body(const GemmArgs& g, const int 
             mfma_step(f0, 1);
             sync_tile();
         }
+    }
     }
 
     if constexpr (AKM) {
@@ -609,9 +670,9 @@ __device__ __forceinline__ void gemm_bf16_dma_body(const GemmArgs& g, const int 
         std::make_integer_sequence<int, TM * TN / 2>{});
 }
 
-template <int BM, int BN, int WM, int WN, bool AKM, bool BKM, bool DB, int STAGES>
+template <int BM, int BN, int WM, int WN, bool AKM, bool BKM, bool DB, int STAGES, int BK>
 __global__ __launch_bounds__(WM* WN * 64) void gemm_bf16_dma_kernel(const GemmArgs g) {
-    gemm_bf16_dma_body<BM, BN, WM, WN, AKM, BKM, DB, STAGES>(g, blockIdx.x, blockIdx.z);
+    gemm_bf16_dma_body<BM, BN, WM, WN, AKM, BKM, DB, STAGES, BK>(g, blockIdx.x, blockIdx.z);
 }
 
 // Several independent problems of one kind in a single launch (the four weight-gradient GEMMs
@@ -772,10 +833,10 @@ static Bf16Tile pick_bf16_tile(int M, int N, int64_t batches) {
     return T128x128;
 }
 
-template <int BM, int BN, int WM, int WN, bool AKM, bool BKM, bool DB, int STAGES = 4>
+template <int BM, int BN, int WM, int WN, bool AKM, bool BKM, bool DB, int STAGES = 4, int BK = 32>
 static int launch_bf16_dma(GemmArgs& g, int batches, hipStream_t st) {
-    constexpr int smem = STAGES * (BM + BN) * 32 * 2;
-    auto kern = gemm_bf16_dma_kernel<BM, BN, WM, WN, AKM, BKM, DB, STAGES>;
+    constexpr int smem = STAGES * (BM + BN) * BK * 2;
+    auto kern = gemm_bf16_dma_kernel<BM, BN, WM, WN, AKM, BKM, DB, STAGES, BK>;
     static bool configured = false;
     if (!configured) {
         BB_HIP_CHECK(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, smem));
@@ -791,10 +852,11 @@ static int launch_bf16_dma(GemmArgs& g, int batches, hipStream_t st) {
 
 // DMA kernels need K % 32 == 0 and at least one full vector of rows; tile by problem size
 enum DmaTile { D_NONE = 0, D256x256, D256x128, D128x128, D_OFF, D256x256w8, D256x128w8, D256x256w8db, D256x128w8db,
-               D256x128w8s3, D128x128s3, D256x256w8s5, D256x128w8s6, D256x256w8s3, D256x128w4s3 };
+               D256x128w8s3, D128x128s3, D256x256w8s5, D256x128w8s6, D256x256w8s3, D256x128w4s3, D256x256k64, D256x128k64, D256x128k64s3, D128x128k64 };
 static const char* const kDmaTileNames[] = {"", "dma256x256", "dma256x128", "dma128x128", "", "dma256x256w8", "dma256x128w8",
                                             "dma256x256w8db", "dma256x128w8db", "dma256x128w8s3", "dma128x128s3",
-                                            "dma256x256w8s5", "dma256x128w8s6", "dma256x256w8s3", "dma256x128w4s3"};
+                                            "dma256x256w8s5", "dma256x128w8s6", "dma256x256w8s3", "dma256x128w4s3", "dma256x256k64",
+                                            "dma256x128k64", "dma256x128k64s3", "dma128x128k64"};
 // BB_DMA_TILE (tuning aid): 1..3 force a DMA tile where it is legal, 4 disables the DMA kernels.
 static int dma_tile_override() {
     static const int v = [] {
@@ -803,33 +865,42 @@ static int dma_tile_override() {
     }();
     return v;
 }
-static DmaTile pick_dma_tile(int M, int N, int K, int64_t batches) {
+static DmaTile pick_dma_tile(int M, int N, int K, int64_t batches, int layout) {
     if (K % 32 != 0 || K < 64 || M < 128 || N < 128 || N % 8 != 0) return D_NONE;
     const int ov = dma_tile_override();
     if (ov == 4) return D_NONE;
-    if ((ov >= 1 && ov <= 3) || (ov >= 5 && ov <= 14)) return (DmaTile)ov;
-    // Rules read off a sweep of M 2048..16384 x N 768..6400 x K 1024/4096 on MI355X (256 CUs, one block
-    // of the 256-row tiles per CU):
-    //  - above one round of 256x256 tiles they win while the last round is at least ~70 % full;
-    //    a thinner last round goes to them only for long K (their main loop is the most efficient),
-    //    otherwise to 128x128 tiles, whose three blocks per CU smooth the tail
-    //  - within one round: 256x256 once 256x128 tiles would need a second round, 256x128 from about half
-    //    a round on, and 128x128 tiles for anything smaller
+    if ((ov >= 1 && ov <= 3) || (ov >= 5 && ov <= 14) || (ov >= 15 && ov <= 18 && K % 64 == 0 && K >= 128)) return (DmaTile)ov;
+    // Rules read off sweeps of M 2048..16384 x N 768..6400 x K 1024/4096 (NT and NN) on MI355X (256 CUs,
+    // one block of the 256-row tiles per CU).
+    //  - Operands whose rows are k-contiguous (both of NT, A of NN) load faster as 64-wide k-tiles: one
+    //    DMA instruction then covers 8 whole 128-byte lines instead of 16 half lines.  The smaller the
+    //    tile, the more of its time is loading and the more that buys (128x128: up to +19 %, 256x128:
+    //    +3..8 %, 256x256: nothing, and its two 64 KB stages cost prologue time).
+    //  - Above one round of 256x256 tiles they win while the last round is well filled; otherwise the
+    //    small tiles, several blocks per CU, smooth the tail.
+    //  - Within one round: 256x256 once 256x128 tiles would need a second round, 256x128 from about half
+    //    a round on, and 128x128 tiles for anything smaller.
+    const bool nt = layout == BB_NT, nn = layout == BB_NN;
+    const bool k64 = (nt || nn) && K % 64 == 0 && K >= 128;
+    const DmaTile small = k64 && (nt || K >= 2048) ? D128x128k64 : D128x128s3;
+    const DmaTile mid = !k64 ? D256x128w8db : (nt && K < 2048) ? D256x128k64 : D256x128k64s3;
     const int64_t t256 = (int64_t)((M + 255) / 256) * ((N + 255) / 256) * batches;
     const int64_t t2128 = (int64_t)((M + 255) / 256) * ((N + 127) / 128) * batches;
     const bool big_ok = M >= 256 && N >= 256;
     if (t256 > 256) {
-        const int64_t rounds = (t256 + 255) / 256;
-        if (big_ok && (t256 * 10 >= rounds * 256 * 7 || K >= 1536)) return D256x256w8db;
-        return D128x128s3;
+        const int64_t slots = (t256 + 255) / 256 * 256;
+        const bool full85 = t256 * 100 >= slots * 85, full70 = t256 * 10 >= slots * 7;
+        if (!big_ok) return small;
+        if (k64) return full85 || (nn && K >= 2048 && full70) ? D256x256w8db : small;
+        return full70 || K >= 1536 ? D256x256w8db : small;
     }
     if (big_ok && t2128 > 256) return D256x256w8db;
-    if (M >= 256 && t2128 > 136) return D256x128w8db;
-    return D128x128s3;
+    if (M >= 256 && t2128 > 136) return mid;
+    return small;
 }
 
 template <bool TA, bool TB> static int dispatch_bf16(GemmArgs& g, int batches, hipStream_t st) {
-    switch (pick_dma_tile(g.M, g.N, g.K, batches)) {
+    switch (pick_dma_tile(g.M, g.N, g.K, batches, TA ? BB_TN : TB ? BB_NN : BB_NT)) {
         case D256x256: return launch_bf16_dma<256, 256, 2, 2, TA, TB, true>(g, batches, st);
         case D256x128: return launch_bf16_dma<256, 128, 2, 2, TA, TB, true>(g, batches, st);
         case D128x128: return launch_bf16_dma<128, 128, 2, 2, TA, TB, true>(g, batches, st);
@@ -843,6 +914,10 @@ template <bool TA, bool TB> static int dispatch_bf16(GemmArgs& g, int batches, h
         case D256x128w8s6: return launch_bf16_dma<256, 128, 4, 2, TA, TB, true, 6>(g, batches, st);
         case D256x256w8s3: return launch_bf16_dma<256, 256, 2, 4, TA, TB, true, 3>(g, batches, st);
         case D256x128w4s3: return launch_bf16_dma<256, 128, 2, 2, TA, TB, true, 3>(g, batches, st);
+        case D256x256k64: return launch_bf16_dma<256, 256, 2, 4, TA, TB, true, 2, 64>(g, batches, st);
+        case D256x128k64: return launch_bf16_dma<256, 128, 4, 2, TA, TB, true, 2, 64>(g, batches, st);
+        case D256x128k64s3: return launch_bf16_dma<256, 128, 4, 2, TA, TB, true, 3, 64>(g, batches, st);
+        case D128x128k64: return launch_bf16_dma<128, 128, 2, 2, TA, TB, true, 2, 64>(g, batches, st);
         default: break;
     }
     switch (pick_bf16_tile(g.M, g.N, batches)) {
@@ -868,7 +943,7 @@ extern "C" int bb_gemm_variant(const bb_gemm_desc* d, char* out, int out_len) {
     BB_REQUIRE(d->layout >= BB_NT && d->layout <= BB_TN, "bb_gemm_variant: bad layout %d", d->layout);
     const int64_t batches = (int64_t)(d->nb1 > 0 ? d->nb1 : 1) * (d->nb2 > 0 ? d->nb2 : 1);
     if (d->dtype == BB_BF16) {
-        const DmaTile dt = pick_dma_tile(d->M, d->N, d->K, batches);
+        const DmaTile dt = pick_dma_tile(d->M, d->N, d->K, batches, d->layout);
         snprintf(out, out_len, "bf16_%s_%s", layouts[d->layout],
                  dt != D_NONE ? kDmaTileNames[dt] : kBf16TileNames[pick_bf16_tile(d->M, d->N, batches)]);
     }
@@ -920,7 +995,7 @@ static int fill_args(const bb_gemm_desc* d, GemmArgs& g, int64_t& batches, bool&
 // The bias-gradient column sums ride inside the DMA kernel when it runs the problem; otherwise
 // the stand-alone reduction computes them.
 static bool colsum_fusable(const bb_gemm_desc* d, int64_t batches) {
-    return d->colsum_out && d->dtype == BB_BF16 && batches == 1 && pick_dma_tile(d->M, d->N, d->K, 1) != D_NONE;
+    return d->colsum_out && d->dtype == BB_BF16 && batches == 1 && pick_dma_tile(d->M, d->N, d->K, 1, d->layout) != D_NONE;
 }
 static int colsum_standalone(const bb_gemm_desc* d, void* stream) {
     BB_REQUIRE(d->colsum_ws, "bb_gemm: colsum_out on this problem needs colsum_ws");
@@ -981,7 +1056,7 @@ extern "C" int bb_gemm_grouped(const bb_gemm_desc* descs, int count, void* strea
     for (int i = 0; i < count && fuse; ++i) {
         const bb_gemm_desc& d = descs[i];
         fuse = d.dtype == BB_BF16 && d.layout == descs[0].layout && d.nb1 <= 1 && d.nb2 <= 1 && d.M > 0 && d.N > 0 &&
-               pick_dma_tile(d.M, d.N, d.K, 1) != D_NONE && dma_tile_override() != 4;
+               pick_dma_tile(d.M, d.N, d.K, 1, d.layout) != D_NONE && dma_tile_override() != 4;
     }
     if (!fuse) {
         for (int i = 0; i < count; ++i) {
@@ -1041,7 +1116,7 @@ static int pick_splits(const bb_gemm_desc* descs, int count) {
         const bb_gemm_desc& d = descs[i];
         if (d.dtype != BB_BF16 || d.c_dtype != BB_F32 || d.layout != descs[0].layout || d.nb1 > 1 || d.nb2 > 1 || d.M <= 0 ||
             d.N <= 0 || d.colsum_out || d.bias || d.epilogue != BB_EPI_NONE || d.alpha != 1.0f || d.N % 4 != 0 ||
-            pick_dma_tile(d.M, d.N, d.K, 1) == D_NONE)
+            pick_dma_tile(d.M, d.N, d.K, 1, d.layout) == D_NONE)
             return 0;
         tiles += (int64_t)((d.M + 127) / 128) * ((d.N + 127) / 128);
         kmin = d.K < kmin ? d.K : kmin;
