@@ -1,5 +1,6 @@
 """The C-ABI library builds, loads without a GPU, and exports every symbol the header declares."""
 import ctypes
+import json
 import os
 import re
 
@@ -57,20 +58,37 @@ def test_gemm_desc_layout_matches_header():
     assert names == [f[0] for f in hip.GemmDesc._fields_]
 
 
+GOLDEN = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "reference_known_answers.json")
+
+
 def test_partition_known_answers():
-    # tests/unit/test_partition.py:103-190 of the reference tree
+    """The partitioning known answers of the reference's unit tests (tests/unit/test_partition.py:95-193),
+    kept as data in tests/golden/."""
     from bamboo_amd.utils import partition_balanced, partition_uniform
-    assert partition_uniform(8, 4) == [0, 2, 4, 6, 8]
+    kat = json.load(open(GOLDEN))
+    for c in kat["partition_uniform"]["cases"]:
+        assert partition_uniform(c["num_items"], c["num_parts"]) == c["parts"]
     assert partition_uniform(2, 4) == [0, 1, 2, 2, 2]
-    assert partition_balanced([1] * 8, 4) == [0, 2, 4, 6, 8]
-    assert partition_balanced([0, 1, 2, 3, 3, 3], 4) == [0, 3, 4, 5, 6]
-    assert partition_balanced([0., 1.1, 1.9, 3., 3., 3.], 4) == [0, 3, 4, 5, 6]
-    assert partition_balanced([0., 1.1, 30, 3.], 3) == [0, 2, 3, 4]
-    w = [52559872] + [12596224] * 24 + [0, 52559872]
+    for c in kat["partition_balanced"]["cases"]:
+        assert partition_balanced(c["weights"], c["num_parts"]) == c["parts"]
+    for c in kat["partition_balanced_valid_only"]["cases"]:
+        w, parts = c["weights"], partition_balanced(c["weights"], c["num_parts"])
+        # assert_valid_partition of the reference: P+1 non-decreasing bounds from 0 to N
+        assert len(parts) == c["num_parts"] + 1 and parts[0] == 0 and parts[-1] == len(w)
+        assert all(a <= b for a, b in zip(parts, parts[1:]))
+    w = kat["partition_balanced_valid_only"]["cases"][1]["weights"]
     parts = partition_balanced(w, 8)
-    assert parts[0] == 0 and parts[-1] == len(w) and all(a <= b for a, b in zip(parts, parts[1:]))
     heaviest = max(sum(w[a:b]) for a, b in zip(parts, parts[1:]))
     assert heaviest <= 52559872 + 12596224        # optimum: one end layer plus at most one transformer layer
+
+
+def test_layer_parameter_count_matches_reference_figure():
+    """12h^2 + 13h parameters per encoder layer at f = 4h: the figure the reference's partition test uses."""
+    kat = json.load(open(GOLDEN))["transformer_layer_parameters"]
+    h, f = kat["hidden"], kat["ffn"]
+    assert 4 * (h * h + h) + 2 * h * f + f + h + 4 * h == kat["params"]
+    from bamboo_amd.layers import TransformerLayer
+    assert TransformerLayer(h, 16, f).num_params() == kat["params"]
 
 
 def test_config_batch_triad():

@@ -1,4 +1,7 @@
 """The product's schedule classes against the oracle streams, instruction by instruction."""
+import json
+import os
+
 import pytest
 
 from bamboo_amd import schedule as S
@@ -82,12 +85,9 @@ def test_upstream_invariants():
 
 def test_repr_and_call_to_str():
     # tests/unit/test_runtime_utils.py:14-22 of the reference tree
-    c2s = S.call_to_str
-    assert c2s("int") == "int()"
-    assert c2s("int", 3) == "int(3)"
-    assert c2s("int", 3, "jeff") == "int(3, 'jeff')"
-    assert c2s("hello", val=3) == "hello(val=3)"
-    assert c2s("hello", 1138, val=3) == "hello(1138, val=3)"
+    golden = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "reference_known_answers.json")
+    for c in json.load(open(golden))["call_to_str"]["cases"]:
+        assert S.call_to_str(*c["args"], **c["kwargs"]) == c["out"]
     assert repr(S.ForwardPass(2, 1)) == "ForwardPass(buffer_id=2, stage_id=1)"
     assert repr(S.OptimizerStep()) == "OptimizerStep()"
 
