@@ -128,8 +128,14 @@ class PipelineModule:
                  dtype=torch.float32, device=None):
         if num_stages is None and topology is None:
             raise RuntimeError("must provide num_stages or topology")
-        if activation_checkpoint_interval != 0:
-            raise NotImplementedError("activation checkpointing is not part of the accelerated stage path")
+        if activation_checkpoint_interval < 0:
+            raise ValueError("activation_checkpoint_interval must be >= 0")
+        # Groups of this many layers keep only their input per micro-batch; the backward pass runs the
+        # group's forward again (same kernels, same bits) into a work stash shared by all micro-batches
+        # (reference: module.py:551-573; activation_checkpoint_func is accepted and unused: the stash is
+        # explicit here, there is no autograd graph to cut).
+        self.activation_checkpoint_interval = int(activation_checkpoint_interval)
+        self.activation_checkpoint_func = activation_checkpoint_func
         self.num_stages = num_stages if num_stages is not None else topology.get_dim("pipe")
         if stage_id is None:
             stage_id = self._stage_from_env()
@@ -301,9 +307,16 @@ class PipelineModule:
         return self.parts[stage_id + 1] - self.parts[stage_id]
 
     # ------------------------------------------------------------------ stash
+    def _checkpoint_groups(self, stage_id):
+        n, every = len(self.func_buckets[stage_id]), self.activation_checkpoint_interval
+        return [(a, min(a + every, n)) for a in range(0, n, every)]
+
     def allocate_stash(self, stage_id, ctx, slots):
-        """One arena holding, for every (slot, layer), the activations its backward needs."""
+        """One arena holding, for every (slot, layer), the activations its backward needs.  With
+        activation checkpointing: one such set of per-layer buffers for the whole stage (the work
+        stash) plus, per slot, the input of every layer group and the stage output."""
         layers = self.func_buckets[stage_id]
+        ckpt = self.activation_checkpoint_interval > 0
         plans, total = [], 0
         for layer in layers:
             plan = []
@@ -312,9 +325,10 @@ class PipelineModule:
                 plan.append((name, shape, dtype, total, nbytes))
                 total += (nbytes + 255) // 256 * 256
             plans.append(plan)
-        arena = torch.empty(total * slots, dtype=torch.uint8, device=self.device)
+        full_sets = 1 if ckpt else slots
+        arena = torch.empty(total * full_sets, dtype=torch.uint8, device=self.device)
         table = []
-        for s in range(slots):
+        for s in range(full_sets):
             per_layer = []
             for plan in plans:
                 views = {}
@@ -323,10 +337,29 @@ class PipelineModule:
                     views[name] = arena[lo: lo + nbytes].view(dtype).view(shape)
                 per_layer.append(views)
             table.append(per_layer)
-        self._stash[stage_id] = table
+        nbytes_total = total * full_sets
         self._stash_arena = getattr(self, "_stash_arena", {})
         self._stash_arena[stage_id] = arena
-        return total * slots
+        if ckpt:
+            groups = self._checkpoint_groups(stage_id)
+            es = torch.empty((), dtype=self.dtype).element_size()
+            sizes = [ctx.rows * layers[a].feature_dim for a, _ in groups] + [ctx.rows * layers[-1].feature_dim]
+            per_slot = sum((n * es + 255) // 256 * 256 for n in sizes)
+            keep = torch.empty(per_slot * slots, dtype=torch.uint8, device=self.device)
+            kept = []
+            for s in range(slots):
+                lo, bufs = s * per_slot, []
+                for n in sizes:
+                    bufs.append(keep[lo: lo + n * es].view(self.dtype).view(ctx.rows, n // ctx.rows))
+                    lo += (n * es + 255) // 256 * 256
+                kept.append(bufs)          # [group inputs ..., stage output]
+            self._kept = getattr(self, "_kept", {})
+            self._kept[stage_id] = kept
+            self._stash_arena[(stage_id, "kept")] = keep
+            nbytes_total += per_slot * slots
+            table = [table[0]] * slots     # every slot works in the one shared set
+        self._stash[stage_id] = table
+        return nbytes_total
 
     # ------------------------------------------------------------------ execution
     def forward(self, forward_input, stage_id, slot=0, ctx=None):
@@ -335,9 +368,19 @@ class PipelineModule:
             raise Exception(f"Unregistered stage id {stage_id}")
         self.micro_offset += 1
         x = forward_input
-        for layer, st in zip(layers, self._stash[stage_id][slot]):
-            x = layer.forward(x, st, ctx)
-        return x
+        stash = self._stash[stage_id][slot]
+        if self.activation_checkpoint_interval == 0:
+            for layer, st in zip(layers, stash):
+                x = layer.forward(x, st, ctx)
+            return x
+        kept = self._kept[stage_id][slot]
+        for g, (a, b) in enumerate(self._checkpoint_groups(stage_id)):
+            hip.cast(x, kept[g], stream=ctx.stream)   # same-type copy: the group's input outlives the work stash
+            x = kept[g]
+            for i in range(a, b):
+                x = layers[i].forward(x, stash[i], ctx)
+        hip.cast(x, kept[-1], stream=ctx.stream)
+        return kept[-1]
 
     def backward(self, grad_output, grad_input, stage_id, slot=0, ctx=None):
         """Back-propagate through the layers of ``stage_id`` from the stash of ``slot``; parameter
@@ -347,10 +390,21 @@ class PipelineModule:
         stash = self._stash[stage_id][slot]
         n = len(layers)
         d = grad_output
-        for i in range(n - 1, -1, -1):
-            dst = grad_input if i == 0 else ctx.buf(f"d_layer{i % 2}", tuple(grad_output.shape))
-            layers[i].backward(d, dst, stash[i], ctx)
-            d = dst
+        groups = self._checkpoint_groups(stage_id) if self.activation_checkpoint_interval > 0 else [(0, n)]
+        for g in range(len(groups) - 1, -1, -1):
+            a, b = groups[g]
+            if self.activation_checkpoint_interval > 0:
+                # run the group's forward again from its kept input; like a redundant forward it must not
+                # update running statistics a second time
+                was, ctx.redundant = ctx.redundant, True
+                x = self._kept[stage_id][slot][g]
+                for i in range(a, b):
+                    x = layers[i].forward(x, stash[i], ctx)
+                ctx.redundant = was
+            for i in range(b - 1, a - 1, -1):
+                dst = grad_input if i == 0 else ctx.buf(f"d_layer{i % 2}", tuple(grad_output.shape))
+                layers[i].backward(d, dst, stash[i], ctx)
+                d = dst
         return grad_input
 
     def prepare_context(self, stage_ids, batch, seq, stream=None, forward_only=False):

@@ -34,9 +34,10 @@ def grad_floor(ref_grads):
 
 
 def build(hidden, heads, ffn, layers_per_stage, stages, stage_id, mb, M, seq, dtype, variant, rl, eager,
-          grad_mode="queue", rc_stream=False, key_len_range=None, **engine_kwargs):
+          grad_mode="queue", rc_stream=False, key_len_range=None, checkpoint_interval=0, **engine_kwargs):
     specs = [LayerSpec(TransformerLayer, hidden, heads, ffn, **variant) for _ in range(layers_per_stage * stages)]
-    model = PipelineModule(specs, num_stages=stages, partition_method="uniform", stage_id=stage_id, dtype=dtype, device=DEV)
+    model = PipelineModule(specs, num_stages=stages, partition_method="uniform", stage_id=stage_id, dtype=dtype, device=DEV,
+                           activation_checkpoint_interval=checkpoint_interval)
     q = SeededActivationQueue((mb, seq, hidden), dtype, M, stage_ids=[stage_id, (stage_id + 1) % stages], seed=7,
                               grad_mode=grad_mode, device=DEV, key_len_range=key_len_range)
     cfg = {"train_micro_batch_size_per_gpu": mb, "gradient_accumulation_steps": M,
@@ -348,6 +349,64 @@ def test_graph_replay_equals_eager(hiplib, variant, klr, rc_stream):
         a, b = engine.module.stage_params[s_], eager_engine.module.stage_params[s_]
         assert torch.equal(a.master, b.master) and torch.equal(a.compute, b.compute)
     assert losses[4] != losses[0]
+
+
+@pytest.mark.parametrize("interval", [1, 2, 3])
+@pytest.mark.parametrize("rc_stream", [False, True], ids=["one-stream", "rc-stream"])
+def test_activation_checkpointing_equals_full_stash(hiplib, interval, rc_stream):
+    """activation_checkpoint_interval > 0 (reference module.py:551-573): only the input of every layer group is
+    kept per micro-batch and the group's forward runs again in the backward pass.  Losses of batches with
+    optimizer steps, a batch that loses the successor at micro-batch 2 (backward of the promoted layers from
+    their kept inputs), the batch after it, and all weights are bit-equal to the full stash, which takes
+    several times the memory."""
+    hid, heads, ffn, L, S, sid, mb, M, seq = 128, 2, 256, 3, 4, 1, 2, 4, 64
+    dtype = torch.bfloat16
+    runs = []
+    for every in (0, interval):
+        engine, q = build(hid, heads, ffn, L, S, sid, mb, M, seq, dtype, GPT_VARIANT, 1, True, grad_mode="mse",
+                          rc_stream=rc_stream, checkpoint_interval=every)
+        losses = [float(engine.train_batch()) for _ in range(3)]
+        q.preempt_successor(2, sid)
+        losses += [float(engine.train_batch()), float(engine.train_batch())]
+        torch.cuda.synchronize()
+        runs.append((engine, losses))
+    (full, lf), (ck, lc) = runs
+    assert lf == lc and lf[2] != lf[0]
+    assert ck.stash_bytes * 2 < full.stash_bytes
+    for s_ in (sid, sid + 1):
+        a, b = full.module.stage_params[s_], ck.module.stage_params[s_]
+        assert torch.equal(a.master, b.master) and torch.equal(a.compute, b.compute)
+        assert torch.equal(a.exp_avg, b.exp_avg) and torch.equal(a.exp_avg_sq, b.exp_avg_sq)
+
+
+def test_activation_checkpointing_resnet_keeps_running_statistics(hiplib):
+    """Bottleneck stage with checkpoint groups of one block: gradients, outputs and the BatchNorm running
+    statistics (updated once per forward, not again by the recomputation) equal the full stash bit for bit."""
+    from bamboo_amd import BottleNeck
+    cin, cmid, side, L, S, sid, mb, M = 64, 16, 6, 2, 4, 1, 4, 4
+    dtype = torch.bfloat16
+    runs = []
+    for every in (0, 1):
+        specs = [LayerSpec(BottleNeck, cin, cmid, height=side, width=side) for _ in range(L * S)]
+        model = PipelineModule(specs, num_stages=S, partition_method="uniform", stage_id=sid, dtype=dtype, device=DEV,
+                               activation_checkpoint_interval=every)
+        q = SeededActivationQueue((mb, side * side, cin), dtype, M, stage_ids=[sid, sid + 1], seed=9, device=DEV)
+        cfg = {"train_micro_batch_size_per_gpu": mb, "gradient_accumulation_steps": M, "bf16": {"enabled": True}}
+        engine, _, _, _ = bamboo_amd.initialize(model=model, config=cfg, redundancy_level=1, eager_recovery=True,
+                                                activation_queue=q, install_signal_handler=False)
+        for _ in range(2):
+            engine.train_batch()
+        torch.cuda.synchronize()
+        runs.append(engine)
+    a, b = runs
+    for s_ in (sid, sid + 1):
+        pa, pb = a.module.stage_params[s_], b.module.stage_params[s_]
+        assert torch.equal(pa.master, pb.master) and torch.equal(pa.exp_avg_sq, pb.exp_avg_sq)
+    for la, lb in zip(a.module.func_buckets[sid], b.module.func_buckets[sid]):
+        ra, rb = la._running(DEV), lb._running(DEV)
+        for idx in ra:
+            assert torch.equal(ra[idx][0], rb[idx][0]) and torch.equal(ra[idx][1], rb[idx][1])
+            assert float(ra[idx][0].abs().sum()) > 0      # the running mean has moved off its zero start
 
 
 def test_optimizer_step_matches_oracle(hiplib):
