@@ -384,6 +384,10 @@ template <int BR, bool KM, int NW, int BK = 32> struct DmaOperand {
             src[i] += step;
         }
     }
+    template <int I> __device__ __forceinline__ void issue_one(unsigned char* tile, int wave) {
+        dma16(src[I], tile + (I * NW + wave) * 1024);
+        src[I] += step;
+    }
 };
 
 // per-lane fragment offsets (bytes inside an operand tile) and the fragment fetch
@@ -512,6 +516,48 @@ __device__ __forceinline__ void gemm_bf16_dma_body(const GemmArgs& g, const int 
             }
         }
     };
+    // One quarter / half of a tile placed by hand: MFMA m of step ks, then its share of ND DMA
+    // instructions into stage `dst` and of the fragment reads of (stage `src`, half h) into `nf` (the
+    // reads ride on the first FM MFMAs so that the last ones cover their latency), each group fenced:
+    // the DMA instructions are inline assembly, opaque to the scheduler's group hints, and unfenced
+    // they end up bunched behind the barrier.
+    auto placed_step = [&](const Frags& f, auto ks_c, auto nd_c, unsigned char* dst, auto reads_c, Frags& nf,
+                           const unsigned char* src, int h) {
+        constexpr int ks = decltype(ks_c)::value, ND = decltype(nd_c)::value;
+        constexpr bool READS = decltype(reads_c)::value;
+        constexpr int NM = TM * TN, NF = 2 * (TM + TN), FM = NM > 2 ? NM - 2 : NM;
+        static_for(
+            [&](auto idx) {
+                constexpr int m = decltype(idx)::value, i = m / TN, j = m % TN;
+                acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(f.a[ks][i], f.b[ks][j], acc[i][j], 0, 0, 0);
+                if constexpr (AKM && j == 0) {
+                    if (do_colsum) {
+                        float t = 0.f;
+#pragma unroll
+                        for (int e = 0; e < 8; ++e) t += (float)f.a[ks][i][e];
+                        csum[i] += t;
+                    }
+                }
+                static_for(
+                    [&](auto d) {
+                        constexpr int k = (ND * m) / NM + decltype(d)::value;
+                        if constexpr (k < OpA::ROUNDS) opa.template issue_one<k>(dst, wave);
+                        else opb.template issue_one<k - OpA::ROUNDS>(dst + OpA::BYTES, wave);
+                    },
+                    std::make_integer_sequence<int, (ND * (m + 1)) / NM - (ND * m) / NM>{});
+                if constexpr (READS && m < FM) {
+                    static_for(
+                        [&](auto r) {
+                            constexpr int q = (NF * m) / FM + decltype(r)::value, fk = q / (TM + TN), t = q % (TM + TN);
+                            if constexpr (t < TM) nf.a[fk][t] = fa.load(src, t, h * 2 + fk);
+                            else nf.b[fk][t - TM] = fb.load(src + OpA::BYTES, t - TM, h * 2 + fk);
+                        },
+                        std::make_integer_sequence<int, (NF * (m + 1)) / FM - (NF * m) / FM>{});
+                }
+                __builtin_amdgcn_sched_barrier(0);
+            },
+            std::make_integer_sequence<int, NM>{});
+    };
     // Steady state is branch-free: a tile is issued every iteration (past the end of K the
     // sources stop advancing, so the last tile is fetched again into a stage nobody reads),
     // hence exactly STAGES-2 newer tiles are in flight whenever a wave waits for the next tile.
@@ -567,17 +613,24 @@ __device__ __forceinline__ void gemm_bf16_dma_body(const GemmArgs& g, const int 
             mfma_step(f0, 1);
             interleave_mfma_with<2 * TM * TN, FRAG_READS, 0x100>();
             mfma_step(f1, 0);
+            // scheduling fences: without them the compiler sinks this third quarter below the barrier
+            // and bunches the next tile's fragment reads at the end of the iteration, right in front
+            // of the wait for them
+            __builtin_amdgcn_sched_barrier(0);
             asm volatile("" ::: "memory");
             wait_vmcnt_lgkm0<(STAGES - 2) * LOADS>();
             __builtin_amdgcn_s_barrier();
             asm volatile("" ::: "memory");
+            // last quarter: the DMA instructions of tile kt+2 (two stages: into the stage of tile kt)
+            // and the first fragment reads of tile kt+1 between its MFMAs
+            unsigned char* dst = smem + issue_stage * STAGE_BYTES;
             if constexpr (STAGES == 2) {
                 stop_at_end(kt + 3);
-                issue_tile();  // tile kt+2 into the stage of tile kt
+                issue_stage = issue_stage + 1 == STAGES ? 0 : issue_stage + 1;
             }
-            load_half(f0, nxt, 0);
-            mfma_step(f1, 1);
-            interleave_mfma_with<TM * TN, FRAG_READS, 0x100>();
+            placed_step(f1, std::integral_constant<int, 1>{}, std::integral_constant<int, STAGES == 2 ? LOADS : 0>{}, dst,
+                        std::true_type{}, f0, nxt, 0);
+            __builtin_amdgcn_sched_barrier(0);
         }
     } else {
     // prologue: tiles 0..STAGES-2 (clamped to the last tile when K is short)
@@ -590,7 +643,25 @@ __device__ __forceinline__ void gemm_bf16_dma_body(const GemmArgs& g, const int 
     if constexpr (DB) {
         // fragments of tile kt+1 are fetched while the second half of tile kt is multiplied,
         // into the other register set
+        // Hand placement pays on the 256x256 tile (eight MFMAs per half to place things between: +1..5 %);
+        // on the smaller tiles and with two k-major operands (twice the fragment read instructions) the
+        // scheduler's own order is as good or better.
+        constexpr bool PLACED = BM == 256 && BN == 256 && !AKM;
         auto body = [&](int kt, Frags& cur, Frags& nxt) {
+          if constexpr (PLACED) {
+            // first half: the DMA instructions of tile kt+STAGES-1 between its MFMAs; second half, behind
+            // the barrier: the fragment reads of tile kt+1
+            stop_at_end(kt + STAGES);
+            unsigned char* dst = smem + issue_stage * STAGE_BYTES;
+            issue_stage = issue_stage + 1 == STAGES ? 0 : issue_stage + 1;
+            placed_step(cur, std::integral_constant<int, 0>{}, std::integral_constant<int, LOADS>{}, dst, std::false_type{},
+                        nxt, smem, 0);
+            sync_tile();
+            const unsigned char* st = smem + read_stage * STAGE_BYTES;
+            read_stage = read_stage + 1 == STAGES ? 0 : read_stage + 1;
+            placed_step(cur, std::integral_constant<int, 1>{}, std::integral_constant<int, 0>{}, dst, std::true_type{}, nxt,
+                        st, 0);
+          } else {
             constexpr int FRAG_READS = 2 * (TM * (AKM ? 2 : 1) + TN * (BKM ? 2 : 1));
             stop_at_end(kt + STAGES);
             issue_tile();
@@ -600,6 +671,7 @@ __device__ __forceinline__ void gemm_bf16_dma_body(const GemmArgs& g, const int 
             load_frags(nxt);
             mfma_step(cur, 1);
             interleave_mfma_with<TM * TN, FRAG_READS, 0x100>();  // next tile's fragment reads between the rest
+          }
         };
         load_frags(f0);
         int kt = 0;
@@ -875,7 +947,7 @@ static DmaTile pick_dma_tile(int M, int N, int K, int64_t batches, int layout) {
     //  - Operands whose rows are k-contiguous (both of NT, A of NN) load faster as 64-wide k-tiles: one
     //    DMA instruction then covers 8 whole 128-byte lines instead of 16 half lines.  The smaller the
     //    tile, the more of its time is loading and the more that buys (128x128: up to +19 %, 256x128:
-    //    +3..8 %, 256x256: nothing, and its two 64 KB stages cost prologue time).
+    //    +3..8 %, 256x256: +4 % for long K only, its two 64 KB stages cost prologue time).
     //  - Above one round of 256x256 tiles they win while the last round is well filled; otherwise the
     //    small tiles, several blocks per CU, smooth the tail.
     //  - Within one round: 256x256 once 256x128 tiles would need a second round, 256x128 from about half
@@ -891,10 +963,10 @@ static DmaTile pick_dma_tile(int M, int N, int K, int64_t batches, int layout) {
         const int64_t slots = (t256 + 255) / 256 * 256;
         const bool full85 = t256 * 100 >= slots * 85, full70 = t256 * 10 >= slots * 7;
         if (!big_ok) return small;
-        if (k64) return full85 || (nn && K >= 2048 && full70) ? D256x256w8db : small;
+        if (k64) return full85 || (nn && K >= 2048 && full70) ? (nt && K >= 2048 ? D256x256k64 : D256x256w8db) : small;
         return full70 || K >= 1536 ? D256x256w8db : small;
     }
-    if (big_ok && t2128 > 256) return D256x256w8db;
+    if (big_ok && t2128 > 256) return k64 && nt && K >= 2048 ? D256x256k64 : D256x256w8db;
     if (M >= 256 && t2128 > 136) return mid;
     return small;
 }
