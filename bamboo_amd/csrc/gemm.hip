@@ -947,7 +947,7 @@ static DmaTile pick_dma_tile(int M, int N, int K, int64_t batches, int layout) {
     //  - Operands whose rows are k-contiguous (both of NT, A of NN) load faster as 64-wide k-tiles: one
     //    DMA instruction then covers 8 whole 128-byte lines instead of 16 half lines.  The smaller the
     //    tile, the more of its time is loading and the more that buys (128x128: up to +19 %, 256x128:
-    //    +3..8 %, 256x256: +4 % for long K only, its two 64 KB stages cost prologue time).
+    //    +3..8 %, 256x256: +4 % at long K, and +2 % on the whole stage with the K = 1024 FFN product on it).
     //  - Above one round of 256x256 tiles they win while the last round is well filled; otherwise the
     //    small tiles, several blocks per CU, smooth the tail.
     //  - Within one round: 256x256 once 256x128 tiles would need a second round, 256x128 from about half
@@ -963,10 +963,10 @@ static DmaTile pick_dma_tile(int M, int N, int K, int64_t batches, int layout) {
         const int64_t slots = (t256 + 255) / 256 * 256;
         const bool full85 = t256 * 100 >= slots * 85, full70 = t256 * 10 >= slots * 7;
         if (!big_ok) return small;
-        if (k64) return full85 || (nn && K >= 2048 && full70) ? (nt && K >= 2048 ? D256x256k64 : D256x256w8db) : small;
+        if (k64) return full85 || (nn && K >= 2048 && full70) ? (nt ? D256x256k64 : D256x256w8db) : small;
         return full70 || K >= 1536 ? D256x256w8db : small;
     }
-    if (big_ok && t2128 > 256) return k64 && nt && K >= 2048 ? D256x256k64 : D256x256w8db;
+    if (big_ok && t2128 > 256) return k64 && nt ? D256x256k64 : D256x256w8db;
     if (M >= 256 && t2128 > 136) return mid;
     return small;
 }
