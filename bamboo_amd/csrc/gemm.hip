@@ -949,13 +949,16 @@ static DmaTile pick_dma_tile(int M, int N, int K, int64_t batches, int layout) {
     //    tile, the more of its time is loading and the more that buys (128x128: up to +19 %, 256x128:
     //    +3..8 %, 256x256: +4 % at long K, and +2 % on the whole stage with the K = 1024 FFN product on it).
     //  - Above one round of 256x256 tiles they win while the last round is well filled; otherwise the
-    //    small tiles, several blocks per CU, smooth the tail.
+    //    small tiles, several blocks per CU, smooth the tail.  Where the sweep (outputs that stay in the
+    //    last-level cache) and the stage itself (outputs that go to HBM) disagree, the stage decides: it
+    //    wants the 256x256 tile from a 70 % full last round on for NT, and three stages for every 256x128
+    //    problem.
     //  - Within one round: 256x256 once 256x128 tiles would need a second round, 256x128 from about half
     //    a round on, and 128x128 tiles for anything smaller.
     const bool nt = layout == BB_NT, nn = layout == BB_NN;
     const bool k64 = (nt || nn) && K % 64 == 0 && K >= 128;
     const DmaTile small = k64 && (nt || K >= 2048) ? D128x128k64 : D128x128s3;
-    const DmaTile mid = !k64 ? D256x128w8db : (nt && K < 2048) ? D256x128k64 : D256x128k64s3;
+    const DmaTile mid = !k64 ? D256x128w8db : D256x128k64s3;
     const int64_t t256 = (int64_t)((M + 255) / 256) * ((N + 255) / 256) * batches;
     const int64_t t2128 = (int64_t)((M + 255) / 256) * ((N + 127) / 128) * batches;
     const bool big_ok = M >= 256 && N >= 256;
@@ -963,7 +966,7 @@ static DmaTile pick_dma_tile(int M, int N, int K, int64_t batches, int layout) {
         const int64_t slots = (t256 + 255) / 256 * 256;
         const bool full85 = t256 * 100 >= slots * 85, full70 = t256 * 10 >= slots * 7;
         if (!big_ok) return small;
-        if (k64) return full85 || (nn && K >= 2048 && full70) ? (nt ? D256x256k64 : D256x256w8db) : small;
+        if (k64) return (nt ? full70 : full85 || (K >= 2048 && full70)) ? (nt ? D256x256k64 : D256x256w8db) : small;
         return full70 || K >= 1536 ? D256x256w8db : small;
     }
     if (big_ok && t2128 > 256) return k64 && nt ? D256x256k64 : D256x256w8db;
