@@ -429,9 +429,9 @@ template <int BM, int BN, int WM, int WN, bool AKM, bool BKM, bool DB, int STAGE
 __device__ __forceinline__ void gemm_bf16_dma_body(const GemmArgs& g, const int block_id, const int batch_id,
                                                    const bool logical_id = false) {
     constexpr int NW = WM * WN;
-    static_assert(BK == 64 ? ((STAGES == 2 || STAGES == 3) && DB) : STAGES >= 3,
+    static_assert(BK == 64 ? (STAGES >= 2 && DB) : STAGES >= 3,
                   "32-wide k-tiles: the ring needs one stage being read, one landing, one in flight; "
-                  "64-wide k-tiles alternate between two stages or rotate through three");
+                  "64-wide k-tiles alternate between two stages or rotate through more");
     constexpr int WTM = BM / WM, WTN = BN / WN, TM = WTM / 32, TN = WTN / 32;
     using OpA = DmaOperand<BM, AKM, NW, BK>;
     using OpB = DmaOperand<BN, BKM, NW, BK>;
@@ -589,12 +589,16 @@ __device__ __forceinline__ void gemm_bf16_dma_body(const GemmArgs& g, const int 
             }
         };
         constexpr int FRAG_READS = 2 * (TM * (AKM ? 2 : 1) + TN * (BKM ? 2 : 1));
-        stop_at_end(1);
-        issue_tile();
-        stop_at_end(2);
-        issue_tile();
+        // prologue: tiles 0 and 1 with two stages, 0..STAGES-2 with more (tile kt+STAGES-1 then goes out
+        // at the top of iteration kt, into the stage tile kt-1 has left)
+        constexpr int PRO = STAGES == 2 ? 2 : STAGES - 1;
+#pragma unroll
+        for (int t = 0; t < PRO; ++t) {
+            stop_at_end(t + 1);
+            issue_tile();
+        }
         asm volatile("" ::: "memory");
-        wait_vmcnt_lgkm0<LOADS>();
+        wait_vmcnt_lgkm0<(PRO - 1) * LOADS>();
         __builtin_amdgcn_s_barrier();
         asm volatile("" ::: "memory");
         load_half(f0, smem, 0);
@@ -603,9 +607,8 @@ __device__ __forceinline__ void gemm_bf16_dma_body(const GemmArgs& g, const int 
             const unsigned char* cur = smem + rs * STAGE_BYTES;
             rs = rs + 1 == STAGES ? 0 : rs + 1;
             const unsigned char* nxt = smem + rs * STAGE_BYTES;
-            if constexpr (STAGES == 3) {
-                // a third stage lets tile kt+2 start a whole tile earlier: its stage held tile kt-1
-                stop_at_end(kt + 3);
+            if constexpr (STAGES >= 3) {
+                stop_at_end(kt + STAGES);
                 issue_tile();
             }
             load_half(f1, cur, 1);
@@ -924,11 +927,12 @@ static int launch_bf16_dma(GemmArgs& g, int batches, hipStream_t st) {
 
 // DMA kernels need K % 32 == 0 and at least one full vector of rows; tile by problem size
 enum DmaTile { D_NONE = 0, D256x256, D256x128, D128x128, D_OFF, D256x256w8, D256x128w8, D256x256w8db, D256x128w8db,
-               D256x128w8s3, D128x128s3, D256x256w8s5, D256x128w8s6, D256x256w8s3, D256x128w4s3, D256x256k64, D256x128k64, D256x128k64s3, D128x128k64 };
+               D256x128w8s3, D128x128s3, D256x256w8s5, D256x128w8s6, D256x256w8s3, D256x128w4s3, D256x256k64, D256x128k64, D256x128k64s3, D128x128k64, D128x64k64s3, D128x64s3, D64x128k64s3, D64x128s3 };
 static const char* const kDmaTileNames[] = {"", "dma256x256", "dma256x128", "dma128x128", "", "dma256x256w8", "dma256x128w8",
                                             "dma256x256w8db", "dma256x128w8db", "dma256x128w8s3", "dma128x128s3",
                                             "dma256x256w8s5", "dma256x128w8s6", "dma256x256w8s3", "dma256x128w4s3", "dma256x256k64",
-                                            "dma256x128k64", "dma256x128k64s3", "dma128x128k64"};
+                                            "dma256x128k64", "dma256x128k64s3", "dma128x128k64", "dma128x64k64s3",
+                                            "dma128x64s3", "dma64x128k64s3", "dma64x128s3"};
 // BB_DMA_TILE (tuning aid): 1..3 force a DMA tile where it is legal, 4 disables the DMA kernels.
 static int dma_tile_override() {
     static const int v = [] {
@@ -942,6 +946,9 @@ static DmaTile pick_dma_tile(int M, int N, int K, int64_t batches, int layout) {
     const int ov = dma_tile_override();
     if (ov == 4) return D_NONE;
     if ((ov >= 1 && ov <= 3) || (ov >= 5 && ov <= 14) || (ov >= 15 && ov <= 18 && K % 64 == 0 && K >= 128)) return (DmaTile)ov;
+    // 19..22: the narrow tiles, where their k-major operand is 128 wide (NT: 128x64, NN: 64x128)
+    if (ov == 19 || ov == 20) return layout == BB_NT ? (ov == 19 && K % 64 == 0 && K >= 128 ? D128x64k64s3 : D128x64s3) : D_NONE;
+    if (ov == 21 || ov == 22) return layout == BB_NN ? (ov == 21 && K % 64 == 0 && K >= 128 ? D64x128k64s3 : D64x128s3) : D_NONE;
     // Rules read off sweeps of M 2048..16384 x N 768..6400 x K 1024/4096 (NT and NN) on MI355X (256 CUs,
     // one block of the 256-row tiles per CU).
     //  - Operands whose rows are k-contiguous (both of NT, A of NN) load faster as 64-wide k-tiles: one
@@ -961,7 +968,14 @@ static DmaTile pick_dma_tile(int M, int N, int K, int64_t batches, int layout) {
     const DmaTile mid = !k64 ? D256x128w8db : D256x128k64s3;
     const int64_t t256 = (int64_t)((M + 255) / 256) * ((N + 255) / 256) * batches;
     const int64_t t2128 = (int64_t)((M + 255) / 256) * ((N + 127) / 128) * batches;
+    const int64_t t128 = (int64_t)((M + 127) / 128) * ((N + 127) / 128) * batches;
     const bool big_ok = M >= 256 && N >= 256;
+    //  - Problems with so few 128x128 tiles that half the CUs would idle (the 256-channel convolutions of a
+    //    ResNet stage: 98 tiles) take 128x64 tiles: twice the blocks.
+    //    (a k-major operand needs 128 rows for its swizzle, so NT narrows N and NN narrows M; TN keeps
+    //    128x128).
+    if (t128 <= 128 && nt) return k64 ? D128x64k64s3 : D128x64s3;
+    if (t128 <= 128 && nn) return k64 ? D64x128k64s3 : D64x128s3;
     if (t256 > 256) {
         const int64_t slots = (t256 + 255) / 256 * 256;
         const bool full85 = t256 * 100 >= slots * 85, full70 = t256 * 10 >= slots * 7;
@@ -993,6 +1007,10 @@ template <bool TA, bool TB> static int dispatch_bf16(GemmArgs& g, int batches, h
         case D256x128k64: return launch_bf16_dma<256, 128, 4, 2, TA, TB, true, 2, 64>(g, batches, st);
         case D256x128k64s3: return launch_bf16_dma<256, 128, 4, 2, TA, TB, true, 3, 64>(g, batches, st);
         case D128x128k64: return launch_bf16_dma<128, 128, 2, 2, TA, TB, true, 2, 64>(g, batches, st);
+        case D128x64k64s3: return launch_bf16_dma<128, 64, 4, 1, TA, TB, true, 3, 64>(g, batches, st);
+        case D128x64s3: return launch_bf16_dma<128, 64, 4, 1, TA, TB, true, 3>(g, batches, st);
+        case D64x128k64s3: return launch_bf16_dma<64, 128, 2, 2, TA, TB, true, 3, 64>(g, batches, st);
+        case D64x128s3: return launch_bf16_dma<64, 128, 2, 2, TA, TB, true, 3>(g, batches, st);
         default: break;
     }
     switch (pick_bf16_tile(g.M, g.N, batches)) {
