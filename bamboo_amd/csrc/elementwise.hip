@@ -737,40 +737,45 @@ extern "C" int bb_mse_fwd_bwd(int dtype, int64_t n, const void* y, const void* t
 // (DeepSpeedExamples/pipeline_parallelism/resnet.py:49-75).
 // =========================================================================================
 constexpr int BN_SPLITS = 64;
+constexpr int BN_WAVES = 16;  // row streams per block; with 64 splits 1024 waves share the rows
 
-// column partial sums of f(x): MODE 0: x ; MODE 1: (x - mean[c])^2 ;
-// MODE 2 (backward): two sums, g and g * xhat, with g = dy * (out > 0 if relu_out given)
+// Column partial sums, two per channel, over the rows of one split:
+// MODE 0 (forward statistics in one pass): sum (x - p) and sum (x - p)^2 with the pivot p = row 0 of x
+//   (mean = p + S1/n, var = S2/n - (S1/n)^2: shifted by a sample of the data the subtraction does not
+//   cancel, unlike sum x^2 - n mean^2);
+// MODE 2 (backward): sum g and sum g * xhat, with g = dy * (out > 0 if relu_out given).
+// Waves take rows wave, wave + BN_WAVES * splits, ... of their split; fixed order everywhere.
 template <typename T, int MODE>
-__global__ __launch_bounds__(256) void bn_colred_kernel(int rows, int cols, const T* __restrict__ x,
+__global__ __launch_bounds__(BN_WAVES * 64) void bn_colred_kernel(int rows, int cols, const T* __restrict__ x,
                                                         const float* __restrict__ mean, const float* __restrict__ rstd,
                                                         const T* __restrict__ dy, const T* __restrict__ relu_out,
                                                         float* __restrict__ partial) {
     constexpr int VEC = Elem<T>::VEC;
-    __shared__ float red[3][2][64 * VEC];
+    constexpr int SLOTS = 5;   // the cross-wave sum goes through LDS five waves at a time
+    __shared__ float red[SLOTS][2][64 * VEC];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int c0 = (blockIdx.x * 64 + lane) * VEC;
     float a0[VEC], a1[VEC], mu[VEC], rs[VEC];
 #pragma unroll
     for (int e = 0; e < VEC; ++e) a0[e] = a1[e] = mu[e] = rs[e] = 0.f;
     if (c0 < cols) {
-        if (MODE >= 1) {
+        if (MODE == 0) {
+            load_vec(x + c0, mu);   // the pivot
+        } else {
 #pragma unroll
-            for (int e = 0; e < VEC; ++e) mu[e] = mean[c0 + e];
-        }
-        if (MODE == 2) {
-#pragma unroll
-            for (int e = 0; e < VEC; ++e) rs[e] = rstd[c0 + e];
+            for (int e = 0; e < VEC; ++e) {
+                mu[e] = mean[c0 + e];
+                rs[e] = rstd[c0 + e];
+            }
         }
         // rows r0, r0 + step, ... in that order; four rows' loads are issued before their sums
         auto add_row = [&](const float (&v)[VEC], const float (&g)[VEC]) {
             if (MODE == 0) {
 #pragma unroll
-                for (int e = 0; e < VEC; ++e) a0[e] += v[e];
-            } else if (MODE == 1) {
-#pragma unroll
                 for (int e = 0; e < VEC; ++e) {
                     const float d = v[e] - mu[e];
-                    a0[e] += d * d;
+                    a0[e] += d;
+                    a1[e] += d * d;
                 }
             } else {
 #pragma unroll
@@ -792,8 +797,8 @@ __global__ __launch_bounds__(256) void bn_colred_kernel(int rows, int cols, cons
                 }
             }
         };
-        const int step = gridDim.y * 4;
-        int r = blockIdx.y * 4 + wave;
+        const int step = gridDim.y * BN_WAVES;
+        int r = blockIdx.y * BN_WAVES + wave;
         for (; r + 3 * step < rows; r += 4 * step) {
             float v[4][VEC], g[4][VEC];
 #pragma unroll
@@ -807,33 +812,44 @@ __global__ __launch_bounds__(256) void bn_colred_kernel(int rows, int cols, cons
             add_row(v, g);
         }
     }
-    if (wave > 0) {
+    // wave 0 + 1 + 2 + ... in that order, SLOTS waves per round through LDS
+    for (int w0 = 1; w0 < BN_WAVES; w0 += SLOTS) {
+        if (wave >= w0 && wave < w0 + SLOTS) {
 #pragma unroll
-        for (int e = 0; e < VEC; ++e) {
-            red[wave - 1][0][lane * VEC + e] = a0[e];
-            red[wave - 1][1][lane * VEC + e] = a1[e];
+            for (int e = 0; e < VEC; ++e) {
+                red[wave - w0][0][lane * VEC + e] = a0[e];
+                red[wave - w0][1][lane * VEC + e] = a1[e];
+            }
         }
+        __syncthreads();
+        if (wave == 0) {
+            const int n = min(SLOTS, BN_WAVES - w0);
+            for (int w = 0; w < n; ++w) {
+#pragma unroll
+                for (int e = 0; e < VEC; ++e) {
+                    a0[e] += red[w][0][lane * VEC + e];
+                    a1[e] += red[w][1][lane * VEC + e];
+                }
+            }
+        }
+        __syncthreads();
     }
-    __syncthreads();
     if (wave == 0 && c0 < cols) {
 #pragma unroll
         for (int e = 0; e < VEC; ++e) {
-            float s0 = a0[e], s1 = a1[e];
-            for (int w = 0; w < 3; ++w) {
-                s0 += red[w][0][lane * VEC + e];
-                s1 += red[w][1][lane * VEC + e];
-            }
-            partial[((int64_t)blockIdx.y * 2) * cols + c0 + e] = s0;
-            partial[((int64_t)blockIdx.y * 2 + 1) * cols + c0 + e] = s1;
+            partial[((int64_t)blockIdx.y * 2) * cols + c0 + e] = a0[e];
+            partial[((int64_t)blockIdx.y * 2 + 1) * cols + c0 + e] = a1[e];
         }
     }
 }
 
 // finish: sums over the BN_SPLITS partial rows in fixed order.
-// what 0: mean = s0/rows ; 1: rstd = 1/sqrt(s0/rows + eps) (+ running stats) ; 2: dbeta += s0, dgamma += s1,
-// and keep the batch means of g and g*xhat for the apply pass
+// what 1 (forward): mean = p + S1/n, var = S2/n - (S1/n)^2, rstd = 1/sqrt(var + eps) (+ running stats);
+// what 2 (backward): dbeta += s0, dgamma += s1, and the batch means of g and g*xhat for the apply pass
+template <typename T>
 __global__ __launch_bounds__(64) void bn_finish_kernel(int what, int rows, int cols, float eps, float momentum,
-                                                        const float* __restrict__ partial, float* __restrict__ mean,
+                                                        const float* __restrict__ partial, const T* __restrict__ x,
+                                                        float* __restrict__ mean,
                                                         float* __restrict__ rstd, float* __restrict__ run_mean,
                                                         float* __restrict__ run_var, float* __restrict__ dgamma,
                                                         float* __restrict__ dbeta, float* __restrict__ sums) {
@@ -845,7 +861,7 @@ __global__ __launch_bounds__(64) void bn_finish_kernel(int what, int rows, int c
 #pragma unroll
         for (int j = 0; j < 8; ++j) {
             t0[j] = partial[((int64_t)(p0 + j) * 2) * cols + c];
-            t1[j] = what == 2 ? partial[((int64_t)(p0 + j) * 2 + 1) * cols + c] : 0.f;
+            t1[j] = partial[((int64_t)(p0 + j) * 2 + 1) * cols + c];
         }
 #pragma unroll
         for (int j = 0; j < 8; ++j) {
@@ -853,13 +869,14 @@ __global__ __launch_bounds__(64) void bn_finish_kernel(int what, int rows, int c
             s1 += t1[j];
         }
     }
-    if (what == 0) {
-        mean[c] = s0 / (float)rows;
-    } else if (what == 1) {
-        const float var = s0 / (float)rows;
+    if (what == 1) {
+        const float d = s0 / (float)rows;
+        const float m = Elem<T>::load(x + c) + d;
+        const float var = fmaxf(s1 / (float)rows - d * d, 0.f);
+        mean[c] = m;
         rstd[c] = 1.0f / sqrtf(var + eps);
         if (run_mean) {  // nn.BatchNorm2d: running_var uses the unbiased estimate
-            run_mean[c] = (1.f - momentum) * run_mean[c] + momentum * mean[c];
+            run_mean[c] = (1.f - momentum) * run_mean[c] + momentum * m;
             run_var[c] = (1.f - momentum) * run_var[c] + momentum * var * (float)rows / (float)(rows - 1);
         }
     } else {
@@ -979,17 +996,14 @@ extern "C" int bb_batchnorm_fwd(int dtype, int rows, int cols, float eps, float 
     const int vec = dtype == BB_BF16 ? 8 : 4;
     dim3 grid((cols + 64 * vec - 1) / (64 * vec), BN_SPLITS), fgrid((cols + 63) / 64);
     const int64_t nvec = (int64_t)rows * cols / vec;
+    const dim3 block(BN_WAVES * 64);
     if (dtype == BB_BF16) {
-        hipLaunchKernelGGL((bn_colred_kernel<bf16, 0>), grid, dim3(256), 0, st, rows, cols, (const bf16*)x, nullptr, nullptr, nullptr, nullptr, workspace);
-        hipLaunchKernelGGL(bn_finish_kernel, fgrid, dim3(64), 0, st, 0, rows, cols, eps, momentum, workspace, mean, rstd, nullptr, nullptr, nullptr, nullptr, nullptr);
-        hipLaunchKernelGGL((bn_colred_kernel<bf16, 1>), grid, dim3(256), 0, st, rows, cols, (const bf16*)x, mean, nullptr, nullptr, nullptr, workspace);
-        hipLaunchKernelGGL(bn_finish_kernel, fgrid, dim3(64), 0, st, 1, rows, cols, eps, momentum, workspace, mean, rstd, running_mean, running_var, nullptr, nullptr, nullptr);
+        hipLaunchKernelGGL((bn_colred_kernel<bf16, 0>), grid, block, 0, st, rows, cols, (const bf16*)x, nullptr, nullptr, nullptr, nullptr, workspace);
+        hipLaunchKernelGGL(bn_finish_kernel<bf16>, fgrid, dim3(64), 0, st, 1, rows, cols, eps, momentum, workspace, (const bf16*)x, mean, rstd, running_mean, running_var, nullptr, nullptr, nullptr);
         hipLaunchKernelGGL(bn_apply_kernel<bf16>, dim3(grid_for(nvec)), dim3(256), 0, st, nvec, cols, relu, (const bf16*)x, mean, rstd, (const bf16*)gamma, (const bf16*)beta, (const bf16*)resid, (bf16*)y);
     } else {
-        hipLaunchKernelGGL((bn_colred_kernel<float, 0>), grid, dim3(256), 0, st, rows, cols, (const float*)x, nullptr, nullptr, nullptr, nullptr, workspace);
-        hipLaunchKernelGGL(bn_finish_kernel, fgrid, dim3(64), 0, st, 0, rows, cols, eps, momentum, workspace, mean, rstd, nullptr, nullptr, nullptr, nullptr, nullptr);
-        hipLaunchKernelGGL((bn_colred_kernel<float, 1>), grid, dim3(256), 0, st, rows, cols, (const float*)x, mean, nullptr, nullptr, nullptr, workspace);
-        hipLaunchKernelGGL(bn_finish_kernel, fgrid, dim3(64), 0, st, 1, rows, cols, eps, momentum, workspace, mean, rstd, running_mean, running_var, nullptr, nullptr, nullptr);
+        hipLaunchKernelGGL((bn_colred_kernel<float, 0>), grid, block, 0, st, rows, cols, (const float*)x, nullptr, nullptr, nullptr, nullptr, workspace);
+        hipLaunchKernelGGL(bn_finish_kernel<float>, fgrid, dim3(64), 0, st, 1, rows, cols, eps, momentum, workspace, (const float*)x, mean, rstd, running_mean, running_var, nullptr, nullptr, nullptr);
         hipLaunchKernelGGL(bn_apply_kernel<float>, dim3(grid_for(nvec)), dim3(256), 0, st, nvec, cols, relu, (const float*)x, mean, rstd, (const float*)gamma, (const float*)beta, (const float*)resid, (float*)y);
     }
     BB_LAUNCH_CHECK();
@@ -1007,13 +1021,14 @@ extern "C" int bb_batchnorm_bwd(int dtype, int rows, int cols, const void* x, co
     dim3 grid((cols + 64 * vec - 1) / (64 * vec), BN_SPLITS), fgrid((cols + 63) / 64);
     const int64_t nvec = (int64_t)rows * cols / vec;
     float* sums = workspace + (int64_t)BN_SPLITS * 2 * cols;
+    const dim3 block(BN_WAVES * 64);
     if (dtype == BB_BF16) {
-        hipLaunchKernelGGL((bn_colred_kernel<bf16, 2>), grid, dim3(256), 0, st, rows, cols, (const bf16*)x, mean, rstd, (const bf16*)dy, (const bf16*)relu_out, workspace);
-        hipLaunchKernelGGL(bn_finish_kernel, fgrid, dim3(64), 0, st, 2, rows, cols, 0.f, 0.f, workspace, nullptr, nullptr, nullptr, nullptr, dgamma, dbeta, sums);
+        hipLaunchKernelGGL((bn_colred_kernel<bf16, 2>), grid, block, 0, st, rows, cols, (const bf16*)x, mean, rstd, (const bf16*)dy, (const bf16*)relu_out, workspace);
+        hipLaunchKernelGGL(bn_finish_kernel<bf16>, fgrid, dim3(64), 0, st, 2, rows, cols, 0.f, 0.f, workspace, (const bf16*)x, nullptr, nullptr, nullptr, nullptr, dgamma, dbeta, sums);
         hipLaunchKernelGGL(bn_bwd_apply_kernel<bf16>, dim3(grid_for(nvec)), dim3(256), 0, st, nvec, cols, (const bf16*)x, mean, rstd, (const bf16*)gamma, sums, (const bf16*)dy, (const bf16*)relu_out, (bf16*)dx, (bf16*)g_out);
     } else {
-        hipLaunchKernelGGL((bn_colred_kernel<float, 2>), grid, dim3(256), 0, st, rows, cols, (const float*)x, mean, rstd, (const float*)dy, (const float*)relu_out, workspace);
-        hipLaunchKernelGGL(bn_finish_kernel, fgrid, dim3(64), 0, st, 2, rows, cols, 0.f, 0.f, workspace, nullptr, nullptr, nullptr, nullptr, dgamma, dbeta, sums);
+        hipLaunchKernelGGL((bn_colred_kernel<float, 2>), grid, block, 0, st, rows, cols, (const float*)x, mean, rstd, (const float*)dy, (const float*)relu_out, workspace);
+        hipLaunchKernelGGL(bn_finish_kernel<float>, fgrid, dim3(64), 0, st, 2, rows, cols, 0.f, 0.f, workspace, (const float*)x, nullptr, nullptr, nullptr, nullptr, dgamma, dbeta, sums);
         hipLaunchKernelGGL(bn_bwd_apply_kernel<float>, dim3(grid_for(nvec)), dim3(256), 0, st, nvec, cols, (const float*)x, mean, rstd, (const float*)gamma, sums, (const float*)dy, (const float*)relu_out, (float*)dx, (float*)g_out);
     }
     BB_LAUNCH_CHECK();

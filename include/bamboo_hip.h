@@ -188,7 +188,7 @@ int bb_residual_add(int dtype, int64_t n, const void* a, const void* b, void* ou
 int bb_act_fwd(int dtype, int act, int64_t n, const void* x, void* out, void* dact, void* stream);
 
 /* BatchNorm2d in training mode on an NHWC activation viewed as [rows = N*H*W, cols = channels]
- * (resnet.py:56,59,62): per-channel batch mean and biased variance (two passes), then
+ * (resnet.py:56,59,62): per-channel batch mean and biased variance (one pass, sums shifted by row 0), then
  * y = gamma * (x - mean) * rstd + beta (+ resid) with optional ReLU (the block's final
  * ReLU(residual_function(x) + shortcut(x)), resnet.py:75).  mean / rstd: fp32 [cols], kept for the
  * backward.  running_mean / running_var (both or neither; may be NULL for a redundant forward,
