@@ -847,27 +847,41 @@ __global__ __launch_bounds__(BN_WAVES * 64) void bn_colred_kernel(int rows, int 
 // what 1 (forward): mean = p + S1/n, var = S2/n - (S1/n)^2, rstd = 1/sqrt(var + eps) (+ running stats);
 // what 2 (backward): dbeta += s0, dgamma += s1, and the batch means of g and g*xhat for the apply pass
 template <typename T>
-__global__ __launch_bounds__(64) void bn_finish_kernel(int what, int rows, int cols, float eps, float momentum,
+__global__ __launch_bounds__(256) void bn_finish_kernel(int what, int rows, int cols, float eps, float momentum,
                                                         const float* __restrict__ partial, const T* __restrict__ x,
                                                         float* __restrict__ mean,
                                                         float* __restrict__ rstd, float* __restrict__ run_mean,
                                                         float* __restrict__ run_var, float* __restrict__ dgamma,
                                                         float* __restrict__ dbeta, float* __restrict__ sums) {
-    const int c = blockIdx.x * 64 + threadIdx.x;
-    if (c >= cols) return;
+    // 32 channels per block, 8 threads per channel: each takes eight consecutive partial rows (one round
+    // of loads), the eight sums are added in row order through LDS
+    static_assert(BN_SPLITS == 64, "eight row groups of eight");
+    __shared__ float red[7][2][32];
+    const int col = threadIdx.x & 31, rg = threadIdx.x >> 5;
+    const int c = blockIdx.x * 32 + col;
     float s0 = 0.f, s1 = 0.f;
-    for (int p0 = 0; p0 < BN_SPLITS; p0 += 8) {  // eight rows' loads in flight, summed in row order
+    if (c < cols) {
         float t0[8], t1[8];
 #pragma unroll
         for (int j = 0; j < 8; ++j) {
-            t0[j] = partial[((int64_t)(p0 + j) * 2) * cols + c];
-            t1[j] = partial[((int64_t)(p0 + j) * 2 + 1) * cols + c];
+            t0[j] = partial[((int64_t)(rg * 8 + j) * 2) * cols + c];
+            t1[j] = partial[((int64_t)(rg * 8 + j) * 2 + 1) * cols + c];
         }
 #pragma unroll
         for (int j = 0; j < 8; ++j) {
             s0 += t0[j];
             s1 += t1[j];
         }
+    }
+    if (rg > 0) {
+        red[rg - 1][0][col] = s0;
+        red[rg - 1][1][col] = s1;
+    }
+    __syncthreads();
+    if (rg > 0 || c >= cols) return;
+    for (int q = 0; q < 7; ++q) {
+        s0 += red[q][0][col];
+        s1 += red[q][1][col];
     }
     if (what == 1) {
         const float d = s0 / (float)rows;
@@ -994,16 +1008,16 @@ extern "C" int bb_batchnorm_fwd(int dtype, int rows, int cols, float eps, float 
     BB_REQUIRE((running_mean == nullptr) == (running_var == nullptr), "bb_batchnorm_fwd: give both running buffers or none");
     hipStream_t st = (hipStream_t)stream;
     const int vec = dtype == BB_BF16 ? 8 : 4;
-    dim3 grid((cols + 64 * vec - 1) / (64 * vec), BN_SPLITS), fgrid((cols + 63) / 64);
+    dim3 grid((cols + 64 * vec - 1) / (64 * vec), BN_SPLITS), fgrid((cols + 31) / 32);
     const int64_t nvec = (int64_t)rows * cols / vec;
     const dim3 block(BN_WAVES * 64);
     if (dtype == BB_BF16) {
         hipLaunchKernelGGL((bn_colred_kernel<bf16, 0>), grid, block, 0, st, rows, cols, (const bf16*)x, nullptr, nullptr, nullptr, nullptr, workspace);
-        hipLaunchKernelGGL(bn_finish_kernel<bf16>, fgrid, dim3(64), 0, st, 1, rows, cols, eps, momentum, workspace, (const bf16*)x, mean, rstd, running_mean, running_var, nullptr, nullptr, nullptr);
+        hipLaunchKernelGGL(bn_finish_kernel<bf16>, fgrid, dim3(256), 0, st, 1, rows, cols, eps, momentum, workspace, (const bf16*)x, mean, rstd, running_mean, running_var, nullptr, nullptr, nullptr);
         hipLaunchKernelGGL(bn_apply_kernel<bf16>, dim3(grid_for(nvec)), dim3(256), 0, st, nvec, cols, relu, (const bf16*)x, mean, rstd, (const bf16*)gamma, (const bf16*)beta, (const bf16*)resid, (bf16*)y);
     } else {
         hipLaunchKernelGGL((bn_colred_kernel<float, 0>), grid, block, 0, st, rows, cols, (const float*)x, nullptr, nullptr, nullptr, nullptr, workspace);
-        hipLaunchKernelGGL(bn_finish_kernel<float>, fgrid, dim3(64), 0, st, 1, rows, cols, eps, momentum, workspace, (const float*)x, mean, rstd, running_mean, running_var, nullptr, nullptr, nullptr);
+        hipLaunchKernelGGL(bn_finish_kernel<float>, fgrid, dim3(256), 0, st, 1, rows, cols, eps, momentum, workspace, (const float*)x, mean, rstd, running_mean, running_var, nullptr, nullptr, nullptr);
         hipLaunchKernelGGL(bn_apply_kernel<float>, dim3(grid_for(nvec)), dim3(256), 0, st, nvec, cols, relu, (const float*)x, mean, rstd, (const float*)gamma, (const float*)beta, (const float*)resid, (float*)y);
     }
     BB_LAUNCH_CHECK();
@@ -1018,17 +1032,17 @@ extern "C" int bb_batchnorm_bwd(int dtype, int rows, int cols, const void* x, co
     BB_REQUIRE(x && gamma && mean && rstd && dy && dx && dgamma && dbeta && workspace, "bb_batchnorm_bwd: null pointer");
     hipStream_t st = (hipStream_t)stream;
     const int vec = dtype == BB_BF16 ? 8 : 4;
-    dim3 grid((cols + 64 * vec - 1) / (64 * vec), BN_SPLITS), fgrid((cols + 63) / 64);
+    dim3 grid((cols + 64 * vec - 1) / (64 * vec), BN_SPLITS), fgrid((cols + 31) / 32);
     const int64_t nvec = (int64_t)rows * cols / vec;
     float* sums = workspace + (int64_t)BN_SPLITS * 2 * cols;
     const dim3 block(BN_WAVES * 64);
     if (dtype == BB_BF16) {
         hipLaunchKernelGGL((bn_colred_kernel<bf16, 2>), grid, block, 0, st, rows, cols, (const bf16*)x, mean, rstd, (const bf16*)dy, (const bf16*)relu_out, workspace);
-        hipLaunchKernelGGL(bn_finish_kernel<bf16>, fgrid, dim3(64), 0, st, 2, rows, cols, 0.f, 0.f, workspace, (const bf16*)x, nullptr, nullptr, nullptr, nullptr, dgamma, dbeta, sums);
+        hipLaunchKernelGGL(bn_finish_kernel<bf16>, fgrid, dim3(256), 0, st, 2, rows, cols, 0.f, 0.f, workspace, (const bf16*)x, nullptr, nullptr, nullptr, nullptr, dgamma, dbeta, sums);
         hipLaunchKernelGGL(bn_bwd_apply_kernel<bf16>, dim3(grid_for(nvec)), dim3(256), 0, st, nvec, cols, (const bf16*)x, mean, rstd, (const bf16*)gamma, sums, (const bf16*)dy, (const bf16*)relu_out, (bf16*)dx, (bf16*)g_out);
     } else {
         hipLaunchKernelGGL((bn_colred_kernel<float, 2>), grid, block, 0, st, rows, cols, (const float*)x, mean, rstd, (const float*)dy, (const float*)relu_out, workspace);
-        hipLaunchKernelGGL(bn_finish_kernel<float>, fgrid, dim3(64), 0, st, 2, rows, cols, 0.f, 0.f, workspace, (const float*)x, nullptr, nullptr, nullptr, nullptr, dgamma, dbeta, sums);
+        hipLaunchKernelGGL(bn_finish_kernel<float>, fgrid, dim3(256), 0, st, 2, rows, cols, 0.f, 0.f, workspace, (const float*)x, nullptr, nullptr, nullptr, nullptr, dgamma, dbeta, sums);
         hipLaunchKernelGGL(bn_bwd_apply_kernel<float>, dim3(grid_for(nvec)), dim3(256), 0, st, nvec, cols, (const float*)x, mean, rstd, (const float*)gamma, sums, (const float*)dy, (const float*)relu_out, (float*)dx, (float*)g_out);
     }
     BB_LAUNCH_CHECK();
