@@ -315,9 +315,10 @@ def test_lazy_recovery_failover(hiplib, dead_from):
     assert abs(float(loss) - float(peer.loss) / M) < 1e-4 * max(1.0, float(peer.loss) / M)
 
 
+@pytest.mark.parametrize("ckpt", [0, 1], ids=["full-stash", "checkpointed"])
 @pytest.mark.parametrize("rc_stream", [False, True], ids=["one-stream", "rc-stream"])
 @pytest.mark.parametrize("variant,klr", [(GPT_VARIANT, None), (BERT_VARIANT, (5, 64))], ids=["gpt", "bert"])
-def test_graph_replay_equals_eager(hiplib, variant, klr, rc_stream):
+def test_graph_replay_equals_eager(hiplib, variant, klr, rc_stream, ckpt):
     """Forward / backward launch sequences replayed as HIP graphs: five batches with optimizer steps
     (eager work and synchronisation between the replays), loss after every batch and the weights at
     the end bit-equal to an engine that launches every kernel itself.  Batch 1 runs eagerly, batch 2
@@ -325,7 +326,7 @@ def test_graph_replay_equals_eager(hiplib, variant, klr, rc_stream):
     hid, heads, ffn, L, S, sid, mb, M, seq = 128, 2, 256, 2, 4, 1, 2, 4, 64
     dtype = torch.bfloat16
     eager_engine, _ = build(hid, heads, ffn, L, S, sid, mb, M, seq, dtype, variant, 1, True, grad_mode="mse",
-                            rc_stream=rc_stream, key_len_range=klr)
+                            rc_stream=rc_stream, key_len_range=klr, checkpoint_interval=ckpt)
     ref_losses = []
     for _ in range(5):
         ref_losses.append(float(eager_engine.train_batch()))
@@ -337,7 +338,7 @@ def test_graph_replay_equals_eager(hiplib, variant, klr, rc_stream):
             with torch.cuda.stream(pass_default):
                 build(hid, heads, ffn, L, S, sid, mb, M, seq, dtype, variant, 1, True, grad_mode="mse", use_graphs=True)
         engine, _ = build(hid, heads, ffn, L, S, sid, mb, M, seq, dtype, variant, 1, True, grad_mode="mse",
-                          rc_stream=rc_stream, key_len_range=klr, use_graphs=True)
+                          rc_stream=rc_stream, key_len_range=klr, use_graphs=True, checkpoint_interval=ckpt)
         torch.cuda.synchronize()
         losses = []
         for _ in range(5):
