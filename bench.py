@@ -249,18 +249,15 @@ def main():
     # no other stream shares the GPU, so the durations are the kernels' own
     engine, q = build_engine(cfg, rc=True, rc_stream=False)
     probe = None
-    for _ in range(args.warmup):
-        engine.train_batch()
-    torch.cuda.synchronize()
+    t_on_serial = time_steps(engine, args.steps, args.warmup)      # the leg's own rate, no event brackets
     if not args.no_probe:
+        # the same steps again with every GEMM launch bracketed (costs ~10 % of the rate: not what is reported)
         probe = GemmProbe()
         hip.gemm_hook = probe
-    t0 = time.perf_counter()
-    for _ in range(args.steps):
-        engine.train_batch()
-    torch.cuda.synchronize()
-    t_on_serial = (time.perf_counter() - t0) / args.steps
-    hip.gemm_hook = None
+        for _ in range(args.steps):
+            engine.train_batch()
+        torch.cuda.synchronize()
+        hip.gemm_hook = None
     t_on = t_on_serial
 
     # leg 3 (default): RC on with the redundant forwards on a second HIP stream; this is the
@@ -310,8 +307,8 @@ def main():
         roofline = {"bound": "mfma", "achieved": round(achieved, 2), "peak": peak, "unit": "TFLOP/s",
                     "frac": round(achieved / peak, 4),
                     "traffic": MEASURED_TRAFFIC_BYTES.get((args.config, f"gemm_{name}")), "kernel": f"gemm_{name}",
-                    "measured_in": "timed steps of the RC-on single-stream leg, HIP events around each launch on its "
-                                   "stream, minus the reading of an empty event bracket",
+                    "measured_in": "a repeat of the timed steps of the RC-on single-stream leg with HIP events around "
+                                   "each GEMM launch on its stream, minus the reading of an empty event bracket",
                     "event_bracket_overhead_us": round(overhead_s * 1e6, 2),
                     "launches": count, "avg_launch_us": round(secs / count * 1e6, 2),
                     "avg_launch_gflop": round(flops / count / 1e9, 3),
