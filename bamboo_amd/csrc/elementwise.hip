@@ -650,6 +650,15 @@ __global__ __launch_bounds__(256) void cast_kernel(int64_t n, const S* __restric
     for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (int64_t)gridDim.x * 256)
         Elem<D>::store(dst + i, Elem<S>::load(src + i));
 }
+// same-type copy, 16 bytes per lane (pointers 16-byte aligned); the tail goes element by element
+template <typename T>
+__global__ __launch_bounds__(256) void copy_kernel(int64_t n, const T* __restrict__ src, T* __restrict__ dst) {
+    constexpr int V = 16 / sizeof(T);
+    const int64_t nv = n / V;
+    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < nv; i += (int64_t)gridDim.x * 256)
+        ((f32x4*)dst)[i] = ((const f32x4*)src)[i];
+    for (int64_t i = nv * V + (int64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (int64_t)gridDim.x * 256) dst[i] = src[i];
+}
 
 extern "C" int bb_cast(int src_dtype, int dst_dtype, int64_t n, const void* src, void* dst, void* stream) {
     BB_REQUIRE((src_dtype == BB_F32 || src_dtype == BB_BF16) && (dst_dtype == BB_F32 || dst_dtype == BB_BF16),
@@ -664,6 +673,8 @@ extern "C" int bb_cast(int src_dtype, int dst_dtype, int64_t n, const void* src,
         hipLaunchKernelGGL((cast_kernel<bf16, float>), grid, block, 0, st, n, (const bf16*)src, (float*)dst);
     else if (src_dtype == BB_F32)
         hipLaunchKernelGGL((cast_kernel<float, float>), grid, block, 0, st, n, (const float*)src, (float*)dst);
+    else if ((((uintptr_t)src | (uintptr_t)dst) & 15) == 0)
+        hipLaunchKernelGGL((copy_kernel<bf16>), dim3(grid_for(n / 8 + 1)), block, 0, st, n, (const bf16*)src, (bf16*)dst);
     else
         hipLaunchKernelGGL((cast_kernel<bf16, bf16>), grid, block, 0, st, n, (const bf16*)src, (bf16*)dst);
     BB_LAUNCH_CHECK();

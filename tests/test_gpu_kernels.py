@@ -485,3 +485,13 @@ def test_adam_rejects_bad_arguments(hiplib):
     with pytest.raises(hiplib.HipKernelError):
         hiplib.adam_multi([t], [t], [t], [t], None, lr=1e-3, beta1=0.9, beta2=0.999, eps=1e-8, step=0)
     hiplib.adam_multi([], [], [], [], None, lr=1e-3, beta1=0.9, beta2=0.999, eps=1e-8, step=1)  # empty list is fine
+
+def test_same_type_copy(hiplib):
+    """cast with equal types is a copy: 16 bytes per lane when both pointers allow it, with a scalar tail,
+    element by element otherwise; the bytes beyond the range stay untouched."""
+    for n, off in ((8 * 1000 + 3, 0), (8 * 1000 + 3, 1), (5, 0), (1 << 20, 0)):
+        src = randn(n + 16, dtype=torch.bfloat16, seed=91)
+        dst = torch.full((n + 16,), 7.0, dtype=torch.bfloat16, device=DEV)
+        hiplib.cast(src[off:off + n], dst[off:off + n])
+        assert torch.equal(dst[off:off + n], src[off:off + n])
+        assert torch.all(dst[off + n:] == 7.0) and torch.all(dst[:off] == 7.0)
