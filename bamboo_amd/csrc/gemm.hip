@@ -711,22 +711,26 @@ __device__ __forceinline__ void gemm_bf16_dma_body(const GemmArgs& g, const int 
     // private [32][64 (+4 pad)] fp32 patch; then one wave instruction covers 8 rows x 64 columns, lane l
     // taking 8 consecutive columns of row l/8, so every global load / store of the epilogue moves whole
     // 128-byte row segments (256 bytes for fp32 outputs).
-    static_assert(TN % 2 == 0, "the epilogue walks the accumulator tiles in pairs");
+    // An odd tile count per row ends with a single tile: its 32 columns use half of the patch and half of
+    // the lanes of the row pass.
     wait_vmcnt_lgkm0<0>();  // the tiles issued past the end of K have to land before their stages become the patch
     __syncthreads();
     constexpr int PLD = 68;
+    constexpr int NP = (TN + 1) / 2;   // pairs per row of accumulator tiles, the last one possibly a single
     float* patch = (float*)smem + wave * (32 * PLD);
     const int prow = lane >> 3, pcol = (lane & 7) * 8;
     static_for(
         [&](auto idx) {
-            constexpr int i = decltype(idx)::value / (TN / 2), jp = decltype(idx)::value % (TN / 2);
+            constexpr int i = decltype(idx)::value / NP, jp = decltype(idx)::value % NP;
+            constexpr int NH = (jp * 2 + 1 < TN) ? 2 : 1;
 #pragma unroll
-            for (int h = 0; h < 2; ++h)
+            for (int h = 0; h < NH; ++h)
 #pragma unroll
                 for (int r = 0; r < 16; ++r)
                     patch[(8 * (r >> 2) + 4 * (lane >> 5) + (r & 3)) * PLD + h * 32 + (lane & 31)] = acc[i][jp * 2 + h][r] * g.alpha;
             asm volatile("" ::: "memory");
             const int n = n0 + wn * WTN + jp * 64 + pcol;
+            const bool live = NH == 2 || pcol < 32;
 #pragma unroll
             for (int it = 0; it < 4; ++it) {
                 const int m = m0 + wm * WTM + i * 32 + it * 8 + prow;
@@ -738,11 +742,11 @@ __device__ __forceinline__ void gemm_bf16_dma_body(const GemmArgs& g, const int 
                     v[e] = lo[e];
                     v[4 + e] = hi[e];
                 }
-                if (m < g.M && n < g.N) epilogue_vec8(g, coff, m, n, v);
+                if (live && m < g.M && n < g.N) epilogue_vec8(g, coff, m, n, v);
             }
             asm volatile("" ::: "memory");
         },
-        std::make_integer_sequence<int, TM * TN / 2>{});
+        std::make_integer_sequence<int, TM * NP>{});
 }
 
 template <int BM, int BN, int WM, int WN, bool AKM, bool BKM, bool DB, int STAGES, int BK>
@@ -927,12 +931,12 @@ static int launch_bf16_dma(GemmArgs& g, int batches, hipStream_t st) {
 
 // DMA kernels need K % 32 == 0 and at least one full vector of rows; tile by problem size
 enum DmaTile { D_NONE = 0, D256x256, D256x128, D128x128, D_OFF, D256x256w8, D256x128w8, D256x256w8db, D256x128w8db,
-               D256x128w8s3, D128x128s3, D256x256w8s5, D256x128w8s6, D256x256w8s3, D256x128w4s3, D256x256k64, D256x128k64, D256x128k64s3, D128x128k64, D128x64k64s3, D128x64s3, D64x128k64s3, D64x128s3 };
+               D256x128w8s3, D128x128s3, D256x256w8s5, D256x128w8s6, D256x256w8s3, D256x128w4s3, D256x256k64, D256x128k64, D256x128k64s3, D128x128k64, D128x64k64s3, D128x64s3, D64x128k64s3, D64x128s3, D256x192k64 };
 static const char* const kDmaTileNames[] = {"", "dma256x256", "dma256x128", "dma128x128", "", "dma256x256w8", "dma256x128w8",
                                             "dma256x256w8db", "dma256x128w8db", "dma256x128w8s3", "dma128x128s3",
                                             "dma256x256w8s5", "dma256x128w8s6", "dma256x256w8s3", "dma256x128w4s3", "dma256x256k64",
                                             "dma256x128k64", "dma256x128k64s3", "dma128x128k64", "dma128x64k64s3",
-                                            "dma128x64s3", "dma64x128k64s3", "dma64x128s3"};
+                                            "dma128x64s3", "dma64x128k64s3", "dma64x128s3", "dma256x192k64"};
 // BB_DMA_TILE (tuning aid): 1..3 force a DMA tile where it is legal, 4 disables the DMA kernels.
 static int dma_tile_override() {
     static const int v = [] {
@@ -946,6 +950,7 @@ static DmaTile pick_dma_tile(int M, int N, int K, int64_t batches, int layout) {
     const int ov = dma_tile_override();
     if (ov == 4) return D_NONE;
     if ((ov >= 1 && ov <= 3) || (ov >= 5 && ov <= 14) || (ov >= 15 && ov <= 18 && K % 64 == 0 && K >= 128)) return (DmaTile)ov;
+    if (ov == 23) return layout == BB_NT && K % 64 == 0 && K >= 128 ? D256x192k64 : D_NONE;
     // 19..22: the narrow tiles, where their k-major operand is 128 wide (NT: 128x64, NN: 64x128)
     if (ov == 19 || ov == 20) return layout == BB_NT ? (ov == 19 && K % 64 == 0 && K >= 128 ? D128x64k64s3 : D128x64s3) : D_NONE;
     if (ov == 21 || ov == 22) return layout == BB_NN ? (ov == 21 && K % 64 == 0 && K >= 128 ? D64x128k64s3 : D64x128s3) : D_NONE;
@@ -976,6 +981,19 @@ static DmaTile pick_dma_tile(int M, int N, int K, int64_t batches, int layout) {
     //    128x128).
     if (t128 <= 128 && nt) return k64 ? D128x64k64s3 : D128x64s3;
     if (t128 <= 128 && nn) return k64 ? D64x128k64s3 : D64x128s3;
+    //  - NT problems whose 256x256 tiles would fill under 70 % of their rounds may take 256x192 tiles (six
+    //    accumulator tiles per wave, about 9 % below the 256x256 tile at equal fill) instead of falling back
+    //    to 128x128: compared by the share of the occupied tile slots that is real output.  (Alone, the QKV
+    //    projection 8192x3072 - 1.5 rounds of 256x256 tiles, exactly two of 256x192 - is 19 % faster on them;
+    //    inside the power-limited stage the whole batch is 1 % slower, so 75 % full rounds stay on 256x256.)
+    if (nt && k64 && big_ok && t2128 > 256) {
+        auto useful = [&](int bn) {   // real output / output slots of whole rounds
+            const int64_t t = (int64_t)((M + 255) / 256) * ((N + bn - 1) / bn) * batches;
+            return (double)M * N * batches / ((double)((t + 255) / 256 * 256) * 256 * bn);
+        };
+        const double s256 = useful(256), s192 = 0.91 * useful(192);
+        if (s256 < 0.70 && s192 > s256 && s192 >= 0.65) return D256x192k64;
+    }
     if (t256 > 256) {
         const int64_t slots = (t256 + 255) / 256 * 256;
         const bool full85 = t256 * 100 >= slots * 85, full70 = t256 * 10 >= slots * 7;
@@ -1011,6 +1029,10 @@ template <bool TA, bool TB> static int dispatch_bf16(GemmArgs& g, int batches, h
         case D128x64s3: return launch_bf16_dma<128, 64, 4, 1, TA, TB, true, 3>(g, batches, st);
         case D64x128k64s3: return launch_bf16_dma<64, 128, 2, 2, TA, TB, true, 3, 64>(g, batches, st);
         case D64x128s3: return launch_bf16_dma<64, 128, 2, 2, TA, TB, true, 3>(g, batches, st);
+        case D256x192k64:
+            // k-contiguous operands only (192 rows do not divide into the k-major loader's instructions)
+            if constexpr (!TA && !TB) return launch_bf16_dma<256, 192, 4, 2, TA, TB, true, 2, 64>(g, batches, st);
+            else break;
         default: break;
     }
     switch (pick_bf16_tile(g.M, g.N, batches)) {

@@ -35,7 +35,9 @@ def randn(*shape, dtype=torch.float32, seed=0, scale=1.0):
 GEMM_SHAPES = [(256, 256, 64), (512, 384, 128), (304, 200, 96), (64, 1024, 256), (1024, 64, 512),
                (136, 72, 40), (2048, 768, 768), (8, 8, 8),
                # ragged edges under the 256x128 tiles with 64-wide k-tiles (two and three stages)
-               (4000, 1496, 1024), (2104, 2000, 2048), (4000, 1496, 128)]
+               (4000, 1496, 1024), (2104, 2000, 2048), (4000, 1496, 128),
+               # NT: 256x192 tiles (three accumulator tiles across a wave: the epilogue's single-tile tail)
+               (4000, 4792, 192)]
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
