@@ -111,6 +111,19 @@ __device__ __forceinline__ float dgelu_tanh_f(float x) {
     const float dz2 = 2.0f * k0 * (1.0f + 3.0f * k1 * x * x);
     return s + x * s * (1.0f - s) * dz2;
 }
+// act(x) and act'(x) together (one sigmoid for both)
+__device__ __forceinline__ void act_dact_f(float x, int kind, float& a, float& d) {
+    if (kind == BB_ACT_RELU) {
+        a = fmaxf(x, 0.0f);
+        d = x > 0.0f ? 1.0f : 0.0f;
+    } else {
+        const float k0 = 0.7978845608028654f, k1 = 0.044715f;
+        const float s = sigmoid2z_f(x);
+        const float dz2 = 2.0f * k0 * (1.0f + 3.0f * k1 * x * x);
+        a = x * s;
+        d = s + x * s * (1.0f - s) * dz2;
+    }
+}
 __device__ __forceinline__ float act_f(float x, int kind) {
     return kind == BB_ACT_RELU ? fmaxf(x, 0.0f) : gelu_tanh_f(x);
 }

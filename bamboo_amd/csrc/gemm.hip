@@ -67,6 +67,11 @@ __device__ __forceinline__ void epilogue_elem(const GemmArgs& g, int64_t coff, i
         v += Elem<T>::load((const T*)g.resid + xi);
     } else if (g.epilogue == BB_EPI_MUL) {
         v *= Elem<T>::load((const T*)g.aux_in + xi);
+    } else if (g.epilogue == BB_EPI_ACT_DACT) {
+        float a, d;
+        act_dact_f(v, g.act, a, d);
+        Elem<T>::store((T*)g.aux_out + xi, d);
+        v = a;
     }
     if (g.c_f32) {
         float* c = (float*)g.C + ci;
@@ -105,6 +110,11 @@ __device__ __forceinline__ void epilogue_vec8(const GemmArgs& g, int64_t coff, i
         load_vec((const bf16*)g.aux_in + xi, d);
 #pragma unroll
         for (int e = 0; e < 8; ++e) v[e] *= d[e];
+    } else if (g.epilogue == BB_EPI_ACT_DACT) {
+        float d[8];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) act_dact_f(v[e], g.act, v[e], d[e]);
+        store_vec((bf16*)g.aux_out + xi, d);
     }
     if (g.c_f32) {
         float* c = (float*)g.C + ci;
@@ -1080,7 +1090,7 @@ static int fill_args(const bb_gemm_desc* d, GemmArgs& g, int64_t& batches, bool&
     BB_REQUIRE(d->layout >= BB_NT && d->layout <= BB_TN, "bb_gemm: bad layout %d", d->layout);
     BB_REQUIRE(d->M >= 0 && d->N >= 0 && d->K >= 0, "bb_gemm: negative dimension");
     BB_REQUIRE(!d->accumulate || d->c_dtype == BB_F32, "bb_gemm: accumulate needs an fp32 C");
-    BB_REQUIRE(d->epilogue >= BB_EPI_NONE && d->epilogue <= BB_EPI_MUL, "bb_gemm: bad epilogue");
+    BB_REQUIRE(d->epilogue >= BB_EPI_NONE && d->epilogue <= BB_EPI_ACT_DACT, "bb_gemm: bad epilogue");
     const int nb1 = d->nb1 > 0 ? d->nb1 : 1, nb2 = d->nb2 > 0 ? d->nb2 : 1;
     batches = (int64_t)nb1 * nb2;
     ta = d->layout == BB_TN;
@@ -1090,6 +1100,7 @@ static int fill_args(const bb_gemm_desc* d, GemmArgs& g, int64_t& batches, bool&
     BB_REQUIRE(d->A && d->B && d->C, "bb_gemm: null operand");
     BB_REQUIRE((d->epilogue != BB_EPI_DACT && d->epilogue != BB_EPI_MUL) || d->aux_in, "bb_gemm: DACT/MUL epilogue needs aux_in");
     BB_REQUIRE(d->epilogue != BB_EPI_RESIDUAL || d->resid, "bb_gemm: RESIDUAL epilogue needs resid");
+    BB_REQUIRE(d->epilogue != BB_EPI_ACT_DACT || d->aux_out, "bb_gemm: ACT_DACT epilogue needs aux_out");
     BB_REQUIRE(batches <= 65535, "bb_gemm: too many batches (%lld)", (long long)batches);
     const int vec = d->dtype == BB_BF16 ? 8 : 4;
     // the contiguous dimension of every operand is read in 16-byte vectors

@@ -149,7 +149,7 @@ class TransformerLayer:
         return [
             ("n1", (R, h), dt), ("qkv", (R, 3 * h), dt), attn,
             ("ctx", (R, h), dt), ("x1", (R, h), dt), ("n2", (R, h), dt),
-            ("u", (R, f), dt), ("act", (R, f), dt), ("out", (R, h), dt),
+            ("dact", (R, f), dt), ("act", (R, f), dt), ("out", (R, h), dt),
             ("mean1", (R,), f32), ("rinv1", (R,), f32), ("mean2", (R,), f32), ("rinv2", (R,), f32),
         ]
 
@@ -235,11 +235,12 @@ class TransformerLayer:
                  epilogue=hip.EPI_RESIDUAL, resid=x, stream=sm)
         hip.layernorm_fwd(st["x1"], w["sublayer.1.norm.a_2"], w["sublayer.1.norm.b_2"], st["n2"], st["mean2"],
                           st["rinv2"], kind, self.eps, stream=sm)
-        # pre-activation (kept for act') and activation both leave the GEMM epilogue: on the power-limited
-        # stage the saved pass over u (read 64 MB, write 64 MB at the GPT-2-medium shapes) outweighs the
-        # epilogue's transcendental work (measured inside the stage, not on the kernel alone)
+        # activation and its derivative (kept for the backward pass, which then multiplies instead of
+        # evaluating act') both leave the GEMM epilogue: on the power-limited stage the saved pass over the
+        # pre-activation (read 64 MB, write 64 MB at the GPT-2-medium shapes) outweighs the epilogue's
+        # transcendental work (measured inside the stage, not on the kernel alone)
         hip.gemm(hip.NT, st["n2"], w["feed_forward.w_1.weight"], st["act"], bias=w["feed_forward.w_1.bias"],
-                 epilogue=hip.EPI_ACT, act=act, aux_out=st["u"], stream=sm)
+                 epilogue=hip.EPI_ACT_DACT, act=act, aux_out=st["dact"], stream=sm)
         hip.gemm(hip.NT, st["act"], w["feed_forward.w_2.weight"], st["out"], bias=w["feed_forward.w_2.bias"],
                  epilogue=hip.EPI_RESIDUAL, resid=st["x1"], stream=sm)
         return st["out"]
@@ -260,8 +261,7 @@ class TransformerLayer:
             hip.TN, dy, x, g[name], accumulate=True, colsum_out=g[name[:-len("weight")] + "bias"], colsum_ws=ws))
         # feed-forward
         wgrad(d_out, st["act"], "feed_forward.w_2.weight")
-        hip.gemm(hip.NN, d_out, w["feed_forward.w_2.weight"], d_ffn, epilogue=hip.EPI_DACT, act=act,
-                 aux_in=st["u"], stream=sm)
+        hip.gemm(hip.NN, d_out, w["feed_forward.w_2.weight"], d_ffn, epilogue=hip.EPI_MUL, aux_in=st["dact"], stream=sm)
         wgrad(d_ffn, st["n2"], "feed_forward.w_1.weight")
         hip.gemm(hip.NN, d_ffn, w["feed_forward.w_1.weight"], d_h0, stream=sm)
         # d_x1 = d_out + LN2'(d_n2)

@@ -50,13 +50,16 @@ extern "C" {
  *   BB_EPI_ACT       aux_out = v (if aux_out != NULL);  C = act(v)
  *   BB_EPI_DACT      C = v * act'(aux_in[m,n])
  *   BB_EPI_RESIDUAL  C = v + resid[m,n]
- *   BB_EPI_MUL       C = v * aux_in[m,n]  (e.g. aux_in = act'(u) kept by bb_act_fwd)
+ *   BB_EPI_MUL       C = v * aux_in[m,n]  (e.g. aux_in = act'(u) kept by BB_EPI_ACT_DACT or bb_act_fwd)
+ *   BB_EPI_ACT_DACT  aux_out = act'(v);  C = act(v)   (forward of an FFN whose backward then needs no
+ *                    transcendental: its input gradient is a BB_EPI_MUL product with aux_out)
  * `accumulate` != 0 adds the result to the existing contents of C (C must be fp32).       */
 #define BB_EPI_NONE 0
 #define BB_EPI_ACT 1
 #define BB_EPI_DACT 2
 #define BB_EPI_RESIDUAL 3
 #define BB_EPI_MUL 4
+#define BB_EPI_ACT_DACT 5
 
 #define BB_ACT_RELU 0
 #define BB_ACT_GELU_TANH 1

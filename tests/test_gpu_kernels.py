@@ -80,6 +80,17 @@ def test_gemm_epilogues(hiplib, dtype):
         ol.activation(Uf, name).sum().backward()
         hiplib.gemm(hiplib.NT, A, W, C, epilogue=hiplib.EPI_DACT, act=act, aux_in=U)
         assert rel_err(C, (Af @ Wf.t()) * Uf.grad) < tol(dtype)
+        # act and act' from one epilogue: C = act(v), aux_out = act'(v) (from the unrounded v)
+        D = torch.empty_like(C)
+        hiplib.gemm(hiplib.NT, A, W, C, bias=bias, epilogue=hiplib.EPI_ACT_DACT, act=act, aux_out=D)
+        lf = lin.clone().requires_grad_(True)
+        ol.activation(lf, name).sum().backward()
+        assert rel_err(C, ol.activation(lin, name)) < tol(dtype)
+        if name == "relu":   # a step function: compare away from the step
+            far = lin.abs() > 1e-2
+            assert torch.equal(D.double().cpu()[far], lf.grad[far])
+        else:
+            assert rel_err(D, lf.grad) < tol(dtype)
     # mul: C = (A W^T) * R
     hiplib.gemm(hiplib.NT, A, W, C, epilogue=hiplib.EPI_MUL, aux_in=R)
     assert rel_err(C, (Af @ Wf.t()) * Rf) < tol(dtype)
