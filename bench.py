@@ -44,8 +44,9 @@ PEAK_BF16_TFLOPS, PEAK_F32_TFLOPS = 2500.0, 157.3
 # counters cannot be read from inside this process, so the figure is carried here per
 # (config, kernel) and is null for anything that was not profiled.
 MEASURED_TRAFFIC_BYTES = {
-    ("c2", "gemm_bf16_nt_dma256x256k64"): int((47551.3 * 2.0 + 57344.0) * 1024),
-    ("c2", "gemm_grouped_bf16_tn"): int((368936.1 * 2.0 + 49188.6) * 1024),
+    ("c2", "gemm_grouped_bf16_tn"): int((239928.6 * 2.0 + 49188.4) * 1024),
+    ("c2", "gemm_bf16_nt_dma256x256k64+act_dact"): int((49965.8 * 2.0 + 131072.0) * 1024),
+    ("c2", "gemm_bf16_nt_dma256x256k64"): int((45853.1 * 2.0 + 49152.0) * 1024),
 }
 
 
@@ -103,6 +104,9 @@ class GemmProbe:
             shape = "+".join(f"{d.M}x{d.N}x{d.K}" for d in desc)
         else:
             name, flops = hip.gemm_variant(desc), 2.0 * desc.M * desc.N * desc.K
+            # an epilogue that evaluates the activation is a different code path with work of its own
+            # (two transcendental-heavy outputs for act_dact): its launches are listed apart
+            name += {hip.EPI_ACT: "+act", hip.EPI_DACT: "+dact", hip.EPI_ACT_DACT: "+act_dact"}.get(desc.epilogue, "")
             shape = f"{desc.M}x{desc.N}x{desc.K}"
         e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         stream = stream if stream is not None else torch.cuda.current_stream()
