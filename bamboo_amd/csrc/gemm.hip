@@ -1014,7 +1014,15 @@ static DmaTile pick_dma_tile(int M, int N, int K, int64_t batches, int layout) {
         const int64_t slots = (t256 + 255) / 256 * 256;
         const bool full85 = t256 * 100 >= slots * 85, full70 = t256 * 10 >= slots * 7;
         if (!big_ok) return small;
-        if (k64) return (nt ? full70 : full85 || (K >= 2048 && full70)) ? (nt ? D256x256k64 : D256x256w8db) : small;
+        if (k64 && nt) {
+            // a last round under 85 %: 256x128 tiles if those come out in whole rounds (the QKV projection
+            // 8192x3072: 1.5 rounds of 256x256, exactly three of 256x128; +1 % on the stage)
+            const int64_t slots2 = (t2128 + 255) / 256 * 256;
+            if (full85) return D256x256k64;
+            if (t2128 * 10 >= slots2 * 9) return mid;
+            return full70 ? D256x256k64 : small;
+        }
+        if (k64) return full85 || (K >= 2048 && full70) ? D256x256w8db : small;
         return full70 || K >= 1536 ? D256x256w8db : small;
     }
     if (big_ok && t2128 > 256) return k64 && nt ? D256x256k64 : D256x256w8db;
