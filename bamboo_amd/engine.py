@@ -115,6 +115,7 @@ class PipelineEngine:
         for sid in built:
             self.stash_bytes += model.allocate_stash(sid, self.ctx, self.micro_batches)
         self._fwd_done = [torch.cuda.Event() for _ in range(self.micro_batches)]
+        self._deferred = {}   # (stage, slot) -> the slot's last forward left backward-only outputs out
 
         act_shape = (self.batch * self.seq, self.queue.shape[2])
         self._input_grad_store = {
@@ -468,7 +469,11 @@ class PipelineEngine:
             self.rc_stream.wait_event(self._fwd_done[buffer_id])
         kl = ctx.key_len
         key = ("F", stage_id, buffer_id, id(ctx), inputs.data_ptr(), None if kl is None else kl.data_ptr())
-        out = self._graphed(key, ctx.stream, lambda: self.module.forward(inputs, stage_id, slot=buffer_id, ctx=ctx))
+        # a redundant forward's stash is read by a backward pass only after a failover: it leaves out
+        # what that backward pass can produce itself
+        self._deferred[(stage_id, buffer_id)] = redundant
+        out = self._graphed(key, ctx.stream, lambda: self.module.forward(inputs, stage_id, slot=buffer_id, ctx=ctx,
+                                                                         defer=redundant))
         self.pipe_buffers[out_key][buffer_id] = out
         if not redundant and self.rc_stream is not None:
             self._fwd_done[buffer_id].record(self.main_stream)
@@ -485,8 +490,11 @@ class PipelineEngine:
         self.ctx.key_len = self.queue.key_len(buffer_id)
         dst = self._input_grad_store[stage_id][buffer_id]
         kl = self.ctx.key_len
-        key = ("B", stage_id, buffer_id, id(self.ctx), grad.data_ptr(), dst.data_ptr(), None if kl is None else kl.data_ptr())
-        self._graphed(key, self.ctx.stream, lambda: self.module.backward(grad, dst, stage_id, slot=buffer_id, ctx=self.ctx))
+        deferred = self._deferred.get((stage_id, buffer_id), False)
+        key = ("B", stage_id, buffer_id, id(self.ctx), grad.data_ptr(), dst.data_ptr(),
+               None if kl is None else kl.data_ptr(), deferred)
+        self._graphed(key, self.ctx.stream, lambda: self.module.backward(grad, dst, stage_id, slot=buffer_id, ctx=self.ctx,
+                                                                         deferred=deferred))
         key = f"input_grad_{stage_id}"
         if key in self.pipe_buffers:
             self.pipe_buffers[key][buffer_id] = dst

@@ -34,6 +34,10 @@ class StageContext:
         self.key_len = None
         self.workspace = None
         self.redundant = False   # set per forward call: a redundant forward must not touch running statistics
+        # set per forward call: leave out what only a backward pass reads (a redundant forward's stash is used
+        # by a backward pass only after a failover); ``deferred`` tells that backward pass to produce it first
+        self.defer = False
+        self.deferred = False
 
     @property
     def rows(self):
@@ -239,11 +243,20 @@ class TransformerLayer:
         # evaluating act') both leave the GEMM epilogue: on the power-limited stage the saved pass over the
         # pre-activation (read 64 MB, write 64 MB at the GPT-2-medium shapes) outweighs the epilogue's
         # transcendental work (measured inside the stage, not on the kernel alone)
-        hip.gemm(hip.NT, st["n2"], w["feed_forward.w_1.weight"], st["act"], bias=w["feed_forward.w_1.bias"],
-                 epilogue=hip.EPI_ACT_DACT, act=act, aux_out=st["dact"], stream=sm)
+        if ctx.defer:
+            # act' is read by the backward pass only: a forward that most likely has none writes act alone
+            hip.gemm(hip.NT, st["n2"], w["feed_forward.w_1.weight"], st["act"], bias=w["feed_forward.w_1.bias"],
+                     epilogue=hip.EPI_ACT, act=act, stream=sm)
+        else:
+            self._ffn1(st, sm)
         hip.gemm(hip.NT, st["act"], w["feed_forward.w_2.weight"], st["out"], bias=w["feed_forward.w_2.bias"],
                  epilogue=hip.EPI_RESIDUAL, resid=st["x1"], stream=sm)
         return st["out"]
+
+    def _ffn1(self, st, sm):
+        w = self.w
+        hip.gemm(hip.NT, st["n2"], w["feed_forward.w_1.weight"], st["act"], bias=w["feed_forward.w_1.bias"],
+                 epilogue=hip.EPI_ACT_DACT, act=hip.ACT_CODES[self.activation], aux_out=st["dact"], stream=sm)
 
     def backward(self, d_out, d_x, st, ctx):
         """d_out: gradient of st['out']; writes the input gradient into d_x; parameter
@@ -259,6 +272,8 @@ class TransformerLayer:
         # ... and each carries its bias gradient (column sums of dy) in the same kernel
         wgrad = lambda dy, x, name: wgrads.append(hip.gemm_desc(
             hip.TN, dy, x, g[name], accumulate=True, colsum_out=g[name[:-len("weight")] + "bias"], colsum_ws=ws))
+        if ctx.deferred:
+            self._ffn1(st, sm)   # the forward of this stash left act' out: same kernel, same bits as a normal forward
         # feed-forward
         wgrad(d_out, st["act"], "feed_forward.w_2.weight")
         hip.gemm(hip.NN, d_out, w["feed_forward.w_2.weight"], d_ffn, epilogue=hip.EPI_MUL, aux_in=st["dact"], stream=sm)

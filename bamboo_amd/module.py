@@ -362,7 +362,9 @@ class PipelineModule:
         return nbytes_total
 
     # ------------------------------------------------------------------ execution
-    def forward(self, forward_input, stage_id, slot=0, ctx=None):
+    def forward(self, forward_input, stage_id, slot=0, ctx=None, defer=False):
+        """``defer``: leave out of the stash what only a backward pass reads and this forward can
+        produce later from what it does keep (``backward(..., deferred=True)`` then produces it first)."""
         layers = self.func_buckets.get(stage_id)
         if layers is None:
             raise Exception(f"Unregistered stage id {stage_id}")
@@ -370,8 +372,10 @@ class PipelineModule:
         x = forward_input
         stash = self._stash[stage_id][slot]
         if self.activation_checkpoint_interval == 0:
+            ctx.defer = defer
             for layer, st in zip(layers, stash):
                 x = layer.forward(x, st, ctx)
+            ctx.defer = False
             return x
         kept = self._kept[stage_id][slot]
         for g, (a, b) in enumerate(self._checkpoint_groups(stage_id)):
@@ -382,11 +386,12 @@ class PipelineModule:
         hip.cast(x, kept[-1], stream=ctx.stream)
         return kept[-1]
 
-    def backward(self, grad_output, grad_input, stage_id, slot=0, ctx=None):
+    def backward(self, grad_output, grad_input, stage_id, slot=0, ctx=None, deferred=False):
         """Back-propagate through the layers of ``stage_id`` from the stash of ``slot``; parameter
         gradients accumulate in the stage's fp32 gradient arena, the input gradient is written to
-        ``grad_input``."""
+        ``grad_input``.  ``deferred``: the stash was written by ``forward(..., defer=True)``."""
         layers = self.func_buckets[stage_id]
+        ctx.deferred = deferred and self.activation_checkpoint_interval == 0
         stash = self._stash[stage_id][slot]
         n = len(layers)
         d = grad_output
@@ -405,6 +410,7 @@ class PipelineModule:
                 dst = grad_input if i == 0 else ctx.buf(f"d_layer{i % 2}", tuple(grad_output.shape))
                 layers[i].backward(d, dst, stash[i], ctx)
                 d = dst
+        ctx.deferred = False
         return grad_input
 
     def prepare_context(self, stage_ids, batch, seq, stream=None, forward_only=False):

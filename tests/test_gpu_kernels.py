@@ -91,6 +91,11 @@ def test_gemm_epilogues(hiplib, dtype):
             assert torch.equal(D.double().cpu()[far], lf.grad[far])
         else:
             assert rel_err(D, lf.grad) < tol(dtype)
+        # a redundant forward writes act alone and the backward after a failover runs ACT_DACT over the
+        # same operands: both must give the same act, bit for bit
+        C1 = torch.empty_like(C)
+        hiplib.gemm(hiplib.NT, A, W, C1, bias=bias, epilogue=hiplib.EPI_ACT, act=act)
+        assert torch.equal(C1, C)
     # mul: C = (A W^T) * R
     hiplib.gemm(hiplib.NT, A, W, C, epilogue=hiplib.EPI_MUL, aux_in=R)
     assert rel_err(C, (Af @ Wf.t()) * Rf) < tol(dtype)
