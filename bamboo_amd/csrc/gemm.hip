@@ -354,14 +354,38 @@ __device__ __forceinline__ void dma16(const void* src, const unsigned char* lds_
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(m0), "v"(src) : "m0");
 }
 
+// 3x3 convolution (stride 1, pad 1, NHWC) as an implicit GEMM: the patch matrix [pixels, 9 * channels] is never
+// built, the A loader gathers its rows from the activation tensor instead.
+struct ConvArgs {
+    int h, w, c;      // image height / width, channels of the gathered tensor (a multiple of the 64-wide k-tile)
+    int b_every;      // input-gradient mode: k-tiles per tap of the B operand ...
+    int64_t b_wrap;   // ... and what its pointers move by (on top of the k-tile step) when the tap changes
+};
+// what the taps outside the image read
+__device__ __attribute__((aligned(128))) unsigned char bb_zero_line[128];
+
 // VIS: issue through the compiler builtin instead (the compiler then sees the load and waits lgkmcnt(0)
 // for every fragment read, which keeps the waves of a block in lock step)
-template <int BR, bool KM, int NW, int BK = 32, bool VIS = false> struct DmaOperand {
+// CONV 1 (row-contiguous operand, 64-wide k-tiles): row p of the operand is pixel p's 3x3 neighbourhood,
+// k = tap * channels + channel; a k-tile lies inside one tap, so each lane reads 16 bytes of the neighbouring
+// pixel's channel vector, or of a line of zeros where the tap falls outside the image.
+// CONV 2 (k-major operand): the weight [out, 9, in] read as B[k = (8 - tap) * out + o, n = i] (the flipped
+// filter of the input gradient): rows o advance by the k-tile, and every out / 64 k-tiles the tap changes.
+template <int BR, bool KM, int NW, int BK = 32, bool VIS = false, int CONV = 0> struct DmaOperand {
     static constexpr int BYTES = BR * BK * 2;
     static constexpr int ROUNDS = BYTES / (1024 * NW);  // instructions per thread per k-tile
     static_assert(ROUNDS >= 1, "tile too small for the block");
+    static_assert(CONV == 0 || (CONV == 1 && !KM && BK == 64) || (CONV == 2 && KM), "convolution loaders: see above");
     const bf16* src[ROUNDS];
     int64_t step;  // elements to advance per k-tile
+    // CONV 1: per round the taps that lie inside the image (bit t = tap t), then wave-uniform position in K
+    unsigned inside[ROUNDS];
+    const bf16* zero;
+    int tap, c0, kstep, cw, cc;
+    int64_t tapoff;
+    // CONV 2
+    int cnt, every;
+    int64_t wrap;
 
     __device__ __forceinline__ void init(const bf16* base, int64_t ld, int row0, int rows, int tid) {
         const int lane = tid & 63, wave = tid >> 6;
@@ -389,17 +413,74 @@ template <int BR, bool KM, int NW, int BK = 32, bool VIS = false> struct DmaOper
         }
         step = KM ? BK * ld : BK;
     }
+    // CONV 1: base = the activation tensor [pixels, cv.c]; src[i] points at the lane's chunk of the centre pixel
+    __device__ __forceinline__ void init_conv(const bf16* base, int row0, int rows, int tid, const ConvArgs& cv) {
+        const int lane = tid & 63, wave = tid >> 6;
+#pragma unroll
+        for (int i = 0; i < ROUNDS; ++i) {
+            const int q = i * NW + wave;
+            const int r = q * 8 + (lane >> 3);
+            const int c = (lane & 7) ^ ((r >> 1) & 7);
+            const int gr = min(row0 + r, rows - 1);
+            const int pix = gr % (cv.h * cv.w), py = pix / cv.w, px = pix % cv.w;
+            unsigned m = 0;
+#pragma unroll
+            for (int t = 0; t < 9; ++t) {
+                const int sy = py + t / 3 - 1, sx = px + t % 3 - 1;
+                if (sy >= 0 && sy < cv.h && sx >= 0 && sx < cv.w) m |= 1u << t;
+            }
+            inside[i] = m;
+            src[i] = base + (int64_t)gr * cv.c + c * 8;
+        }
+        zero = (const bf16*)(bb_zero_line + (lane & 7) * 16);
+        step = 0;
+        tap = 0; c0 = 0; kstep = BK; cw = cv.w; cc = cv.c;
+        tapoff = (int64_t)(-cv.w - 1) * cv.c;
+    }
+    // CONV 2: after init() with base already at tap 8 of the weight
+    __device__ __forceinline__ void init_wrap(const ConvArgs& cv) {
+        cnt = 0; every = cv.b_every; wrap = cv.b_wrap;
+    }
+    // past the end of K: the last tile is fetched again and again
+    __device__ __forceinline__ void stop() {
+        step = 0;
+        if constexpr (CONV == 1) kstep = 0;
+        if constexpr (CONV == 2) wrap = 0;
+    }
+    __device__ __forceinline__ const bf16* source(int i) const {
+        if constexpr (CONV == 1) return ((inside[i] >> tap) & 1u) ? src[i] + (tapoff + c0) : zero;
+        else return src[i];
+    }
+    // after the last instruction of a k-tile
+    __device__ __forceinline__ void advance() {
+        if constexpr (CONV == 1) {
+            c0 += kstep;
+            if (c0 >= cc) {
+                c0 = 0;
+                ++tap;
+                tapoff = (int64_t)((tap / 3 - 1) * cw + (tap % 3 - 1)) * cc;
+            }
+        } else if constexpr (CONV == 2) {
+            if (++cnt == every) {
+                cnt = 0;
+#pragma unroll
+                for (int i = 0; i < ROUNDS; ++i) src[i] += wrap;
+            }
+        }
+    }
     __device__ __forceinline__ void issue(unsigned char* tile, int wave) {
 #pragma unroll
         for (int i = 0; i < ROUNDS; ++i) {
-            if constexpr (VIS) __builtin_amdgcn_global_load_lds((gbl_ptr_t*)src[i], (lds_ptr_t*)(tile + (i * NW + wave) * 1024), 16, 0, 0);
-            else dma16(src[i], tile + (i * NW + wave) * 1024);
+            if constexpr (VIS) __builtin_amdgcn_global_load_lds((gbl_ptr_t*)source(i), (lds_ptr_t*)(tile + (i * NW + wave) * 1024), 16, 0, 0);
+            else dma16(source(i), tile + (i * NW + wave) * 1024);
             src[i] += step;
         }
+        advance();
     }
     template <int I> __device__ __forceinline__ void issue_one(unsigned char* tile, int wave) {
-        dma16(src[I], tile + (I * NW + wave) * 1024);
+        dma16(source(I), tile + (I * NW + wave) * 1024);
         src[I] += step;
+        if constexpr (I == ROUNDS - 1) advance();
     }
 };
 
@@ -438,16 +519,18 @@ template <int BR, int T, bool KM, int BK = 32> struct FragReader {
     }
 };
 
-template <int BM, int BN, int WM, int WN, bool AKM, bool BKM, bool DB, int STAGES, int BK = 32, bool VIS = false>
+template <int BM, int BN, int WM, int WN, bool AKM, bool BKM, bool DB, int STAGES, int BK = 32, bool VIS = false, int CONV = 0>
 __device__ __forceinline__ void gemm_bf16_dma_body(const GemmArgs& g, const int block_id, const int batch_id,
-                                                   const bool logical_id = false) {
+                                                   const bool logical_id = false, const ConvArgs& cv = ConvArgs{}) {
     constexpr int NW = WM * WN;
     static_assert(BK == 64 ? (STAGES >= 2 && DB) : STAGES >= 3,
                   "32-wide k-tiles: the ring needs one stage being read, one landing, one in flight; "
                   "64-wide k-tiles alternate between two stages or rotate through more");
     constexpr int WTM = BM / WM, WTN = BN / WN, TM = WTM / 32, TN = WTN / 32;
-    using OpA = DmaOperand<BM, AKM, NW, BK, VIS>;
-    using OpB = DmaOperand<BN, BKM, NW, BK, VIS>;
+    // CONV 1: forward 3x3 convolution (A gathered); CONV 2: its input gradient (A gathered, B the flipped filter)
+    static_assert(CONV == 0 || (!AKM && (CONV == 2) == BKM), "implicit convolution: NT forward, NN input gradient");
+    using OpA = DmaOperand<BM, AKM, NW, BK, VIS, CONV ? 1 : 0>;
+    using OpB = DmaOperand<BN, BKM, NW, BK, VIS, CONV == 2 ? 2 : 0>;
     constexpr int STAGE_BYTES = OpA::BYTES + OpB::BYTES;
     constexpr int LOADS = OpA::ROUNDS + OpB::ROUNDS;
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
@@ -465,8 +548,10 @@ __device__ __forceinline__ void gemm_bf16_dma_body(const GemmArgs& g, const int 
 
     OpA opa;
     OpB opb;
-    opa.init(A, g.lda, m0, g.M, tid);
+    if constexpr (CONV != 0) opa.init_conv(A, m0, g.M, tid, cv);
+    else opa.init(A, g.lda, m0, g.M, tid);
     opb.init(B, g.ldb, n0, g.N, tid);
+    if constexpr (CONV == 2) opb.init_wrap(cv);
     FragReader<BM, TM, AKM, BK> fa;
     FragReader<BN, TN, BKM, BK> fb;
     fa.init(wm * WTM, lane);
@@ -582,8 +667,8 @@ __device__ __forceinline__ void gemm_bf16_dma_body(const GemmArgs& g, const int 
     };
     auto stop_at_end = [&](int next_tile) {
         if (next_tile >= KT) {
-            opa.step = 0;
-            opb.step = 0;
+            opa.stop();
+            opb.stop();
         }
     };
 
@@ -765,6 +850,13 @@ __device__ __forceinline__ void gemm_bf16_dma_body(const GemmArgs& g, const int 
 template <int BM, int BN, int WM, int WN, bool AKM, bool BKM, bool DB, int STAGES, int BK>
 __global__ __launch_bounds__(WM* WN * 64) void gemm_bf16_dma_kernel(const GemmArgs g) {
     gemm_bf16_dma_body<BM, BN, WM, WN, AKM, BKM, DB, STAGES, BK>(g, blockIdx.x, blockIdx.z);
+}
+
+// 3x3 convolution as an implicit GEMM: forward (BKM = false: y = patches(x) W^T) and input gradient
+// (BKM = true: dx = patches(dy) W_flipped) on the same main loop, operands gathered by the loaders.
+template <int BM, int BN, int WM, int WN, bool BKM, int STAGES>
+__global__ __launch_bounds__(WM* WN * 64) void conv3x3_bf16_igemm_kernel(const GemmArgs g, const ConvArgs cv) {
+    gemm_bf16_dma_body<BM, BN, WM, WN, false, BKM, true, STAGES, 64, false, BKM ? 2 : 1>(g, blockIdx.x, 0, false, cv);
 }
 
 // Several independent problems of one kind in a single launch (the four weight-gradient GEMMs
@@ -1162,6 +1254,69 @@ extern "C" int bb_gemm(const bb_gemm_desc* d, void* stream) {
     if (!ta && !tb) return dispatch_f32<false, false>(g, (int)batches, st);
     if (!ta && tb) return dispatch_f32<false, true>(g, (int)batches, st);
     return dispatch_f32<true, true>(g, (int)batches, st);
+}
+
+template <int BM, int BN, int WM, int WN, bool BKM, int STAGES>
+static int launch_conv3x3(GemmArgs& g, const ConvArgs& cv, hipStream_t st) {
+    constexpr int smem = STAGES * (BM + BN) * 64 * 2;
+    auto kern = conv3x3_bf16_igemm_kernel<BM, BN, WM, WN, BKM, STAGES>;
+    static bool configured = false;
+    if (!configured) {
+        BB_HIP_CHECK(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, smem));
+        configured = true;
+    }
+    g.tiles_m = (g.M + BM - 1) / BM;
+    g.tiles_n = (g.N + BN - 1) / BN;
+    hipLaunchKernelGGL(kern, dim3(g.tiles_m * g.tiles_n), dim3(WM * WN * 64), smem, st, g, cv);
+    BB_LAUNCH_CHECK();
+    return BB_OK;
+}
+
+extern "C" int bb_conv3x3_supported(int dtype, int mode, int n, int h, int w, int cin, int cout) {
+    const int64_t rows = (int64_t)n * h * w;
+    const int gathered = mode == BB_CONV_DGRAD ? cout : cin, produced = mode == BB_CONV_DGRAD ? cin : cout;
+    return dtype == BB_BF16 && (mode == BB_CONV_FWD || mode == BB_CONV_DGRAD) && n > 0 && h > 0 && w > 0 &&
+           rows >= 128 && rows < (1ll << 31) && gathered >= 64 && gathered % 64 == 0 && produced % 8 == 0 &&
+           produced >= 64;
+}
+
+extern "C" int bb_conv3x3(int dtype, int mode, int n, int h, int w, int cin, int cout, const void* src, const void* weight,
+                          void* dst, void* stream) {
+    BB_REQUIRE(src && weight && dst, "bb_conv3x3: null operand");
+    BB_REQUIRE(bb_conv3x3_supported(dtype, mode, n, h, w, cin, cout),
+               "bb_conv3x3: unsupported problem (bf16, >= 128 pixels, gathered channels a multiple of 64, produced channels "
+               "a multiple of 8 and >= 64): dtype %d mode %d n %d h %d w %d cin %d cout %d",
+               dtype, mode, n, h, w, cin, cout);
+    BB_REQUIRE(((uintptr_t)src % 16) == 0 && ((uintptr_t)weight % 16) == 0 && ((uintptr_t)dst % 16) == 0,
+               "bb_conv3x3: operands must be 16-byte aligned");
+    const bool dgrad = mode == BB_CONV_DGRAD;
+    GemmArgs g = {};
+    ConvArgs cv = {};
+    g.M = n * h * w;
+    g.N = dgrad ? cin : cout;
+    g.K = 9 * (dgrad ? cout : cin);
+    g.nb2 = 1;
+    g.A = src;
+    g.C = dst;
+    g.lda = dgrad ? cout : cin;
+    g.ldc = g.ldaux = g.N;
+    g.alpha = 1.f;
+    g.epilogue = BB_EPI_NONE;
+    cv.h = h; cv.w = w; cv.c = dgrad ? cout : cin;
+    hipStream_t st = (hipStream_t)stream;
+    if (!dgrad) {
+        // B = the weight as it lies: [cout, 9 * cin], k-contiguous
+        g.B = weight;
+        g.ldb = 9 * (int64_t)cin;
+        return launch_conv3x3<128, 64, 4, 1, false, 3>(g, cv, st);
+    }
+    // B[k = t * cout + o, n = i] = weight[o, 8 - t, i]: k-major with row stride 9 * cin, starting at tap 8; after
+    // the cout / 64 k-tiles of a tap the rows go back to o = 0 and one tap down
+    g.B = (const bf16*)weight + 8 * (int64_t)cin;
+    g.ldb = 9 * (int64_t)cin;
+    cv.b_every = cout / 64;
+    cv.b_wrap = -(int64_t)cout * g.ldb - cin;
+    return launch_conv3x3<64, 128, 2, 2, true, 3>(g, cv, st);
 }
 
 template <bool TA, bool TB> static int launch_grouped(GroupedArgs& G, hipStream_t st) {

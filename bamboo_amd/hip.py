@@ -25,7 +25,7 @@ LN_CODES = {"standard": LN_STANDARD, "annotated": LN_ANNOTATED}
 EXPORTS = (
     "bb_version", "bb_last_error", "bb_init", "bb_gemm", "bb_gemm_grouped", "bb_gemm_splitk_workspace", "bb_gemm_grouped_splitk", "bb_gemm_variant", "bb_layernorm_fwd",
     "bb_layernorm_bwd_workspace", "bb_layernorm_bwd", "bb_colsum_workspace", "bb_colsum_acc",
-    "bb_softmax_fwd", "bb_softmax_bwd", "bb_attention_fwd", "bb_attention_bwd", "bb_residual_add", "bb_act_fwd", "bb_bn_workspace", "bb_batchnorm_fwd", "bb_batchnorm_bwd", "bb_patch3x3", "bb_mse_workspace", "bb_mse_fwd_bwd", "bb_graph_begin", "bb_graph_end", "bb_graph_launch", "bb_graph_destroy",
+    "bb_softmax_fwd", "bb_softmax_bwd", "bb_attention_fwd", "bb_attention_bwd", "bb_residual_add", "bb_act_fwd", "bb_bn_workspace", "bb_batchnorm_fwd", "bb_batchnorm_bwd", "bb_patch3x3", "bb_conv3x3_supported", "bb_conv3x3", "bb_mse_workspace", "bb_mse_fwd_bwd", "bb_graph_begin", "bb_graph_end", "bb_graph_launch", "bb_graph_destroy",
     "bb_adam_multi", "bb_cast", "bb_fill_f32",
 )
 
@@ -102,6 +102,8 @@ def lib():
     L.bb_batchnorm_fwd.argtypes = [c_int, c_int, c_int, c_float, c_float, c_int] + [c_void_p] * 11
     L.bb_batchnorm_bwd.argtypes = [c_int, c_int, c_int] + [c_void_p] * 12
     L.bb_patch3x3.argtypes = [c_int, c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p]
+    L.bb_conv3x3_supported.argtypes = [c_int] * 7
+    L.bb_conv3x3.argtypes = [c_int] * 7 + [c_void_p] * 4
     L.bb_mse_workspace.restype = c_int64
     L.bb_mse_fwd_bwd.argtypes = [c_int, c_int64, c_void_p, c_void_p, c_void_p, c_float, c_void_p, c_int,
                                  c_void_p, c_void_p]
@@ -402,6 +404,43 @@ def batchnorm_bwd(x, gamma, mean, rstd, dy, relu_out, dx, g_out, dgamma, dbeta, 
 def patch3x3(src, dst, n, h, w, c, adjoint=False, stream=None):
     check(lib().bb_patch3x3(dtype_code(src.dtype), int(adjoint), n, h, w, c, _ptr(src), _ptr(dst), stream_ptr(stream)),
           "bb_patch3x3")
+
+
+CONV_FWD, CONV_DGRAD = 0, 1
+
+
+def conv3x3_supported(dtype, mode, n, h, w, cin, cout):
+    """Whether the implicit-GEMM 3x3 convolution takes this problem (else: patch matrix + GEMM)."""
+    return bool(lib().bb_conv3x3_supported(dtype_code(dtype), mode, n, h, w, cin, cout))
+
+
+def conv3x3(mode, src, weight, dst, n, h, w, cin, cout, stream=None):
+    """``CONV_FWD``: dst[n*h*w, cout] = conv3x3(src[n*h*w, cin]); ``CONV_DGRAD``: dst[n*h*w, cin] = the input
+    gradient for src = dy[n*h*w, cout]; weight [cout, 3, 3, cin]."""
+    rows = n * h * w
+    want_src, want_dst = ((rows, cin), (rows, cout)) if mode == CONV_FWD else ((rows, cout), (rows, cin))
+    if tuple(src.shape) != want_src or tuple(dst.shape) != want_dst or weight.numel() != 9 * cin * cout:
+        raise HipKernelError(f"conv3x3: shapes {tuple(src.shape)} {tuple(weight.shape)} {tuple(dst.shape)} do not fit "
+                             f"n={n} h={h} w={w} cin={cin} cout={cout} mode={mode}")
+    if not (src.is_contiguous() and dst.is_contiguous() and weight.is_contiguous()):
+        raise HipKernelError("conv3x3: operands must be contiguous")
+    if not (src.dtype == weight.dtype == dst.dtype):
+        raise HipKernelError("conv3x3: operands must share one dtype")
+    call = lambda: check(lib().bb_conv3x3(dtype_code(src.dtype), mode, n, h, w, cin, cout, _ptr(src), _ptr(weight),
+                                          _ptr(dst), stream_ptr(stream)), "bb_conv3x3")
+    if gemm_hook is not None:
+        gemm_hook(ConvLaunch(mode, rows, cin, cout), call, stream)
+    else:
+        call()
+
+
+class ConvLaunch:
+    """What ``gemm_hook`` is handed for an implicit-GEMM convolution: the GEMM it amounts to."""
+
+    def __init__(self, mode, rows, cin, cout):
+        self.variant_name = "bf16_conv3x3_fwd_igemm128x64k64s3" if mode == CONV_FWD else "bf16_conv3x3_dgrad_igemm64x128k64s3"
+        self.M, self.N, self.K = (rows, cout, 9 * cin) if mode == CONV_FWD else (rows, cin, 9 * cout)
+        self.epilogue = EPI_NONE
 
 
 def mse_workspace():

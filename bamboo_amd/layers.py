@@ -302,7 +302,10 @@ class BottleNeck:
     identity shortcut (reference ``BottleNeck``, DeepSpeedExamples/pipeline_parallelism/resnet.py:49-75:
     stride 1 and ``in_channels == 4 * out_channels``), on NHWC activations viewed as
     ``[rows = N*H*W, channels]``.  The 1x1 convolutions are plain GEMMs on that view; the 3x3
-    convolution is a GEMM over the gathered patch matrix ``[rows, 9*C]``.  Parameter names are the
+    convolution and its input gradient are implicit GEMMs (``hip.conv3x3``: the operand loader gathers the
+    3x3 neighbourhoods, no patch matrix is written); its weight gradient, and all three where the implicit
+    kernel does not take the problem (fp32, channel counts that are not multiples of 64), are GEMMs over the
+    gathered patch matrix ``[rows, 9*C]``.  Parameter names are the
     reference's; the 3x3 weight is kept as ``[out, 3, 3, in]`` (tap-major, channel-minor) so that it is the
     ``[out, 9*in]`` GEMM operand as it lies in memory (the reference holds ``[out, in, 3, 3]``)."""
 
@@ -400,16 +403,23 @@ class BottleNeck:
                           resid, y, mean, rstd, run[0], run[1], ctx.workspace, self.eps, self.momentum, relu,
                           stream=ctx.stream)
 
+    def _implicit(self, ctx, mode):
+        return hip.conv3x3_supported(ctx.dtype, mode, ctx.batch, self.h, self.w, self.cmid, self.cmid)
+
     def forward(self, x, st, ctx):
         if ctx.seq != self.h * self.w:
             raise hip.HipKernelError(f"activation has {ctx.seq} positions, the block expects {self.h}x{self.w}")
         w, sm = self.w_, ctx.stream
         st["x0"] = x
-        col = ctx.buf("col", (ctx.rows, 9 * self.cmid))
         hip.gemm(hip.NT, x, w["residual_function.0.weight"], st["y1"], stream=sm)
         self._bn_fwd(1, st["y1"], None, st["a1"], st["mean1"], st["rstd1"], True, ctx)
-        hip.patch3x3(st["a1"], col, ctx.batch, self.h, self.w, self.cmid, stream=sm)
-        hip.gemm(hip.NT, col, w["conv2"], st["y2"], stream=sm)
+        if self._implicit(ctx, hip.CONV_FWD):
+            hip.conv3x3(hip.CONV_FWD, st["a1"], w["residual_function.3.weight"], st["y2"], ctx.batch, self.h, self.w,
+                        self.cmid, self.cmid, stream=sm)
+        else:
+            col = ctx.buf("col", (ctx.rows, 9 * self.cmid))
+            hip.patch3x3(st["a1"], col, ctx.batch, self.h, self.w, self.cmid, stream=sm)
+            hip.gemm(hip.NT, col, w["conv2"], st["y2"], stream=sm)
         self._bn_fwd(4, st["y2"], None, st["a2"], st["mean2"], st["rstd2"], True, ctx)
         hip.gemm(hip.NT, st["a2"], w["residual_function.6.weight"], st["y3"], stream=sm)
         self._bn_fwd(7, st["y3"], x, st["out"], st["mean3"], st["rstd3"], True, ctx)
@@ -428,10 +438,14 @@ class BottleNeck:
         bn(7, "y3", "mean3", "rstd3", d_out, st["out"], d_y3, d_res)
         hip.gemm(hip.NN, d_y3, w["residual_function.6.weight"], d_m0, stream=sm)          # d_a2
         bn(4, "y2", "mean2", "rstd2", d_m0, st["a2"], d_m1, None)                          # d_y2
-        hip.patch3x3(st["a1"], col, ctx.batch, self.h, self.w, cm, stream=sm)              # patches again: cheaper than stashing
-        hip.gemm(hip.NN, d_m1, w["conv2"], d_col, stream=sm)
+        hip.patch3x3(st["a1"], col, ctx.batch, self.h, self.w, cm, stream=sm)              # for the weight gradient: cheaper than stashing
         d_a1, d_m2 = ctx.buf("d_m0", (R, cm)), ctx.buf("d_m2", (R, cm))
-        hip.patch3x3(d_col, d_a1, ctx.batch, self.h, self.w, cm, adjoint=True, stream=sm)
+        if self._implicit(ctx, hip.CONV_DGRAD):
+            hip.conv3x3(hip.CONV_DGRAD, d_m1, w["residual_function.3.weight"], d_a1, ctx.batch, self.h, self.w, cm, cm,
+                        stream=sm)
+        else:
+            hip.gemm(hip.NN, d_m1, w["conv2"], d_col, stream=sm)
+            hip.patch3x3(d_col, d_a1, ctx.batch, self.h, self.w, cm, adjoint=True, stream=sm)
         bn(1, "y1", "mean1", "rstd1", d_a1, st["a1"], d_m2, None)                          # d_y1
         hip.gemm(hip.NN, d_m2, w["residual_function.0.weight"], d_x, epilogue=hip.EPI_RESIDUAL, resid=d_res, stream=sm)
         # the three weight gradients in one launch: 68 output tiles over 6272 rows, cut along the rows

@@ -102,6 +102,8 @@ class GemmProbe:
             name = "grouped_" + hip.gemm_variant(desc[0]).rsplit("_", 1)[0]
             flops = sum(2.0 * d.M * d.N * d.K for d in desc)
             shape = "+".join(f"{d.M}x{d.N}x{d.K}" for d in desc)
+        elif hasattr(desc, "variant_name"):      # implicit-GEMM convolution
+            name, flops, shape = desc.variant_name, 2.0 * desc.M * desc.N * desc.K, f"{desc.M}x{desc.N}x{desc.K}"
         else:
             name, flops = hip.gemm_variant(desc), 2.0 * desc.M * desc.N * desc.K
             # an epilogue that evaluates the activation is a different code path with work of its own

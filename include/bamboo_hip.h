@@ -211,6 +211,18 @@ int bb_batchnorm_bwd(int dtype, int rows, int cols, const void* x, const void* g
  * (adjoint = 0), or its adjoint dx[p, c] = sum of the patch entries that read x[p, c]
  * (adjoint = 1); turns nn.Conv2d(k=3, padding=1) (resnet.py:58) and its input gradient into GEMMs. */
 int bb_patch3x3(int dtype, int adjoint, int n, int h, int w, int c, const void* src, void* dst, void* stream);
+/* nn.Conv2d(cin, cout, kernel_size=3, padding=1, bias=False) (resnet.py:58) on NHWC rows as an implicit
+ * GEMM on the matrix cores: the patch matrix is never written, the operand loader gathers it.
+ *   BB_CONV_FWD    dst[p, o] = sum_{t, i} src[p + shift(t), i] * weight[o, t, i]     src [n*h*w, cin], dst [n*h*w, cout]
+ *   BB_CONV_DGRAD  dst[p, i] = sum_{t, o} src[p - shift(t), o] * weight[o, t, i]     src [n*h*w, cout], dst [n*h*w, cin]
+ * with tap t = (dy + 1) * 3 + (dx + 1), shift(t) = dy * w + dx inside one image and zero outside it, and
+ * weight [cout, 3, 3, cin] (tap-major, channel-minor).  bf16 only; bb_conv3x3_supported() says (1 / 0) whether
+ * a problem is taken (channel counts: gathered side a multiple of 64), bb_conv3x3 refuses the others.     */
+#define BB_CONV_FWD 0
+#define BB_CONV_DGRAD 1
+int bb_conv3x3_supported(int dtype, int mode, int n, int h, int w, int cin, int cout);
+int bb_conv3x3(int dtype, int mode, int n, int h, int w, int cin, int cout, const void* src, const void* weight,
+               void* dst, void* stream);
 
 /* Mean-squared-error head (nn.MSELoss, transformer.py:264) fused with its gradient:
  * loss_out[0] (+)= mean((y-t)^2);  dy = grad_scale * 2 (y-t) / n.  Deterministic two-pass

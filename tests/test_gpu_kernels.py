@@ -453,6 +453,62 @@ def test_patch3x3_and_adjoint(hiplib, dtype):
     assert rel_err(back, fold) < (1e-6 if dtype == torch.float32 else 1e-2)
 
 
+CONV_SHAPES = [(4, 5, 7, 64, 64),        # 140 pixels: one ragged row tile, one k-tile per tap
+               (4, 6, 6, 64, 128),        # 144 pixels, as many output as a dgrad column tile
+               (3, 9, 8, 128, 192),       # cin != cout, two k-tiles per tap forward and three backward
+               (32, 14, 14, 256, 256),    # a ResNet-152 conv4_x block at micro-batch 32 (6272 pixels)
+               (2, 1, 70, 64, 128), (2, 70, 1, 128, 128)]   # degenerate images: whole rows / columns of taps fall outside
+
+
+@pytest.mark.parametrize("n,h,w,cin,cout", CONV_SHAPES)
+def test_conv3x3_implicit_gemm(hiplib, n, h, w, cin, cout):
+    """nn.Conv2d(cin, cout, 3, padding=1, bias=False) (reference resnet.py:58) and its input gradient as implicit
+    GEMMs, against torch's conv2d and its autograd in fp64 on the same bf16 values; the forward is also
+    bit-equal to the patch matrix followed by the GEMM kernel of the same tile shape, which multiplies the
+    same numbers in the same order."""
+    dt = torch.bfloat16
+    rows = n * h * w
+    assert hiplib.conv3x3_supported(dt, hiplib.CONV_FWD, n, h, w, cin, cout)
+    assert hiplib.conv3x3_supported(dt, hiplib.CONV_DGRAD, n, h, w, cin, cout)
+    x = randn(rows, cin, dtype=dt, seed=60)
+    wt = randn(cout, 3, 3, cin, dtype=dt, seed=61, scale=math.sqrt(2.0 / (9 * cin)))   # [out, tap, in]
+    dy = randn(rows, cout, dtype=dt, seed=62)
+    y = torch.full((rows, cout), float("nan"), dtype=dt, device=DEV)
+    dx = torch.full((rows, cin), float("nan"), dtype=dt, device=DEV)
+    hiplib.conv3x3(hiplib.CONV_FWD, x, wt, y, n, h, w, cin, cout)
+    hiplib.conv3x3(hiplib.CONV_DGRAD, dy, wt, dx, n, h, w, cin, cout)
+    xr = x.double().cpu().view(n, h, w, cin).permute(0, 3, 1, 2).requires_grad_(True)
+    wr = wt.double().cpu().permute(0, 3, 1, 2)                                            # the reference's [O, I, kh, kw]
+    yr = torch.nn.functional.conv2d(xr, wr, padding=1)
+    yr.backward(dy.double().cpu().view(n, h, w, cout).permute(0, 3, 1, 2))
+    assert rel_err(y, yr.detach().permute(0, 2, 3, 1).reshape(rows, cout)) < tol(dt)
+    assert rel_err(dx, xr.grad.permute(0, 2, 3, 1).reshape(rows, cin)) < tol(dt)
+    # deterministic
+    y2, dx2 = torch.empty_like(y), torch.empty_like(dx)
+    hiplib.conv3x3(hiplib.CONV_FWD, x, wt, y2, n, h, w, cin, cout)
+    hiplib.conv3x3(hiplib.CONV_DGRAD, dy, wt, dx2, n, h, w, cin, cout)
+    assert torch.equal(y, y2) and torch.equal(dx, dx2)
+    # the explicit route: patch matrix, then the GEMM
+    col = torch.empty(rows, 9 * cin, dtype=dt, device=DEV)
+    hiplib.patch3x3(x, col, n, h, w, cin)
+    y3 = torch.empty_like(y)
+    hiplib.gemm(hiplib.NT, col, wt.view(cout, 9 * cin), y3)
+    if hiplib.gemm_variant(hiplib.gemm_desc(hiplib.NT, col, wt.view(cout, 9 * cin), y3)).endswith("dma128x64k64s3"):
+        assert torch.equal(y, y3)
+    else:
+        assert rel_err(y, y3.double()) < 1e-2
+
+
+def test_conv3x3_refuses_what_it_does_not_take(hiplib):
+    dt = torch.bfloat16
+    assert not hiplib.conv3x3_supported(dt, hiplib.CONV_FWD, 4, 6, 6, 16, 64)            # 16 gathered channels
+    assert not hiplib.conv3x3_supported(torch.float32, hiplib.CONV_FWD, 4, 6, 6, 64, 64)
+    assert not hiplib.conv3x3_supported(dt, hiplib.CONV_FWD, 1, 6, 6, 64, 64)            # 36 pixels
+    x, wt, y = randn(144, 16, dtype=dt), randn(64, 3, 3, 16, dtype=dt), torch.empty(144, 64, dtype=dt, device=DEV)
+    with pytest.raises(hiplib.HipKernelError):
+        hiplib.conv3x3(hiplib.CONV_FWD, x, wt, y, 4, 6, 6, 16, 64)
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 def test_mse(hiplib, dtype):
     n = 4 * 128 * 768

@@ -216,12 +216,15 @@ def test_failover_promotion_matches_oracle(hiplib, dead_from, dtype):
     assert engine.global_steps == 1 or engine.global_steps == 2
 
 
-@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["fp32", "bf16"])
-def test_resnet_stage_matches_oracle_with_rc(hiplib, dtype):
+@pytest.mark.parametrize("dtype,cin,cmid", [(torch.float32, 64, 16), (torch.bfloat16, 64, 16), (torch.bfloat16, 512, 128)],
+                         ids=["fp32", "bf16", "bf16-implicit-gemm"])
+def test_resnet_stage_matches_oracle_with_rc(hiplib, dtype, cin, cmid):
     """Bottleneck stage (conv 1x1 -> 3x3 -> 1x1, train-mode BatchNorm, ReLU, identity shortcut) with
-    redundant forwards of the shadow blocks, against the torch conv2d / batch_norm oracle."""
+    redundant forwards of the shadow blocks, against the torch conv2d / batch_norm oracle.  With 128 middle
+    channels the 3x3 convolution and its input gradient run as implicit GEMMs, with 16 through the patch matrix."""
     from bamboo_amd import BottleNeck
-    cin, cmid, side, L, S, sid, mb, M = 64, 16, 6, 2, 4, 1, 4, 4
+    side, L, S, sid, mb, M = 6, 2, 4, 1, 4, 4
+    assert hiplib.conv3x3_supported(dtype, hiplib.CONV_DGRAD, mb, side, side, cmid, cmid) == (cmid == 128)
     specs = [LayerSpec(BottleNeck, cin, cmid, height=side, width=side) for _ in range(L * S)]
     model = PipelineModule(specs, num_stages=S, partition_method="uniform", stage_id=sid, dtype=dtype, device=DEV)
     q = SeededActivationQueue((mb, side * side, cin), dtype, M, stage_ids=[sid, sid + 1], seed=9, device=DEV)
