@@ -25,6 +25,7 @@ struct GemmArgs {
     float alpha;
     int epilogue, act, accumulate, c_f32;
     int tiles_m, tiles_n;
+    int conv_h, conv_w, conv_c, conv_row0;  // TN: B is the 3x3 patch matrix of an NHWC tensor (conv_c > 0)
 };
 
 // ---- tile order: consecutive logical tiles land on the same XCD (workgroups are dealt
@@ -375,7 +376,7 @@ template <int BR, bool KM, int NW, int BK = 32, bool VIS = false, int CONV = 0> 
     static constexpr int BYTES = BR * BK * 2;
     static constexpr int ROUNDS = BYTES / (1024 * NW);  // instructions per thread per k-tile
     static_assert(ROUNDS >= 1, "tile too small for the block");
-    static_assert(CONV == 0 || (CONV == 1 && !KM && BK == 64) || (CONV == 2 && KM), "convolution loaders: see above");
+    static_assert(CONV == 0 || (CONV == 1 && !KM && BK == 64) || ((CONV == 2 || CONV == 3) && KM), "convolution loaders: see above");
     const bf16* src[ROUNDS];
     int64_t step;  // elements to advance per k-tile
     // CONV 1: per round the taps that lie inside the image (bit t = tap t), then wave-uniform position in K
@@ -386,6 +387,9 @@ template <int BR, bool KM, int NW, int BK = 32, bool VIS = false, int CONV = 0> 
     // CONV 2
     int cnt, every;
     int64_t wrap;
+    // CONV 3: image coordinates of the pixel each round reads next, the block's tap, the k-tile step in pixels
+    int py[ROUNDS], px[ROUNDS];
+    int tdy, tdx, dpy, dpx, ch;
 
     __device__ __forceinline__ void init(const bf16* base, int64_t ld, int row0, int rows, int tid) {
         const int lane = tid & 63, wave = tid >> 6;
@@ -441,15 +445,52 @@ template <int BR, bool KM, int NW, int BK = 32, bool VIS = false, int CONV = 0> 
     __device__ __forceinline__ void init_wrap(const ConvArgs& cv) {
         cnt = 0; every = cv.b_every; wrap = cv.b_wrap;
     }
+    // CONV 3 (k-major operand): the patch matrix [pixels, 9 * c] of the tensor at base as the B operand of a
+    // weight gradient.  A column tile (col0 .. col0 + BR - 1, inside one tap since c % BR == 0) reads channels
+    // of the pixel `tap` away from pixel k: rows advance by the k-tile, the lane's image coordinates with them.
+    __device__ __forceinline__ void init_conv_km(const bf16* base, int col0, int tid, int h, int w, int c, int pix0) {
+        const int lane = tid & 63, wave = tid >> 6;
+        const int t = col0 / c, ci0 = col0 - t * c;
+        tdy = t / 3 - 1; tdx = t % 3 - 1; ch = h; cw = w;
+        dpy = BK / w; dpx = BK % w;
+#pragma unroll
+        for (int i = 0; i < ROUNDS; ++i) {
+            const int q = i * NW + wave;
+            constexpr int CPR = BR / 8, RPI = 64 / CPR;
+            const int k = q * RPI + lane / CPR;
+            const int cch = (lane % CPR) ^ (4 * (k & 3));
+            const int p = pix0 + k, pix = p % (h * w);
+            py[i] = pix / w;
+            px[i] = pix - py[i] * w;
+            src[i] = base + ((int64_t)p + tdy * w + tdx) * c + ci0 + cch * 8;
+        }
+        zero = (const bf16*)(bb_zero_line + (lane & 7) * 16);
+        step = (int64_t)BK * c;
+    }
     // past the end of K: the last tile is fetched again and again
     __device__ __forceinline__ void stop() {
         step = 0;
         if constexpr (CONV == 1) kstep = 0;
         if constexpr (CONV == 2) wrap = 0;
+        if constexpr (CONV == 3) dpy = dpx = 0;
     }
     __device__ __forceinline__ const bf16* source(int i) const {
         if constexpr (CONV == 1) return ((inside[i] >> tap) & 1u) ? src[i] + (tapoff + c0) : zero;
+        else if constexpr (CONV == 3)
+            return ((unsigned)(py[i] + tdy) < (unsigned)ch && (unsigned)(px[i] + tdx) < (unsigned)cw) ? src[i] : zero;
         else return src[i];
+    }
+    // CONV 3: round i moves on by one k-tile of pixels (BK / w + 1 <= h: at most one image boundary per step)
+    __device__ __forceinline__ void next_pixels(int i) {
+        if constexpr (CONV == 3) {
+            px[i] += dpx;
+            py[i] += dpy;
+            if (px[i] >= cw) {
+                px[i] -= cw;
+                ++py[i];
+            }
+            if (py[i] >= ch) py[i] -= ch;
+        }
     }
     // after the last instruction of a k-tile
     __device__ __forceinline__ void advance() {
@@ -474,12 +515,14 @@ template <int BR, bool KM, int NW, int BK = 32, bool VIS = false, int CONV = 0> 
             if constexpr (VIS) __builtin_amdgcn_global_load_lds((gbl_ptr_t*)source(i), (lds_ptr_t*)(tile + (i * NW + wave) * 1024), 16, 0, 0);
             else dma16(source(i), tile + (i * NW + wave) * 1024);
             src[i] += step;
+            next_pixels(i);
         }
         advance();
     }
     template <int I> __device__ __forceinline__ void issue_one(unsigned char* tile, int wave) {
         dma16(source(I), tile + (I * NW + wave) * 1024);
         src[I] += step;
+        next_pixels(I);
         if constexpr (I == ROUNDS - 1) advance();
     }
 };
@@ -528,9 +571,11 @@ __device__ __forceinline__ void gemm_bf16_dma_body(const GemmArgs& g, const int 
                   "64-wide k-tiles alternate between two stages or rotate through more");
     constexpr int WTM = BM / WM, WTN = BN / WN, TM = WTM / 32, TN = WTN / 32;
     // CONV 1: forward 3x3 convolution (A gathered); CONV 2: its input gradient (A gathered, B the flipped filter)
-    static_assert(CONV == 0 || (!AKM && (CONV == 2) == BKM), "implicit convolution: NT forward, NN input gradient");
-    using OpA = DmaOperand<BM, AKM, NW, BK, VIS, CONV ? 1 : 0>;
-    using OpB = DmaOperand<BN, BKM, NW, BK, VIS, CONV == 2 ? 2 : 0>;
+    // CONV 3: its weight gradient (B = the patch matrix, gathered)
+    static_assert(CONV == 0 || (CONV == 3 ? AKM && BKM : !AKM && (CONV == 2) == BKM),
+                  "implicit convolution: NT forward, NN input gradient, TN weight gradient");
+    using OpA = DmaOperand<BM, AKM, NW, BK, VIS, CONV == 1 || CONV == 2 ? 1 : 0>;
+    using OpB = DmaOperand<BN, BKM, NW, BK, VIS, CONV >= 2 ? CONV : 0>;
     constexpr int STAGE_BYTES = OpA::BYTES + OpB::BYTES;
     constexpr int LOADS = OpA::ROUNDS + OpB::ROUNDS;
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
@@ -548,9 +593,10 @@ __device__ __forceinline__ void gemm_bf16_dma_body(const GemmArgs& g, const int 
 
     OpA opa;
     OpB opb;
-    if constexpr (CONV != 0) opa.init_conv(A, m0, g.M, tid, cv);
+    if constexpr (CONV == 1 || CONV == 2) opa.init_conv(A, m0, g.M, tid, cv);
     else opa.init(A, g.lda, m0, g.M, tid);
-    opb.init(B, g.ldb, n0, g.N, tid);
+    if constexpr (CONV == 3) opb.init_conv_km(B, n0, tid, g.conv_h, g.conv_w, g.conv_c, g.conv_row0);
+    else opb.init(B, g.ldb, n0, g.N, tid);
     if constexpr (CONV == 2) opb.init_wrap(cv);
     FragReader<BM, TM, AKM, BK> fa;
     FragReader<BN, TN, BKM, BK> fb;
@@ -867,7 +913,8 @@ struct GroupedArgs {
     int first_block[GROUP_MAX + 1];
     int count;
 };
-template <int BM, int BN, int WM, int WN, bool AKM, bool BKM, bool DB, int STAGES>
+// CONVB: some problems of the group read their B operand as the patch matrix of a 3x3 convolution
+template <int BM, int BN, int WM, int WN, bool AKM, bool BKM, bool DB, int STAGES, bool CONVB = false>
 __global__ __launch_bounds__(WM* WN * 64) void gemm_bf16_dma_grouped_kernel(const GroupedArgs G) {
     // The tiles of all problems form one list; an XCD takes a contiguous stretch of it, so its
     // resident blocks are a few wide rectangles of one or two problems (few distinct operand
@@ -878,6 +925,12 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_bf16_dma_grouped_kernel(cons
     // compiler-visible DMA here: the lock step it forces on the waves keeps the three resident blocks of a CU
     // on the same operand panels (459 instead of 720 MiB read per launch at the same kernel speed; the stage
     // gains half a percent with the second stream running)
+    if constexpr (CONVB) {
+        if (G.p[pi].conv_c > 0) {
+            gemm_bf16_dma_body<BM, BN, WM, WN, AKM, BKM, DB, STAGES, 32, true, 3>(G.p[pi], lid - G.first_block[pi], 0, true);
+            return;
+        }
+    }
     gemm_bf16_dma_body<BM, BN, WM, WN, AKM, BKM, DB, STAGES, 32, true>(G.p[pi], lid - G.first_block[pi], 0, true);
 }
 
@@ -1203,19 +1256,33 @@ static int fill_args(const bb_gemm_desc* d, GemmArgs& g, int64_t& batches, bool&
     BB_REQUIRE(d->epilogue != BB_EPI_ACT_DACT || d->aux_out, "bb_gemm: ACT_DACT epilogue needs aux_out");
     BB_REQUIRE(batches <= 65535, "bb_gemm: too many batches (%lld)", (long long)batches);
     const int vec = d->dtype == BB_BF16 ? 8 : 4;
+    const bool conv = d->conv_c != 0 || d->conv_h != 0 || d->conv_w != 0 || d->conv_row0 != 0;
+    if (conv) {
+        // B = patch matrix of an NHWC tensor, gathered by the grouped DMA kernel's loader
+        BB_REQUIRE(d->layout == BB_TN && d->dtype == BB_BF16 && batches == 1, "bb_gemm: a patch-matrix B needs BB_TN, bf16, no batching");
+        BB_REQUIRE(d->conv_c > 0 && d->conv_c % 128 == 0 && d->conv_h > 0 && d->conv_w > 0 && d->conv_row0 >= 0,
+                   "bb_gemm: patch-matrix B: conv_c (%d) must be a positive multiple of 128, conv_h/conv_w positive", d->conv_c);
+        BB_REQUIRE(d->N == 9 * d->conv_c, "bb_gemm: patch-matrix B: N (%d) must be 9 * conv_c (%d)", d->N, d->conv_c);
+        BB_REQUIRE(d->K % 32 == 0 && d->K >= 64 && d->M >= 128 && 32 / d->conv_w + 1 <= d->conv_h,
+                   "bb_gemm: patch-matrix B: K (%d) must be a multiple of 32 and >= 64, M (%d) >= 128, and 32 pixels must "
+                   "not span more than one image boundary (%d x %d)", d->K, d->M, d->conv_h, d->conv_w);
+        BB_REQUIRE(!d->bias && d->epilogue == BB_EPI_NONE, "bb_gemm: patch-matrix B takes no bias / epilogue");
+    }
     // the contiguous dimension of every operand is read in 16-byte vectors
-    const int a_contig = ta ? d->M : d->K, b_contig = tb ? d->N : d->K;
+    const int a_contig = ta ? d->M : d->K, b_contig = conv ? d->conv_c : tb ? d->N : d->K;
+    const int64_t ldb = conv ? d->conv_c : d->ldb;
     BB_REQUIRE(a_contig % vec == 0 && d->lda % vec == 0, "bb_gemm: A contiguous dim/lda must be a multiple of %d", vec);
-    BB_REQUIRE(b_contig % vec == 0 && d->ldb % vec == 0, "bb_gemm: B contiguous dim/ldb must be a multiple of %d", vec);
+    BB_REQUIRE(b_contig % vec == 0 && ldb % vec == 0, "bb_gemm: B contiguous dim/ldb must be a multiple of %d", vec);
     BB_REQUIRE(((uintptr_t)d->A % 16) == 0 && ((uintptr_t)d->B % 16) == 0, "bb_gemm: operands must be 16-byte aligned");
     BB_REQUIRE(d->sA1 % vec == 0 && d->sA2 % vec == 0 && d->sB1 % vec == 0 && d->sB2 % vec == 0,
                "bb_gemm: batch strides of A/B must be multiples of %d", vec);
-    BB_REQUIRE(d->lda >= a_contig && d->ldb >= b_contig && d->ldc >= d->N, "bb_gemm: leading dimension too small");
+    BB_REQUIRE(d->lda >= a_contig && ldb >= b_contig && d->ldc >= d->N, "bb_gemm: leading dimension too small");
     g.A = d->A; g.B = d->B; g.C = d->C;
     g.bias = d->bias; g.aux_in = d->aux_in; g.aux_out = d->aux_out; g.resid = d->resid;
     g.colsum = nullptr;
     BB_REQUIRE(!d->colsum_out || d->layout == BB_TN, "bb_gemm: colsum_out needs the BB_TN layout");
-    g.lda = d->lda; g.ldb = d->ldb; g.ldc = d->ldc; g.ldaux = d->ldaux > 0 ? d->ldaux : d->ldc;
+    g.lda = d->lda; g.ldb = ldb; g.ldc = d->ldc; g.ldaux = d->ldaux > 0 ? d->ldaux : d->ldc;
+    g.conv_h = d->conv_h; g.conv_w = d->conv_w; g.conv_c = d->conv_c; g.conv_row0 = d->conv_row0;
     g.sA1 = d->sA1; g.sA2 = d->sA2; g.sB1 = d->sB1; g.sB2 = d->sB2; g.sC1 = d->sC1; g.sC2 = d->sC2;
     g.alpha = d->alpha;
     g.epilogue = d->epilogue; g.act = d->act; g.accumulate = d->accumulate;
@@ -1235,6 +1302,7 @@ static int colsum_standalone(const bb_gemm_desc* d, void* stream) {
 }
 
 extern "C" int bb_gemm(const bb_gemm_desc* d, void* stream) {
+    if (d && d->conv_c != 0) return bb_gemm_grouped(d, 1, stream);   // only the grouped kernel gathers a patch-matrix B
     GemmArgs g;
     int64_t batches;
     bool ta, tb;
@@ -1319,10 +1387,10 @@ extern "C" int bb_conv3x3(int dtype, int mode, int n, int h, int w, int cin, int
     return launch_conv3x3<64, 128, 2, 2, true, 3>(g, cv, st);
 }
 
-template <bool TA, bool TB> static int launch_grouped(GroupedArgs& G, hipStream_t st) {
+template <bool TA, bool TB, bool CONVB = false> static int launch_grouped(GroupedArgs& G, hipStream_t st) {
     constexpr int BM = 128, BN = 128, STAGES = 3;
     constexpr int smem = STAGES * (BM + BN) * 32 * 2;
-    auto kern = gemm_bf16_dma_grouped_kernel<BM, BN, 2, 2, TA, TB, true, STAGES>;
+    auto kern = gemm_bf16_dma_grouped_kernel<BM, BN, 2, 2, TA, TB, true, STAGES, CONVB>;
     static bool configured = false;
     if (!configured) {
         BB_HIP_CHECK(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, smem));
@@ -1347,12 +1415,17 @@ extern "C" int bb_gemm_grouped(const bb_gemm_desc* descs, int count, void* strea
     hipStream_t st = (hipStream_t)stream;
     // one launch when every problem is an unbatched bf16 problem of one layout that the DMA
     // kernel accepts; otherwise the problems run one after the other (same results)
-    bool fuse = count >= 2 && count <= GROUP_MAX;
+    bool has_conv = false;
+    for (int i = 0; i < count; ++i) has_conv = has_conv || descs[i].conv_c != 0;
+    bool fuse = count >= (has_conv ? 1 : 2) && count <= GROUP_MAX;
     for (int i = 0; i < count && fuse; ++i) {
         const bb_gemm_desc& d = descs[i];
         fuse = d.dtype == BB_BF16 && d.layout == descs[0].layout && d.nb1 <= 1 && d.nb2 <= 1 && d.M > 0 && d.N > 0 &&
                pick_dma_tile(d.M, d.N, d.K, 1, d.layout) != D_NONE && dma_tile_override() != 4;
     }
+    // a patch-matrix B exists only inside the grouped kernel: no one-by-one route for it
+    BB_REQUIRE(fuse || !has_conv, "bb_gemm_grouped: a problem with a patch-matrix B must share a launch of bf16 BB_TN "
+                                  "problems the DMA kernel takes (M, N >= 128, K %% 32 == 0)");
     if (!fuse) {
         for (int i = 0; i < count; ++i) {
             int rc = bb_gemm(&descs[i], stream);
@@ -1372,6 +1445,7 @@ extern "C" int bb_gemm_grouped(const bb_gemm_desc* descs, int count, void* strea
     const int layout = descs[0].layout;
     if (layout == BB_NT) return launch_grouped<false, false>(G, st);
     if (layout == BB_NN) return launch_grouped<false, true>(G, st);
+    if (has_conv) return launch_grouped<true, true, true>(G, st);
     return launch_grouped<true, true>(G, st);
 }
 
@@ -1456,7 +1530,8 @@ extern "C" int bb_gemm_grouped_splitk(const bb_gemm_desc* descs, int count, void
             // A advances along its contraction index: rows for TN ([K, M]), columns otherwise ([M, K])
             t.A = (const char*)d.A + (d.layout == BB_TN ? (int64_t)k0 * d.lda : (int64_t)k0) * 2;
             // B: [N, K] for NT, [K, N] for NN and TN
-            t.B = (const char*)d.B + (d.layout == BB_NT ? (int64_t)k0 : (int64_t)k0 * d.ldb) * 2;
+            if (d.conv_c != 0) t.conv_row0 = d.conv_row0 + k0;   // the tensor stays put, the chunk starts k0 pixels in
+            else t.B = (const char*)d.B + (d.layout == BB_NT ? (int64_t)k0 : (int64_t)k0 * d.ldb) * 2;
             t.C = ws + (int64_t)p * d.M * d.N;
             t.ldc = d.N;
             t.accumulate = 0;

@@ -47,6 +47,7 @@ class GemmDesc(Structure):
         ("alpha", c_float), ("epilogue", c_int32), ("act", c_int32), ("accumulate", c_int32),
         ("bias", c_void_p), ("aux_in", c_void_p), ("aux_out", c_void_p), ("resid", c_void_p),
         ("ldaux", c_int64), ("colsum_out", c_void_p), ("colsum_ws", c_void_p),
+        ("conv_h", c_int32), ("conv_w", c_int32), ("conv_c", c_int32), ("conv_row0", c_int32),
     ]
 
 
@@ -152,10 +153,16 @@ def _row_major(t, name):
 
 # ------------------------------------------------------------------------------------- GEMM
 def gemm_desc(layout, A, B, C, *, alpha=1.0, bias=None, epilogue=EPI_NONE, act=ACT_RELU, accumulate=False,
-              aux_in=None, aux_out=None, resid=None, colsum_out=None, colsum_ws=None):
-    """Descriptor of C = epilogue(alpha * op(A) op(B) [+ bias]) on 2-D row-major views."""
+              aux_in=None, aux_out=None, resid=None, colsum_out=None, colsum_ws=None, conv=None):
+    """Descriptor of C = epilogue(alpha * op(A) op(B) [+ bias]) on 2-D row-major views.
+    ``conv=(h, w)`` (TN only): B is the NHWC tensor ``[pixels, c]`` whose 3x3 patch matrix ``[pixels, 9c]`` is
+    the operand, gathered inside the kernel (weight gradient of a 3x3 convolution)."""
     lda, ldb, ldc = _row_major(A, "A"), _row_major(B, "B"), _row_major(C, "C")
-    if layout == NT:
+    if conv is not None:
+        if layout != TN or not B.is_contiguous():
+            raise HipKernelError("gemm: conv= needs the TN layout and a contiguous NHWC tensor as B")
+        K, M = A.shape; Kb, N = B.shape[0], 9 * B.shape[1]
+    elif layout == NT:
         M, K = A.shape; N, Kb = B.shape
     elif layout == NN:
         M, K = A.shape; Kb, N = B.shape
@@ -172,6 +179,8 @@ def gemm_desc(layout, A, B, C, *, alpha=1.0, bias=None, epilogue=EPI_NONE, act=A
     d.M, d.N, d.K = M, N, K
     d.A, d.lda, d.B, d.ldb, d.C, d.ldc = A.data_ptr(), lda, B.data_ptr(), ldb, C.data_ptr(), ldc
     d.nb1 = d.nb2 = 1
+    if conv is not None:
+        d.conv_h, d.conv_w, d.conv_c, d.conv_row0 = conv[0], conv[1], B.shape[1], 0
     d.alpha, d.epilogue, d.act, d.accumulate = alpha, epilogue, act, int(accumulate)
     ldaux = 0
     for t in (aux_in, aux_out, resid):

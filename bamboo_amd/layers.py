@@ -302,10 +302,10 @@ class BottleNeck:
     identity shortcut (reference ``BottleNeck``, DeepSpeedExamples/pipeline_parallelism/resnet.py:49-75:
     stride 1 and ``in_channels == 4 * out_channels``), on NHWC activations viewed as
     ``[rows = N*H*W, channels]``.  The 1x1 convolutions are plain GEMMs on that view; the 3x3
-    convolution and its input gradient are implicit GEMMs (``hip.conv3x3``: the operand loader gathers the
-    3x3 neighbourhoods, no patch matrix is written); its weight gradient, and all three where the implicit
-    kernel does not take the problem (fp32, channel counts that are not multiples of 64), are GEMMs over the
-    gathered patch matrix ``[rows, 9*C]``.  Parameter names are the
+    convolution, its input gradient (``hip.conv3x3``) and its weight gradient (``gemm_desc(..., conv=)``) are
+    implicit GEMMs: the operand loader gathers the 3x3 neighbourhoods, no patch matrix is written.  Where the
+    implicit kernels do not take the problem (fp32, channel counts that are not multiples of 64, resp. 128 for
+    the weight gradient) the same products run as GEMMs over the gathered patch matrix ``[rows, 9*C]``.  Parameter names are the
     reference's; the 3x3 weight is kept as ``[out, 3, 3, in]`` (tap-major, channel-minor) so that it is the
     ``[out, 9*in]`` GEMM operand as it lies in memory (the reference holds ``[out, in, 3, 3]``)."""
 
@@ -438,7 +438,11 @@ class BottleNeck:
         bn(7, "y3", "mean3", "rstd3", d_out, st["out"], d_y3, d_res)
         hip.gemm(hip.NN, d_y3, w["residual_function.6.weight"], d_m0, stream=sm)          # d_a2
         bn(4, "y2", "mean2", "rstd2", d_m0, st["a2"], d_m1, None)                          # d_y2
-        hip.patch3x3(st["a1"], col, ctx.batch, self.h, self.w, cm, stream=sm)              # for the weight gradient: cheaper than stashing
+        # weight gradient of the 3x3 convolution: patch matrix gathered inside the GEMM, else built again here
+        # (cheaper than stashing it)
+        wgrad_implicit = (self._implicit(ctx, hip.CONV_DGRAD) and cm % 128 == 0 and R % 32 == 0 and 32 // self.w + 1 <= self.h)
+        if not wgrad_implicit:
+            hip.patch3x3(st["a1"], col, ctx.batch, self.h, self.w, cm, stream=sm)
         d_a1, d_m2 = ctx.buf("d_m0", (R, cm)), ctx.buf("d_m2", (R, cm))
         if self._implicit(ctx, hip.CONV_DGRAD):
             hip.conv3x3(hip.CONV_DGRAD, d_m1, w["residual_function.3.weight"], d_a1, ctx.batch, self.h, self.w, cm, cm,
@@ -450,7 +454,8 @@ class BottleNeck:
         hip.gemm(hip.NN, d_m2, w["residual_function.0.weight"], d_x, epilogue=hip.EPI_RESIDUAL, resid=d_res, stream=sm)
         # the three weight gradients in one launch: 68 output tiles over 6272 rows, cut along the rows
         hip.gemm_grouped([hip.gemm_desc(hip.TN, d_y3, st["a2"], g["residual_function.6.weight"], accumulate=True),
-                          hip.gemm_desc(hip.TN, d_m1, col, g["conv2"], accumulate=True),
+                          hip.gemm_desc(hip.TN, d_m1, st["a1"], g["conv2"], accumulate=True, conv=(self.h, self.w))
+                          if wgrad_implicit else hip.gemm_desc(hip.TN, d_m1, col, g["conv2"], accumulate=True),
                           hip.gemm_desc(hip.TN, d_m2, st["x0"], g["residual_function.0.weight"], accumulate=True)],
                          stream=sm, splitk_ws=ctx.buf("splitk", (8 * (ci * cm + 9 * cm * cm + cm * ci),)))
         return d_x

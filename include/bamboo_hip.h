@@ -101,6 +101,14 @@ typedef struct bb_gemm_desc {
      * fp32 summation order.                                                                */
     float* colsum_out;
     float* colsum_ws;
+    /* BB_TN, bf16, unbatched only: with conv_c > 0, B is not a matrix in memory but the 3x3 / pad 1 patch
+     * matrix [K pixels, N = 9 * conv_c] of the NHWC tensor at B ([pixels, conv_c], images of conv_h x conv_w;
+     * column tap * conv_c + c of row p = the tensor at pixel p + shift(tap), zero outside the image), gathered
+     * by the operand loader: with A = dy this is the weight gradient of nn.Conv2d(k=3, padding=1)
+     * (resnet.py:58) in [out, 3, 3, in] order.  ldb is ignored; conv_c % 128 == 0; K % 32 == 0; B points at
+     * pixel 0 of the tensor and the K rows of the problem are its pixels conv_row0 .. conv_row0 + K - 1 (A's
+     * rows start at A as usual).  All four zero: an ordinary B.                                        */
+    int32_t conv_h, conv_w, conv_c, conv_row0;
 } bb_gemm_desc;
 
 /* library ------------------------------------------------------------------------------ */

@@ -499,6 +499,48 @@ def test_conv3x3_implicit_gemm(hiplib, n, h, w, cin, cout):
         assert rel_err(y, y3.double()) < 1e-2
 
 
+@pytest.mark.parametrize("n,h,w,c,cout", [(4, 6, 6, 128, 128),      # 144 pixels... rounded to 128 below; 32-pixel k-tiles cross image borders
+                                          (8, 4, 9, 128, 256),      # 288 pixels, images of 36 pixels: a k-tile nearly spans one
+                                          (32, 14, 14, 256, 256)])  # the ResNet-152 conv4_x block (6272 pixels)
+def test_conv3x3_weight_gradient_implicit_gemm(hiplib, n, h, w, c, cout):
+    """dW[o, tap, i] += sum_p dy[p, o] * x[p + shift(tap), i] with the patch matrix gathered inside the GEMM
+    (``conv=``): bit-equal to the same GEMM over the explicit patch matrix (same tiles, same order), alone,
+    in a group, and cut along the pixels; and equal to torch's conv2d weight gradient."""
+    dt = torch.bfloat16
+    rows = n * h * w // 32 * 32                                      # K must be a multiple of 32: drop the tail pixels
+    x_full = randn(n * h * w, c, dtype=dt, seed=70)
+    dy_full = randn(n * h * w, cout, dtype=dt, seed=71)
+    if rows != n * h * w:
+        dy_full[rows:] = 0                                           # ... by giving them no gradient
+    x, dy = x_full, dy_full[:rows]
+    col = torch.empty(n * h * w, 9 * c, dtype=dt, device=DEV)
+    hiplib.patch3x3(x_full, col, n, h, w, c)
+    base = randn(cout, 9 * c, seed=72)
+    want, got = base.clone(), base.clone()
+    hiplib.gemm_grouped([hiplib.gemm_desc(hiplib.TN, dy, col[:rows], want, accumulate=True)])
+    hiplib.gemm(hiplib.TN, dy, x[:rows], got, accumulate=True, conv=(h, w))
+    assert torch.equal(got, want)
+    xr = x_full.double().cpu().view(n, h, w, c).permute(0, 3, 1, 2)
+    wr = torch.zeros(cout, c, 3, 3, dtype=torch.float64, requires_grad=True)
+    torch.nn.functional.conv2d(xr, wr, padding=1).backward(dy_full.double().cpu().view(n, h, w, cout).permute(0, 3, 1, 2))
+    ref = wr.grad.permute(0, 2, 3, 1).reshape(cout, 9 * c)
+    assert rel_err(got.double().cpu() - base.double().cpu(), ref) < tol(dt)
+    # in a group with an ordinary problem, whole and cut along the contraction
+    a2, w2 = randn(rows, 256, dtype=dt, seed=73), randn(256, 128, seed=74)
+    for splitk in (False, True):
+        outs = []
+        for implicit in (False, True):
+            g1, g2 = base.clone(), w2.clone()
+            descs = [hiplib.gemm_desc(hiplib.TN, a2, dy[:, :128].contiguous(), g2, accumulate=True),
+                     hiplib.gemm_desc(hiplib.TN, dy, x[:rows], g1, accumulate=True, conv=(h, w)) if implicit
+                     else hiplib.gemm_desc(hiplib.TN, dy, col[:rows], g1, accumulate=True)]
+            ws = torch.empty(hiplib.gemm_splitk_workspace(descs) // 4, dtype=torch.float32, device=DEV) if splitk else None
+            hiplib.gemm_grouped(descs, splitk_ws=ws)
+            outs.append((g1, g2))
+        assert torch.equal(outs[0][0], outs[1][0]) and torch.equal(outs[0][1], outs[1][1])
+        assert rel_err(outs[1][0].double().cpu() - base.double().cpu(), ref) < tol(dt)
+
+
 def test_conv3x3_refuses_what_it_does_not_take(hiplib):
     dt = torch.bfloat16
     assert not hiplib.conv3x3_supported(dt, hiplib.CONV_FWD, 4, 6, 6, 16, 64)            # 16 gathered channels

@@ -223,7 +223,7 @@ def test_resnet_stage_matches_oracle_with_rc(hiplib, dtype, cin, cmid):
     redundant forwards of the shadow blocks, against the torch conv2d / batch_norm oracle.  With 128 middle
     channels the 3x3 convolution and its input gradient run as implicit GEMMs, with 16 through the patch matrix."""
     from bamboo_amd import BottleNeck
-    side, L, S, sid, mb, M = 6, 2, 4, 1, 4, 4
+    side, L, S, sid, mb, M = 6, 2, 4, 1, (8 if cmid == 128 else 4), 4     # 288 pixels: whole 32-pixel k-tiles for the weight gradient
     assert hiplib.conv3x3_supported(dtype, hiplib.CONV_DGRAD, mb, side, side, cmid, cmid) == (cmid == 128)
     specs = [LayerSpec(BottleNeck, cin, cmid, height=side, width=side) for _ in range(L * S)]
     model = PipelineModule(specs, num_stages=S, partition_method="uniform", stage_id=sid, dtype=dtype, device=DEV)
