@@ -1457,9 +1457,21 @@ extern "C" int bb_gemm_grouped(const bb_gemm_desc* descs, int count, void* strea
 // =========================================================================================
 constexpr int SPLITK_MAX = 8;
 
-__global__ __launch_bounds__(256) void splitk_reduce_kernel(const float* __restrict__ ws, int splits, int64_t part, int M,
-                                                            int N, float* __restrict__ C, int64_t ldc, int accumulate) {
-    const int64_t nvec = (int64_t)M * N / 4;
+// every problem of the group in one launch: blockIdx.y = problem
+struct SplitkReduceArgs {
+    const float* ws[GROUP_MAX];
+    float* C[GROUP_MAX];
+    int64_t ldc[GROUP_MAX];
+    int M[GROUP_MAX], N[GROUP_MAX], accumulate[GROUP_MAX];
+    int splits;
+};
+__global__ __launch_bounds__(256) void splitk_reduce_kernel(const SplitkReduceArgs a) {
+    const int pi = blockIdx.y;
+    const int M = a.M[pi], N = a.N[pi], splits = a.splits, accumulate = a.accumulate[pi];
+    const float* __restrict__ ws = a.ws[pi];
+    float* __restrict__ C = a.C[pi];
+    const int64_t ldc = a.ldc[pi], part = (int64_t)M * N;
+    const int64_t nvec = part / 4;
     for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < nvec; i += (int64_t)gridDim.x * 256) {
         const int64_t e = i * 4;
         const int m = (int)(e / N), n = (int)(e % N);
@@ -1541,15 +1553,20 @@ extern "C" int bb_gemm_grouped_splitk(const bb_gemm_desc* descs, int count, void
     }
     int rc = bb_gemm_grouped(sub, ns, stream);
     if (rc) return rc;
+    SplitkReduceArgs ra;
+    ra.splits = splits;
     ws = (float*)workspace;
+    int64_t most = 0;
     for (int i = 0; i < count; ++i) {
         const bb_gemm_desc& d = descs[i];
         const int64_t part = (int64_t)d.M * d.N;
-        const int64_t nvec = part / 4;
-        hipLaunchKernelGGL(splitk_reduce_kernel, dim3((unsigned)((nvec + 255) / 256 > 1024 ? 1024 : (nvec + 255) / 256)),
-                           dim3(256), 0, (hipStream_t)stream, ws, splits, part, d.M, d.N, (float*)d.C, d.ldc, d.accumulate);
+        ra.ws[i] = ws; ra.C[i] = (float*)d.C; ra.ldc[i] = d.ldc;
+        ra.M[i] = d.M; ra.N[i] = d.N; ra.accumulate[i] = d.accumulate;
+        most = part / 4 > most ? part / 4 : most;
         ws += (int64_t)splits * part;
     }
+    const unsigned bx = (unsigned)((most + 255) / 256 > 1024 ? 1024 : (most + 255) / 256);
+    hipLaunchKernelGGL(splitk_reduce_kernel, dim3(bx, (unsigned)count), dim3(256), 0, (hipStream_t)stream, ra);
     BB_LAUNCH_CHECK();
     return BB_OK;
 }
