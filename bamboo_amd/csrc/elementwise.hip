@@ -912,6 +912,69 @@ __global__ __launch_bounds__(256) void bn_finish_kernel(int what, int rows, int 
     }
 }
 
+// Forward statistics from the strip triples a convolution's GEMM epilogue leaves (per 32 rows and channel:
+// pivot p, S1 = sum (x - p), S2 = sum (x - p)^2).  A strip's mean is p + S1/n and its sum of squared deviations
+// M2 = S2 - S1^2/n (no cancellation: p is a sample of the strip).  Two passes over the triples, which stay in
+// registers (at most 8192 rows): mean = sum n_s mean_s / rows, then sum of squared deviations = sum (M2_s + n_s (mean_s - mean)^2) -
+// again no cancellation.  One block owns 64 channels (lane = channel: 256-byte reads); its sixteen waves take
+// strips w, w + 16, ...; the sixteen partial sums are added in wave order by every thread (fixed order).
+constexpr int BN_STRIP_WAVES = 16, BN_STRIP_MAX = 16;   // 16 * 16 strips = up to 8192 rows
+__global__ __launch_bounds__(BN_STRIP_WAVES * 64) void bn_finish_strips_kernel(int rows, int cols, float eps, float momentum,
+                                                               const float* __restrict__ strips, float* __restrict__ mean,
+                                                               float* __restrict__ rstd, float* __restrict__ run_mean,
+                                                               float* __restrict__ run_var) {
+    __shared__ float red[2][BN_STRIP_WAVES][64];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int c = min(blockIdx.x * 64 + lane, cols - 1);   // lanes past the last channel repeat it and store nothing
+    const int nstrips = (rows + 31) / 32;
+    float p[BN_STRIP_MAX], a[BN_STRIP_MAX], b[BN_STRIP_MAX];
+#pragma unroll
+    for (int j = 0; j < BN_STRIP_MAX; ++j) {
+        const int s = min(j * BN_STRIP_WAVES + wave, nstrips - 1);   // clamped: every load is issued, unused ones get n = 0
+        const float* t = strips + ((int64_t)s * 3) * cols + c;
+        p[j] = t[0];
+        a[j] = t[cols];
+        b[j] = t[2 * (int64_t)cols];
+    }
+    float sm = 0.f;
+#pragma unroll
+    for (int j = 0; j < BN_STRIP_MAX; ++j) {
+        const int s = j * BN_STRIP_WAVES + wave;
+        const int cnt = s < nstrips ? min(32, rows - s * 32) : 0;
+        const float n = (float)cnt, inv = cnt == 32 ? 0.03125f : cnt > 0 ? 1.0f / n : 0.f;
+        const float m = p[j] + a[j] * inv;           // the strip's mean
+        b[j] = cnt > 0 ? b[j] - a[j] * a[j] * inv : 0.f;   // its sum of squared deviations
+        p[j] = m;
+        a[j] = n;
+        sm += n * m;
+    }
+    red[0][wave][lane] = sm;
+    __syncthreads();
+    float tot = 0.f;
+#pragma unroll
+    for (int w = 0; w < BN_STRIP_WAVES; ++w) tot += red[0][w][lane];
+    const float mu = tot / (float)rows;
+    float sq = 0.f;
+#pragma unroll
+    for (int j = 0; j < BN_STRIP_MAX; ++j) {
+        const float d = p[j] - mu;
+        sq += b[j] + a[j] * d * d;
+    }
+    red[1][wave][lane] = sq;
+    __syncthreads();
+    if (wave != 0 || blockIdx.x * 64 + lane >= cols) return;
+    float q = 0.f;
+#pragma unroll
+    for (int w = 0; w < BN_STRIP_WAVES; ++w) q += red[1][w][lane];
+    const float var = fmaxf(q / (float)rows, 0.f);
+    mean[c] = mu;
+    rstd[c] = 1.0f / sqrtf(var + eps);
+    if (run_mean) {  // nn.BatchNorm2d: running_var uses the unbiased estimate
+        run_mean[c] = (1.f - momentum) * run_mean[c] + momentum * mu;
+        run_var[c] = (1.f - momentum) * run_var[c] + momentum * var * (float)rows / (float)(rows - 1);
+    }
+}
+
 // forward apply: y = gamma * (x - mean) * rstd + beta (+ resid), optional ReLU
 template <typename T>
 __global__ __launch_bounds__(256) void bn_apply_kernel(int64_t nvec, int cols, int relu, const T* __restrict__ x,
@@ -1031,6 +1094,26 @@ extern "C" int bb_batchnorm_fwd(int dtype, int rows, int cols, float eps, float 
         hipLaunchKernelGGL(bn_finish_kernel<float>, fgrid, dim3(256), 0, st, 1, rows, cols, eps, momentum, workspace, (const float*)x, mean, rstd, running_mean, running_var, nullptr, nullptr, nullptr);
         hipLaunchKernelGGL(bn_apply_kernel<float>, dim3(grid_for(nvec)), dim3(256), 0, st, nvec, cols, relu, (const float*)x, mean, rstd, (const float*)gamma, (const float*)beta, (const float*)resid, (float*)y);
     }
+    BB_LAUNCH_CHECK();
+    return BB_OK;
+}
+
+extern "C" int bb_batchnorm_fwd_strips(int dtype, int rows, int cols, float eps, float momentum, int relu, const void* x,
+                                       const void* gamma, const void* beta, const void* resid, void* y, float* mean,
+                                       float* rstd, float* running_mean, float* running_var, const float* strip_stats,
+                                       void* stream) {
+    int rc = check_bn("bb_batchnorm_fwd_strips", dtype, rows, cols);
+    if (rc) return rc;
+    BB_REQUIRE(dtype == BB_BF16, "bb_batchnorm_fwd_strips: bf16 only (the kernels that leave strip statistics are)");
+    BB_REQUIRE(x && gamma && beta && y && mean && rstd && strip_stats, "bb_batchnorm_fwd_strips: null pointer");
+    BB_REQUIRE(rows <= 32 * BN_STRIP_WAVES * BN_STRIP_MAX, "bb_batchnorm_fwd_strips: at most %d rows", 32 * BN_STRIP_WAVES * BN_STRIP_MAX);
+    BB_REQUIRE((running_mean == nullptr) == (running_var == nullptr), "bb_batchnorm_fwd_strips: give both running buffers or none");
+    hipStream_t st = (hipStream_t)stream;
+    const int64_t nvec = (int64_t)rows * cols / 8;
+    hipLaunchKernelGGL(bn_finish_strips_kernel, dim3((cols + 63) / 64), dim3(BN_STRIP_WAVES * 64), 0, st, rows, cols, eps, momentum, strip_stats,
+                       mean, rstd, running_mean, running_var);
+    hipLaunchKernelGGL(bn_apply_kernel<bf16>, dim3(grid_for(nvec)), dim3(256), 0, st, nvec, cols, relu, (const bf16*)x, mean, rstd,
+                       (const bf16*)gamma, (const bf16*)beta, (const bf16*)resid, (bf16*)y);
     BB_LAUNCH_CHECK();
     return BB_OK;
 }

@@ -26,6 +26,7 @@ struct GemmArgs {
     int epilogue, act, accumulate, c_f32;
     int tiles_m, tiles_n;
     int conv_h, conv_w, conv_c, conv_row0;  // TN: B is the 3x3 patch matrix of an NHWC tensor (conv_c > 0)
+    float* strip_stats;  // [ceil(M / 32)][3][N]: per 32-row strip and output column (pivot, sum (c - pivot), sum (c - pivot)^2)
 };
 
 // ---- tile order: consecutive logical tiles land on the same XCD (workgroups are dealt
@@ -562,7 +563,10 @@ template <int BR, int T, bool KM, int BK = 32> struct FragReader {
     }
 };
 
-template <int BM, int BN, int WM, int WN, bool AKM, bool BKM, bool DB, int STAGES, int BK = 32, bool VIS = false, int CONV = 0>
+// STATS: the epilogue also leaves the column statistics of the stored (bf16-rounded) output per 32-row strip, for the
+// batch normalisation that follows a convolution (its statistics pass then has nothing left to read).
+template <int BM, int BN, int WM, int WN, bool AKM, bool BKM, bool DB, int STAGES, int BK = 32, bool VIS = false, int CONV = 0,
+          bool STATS = false>
 __device__ __forceinline__ void gemm_bf16_dma_body(const GemmArgs& g, const int block_id, const int batch_id,
                                                    const bool logical_id = false, const ConvArgs& cv = ConvArgs{}) {
     constexpr int NW = WM * WN;
@@ -888,6 +892,29 @@ __device__ __forceinline__ void gemm_bf16_dma_body(const GemmArgs& g, const int 
                 }
                 if (live && m < g.M && n < g.N) epilogue_vec8(g, coff, m, n, v);
             }
+            if constexpr (STATS) {
+                // Column statistics of this 32-row strip straight from the patch: lane = column, 32 conflict-free LDS
+                // reads.  The patch holds what is stored (alpha = 1, no bias, no epilogue), rounded here as the
+                // store rounds it; the pivot is the strip's first row.
+                const int strip_row = m0 + wm * WTM + i * 32, nrows = min(32, g.M - strip_row);
+                const int nc = n0 + wn * WTN + jp * 64 + lane;
+                const float piv = bf2f(f2bf(patch[lane]));
+                float s1 = 0.f, s2 = 0.f;
+#pragma unroll
+                for (int r = 0; r < 32; ++r) {
+                    const float dv = bf2f(f2bf(patch[r * PLD + lane])) - piv;
+                    if (r < nrows) {
+                        s1 += dv;
+                        s2 += dv * dv;
+                    }
+                }
+                if (g.strip_stats && nrows > 0 && nc < g.N && (NH == 2 || lane < 32)) {
+                    float* o = g.strip_stats + ((int64_t)(strip_row >> 5) * 3) * g.N + nc;
+                    o[0] = piv;
+                    o[g.N] = s1;
+                    o[2 * (int64_t)g.N] = s2;
+                }
+            }
             asm volatile("" ::: "memory");
         },
         std::make_integer_sequence<int, TM * NP>{});
@@ -897,12 +924,17 @@ template <int BM, int BN, int WM, int WN, bool AKM, bool BKM, bool DB, int STAGE
 __global__ __launch_bounds__(WM* WN * 64) void gemm_bf16_dma_kernel(const GemmArgs g) {
     gemm_bf16_dma_body<BM, BN, WM, WN, AKM, BKM, DB, STAGES, BK>(g, blockIdx.x, blockIdx.z);
 }
+// the same with the strip statistics of the output (NT, 64-wide k-tiles, three stages)
+template <int BM, int BN, int WM, int WN>
+__global__ __launch_bounds__(WM* WN * 64) void gemm_bf16_dma_stats_kernel(const GemmArgs g) {
+    gemm_bf16_dma_body<BM, BN, WM, WN, false, false, true, 3, 64, false, 0, true>(g, blockIdx.x, blockIdx.z);
+}
 
 // 3x3 convolution as an implicit GEMM: forward (BKM = false: y = patches(x) W^T) and input gradient
 // (BKM = true: dx = patches(dy) W_flipped) on the same main loop, operands gathered by the loaders.
-template <int BM, int BN, int WM, int WN, bool BKM, int STAGES>
+template <int BM, int BN, int WM, int WN, bool BKM, int STAGES, bool STATS = false>
 __global__ __launch_bounds__(WM* WN * 64) void conv3x3_bf16_igemm_kernel(const GemmArgs g, const ConvArgs cv) {
-    gemm_bf16_dma_body<BM, BN, WM, WN, false, BKM, true, STAGES, 64, false, BKM ? 2 : 1>(g, blockIdx.x, 0, false, cv);
+    gemm_bf16_dma_body<BM, BN, WM, WN, false, BKM, true, STAGES, 64, false, BKM ? 2 : 1, STATS>(g, blockIdx.x, 0, false, cv);
 }
 
 // Several independent problems of one kind in a single launch (the four weight-gradient GEMMs
@@ -1086,6 +1118,22 @@ static int launch_bf16_dma(GemmArgs& g, int batches, hipStream_t st) {
     g.tiles_n = (g.N + BN - 1) / BN;
     dim3 grid(g.tiles_m * g.tiles_n, 1, batches);
     hipLaunchKernelGGL(kern, grid, dim3(WM * WN * 64), smem, st, g);
+    BB_LAUNCH_CHECK();
+    return BB_OK;
+}
+
+template <int BM, int BN, int WM, int WN>
+static int launch_bf16_dma_stats(GemmArgs& g, hipStream_t st) {
+    constexpr int smem = 3 * (BM + BN) * 64 * 2;
+    auto kern = gemm_bf16_dma_stats_kernel<BM, BN, WM, WN>;
+    static bool configured = false;
+    if (!configured) {
+        BB_HIP_CHECK(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, smem));
+        configured = true;
+    }
+    g.tiles_m = (g.M + BM - 1) / BM;
+    g.tiles_n = (g.N + BN - 1) / BN;
+    hipLaunchKernelGGL(kern, dim3(g.tiles_m * g.tiles_n), dim3(WM * WN * 64), smem, st, g);
     BB_LAUNCH_CHECK();
     return BB_OK;
 }
@@ -1283,6 +1331,7 @@ static int fill_args(const bb_gemm_desc* d, GemmArgs& g, int64_t& batches, bool&
     BB_REQUIRE(!d->colsum_out || d->layout == BB_TN, "bb_gemm: colsum_out needs the BB_TN layout");
     g.lda = d->lda; g.ldb = ldb; g.ldc = d->ldc; g.ldaux = d->ldaux > 0 ? d->ldaux : d->ldc;
     g.conv_h = d->conv_h; g.conv_w = d->conv_w; g.conv_c = d->conv_c; g.conv_row0 = d->conv_row0;
+    g.strip_stats = nullptr;   // bb_gemm sets it where the kernel that runs the problem produces them
     g.sA1 = d->sA1; g.sA2 = d->sA2; g.sB1 = d->sB1; g.sB2 = d->sB2; g.sC1 = d->sC1; g.sC2 = d->sC2;
     g.alpha = d->alpha;
     g.epilogue = d->epilogue; g.act = d->act; g.accumulate = d->accumulate;
@@ -1301,8 +1350,29 @@ static int colsum_standalone(const bb_gemm_desc* d, void* stream) {
     return bb_colsum_acc(d->dtype, d->K, d->M, d->A, d->lda, d->colsum_out, d->colsum_ws, stream);
 }
 
+extern "C" int bb_gemm_strip_stats_supported(const bb_gemm_desc* d) {
+    return d && d->dtype == BB_BF16 && d->c_dtype == BB_BF16 && d->layout == BB_NT && d->nb1 <= 1 && d->nb2 <= 1 &&
+           d->M >= 128 && d->N >= 64 && d->N % 8 == 0 && d->K >= 128 && d->K % 64 == 0 && d->conv_c == 0 && !d->colsum_out &&
+           !d->bias && d->epilogue == BB_EPI_NONE && d->alpha == 1.0f && dma_tile_override() == 0;
+}
+extern "C" int64_t bb_strip_stats_workspace(int rows, int cols) { return (int64_t)((rows + 31) / 32) * 3 * cols; }
+
 extern "C" int bb_gemm(const bb_gemm_desc* d, void* stream) {
     if (d && d->conv_c != 0) return bb_gemm_grouped(d, 1, stream);   // only the grouped kernel gathers a patch-matrix B
+    if (d && d->strip_stats) {
+        BB_REQUIRE(bb_gemm_strip_stats_supported(d), "bb_gemm: strip_stats needs an unbatched bf16 BB_NT problem with a bf16 C, "
+                   "M >= 128, N >= 64, N %% 8 == 0, K >= 128, K %% 64 == 0, alpha = 1, no bias, no epilogue");
+        BB_REQUIRE(((uintptr_t)d->strip_stats % 16) == 0, "bb_gemm: strip_stats must be 16-byte aligned");
+        GemmArgs g;
+        int64_t batches;
+        bool ta, tb;
+        int rc = fill_args(d, g, batches, ta, tb);
+        if (rc) return rc;
+        g.strip_stats = d->strip_stats;
+        // the two tiles that carry the statistics: 256x128 where the ordinary choice would be that tile, else 128x64
+        if (pick_dma_tile(d->M, d->N, d->K, 1, BB_NT) == D256x128k64s3) return launch_bf16_dma_stats<256, 128, 4, 2>(g, (hipStream_t)stream);
+        return launch_bf16_dma_stats<128, 64, 4, 1>(g, (hipStream_t)stream);
+    }
     GemmArgs g;
     int64_t batches;
     bool ta, tb;
@@ -1324,10 +1394,10 @@ extern "C" int bb_gemm(const bb_gemm_desc* d, void* stream) {
     return dispatch_f32<true, true>(g, (int)batches, st);
 }
 
-template <int BM, int BN, int WM, int WN, bool BKM, int STAGES>
+template <int BM, int BN, int WM, int WN, bool BKM, int STAGES, bool STATS = false>
 static int launch_conv3x3(GemmArgs& g, const ConvArgs& cv, hipStream_t st) {
     constexpr int smem = STAGES * (BM + BN) * 64 * 2;
-    auto kern = conv3x3_bf16_igemm_kernel<BM, BN, WM, WN, BKM, STAGES>;
+    auto kern = conv3x3_bf16_igemm_kernel<BM, BN, WM, WN, BKM, STAGES, STATS>;
     static bool configured = false;
     if (!configured) {
         BB_HIP_CHECK(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, smem));
@@ -1349,8 +1419,10 @@ extern "C" int bb_conv3x3_supported(int dtype, int mode, int n, int h, int w, in
 }
 
 extern "C" int bb_conv3x3(int dtype, int mode, int n, int h, int w, int cin, int cout, const void* src, const void* weight,
-                          void* dst, void* stream) {
+                          void* dst, float* strip_stats, void* stream) {
     BB_REQUIRE(src && weight && dst, "bb_conv3x3: null operand");
+    BB_REQUIRE(!strip_stats || (mode == BB_CONV_FWD && ((uintptr_t)strip_stats % 16) == 0),
+               "bb_conv3x3: strip_stats goes with BB_CONV_FWD only and must be 16-byte aligned");
     BB_REQUIRE(bb_conv3x3_supported(dtype, mode, n, h, w, cin, cout),
                "bb_conv3x3: unsupported problem (bf16, >= 128 pixels, gathered channels a multiple of 64, produced channels "
                "a multiple of 8 and >= 64): dtype %d mode %d n %d h %d w %d cin %d cout %d",
@@ -1376,6 +1448,10 @@ extern "C" int bb_conv3x3(int dtype, int mode, int n, int h, int w, int cin, int
         // B = the weight as it lies: [cout, 9 * cin], k-contiguous
         g.B = weight;
         g.ldb = 9 * (int64_t)cin;
+        if (strip_stats) {
+            g.strip_stats = strip_stats;
+            return launch_conv3x3<128, 64, 4, 1, false, 3, true>(g, cv, st);
+        }
         return launch_conv3x3<128, 64, 4, 1, false, 3>(g, cv, st);
     }
     // B[k = t * cout + o, n = i] = weight[o, 8 - t, i]: k-major with row stride 9 * cin, starting at tap 8; after

@@ -25,7 +25,7 @@ LN_CODES = {"standard": LN_STANDARD, "annotated": LN_ANNOTATED}
 EXPORTS = (
     "bb_version", "bb_last_error", "bb_init", "bb_gemm", "bb_gemm_grouped", "bb_gemm_splitk_workspace", "bb_gemm_grouped_splitk", "bb_gemm_variant", "bb_layernorm_fwd",
     "bb_layernorm_bwd_workspace", "bb_layernorm_bwd", "bb_colsum_workspace", "bb_colsum_acc",
-    "bb_softmax_fwd", "bb_softmax_bwd", "bb_attention_fwd", "bb_attention_bwd", "bb_residual_add", "bb_act_fwd", "bb_bn_workspace", "bb_batchnorm_fwd", "bb_batchnorm_bwd", "bb_patch3x3", "bb_conv3x3_supported", "bb_conv3x3", "bb_mse_workspace", "bb_mse_fwd_bwd", "bb_graph_begin", "bb_graph_end", "bb_graph_launch", "bb_graph_destroy",
+    "bb_softmax_fwd", "bb_softmax_bwd", "bb_attention_fwd", "bb_attention_bwd", "bb_residual_add", "bb_act_fwd", "bb_bn_workspace", "bb_batchnorm_fwd", "bb_batchnorm_bwd", "bb_patch3x3", "bb_conv3x3_supported", "bb_conv3x3", "bb_gemm_strip_stats_supported", "bb_strip_stats_workspace", "bb_batchnorm_fwd_strips", "bb_mse_workspace", "bb_mse_fwd_bwd", "bb_graph_begin", "bb_graph_end", "bb_graph_launch", "bb_graph_destroy",
     "bb_adam_multi", "bb_cast", "bb_fill_f32",
 )
 
@@ -48,6 +48,7 @@ class GemmDesc(Structure):
         ("bias", c_void_p), ("aux_in", c_void_p), ("aux_out", c_void_p), ("resid", c_void_p),
         ("ldaux", c_int64), ("colsum_out", c_void_p), ("colsum_ws", c_void_p),
         ("conv_h", c_int32), ("conv_w", c_int32), ("conv_c", c_int32), ("conv_row0", c_int32),
+        ("strip_stats", c_void_p),
     ]
 
 
@@ -104,7 +105,11 @@ def lib():
     L.bb_batchnorm_bwd.argtypes = [c_int, c_int, c_int] + [c_void_p] * 12
     L.bb_patch3x3.argtypes = [c_int, c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p]
     L.bb_conv3x3_supported.argtypes = [c_int] * 7
-    L.bb_conv3x3.argtypes = [c_int] * 7 + [c_void_p] * 4
+    L.bb_conv3x3.argtypes = [c_int] * 7 + [c_void_p] * 5
+    L.bb_gemm_strip_stats_supported.argtypes = [POINTER(GemmDesc)]
+    L.bb_strip_stats_workspace.argtypes = [c_int, c_int]
+    L.bb_strip_stats_workspace.restype = c_int64
+    L.bb_batchnorm_fwd_strips.argtypes = [c_int, c_int, c_int, c_float, c_float, c_int] + [c_void_p] * 11
     L.bb_mse_workspace.restype = c_int64
     L.bb_mse_fwd_bwd.argtypes = [c_int, c_int64, c_void_p, c_void_p, c_void_p, c_float, c_void_p, c_int,
                                  c_void_p, c_void_p]
@@ -153,7 +158,7 @@ def _row_major(t, name):
 
 # ------------------------------------------------------------------------------------- GEMM
 def gemm_desc(layout, A, B, C, *, alpha=1.0, bias=None, epilogue=EPI_NONE, act=ACT_RELU, accumulate=False,
-              aux_in=None, aux_out=None, resid=None, colsum_out=None, colsum_ws=None, conv=None):
+              aux_in=None, aux_out=None, resid=None, colsum_out=None, colsum_ws=None, conv=None, strip_stats=None):
     """Descriptor of C = epilogue(alpha * op(A) op(B) [+ bias]) on 2-D row-major views.
     ``conv=(h, w)`` (TN only): B is the NHWC tensor ``[pixels, c]`` whose 3x3 patch matrix ``[pixels, 9c]`` is
     the operand, gathered inside the kernel (weight gradient of a 3x3 convolution)."""
@@ -205,7 +210,25 @@ def gemm_desc(layout, A, B, C, *, alpha=1.0, bias=None, epilogue=EPI_NONE, act=A
             raise HipKernelError("gemm: colsum_ws too small")
         d.colsum_out = colsum_out.data_ptr()
         d.colsum_ws = None if colsum_ws is None else colsum_ws.data_ptr()
+    if strip_stats is not None:
+        _check_strip_stats(strip_stats, M, N)
+        d.strip_stats = strip_stats.data_ptr()
     return d
+
+
+def strip_stats_workspace(rows, cols):
+    """fp32 elements of the per-32-row-strip column statistics a GEMM / convolution leaves for batchnorm_fwd."""
+    return int(lib().bb_strip_stats_workspace(rows, cols))
+
+
+def _check_strip_stats(t, rows, cols):
+    if t.dtype != torch.float32 or not t.is_contiguous() or t.numel() < strip_stats_workspace(rows, cols):
+        raise HipKernelError(f"strip_stats must be a contiguous fp32 tensor of >= {strip_stats_workspace(rows, cols)} elements")
+
+
+def gemm_strip_stats_supported(layout, A, B, C):
+    """Whether ``gemm(layout, A, B, C, strip_stats=...)`` is taken (bf16 NT problems of the convolution shapes)."""
+    return bool(lib().bb_gemm_strip_stats_supported(byref(gemm_desc(layout, A, B, C))))
 
 
 def gemm(layout, A, B, C, *, stream=None, **kw):
@@ -392,8 +415,17 @@ def bn_workspace(cols):
     return int(lib().bb_bn_workspace(cols))
 
 
-def batchnorm_fwd(x, gamma, beta, resid, y, mean, rstd, run_mean, run_var, workspace, eps, momentum, relu, stream=None):
+def batchnorm_fwd(x, gamma, beta, resid, y, mean, rstd, run_mean, run_var, workspace, eps, momentum, relu, stream=None,
+                  strip_stats=None):
+    """``strip_stats``: the statistics the kernel that produced ``x`` left (``gemm(..., strip_stats=)``,
+    ``conv3x3(..., strip_stats=)``); the statistics pass over ``x`` is then skipped."""
     rows, cols = x.shape
+    if strip_stats is not None:
+        _check_strip_stats(strip_stats, rows, cols)
+        check(lib().bb_batchnorm_fwd_strips(dtype_code(x.dtype), rows, cols, eps, momentum, int(relu), _ptr(x), _ptr(gamma),
+                                            _ptr(beta), _ptr(resid), _ptr(y), _ptr(mean), _ptr(rstd), _ptr(run_mean),
+                                            _ptr(run_var), _ptr(strip_stats), stream_ptr(stream)), "bb_batchnorm_fwd_strips")
+        return
     if workspace.numel() < bn_workspace(cols):
         raise HipKernelError("batchnorm_fwd: workspace too small")
     check(lib().bb_batchnorm_fwd(dtype_code(x.dtype), rows, cols, eps, momentum, int(relu), _ptr(x), _ptr(gamma),
@@ -423,7 +455,7 @@ def conv3x3_supported(dtype, mode, n, h, w, cin, cout):
     return bool(lib().bb_conv3x3_supported(dtype_code(dtype), mode, n, h, w, cin, cout))
 
 
-def conv3x3(mode, src, weight, dst, n, h, w, cin, cout, stream=None):
+def conv3x3(mode, src, weight, dst, n, h, w, cin, cout, strip_stats=None, stream=None):
     """``CONV_FWD``: dst[n*h*w, cout] = conv3x3(src[n*h*w, cin]); ``CONV_DGRAD``: dst[n*h*w, cin] = the input
     gradient for src = dy[n*h*w, cout]; weight [cout, 3, 3, cin]."""
     rows = n * h * w
@@ -435,8 +467,10 @@ def conv3x3(mode, src, weight, dst, n, h, w, cin, cout, stream=None):
         raise HipKernelError("conv3x3: operands must be contiguous")
     if not (src.dtype == weight.dtype == dst.dtype):
         raise HipKernelError("conv3x3: operands must share one dtype")
+    if strip_stats is not None:
+        _check_strip_stats(strip_stats, rows, cout)
     call = lambda: check(lib().bb_conv3x3(dtype_code(src.dtype), mode, n, h, w, cin, cout, _ptr(src), _ptr(weight),
-                                          _ptr(dst), stream_ptr(stream)), "bb_conv3x3")
+                                          _ptr(dst), _ptr(strip_stats), stream_ptr(stream)), "bb_conv3x3")
     if gemm_hook is not None:
         gemm_hook(ConvLaunch(mode, rows, cin, cout), call, stream)
     else:

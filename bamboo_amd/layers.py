@@ -316,6 +316,7 @@ class BottleNeck:
         self.eps, self.momentum = bn_eps, bn_momentum
         self.w_ = self.g_ = None
         self.running = None
+        self._stats_ok = {}    # (shapes, dtype) -> whether the GEMM of a 1x1 convolution leaves strip statistics
 
     @property
     def feature_dim(self):
@@ -380,10 +381,12 @@ class BottleNeck:
         # split-K partial products of the three weight gradients (8 chunks of each, fp32)
         nws = 8 * (ci * cm + 9 * cm * cm + cm * ci)
         return [("col", (R, 9 * cm), dt), ("d_col", (R, 9 * cm), dt), ("d_y3", (R, ci), dt), ("d_res", (R, ci), dt),
-                ("d_m0", (R, cm), dt), ("d_m1", (R, cm), dt), ("d_m2", (R, cm), dt), ("splitk", (nws,), torch.float32)]
+                ("d_m0", (R, cm), dt), ("d_m1", (R, cm), dt), ("d_m2", (R, cm), dt), ("splitk", (nws,), torch.float32),
+                ("strips", (hip.strip_stats_workspace(R, ci),), torch.float32)]
 
     def forward_scratch_specs(self, ctx):
-        return [("col", (ctx.rows, 9 * self.cmid), ctx.dtype)]
+        return [("col", (ctx.rows, 9 * self.cmid), ctx.dtype),
+                ("strips", (hip.strip_stats_workspace(ctx.rows, self.cin),), torch.float32)]
 
     def workspace_elems(self):
         return max(hip.bn_workspace(self.cin), hip.colsum_workspace(self.cin))
@@ -397,11 +400,23 @@ class BottleNeck:
             self.running = {i: (z(n, 0.0), z(n, 1.0)) for i, n in ((1, self.cmid), (4, self.cmid), (7, self.cin))}
         return self.running
 
-    def _bn_fwd(self, idx, x, resid, y, mean, rstd, relu, ctx):
+    def _bn_fwd(self, idx, x, resid, y, mean, rstd, relu, ctx, strips=None):
         run = (None, None) if ctx.redundant else self._running(x.device)[idx]
         hip.batchnorm_fwd(x, self.w_[f"residual_function.{idx}.weight"], self.w_[f"residual_function.{idx}.bias"],
                           resid, y, mean, rstd, run[0], run[1], ctx.workspace, self.eps, self.momentum, relu,
-                          stream=ctx.stream)
+                          stream=ctx.stream, strip_stats=strips)
+
+    def _conv1x1(self, x, weight, y, ctx):
+        """1x1 convolution = GEMM on the NHWC rows; where the kernel can, it also leaves the strip statistics of
+        its output for the BatchNorm that follows (returned, else None: that BatchNorm then reads y for them)."""
+        strips = None
+        key = (tuple(x.shape), tuple(weight.shape), x.dtype)
+        if key not in self._stats_ok:
+            self._stats_ok[key] = ctx.rows <= 8192 and hip.gemm_strip_stats_supported(hip.NT, x, weight, y)
+        if self._stats_ok[key]:
+            strips = ctx.buf("strips", (hip.strip_stats_workspace(ctx.rows, y.shape[1]),))
+        hip.gemm(hip.NT, x, weight, y, stream=ctx.stream, strip_stats=strips)
+        return strips
 
     def _implicit(self, ctx, mode):
         return hip.conv3x3_supported(ctx.dtype, mode, ctx.batch, self.h, self.w, self.cmid, self.cmid)
@@ -411,18 +426,19 @@ class BottleNeck:
             raise hip.HipKernelError(f"activation has {ctx.seq} positions, the block expects {self.h}x{self.w}")
         w, sm = self.w_, ctx.stream
         st["x0"] = x
-        hip.gemm(hip.NT, x, w["residual_function.0.weight"], st["y1"], stream=sm)
-        self._bn_fwd(1, st["y1"], None, st["a1"], st["mean1"], st["rstd1"], True, ctx)
+        strips = self._conv1x1(x, w["residual_function.0.weight"], st["y1"], ctx)
+        self._bn_fwd(1, st["y1"], None, st["a1"], st["mean1"], st["rstd1"], True, ctx, strips)
         if self._implicit(ctx, hip.CONV_FWD):
+            strips = ctx.buf("strips", (hip.strip_stats_workspace(ctx.rows, self.cmid),)) if ctx.rows <= 8192 else None
             hip.conv3x3(hip.CONV_FWD, st["a1"], w["residual_function.3.weight"], st["y2"], ctx.batch, self.h, self.w,
-                        self.cmid, self.cmid, stream=sm)
+                        self.cmid, self.cmid, strip_stats=strips, stream=sm)
         else:
             col = ctx.buf("col", (ctx.rows, 9 * self.cmid))
             hip.patch3x3(st["a1"], col, ctx.batch, self.h, self.w, self.cmid, stream=sm)
-            hip.gemm(hip.NT, col, w["conv2"], st["y2"], stream=sm)
-        self._bn_fwd(4, st["y2"], None, st["a2"], st["mean2"], st["rstd2"], True, ctx)
-        hip.gemm(hip.NT, st["a2"], w["residual_function.6.weight"], st["y3"], stream=sm)
-        self._bn_fwd(7, st["y3"], x, st["out"], st["mean3"], st["rstd3"], True, ctx)
+            strips = self._conv1x1(col, w["conv2"], st["y2"], ctx)
+        self._bn_fwd(4, st["y2"], None, st["a2"], st["mean2"], st["rstd2"], True, ctx, strips)
+        strips = self._conv1x1(st["a2"], w["residual_function.6.weight"], st["y3"], ctx)
+        self._bn_fwd(7, st["y3"], x, st["out"], st["mean3"], st["rstd3"], True, ctx, strips)
         return st["out"]
 
     def backward(self, d_out, d_x, st, ctx):

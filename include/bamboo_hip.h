@@ -109,6 +109,12 @@ typedef struct bb_gemm_desc {
      * pixel 0 of the tensor and the K rows of the problem are its pixels conv_row0 .. conv_row0 + K - 1 (A's
      * rows start at A as usual).  All four zero: an ordinary B.                                        */
     int32_t conv_h, conv_w, conv_c, conv_row0;
+    /* bb_gemm only, where bb_gemm_strip_stats_supported() says so: the kernel also leaves, per strip of 32
+     * consecutive rows of C and per column, the triple (pivot = the strip's first row, sum (c - pivot),
+     * sum (c - pivot)^2) of the stored bf16 values: strip_stats[(strip * 3 + j) * N + n], fp32,
+     * >= bb_strip_stats_workspace(M, N) floats.  bb_batchnorm_fwd_strips turns them into the batch statistics
+     * of nn.BatchNorm2d without reading C again (resnet.py:55-62: every convolution feeds a BatchNorm).    */
+    float* strip_stats;
 } bb_gemm_desc;
 
 /* library ------------------------------------------------------------------------------ */
@@ -122,6 +128,8 @@ int bb_init(void);
  * (engine.py:1701-1709 torch.autograd.backward).  bf16 needs K, lda, ldb, ldc % 8 == 0;
  * fp32 needs them % 4 == 0.                                                               */
 int bb_gemm(const bb_gemm_desc* desc, void* stream);
+int bb_gemm_strip_stats_supported(const bb_gemm_desc* desc);
+int64_t bb_strip_stats_workspace(int rows, int cols);
 /* `count` independent GEMMs of one layout/dtype; results are identical to calling bb_gemm on
  * each descriptor in turn.  When all are unbatched bf16 problems they share one launch, which
  * is how the four weight-gradient products of a layer (autograd of transformer.py:136-146,158)
@@ -209,6 +217,13 @@ int64_t bb_bn_workspace(int cols);
 int bb_batchnorm_fwd(int dtype, int rows, int cols, float eps, float momentum, int relu, const void* x,
                      const void* gamma, const void* beta, const void* resid, void* y, float* mean,
                      float* rstd, float* running_mean, float* running_var, float* workspace, void* stream);
+/* bb_batchnorm_fwd with the statistics pass replaced by the strip statistics of x that the kernel which
+ * produced x left behind (bb_gemm_desc.strip_stats, bb_conv3x3): same outputs up to the fp32 rounding of the
+ * statistics (strips are merged with the pairwise update of Chan et al., no cancellation).  bf16 only.      */
+int bb_batchnorm_fwd_strips(int dtype, int rows, int cols, float eps, float momentum, int relu, const void* x,
+                            const void* gamma, const void* beta, const void* resid, void* y, float* mean,
+                            float* rstd, float* running_mean, float* running_var, const float* strip_stats,
+                            void* stream);
 /* Backward through (optional ReLU given by its output relu_out) and the batch normalisation:
  * g = dy * (relu_out > 0); dgamma += sum g*xhat; dbeta += sum g;
  * dx = gamma * rstd * (g - mean(g) - xhat * mean(g*xhat)); g_out (optional) receives g.       */
@@ -230,7 +245,7 @@ int bb_patch3x3(int dtype, int adjoint, int n, int h, int w, int c, const void* 
 #define BB_CONV_DGRAD 1
 int bb_conv3x3_supported(int dtype, int mode, int n, int h, int w, int cin, int cout);
 int bb_conv3x3(int dtype, int mode, int n, int h, int w, int cin, int cout, const void* src, const void* weight,
-               void* dst, void* stream);
+               void* dst, float* strip_stats /* BB_CONV_FWD: as bb_gemm_desc.strip_stats, or NULL */, void* stream);
 
 /* Mean-squared-error head (nn.MSELoss, transformer.py:264) fused with its gradient:
  * loss_out[0] (+)= mean((y-t)^2);  dy = grad_scale * 2 (y-t) / n.  Deterministic two-pass

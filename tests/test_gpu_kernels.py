@@ -541,6 +541,79 @@ def test_conv3x3_weight_gradient_implicit_gemm(hiplib, n, h, w, c, cout):
         assert rel_err(outs[1][0].double().cpu() - base.double().cpu(), ref) < tol(dt)
 
 
+def _strip_reference(y, rows, cols):
+    """(pivot, sum (y - pivot), sum (y - pivot)^2) per 32-row strip and column, in fp64, from the stored tensor."""
+    yd = y.double().cpu()
+    out = []
+    for s0 in range(0, rows, 32):
+        blk = yd[s0:s0 + 32]
+        d = blk - blk[0]
+        out.append(torch.stack([blk[0], d.sum(0), (d * d).sum(0)]))
+    return torch.stack(out)                                              # [strips, 3, cols]
+
+
+@pytest.mark.parametrize("M,N,K", [(6272, 256, 1024),     # conv1 of the ResNet block: 128x64 tiles
+                                   (6272, 1024, 256),     # conv3: 256x128 tiles
+                                   (300, 72, 128)])       # ragged: 12 rows in the last strip, 8 columns in the last group
+def test_gemm_strip_statistics_feed_batchnorm(hiplib, M, N, K):
+    """The GEMM epilogue's per-strip column statistics: the product is bit-equal to the plain call, the triples
+    equal an fp64 restatement on the stored values, and BatchNorm fed from them equals BatchNorm reading the tensor."""
+    dt = torch.bfloat16
+    A, B = randn(M, K, dtype=dt, seed=80), randn(N, K, dtype=dt, seed=81, scale=0.05)
+    A += 3.0                                                              # a mean far from zero: what the pivot is for
+    y0 = torch.empty(M, N, dtype=dt, device=DEV)
+    y1 = torch.empty_like(y0)
+    assert hiplib.gemm_strip_stats_supported(hiplib.NT, A, B, y0)
+    strips = torch.full((hiplib.strip_stats_workspace(M, N),), float("nan"), device=DEV)
+    hiplib.gemm(hiplib.NT, A, B, y1, strip_stats=strips)
+    ref_prod = A.double().cpu() @ B.double().cpu().t()
+    assert rel_err(y1, ref_prod) < tol(dt)
+    ns = (M + 31) // 32
+    got = strips[: ns * 3 * N].view(ns, 3, N).double().cpu()
+    want = _strip_reference(y1, M, N)
+    assert torch.equal(got[:, 0], want[:, 0])
+    assert rel_err(got[:, 1], want[:, 1]) < 1e-5 and rel_err(got[:, 2], want[:, 2]) < 1e-5
+    _check_batchnorm_from_strips(hiplib, y1, strips, M, N)
+
+
+def _check_batchnorm_from_strips(hiplib, y, strips, M, N):
+    dt = torch.bfloat16
+    gamma, beta = randn(N, dtype=dt, seed=82) * 0.1 + 1.0, randn(N, dtype=dt, seed=83) * 0.1
+    ws = torch.empty(hiplib.bn_workspace(N), device=DEV)
+    outs = []
+    for st in (None, strips):
+        o = torch.empty_like(y)
+        mean, rstd = torch.empty(N, device=DEV), torch.empty(N, device=DEV)
+        rm, rv = torch.zeros(N, device=DEV), torch.ones(N, device=DEV)
+        hiplib.batchnorm_fwd(y, gamma, beta, None, o, mean, rstd, rm, rv, ws, 1e-5, 0.1, True, strip_stats=st)
+        outs.append((o, mean, rstd, rm, rv))
+    yd = y.double().cpu()
+    mu, var = yd.mean(0), yd.var(0, unbiased=False)
+    for o, mean, rstd, rm, rv in outs:
+        assert rel_err(mean, mu) < 1e-5
+        assert float(((rstd.double().cpu() - 1 / torch.sqrt(var + 1e-5)).abs() * torch.sqrt(var + 1e-5)).max()) < 1e-5
+        assert rel_err(rv, 0.9 + 0.1 * yd.var(0, unbiased=True)) < 1e-5
+    assert rel_err(outs[1][0], outs[0][0].double()) < 1e-2               # bf16 outputs: a rounding step apart at most
+
+
+def test_conv3x3_strip_statistics(hiplib):
+    n, h, w, cin, cout = 8, 6, 6, 128, 192
+    dt = torch.bfloat16
+    rows = n * h * w
+    x = randn(rows, cin, dtype=dt, seed=84)
+    wt = randn(cout, 3, 3, cin, dtype=dt, seed=85, scale=0.03)
+    y0, y1 = torch.empty(rows, cout, dtype=dt, device=DEV), torch.empty(rows, cout, dtype=dt, device=DEV)
+    strips = torch.full((hiplib.strip_stats_workspace(rows, cout),), float("nan"), device=DEV)
+    hiplib.conv3x3(hiplib.CONV_FWD, x, wt, y0, n, h, w, cin, cout)
+    hiplib.conv3x3(hiplib.CONV_FWD, x, wt, y1, n, h, w, cin, cout, strip_stats=strips)
+    assert torch.equal(y0, y1)
+    got = strips.view(rows // 32, 3, cout).double().cpu()
+    want = _strip_reference(y1, rows, cout)
+    assert torch.equal(got[:, 0], want[:, 0])
+    assert rel_err(got[:, 1], want[:, 1]) < 1e-5 and rel_err(got[:, 2], want[:, 2]) < 1e-5
+    _check_batchnorm_from_strips(hiplib, y1, strips, rows, cout)
+
+
 def test_conv3x3_refuses_what_it_does_not_take(hiplib):
     dt = torch.bfloat16
     assert not hiplib.conv3x3_supported(dt, hiplib.CONV_FWD, 4, 6, 6, 16, 64)            # 16 gathered channels
