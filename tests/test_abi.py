@@ -40,6 +40,47 @@ def test_version_and_error_string():
     assert L.bb_adam_multi(1, None, None, None, None, None, None, 1e-3, 0.9, 0.999, 1e-8, 0, 1, 1, 0.0, 0, None) == -1
 
 
+def test_convolution_entry_points_validate_on_the_host():
+    """What the implicit-GEMM convolution entry points take and refuse is decided on the host, before any HIP call."""
+    from bamboo_amd import hip
+    L = hip.lib()
+    BF16, F32, FWD, DGRAD = hip.BF16, hip.F32, hip.CONV_FWD, hip.CONV_DGRAD
+    ok = L.bb_conv3x3_supported
+    assert ok(BF16, FWD, 32, 14, 14, 256, 256) == 1 and ok(BF16, DGRAD, 32, 14, 14, 256, 256) == 1
+    assert ok(BF16, FWD, 4, 6, 6, 64, 72) == 1            # gathered channels % 64, produced % 8
+    assert ok(BF16, FWD, 4, 6, 6, 96, 64) == 0            # 96 gathered channels: a k-tile would straddle two taps
+    assert ok(BF16, DGRAD, 4, 6, 6, 64, 96) == 0          # the input gradient gathers the output channels
+    assert ok(F32, FWD, 4, 6, 6, 64, 64) == 0 and ok(BF16, 2, 4, 6, 6, 64, 64) == 0
+    assert ok(BF16, FWD, 3, 6, 6, 64, 64) == 0            # 108 pixels: fewer than one 128-row tile
+    assert L.bb_conv3x3(BF16, FWD, 4, 6, 6, 96, 64, 16, 16, 16, None, None) == -1
+    assert b"unsupported problem" in L.bb_last_error()
+    assert L.bb_conv3x3(BF16, FWD, 4, 6, 6, 64, 64, None, None, None, None, None) == -1
+    assert b"null operand" in L.bb_last_error()
+    assert L.bb_strip_stats_workspace(6272, 256) == 196 * 3 * 256 and L.bb_strip_stats_workspace(33, 8) == 2 * 3 * 8
+    # a patch-matrix B (weight gradient of the 3x3 convolution) is a BB_TN, bf16, unbatched affair
+    d = hip.GemmDesc()
+    d.layout, d.dtype, d.c_dtype = hip.TN, BF16, F32
+    d.M, d.N, d.K, d.nb1, d.nb2 = 256, 9 * 128, 288, 1, 1
+    d.A, d.B, d.C, d.lda, d.ldb, d.ldc = 4096, 8192, 12288, 256, 128, 9 * 128
+    d.alpha, d.accumulate = 1.0, 1
+    d.conv_h, d.conv_w, d.conv_c = 6, 6, 96
+    assert L.bb_gemm(ctypes.byref(d), None) == -1 and b"multiple of 128" in L.bb_last_error()
+    d.conv_c, d.N = 128, 9 * 128 + 8
+    assert L.bb_gemm(ctypes.byref(d), None) == -1 and b"9 * conv_c" in L.bb_last_error()
+    d.N, d.layout = 9 * 128, hip.NN
+    assert L.bb_gemm(ctypes.byref(d), None) == -1 and b"BB_TN" in L.bb_last_error()
+    d.layout, d.conv_h, d.conv_w = hip.TN, 2, 8          # 32 consecutive pixels span two whole images
+    assert L.bb_gemm(ctypes.byref(d), None) == -1 and b"image boundary" in L.bb_last_error()
+    # strip statistics: only where the kernels that carry them run
+    s = hip.GemmDesc()
+    s.layout, s.dtype, s.c_dtype, s.M, s.N, s.K, s.nb1, s.nb2, s.alpha = hip.NT, BF16, BF16, 6272, 256, 1024, 1, 1, 1.0
+    assert L.bb_gemm_strip_stats_supported(ctypes.byref(s)) == 1
+    s.K = 96
+    assert L.bb_gemm_strip_stats_supported(ctypes.byref(s)) == 0
+    s.K, s.layout = 1024, hip.NN
+    assert L.bb_gemm_strip_stats_supported(ctypes.byref(s)) == 0
+
+
 def test_gemm_desc_layout_matches_header():
     """Field order of the ctypes mirror follows the struct in the header."""
     from bamboo_amd import hip
