@@ -755,21 +755,26 @@ constexpr int BN_WAVES = 16;  // row streams per block; with 64 splits 1024 wave
 //   (mean = p + S1/n, var = S2/n - (S1/n)^2: shifted by a sample of the data the subtraction does not
 //   cancel, unlike sum x^2 - n mean^2);
 // MODE 2 (backward): sum g and sum g * xhat, with g = dy * (out > 0 if relu_out given).
-// Waves take rows wave, wave + BN_WAVES * splits, ... of their split; fixed order everywhere.
+// A block column covers 64 vectors of a row; where the tensor has at most 32 left for it (256 bf16 channels)
+// the two halves of a wave take alternate rows, so no lane idles.  Row streams (waves, or half waves) take rows
+// s, s + streams, ...: four rows' loads go out together (the rows of a stage-sized tensor fit in one such round),
+// sums are added in row order, halves then waves combined in fixed order.
 template <typename T, int MODE>
 __global__ __launch_bounds__(BN_WAVES * 64) void bn_colred_kernel(int rows, int cols, const T* __restrict__ x,
                                                         const float* __restrict__ mean, const float* __restrict__ rstd,
                                                         const T* __restrict__ dy, const T* __restrict__ relu_out,
                                                         float* __restrict__ partial) {
     constexpr int VEC = Elem<T>::VEC;
-    constexpr int SLOTS = 5;   // the cross-wave sum goes through LDS five waves at a time
-    __shared__ float red[SLOTS][2][64 * VEC];
+    __shared__ float red[BN_WAVES / 2][2][64 * VEC];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const int c0 = (blockIdx.x * 64 + lane) * VEC;
+    const int left = cols / VEC - blockIdx.x * 64;          // vectors of a row from this block column on
+    const bool halves = left <= 32;
+    const int lv = halves ? (lane & 31) : lane, sub = halves ? (lane >> 5) : 0, nsub = halves ? 2 : 1;
+    const int c0 = (blockIdx.x * 64 + lv) * VEC;
     float a0[VEC], a1[VEC], mu[VEC], rs[VEC];
 #pragma unroll
     for (int e = 0; e < VEC; ++e) a0[e] = a1[e] = mu[e] = rs[e] = 0.f;
-    if (c0 < cols) {
+    if (lv < left) {
         if (MODE == 0) {
             load_vec(x + c0, mu);   // the pivot
         } else {
@@ -779,78 +784,80 @@ __global__ __launch_bounds__(BN_WAVES * 64) void bn_colred_kernel(int rows, int 
                 rs[e] = rstd[c0 + e];
             }
         }
-        // rows r0, r0 + step, ... in that order; four rows' loads are issued before their sums
-        auto add_row = [&](const float (&v)[VEC], const float (&g)[VEC]) {
-            if (MODE == 0) {
-#pragma unroll
-                for (int e = 0; e < VEC; ++e) {
-                    const float d = v[e] - mu[e];
-                    a0[e] += d;
-                    a1[e] += d * d;
-                }
-            } else {
-#pragma unroll
-                for (int e = 0; e < VEC; ++e) {
-                    a0[e] += g[e];
-                    a1[e] += g[e] * (v[e] - mu[e]) * rs[e];
-                }
-            }
-        };
-        auto load_row = [&](int r, float (&v)[VEC], float (&g)[VEC]) {
-            load_vec(x + (int64_t)r * cols + c0, v);
-            if (MODE == 2) {
-                load_vec(dy + (int64_t)r * cols + c0, g);
-                if (relu_out) {
-                    float o[VEC];
-                    load_vec(relu_out + (int64_t)r * cols + c0, o);
-#pragma unroll
-                    for (int e = 0; e < VEC; ++e) g[e] = o[e] > 0.f ? g[e] : 0.f;
-                }
-            }
-        };
-        const int step = gridDim.y * BN_WAVES;
-        int r = blockIdx.y * BN_WAVES + wave;
-        for (; r + 3 * step < rows; r += 4 * step) {
+        const int streams = gridDim.y * BN_WAVES * nsub;
+        for (int r = (blockIdx.y * BN_WAVES + wave) * nsub + sub; r < rows; r += 4 * streams) {
             float v[4][VEC], g[4][VEC];
 #pragma unroll
-            for (int j = 0; j < 4; ++j) load_row(r + j * step, v[j], g[j]);
+            for (int j = 0; j < 4; ++j) {
+                const int rj = r + j * streams;
+                if (rj < rows) {
+                    load_vec(x + (int64_t)rj * cols + c0, v[j]);
+                    if (MODE == 2) {
+                        load_vec(dy + (int64_t)rj * cols + c0, g[j]);
+                        if (relu_out) {
+                            float o[VEC];
+                            load_vec(relu_out + (int64_t)rj * cols + c0, o);
 #pragma unroll
-            for (int j = 0; j < 4; ++j) add_row(v[j], g[j]);
-        }
-        for (; r < rows; r += step) {
-            float v[VEC], g[VEC];
-            load_row(r, v, g);
-            add_row(v, g);
-        }
-    }
-    // wave 0 + 1 + 2 + ... in that order, SLOTS waves per round through LDS
-    for (int w0 = 1; w0 < BN_WAVES; w0 += SLOTS) {
-        if (wave >= w0 && wave < w0 + SLOTS) {
-#pragma unroll
-            for (int e = 0; e < VEC; ++e) {
-                red[wave - w0][0][lane * VEC + e] = a0[e];
-                red[wave - w0][1][lane * VEC + e] = a1[e];
+                            for (int e = 0; e < VEC; ++e) g[j][e] = o[e] > 0.f ? g[j][e] : 0.f;
+                        }
+                    }
+                }
             }
-        }
-        __syncthreads();
-        if (wave == 0) {
-            const int n = min(SLOTS, BN_WAVES - w0);
-            for (int w = 0; w < n; ++w) {
 #pragma unroll
-                for (int e = 0; e < VEC; ++e) {
-                    a0[e] += red[w][0][lane * VEC + e];
-                    a1[e] += red[w][1][lane * VEC + e];
+            for (int j = 0; j < 4; ++j) {
+                if (r + j * streams < rows) {
+#pragma unroll
+                    for (int e = 0; e < VEC; ++e) {
+                        if (MODE == 0) {
+                            const float d = v[j][e] - mu[e];
+                            a0[e] += d;
+                            a1[e] += d * d;
+                        } else {
+                            a0[e] += g[j][e];
+                            a1[e] += g[j][e] * (v[j][e] - mu[e]) * rs[e];
+                        }
+                    }
                 }
             }
         }
-        __syncthreads();
     }
-    if (wave == 0 && c0 < cols) {
+    if (halves) {   // both halves end with the sum of the two (a + b = b + a bit for bit)
 #pragma unroll
         for (int e = 0; e < VEC; ++e) {
-            partial[((int64_t)blockIdx.y * 2) * cols + c0 + e] = a0[e];
-            partial[((int64_t)blockIdx.y * 2 + 1) * cols + c0 + e] = a1[e];
+            a0[e] += __shfl_xor(a0[e], 32, 64);
+            a1[e] += __shfl_xor(a1[e], 32, 64);
         }
+    }
+    // waves: upper half onto lower half, then every thread adds up one output value over the eight left
+    constexpr int HW = BN_WAVES / 2;
+    auto put = [&](int slot) {
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) {
+            red[slot][0][lane * VEC + e] = a0[e];
+            red[slot][1][lane * VEC + e] = a1[e];
+        }
+    };
+    if (wave >= HW) put(wave - HW);
+    __syncthreads();
+    if (wave < HW) {
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) {
+            a0[e] += red[wave][0][lane * VEC + e];
+            a1[e] += red[wave][1][lane * VEC + e];
+        }
+    }
+    __syncthreads();
+    if (wave < HW) put(wave);
+    __syncthreads();
+    // lanes of the second half hold the same columns as the first where rows were shared between halves
+    const int width = halves ? 32 * VEC : 64 * VEC;
+    for (int t = threadIdx.x; t < 2 * width; t += BN_WAVES * 64) {
+        const int j = t / width, col = t - j * width;
+        float sum = red[0][j][col];
+#pragma unroll
+        for (int w = 1; w < HW; ++w) sum += red[w][j][col];
+        const int c = blockIdx.x * 64 * VEC + col;
+        if (c < cols) partial[((int64_t)blockIdx.y * 2 + j) * cols + c] = sum;
     }
 }
 
