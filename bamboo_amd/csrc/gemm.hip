@@ -1188,6 +1188,10 @@ static DmaTile pick_dma_tile(int M, int N, int K, int64_t batches, int layout) {
     //    ResNet stage: 98 tiles) take 128x64 tiles: twice the blocks.
     //    (a k-major operand needs 128 rows for its swizzle, so NT narrows N and NN narrows M; TN keeps
     //    128x128).
+    //  - A short forward contraction (K <= 512: the 1x1 convolution out of 256 channels) leaves a launch that is mostly
+    //    its epilogue: 128x64 tiles, so that every CU stores a share (6272x1024x256: 15 us on 100 tiles of 256x128,
+    //    13 us on 784 of 128x64; the input gradient of the same shape gains nothing from 64x128 tiles).
+    if (K <= 512 && nt) return k64 ? D128x64k64s3 : D128x64s3;
     if (t128 <= 128 && nt) return k64 ? D128x64k64s3 : D128x64s3;
     if (t128 <= 128 && nn) return k64 ? D64x128k64s3 : D64x128s3;
     //  - NT problems whose 256x256 tiles would fill under 70 % of their rounds may take 256x192 tiles (six
@@ -1450,9 +1454,11 @@ extern "C" int bb_conv3x3(int dtype, int mode, int n, int h, int w, int cin, int
         g.ldb = 9 * (int64_t)cin;
         if (strip_stats) {
             g.strip_stats = strip_stats;
-            return launch_conv3x3<128, 64, 4, 1, false, 3, true>(g, cv, st);
+            return launch_conv3x3<128, 64, 4, 2, false, 3, true>(g, cv, st);
         }
-        return launch_conv3x3<128, 64, 4, 1, false, 3>(g, cv, st);
+        // eight waves on a 128x64 tile (32x32 per wave): with one block per CU, two waves per SIMD hide each other's
+        // LDS and barrier waits (four waves: 21.6 us, eight: 19.4 us at 6272 pixels, 256 channels)
+        return launch_conv3x3<128, 64, 4, 2, false, 3>(g, cv, st);
     }
     // B[k = t * cout + o, n = i] = weight[o, 8 - t, i]: k-major with row stride 9 * cin, starting at tap 8; after
     // the cout / 64 k-tiles of a tap the rows go back to o = 0 and one tap down
@@ -1460,7 +1466,7 @@ extern "C" int bb_conv3x3(int dtype, int mode, int n, int h, int w, int cin, int
     g.ldb = 9 * (int64_t)cin;
     cv.b_every = cout / 64;
     cv.b_wrap = -(int64_t)cout * g.ldb - cin;
-    return launch_conv3x3<64, 128, 2, 2, true, 3>(g, cv, st);
+    return launch_conv3x3<64, 128, 2, 4, true, 3>(g, cv, st);
 }
 
 template <bool TA, bool TB, bool CONVB = false> static int launch_grouped(GroupedArgs& G, hipStream_t st) {
@@ -1578,7 +1584,14 @@ static int pick_splits(const bb_gemm_desc* descs, int count) {
         tiles += (int64_t)((d.M + 127) / 128) * ((d.N + 127) / 128);
         kmin = d.K < kmin ? d.K : kmin;
     }
-    int splits = (int)(256 / tiles);                 // fill the 256 CUs once
+    // Two blocks per CU on average: with one, a CU's four waves have nobody to hide their load and barrier waits
+    // behind (the weight gradients of a ResNet block: 61.7 us at three chunks, 50.8 us at five).
+    // BB_SPLITK_FILL (tuning aid) overrides the 2.
+    static const int fill = [] {
+        const char* e = getenv("BB_SPLITK_FILL");
+        return e && atoi(e) > 0 ? atoi(e) : 2;
+    }();
+    int splits = (int)(256 * fill / tiles);
     if (splits > SPLITK_MAX) splits = SPLITK_MAX;
     if (splits > GROUP_MAX / count) splits = GROUP_MAX / count;
     while (splits > 1 && kmin / splits < 512) --splits;  // keep the pipelines of the chunks long

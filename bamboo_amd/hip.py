@@ -481,7 +481,7 @@ class ConvLaunch:
     """What ``gemm_hook`` is handed for an implicit-GEMM convolution: the GEMM it amounts to."""
 
     def __init__(self, mode, rows, cin, cout):
-        self.variant_name = "bf16_conv3x3_fwd_igemm128x64k64s3" if mode == CONV_FWD else "bf16_conv3x3_dgrad_igemm64x128k64s3"
+        self.variant_name = "bf16_conv3x3_fwd_igemm128x64w8k64s3" if mode == CONV_FWD else "bf16_conv3x3_dgrad_igemm64x128w8k64s3"
         self.M, self.N, self.K = (rows, cout, 9 * cin) if mode == CONV_FWD else (rows, cin, 9 * cout)
         self.epilogue = EPI_NONE
 
