@@ -8,9 +8,10 @@
  *     aligned, row-major; leading dimensions and strides are in ELEMENTS.
  *   - `stream` is a hipStream_t passed as void*; work is stream-ordered, no hidden
  *     synchronisation, no allocation (workspaces are caller-provided).
- *   - results are deterministic: no atomics in reductions, no split-K, so running the same
- *     call twice on the same inputs gives bit-identical outputs (this is what makes the
- *     redundant forward of shadow layers bit-exact with the normal forward).
+ *   - results are deterministic: no atomics in reductions, partial sums (split contractions,
+ *     per-block partials) added in a fixed order, so running the same call twice on the same
+ *     inputs gives bit-identical outputs (this is what makes the redundant forward of shadow
+ *     layers bit-exact with the normal forward).
  *   - dtype codes: BB_F32 = 0, BB_BF16 = 1.
  *
  * The reference has exactly one native entry point on this path, the torch extension
