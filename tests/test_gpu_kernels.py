@@ -553,7 +553,8 @@ def _strip_reference(y, rows, cols):
 
 
 @pytest.mark.parametrize("M,N,K", [(6272, 256, 1024),     # conv1 of the ResNet block: 128x64 tiles
-                                   (6272, 1024, 256),     # conv3: 256x128 tiles
+                                   (6272, 1024, 256),     # conv3: short contraction, 128x64 tiles
+                                   (6272, 1024, 1024),    # the 256x128 tile (two strips per wave)
                                    (300, 72, 128)])       # ragged: 12 rows in the last strip, 8 columns in the last group
 def test_gemm_strip_statistics_feed_batchnorm(hiplib, M, N, K):
     """The GEMM epilogue's per-strip column statistics: the product is bit-equal to the plain call, the triples
@@ -566,6 +567,8 @@ def test_gemm_strip_statistics_feed_batchnorm(hiplib, M, N, K):
     assert hiplib.gemm_strip_stats_supported(hiplib.NT, A, B, y0)
     strips = torch.full((hiplib.strip_stats_workspace(M, N),), float("nan"), device=DEV)
     hiplib.gemm(hiplib.NT, A, B, y1, strip_stats=strips)
+    if (M, N, K) == (6272, 1024, 1024):
+        assert hiplib.gemm_variant(hiplib.gemm_desc(hiplib.NT, A, B, y1)).endswith("dma256x128k64s3")
     ref_prod = A.double().cpu() @ B.double().cpu().t()
     assert rel_err(y1, ref_prod) < tol(dt)
     ns = (M + 31) // 32
