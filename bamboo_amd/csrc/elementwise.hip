@@ -103,6 +103,19 @@ template <int N> __device__ __forceinline__ void store_f32s(float* dst, const fl
     for (int e = 0; e < N; e += 4) *(f32x4*)(dst + e) = f32x4{v[e], v[e + 1], v[e + 2], v[e + 3]};
 }
 
+// 16 raw bytes -> VEC floats
+__device__ __forceinline__ void unpack16(const u32x4& t, float (&v)[4]) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) v[i] = __uint_as_float(t[i]);
+}
+__device__ __forceinline__ void unpack16(const u32x4& t, float (&v)[8]) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        v[2 * i] = __uint_as_float(t[i] << 16);
+        v[2 * i + 1] = __uint_as_float(t[i] & 0xffff0000u);
+    }
+}
+
 constexpr int LN_BWD_BLOCKS = 256;
 constexpr int LN_BWD_WAVES = 16;  // one block per CU, four waves per SIMD to cover the load latency
 
@@ -113,9 +126,9 @@ __global__ __launch_bounds__(LN_BWD_WAVES * 64) void layernorm_bwd_kernel(int ki
                                                             const float* __restrict__ mean_in,
                                                             const float* __restrict__ rinv_in, const T* __restrict__ dy,
                                                             const T* __restrict__ dres, T* __restrict__ dx,
-                                                            float* __restrict__ partial) {
+                                                            float* __restrict__ partial, int one_pass) {
     constexpr int VEC = Elem<T>::VEC;
-    extern __shared__ float red[];  // [3 waves][2][cols] for the cross-wave sum
+    extern __shared__ float red[];  // [16 waves][2][cols] (one pass) or [3 waves][2][cols] for the cross-wave sum
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int nvec = cols / VEC;
     float gv[IT][VEC], dg[IT][VEC], db[IT][VEC];
@@ -131,7 +144,13 @@ __global__ __launch_bounds__(LN_BWD_WAVES * 64) void layernorm_bwd_kernel(int ki
         const T* xr = x + (int64_t)row * cols;
         const T* dyr = dy + (int64_t)row * cols;
         float xh[IT][VEC], dyh[IT][VEC];
+        u32x4 rres[IT];   // the residual gradient, fetched with the row (16 bytes per vector, unpacked at the end)
         float s1 = 0.f, s2 = 0.f;
+#pragma unroll
+        for (int i = 0; i < IT; ++i) {
+            const int c = lane + i * 64;
+            if (dres && c < nvec) rres[i] = *(const u32x4*)(dres + (int64_t)row * cols + c * VEC);
+        }
 #pragma unroll
         for (int i = 0; i < IT; ++i) {
             const int c = lane + i * 64;
@@ -172,7 +191,7 @@ __global__ __launch_bounds__(LN_BWD_WAVES * 64) void layernorm_bwd_kernel(int ki
                 for (int e = 0; e < VEC; ++e) o[e] = rinv * (dyh[i][e] - s1) - xh[i][e] * c2;
                 if (dres) {
                     float rv[VEC];
-                    load_vec(dres + (int64_t)row * cols + c * VEC, rv);
+                    unpack16(rres[i], rv);
 #pragma unroll
                     for (int e = 0; e < VEC; ++e) o[e] += rv[e];
                 }
@@ -180,8 +199,29 @@ __global__ __launch_bounds__(LN_BWD_WAVES * 64) void layernorm_bwd_kernel(int ki
             }
         }
     }
-    // cross-wave sum in fixed order (wave 0 + 1 + 2 + ... ), three waves per round through the
-    // three LDS slots, then one partial row per block
+    // cross-wave sum.  Where the LDS holds all sixteen waves' sums (2 * cols floats each): one barrier, then every
+    // thread adds up its share of the 2 * cols outputs over the waves in wave order, and the block's partial row is
+    // written by all threads.  Wider rows go three waves per round through three slots (fixed order as well).
+    if (one_pass) {
+        float* r = red + (int64_t)wave * 2 * cols;
+#pragma unroll
+        for (int i = 0; i < IT; ++i) {
+            const int c = lane + i * 64;
+            if (c < nvec) {
+                store_f32s<VEC>(r + c * VEC, dg[i]);
+                store_f32s<VEC>(r + cols + c * VEC, db[i]);
+            }
+        }
+        __syncthreads();
+        float* out = partial + (int64_t)blockIdx.x * 2 * cols;
+        for (int t = threadIdx.x; t < 2 * cols; t += LN_BWD_WAVES * 64) {
+            float sum = red[t];
+#pragma unroll
+            for (int w = 1; w < LN_BWD_WAVES; ++w) sum += red[(int64_t)w * 2 * cols + t];
+            out[t] = sum;
+        }
+        return;
+    }
     for (int w0 = 1; w0 < LN_BWD_WAVES; w0 += 3) {
         if (wave >= w0 && wave < w0 + 3) {
             float* r = red + (int64_t)(wave - w0) * 2 * cols;
@@ -292,11 +332,17 @@ static int ln_fwd_launch(int kind, int rows, int cols, float eps, const void* x,
 template <typename T, int IT>
 static int ln_bwd_launch(int kind, int rows, int cols, float eps, const void* x, const void* gain, const float* mean,
                          const float* rinv, const void* dy, const void* dres, void* dx, float* ws, hipStream_t st) {
-    const size_t smem = (size_t)3 * 2 * cols * sizeof(float);
+    const size_t all = (size_t)LN_BWD_WAVES * 2 * cols * sizeof(float);
+    const int one_pass = all <= 128 * 1024;
+    const size_t smem = one_pass ? all : (size_t)3 * 2 * cols * sizeof(float);
     auto kern = layernorm_bwd_kernel<T, IT>;
-    if (smem > 64 * 1024) BB_HIP_CHECK(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
+    static size_t allowed = 64 * 1024;   // raised once per size, on the first (never captured) call that needs it
+    if (smem > allowed) {
+        BB_HIP_CHECK(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
+        allowed = smem;
+    }
     hipLaunchKernelGGL(kern, dim3(LN_BWD_BLOCKS), dim3(LN_BWD_WAVES * 64), smem, st, kind, rows, cols, eps, (const T*)x,
-                       (const T*)gain, mean, rinv, (const T*)dy, (const T*)dres, (T*)dx, ws);
+                       (const T*)gain, mean, rinv, (const T*)dy, (const T*)dres, (T*)dx, ws, one_pass);
     BB_LAUNCH_CHECK();
     return BB_OK;
 }

@@ -46,7 +46,7 @@ PEAK_BF16_TFLOPS, PEAK_F32_TFLOPS = 2500.0, 157.3
 MEASURED_TRAFFIC_BYTES = {
     # average over the three forward products that run on this tile (QKV, attention output, FFN2)
     ("c2", "gemm_bf16_nt_dma256x128k64s3"): int((60311.8 * 2.0 + 27306.7) * 1024),
-    ("c2", "gemm_grouped_bf16_tn"): int((233331.0 * 2.0 + 49188.7) * 1024),
+    ("c2", "gemm_grouped_bf16_tn"): int((235172.6 * 2.0 + 49188.7) * 1024),
     ("c2", "gemm_bf16_nt_dma256x256k64+act_dact"): int((50033.1 * 2.0 + 131072.0) * 1024),
     ("c2", "gemm_bf16_nt_dma256x256k64+act"): int((50033.1 * 2.0 + 65536.0) * 1024),
 }
