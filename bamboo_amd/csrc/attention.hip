@@ -288,24 +288,25 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const AttnArgs a) {
 // backward, preparation: delta[b, head, q] = sum_d dO[q, d] * O[q, d]
 // =========================================================================================
 __global__ __launch_bounds__(256) void attn_delta_kernel(const AttnArgs a) {
-    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;  // (row, head), head fastest
+    // Eight lanes per (row, head): each takes 16 bytes of the head's 128-byte slice of O and of dO (one cache line per
+    // group and tensor), products summed over the group by three shuffles.  A block covers 32 consecutive rows of one
+    // head, so the results leave as one run of 32 floats.
+    const int lane8 = threadIdx.x & 7, g = threadIdx.x >> 3;
+    const int head = blockIdx.y;
     const int64_t rows = (int64_t)a.batch * a.seq;
-    if (i >= rows * a.heads) return;
-    const int head = (int)(i % a.heads);
-    const int64_t row = i / a.heads;
-    const bf16* op = a.o + row * a.ld_o + head * 64;
-    const bf16* gp = a.d_o + row * a.ld_o + head * 64;
+    const int64_t row = min((int64_t)blockIdx.x * 32 + g, rows - 1);   // rows past the end repeat the last one, store nothing
+    float x[8], y[8];
+    load_vec(a.o + row * a.ld_o + head * 64 + lane8 * 8, x);
+    load_vec(a.d_o + row * a.ld_o + head * 64 + lane8 * 8, y);
     float s = 0.f;
 #pragma unroll
-    for (int c = 0; c < 8; ++c) {
-        float x[8], y[8];
-        load_vec(op + c * 8, x);
-        load_vec(gp + c * 8, y);
+    for (int e = 0; e < 8; ++e) s += x[e] * y[e];
 #pragma unroll
-        for (int e = 0; e < 8; ++e) s += x[e] * y[e];
+    for (int o = 1; o < 8; o <<= 1) s += __shfl_xor(s, o, 64);
+    if (lane8 == 0 && (int64_t)blockIdx.x * 32 + g < rows) {
+        const int b = (int)(row / a.seq), q = (int)(row % a.seq);
+        a.delta[((int64_t)b * a.heads + head) * a.seq + q] = s;
     }
-    const int b = (int)(row / a.seq), q = (int)(row % a.seq);
-    a.delta[((int64_t)b * a.heads + head) * a.seq + q] = s;
 }
 
 // =========================================================================================
@@ -620,8 +621,7 @@ extern "C" int bb_attention_bwd(int dtype, int mask, int batch, int heads, int s
     a.scale = 1.0f / sqrtf((float)head_dim);
     a.scale_log2 = a.scale * 1.4426950408889634f;
     hipStream_t st = (hipStream_t)stream;
-    const int64_t n = (int64_t)batch * seq * heads;
-    hipLaunchKernelGGL(attn_delta_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st, a);
+    hipLaunchKernelGGL(attn_delta_kernel, dim3((unsigned)(((int64_t)batch * seq + 31) / 32), (unsigned)heads), dim3(256), 0, st, a);
     dim3 grid(attn_grid(seq, batch * heads));
     hipLaunchKernelGGL(attn_bwd_dkv_kernel, grid, dim3(256), 0, st, a);
     hipLaunchKernelGGL(attn_bwd_dq_kernel, grid, dim3(256), 0, st, a);
