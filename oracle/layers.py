@@ -6,6 +6,9 @@ Follows DeepSpeedExamples/pipeline_parallelism/transformer.py of the reference:
   feed_forward        transformer.py:149-158 (PositionwiseFeedForward)
   transformer_layer   transformer.py:91-103,161-172 (SublayerConnection + EncoderLayer, pre-LN)
   bottleneck          resnet.py:49-75        (BottleNeck, bias-free convs, train-mode BN)
+  batch_stats_from_strips  resnet.py:56,59,62 (nn.BatchNorm2d batch statistics, restated over
+                      32-row strips as the HIP path computes them; pinned against torch's
+                      mean / var in tests/test_oracle_layers.py)
 Dropout is fixed to 0 (the reference's own parity test disables it,
 tests/unit/test_pipe.py:144-145).  Switches beyond the reference's setting
 (`relu`, `annotated`, no mask) exist because the benchmark configurations ask
@@ -180,3 +183,29 @@ def bottleneck(x, p, cfg):
     y = F.relu(bn(F.conv2d(y, p["residual_function.3.weight"], stride=cfg.stride, padding=1), 4))
     y = bn(F.conv2d(y, p["residual_function.6.weight"]), 7)
     return F.relu(y + x)
+
+
+def strip_triples(y, strip=32):
+    """Per strip of `strip` consecutive rows and per column: (pivot = the strip's first row,
+    sum (y - pivot), sum (y - pivot)^2).  y: [rows, cols]; returns [strips, 3, cols] in float64."""
+    yd = y.double()
+    out = []
+    for s0 in range(0, yd.shape[0], strip):
+        blk = yd[s0:s0 + strip]
+        d = blk - blk[0]
+        out.append(torch.stack([blk[0], d.sum(0), (d * d).sum(0)]))
+    return torch.stack(out)
+
+
+def batch_stats_from_strips(triples, rows, strip=32):
+    """Mean and biased variance over all rows from the strip triples: a strip's mean is
+    pivot + S1/n and its sum of squared deviations S2 - S1^2/n; the batch mean is the
+    n-weighted mean of the strip means, the batch sum of squared deviations is
+    sum_s [M2_s + n_s (mean_s - mean)^2]."""
+    ns = torch.tensor([min(strip, rows - i * strip) for i in range(triples.shape[0])], dtype=torch.float64)[:, None]
+    piv, s1, s2 = triples[:, 0], triples[:, 1], triples[:, 2]
+    mean_s = piv + s1 / ns
+    m2_s = s2 - s1 * s1 / ns
+    mean = (ns * mean_s).sum(0) / rows
+    m2 = (m2_s + ns * (mean_s - mean) ** 2).sum(0)
+    return mean, m2 / rows

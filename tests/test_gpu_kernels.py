@@ -543,13 +543,7 @@ def test_conv3x3_weight_gradient_implicit_gemm(hiplib, n, h, w, c, cout):
 
 def _strip_reference(y, rows, cols):
     """(pivot, sum (y - pivot), sum (y - pivot)^2) per 32-row strip and column, in fp64, from the stored tensor."""
-    yd = y.double().cpu()
-    out = []
-    for s0 in range(0, rows, 32):
-        blk = yd[s0:s0 + 32]
-        d = blk - blk[0]
-        out.append(torch.stack([blk[0], d.sum(0), (d * d).sum(0)]))
-    return torch.stack(out)                                              # [strips, 3, cols]
+    return ol.strip_triples(y.double().cpu())                           # [strips, 3, cols]
 
 
 @pytest.mark.parametrize("M,N,K", [(6272, 256, 1024),     # conv1 of the ResNet block: 128x64 tiles
@@ -592,6 +586,8 @@ def _check_batchnorm_from_strips(hiplib, y, strips, M, N):
         outs.append((o, mean, rstd, rm, rv))
     yd = y.double().cpu()
     mu, var = yd.mean(0), yd.var(0, unbiased=False)
+    mu_s, var_s = ol.batch_stats_from_strips(strips[: ((M + 31) // 32) * 3 * N].view(-1, 3, N).double().cpu(), M)
+    assert rel_err(mu_s, mu) < 1e-6 and rel_err(var_s, var) < 1e-5     # the GPU's triples through the oracle's finish
     for o, mean, rstd, rm, rv in outs:
         assert rel_err(mean, mu) < 1e-5
         assert float(((rstd.double().cpu() - 1 / torch.sqrt(var + 1e-5)).abs() * torch.sqrt(var + 1e-5)).max()) < 1e-5

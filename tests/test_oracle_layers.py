@@ -125,3 +125,19 @@ def test_adam_first_step_closed_form():
     m, v = np.zeros(3, np.float32), np.zeros(3, np.float32)
     oadam.adam_step(p, g, m, v, 1, lr=0.1)
     np.testing.assert_allclose(p, [0.9, -1.9, 2.9], rtol=1e-5)
+
+
+def test_batch_statistics_from_strips_equal_the_direct_ones():
+    """The strip restatement of BatchNorm's batch statistics (what the convolution epilogues and the finish
+    kernel compute) is an identity: checked against torch's mean / var on data with a mean far from zero,
+    a ragged last strip, and a single-strip tensor."""
+    g = torch.Generator().manual_seed(5)
+    for rows, cols, shift in ((6272, 24, 0.0), (300, 8, 50.0), (20, 16, -3.0), (33, 8, 1e3)):
+        y = torch.randn(rows, cols, generator=g, dtype=torch.float64) * 0.7 + shift
+        mean, var = ol.batch_stats_from_strips(ol.strip_triples(y), rows)
+        torch.testing.assert_close(mean, y.mean(0), rtol=1e-12, atol=1e-12)
+        torch.testing.assert_close(var, y.var(0, unbiased=False), rtol=1e-9, atol=1e-12)
+    # one row per strip degenerates to the textbook two-pass formula
+    y = torch.randn(7, 4, generator=g, dtype=torch.float64)
+    mean, var = ol.batch_stats_from_strips(ol.strip_triples(y, strip=1), 7, strip=1)
+    torch.testing.assert_close(var, ((y - y.mean(0)) ** 2).mean(0))
