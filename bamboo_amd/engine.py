@@ -277,6 +277,7 @@ class PipelineEngine:
         self._reserve_pipe_buffers(self.micro_batches)
         self.queue.start_batch()
         self.total_loss.zero_()
+        self._loss_done = set()
         self._debug = debug
         t0 = time.perf_counter()
 
@@ -422,7 +423,9 @@ class PipelineEngine:
 
     def _exec_recv_activations(self, buffer_id, stage_id):
         if buffer_id == -1:
-            self.queue.ping(self._dec(stage_id))
+            # one-element receive from the predecessor (reference engine.py:2012-2035): a dead
+            # predecessor surfaces as PrevStageException
+            self.queue.ping_prev(stage_id)
             return
         key = f"input_{stage_id}"
         if self.pipe_buffers[key][buffer_id] is not None:
@@ -437,7 +440,9 @@ class PipelineEngine:
 
     def _exec_send_activations(self, buffer_id, stage_id):
         if buffer_id == -1:
-            self.queue.ping(stage_id)
+            # one-element send to the successor (reference engine.py:1903-1930): a dead successor
+            # surfaces as NextStageException
+            self.queue.ping_next(stage_id)
             return
         if stage_id + 1 in self.stage_ids:
             return
@@ -458,7 +463,14 @@ class PipelineEngine:
 
     def _exec_forward_pass(self, buffer_id, stage_id):
         out_key = f"output_{stage_id}"
+        last_with_loss = stage_id == self.num_stages - 1 and self.module.loss_fn is not None
         if self.pipe_buffers[out_key][buffer_id] is not None:
+            # The reference keeps no output of the last stage (engine.py:1646), so a replayed forward of
+            # an absorbed last stage computes the loss again.  Here the redundant forward's output is
+            # kept for the backward pass from the stash, and only the loss head still has to run on it.
+            if (last_with_loss and stage_id in self.stage_ids and self._deferred.get((stage_id, buffer_id))
+                    and (stage_id, buffer_id) not in self._loss_done):
+                self._loss_head(buffer_id, stage_id, self.pipe_buffers[out_key][buffer_id])
             return
         inputs = self.pipe_buffers["data" if stage_id == 0 else f"input_{stage_id}"][buffer_id]
         redundant = stage_id in self.r_stage_ids
@@ -477,11 +489,23 @@ class PipelineEngine:
         self.pipe_buffers[out_key][buffer_id] = out
         if not redundant and self.rc_stream is not None:
             self._fwd_done[buffer_id].record(self.main_stream)
-        if stage_id == self.num_stages - 1 and not redundant and self.module.loss_fn is not None:
-            labels = self.pipe_buffers["label"][buffer_id]
-            self.module.loss_fn(out, labels, self._loss_grad, 1.0 / self.micro_batches, self.total_loss, True,
-                                self._loss_ws, stream=self.main_stream)
-            self.grad_layer[stage_id] = self._loss_grad
+        if last_with_loss and not redundant:
+            self._loss_head(buffer_id, stage_id, out)
+
+    def _loss_head(self, buffer_id, stage_id, out):
+        """Loss of one micro-batch on the last stage and its gradient scaled by 1 / micro_batches
+        (reference engine.py:1649-1663, deepspeed/runtime/engine.py:1430-1431)."""
+        labels = self.pipe_buffers["label"][buffer_id]
+        if labels is None:
+            raise PipelineError(f"ForwardPass({buffer_id}, {stage_id}): the last stage has no labels for this micro-batch")
+        if self._loss_grad is None:
+            act_shape = (self.batch * self.seq, self.queue.shape[2])
+            self._loss_grad = torch.empty(act_shape, dtype=self.module.dtype, device=self.device)
+            self._loss_ws = torch.empty(hip.mse_workspace(), dtype=torch.float32, device=self.device)
+        self.module.loss_fn(out, labels, self._loss_grad, 1.0 / self.micro_batches, self.total_loss, True,
+                            self._loss_ws, stream=self.main_stream)
+        self.grad_layer[stage_id] = self._loss_grad
+        self._loss_done.add((stage_id, buffer_id))
 
     def _exec_backward_pass(self, buffer_id, stage_id):
         grad = self.grad_layer.get(stage_id)

@@ -125,9 +125,16 @@ class SeededActivationQueue:
     def send_grad(self, k, tensor, stage_id):
         self.sent_grads[(stage_id, k)] = tensor
 
-    def ping(self, stage_id):
+    def ping_next(self, stage_id):
+        """One-element send from ``stage_id`` to its successor (``SendActivation(-1, stage_id)`` of the
+        lazy schedule): fails like any other transfer with a successor that is gone."""
         if self.dead_from is not None and stage_id == self.dead_stage and self.dead_from <= 0:
             raise NextStageException(f"successor of stage {stage_id} does not answer")
+
+    def ping_prev(self, stage_id):
+        """One-element receive of ``stage_id`` from its predecessor (``RecvActivation(-1, stage_id)``).  This
+        queue models the loss of a successor only; the activations it serves are always there."""
+        return
 
 
 # =============================================================================================
@@ -269,10 +276,21 @@ class FabricEndpoint:
         self._check_kill(k)
         self._put("grad", stage_id, stage_id - 1, k, tensor, PrevStageException)
 
-    def ping(self, stage_id):
+    def _ping(self, peer, exc):
+        peer %= self.f.num_stages   # the pings of the first and the last stage close the ring (reference engine.py:_inc/_dec)
         with self.f.cv:
-            if stage_id in self.f.dead and stage_id not in self.acknowledged:
-                raise NextStageException(f"stage {stage_id} does not answer")
+            if peer in self.f.dead and peer not in self.acknowledged:
+                raise exc(f"stage {peer} does not answer")
+
+    def ping_next(self, stage_id):
+        """``SendActivation(-1, stage_id)``: a dead successor raises :class:`NextStageException`
+        (reference engine.py:1903-1930)."""
+        self._ping(stage_id + 1, NextStageException)
+
+    def ping_prev(self, stage_id):
+        """``RecvActivation(-1, stage_id)``: a dead predecessor raises :class:`PrevStageException`
+        (reference engine.py:2012-2035)."""
+        self._ping(stage_id - 1, PrevStageException)
 
     # ---------------------------------------------------------------- weights of a stage for its shadow
     def send_weights(self, stage_id, arenas):

@@ -146,9 +146,15 @@ class BottleneckCfg:
         return 4 * self.mid_channels
 
 
+    @property
+    def projection(self):
+        """The shortcut is conv1x1(stride) + BN instead of the identity (resnet.py:68-72)."""
+        return self.stride != 1 or self.in_channels != self.out_channels
+
+
 def bottleneck_param_shapes(cfg):
     ci, cm, co = cfg.in_channels, cfg.mid_channels, cfg.out_channels
-    return {
+    shapes = {
         "residual_function.0.weight": (cm, ci, 1, 1),
         "residual_function.1.weight": (cm,), "residual_function.1.bias": (cm,),
         "residual_function.3.weight": (cm, cm, 3, 3),
@@ -156,6 +162,9 @@ def bottleneck_param_shapes(cfg):
         "residual_function.6.weight": (co, cm, 1, 1),
         "residual_function.7.weight": (co,), "residual_function.7.bias": (co,),
     }
+    if cfg.projection:
+        shapes.update({"shortcut.0.weight": (co, ci, 1, 1), "shortcut.1.weight": (co,), "shortcut.1.bias": (co,)})
+    return shapes
 
 
 def init_bottleneck_params(cfg, seed, dtype=torch.float32):
@@ -175,14 +184,16 @@ def init_bottleneck_params(cfg, seed, dtype=torch.float32):
 
 
 def bottleneck(x, p, cfg):
-    """x is NCHW here (torch's convention); identity shortcut (stride 1, Cin == 4*Cmid)."""
-    assert cfg.stride == 1 and cfg.in_channels == cfg.out_channels
-    bn = lambda t, i: F.batch_norm(t, None, None, p[f"residual_function.{i}.weight"],
-                                   p[f"residual_function.{i}.bias"], training=True, eps=cfg.bn_eps)
-    y = F.relu(bn(F.conv2d(x, p["residual_function.0.weight"]), 1))
-    y = F.relu(bn(F.conv2d(y, p["residual_function.3.weight"], stride=cfg.stride, padding=1), 4))
-    y = bn(F.conv2d(y, p["residual_function.6.weight"]), 7)
-    return F.relu(y + x)
+    """x is NCHW here (torch's convention).  Shortcut: the identity when stride is 1 and
+    Cin == 4*Cmid, else conv1x1(stride) + BN (resnet.py:66-72)."""
+    bn = lambda t, key: F.batch_norm(t, None, None, p[f"{key}.weight"], p[f"{key}.bias"], training=True, eps=cfg.bn_eps)
+    y = F.relu(bn(F.conv2d(x, p["residual_function.0.weight"]), "residual_function.1"))
+    y = F.relu(bn(F.conv2d(y, p["residual_function.3.weight"], stride=cfg.stride, padding=1), "residual_function.4"))
+    y = bn(F.conv2d(y, p["residual_function.6.weight"]), "residual_function.7")
+    sc = x
+    if cfg.projection:
+        sc = bn(F.conv2d(x, p["shortcut.0.weight"], stride=cfg.stride), "shortcut.1")
+    return F.relu(y + sc)
 
 
 def strip_triples(y, strip=32):

@@ -9,6 +9,7 @@ Follows deepspeed/runtime/pipe/schedule.py of the reference:
   train_schedule        schedule.py:225-310  (TrainSchedule.steps)
   eager_merge           schedule.py:504-524  (EagerRecoverySchedule._merge_cmds)
   next_stage_failover   schedule.py:343-430  (NextStageFailoverSchedule._merge_cmds)
+  lazy_merge            schedule.py:469-501  (LazyRecoverySchedule._merge_cmds)
 """
 
 RC_KINDS = ("RecvActivation", "LoadMicroBatch", "ForwardPass")
@@ -72,6 +73,42 @@ def eager_merge(own_steps, next_steps):
         if any(c[0] in RC_KINDS for c in nxt):
             fifo.append(nxt)
         out.append(cmds + list(own))
+    return out
+
+
+COMM_KINDS = ("SendActivation", "RecvActivation", "SendGrad", "RecvGrad")
+
+
+def lazy_merge(own_steps, micro_batches, stages, stage_id):
+    """Lazy recovery (schedule.py:483-501): no redundant work, the own stream plus one-element
+    "pings" (buffer id -1) in front of some steps so that a dead neighbour is noticed while the
+    stage would otherwise not talk to it.  Per step ``i`` of stage ``s`` (``half`` = the first
+    ``M + S - 1`` steps, ``F(x)`` = step i is a forward step of stage x, ``quiet`` = the own step
+    holds no send/recv):
+      first stage:   listen (RecvActivation(-1)) on every F(s) step;
+      last stage:    listen on quiet F(s) steps of the first half, and -- independently, placed in
+                     front of it -- call (SendActivation(-1)) on every step that is F(0): the ring
+                     last -> first;
+      middle stages: on quiet steps of the first half, listen if F(s) else call."""
+    M, S, s = micro_batches, stages, stage_id
+    out = []
+    for i, own in enumerate(own_steps):
+        cmds = list(own)
+        fwd = step_to_micro_batch(S, s, i)[1]
+        quiet = not any(c[0] in COMM_KINDS for c in cmds)
+        half = i < M + S - 1
+        listen, call = ("RecvActivation", -1, s), ("SendActivation", -1, s)
+        if s == 0:
+            if fwd:
+                cmds.insert(0, listen)
+        elif s == S - 1:
+            if quiet and fwd and half:
+                cmds.insert(0, listen)
+            if step_to_micro_batch(S, 0, i)[1]:
+                cmds.insert(0, call)
+        elif quiet and half:
+            cmds.insert(0, listen if fwd else call)
+        out.append(cmds)
     return out
 
 

@@ -9,6 +9,7 @@ Follows the reference engine's handlers (deepspeed/runtime/pipe/engine.py):
   BackwardPass    :1680-1727  torch.autograd.backward(output, grad)
   SendGrad        :1935-1997
   OptimizerStep   :2139-2147 -> FusedAdam.step (deepspeed/ops/adam/fused_adam.py:85-182)
+  last stage      :1649-1663  loss_model(outputs, labels) in the forward, backward of loss / GAS
 and the failover branch of train_batch (:1190-1264): promote the shadow stage, run the
 NextStageFailoverSchedule from step 0, one optimizer step for both stages.  The neighbours
 are modelled exactly as the product's in-process queue models them: seeded activations in,
@@ -30,9 +31,10 @@ class PeerFailure(Exception):
 class OraclePeer:
     """Neighbour model: ``grads[stage][k]`` tensors (queue mode) or ``targets[stage][k]`` (mse)."""
 
-    def __init__(self, activations, micro_batches, grads=None, targets=None, key_lens=None):
+    def __init__(self, activations, micro_batches, grads=None, targets=None, key_lens=None, labels=None):
         self.activations, self.M = activations, micro_batches
         self.grads, self.targets, self.key_lens = grads or {}, targets or {}, key_lens
+        self.labels = labels      # labels[k] of the last stage's own loss (LoadMicroBatch), if this process hosts it
         self.loss = 0.0
         self.dead_from, self.dead_stage = None, None
         self._mse_grads = {}
@@ -141,9 +143,25 @@ class OracleStage:
 
     def _ForwardPass(self, k, s, peer, bufs):
         if bufs["out"].get((s, k)) is not None:
+            if (s == self.S - 1 and peer.labels is not None and s in self.stage_ids
+                    and (s, k) not in bufs.get("loss", {})):
+                # replay after absorbing the last stage: the redundant forward left the output, the loss
+                # is still to be computed
+                out = bufs["out"][(s, k)]
+                loss = F.mse_loss(out, peer.labels[k].view_as(out))
+                bufs.setdefault("loss", {})[(s, k)] = loss
+                peer.loss = peer.loss + loss.detach()
             return
         kl = None if peer.key_lens is None else peer.key_lens[k]
-        bufs["out"][(s, k)] = self.forward(bufs["in"][(s, k)], s, kl)
+        out = self.forward(bufs["in"][(s, k)], s, kl)
+        bufs["out"][(s, k)] = out
+        if s == self.S - 1 and peer.labels is not None and s in self.stage_ids:
+            # last stage: loss_model(outputs, labels), summed into total_loss (engine.py:1649-1663); counted
+            # once per micro-batch (the reference recomputes the forward of an absorbed last stage, whose
+            # output it never keeps, :1646 -- same value)
+            loss = F.mse_loss(out, peer.labels[k].view_as(out))
+            bufs.setdefault("loss", {})[(s, k)] = loss
+            peer.loss = peer.loss + loss.detach()
 
     def _SendActivation(self, k, s, peer, bufs):
         if s + 1 in self.stage_ids:
@@ -157,6 +175,10 @@ class OracleStage:
             bufs["grad"][s] = peer.recv_grad(k, s)
 
     def _BackwardPass(self, k, s, peer, bufs):
+        if s == self.S - 1 and (s, k) in bufs.get("loss", {}):
+            # loss / gradient_accumulation_steps, then backward (deepspeed/runtime/engine.py:1430-1431,1478)
+            (bufs["loss"][(s, k)] / self.M).backward()
+            return
         out = bufs["out"][(s, k)]
         torch.autograd.backward(out, bufs["grad"][s].view_as(out))
 

@@ -112,3 +112,36 @@ def test_weights_mailbox():
     msg = {"master": torch.ones(8), "exp_avg": torch.zeros(8), "exp_avg_sq": torch.zeros(8), "step": 3}
     b.send_weights(2, msg)
     assert a.recv_weights(2) is msg
+
+
+def test_pings_have_a_direction():
+    """The lazy schedule's one-element transfers (reference engine.py:1903-1930, 2012-2035): a receive-ping
+    reports a dead predecessor as PrevStageException, a send-ping a dead successor as NextStageException,
+    and neither reports the neighbour on the other side."""
+    f = fabric()
+    eps = [f.endpoint(s) for s in range(4)]
+    for e in eps:
+        e.start_batch()
+    for e in eps:                       # everybody alive: silent
+        e.ping_prev(e.stage)
+        e.ping_next(e.stage)
+    with f.cv:
+        f.dead.add(2)
+    with pytest.raises(PrevStageException):
+        eps[3].ping_prev(3)             # stage 3 listens to stage 2
+    eps[3].ping_next(3)                 # its successor (the ring closes on stage 0) is fine
+    with pytest.raises(NextStageException):
+        eps[1].ping_next(1)             # stage 1 sends to stage 2
+    eps[1].ping_prev(1)
+    eps[0].ping_prev(0)
+    eps[0].ping_next(0)
+    # once the loss has been reported the pings wait for the adopter like every other transfer
+    eps[1].acknowledged.add(2)
+    eps[1].ping_next(1)
+    with f.cv:
+        f.dead.discard(2)
+        f.dead.add(3)
+    with pytest.raises(PrevStageException):
+        eps[0].ping_prev(0)             # the first stage's predecessor in the ring is the last stage
+    with pytest.raises(NextStageException):
+        eps[2].ping_next(2)

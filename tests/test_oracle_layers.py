@@ -102,6 +102,87 @@ def test_bottleneck_identity_shapes_and_relu():
     torch.testing.assert_close(ol.bottleneck(x, p, cfg), F.relu(x))
 
 
+def _module_bottleneck(cfg):
+    """The block as torch.nn modules in the arrangement of the reference's ``BottleNeck``
+    (resnet.py:53-72): Sequential(conv1x1, BN, ReLU, conv3x3(stride, pad 1), BN, ReLU, conv1x1, BN),
+    a shortcut Sequential (empty, or conv1x1(stride) + BN), ReLU of the sum; all convolutions bias-free."""
+    nn = torch.nn
+    ci, cm, co = cfg.in_channels, cfg.mid_channels, cfg.out_channels
+
+    class Block(nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.residual_function = nn.Sequential(
+                nn.Conv2d(ci, cm, 1, bias=False), nn.BatchNorm2d(cm, eps=cfg.bn_eps), nn.ReLU(),
+                nn.Conv2d(cm, cm, 3, stride=cfg.stride, padding=1, bias=False), nn.BatchNorm2d(cm, eps=cfg.bn_eps), nn.ReLU(),
+                nn.Conv2d(cm, co, 1, bias=False), nn.BatchNorm2d(co, eps=cfg.bn_eps))
+            self.shortcut = nn.Sequential()
+            if cfg.stride != 1 or ci != co:
+                self.shortcut = nn.Sequential(nn.Conv2d(ci, co, 1, stride=cfg.stride, bias=False), nn.BatchNorm2d(co, eps=cfg.bn_eps))
+
+        def forward(self, x):
+            return torch.relu(self.residual_function(x) + self.shortcut(x))
+    return Block().double().train()
+
+
+def _bottleneck_case(cfg, seed):
+    g = torch.Generator().manual_seed(seed)
+    p = ol.init_bottleneck_params(cfg, seed, dtype=torch.float64)
+    for k in p:     # BN gains and shifts away from 1 / 0, so that swapping two of them shows
+        if p[k].dim() == 1:
+            p[k] = (1.0 if k.endswith("weight") else 0.0) + 0.3 * torch.randn(p[k].shape, generator=g, dtype=torch.float64)
+    p = {k: v.requires_grad_(True) for k, v in p.items()}
+    x = torch.randn(3, cfg.in_channels, 6, 6, generator=g, dtype=torch.float64, requires_grad=True)
+    return p, x
+
+
+def _compare_with_modules(fn, cfg, seed=4):
+    """Forward and every gradient of ``fn(x, p, cfg)`` against the nn.Module block with the same weights."""
+    p, x = _bottleneck_case(cfg, seed)
+    ref = _module_bottleneck(cfg)
+    # the oracle's parameter names are the module's: a strict load (running statistics aside) must succeed
+    missing, unexpected = ref.load_state_dict({k: v.detach() for k, v in p.items()}, strict=False)
+    assert not unexpected and all("running_" in k or "num_batches" in k for k in missing)
+    xr = x.detach().clone().requires_grad_(True)
+    y, yr = fn(x, p, cfg), ref(xr)
+    dy = torch.randn(yr.shape, generator=torch.Generator().manual_seed(seed + 1), dtype=torch.float64)
+    y.backward(dy)
+    yr.backward(dy)
+    torch.testing.assert_close(y, yr, rtol=1e-10, atol=1e-10)
+    torch.testing.assert_close(x.grad, xr.grad, rtol=1e-9, atol=1e-10)
+    for k, v in ref.named_parameters():
+        torch.testing.assert_close(p[k].grad, v.grad, rtol=1e-9, atol=1e-10, msg=k)
+
+
+@pytest.mark.parametrize("ci,cm,stride", [(64, 16, 1), (32, 16, 1), (64, 16, 2), (48, 8, 2)],
+                         ids=["identity", "projection", "strided", "strided-projection"])
+def test_bottleneck_equals_the_module_composition(ci, cm, stride):
+    """oracle.layers.bottleneck against Conv2d / BatchNorm2d (training mode) / ReLU modules arranged as the
+    reference arranges them (resnet.py:53-75), same weights, fp64: outputs, input gradient and all parameter
+    gradients."""
+    _compare_with_modules(ol.bottleneck, ol.BottleneckCfg(in_channels=ci, mid_channels=cm, stride=stride), seed=ci + stride)
+
+
+@pytest.mark.parametrize("mistake", ["dropped-relu", "swapped-bn", "no-padding-shift", "shortcut-before-relu"])
+def test_bottleneck_pin_catches_plausible_mistakes(mistake):
+    """Negative controls: each of these variants of the oracle must fail the comparison above."""
+    def wrong(x, p, cfg):
+        bn = lambda t, i: F.batch_norm(t, None, None, p[f"residual_function.{i}.weight"], p[f"residual_function.{i}.bias"],
+                                       training=True, eps=cfg.bn_eps)
+        a, b = (4, 1) if mistake == "swapped-bn" else (1, 4)
+        y = F.relu(bn(F.conv2d(x, p["residual_function.0.weight"]), a))
+        w3 = p["residual_function.3.weight"]
+        if mistake == "no-padding-shift":
+            w3 = w3.flip(-1)            # a mirrored filter: what a wrong tap order gives
+        y = bn(F.conv2d(y, w3, padding=1), b)
+        if mistake != "dropped-relu":
+            y = F.relu(y)
+        y = bn(F.conv2d(y, p["residual_function.6.weight"]), 7)
+        return F.relu(y) + x if mistake == "shortcut-before-relu" else F.relu(y + x)
+    with pytest.raises(AssertionError):
+        _compare_with_modules(wrong, ol.BottleneckCfg(in_channels=64, mid_channels=16))
+
+
 @pytest.mark.parametrize("adam_w,wd", [(True, 0.0), (True, 0.01), (False, 0.01)])
 def test_adam_matches_torch(adam_w, wd):
     torch.manual_seed(3)

@@ -145,3 +145,41 @@ def test_redundancy_ids():
     assert osched.redundant_stage_ids(1, 3, 4) == [0]
     assert osched.redundant_user_stage_ids(1, 2, 4) == [1]
     assert osched.redundant_user_stage_ids(1, 0, 4) == [3]
+
+
+def test_lazy_merge_hand_trace():
+    """S = 4, M = 2, worked by hand from the three branches of the reference
+    (schedule.py:483-501).  T = 10 steps, first half = steps 0..4.  L = RecvActivation(-1), C = SendActivation(-1);
+    a stage's forward steps are those of its own parity.
+      stage 0: L on steps 0, 2, 4, 6, 8 (every forward step, valid micro-batch or not)
+      stage 1: quiet steps of the first half are 0 (backward parity -> C) only (1..4 carry transfers)
+      stage 2: quiet steps 0 (forward parity -> L) and 1 (-> C)
+      stage 3: L on quiet forward steps of the first half: 1 (3 carries RecvActivation(0));
+               C on every step with stage 0's forward parity: 0, 2, 4, 6, 8, in front of everything else"""
+    M, S = 2, 4
+    pings = {}
+    for s in range(S):
+        steps = osched.lazy_merge(osched.train_schedule(M, S, s), M, S, s)
+        pings[s] = {i: [c[0][0] for c in cmds if c[1] == -1] for i, cmds in enumerate(steps) if any(c[1] == -1 for c in cmds)}
+        # nothing but pings is added, and pings come first
+        for got, own in zip(steps, osched.train_schedule(M, S, s)):
+            assert [c for c in got if c[1] != -1] == own
+            n = sum(1 for c in got if c[1] == -1)
+            assert all(c[1] == -1 for c in got[:n])
+    assert pings[0] == {0: ["R"], 2: ["R"], 4: ["R"], 6: ["R"], 8: ["R"]}
+    assert pings[1] == {0: ["S"]}
+    assert pings[2] == {0: ["R"], 1: ["S"]}
+    assert pings[3] == {0: ["S"], 1: ["R"], 2: ["S"], 4: ["S"], 6: ["S"], 8: ["S"]}
+
+
+@pytest.mark.parametrize("S,M", [(S, M) for S in range(2, 7) for M in range(1, 11) if M >= S - 1])
+def test_lazy_pings_pair_up_around_the_ring(S, M):
+    """A one-element send is a blocking transfer: whenever stage s calls its successor, the successor (the
+    first stage for the last one) listens in the same step, and nobody listens without a caller.  Holds from
+    M >= S - 1 on (with fewer micro-batches the reference's own rule leaves a few pings unanswered)."""
+    streams = [osched.lazy_merge(osched.train_schedule(M, S, s), M, S, s) for s in range(S)]
+    for i in range(osched.total_steps(M, S)):
+        for s in range(S):
+            calls = [c for c in streams[s][i] if c[:2] == ("SendActivation", -1)]
+            listens = [c for c in streams[(s + 1) % S][i] if c[:2] == ("RecvActivation", -1)]
+            assert len(calls) == len(listens) <= 1, (i, s)

@@ -105,6 +105,15 @@ def test_lazy_schedule_pings():
         assert len(extra) == (0 if talks or not first_half else 1)
 
 
+@pytest.mark.parametrize("stages,mbs", [(s, m) for s in range(2, 7) for m in range(1, 11)])
+def test_lazy_schedule_equals_oracle(stages, mbs):
+    """First, middle and last stage branches of LazyRecoverySchedule (reference schedule.py:483-501)."""
+    for sid in range(stages):
+        mk = lambda s: S.TrainSchedule(micro_batches=mbs, stages=stages, stage_id=s)
+        got = as_tuples(S.LazyRecoverySchedule(mk(sid), mk((sid + 1) % stages)))
+        assert got == osched.lazy_merge(osched.train_schedule(mbs, stages, sid), mbs, stages, sid)
+
+
 def test_redundancy_helpers():
     for level in (0, 1):
         for stages in range(1, 6):
