@@ -86,9 +86,13 @@ def layer_norm(x, gain, shift, kind, eps):
     return F.layer_norm(x, x.shape[-1:], gain, shift, eps)
 
 
-def activation(x, kind):
+def activation(x, kind, mask=None):
+    """``mask`` (relu only): use this 0/1 tensor as the ReLU's decision instead of ``x > 0``.  A low-precision
+    run decides ``x > 0`` on its own rounded ``x``; for the few pre-activations closer to zero than the
+    rounding error the decision differs from the exact one and the derivative jumps.  Feeding the run's own
+    decisions makes the comparison one of arithmetic, not of tie-breaking at the kink."""
     if kind == "relu":
-        return F.relu(x)
+        return F.relu(x) if mask is None else x * mask.to(x.dtype)
     if kind == "gelu_tanh":
         return F.gelu(x, approximate="tanh")
     raise ValueError(kind)
@@ -120,16 +124,16 @@ def attention(x, p, cfg, key_lens=None):
     return lin(3, ctx)
 
 
-def feed_forward(x, p, cfg):
+def feed_forward(x, p, cfg, relu_mask=None):
     u = F.linear(x, p["feed_forward.w_1.weight"], p["feed_forward.w_1.bias"])
-    return F.linear(activation(u, cfg.activation), p["feed_forward.w_2.weight"], p["feed_forward.w_2.bias"])
+    return F.linear(activation(u, cfg.activation, relu_mask), p["feed_forward.w_2.weight"], p["feed_forward.w_2.bias"])
 
 
-def transformer_layer(x, p, cfg, key_lens=None):
+def transformer_layer(x, p, cfg, key_lens=None, relu_mask=None):
     n1 = layer_norm(x, p["sublayer.0.norm.a_2"], p["sublayer.0.norm.b_2"], cfg.ln, cfg.eps)
     x = x + attention(n1, p, cfg, key_lens)
     n2 = layer_norm(x, p["sublayer.1.norm.a_2"], p["sublayer.1.norm.b_2"], cfg.ln, cfg.eps)
-    return x + feed_forward(n2, p, cfg)
+    return x + feed_forward(n2, p, cfg, relu_mask)
 
 
 # ---------------------------------------------------------------- ResNet bottleneck
@@ -183,17 +187,19 @@ def init_bottleneck_params(cfg, seed, dtype=torch.float32):
     return out
 
 
-def bottleneck(x, p, cfg):
+def bottleneck(x, p, cfg, relu_masks=None):
     """x is NCHW here (torch's convention).  Shortcut: the identity when stride is 1 and
-    Cin == 4*Cmid, else conv1x1(stride) + BN (resnet.py:66-72)."""
+    Cin == 4*Cmid, else conv1x1(stride) + BN (resnet.py:66-72).  ``relu_masks``: the decisions of
+    the block's three ReLUs, in order, to use instead of ``> 0`` (see :func:`activation`)."""
     bn = lambda t, key: F.batch_norm(t, None, None, p[f"{key}.weight"], p[f"{key}.bias"], training=True, eps=cfg.bn_eps)
-    y = F.relu(bn(F.conv2d(x, p["residual_function.0.weight"]), "residual_function.1"))
-    y = F.relu(bn(F.conv2d(y, p["residual_function.3.weight"], stride=cfg.stride, padding=1), "residual_function.4"))
+    m = relu_masks if relu_masks is not None else (None, None, None)
+    y = activation(bn(F.conv2d(x, p["residual_function.0.weight"]), "residual_function.1"), "relu", m[0])
+    y = activation(bn(F.conv2d(y, p["residual_function.3.weight"], stride=cfg.stride, padding=1), "residual_function.4"), "relu", m[1])
     y = bn(F.conv2d(y, p["residual_function.6.weight"]), "residual_function.7")
     sc = x
     if cfg.projection:
         sc = bn(F.conv2d(x, p["shortcut.0.weight"], stride=cfg.stride), "shortcut.1")
-    return F.relu(y + sc)
+    return activation(y + sc, "relu", m[2])
 
 
 def strip_triples(y, strip=32):

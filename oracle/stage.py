@@ -34,6 +34,7 @@ class OraclePeer:
     def __init__(self, activations, micro_batches, grads=None, targets=None, key_lens=None, labels=None):
         self.activations, self.M = activations, micro_batches
         self.grads, self.targets, self.key_lens = grads or {}, targets or {}, key_lens
+        self.relu_masks = {}      # (stage, k) -> per-layer ReLU decisions of the run the oracle is compared with
         self.labels = labels      # labels[k] of the last stage's own loss (LoadMicroBatch), if this process hosts it
         self.loss = 0.0
         self.dead_from, self.dead_stage = None, None
@@ -90,17 +91,20 @@ class OracleStage:
             layers.append({k: v.requires_grad_(True) for k, v in p.items()})
         self.params[stage] = layers
 
-    def forward(self, x, stage, key_lens=None):
+    def forward(self, x, stage, key_lens=None, relu_masks=None):
+        """``relu_masks``: per layer of the stage, the ReLU decisions to use (``oracle.layers.activation``):
+        one tensor [batch, seq, ffn] per transformer layer, three NCHW tensors per bottleneck block."""
+        masks = relu_masks if relu_masks is not None else [None] * len(self.params[stage])
         if isinstance(self.cfg, olayers.BottleneckCfg):
             # activations travel as [batch, H*W, C] (NHWC); torch convolutions want NCHW
             b, hw, c = x.shape
             side = int(round(hw ** 0.5))
             y = x.view(b, side, side, c).permute(0, 3, 1, 2)
-            for p in self.params[stage]:
-                y = olayers.bottleneck(y, p, self.cfg)
+            for p, m in zip(self.params[stage], masks):
+                y = olayers.bottleneck(y, p, self.cfg, m)
             return y.permute(0, 2, 3, 1).reshape(b, hw, c)
-        for p in self.params[stage]:
-            x = olayers.transformer_layer(x, p, self.cfg, key_lens)
+        for p, m in zip(self.params[stage], masks):
+            x = olayers.transformer_layer(x, p, self.cfg, key_lens, m)
         return x
 
     def named_grads(self, stage):
@@ -153,7 +157,7 @@ class OracleStage:
                 peer.loss = peer.loss + loss.detach()
             return
         kl = None if peer.key_lens is None else peer.key_lens[k]
-        out = self.forward(bufs["in"][(s, k)], s, kl)
+        out = self.forward(bufs["in"][(s, k)], s, kl, peer.relu_masks.get((s, k)))
         bufs["out"][(s, k)] = out
         if s == self.S - 1 and peer.labels is not None and s in self.stage_ids:
             # last stage: loss_model(outputs, labels), summed into total_loss (engine.py:1649-1663); counted

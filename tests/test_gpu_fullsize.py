@@ -1,6 +1,8 @@
-"""Checks at the full shapes of the benchmark configuration (GPT-2-medium stage: rows 8192, hidden 1024,
-ffn 4096, 16 heads, seq 1024) through properties that do not need a full CPU run: bit-reproducibility,
-oracle values on sampled rows / heads, softmax normalisation, causality, RC bit-exactness."""
+"""Checks at the full shapes of the benchmark configurations -- the GPT-2-medium stage (rows 8192, hidden 1024,
+ffn 4096, 16 heads, seq 1024) and the GPT-2-1.5B stage (rows 4096, hidden 1600, ffn 6400, 25 heads, seq 1024:
+1600 = 25 x 64 is no multiple of the 128- and 256-wide tiles) -- through properties that do not need a full CPU
+run: bit-reproducibility, oracle values on sampled rows / heads, softmax normalisation, causality, RC
+bit-exactness; plus one failover at the 1.5B layer shape against the CPU oracle."""
 import math
 
 import numpy as np
@@ -16,6 +18,9 @@ pytestmark = pytest.mark.gpu
 DEV = "cuda:0"
 MB, SEQ, HID, HEADS, FFN = 8, 1024, 1024, 16, 4096
 ROWS = MB * SEQ
+# GPT-2-1.5B stage
+MB5, HID5, HEADS5, FFN5 = 4, 1600, 25, 6400
+ROWS5 = MB5 * SEQ
 
 
 def randn(*shape, seed=0, scale=1.0, dtype=torch.bfloat16):
@@ -28,8 +33,13 @@ def l2(a, b):
     return float((a - b).norm() / b.norm())
 
 
-@pytest.mark.parametrize("layout,M,N,K", [(0, ROWS, FFN, HID), (0, ROWS, 3 * HID, HID), (0, ROWS, HID, FFN),
-                                          (1, ROWS, HID, FFN), (1, ROWS, FFN, HID), (2, FFN, HID, ROWS), (2, HID, HID, ROWS)])
+@pytest.mark.parametrize("layout,M,N,K", [
+    (0, ROWS, FFN, HID), (0, ROWS, 3 * HID, HID), (0, ROWS, HID, FFN),
+    (1, ROWS, HID, FFN), (1, ROWS, FFN, HID), (2, FFN, HID, ROWS), (2, HID, HID, ROWS),
+    # every product of a GPT-2-1.5B layer: forward (NT), input gradients (NN), weight gradients (TN)
+    (0, ROWS5, 3 * HID5, HID5), (0, ROWS5, HID5, HID5), (0, ROWS5, FFN5, HID5), (0, ROWS5, HID5, FFN5),
+    (1, ROWS5, HID5, 3 * HID5), (1, ROWS5, HID5, HID5), (1, ROWS5, HID5, FFN5), (1, ROWS5, FFN5, HID5),
+    (2, 3 * HID5, HID5, ROWS5), (2, HID5, HID5, ROWS5), (2, FFN5, HID5, ROWS5), (2, HID5, FFN5, ROWS5)])
 def test_gemm_full_shapes_sampled(hiplib, layout, M, N, K):
     a_shape = (K, M) if layout == hiplib.TN else (M, K)
     b_shape = (N, K) if layout == hiplib.NT else (K, N)
@@ -38,10 +48,12 @@ def test_gemm_full_shapes_sampled(hiplib, layout, M, N, K):
     if layout == hiplib.TN:
         C.zero_()
     hiplib.gemm(layout, A, B, C, accumulate=layout == hiplib.TN)
-    idx = torch.randint(0, M, (48,), generator=torch.Generator().manual_seed(3)).to(DEV)
+    # sampled rows, always with the first and the last one (the edges of the first and the last tile)
+    idx = torch.cat([torch.tensor([0, M - 1]), torch.randint(0, M, (46,), generator=torch.Generator().manual_seed(3))]).to(DEV)
     Ar = (A[:, idx].t() if layout == hiplib.TN else A[idx]).double()
     ref = Ar @ (B.double().t() if layout == hiplib.NT else B.double())
     assert l2(C[idx], ref) < 1e-2
+    assert l2(C[idx][:, -64:], ref[:, -64:]) < 1e-2       # the last columns: a partly filled tile when N % 256 != 0
     C2 = torch.zeros_like(C)
     hiplib.gemm(layout, A, B, C2, accumulate=layout == hiplib.TN)
     assert torch.equal(C, C2)
@@ -51,8 +63,10 @@ def test_gemm_full_shapes_sampled(hiplib, layout, M, N, K):
     assert torch.equal(C3.float(), C.float() * 2)
 
 
+@pytest.mark.parametrize("MB,HEADS", [(MB, HEADS), (MB5, HEADS5)], ids=["gpt2-medium", "gpt2-1.5b"])
 @pytest.mark.parametrize("mask", ["causal", "key_padding"])
-def test_attention_full_shape_properties(hiplib, mask):
+def test_attention_full_shape_properties(hiplib, mask, MB, HEADS):
+    ROWS = MB * SEQ
     h = HEADS * 64
     qkv = randn(ROWS, 3 * h, seed=4, scale=0.7)
     out, lse = torch.empty(ROWS, h, dtype=torch.bfloat16, device=DEV), torch.empty(MB, HEADS, SEQ, device=DEV)
@@ -99,7 +113,8 @@ def test_attention_full_shape_properties(hiplib, mask):
         assert float(dead.float().abs().max()) == 0.0
 
 
-def test_rc_bit_exact_full_layer(hiplib):
+@pytest.mark.parametrize("MB,HID,HEADS,FFN", [(MB, HID, HEADS, FFN), (MB5, HID5, HEADS5, FFN5)], ids=["gpt2-medium", "gpt2-1.5b"])
+def test_rc_bit_exact_full_layer(hiplib, MB, HID, HEADS, FFN):
     """One own + one shadow layer at the benchmark's layer shape: the redundant forward equals a normal
     forward of the same layer bit for bit, on either stream arrangement."""
     variant = dict(activation="gelu_tanh", ln="standard", mask="causal")
@@ -149,3 +164,62 @@ def test_adam_full_stage_arena(hiplib):
     assert torch.equal(LP, P.to(torch.bfloat16)) and float(G.abs().max()) == 0.0
     # first step with zero moments moves every parameter by lr * g/(|g| + eps') ~ lr
     assert float((P - p0).abs().max()) <= 1.001e-3
+
+
+def test_failover_at_the_gpt2_1p5b_layer_shape(hiplib):
+    """One own and one shadow layer of the GPT-2-1.5B stage (hidden 1600, 25 heads, ffn 6400, seq 1024,
+    micro-batch 4), two micro-batches, the successor preempted at the second: the promoted layer's backward runs
+    from the stashed redundant forward for micro-batch 0 and after a normal forward for micro-batch 1.  Gradients
+    of both stages and the loss against the CPU oracle (fp32 arithmetic on the engine's bf16 weights), 2e-2."""
+    from oracle.stage import OraclePeer, OracleStage
+    variant = dict(activation="gelu_tanh", ln="standard", mask="causal")
+    S, sid, M = 4, 1, 2
+    specs = [LayerSpec(TransformerLayer, HID5, HEADS5, FFN5, **variant) for _ in range(S)]
+    model = PipelineModule(specs, num_stages=S, partition_method="uniform", stage_id=sid, dtype=torch.bfloat16, device=DEV)
+    q = SeededActivationQueue((MB5, SEQ, HID5), torch.bfloat16, M, stage_ids=[sid, sid + 1], seed=13, grad_mode="mse", device=DEV)
+    cfg = {"train_micro_batch_size_per_gpu": MB5, "gradient_accumulation_steps": M, "bf16": {"enabled": True}}
+    engine, _, _, _ = bamboo_amd.initialize(model=model, config=cfg, redundancy_level=1, eager_recovery=True,
+                                            activation_queue=q, install_signal_handler=False)
+    st = OracleStage(ol.TransformerCfg(hidden=HID5, heads=HEADS5, ffn=FFN5, **variant), list(range(S + 1)), sid, M,
+                     dtype=torch.float32, redundancy_level=1, eager=True)
+    for s_ in list(st.params):
+        sp = engine.module.stage_params[s_]
+        named = sp.named(sp.compute)
+        for key, t in st.named_params(s_).items():
+            with torch.no_grad():
+                t.copy_(named[key].float().cpu())
+    acts = [a.float().cpu() for a in q.activations]
+    targets = [t.float().cpu() for t in q.targets[sid + 1]]
+    true_grads = []
+    for k in range(M):
+        o1 = st.forward(acts[k], sid).detach().requires_grad_(True)
+        (torch.nn.functional.mse_loss(st.forward(o1, sid + 1), targets[k]) / M).backward()
+        true_grads.append(o1.grad)
+    for layers in st.params.values():
+        for p in layers:
+            for t in p.values():
+                t.grad = None
+    peer = OraclePeer(acts, M, grads={sid: true_grads}, targets={sid + 1: targets})
+    peer.dead_from, peer.dead_stage = 1, sid
+    st.run_batch(peer, optimizer_step=False)
+
+    q.set_grads(sid, [g.view(MB5, SEQ, HID5) for g in true_grads])
+    q.targets.pop(sid)                      # own outputs go to a live successor, not to a loss head
+    orig_send = q.send_activation
+    q.send_activation = lambda k, t, stage_id, stream=None: (q._check_alive(k, stage_id) if stage_id == sid
+                                                              else orig_send(k, t, stage_id, stream=stream))
+    q.preempt_successor(1, sid)
+    from bamboo_amd import schedule
+    engine._INSTRUCTION_MAP = dict(engine._INSTRUCTION_MAP)
+    engine._INSTRUCTION_MAP[schedule.OptimizerStep] = lambda self_: None
+    loss = engine.train_batch()
+    torch.cuda.synchronize()
+    assert engine.stage_ids == [sid, sid + 1]
+    for s_ in (sid, sid + 1):
+        ref = st.named_grads(s_)
+        floor = 1e-3 * max(float(g.abs().max()) for g in ref.values())
+        for name, g in engine.module.get_named_grad(s_):
+            r = ref[name].double()
+            err = float((g.double().cpu() - r).norm() / r.norm().clamp_min(floor * r.numel() ** 0.5))
+            assert err < 2e-2, (s_, name, err)
+    assert abs(float(loss) - float(peer.loss) / M) < 2e-2 * float(peer.loss) / M

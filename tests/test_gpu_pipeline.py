@@ -132,6 +132,34 @@ def test_lost_stage_is_recovered_bit_exact(hiplib, dtype, victim, dead_from):
         assert torch.equal(got2[name], g), name
 
 
+@pytest.mark.parametrize("dead_from", [0, 1])
+@pytest.mark.parametrize("victim", [1, 2])
+def test_lazy_pipeline_notices_a_loss_through_its_pings(hiplib, victim, dead_from):
+    """Lazy recovery (no redundant forwards, one-element pings on silent steps): a stage lost at its first
+    micro-batches is noticed by its successor through a receive-ping (PrevStageException -- the successor keeps
+    its own stream and re-sends gradients) and by its predecessor through a send (NextStageException -- it
+    promotes the shadow stage from its host mirrors).  Gradients and loss equal the failure-free run bit for bit."""
+    dtype = torch.float32
+    data = make_data(dtype)
+    good = make_pipeline(dtype, data=data, eager=False)
+    freeze_optimizer(good)
+    loss_good = good.train_batch(sync_weights=False)
+    ref = all_grads(good)
+    pipe = make_pipeline(dtype, data=data, eager=False)
+    freeze_optimizer(pipe)
+    pipe.kill(victim, at_micro_batch=dead_from)
+    loss = pipe.train_batch(sync_weights=False)
+    torch.cuda.synchronize()
+    assert pipe.lost == [victim]
+    pred, succ = pipe.engines[victim - 1], pipe.engines[victim + 1]
+    assert pred.stage_ids == [victim - 1, victim] and succ.stage_ids == [victim + 1]
+    assert succ.last_failover is not None and succ.last_failover.get("role") == "successor of the lost stage"
+    assert float(loss) == float(loss_good)
+    got = all_grads(pipe)
+    for name, g in ref.items():
+        assert torch.equal(got[name], g), name
+
+
 @pytest.mark.parametrize("eager", [True, False], ids=["eager", "lazy"])
 @pytest.mark.parametrize("rc_stream", [False, True], ids=["one-stream", "rc-stream"])
 def test_training_through_a_failure_equals_training_without(hiplib, rc_stream, eager):

@@ -183,6 +183,35 @@ def test_bottleneck_pin_catches_plausible_mistakes(mistake):
         _compare_with_modules(wrong, ol.BottleneckCfg(in_channels=64, mid_channels=16))
 
 
+def test_relu_decisions_handed_in_reproduce_the_plain_run():
+    """With the decisions an exact run makes itself (x > 0) the masked variants are the plain functions, bit for
+    bit, outputs and gradients; with one decision flipped they are not."""
+    cfg = ol.BottleneckCfg(in_channels=64, mid_channels=16)
+    p, x = _bottleneck_case(cfg, 9)
+    y = ol.bottleneck(x, p, cfg)
+    y.sum().backward()
+    gx = x.grad.clone()
+    bn = lambda t, i: F.batch_norm(t, None, None, p[f"residual_function.{i}.weight"], p[f"residual_function.{i}.bias"], training=True, eps=cfg.bn_eps)
+    with torch.no_grad():
+        u1 = bn(F.conv2d(x, p["residual_function.0.weight"]), 1)
+        u2 = bn(F.conv2d(F.relu(u1), p["residual_function.3.weight"], padding=1), 4)
+        u3 = bn(F.conv2d(F.relu(u2), p["residual_function.6.weight"]), 7) + x
+    masks = (u1 > 0, u2 > 0, u3 > 0)
+    x.grad = None
+    ym = ol.bottleneck(x, p, cfg, masks)
+    ym.sum().backward()
+    assert torch.equal(ym, y) and torch.equal(x.grad, gx)
+    flipped = (masks[0].clone(), masks[1], masks[2])
+    flipped[0][0, 0, 0, 0] = ~flipped[0][0, 0, 0, 0]
+    assert not torch.equal(ol.bottleneck(x, p, cfg, flipped), y)
+    # transformer feed-forward
+    tcfg = ol.TransformerCfg(hidden=32, heads=4, ffn=64)
+    tp = {k: v.double() for k, v in ol.init_params(tcfg, 3).items()}
+    t = torch.randn(2, 5, 32, dtype=torch.float64)
+    u = F.linear(t, tp["feed_forward.w_1.weight"], tp["feed_forward.w_1.bias"])
+    assert torch.equal(ol.feed_forward(t, tp, tcfg, u > 0), ol.feed_forward(t, tp, tcfg))
+
+
 @pytest.mark.parametrize("adam_w,wd", [(True, 0.0), (True, 0.01), (False, 0.01)])
 def test_adam_matches_torch(adam_w, wd):
     torch.manual_seed(3)

@@ -20,12 +20,6 @@ def make_inputs(seed=0):
     return acts, targets, grads
 
 
-def single_stage_reference(acts, targets, stage_layers):
-    """own+shadow layers as ONE stage under plain gradient accumulation with the MSE head."""
-    st = OracleStage(CFG, [0, 0, 4, 4, 8], 1, M, dtype=torch.float64)  # stage 1 owns layers 0..3 ... see below
-    return st
-
-
 def test_rc_does_not_change_results():
     acts, targets, grads = make_inputs()
     res = []
@@ -80,6 +74,39 @@ def test_failover_equals_merged_stage(dead_from):
     for k in range(M):
         torch.testing.assert_close(bufs["sent_grad"][(1, k)], ref_bufs["sent_grad"][(1, k)], rtol=1e-9, atol=1e-11)
     assert abs(float(peer.loss) - float(ref_peer.loss)) < 1e-9
+
+
+@pytest.mark.parametrize("dead_from", [0, 1, 2, 3])
+def test_failover_onto_the_last_stage_equals_merged_stage(dead_from):
+    """Stage 2 of 4 shadows the LAST stage, which computes the loss from its own labels.  After the last
+    stage is lost, stage 2 ends the batch with the gradients and the loss of layers 4..7 run as one last
+    stage (3 stages, partition [0, 2, 4, 8]) on the same labels."""
+    acts, labels, _ = make_inputs(5)
+    ref = OracleStage(CFG, [0, 2, 4, 8], 2, M, dtype=torch.float64)
+    ref_peer = OraclePeer(acts, M, labels=labels)
+    ref_bufs, _ = ref.run_batch(ref_peer, optimizer_step=False)
+    ref_grads = ref.named_grads(2)
+
+    last = OracleStage(CFG, PARTS, 3, M, dtype=torch.float64)
+    own_probe = OracleStage(CFG, PARTS, 2, M, dtype=torch.float64)
+    true_grads = []
+    for k in range(M):
+        o1 = own_probe.forward(acts[k], 2).detach().requires_grad_(True)
+        (torch.nn.functional.mse_loss(last.forward(o1, 3), labels[k]) / M).backward()
+        true_grads.append(o1.grad)
+
+    st = OracleStage(CFG, PARTS, 2, M, dtype=torch.float64, redundancy_level=1, eager=True)
+    peer = OraclePeer(acts, M, grads={2: true_grads}, labels=labels)
+    peer.dead_from, peer.dead_stage = dead_from, 2
+    bufs, info = st.run_batch(peer, optimizer_step=False)
+    assert info["failed_step"] is not None and st.stage_ids == [2, 3]
+    got = {**st.named_grads(2), **st.named_grads(3)}
+    assert set(got) == set(ref_grads)
+    for k in ref_grads:
+        torch.testing.assert_close(got[k], ref_grads[k], rtol=1e-9, atol=1e-11)
+    for k in range(M):
+        torch.testing.assert_close(bufs["sent_grad"][(2, k)], ref_bufs["sent_grad"][(2, k)], rtol=1e-9, atol=1e-11)
+    assert abs(float(peer.loss) - float(ref_peer.loss)) < 1e-9 and float(peer.loss) > 0
 
 
 def test_optimizer_step_moves_parameters():
