@@ -5,6 +5,9 @@
 #include <stdio.h>
 #include <string.h>
 
+#include <mutex>
+#include <unordered_map>
+
 #include "../../include/bamboo_hip.h"
 
 typedef __bf16 bf16;
@@ -38,6 +41,24 @@ void bb_set_error(const char* fmt, ...);
     } while (0)
 
 #define BB_LAUNCH_CHECK() BB_HIP_CHECK(hipGetLastError())
+
+// Raises a kernel's dynamic-LDS limit to at least `bytes`, once per kernel, size and process.  Callers on several
+// threads may arrive together (one thread per pipeline stage, the interpreter lock released during the call): the
+// table is guarded, and a kernel counts as configured only after the call has succeeded.
+static inline hipError_t bb_allow_dynamic_lds(const void* kern, size_t bytes) {
+    static std::mutex mu;
+    static std::unordered_map<const void*, size_t> allowed;
+    std::lock_guard<std::mutex> lock(mu);
+    auto it = allowed.find(kern);
+    if (it != allowed.end() && it->second >= bytes) return hipSuccess;
+    if (bytes <= 64 * 1024 && it == allowed.end()) {   // the default limit covers it
+        allowed[kern] = 64 * 1024;
+        return hipSuccess;
+    }
+    const hipError_t e = hipFuncSetAttribute(kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes);
+    if (e == hipSuccess) allowed[kern] = bytes;
+    return e;
+}
 
 // ---- scalar conversions -----------------------------------------------------------------
 __device__ __forceinline__ float bf2f(uint16_t b) { return __uint_as_float(((uint32_t)b) << 16); }

@@ -336,11 +336,7 @@ static int ln_bwd_launch(int kind, int rows, int cols, float eps, const void* x,
     const int one_pass = all <= 128 * 1024;
     const size_t smem = one_pass ? all : (size_t)3 * 2 * cols * sizeof(float);
     auto kern = layernorm_bwd_kernel<T, IT>;
-    static size_t allowed = 64 * 1024;   // raised once per size, on the first (never captured) call that needs it
-    if (smem > allowed) {
-        BB_HIP_CHECK(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
-        allowed = smem;
-    }
+    BB_HIP_CHECK(bb_allow_dynamic_lds((const void*)kern, smem));   // raised on the first (never captured) call that needs it
     hipLaunchKernelGGL(kern, dim3(LN_BWD_BLOCKS), dim3(LN_BWD_WAVES * 64), smem, st, kind, rows, cols, eps, (const T*)x,
                        (const T*)gain, mean, rinv, (const T*)dy, (const T*)dres, (T*)dx, ws, one_pass);
     BB_LAUNCH_CHECK();

@@ -12,7 +12,6 @@
 // store, so the MFMA side never changes.
 #include "common.h"
 
-#include <stdlib.h>
 #include <utility>
 
 struct GemmArgs {
@@ -1079,11 +1078,7 @@ template <int BM, int BN, int WM, int WN, bool TA, bool TB>
 static int launch_bf16(GemmArgs& g, int batches, hipStream_t st) {
     constexpr int smem = 2 * (BM + BN) * 64 * 2;
     auto kern = gemm_bf16_kernel<BM, BN, WM, WN, TA, TB>;
-    static bool configured = false;
-    if (!configured) {
-        BB_HIP_CHECK(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, smem));
-        configured = true;
-    }
+    BB_HIP_CHECK(bb_allow_dynamic_lds((const void*)kern, smem));
     g.tiles_m = (g.M + BM - 1) / BM;
     g.tiles_n = (g.N + BN - 1) / BN;
     dim3 grid(g.tiles_m * g.tiles_n, 1, batches);
@@ -1109,11 +1104,7 @@ template <int BM, int BN, int WM, int WN, bool AKM, bool BKM, bool DB, int STAGE
 static int launch_bf16_dma(GemmArgs& g, int batches, hipStream_t st) {
     constexpr int smem = STAGES * (BM + BN) * BK * 2;
     auto kern = gemm_bf16_dma_kernel<BM, BN, WM, WN, AKM, BKM, DB, STAGES, BK>;
-    static bool configured = false;
-    if (!configured) {
-        BB_HIP_CHECK(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, smem));
-        configured = true;
-    }
+    BB_HIP_CHECK(bb_allow_dynamic_lds((const void*)kern, smem));
     g.tiles_m = (g.M + BM - 1) / BM;
     g.tiles_n = (g.N + BN - 1) / BN;
     dim3 grid(g.tiles_m * g.tiles_n, 1, batches);
@@ -1126,11 +1117,7 @@ template <int BM, int BN, int WM, int WN>
 static int launch_bf16_dma_stats(GemmArgs& g, hipStream_t st) {
     constexpr int smem = 3 * (BM + BN) * 64 * 2;
     auto kern = gemm_bf16_dma_stats_kernel<BM, BN, WM, WN>;
-    static bool configured = false;
-    if (!configured) {
-        BB_HIP_CHECK(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, smem));
-        configured = true;
-    }
+    BB_HIP_CHECK(bb_allow_dynamic_lds((const void*)kern, smem));
     g.tiles_m = (g.M + BM - 1) / BM;
     g.tiles_n = (g.N + BN - 1) / BN;
     hipLaunchKernelGGL(kern, dim3(g.tiles_m * g.tiles_n), dim3(WM * WN * 64), smem, st, g);
@@ -1139,30 +1126,15 @@ static int launch_bf16_dma_stats(GemmArgs& g, hipStream_t st) {
 }
 
 // DMA kernels need K % 32 == 0 and at least one full vector of rows; tile by problem size
-enum DmaTile { D_NONE = 0, D256x256, D256x128, D128x128, D_OFF, D256x256w8, D256x128w8, D256x256w8db, D256x128w8db,
-               D256x128w8s3, D128x128s3, D256x256w8s5, D256x128w8s6, D256x256w8s3, D256x128w4s3, D256x256k64, D256x128k64, D256x128k64s3, D128x128k64, D128x64k64s3, D128x64s3, D64x128k64s3, D64x128s3, D256x192k64 };
-static const char* const kDmaTileNames[] = {"", "dma256x256", "dma256x128", "dma128x128", "", "dma256x256w8", "dma256x128w8",
-                                            "dma256x256w8db", "dma256x128w8db", "dma256x128w8s3", "dma128x128s3",
-                                            "dma256x256w8s5", "dma256x128w8s6", "dma256x256w8s3", "dma256x128w4s3", "dma256x256k64",
-                                            "dma256x128k64", "dma256x128k64s3", "dma128x128k64", "dma128x64k64s3",
-                                            "dma128x64s3", "dma64x128k64s3", "dma64x128s3", "dma256x192k64"};
-// BB_DMA_TILE (tuning aid): 1..3 force a DMA tile where it is legal, 4 disables the DMA kernels.
-static int dma_tile_override() {
-    static const int v = [] {
-        const char* e = getenv("BB_DMA_TILE");
-        return e ? atoi(e) : 0;
-    }();
-    return v;
-}
+enum DmaTile { D_NONE = 0, D256x256w8db, D256x128w8db, D128x128s3, D256x256k64, D256x128k64s3, D128x128k64, D128x64k64s3, D128x64s3,
+               D64x128k64s3, D64x128s3, D256x192k64 };
+static const char* const kDmaTileNames[] = {"", "dma256x256w8db", "dma256x128w8db", "dma128x128s3", "dma256x256k64", "dma256x128k64s3",
+                                            "dma128x128k64", "dma128x64k64s3", "dma128x64s3", "dma64x128k64s3", "dma64x128s3",
+                                            "dma256x192k64"};
+// The tile of a problem depends on its shape and layout only (never on the stream, the environment or what ran
+// before): a redundant forward and a normal forward of the same layer run the same kernel and give the same bits.
 static DmaTile pick_dma_tile(int M, int N, int K, int64_t batches, int layout) {
     if (K % 32 != 0 || K < 64 || M < 128 || N < 128 || N % 8 != 0) return D_NONE;
-    const int ov = dma_tile_override();
-    if (ov == 4) return D_NONE;
-    if ((ov >= 1 && ov <= 3) || (ov >= 5 && ov <= 14) || (ov >= 15 && ov <= 18 && K % 64 == 0 && K >= 128)) return (DmaTile)ov;
-    if (ov == 23) return layout == BB_NT && K % 64 == 0 && K >= 128 ? D256x192k64 : D_NONE;
-    // 19..22: the narrow tiles, where their k-major operand is 128 wide (NT: 128x64, NN: 64x128)
-    if (ov == 19 || ov == 20) return layout == BB_NT ? (ov == 19 && K % 64 == 0 && K >= 128 ? D128x64k64s3 : D128x64s3) : D_NONE;
-    if (ov == 21 || ov == 22) return layout == BB_NN ? (ov == 21 && K % 64 == 0 && K >= 128 ? D64x128k64s3 : D64x128s3) : D_NONE;
     // Rules read off sweeps of M 2048..16384 x N 768..6400 x K 1024/4096 (NT and NN) on MI355X (256 CUs,
     // one block of the 256-row tiles per CU).
     //  - Operands whose rows are k-contiguous (both of NT, A of NN) load faster as 64-wide k-tiles: one
@@ -1229,21 +1201,10 @@ static DmaTile pick_dma_tile(int M, int N, int K, int64_t batches, int layout) {
 
 template <bool TA, bool TB> static int dispatch_bf16(GemmArgs& g, int batches, hipStream_t st) {
     switch (pick_dma_tile(g.M, g.N, g.K, batches, TA ? BB_TN : TB ? BB_NN : BB_NT)) {
-        case D256x256: return launch_bf16_dma<256, 256, 2, 2, TA, TB, true>(g, batches, st);
-        case D256x128: return launch_bf16_dma<256, 128, 2, 2, TA, TB, true>(g, batches, st);
-        case D128x128: return launch_bf16_dma<128, 128, 2, 2, TA, TB, true>(g, batches, st);
-        case D256x256w8: return launch_bf16_dma<256, 256, 2, 4, TA, TB, false>(g, batches, st);
-        case D256x128w8: return launch_bf16_dma<256, 128, 4, 2, TA, TB, false>(g, batches, st);
         case D256x256w8db: return launch_bf16_dma<256, 256, 2, 4, TA, TB, true>(g, batches, st);
         case D256x128w8db: return launch_bf16_dma<256, 128, 4, 2, TA, TB, true>(g, batches, st);
-        case D256x128w8s3: return launch_bf16_dma<256, 128, 4, 2, TA, TB, true, 3>(g, batches, st);
         case D128x128s3: return launch_bf16_dma<128, 128, 2, 2, TA, TB, true, 3>(g, batches, st);
-        case D256x256w8s5: return launch_bf16_dma<256, 256, 2, 4, TA, TB, true, 5>(g, batches, st);
-        case D256x128w8s6: return launch_bf16_dma<256, 128, 4, 2, TA, TB, true, 6>(g, batches, st);
-        case D256x256w8s3: return launch_bf16_dma<256, 256, 2, 4, TA, TB, true, 3>(g, batches, st);
-        case D256x128w4s3: return launch_bf16_dma<256, 128, 2, 2, TA, TB, true, 3>(g, batches, st);
         case D256x256k64: return launch_bf16_dma<256, 256, 2, 4, TA, TB, true, 2, 64>(g, batches, st);
-        case D256x128k64: return launch_bf16_dma<256, 128, 4, 2, TA, TB, true, 2, 64>(g, batches, st);
         case D256x128k64s3: return launch_bf16_dma<256, 128, 4, 2, TA, TB, true, 3, 64>(g, batches, st);
         case D128x128k64: return launch_bf16_dma<128, 128, 2, 2, TA, TB, true, 2, 64>(g, batches, st);
         case D128x64k64s3: return launch_bf16_dma<128, 64, 4, 1, TA, TB, true, 3, 64>(g, batches, st);
@@ -1357,7 +1318,7 @@ static int colsum_standalone(const bb_gemm_desc* d, void* stream) {
 extern "C" int bb_gemm_strip_stats_supported(const bb_gemm_desc* d) {
     return d && d->dtype == BB_BF16 && d->c_dtype == BB_BF16 && d->layout == BB_NT && d->nb1 <= 1 && d->nb2 <= 1 &&
            d->M >= 128 && d->N >= 64 && d->N % 8 == 0 && d->K >= 128 && d->K % 64 == 0 && d->conv_c == 0 && !d->colsum_out &&
-           !d->bias && d->epilogue == BB_EPI_NONE && d->alpha == 1.0f && dma_tile_override() == 0;
+           !d->bias && d->epilogue == BB_EPI_NONE && d->alpha == 1.0f;
 }
 extern "C" int64_t bb_strip_stats_workspace(int rows, int cols) { return (int64_t)((rows + 31) / 32) * 3 * cols; }
 
@@ -1402,11 +1363,7 @@ template <int BM, int BN, int WM, int WN, bool BKM, int STAGES, bool STATS = fal
 static int launch_conv3x3(GemmArgs& g, const ConvArgs& cv, hipStream_t st) {
     constexpr int smem = STAGES * (BM + BN) * 64 * 2;
     auto kern = conv3x3_bf16_igemm_kernel<BM, BN, WM, WN, BKM, STAGES, STATS>;
-    static bool configured = false;
-    if (!configured) {
-        BB_HIP_CHECK(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, smem));
-        configured = true;
-    }
+    BB_HIP_CHECK(bb_allow_dynamic_lds((const void*)kern, smem));
     g.tiles_m = (g.M + BM - 1) / BM;
     g.tiles_n = (g.N + BN - 1) / BN;
     hipLaunchKernelGGL(kern, dim3(g.tiles_m * g.tiles_n), dim3(WM * WN * 64), smem, st, g, cv);
@@ -1473,11 +1430,7 @@ template <bool TA, bool TB, bool CONVB = false> static int launch_grouped(Groupe
     constexpr int BM = 128, BN = 128, STAGES = 3;
     constexpr int smem = STAGES * (BM + BN) * 32 * 2;
     auto kern = gemm_bf16_dma_grouped_kernel<BM, BN, 2, 2, TA, TB, true, STAGES, CONVB>;
-    static bool configured = false;
-    if (!configured) {
-        BB_HIP_CHECK(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, smem));
-        configured = true;
-    }
+    BB_HIP_CHECK(bb_allow_dynamic_lds((const void*)kern, smem));
     int blocks = 0;
     for (int i = 0; i < G.count; ++i) {
         GemmArgs& g = G.p[i];
@@ -1503,7 +1456,7 @@ extern "C" int bb_gemm_grouped(const bb_gemm_desc* descs, int count, void* strea
     for (int i = 0; i < count && fuse; ++i) {
         const bb_gemm_desc& d = descs[i];
         fuse = d.dtype == BB_BF16 && d.layout == descs[0].layout && d.nb1 <= 1 && d.nb2 <= 1 && d.M > 0 && d.N > 0 &&
-               pick_dma_tile(d.M, d.N, d.K, 1, d.layout) != D_NONE && dma_tile_override() != 4;
+               pick_dma_tile(d.M, d.N, d.K, 1, d.layout) != D_NONE;
     }
     // a patch-matrix B exists only inside the grouped kernel: no one-by-one route for it
     BB_REQUIRE(fuse || !has_conv, "bb_gemm_grouped: a problem with a patch-matrix B must share a launch of bf16 BB_TN "
@@ -1572,7 +1525,7 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(const SplitkReduceAr
 
 // chunks of the contraction: 0 or 1 = run the group whole
 static int pick_splits(const bb_gemm_desc* descs, int count) {
-    if (count < 1 || count > GROUP_MAX || dma_tile_override() != 0) return 0;
+    if (count < 1 || count > GROUP_MAX) return 0;
     int64_t tiles = 0;
     int kmin = 1 << 30;
     for (int i = 0; i < count; ++i) {
@@ -1586,12 +1539,7 @@ static int pick_splits(const bb_gemm_desc* descs, int count) {
     }
     // Two blocks per CU on average: with one, a CU's four waves have nobody to hide their load and barrier waits
     // behind (the weight gradients of a ResNet block: 61.7 us at three chunks, 50.8 us at five).
-    // BB_SPLITK_FILL (tuning aid) overrides the 2.
-    static const int fill = [] {
-        const char* e = getenv("BB_SPLITK_FILL");
-        return e && atoi(e) > 0 ? atoi(e) : 2;
-    }();
-    int splits = (int)(256 * fill / tiles);
+    int splits = (int)(256 * 2 / tiles);
     if (splits > SPLITK_MAX) splits = SPLITK_MAX;
     if (splits > GROUP_MAX / count) splits = GROUP_MAX / count;
     while (splits > 1 && kmin / splits < 512) --splits;  // keep the pipelines of the chunks long

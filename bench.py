@@ -332,7 +332,8 @@ def main():
                    "eager_recovery": True, "rc_stream": bool(args.rc_stream), "hip_graphs": n_graphs if graphs else 0,
                    "samples_per_step": samples,
                    "attention": "n/a (convolutions as GEMMs over NHWC rows, 3x3 as implicit GEMMs)" if cfg.get("kind") == "resnet"
-                   else "fused (no score matrix in HBM); flops counted dense, the causal kernel skips masked tiles"},
+                   else ("unfused (fp32: scores and probabilities in HBM, as the reference); flops counted dense" if cfg["dtype"] == "fp32"
+                         else "fused (no score matrix in HBM); flops counted dense, the causal kernel skips masked tiles")},
         "rc_on_samples_per_s": round(samples / t_on, 3),
         "rc_off_samples_per_s": None if t_off is None else round(samples / t_off, 3),
         "rc_overhead_pct": None if t_off is None else round(100.0 * (t_on - t_off) / t_off, 2),
@@ -355,7 +356,12 @@ def main():
     if failover is not None:
         out["failover"] = failover
     if not args.no_cpu_baseline:
-        threads = min(os.cpu_count() or 1, 16)
+        # all host cores this process may run on (the affinity mask is what the box really grants; os.cpu_count()
+        # reports the machine's)
+        threads = len(os.sched_getaffinity(0)) if hasattr(os, "sched_getaffinity") else (os.cpu_count() or 1)
+        if os.environ.get("OMP_NUM_THREADS", "").isdigit():
+            # a GPU box exports its CPU share of the host here; more threads than that would be time-sliced
+            threads = min(threads, int(os.environ["OMP_NUM_THREADS"]))
         out["cpu_baseline"] = cpu_baseline(cfg, threads)
     print(json.dumps(out))
 
