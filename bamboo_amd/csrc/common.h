@@ -46,17 +46,18 @@ void bb_set_error(const char* fmt, ...);
 // threads may arrive together (one thread per pipeline stage, the interpreter lock released during the call): the
 // table is guarded, and a kernel counts as configured only after the call has succeeded.
 static inline hipError_t bb_allow_dynamic_lds(const void* kern, size_t bytes) {
+    if (bytes <= 64 * 1024) return hipSuccess;   // the default limit covers it
     static std::mutex mu;
-    static std::unordered_map<const void*, size_t> allowed;
+    static std::unordered_map<uintptr_t, size_t> allowed;   // (kernel, device) -> limit set so far
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return e;
+    const uintptr_t key = (uintptr_t)kern ^ ((uintptr_t)(dev + 1) << 56);
     std::lock_guard<std::mutex> lock(mu);
-    auto it = allowed.find(kern);
+    auto it = allowed.find(key);
     if (it != allowed.end() && it->second >= bytes) return hipSuccess;
-    if (bytes <= 64 * 1024 && it == allowed.end()) {   // the default limit covers it
-        allowed[kern] = 64 * 1024;
-        return hipSuccess;
-    }
-    const hipError_t e = hipFuncSetAttribute(kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes);
-    if (e == hipSuccess) allowed[kern] = bytes;
+    e = hipFuncSetAttribute(kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes);
+    if (e == hipSuccess) allowed[key] = bytes;
     return e;
 }
 

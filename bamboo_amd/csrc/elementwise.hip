@@ -18,6 +18,7 @@ void bb_set_error(const char* fmt, ...) {
 }
 extern "C" const char* bb_last_error(void) { return g_err; }
 extern "C" int bb_version(void) { return 1; }
+static int ln_bwd_static_setup(int dev);
 extern "C" int bb_init(void) {
     int dev = 0;
     BB_HIP_CHECK(hipGetDevice(&dev));
@@ -27,7 +28,7 @@ extern "C" int bb_init(void) {
         bb_set_error("bb_init: device %d is %s, this library is built for gfx950 only", dev, prop.gcnArchName);
         return BB_EHIP;
     }
-    return BB_OK;
+    return ln_bwd_static_setup(dev);   // so that bb_layernorm_bwd_static has nothing left to set up on this device
 }
 
 // =========================================================================================
@@ -379,16 +380,15 @@ extern "C" int bb_layernorm_fwd(int dtype, int kind, int rows, int cols, float e
 
 extern "C" int64_t bb_layernorm_bwd_workspace(int cols) { return (int64_t)LN_BWD_BLOCKS * 2 * cols; }
 
-extern "C" int bb_layernorm_bwd(int dtype, int kind, int rows, int cols, float eps, const void* x, const void* gain,
-                                const float* mean, const float* rinv, const void* dy, const void* dres, void* dx,
-                                float* dgain, float* dshift, float* workspace, void* stream) {
-    int rc = check_rowop("bb_layernorm_bwd", dtype, rows, cols);
+static int ln_bwd_run(const char* who, int dtype, int kind, int rows, int cols, float eps, const void* x, const void* gain,
+                      const float* mean, const float* rinv, const void* dy, const void* dres, void* dx, float* dgain,
+                      float* dshift, float* workspace, hipStream_t st) {
+    int rc = check_rowop(who, dtype, rows, cols);
     if (rc) return rc;
-    BB_REQUIRE(kind == BB_LN_STANDARD || kind == BB_LN_ANNOTATED, "bb_layernorm_bwd: bad kind %d", kind);
-    BB_REQUIRE(x && gain && mean && rinv && dy && dx && dgain && dshift && workspace, "bb_layernorm_bwd: null pointer");
-    BB_REQUIRE((size_t)3 * 2 * cols * sizeof(float) <= 160 * 1024, "bb_layernorm_bwd: cols (%d) too large (max 6826)", cols);
+    BB_REQUIRE(kind == BB_LN_STANDARD || kind == BB_LN_ANNOTATED, "%s: bad kind %d", who, kind);
+    BB_REQUIRE(x && gain && mean && rinv && dy && dx && dgain && dshift && workspace, "%s: null pointer", who);
+    BB_REQUIRE((size_t)3 * 2 * cols * sizeof(float) <= 160 * 1024, "%s: cols (%d) too large (max 6826)", who, cols);
     if (rows == 0) return BB_OK;
-    hipStream_t st = (hipStream_t)stream;
     auto finish = [&]() -> int {
         const int nb = (cols + 63) / 64;
         hipLaunchKernelGGL(reduce_partials_acc2_kernel, dim3(nb, 2), dim3(RED_WAVES * 64), 0, st, workspace, LN_BWD_BLOCKS,
@@ -405,6 +405,66 @@ extern "C" int bb_layernorm_bwd(int dtype, int kind, int rows, int cols, float e
     else
         BB_DISPATCH_IT(float, cols / 4, run(ln_bwd_launch<float, IT>(kind, rows, cols, eps, x, gain, mean, rinv, dy, dres, dx, workspace, st)));
     return BB_EINVAL;
+}
+
+extern "C" int bb_layernorm_bwd(int dtype, int kind, int rows, int cols, float eps, const void* x, const void* gain,
+                                const float* mean, const float* rinv, const void* dy, const void* dres, void* dx,
+                                float* dgain, float* dshift, float* workspace, void* stream) {
+    return ln_bwd_run("bb_layernorm_bwd", dtype, kind, rows, cols, eps, x, gain, mean, rinv, dy, dres, dx, dgain, dshift, workspace,
+                      (hipStream_t)stream);
+}
+
+// ---- the same for callers that cannot allocate ---------------------------------------------------------------
+// The per-block partial sums of dgain / dshift ([LN_BWD_BLOCKS][2][cols] floats) live in an array that is part of the
+// library's device image instead of a caller's workspace.  Every GPU the library runs on holds its own copy (2 MiB,
+// until the process ends) at its own address; host code reaches it only through the address that
+// hipGetSymbolAddress returns with that device current -- the array's name is no device address on the host.
+static __device__ __align__(256) float ln_bwd_static_scratch[LN_BWD_BLOCKS * 2 * BB_LN_BWD_STATIC_MAX_COLS];
+constexpr int LN_STATIC_MAX_DEVICES = 64;
+static float* g_ln_static_ptr[LN_STATIC_MAX_DEVICES];   // per device: address of its copy, null until set up
+static std::mutex g_ln_static_mu;
+
+template <typename T, int IT> static hipError_t ln_bwd_allow_one_pass() {
+    // the largest dynamic LDS request the kernel makes for cols <= BB_LN_BWD_STATIC_MAX_COLS: the one-pass layout
+    return bb_allow_dynamic_lds((const void*)layernorm_bwd_kernel<T, IT>, 128 * 1024);
+}
+// once per device, with that device current: the address of the device's copy, and every LDS-limit change the
+// entry point could otherwise need on its first call
+static int ln_bwd_static_setup(int dev) {
+    BB_REQUIRE(dev >= 0 && dev < LN_STATIC_MAX_DEVICES, "bb_layernorm_bwd_static: device ordinal %d out of range", dev);
+    std::lock_guard<std::mutex> lock(g_ln_static_mu);
+    if (g_ln_static_ptr[dev]) return BB_OK;
+    float* ptr = nullptr;
+    BB_HIP_CHECK(hipGetSymbolAddress((void**)&ptr, HIP_SYMBOL(ln_bwd_static_scratch)));
+    BB_REQUIRE(ptr != nullptr, "bb_layernorm_bwd_static: no address for the scratch array on device %d", dev);
+    BB_HIP_CHECK((ln_bwd_allow_one_pass<bf16, 2>()));
+    BB_HIP_CHECK((ln_bwd_allow_one_pass<bf16, 4>()));
+    BB_HIP_CHECK((ln_bwd_allow_one_pass<bf16, 8>()));
+    BB_HIP_CHECK((ln_bwd_allow_one_pass<bf16, 16>()));
+    BB_HIP_CHECK((ln_bwd_allow_one_pass<float, 2>()));
+    BB_HIP_CHECK((ln_bwd_allow_one_pass<float, 4>()));
+    BB_HIP_CHECK((ln_bwd_allow_one_pass<float, 8>()));
+    BB_HIP_CHECK((ln_bwd_allow_one_pass<float, 16>()));
+    g_ln_static_ptr[dev] = ptr;
+    return BB_OK;
+}
+
+extern "C" int bb_layernorm_bwd_static(int dtype, int kind, int rows, int cols, float eps, const void* x, const void* gain,
+                                       const float* mean, const float* rinv, const void* dy, const void* dres, void* dx,
+                                       float* dgain, float* dshift, void* stream) {
+    BB_REQUIRE(cols <= BB_LN_BWD_STATIC_MAX_COLS, "bb_layernorm_bwd_static: cols (%d) beyond the built-in scratch (max %d); "
+               "use bb_layernorm_bwd with a workspace", cols, BB_LN_BWD_STATIC_MAX_COLS);
+    int dev = 0;
+    BB_HIP_CHECK(hipGetDevice(&dev));
+    BB_REQUIRE(dev >= 0 && dev < LN_STATIC_MAX_DEVICES, "bb_layernorm_bwd_static: device ordinal %d out of range", dev);
+    if (!g_ln_static_ptr[dev]) {    // bb_init was not called on this device: set up now (not under stream capture)
+        int rc = ln_bwd_static_setup(dev);
+        if (rc) return rc;
+    }
+    // every block of the kernel writes its whole partial row (zeros where it had no rows) before the reduction
+    // reads it: nothing of the previous call's contents is read, so nothing has to be cleared
+    return ln_bwd_run("bb_layernorm_bwd_static", dtype, kind, rows, cols, eps, x, gain, mean, rinv, dy, dres, dx, dgain, dshift,
+                      g_ln_static_ptr[dev], (hipStream_t)stream);
 }
 
 // =========================================================================================

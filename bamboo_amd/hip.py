@@ -24,7 +24,7 @@ LN_CODES = {"standard": LN_STANDARD, "annotated": LN_ANNOTATED}
 
 EXPORTS = (
     "bb_version", "bb_last_error", "bb_init", "bb_gemm", "bb_gemm_grouped", "bb_gemm_splitk_workspace", "bb_gemm_grouped_splitk", "bb_gemm_variant", "bb_layernorm_fwd",
-    "bb_layernorm_bwd_workspace", "bb_layernorm_bwd", "bb_colsum_workspace", "bb_colsum_acc",
+    "bb_layernorm_bwd_workspace", "bb_layernorm_bwd", "bb_layernorm_bwd_static", "bb_colsum_workspace", "bb_colsum_acc",
     "bb_softmax_fwd", "bb_softmax_bwd", "bb_attention_fwd", "bb_attention_bwd", "bb_residual_add", "bb_act_fwd", "bb_bn_workspace", "bb_batchnorm_fwd", "bb_batchnorm_bwd", "bb_patch3x3", "bb_conv3x3_supported", "bb_conv3x3", "bb_gemm_strip_stats_supported", "bb_strip_stats_workspace", "bb_batchnorm_fwd_strips", "bb_mse_workspace", "bb_mse_fwd_bwd", "bb_graph_begin", "bb_graph_end", "bb_graph_launch", "bb_graph_destroy",
     "bb_adam_multi", "bb_cast", "bb_fill_f32",
 )
@@ -84,6 +84,7 @@ def lib():
     L.bb_layernorm_bwd_workspace.argtypes = [c_int]
     L.bb_layernorm_bwd_workspace.restype = c_int64
     L.bb_layernorm_bwd.argtypes = [c_int, c_int, c_int, c_int, c_float] + [c_void_p] * 11
+    L.bb_layernorm_bwd_static.argtypes = [c_int, c_int, c_int, c_int, c_float] + [c_void_p] * 10
     L.bb_colsum_workspace.argtypes = [c_int]
     L.bb_colsum_workspace.restype = c_int64
     L.bb_colsum_acc.argtypes = [c_int, c_int, c_int, c_void_p, c_int64, c_void_p, c_void_p, c_void_p]
@@ -309,6 +310,15 @@ def layernorm_bwd(x, gain, mean, rinv, dy, dres, dx, dgain, dshift, workspace, k
     check(lib().bb_layernorm_bwd(dtype_code(x.dtype), kind, rows, cols, eps, _ptr(x), _ptr(gain), _ptr(mean),
                                  _ptr(rinv), _ptr(dy), _ptr(dres), _ptr(dx), _ptr(dgain), _ptr(dshift),
                                  _ptr(workspace), stream_ptr(stream)), "bb_layernorm_bwd")
+
+
+def layernorm_bwd_static(x, gain, mean, rinv, dy, dres, dx, dgain, dshift, kind, eps, stream=None):
+    """:func:`layernorm_bwd` on the library's built-in scratch array: allocates nothing, cols <= 2048, calls that
+    overlap on one GPU race."""
+    rows, cols = x.shape
+    check(lib().bb_layernorm_bwd_static(dtype_code(x.dtype), kind, rows, cols, eps, _ptr(x), _ptr(gain), _ptr(mean),
+                                        _ptr(rinv), _ptr(dy), _ptr(dres), _ptr(dx), _ptr(dgain), _ptr(dshift),
+                                        stream_ptr(stream)), "bb_layernorm_bwd_static")
 
 
 def colsum_workspace(cols):

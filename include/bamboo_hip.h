@@ -163,6 +163,18 @@ int bb_layernorm_bwd(int dtype, int kind, int rows, int cols, float eps, const v
                      const void* gain, const float* mean, const float* rinv, const void* dy,
                      const void* dres, void* dx, float* dgain, float* dshift,
                      float* workspace, void* stream);
+/* The same without a workspace, for callers that cannot allocate device memory (code under HIP graph
+ * capture, serving loops, harnesses that forbid hipMalloc).  No counterpart in the reference.  The
+ * per-block partial sums live in an array inside the library's device image (2 MiB per GPU, held until
+ * the process ends); the call allocates nothing.  cols <= BB_LN_BWD_STATIC_MAX_COLS, else BB_EINVAL.
+ * All calls on one GPU share that array: calls that overlap in time on one GPU (two streams, two
+ * threads) race; calls on one stream are ordered and independent (nothing of an earlier call's contents
+ * is read).  bb_init() on a device completes the one-time set-up; otherwise the first call on that
+ * device does (do not make that first call under stream capture).                                  */
+#define BB_LN_BWD_STATIC_MAX_COLS 2048
+int bb_layernorm_bwd_static(int dtype, int kind, int rows, int cols, float eps, const void* x,
+                            const void* gain, const float* mean, const float* rinv, const void* dy,
+                            const void* dres, void* dx, float* dgain, float* dshift, void* stream);
 
 /* Column sums of a [rows, cols] matrix accumulated into an fp32 vector: the bias gradient of
  * nn.Linear (autograd of transformer.py:136-146,158).  workspace: fp32, at least

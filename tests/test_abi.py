@@ -38,6 +38,10 @@ def test_version_and_error_string():
     assert b"bad layout" in L.bb_last_error()
     assert L.bb_residual_add(1, 12, 1, 1, 1, None) == -1      # bf16 needs n % 8 == 0
     assert L.bb_adam_multi(1, None, None, None, None, None, None, 1e-3, 0.9, 0.999, 1e-8, 0, 1, 1, 0.0, 0, None) == -1
+    # the allocation-free LayerNorm backward refuses rows wider than its built-in scratch array
+    one = ctypes.c_void_p(16)
+    assert L.bb_layernorm_bwd_static(1, 0, 8, 4096, 1e-5, one, one, one, one, one, None, one, one, one, None) == -1
+    assert b"beyond the built-in scratch" in L.bb_last_error()
 
 
 def test_convolution_entry_points_validate_on_the_host():

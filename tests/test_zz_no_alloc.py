@@ -1,0 +1,71 @@
+"""The allocation-free entry point ``bb_layernorm_bwd_static`` against ``bb_layernorm_bwd`` (same kernels, the
+partial sums in the library's built-in scratch array instead of a caller's workspace): bit-equal results through
+the C ABI on two calls in a row, the second on a smaller input, for both dtypes and both LayerNorm kinds."""
+import ctypes
+
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+def _case(hip, dtype, rows, cols, seed, kind):
+    g = torch.Generator(device=DEV).manual_seed(seed)
+    mk = lambda *s: torch.randn(*s, generator=g, device=DEV).to(dtype)
+    x, dy, dres, gain, shift = mk(rows, cols), mk(rows, cols), mk(rows, cols), mk(cols), mk(cols)
+    y = torch.empty_like(x)
+    mean, rinv = torch.empty(rows, device=DEV), torch.empty(rows, device=DEV)
+    eps = 1e-5 if kind == hip.LN_STANDARD else 1e-6
+    hip.layernorm_fwd(x, gain, shift, y, mean, rinv, kind, eps)
+    return x, gain, mean, rinv, dy, dres, eps
+
+
+def _run(hip, static, case, kind, fill):
+    x, gain, mean, rinv, dy, dres, eps = case
+    rows, cols = x.shape
+    dx = torch.full_like(x, fill)
+    # dgain / dshift are accumulated: start both runs from the same non-zero contents
+    dgain = torch.full((cols,), 0.25, device=DEV)
+    dshift = torch.full((cols,), -0.5, device=DEV)
+    if static:
+        # torch's allocator sees no request during the call (the library's own hipMalloc calls would not show
+        # here; it makes none: the scratch is part of its device image)
+        n0 = torch.cuda.memory_stats()["allocation.all.allocated"]
+        hip.layernorm_bwd_static(x, gain, mean, rinv, dy, dres, dx, dgain, dshift, kind, eps)
+        assert torch.cuda.memory_stats()["allocation.all.allocated"] == n0
+    else:
+        ws = torch.full((hip.layernorm_bwd_workspace(cols),), float("nan"), device=DEV)
+        hip.layernorm_bwd(x, gain, mean, rinv, dy, dres, dx, dgain, dshift, ws, kind, eps)
+    torch.cuda.synchronize()
+    return dx, dgain, dshift
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32], ids=["bf16", "fp32"])
+@pytest.mark.parametrize("kind_name", ["standard", "annotated"])
+def test_static_entry_point_equals_the_workspace_one(hiplib, dtype, kind_name):
+    hip = hiplib
+    kind = hip.LN_CODES[kind_name]
+    # first call: GPT-2-1.5B rows (1600 columns, the two-phase reduction); second, right after it: fewer and
+    # narrower rows (one-pass reduction), so stale partial sums of the first call lie beyond and inside its range
+    shapes = [(4096, 1600), (520, 1024), (24, 2048), (8, 64)]
+    for i, (rows, cols) in enumerate(shapes):
+        case = _case(hip, dtype, rows, cols, seed=31 + i, kind=kind)
+        ref = _run(hip, False, case, kind, fill=1.0)
+        got = _run(hip, True, case, kind, fill=2.0)
+        for a, b, name in zip(got, ref, ("dx", "dgain", "dshift")):
+            assert torch.equal(a, b), (rows, cols, name)
+        assert float(got[1].abs().max()) > 1.0      # the gradients did land on top of the initial contents
+        del case, ref, got
+
+
+def test_static_entry_point_rejects_what_does_not_fit(hiplib):
+    hip = hiplib
+    L = hip.lib()
+    one = ctypes.c_void_p(16)
+    rc = L.bb_layernorm_bwd_static(hip.BF16, hip.LN_STANDARD, 8, 2056, 1e-5, one, one, one, one, one, None, one, one, one, None)
+    assert rc == -1 and b"beyond the built-in scratch" in L.bb_last_error()
+    x = torch.zeros(4, 4096, dtype=torch.bfloat16, device=DEV)
+    v = torch.zeros(4096, device=DEV)
+    with pytest.raises(hip.HipKernelError):
+        hip.layernorm_bwd_static(x, x[0], v[:4], v[:4], x, None, x, v, v, hip.LN_STANDARD, 1e-5)
