@@ -46,7 +46,8 @@ class PipelineEngine:
     def __init__(self, args=None, model=None, optimizer=None, model_parameters=None, training_data=None,
                  lr_scheduler=None, mpu=None, dist_init_required=None, collate_fn=None, config=None,
                  config_params=None, redundancy_level=0, sync_save=False, eager_recovery=False, prev_state={},
-                 activation_queue=None, rc_stream=False, install_signal_handler=True, use_graphs=False):
+                 activation_queue=None, rc_stream=False, install_signal_handler=True, use_graphs=False,
+                 rc_issue="reference", rc_backlog=None):
         if not isinstance(model, PipelineModule):
             raise PipelineError("model must base PipelineModule")
         hip.init()
@@ -105,6 +106,30 @@ class PipelineEngine:
                                 "(torch.cuda.stream(...)): the default stream cannot be captured")
         self._graphs = {}
         self.rc_stream = torch.cuda.Stream(self.device) if (rc_stream and self.r_stage_ids and eager_recovery) else None
+        # When a redundant forward is issued (results never depend on it, only timing):
+        #   "reference": where EagerRecoverySchedule puts it, in front of the own step that waits for a gradient
+        #                (schedule.py:504-524);
+        #   "asap":      onto the second stream as soon as the own forward it depends on has been issued;
+        #   "bubble":    into the pipeline's bubbles.  A redundant forward becomes *pending* once its input exists.
+        #                Whenever the own stream is about to wait for a neighbour (a receive whose tensor is not
+        #                there yet), pending forwards go to the second stream one layer at a time until the tensor
+        #                arrives.  Only when more than `rc_backlog` are pending (the number the idle time behind the
+        #                last own forward can absorb: cool-down, the wait for the stages in front to finish, the
+        #                next batch's fill) is the oldest issued alongside own work; what is pending at the end of
+        #                the batch is issued then.
+        if rc_issue not in ("reference", "asap", "bubble"):
+            raise PipelineError(f"rc_issue must be 'reference', 'asap' or 'bubble', got {rc_issue!r}")
+        if rc_issue != "reference" and self.r_stage_ids and eager_recovery and self.rc_stream is None:
+            raise PipelineError(f"rc_issue={rc_issue!r} needs rc_stream=True: on one stream an early redundant forward "
+                                "would run in front of the own work instead of in its gaps")
+        self.rc_issue = rc_issue
+        # idle time behind the last own forward, in forward slots (a backward taken as two): S-1-s cool-down gaps,
+        # s backward slots until stage 0 has finished, s forward slots until the next batch reaches this stage
+        self.rc_backlog = rc_backlog if rc_backlog is not None else (self.num_stages - 1 - self.stage_id) + 3 * self.stage_id
+        self._rc_pending = []      # micro-batches whose redundant forward is still to be issued, oldest first
+        self._rc_partial = None    # [micro-batch, next layer, its input] of a forward issued layer by layer
+        self._rc_forced = False
+        self._own_tail = None      # event behind the last pass issued to the own stream
         built = list(self.stage_ids) + (list(self.r_stage_ids) if self.eager_recovery else [])
         self.ctx = model.prepare_context(built, self.batch, self.seq, stream=self.main_stream)
         self.rc_ctx = self.ctx
@@ -278,6 +303,7 @@ class PipelineEngine:
         self.queue.start_batch()
         self.total_loss.zero_()
         self._loss_done = set()
+        self._rc_forced = False
         self._debug = debug
         t0 = time.perf_counter()
 
@@ -302,6 +328,8 @@ class PipelineEngine:
                 self._install_sched_generator()
             else:
                 raise exc
+        if self.rc_issue == "bubble" and self.r_stage_ids:
+            self._rc_flush()     # runs while the stages in front finish the batch and the next one fills the pipeline
         if hasattr(self.queue, "end_batch"):
             self.queue.end_batch(self.stage_ids)
         if self.rc_stream is not None:
@@ -379,6 +407,8 @@ class PipelineEngine:
                 self.pipe_buffers[key] = [None] * self.micro_batches
         if self.rc_stream is not None:
             self.main_stream.wait_stream(self.rc_stream)
+        # redundant forwards not issued, or issued in part: the replay runs them as ordinary forwards
+        self._rc_pending, self._rc_partial = [], None
         self.rc_ctx = self.ctx
         self.optimizer.add_stage(absorbed, self.module.stage_params[absorbed])
         self.stage_ids.append(absorbed)
@@ -435,6 +465,8 @@ class PipelineEngine:
             # local hand-off: the producer's output buffer stays valid until the end of the batch
             self.pipe_buffers[key][buffer_id] = self.pipe_buffers[f"output_{producer}"][buffer_id]
         else:
+            if hasattr(self.queue, "activation_arrived"):
+                self._fill_bubble(lambda: self.queue.activation_arrived(buffer_id))
             x = self.queue.recv_activation(buffer_id)
             self.pipe_buffers[key][buffer_id] = x.view(-1, x.shape[-1])
 
@@ -453,6 +485,8 @@ class PipelineEngine:
         if stage_id + 1 in self.stage_ids:
             self.grad_layer[stage_id] = self.pipe_buffers[f"input_grad_{stage_id + 1}"][buffer_id]
         else:
+            if hasattr(self.queue, "grad_arrived"):
+                self._fill_bubble(lambda: self.queue.grad_arrived(buffer_id, stage_id))
             g = self.queue.recv_grad(buffer_id, stage_id)
             self.grad_layer[stage_id] = g.view(-1, g.shape[-1])
 
@@ -474,6 +508,8 @@ class PipelineEngine:
             return
         inputs = self.pipe_buffers["data" if stage_id == 0 else f"input_{stage_id}"][buffer_id]
         redundant = stage_id in self.r_stage_ids
+        if redundant and self.rc_issue == "bubble" and not self._rc_forced:
+            return      # issued from the bubbles, the backlog limit or the end of the batch instead
         ctx = self.rc_ctx if redundant else self.ctx
         ctx.key_len = self.queue.key_len(buffer_id)
         ctx.redundant = redundant
@@ -489,8 +525,105 @@ class PipelineEngine:
         self.pipe_buffers[out_key][buffer_id] = out
         if not redundant and self.rc_stream is not None:
             self._fwd_done[buffer_id].record(self.main_stream)
+        if not redundant and hasattr(self.queue, "note_done"):
+            self.queue.note_done("F", buffer_id, stage_id, self.main_stream)
+        if not redundant and self.rc_issue == "bubble":
+            self._mark_own_tail()
+        if (not redundant and self.rc_stream is not None and stage_id == self.stage_id and self.r_stage_ids
+                and self.eager_recovery):
+            if self.rc_issue == "asap":
+                self._rc_issue_whole(buffer_id)
+            elif self.rc_issue == "bubble":
+                self._rc_pending.append(buffer_id)
+                while len(self._rc_pending) > self.rc_backlog:
+                    self._rc_issue_oldest()
         if last_with_loss and not redundant:
             self._loss_head(buffer_id, stage_id, out)
+
+    # ------------------------------------------------------------------ redundant forwards outside the stream's order
+    def _rc_issue_whole(self, k):
+        """The redundant forward of micro-batch ``k`` now (second stream, behind the own forward it reads)."""
+        nxt = self.r_stage_ids[0]
+        if nxt == self.num_stages - 1 and self.data_iterator is not None:
+            self._exec_load_micro_batch(k)
+        self._rc_forced = True
+        try:
+            self._exec_recv_activations(k, nxt)
+            self._exec_forward_pass(k, nxt)
+        finally:
+            self._rc_forced = False
+
+    def _rc_issue_oldest(self):
+        """Issue what is left of the oldest pending redundant forward in one go."""
+        k = self._rc_pending[0]
+        if self._rc_partial is not None and self._rc_partial[0] == k:
+            while self._rc_issue_layer() is not None and self._rc_partial is not None:
+                pass
+            return
+        self._rc_pending.pop(0)
+        self._rc_issue_whole(k)
+
+    def _rc_issue_layer(self):
+        """Issue ONE layer of the oldest pending redundant forward on the second stream; returns an event that
+        completes with it (None when nothing is pending).  Same kernels on the same operands as the whole forward:
+        the result does not depend on how the forward was cut."""
+        if not self._rc_pending:
+            return None
+        k, nxt = self._rc_pending[0], self.r_stage_ids[0]
+        n_layers = len(self.module.func_buckets[nxt])
+        if self.module.activation_checkpoint_interval > 0:
+            self._rc_pending.pop(0)      # checkpointed stashes are filled by whole forwards only
+            self._rc_issue_whole(k)
+        else:
+            ctx = self.rc_ctx
+            if self._rc_partial is None or self._rc_partial[0] != k:
+                if nxt == self.num_stages - 1 and self.data_iterator is not None:
+                    self._exec_load_micro_batch(k)
+                self._exec_recv_activations(k, nxt)
+                self.rc_stream.wait_event(self._fwd_done[k])
+                self._rc_partial = [k, 0, self.pipe_buffers[f"input_{nxt}"][k]]
+                self._deferred[(nxt, k)] = True
+            _, i, x = self._rc_partial
+            ctx.key_len = self.queue.key_len(k)
+            ctx.redundant = True
+            out = self.module.forward(x, nxt, slot=k, ctx=ctx, defer=True, layers=(i, i + 1))
+            if i + 1 == n_layers:
+                self.pipe_buffers[f"output_{nxt}"][k] = out
+                self._rc_pending.pop(0)
+                self._rc_partial = None
+            else:
+                self._rc_partial = [k, i + 1, out]
+        ev = torch.cuda.Event()
+        ev.record(self.rc_stream)
+        return ev
+
+    def _fill_bubble(self, arrived):
+        """The own stream is about to wait for a neighbour: pending redundant forwards go out, one layer at a time,
+        until ``arrived()`` says the awaited tensor is there (the layer in flight then overlaps the own pass that
+        follows, for a fraction of a millisecond)."""
+        if self.rc_issue != "bubble" or self.rc_stream is None or not self.r_stage_ids:
+            return
+        while self._rc_pending and not arrived():
+            if self._own_tail is not None and not self._own_tail.query():
+                time.sleep(0)      # the host is ahead of the GPU: the own stream still has work, this is no bubble yet
+                continue
+            ev = self._rc_issue_layer()
+            while ev is not None and not ev.query():
+                if arrived():
+                    return
+                time.sleep(0)
+
+    def _mark_own_tail(self):
+        self._own_tail = torch.cuda.Event()
+        self._own_tail.record(self.main_stream)
+
+    def _rc_flush(self):
+        """End of the batch: what is still pending goes out once the own stream has drained (the last own backward
+        is what the stages in front are waiting for; nothing may share the GPU with it)."""
+        if self._rc_pending and self._own_tail is not None:
+            self._own_tail.synchronize()
+        while self._rc_pending:
+            self._rc_issue_oldest()
 
     def _loss_head(self, buffer_id, stage_id, out):
         """Loss of one micro-batch on the last stage and its gradient scaled by 1 / micro_batches
@@ -523,6 +656,10 @@ class PipelineEngine:
         if key in self.pipe_buffers:
             self.pipe_buffers[key][buffer_id] = dst
         self.grad_layer[stage_id] = None
+        if hasattr(self.queue, "note_done"):
+            self.queue.note_done("B", buffer_id, stage_id, self.main_stream)
+        if self.rc_issue == "bubble":
+            self._mark_own_tail()
 
     def _exec_reduce_grads(self, stage_id):
         # data-parallel world of one: the all-reduce of deepspeed/runtime/engine.py:1773-1802 is the identity

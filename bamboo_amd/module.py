@@ -362,15 +362,29 @@ class PipelineModule:
         return nbytes_total
 
     # ------------------------------------------------------------------ execution
-    def forward(self, forward_input, stage_id, slot=0, ctx=None, defer=False):
+    def forward(self, forward_input, stage_id, slot=0, ctx=None, defer=False, layers=None):
         """``defer``: leave out of the stash what only a backward pass reads and this forward can
-        produce later from what it does keep (``backward(..., deferred=True)`` then produces it first)."""
-        layers = self.func_buckets.get(stage_id)
-        if layers is None:
+        produce later from what it does keep (``backward(..., deferred=True)`` then produces it first).
+        ``layers=(a, b)``: only layers a..b-1 of the stage (``forward_input`` is then the input of layer a):
+        a forward cut into pieces runs the same kernels on the same operands as a whole one."""
+        stage_layers = self.func_buckets.get(stage_id)
+        if stage_layers is None:
             raise Exception(f"Unregistered stage id {stage_id}")
-        self.micro_offset += 1
         x = forward_input
         stash = self._stash[stage_id][slot]
+        if layers is not None:
+            if self.activation_checkpoint_interval != 0:
+                raise PipelineError("a forward cut into layer ranges needs the full stash (no activation checkpointing)")
+            a, b = layers
+            if a == 0:
+                self.micro_offset += 1
+            ctx.defer = defer
+            for i in range(a, b):
+                x = stage_layers[i].forward(x, stash[i], ctx)
+            ctx.defer = False
+            return x
+        layers = stage_layers
+        self.micro_offset += 1
         if self.activation_checkpoint_interval == 0:
             ctx.defer = defer
             for layer, st in zip(layers, stash):

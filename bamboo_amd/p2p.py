@@ -138,6 +138,182 @@ class SeededActivationQueue:
 
 
 # =============================================================================================
+# A seeded queue that makes the stage wait as a real pipeline would: the bubbles of 1F1B
+# =============================================================================================
+import time  # noqa: E402
+
+
+class PipelineClock:
+    """Closed-loop model of the OTHER stages of an S-stage 1F1B pipeline around one real stage.
+
+    Every other stage executes the forward / backward passes of its ``TrainSchedule`` stream in order; a
+    forward takes ``t_fwd`` seconds, a backward ``t_bwd``; ``F(s, k)`` starts when stage ``s`` is free and
+    ``F(s-1, k)`` has ended, ``B(s, k)`` when stage ``s`` is free and ``B(s+1, k)`` has ended (transfers
+    take no time: the reference's p2p moves 17 MB over a link that does it in 0.1 ms).  The passes of the
+    real stage enter with the times the GPU really finished them (:meth:`note_done`), so a real stage that
+    falls behind delays its neighbours and, through them, what it receives later -- the loop is closed.
+
+    What the real stage asks: when does ``RecvActivation(k)`` find its tensor (= end of ``F(s-1, k)``), when
+    ``RecvGrad(k)`` (= end of ``B(s+1, k)``), and when does the whole pipeline finish the batch (= the last
+    backward of stage 0)."""
+
+    def __init__(self, stages, stage_id, micro_batches, t_fwd, t_bwd):
+        from .schedule import BackwardPass, ForwardPass, TrainSchedule
+        self.S, self.sid, self.M, self.t_fwd, self.t_bwd = stages, stage_id, micro_batches, float(t_fwd), float(t_bwd)
+        self.order = {}     # stage -> [(kind, k)] in execution order
+        self.before = {}    # (stage, kind, k) -> the pass the stage runs right before it
+        for s in range(stages):
+            seq = []
+            for cmds in TrainSchedule(micro_batches=micro_batches, stages=stages, stage_id=s):
+                for c in cmds:
+                    if type(c) is ForwardPass:
+                        seq.append(("F", c.buffer_id))
+                    elif type(c) is BackwardPass:
+                        seq.append(("B", c.buffer_id))
+            self.order[s] = seq
+            for i, (kind, k) in enumerate(seq):
+                self.before[(s, kind, k)] = None if i == 0 else (s,) + seq[i - 1]
+        self.start_batch(0.0)
+
+    def start_batch(self, t0):
+        """A batch whose first pass (stage 0's first forward) may start at ``t0`` (seconds on the clock's axis): 0 for
+        a pipeline that starts empty, the previous batch's :meth:`pipeline_end` for batches run back to back."""
+        self.t0 = t0
+        self.end = {}        # (stage, kind, k) -> seconds on the clock's axis
+        self.real = {}       # (kind, k) of the real stage -> callable returning seconds on that axis (blocks until known)
+
+    def note_done(self, kind, k, when):
+        """``when()``: the time on the clock's axis at which the real stage finished this pass (may block
+        until the GPU has got there)."""
+        self.real[(kind, k)] = when
+
+    def end_of(self, s, kind, k):
+        key = (s, kind, k)
+        if key in self.end:
+            return self.end[key]
+        if s == self.sid:
+            if (kind, k) not in self.real:
+                raise RuntimeError(f"pipeline clock: {kind}({k}) of the real stage {s} is needed before it was issued")
+            t = self.real[(kind, k)]()
+        else:
+            prev = self.before[key]
+            t = self.t0 if prev is None else self.end_of(*prev)
+            if kind == "F" and s > 0:
+                t = max(t, self.end_of(s - 1, "F", k))
+            if kind == "B" and s < self.S - 1:
+                t = max(t, self.end_of(s + 1, "B", k))
+            t += self.t_fwd if kind == "F" else self.t_bwd
+        self.end[key] = t
+        return t
+
+    def activation_at(self, k):
+        return self.end_of(self.sid - 1, "F", k) if self.sid > 0 else self.t0
+
+    def grad_at(self, k):
+        return self.end_of(self.sid + 1, "B", k) if self.sid < self.S - 1 else self.t0
+
+    def pipeline_end(self):
+        """When the last stage to finish the batch (stage 0, with its last backward) is done."""
+        return max(self.end_of(s, *self.order[s][-1]) for s in range(self.S))
+
+
+class PacedActivationQueue(SeededActivationQueue):
+    """:class:`SeededActivationQueue` whose receives return when a real pipeline would deliver.
+
+    ``RecvActivation(k)`` / ``RecvGrad(k)`` wait ON THE HOST (no kernel spins) until the moment a
+    :class:`PipelineClock` gives for the tensor, then hand over the resident seeded tensor.  Because the
+    engine issues a pass only after its receive has returned, the GPU really idles in the warm-up, wherever
+    the stage is ahead of its neighbours, and in the cool-down: the bubbles of 1F1B exist, and what the
+    engine has queued on another stream (redundant forwards) runs in them.  The stage's own passes are
+    timed with events on their stream; their GPU completion times feed the clock."""
+
+    def __init__(self, shape, dtype, micro_batches, stage_ids, stages, stage_id, t_fwd, t_bwd, **kw):
+        super().__init__(shape, dtype, micro_batches, stage_ids, **kw)
+        self.clock = PipelineClock(stages, stage_id, micro_batches, t_fwd, t_bwd)
+        self.stage_id = stage_id
+        self.waited = 0.0          # host seconds spent waiting for deliveries in this batch
+        self.batch_seconds = None  # of the last finished batch: from its start to the pipeline's end
+        self.batches = 0           # batches since the last reset()
+        self._base = None
+
+    def reset(self):
+        """The next batch starts a new run: GPU drained, empty pipeline, time zero."""
+        self._base = None
+
+    def start_batch(self):
+        """Batches run back to back: a batch starts on the pipeline's clock when the previous one has ended there
+        (stage 0 is free for its first forward), whatever this stage's GPU still has queued -- redundant forwards left
+        over from the previous batch run in the pipeline's fill time, as they would between real batches."""
+        super().start_batch()
+        if self._base is None:
+            torch.cuda.synchronize(self.device)
+            self._base = torch.cuda.Event(enable_timing=True)
+            self._base.record(torch.cuda.current_stream(self.device))
+            self._base.synchronize()
+            self._t0 = time.perf_counter()
+            self.clock.start_batch(0.0)
+            self.batches = 0
+        else:
+            self.clock.start_batch(self._last_end)
+        self.waited = 0.0
+
+    def note_done(self, kind, k, stage_id, stream):
+        """Called by the engine after it has issued forward / backward pass ``k`` of its own stage."""
+        if stage_id != self.stage_id:
+            return
+        ev = torch.cuda.Event(enable_timing=True)
+        ev.record(stream)
+        base = self._base
+
+        def when():
+            ev.synchronize()
+            return base.elapsed_time(ev) * 1e-3
+        self.clock.note_done(kind, k, when)
+
+    def _wait_until(self, t):
+        target = self._t0 + t
+        t_in = time.perf_counter()
+        while True:
+            left = target - time.perf_counter()
+            if left <= 0:
+                break
+            time.sleep(min(left, 2e-4) if left > 3e-4 else 0)
+        self.waited += time.perf_counter() - t_in
+
+    def activation_arrived(self, k):
+        """Non-consuming: has ``RecvActivation(k)`` nothing left to wait for?  (May itself wait for this stage's own
+        earlier passes to finish on the GPU: what the neighbours send depends on them.)"""
+        return time.perf_counter() >= self._t0 + self.clock.activation_at(k)
+
+    def grad_arrived(self, k, stage_id):
+        return stage_id != self.stage_id or time.perf_counter() >= self._t0 + self.clock.grad_at(k)
+
+    def recv_activation(self, k):
+        self._wait_until(self.clock.activation_at(k))
+        return super().recv_activation(k)
+
+    def recv_grad(self, k, stage_id):
+        self._check_alive(k, stage_id)
+        if stage_id == self.stage_id:
+            self._wait_until(self.clock.grad_at(k))
+        return super().recv_grad(k, stage_id)
+
+    def end_batch(self, stage_ids):
+        """The batch ends when the pipeline's last pass does (stage 0's last backward, which waits for every gradient
+        this stage sends: the delays this stage caused are in it)."""
+        self._last_end = self.clock.pipeline_end()
+        self.batch_seconds = self._last_end - self.clock.t0
+        self.batches += 1
+
+    def finish(self):
+        """Seconds from the start of the first batch after :meth:`reset` to the later of the pipeline's end of the
+        last batch and the moment this stage's GPU work, redundant forwards included, has drained."""
+        torch.cuda.synchronize(self.device)
+        drained = time.perf_counter() - self._t0
+        return max(self._last_end, drained)
+
+
+# =============================================================================================
 # Several stages in one process: a mailbox fabric between engines that run in threads
 # =============================================================================================
 import threading  # noqa: E402

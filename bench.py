@@ -10,6 +10,7 @@ the dominant kernel (measured with HIP events around its launches inside the tim
 and a ``cpu_baseline`` object (the CPU oracle timed on a bounded sample of the same workload).
 """
 import argparse
+import gc
 import json
 import os
 import sys
@@ -52,11 +53,14 @@ MEASURED_TRAFFIC_BYTES = {
 }
 
 
-def build_engine(cfg, rc, rc_stream, seed=1138, use_graphs=False):
+def build_engine(cfg, rc, rc_stream, seed=1138, use_graphs=False, paced=None, rc_issue="reference"):
+    """``paced=(t_fwd, t_bwd)``: the neighbours are a closed-loop model of the other stages of a 1F1B pipeline whose
+    forward / backward passes take that long, so the stage waits for its inputs as in a real pipeline."""
     import torch
 
     import bamboo_amd
     from bamboo_amd import BottleNeck, LayerSpec, PipelineModule, SeededActivationQueue, TransformerLayer
+    from bamboo_amd.p2p import PacedActivationQueue
     dtype = torch.bfloat16 if cfg["dtype"] == "bf16" else torch.float32
     if cfg.get("kind") == "resnet":
         specs = [LayerSpec(BottleNeck, cfg["hidden"], cfg["mid"], height=cfg["side"], width=cfg["side"])
@@ -66,16 +70,72 @@ def build_engine(cfg, rc, rc_stream, seed=1138, use_graphs=False):
                  for _ in range(cfg["layers"] * STAGES)]
     model = PipelineModule(specs, num_stages=STAGES, partition_method="uniform", stage_id=STAGE_ID, dtype=dtype,
                            device="cuda:0")
-    q = SeededActivationQueue((cfg["mb"], cfg["seq"], cfg["hidden"]), dtype, cfg["M"],
-                              stage_ids=[STAGE_ID, STAGE_ID + 1], seed=seed, grad_mode=cfg["grad_mode"],
-                              device="cuda:0", key_len_range=cfg.get("key_len_range"))
+    qargs = dict(stage_ids=[STAGE_ID, STAGE_ID + 1], seed=seed, grad_mode=cfg["grad_mode"], device="cuda:0",
+                 key_len_range=cfg.get("key_len_range"))
+    if paced is not None:
+        q = PacedActivationQueue((cfg["mb"], cfg["seq"], cfg["hidden"]), dtype, cfg["M"], stages=STAGES, stage_id=STAGE_ID,
+                                 t_fwd=paced[0], t_bwd=paced[1], **qargs)
+    else:
+        q = SeededActivationQueue((cfg["mb"], cfg["seq"], cfg["hidden"]), dtype, cfg["M"], **qargs)
     ds = {"train_micro_batch_size_per_gpu": cfg["mb"], "gradient_accumulation_steps": cfg["M"],
           "optimizer": {"type": "Adam", "params": {"lr": 1e-3, "betas": [0.9, 0.999], "eps": 1e-8}},
           "bf16": {"enabled": cfg["dtype"] == "bf16"}}
     engine, _, _, _ = bamboo_amd.initialize(model=model, config=ds, redundancy_level=1 if rc else 0,
                                             eager_recovery=rc, activation_queue=q, rc_stream=rc_stream,
-                                            install_signal_handler=False, use_graphs=use_graphs)
+                                            install_signal_handler=False, use_graphs=use_graphs, rc_issue=rc_issue)
     return engine, q
+
+
+def measure_pass_times(engine, q):
+    """Median GPU time of one forward and one backward pass of the stage's own layers (seconds), from events
+    recorded behind every pass of one batch on an otherwise idle GPU: consecutive passes run back to back on one
+    stream, so a pass lasts from the previous pass's end to its own."""
+    import torch
+    marks = []
+
+    def note_done(kind, k, stage_id, stream):
+        ev = torch.cuda.Event(enable_timing=True)
+        ev.record(stream)
+        marks.append((kind, ev))
+    q.note_done = note_done
+    torch.cuda.synchronize()
+    base = torch.cuda.Event(enable_timing=True)
+    base.record(torch.cuda.current_stream())
+    engine.train_batch()
+    torch.cuda.synchronize()
+    del q.note_done
+    durs = {"F": [], "B": []}
+    prev = base
+    for i, (kind, ev) in enumerate(marks):
+        if i > 0:                        # the first pass also carries the start of the batch
+            durs[kind].append(prev.elapsed_time(ev) * 1e-3)
+        prev = ev
+    med = lambda v: sorted(v)[len(v) // 2]
+    return med(durs["F"]), med(durs["B"])
+
+
+def paced_leg(cfg, rc, rc_issue, t_fwd, t_bwd, steps, warmup):
+    """Batch time (seconds, mean of ``steps`` batches) of the stage inside the closed-loop pipeline model, graphs on
+    (one launch per pass: the host never holds the GPU back after a receive has returned)."""
+    import torch
+    work = torch.cuda.Stream()
+    work.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(work):
+        engine, q = build_engine(cfg, rc=rc, rc_stream=rc, use_graphs=True, paced=(t_fwd, t_bwd), rc_issue=rc_issue)
+        for _ in range(max(warmup, 3)):      # eager batch, capturing batch, first replay
+            engine.train_batch()
+        q.reset()
+        waits, per_batch = [], []
+        for _ in range(steps):
+            engine.train_batch()
+            waits.append(q.waited)
+            per_batch.append(q.batch_seconds)
+        total = q.finish()
+    del engine, q
+    gc.collect()
+    torch.cuda.empty_cache()
+    mean = lambda v: sum(v) / len(v)
+    return {"batch_s": total / steps, "host_wait_s": mean(waits), "first_batch_s": per_batch[0], "later_batches_s": mean(per_batch[1:] or per_batch)}
 
 
 def time_steps(engine, steps, warmup):
@@ -217,6 +277,8 @@ def main():
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="first run three 256 MiB fp32 copies (cast_kernel<float,float>): the known-size kernel that "
                          "FETCH_SIZE / WRITE_SIZE counters of a --pmc run are scaled by")
+    ap.add_argument("--no-paced", action="store_true",
+                    help="skip the legs that run the stage inside the closed-loop model of a 4-stage 1F1B pipeline")
     ap.add_argument("--failover-at", type=int, default=None,
                     help="also measure a failover: the successor is preempted at this micro-batch (config c5: 7)")
     args = ap.parse_args()
@@ -247,10 +309,14 @@ def main():
 
     # leg 1: RC off (plain 1F1B stream of the stage)
     t_off = None
+    pass_times = None
     if not args.skip_rc_off:
         engine, q = build_engine(cfg, rc=False, rc_stream=False, use_graphs=graphs)
         t_off = time_steps(engine, args.steps, args.warmup)
+        if not args.no_paced:
+            pass_times = measure_pass_times(engine, q)
         del engine, q
+        gc.collect()      # engines hold reference cycles (schedule generators, captured graphs)
         torch.cuda.empty_cache()
 
     # leg 2: RC on, everything on one stream; GEMM launches are bracketed with events here, where
@@ -272,6 +338,7 @@ def main():
     # configuration `value` is quoted on
     if args.rc_stream:
         del engine, q
+        gc.collect()      # engines hold reference cycles (schedule generators, captured graphs)
         torch.cuda.empty_cache()
         engine, q = build_engine(cfg, rc=True, rc_stream=True, use_graphs=graphs)
         t_on = time_steps(engine, args.steps, args.warmup)
@@ -353,6 +420,30 @@ def main():
         model = lambda t_with_rc: round(100.0 * max(0.0, (t_with_rc - t_off) - idle) / (t_off + idle), 2)
         out["rc_overhead_bubble_model_pct"] = {"stages": STAGES, "single_stream": model(t_on_serial),
                                                "second_stream": model(t_on)}
+    if pass_times is not None:
+        # The stage inside a pipeline that has bubbles: the other three stages are a closed-loop model (their passes
+        # take what this stage's own passes take, they react to what this stage really sends and when), receives
+        # wait on the host until the model delivers.  RC off and RC on run under the same model; the redundant
+        # forwards go to the second stream either where the reference places them or as soon as their input exists.
+        t_fwd, t_bwd = pass_times
+        off = paced_leg(cfg, False, "reference", t_fwd, t_bwd, args.steps, args.warmup)
+        legs = {issue: paced_leg(cfg, True, issue, t_fwd, t_bwd, args.steps, args.warmup) for issue in ("reference", "asap", "bubble")}
+        best = min(legs, key=lambda k: legs[k]["batch_s"])
+        pct = lambda leg: round(100.0 * (leg["batch_s"] - off["batch_s"]) / off["batch_s"], 2)
+        r3 = lambda d: {k: round(v * 1e3, 3) for k, v in d.items()}
+        out["rc_overhead_paced_pct"] = pct(legs[best])
+        out["paced"] = {
+            "model": f"closed-loop {STAGES}-stage 1F1B, stage {STAGE_ID} real, neighbours' passes = this stage's measured "
+                     "forward/backward, host-side waits, HIP graphs; batches back to back (a batch starts when the pipeline has finished the "
+                     "previous one), batch_s = (start of the first batch -> max(pipeline end of the last, own GPU work drained)) / steps",
+            "t_fwd_ms": round(t_fwd * 1e3, 3), "t_bwd_ms": round(t_bwd * 1e3, 3),
+            "ideal_batch_ms": round((cfg["M"] + STAGES - 1) * (t_fwd + t_bwd) * 1e3, 3),
+            "rc_off_ms": r3(off), "rc_on_reference_ms": r3(legs["reference"]), "rc_on_asap_ms": r3(legs["asap"]), "rc_on_bubble_ms": r3(legs["bubble"]),
+            "rc_overhead_reference_pct": pct(legs["reference"]), "rc_overhead_asap_pct": pct(legs["asap"]),
+            "rc_overhead_bubble_pct": pct(legs["bubble"]),
+            "rc_issue_quoted": best,
+            "rc_off_samples_per_s": round(samples / off["batch_s"], 3),
+            "rc_on_samples_per_s": round(samples / legs[best]["batch_s"], 3)}
     if failover is not None:
         out["failover"] = failover
     if not args.no_cpu_baseline:

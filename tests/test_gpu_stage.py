@@ -483,6 +483,43 @@ def test_activation_checkpointing_resnet_keeps_running_statistics(hiplib):
             assert float(ra[idx][0].abs().sum()) > 0      # the running mean has moved off its zero start
 
 
+@pytest.mark.parametrize("rc_issue", ["reference", "asap", "bubble"])
+def test_paced_pipeline_changes_timing_not_results(hiplib, rc_issue):
+    """The stage inside the closed-loop pipeline model (receives wait on the host until a 4-stage 1F1B pipeline
+    would deliver; redundant forwards on the second stream, placed as the reference places them or issued as soon
+    as their input exists): losses and weights after three batches are bit-equal to the always-ready queue, the
+    stage really waited, and no batch beat the pipeline's own length."""
+    from bamboo_amd.p2p import PacedActivationQueue
+    hid, heads, ffn, L, S, sid, mb, M, seq = 128, 2, 256, 2, 4, 1, 2, 6, 64
+    dtype = torch.bfloat16
+    ref_engine, _ = build(hid, heads, ffn, L, S, sid, mb, M, seq, dtype, GPT_VARIANT, 1, True, grad_mode="mse", rc_stream=True)
+    ref_losses = [float(ref_engine.train_batch()) for _ in range(3)]
+    t_fwd, t_bwd = 2e-3, 4e-3
+    specs = [LayerSpec(TransformerLayer, hid, heads, ffn, **GPT_VARIANT) for _ in range(L * S)]
+    model = PipelineModule(specs, num_stages=S, partition_method="uniform", stage_id=sid, dtype=dtype, device=DEV)
+    q = PacedActivationQueue((mb, seq, hid), dtype, M, stage_ids=[sid, sid + 1], stages=S, stage_id=sid, t_fwd=t_fwd,
+                             t_bwd=t_bwd, seed=7, grad_mode="mse", device=DEV)
+    cfg = {"train_micro_batch_size_per_gpu": mb, "gradient_accumulation_steps": M,
+           "optimizer": {"type": "Adam", "params": {"lr": 1e-3}}, "bf16": {"enabled": True}}
+    engine, _, _, _ = bamboo_amd.initialize(model=model, config=cfg, redundancy_level=1, eager_recovery=True,
+                                            activation_queue=q, rc_stream=True, rc_issue=rc_issue, install_signal_handler=False)
+    losses = []
+    for _ in range(3):
+        losses.append(float(engine.train_batch()))
+        # this stage's own passes are far shorter than its neighbours': the batch is at most one slot shorter than
+        # a balanced pipeline's (M + S - 1) slots
+        assert q.batch_seconds >= (M + S - 2) * (t_fwd + t_bwd)
+        assert q.waited > (S - 1) * t_fwd          # at least the warm-up of the pipeline was spent waiting
+    assert q.finish() >= 3 * (M + S - 2) * (t_fwd + t_bwd) and q.batches == 3
+    torch.cuda.synchronize()
+    assert losses == ref_losses
+    for s_ in (sid, sid + 1):
+        a, b = engine.module.stage_params[s_], ref_engine.module.stage_params[s_]
+        assert torch.equal(a.master, b.master) and torch.equal(a.exp_avg_sq, b.exp_avg_sq)
+    with pytest.raises(bamboo_amd.PipelineError):
+        build(hid, heads, ffn, L, S, sid, mb, M, seq, dtype, GPT_VARIANT, 1, True, rc_issue="asap")   # needs the second stream
+
+
 def test_optimizer_step_matches_oracle(hiplib):
     rel_err.lowp = False
     hid, heads, ffn, L, S, sid, mb, M, seq = 128, 2, 256, 2, 4, 1, 2, 4, 64
