@@ -1,0 +1,1064 @@
+// Device side of the GEMM family (kernels, operand loaders, fragment readers, epilogues) and the per-kernel launch
+// templates; the host-side tile choice and the C entry points are in gemm.hip.
+#pragma once
+#include "common.h"
+
+#include <utility>
+
+struct GemmArgs {
+    const void* A; const void* B; void* C;
+    const void* bias; const void* aux_in; void* aux_out; const void* resid;
+    float* colsum;  // TN only: += column sums of A over K (the bias gradient of a linear layer)
+    int64_t lda, ldb, ldc, ldaux;
+    int64_t sA1, sA2, sB1, sB2, sC1, sC2;
+    int M, N, K, nb2;
+    float alpha;
+    int epilogue, act, accumulate, c_f32;
+    int tiles_m, tiles_n;
+    int conv_h, conv_w, conv_c, conv_row0;  // TN: B is the 3x3 patch matrix of an NHWC tensor (conv_c > 0)
+    float* strip_stats;  // [ceil(M / 32)][3][N]: per 32-row strip and output column (pivot, sum (c - pivot), sum (c - pivot)^2)
+};
+
+// ---- tile order: consecutive logical tiles land on the same XCD (workgroups are dealt
+// round-robin over the 8 XCDs, each with a private L2), and walk the output in column
+// panels of GROUP_M row-tiles so that an XCD's resident tiles share A rows and B columns.
+// logical tile -> (row tile, column tile): column panels of GROUP_M row-tiles
+__device__ __forceinline__ void panel_coords(int lid, int tiles_m, int tiles_n, int& tm, int& tn) {
+    constexpr int GROUP_M = 8;
+    const int width = GROUP_M * tiles_n;
+    const int group = lid / width;
+    const int first_m = group * GROUP_M;
+    const int gsize = min(tiles_m - first_m, GROUP_M);
+    tm = first_m + (lid % width) % gsize;
+    tn = (lid % width) / gsize;
+}
+// block id -> logical tile such that XCD x (which receives the block ids = x mod 8) owns the
+// contiguous range [x * total / 8, (x + 1) * total / 8) of logical tiles
+__device__ __forceinline__ int xcd_contiguous(int bid, int total) {
+    const int per = total / 8;
+    return (per > 0 && bid < per * 8) ? (bid % 8) * per + bid / 8 : bid;
+}
+__device__ __forceinline__ void tile_coords(int bid, int tiles_m, int tiles_n, int& tm, int& tn) {
+    panel_coords(xcd_contiguous(bid, tiles_m * tiles_n), tiles_m, tiles_n, tm, tn);
+}
+
+// Generic scalar epilogue.  T = operand dtype (bias/aux/resid), output fp32 or T.
+template <typename T>
+__device__ __forceinline__ void epilogue_elem(const GemmArgs& g, int64_t coff, int64_t xoff, int m,
+                                              int n, float acc) {
+    float v = acc * g.alpha;
+    if (g.bias) v += Elem<T>::load((const T*)g.bias + n);
+    const int64_t ci = coff + (int64_t)m * g.ldc + n;
+    const int64_t xi = xoff + (int64_t)m * g.ldaux + n;
+    if (g.epilogue == BB_EPI_ACT) {
+        if (g.aux_out) Elem<T>::store((T*)g.aux_out + xi, v);
+        v = act_f(v, g.act);
+    } else if (g.epilogue == BB_EPI_DACT) {
+        v *= dact_f(Elem<T>::load((const T*)g.aux_in + xi), g.act);
+    } else if (g.epilogue == BB_EPI_RESIDUAL) {
+        v += Elem<T>::load((const T*)g.resid + xi);
+    } else if (g.epilogue == BB_EPI_MUL) {
+        v *= Elem<T>::load((const T*)g.aux_in + xi);
+    } else if (g.epilogue == BB_EPI_ACT_DACT) {
+        float a, d;
+        act_dact_f(v, g.act, a, d);
+        Elem<T>::store((T*)g.aux_out + xi, d);
+        v = a;
+    }
+    if (g.c_f32) {
+        float* c = (float*)g.C + ci;
+        *c = g.accumulate ? (*c + v) : v;
+    } else {
+        Elem<T>::store((T*)g.C + ci, v);
+    }
+}
+
+// Vector epilogue for bf16 operands: 8 consecutive columns of one row (n % 8 == 0, n + 8 <= N).
+__device__ __forceinline__ void epilogue_vec8(const GemmArgs& g, int64_t coff, int m, int n, float (&v)[8]) {
+    const int64_t ci = coff + (int64_t)m * g.ldc + n;
+    const int64_t xi = coff + (int64_t)m * g.ldaux + n;
+    if (g.bias) {
+        float b[8];
+        load_vec((const bf16*)g.bias + n, b);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) v[e] += b[e];
+    }
+    if (g.epilogue == BB_EPI_ACT) {
+        if (g.aux_out) store_vec((bf16*)g.aux_out + xi, v);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) v[e] = act_f(v[e], g.act);
+    } else if (g.epilogue == BB_EPI_DACT) {
+        float u[8];
+        load_vec((const bf16*)g.aux_in + xi, u);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) v[e] *= dact_f(u[e], g.act);
+    } else if (g.epilogue == BB_EPI_RESIDUAL) {
+        float r[8];
+        load_vec((const bf16*)g.resid + xi, r);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) v[e] += r[e];
+    } else if (g.epilogue == BB_EPI_MUL) {
+        float d[8];
+        load_vec((const bf16*)g.aux_in + xi, d);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) v[e] *= d[e];
+    } else if (g.epilogue == BB_EPI_ACT_DACT) {
+        float d[8];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) act_dact_f(v[e], g.act, v[e], d[e]);
+        store_vec((bf16*)g.aux_out + xi, d);
+    }
+    if (g.c_f32) {
+        float* c = (float*)g.C + ci;
+        f32x4 lo = {v[0], v[1], v[2], v[3]}, hi = {v[4], v[5], v[6], v[7]};
+        if (g.accumulate) {
+            lo += *(const f32x4*)c;
+            hi += *(const f32x4*)(c + 4);
+        }
+        *(f32x4*)c = lo;
+        *(f32x4*)(c + 4) = hi;
+    } else {
+        store_vec((bf16*)g.C + ci, v);
+    }
+}
+
+template <typename F, int... Is> __device__ __forceinline__ void static_for(F&& f, std::integer_sequence<int, Is...>) {
+    (f(std::integral_constant<int, Is>{}), ...);
+}
+
+// =========================================================================================
+// bf16 kernel
+// =========================================================================================
+__device__ __forceinline__ int swz(int row) {
+    return ((row >> 1) & 7) ^ ((row & 1) << 2) ^ ((row >> 4) & 7);
+}
+
+// Loader of one operand tile: R tile rows (m or n index) x 64 k.  TR = operand memory is
+// k-major ([K, rows], rows contiguous).
+template <int R, int NT, bool TR> struct TileLoader;
+
+template <int R, int NT> struct TileLoader<R, NT, false> {
+    static constexpr int NCH = R * 8 / NT;  // 16-byte chunks per thread
+    static_assert(NCH >= 1, "tile too small for the block");
+    u32x4 regs[NCH];
+    __device__ __forceinline__ void gload(const bf16* base, int64_t ld, int row0, int rows, int k0,
+                                          int K, int tid) {
+#pragma unroll
+        for (int i = 0; i < NCH; ++i) {
+            const int c = tid + i * NT;
+            const int r = c >> 3, kc = c & 7;
+            const int gr = row0 + r, gk = k0 + kc * 8;
+            u32x4 v = {0u, 0u, 0u, 0u};
+            if (gr < rows && gk < K) v = *(const u32x4*)(base + (int64_t)gr * ld + gk);
+            regs[i] = v;
+        }
+    }
+    __device__ __forceinline__ void sstore(bf16* lds, int tid) const {
+#pragma unroll
+        for (int i = 0; i < NCH; ++i) {
+            const int c = tid + i * NT;
+            const int r = c >> 3, kc = c & 7;
+            *(u32x4*)(lds + r * 64 + ((kc ^ swz(r)) << 3)) = regs[i];
+        }
+    }
+};
+
+template <int R, int NT> struct TileLoader<R, NT, true> {
+    // each thread owns an 8-row x KB-k block: KB 16-byte loads, each 8 rows at one k
+    static constexpr int KB = 8 * R / NT;
+    static_assert(KB == 2 || KB == 4 || KB == 8, "unsupported tile/block combination");
+    static constexpr int NRB = R / 8;
+    u32x4 regs[KB];
+    __device__ __forceinline__ void gload(const bf16* base, int64_t ld, int row0, int rows, int k0,
+                                          int K, int tid) {
+        const int rb = tid % NRB, kb = tid / NRB;
+        const int gr = row0 + rb * 8;
+#pragma unroll
+        for (int j = 0; j < KB; ++j) {
+            const int gk = k0 + kb * KB + j;
+            u32x4 v = {0u, 0u, 0u, 0u};
+            if (gr < rows && gk < K) v = *(const u32x4*)(base + (int64_t)gk * ld + gr);
+            regs[j] = v;
+        }
+    }
+    __device__ __forceinline__ void sstore(bf16* lds, int tid) const {
+        const int rb = tid % NRB, kb = tid / NRB;
+        const int ko = kb * KB;  // k offset inside the 64-wide tile
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            // row i of the block: element i of every loaded vector
+            uint32_t w[KB / 2];
+#pragma unroll
+            for (int j = 0; j < KB / 2; ++j) {
+                const uint32_t lo = regs[2 * j][i >> 1], hi = regs[2 * j + 1][i >> 1];
+                w[j] = (i & 1) ? ((lo >> 16) | (hi & 0xffff0000u)) : ((lo & 0xffffu) | (hi << 16));
+            }
+            const int r = rb * 8 + i;
+            bf16* dst = lds + r * 64 + ((((ko >> 3) ^ swz(r))) << 3) + (ko & 7);
+            if constexpr (KB == 8) {
+                u32x4 t = {w[0], w[1], w[2], w[3]};
+                *(u32x4*)dst = t;
+            } else if constexpr (KB == 4) {
+                u32x2 t = {w[0], w[1]};
+                *(u32x2*)dst = t;
+            } else {
+                *(uint32_t*)dst = w[0];
+            }
+        }
+    }
+};
+
+template <int BM, int BN, int WM, int WN, bool TA, bool TB>
+__global__ __launch_bounds__(WM* WN * 64) void gemm_bf16_kernel(const GemmArgs g) {
+    constexpr int NT = WM * WN * 64, BK = 64;
+    constexpr int WTM = BM / WM, WTN = BN / WN, TM = WTM / 32, TN = WTN / 32;
+    static_assert(TM >= 1 && TN >= 1, "wave tile must hold a 32x32 MFMA tile");
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+    bf16* As = (bf16*)smem;            // [2][BM*BK]
+    bf16* Bs = As + 2 * BM * BK;       // [2][BN*BK]
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wm = wave / WN, wn = wave % WN;
+    int tile_m, tile_n;
+    tile_coords(blockIdx.x, g.tiles_m, g.tiles_n, tile_m, tile_n);
+    const int m0 = tile_m * BM, n0 = tile_n * BN;
+    const int b1 = blockIdx.z / g.nb2, b2 = blockIdx.z % g.nb2;
+    const bf16* A = (const bf16*)g.A + b1 * g.sA1 + b2 * g.sA2;
+    const bf16* B = (const bf16*)g.B + b1 * g.sB1 + b2 * g.sB2;
+    const int64_t coff = b1 * g.sC1 + b2 * g.sC2;
+
+    TileLoader<BM, NT, TA> la;
+    TileLoader<BN, NT, TB> lb;
+
+    f32x16 acc[TM][TN];
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+
+    const int KT = (g.K + BK - 1) / BK;
+    la.gload(A, g.lda, m0, g.M, 0, g.K, tid);
+    lb.gload(B, g.ldb, n0, g.N, 0, g.K, tid);
+    la.sstore(As, tid);
+    lb.sstore(Bs, tid);
+    __syncthreads();
+
+    const int frow = lane & 31, fk = lane >> 5;
+    for (int kt = 0; kt < KT; ++kt) {
+        const int cur = kt & 1;
+        const bool more = kt + 1 < KT;
+        if (more) {
+            la.gload(A, g.lda, m0, g.M, (kt + 1) * BK, g.K, tid);
+            lb.gload(B, g.ldb, n0, g.N, (kt + 1) * BK, g.K, tid);
+        }
+        const bf16* as = As + cur * BM * BK;
+        const bf16* bs = Bs + cur * BN * BK;
+#pragma unroll
+        for (int ks = 0; ks < BK / 16; ++ks) {
+            bf16x8 af[TM], bfr[TN];
+#pragma unroll
+            for (int i = 0; i < TM; ++i) {
+                const int r = wm * WTM + i * 32 + frow;
+                af[i] = *(const bf16x8*)(as + r * 64 + (((ks * 2 + fk) ^ swz(r)) << 3));
+            }
+#pragma unroll
+            for (int j = 0; j < TN; ++j) {
+                const int r = wn * WTN + j * 32 + frow;
+                bfr[j] = *(const bf16x8*)(bs + r * 64 + (((ks * 2 + fk) ^ swz(r)) << 3));
+            }
+#pragma unroll
+            for (int i = 0; i < TM; ++i)
+#pragma unroll
+                for (int j = 0; j < TN; ++j)
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[i], bfr[j], acc[i][j], 0, 0, 0);
+        }
+        if (more) {
+            la.sstore(As + (cur ^ 1) * BM * BK, tid);
+            lb.sstore(Bs + (cur ^ 1) * BN * BK, tid);
+        }
+        __syncthreads();
+    }
+
+    // epilogue: lane holds column (lane & 31); register r is row 8*(r/4) + 4*(lane/32) + r%4
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j) {
+            const int n = n0 + wn * WTN + j * 32 + (lane & 31);
+            if (n >= g.N) continue;
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int m = m0 + wm * WTM + i * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
+                if (m < g.M) epilogue_elem<bf16>(g, coff, coff, m, n, acc[i][j][r]);
+            }
+        }
+}
+
+// =========================================================================================
+// bf16 kernel, DMA generation: tiles go global -> LDS directly (global_load_lds_dwordx4, no
+// VGPR staging) through a 4-stage ring of 32-wide k-tiles, MFMA fragments are double-buffered
+// in registers so LDS reads of tile t+1 overlap the MFMAs of tile t.
+//
+// LDS tile formats (one wave-instruction always fills 1024 contiguous bytes, 16 B per lane):
+//   KC operand (memory rows are k-contiguous): [rows][32 k], 64 B per row = 4 chunks of 16 B,
+//       chunk c of row r at slot c ^ ((r >> 2) & 3); fragments by ds_read_b128.
+//   KM operand (memory is k-major, rows contiguous): [32 k][rows], chunk c of k-row k at slot
+//       c ^ (4 * (k & 3)); fragments by two ds_read_b64_tr_b16 (the hardware transposes a
+//       4k x 16row block across 16 lanes: lane j reads row k0 + j/4, cols 4*(j%4)..+3 and
+//       receives column j, k0..k0+3).
+// Rows beyond M / N are clamped to the last valid row (their results are never stored);
+// K must be a multiple of 32.
+// =========================================================================================
+typedef __attribute__((address_space(3))) void lds_ptr_t;
+typedef const __attribute__((address_space(1))) void gbl_ptr_t;
+typedef __attribute__((ext_vector_type(4))) short s16x4;
+
+// Ask the machine scheduler for "one MFMA, then its share of NMEM memory instructions" NMFMA times:
+// the memory instructions of a region (LDS fragment reads or DMA issues) are spread between the
+// MFMAs instead of being bunched in front of a full wait.
+template <int NMFMA, int NMEM, int MEM_MASK> __device__ __forceinline__ void interleave_mfma_with() {
+    static_for(
+        [&](auto idx) {
+            constexpr int i = decltype(idx)::value;
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+            constexpr int n = (NMEM * (i + 1)) / NMFMA - (NMEM * i) / NMFMA;
+            if constexpr (n > 0) __builtin_amdgcn_sched_group_barrier(MEM_MASK, n, 0);
+        },
+        std::make_integer_sequence<int, NMFMA>{});
+}
+
+template <int N> __device__ __forceinline__ void wait_vmcnt_lgkm0() {
+    // s_waitcnt vmcnt(N) lgkmcnt(0): vmcnt[3:0] | expcnt(7) << 4 | lgkmcnt << 8 | vmcnt[5:4] << 14
+    __builtin_amdgcn_s_waitcnt((N & 15) | (7 << 4) | (0 << 8) | ((N >> 4) << 14));
+}
+
+// One wave-wide 16-byte-per-lane global -> LDS transfer (global_load_lds_dwordx4; the LDS target
+// is M0 + lane * 16).  Issued as inline assembly on purpose: while the compiler sees such a load in
+// flight it turns EVERY wait for an LDS read into lgkmcnt(0), i.e. each fragment wait would drain
+// all outstanding fragment reads.  Unseen, the fragment waits keep their exact counts.  The price:
+// the compiler does not count these loads in vmcnt either - the main loop waits for them explicitly
+// (it always did), and nothing else may touch the target stage or leave the kernel's main loop
+// without an explicit vmcnt wait.
+__device__ __forceinline__ void dma16(const void* src, const unsigned char* lds_dst) {
+    const unsigned m0 = __builtin_amdgcn_readfirstlane((unsigned)(uintptr_t)(lds_ptr_t*)lds_dst);
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(m0), "v"(src) : "m0");
+}
+
+// 3x3 convolution (stride 1, pad 1, NHWC) as an implicit GEMM: the patch matrix [pixels, 9 * channels] is never
+// built, the A loader gathers its rows from the activation tensor instead.
+struct ConvArgs {
+    int h, w, c;      // image height / width, channels of the gathered tensor (a multiple of the 64-wide k-tile)
+    int b_every;      // input-gradient mode: k-tiles per tap of the B operand ...
+    int64_t b_wrap;   // ... and what its pointers move by (on top of the k-tile step) when the tap changes
+};
+// what the taps outside the image read
+__device__ __attribute__((aligned(128))) unsigned char bb_zero_line[128];
+
+// VIS: issue through the compiler builtin instead (the compiler then sees the load and waits lgkmcnt(0)
+// for every fragment read, which keeps the waves of a block in lock step)
+// CONV 1 (row-contiguous operand, 64-wide k-tiles): row p of the operand is pixel p's 3x3 neighbourhood,
+// k = tap * channels + channel; a k-tile lies inside one tap, so each lane reads 16 bytes of the neighbouring
+// pixel's channel vector, or of a line of zeros where the tap falls outside the image.
+// CONV 2 (k-major operand): the weight [out, 9, in] read as B[k = (8 - tap) * out + o, n = i] (the flipped
+// filter of the input gradient): rows o advance by the k-tile, and every out / 64 k-tiles the tap changes.
+template <int BR, bool KM, int NW, int BK = 32, bool VIS = false, int CONV = 0> struct DmaOperand {
+    static constexpr int BYTES = BR * BK * 2;
+    static constexpr int ROUNDS = BYTES / (1024 * NW);  // instructions per thread per k-tile
+    static_assert(ROUNDS >= 1, "tile too small for the block");
+    static_assert(CONV == 0 || (CONV == 1 && !KM && BK == 64) || ((CONV == 2 || CONV == 3) && KM), "convolution loaders: see above");
+    const bf16* src[ROUNDS];
+    int64_t step;  // elements to advance per k-tile
+    // CONV 1: per round the taps that lie inside the image (bit t = tap t), then wave-uniform position in K
+    unsigned inside[ROUNDS];
+    const bf16* zero;
+    int tap, c0, kstep, cw, cc;
+    int64_t tapoff;
+    // CONV 2
+    int cnt, every;
+    int64_t wrap;
+    // CONV 3: image coordinates of the pixel each round reads next, the block's tap, the k-tile step in pixels
+    int py[ROUNDS], px[ROUNDS];
+    int tdy, tdx, dpy, dpx, ch;
+
+    __device__ __forceinline__ void init(const bf16* base, int64_t ld, int row0, int rows, int tid) {
+        const int lane = tid & 63, wave = tid >> 6;
+#pragma unroll
+        for (int i = 0; i < ROUNDS; ++i) {
+            const int q = i * NW + wave;
+            if constexpr (!KM && BK == 64) {
+                // 64-wide k-tiles: one instruction takes 8 rows x 128 B, whole cache lines
+                const int r = q * 8 + (lane >> 3);
+                const int c = (lane & 7) ^ ((r >> 1) & 7);
+                const int gr = min(row0 + r, rows - 1);
+                src[i] = base + (int64_t)gr * ld + c * 8;
+            } else if constexpr (!KM) {
+                const int r = q * 16 + (lane >> 2);
+                const int c = (lane & 3) ^ ((r >> 2) & 3);
+                const int gr = min(row0 + r, rows - 1);
+                src[i] = base + (int64_t)gr * ld + c * 8;
+            } else {
+                constexpr int CPR = BR / 8, RPI = 64 / CPR;
+                const int k = q * RPI + lane / CPR;
+                const int c = (lane % CPR) ^ (4 * (k & 3));
+                const int gc = min(row0 + c * 8, rows - 8);
+                src[i] = base + (int64_t)k * ld + gc;
+            }
+        }
+        step = KM ? BK * ld : BK;
+    }
+    // CONV 1: base = the activation tensor [pixels, cv.c]; src[i] points at the lane's chunk of the centre pixel
+    __device__ __forceinline__ void init_conv(const bf16* base, int row0, int rows, int tid, const ConvArgs& cv) {
+        const int lane = tid & 63, wave = tid >> 6;
+#pragma unroll
+        for (int i = 0; i < ROUNDS; ++i) {
+            const int q = i * NW + wave;
+            const int r = q * 8 + (lane >> 3);
+            const int c = (lane & 7) ^ ((r >> 1) & 7);
+            const int gr = min(row0 + r, rows - 1);
+            const int pix = gr % (cv.h * cv.w), py = pix / cv.w, px = pix % cv.w;
+            unsigned m = 0;
+#pragma unroll
+            for (int t = 0; t < 9; ++t) {
+                const int sy = py + t / 3 - 1, sx = px + t % 3 - 1;
+                if (sy >= 0 && sy < cv.h && sx >= 0 && sx < cv.w) m |= 1u << t;
+            }
+            inside[i] = m;
+            src[i] = base + (int64_t)gr * cv.c + c * 8;
+        }
+        zero = (const bf16*)(bb_zero_line + (lane & 7) * 16);
+        step = 0;
+        tap = 0; c0 = 0; kstep = BK; cw = cv.w; cc = cv.c;
+        tapoff = (int64_t)(-cv.w - 1) * cv.c;
+    }
+    // CONV 2: after init() with base already at tap 8 of the weight
+    __device__ __forceinline__ void init_wrap(const ConvArgs& cv) {
+        cnt = 0; every = cv.b_every; wrap = cv.b_wrap;
+    }
+    // CONV 3 (k-major operand): the patch matrix [pixels, 9 * c] of the tensor at base as the B operand of a
+    // weight gradient.  A column tile (col0 .. col0 + BR - 1, inside one tap since c % BR == 0) reads channels
+    // of the pixel `tap` away from pixel k: rows advance by the k-tile, the lane's image coordinates with them.
+    __device__ __forceinline__ void init_conv_km(const bf16* base, int col0, int tid, int h, int w, int c, int pix0) {
+        const int lane = tid & 63, wave = tid >> 6;
+        const int t = col0 / c, ci0 = col0 - t * c;
+        tdy = t / 3 - 1; tdx = t % 3 - 1; ch = h; cw = w;
+        dpy = BK / w; dpx = BK % w;
+#pragma unroll
+        for (int i = 0; i < ROUNDS; ++i) {
+            const int q = i * NW + wave;
+            constexpr int CPR = BR / 8, RPI = 64 / CPR;
+            const int k = q * RPI + lane / CPR;
+            const int cch = (lane % CPR) ^ (4 * (k & 3));
+            const int p = pix0 + k, pix = p % (h * w);
+            py[i] = pix / w;
+            px[i] = pix - py[i] * w;
+            src[i] = base + ((int64_t)p + tdy * w + tdx) * c + ci0 + cch * 8;
+        }
+        zero = (const bf16*)(bb_zero_line + (lane & 7) * 16);
+        step = (int64_t)BK * c;
+    }
+    // past the end of K: the last tile is fetched again and again
+    __device__ __forceinline__ void stop() {
+        step = 0;
+        if constexpr (CONV == 1) kstep = 0;
+        if constexpr (CONV == 2) wrap = 0;
+        if constexpr (CONV == 3) dpy = dpx = 0;
+    }
+    __device__ __forceinline__ const bf16* source(int i) const {
+        if constexpr (CONV == 1) return ((inside[i] >> tap) & 1u) ? src[i] + (tapoff + c0) : zero;
+        else if constexpr (CONV == 3)
+            return ((unsigned)(py[i] + tdy) < (unsigned)ch && (unsigned)(px[i] + tdx) < (unsigned)cw) ? src[i] : zero;
+        else return src[i];
+    }
+    // CONV 3: round i moves on by one k-tile of pixels (BK / w + 1 <= h: at most one image boundary per step)
+    __device__ __forceinline__ void next_pixels(int i) {
+        if constexpr (CONV == 3) {
+            px[i] += dpx;
+            py[i] += dpy;
+            if (px[i] >= cw) {
+                px[i] -= cw;
+                ++py[i];
+            }
+            if (py[i] >= ch) py[i] -= ch;
+        }
+    }
+    // after the last instruction of a k-tile
+    __device__ __forceinline__ void advance() {
+        if constexpr (CONV == 1) {
+            c0 += kstep;
+            if (c0 >= cc) {
+                c0 = 0;
+                ++tap;
+                tapoff = (int64_t)((tap / 3 - 1) * cw + (tap % 3 - 1)) * cc;
+            }
+        } else if constexpr (CONV == 2) {
+            if (++cnt == every) {
+                cnt = 0;
+#pragma unroll
+                for (int i = 0; i < ROUNDS; ++i) src[i] += wrap;
+            }
+        }
+    }
+    __device__ __forceinline__ void issue(unsigned char* tile, int wave) {
+#pragma unroll
+        for (int i = 0; i < ROUNDS; ++i) {
+            if constexpr (VIS) __builtin_amdgcn_global_load_lds((gbl_ptr_t*)source(i), (lds_ptr_t*)(tile + (i * NW + wave) * 1024), 16, 0, 0);
+            else dma16(source(i), tile + (i * NW + wave) * 1024);
+            src[i] += step;
+            next_pixels(i);
+        }
+        advance();
+    }
+    template <int I> __device__ __forceinline__ void issue_one(unsigned char* tile, int wave) {
+        dma16(source(I), tile + (I * NW + wave) * 1024);
+        src[I] += step;
+        next_pixels(I);
+        if constexpr (I == ROUNDS - 1) advance();
+    }
+};
+
+// per-lane fragment offsets (bytes inside an operand tile) and the fragment fetch
+template <int BR, int T, bool KM, int BK = 32> struct FragReader {
+    int off[KM ? T : 1];
+    int sw, hi;
+    __device__ __forceinline__ void init(int wbase, int lane) {
+        hi = lane >> 5;
+        if constexpr (!KM) {
+            sw = BK == 64 ? ((lane & 31) >> 1) & 7 : ((lane & 31) >> 2) & 3;
+            off[0] = (wbase + (lane & 31)) * (BK * 2);
+        } else {
+            const int j4 = (lane & 15) >> 2;
+            const int lo = ((lane >> 4) & 1) * 2 + ((lane & 3) >> 1);
+            const int within = (lane & 1) * 4;  // element offset inside the 16-byte chunk
+            sw = 0;
+#pragma unroll
+            for (int t = 0; t < T; ++t) {
+                const int c4 = ((wbase >> 5) + t) ^ j4;  // chunk-of-four index after the swizzle
+                off[t] = (hi * 8 + j4) * (BR * 2) + ((c4 * 4 + lo) << 4) + within * 2;
+            }
+        }
+    }
+    __device__ __forceinline__ bf16x8 load(const unsigned char* tile, int t, int ks) const {
+        if constexpr (!KM) {
+            return *(const bf16x8*)(tile + off[0] + t * (32 * BK * 2) + (((ks * 2 + hi) ^ sw) << 4));
+        } else {
+            const unsigned char* p = tile + off[t] + ks * 16 * (BR * 2);
+            s16x4 lo4 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4*)(p));
+            s16x4 hi4 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4*)(p + 4 * (BR * 2)));
+            typedef __attribute__((ext_vector_type(8))) short s16x8;
+            s16x8 v = __builtin_shufflevector(lo4, hi4, 0, 1, 2, 3, 4, 5, 6, 7);
+            return __builtin_bit_cast(bf16x8, v);
+        }
+    }
+};
+
+// STATS: the epilogue also leaves the column statistics of the stored (bf16-rounded) output per 32-row strip, for the
+// batch normalisation that follows a convolution (its statistics pass then has nothing left to read).
+template <int BM, int BN, int WM, int WN, bool AKM, bool BKM, bool DB, int STAGES, int BK = 32, bool VIS = false, int CONV = 0,
+          bool STATS = false>
+__device__ __forceinline__ void gemm_bf16_dma_body(const GemmArgs& g, const int block_id, const int batch_id,
+                                                   const bool logical_id = false, const ConvArgs& cv = ConvArgs{}) {
+    constexpr int NW = WM * WN;
+    static_assert(BK == 64 ? (STAGES >= 2 && DB) : STAGES >= 3,
+                  "32-wide k-tiles: the ring needs one stage being read, one landing, one in flight; "
+                  "64-wide k-tiles alternate between two stages or rotate through more");
+    constexpr int WTM = BM / WM, WTN = BN / WN, TM = WTM / 32, TN = WTN / 32;
+    // CONV 1: forward 3x3 convolution (A gathered); CONV 2: its input gradient (A gathered, B the flipped filter)
+    // CONV 3: its weight gradient (B = the patch matrix, gathered)
+    static_assert(CONV == 0 || (CONV == 3 ? AKM && BKM : !AKM && (CONV == 2) == BKM),
+                  "implicit convolution: NT forward, NN input gradient, TN weight gradient");
+    using OpA = DmaOperand<BM, AKM, NW, BK, VIS, CONV == 1 || CONV == 2 ? 1 : 0>;
+    using OpB = DmaOperand<BN, BKM, NW, BK, VIS, CONV >= 2 ? CONV : 0>;
+    constexpr int STAGE_BYTES = OpA::BYTES + OpB::BYTES;
+    constexpr int LOADS = OpA::ROUNDS + OpB::ROUNDS;
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wm = wave / WN, wn = wave % WN;
+    int tile_m, tile_n;
+    if (logical_id) panel_coords(block_id, g.tiles_m, g.tiles_n, tile_m, tile_n);
+    else tile_coords(block_id, g.tiles_m, g.tiles_n, tile_m, tile_n);
+    const int m0 = tile_m * BM, n0 = tile_n * BN;
+    const int b1 = batch_id / g.nb2, b2 = batch_id % g.nb2;
+    const bf16* A = (const bf16*)g.A + b1 * g.sA1 + b2 * g.sA2;
+    const bf16* B = (const bf16*)g.B + b1 * g.sB1 + b2 * g.sB2;
+    const int64_t coff = b1 * g.sC1 + b2 * g.sC2;
+
+    OpA opa;
+    OpB opb;
+    if constexpr (CONV == 1 || CONV == 2) opa.init_conv(A, m0, g.M, tid, cv);
+    else opa.init(A, g.lda, m0, g.M, tid);
+    if constexpr (CONV == 3) opb.init_conv_km(B, n0, tid, g.conv_h, g.conv_w, g.conv_c, g.conv_row0);
+    else opb.init(B, g.ldb, n0, g.N, tid);
+    if constexpr (CONV == 2) opb.init_wrap(cv);
+    FragReader<BM, TM, AKM, BK> fa;
+    FragReader<BN, TN, BKM, BK> fb;
+    fa.init(wm * WTM, lane);
+    fb.init(wn * WTN, lane);
+
+    f32x16 acc[TM][TN];
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+
+    struct Frags {
+        bf16x8 a[2][TM], b[2][TN];
+    };
+    Frags f0, f1;
+    const int KT = g.K / BK;
+
+    // ring positions: tile t lives in stage t % STAGES
+    int issue_stage = 0, read_stage = 0;
+    auto issue_tile = [&]() {
+        unsigned char* st = smem + issue_stage * STAGE_BYTES;
+        opa.issue(st, wave);
+        opb.issue(st + OpA::BYTES, wave);
+        issue_stage = issue_stage + 1 == STAGES ? 0 : issue_stage + 1;
+    };
+    auto load_frags = [&](Frags& f) {
+        const unsigned char* st = smem + read_stage * STAGE_BYTES;
+#pragma unroll
+        for (int ks = 0; ks < 2; ++ks) {
+#pragma unroll
+            for (int i = 0; i < TM; ++i) f.a[ks][i] = fa.load(st, i, ks);
+#pragma unroll
+            for (int j = 0; j < TN; ++j) f.b[ks][j] = fb.load(st + OpA::BYTES, j, ks);
+        }
+        read_stage = read_stage + 1 == STAGES ? 0 : read_stage + 1;
+    };
+    // bias gradient riding along: the waves of the first block column (and first wave column)
+    // add up the A fragments they hold anyway: lane (m, kg) sees 8 of the 16 k values per step
+    const bool do_colsum = AKM && g.colsum != nullptr && tile_n == 0 && wn == 0;
+    float csum[TM];
+#pragma unroll
+    for (int i = 0; i < TM; ++i) csum[i] = 0.f;
+    auto mfma_step = [&](const Frags& f, int ks) {
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+            for (int j = 0; j < TN; ++j)
+                acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(f.a[ks][i], f.b[ks][j], acc[i][j], 0, 0, 0);
+        if constexpr (AKM) {
+            if (do_colsum) {
+#pragma unroll
+                for (int i = 0; i < TM; ++i) {
+                    float t = 0.f;
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) t += (float)f.a[ks][i][e];
+                    csum[i] += t;
+                }
+            }
+        }
+    };
+    // One quarter / half of a tile placed by hand: MFMA m of step ks, then its share of ND DMA
+    // instructions into stage `dst` and of the fragment reads of (stage `src`, half h) into `nf` (the
+    // reads ride on the first FM MFMAs so that the last ones cover their latency), each group fenced:
+    // the DMA instructions are inline assembly, opaque to the scheduler's group hints, and unfenced
+    // they end up bunched behind the barrier.
+    auto placed_step = [&](const Frags& f, auto ks_c, auto nd_c, unsigned char* dst, auto reads_c, Frags& nf,
+                           const unsigned char* src, int h) {
+        constexpr int ks = decltype(ks_c)::value, ND = decltype(nd_c)::value;
+        constexpr bool READS = decltype(reads_c)::value;
+        constexpr int NM = TM * TN, NF = 2 * (TM + TN), FM = NM > 2 ? NM - 2 : NM;
+        static_for(
+            [&](auto idx) {
+                constexpr int m = decltype(idx)::value, i = m / TN, j = m % TN;
+                acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(f.a[ks][i], f.b[ks][j], acc[i][j], 0, 0, 0);
+                if constexpr (AKM && j == 0) {
+                    if (do_colsum) {
+                        float t = 0.f;
+#pragma unroll
+                        for (int e = 0; e < 8; ++e) t += (float)f.a[ks][i][e];
+                        csum[i] += t;
+                    }
+                }
+                static_for(
+                    [&](auto d) {
+                        constexpr int k = (ND * m) / NM + decltype(d)::value;
+                        if constexpr (k < OpA::ROUNDS) opa.template issue_one<k>(dst, wave);
+                        else opb.template issue_one<k - OpA::ROUNDS>(dst + OpA::BYTES, wave);
+                    },
+                    std::make_integer_sequence<int, (ND * (m + 1)) / NM - (ND * m) / NM>{});
+                if constexpr (READS && m < FM) {
+                    static_for(
+                        [&](auto r) {
+                            constexpr int q = (NF * m) / FM + decltype(r)::value, fk = q / (TM + TN), t = q % (TM + TN);
+                            if constexpr (t < TM) nf.a[fk][t] = fa.load(src, t, h * 2 + fk);
+                            else nf.b[fk][t - TM] = fb.load(src + OpA::BYTES, t - TM, h * 2 + fk);
+                        },
+                        std::make_integer_sequence<int, (NF * (m + 1)) / FM - (NF * m) / FM>{});
+                }
+                __builtin_amdgcn_sched_barrier(0);
+            },
+            std::make_integer_sequence<int, NM>{});
+    };
+    // Steady state is branch-free: a tile is issued every iteration (past the end of K the
+    // sources stop advancing, so the last tile is fetched again into a stage nobody reads),
+    // hence exactly STAGES-2 newer tiles are in flight whenever a wave waits for the next tile.
+    auto sync_tile = [&]() {
+        asm volatile("" ::: "memory");
+        wait_vmcnt_lgkm0<(STAGES - 2) * LOADS>();
+        __builtin_amdgcn_s_barrier();
+        asm volatile("" ::: "memory");
+    };
+    auto stop_at_end = [&](int next_tile) {
+        if (next_tile >= KT) {
+            opa.stop();
+            opb.stop();
+        }
+    };
+
+    if constexpr (BK == 64) {
+        // Two stages of 64-wide k-tiles, each multiplied as two 32-wide halves from the two fragment
+        // sets.  Per tile one barrier, in the middle of its second half: by then every wave has read
+        // the tile's last fragments (so its stage can take tile kt+2) and tile kt+1, issued one whole
+        // tile earlier, has to have landed (its first fragments are read right after).
+        auto load_half = [&](Frags& f, const unsigned char* st, int h) {
+#pragma unroll
+            for (int ks = 0; ks < 2; ++ks) {
+#pragma unroll
+                for (int i = 0; i < TM; ++i) f.a[ks][i] = fa.load(st, i, h * 2 + ks);
+#pragma unroll
+                for (int j = 0; j < TN; ++j) f.b[ks][j] = fb.load(st + OpA::BYTES, j, h * 2 + ks);
+            }
+        };
+        constexpr int FRAG_READS = 2 * (TM * (AKM ? 2 : 1) + TN * (BKM ? 2 : 1));
+        // prologue: tiles 0 and 1 with two stages, 0..STAGES-2 with more (tile kt+STAGES-1 then goes out
+        // at the top of iteration kt, into the stage tile kt-1 has left)
+        constexpr int PRO = STAGES == 2 ? 2 : STAGES - 1;
+#pragma unroll
+        for (int t = 0; t < PRO; ++t) {
+            stop_at_end(t + 1);
+            issue_tile();
+        }
+        asm volatile("" ::: "memory");
+        wait_vmcnt_lgkm0<(PRO - 1) * LOADS>();
+        __builtin_amdgcn_s_barrier();
+        asm volatile("" ::: "memory");
+        load_half(f0, smem, 0);
+        int rs = 0;
+        for (int kt = 0; kt < KT; ++kt) {
+            const unsigned char* cur = smem + rs * STAGE_BYTES;
+            rs = rs + 1 == STAGES ? 0 : rs + 1;
+            const unsigned char* nxt = smem + rs * STAGE_BYTES;
+            if constexpr (STAGES >= 3) {
+                stop_at_end(kt + STAGES);
+                issue_tile();
+            }
+            load_half(f1, cur, 1);
+            mfma_step(f0, 0);
+            mfma_step(f0, 1);
+            interleave_mfma_with<2 * TM * TN, FRAG_READS, 0x100>();
+            mfma_step(f1, 0);
+            // scheduling fences: without them the compiler sinks this third quarter below the barrier
+            // and bunches the next tile's fragment reads at the end of the iteration, right in front
+            // of the wait for them
+            __builtin_amdgcn_sched_barrier(0);
+            asm volatile("" ::: "memory");
+            wait_vmcnt_lgkm0<(STAGES - 2) * LOADS>();
+            __builtin_amdgcn_s_barrier();
+            asm volatile("" ::: "memory");
+            // last quarter: the DMA instructions of tile kt+2 (two stages: into the stage of tile kt)
+            // and the first fragment reads of tile kt+1 between its MFMAs
+            unsigned char* dst = smem + issue_stage * STAGE_BYTES;
+            if constexpr (STAGES == 2) {
+                stop_at_end(kt + 3);
+                issue_stage = issue_stage + 1 == STAGES ? 0 : issue_stage + 1;
+            }
+            placed_step(f1, std::integral_constant<int, 1>{}, std::integral_constant<int, STAGES == 2 ? LOADS : 0>{}, dst,
+                        std::true_type{}, f0, nxt, 0);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    } else {
+    // prologue: tiles 0..STAGES-2 (clamped to the last tile when K is short)
+#pragma unroll
+    for (int t = 0; t < STAGES - 1; ++t) {
+        stop_at_end(t + 1);
+        issue_tile();
+    }
+    sync_tile();
+    if constexpr (DB) {
+        // fragments of tile kt+1 are fetched while the second half of tile kt is multiplied,
+        // into the other register set
+        // Hand placement pays on the 256x256 tile (eight MFMAs per half to place things between: +1..5 %);
+        // on the smaller tiles and with two k-major operands (twice the fragment read instructions) the
+        // scheduler's own order is as good or better.
+        constexpr bool PLACED = BM == 256 && BN == 256 && !AKM;
+        auto body = [&](int kt, Frags& cur, Frags& nxt) {
+          if constexpr (PLACED) {
+            // first half: the DMA instructions of tile kt+STAGES-1 between its MFMAs; second half, behind
+            // the barrier: the fragment reads of tile kt+1
+            stop_at_end(kt + STAGES);
+            unsigned char* dst = smem + issue_stage * STAGE_BYTES;
+            issue_stage = issue_stage + 1 == STAGES ? 0 : issue_stage + 1;
+            placed_step(cur, std::integral_constant<int, 0>{}, std::integral_constant<int, LOADS>{}, dst, std::false_type{},
+                        nxt, smem, 0);
+            sync_tile();
+            const unsigned char* st = smem + read_stage * STAGE_BYTES;
+            read_stage = read_stage + 1 == STAGES ? 0 : read_stage + 1;
+            placed_step(cur, std::integral_constant<int, 1>{}, std::integral_constant<int, 0>{}, dst, std::true_type{}, nxt,
+                        st, 0);
+          } else {
+            constexpr int FRAG_READS = 2 * (TM * (AKM ? 2 : 1) + TN * (BKM ? 2 : 1));
+            stop_at_end(kt + STAGES);
+            issue_tile();
+            mfma_step(cur, 0);
+            interleave_mfma_with<TM * TN, LOADS, 0x020>();   // DMA issues between the first-half MFMAs
+            sync_tile();
+            load_frags(nxt);
+            mfma_step(cur, 1);
+            interleave_mfma_with<TM * TN, FRAG_READS, 0x100>();  // next tile's fragment reads between the rest
+          }
+        };
+        load_frags(f0);
+        int kt = 0;
+        for (; kt + 1 < KT; kt += 2) {
+            body(kt, f0, f1);
+            body(kt + 1, f1, f0);
+        }
+        if (kt < KT) body(kt, f0, f1);
+    } else {
+        // single fragment set: other resident waves cover LDS latency and barrier waits
+        for (int kt = 0; kt < KT; ++kt) {
+            stop_at_end(kt + STAGES);
+            issue_tile();
+            load_frags(f0);
+            mfma_step(f0, 0);
+            mfma_step(f0, 1);
+            sync_tile();
+        }
+    }
+    }
+
+    if constexpr (AKM) {
+        if (do_colsum) {
+#pragma unroll
+            for (int i = 0; i < TM; ++i) {
+                const float t = csum[i] + __shfl_xor(csum[i], 32, 64);
+                const int m = m0 + wm * WTM + i * 32 + (lane & 31);
+                if (lane < 32 && m < g.M) g.colsum[m] += t;
+            }
+        }
+    }
+
+    // Epilogue through LDS: every wave parks two horizontally adjacent 32x32 accumulator tiles in a
+    // private [32][64 (+4 pad)] fp32 patch; then one wave instruction covers 8 rows x 64 columns, lane l
+    // taking 8 consecutive columns of row l/8, so every global load / store of the epilogue moves whole
+    // 128-byte row segments (256 bytes for fp32 outputs).
+    // An odd tile count per row ends with a single tile: its 32 columns use half of the patch and half of
+    // the lanes of the row pass.
+    wait_vmcnt_lgkm0<0>();  // the tiles issued past the end of K have to land before their stages become the patch
+    __syncthreads();
+    constexpr int PLD = 68;
+    constexpr int NP = (TN + 1) / 2;   // pairs per row of accumulator tiles, the last one possibly a single
+    float* patch = (float*)smem + wave * (32 * PLD);
+    const int prow = lane >> 3, pcol = (lane & 7) * 8;
+    static_for(
+        [&](auto idx) {
+            constexpr int i = decltype(idx)::value / NP, jp = decltype(idx)::value % NP;
+            constexpr int NH = (jp * 2 + 1 < TN) ? 2 : 1;
+#pragma unroll
+            for (int h = 0; h < NH; ++h)
+#pragma unroll
+                for (int r = 0; r < 16; ++r)
+                    patch[(8 * (r >> 2) + 4 * (lane >> 5) + (r & 3)) * PLD + h * 32 + (lane & 31)] = acc[i][jp * 2 + h][r] * g.alpha;
+            asm volatile("" ::: "memory");
+            const int n = n0 + wn * WTN + jp * 64 + pcol;
+            const bool live = NH == 2 || pcol < 32;
+#pragma unroll
+            for (int it = 0; it < 4; ++it) {
+                const int m = m0 + wm * WTM + i * 32 + it * 8 + prow;
+                float v[8];
+                const f32x4 lo = *(const f32x4*)(patch + (it * 8 + prow) * PLD + pcol);
+                const f32x4 hi = *(const f32x4*)(patch + (it * 8 + prow) * PLD + pcol + 4);
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    v[e] = lo[e];
+                    v[4 + e] = hi[e];
+                }
+                if (live && m < g.M && n < g.N) epilogue_vec8(g, coff, m, n, v);
+            }
+            if constexpr (STATS) {
+                // Column statistics of this 32-row strip straight from the patch: lane = column, 32 conflict-free LDS
+                // reads.  The patch holds what is stored (alpha = 1, no bias, no epilogue), rounded here as the
+                // store rounds it; the pivot is the strip's first row.
+                const int strip_row = m0 + wm * WTM + i * 32, nrows = min(32, g.M - strip_row);
+                const int nc = n0 + wn * WTN + jp * 64 + lane;
+                const float piv = bf2f(f2bf(patch[lane]));
+                float s1 = 0.f, s2 = 0.f;
+#pragma unroll
+                for (int r = 0; r < 32; ++r) {
+                    const float dv = bf2f(f2bf(patch[r * PLD + lane])) - piv;
+                    if (r < nrows) {
+                        s1 += dv;
+                        s2 += dv * dv;
+                    }
+                }
+                if (g.strip_stats && nrows > 0 && nc < g.N && (NH == 2 || lane < 32)) {
+                    float* o = g.strip_stats + ((int64_t)(strip_row >> 5) * 3) * g.N + nc;
+                    o[0] = piv;
+                    o[g.N] = s1;
+                    o[2 * (int64_t)g.N] = s2;
+                }
+            }
+            asm volatile("" ::: "memory");
+        },
+        std::make_integer_sequence<int, TM * NP>{});
+}
+
+template <int BM, int BN, int WM, int WN, bool AKM, bool BKM, bool DB, int STAGES, int BK>
+__global__ __launch_bounds__(WM* WN * 64) void gemm_bf16_dma_kernel(const GemmArgs g) {
+    gemm_bf16_dma_body<BM, BN, WM, WN, AKM, BKM, DB, STAGES, BK>(g, blockIdx.x, blockIdx.z);
+}
+// the same with the strip statistics of the output (NT, 64-wide k-tiles, three stages)
+template <int BM, int BN, int WM, int WN>
+__global__ __launch_bounds__(WM* WN * 64) void gemm_bf16_dma_stats_kernel(const GemmArgs g) {
+    gemm_bf16_dma_body<BM, BN, WM, WN, false, false, true, 3, 64, false, 0, true>(g, blockIdx.x, blockIdx.z);
+}
+
+// 3x3 convolution as an implicit GEMM: forward (BKM = false: y = patches(x) W^T) and input gradient
+// (BKM = true: dx = patches(dy) W_flipped) on the same main loop, operands gathered by the loaders.
+template <int BM, int BN, int WM, int WN, bool BKM, int STAGES, bool STATS = false>
+__global__ __launch_bounds__(WM* WN * 64) void conv3x3_bf16_igemm_kernel(const GemmArgs g, const ConvArgs cv) {
+    gemm_bf16_dma_body<BM, BN, WM, WN, false, BKM, true, STAGES, 64, false, BKM ? 2 : 1, STATS>(g, blockIdx.x, 0, false, cv);
+}
+
+// Several independent problems of one kind in a single launch (the four weight-gradient GEMMs
+// of a transformer layer: each alone has too few output tiles to fill 256 CUs).
+constexpr int GROUP_MAX = 16;
+struct GroupedArgs {
+    GemmArgs p[GROUP_MAX];
+    int first_block[GROUP_MAX + 1];
+    int count;
+};
+// CONVB: some problems of the group read their B operand as the patch matrix of a 3x3 convolution
+template <int BM, int BN, int WM, int WN, bool AKM, bool BKM, bool DB, int STAGES, bool CONVB = false>
+__global__ __launch_bounds__(WM* WN * 64) void gemm_bf16_dma_grouped_kernel(const GroupedArgs G) {
+    // The tiles of all problems form one list; an XCD takes a contiguous stretch of it, so its
+    // resident blocks are a few wide rectangles of one or two problems (few distinct operand
+    // panels in its L2) rather than a narrow slice of every problem.
+    const int lid = xcd_contiguous(blockIdx.x, G.first_block[G.count]);
+    int pi = 0;
+    while (pi + 1 < G.count && lid >= G.first_block[pi + 1]) ++pi;
+    // compiler-visible DMA here: the lock step it forces on the waves keeps the three resident blocks of a CU
+    // on the same operand panels (459 instead of 720 MiB read per launch at the same kernel speed; the stage
+    // gains half a percent with the second stream running)
+    if constexpr (CONVB) {
+        if (G.p[pi].conv_c > 0) {
+            gemm_bf16_dma_body<BM, BN, WM, WN, AKM, BKM, DB, STAGES, 32, true, 3>(G.p[pi], lid - G.first_block[pi], 0, true);
+            return;
+        }
+    }
+    gemm_bf16_dma_body<BM, BN, WM, WN, AKM, BKM, DB, STAGES, 32, true>(G.p[pi], lid - G.first_block[pi], 0, true);
+}
+
+// =========================================================================================
+// fp32 kernel: 128x128x16 tiles, 4 waves (2x2), LDS k-major with padded rows.
+// =========================================================================================
+template <bool TA, bool TB>
+__global__ __launch_bounds__(256) void gemm_f32_kernel(const GemmArgs g) {
+    constexpr int BM = 128, BN = 128, BK = 16, LDS_LD = 132, NT = 256;
+    __shared__ __attribute__((aligned(16))) float As[2][BK * LDS_LD];
+    __shared__ __attribute__((aligned(16))) float Bs[2][BK * LDS_LD];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wm = wave >> 1, wn = wave & 1;
+    int tile_m, tile_n;
+    tile_coords(blockIdx.x, g.tiles_m, g.tiles_n, tile_m, tile_n);
+    const int m0 = tile_m * BM, n0 = tile_n * BN;
+    const int b1 = blockIdx.z / g.nb2, b2 = blockIdx.z % g.nb2;
+    const float* A = (const float*)g.A + b1 * g.sA1 + b2 * g.sA2;
+    const float* B = (const float*)g.B + b1 * g.sB1 + b2 * g.sB2;
+    const int64_t coff = b1 * g.sC1 + b2 * g.sC2;
+
+    f32x4 ra[2], rb[2];
+    auto gload = [&](const float* base, int64_t ld, int row0, int rows, int k0, bool tr, f32x4 (&r)[2]) {
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+            const int c = tid + i * NT;
+            f32x4 v = {0.f, 0.f, 0.f, 0.f};
+            if (!tr) {
+                const int row = c >> 2, kq = c & 3;
+                if (row0 + row < rows && k0 + kq * 4 < g.K)
+                    v = *(const f32x4*)(base + (int64_t)(row0 + row) * ld + k0 + kq * 4);
+            } else {
+                const int k = c >> 5, rq = c & 31;
+                if (row0 + rq * 4 < rows && k0 + k < g.K)
+                    v = *(const f32x4*)(base + (int64_t)(k0 + k) * ld + row0 + rq * 4);
+            }
+            r[i] = v;
+        }
+    };
+    auto sstore = [&](float* lds, bool tr, const f32x4 (&r)[2]) {
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+            const int c = tid + i * NT;
+            if (!tr) {
+                const int row = c >> 2, kq = c & 3;
+#pragma unroll
+                for (int e = 0; e < 4; ++e) lds[(kq * 4 + e) * LDS_LD + row] = r[i][e];
+            } else {
+                const int k = c >> 5, rq = c & 31;
+                *(f32x4*)(lds + k * LDS_LD + rq * 4) = r[i];
+            }
+        }
+    };
+
+    f32x16 acc[2][2];
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+
+    const int KT = (g.K + BK - 1) / BK;
+    gload(A, g.lda, m0, g.M, 0, TA, ra);
+    gload(B, g.ldb, n0, g.N, 0, TB, rb);
+    sstore(As[0], TA, ra);
+    sstore(Bs[0], TB, rb);
+    __syncthreads();
+    for (int kt = 0; kt < KT; ++kt) {
+        const int cur = kt & 1;
+        const bool more = kt + 1 < KT;
+        if (more) {
+            gload(A, g.lda, m0, g.M, (kt + 1) * BK, TA, ra);
+            gload(B, g.ldb, n0, g.N, (kt + 1) * BK, TB, rb);
+        }
+#pragma unroll
+        for (int ks = 0; ks < BK / 2; ++ks) {
+            float af[2], bfr[2];
+            const int kk = ks * 2 + (lane >> 5);
+#pragma unroll
+            for (int i = 0; i < 2; ++i) af[i] = As[cur][kk * LDS_LD + wm * 64 + i * 32 + (lane & 31)];
+#pragma unroll
+            for (int j = 0; j < 2; ++j) bfr[j] = Bs[cur][kk * LDS_LD + wn * 64 + j * 32 + (lane & 31)];
+#pragma unroll
+            for (int i = 0; i < 2; ++i)
+#pragma unroll
+                for (int j = 0; j < 2; ++j)
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(af[i], bfr[j], acc[i][j], 0, 0, 0);
+        }
+        if (more) {
+            sstore(As[cur ^ 1], TA, ra);
+            sstore(Bs[cur ^ 1], TB, rb);
+        }
+        __syncthreads();
+    }
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+            const int n = n0 + wn * 64 + j * 32 + (lane & 31);
+            if (n >= g.N) continue;
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int m = m0 + wm * 64 + i * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
+                if (m < g.M) epilogue_elem<float>(g, coff, coff, m, n, acc[i][j][r]);
+            }
+        }
+}
+
