@@ -1,0 +1,92 @@
+"""Taking over the layers of the reference's model scripts.
+
+The reference's ``PipelineModule`` accepts ``nn.Module`` instances, ``LayerSpec`` of module classes and bare
+callables in its layer list (deepspeed/runtime/pipe/module.py:281-318).  This engine runs hand-written kernels
+with explicit backward passes, so it cannot execute an arbitrary module; what it can do is recognise the layers
+the reference's own scripts are made of -- by the names and shapes of their parameters, not by their class, so a
+script's local copy of the class is recognised too -- build the native layer that computes the same function, and
+take the module's weights into the stage's arenas:
+
+  ``EncoderLayer``   (DeepSpeedExamples/pipeline_parallelism/transformer.py:161-172)  -> :class:`TransformerLayer`
+  ``LayerNorm``      (transformer.py:77-88, the ``encoder.norm`` of :181,250)          -> :class:`FinalLayerNorm`
+  ``lambda x: x.sum(-1)`` (transformer.py:250)                                        -> :class:`SumLast`
+  ``BottleNeck``     (DeepSpeedExamples/pipeline_parallelism/resnet.py:49-75)          -> :class:`BottleNeck`
+  ``nn.MSELoss()``   (transformer.py:264, as ``loss_fn``)                              -> :class:`MSELoss`
+
+Anything else is refused with an error that says what was found: there is no autograd fallback.
+"""
+import torch
+
+from .layers import BottleNeck, FinalLayerNorm, MSELoss, SumLast, TransformerLayer
+
+
+class AdoptionError(Exception):
+    pass
+
+
+def _dropout_probabilities(module):
+    return sorted({float(m.p) for m in module.modules() if isinstance(m, torch.nn.Dropout)})
+
+
+def _is_sum_last(fn):
+    """Behavioural check of a bare callable: does it reduce the last dimension by summation?"""
+    g = torch.Generator().manual_seed(0)
+    for shape in ((2, 3, 8), (1, 5, 16)):
+        x = torch.randn(shape, generator=g, dtype=torch.float64)
+        try:
+            y = fn(x)
+        except Exception:
+            return False
+        if not (isinstance(y, torch.Tensor) and y.shape == x.shape[:-1] and torch.allclose(y, x.sum(-1), rtol=1e-12, atol=1e-12)):
+            return False
+    return True
+
+
+def adopt_layer(obj, training=True):
+    """``(native layer, {parameter name: tensor in the reference's layout} or None)`` for a layer object of the
+    reference's scripts.  ``training``: dropout probabilities count (a module in ``eval()`` mode applies none)."""
+    if all(hasattr(obj, a) for a in ("forward", "backward", "param_specs")):
+        return obj, None                                     # already native
+    if not isinstance(obj, torch.nn.Module):
+        if callable(obj) and _is_sum_last(obj):
+            return SumLast(hidden=None), None
+        raise AdoptionError(f"layer {obj!r} is neither a layer of this package nor one of the reference scripts' layers "
+                            "(a bare callable is taken only if it computes x.sum(-1)); this engine has no autograd fallback")
+    params = {n: p.detach() for n, p in obj.named_parameters()}
+    names = set(params)
+    drops = _dropout_probabilities(obj) if (training and obj.training) else []
+    if names == set(TransformerLayer.REFERENCE_ORDER):
+        hidden = params["sublayer.0.norm.a_2"].numel()
+        ffn = params["feed_forward.w_1.weight"].shape[0]
+        heads = getattr(getattr(obj, "self_attn", None), "h", None)
+        if heads is None:
+            raise AdoptionError("EncoderLayer-shaped module without self_attn.h (number of heads)")
+        if any(p > 0 for p in drops):
+            raise AdoptionError(f"EncoderLayer-shaped module with dropout {drops}: dropout is not built "
+                                "(set the probabilities to 0 or put the module in eval() mode)")
+        eps = float(getattr(obj.sublayer[0].norm, "eps", 1e-6))
+        layer = TransformerLayer(hidden, int(heads), ffn, activation="relu", ln="annotated", mask="none", ln_eps=eps)
+        return layer, params
+    if names == set(BottleNeck.REFERENCE_ORDER):
+        w0, conv3 = params["residual_function.0.weight"], obj.residual_function[3]
+        stride = conv3.stride[0] if isinstance(conv3.stride, tuple) else int(conv3.stride)
+        bn = obj.residual_function[1]
+        layer = BottleNeck(w0.shape[1], w0.shape[0], stride=stride, height=None, width=None, bn_eps=float(bn.eps),
+                           bn_momentum=float(bn.momentum))
+        layer.adopted_running = {i: (obj.residual_function[i].running_mean.detach().clone(),
+                                     obj.residual_function[i].running_var.detach().clone()) for i in (1, 4, 7)}
+        return layer, params
+    if names == {"a_2", "b_2"}:
+        return FinalLayerNorm(params["a_2"].numel(), ln="annotated", ln_eps=float(getattr(obj, "eps", 1e-6))), params
+    raise AdoptionError(f"module {type(obj).__name__} with parameters {sorted(names)[:6]}... is not one of the layers this "
+                        "engine accelerates (EncoderLayer, LayerNorm, BottleNeck of the reference's pipeline_parallelism scripts)")
+
+
+def adopt_loss(loss_fn):
+    if loss_fn is None or isinstance(loss_fn, MSELoss):
+        return loss_fn
+    if isinstance(loss_fn, torch.nn.MSELoss):
+        if loss_fn.reduction != "mean":
+            raise AdoptionError("nn.MSELoss is taken with reduction='mean' only")
+        return MSELoss()
+    raise AdoptionError(f"loss_fn {loss_fn!r}: only nn.MSELoss() (the reference scripts' loss) has a kernel here")

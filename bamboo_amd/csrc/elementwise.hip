@@ -707,6 +707,67 @@ extern "C" int bb_residual_add(int dtype, int64_t n, const void* a, const void* 
     return BB_OK;
 }
 
+// y[r] = sum over the columns of row r (the ``lambda x: x.sum(-1)`` that ends the reference's transformer script,
+// DeepSpeedExamples/pipeline_parallelism/transformer.py:250) and its backward, dx[r, :] = dy[r].  One wave per row,
+// fixed summation order (lane-strided partial sums, then the butterfly).
+template <typename T>
+__global__ __launch_bounds__(256) void rowsum_fwd_kernel(int rows, int cols, const T* __restrict__ x, T* __restrict__ y) {
+    constexpr int VEC = Elem<T>::VEC;
+    const int lane = threadIdx.x & 63;
+    const int row = blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (row >= rows) return;
+    const T* xr = x + (int64_t)row * cols;
+    float s = 0.f;
+    for (int c = lane; c < cols / VEC; c += 64) {
+        float v[VEC];
+        load_vec(xr + c * VEC, v);
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) s += v[e];
+    }
+    s = wave_sum(s);
+    if (lane == 0) Elem<T>::store(y + row, s);
+}
+template <typename T>
+__global__ __launch_bounds__(256) void rowsum_bwd_kernel(int rows, int cols, const T* __restrict__ dy, T* __restrict__ dx) {
+    constexpr int VEC = Elem<T>::VEC;
+    const int lane = threadIdx.x & 63;
+    const int row = blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (row >= rows) return;
+    const float g = Elem<T>::load(dy + row);
+    float v[VEC];
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) v[e] = g;
+    T* dr = dx + (int64_t)row * cols;
+    for (int c = lane; c < cols / VEC; c += 64) store_vec(dr + c * VEC, v);
+}
+
+extern "C" int bb_rowsum_fwd(int dtype, int rows, int cols, const void* x, void* y, void* stream) {
+    int rc = check_rowop("bb_rowsum_fwd", dtype, rows, cols);
+    if (rc) return rc;
+    BB_REQUIRE(x && y, "bb_rowsum_fwd: null pointer");
+    if (rows == 0) return BB_OK;
+    hipStream_t st = (hipStream_t)stream;
+    if (dtype == BB_BF16)
+        hipLaunchKernelGGL(rowsum_fwd_kernel<bf16>, dim3((rows + 3) / 4), dim3(256), 0, st, rows, cols, (const bf16*)x, (bf16*)y);
+    else
+        hipLaunchKernelGGL(rowsum_fwd_kernel<float>, dim3((rows + 3) / 4), dim3(256), 0, st, rows, cols, (const float*)x, (float*)y);
+    BB_LAUNCH_CHECK();
+    return BB_OK;
+}
+extern "C" int bb_rowsum_bwd(int dtype, int rows, int cols, const void* dy, void* dx, void* stream) {
+    int rc = check_rowop("bb_rowsum_bwd", dtype, rows, cols);
+    if (rc) return rc;
+    BB_REQUIRE(dy && dx, "bb_rowsum_bwd: null pointer");
+    if (rows == 0) return BB_OK;
+    hipStream_t st = (hipStream_t)stream;
+    if (dtype == BB_BF16)
+        hipLaunchKernelGGL(rowsum_bwd_kernel<bf16>, dim3((rows + 3) / 4), dim3(256), 0, st, rows, cols, (const bf16*)dy, (bf16*)dx);
+    else
+        hipLaunchKernelGGL(rowsum_bwd_kernel<float>, dim3((rows + 3) / 4), dim3(256), 0, st, rows, cols, (const float*)dy, (float*)dx);
+    BB_LAUNCH_CHECK();
+    return BB_OK;
+}
+
 // out = act(x) and, if wanted, dact = act'(x), elementwise (the activation between the two
 // feed-forward GEMMs).  dact may alias x: a thread reads its elements before it writes them.
 template <typename T, bool DACT>

@@ -146,10 +146,7 @@ class PipelineEngine:
         self._input_grad_store = {
             sid: [torch.empty(act_shape, dtype=model.dtype, device=self.device) for _ in range(self.micro_batches)]
             for sid in built}
-        self._loss_grad = None
-        if model.loss_fn is not None:
-            self._loss_grad = torch.empty(act_shape, dtype=model.dtype, device=self.device)
-            self._loss_ws = torch.empty(hip.mse_workspace(), dtype=torch.float32, device=self.device)
+        self._loss_grad = None     # gradient of the loss head: allocated with the first last-stage output it sees
         self.total_loss = torch.zeros(1, dtype=torch.float32, device=self.device)
 
         self.optimizer = optimizer if optimizer is not None else FusedAdam(
@@ -631,9 +628,10 @@ class PipelineEngine:
         labels = self.pipe_buffers["label"][buffer_id]
         if labels is None:
             raise PipelineError(f"ForwardPass({buffer_id}, {stage_id}): the last stage has no labels for this micro-batch")
-        if self._loss_grad is None:
-            act_shape = (self.batch * self.seq, self.queue.shape[2])
-            self._loss_grad = torch.empty(act_shape, dtype=self.module.dtype, device=self.device)
+        if labels.numel() != out.numel():
+            raise PipelineError(f"labels of micro-batch {buffer_id} have {labels.numel()} elements, the last stage's output {out.numel()}")
+        if self._loss_grad is None or self._loss_grad.shape != out.shape:
+            self._loss_grad = torch.empty(tuple(out.shape), dtype=self.module.dtype, device=self.device)
             self._loss_ws = torch.empty(hip.mse_workspace(), dtype=torch.float32, device=self.device)
         self.module.loss_fn(out, labels, self._loss_grad, 1.0 / self.micro_batches, self.total_loss, True,
                             self._loss_ws, stream=self.main_stream)
@@ -714,9 +712,8 @@ class PipelineEngine:
 
     # ------------------------------------------------------------------ moving layers (reconfiguration)
     def _stage_of_layer(self, layer_idx):
-        prefix = f"{layer_idx}."
-        for sid, sp in self.module.stage_params.items():
-            if any(k.startswith(prefix) for k in sp.index):
+        for sid in self.module.stage_params:
+            if self.module.parts[sid] <= layer_idx < self.module.parts[sid + 1]:
                 return sid
         raise PipelineError(f"layer {layer_idx} is not built in this process")
 
@@ -725,11 +722,9 @@ class PipelineEngine:
         ``send_layers`` (reference engine.py:893-901, ``get_optimizer_state`` :1005-1014)."""
         out = {}
         for idx in layer_idxs:
-            sp = self.module.stage_params[self._stage_of_layer(idx)]
             sd = self.module.layer_state_dict(idx)
-            opt = [{"exp_avg": sp.view(sp.exp_avg, f"{idx}.{name}"), "exp_avg_sq": sp.view(sp.exp_avg_sq, f"{idx}.{name}")}
-                   for name in sd]
-            out[idx] = [sd, opt]
+            m, v = self.module.layer_state_dict(idx, "exp_avg"), self.module.layer_state_dict(idx, "exp_avg_sq")
+            out[idx] = [sd, [{"exp_avg": m[name], "exp_avg_sq": v[name]} for name in sd]]
         return out
 
     def send_layers(self, dst_rank, layer_idxs, state):
@@ -758,9 +753,9 @@ class PipelineEngine:
         for idx, (sd, opt) in recvd_state.items():
             sp = self.module.stage_params[self._stage_of_layer(idx)]
             for (name, t), moments in zip(sd.items(), opt):
-                sp.view(sp.master, f"{idx}.{name}").copy_(t)
-                sp.view(sp.exp_avg, f"{idx}.{name}").copy_(moments["exp_avg"])
-                sp.view(sp.exp_avg_sq, f"{idx}.{name}").copy_(moments["exp_avg_sq"])
+                self.module.load_layer_tensor(idx, name, t)
+                self.module.load_layer_tensor(idx, name, moments["exp_avg"], "exp_avg")
+                self.module.load_layer_tensor(idx, name, moments["exp_avg_sq"], "exp_avg_sq")
             sp.refresh_compute()
 
     _INSTRUCTION_MAP = {

@@ -24,7 +24,7 @@ LN_CODES = {"standard": LN_STANDARD, "annotated": LN_ANNOTATED}
 
 EXPORTS = (
     "bb_version", "bb_last_error", "bb_init", "bb_gemm", "bb_gemm_grouped", "bb_gemm_splitk_workspace", "bb_gemm_grouped_splitk", "bb_gemm_variant", "bb_layernorm_fwd",
-    "bb_layernorm_bwd_workspace", "bb_layernorm_bwd", "bb_layernorm_bwd_static", "bb_colsum_workspace", "bb_colsum_acc",
+    "bb_layernorm_bwd_workspace", "bb_layernorm_bwd", "bb_layernorm_bwd_static", "bb_colsum_workspace", "bb_colsum_acc", "bb_rowsum_fwd", "bb_rowsum_bwd",
     "bb_softmax_fwd", "bb_softmax_bwd", "bb_attention_fwd", "bb_attention_bwd", "bb_residual_add", "bb_act_fwd", "bb_bn_workspace", "bb_batchnorm_fwd", "bb_batchnorm_bwd", "bb_patch3x3", "bb_conv3x3_supported", "bb_conv3x3", "bb_gemm_strip_stats_supported", "bb_strip_stats_workspace", "bb_batchnorm_fwd_strips", "bb_mse_workspace", "bb_mse_fwd_bwd", "bb_graph_begin", "bb_graph_end", "bb_graph_launch", "bb_graph_destroy",
     "bb_adam_multi", "bb_cast", "bb_fill_f32",
 )
@@ -85,6 +85,8 @@ def lib():
     L.bb_layernorm_bwd_workspace.restype = c_int64
     L.bb_layernorm_bwd.argtypes = [c_int, c_int, c_int, c_int, c_float] + [c_void_p] * 11
     L.bb_layernorm_bwd_static.argtypes = [c_int, c_int, c_int, c_int, c_float] + [c_void_p] * 10
+    L.bb_rowsum_fwd.argtypes = [c_int, c_int, c_int, c_void_p, c_void_p, c_void_p]
+    L.bb_rowsum_bwd.argtypes = [c_int, c_int, c_int, c_void_p, c_void_p, c_void_p]
     L.bb_colsum_workspace.argtypes = [c_int]
     L.bb_colsum_workspace.restype = c_int64
     L.bb_colsum_acc.argtypes = [c_int, c_int, c_int, c_void_p, c_int64, c_void_p, c_void_p, c_void_p]
@@ -319,6 +321,22 @@ def layernorm_bwd_static(x, gain, mean, rinv, dy, dres, dx, dgain, dshift, kind,
     check(lib().bb_layernorm_bwd_static(dtype_code(x.dtype), kind, rows, cols, eps, _ptr(x), _ptr(gain), _ptr(mean),
                                         _ptr(rinv), _ptr(dy), _ptr(dres), _ptr(dx), _ptr(dgain), _ptr(dshift),
                                         stream_ptr(stream)), "bb_layernorm_bwd_static")
+
+
+def rowsum_fwd(x, y, stream=None):
+    """y[r] = sum of row r of x ([rows, cols] -> [rows])."""
+    rows, cols = x.shape
+    if y.numel() != rows or y.dtype != x.dtype:
+        raise HipKernelError("rowsum_fwd: y must hold one element of x's dtype per row")
+    check(lib().bb_rowsum_fwd(dtype_code(x.dtype), rows, cols, _ptr(x), _ptr(y), stream_ptr(stream)), "bb_rowsum_fwd")
+
+
+def rowsum_bwd(dy, dx, stream=None):
+    """dx[r, :] = dy[r]."""
+    rows, cols = dx.shape
+    if dy.numel() != rows or dy.dtype != dx.dtype:
+        raise HipKernelError("rowsum_bwd: dy must hold one element of dx's dtype per row")
+    check(lib().bb_rowsum_bwd(dtype_code(dx.dtype), rows, cols, _ptr(dy), _ptr(dx), stream_ptr(stream)), "bb_rowsum_bwd")
 
 
 def colsum_workspace(cols):

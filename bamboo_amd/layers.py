@@ -67,6 +67,14 @@ class TransformerLayer:
     agree bit for bit.
     """
 
+    # parameter registration order of the reference's ``EncoderLayer`` (self_attn, feed_forward, sublayer:
+    # transformer.py:161-168): the order of its ``state_dict()``, hence of the layer wire format
+    REFERENCE_ORDER = (
+        "self_attn.linears.0.weight", "self_attn.linears.0.bias", "self_attn.linears.1.weight", "self_attn.linears.1.bias",
+        "self_attn.linears.2.weight", "self_attn.linears.2.bias", "self_attn.linears.3.weight", "self_attn.linears.3.bias",
+        "feed_forward.w_1.weight", "feed_forward.w_1.bias", "feed_forward.w_2.weight", "feed_forward.w_2.bias",
+        "sublayer.0.norm.a_2", "sublayer.0.norm.b_2", "sublayer.1.norm.a_2", "sublayer.1.norm.b_2")
+
     def __init__(self, hidden, heads, ffn, activation="relu", ln="annotated", mask="none", ln_eps=None,
                  init_std=0.02):
         if hidden % heads:
@@ -134,6 +142,10 @@ class TransformerLayer:
     # ------------------------------------------------------------------ memory plans
     @property
     def feature_dim(self):
+        return self.hidden
+
+    @property
+    def out_features(self):
         return self.hidden
 
     def fused_attention(self, ctx):
@@ -297,6 +309,107 @@ class TransformerLayer:
         return d_x
 
 
+class FinalLayerNorm:
+    """A LayerNorm as a layer of its own: ``encoder.norm``, the first of the two layers that end the reference's
+    transformer script (transformer.py:181,250).  Parameters ``a_2`` / ``b_2`` as in the reference's ``LayerNorm``
+    module (transformer.py:77-88)."""
+
+    REFERENCE_ORDER = ("a_2", "b_2")
+
+    def __init__(self, hidden, ln="annotated", ln_eps=None):
+        if ln not in hip.LN_CODES:
+            raise ValueError(f"unsupported LayerNorm kind {ln}")
+        self.hidden, self.ln = hidden, ln
+        self.eps = ln_eps if ln_eps is not None else (1e-6 if ln == "annotated" else 1e-5)
+        self.w = self.g = None
+
+    feature_dim = property(lambda self: self.hidden)
+    out_features = property(lambda self: self.hidden)
+
+    def param_specs(self):
+        return OrderedDict([("a_2", (self.hidden,)), ("b_2", (self.hidden,))])
+
+    def num_params(self):
+        return 2 * self.hidden
+
+    def init_params(self, master, seed):
+        master["a_2"].fill_(1.0)
+        master["b_2"].zero_()
+
+    def bind(self, compute, grads):
+        self.w, self.g = dict(compute), dict(grads)
+
+    def stash_specs(self, ctx):
+        R, f32 = ctx.rows, torch.float32
+        return [("out", (R, self.hidden), ctx.dtype), ("mean", (R,), f32), ("rinv", (R,), f32)]
+
+    def scratch_specs(self, ctx):
+        return []
+
+    def workspace_elems(self):
+        return hip.layernorm_bwd_workspace(self.hidden)
+
+    def flops_fwd(self, batch, seq):
+        return 0
+
+    def forward(self, x, st, ctx):
+        st["x0"] = x
+        hip.layernorm_fwd(x, self.w["a_2"], self.w["b_2"], st["out"], st["mean"], st["rinv"], hip.LN_CODES[self.ln],
+                          self.eps, stream=ctx.stream)
+        return st["out"]
+
+    def backward(self, d_out, d_x, st, ctx):
+        hip.layernorm_bwd(st["x0"], self.w["a_2"], st["mean"], st["rinv"], d_out, None, d_x, self.g["a_2"], self.g["b_2"],
+                          ctx.workspace, hip.LN_CODES[self.ln], self.eps, stream=ctx.stream)
+        return d_x
+
+
+class SumLast:
+    """``lambda x: x.sum(-1)``: the parameter-free layer that ends the reference's transformer script
+    (transformer.py:250); ``[rows, hidden] -> [rows, 1]``, so that ``MSELoss`` compares with ``[batch, seq]`` labels
+    (transformer.py:205-219,264)."""
+
+    REFERENCE_ORDER = ()
+
+    def __init__(self, hidden):
+        self.hidden = hidden
+
+    feature_dim = property(lambda self: self.hidden)
+    out_features = 1
+
+    def param_specs(self):
+        return OrderedDict()
+
+    def num_params(self):
+        return 0
+
+    def init_params(self, master, seed):
+        pass
+
+    def bind(self, compute, grads):
+        pass
+
+    def stash_specs(self, ctx):
+        return [("out", (ctx.rows, 1), ctx.dtype)]
+
+    def scratch_specs(self, ctx):
+        return []
+
+    def workspace_elems(self):
+        return 0
+
+    def flops_fwd(self, batch, seq):
+        return 0
+
+    def forward(self, x, st, ctx):
+        hip.rowsum_fwd(x, st["out"], stream=ctx.stream)
+        return st["out"]
+
+    def backward(self, d_out, d_x, st, ctx):
+        hip.rowsum_bwd(d_out, d_x, stream=ctx.stream)
+        return d_x
+
+
 class BottleNeck:
     """ResNet bottleneck block ``ReLU(BN(conv1x1(ReLU(BN(conv3x3(ReLU(BN(conv1x1 x)))))) + x)`` with the
     identity shortcut (reference ``BottleNeck``, DeepSpeedExamples/pipeline_parallelism/resnet.py:49-75:
@@ -322,6 +435,10 @@ class BottleNeck:
     def feature_dim(self):
         return self.cin
 
+    @property
+    def out_features(self):
+        return self.cin
+
     def param_specs(self):
         ci, cm = self.cin, self.cmid
         return OrderedDict([
@@ -336,12 +453,27 @@ class BottleNeck:
     def num_params(self):
         return sum(math.prod(s) for s in self.param_specs().values())
 
+    # registration order of the reference's ``residual_function`` (resnet.py:55-64)
+    REFERENCE_ORDER = ("residual_function.0.weight", "residual_function.1.weight", "residual_function.1.bias",
+                       "residual_function.3.weight", "residual_function.4.weight", "residual_function.4.bias",
+                       "residual_function.6.weight", "residual_function.7.weight", "residual_function.7.bias")
+
     @staticmethod
     def to_native(name, tensor):
         """Reference layout -> arena layout: conv weights [O, I, kh, kw] -> [O, kh, kw, I]."""
         if tensor.dim() == 4:
             t = tensor.permute(0, 2, 3, 1).contiguous()
             return t.view(t.shape[0], -1) if t.shape[1] == 1 else t
+        return tensor
+
+    @staticmethod
+    def to_reference(name, tensor):
+        """Arena layout -> the reference's: 1x1 convolutions [O, I] -> [O, I, 1, 1], the 3x3 one [O, kh, kw, I] ->
+        [O, I, kh, kw] (a copy)."""
+        if name in ("residual_function.0.weight", "residual_function.6.weight"):
+            return tensor.reshape(tensor.shape[0], tensor.shape[1], 1, 1)
+        if name == "residual_function.3.weight":
+            return tensor.permute(0, 3, 1, 2).contiguous()
         return tensor
 
     def init_params(self, master, seed):
@@ -398,6 +530,9 @@ class BottleNeck:
         if self.running is None:
             z = lambda n, v: torch.full((n,), v, dtype=torch.float32, device=device)
             self.running = {i: (z(n, 0.0), z(n, 1.0)) for i, n in ((1, self.cmid), (4, self.cmid), (7, self.cin))}
+            for i, (m, v) in getattr(self, "adopted_running", {}).items():   # statistics of the module the block came from
+                self.running[i][0].copy_(m)
+                self.running[i][1].copy_(v)
         return self.running
 
     def _bn_fwd(self, idx, x, resid, y, mean, rstd, relu, ctx, strips=None):
@@ -421,7 +556,16 @@ class BottleNeck:
     def _implicit(self, ctx, mode):
         return hip.conv3x3_supported(ctx.dtype, mode, ctx.batch, self.h, self.w, self.cmid, self.cmid)
 
+    def _bind_image(self, ctx):
+        """A block taken over from a module does not know its image size: square images, side = sqrt(positions)."""
+        if self.h is None or self.w is None:
+            side = math.isqrt(ctx.seq)
+            if side * side != ctx.seq:
+                raise hip.HipKernelError(f"cannot infer a square image from {ctx.seq} positions: pass height= and width=")
+            self.h = self.w = side
+
     def forward(self, x, st, ctx):
+        self._bind_image(ctx)
         if ctx.seq != self.h * self.w:
             raise hip.HipKernelError(f"activation has {ctx.seq} positions, the block expects {self.h}x{self.w}")
         w, sm = self.w_, ctx.stream

@@ -142,7 +142,11 @@ class PipelineModule:
         if not 0 <= stage_id < self.num_stages:
             raise PipelineError(f"stage_id {stage_id} outside [0, {self.num_stages})")
         self.stage_id = stage_id
-        self.loss_fn = loss_fn
+        from .adopt import AdoptionError, adopt_loss
+        try:
+            self.loss_fn = adopt_loss(loss_fn)
+        except AdoptionError as e:
+            raise PipelineError(str(e)) from None
         self.seed_layers, self.seed_fn, self.base_seed = seed_layers, seed_fn, base_seed
         self.micro_offset = 0
         self._layer_specs = list(layers)
@@ -171,10 +175,16 @@ class PipelineModule:
 
     # ------------------------------------------------------------------ partitioning
     def _count_layer_params(self):
+        """Trainable parameters per layer (reference module.py:337-360: modules count theirs, bare callables 0)."""
         counts = []
         for spec in self._layer_specs:
             layer = spec.build() if isinstance(spec, LayerSpec) else spec
-            counts.append(layer.num_params() if hasattr(layer, "num_params") else 0)
+            if hasattr(layer, "num_params"):
+                counts.append(layer.num_params())
+            elif isinstance(layer, torch.nn.Module):
+                counts.append(sum(p.numel() for p in layer.parameters() if p.requires_grad))
+            else:
+                counts.append(0)
         return counts
 
     def _find_layer_type(self, layername):
@@ -208,17 +218,40 @@ class PipelineModule:
 
     # ------------------------------------------------------------------ building
     def _instantiate(self, stage_id):
-        built = []
-        for spec in self._layer_specs[self.parts[stage_id]: self.parts[stage_id + 1]]:
+        """Layer objects of a stage.  Layers of the reference's scripts (``nn.Module`` instances, ``LayerSpec`` of
+        module classes, the ``x.sum(-1)`` callable; reference module.py:281-318) are replaced by the native layer
+        that computes the same function; their weights are kept to be loaded into the arenas."""
+        from .adopt import AdoptionError, adopt_layer
+        built, weights = [], {}
+        prev_features = None
+        for li, spec in enumerate(self._layer_specs[self.parts[stage_id]: self.parts[stage_id + 1]]):
             if isinstance(spec, TiedLayerSpec):
                 raise NotImplementedError("tied layers are not supported on the accelerated stage path")
             layer = spec.build() if isinstance(spec, LayerSpec) else spec
-            if not (hasattr(layer, "forward") and hasattr(layer, "backward") and hasattr(layer, "param_specs")):
-                raise PipelineError(
-                    f"layer {layer!r} is not a native bamboo_amd layer: this engine runs hand-written HIP kernels "
-                    "only and has no autograd fallback")
+            try:
+                layer, taken = adopt_layer(layer)
+            except AdoptionError as e:
+                raise PipelineError(str(e)) from None
+            if getattr(layer, "hidden", 0) is None:      # a parameter-free layer takes its width from its predecessor
+                if prev_features is None:
+                    prev_features = self._features_before(self.parts[stage_id] + li)
+                layer.hidden = prev_features
+            prev_features = layer.out_features
+            if taken:
+                idx = self.parts[stage_id] + li
+                weights.update({f"{idx}.{name}": t for name, t in taken.items()})
             built.append(layer)
+        self._adopted_weights = weights
         return built
+
+    def _features_before(self, layer_idx):
+        """Output width of the layer in front of ``layer_idx`` (for a width-less layer that opens a stage)."""
+        from .adopt import adopt_layer
+        if layer_idx == 0:
+            raise PipelineError("the first layer of the model must state its width")
+        spec = self._layer_specs[layer_idx - 1]
+        layer, _ = adopt_layer(spec.build() if isinstance(spec, LayerSpec) else spec)
+        return layer.out_features
 
     def build_layers(self, stage_id, buffer=None):
         """Materialise the layers of ``stage_id`` on the GPU (own stage, or a stage this process
@@ -230,6 +263,9 @@ class PipelineModule:
         layers = self._instantiate(stage_id)
         sp = StageParams(layers, self.parts[stage_id], self.dtype, self.device)
         sp.init(self.base_seed)
+        if self._adopted_weights:
+            sp.load(self._adopted_weights)       # weights of the modules the layers were taken from
+            self._adopted_weights = {}
         if buffer is not None:
             sp.load(buffer)
         self.func_buckets[stage_id] = layers
@@ -250,14 +286,33 @@ class PipelineModule:
         return names
 
     # ------------------------------------------------------------------ layer state and checkpoints
-    def layer_state_dict(self, layer_idx):
-        """``state_dict`` of one layer (global index): ordered ``{name: fp32 master view}``."""
+    def _layer_home(self, layer_idx):
+        """(stage parameters, layer object) of a built layer (global index)."""
         for sid, sp in self.stage_params.items():
-            prefix = f"{layer_idx}."
-            keys = [k for k in sp.index if k.startswith(prefix)]
-            if keys:
-                return OrderedDict((k[len(prefix):], sp.view(sp.master, k)) for k in keys)
+            if self.parts[sid] <= layer_idx < self.parts[sid + 1]:
+                return sp, sp.layers[layer_idx - self.parts[sid]]
         raise PipelineError(f"layer {layer_idx} is not built in this process")
+
+    def layer_state_dict(self, layer_idx, arena="master"):
+        """``state_dict`` of one layer (global index) as the reference module would give it: parameters in the
+        reference's registration order and layout (convolution weights ``[O, I, kh, kw]``), fp32.  Views of the
+        arena where the layouts agree, copies where they do not; ``arena`` may also name a moment arena
+        (``exp_avg``, ``exp_avg_sq``), whose entries travel in the same order and layout."""
+        sp, layer = self._layer_home(layer_idx)
+        names = getattr(layer, "REFERENCE_ORDER", None) or tuple(layer.param_specs())
+        if set(names) != set(layer.param_specs()):
+            raise PipelineError(f"{type(layer).__name__}.REFERENCE_ORDER does not list the layer's parameters")
+        to_ref = getattr(layer, "to_reference", lambda name, t: t)
+        src = getattr(sp, arena)
+        return OrderedDict((n, to_ref(n, sp.view(src, f"{layer_idx}.{n}"))) for n in names)
+
+    def load_layer_tensor(self, layer_idx, name, tensor, arena="master"):
+        """Inverse of :meth:`layer_state_dict` for one entry: a tensor in the reference's layout into the arena."""
+        sp, layer = self._layer_home(layer_idx)
+        dst = sp.view(getattr(sp, arena), f"{layer_idx}.{name}")
+        if tuple(tensor.shape) != tuple(dst.shape) and hasattr(layer, "to_native"):
+            tensor = layer.to_native(name, tensor)
+        dst.copy_(tensor.to(torch.float32).reshape(dst.shape))
 
     def save_state_dict(self, save_dir, stage_id=None):
         """One ``layer_XX-model_states.pt`` per layer of the stage (reference module.py:804-826)."""
@@ -343,7 +398,7 @@ class PipelineModule:
         if ckpt:
             groups = self._checkpoint_groups(stage_id)
             es = torch.empty((), dtype=self.dtype).element_size()
-            sizes = [ctx.rows * layers[a].feature_dim for a, _ in groups] + [ctx.rows * layers[-1].feature_dim]
+            sizes = [ctx.rows * layers[a].feature_dim for a, _ in groups] + [ctx.rows * layers[-1].out_features]
             per_slot = sum((n * es + 255) // 256 * 256 for n in sizes)
             keep = torch.empty(per_slot * slots, dtype=torch.uint8, device=self.device)
             kept = []
@@ -421,7 +476,7 @@ class PipelineModule:
                     x = layers[i].forward(x, stash[i], ctx)
                 ctx.redundant = was
             for i in range(b - 1, a - 1, -1):
-                dst = grad_input if i == 0 else ctx.buf(f"d_layer{i % 2}", tuple(grad_output.shape))
+                dst = grad_input if i == 0 else ctx.buf(f"d_layer{i % 2}", (grad_output.shape[0], layers[i].feature_dim))
                 layers[i].backward(d, dst, stash[i], ctx)
                 d = dst
         ctx.deferred = False

@@ -176,6 +176,12 @@ int bb_layernorm_bwd_static(int dtype, int kind, int rows, int cols, float eps, 
                             const void* gain, const float* mean, const float* rinv, const void* dy,
                             const void* dres, void* dx, float* dgain, float* dshift, void* stream);
 
+/* Sum over the last dimension and its backward: y[r] = sum_c x[r, c]; dx[r, c] = dy[r]
+ * (the ``lambda x: x.sum(-1)`` tail layer of transformer.py:250 and its autograd).
+ * x, dx: [rows, cols]; y, dy: [rows], all of `dtype`.                                      */
+int bb_rowsum_fwd(int dtype, int rows, int cols, const void* x, void* y, void* stream);
+int bb_rowsum_bwd(int dtype, int rows, int cols, const void* dy, void* dx, void* stream);
+
 /* Column sums of a [rows, cols] matrix accumulated into an fp32 vector: the bias gradient of
  * nn.Linear (autograd of transformer.py:136-146,158).  workspace: fp32, at least
  * bb_colsum_workspace(cols) elements.                                                     */

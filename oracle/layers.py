@@ -5,6 +5,7 @@ Follows DeepSpeedExamples/pipeline_parallelism/transformer.py of the reference:
   attention           transformer.py:106-146 (MultiHeadedAttention, masked_fill(mask==0,-1e9))
   feed_forward        transformer.py:149-158 (PositionwiseFeedForward)
   transformer_layer   transformer.py:91-103,161-172 (SublayerConnection + EncoderLayer, pre-LN)
+  script_tail         transformer.py:181,250 (final LayerNorm, then sum over the hidden dimension)
   bottleneck          resnet.py:49-75        (BottleNeck, bias-free convs, train-mode BN)
   batch_stats_from_strips  resnet.py:56,59,62 (nn.BatchNorm2d batch statistics, restated over
                       32-row strips as the HIP path computes them; pinned against torch's
@@ -134,6 +135,13 @@ def transformer_layer(x, p, cfg, key_lens=None, relu_mask=None):
     x = x + attention(n1, p, cfg, key_lens)
     n2 = layer_norm(x, p["sublayer.1.norm.a_2"], p["sublayer.1.norm.b_2"], cfg.ln, cfg.eps)
     return x + feed_forward(n2, p, cfg, relu_mask)
+
+
+def script_tail(x, p, kind="annotated", eps=1e-6):
+    """The two layers that end the reference's transformer script (transformer.py:250): the encoder's final
+    LayerNorm (:181, parameters a_2 / b_2) and ``lambda x: x.sum(-1)``; [b, s, h] -> [b, s], to be compared with
+    [b, s] labels by ``nn.MSELoss()`` (:205-219, :264)."""
+    return layer_norm(x, p["a_2"], p["b_2"], kind, eps).sum(-1)
 
 
 # ---------------------------------------------------------------- ResNet bottleneck

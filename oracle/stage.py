@@ -62,7 +62,10 @@ class OraclePeer:
 
 class OracleStage:
     def __init__(self, cfg, parts, stage_id, micro_batches, base_seed=1234, dtype=torch.float32,
-                 redundancy_level=0, eager=False, adam=None):
+                 redundancy_level=0, eager=False, adam=None, tail=False):
+        """``tail``: the model ends with the reference script's two extra layers (final LayerNorm, sum over the hidden
+        dimension; transformer.py:250): ``parts[-1]`` then counts them, and the last stage applies them."""
+        self.tail = tail
         self.cfg, self.parts, self.stage_id, self.M = cfg, parts, stage_id, micro_batches
         self.S = len(parts) - 1
         self.dtype = dtype
@@ -83,7 +86,16 @@ class OracleStage:
     def build(self, stage):
         conv = isinstance(self.cfg, olayers.BottleneckCfg)
         layers = []
+        n_blocks = self.parts[-1] - (2 if self.tail else 0)
         for li in range(self.parts[stage], self.parts[stage + 1]):
+            if li == n_blocks:            # the final LayerNorm: gain 1, shift 0
+                h = self.cfg.hidden
+                layers.append({"a_2": torch.ones(h, dtype=self.dtype).requires_grad_(True),
+                               "b_2": torch.zeros(h, dtype=self.dtype).requires_grad_(True)})
+                continue
+            if li > n_blocks:             # x.sum(-1): no parameters
+                layers.append({})
+                continue
             if conv:
                 p = olayers.init_bottleneck_params(self.cfg, self.base_seed + li, dtype=self.dtype)
             else:
@@ -104,7 +116,10 @@ class OracleStage:
                 y = olayers.bottleneck(y, p, self.cfg, m)
             return y.permute(0, 2, 3, 1).reshape(b, hw, c)
         for p, m in zip(self.params[stage], masks):
-            x = olayers.transformer_layer(x, p, self.cfg, key_lens, m)
+            if set(p) == {"a_2", "b_2"}:
+                x = olayers.script_tail(x, p, self.cfg.ln, self.cfg.eps)
+            elif p:
+                x = olayers.transformer_layer(x, p, self.cfg, key_lens, m)
         return x
 
     def named_grads(self, stage):

@@ -1,0 +1,99 @@
+"""Layers of the reference's scripts handed to PipelineModule as they are (nn.Module instances, LayerSpec of module
+classes, the x.sum(-1) callable): recognised by their parameters, replaced by native layers, weights taken over; and
+the order / layout in which a layer's state travels (state_dict order of the reference module).  CPU only: building
+the arenas runs no kernel in fp32."""
+import pytest
+import torch
+
+from bamboo_amd import (BottleNeck, FinalLayerNorm, LayerSpec, MSELoss, PipelineError, PipelineModule, SumLast,
+                        TransformerLayer)
+from tests.reference_shapes import RefBottleNeck, RefEncoderLayer, RefLayerNorm
+
+
+def encoder_script_layers(n=4, d=32, h=4, ff=64, p=0.0):
+    """The layer list of the reference's transformer script (transformer.py:246-250): the encoder's layers, its
+    final norm, and the sum over the hidden dimension."""
+    torch.manual_seed(0)
+    layers = [RefEncoderLayer(d, h, ff, p) for _ in range(n)]
+    return layers + [RefLayerNorm(d), lambda x: x.sum(-1)]
+
+
+def test_script_layer_list_is_taken_over():
+    layers = encoder_script_layers()
+    with torch.no_grad():
+        for m in layers[:-1]:
+            for prm in m.parameters():
+                prm.add_(0.01 * torch.randn_like(prm))
+    model = PipelineModule(layers, num_stages=2, loss_fn=torch.nn.MSELoss(), partition_method="uniform", stage_id=1,
+                           dtype=torch.float32, device="cpu")
+    assert isinstance(model.loss_fn, MSELoss)
+    built = model.func_buckets[1]
+    assert [type(b) for b in built] == [TransformerLayer, FinalLayerNorm, SumLast]
+    assert (built[0].hidden, built[0].heads, built[0].ffn, built[0].activation, built[0].ln, built[0].mask) == (32, 4, 64, "relu", "annotated", "none")
+    assert built[2].hidden == 32 and built[2].out_features == 1
+    # weights: every parameter of the modules is in the arena under the reference's key "{layer_idx}.{name}"
+    sp = model.stage_params[1]
+    named = sp.named(sp.master)
+    for li in (3, 4):
+        for name, prm in layers[li].named_parameters():
+            assert torch.equal(named[f"{li}.{name}"], prm.detach()), (li, name)
+    assert set(named) == {f"{li}.{n}" for li in (3, 4) for n, _ in layers[li].named_parameters()}
+    # the state of a layer travels in the module's own state_dict order
+    assert list(model.layer_state_dict(3)) == list(layers[3].state_dict())
+    assert list(model.layer_state_dict(4)) == list(layers[4].state_dict())
+    assert list(model.layer_state_dict(5)) == []
+
+
+def test_parameter_partitioning_counts_module_parameters():
+    layers = encoder_script_layers(n=6)
+    model = PipelineModule(layers, num_stages=3, partition_method="parameters", stage_id=0, dtype=torch.float32, device="cpu")
+    assert model._count_layer_params()[:6] == [sum(p.numel() for p in layers[0].parameters())] * 6
+    assert model._count_layer_params()[6:] == [64, 0]
+    assert model.parts[0] == 0 and model.parts[-1] == 8 and model.parts == sorted(model.parts)
+
+
+def test_layerspec_of_a_module_class_and_a_stage_that_opens_with_the_callable():
+    torch.manual_seed(1)
+    specs = [LayerSpec(RefEncoderLayer, 32, 4, 64, 0.0), LayerSpec(RefLayerNorm, 32), lambda x: x.sum(-1)]
+    model = PipelineModule(specs, num_stages=2, partition_method="custom", custom_partitions=[0, 2, 3], stage_id=1,
+                           dtype=torch.float32, device="cpu")
+    (tail,) = model.func_buckets[1]
+    assert isinstance(tail, SumLast) and tail.hidden == 32        # width taken from the layer in front of the stage
+
+
+def test_what_is_not_recognised_is_refused():
+    with pytest.raises(PipelineError, match="not one of the layers"):
+        PipelineModule([torch.nn.Linear(8, 8)], num_stages=1, stage_id=0, dtype=torch.float32, device="cpu")
+    with pytest.raises(PipelineError, match="bare callable"):
+        PipelineModule([RefEncoderLayer(32, 4, 64, 0.0), lambda x: x * 2], num_stages=1, stage_id=0, dtype=torch.float32, device="cpu")
+    with pytest.raises(PipelineError, match="dropout"):
+        PipelineModule([RefEncoderLayer(32, 4, 64, 0.1)], num_stages=1, stage_id=0, dtype=torch.float32, device="cpu")
+    # the same module in eval() mode applies no dropout: taken
+    m = RefEncoderLayer(32, 4, 64, 0.1).eval()
+    assert isinstance(PipelineModule([m], num_stages=1, stage_id=0, dtype=torch.float32, device="cpu").func_buckets[0][0], TransformerLayer)
+    with pytest.raises(PipelineError, match="MSELoss"):
+        PipelineModule([m], num_stages=1, stage_id=0, loss_fn=torch.nn.L1Loss(), dtype=torch.float32, device="cpu")
+
+
+def test_bottleneck_module_is_taken_over_with_layouts_and_running_statistics():
+    torch.manual_seed(2)
+    ref = RefBottleNeck(64, 16)
+    with torch.no_grad():
+        ref.residual_function[4].running_mean.add_(0.5)
+    model = PipelineModule([ref, RefBottleNeck(64, 16)], num_stages=1, stage_id=0, dtype=torch.float32, device="cpu")
+    blk = model.func_buckets[0][0]
+    assert isinstance(blk, BottleNeck) and (blk.cin, blk.cmid, blk.h) == (64, 16, None)
+    sd = model.layer_state_dict(0)
+    ref_params = dict(ref.named_parameters())
+    assert list(sd) == [k for k in ref.state_dict() if k in ref_params]       # parameters in registration order
+    for k, v in sd.items():
+        assert v.shape == ref_params[k].shape and torch.equal(v, ref_params[k].detach()), k     # [O, I, kh, kw] on the wire
+    # in the arena the 3x3 weight is tap-major
+    sp = model.stage_params[0]
+    w3 = sp.view(sp.master, "0.residual_function.3.weight")
+    assert w3.shape == (16, 3, 3, 16) and torch.equal(w3.permute(0, 3, 1, 2), ref_params["residual_function.3.weight"].detach())
+    # a tensor in the reference's layout goes back into the arena through the inverse conversion
+    new = torch.randn(16, 16, 3, 3)
+    model.load_layer_tensor(0, "residual_function.3.weight", new)
+    assert torch.equal(model.layer_state_dict(0)["residual_function.3.weight"], new)
+    assert float(blk._running("cpu")[4][0][0]) == 0.5

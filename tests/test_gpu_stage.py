@@ -520,6 +520,90 @@ def test_paced_pipeline_changes_timing_not_results(hiplib, rc_issue):
         build(hid, heads, ffn, L, S, sid, mb, M, seq, dtype, GPT_VARIANT, 1, True, rc_issue="asap")   # needs the second stream
 
 
+def test_script_layers_taken_over_run_as_the_last_stage(hiplib):
+    """The reference script's own layer list -- EncoderLayer modules, the final LayerNorm, ``lambda x: x.sum(-1)``,
+    ``nn.MSELoss()`` against [batch, seq] labels (transformer.py:246-264) -- handed over as it is.  The last stage
+    (one encoder layer, norm, sum) runs on the HIP kernels; loss, parameter gradients and the gradient sent
+    upstream equal torch autograd on the modules themselves (fp32)."""
+    from tests.reference_shapes import RefEncoderLayer, RefLayerNorm
+    hid, heads, ffn, mb, M, seq = 128, 2, 256, 2, 4, 64
+    torch.manual_seed(11)
+    mods = [RefEncoderLayer(hid, heads, ffn, 0.0) for _ in range(2)] + [RefLayerNorm(hid)]
+    with torch.no_grad():
+        for m in mods:
+            for prm in m.parameters():
+                prm.add_(0.05 * torch.randn_like(prm))
+    layers = mods + [lambda x: x.sum(-1)]
+    g = torch.Generator().manual_seed(12)
+    labels = [torch.randn(mb, seq, generator=g) for _ in range(M)]
+    model = PipelineModule(layers, num_stages=2, partition_method="custom", custom_partitions=[0, 1, 4], stage_id=1,
+                           loss_fn=torch.nn.MSELoss(), dtype=torch.float32, device=DEV)
+    q = SeededActivationQueue((mb, seq, hid), torch.float32, M, stage_ids=[1], seed=5, device=DEV)
+    cfg = {"train_micro_batch_size_per_gpu": mb, "gradient_accumulation_steps": M}
+    engine, _, _, _ = bamboo_amd.initialize(model=model, config=cfg, activation_queue=q, install_signal_handler=False,
+                                            training_data=[(torch.zeros(1), y) for y in labels])
+    with NoStep(engine):
+        loss = engine.train_batch()
+    torch.cuda.synchronize()
+    total, xgrads = 0.0, []
+    for k in range(M):
+        x = q.activations[k].cpu().clone().requires_grad_(True)
+        out = layers[3](mods[2](mods[1](x)))
+        l = torch.nn.functional.mse_loss(out, labels[k])
+        (l / M).backward()
+        total += float(l)
+        xgrads.append(x.grad)
+    rel_err.lowp = False
+    assert abs(float(loss) - total / M) < 1e-5 * total / M
+    ref = {f"{li}.{n}": p.grad for li in (1, 2) for n, p in mods[li].named_parameters()}
+    got = dict(engine.module.get_named_grad(1))
+    assert set(got) == set(ref)
+    floor = grad_floor(ref)
+    for name, gr in got.items():
+        assert rel_err(gr, ref[name], floor) < 1e-4, name
+    for k in range(M):
+        assert rel_err(q.sent_grads[(1, k)], xgrads[k].view(mb * seq, hid)) < 1e-4
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["fp32", "bf16"])
+def test_last_stage_with_the_script_tail_matches_oracle(hiplib, dtype):
+    """Last stage = transformer layer, final LayerNorm, sum over the hidden dimension, MSE against [batch, seq]
+    labels (native layer specs, GPT variant) against the oracle stage with the same tail."""
+    from bamboo_amd import FinalLayerNorm, MSELoss, SumLast
+    hid, heads, ffn, mb, M, seq = 128, 2, 256, 2, 4, 64
+    specs = [LayerSpec(TransformerLayer, hid, heads, ffn, **GPT_VARIANT) for _ in range(2)]
+    specs += [LayerSpec(FinalLayerNorm, hid, ln="standard"), LayerSpec(SumLast, hid)]
+    model = PipelineModule(specs, num_stages=2, partition_method="custom", custom_partitions=[0, 1, 4], stage_id=1,
+                           loss_fn=MSELoss(), dtype=dtype, device=DEV)
+    # a final norm with gain 1 and shift 0 sums to zero: move it off that point
+    sp = model.stage_params[1]
+    gen = torch.Generator().manual_seed(3)
+    sp.load({"2.a_2": 1 + 0.3 * torch.randn(hid, generator=gen), "2.b_2": 0.3 * torch.randn(hid, generator=gen)})
+    q = SeededActivationQueue((mb, seq, hid), dtype, M, stage_ids=[1], seed=5, device=DEV)
+    labels = [torch.randn(mb, seq, generator=gen).to(dtype) for _ in range(M)]
+    cfg = {"train_micro_batch_size_per_gpu": mb, "gradient_accumulation_steps": M, "bf16": {"enabled": dtype == torch.bfloat16}}
+    engine, _, _, _ = bamboo_amd.initialize(model=model, config=cfg, activation_queue=q, install_signal_handler=False,
+                                            training_data=[(torch.zeros(1), y) for y in labels])
+    st = OracleStage(ol.TransformerCfg(hidden=hid, heads=heads, ffn=ffn, **GPT_VARIANT), [0, 1, 4], 1, M, dtype=torch.float64, tail=True)
+    named = sp.named(sp.compute)
+    for key, t in st.named_params(1).items():
+        with torch.no_grad():
+            t.copy_(named[key].double().cpu())
+    peer = OraclePeer([a.double().cpu() for a in q.activations], M, labels=[y.double() for y in labels])
+    bufs, _ = st.run_batch(peer, optimizer_step=False)
+    with NoStep(engine):
+        loss = engine.train_batch()
+    torch.cuda.synchronize()
+    tol = 1e-4 if dtype == torch.float32 else 2e-2
+    rel_err.lowp = dtype == torch.bfloat16
+    assert abs(float(loss) - float(peer.loss) / M) < tol * float(peer.loss) / M
+    ref = st.named_grads(1)
+    for name, gr in engine.module.get_named_grad(1):
+        assert rel_err(gr, ref[name], grad_floor(ref)) < tol, name
+    for k in range(M):
+        assert rel_err(q.sent_grads[(1, k)], bufs["sent_grad"][(1, k)].view(mb * seq, hid)) < tol
+
+
 def test_optimizer_step_matches_oracle(hiplib):
     rel_err.lowp = False
     hid, heads, ffn, L, S, sid, mb, M, seq = 128, 2, 256, 2, 4, 1, 2, 4, 64

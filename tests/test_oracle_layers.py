@@ -79,6 +79,31 @@ def test_layer_matches_torch_encoder_layer():
     torch.testing.assert_close(ol.transformer_layer(x, p, cfg_c), ref(x, src_mask=cm, is_causal=True), rtol=1e-9, atol=1e-9)
 
 
+def test_script_tail_equals_the_module_form():
+    """final LayerNorm + sum over the hidden dimension against the stand-in of the reference's LayerNorm module
+    followed by the script's lambda, values and gradients."""
+    from tests.reference_shapes import RefLayerNorm
+    torch.manual_seed(5)
+    norm = RefLayerNorm(24).double()
+    with torch.no_grad():
+        norm.a_2.add_(0.2 * torch.randn(24, dtype=torch.float64))
+        norm.b_2.add_(0.2 * torch.randn(24, dtype=torch.float64))
+    x = torch.randn(2, 7, 24, dtype=torch.float64, requires_grad=True)
+    p = {"a_2": norm.a_2.detach().clone().requires_grad_(True), "b_2": norm.b_2.detach().clone().requires_grad_(True)}
+    y = ol.script_tail(x, p)
+    ref = (lambda t: t.sum(-1))(norm(x))
+    assert y.shape == (2, 7)
+    torch.testing.assert_close(y, ref, rtol=1e-12, atol=1e-12)
+    w = torch.randn(2, 7, dtype=torch.float64)
+    gx, ga = torch.autograd.grad((y * w).sum(), [x, p["a_2"]])
+    rx, ra = torch.autograd.grad((ref * w).sum(), [x, norm.a_2])
+    torch.testing.assert_close(gx, rx, rtol=1e-10, atol=1e-12)
+    torch.testing.assert_close(ga, ra, rtol=1e-10, atol=1e-12)
+    # with unit gain and zero shift the normalised row sums to zero: the tail's output is 0 whatever x
+    unit = {"a_2": torch.ones(24, dtype=torch.float64), "b_2": torch.zeros(24, dtype=torch.float64)}
+    assert float(ol.script_tail(x.detach(), unit).abs().max()) < 1e-12
+
+
 def test_gelu_tanh_formula():
     x = torch.linspace(-4, 4, 101, dtype=torch.float64)
     ref = 0.5 * x * (1 + torch.tanh(0.7978845608028654 * (x + 0.044715 * x ** 3)))
