@@ -53,7 +53,7 @@ MEASURED_TRAFFIC_BYTES = {
 }
 
 
-def build_engine(cfg, rc, rc_stream, seed=1138, use_graphs=False, paced=None, rc_issue="reference"):
+def build_engine(cfg, rc, rc_stream, seed=1138, use_graphs=False, paced=None, rc_issue="reference", eager=True):
     """``paced=(t_fwd, t_bwd)``: the neighbours are a closed-loop model of the other stages of a 1F1B pipeline whose
     forward / backward passes take that long, so the stage waits for its inputs as in a real pipeline."""
     import torch
@@ -81,7 +81,7 @@ def build_engine(cfg, rc, rc_stream, seed=1138, use_graphs=False, paced=None, rc
           "optimizer": {"type": "Adam", "params": {"lr": 1e-3, "betas": [0.9, 0.999], "eps": 1e-8}},
           "bf16": {"enabled": cfg["dtype"] == "bf16"}}
     engine, _, _, _ = bamboo_amd.initialize(model=model, config=ds, redundancy_level=1 if rc else 0,
-                                            eager_recovery=rc, activation_queue=q, rc_stream=rc_stream,
+                                            eager_recovery=rc and eager, activation_queue=q, rc_stream=rc_stream,
                                             install_signal_handler=False, use_graphs=use_graphs, rc_issue=rc_issue)
     return engine, q
 
@@ -362,6 +362,25 @@ def main():
                     "post_failover_ms_per_step": round(t_post * 1e3, 3),
                     "note": "pause = failure detected (GPU drained) -> successor's lost work replayed from the RC stash; "
                             "post-failover = own + promoted layers as two local stages"}
+        # the same failure without redundant forwards (lazy recovery: host mirrors of the shadow parameters, nothing
+        # computed ahead): promotion materialises the layers and the replay recomputes the successor's forwards
+        del engine, q
+        gc.collect()
+        torch.cuda.empty_cache()
+        engine, q = build_engine(cfg, rc=True, rc_stream=False, eager=False)
+        t_lazy = time_steps(engine, args.steps, args.warmup)
+        q.preempt_successor(args.failover_at, STAGE_ID)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        engine.train_batch()
+        torch.cuda.synchronize()
+        t_fail_lazy = time.perf_counter() - t0
+        q.revive()
+        fo = engine.last_failover
+        failover["lazy"] = {"samples_per_s_before": round(samples / t_lazy, 3), "promote_ms": round(fo["promote_s"] * 1e3, 3),
+                            "pause_ms": round(fo["pause_s"] * 1e3, 3), "failover_batch_ms": round(t_fail_lazy * 1e3, 3),
+                            "note": "redundancy_level=1 without eager recovery: no RC overhead before the failure, the "
+                                    "pause pays for building the layers from host mirrors and for the lost forwards"}
 
     n_graphs = sum(1 for v in engine._graphs.values() if isinstance(v, tuple))
     layer = engine.module.func_buckets[STAGE_ID][0]
