@@ -61,11 +61,12 @@ def adopt_layer(obj, training=True):
         heads = getattr(getattr(obj, "self_attn", None), "h", None)
         if heads is None:
             raise AdoptionError("EncoderLayer-shaped module without self_attn.h (number of heads)")
-        if any(p > 0 for p in drops):
-            raise AdoptionError(f"EncoderLayer-shaped module with dropout {drops}: dropout is not built "
-                                "(set the probabilities to 0 or put the module in eval() mode)")
+        if len(drops) > 1:
+            raise AdoptionError(f"EncoderLayer-shaped module with different dropout probabilities {drops}: the layer "
+                                "takes one probability for its four dropout sites, as the reference's make_encoder sets them")
         eps = float(getattr(obj.sublayer[0].norm, "eps", 1e-6))
-        layer = TransformerLayer(hidden, int(heads), ffn, activation="relu", ln="annotated", mask="none", ln_eps=eps)
+        layer = TransformerLayer(hidden, int(heads), ffn, activation="relu", ln="annotated", mask="none", ln_eps=eps,
+                                 dropout=drops[0] if drops else 0.0)
         return layer, params
     if names == set(BottleNeck.REFERENCE_ORDER):
         w0, conv3 = params["residual_function.0.weight"], obj.residual_function[3]

@@ -34,7 +34,12 @@ struct AttnArgs {
     int batch, heads, seq, mask;
     float scale_log2;                              // log2(e) / sqrt(d)
     float scale;                                   // 1 / sqrt(d)
+    DropKey drop;                                  // dropout on the probabilities (thresh 0: none)
 };
+// index of probability (b, head, q, kv) in the [batch, heads, seq, seq] tensor that is never stored
+__device__ __forceinline__ uint64_t prob_index(const AttnArgs& a, int b, int head, int q) {
+    return ((uint64_t)(b * a.heads + head) * a.seq + q) * a.seq;
+}
 
 // Global -> LDS transfers (16 or 4 bytes per lane; the LDS target is M0 + lane * size), issued as
 // inline assembly: while the compiler sees such a load in flight it turns every wait for an LDS
@@ -250,6 +255,15 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const AttnArgs a) {
                 }
             lsum = lsum * alpha + psum;
             m = mnew;
+            if (a.drop.thresh) {   // the normaliser takes every probability, the context only the kept ones
+                const uint64_t base = prob_index(a, b, head, min(myq, last)) + kv0;
+#pragma unroll
+                for (int u = 0; u < 2; ++u)
+#pragma unroll
+                    for (int r = 0; r < 16; ++r)
+                        s[u][r] = bb_dropout_keep(a.drop.k0, a.drop.k1, a.drop.thresh, base + u * 32 + acc_row(r, lane))
+                                      ? s[u][r] * a.drop.scale : 0.f;
+            }
             if (__any(alpha != 1.0f)) {  // wave-uniform: once the maxima have settled nothing is rescaled
 #pragma unroll
                 for (int t2 = 0; t2 < 2; ++t2)
@@ -413,6 +427,21 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dkv_kernel(const AttnArgs a) 
                     s[r] = q >= qmin && q < a.seq ? s[r] : 0.f;
                 }
             }
+            // dropout: dP = dP~ o mask / (1 - p) before it meets P; P itself is masked (into what multiplied V in
+            // the forward) only after dS has been formed from the unmasked probabilities
+            unsigned kept = 0xffffu;
+            if (a.drop.thresh) {
+                asm volatile("" ::: "memory");
+                const int qlane = t * 64 + u * 32 + 4 * (lane >> 5);
+                kept = 0u;
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    const int q = min(qlane + 8 * (r >> 2) + (r & 3), last);
+                    const bool keep = bb_dropout_keep(a.drop.k0, a.drop.k1, a.drop.thresh, prob_index(a, b, head, q) + min(mykv, last));
+                    kept |= keep ? 1u << r : 0u;
+                    dp[r] = keep ? dp[r] * a.drop.scale : 0.f;
+                }
+            }
 #pragma unroll
             for (int g4 = 0; g4 < 4; ++g4) {
                 const int ql = u * 32 + 8 * g4 + 4 * (lane >> 5);
@@ -420,7 +449,11 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dkv_kernel(const AttnArgs a) 
 #pragma unroll
                 for (int e = 0; e < 4; ++e) dp[g4 * 4 + e] = s[g4 * 4 + e] * (dp[g4 * 4 + e] - d4[e]);
             }
-            // dV^T += dO^T P ; dK^T += Q^T dS   (contraction over the 32 queries of this sub-tile)
+            if (a.drop.thresh) {
+#pragma unroll
+                for (int r = 0; r < 16; ++r) s[r] = (kept >> r) & 1u ? s[r] * a.drop.scale : 0.f;
+            }
+            // dV^T += dO^T P~ ; dK^T += Q^T dS   (contraction over the 32 queries of this sub-tile)
 #pragma unroll
             for (int kk = 0; kk < 2; ++kk) {
                 const bf16x8 pf = pack_acc(s, kk), dsf = pack_acc(dp, kk);
@@ -539,6 +572,13 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dq_kernel(const AttnArgs a) {
 #pragma unroll
                     for (int r = 0; r < 16; ++r) s[r] = 8 * (r >> 2) + (r & 3) < lim ? s[r] : 0.f;
                 }
+                if (a.drop.thresh) {
+                    asm volatile("" ::: "memory");
+                    const uint64_t base = prob_index(a, b, head, min(myq, last)) + kv0 + u * 32;
+#pragma unroll
+                    for (int r = 0; r < 16; ++r)
+                        dp[r] = bb_dropout_keep(a.drop.k0, a.drop.k1, a.drop.thresh, base + acc_row(r, lane)) ? dp[r] * a.drop.scale : 0.f;
+                }
 #pragma unroll
                 for (int r = 0; r < 16; ++r) dp[r] = s[r] * (dp[r] - my_delta);
                 // dQ^T += K^T dS^T (contraction over the 32 keys of this sub-tile)
@@ -585,12 +625,15 @@ static int check_attn(const char* name, int dtype, int mask, int batch, int head
 
 extern "C" int bb_attention_fwd(int dtype, int mask, int batch, int heads, int seq, int head_dim, const void* q,
                                 const void* k, const void* v, int64_t ld_qkv, void* out, int64_t ld_out, float* lse,
-                                const int32_t* key_len, void* stream) {
+                                const int32_t* key_len, float dropout_p, uint32_t dropout_k0, uint32_t dropout_k1,
+                                void* stream) {
     int rc = check_attn("bb_attention_fwd", dtype, mask, batch, heads, seq, head_dim, ld_qkv, ld_out, key_len);
     if (rc) return rc;
     if (batch == 0 || seq == 0) return BB_OK;
     BB_REQUIRE(q && k && v && out && lse, "bb_attention_fwd: null pointer");
+    BB_REQUIRE(dropout_p >= 0.f && dropout_p < 1.f, "bb_attention_fwd: dropout_p must be in [0, 1)");
     AttnArgs a = {};
+    a.drop = bb_drop_key(dropout_p, dropout_k0, dropout_k1);
     a.q = (const bf16*)q; a.k = (const bf16*)k; a.v = (const bf16*)v;
     a.out = (bf16*)out; a.lse = lse; a.key_len = key_len;
     a.ld_qkv = ld_qkv; a.ld_o = ld_out;
@@ -605,13 +648,16 @@ extern "C" int bb_attention_fwd(int dtype, int mask, int batch, int heads, int s
 extern "C" int bb_attention_bwd(int dtype, int mask, int batch, int heads, int seq, int head_dim, const void* q,
                                 const void* k, const void* v, int64_t ld_qkv, const void* out, const void* d_out,
                                 int64_t ld_out, const float* lse, float* delta, void* dq, void* dk, void* dv,
-                                int64_t ld_dqkv, const int32_t* key_len, void* stream) {
+                                int64_t ld_dqkv, const int32_t* key_len, float dropout_p, uint32_t dropout_k0,
+                                uint32_t dropout_k1, void* stream) {
     int rc = check_attn("bb_attention_bwd", dtype, mask, batch, heads, seq, head_dim, ld_qkv, ld_out, key_len);
     if (rc) return rc;
     if (batch == 0 || seq == 0) return BB_OK;
     BB_REQUIRE(q && k && v && out && d_out && lse && delta && dq && dk && dv, "bb_attention_bwd: null pointer");
     BB_REQUIRE(ld_dqkv % 4 == 0 && ld_dqkv >= heads * 64, "bb_attention_bwd: bad gradient leading dimension");
+    BB_REQUIRE(dropout_p >= 0.f && dropout_p < 1.f, "bb_attention_bwd: dropout_p must be in [0, 1)");
     AttnArgs a = {};
+    a.drop = bb_drop_key(dropout_p, dropout_k0, dropout_k1);
     a.q = (const bf16*)q; a.k = (const bf16*)k; a.v = (const bf16*)v;
     a.o = (const bf16*)out; a.d_o = (const bf16*)d_out;
     a.dq = (bf16*)dq; a.dk = (bf16*)dk; a.dv = (bf16*)dv;

@@ -153,4 +153,34 @@ __device__ __forceinline__ float dact_f(float x, int kind) {
     return kind == BB_ACT_RELU ? (x > 0.0f ? 1.0f : 0.0f) : dgelu_tanh_f(x);
 }
 
+// ---- dropout -------------------------------------------------------------------------------
+// Counter-based keep/drop decision: a pure function of (key, element index), so a redundant forward, a normal
+// forward and the backward pass of the same (layer, site, micro-batch) make the same decisions without a mask ever
+// being stored.  Two rounds of a 32-bit finalizer (xorshift-multiply), the key words and the high half of the
+// counter injected between them; an element is kept when the result is >= thresh = p * 2^32.
+struct DropKey {
+    uint32_t k0, k1, thresh;   // thresh == 0: no dropout
+    float scale;               // 1 / (1 - p)
+};
+__host__ __device__ __forceinline__ uint32_t bb_mix32(uint32_t x) {
+    x ^= x >> 16; x *= 0x7feb352du;
+    x ^= x >> 15; x *= 0x846ca68bu;
+    x ^= x >> 16;
+    return x;
+}
+__host__ __device__ __forceinline__ bool bb_dropout_keep(uint32_t k0, uint32_t k1, uint32_t thresh, uint64_t idx) {
+    uint32_t x = bb_mix32((uint32_t)idx ^ k0);
+    x = bb_mix32(x + ((uint32_t)(idx >> 32) ^ k1));
+    return x >= thresh;
+}
+static inline DropKey bb_drop_key(float p, uint32_t k0, uint32_t k1) {
+    DropKey d = {k0, k1, 0u, 1.0f};
+    if (p > 0.f) {
+        const double t = (double)p * 4294967296.0;
+        d.thresh = t >= 4294967295.0 ? 4294967295u : (uint32_t)(t + 0.5);
+        d.scale = 1.0f / (1.0f - p);
+    }
+    return d;
+}
+
 static inline int64_t ceil_div64(int64_t a, int64_t b) { return (a + b - 1) / b; }

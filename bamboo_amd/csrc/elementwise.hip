@@ -707,6 +707,43 @@ extern "C" int bb_residual_add(int dtype, int64_t n, const void* a, const void* 
     return BB_OK;
 }
 
+// dst = dropout(src) with the decisions of key (k0, k1): element i of the contiguous tensor is kept (and scaled by
+// 1 / (1 - p)) when bb_dropout_keep says so.  nn.Dropout in training mode (transformer.py:98-103,125-126,154-158)
+// with a mask that is a pure function of (key, i); the same call on a gradient is its backward.
+template <typename T>
+__global__ __launch_bounds__(256) void dropout_kernel(int64_t nvec, const T* src, T* dst, DropKey key) {
+    constexpr int VEC = Elem<T>::VEC;
+    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < nvec; i += (int64_t)gridDim.x * 256) {
+        float v[VEC];
+        load_vec(src + i * VEC, v);
+#pragma unroll
+        for (int e = 0; e < VEC; ++e)
+            v[e] = bb_dropout_keep(key.k0, key.k1, key.thresh, (uint64_t)(i * VEC + e)) ? v[e] * key.scale : 0.f;
+        store_vec(dst + i * VEC, v);
+    }
+}
+extern "C" int bb_dropout_apply(int dtype, int64_t n, const void* src, void* dst, float p, uint32_t k0, uint32_t k1, void* stream) {
+    BB_REQUIRE(dtype == BB_F32 || dtype == BB_BF16, "bb_dropout_apply: bad dtype %d", dtype);
+    const int vec = dtype == BB_BF16 ? 8 : 4;
+    BB_REQUIRE(n >= 0 && n % vec == 0, "bb_dropout_apply: n (%lld) must be a multiple of %d", (long long)n, vec);
+    BB_REQUIRE(p >= 0.f && p < 1.f, "bb_dropout_apply: p must be in [0, 1)");
+    BB_REQUIRE(src && dst, "bb_dropout_apply: null pointer");
+    if (n == 0) return BB_OK;
+    const DropKey key = bb_drop_key(p, k0, k1);
+    const int64_t nvec = n / vec;
+    hipStream_t st = (hipStream_t)stream;
+    if (dtype == BB_BF16)
+        hipLaunchKernelGGL(dropout_kernel<bf16>, dim3(grid_for(nvec)), dim3(256), 0, st, nvec, (const bf16*)src, (bf16*)dst, key);
+    else
+        hipLaunchKernelGGL(dropout_kernel<float>, dim3(grid_for(nvec)), dim3(256), 0, st, nvec, (const float*)src, (float*)dst, key);
+    BB_LAUNCH_CHECK();
+    return BB_OK;
+}
+extern "C" int bb_dropout_keep_host(float p, uint32_t k0, uint32_t k1, uint64_t index) {
+    const DropKey key = bb_drop_key(p, k0, k1);
+    return bb_dropout_keep(key.k0, key.k1, key.thresh, index) ? 1 : 0;
+}
+
 // y[r] = sum over the columns of row r (the ``lambda x: x.sum(-1)`` that ends the reference's transformer script,
 // DeepSpeedExamples/pipeline_parallelism/transformer.py:250) and its backward, dx[r, :] = dy[r].  One wave per row,
 // fixed summation order (lane-strided partial sums, then the butterfly).

@@ -242,6 +242,10 @@ static int fill_args(const bb_gemm_desc* d, GemmArgs& g, int64_t& batches, bool&
     g.alpha = d->alpha;
     g.epilogue = d->epilogue; g.act = d->act; g.accumulate = d->accumulate;
     g.c_f32 = (d->c_dtype == BB_F32);
+    BB_REQUIRE(d->dropout_p >= 0.f && d->dropout_p < 1.f, "bb_gemm: dropout_p must be in [0, 1)");
+    BB_REQUIRE(d->dropout_p == 0.f || (batches == 1 && d->epilogue != BB_EPI_DACT && d->epilogue != BB_EPI_MUL && !d->accumulate),
+               "bb_gemm: dropout goes with an unbatched, non-accumulating problem and not with the DACT / MUL epilogues");
+    g.drop = bb_drop_key(d->dropout_p, d->dropout_k0, d->dropout_k1);
     g.tiles_m = g.tiles_n = 0;
     return BB_OK;
 }
@@ -259,7 +263,7 @@ static int colsum_standalone(const bb_gemm_desc* d, void* stream) {
 extern "C" int bb_gemm_strip_stats_supported(const bb_gemm_desc* d) {
     return d && d->dtype == BB_BF16 && d->c_dtype == BB_BF16 && d->layout == BB_NT && d->nb1 <= 1 && d->nb2 <= 1 &&
            d->M >= 128 && d->N >= 64 && d->N % 8 == 0 && d->K >= 128 && d->K % 64 == 0 && d->conv_c == 0 && !d->colsum_out &&
-           !d->bias && d->epilogue == BB_EPI_NONE && d->alpha == 1.0f;
+           !d->bias && d->epilogue == BB_EPI_NONE && d->alpha == 1.0f && d->dropout_p == 0.f;
 }
 extern "C" int64_t bb_strip_stats_workspace(int rows, int cols) { return (int64_t)((rows + 31) / 32) * 3 * cols; }
 
@@ -472,7 +476,7 @@ static int pick_splits(const bb_gemm_desc* descs, int count) {
     for (int i = 0; i < count; ++i) {
         const bb_gemm_desc& d = descs[i];
         if (d.dtype != BB_BF16 || d.c_dtype != BB_F32 || d.layout != descs[0].layout || d.nb1 > 1 || d.nb2 > 1 || d.M <= 0 ||
-            d.N <= 0 || d.colsum_out || d.bias || d.epilogue != BB_EPI_NONE || d.alpha != 1.0f || d.N % 4 != 0 ||
+            d.N <= 0 || d.colsum_out || d.bias || d.epilogue != BB_EPI_NONE || d.alpha != 1.0f || d.N % 4 != 0 || d.dropout_p != 0.f ||
             pick_dma_tile(d.M, d.N, d.K, 1, d.layout) == D_NONE)
             return 0;
         tiles += (int64_t)((d.M + 127) / 128) * ((d.N + 127) / 128);

@@ -17,7 +17,12 @@ struct GemmArgs {
     int tiles_m, tiles_n;
     int conv_h, conv_w, conv_c, conv_row0;  // TN: B is the 3x3 patch matrix of an NHWC tensor (conv_c > 0)
     float* strip_stats;  // [ceil(M / 32)][3][N]: per 32-row strip and output column (pivot, sum (c - pivot), sum (c - pivot)^2)
+    DropKey drop;        // dropout on the product after bias and activation, before the residual (thresh 0: none)
 };
+// keep-and-scale factor of element (m, n) of the [M, N] product
+__device__ __forceinline__ float drop_factor(const GemmArgs& g, int m, int n) {
+    return bb_dropout_keep(g.drop.k0, g.drop.k1, g.drop.thresh, (uint64_t)m * (uint64_t)g.N + (uint64_t)n) ? g.drop.scale : 0.f;
+}
 
 // ---- tile order: consecutive logical tiles land on the same XCD (workgroups are dealt
 // round-robin over the 8 XCDs, each with a private L2), and walk the output in column
@@ -50,20 +55,23 @@ __device__ __forceinline__ void epilogue_elem(const GemmArgs& g, int64_t coff, i
     if (g.bias) v += Elem<T>::load((const T*)g.bias + n);
     const int64_t ci = coff + (int64_t)m * g.ldc + n;
     const int64_t xi = xoff + (int64_t)m * g.ldaux + n;
+    const float keep = g.drop.thresh ? drop_factor(g, m, n) : 1.0f;
     if (g.epilogue == BB_EPI_ACT) {
         if (g.aux_out) Elem<T>::store((T*)g.aux_out + xi, v);
-        v = act_f(v, g.act);
+        v = act_f(v, g.act) * keep;
     } else if (g.epilogue == BB_EPI_DACT) {
         v *= dact_f(Elem<T>::load((const T*)g.aux_in + xi), g.act);
     } else if (g.epilogue == BB_EPI_RESIDUAL) {
-        v += Elem<T>::load((const T*)g.resid + xi);
+        v = v * keep + Elem<T>::load((const T*)g.resid + xi);
     } else if (g.epilogue == BB_EPI_MUL) {
         v *= Elem<T>::load((const T*)g.aux_in + xi);
     } else if (g.epilogue == BB_EPI_ACT_DACT) {
         float a, d;
         act_dact_f(v, g.act, a, d);
-        Elem<T>::store((T*)g.aux_out + xi, d);
-        v = a;
+        Elem<T>::store((T*)g.aux_out + xi, d * keep);
+        v = a * keep;
+    } else {
+        v *= keep;
     }
     if (g.c_f32) {
         float* c = (float*)g.C + ci;
@@ -83,10 +91,19 @@ __device__ __forceinline__ void epilogue_vec8(const GemmArgs& g, int64_t coff, i
 #pragma unroll
         for (int e = 0; e < 8; ++e) v[e] += b[e];
     }
+    float keep[8];
+    if (g.drop.thresh) {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) keep[e] = drop_factor(g, m, n + e);
+    }
     if (g.epilogue == BB_EPI_ACT) {
         if (g.aux_out) store_vec((bf16*)g.aux_out + xi, v);
 #pragma unroll
         for (int e = 0; e < 8; ++e) v[e] = act_f(v[e], g.act);
+        if (g.drop.thresh) {
+#pragma unroll
+            for (int e = 0; e < 8; ++e) v[e] *= keep[e];
+        }
     } else if (g.epilogue == BB_EPI_DACT) {
         float u[8];
         load_vec((const bf16*)g.aux_in + xi, u);
@@ -95,6 +112,10 @@ __device__ __forceinline__ void epilogue_vec8(const GemmArgs& g, int64_t coff, i
     } else if (g.epilogue == BB_EPI_RESIDUAL) {
         float r[8];
         load_vec((const bf16*)g.resid + xi, r);
+        if (g.drop.thresh) {
+#pragma unroll
+            for (int e = 0; e < 8; ++e) v[e] *= keep[e];
+        }
 #pragma unroll
         for (int e = 0; e < 8; ++e) v[e] += r[e];
     } else if (g.epilogue == BB_EPI_MUL) {
@@ -106,7 +127,17 @@ __device__ __forceinline__ void epilogue_vec8(const GemmArgs& g, int64_t coff, i
         float d[8];
 #pragma unroll
         for (int e = 0; e < 8; ++e) act_dact_f(v[e], g.act, v[e], d[e]);
+        if (g.drop.thresh) {
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                v[e] *= keep[e];
+                d[e] *= keep[e];
+            }
+        }
         store_vec((bf16*)g.aux_out + xi, d);
+    } else if (g.drop.thresh) {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) v[e] *= keep[e];
     }
     if (g.c_f32) {
         float* c = (float*)g.C + ci;

@@ -101,6 +101,9 @@ class PipelineEngine:
         # of (stage, micro-batch) touches the same static buffers in every batch, so its ~100
         # launches are captured the second time they occur and launched as one graph afterwards.
         self.use_graphs = bool(use_graphs)
+        if self.use_graphs and any(getattr(l, "dropout", 0) > 0 for ls in model.func_buckets.values() for l in ls):
+            raise PipelineError("use_graphs with dropout: the dropout keys change with every batch and are kernel "
+                                "arguments, a replayed graph would repeat the first batch's masks")
         if self.use_graphs and self.main_stream.cuda_stream == 0:
             raise PipelineError("use_graphs needs the engine built and run under a created stream "
                                 "(torch.cuda.stream(...)): the default stream cannot be captured")
@@ -510,6 +513,10 @@ class PipelineEngine:
         ctx = self.rc_ctx if redundant else self.ctx
         ctx.key_len = self.queue.key_len(buffer_id)
         ctx.redundant = redundant
+        # what names this micro-batch's dropout masks: the same for the redundant forward, the normal forward of
+        # the same layers, a replay and the backward pass (the reference reseeds per layer and micro-batch for
+        # the same purpose, deepspeed/runtime/pipe/module.py:538-545)
+        ctx.dropout_base = (self.module.base_seed, self.global_steps, buffer_id)
         if redundant and self.rc_stream is not None:
             self.rc_stream.wait_event(self._fwd_done[buffer_id])
         kl = ctx.key_len
@@ -583,6 +590,7 @@ class PipelineEngine:
             _, i, x = self._rc_partial
             ctx.key_len = self.queue.key_len(k)
             ctx.redundant = True
+            ctx.dropout_base = (self.module.base_seed, self.global_steps, k)
             out = self.module.forward(x, nxt, slot=k, ctx=ctx, defer=True, layers=(i, i + 1))
             if i + 1 == n_layers:
                 self.pipe_buffers[f"output_{nxt}"][k] = out
@@ -643,6 +651,7 @@ class PipelineEngine:
         if grad is None:
             raise PipelineError(f"BackwardPass({buffer_id}, {stage_id}) without a received gradient")
         self.ctx.key_len = self.queue.key_len(buffer_id)
+        self.ctx.dropout_base = (self.module.base_seed, self.global_steps, buffer_id)
         dst = self._input_grad_store[stage_id][buffer_id]
         kl = self.ctx.key_len
         deferred = self._deferred.get((stage_id, buffer_id), False)

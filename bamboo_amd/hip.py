@@ -7,7 +7,7 @@ own device memory and streams.
 """
 import ctypes
 import os
-from ctypes import POINTER, Structure, byref, c_char_p, c_float, c_int, c_int32, c_int64, c_void_p
+from ctypes import POINTER, Structure, byref, c_char_p, c_float, c_int, c_int32, c_int64, c_uint32, c_uint64, c_void_p
 
 import torch
 
@@ -24,7 +24,7 @@ LN_CODES = {"standard": LN_STANDARD, "annotated": LN_ANNOTATED}
 
 EXPORTS = (
     "bb_version", "bb_last_error", "bb_init", "bb_gemm", "bb_gemm_grouped", "bb_gemm_splitk_workspace", "bb_gemm_grouped_splitk", "bb_gemm_variant", "bb_layernorm_fwd",
-    "bb_layernorm_bwd_workspace", "bb_layernorm_bwd", "bb_layernorm_bwd_static", "bb_colsum_workspace", "bb_colsum_acc", "bb_rowsum_fwd", "bb_rowsum_bwd",
+    "bb_layernorm_bwd_workspace", "bb_layernorm_bwd", "bb_layernorm_bwd_static", "bb_colsum_workspace", "bb_colsum_acc", "bb_rowsum_fwd", "bb_rowsum_bwd", "bb_dropout_apply", "bb_dropout_keep_host",
     "bb_softmax_fwd", "bb_softmax_bwd", "bb_attention_fwd", "bb_attention_bwd", "bb_residual_add", "bb_act_fwd", "bb_bn_workspace", "bb_batchnorm_fwd", "bb_batchnorm_bwd", "bb_patch3x3", "bb_conv3x3_supported", "bb_conv3x3", "bb_gemm_strip_stats_supported", "bb_strip_stats_workspace", "bb_batchnorm_fwd_strips", "bb_mse_workspace", "bb_mse_fwd_bwd", "bb_graph_begin", "bb_graph_end", "bb_graph_launch", "bb_graph_destroy",
     "bb_adam_multi", "bb_cast", "bb_fill_f32",
 )
@@ -49,6 +49,7 @@ class GemmDesc(Structure):
         ("ldaux", c_int64), ("colsum_out", c_void_p), ("colsum_ws", c_void_p),
         ("conv_h", c_int32), ("conv_w", c_int32), ("conv_c", c_int32), ("conv_row0", c_int32),
         ("strip_stats", c_void_p),
+        ("dropout_p", c_float), ("dropout_k0", c_uint32), ("dropout_k1", c_uint32),
     ]
 
 
@@ -93,9 +94,12 @@ def lib():
     L.bb_softmax_fwd.argtypes = [c_int, c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p]
     L.bb_softmax_bwd.argtypes = [c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p]
     L.bb_attention_fwd.argtypes = [c_int] * 6 + [c_void_p, c_void_p, c_void_p, c_int64, c_void_p, c_int64, c_void_p,
-                                   c_void_p, c_void_p]
+                                   c_void_p, c_float, c_uint32, c_uint32, c_void_p]
     L.bb_attention_bwd.argtypes = [c_int] * 6 + [c_void_p, c_void_p, c_void_p, c_int64, c_void_p, c_void_p, c_int64,
-                                   c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_void_p, c_void_p]
+                                   c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_void_p, c_float, c_uint32,
+                                   c_uint32, c_void_p]
+    L.bb_dropout_apply.argtypes = [c_int, c_int64, c_void_p, c_void_p, c_float, c_uint32, c_uint32, c_void_p]
+    L.bb_dropout_keep_host.argtypes = [c_float, c_uint32, c_uint32, c_uint64]
     L.bb_residual_add.argtypes = [c_int, c_int64, c_void_p, c_void_p, c_void_p, c_void_p]
     L.bb_graph_begin.argtypes = [c_void_p]
     L.bb_graph_end.argtypes = [c_void_p, POINTER(c_void_p)]
@@ -161,7 +165,8 @@ def _row_major(t, name):
 
 # ------------------------------------------------------------------------------------- GEMM
 def gemm_desc(layout, A, B, C, *, alpha=1.0, bias=None, epilogue=EPI_NONE, act=ACT_RELU, accumulate=False,
-              aux_in=None, aux_out=None, resid=None, colsum_out=None, colsum_ws=None, conv=None, strip_stats=None):
+              aux_in=None, aux_out=None, resid=None, colsum_out=None, colsum_ws=None, conv=None, strip_stats=None,
+              dropout=None):
     """Descriptor of C = epilogue(alpha * op(A) op(B) [+ bias]) on 2-D row-major views.
     ``conv=(h, w)`` (TN only): B is the NHWC tensor ``[pixels, c]`` whose 3x3 patch matrix ``[pixels, 9c]`` is
     the operand, gathered inside the kernel (weight gradient of a 3x3 convolution)."""
@@ -216,6 +221,9 @@ def gemm_desc(layout, A, B, C, *, alpha=1.0, bias=None, epilogue=EPI_NONE, act=A
     if strip_stats is not None:
         _check_strip_stats(strip_stats, M, N)
         d.strip_stats = strip_stats.data_ptr()
+    if dropout is not None and dropout[0] > 0:
+        # (p, (k0, k1)): dropout on the product after bias / activation, before the residual
+        d.dropout_p, (d.dropout_k0, d.dropout_k1) = dropout[0], dropout[1]
     return d
 
 
@@ -368,17 +376,25 @@ def softmax_bwd(p, dp, stream=None):
           "bb_softmax_bwd")
 
 
-def attention_fwd(qkv, out, lse, batch, heads, seq, mask, key_len=None, stream=None):
-    """qkv: [batch*seq, 3*heads*64] (Q | K | V thirds), out: [batch*seq, heads*64], lse: fp32 [batch, heads, seq]."""
+def _drop_args(dropout):
+    if dropout is None or dropout[0] <= 0:
+        return 0.0, 0, 0
+    return float(dropout[0]), int(dropout[1][0]), int(dropout[1][1])
+
+
+def attention_fwd(qkv, out, lse, batch, heads, seq, mask, key_len=None, stream=None, dropout=None):
+    """qkv: [batch*seq, 3*heads*64] (Q | K | V thirds), out: [batch*seq, heads*64], lse: fp32 [batch, heads, seq].
+    ``dropout=(p, (k0, k1))``: dropout on the probabilities with the decisions of that key."""
     h = heads * 64
     es = qkv.element_size()
     q = qkv.data_ptr()
     check(lib().bb_attention_fwd(dtype_code(qkv.dtype), mask, batch, heads, seq, qkv.shape[1] // (3 * heads),
                                  c_void_p(q), c_void_p(q + h * es), c_void_p(q + 2 * h * es), qkv.stride(0), _ptr(out),
-                                 out.stride(0), _ptr(lse), _ptr(key_len), stream_ptr(stream)), "bb_attention_fwd")
+                                 out.stride(0), _ptr(lse), _ptr(key_len), *_drop_args(dropout), stream_ptr(stream)),
+          "bb_attention_fwd")
 
 
-def attention_bwd(qkv, out, d_out, lse, delta, d_qkv, batch, heads, seq, mask, key_len=None, stream=None):
+def attention_bwd(qkv, out, d_out, lse, delta, d_qkv, batch, heads, seq, mask, key_len=None, stream=None, dropout=None):
     h = heads * 64
     es = qkv.element_size()
     q, dq = qkv.data_ptr(), d_qkv.data_ptr()
@@ -386,7 +402,35 @@ def attention_bwd(qkv, out, d_out, lse, delta, d_qkv, batch, heads, seq, mask, k
                                  c_void_p(q), c_void_p(q + h * es), c_void_p(q + 2 * h * es), qkv.stride(0), _ptr(out),
                                  _ptr(d_out), out.stride(0), _ptr(lse), _ptr(delta), c_void_p(dq),
                                  c_void_p(dq + h * es), c_void_p(dq + 2 * h * es), d_qkv.stride(0), _ptr(key_len),
-                                 stream_ptr(stream)), "bb_attention_bwd")
+                                 *_drop_args(dropout), stream_ptr(stream)), "bb_attention_bwd")
+
+
+def dropout_apply(src, dst, p, key, stream=None):
+    """dst = src / (1 - p) where kept, 0 elsewhere; element i of the contiguous tensor is kept when
+    ``dropout_keep(p, key, i)``.  The same call on a gradient is the backward."""
+    if not (src.is_contiguous() and dst.is_contiguous()) or src.shape != dst.shape or src.dtype != dst.dtype:
+        raise HipKernelError("dropout_apply: src and dst must be contiguous tensors of one shape and dtype")
+    check(lib().bb_dropout_apply(dtype_code(src.dtype), src.numel(), _ptr(src), _ptr(dst), float(p), int(key[0]), int(key[1]),
+                                 stream_ptr(stream)), "bb_dropout_apply")
+
+
+def dropout_keep(p, key, index):
+    """The decision for one element, evaluated on the host (no GPU needed)."""
+    return bool(lib().bb_dropout_keep_host(float(p), int(key[0]), int(key[1]), int(index)))
+
+
+def dropout_key(base_seed, step, micro_batch, layer_idx, site):
+    """Two 32-bit key words from what identifies one dropout mask: the model's base seed, the batch counter, the
+    micro-batch, the layer (global index) and the dropout site inside the layer (splitmix64 over the five)."""
+    z = 0x9E3779B97F4A7C15
+    for v in (base_seed, step, micro_batch, layer_idx, site):
+        z = (z + (int(v) & 0xFFFFFFFFFFFFFFFF) * 0xBF58476D1CE4E5B9 + 0x9E3779B97F4A7C15) & 0xFFFFFFFFFFFFFFFF
+        z ^= z >> 30
+        z = (z * 0xBF58476D1CE4E5B9) & 0xFFFFFFFFFFFFFFFF
+        z ^= z >> 27
+        z = (z * 0x94D049BB133111EB) & 0xFFFFFFFFFFFFFFFF
+        z ^= z >> 31
+    return z & 0xFFFFFFFF, z >> 32
 
 
 def residual_add(a, b, out, stream=None):

@@ -33,6 +33,9 @@ class StageContext:
         self.scratch = {}
         self.key_len = None
         self.workspace = None
+        # (base seed, batch counter, micro-batch): with a layer's index and the site inside it this names a dropout
+        # mask; set per forward / backward call by whoever drives the stage
+        self.dropout_base = None
         self.redundant = False   # set per forward call: a redundant forward must not touch running statistics
         # set per forward call: leave out what only a backward pass reads (a redundant forward's stash is used
         # by a backward pass only after a failover); ``deferred`` tells that backward pass to produce it first
@@ -63,9 +66,16 @@ class TransformerLayer:
 
     activation: ``relu`` (reference) or ``gelu_tanh``; ln: ``annotated`` (reference: unbiased
     std, eps added to the std) or ``standard``; mask: ``none`` (reference scripts), ``causal``
-    or ``key_padding``.  Dropout is not implemented (p = 0): redundant and normal forward must
-    agree bit for bit.
+    or ``key_padding``.
+
+    dropout: probability of the reference's four ``nn.Dropout`` sites (attention probabilities, the two sublayer
+    outputs, the feed-forward's hidden activation; transformer.py:98-103,125-126,154-158).  No mask is stored: each
+    decision is a pure function of (base seed, batch counter, micro-batch, layer, site, element), evaluated inside
+    the attention kernels and the GEMM epilogues, so the redundant forward of a layer, its normal forward and its
+    backward pass agree bit for bit.
     """
+
+    SITE_ATTENTION, SITE_SUBLAYER0, SITE_FFN, SITE_SUBLAYER1 = 0, 1, 2, 3
 
     # parameter registration order of the reference's ``EncoderLayer`` (self_attn, feed_forward, sublayer:
     # transformer.py:161-168): the order of its ``state_dict()``, hence of the layer wire format
@@ -76,9 +86,13 @@ class TransformerLayer:
         "sublayer.0.norm.a_2", "sublayer.0.norm.b_2", "sublayer.1.norm.a_2", "sublayer.1.norm.b_2")
 
     def __init__(self, hidden, heads, ffn, activation="relu", ln="annotated", mask="none", ln_eps=None,
-                 init_std=0.02):
+                 init_std=0.02, dropout=0.0):
         if hidden % heads:
             raise ValueError("hidden must be divisible by heads")
+        if not 0.0 <= dropout < 1.0:
+            raise ValueError("dropout must be in [0, 1)")
+        self.dropout = float(dropout)
+        self.layer_idx = None     # global index, set when the layer is bound to a stage's arenas
         self.hidden, self.heads, self.ffn = hidden, heads, ffn
         self.head_dim = hidden // heads
         if activation not in hip.ACT_CODES or ln not in hip.LN_CODES or mask not in hip.MASK_CODES:
@@ -174,7 +188,25 @@ class TransformerLayer:
         dt = ctx.dtype
         attn = ("attn_delta", (ctx.batch, self.heads, ctx.seq), torch.float32) if self.fused_attention(ctx) else \
             ("d_prob", (ctx.batch, self.heads, ctx.seq, ctx.seq), dt)
-        return [("d_ffn", (R, f), dt), ("d_h0", (R, h), dt), ("d_h1", (R, h), dt), ("d_qkv", (R, 3 * h), dt), attn]
+        specs = [("d_ffn", (R, f), dt), ("d_h0", (R, h), dt), ("d_h1", (R, h), dt), ("d_qkv", (R, 3 * h), dt), attn]
+        if self.dropout > 0:
+            # the gradients behind the two sublayer dropouts: the weight gradients read them at the end of the layer
+            specs += [("d_drop0", (R, h), dt), ("d_drop1", (R, h), dt)]
+        return specs + self.forward_scratch_specs(ctx)
+
+    def forward_scratch_specs(self, ctx):
+        if self.dropout > 0 and not self.fused_attention(ctx):
+            return [("prob_drop", (ctx.batch, self.heads, ctx.seq, ctx.seq), ctx.dtype)]   # dropped-out probabilities
+        return []
+
+    def _drop(self, ctx, site):
+        """``(p, key)`` of one dropout site for the call in progress, or None."""
+        if self.dropout <= 0:
+            return None
+        if ctx.dropout_base is None or self.layer_idx is None:
+            raise hip.HipKernelError("a layer with dropout needs ctx.dropout_base = (base seed, batch counter, micro-batch) "
+                                     "and its layer index")
+        return self.dropout, hip.dropout_key(*ctx.dropout_base, self.layer_idx, site)
 
     def workspace_elems(self):
         n = max(self.hidden * 3, self.ffn)
@@ -191,9 +223,10 @@ class TransformerLayer:
 
     def _attention_fwd(self, st, ctx):
         h, d, s = self.hidden, self.head_dim, ctx.seq
+        drop = self._drop(ctx, self.SITE_ATTENTION)
         if self.fused_attention(ctx):
             hip.attention_fwd(st["qkv"], st["ctx"], st["lse"], ctx.batch, self.heads, s, hip.MASK_CODES[self.mask],
-                              ctx.key_len, stream=ctx.stream)
+                              ctx.key_len, stream=ctx.stream, dropout=drop)
             return
         es = st["qkv"].element_size()
         q = st["qkv"].data_ptr()
@@ -204,16 +237,22 @@ class TransformerLayer:
         self._heads_gemm(ctx, hip.NT, s, s, d, q, 3 * h, head_in, k, 3 * h, head_in,
                          prob.data_ptr(), s, (self.heads * s * s, s * s), alpha=1.0 / math.sqrt(d))
         hip.softmax_fwd(prob, hip.MASK_CODES[self.mask], ctx.key_len, stream=ctx.stream)
+        if drop is not None:
+            # the stash keeps the probabilities themselves (the softmax backward needs them); V meets the dropped-out copy
+            kept = ctx.buf("prob_drop", tuple(prob.shape))
+            hip.dropout_apply(prob, kept, drop[0], drop[1], stream=ctx.stream)
+            prob = kept
         # ctx = P V, written straight into the [rows, hidden] layout (head j -> columns j*d..)
         self._heads_gemm(ctx, hip.NN, s, d, s, prob.data_ptr(), s, (self.heads * s * s, s * s), v, 3 * h, head_in,
                          st["ctx"].data_ptr(), h, (s * h, d))
 
     def _attention_bwd(self, d_ctx, d_qkv, st, ctx):
         h, d, s = self.hidden, self.head_dim, ctx.seq
+        drop = self._drop(ctx, self.SITE_ATTENTION)
         if self.fused_attention(ctx):
             delta = ctx.buf("attn_delta", (ctx.batch, self.heads, s))
             hip.attention_bwd(st["qkv"], st["ctx"], d_ctx, st["lse"], delta, d_qkv, ctx.batch, self.heads, s,
-                              hip.MASK_CODES[self.mask], ctx.key_len, stream=ctx.stream)
+                              hip.MASK_CODES[self.mask], ctx.key_len, stream=ctx.stream, dropout=drop)
             return
         es = st["qkv"].element_size()
         q = st["qkv"].data_ptr()
@@ -224,12 +263,18 @@ class TransformerLayer:
         prob = st["prob"]
         d_prob = ctx.buf("d_prob", tuple(prob.shape))
         scale = 1.0 / math.sqrt(d)
-        # dV = P^T dctx
-        self._heads_gemm(ctx, hip.TN, s, d, s, prob.data_ptr(), s, head_p, d_ctx.data_ptr(), h, head_ctx,
+        # dV = P~^T dctx, P~ = what multiplied V in the forward (the dropped-out probabilities, made again)
+        p_fwd = prob
+        if drop is not None:
+            p_fwd = ctx.buf("prob_drop", tuple(prob.shape))
+            hip.dropout_apply(prob, p_fwd, drop[0], drop[1], stream=ctx.stream)
+        self._heads_gemm(ctx, hip.TN, s, d, s, p_fwd.data_ptr(), s, head_p, d_ctx.data_ptr(), h, head_ctx,
                          dv, 3 * h, head_in)
-        # dP = dctx V^T ; dS = P * (dP - rowsum(dP * P))
+        # dP~ = dctx V^T ; dP = dropout'(dP~) ; dS = P * (dP - rowsum(dP * P))
         self._heads_gemm(ctx, hip.NT, s, s, d, d_ctx.data_ptr(), h, head_ctx, v, 3 * h, head_in,
                          d_prob.data_ptr(), s, head_p)
+        if drop is not None:
+            hip.dropout_apply(d_prob, d_prob, drop[0], drop[1], stream=ctx.stream)
         hip.softmax_bwd(prob, d_prob, stream=ctx.stream)
         # dQ = dS K / sqrt(d) ; dK = dS^T Q / sqrt(d)
         self._heads_gemm(ctx, hip.NN, s, d, s, d_prob.data_ptr(), s, head_p, k, 3 * h, head_in,
@@ -248,7 +293,7 @@ class TransformerLayer:
         hip.gemm(hip.NT, st["n1"], w["qkv.weight"], st["qkv"], bias=w["qkv.bias"], stream=sm)
         self._attention_fwd(st, ctx)
         hip.gemm(hip.NT, st["ctx"], w["self_attn.linears.3.weight"], st["x1"], bias=w["self_attn.linears.3.bias"],
-                 epilogue=hip.EPI_RESIDUAL, resid=x, stream=sm)
+                 epilogue=hip.EPI_RESIDUAL, resid=x, dropout=self._drop(ctx, self.SITE_SUBLAYER0), stream=sm)
         hip.layernorm_fwd(st["x1"], w["sublayer.1.norm.a_2"], w["sublayer.1.norm.b_2"], st["n2"], st["mean2"],
                           st["rinv2"], kind, self.eps, stream=sm)
         # activation and its derivative (kept for the backward pass, which then multiplies instead of
@@ -258,17 +303,20 @@ class TransformerLayer:
         if ctx.defer:
             # act' is read by the backward pass only: a forward that most likely has none writes act alone
             hip.gemm(hip.NT, st["n2"], w["feed_forward.w_1.weight"], st["act"], bias=w["feed_forward.w_1.bias"],
-                     epilogue=hip.EPI_ACT, act=act, stream=sm)
+                     epilogue=hip.EPI_ACT, act=act, dropout=self._drop(ctx, self.SITE_FFN), stream=sm)
         else:
-            self._ffn1(st, sm)
+            self._ffn1(st, ctx)
         hip.gemm(hip.NT, st["act"], w["feed_forward.w_2.weight"], st["out"], bias=w["feed_forward.w_2.bias"],
-                 epilogue=hip.EPI_RESIDUAL, resid=st["x1"], stream=sm)
+                 epilogue=hip.EPI_RESIDUAL, resid=st["x1"], dropout=self._drop(ctx, self.SITE_SUBLAYER1), stream=sm)
         return st["out"]
 
-    def _ffn1(self, st, sm):
+    def _ffn1(self, st, ctx):
+        """act and act' of the feed-forward's hidden layer; under dropout both carry the keep factor, so the backward
+        pass multiplies by the stored derivative as before."""
         w = self.w
         hip.gemm(hip.NT, st["n2"], w["feed_forward.w_1.weight"], st["act"], bias=w["feed_forward.w_1.bias"],
-                 epilogue=hip.EPI_ACT_DACT, act=hip.ACT_CODES[self.activation], aux_out=st["dact"], stream=sm)
+                 epilogue=hip.EPI_ACT_DACT, act=hip.ACT_CODES[self.activation], aux_out=st["dact"],
+                 dropout=self._drop(ctx, self.SITE_FFN), stream=ctx.stream)
 
     def backward(self, d_out, d_x, st, ctx):
         """d_out: gradient of st['out']; writes the input gradient into d_x; parameter
@@ -285,18 +333,27 @@ class TransformerLayer:
         wgrad = lambda dy, x, name: wgrads.append(hip.gemm_desc(
             hip.TN, dy, x, g[name], accumulate=True, colsum_out=g[name[:-len("weight")] + "bias"], colsum_ws=ws))
         if ctx.deferred:
-            self._ffn1(st, sm)   # the forward of this stash left act' out: same kernel, same bits as a normal forward
+            self._ffn1(st, ctx)   # the forward of this stash left act' out: same kernel, same bits as a normal forward
+        # the gradient behind a sublayer's dropout feeds the sublayer; the residual branch takes the one in front of it
+        d_ff2, d_proj = d_out, None
+        if self.dropout > 0:
+            d_ff2 = ctx.buf("d_drop1", (R, h))
+            hip.dropout_apply(d_out, d_ff2, *self._drop(ctx, self.SITE_SUBLAYER1), stream=sm)
         # feed-forward
-        wgrad(d_out, st["act"], "feed_forward.w_2.weight")
-        hip.gemm(hip.NN, d_out, w["feed_forward.w_2.weight"], d_ffn, epilogue=hip.EPI_MUL, aux_in=st["dact"], stream=sm)
+        wgrad(d_ff2, st["act"], "feed_forward.w_2.weight")
+        hip.gemm(hip.NN, d_ff2, w["feed_forward.w_2.weight"], d_ffn, epilogue=hip.EPI_MUL, aux_in=st["dact"], stream=sm)
         wgrad(d_ffn, st["n2"], "feed_forward.w_1.weight")
         hip.gemm(hip.NN, d_ffn, w["feed_forward.w_1.weight"], d_h0, stream=sm)
         # d_x1 = d_out + LN2'(d_n2)
         hip.layernorm_bwd(st["x1"], w["sublayer.1.norm.a_2"], st["mean2"], st["rinv2"], d_h0, d_out, d_h1,
                           g["sublayer.1.norm.a_2"], g["sublayer.1.norm.b_2"], ws, kind, self.eps, stream=sm)
         # attention output projection
-        wgrad(d_h1, st["ctx"], "self_attn.linears.3.weight")
-        hip.gemm(hip.NN, d_h1, w["self_attn.linears.3.weight"], d_h0, stream=sm)
+        d_proj = d_h1
+        if self.dropout > 0:
+            d_proj = ctx.buf("d_drop0", (R, h))
+            hip.dropout_apply(d_h1, d_proj, *self._drop(ctx, self.SITE_SUBLAYER0), stream=sm)
+        wgrad(d_proj, st["ctx"], "self_attn.linears.3.weight")
+        hip.gemm(hip.NN, d_proj, w["self_attn.linears.3.weight"], d_h0, stream=sm)
         self._attention_bwd(d_h0, d_qkv, st, ctx)
         # QKV projection
         wgrad(d_qkv, st["n1"], "qkv.weight")
@@ -304,7 +361,7 @@ class TransformerLayer:
         # d_x0 = d_x1 + LN1'(d_n1)
         hip.layernorm_bwd(st["x0"], w["sublayer.0.norm.a_2"], st["mean1"], st["rinv1"], d_h0, d_h1, d_x,
                           g["sublayer.0.norm.a_2"], g["sublayer.0.norm.b_2"], ws, kind, self.eps, stream=sm)
-        # d_out, d_ffn, d_h1 and d_qkv still hold the four output gradients here
+        # d_out (d_drop1), d_ffn, d_h1 (d_drop0) and d_qkv still hold the four output gradients here
         hip.gemm_grouped(wgrads, stream=sm)
         return d_x
 

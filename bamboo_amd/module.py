@@ -78,6 +78,7 @@ class StageParams:
         for li, layer in enumerate(layers):
             prefix = f"{first_layer_idx + li}."
             names = [k[len(prefix):] for k in self.index if k.startswith(prefix)]
+            layer.layer_idx = first_layer_idx + li
             layer.bind({n: self.view(self.compute, prefix + n) for n in names},
                        {n: self.view(self.grad, prefix + n) for n in names})
 

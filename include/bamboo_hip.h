@@ -116,6 +116,13 @@ typedef struct bb_gemm_desc {
      * >= bb_strip_stats_workspace(M, N) floats.  bb_batchnorm_fwd_strips turns them into the batch statistics
      * of nn.BatchNorm2d without reading C again (resnet.py:55-62: every convolution feeds a BatchNorm).    */
     float* strip_stats;
+    /* Dropout on the product, after bias and activation and before the residual is added
+     * (nn.Dropout of SublayerConnection and PositionwiseFeedForward, transformer.py:98-103,154-158):
+     * element (m, n) is kept and scaled by 1 / (1 - dropout_p) when bb_dropout_keep(key, m * N + n) says so
+     * (the decision function of bb_dropout_apply), else zero; with BB_EPI_ACT_DACT the stored derivative gets
+     * the same factor.  dropout_p = 0: none.  Not with BB_EPI_DACT / BB_EPI_MUL, not batched.            */
+    float dropout_p;
+    uint32_t dropout_k0, dropout_k1;
 } bb_gemm_desc;
 
 /* library ------------------------------------------------------------------------------ */
@@ -182,6 +189,16 @@ int bb_layernorm_bwd_static(int dtype, int kind, int rows, int cols, float eps, 
 int bb_rowsum_fwd(int dtype, int rows, int cols, const void* x, void* y, void* stream);
 int bb_rowsum_bwd(int dtype, int rows, int cols, const void* dy, void* dx, void* stream);
 
+/* dst[i] = src[i] / (1 - p) where element i is kept, else 0 (F.dropout in training mode with the mask of
+ * key (k0, k1)): i counts the n elements of a contiguous tensor.  The decision for element i is a pure
+ * function of (k0, k1, i) -- see bb_dropout_keep_host -- shared by the GEMM epilogues (i = m * N + n) and the
+ * attention kernels (i = ((batch * heads + head) * seq + query) * seq + key).  src == dst allowed.
+ * The backward of dropout is the same call on the gradient.                                         */
+int bb_dropout_apply(int dtype, int64_t n, const void* src, void* dst, float p, uint32_t k0, uint32_t k1,
+                     void* stream);
+/* The decision itself, on the host (1 = keep): for tests and for callers that need the mask. */
+int bb_dropout_keep_host(float p, uint32_t k0, uint32_t k1, uint64_t index);
+
 /* Column sums of a [rows, cols] matrix accumulated into an fp32 vector: the bias gradient of
  * nn.Linear (autograd of transformer.py:136-146,158).  workspace: fp32, at least
  * bb_colsum_workspace(cols) elements.                                                     */
@@ -203,17 +220,20 @@ int bb_softmax_bwd(int dtype, int batch, int heads, int sq, int sk, const void* 
  * q, k, v point at head 0 of batch 0; rows are tokens (batch-major), head j occupies columns
  * j*64.. of each pointer, row stride ld_qkv (the three pointers may alias one [rows, 3h] buffer).
  * out: [rows, heads*64] with row stride ld_out.  lse: fp32 [batch, heads, seq] log-sum-exp (base 2,
- * scaled scores) kept for the backward.                                                     */
+ * scaled scores) kept for the backward.
+ * dropout_p > 0: dropout on the probabilities (transformer.py:125-126), out = (P o mask / (1 - p)) V with the
+ * decisions of key (dropout_k0, dropout_k1) at element ((batch * heads + head) * seq + query) * seq + key;
+ * the backward is given the same p and key and makes the same decisions again.                          */
 int bb_attention_fwd(int dtype, int mask, int batch, int heads, int seq, int head_dim, const void* q,
                      const void* k, const void* v, int64_t ld_qkv, void* out, int64_t ld_out, float* lse,
-                     const int32_t* key_len, void* stream);
+                     const int32_t* key_len, float dropout_p, uint32_t dropout_k0, uint32_t dropout_k1, void* stream);
 /* Backward of bb_attention_fwd: dq, dk, dv (same addressing as q, k, v with row stride ld_dqkv)
  * from d_out, the forward's out and lse.  delta: fp32 workspace [batch, heads, seq].
  * Deterministic (no atomics): dK/dV and dQ are produced by two passes over the score tiles. */
 int bb_attention_bwd(int dtype, int mask, int batch, int heads, int seq, int head_dim, const void* q,
                      const void* k, const void* v, int64_t ld_qkv, const void* out, const void* d_out,
                      int64_t ld_out, const float* lse, float* delta, void* dq, void* dk, void* dv,
-                     int64_t ld_dqkv, const int32_t* key_len, void* stream);
+                     int64_t ld_dqkv, const int32_t* key_len, float dropout_p, uint32_t dropout_k0, uint32_t dropout_k1, void* stream);
 
 /* out = a + b, elementwise (SublayerConnection residual, transformer.py:103).             */
 int bb_residual_add(int dtype, int64_t n, const void* a, const void* b, void* out,

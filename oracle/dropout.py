@@ -1,0 +1,60 @@
+"""Dropout masks as pure functions of a key and an element index (TEST ORACLE, numpy).
+
+The reference applies ``nn.Dropout`` at four places of an encoder layer (DeepSpeedExamples/pipeline_parallelism/
+transformer.py: attention probabilities :125-126, the two ``SublayerConnection`` outputs :98-103, the feed-forward's
+hidden activation :154-158) and reseeds torch's generator per layer and micro-batch so that a forward can be repeated
+(deepspeed/runtime/pipe/module.py:538-545).  Which elements torch's generator drops is not part of the reference
+(it depends on the device kernel's launch shape): **parity unpinned** for the mask bits themselves.  What is
+fixed, and restated here, is the arithmetic -- kept elements are scaled by 1 / (1 - p), dropped ones are zero, an
+element is kept with probability 1 - p -- and, for this build, the decision function the HIP kernels evaluate
+(two rounds of a 32-bit xorshift-multiply finalizer over (index, key)), restated with numpy integer arithmetic and
+pinned against the library's own host-side evaluation of it (tests/test_dropout.py)."""
+import numpy as np
+
+M64 = (1 << 64) - 1
+
+# the four dropout sites of an encoder layer
+SITE_ATTENTION, SITE_SUBLAYER0, SITE_FFN, SITE_SUBLAYER1 = 0, 1, 2, 3
+
+
+def key(base_seed, step, micro_batch, layer_idx, site):
+    """(k0, k1): splitmix64 chained over what identifies one mask."""
+    z = 0x9E3779B97F4A7C15
+    for v in (base_seed, step, micro_batch, layer_idx, site):
+        z = (z + (int(v) & M64) * 0xBF58476D1CE4E5B9 + 0x9E3779B97F4A7C15) & M64
+        z ^= z >> 30
+        z = (z * 0xBF58476D1CE4E5B9) & M64
+        z ^= z >> 27
+        z = (z * 0x94D049BB133111EB) & M64
+        z ^= z >> 31
+    return z & 0xFFFFFFFF, z >> 32
+
+
+def _mix32(x):
+    x = x.astype(np.uint64)
+    x ^= x >> np.uint64(16)
+    x = (x * np.uint64(0x7FEB352D)) & np.uint64(0xFFFFFFFF)
+    x ^= x >> np.uint64(15)
+    x = (x * np.uint64(0x846CA68B)) & np.uint64(0xFFFFFFFF)
+    x ^= x >> np.uint64(16)
+    return x
+
+
+def threshold(p):
+    t = float(np.float32(p)) * 4294967296.0
+    return 4294967295 if t >= 4294967295.0 else int(t + 0.5)
+
+
+def keep(p, k, index):
+    """Boolean array: element ``index`` (array of non-negative ints) is kept under probability-to-drop ``p``."""
+    idx = np.asarray(index, dtype=np.uint64)
+    lo, hi = idx & np.uint64(0xFFFFFFFF), idx >> np.uint64(32)
+    x = _mix32(lo ^ np.uint64(k[0]))
+    x = _mix32((x + (hi ^ np.uint64(k[1]))) & np.uint64(0xFFFFFFFF))
+    return x >= np.uint64(threshold(p))
+
+
+def mask(p, k, shape):
+    """0/1 float64 mask of a contiguous tensor of ``shape`` (element index = row-major position)."""
+    n = int(np.prod(shape))
+    return keep(p, k, np.arange(n, dtype=np.uint64)).reshape(shape).astype(np.float64)

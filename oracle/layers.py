@@ -42,6 +42,7 @@ class TransformerCfg:
     ln: str = "annotated"         # annotated (reference) | standard
     mask: str = "none"            # none | causal | key_padding
     ln_eps: float = None
+    dropout: float = 0.0          # the reference scripts run 0.1 (transformer.py:196); masks are handed in explicitly
 
     @property
     def eps(self):
@@ -111,7 +112,14 @@ def build_mask(cfg, batch, seq, key_lens=None):
     raise ValueError(cfg.mask)
 
 
-def attention(x, p, cfg, key_lens=None):
+def drop(x, mask, p_drop):
+    """nn.Dropout in training mode with a given 0/1 mask: kept elements scaled by 1 / (1 - p)."""
+    if mask is None:
+        return x
+    return x * mask.to(x.dtype).view_as(x) / (1.0 - p_drop)
+
+
+def attention(x, p, cfg, key_lens=None, prob_mask=None):
     b, s, h = x.shape
     a, d = cfg.heads, cfg.hidden // cfg.heads
     lin = lambda i, t: F.linear(t, p[f"self_attn.linears.{i}.weight"], p[f"self_attn.linears.{i}.bias"])
@@ -120,21 +128,34 @@ def attention(x, p, cfg, key_lens=None):
     mask = build_mask(cfg, b, s, key_lens)
     if mask is not None:
         scores = scores.masked_fill(~mask, -1e9)
-    prob = F.softmax(scores, dim=-1)
+    prob = drop(F.softmax(scores, dim=-1), prob_mask, cfg.dropout)          # transformer.py:125-126
     ctx = torch.matmul(prob, v).transpose(1, 2).contiguous().view(b, s, h)
     return lin(3, ctx)
 
 
-def feed_forward(x, p, cfg, relu_mask=None):
+def feed_forward(x, p, cfg, relu_mask=None, hidden_mask=None):
     u = F.linear(x, p["feed_forward.w_1.weight"], p["feed_forward.w_1.bias"])
-    return F.linear(activation(u, cfg.activation, relu_mask), p["feed_forward.w_2.weight"], p["feed_forward.w_2.bias"])
+    a = drop(activation(u, cfg.activation, relu_mask), hidden_mask, cfg.dropout)    # transformer.py:158
+    return F.linear(a, p["feed_forward.w_2.weight"], p["feed_forward.w_2.bias"])
 
 
-def transformer_layer(x, p, cfg, key_lens=None, relu_mask=None):
+def transformer_layer(x, p, cfg, key_lens=None, relu_mask=None, drop_masks=None):
+    """``drop_masks``: {site: 0/1 tensor} for the layer's four dropout sites (oracle.dropout.SITE_*): attention
+    probabilities [b, heads, s, s], sublayer outputs [b, s, h], feed-forward hidden [b, s, ffn]."""
+    dm = drop_masks or {}
     n1 = layer_norm(x, p["sublayer.0.norm.a_2"], p["sublayer.0.norm.b_2"], cfg.ln, cfg.eps)
-    x = x + attention(n1, p, cfg, key_lens)
+    x = x + drop(attention(n1, p, cfg, key_lens, dm.get(0)), dm.get(1), cfg.dropout)      # transformer.py:103
     n2 = layer_norm(x, p["sublayer.1.norm.a_2"], p["sublayer.1.norm.b_2"], cfg.ln, cfg.eps)
-    return x + feed_forward(n2, p, cfg, relu_mask)
+    return x + drop(feed_forward(n2, p, cfg, relu_mask, dm.get(2)), dm.get(3), cfg.dropout)
+
+
+def layer_drop_masks(cfg, base_seed, step, micro_batch, layer_idx, batch, seq):
+    """The four masks of one layer forward under this build's decision function (oracle.dropout)."""
+    from . import dropout as od
+    shapes = {od.SITE_ATTENTION: (batch, cfg.heads, seq, seq), od.SITE_SUBLAYER0: (batch, seq, cfg.hidden),
+              od.SITE_FFN: (batch, seq, cfg.ffn), od.SITE_SUBLAYER1: (batch, seq, cfg.hidden)}
+    return {site: torch.from_numpy(od.mask(cfg.dropout, od.key(base_seed, step, micro_batch, layer_idx, site), shape))
+            for site, shape in shapes.items()}
 
 
 def script_tail(x, p, kind="annotated", eps=1e-6):

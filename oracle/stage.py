@@ -103,7 +103,7 @@ class OracleStage:
             layers.append({k: v.requires_grad_(True) for k, v in p.items()})
         self.params[stage] = layers
 
-    def forward(self, x, stage, key_lens=None, relu_masks=None):
+    def forward(self, x, stage, key_lens=None, relu_masks=None, drop_id=None):
         """``relu_masks``: per layer of the stage, the ReLU decisions to use (``oracle.layers.activation``):
         one tensor [batch, seq, ffn] per transformer layer, three NCHW tensors per bottleneck block."""
         masks = relu_masks if relu_masks is not None else [None] * len(self.params[stage])
@@ -115,11 +115,17 @@ class OracleStage:
             for p, m in zip(self.params[stage], masks):
                 y = olayers.bottleneck(y, p, self.cfg, m)
             return y.permute(0, 2, 3, 1).reshape(b, hw, c)
-        for p, m in zip(self.params[stage], masks):
+        for li, (p, m) in enumerate(zip(self.params[stage], masks)):
             if set(p) == {"a_2", "b_2"}:
                 x = olayers.script_tail(x, p, self.cfg.ln, self.cfg.eps)
             elif p:
-                x = olayers.transformer_layer(x, p, self.cfg, key_lens, m)
+                dm = None
+                if getattr(self.cfg, "dropout", 0.0) > 0 and drop_id is not None:
+                    # drop_id = (step, micro-batch): with the model's base seed and the layer's global index it names
+                    # the masks, the same for a redundant forward, a normal one and a replay
+                    dm = olayers.layer_drop_masks(self.cfg, self.base_seed, drop_id[0], drop_id[1], self.parts[stage] + li,
+                                                  x.shape[0], x.shape[1])
+                x = olayers.transformer_layer(x, p, self.cfg, key_lens, m, dm)
         return x
 
     def named_grads(self, stage):
@@ -172,7 +178,7 @@ class OracleStage:
                 peer.loss = peer.loss + loss.detach()
             return
         kl = None if peer.key_lens is None else peer.key_lens[k]
-        out = self.forward(bufs["in"][(s, k)], s, kl, peer.relu_masks.get((s, k)))
+        out = self.forward(bufs["in"][(s, k)], s, kl, peer.relu_masks.get((s, k)), (self.step_count, k))
         bufs["out"][(s, k)] = out
         if s == self.S - 1 and peer.labels is not None and s in self.stage_ids:
             # last stage: loss_model(outputs, labels), summed into total_loss (engine.py:1649-1663); counted

@@ -66,11 +66,15 @@ def test_what_is_not_recognised_is_refused():
         PipelineModule([torch.nn.Linear(8, 8)], num_stages=1, stage_id=0, dtype=torch.float32, device="cpu")
     with pytest.raises(PipelineError, match="bare callable"):
         PipelineModule([RefEncoderLayer(32, 4, 64, 0.0), lambda x: x * 2], num_stages=1, stage_id=0, dtype=torch.float32, device="cpu")
-    with pytest.raises(PipelineError, match="dropout"):
-        PipelineModule([RefEncoderLayer(32, 4, 64, 0.1)], num_stages=1, stage_id=0, dtype=torch.float32, device="cpu")
-    # the same module in eval() mode applies no dropout: taken
+    # dropout: the module's probability in training mode, none in eval() mode; mixed probabilities are refused
+    taken = PipelineModule([RefEncoderLayer(32, 4, 64, 0.1)], num_stages=1, stage_id=0, dtype=torch.float32, device="cpu").func_buckets[0][0]
+    assert isinstance(taken, TransformerLayer) and abs(taken.dropout - 0.1) < 1e-7 and taken.layer_idx == 0
     m = RefEncoderLayer(32, 4, 64, 0.1).eval()
-    assert isinstance(PipelineModule([m], num_stages=1, stage_id=0, dtype=torch.float32, device="cpu").func_buckets[0][0], TransformerLayer)
+    assert PipelineModule([m], num_stages=1, stage_id=0, dtype=torch.float32, device="cpu").func_buckets[0][0].dropout == 0.0
+    mixed = RefEncoderLayer(32, 4, 64, 0.1)
+    mixed.feed_forward.dropout.p = 0.3
+    with pytest.raises(PipelineError, match="different dropout"):
+        PipelineModule([mixed], num_stages=1, stage_id=0, dtype=torch.float32, device="cpu")
     with pytest.raises(PipelineError, match="MSELoss"):
         PipelineModule([m], num_stages=1, stage_id=0, loss_fn=torch.nn.L1Loss(), dtype=torch.float32, device="cpu")
 

@@ -180,21 +180,22 @@ def test_rc_forward_bit_exact_and_rc_neutral(hiplib, rc_stream):
         assert torch.equal(normal, keep[f"output_{sid + 1}"][k]), f"micro-batch {k}"
 
 
-@pytest.mark.parametrize("dead_from", [0, 2, 3])
+@pytest.mark.parametrize("dead_from,dropout", [(0, 0.0), (2, 0.0), (3, 0.0), (2, 0.1)])
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["fp32", "bf16"])
-def test_failover_promotion_matches_oracle(hiplib, dead_from, dtype):
+def test_failover_promotion_matches_oracle(hiplib, dead_from, dtype, dropout):
     """The successor is preempted at micro-batch ``dead_from``: the engine promotes the shadow
     layers, replays the successor's backward passes from the stashed redundant activations and
-    ends the batch with the gradients of both stages (oracle: same stream on CPU autograd)."""
+    ends the batch with the gradients of both stages (oracle: same stream on CPU autograd).  With dropout the
+    promoted layers' backward passes make the decisions of the redundant forwards again."""
     hid, heads, ffn, L, S, sid, mb, M, seq = 128, 2, 256, 2, 4, 1, 2, 4, 64
-    engine, q = build(hid, heads, ffn, L, S, sid, mb, M, seq, dtype, GPT_VARIANT, 1, True, grad_mode="mse")
-    st, peer = oracle_for(engine, q, GPT_VARIANT, hid, heads, ffn, L, S, sid, M, 1, True)
+    variant = dict(GPT_VARIANT, dropout=dropout)
+    engine, q = build(hid, heads, ffn, L, S, sid, mb, M, seq, dtype, variant, 1, True, grad_mode="mse")
+    st, peer = oracle_for(engine, q, variant, hid, heads, ffn, L, S, sid, M, 1, True)
     # while alive, the successor returns the true gradients of the downstream loss
-    succ_cfg = ol.TransformerCfg(hidden=hid, heads=heads, ffn=ffn, **GPT_VARIANT)
     true_grads = []
     for k in range(M):
-        o1 = st.forward(peer.activations[k], sid).detach().requires_grad_(True)
-        o2 = st.forward(o1, sid + 1)
+        o1 = st.forward(peer.activations[k], sid, drop_id=(0, k)).detach().requires_grad_(True)
+        o2 = st.forward(o1, sid + 1, drop_id=(0, k))
         (torch.nn.functional.mse_loss(o2, peer.targets[sid + 1][k]) / M).backward()
         true_grads.append(o1.grad)
     for s_ in st.params.values():
