@@ -40,17 +40,22 @@ CONFIGS = {
 STAGES, STAGE_ID = 4, 1
 PEAK_BF16_TFLOPS, PEAK_F32_TFLOPS = 2500.0, 157.3
 
-# HBM bytes per launch of the dominant kernel, from the two rocprofv3 --pmc runs summarised in
-# profiles/ (FETCH_SIZE x 2.0 and WRITE_SIZE x 1.0, the factors a 256 MiB copy kernel gives);
-# counters cannot be read from inside this process, so the figure is carried here per
-# (config, kernel) and is null for anything that was not profiled.
-MEASURED_TRAFFIC_BYTES = {
-    # average over the three forward products that run on this tile (QKV, attention output, FFN2)
-    ("c2", "gemm_bf16_nt_dma256x128k64s3"): int((60311.8 * 2.0 + 27306.7) * 1024),
-    ("c2", "gemm_grouped_bf16_tn"): int((235172.6 * 2.0 + 49188.7) * 1024),
-    ("c2", "gemm_bf16_nt_dma256x256k64+act_dact"): int((50033.1 * 2.0 + 131072.0) * 1024),
-    ("c2", "gemm_bf16_nt_dma256x256k64+act"): int((50033.1 * 2.0 + 65536.0) * 1024),
-}
+TRAFFIC_SUMMARY = os.path.join(ROOT, "profiles", "gemm_bf16_dma_c2_gpt2_medium_stage_hbm_traffic.md")
+
+
+def measured_traffic_bytes(config, kernel):
+    """HBM bytes per launch of a GEMM variant as the two ``rocprofv3 --pmc`` runs summarised under profiles/ counted
+    them (FETCH_SIZE and WRITE_SIZE, each scaled by what the same counter reads for a copy of known size).  Counters
+    cannot be read from inside this process, so the figure is looked up in that summary's table ``| config | variant |
+    bytes per launch |``; None for anything that was not profiled, or where the summary is not at hand."""
+    try:
+        for line in open(TRAFFIC_SUMMARY):
+            cells = [c.strip().strip("`") for c in line.strip().strip("|").split("|")]
+            if len(cells) == 3 and cells[0] == config and cells[1] == kernel and cells[2].isdigit():
+                return int(cells[2])
+    except OSError:
+        pass
+    return None
 
 
 def build_engine(cfg, rc, rc_stream, seed=1138, use_graphs=False, paced=None, rc_issue="reference", eager=True):
@@ -400,7 +405,7 @@ def main():
         achieved = flops / secs / 1e12
         roofline = {"bound": "mfma", "achieved": round(achieved, 2), "peak": peak, "unit": "TFLOP/s",
                     "frac": round(achieved / peak, 4),
-                    "traffic": MEASURED_TRAFFIC_BYTES.get((args.config, f"gemm_{name}")), "kernel": f"gemm_{name}",
+                    "traffic": measured_traffic_bytes(args.config, f"gemm_{name}"), "kernel": f"gemm_{name}",
                     "measured_in": "a repeat of the timed steps of the RC-on single-stream leg with HIP events around "
                                    "each GEMM launch on its stream, minus the reading of an empty event bracket",
                     "event_bracket_overhead_us": round(overhead_s * 1e6, 2),
