@@ -154,6 +154,7 @@ static unsigned attn_grid(int seq, int nbh) { return (unsigned)(8 * ((nbh + 7) /
 // =========================================================================================
 // forward: block = 128 queries (4 waves x 32), loop over 64-key tiles
 // =========================================================================================
+template <bool DROP>
 __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const AttnArgs a) {
     __shared__ __attribute__((aligned(16))) unsigned char smem[2 * 2 * 8192];  // 2 stages x (K, V)
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -255,7 +256,7 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const AttnArgs a) {
                 }
             lsum = lsum * alpha + psum;
             m = mnew;
-            if (a.drop.thresh) {   // the normaliser takes every probability, the context only the kept ones
+            if (DROP && a.drop.thresh) {   // the normaliser takes every probability, the context only the kept ones
                 const uint64_t base = prob_index(a, b, head, min(myq, last)) + kv0;
 #pragma unroll
                 for (int u = 0; u < 2; ++u)
@@ -326,6 +327,7 @@ __global__ __launch_bounds__(256) void attn_delta_kernel(const AttnArgs a) {
 // =========================================================================================
 // backward dK, dV: block = 128 keys (4 waves x 32), loop over 64-query tiles
 // =========================================================================================
+template <bool DROP>
 __global__ __launch_bounds__(256, 2) void attn_bwd_dkv_kernel(const AttnArgs a) {
     // 2 stages x (Q tile 8 KiB, dO tile 8 KiB, lse 256 B, delta 256 B)
     constexpr int STAGE = 2 * 8192 + 512;
@@ -430,7 +432,7 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dkv_kernel(const AttnArgs a) 
             // dropout: dP = dP~ o mask / (1 - p) before it meets P; P itself is masked (into what multiplied V in
             // the forward) only after dS has been formed from the unmasked probabilities
             unsigned kept = 0xffffu;
-            if (a.drop.thresh) {
+            if (DROP && a.drop.thresh) {
                 asm volatile("" ::: "memory");
                 const int qlane = t * 64 + u * 32 + 4 * (lane >> 5);
                 kept = 0u;
@@ -449,7 +451,7 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dkv_kernel(const AttnArgs a) 
 #pragma unroll
                 for (int e = 0; e < 4; ++e) dp[g4 * 4 + e] = s[g4 * 4 + e] * (dp[g4 * 4 + e] - d4[e]);
             }
-            if (a.drop.thresh) {
+            if (DROP && a.drop.thresh) {
 #pragma unroll
                 for (int r = 0; r < 16; ++r) s[r] = (kept >> r) & 1u ? s[r] * a.drop.scale : 0.f;
             }
@@ -492,6 +494,7 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dkv_kernel(const AttnArgs a) 
 // =========================================================================================
 // backward dQ: block = 128 queries (4 waves x 32), loop over 64-key tiles
 // =========================================================================================
+template <bool DROP>
 __global__ __launch_bounds__(256, 2) void attn_bwd_dq_kernel(const AttnArgs a) {
     __shared__ __attribute__((aligned(16))) unsigned char smem[2 * 2 * 8192];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -572,7 +575,7 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dq_kernel(const AttnArgs a) {
 #pragma unroll
                     for (int r = 0; r < 16; ++r) s[r] = 8 * (r >> 2) + (r & 3) < lim ? s[r] : 0.f;
                 }
-                if (a.drop.thresh) {
+                if (DROP && a.drop.thresh) {
                     asm volatile("" ::: "memory");
                     const uint64_t base = prob_index(a, b, head, min(myq, last)) + kv0 + u * 32;
 #pragma unroll
@@ -640,7 +643,9 @@ extern "C" int bb_attention_fwd(int dtype, int mask, int batch, int heads, int s
     a.batch = batch; a.heads = heads; a.seq = seq; a.mask = mask;
     a.scale = 1.0f / sqrtf((float)head_dim);
     a.scale_log2 = a.scale * 1.4426950408889634f;
-    hipLaunchKernelGGL(attn_fwd_kernel, dim3(attn_grid(seq, batch * heads)), dim3(256), 0, (hipStream_t)stream, a);
+    // dropout is a kernel of its own: its keep decisions cost registers that decide how many blocks a CU holds
+    if (a.drop.thresh) hipLaunchKernelGGL(attn_fwd_kernel<true>, dim3(attn_grid(seq, batch * heads)), dim3(256), 0, (hipStream_t)stream, a);
+    else hipLaunchKernelGGL(attn_fwd_kernel<false>, dim3(attn_grid(seq, batch * heads)), dim3(256), 0, (hipStream_t)stream, a);
     BB_LAUNCH_CHECK();
     return BB_OK;
 }
@@ -669,8 +674,13 @@ extern "C" int bb_attention_bwd(int dtype, int mask, int batch, int heads, int s
     hipStream_t st = (hipStream_t)stream;
     hipLaunchKernelGGL(attn_delta_kernel, dim3((unsigned)(((int64_t)batch * seq + 31) / 32), (unsigned)heads), dim3(256), 0, st, a);
     dim3 grid(attn_grid(seq, batch * heads));
-    hipLaunchKernelGGL(attn_bwd_dkv_kernel, grid, dim3(256), 0, st, a);
-    hipLaunchKernelGGL(attn_bwd_dq_kernel, grid, dim3(256), 0, st, a);
+    if (a.drop.thresh) {
+        hipLaunchKernelGGL(attn_bwd_dkv_kernel<true>, grid, dim3(256), 0, st, a);
+        hipLaunchKernelGGL(attn_bwd_dq_kernel<true>, grid, dim3(256), 0, st, a);
+    } else {
+        hipLaunchKernelGGL(attn_bwd_dkv_kernel<false>, grid, dim3(256), 0, st, a);
+        hipLaunchKernelGGL(attn_bwd_dq_kernel<false>, grid, dim3(256), 0, st, a);
+    }
     BB_LAUNCH_CHECK();
     return BB_OK;
 }

@@ -45,6 +45,9 @@ template <int BM, int BN, int WM, int WN, bool AKM, bool BKM, bool DB, int STAGE
 static int launch_bf16_dma(GemmArgs& g, int batches, hipStream_t st) {
     constexpr int smem = STAGES * (BM + BN) * BK * 2;
     auto kern = gemm_bf16_dma_kernel<BM, BN, WM, WN, AKM, BKM, DB, STAGES, BK>;
+    if constexpr (!AKM && !BKM) {       // dropout goes with forward (NT) products only: fill_args refuses the others
+        if (g.drop.thresh) kern = gemm_bf16_dma_kernel<BM, BN, WM, WN, AKM, BKM, DB, STAGES, BK, true>;
+    }
     BB_HIP_CHECK(bb_allow_dynamic_lds((const void*)kern, smem));
     g.tiles_m = (g.M + BM - 1) / BM;
     g.tiles_n = (g.N + BN - 1) / BN;
@@ -243,8 +246,9 @@ static int fill_args(const bb_gemm_desc* d, GemmArgs& g, int64_t& batches, bool&
     g.epilogue = d->epilogue; g.act = d->act; g.accumulate = d->accumulate;
     g.c_f32 = (d->c_dtype == BB_F32);
     BB_REQUIRE(d->dropout_p >= 0.f && d->dropout_p < 1.f, "bb_gemm: dropout_p must be in [0, 1)");
-    BB_REQUIRE(d->dropout_p == 0.f || (batches == 1 && d->epilogue != BB_EPI_DACT && d->epilogue != BB_EPI_MUL && !d->accumulate),
-               "bb_gemm: dropout goes with an unbatched, non-accumulating problem and not with the DACT / MUL epilogues");
+    BB_REQUIRE(d->dropout_p == 0.f || (batches == 1 && d->layout == BB_NT && d->epilogue != BB_EPI_DACT && d->epilogue != BB_EPI_MUL &&
+                                       !d->accumulate),
+               "bb_gemm: dropout goes with an unbatched, non-accumulating NT problem and not with the DACT / MUL epilogues");
     g.drop = bb_drop_key(d->dropout_p, d->dropout_k0, d->dropout_k1);
     g.tiles_m = g.tiles_n = 0;
     return BB_OK;

@@ -82,6 +82,7 @@ __device__ __forceinline__ void epilogue_elem(const GemmArgs& g, int64_t coff, i
 }
 
 // Vector epilogue for bf16 operands: 8 consecutive columns of one row (n % 8 == 0, n + 8 <= N).
+template <bool DROP>
 __device__ __forceinline__ void epilogue_vec8(const GemmArgs& g, int64_t coff, int m, int n, float (&v)[8]) {
     const int64_t ci = coff + (int64_t)m * g.ldc + n;
     const int64_t xi = coff + (int64_t)m * g.ldaux + n;
@@ -92,7 +93,8 @@ __device__ __forceinline__ void epilogue_vec8(const GemmArgs& g, int64_t coff, i
         for (int e = 0; e < 8; ++e) v[e] += b[e];
     }
     float keep[8];
-    if (g.drop.thresh) {
+    const bool drop = DROP && g.drop.thresh != 0;   // DROP = false: no dropout code in the kernel at all
+    if (drop) {
 #pragma unroll
         for (int e = 0; e < 8; ++e) keep[e] = drop_factor(g, m, n + e);
     }
@@ -100,7 +102,7 @@ __device__ __forceinline__ void epilogue_vec8(const GemmArgs& g, int64_t coff, i
         if (g.aux_out) store_vec((bf16*)g.aux_out + xi, v);
 #pragma unroll
         for (int e = 0; e < 8; ++e) v[e] = act_f(v[e], g.act);
-        if (g.drop.thresh) {
+        if (drop) {
 #pragma unroll
             for (int e = 0; e < 8; ++e) v[e] *= keep[e];
         }
@@ -112,7 +114,7 @@ __device__ __forceinline__ void epilogue_vec8(const GemmArgs& g, int64_t coff, i
     } else if (g.epilogue == BB_EPI_RESIDUAL) {
         float r[8];
         load_vec((const bf16*)g.resid + xi, r);
-        if (g.drop.thresh) {
+        if (drop) {
 #pragma unroll
             for (int e = 0; e < 8; ++e) v[e] *= keep[e];
         }
@@ -127,7 +129,7 @@ __device__ __forceinline__ void epilogue_vec8(const GemmArgs& g, int64_t coff, i
         float d[8];
 #pragma unroll
         for (int e = 0; e < 8; ++e) act_dact_f(v[e], g.act, v[e], d[e]);
-        if (g.drop.thresh) {
+        if (drop) {
 #pragma unroll
             for (int e = 0; e < 8; ++e) {
                 v[e] *= keep[e];
@@ -135,7 +137,7 @@ __device__ __forceinline__ void epilogue_vec8(const GemmArgs& g, int64_t coff, i
             }
         }
         store_vec((bf16*)g.aux_out + xi, d);
-    } else if (g.drop.thresh) {
+    } else if (drop) {
 #pragma unroll
         for (int e = 0; e < 8; ++e) v[e] *= keep[e];
     }
@@ -587,7 +589,7 @@ template <int BR, int T, bool KM, int BK = 32> struct FragReader {
 // STATS: the epilogue also leaves the column statistics of the stored (bf16-rounded) output per 32-row strip, for the
 // batch normalisation that follows a convolution (its statistics pass then has nothing left to read).
 template <int BM, int BN, int WM, int WN, bool AKM, bool BKM, bool DB, int STAGES, int BK = 32, bool VIS = false, int CONV = 0,
-          bool STATS = false>
+          bool STATS = false, bool DROP = false>
 __device__ __forceinline__ void gemm_bf16_dma_body(const GemmArgs& g, const int block_id, const int batch_id,
                                                    const bool logical_id = false, const ConvArgs& cv = ConvArgs{}) {
     constexpr int NW = WM * WN;
@@ -911,7 +913,7 @@ __device__ __forceinline__ void gemm_bf16_dma_body(const GemmArgs& g, const int 
                     v[e] = lo[e];
                     v[4 + e] = hi[e];
                 }
-                if (live && m < g.M && n < g.N) epilogue_vec8(g, coff, m, n, v);
+                if (live && m < g.M && n < g.N) epilogue_vec8<DROP>(g, coff, m, n, v);
             }
             if constexpr (STATS) {
                 // Column statistics of this 32-row strip straight from the patch: lane = column, 32 conflict-free LDS
@@ -941,9 +943,11 @@ __device__ __forceinline__ void gemm_bf16_dma_body(const GemmArgs& g, const int 
         std::make_integer_sequence<int, TM * NP>{});
 }
 
-template <int BM, int BN, int WM, int WN, bool AKM, bool BKM, bool DB, int STAGES, int BK>
+// DROP: the epilogue can apply dropout (g.drop).  A kernel of its own, so that the keep decisions' registers cost the
+// kernels without dropout nothing (they decide how many blocks of the small tiles a CU holds).
+template <int BM, int BN, int WM, int WN, bool AKM, bool BKM, bool DB, int STAGES, int BK, bool DROP = false>
 __global__ __launch_bounds__(WM* WN * 64) void gemm_bf16_dma_kernel(const GemmArgs g) {
-    gemm_bf16_dma_body<BM, BN, WM, WN, AKM, BKM, DB, STAGES, BK>(g, blockIdx.x, blockIdx.z);
+    gemm_bf16_dma_body<BM, BN, WM, WN, AKM, BKM, DB, STAGES, BK, false, 0, false, DROP>(g, blockIdx.x, blockIdx.z);
 }
 // the same with the strip statistics of the output (NT, 64-wide k-tiles, three stages)
 template <int BM, int BN, int WM, int WN>

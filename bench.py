@@ -71,7 +71,8 @@ def build_engine(cfg, rc, rc_stream, seed=1138, use_graphs=False, paced=None, rc
         specs = [LayerSpec(BottleNeck, cfg["hidden"], cfg["mid"], height=cfg["side"], width=cfg["side"])
                  for _ in range(cfg["layers"] * STAGES)]
     else:
-        specs = [LayerSpec(TransformerLayer, cfg["hidden"], cfg["heads"], cfg["ffn"], **cfg["variant"])
+        specs = [LayerSpec(TransformerLayer, cfg["hidden"], cfg["heads"], cfg["ffn"], dropout=cfg.get("dropout", 0.0),
+                           **cfg["variant"])
                  for _ in range(cfg["layers"] * STAGES)]
     model = PipelineModule(specs, num_stages=STAGES, partition_method="uniform", stage_id=STAGE_ID, dtype=dtype,
                            device="cuda:0")
@@ -282,6 +283,9 @@ def main():
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="first run three 256 MiB fp32 copies (cast_kernel<float,float>): the known-size kernel that "
                          "FETCH_SIZE / WRITE_SIZE counters of a --pmc run are scaled by")
+    ap.add_argument("--dropout", type=float, default=0.0,
+                    help="dropout probability of the transformer layers (the reference scripts run 0.1; the benchmark "
+                         "line is quoted at 0, the configuration names none)")
     ap.add_argument("--no-paced", action="store_true",
                     help="skip the legs that run the stage inside the closed-loop model of a 4-stage 1F1B pipeline")
     ap.add_argument("--failover-at", type=int, default=None,
@@ -295,6 +299,13 @@ def main():
 
     from bamboo_amd import hip
     cfg = CONFIGS[args.config]
+    if args.dropout > 0.0:
+        # keys change every batch, so no HIP graphs, and the paced legs (which replay graphs) are left out
+        if args.graphs or cfg.get("kind") == "resnet":
+            print("bench.py: --dropout goes with the transformer configurations and without --graphs", file=sys.stderr)
+            sys.exit(2)
+        cfg = dict(cfg, dropout=args.dropout)
+        args.no_paced = True
     samples = cfg["mb"] * cfg["M"]
     graphs = bool(args.graphs)
     if graphs:
@@ -421,7 +432,7 @@ def main():
         "vs_baseline": None, "dtype": cfg["dtype"], "data": "synthetic",
         "config": {"workload": cfg["label"], "stage": f"{STAGE_ID} of {STAGES}", "redundancy_level": 1,
                    "eager_recovery": True, "rc_stream": bool(args.rc_stream), "hip_graphs": n_graphs if graphs else 0,
-                   "samples_per_step": samples,
+                   "samples_per_step": samples, "dropout": cfg.get("dropout", 0.0),
                    "attention": "n/a (convolutions as GEMMs over NHWC rows, 3x3 as implicit GEMMs)" if cfg.get("kind") == "resnet"
                    else ("unfused (fp32: scores and probabilities in HBM, as the reference); flops counted dense" if cfg["dtype"] == "fp32"
                          else "fused (no score matrix in HBM); flops counted dense, the causal kernel skips masked tiles")},

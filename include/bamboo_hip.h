@@ -172,7 +172,7 @@ int bb_layernorm_bwd(int dtype, int kind, int rows, int cols, float eps, const v
                      float* workspace, void* stream);
 /* The same without a workspace, for callers that cannot allocate device memory (code under HIP graph
  * capture, serving loops, harnesses that forbid hipMalloc).  No counterpart in the reference.  The
- * per-block partial sums live in an array inside the library's device image (2 MiB per GPU, held until
+ * per-block partial sums live in an array inside the library's device image (4 MiB per GPU, held until
  * the process ends); the call allocates nothing.  cols <= BB_LN_BWD_STATIC_MAX_COLS, else BB_EINVAL.
  * All calls on one GPU share that array: calls that overlap in time on one GPU (two streams, two
  * threads) race; calls on one stream are ordered and independent (nothing of an earlier call's contents
@@ -273,6 +273,16 @@ int bb_batchnorm_bwd(int dtype, int rows, int cols, const void* x, const void* g
  * (adjoint = 0), or its adjoint dx[p, c] = sum of the patch entries that read x[p, c]
  * (adjoint = 1); turns nn.Conv2d(k=3, padding=1) (resnet.py:58) and its input gradient into GEMMs. */
 int bb_patch3x3(int dtype, int adjoint, int n, int h, int w, int c, const void* src, void* dst, void* stream);
+/* The same with a stride (nn.Conv2d(k=3, stride=s, padding=1) of a down-sampling bottleneck, resnet.py:58 with
+ * stride = 2): col has one row per output pixel of the [(h-1)/s + 1, (w-1)/s + 1] grid; the adjoint writes the
+ * [n*h*w, c] input gradient from it.  stride 1..4.                                                           */
+int bb_patch3x3_strided(int dtype, int adjoint, int n, int h, int w, int c, int stride, const void* src, void* dst,
+                        void* stream);
+/* What a 1x1 convolution with stride s reads (the projection shortcut, resnet.py:69): adjoint = 0:
+ * dst[n, oy, ox, :] = src[n, s*oy, s*ox, :]; adjoint = 1, in place: dst[n, s*oy, s*ox, :] += src[n, oy, ox, :]
+ * (dst [n*h*w, c] keeps its other pixels).                                                                    */
+int bb_subsample(int dtype, int adjoint, int n, int h, int w, int c, int stride, const void* src, void* dst,
+                 void* stream);
 /* nn.Conv2d(cin, cout, kernel_size=3, padding=1, bias=False) (resnet.py:58) on NHWC rows as an implicit
  * GEMM on the matrix cores: the patch matrix is never written, the operand loader gathers it.
  *   BB_CONV_FWD    dst[p, o] = sum_{t, i} src[p + shift(t), i] * weight[o, t, i]     src [n*h*w, cin], dst [n*h*w, cout]
