@@ -68,14 +68,24 @@ def adopt_layer(obj, training=True):
         layer = TransformerLayer(hidden, int(heads), ffn, activation="relu", ln="annotated", mask="none", ln_eps=eps,
                                  dropout=drops[0] if drops else 0.0)
         return layer, params
-    if names == set(BottleNeck.REFERENCE_ORDER):
+    if names in (set(BottleNeck.RESIDUAL_ORDER), set(BottleNeck.RESIDUAL_ORDER + BottleNeck.SHORTCUT_ORDER)):
         w0, conv3 = params["residual_function.0.weight"], obj.residual_function[3]
         stride = conv3.stride[0] if isinstance(conv3.stride, tuple) else int(conv3.stride)
         bn = obj.residual_function[1]
         layer = BottleNeck(w0.shape[1], w0.shape[0], stride=stride, height=None, width=None, bn_eps=float(bn.eps),
                            bn_momentum=float(bn.momentum))
-        layer.adopted_running = {i: (obj.residual_function[i].running_mean.detach().clone(),
-                                     obj.residual_function[i].running_var.detach().clone()) for i in (1, 4, 7)}
+        if layer.projection != ("shortcut.0.weight" in names):
+            raise AdoptionError(f"BottleNeck-shaped module: stride {stride}, {w0.shape[1]} -> {4 * w0.shape[0]} channels "
+                                f"{'needs' if layer.projection else 'cannot have'} a projection shortcut (resnet.py:68-72)")
+        stats = lambda m: (m.running_mean.detach().clone(), m.running_var.detach().clone())
+        layer.adopted_running = {i: stats(obj.residual_function[i]) for i in (1, 4, 7)}
+        if layer.projection:
+            sc = obj.shortcut[0]
+            sc_stride = sc.stride[0] if isinstance(sc.stride, tuple) else int(sc.stride)
+            if sc_stride != stride:
+                raise AdoptionError(f"BottleNeck-shaped module: shortcut stride {sc_stride} differs from the 3x3 "
+                                    f"convolution's {stride}")
+            layer.adopted_running["shortcut"] = stats(obj.shortcut[1])
         return layer, params
     if names == {"a_2", "b_2"}:
         return FinalLayerNorm(params["a_2"].numel(), ln="annotated", ln_eps=float(getattr(obj, "eps", 1e-6))), params

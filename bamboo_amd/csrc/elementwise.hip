@@ -416,7 +416,7 @@ extern "C" int bb_layernorm_bwd(int dtype, int kind, int rows, int cols, float e
 
 // ---- the same for callers that cannot allocate ---------------------------------------------------------------
 // The per-block partial sums of dgain / dshift ([LN_BWD_BLOCKS][2][cols] floats) live in an array that is part of the
-// library's device image instead of a caller's workspace.  Every GPU the library runs on holds its own copy (2 MiB,
+// library's device image instead of a caller's workspace.  Every GPU the library runs on holds its own copy (4 MiB,
 // until the process ends) at its own address; host code reaches it only through the address that
 // hipGetSymbolAddress returns with that device current -- the array's name is no device address on the host.
 static __device__ __align__(256) float ln_bwd_static_scratch[LN_BWD_BLOCKS * 2 * BB_LN_BWD_STATIC_MAX_COLS];
@@ -1350,41 +1350,44 @@ extern "C" int bb_batchnorm_bwd(int dtype, int rows, int cols, const void* x, co
     return BB_OK;
 }
 
-// 3x3, stride 1, pad 1 patch gather on NHWC: col[p][tap*C + c] = x[n, y+dy, x+dx, c] (0 outside), and its
-// adjoint as a gather (every input pixel sums the nine patch entries that referenced it: no atomics)
+// 3x3, pad 1 patch gather on NHWC with stride s: col[q][tap*C + c] = x[n, s*oy+dy, s*ox+dx, c] (0 outside) for the
+// output pixel q = (n, oy, ox) of the [ho, wo] = [(h-1)/s + 1, (w-1)/s + 1] grid, and its adjoint as a gather (every
+// input pixel sums the patch entries that referenced it: no atomics)
 template <typename T, bool ADJOINT>
-__global__ __launch_bounds__(256) void patch3x3_kernel(int n, int h, int w, int c, const T* __restrict__ src,
+__global__ __launch_bounds__(256) void patch3x3_kernel(int n, int h, int w, int c, int s, const T* __restrict__ src,
                                                        T* __restrict__ dst) {
     constexpr int VEC = Elem<T>::VEC;
     const int cv = c / VEC;
-    const int64_t pixels = (int64_t)n * h * w;
-    const int64_t total = ADJOINT ? pixels * cv : pixels * 9 * cv;
+    const int ho = (h - 1) / s + 1, wo = (w - 1) / s + 1;
+    const int64_t total = ADJOINT ? (int64_t)n * h * w * cv : (int64_t)n * ho * wo * 9 * cv;
     for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < total; i += (int64_t)gridDim.x * 256) {
         if (!ADJOINT) {
             const int ch = (int)(i % cv) * VEC;
             const int tap = (int)((i / cv) % 9);
-            const int64_t p = i / (cv * 9);
-            const int px = (int)(p % w), py = (int)((p / w) % h);
-            const int sy = py + tap / 3 - 1, sx = px + tap % 3 - 1;
+            const int64_t q = i / (cv * 9);
+            const int ox = (int)(q % wo), oy = (int)((q / wo) % ho);
+            const int64_t img = q / ((int64_t)wo * ho);
+            const int sy = oy * s + tap / 3 - 1, sx = ox * s + tap % 3 - 1;
             float v[VEC];
 #pragma unroll
             for (int e = 0; e < VEC; ++e) v[e] = 0.f;
-            if (sy >= 0 && sy < h && sx >= 0 && sx < w) load_vec(src + (p + (int64_t)(sy - py) * w + (sx - px)) * c + ch, v);
-            store_vec(dst + (p * 9 + tap) * c + ch, v);
+            if (sy >= 0 && sy < h && sx >= 0 && sx < w) load_vec(src + ((img * h + sy) * w + sx) * c + ch, v);
+            store_vec(dst + (q * 9 + tap) * c + ch, v);
         } else {
             const int ch = (int)(i % cv) * VEC;
             const int64_t p = i / cv;
             const int px = (int)(p % w), py = (int)((p / w) % h);
+            const int64_t img = p / ((int64_t)w * h);
             float acc[VEC];
 #pragma unroll
             for (int e = 0; e < VEC; ++e) acc[e] = 0.f;
 #pragma unroll
             for (int tap = 0; tap < 9; ++tap) {
-                // patch of pixel q = p - shift(tap) holds x[p] at position tap
-                const int qy = py - (tap / 3 - 1), qx = px - (tap % 3 - 1);
-                if (qy >= 0 && qy < h && qx >= 0 && qx < w) {
+                // the patch of output pixel (qy, qx) holds x[p] at position tap when s*q + shift(tap) = p
+                const int ny = py - (tap / 3 - 1), nx = px - (tap % 3 - 1);
+                if (ny >= 0 && nx >= 0 && ny % s == 0 && nx % s == 0 && ny / s < ho && nx / s < wo) {
                     float v[VEC];
-                    load_vec(src + ((p + (int64_t)(qy - py) * w + (qx - px)) * 9 + tap) * c + ch, v);
+                    load_vec(src + (((img * ho + ny / s) * wo + nx / s) * 9 + tap) * c + ch, v);
 #pragma unroll
                     for (int e = 0; e < VEC; ++e) acc[e] += v[e];
                 }
@@ -1394,19 +1397,76 @@ __global__ __launch_bounds__(256) void patch3x3_kernel(int n, int h, int w, int 
     }
 }
 
-extern "C" int bb_patch3x3(int dtype, int adjoint, int n, int h, int w, int c, const void* src, void* dst, void* stream) {
+extern "C" int bb_patch3x3_strided(int dtype, int adjoint, int n, int h, int w, int c, int stride, const void* src,
+                                   void* dst, void* stream) {
     BB_REQUIRE(dtype == BB_F32 || dtype == BB_BF16, "bb_patch3x3: bad dtype %d", dtype);
     const int vec = dtype == BB_BF16 ? 8 : 4;
-    BB_REQUIRE(n > 0 && h > 0 && w > 0 && c > 0 && c % vec == 0 && src && dst, "bb_patch3x3: bad arguments");
+    BB_REQUIRE(n > 0 && h > 0 && w > 0 && c > 0 && c % vec == 0 && stride >= 1 && stride <= 4 && src && dst,
+               "bb_patch3x3: bad arguments (n=%d h=%d w=%d c=%d stride=%d)", n, h, w, c, stride);
     hipStream_t st = (hipStream_t)stream;
-    const int64_t items = (int64_t)n * h * w * (adjoint ? 1 : 9) * (c / vec);
+    const int ho = (h - 1) / stride + 1, wo = (w - 1) / stride + 1;
+    const int64_t items = adjoint ? (int64_t)n * h * w * (c / vec) : (int64_t)n * ho * wo * 9 * (c / vec);
     dim3 grid(grid_for(items));
     if (dtype == BB_BF16) {
-        if (adjoint) hipLaunchKernelGGL((patch3x3_kernel<bf16, true>), grid, dim3(256), 0, st, n, h, w, c, (const bf16*)src, (bf16*)dst);
-        else hipLaunchKernelGGL((patch3x3_kernel<bf16, false>), grid, dim3(256), 0, st, n, h, w, c, (const bf16*)src, (bf16*)dst);
+        if (adjoint) hipLaunchKernelGGL((patch3x3_kernel<bf16, true>), grid, dim3(256), 0, st, n, h, w, c, stride, (const bf16*)src, (bf16*)dst);
+        else hipLaunchKernelGGL((patch3x3_kernel<bf16, false>), grid, dim3(256), 0, st, n, h, w, c, stride, (const bf16*)src, (bf16*)dst);
     } else {
-        if (adjoint) hipLaunchKernelGGL((patch3x3_kernel<float, true>), grid, dim3(256), 0, st, n, h, w, c, (const float*)src, (float*)dst);
-        else hipLaunchKernelGGL((patch3x3_kernel<float, false>), grid, dim3(256), 0, st, n, h, w, c, (const float*)src, (float*)dst);
+        if (adjoint) hipLaunchKernelGGL((patch3x3_kernel<float, true>), grid, dim3(256), 0, st, n, h, w, c, stride, (const float*)src, (float*)dst);
+        else hipLaunchKernelGGL((patch3x3_kernel<float, false>), grid, dim3(256), 0, st, n, h, w, c, stride, (const float*)src, (float*)dst);
+    }
+    BB_LAUNCH_CHECK();
+    return BB_OK;
+}
+
+extern "C" int bb_patch3x3(int dtype, int adjoint, int n, int h, int w, int c, const void* src, void* dst, void* stream) {
+    return bb_patch3x3_strided(dtype, adjoint, n, h, w, c, 1, src, dst, stream);
+}
+
+// Every s-th pixel of every s-th row of an NHWC tensor (what a 1x1 convolution with stride s reads), and the adjoint
+// added in place: dst[n, s*oy, s*ox, :] += src[n, oy, ox, :] (each target is written by one thread).
+template <typename T, bool ADJOINT>
+__global__ __launch_bounds__(256) void subsample_kernel(int n, int h, int w, int c, int s, const T* __restrict__ src,
+                                                        T* __restrict__ dst) {
+    constexpr int VEC = Elem<T>::VEC;
+    const int cv = c / VEC;
+    const int ho = (h - 1) / s + 1, wo = (w - 1) / s + 1;
+    const int64_t total = (int64_t)n * ho * wo * cv;
+    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < total; i += (int64_t)gridDim.x * 256) {
+        const int ch = (int)(i % cv) * VEC;
+        const int64_t q = i / cv;
+        const int ox = (int)(q % wo), oy = (int)((q / wo) % ho);
+        const int64_t img = q / ((int64_t)wo * ho);
+        const int64_t p = (img * h + (int64_t)oy * s) * w + (int64_t)ox * s;
+        float v[VEC];
+        if (!ADJOINT) {
+            load_vec(src + p * c + ch, v);
+            store_vec(dst + q * c + ch, v);
+        } else {
+            float d[VEC];
+            load_vec(src + q * c + ch, v);
+            load_vec(dst + p * c + ch, d);
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) d[e] += v[e];
+            store_vec(dst + p * c + ch, d);
+        }
+    }
+}
+
+extern "C" int bb_subsample(int dtype, int adjoint, int n, int h, int w, int c, int stride, const void* src, void* dst,
+                            void* stream) {
+    BB_REQUIRE(dtype == BB_F32 || dtype == BB_BF16, "bb_subsample: bad dtype %d", dtype);
+    const int vec = dtype == BB_BF16 ? 8 : 4;
+    BB_REQUIRE(n > 0 && h > 0 && w > 0 && c > 0 && c % vec == 0 && stride >= 1 && stride <= 4 && src && dst,
+               "bb_subsample: bad arguments (n=%d h=%d w=%d c=%d stride=%d)", n, h, w, c, stride);
+    hipStream_t st = (hipStream_t)stream;
+    const int ho = (h - 1) / stride + 1, wo = (w - 1) / stride + 1;
+    dim3 grid(grid_for((int64_t)n * ho * wo * (c / vec)));
+    if (dtype == BB_BF16) {
+        if (adjoint) hipLaunchKernelGGL((subsample_kernel<bf16, true>), grid, dim3(256), 0, st, n, h, w, c, stride, (const bf16*)src, (bf16*)dst);
+        else hipLaunchKernelGGL((subsample_kernel<bf16, false>), grid, dim3(256), 0, st, n, h, w, c, stride, (const bf16*)src, (bf16*)dst);
+    } else {
+        if (adjoint) hipLaunchKernelGGL((subsample_kernel<float, true>), grid, dim3(256), 0, st, n, h, w, c, stride, (const float*)src, (float*)dst);
+        else hipLaunchKernelGGL((subsample_kernel<float, false>), grid, dim3(256), 0, st, n, h, w, c, stride, (const float*)src, (float*)dst);
     }
     BB_LAUNCH_CHECK();
     return BB_OK;

@@ -137,17 +137,21 @@ class PipelineEngine:
         self.ctx = model.prepare_context(built, self.batch, self.seq, stream=self.main_stream)
         self.rc_ctx = self.ctx
         if self.rc_stream is not None:
-            self.rc_ctx = model.prepare_context(self.r_stage_ids, self.batch, self.seq, stream=self.rc_stream,
-                                                forward_only=True)
+            # the shadowed stage takes what the own stage leaves (a down-sampling stage changes the positions)
+            self.rc_ctx = model.prepare_context(self.r_stage_ids, self.batch, model.stage_seq[self.r_stage_ids[0]][0],
+                                                stream=self.rc_stream, forward_only=True)
         self.stash_bytes = 0
         for sid in built:
             self.stash_bytes += model.allocate_stash(sid, self.ctx, self.micro_batches)
         self._fwd_done = [torch.cuda.Event() for _ in range(self.micro_batches)]
         self._deferred = {}   # (stage, slot) -> the slot's last forward left backward-only outputs out
 
-        act_shape = (self.batch * self.seq, self.queue.shape[2])
+        if model.stage_io_shapes(self.stage_id, self.batch)[0] != (self.batch * self.seq, self.queue.shape[2]):
+            raise PipelineError(f"the activation queue delivers {tuple(self.queue.shape)}, the stage's first layer takes "
+                                f"{model.stage_io_shapes(self.stage_id, self.batch)[0]} (rows, features)")
         self._input_grad_store = {
-            sid: [torch.empty(act_shape, dtype=model.dtype, device=self.device) for _ in range(self.micro_batches)]
+            sid: [torch.empty(model.stage_io_shapes(sid, self.batch)[0], dtype=model.dtype, device=self.device)
+                  for _ in range(self.micro_batches)]
             for sid in built}
         self._loss_grad = None     # gradient of the loss head: allocated with the first last-stage output it sees
         self.total_loss = torch.zeros(1, dtype=torch.float32, device=self.device)
@@ -400,7 +404,7 @@ class PipelineEngine:
                 sp.view(sp.exp_avg_sq, name).copy_(self.state_buffers[absorbed][f"{i}.exp_avg_sq"])
             self.ctx = self.module.prepare_context(self.stage_ids + [absorbed], self.batch, self.seq, stream=self.main_stream)
             self.stash_bytes += self.module.allocate_stash(absorbed, self.ctx, self.micro_batches)
-            act_shape = (self.batch * self.seq, self.queue.shape[2])
+            act_shape = self.module.stage_io_shapes(absorbed, self.batch)[0]
             self._input_grad_store[absorbed] = [torch.empty(act_shape, dtype=self.module.dtype, device=self.device)
                                                 for _ in range(self.micro_batches)]
             for key in (f"input_{absorbed}", f"output_{absorbed}", f"input_grad_{absorbed}"):

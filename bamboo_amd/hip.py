@@ -25,7 +25,7 @@ LN_CODES = {"standard": LN_STANDARD, "annotated": LN_ANNOTATED}
 EXPORTS = (
     "bb_version", "bb_last_error", "bb_init", "bb_gemm", "bb_gemm_grouped", "bb_gemm_splitk_workspace", "bb_gemm_grouped_splitk", "bb_gemm_variant", "bb_layernorm_fwd",
     "bb_layernorm_bwd_workspace", "bb_layernorm_bwd", "bb_layernorm_bwd_static", "bb_colsum_workspace", "bb_colsum_acc", "bb_rowsum_fwd", "bb_rowsum_bwd", "bb_dropout_apply", "bb_dropout_keep_host",
-    "bb_softmax_fwd", "bb_softmax_bwd", "bb_attention_fwd", "bb_attention_bwd", "bb_residual_add", "bb_act_fwd", "bb_bn_workspace", "bb_batchnorm_fwd", "bb_batchnorm_bwd", "bb_patch3x3", "bb_conv3x3_supported", "bb_conv3x3", "bb_gemm_strip_stats_supported", "bb_strip_stats_workspace", "bb_batchnorm_fwd_strips", "bb_mse_workspace", "bb_mse_fwd_bwd", "bb_graph_begin", "bb_graph_end", "bb_graph_launch", "bb_graph_destroy",
+    "bb_softmax_fwd", "bb_softmax_bwd", "bb_attention_fwd", "bb_attention_bwd", "bb_residual_add", "bb_act_fwd", "bb_bn_workspace", "bb_batchnorm_fwd", "bb_batchnorm_bwd", "bb_patch3x3", "bb_patch3x3_strided", "bb_subsample", "bb_conv3x3_supported", "bb_conv3x3", "bb_gemm_strip_stats_supported", "bb_strip_stats_workspace", "bb_batchnorm_fwd_strips", "bb_mse_workspace", "bb_mse_fwd_bwd", "bb_graph_begin", "bb_graph_end", "bb_graph_launch", "bb_graph_destroy",
     "bb_adam_multi", "bb_cast", "bb_fill_f32",
 )
 
@@ -111,6 +111,8 @@ def lib():
     L.bb_batchnorm_fwd.argtypes = [c_int, c_int, c_int, c_float, c_float, c_int] + [c_void_p] * 11
     L.bb_batchnorm_bwd.argtypes = [c_int, c_int, c_int] + [c_void_p] * 12
     L.bb_patch3x3.argtypes = [c_int, c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p]
+    L.bb_patch3x3_strided.argtypes = [c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p]
+    L.bb_subsample.argtypes = [c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p]
     L.bb_conv3x3_supported.argtypes = [c_int] * 7
     L.bb_conv3x3.argtypes = [c_int] * 7 + [c_void_p] * 5
     L.bb_gemm_strip_stats_supported.argtypes = [POINTER(GemmDesc)]
@@ -514,9 +516,33 @@ def batchnorm_bwd(x, gamma, mean, rstd, dy, relu_out, dx, g_out, dgamma, dbeta, 
                                  _ptr(workspace), stream_ptr(stream)), "bb_batchnorm_bwd")
 
 
-def patch3x3(src, dst, n, h, w, c, adjoint=False, stream=None):
-    check(lib().bb_patch3x3(dtype_code(src.dtype), int(adjoint), n, h, w, c, _ptr(src), _ptr(dst), stream_ptr(stream)),
-          "bb_patch3x3")
+def _out_side(side, stride):
+    return (side - 1) // stride + 1
+
+
+def patch3x3(src, dst, n, h, w, c, adjoint=False, stride=1, stream=None):
+    """Patch matrix of nn.Conv2d(k=3, stride, padding=1) over NHWC rows: ``dst[n*ho*wo, 9*c]`` from ``src[n*h*w, c]``;
+    ``adjoint``: ``dst[n*h*w, c]`` from ``src[n*ho*wo, 9*c]``."""
+    rows_in, rows_out = n * h * w, n * _out_side(h, stride) * _out_side(w, stride)
+    want_src, want_dst = (rows_out * 9 * c, rows_in * c) if adjoint else (rows_in * c, rows_out * 9 * c)
+    if src.numel() != want_src or dst.numel() != want_dst or not (src.is_contiguous() and dst.is_contiguous()):
+        raise HipKernelError(f"patch3x3: {tuple(src.shape)} -> {tuple(dst.shape)} does not fit n={n} h={h} w={w} c={c} "
+                             f"stride={stride} adjoint={adjoint}")
+    check(lib().bb_patch3x3_strided(dtype_code(src.dtype), int(adjoint), n, h, w, c, stride, _ptr(src), _ptr(dst),
+                                    stream_ptr(stream)), "bb_patch3x3_strided")
+
+
+def subsample(src, dst, n, h, w, c, stride, adjoint=False, stream=None):
+    """Rows of the pixels a strided 1x1 convolution reads: ``dst[n*ho*wo, c]`` from ``src[n*h*w, c]``; ``adjoint``:
+    ``dst[n*h*w, c]`` gets ``src[n*ho*wo, c]`` ADDED at those pixels."""
+    rows_in, rows_out = n * h * w, n * _out_side(h, stride) * _out_side(w, stride)
+    want_src, want_dst = (rows_out * c, rows_in * c) if adjoint else (rows_in * c, rows_out * c)
+    if src.numel() != want_src or dst.numel() != want_dst or src.dtype != dst.dtype or \
+            not (src.is_contiguous() and dst.is_contiguous()):
+        raise HipKernelError(f"subsample: {tuple(src.shape)} -> {tuple(dst.shape)} does not fit n={n} h={h} w={w} c={c} "
+                             f"stride={stride} adjoint={adjoint}")
+    check(lib().bb_subsample(dtype_code(src.dtype), int(adjoint), n, h, w, c, stride, _ptr(src), _ptr(dst),
+                             stream_ptr(stream)), "bb_subsample")
 
 
 CONV_FWD, CONV_DGRAD = 0, 1

@@ -468,21 +468,28 @@ class SumLast:
 
 
 class BottleNeck:
-    """ResNet bottleneck block ``ReLU(BN(conv1x1(ReLU(BN(conv3x3(ReLU(BN(conv1x1 x)))))) + x)`` with the
-    identity shortcut (reference ``BottleNeck``, DeepSpeedExamples/pipeline_parallelism/resnet.py:49-75:
-    stride 1 and ``in_channels == 4 * out_channels``), on NHWC activations viewed as
-    ``[rows = N*H*W, channels]``.  The 1x1 convolutions are plain GEMMs on that view; the 3x3
-    convolution, its input gradient (``hip.conv3x3``) and its weight gradient (``gemm_desc(..., conv=)``) are
-    implicit GEMMs: the operand loader gathers the 3x3 neighbourhoods, no patch matrix is written.  Where the
-    implicit kernels do not take the problem (fp32, channel counts that are not multiples of 64, resp. 128 for
-    the weight gradient) the same products run as GEMMs over the gathered patch matrix ``[rows, 9*C]``.  Parameter names are the
-    reference's; the 3x3 weight is kept as ``[out, 3, 3, in]`` (tap-major, channel-minor) so that it is the
-    ``[out, 9*in]`` GEMM operand as it lies in memory (the reference holds ``[out, in, 3, 3]``)."""
+    """ResNet bottleneck block ``ReLU(BN(conv1x1(ReLU(BN(conv3x3(ReLU(BN(conv1x1 x)))))) + shortcut(x))`` (reference
+    ``BottleNeck``, DeepSpeedExamples/pipeline_parallelism/resnet.py:49-75) on NHWC activations viewed as
+    ``[rows = N*H*W, channels]``.  The shortcut is the identity when ``stride == 1`` and ``in_channels == 4 *
+    out_channels``, else ``BN(conv1x1(x, stride))`` (resnet.py:68-72); ``stride`` sits on the 3x3 convolution
+    (resnet.py:58), so a down-sampling block turns ``N*H*W`` input rows into ``N*ceil(H/s)*ceil(W/s)`` output rows.
+    The 1x1 convolutions are plain GEMMs on the row view (the strided one on the rows of every s-th pixel,
+    ``hip.subsample``); the 3x3 convolution with stride 1, its input gradient (``hip.conv3x3``) and its weight
+    gradient (``gemm_desc(..., conv=)``) are implicit GEMMs: the operand loader gathers the 3x3 neighbourhoods, no
+    patch matrix is written.  Where the implicit kernels do not take the problem (a stride, fp32, channel counts that
+    are not multiples of 64, resp. 128 for the weight gradient) the same products run as GEMMs over the gathered patch
+    matrix ``[rows, 9*C]``.  Parameter names are the reference's; the 3x3 weight is kept as ``[out, 3, 3, in]``
+    (tap-major, channel-minor) so that it is the ``[out, 9*in]`` GEMM operand as it lies in memory (the reference
+    holds ``[out, in, 3, 3]``)."""
+
+    EXPANSION = 4
 
     def __init__(self, in_channels, out_channels, stride=1, height=14, width=14, bn_eps=1e-5, bn_momentum=0.1):
-        if stride != 1 or in_channels != 4 * out_channels:
-            raise NotImplementedError("only the identity-shortcut bottleneck (stride 1, in = 4 * out) is built")
-        self.cin, self.cmid, self.h, self.w = in_channels, out_channels, height, width
+        if stride not in (1, 2):
+            raise NotImplementedError(f"bottleneck stride {stride}: the reference's ResNets use 1 and 2")
+        self.cin, self.cmid, self.cout = in_channels, out_channels, self.EXPANSION * out_channels
+        self.stride, self.h, self.w = stride, height, width
+        self.projection = stride != 1 or in_channels != self.cout
         self.eps, self.momentum = bn_eps, bn_momentum
         self.w_ = self.g_ = None
         self.running = None
@@ -494,26 +501,40 @@ class BottleNeck:
 
     @property
     def out_features(self):
-        return self.cin
+        return self.cout
+
+    def out_seq(self, seq):
+        """Pixels per image behind the block, for ``seq`` in front of it."""
+        if self.stride == 1:
+            return seq
+        h, w = self._image(seq)
+        return ((h - 1) // self.stride + 1) * ((w - 1) // self.stride + 1)
 
     def param_specs(self):
-        ci, cm = self.cin, self.cmid
-        return OrderedDict([
-            ("residual_function.0.weight", (cm, ci)),
-            ("residual_function.1.weight", (cm,)), ("residual_function.1.bias", (cm,)),
-            ("residual_function.3.weight", (cm, 3, 3, cm)),
-            ("residual_function.4.weight", (cm,)), ("residual_function.4.bias", (cm,)),
-            ("residual_function.6.weight", (ci, cm)),
-            ("residual_function.7.weight", (ci,)), ("residual_function.7.bias", (ci,)),
-        ])
+        ci, cm, co = self.cin, self.cmid, self.cout
+        specs = [("residual_function.0.weight", (cm, ci)),
+                 ("residual_function.1.weight", (cm,)), ("residual_function.1.bias", (cm,)),
+                 ("residual_function.3.weight", (cm, 3, 3, cm)),
+                 ("residual_function.4.weight", (cm,)), ("residual_function.4.bias", (cm,)),
+                 ("residual_function.6.weight", (co, cm)),
+                 ("residual_function.7.weight", (co,)), ("residual_function.7.bias", (co,))]
+        if self.projection:
+            specs += [("shortcut.0.weight", (co, ci)), ("shortcut.1.weight", (co,)), ("shortcut.1.bias", (co,))]
+        return OrderedDict(specs)
 
     def num_params(self):
         return sum(math.prod(s) for s in self.param_specs().values())
 
-    # registration order of the reference's ``residual_function`` (resnet.py:55-64)
-    REFERENCE_ORDER = ("residual_function.0.weight", "residual_function.1.weight", "residual_function.1.bias",
-                       "residual_function.3.weight", "residual_function.4.weight", "residual_function.4.bias",
-                       "residual_function.6.weight", "residual_function.7.weight", "residual_function.7.bias")
+    # registration order of the reference's ``residual_function`` and ``shortcut`` (resnet.py:55-72)
+    RESIDUAL_ORDER = ("residual_function.0.weight", "residual_function.1.weight", "residual_function.1.bias",
+                      "residual_function.3.weight", "residual_function.4.weight", "residual_function.4.bias",
+                      "residual_function.6.weight", "residual_function.7.weight", "residual_function.7.bias")
+    SHORTCUT_ORDER = ("shortcut.0.weight", "shortcut.1.weight", "shortcut.1.bias")
+    _CONV1X1 = ("residual_function.0.weight", "residual_function.6.weight", "shortcut.0.weight")
+
+    @property
+    def REFERENCE_ORDER(self):
+        return self.RESIDUAL_ORDER + (self.SHORTCUT_ORDER if self.projection else ())
 
     @staticmethod
     def to_native(name, tensor):
@@ -523,11 +544,11 @@ class BottleNeck:
             return t.view(t.shape[0], -1) if t.shape[1] == 1 else t
         return tensor
 
-    @staticmethod
-    def to_reference(name, tensor):
+    @classmethod
+    def to_reference(cls, name, tensor):
         """Arena layout -> the reference's: 1x1 convolutions [O, I] -> [O, I, 1, 1], the 3x3 one [O, kh, kw, I] ->
         [O, I, kh, kw] (a copy)."""
-        if name in ("residual_function.0.weight", "residual_function.6.weight"):
+        if name in cls._CONV1X1:
             return tensor.reshape(tensor.shape[0], tensor.shape[1], 1, 1)
         if name == "residual_function.3.weight":
             return tensor.permute(0, 3, 1, 2).contiguous()
@@ -538,7 +559,8 @@ class BottleNeck:
         the reference's [O, I, kh, kw] layout, BN gain 1 / shift 0."""
         ref_shapes = {"residual_function.0.weight": (self.cmid, self.cin, 1, 1),
                       "residual_function.3.weight": (self.cmid, self.cmid, 3, 3),
-                      "residual_function.6.weight": (self.cin, self.cmid, 1, 1)}
+                      "residual_function.6.weight": (self.cout, self.cmid, 1, 1),
+                      "shortcut.0.weight": (self.cout, self.cin, 1, 1)}
         for i, name in enumerate(self.param_specs()):
             t = master[name]
             if name in ref_shapes:
@@ -556,37 +578,81 @@ class BottleNeck:
         for d in (self.w_, self.g_):
             d["conv2"] = d["residual_function.3.weight"].view(self.cmid, 9 * self.cmid)
 
+    # ---------------------------------------------------------------- shapes
+    def _image(self, seq):
+        """(height, width) of the input image; a block taken over from a module does not know them: square
+        images, side = sqrt(positions)."""
+        if self.h is None or self.w is None:
+            side = math.isqrt(seq)
+            if side * side != seq:
+                raise hip.HipKernelError(f"cannot infer a square image from {seq} positions: pass height= and width=")
+            return side, side
+        return self.h, self.w
+
+    def _bind_image(self, ctx):
+        self.h, self.w = self._image(ctx.seq)
+        if ctx.seq != self.h * self.w:
+            raise hip.HipKernelError(f"activation has {ctx.seq} positions, the block expects {self.h}x{self.w}")
+
+    def _rows(self, ctx):
+        """(input rows, output rows, output height, output width)."""
+        self._bind_image(ctx)
+        ho, wo = (self.h - 1) // self.stride + 1, (self.w - 1) // self.stride + 1
+        return ctx.batch * self.h * self.w, ctx.batch * ho * wo, ho, wo
+
     def stash_specs(self, ctx):
-        R, ci, cm = ctx.rows, self.cin, self.cmid
+        R, R2, _, _ = self._rows(ctx)
+        cm, co = self.cmid, self.cout
         dt, f32 = ctx.dtype, torch.float32
-        return [("y1", (R, cm), dt), ("a1", (R, cm), dt), ("y2", (R, cm), dt), ("a2", (R, cm), dt),
-                ("y3", (R, ci), dt), ("out", (R, ci), dt),
-                ("mean1", (cm,), f32), ("rstd1", (cm,), f32), ("mean2", (cm,), f32), ("rstd2", (cm,), f32),
-                ("mean3", (ci,), f32), ("rstd3", (ci,), f32)]
+        specs = [("y1", (R, cm), dt), ("a1", (R, cm), dt), ("y2", (R2, cm), dt), ("a2", (R2, cm), dt),
+                 ("y3", (R2, co), dt), ("out", (R2, co), dt),
+                 ("mean1", (cm,), f32), ("rstd1", (cm,), f32), ("mean2", (cm,), f32), ("rstd2", (cm,), f32),
+                 ("mean3", (co,), f32), ("rstd3", (co,), f32)]
+        if self.projection:
+            specs += [("ys", (R2, co), dt), ("mean_s", (co,), f32), ("rstd_s", (co,), f32)]
+        return specs
+
+    def _wgrad_elems(self):
+        n = self.cin * self.cmid + 9 * self.cmid * self.cmid + self.cmid * self.cout
+        return n + (self.cout * self.cin if self.projection else 0)
 
     def scratch_specs(self, ctx):
-        R, ci, cm = ctx.rows, self.cin, self.cmid
+        R, R2, _, _ = self._rows(ctx)
+        ci, cm, co = self.cin, self.cmid, self.cout
         dt = ctx.dtype
-        # split-K partial products of the three weight gradients (8 chunks of each, fp32)
-        nws = 8 * (ci * cm + 9 * cm * cm + cm * ci)
-        return [("col", (R, 9 * cm), dt), ("d_col", (R, 9 * cm), dt), ("d_y3", (R, ci), dt), ("d_res", (R, ci), dt),
-                ("d_m0", (R, cm), dt), ("d_m1", (R, cm), dt), ("d_m2", (R, cm), dt), ("splitk", (nws,), torch.float32),
-                ("strips", (hip.strip_stats_workspace(R, ci),), torch.float32)]
+        specs = [("d_col", (R2, 9 * cm), dt), ("d_y3", (R2, co), dt), ("d_res", (R2, co), dt),
+                 ("d_m0", (R, cm), dt), ("d_m1", (R2, cm), dt), ("d_m2", (R, cm), dt),
+                 # split-K partial products of the weight gradients (8 chunks of each, fp32)
+                 ("splitk", (8 * self._wgrad_elems(),), torch.float32)]
+        if self.projection:
+            specs += [("d_ys", (R2, co), dt), ("d_xs", (R2, ci), dt)]
+        return specs + self.forward_scratch_specs(ctx)
 
     def forward_scratch_specs(self, ctx):
-        return [("col", (ctx.rows, 9 * self.cmid), ctx.dtype),
-                ("strips", (hip.strip_stats_workspace(ctx.rows, self.cin),), torch.float32)]
+        R, R2, _, _ = self._rows(ctx)
+        specs = [("col", (R2, 9 * self.cmid), ctx.dtype),
+                 ("strips", (hip.strip_stats_workspace(R, self.cout),), torch.float32)]
+        if self.projection:
+            specs += [("sc", (R2, self.cout), ctx.dtype), ("xs", (R2, self.cin), ctx.dtype)]
+        return specs
 
     def workspace_elems(self):
-        return max(hip.bn_workspace(self.cin), hip.colsum_workspace(self.cin))
+        c = max(self.cin, self.cout)
+        return max(hip.bn_workspace(c), hip.colsum_workspace(c))
 
     def flops_fwd(self, batch, seq):
-        return 2 * batch * seq * (self.cin * self.cmid + 9 * self.cmid * self.cmid + self.cmid * self.cin)
+        out = batch * self.out_seq(seq)
+        f = 2 * batch * seq * self.cin * self.cmid + 2 * out * (9 * self.cmid * self.cmid + self.cmid * self.cout)
+        return f + (2 * out * self.cin * self.cout if self.projection else 0)
+
+    # ---------------------------------------------------------------- pieces
+    _BN_NAMES = {1: "residual_function.1", 4: "residual_function.4", 7: "residual_function.7", "shortcut": "shortcut.1"}
 
     def _running(self, device):
         if self.running is None:
             z = lambda n, v: torch.full((n,), v, dtype=torch.float32, device=device)
-            self.running = {i: (z(n, 0.0), z(n, 1.0)) for i, n in ((1, self.cmid), (4, self.cmid), (7, self.cin))}
+            widths = [(1, self.cmid), (4, self.cmid), (7, self.cout)] + ([("shortcut", self.cout)] if self.projection else [])
+            self.running = {i: (z(n, 0.0), z(n, 1.0)) for i, n in widths}
             for i, (m, v) in getattr(self, "adopted_running", {}).items():   # statistics of the module the block came from
                 self.running[i][0].copy_(m)
                 self.running[i][1].copy_(v)
@@ -594,7 +660,8 @@ class BottleNeck:
 
     def _bn_fwd(self, idx, x, resid, y, mean, rstd, relu, ctx, strips=None):
         run = (None, None) if ctx.redundant else self._running(x.device)[idx]
-        hip.batchnorm_fwd(x, self.w_[f"residual_function.{idx}.weight"], self.w_[f"residual_function.{idx}.bias"],
+        name = self._BN_NAMES[idx]
+        hip.batchnorm_fwd(x, self.w_[f"{name}.weight"], self.w_[f"{name}.bias"],
                           resid, y, mean, rstd, run[0], run[1], ctx.workspace, self.eps, self.momentum, relu,
                           stream=ctx.stream, strip_stats=strips)
 
@@ -604,77 +671,99 @@ class BottleNeck:
         strips = None
         key = (tuple(x.shape), tuple(weight.shape), x.dtype)
         if key not in self._stats_ok:
-            self._stats_ok[key] = ctx.rows <= 8192 and hip.gemm_strip_stats_supported(hip.NT, x, weight, y)
+            self._stats_ok[key] = x.shape[0] <= 8192 and hip.gemm_strip_stats_supported(hip.NT, x, weight, y)
         if self._stats_ok[key]:
-            strips = ctx.buf("strips", (hip.strip_stats_workspace(ctx.rows, y.shape[1]),))
+            strips = ctx.buf("strips", (hip.strip_stats_workspace(x.shape[0], y.shape[1]),))
         hip.gemm(hip.NT, x, weight, y, stream=ctx.stream, strip_stats=strips)
         return strips
 
     def _implicit(self, ctx, mode):
-        return hip.conv3x3_supported(ctx.dtype, mode, ctx.batch, self.h, self.w, self.cmid, self.cmid)
+        return self.stride == 1 and hip.conv3x3_supported(ctx.dtype, mode, ctx.batch, self.h, self.w, self.cmid, self.cmid)
 
-    def _bind_image(self, ctx):
-        """A block taken over from a module does not know its image size: square images, side = sqrt(positions)."""
-        if self.h is None or self.w is None:
-            side = math.isqrt(ctx.seq)
-            if side * side != ctx.seq:
-                raise hip.HipKernelError(f"cannot infer a square image from {ctx.seq} positions: pass height= and width=")
-            self.h = self.w = side
+    def _shortcut_input(self, x, ctx, R2):
+        """Rows the projection shortcut reads: x itself, or the rows of every stride-th pixel."""
+        if self.stride == 1:
+            return x
+        xs = ctx.buf("xs", (R2, self.cin))
+        hip.subsample(x, xs, ctx.batch, self.h, self.w, self.cin, self.stride, stream=ctx.stream)
+        return xs
 
     def forward(self, x, st, ctx):
-        self._bind_image(ctx)
-        if ctx.seq != self.h * self.w:
-            raise hip.HipKernelError(f"activation has {ctx.seq} positions, the block expects {self.h}x{self.w}")
-        w, sm = self.w_, ctx.stream
+        R, R2, _, _ = self._rows(ctx)
+        w, sm, cm = self.w_, ctx.stream, self.cmid
         st["x0"] = x
         strips = self._conv1x1(x, w["residual_function.0.weight"], st["y1"], ctx)
         self._bn_fwd(1, st["y1"], None, st["a1"], st["mean1"], st["rstd1"], True, ctx, strips)
         if self._implicit(ctx, hip.CONV_FWD):
-            strips = ctx.buf("strips", (hip.strip_stats_workspace(ctx.rows, self.cmid),)) if ctx.rows <= 8192 else None
+            strips = ctx.buf("strips", (hip.strip_stats_workspace(R, cm),)) if R <= 8192 else None
             hip.conv3x3(hip.CONV_FWD, st["a1"], w["residual_function.3.weight"], st["y2"], ctx.batch, self.h, self.w,
-                        self.cmid, self.cmid, strip_stats=strips, stream=sm)
+                        cm, cm, strip_stats=strips, stream=sm)
         else:
-            col = ctx.buf("col", (ctx.rows, 9 * self.cmid))
-            hip.patch3x3(st["a1"], col, ctx.batch, self.h, self.w, self.cmid, stream=sm)
+            col = ctx.buf("col", (R2, 9 * cm))
+            hip.patch3x3(st["a1"], col, ctx.batch, self.h, self.w, cm, stride=self.stride, stream=sm)
             strips = self._conv1x1(col, w["conv2"], st["y2"], ctx)
         self._bn_fwd(4, st["y2"], None, st["a2"], st["mean2"], st["rstd2"], True, ctx, strips)
+        if self.projection:
+            # the shortcut first: its normalised output is the residual the last BatchNorm adds before the ReLU
+            sc = ctx.buf("sc", (R2, self.cout))
+            strips = self._conv1x1(self._shortcut_input(x, ctx, R2), w["shortcut.0.weight"], st["ys"], ctx)
+            self._bn_fwd("shortcut", st["ys"], None, sc, st["mean_s"], st["rstd_s"], False, ctx, strips)
+        else:
+            sc = x
         strips = self._conv1x1(st["a2"], w["residual_function.6.weight"], st["y3"], ctx)
-        self._bn_fwd(7, st["y3"], x, st["out"], st["mean3"], st["rstd3"], True, ctx, strips)
+        self._bn_fwd(7, st["y3"], sc, st["out"], st["mean3"], st["rstd3"], True, ctx, strips)
         return st["out"]
 
     def backward(self, d_out, d_x, st, ctx):
         w, g, sm, ws = self.w_, self.g_, ctx.stream, ctx.workspace
-        R, ci, cm = ctx.rows, self.cin, self.cmid
-        col, d_col = ctx.buf("col", (R, 9 * cm)), ctx.buf("d_col", (R, 9 * cm))
-        d_y3, d_res = ctx.buf("d_y3", (R, ci)), ctx.buf("d_res", (R, ci))
-        d_m0, d_m1 = ctx.buf("d_m0", (R, cm)), ctx.buf("d_m1", (R, cm))
-        bn = lambda idx, xk, mk, rk, dy, relu_out, dx, g_out: hip.batchnorm_bwd(
-            st[xk], w[f"residual_function.{idx}.weight"], st[mk], st[rk], dy, relu_out, dx, g_out,
-            g[f"residual_function.{idx}.weight"], g[f"residual_function.{idx}.bias"], ws, stream=sm)
-        # final ReLU + BN3; d_res keeps the masked gradient for the identity shortcut
+        R, R2, _, _ = self._rows(ctx)
+        ci, cm, co = self.cin, self.cmid, self.cout
+        col = ctx.buf("col", (R2, 9 * cm))
+        d_y3, d_res = ctx.buf("d_y3", (R2, co)), ctx.buf("d_res", (R2, co))
+        d_m0, d_m1 = ctx.buf("d_m0", (R2, cm)), ctx.buf("d_m1", (R2, cm))
+
+        def bn(idx, xk, mk, rk, dy, relu_out, dx, g_out):
+            name = self._BN_NAMES[idx]
+            hip.batchnorm_bwd(st[xk], w[f"{name}.weight"], st[mk], st[rk], dy, relu_out, dx, g_out,
+                              g[f"{name}.weight"], g[f"{name}.bias"], ws, stream=sm)
+        # final ReLU + BN3; d_res keeps the masked gradient for the shortcut
         bn(7, "y3", "mean3", "rstd3", d_out, st["out"], d_y3, d_res)
+        d_ys = d_xs = xs = None
+        if self.projection:
+            d_ys, d_xs = ctx.buf("d_ys", (R2, co)), ctx.buf("d_xs", (R2, ci))
+            bn("shortcut", "ys", "mean_s", "rstd_s", d_res, None, d_ys, None)
+            hip.gemm(hip.NN, d_ys, w["shortcut.0.weight"], d_xs, stream=sm)
+            xs = self._shortcut_input(st["x0"], ctx, R2)
         hip.gemm(hip.NN, d_y3, w["residual_function.6.weight"], d_m0, stream=sm)          # d_a2
         bn(4, "y2", "mean2", "rstd2", d_m0, st["a2"], d_m1, None)                          # d_y2
         # weight gradient of the 3x3 convolution: patch matrix gathered inside the GEMM, else built again here
         # (cheaper than stashing it)
         wgrad_implicit = (self._implicit(ctx, hip.CONV_DGRAD) and cm % 128 == 0 and R % 32 == 0 and 32 // self.w + 1 <= self.h)
         if not wgrad_implicit:
-            hip.patch3x3(st["a1"], col, ctx.batch, self.h, self.w, cm, stream=sm)
+            hip.patch3x3(st["a1"], col, ctx.batch, self.h, self.w, cm, stride=self.stride, stream=sm)
         d_a1, d_m2 = ctx.buf("d_m0", (R, cm)), ctx.buf("d_m2", (R, cm))
         if self._implicit(ctx, hip.CONV_DGRAD):
             hip.conv3x3(hip.CONV_DGRAD, d_m1, w["residual_function.3.weight"], d_a1, ctx.batch, self.h, self.w, cm, cm,
                         stream=sm)
         else:
+            d_col = ctx.buf("d_col", (R2, 9 * cm))
             hip.gemm(hip.NN, d_m1, w["conv2"], d_col, stream=sm)
-            hip.patch3x3(d_col, d_a1, ctx.batch, self.h, self.w, cm, adjoint=True, stream=sm)
+            hip.patch3x3(d_col, d_a1, ctx.batch, self.h, self.w, cm, adjoint=True, stride=self.stride, stream=sm)
         bn(1, "y1", "mean1", "rstd1", d_a1, st["a1"], d_m2, None)                          # d_y1
-        hip.gemm(hip.NN, d_m2, w["residual_function.0.weight"], d_x, epilogue=hip.EPI_RESIDUAL, resid=d_res, stream=sm)
-        # the three weight gradients in one launch: 68 output tiles over 6272 rows, cut along the rows
-        hip.gemm_grouped([hip.gemm_desc(hip.TN, d_y3, st["a2"], g["residual_function.6.weight"], accumulate=True),
-                          hip.gemm_desc(hip.TN, d_m1, st["a1"], g["conv2"], accumulate=True, conv=(self.h, self.w))
-                          if wgrad_implicit else hip.gemm_desc(hip.TN, d_m1, col, g["conv2"], accumulate=True),
-                          hip.gemm_desc(hip.TN, d_m2, st["x0"], g["residual_function.0.weight"], accumulate=True)],
-                         stream=sm, splitk_ws=ctx.buf("splitk", (8 * (ci * cm + 9 * cm * cm + cm * ci),)))
+        if self.projection and self.stride > 1:
+            hip.gemm(hip.NN, d_m2, w["residual_function.0.weight"], d_x, stream=sm)
+            hip.subsample(d_xs, d_x, ctx.batch, self.h, self.w, ci, self.stride, adjoint=True, stream=sm)
+        else:
+            hip.gemm(hip.NN, d_m2, w["residual_function.0.weight"], d_x, epilogue=hip.EPI_RESIDUAL,
+                     resid=d_xs if self.projection else d_res, stream=sm)
+        # the weight gradients in one launch: few output tiles over thousands of rows, cut along the rows
+        descs = [hip.gemm_desc(hip.TN, d_y3, st["a2"], g["residual_function.6.weight"], accumulate=True),
+                 hip.gemm_desc(hip.TN, d_m1, st["a1"], g["conv2"], accumulate=True, conv=(self.h, self.w))
+                 if wgrad_implicit else hip.gemm_desc(hip.TN, d_m1, col, g["conv2"], accumulate=True),
+                 hip.gemm_desc(hip.TN, d_m2, st["x0"], g["residual_function.0.weight"], accumulate=True)]
+        if self.projection:
+            descs.append(hip.gemm_desc(hip.TN, d_ys, xs, g["shortcut.0.weight"], accumulate=True))
+        hip.gemm_grouped(descs, stream=sm, splitk_ws=ctx.buf("splitk", (8 * self._wgrad_elems(),)))
         return d_x
 
 

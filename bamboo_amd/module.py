@@ -373,9 +373,11 @@ class PipelineModule:
         stash) plus, per slot, the input of every layer group and the stage output."""
         layers = self.func_buckets[stage_id]
         ckpt = self.activation_checkpoint_interval > 0
+        seqs = self._stage_seqs(stage_id, ctx)
         plans, total = [], 0
-        for layer in layers:
+        for li, layer in enumerate(layers):
             plan = []
+            ctx.seq = seqs[li]
             for name, shape, dtype in layer.stash_specs(ctx):
                 nbytes = math.prod(shape) * torch.empty((), dtype=dtype).element_size()
                 plan.append((name, shape, dtype, total, nbytes))
@@ -399,14 +401,16 @@ class PipelineModule:
         if ckpt:
             groups = self._checkpoint_groups(stage_id)
             es = torch.empty((), dtype=self.dtype).element_size()
-            sizes = [ctx.rows * layers[a].feature_dim for a, _ in groups] + [ctx.rows * layers[-1].out_features]
+            shapes = [(ctx.batch * seqs[a], layers[a].feature_dim) for a, _ in groups] + \
+                     [(ctx.batch * seqs[-1], layers[-1].out_features)]
+            sizes = [r * c for r, c in shapes]
             per_slot = sum((n * es + 255) // 256 * 256 for n in sizes)
             keep = torch.empty(per_slot * slots, dtype=torch.uint8, device=self.device)
             kept = []
             for s in range(slots):
                 lo, bufs = s * per_slot, []
-                for n in sizes:
-                    bufs.append(keep[lo: lo + n * es].view(self.dtype).view(ctx.rows, n // ctx.rows))
+                for n, shape in zip(sizes, shapes):
+                    bufs.append(keep[lo: lo + n * es].view(self.dtype).view(shape))
                     lo += (n * es + 255) // 256 * 256
                 kept.append(bufs)          # [group inputs ..., stage output]
             self._kept = getattr(self, "_kept", {})
@@ -415,7 +419,32 @@ class PipelineModule:
             nbytes_total += per_slot * slots
             table = [table[0]] * slots     # every slot works in the one shared set
         self._stash[stage_id] = table
+        ctx.seq = seqs[0]
         return nbytes_total
+
+    def _stage_seqs(self, stage_id, ctx=None):
+        """Positions per sample in front of every layer of a built stage and behind its last one (a down-sampling
+        bottleneck changes them); set by :meth:`prepare_context`."""
+        seqs = getattr(self, "stage_seq", {}).get(stage_id)
+        if seqs is None:
+            if ctx is None:
+                raise PipelineError(f"stage {stage_id}: prepare_context has not seen this stage")
+            seqs = self._chain_seqs(stage_id, ctx.seq)
+        return seqs
+
+    def _chain_seqs(self, stage_id, seq):
+        seqs = [seq]
+        for layer in self.func_buckets[stage_id]:
+            out_seq = getattr(layer, "out_seq", None)
+            seqs.append(out_seq(seqs[-1]) if out_seq is not None else seqs[-1])
+        self.stage_seq = getattr(self, "stage_seq", {})
+        self.stage_seq[stage_id] = seqs
+        return seqs
+
+    def stage_io_shapes(self, stage_id, batch):
+        """((rows, features) of the stage's input, (rows, features) of its output) once its context is prepared."""
+        seqs, layers = self._stage_seqs(stage_id), self.func_buckets[stage_id]
+        return (batch * seqs[0], layers[0].feature_dim), (batch * seqs[-1], layers[-1].out_features)
 
     # ------------------------------------------------------------------ execution
     def forward(self, forward_input, stage_id, slot=0, ctx=None, defer=False, layers=None):
@@ -428,6 +457,7 @@ class PipelineModule:
             raise Exception(f"Unregistered stage id {stage_id}")
         x = forward_input
         stash = self._stash[stage_id][slot]
+        seqs = self._stage_seqs(stage_id, ctx)
         if layers is not None:
             if self.activation_checkpoint_interval != 0:
                 raise PipelineError("a forward cut into layer ranges needs the full stash (no activation checkpointing)")
@@ -436,6 +466,7 @@ class PipelineModule:
                 self.micro_offset += 1
             ctx.defer = defer
             for i in range(a, b):
+                ctx.seq = seqs[i]
                 x = stage_layers[i].forward(x, stash[i], ctx)
             ctx.defer = False
             return x
@@ -443,7 +474,8 @@ class PipelineModule:
         self.micro_offset += 1
         if self.activation_checkpoint_interval == 0:
             ctx.defer = defer
-            for layer, st in zip(layers, stash):
+            for i, (layer, st) in enumerate(zip(layers, stash)):
+                ctx.seq = seqs[i]
                 x = layer.forward(x, st, ctx)
             ctx.defer = False
             return x
@@ -452,6 +484,7 @@ class PipelineModule:
             hip.cast(x, kept[g], stream=ctx.stream)   # same-type copy: the group's input outlives the work stash
             x = kept[g]
             for i in range(a, b):
+                ctx.seq = seqs[i]
                 x = layers[i].forward(x, stash[i], ctx)
         hip.cast(x, kept[-1], stream=ctx.stream)
         return kept[-1]
@@ -463,6 +496,7 @@ class PipelineModule:
         layers = self.func_buckets[stage_id]
         ctx.deferred = deferred and self.activation_checkpoint_interval == 0
         stash = self._stash[stage_id][slot]
+        seqs = self._stage_seqs(stage_id, ctx)
         n = len(layers)
         d = grad_output
         groups = self._checkpoint_groups(stage_id) if self.activation_checkpoint_interval > 0 else [(0, n)]
@@ -474,10 +508,12 @@ class PipelineModule:
                 was, ctx.redundant = ctx.redundant, True
                 x = self._kept[stage_id][slot][g]
                 for i in range(a, b):
+                    ctx.seq = seqs[i]
                     x = layers[i].forward(x, stash[i], ctx)
                 ctx.redundant = was
             for i in range(b - 1, a - 1, -1):
-                dst = grad_input if i == 0 else ctx.buf(f"d_layer{i % 2}", (grad_output.shape[0], layers[i].feature_dim))
+                dst = grad_input if i == 0 else ctx.buf(f"d_layer{i % 2}", (ctx.batch * seqs[i], layers[i].feature_dim))
+                ctx.seq = seqs[i]
                 layers[i].backward(d, dst, stash[i], ctx)
                 d = dst
         ctx.deferred = False
@@ -488,8 +524,12 @@ class PipelineModule:
         (``forward_only``: a lane that only runs redundant forwards needs no backward scratch)."""
         ctx = StageContext(batch, seq, self.dtype, self.device, stream)
         ws = 0
-        for sid in stage_ids:
-            for layer in self.func_buckets[sid]:
+        for n, sid in enumerate(stage_ids):
+            # the first stage of the list takes ``seq`` positions per sample, each later one what its predecessor
+            # in the list leaves (consecutive stages: own, then shadowed / absorbed)
+            seqs = self._chain_seqs(sid, seq if n == 0 else self.stage_seq[stage_ids[n - 1]][-1])
+            for li, layer in enumerate(self.func_buckets[sid]):
+                ctx.seq = seqs[li]
                 if hasattr(layer, "forward_scratch_specs"):
                     ctx.ensure_scratch(layer.forward_scratch_specs(ctx))
                 ws = max(ws, layer.workspace_elems())
@@ -499,4 +539,5 @@ class PipelineModule:
                 h = (ctx.rows, layer.feature_dim)
                 ctx.ensure_scratch([("d_layer0", h, self.dtype), ("d_layer1", h, self.dtype)])
         ctx.ensure_workspace(ws)
+        ctx.seq = seq
         return ctx

@@ -39,10 +39,12 @@ class AllReduceException(Exception):
 
 class SeededActivationQueue:
     def __init__(self, shape, dtype, micro_batches, stage_ids, seed=1138, grad_mode="queue", device="cuda:0",
-                 key_len_range=None):
-        """shape: activation shape ``[micro_batch, seq, hidden]`` (same for every stage boundary);
-        stage_ids: stages whose *outputs* this queue must answer for (own stage and, for failover,
-        the shadowed stage)."""
+                 key_len_range=None, out_shapes=None):
+        """shape: activation shape ``[micro_batch, seq, hidden]`` the stage receives, and the shape of every stage
+        output unless ``out_shapes = {stage_id: shape}`` says otherwise (a down-sampling ResNet stage leaves fewer
+        positions and more channels than it takes); stage_ids: stages whose *outputs* this queue must answer
+        for (own stage and, for failover, the shadowed stage)."""
+        self.out_shapes = {sid: tuple(s) for sid, s in (out_shapes or {}).items()}
         if grad_mode not in ("queue", "mse"):
             raise ValueError(grad_mode)
         self.shape, self.dtype, self.M = tuple(shape), dtype, micro_batches
@@ -63,11 +65,12 @@ class SeededActivationQueue:
                 self.key_lens.append(torch.randint(lo, hi + 1, (shape[0],), generator=g, dtype=torch.int32).to(self.device))
         self.grads, self.targets = {}, {}
         for sid in stage_ids:
+            out = self.out_shapes.get(sid, self.shape)
             if grad_mode == "queue":
-                self.grads[sid] = [self._randn(("grad", sid, k)) for k in range(micro_batches)]
+                self.grads[sid] = [self._randn(("grad", sid, k), out) for k in range(micro_batches)]
             else:
-                self.targets[sid] = [self._randn(("target", sid, k)) for k in range(micro_batches)]
-                self.grads[sid] = [torch.zeros(self.shape, dtype=dtype, device=self.device) for _ in range(micro_batches)]
+                self.targets[sid] = [self._randn(("target", sid, k), out) for k in range(micro_batches)]
+                self.grads[sid] = [torch.zeros(out, dtype=dtype, device=self.device) for _ in range(micro_batches)]
 
     _TAGS = {"act": 11, "grad": 23, "target": 37, "len": 41}
 
@@ -78,9 +81,9 @@ class SeededActivationQueue:
             h = (h * 1000003 + self._TAGS.get(t, t) + 7) % (2 ** 31 - 1)
         return h
 
-    def _randn(self, tag):
+    def _randn(self, tag, shape=None):
         g = torch.Generator().manual_seed(self._tag_seed(tag))
-        return torch.randn(self.shape, generator=g, dtype=torch.float32).to(self.dtype).to(self.device)
+        return torch.randn(shape or self.shape, generator=g, dtype=torch.float32).to(self.dtype).to(self.device)
 
     # -------------------------------------------------------------- test hooks
     def set_grads(self, stage_id, tensors):

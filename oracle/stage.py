@@ -66,6 +66,10 @@ class OracleStage:
         """``tail``: the model ends with the reference script's two extra layers (final LayerNorm, sum over the hidden
         dimension; transformer.py:250): ``parts[-1]`` then counts them, and the last stage applies them."""
         self.tail = tail
+        # a list of BottleneckCfg gives every block of the model its own shape (down-sampling / widening blocks)
+        self.layer_cfgs = list(cfg) if isinstance(cfg, (list, tuple)) else None
+        if self.layer_cfgs is not None:
+            cfg = self.layer_cfgs[0]
         self.cfg, self.parts, self.stage_id, self.M = cfg, parts, stage_id, micro_batches
         self.S = len(parts) - 1
         self.dtype = dtype
@@ -83,6 +87,9 @@ class OracleStage:
         self.adam_state = {}
         self.step_count = 0
 
+    def block_cfg(self, layer_idx):
+        return self.cfg if self.layer_cfgs is None else self.layer_cfgs[layer_idx]
+
     def build(self, stage):
         conv = isinstance(self.cfg, olayers.BottleneckCfg)
         layers = []
@@ -97,7 +104,7 @@ class OracleStage:
                 layers.append({})
                 continue
             if conv:
-                p = olayers.init_bottleneck_params(self.cfg, self.base_seed + li, dtype=self.dtype)
+                p = olayers.init_bottleneck_params(self.block_cfg(li), self.base_seed + li, dtype=self.dtype)
             else:
                 p = olayers.init_params(self.cfg, self.base_seed + li, dtype=self.dtype)
             layers.append({k: v.requires_grad_(True) for k, v in p.items()})
@@ -112,9 +119,9 @@ class OracleStage:
             b, hw, c = x.shape
             side = int(round(hw ** 0.5))
             y = x.view(b, side, side, c).permute(0, 3, 1, 2)
-            for p, m in zip(self.params[stage], masks):
-                y = olayers.bottleneck(y, p, self.cfg, m)
-            return y.permute(0, 2, 3, 1).reshape(b, hw, c)
+            for li, (p, m) in enumerate(zip(self.params[stage], masks)):
+                y = olayers.bottleneck(y, p, self.block_cfg(self.parts[stage] + li), m)
+            return y.permute(0, 2, 3, 1).reshape(b, -1, y.shape[1])
         for li, (p, m) in enumerate(zip(self.params[stage], masks)):
             if set(p) == {"a_2", "b_2"}:
                 x = olayers.script_tail(x, p, self.cfg.ln, self.cfg.eps)

@@ -101,3 +101,33 @@ def test_bottleneck_module_is_taken_over_with_layouts_and_running_statistics():
     model.load_layer_tensor(0, "residual_function.3.weight", new)
     assert torch.equal(model.layer_state_dict(0)["residual_function.3.weight"], new)
     assert float(blk._running("cpu")[4][0][0]) == 0.5
+
+
+def test_downsampling_bottleneck_module_is_taken_over_with_its_shortcut():
+    """A block with the projection shortcut (resnet.py:68-72): stride read off the 3x3 convolution, the shortcut's
+    parameters follow the residual function's in the reference's registration order, its BatchNorm statistics come
+    along; the partition by parameter count sees the extra parameters."""
+    torch.manual_seed(3)
+    ref = RefBottleNeck(64, 32, stride=2)
+    with torch.no_grad():
+        ref.shortcut[1].running_var.mul_(3.0)
+    model = PipelineModule([ref, RefBottleNeck(128, 32)], num_stages=1, stage_id=0, dtype=torch.float32, device="cpu")
+    blk, plain = model.func_buckets[0]
+    assert (blk.cin, blk.cmid, blk.cout, blk.stride, blk.projection) == (64, 32, 128, 2, True)
+    assert (plain.stride, plain.projection, plain.feature_dim, plain.out_features) == (1, False, 128, 128)
+    assert blk.out_seq(64) == 16 and blk.out_seq(49) == 16 and plain.out_seq(49) == 49
+    sd = model.layer_state_dict(0)
+    ref_params = dict(ref.named_parameters())
+    assert list(sd) == [k for k in ref.state_dict() if k in ref_params]
+    assert list(sd)[-3:] == ["shortcut.0.weight", "shortcut.1.weight", "shortcut.1.bias"]
+    for k, v in sd.items():
+        assert v.shape == ref_params[k].shape and torch.equal(v, ref_params[k].detach()), k
+    assert float(blk._running("cpu")["shortcut"][1][0]) == 3.0
+    assert blk.num_params() == sum(p.numel() for p in ref.parameters())
+
+
+def test_bottleneck_whose_shortcut_contradicts_its_shape_is_refused():
+    ref = RefBottleNeck(64, 16)                      # identity shortcut ...
+    ref.residual_function[3].stride = (2, 2)         # ... but a stride: the reference would have built a projection
+    with pytest.raises(PipelineError, match="projection shortcut"):
+        PipelineModule([ref], num_stages=1, stage_id=0, dtype=torch.float32, device="cpu")

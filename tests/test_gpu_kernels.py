@@ -430,27 +430,57 @@ def test_batchnorm_fwd_bwd(hiplib, dtype, rows, cols, relu, with_resid):
     assert torch.equal(y, y2) and torch.equal(rm, rm2)
 
 
+@pytest.mark.parametrize("stride", [1, 2, 3])
 @pytest.mark.parametrize("dtype", DTYPES)
-def test_patch3x3_and_adjoint(hiplib, dtype):
+def test_patch3x3_and_adjoint(hiplib, dtype, stride):
+    """Patch matrix of nn.Conv2d(k=3, stride, padding=1) against torch's unfold, the product with the weight against
+    conv2d, the adjoint against fold; odd image sides, so the last strided pixel's patch leaves the image."""
+    F = torch.nn.functional
     n, h, w, c = 3, 5, 7, 16
+    ho, wo = (h - 1) // stride + 1, (w - 1) // stride + 1
     x = randn(n * h * w, c, dtype=dtype, seed=38)
-    col = torch.empty(n * h * w, 9 * c, dtype=dtype, device=DEV)
-    hiplib.patch3x3(x, col, n, h, w, c)
+    col = torch.empty(n * ho * wo, 9 * c, dtype=dtype, device=DEV)
+    hiplib.patch3x3(x, col, n, h, w, c, stride=stride)
     xn = x.float().cpu().view(n, h, w, c).permute(0, 3, 1, 2)
-    ref = torch.nn.functional.unfold(xn, 3, padding=1)                      # [n, c*9, h*w], (c, tap) order
-    ref = ref.view(n, c, 9, h * w).permute(0, 3, 2, 1).reshape(n * h * w, 9 * c)
+    ref = F.unfold(xn, 3, padding=1, stride=stride)                         # [n, c*9, ho*wo], (c, tap) order
+    assert ref.shape[2] == ho * wo
+    ref = ref.view(n, c, 9, ho * wo).permute(0, 3, 2, 1).reshape(n * ho * wo, 9 * c)
     assert torch.equal(col.float().cpu(), ref)
     # conv3x3 == patches @ W^T with W in [out, tap, in] order
     wt = randn(8, c, 3, 3, seed=39).cpu()
-    conv = torch.nn.functional.conv2d(xn, wt, padding=1).permute(0, 2, 3, 1).reshape(n * h * w, 8)
+    conv = F.conv2d(xn, wt, padding=1, stride=stride).permute(0, 2, 3, 1).reshape(n * ho * wo, 8)
     assert rel_err(col.float().cpu() @ wt.permute(0, 2, 3, 1).reshape(8, 9 * c).t(), conv) < 1e-5
     # adjoint: <patch(x), d> == <x, adjoint(d)>
-    d = randn(n * h * w, 9 * c, dtype=dtype, seed=40)
-    back = torch.empty_like(x)
-    hiplib.patch3x3(d, back, n, h, w, c, adjoint=True)
-    dn = d.float().cpu().view(n, h * w, 9, c).permute(0, 3, 2, 1).reshape(n, c * 9, h * w)
-    fold = torch.nn.functional.fold(dn, (h, w), 3, padding=1).permute(0, 2, 3, 1).reshape(n * h * w, c)
+    d = randn(n * ho * wo, 9 * c, dtype=dtype, seed=40)
+    back = torch.full_like(x, 7.0)      # every input pixel is written, also those no patch reads
+    hiplib.patch3x3(d, back, n, h, w, c, adjoint=True, stride=stride)
+    dn = d.float().cpu().view(n, ho * wo, 9, c).permute(0, 3, 2, 1).reshape(n, c * 9, ho * wo)
+    fold = F.fold(dn, (h, w), 3, padding=1, stride=stride).permute(0, 2, 3, 1).reshape(n * h * w, c)
     assert rel_err(back, fold) < (1e-6 if dtype == torch.float32 else 1e-2)
+    with pytest.raises(hiplib.HipKernelError):
+        hiplib.patch3x3(x, col[:-1], n, h, w, c, stride=stride)
+
+
+@pytest.mark.parametrize("stride", [1, 2])
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_subsample_and_adjoint(hiplib, dtype, stride):
+    """Rows a strided 1x1 convolution reads (bit-exact against slicing), and the adjoint added in place."""
+    n, h, w, c = 2, 7, 6, 24
+    ho, wo = (h - 1) // stride + 1, (w - 1) // stride + 1
+    x = randn(n * h * w, c, dtype=dtype, seed=41)
+    xs = torch.empty(n * ho * wo, c, dtype=dtype, device=DEV)
+    hiplib.subsample(x, xs, n, h, w, c, stride)
+    ref = x.view(n, h, w, c)[:, ::stride, ::stride].reshape(n * ho * wo, c)
+    assert torch.equal(xs, ref)
+    base = randn(n * h * w, c, dtype=dtype, seed=42)
+    d = randn(n * ho * wo, c, dtype=dtype, seed=43)
+    got = base.clone()
+    hiplib.subsample(d, got, n, h, w, c, stride, adjoint=True)
+    want = base.float().view(n, h, w, c).clone()
+    want[:, ::stride, ::stride] += d.float().view(n, ho, wo, c)
+    assert torch.equal(got, want.to(dtype).view(n * h * w, c))
+    with pytest.raises(hiplib.HipKernelError):
+        hiplib.subsample(x, xs[:-1], n, h, w, c, stride)
 
 
 CONV_SHAPES = [(4, 5, 7, 64, 64),        # 140 pixels: one ragged row tile, one k-tile per tap

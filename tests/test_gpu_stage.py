@@ -342,6 +342,90 @@ def test_resnet_stage_matches_oracle_with_rc(hiplib, dtype, cin, cmid):
         assert float(layer.running[1][0].abs().max()) > 0
 
 
+DOWNSAMPLING_NET = [  # (in, mid, stride) of every block: widening, down-sampling and identity-shortcut blocks mixed
+    (32, 16, 1), (64, 16, 1),            # stage 0: projection 32 -> 64, identity
+    (64, 32, 2), (128, 32, 1),           # stage 1: 16x16 -> 8x8 with 64 -> 128 channels, identity
+    (128, 64, 1), (256, 64, 2),          # stage 2: widening projection at stride 1, then 8x8 -> 4x4
+    (256, 64, 1), (256, 64, 1)]          # stage 3
+# one block per stage: what bf16 storage between the kernels leaves of a gradient that has crossed two blocks
+# forward and two backward stays inside the 2e-2 bar (across four blocks it reaches 1.8 % on the activations alone)
+SHALLOW_DOWNSAMPLING_NET = [(32, 16, 1), (64, 32, 2), (128, 64, 2), (256, 64, 1)]
+
+
+@pytest.mark.parametrize("dtype,net,dead_from", [(torch.float32, DOWNSAMPLING_NET, None), (torch.float32, DOWNSAMPLING_NET, 1),
+                                                 (torch.bfloat16, DOWNSAMPLING_NET, None),
+                                                 (torch.bfloat16, SHALLOW_DOWNSAMPLING_NET, 1)],
+                         ids=["fp32-rc", "fp32-failover", "bf16-rc", "bf16-failover"])
+def test_resnet_stage_with_projection_shortcuts_matches_oracle(hiplib, dtype, net, dead_from):
+    """Bottleneck blocks with the projection shortcut (conv1x1(stride) + BatchNorm, resnet.py:68-72) and a stride on
+    the 3x3 convolution: the own stage halves the image and doubles the channels, the shadowed stage widens at
+    stride 1 and / or halves again, so rows and features differ at every stage boundary (and, in the two-block
+    stages, inside a stage).  Outputs, input gradients and all parameter gradients against the conv2d / batch_norm
+    oracle, with redundant forwards, and through a failover that promotes the shadowed stage."""
+    from bamboo_amd import BottleNeck
+    S, sid, mb, M, side = 4, 1, 8, 4, 16     # the smallest BatchNorm still sees 128 pixels
+    L = len(net) // S
+    specs = [LayerSpec(BottleNeck, ci, cm, stride=st_, height=None, width=None) for ci, cm, st_ in net]
+    model = PipelineModule(specs, num_stages=S, partition_method="uniform", stage_id=sid, dtype=dtype, device=DEV)
+    seq_of = lambda n_blocks: side * side // 4 ** sum(st_ == 2 for _, _, st_ in net[:n_blocks])
+    shapes = {s_: (mb, seq_of((s_ + 1) * L), 4 * net[(s_ + 1) * L - 1][1]) for s_ in (sid, sid + 1)}
+    q = SeededActivationQueue((mb, side * side, 64), dtype, M, stage_ids=[sid, sid + 1], seed=19, device=DEV, out_shapes=shapes)
+    cfg = {"train_micro_batch_size_per_gpu": mb, "gradient_accumulation_steps": M, "bf16": {"enabled": dtype == torch.bfloat16}}
+    engine, _, _, _ = bamboo_amd.initialize(model=model, config=cfg, redundancy_level=1, eager_recovery=True,
+                                            activation_queue=q, install_signal_handler=False)
+    assert model.func_buckets[sid][0].projection and model.func_buckets[sid][0].stride == 2
+    if L == 2:
+        assert model.stage_seq[sid] == [256, 64, 64] and model.stage_seq[sid + 1] == [64, 64, 16]
+        assert shapes == {sid: (mb, 64, 128), sid + 1: (mb, 16, 256)}
+    ocfgs = [ol.BottleneckCfg(in_channels=ci, mid_channels=cm, stride=st_) for ci, cm, st_ in net]
+    st = OracleStage(ocfgs, [i * L for i in range(S + 1)], sid, M, dtype=torch.float64, redundancy_level=1, eager=True)
+    for s_ in list(st.params):
+        sp = engine.module.stage_params[s_]
+        named = sp.named(sp.compute)
+        assert set(named) == set(st.named_params(s_))
+        for key, t in st.named_params(s_).items():
+            src = named[key].double().cpu()
+            if t.dim() == 4:      # arena keeps [O, kh, kw, I]; the oracle the reference's [O, I, kh, kw]
+                src = src.view(t.shape[0], t.shape[2], t.shape[3], t.shape[1]).permute(0, 3, 1, 2)
+            with torch.no_grad():
+                t.copy_(src.reshape(t.shape))
+    peer = OraclePeer([a.double().cpu() for a in q.activations], M,
+                      grads={s_: [g.double().cpu() for g in gs] for s_, gs in q.grads.items()})
+    if dead_from is not None:
+        peer.dead_from, peer.dead_stage = dead_from, sid
+        q.preempt_successor(dead_from, sid)
+    rel_err.lowp = dtype == torch.bfloat16
+    keep = {}
+    with NoStep(engine):
+        clean = engine._clean_pipe_buffers
+        engine._clean_pipe_buffers = lambda: (keep.update({k: list(v) for k, v in engine.pipe_buffers.items()}), clean())
+        engine.train_batch()
+    torch.cuda.synchronize()
+    if dtype == torch.bfloat16:
+        peer.relu_masks = relu_decisions(engine, [sid, sid + 1], M, mb)
+    bufs, info = st.run_batch(peer, optimizer_step=False)
+    assert (info["failed_step"] is not None) == (dead_from is not None)
+    assert engine.stage_ids == ([sid, sid + 1] if dead_from is not None else [sid])
+    t_act = 1e-5 if dtype == torch.float32 else 2e-2
+    t_grad = 1e-4 if dtype == torch.float32 else 2e-2
+    for k in range(M):
+        for s_ in (sid, sid + 1):
+            want = bufs["out"][(s_, k)].detach()
+            assert rel_err(keep[f"output_{s_}"][k], want.reshape(-1, want.shape[-1])) < t_act, (s_, k)
+        want = bufs["sent_grad"][(sid, k)]
+        assert rel_err(keep[f"input_grad_{sid}"][k], want.reshape(-1, want.shape[-1])) < t_grad, k
+    for s_ in engine.stage_ids:
+        ref = st.named_grads(s_)
+        for name, g in engine.module.get_named_grad(s_):
+            r = ref[name]
+            if r.dim() == 4:
+                r = r.permute(0, 2, 3, 1)
+            assert rel_err(g, r.reshape(g.shape), grad_floor(ref)) < t_grad, (s_, name)
+    # the shortcut's BatchNorm keeps running statistics like the others
+    own = engine.module.func_buckets[sid][0]
+    assert float(own.running["shortcut"][0].abs().max()) > 0
+
+
 @pytest.mark.parametrize("dead_from", [0, 2])
 def test_lazy_recovery_failover(hiplib, dead_from):
     """redundancy_level=1 without eager recovery: no redundant forwards (only pings); the shadow stage exists
@@ -454,18 +538,26 @@ def test_activation_checkpointing_equals_full_stash(hiplib, interval, rc_stream)
         assert torch.equal(a.exp_avg, b.exp_avg) and torch.equal(a.exp_avg_sq, b.exp_avg_sq)
 
 
-def test_activation_checkpointing_resnet_keeps_running_statistics(hiplib):
+@pytest.mark.parametrize("net", ["identity", "down-sampling"])
+def test_activation_checkpointing_resnet_keeps_running_statistics(hiplib, net):
     """Bottleneck stage with checkpoint groups of one block: gradients, outputs and the BatchNorm running
-    statistics (updated once per forward, not again by the recomputation) equal the full stash bit for bit."""
+    statistics (updated once per forward, not again by the recomputation) equal the full stash bit for bit; also
+    where the kept group inputs differ in rows and channels (blocks with a stride and a projection shortcut)."""
     from bamboo_amd import BottleNeck
     cin, cmid, side, L, S, sid, mb, M = 64, 16, 6, 2, 4, 1, 4, 4
+    blocks = [(cin, cmid, 1)] * (L * S) if net == "identity" else DOWNSAMPLING_NET
+    if net != "identity":
+        side = 16
+    out_shapes = {s_: (mb, side * side // 4 ** sum(st_ == 2 for _, _, st_ in blocks[:(s_ + 1) * L]), 4 * blocks[(s_ + 1) * L - 1][1])
+                  for s_ in (sid, sid + 1)}
     dtype = torch.bfloat16
     runs = []
     for every in (0, 1):
-        specs = [LayerSpec(BottleNeck, cin, cmid, height=side, width=side) for _ in range(L * S)]
+        specs = [LayerSpec(BottleNeck, ci, cm, stride=st_, height=None, width=None) for ci, cm, st_ in blocks]
         model = PipelineModule(specs, num_stages=S, partition_method="uniform", stage_id=sid, dtype=dtype, device=DEV,
                                activation_checkpoint_interval=every)
-        q = SeededActivationQueue((mb, side * side, cin), dtype, M, stage_ids=[sid, sid + 1], seed=9, device=DEV)
+        q = SeededActivationQueue((mb, side * side, cin), dtype, M, stage_ids=[sid, sid + 1], seed=9, device=DEV,
+                                  out_shapes=out_shapes)
         cfg = {"train_micro_batch_size_per_gpu": mb, "gradient_accumulation_steps": M, "bf16": {"enabled": True}}
         engine, _, _, _ = bamboo_amd.initialize(model=model, config=cfg, redundancy_level=1, eager_recovery=True,
                                                 activation_queue=q, install_signal_handler=False)
