@@ -528,8 +528,13 @@ class PipelineEngine:
         # a redundant forward's stash is read by a backward pass only after a failover: it leaves out
         # what that backward pass can produce itself
         self._deferred[(stage_id, buffer_id)] = redundant
+        note_rc = getattr(self.queue, "note_rc", None) if redundant else None
+        if note_rc is not None:      # a queue that keeps a timeline of the redundant work (measurement only)
+            note_rc(buffer_id, 0, "begin", ctx.stream)
         out = self._graphed(key, ctx.stream, lambda: self.module.forward(inputs, stage_id, slot=buffer_id, ctx=ctx,
                                                                          defer=redundant))
+        if note_rc is not None:
+            note_rc(buffer_id, len(self.module.func_buckets[stage_id]), "end", ctx.stream)
         self.pipe_buffers[out_key][buffer_id] = out
         if not redundant and self.rc_stream is not None:
             self._fwd_done[buffer_id].record(self.main_stream)
@@ -595,7 +600,12 @@ class PipelineEngine:
             ctx.key_len = self.queue.key_len(k)
             ctx.redundant = True
             ctx.dropout_base = (self.module.base_seed, self.global_steps, k)
+            note_rc = getattr(self.queue, "note_rc", None)
+            if note_rc is not None:
+                note_rc(k, i, "begin", self.rc_stream)
             out = self.module.forward(x, nxt, slot=k, ctx=ctx, defer=True, layers=(i, i + 1))
+            if note_rc is not None:
+                note_rc(k, i + 1, "end", self.rc_stream)
             if i + 1 == n_layers:
                 self.pipe_buffers[f"output_{nxt}"][k] = out
                 self._rc_pending.pop(0)

@@ -238,6 +238,7 @@ class PacedActivationQueue(SeededActivationQueue):
         self.batch_seconds = None  # of the last finished batch: from its start to the pipeline's end
         self.batches = 0           # batches since the last reset()
         self._base = None
+        self.rc_marks = None       # set to a list to collect (micro-batch, layer, "begin" | "end", seconds()) of redundant work
 
     def reset(self):
         """The next batch starts a new run: GPU drained, empty pipeline, time zero."""
@@ -272,6 +273,16 @@ class PacedActivationQueue(SeededActivationQueue):
             ev.synchronize()
             return base.elapsed_time(ev) * 1e-3
         self.clock.note_done(kind, k, when)
+
+    def note_rc(self, k, layer, what, stream):
+        """Called by the engine around every piece of a redundant forward it issues (layers ``begin`` .. ``end``
+        of micro-batch ``k``); collected only while ``rc_marks`` is a list."""
+        if self.rc_marks is None or self._base is None:
+            return
+        ev = torch.cuda.Event(enable_timing=True)
+        ev.record(stream)
+        base = self._base
+        self.rc_marks.append((k, layer, what, lambda: base.elapsed_time(ev) * 1e-3))
 
     def _wait_until(self, t):
         target = self._t0 + t

@@ -120,7 +120,46 @@ def measure_pass_times(engine, q):
     return med(durs["F"]), med(durs["B"])
 
 
-def paced_leg(cfg, rc, rc_issue, t_fwd, t_bwd, steps, warmup):
+def paced_timeline(q, t_start):
+    """Markdown rows of the stage's last batch inside the pipeline model: every own pass (when its input arrived,
+    when it ran) and every piece of redundant forward work (when it ran, and beside which own pass, if any)."""
+    c = q.clock
+    sid = q.stage_id
+    ms = lambda t: f"{(t - t_start) * 1e3:8.2f}"
+    own, prev = [], c.t0
+    for kind, k in c.order[sid]:
+        arrive = c.activation_at(k) if kind == "F" else c.grad_at(k)
+        end = c.end_of(sid, kind, k)
+        own.append((f"{kind}{k}", arrive, max(arrive, prev), end))
+        prev = end
+    # pieces of one micro-batch's redundant forward that ran back to back are one row
+    marks = [(k, layer, what, when()) for k, layer, what, when in q.rc_marks]
+    pieces = []
+    for (k, lo, _, t0), (_, hi, _, t1) in zip(marks[0::2], marks[1::2]):
+        if pieces and pieces[-1][0] == k and pieces[-1][2] == lo and t0 - pieces[-1][4] < 50e-6:
+            pieces[-1][2], pieces[-1][4] = hi, t1
+        else:
+            pieces.append([k, lo, hi, t0, t1])
+    lines = ["| own pass | input arrived (ms) | started | ended | idle before it (ms) |", "|---|---:|---:|---:|---:|"]
+    idle_total, last_end = 0.0, c.t0
+    for name, arrive, start, end in own:
+        idle_total += start - last_end
+        lines.append(f"| {name} | {ms(arrive)} | {ms(start)} | {ms(end)} | {(start - last_end) * 1e3:6.2f} |")
+        last_end = end
+    lines += ["", f"Own stream idle inside the batch: {idle_total * 1e3:.2f} ms; pipeline end of the batch at {ms(c.pipeline_end())} ms.", "",
+              "| redundant forward of micro-batch | layers | started (ms) | ended | overlapped with own passes (ms) | beside |", "|---|---|---:|---:|---:|---|"]
+    in_idle = 0
+    for k, lo, hi, t0, t1 in pieces:
+        shared = [(name, max(0.0, min(t1, e) - max(t0, s))) for name, _, s, e in own]
+        shared = [(n, d) for n, d in shared if d > 20e-6]
+        ov = sum(d for _, d in shared)
+        in_idle += ov < 0.1 * (t1 - t0)
+        lines.append(f"| {k} | {lo}-{hi - 1} | {ms(t0)} | {ms(t1)} | {ov * 1e3:6.2f} of {(t1 - t0) * 1e3:5.2f} | {', '.join(n for n, _ in shared) or 'idle GPU'} |")
+    lines += ["", f"{in_idle} of {len(pieces)} pieces ran with less than a tenth of their time beside an own pass."]
+    return "\n".join(lines)
+
+
+def paced_leg(cfg, rc, rc_issue, t_fwd, t_bwd, steps, warmup, timeline=None):
     """Batch time (seconds, mean of ``steps`` batches) of the stage inside the closed-loop pipeline model, graphs on
     (one launch per pass: the host never holds the GPU back after a receive has returned)."""
     import torch
@@ -132,11 +171,17 @@ def paced_leg(cfg, rc, rc_issue, t_fwd, t_bwd, steps, warmup):
             engine.train_batch()
         q.reset()
         waits, per_batch = [], []
-        for _ in range(steps):
+        for i in range(steps):
+            if timeline is not None and i == steps - 1:
+                q.rc_marks = []              # the last batch's redundant work, piece by piece
+                t_start = q._last_end if i > 0 else 0.0
             engine.train_batch()
             waits.append(q.waited)
             per_batch.append(q.batch_seconds)
         total = q.finish()
+        if timeline is not None:
+            with open(timeline, "w") as f:
+                f.write(paced_timeline(q, t_start) + "\n")
     del engine, q
     gc.collect()
     torch.cuda.empty_cache()
@@ -288,6 +333,8 @@ def main():
                          "line is quoted at 0, the configuration names none)")
     ap.add_argument("--no-paced", action="store_true",
                     help="skip the legs that run the stage inside the closed-loop model of a 4-stage 1F1B pipeline")
+    ap.add_argument("--paced-timeline", default=None, metavar="FILE",
+                    help="write the last batch of the paced 'bubble' leg as a table: own passes and pieces of redundant work")
     ap.add_argument("--failover-at", type=int, default=None,
                     help="also measure a failover: the successor is preempted at this micro-batch (config c5: 7)")
     args = ap.parse_args()
@@ -462,7 +509,9 @@ def main():
         # forwards go to the second stream either where the reference places them or as soon as their input exists.
         t_fwd, t_bwd = pass_times
         off = paced_leg(cfg, False, "reference", t_fwd, t_bwd, args.steps, args.warmup)
-        legs = {issue: paced_leg(cfg, True, issue, t_fwd, t_bwd, args.steps, args.warmup) for issue in ("reference", "asap", "bubble")}
+        legs = {issue: paced_leg(cfg, True, issue, t_fwd, t_bwd, args.steps, args.warmup,
+                                 timeline=args.paced_timeline if issue == "bubble" else None)
+                for issue in ("reference", "asap", "bubble")}
         best = min(legs, key=lambda k: legs[k]["batch_s"])
         pct = lambda leg: round(100.0 * (leg["batch_s"] - off["batch_s"]) / off["batch_s"], 2)
         r3 = lambda d: {k: round(v * 1e3, 3) for k, v in d.items()}
