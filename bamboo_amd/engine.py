@@ -28,7 +28,7 @@ import torch
 
 from . import hip, schedule
 from .config import BambooConfig
-from .module import PipelineError, PipelineModule
+from .module import MirrorBuffer, PipelineError, PipelineModule, flat_mirror
 from .optim import FusedAdam
 from .p2p import AllReduceException, NextStageException, PrevStageException, SeededActivationQueue  # noqa: F401
 from .utils import get_redundant_stage_ids, get_redundant_user_stage_ids
@@ -183,7 +183,7 @@ class PipelineEngine:
         self.r_user_stage_ids = get_redundant_user_stage_ids(self.redundancy_level, self.stage_id, self.num_stages)
         self.param_buffers, self.state_buffers = {}, {}
         for sid in self.r_stage_ids:
-            self.param_buffers[sid], self.state_buffers[sid] = {}, {}
+            self.param_buffers[sid], self.state_buffers[sid] = MirrorBuffer(), MirrorBuffer()
             if self.eager_recovery:
                 self.module.build_layers(sid)
                 for name, p in self.module.get_named_param(sid):
@@ -194,10 +194,16 @@ class PipelineEngine:
                     self.state_buffers[sid][f"{i}.exp_avg_sq"] = sp.view(sp.exp_avg_sq, name)
             else:
                 names = self.module.allocate_param(sid, self.param_buffers[sid], "cpu")
+                # both moments of a parameter as views of two flat host tensors in the arena's order
+                total = self.param_buffers[sid].flat.numel()
+                flats = {"exp_avg": flat_mirror(total), "exp_avg_sq": flat_mirror(total)}
+                off = 0
                 for i, name in enumerate(names):
                     z = self.param_buffers[sid][name]
-                    self.state_buffers[sid][f"{i}.exp_avg"] = torch.zeros_like(z)
-                    self.state_buffers[sid][f"{i}.exp_avg_sq"] = torch.zeros_like(z)
+                    for kind, flat in flats.items():
+                        self.state_buffers[sid][f"{i}.{kind}"] = flat[off: off + z.numel()].view(z.shape)
+                    off += z.numel()
+                self.state_buffers[sid].flat = flats
 
     def init_pipe_buffers(self):
         """Per-micro-batch buffer lists keyed like the reference's (engine.py:352-387)."""
@@ -399,9 +405,14 @@ class PipelineEngine:
             # lazy mode keeps CPU mirrors only: materialise the layers from them now
             self.module.build_layers(absorbed, self.param_buffers[absorbed])
             sp = self.module.stage_params[absorbed]
-            for i, name in enumerate(sp.index):
-                sp.view(sp.exp_avg, name).copy_(self.state_buffers[absorbed][f"{i}.exp_avg"])
-                sp.view(sp.exp_avg_sq, name).copy_(self.state_buffers[absorbed][f"{i}.exp_avg_sq"])
+            flats = getattr(self.state_buffers[absorbed], "flat", None)
+            if flats is not None and flats["exp_avg"].numel() == sp.numel:
+                sp.exp_avg.copy_(flats["exp_avg"])          # one transfer per moment arena
+                sp.exp_avg_sq.copy_(flats["exp_avg_sq"])
+            else:
+                for i, name in enumerate(sp.index):
+                    sp.view(sp.exp_avg, name).copy_(self.state_buffers[absorbed][f"{i}.exp_avg"])
+                    sp.view(sp.exp_avg_sq, name).copy_(self.state_buffers[absorbed][f"{i}.exp_avg_sq"])
             self.ctx = self.module.prepare_context(self.stage_ids + [absorbed], self.batch, self.seq, stream=self.main_stream)
             self.stash_bytes += self.module.allocate_stash(absorbed, self.ctx, self.micro_batches)
             act_shape = self.module.stage_io_shapes(absorbed, self.batch)[0]
@@ -715,6 +726,14 @@ class PipelineEngine:
             # lazy mode keeps host mirrors only (engine.py:336-350): parameters and both moments come
             # down as three flat copies and are scattered into the named buffers
             names = self.module.param_name_buckets[stage_id]
+            pflat = getattr(self.param_buffers[stage_id], "flat", None)
+            sflat = getattr(self.state_buffers[stage_id], "flat", None)
+            if pflat is not None and sflat is not None and pflat.numel() == msg["master"].numel():
+                pflat.copy_(msg["master"])                   # the named buffers are views of these three
+                sflat["exp_avg"].copy_(msg["exp_avg"])
+                sflat["exp_avg_sq"].copy_(msg["exp_avg_sq"])
+                self._shadow_step = msg["step"]
+                return
             host = {k: msg[k].cpu() for k in ("master", "exp_avg", "exp_avg_sq")}
             off = 0
             for i, name in enumerate(names):

@@ -53,6 +53,18 @@ class TiedLayerSpec(LayerSpec):
         self.key, self.forward_fn, self.tied_weight_attr = key, forward_fn, tied_weight_attr
 
 
+class MirrorBuffer(dict):
+    """``{name: tensor}`` whose tensors are views of one flat tensor ``flat`` (set by whoever fills it)."""
+    flat = None
+
+
+def flat_mirror(numel, device="cpu"):
+    """Zeroed fp32 tensor for a host mirror: page-locked where a GPU is present (transfers at the link's rate,
+    asynchronous to the host), plain otherwise."""
+    pin = torch.device(device).type == "cpu" and torch.cuda.is_available()
+    return torch.zeros(numel, dtype=torch.float32, device=device, pin_memory=pin)
+
+
 class StageParams:
     """Flat parameter arenas of one stage and the per-layer named views into them."""
 
@@ -256,14 +268,21 @@ class PipelineModule:
 
     def build_layers(self, stage_id, buffer=None):
         """Materialise the layers of ``stage_id`` on the GPU (own stage, or a stage this process
-        shadows).  ``buffer``: optional ``{"{layer_idx}.{name}": tensor}`` to copy weights from."""
+        shadows).  ``buffer``: optional ``{"{layer_idx}.{name}": tensor}`` to copy weights from; where it is the
+        mirror :meth:`allocate_param` made (one flat host tensor behind the named views), it goes over in one copy."""
         if stage_id in self.func_buckets:
             if buffer is not None:
                 self.stage_params[stage_id].load(buffer)
             return self.param_name_buckets[stage_id]
         layers = self._instantiate(stage_id)
         sp = StageParams(layers, self.parts[stage_id], self.dtype, self.device)
-        sp.init(self.base_seed)
+        flat = getattr(buffer, "flat", None)
+        if flat is not None and flat.numel() == sp.numel and not self._adopted_weights:
+            sp.master.copy_(flat)                # every parameter comes from the mirror: no seeded initialisation
+            sp.refresh_compute()
+            buffer = None
+        else:
+            sp.init(self.base_seed)
         if self._adopted_weights:
             sp.load(self._adopted_weights)       # weights of the modules the layers were taken from
             self._adopted_weights = {}
@@ -275,14 +294,22 @@ class PipelineModule:
         return self.param_name_buckets[stage_id]
 
     def allocate_param(self, stage_id, param_buffer, device="cpu"):
-        """Zero mirrors of the parameters of ``stage_id`` (reference module.py:229-260)."""
+        """Zero mirrors of the parameters of ``stage_id`` (reference module.py:229-260): named tensors in
+        ``param_buffer`` that are views of ONE flat tensor in the arena's order (``param_buffer.flat`` where the
+        buffer is a :class:`MirrorBuffer`), page-locked when it lives on the host of a GPU process, so that a
+        refresh and a promotion move it in a single transfer."""
         layers = self.func_buckets.get(stage_id) or self._instantiate(stage_id)
-        names = []
-        for li, layer in enumerate(layers):
-            for name, shape in layer.param_specs().items():
-                key = f"{self.parts[stage_id] + li}.{name}"
-                param_buffer[key] = torch.zeros(shape, dtype=torch.float32, device=device)
-                names.append(key)
+        specs = [(f"{self.parts[stage_id] + li}.{name}", shape) for li, layer in enumerate(layers)
+                 for name, shape in layer.param_specs().items()]
+        flat = flat_mirror(sum(math.prod(shape) for _, shape in specs), device)
+        off = 0
+        for key, shape in specs:
+            n = math.prod(shape)
+            param_buffer[key] = flat[off: off + n].view(shape)
+            off += n
+        if isinstance(param_buffer, MirrorBuffer):
+            param_buffer.flat = flat
+        names = [key for key, _ in specs]
         self.param_name_buckets.setdefault(stage_id, names)
         return names
 
