@@ -2,7 +2,9 @@
 ffn 4096, 16 heads, seq 1024) and the GPT-2-1.5B stage (rows 4096, hidden 1600, ffn 6400, 25 heads, seq 1024:
 1600 = 25 x 64 is no multiple of the 128- and 256-wide tiles) -- through properties that do not need a full CPU
 run: bit-reproducibility, oracle values on sampled rows / heads, softmax normalisation, causality, RC
-bit-exactness; plus one failover at the 1.5B layer shape against the CPU oracle."""
+bit-exactness; plus one failover at the 1.5B layer shape against the CPU oracle, and the BERT-large stage's attention
+(seq 512, ragged key lengths) against fp64 autograd on sampled heads.  (The ResNet stage's block shape is a case of
+tests/test_gpu_stage.py::test_resnet_stage_matches_oracle_with_rc.)"""
 import math
 
 import numpy as np
@@ -111,6 +113,40 @@ def test_attention_full_shape_properties(hiplib, mask, MB, HEADS):
         b = int(torch.argmin(lens))
         dead = d1.view(MB, SEQ, 3 * h)[b, int(lens[b]):, h:]
         assert float(dead.float().abs().max()) == 0.0
+
+
+def test_attention_bert_large_shape_with_ragged_keys(hiplib):
+    """The BERT-large stage's attention (16 samples of 512 positions, 16 heads, key lengths uniform in [128, 512]):
+    forward and all three input gradients of the shortest and the longest sample against fp64 autograd, padded
+    keys without probability mass or gradient, rows normalised."""
+    mb, heads, seq = 16, 16, 512
+    h = heads * 64
+    rows = mb * seq
+    qkv = randn(rows, 3 * h, seed=14, scale=0.7)
+    lens = torch.randint(128, seq + 1, (mb,), generator=torch.Generator().manual_seed(15), dtype=torch.int32)
+    lens[3], lens[11] = 128, 512
+    lens_d = lens.to(DEV)
+    code = hiplib.MASK_CODES["key_padding"]
+    out, lse = torch.empty(rows, h, dtype=torch.bfloat16, device=DEV), torch.empty(mb, heads, seq, device=DEV)
+    hiplib.attention_fwd(qkv, out, lse, mb, heads, seq, code, lens_d)
+    d_out = randn(rows, h, seed=16)
+    delta, d_qkv = torch.empty(mb, heads, seq, device=DEV), torch.empty_like(qkv)
+    hiplib.attention_bwd(qkv, out, d_out, lse, delta, d_qkv, mb, heads, seq, code, lens_d)
+    for b, a in [(3, 0), (11, heads - 1), (7, 5)]:
+        rs = slice(b * seq, (b + 1) * seq)
+        q, k, v = [qkv[rs, i * h + a * 64: i * h + (a + 1) * 64].double().cpu().requires_grad_(True) for i in range(3)]
+        sc = (q @ k.t() / 8.0).masked_fill(torch.arange(seq).view(1, -1) >= int(lens[b]), -1e9)
+        ctx = torch.softmax(sc, -1) @ v
+        ctx.backward(d_out[rs, a * 64:(a + 1) * 64].double().cpu())
+        assert l2(out[rs, a * 64:(a + 1) * 64], ctx.detach()) < 1e-2
+        for i, t in enumerate((q, k, v)):
+            assert l2(d_qkv[rs, i * h + a * 64: i * h + (a + 1) * 64], t.grad) < 2e-2, (b, a, i)
+    dead = d_qkv.view(mb, seq, 3 * h)[3, 128:, h:]
+    assert float(dead.float().abs().max()) == 0.0
+    qkv1 = qkv.clone()
+    qkv1[:, 2 * h:] = 1.0
+    hiplib.attention_fwd(qkv1, out, lse, mb, heads, seq, code, lens_d)
+    assert float((out.float() - 1).abs().max()) < 1e-2
 
 
 @pytest.mark.parametrize("MB,HID,HEADS,FFN", [(MB, HID, HEADS, FFN), (MB5, HID5, HEADS5, FFN5)], ids=["gpt2-medium", "gpt2-1.5b"])

@@ -284,15 +284,20 @@ def test_failover_onto_the_last_stage_computes_the_loss(hiplib, dead_from, dtype
     assert abs(float(loss2) - float(loss)) < 0.1 * float(loss)
 
 
-@pytest.mark.parametrize("dtype,cin,cmid", [(torch.float32, 64, 16), (torch.bfloat16, 64, 16), (torch.bfloat16, 512, 128)],
-                         ids=["fp32", "bf16", "bf16-implicit-gemm"])
+@pytest.mark.parametrize("dtype,cin,cmid", [(torch.float32, 64, 16), (torch.bfloat16, 64, 16), (torch.bfloat16, 512, 128),
+                                            (torch.bfloat16, 1024, 256)],
+                         ids=["fp32", "bf16", "bf16-implicit-gemm", "bf16-resnet152-conv4-shape"])
 def test_resnet_stage_matches_oracle_with_rc(hiplib, dtype, cin, cmid):
     """Bottleneck stage (conv 1x1 -> 3x3 -> 1x1, train-mode BatchNorm, ReLU, identity shortcut) with
     redundant forwards of the shadow blocks, against the torch conv2d / batch_norm oracle.  With 128 middle
-    channels the 3x3 convolution and its input gradient run as implicit GEMMs, with 16 through the patch matrix."""
+    channels the 3x3 convolution and its input gradient run as implicit GEMMs, with 16 through the patch matrix.
+    The last case is the benchmark's own block shape: 32 images of 14x14, 1024 -> 256 -> 256 -> 1024 channels
+    (one own and one shadow block, two micro-batches: the CPU oracle runs it in fp64)."""
     from bamboo_amd import BottleNeck
     side, L, S, sid, mb, M = 6, 2, 4, 1, (8 if cmid == 128 else 4), 4     # 288 pixels: whole 32-pixel k-tiles for the weight gradient
-    assert hiplib.conv3x3_supported(dtype, hiplib.CONV_DGRAD, mb, side, side, cmid, cmid) == (cmid == 128)
+    if cin == 1024:
+        side, L, mb, M = 14, 1, 32, 2
+    assert hiplib.conv3x3_supported(dtype, hiplib.CONV_DGRAD, mb, side, side, cmid, cmid) == (cmid >= 128)
     specs = [LayerSpec(BottleNeck, cin, cmid, height=side, width=side) for _ in range(L * S)]
     model = PipelineModule(specs, num_stages=S, partition_method="uniform", stage_id=sid, dtype=dtype, device=DEV)
     q = SeededActivationQueue((mb, side * side, cin), dtype, M, stage_ids=[sid, sid + 1], seed=9, device=DEV)
