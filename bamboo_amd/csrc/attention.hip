@@ -121,6 +121,26 @@ __device__ __forceinline__ bf16x8 pack_acc(const f32x16& a, int half) {
 }
 // row index (0..31) that register r of a 32x32 accumulator holds in this lane
 __device__ __forceinline__ int acc_row(int r, int lane) { return 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3); }
+// Dropout over the sixteen accumulator registers of a lane whose rows acc_row(r, lane) are consecutive probability
+// indices from `base` on: registers 4g .. 4g + 3 hold four neighbouring indices, i.e. two hash pairs when the first is
+// even (every case with an even sequence length).  Kept values are scaled, dropped ones zeroed.
+__device__ __forceinline__ void drop_acc_rows(const DropKey& k, uint64_t base, int lane, f32x16& v) {
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+        const uint64_t i0 = base + 8 * g + 4 * (lane >> 5);
+        if ((i0 & 1) == 0) {
+            const uint32_t x0 = bb_dropout_pair_bits(k.k0, k.k1, i0 >> 1), x1 = bb_dropout_pair_bits(k.k0, k.k1, (i0 >> 1) + 1);
+            v[4 * g] = bb_keep_even(x0, k.thresh) ? v[4 * g] * k.scale : 0.f;
+            v[4 * g + 1] = bb_keep_odd(x0, k.thresh) ? v[4 * g + 1] * k.scale : 0.f;
+            v[4 * g + 2] = bb_keep_even(x1, k.thresh) ? v[4 * g + 2] * k.scale : 0.f;
+            v[4 * g + 3] = bb_keep_odd(x1, k.thresh) ? v[4 * g + 3] * k.scale : 0.f;
+        } else {
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+                v[4 * g + e] = bb_dropout_keep(k.k0, k.k1, k.thresh, i0 + e) ? v[4 * g + e] * k.scale : 0.f;
+        }
+    }
+}
 
 template <int N> __device__ __forceinline__ void wait_vm() {
     __builtin_amdgcn_s_waitcnt((N & 15) | (7 << 4) | (0 << 8) | ((N >> 4) << 14));
@@ -259,11 +279,7 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const AttnArgs a) {
             if (DROP && a.drop.thresh) {   // the normaliser takes every probability, the context only the kept ones
                 const uint64_t base = prob_index(a, b, head, min(myq, last)) + kv0;
 #pragma unroll
-                for (int u = 0; u < 2; ++u)
-#pragma unroll
-                    for (int r = 0; r < 16; ++r)
-                        s[u][r] = bb_dropout_keep(a.drop.k0, a.drop.k1, a.drop.thresh, base + u * 32 + acc_row(r, lane))
-                                      ? s[u][r] * a.drop.scale : 0.f;
+                for (int u = 0; u < 2; ++u) drop_acc_rows(a.drop, base + u * 32, lane, s[u]);
             }
             if (__any(alpha != 1.0f)) {  // wave-uniform: once the maxima have settled nothing is rescaled
 #pragma unroll
@@ -578,9 +594,7 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dq_kernel(const AttnArgs a) {
                 if (DROP && a.drop.thresh) {
                     asm volatile("" ::: "memory");
                     const uint64_t base = prob_index(a, b, head, min(myq, last)) + kv0 + u * 32;
-#pragma unroll
-                    for (int r = 0; r < 16; ++r)
-                        dp[r] = bb_dropout_keep(a.drop.k0, a.drop.k1, a.drop.thresh, base + acc_row(r, lane)) ? dp[r] * a.drop.scale : 0.f;
+                    drop_acc_rows(a.drop, base, lane, dp);
                 }
 #pragma unroll
                 for (int r = 0; r < 16; ++r) dp[r] = s[r] * (dp[r] - my_delta);

@@ -156,10 +156,9 @@ __device__ __forceinline__ float dact_f(float x, int kind) {
 // ---- dropout -------------------------------------------------------------------------------
 // Counter-based keep/drop decision: a pure function of (key, element index), so a redundant forward, a normal
 // forward and the backward pass of the same (layer, site, micro-batch) make the same decisions without a mask ever
-// being stored.  Two rounds of a 32-bit finalizer (xorshift-multiply), the key words and the high half of the
-// counter injected between them; an element is kept when the result is >= thresh = p * 2^32.
+// being stored.
 struct DropKey {
-    uint32_t k0, k1, thresh;   // thresh == 0: no dropout
+    uint32_t k0, k1, thresh;   // thresh: 16-bit, round(p * 65536); 0: no dropout
     float scale;               // 1 / (1 - p)
 };
 __host__ __device__ __forceinline__ uint32_t bb_mix32(uint32_t x) {
@@ -168,16 +167,27 @@ __host__ __device__ __forceinline__ uint32_t bb_mix32(uint32_t x) {
     x ^= x >> 16;
     return x;
 }
-__host__ __device__ __forceinline__ bool bb_dropout_keep(uint32_t k0, uint32_t k1, uint32_t thresh, uint64_t idx) {
-    uint32_t x = bb_mix32((uint32_t)idx ^ k0);
-    x = bb_mix32(x + ((uint32_t)(idx >> 32) ^ k1));
-    return x >= thresh;
+// Dropout decisions as a pure function of (key, element index).  One 32-bit hash serves the two elements 2j and
+// 2j + 1 of a tensor: x = mix32(((uint32)j ^ k0) + (k1 ^ rotl(j >> 32, 16))), the low 16 bits decide the even
+// element, the high 16 the odd one; an element is kept when its 16 bits are >= thresh = round(p * 65536).  (mix32
+// is a full-avalanche finalizer: every output bit depends on every input bit, so the two halves are as good as
+// two hashes; p is met to within 1 / 131072.)
+__host__ __device__ __forceinline__ uint32_t bb_dropout_pair_bits(uint32_t k0, uint32_t k1, uint64_t pair) {
+    const uint32_t hi = (uint32_t)(pair >> 32);
+    return bb_mix32(((uint32_t)pair ^ k0) + (k1 ^ ((hi << 16) | (hi >> 16))));
 }
+__host__ __device__ __forceinline__ bool bb_dropout_keep(uint32_t k0, uint32_t k1, uint32_t thresh, uint64_t idx) {
+    const uint32_t x = bb_dropout_pair_bits(k0, k1, idx >> 1);
+    return ((idx & 1) ? x >> 16 : x & 0xffffu) >= thresh;
+}
+// both decisions of the pair (even element, odd element) from its hash
+__host__ __device__ __forceinline__ bool bb_keep_even(uint32_t x, uint32_t thresh) { return (x & 0xffffu) >= thresh; }
+__host__ __device__ __forceinline__ bool bb_keep_odd(uint32_t x, uint32_t thresh) { return (x >> 16) >= thresh; }
 static inline DropKey bb_drop_key(float p, uint32_t k0, uint32_t k1) {
     DropKey d = {k0, k1, 0u, 1.0f};
     if (p > 0.f) {
-        const double t = (double)p * 4294967296.0;
-        d.thresh = t >= 4294967295.0 ? 4294967295u : (uint32_t)(t + 0.5);
+        const double t = (double)p * 65536.0;
+        d.thresh = t >= 65535.0 ? 65535u : t < 1.0 ? 1u : (uint32_t)(t + 0.5);
         d.scale = 1.0f / (1.0f - p);
     }
     return d;

@@ -717,8 +717,11 @@ __global__ __launch_bounds__(256) void dropout_kernel(int64_t nvec, const T* src
         float v[VEC];
         load_vec(src + i * VEC, v);
 #pragma unroll
-        for (int e = 0; e < VEC; ++e)
-            v[e] = bb_dropout_keep(key.k0, key.k1, key.thresh, (uint64_t)(i * VEC + e)) ? v[e] * key.scale : 0.f;
+        for (int e = 0; e < VEC; e += 2) {   // VEC is even: one hash per two neighbouring elements
+            const uint32_t x = bb_dropout_pair_bits(key.k0, key.k1, (uint64_t)(i * VEC + e) >> 1);
+            v[e] = bb_keep_even(x, key.thresh) ? v[e] * key.scale : 0.f;
+            v[e + 1] = bb_keep_odd(x, key.thresh) ? v[e + 1] * key.scale : 0.f;
+        }
         store_vec(dst + i * VEC, v);
     }
 }

@@ -7,7 +7,7 @@ hidden activation :154-158) and reseeds torch's generator per layer and micro-ba
 (it depends on the device kernel's launch shape): **parity unpinned** for the mask bits themselves.  What is
 fixed, and restated here, is the arithmetic -- kept elements are scaled by 1 / (1 - p), dropped ones are zero, an
 element is kept with probability 1 - p -- and, for this build, the decision function the HIP kernels evaluate
-(two rounds of a 32-bit xorshift-multiply finalizer over (index, key)), restated with numpy integer arithmetic and
+(a 32-bit xorshift-multiply finalizer over (index / 2, key), sixteen of its bits per element), restated with numpy integer arithmetic and
 pinned against the library's own host-side evaluation of it (tests/test_dropout.py)."""
 import numpy as np
 
@@ -41,17 +41,28 @@ def _mix32(x):
 
 
 def threshold(p):
-    t = float(np.float32(p)) * 4294967296.0
-    return 4294967295 if t >= 4294967295.0 else int(t + 0.5)
+    """16-bit threshold: an element is kept when its 16 hash bits are >= round(p * 65536) (at least 1 for p > 0)."""
+    if p <= 0:
+        return 0
+    t = float(np.float32(p)) * 65536.0
+    return 65535 if t >= 65535.0 else 1 if t < 1.0 else int(t + 0.5)
+
+
+def pair_bits(k, pair):
+    """The 32 hash bits shared by elements 2 * pair and 2 * pair + 1."""
+    pair = np.asarray(pair, dtype=np.uint64)
+    lo, hi = pair & np.uint64(0xFFFFFFFF), pair >> np.uint64(32)
+    rot = ((hi << np.uint64(16)) | (hi >> np.uint64(16))) & np.uint64(0xFFFFFFFF)
+    return _mix32(((lo ^ np.uint64(k[0])) + (np.uint64(k[1]) ^ rot)) & np.uint64(0xFFFFFFFF))
 
 
 def keep(p, k, index):
-    """Boolean array: element ``index`` (array of non-negative ints) is kept under probability-to-drop ``p``."""
+    """Boolean array: element ``index`` (array of non-negative ints) is kept under probability-to-drop ``p``: the low
+    16 bits of its pair's hash decide an even element, the high 16 bits an odd one."""
     idx = np.asarray(index, dtype=np.uint64)
-    lo, hi = idx & np.uint64(0xFFFFFFFF), idx >> np.uint64(32)
-    x = _mix32(lo ^ np.uint64(k[0]))
-    x = _mix32((x + (hi ^ np.uint64(k[1]))) & np.uint64(0xFFFFFFFF))
-    return x >= np.uint64(threshold(p))
+    x = pair_bits(k, idx >> np.uint64(1))
+    bits = np.where((idx & np.uint64(1)) == 1, x >> np.uint64(16), x & np.uint64(0xFFFF))
+    return bits >= np.uint64(threshold(p))
 
 
 def mask(p, k, shape):

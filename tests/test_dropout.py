@@ -21,7 +21,13 @@ def test_decision_function_equals_the_library():
         want = od.keep(p, k, idx)
         got = np.array([hip.dropout_keep(p, k, int(i)) for i in idx])
         assert np.array_equal(want, got)
-    assert od.threshold(0.1) == round(float(np.float32(0.1)) * 2 ** 32)
+    assert od.threshold(0.1) == round(float(np.float32(0.1)) * 2 ** 16) == 6554 and od.threshold(0.0) == 0 and od.threshold(1e-9) == 1
+    # one hand-computed value of the finalizer (x ^= x >> 16; x *= 0x7feb352d; x ^= x >> 15; x *= 0x846ca68b; x ^= x >> 16)
+    # pins the restatement independently of the library: key (0, 0), pair 1 -> mix32(1)
+    x = 1
+    x ^= x >> 16; x = (x * 0x7FEB352D) & 0xFFFFFFFF; x ^= x >> 15; x = (x * 0x846CA68B) & 0xFFFFFFFF; x ^= x >> 16
+    assert int(od.pair_bits((0, 0), 1)) == x
+    assert bool(od.keep(0.5, (0, 0), 2)) == ((x & 0xFFFF) >= 32768) and bool(od.keep(0.5, (0, 0), 3)) == ((x >> 16) >= 32768)
     # p = 0 keeps everything
     assert od.keep(0.0, (1, 2), np.arange(1000)).all()
 
@@ -40,8 +46,9 @@ def test_mask_statistics(p):
         assert abs((x == y).mean() - ((1 - p) ** 2 + p ** 2)) < 6 * (0.25 / n) ** 0.5
     quarters = a.reshape(4, -1).mean(1)
     assert np.abs(quarters - (1 - p)).max() < 5 * 2 * sigma
-    # neighbouring elements are uncorrelated
+    # neighbouring elements are uncorrelated, also the two that share one hash (its low and its high sixteen bits)
     assert abs(np.corrcoef(a[:-1], a[1:])[0, 1]) < 5 / n ** 0.5
+    assert abs(np.corrcoef(a[0::2], a[1::2])[0, 1]) < 5 / (n / 2) ** 0.5
 
 
 def test_dropout_sites_of_the_layer_match_the_module_form():
