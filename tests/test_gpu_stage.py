@@ -618,6 +618,41 @@ def test_paced_pipeline_changes_timing_not_results(hiplib, rc_issue):
         build(hid, heads, ffn, L, S, sid, mb, M, seq, dtype, GPT_VARIANT, 1, True, rc_issue="asap")   # needs the second stream
 
 
+@pytest.mark.parametrize("dead_from", [1, 4])
+@pytest.mark.parametrize("rc_issue", ["asap", "bubble"])
+def test_failover_with_redundant_forwards_issued_out_of_order(hiplib, rc_issue, dead_from):
+    """The successor is lost while redundant forwards are pending, partly issued or ahead of the schedule (issued as
+    soon as their input exists, or held back for the bubbles of the paced pipeline): the promoted stage replays what
+    is missing as ordinary forwards.  Losses of the failing batch and the one after it, and every parameter of both
+    stages after the two optimizer steps, are bit-equal to the same failure under the reference's placement."""
+    from bamboo_amd.p2p import PacedActivationQueue
+    hid, heads, ffn, L, S, sid, mb, M, seq = 128, 2, 256, 2, 4, 1, 2, 6, 64
+    dtype = torch.bfloat16
+
+    def run(issue, paced):
+        specs = [LayerSpec(TransformerLayer, hid, heads, ffn, **GPT_VARIANT) for _ in range(L * S)]
+        model = PipelineModule(specs, num_stages=S, partition_method="uniform", stage_id=sid, dtype=dtype, device=DEV)
+        kw = dict(stage_ids=[sid, sid + 1], seed=7, grad_mode="mse", device=DEV)
+        q = (PacedActivationQueue((mb, seq, hid), dtype, M, stages=S, stage_id=sid, t_fwd=1e-3, t_bwd=2e-3, **kw) if paced
+             else SeededActivationQueue((mb, seq, hid), dtype, M, **kw))
+        cfg = {"train_micro_batch_size_per_gpu": mb, "gradient_accumulation_steps": M,
+               "optimizer": {"type": "Adam", "params": {"lr": 1e-3}}, "bf16": {"enabled": True}}
+        engine, _, _, _ = bamboo_amd.initialize(model=model, config=cfg, redundancy_level=1, eager_recovery=True,
+                                                activation_queue=q, rc_stream=True, rc_issue=issue, install_signal_handler=False)
+        losses = [float(engine.train_batch())]
+        q.preempt_successor(dead_from, sid)
+        losses += [float(engine.train_batch()), float(engine.train_batch())]
+        torch.cuda.synchronize()
+        assert engine.stage_ids == [sid, sid + 1]
+        return engine, losses
+    ref, ref_losses = run("reference", False)
+    eng, losses = run(rc_issue, True)
+    assert losses == ref_losses
+    for s_ in (sid, sid + 1):
+        a, b = eng.module.stage_params[s_], ref.module.stage_params[s_]
+        assert torch.equal(a.master, b.master) and torch.equal(a.exp_avg, b.exp_avg) and torch.equal(a.exp_avg_sq, b.exp_avg_sq)
+
+
 def test_script_layers_taken_over_run_as_the_last_stage(hiplib):
     """The reference script's own layer list -- EncoderLayer modules, the final LayerNorm, ``lambda x: x.sum(-1)``,
     ``nn.MSELoss()`` against [batch, seq] labels (transformer.py:246-264) -- handed over as it is.  The last stage
