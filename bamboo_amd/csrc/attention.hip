@@ -125,20 +125,25 @@ __device__ __forceinline__ int acc_row(int r, int lane) { return 8 * (r >> 2) + 
 // indices from `base` on: registers 4g .. 4g + 3 hold four neighbouring indices, i.e. two hash pairs when the first is
 // even (every case with an even sequence length).  Kept values are scaled, dropped ones zeroed.
 __device__ __forceinline__ void drop_acc_rows(const DropKey& k, uint64_t base, int lane, f32x16& v) {
+    const bool even = (base & 1) == 0;   // 8 g + 4 (lane >> 5) is even
+    if (k.small && even) {               // the rule: fewer than 2^32 probabilities, even sequence length
+        const uint32_t p0 = ((uint32_t)base >> 1) + 2 * (lane >> 5);
 #pragma unroll
-    for (int g = 0; g < 4; ++g) {
-        const uint64_t i0 = base + 8 * g + 4 * (lane >> 5);
-        if ((i0 & 1) == 0) {
-            const uint32_t x0 = bb_dropout_pair_bits(k.k0, k.k1, i0 >> 1), x1 = bb_dropout_pair_bits(k.k0, k.k1, (i0 >> 1) + 1);
+        for (int g = 0; g < 4; ++g) {
+            const uint32_t x0 = bb_dropout_pair_bits32(k.k0, k.k1, p0 + 4 * g), x1 = bb_dropout_pair_bits32(k.k0, k.k1, p0 + 4 * g + 1);
             v[4 * g] = bb_keep_even(x0, k.thresh) ? v[4 * g] * k.scale : 0.f;
             v[4 * g + 1] = bb_keep_odd(x0, k.thresh) ? v[4 * g + 1] * k.scale : 0.f;
             v[4 * g + 2] = bb_keep_even(x1, k.thresh) ? v[4 * g + 2] * k.scale : 0.f;
             v[4 * g + 3] = bb_keep_odd(x1, k.thresh) ? v[4 * g + 3] * k.scale : 0.f;
-        } else {
-#pragma unroll
-            for (int e = 0; e < 4; ++e)
-                v[4 * g + e] = bb_dropout_keep(k.k0, k.k1, k.thresh, i0 + e) ? v[4 * g + e] * k.scale : 0.f;
         }
+        return;
+    }
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+        const uint64_t i0 = base + 8 * g + 4 * (lane >> 5);
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+            v[4 * g + e] = bb_dropout_keep(k.k0, k.k1, k.thresh, i0 + e) ? v[4 * g + e] * k.scale : 0.f;
     }
 }
 
@@ -452,12 +457,26 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dkv_kernel(const AttnArgs a) 
                 asm volatile("" ::: "memory");
                 const int qlane = t * 64 + u * 32 + 4 * (lane >> 5);
                 kept = 0u;
+                if (a.drop.small) {
+                    // 32-bit indices; a query past the end is masked out above, what is decided for it does not matter
+                    const uint32_t i0 = ((uint32_t)(b * a.heads + head) * (uint32_t)a.seq + (uint32_t)qlane) * (uint32_t)a.seq +
+                                        (uint32_t)min(mykv, last);
 #pragma unroll
-                for (int r = 0; r < 16; ++r) {
-                    const int q = min(qlane + 8 * (r >> 2) + (r & 3), last);
-                    const bool keep = bb_dropout_keep(a.drop.k0, a.drop.k1, a.drop.thresh, prob_index(a, b, head, q) + min(mykv, last));
-                    kept |= keep ? 1u << r : 0u;
-                    dp[r] = keep ? dp[r] * a.drop.scale : 0.f;
+                    for (int r = 0; r < 16; ++r) {
+                        const uint32_t idx = i0 + (uint32_t)(8 * (r >> 2) + (r & 3)) * (uint32_t)a.seq;
+                        const uint32_t x = bb_dropout_pair_bits32(a.drop.k0, a.drop.k1, idx >> 1);
+                        const bool keep = (idx & 1) ? bb_keep_odd(x, a.drop.thresh) : bb_keep_even(x, a.drop.thresh);
+                        kept |= keep ? 1u << r : 0u;
+                        dp[r] = keep ? dp[r] * a.drop.scale : 0.f;
+                    }
+                } else {
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) {
+                        const int q = min(qlane + 8 * (r >> 2) + (r & 3), last);
+                        const bool keep = bb_dropout_keep(a.drop.k0, a.drop.k1, a.drop.thresh, prob_index(a, b, head, q) + min(mykv, last));
+                        kept |= keep ? 1u << r : 0u;
+                        dp[r] = keep ? dp[r] * a.drop.scale : 0.f;
+                    }
                 }
             }
 #pragma unroll
@@ -650,7 +669,7 @@ extern "C" int bb_attention_fwd(int dtype, int mask, int batch, int heads, int s
     BB_REQUIRE(q && k && v && out && lse, "bb_attention_fwd: null pointer");
     BB_REQUIRE(dropout_p >= 0.f && dropout_p < 1.f, "bb_attention_fwd: dropout_p must be in [0, 1)");
     AttnArgs a = {};
-    a.drop = bb_drop_key(dropout_p, dropout_k0, dropout_k1);
+    a.drop = bb_drop_key(dropout_p, dropout_k0, dropout_k1, (uint64_t)batch * heads * (uint64_t)seq * (uint64_t)seq);
     a.q = (const bf16*)q; a.k = (const bf16*)k; a.v = (const bf16*)v;
     a.out = (bf16*)out; a.lse = lse; a.key_len = key_len;
     a.ld_qkv = ld_qkv; a.ld_o = ld_out;
@@ -676,7 +695,7 @@ extern "C" int bb_attention_bwd(int dtype, int mask, int batch, int heads, int s
     BB_REQUIRE(ld_dqkv % 4 == 0 && ld_dqkv >= heads * 64, "bb_attention_bwd: bad gradient leading dimension");
     BB_REQUIRE(dropout_p >= 0.f && dropout_p < 1.f, "bb_attention_bwd: dropout_p must be in [0, 1)");
     AttnArgs a = {};
-    a.drop = bb_drop_key(dropout_p, dropout_k0, dropout_k1);
+    a.drop = bb_drop_key(dropout_p, dropout_k0, dropout_k1, (uint64_t)batch * heads * (uint64_t)seq * (uint64_t)seq);
     a.q = (const bf16*)q; a.k = (const bf16*)k; a.v = (const bf16*)v;
     a.o = (const bf16*)out; a.d_o = (const bf16*)d_out;
     a.dq = (bf16*)dq; a.dk = (bf16*)dk; a.dv = (bf16*)dv;

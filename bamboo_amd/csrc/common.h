@@ -160,6 +160,7 @@ __device__ __forceinline__ float dact_f(float x, int kind) {
 struct DropKey {
     uint32_t k0, k1, thresh;   // thresh: 16-bit, round(p * 65536); 0: no dropout
     float scale;               // 1 / (1 - p)
+    uint32_t small;            // the tensor has fewer than 2^32 elements: indices fit 32-bit arithmetic
 };
 __host__ __device__ __forceinline__ uint32_t bb_mix32(uint32_t x) {
     x ^= x >> 16; x *= 0x7feb352du;
@@ -176,6 +177,10 @@ __host__ __device__ __forceinline__ uint32_t bb_dropout_pair_bits(uint32_t k0, u
     const uint32_t hi = (uint32_t)(pair >> 32);
     return bb_mix32(((uint32_t)pair ^ k0) + (k1 ^ ((hi << 16) | (hi >> 16))));
 }
+// the same for a pair index below 2^32 (its high word is zero)
+__host__ __device__ __forceinline__ uint32_t bb_dropout_pair_bits32(uint32_t k0, uint32_t k1, uint32_t pair) {
+    return bb_mix32((pair ^ k0) + k1);
+}
 __host__ __device__ __forceinline__ bool bb_dropout_keep(uint32_t k0, uint32_t k1, uint32_t thresh, uint64_t idx) {
     const uint32_t x = bb_dropout_pair_bits(k0, k1, idx >> 1);
     return ((idx & 1) ? x >> 16 : x & 0xffffu) >= thresh;
@@ -183,8 +188,8 @@ __host__ __device__ __forceinline__ bool bb_dropout_keep(uint32_t k0, uint32_t k
 // both decisions of the pair (even element, odd element) from its hash
 __host__ __device__ __forceinline__ bool bb_keep_even(uint32_t x, uint32_t thresh) { return (x & 0xffffu) >= thresh; }
 __host__ __device__ __forceinline__ bool bb_keep_odd(uint32_t x, uint32_t thresh) { return (x >> 16) >= thresh; }
-static inline DropKey bb_drop_key(float p, uint32_t k0, uint32_t k1) {
-    DropKey d = {k0, k1, 0u, 1.0f};
+static inline DropKey bb_drop_key(float p, uint32_t k0, uint32_t k1, uint64_t numel) {
+    DropKey d = {k0, k1, 0u, 1.0f, numel < (1ull << 32) ? 1u : 0u};
     if (p > 0.f) {
         const double t = (double)p * 65536.0;
         d.thresh = t >= 65535.0 ? 65535u : t < 1.0 ? 1u : (uint32_t)(t + 0.5);

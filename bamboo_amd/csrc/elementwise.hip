@@ -718,7 +718,8 @@ __global__ __launch_bounds__(256) void dropout_kernel(int64_t nvec, const T* src
         load_vec(src + i * VEC, v);
 #pragma unroll
         for (int e = 0; e < VEC; e += 2) {   // VEC is even: one hash per two neighbouring elements
-            const uint32_t x = bb_dropout_pair_bits(key.k0, key.k1, (uint64_t)(i * VEC + e) >> 1);
+            const uint32_t x = key.small ? bb_dropout_pair_bits32(key.k0, key.k1, (uint32_t)(i * VEC + e) >> 1)
+                                         : bb_dropout_pair_bits(key.k0, key.k1, (uint64_t)(i * VEC + e) >> 1);
             v[e] = bb_keep_even(x, key.thresh) ? v[e] * key.scale : 0.f;
             v[e + 1] = bb_keep_odd(x, key.thresh) ? v[e + 1] * key.scale : 0.f;
         }
@@ -732,7 +733,7 @@ extern "C" int bb_dropout_apply(int dtype, int64_t n, const void* src, void* dst
     BB_REQUIRE(p >= 0.f && p < 1.f, "bb_dropout_apply: p must be in [0, 1)");
     BB_REQUIRE(src && dst, "bb_dropout_apply: null pointer");
     if (n == 0) return BB_OK;
-    const DropKey key = bb_drop_key(p, k0, k1);
+    const DropKey key = bb_drop_key(p, k0, k1, (uint64_t)n);
     const int64_t nvec = n / vec;
     hipStream_t st = (hipStream_t)stream;
     if (dtype == BB_BF16)
@@ -743,7 +744,7 @@ extern "C" int bb_dropout_apply(int dtype, int64_t n, const void* src, void* dst
     return BB_OK;
 }
 extern "C" int bb_dropout_keep_host(float p, uint32_t k0, uint32_t k1, uint64_t index) {
-    const DropKey key = bb_drop_key(p, k0, k1);
+    const DropKey key = bb_drop_key(p, k0, k1, ~0ull);
     return bb_dropout_keep(key.k0, key.k1, key.thresh, index) ? 1 : 0;
 }
 

@@ -249,7 +249,7 @@ static int fill_args(const bb_gemm_desc* d, GemmArgs& g, int64_t& batches, bool&
     BB_REQUIRE(d->dropout_p == 0.f || (batches == 1 && d->layout == BB_NT && d->epilogue != BB_EPI_DACT && d->epilogue != BB_EPI_MUL &&
                                        !d->accumulate),
                "bb_gemm: dropout goes with an unbatched, non-accumulating NT problem and not with the DACT / MUL epilogues");
-    g.drop = bb_drop_key(d->dropout_p, d->dropout_k0, d->dropout_k1);
+    g.drop = bb_drop_key(d->dropout_p, d->dropout_k0, d->dropout_k1, (uint64_t)d->M * (uint64_t)d->N);
     g.tiles_m = g.tiles_n = 0;
     return BB_OK;
 }

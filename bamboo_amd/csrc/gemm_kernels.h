@@ -98,9 +98,11 @@ __device__ __forceinline__ void epilogue_vec8(const GemmArgs& g, int64_t coff, i
         // n is a multiple of 8 and so is N (a condition of the kernels that store eight columns at a time): the index
         // is even, one hash serves two neighbouring columns
         const uint64_t pair = ((uint64_t)m * (uint64_t)g.N + (uint64_t)n) >> 1;
+        const uint32_t pair32 = ((uint32_t)m * (uint32_t)g.N + (uint32_t)n) >> 1;
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
-            const uint32_t x = bb_dropout_pair_bits(g.drop.k0, g.drop.k1, pair + e);
+            const uint32_t x = g.drop.small ? bb_dropout_pair_bits32(g.drop.k0, g.drop.k1, pair32 + e)
+                                            : bb_dropout_pair_bits(g.drop.k0, g.drop.k1, pair + e);
             keep[2 * e] = bb_keep_even(x, g.drop.thresh) ? g.drop.scale : 0.f;
             keep[2 * e + 1] = bb_keep_odd(x, g.drop.thresh) ? g.drop.scale : 0.f;
         }

@@ -228,3 +228,77 @@ def test_rc_bit_exact_with_dropout(hiplib, rc_stream):
             bamboo_amd.initialize(model=m3, config={"train_micro_batch_size_per_gpu": mb, "gradient_accumulation_steps": M,
                                                     "bf16": {"enabled": True}}, activation_queue=q3, use_graphs=True,
                                   install_signal_handler=False)
+
+
+def test_dropout_indices_past_32_bits(hiplib):
+    """Tensors of 2^32 elements and more take the 64-bit index arithmetic (smaller ones, i.e. every other test, the
+    32-bit one): the stand-alone kernel over 2^32 + 4096 elements and the epilogue of a 65536 x 65544 product, on
+    sampled elements either side of the 2^32 boundary, against the oracle's decisions."""
+    p = 0.25
+    n = (1 << 32) + 4096
+    x = torch.ones(n, dtype=torch.bfloat16, device=DEV)
+    y = torch.empty_like(x)
+    hiplib.dropout_apply(x, y, p, KEY)
+    rng = np.random.default_rng(8)
+    idx = np.concatenate([np.arange(64), (1 << 32) - 64 + np.arange(128), n - 64 + np.arange(64),
+                          rng.integers(0, n, 4096)]).astype(np.int64)
+    got = y[torch.from_numpy(idx).to(DEV)].float().cpu().numpy() != 0
+    assert np.array_equal(got, od.keep(p, KEY, idx.astype(np.uint64)))
+    assert abs(float((y[: 1 << 24] != 0).float().mean()) - (1 - p)) < 1e-3 and abs(float((y[-(1 << 24):] != 0).float().mean()) - (1 - p)) < 1e-3
+    del x, y
+    M, N, K = 65536, 65544, 64
+    A = torch.full((M, K), 0.125, dtype=torch.bfloat16, device=DEV)
+    B = torch.full((N, K), 0.125, dtype=torch.bfloat16, device=DEV)
+    C = torch.empty(M, N, dtype=torch.bfloat16, device=DEV)           # every element 1 before dropout
+    hiplib.gemm(hiplib.NT, A, B, C, dropout=(p, KEY))
+    ms = np.concatenate([[0, 1, M - 1, 65527, 65528], rng.integers(0, M, 512)]).astype(np.int64)
+    ns = np.concatenate([[0, 7, N - 1, 8, 65543], rng.integers(0, N, 512)]).astype(np.int64)
+    flat = ms * N + ns
+    assert flat.max() >= 1 << 32
+    got = C[torch.from_numpy(ms).to(DEV), torch.from_numpy(ns).to(DEV)].float().cpu().numpy()
+    keep = od.keep(p, KEY, flat.astype(np.uint64))
+    assert np.array_equal(got != 0, keep)
+    assert np.allclose(got[keep], float(torch.tensor(1.0 / (1.0 - np.float32(p))).bfloat16()))
+
+
+def test_attention_dropout_past_32_bits_of_probabilities(hiplib):
+    """One head over 65536 positions: 2^32 probabilities, so the three fused kernels take the 64-bit index arithmetic.
+    Sampled query rows of the context and of dQ, sampled key rows of dK and dV, against fp64 restatements built from
+    the oracle's decisions."""
+    p, s, d = 0.25, 65536, 64
+    g = torch.Generator(device=DEV).manual_seed(21)
+    qkv = (torch.randn(s, 3 * d, generator=g, device=DEV) * 0.5).bfloat16()
+    d_out = torch.randn(s, d, generator=g, device=DEV).bfloat16()
+    out, lse = torch.empty(s, d, dtype=torch.bfloat16, device=DEV), torch.empty(1, 1, s, device=DEV)
+    delta, d_qkv = torch.empty(1, 1, s, device=DEV), torch.empty_like(qkv)
+    code = hiplib.MASK_CODES["none"]
+    hiplib.attention_fwd(qkv, out, lse, 1, 1, s, code, dropout=(p, KEY))
+    hiplib.attention_bwd(qkv, out, d_out, lse, delta, d_qkv, 1, 1, s, code, dropout=(p, KEY))
+    torch.cuda.synchronize()
+    Q, K, V = [qkv[:, i * d:(i + 1) * d].double().cpu() for i in range(3)]
+    dO, O = d_out.double().cpu(), out.double().cpu()
+    scale = 1.0 / (1.0 - p)
+    cols = torch.arange(s, dtype=torch.int64)
+    for q in (0, 1, 40001, s - 1):
+        sc = (K @ Q[q]) / 8.0
+        prob = torch.softmax(sc, 0)
+        keep = torch.from_numpy(od.keep(p, KEY, (q * s + cols.numpy()).astype(np.uint64))).double()
+        pk = prob * keep * scale
+        assert l2(out[q], pk @ V) < 1e-2, q
+        dpk = (V @ dO[q]) * keep * scale                 # gradient of the kept-and-scaled probabilities
+        dlt = float((dO[q] * O[q]).sum())                # rowsum(dO o O) = sum_kv P~ dP (what the kernels subtract)
+        ds = prob * (dpk - dlt)
+        assert l2(d_qkv[q, :d], (ds @ K) / 8.0) < 3e-2, q
+    # full-column checks need every row's normaliser: recompute it in fp64 for all rows, blockwise
+    lse64 = torch.empty(s, dtype=torch.float64)
+    for lo in range(0, s, 4096):
+        lse64[lo:lo + 4096] = torch.logsumexp((Q[lo:lo + 4096] @ K.t()) / 8.0, dim=1)
+    dlt_all = (dO * O).sum(1)
+    rows = torch.arange(s, dtype=torch.int64).numpy()
+    for kv in (0, 3, 33333, s - 1):
+        prob = torch.exp((Q @ K[kv]) / 8.0 - lse64)
+        keep = torch.from_numpy(od.keep(p, KEY, (rows * s + kv).astype(np.uint64))).double()
+        pk = prob * keep * scale
+        assert l2(d_qkv[kv, 2 * d:], pk @ dO) < 3e-2, kv
+        ds = prob * ((dO @ V[kv]) * keep * scale - dlt_all)
+        assert l2(d_qkv[kv, d:2 * d], (ds @ Q) / 8.0) < 3e-2, kv
