@@ -7,7 +7,8 @@ the reference's own scripts are made of -- by the names and shapes of their para
 script's local copy of the class is recognised too -- build the native layer that computes the same function, and
 take the module's weights into the stage's arenas:
 
-  ``EncoderLayer``   (DeepSpeedExamples/pipeline_parallelism/transformer.py:161-172)  -> :class:`TransformerLayer`
+  ``EncoderLayer``   (DeepSpeedExamples/pipeline_parallelism/transformer.py:161-172;
+                     ``EncoderLayerSimple``, bert.py:20-31: same parameters, same function)   -> :class:`TransformerLayer`
   ``LayerNorm``      (transformer.py:77-88, the ``encoder.norm`` of :181,250)          -> :class:`FinalLayerNorm`
   ``lambda x: x.sum(-1)`` (transformer.py:250)                                        -> :class:`SumLast`
   ``BottleNeck``     (DeepSpeedExamples/pipeline_parallelism/resnet.py:49-75)          -> :class:`BottleNeck`
