@@ -1123,21 +1123,40 @@ __global__ __launch_bounds__(256) void bn_finish_kernel(int what, int rows, int 
     }
 }
 
-// Forward statistics from the strip triples a convolution's GEMM epilogue leaves (per 32 rows and channel:
-// pivot p, S1 = sum (x - p), S2 = sum (x - p)^2).  A strip's mean is p + S1/n and its sum of squared deviations
-// M2 = S2 - S1^2/n (no cancellation: p is a sample of the strip).  Two passes over the triples, which stay in
-// registers (at most 8192 rows): mean = sum n_s mean_s / rows, then sum of squared deviations = sum (M2_s + n_s (mean_s - mean)^2) -
-// again no cancellation.  One block owns 64 channels (lane = channel: 256-byte reads); its sixteen waves take
-// strips w, w + 16, ...; the sixteen partial sums are added in wave order by every thread (fixed order).
+// Forward BatchNorm from the strip triples a convolution's GEMM epilogue leaves (per 32 rows and channel: pivot p,
+// S1 = sum (x - p), S2 = sum (x - p)^2), statistics and normalisation in ONE launch.  A block owns 64 channels and
+// one of gridDim.y row ranges.  Every block first turns the strips of its channels into mean and variance -- a
+// strip's mean is p + S1/n and its sum of squared deviations M2 = S2 - S1^2/n (no cancellation: p is a sample of the
+// strip); two passes over the triples, which stay in registers (at most 8192 rows): mean = sum n_s mean_s / rows,
+// then sum (M2_s + n_s (mean_s - mean)^2) -- lane = channel (256-byte reads), its sixteen waves taking strips w,
+// w + 16, ..., the sixteen partial sums added in wave order by every thread (a fixed order, the same in every
+// block: all row ranges of a channel normalise with the same bits).  The block of the first row range also writes
+// mean, rstd and the running statistics.  Then y = gamma (x - mean) rstd + beta (+ resid) (ReLU) over the block's
+// rows, eight lanes per row of the 64 channels (128-byte segments).  The tensor is read once; repeating the small
+// strip reduction per row range is cheaper than a launch of its own.
 constexpr int BN_STRIP_WAVES = 16, BN_STRIP_MAX = 16;   // 16 * 16 strips = up to 8192 rows
-__global__ __launch_bounds__(BN_STRIP_WAVES * 64) void bn_finish_strips_kernel(int rows, int cols, float eps, float momentum,
-                                                               const float* __restrict__ strips, float* __restrict__ mean,
-                                                               float* __restrict__ rstd, float* __restrict__ run_mean,
-                                                               float* __restrict__ run_var) {
+constexpr int BN_FWD_ROW_RANGES = 64;
+__global__ __launch_bounds__(BN_STRIP_WAVES * 64) void bn_fwd_strips_kernel(int rows, int cols, float eps, float momentum, int relu,
+                                                            const float* __restrict__ strips, const bf16* __restrict__ x,
+                                                            const bf16* __restrict__ gamma, const bf16* __restrict__ beta,
+                                                            const bf16* __restrict__ resid, bf16* __restrict__ y,
+                                                            float* __restrict__ mean, float* __restrict__ rstd,
+                                                            float* __restrict__ run_mean, float* __restrict__ run_var) {
     __shared__ float red[2][BN_STRIP_WAVES][64];
+    __shared__ float fold[2][64];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int c = min(blockIdx.x * 64 + lane, cols - 1);   // lanes past the last channel repeat it and store nothing
     const int nstrips = (rows + 31) / 32;
+    // the rows this thread normalises first are fetched now, so that they travel while the statistics are reduced
+    const int v8 = (threadIdx.x & 7) * 8, c0 = blockIdx.x * 64 + v8;
+    const int per = (rows + gridDim.y - 1) / gridDim.y;
+    const int r0 = blockIdx.y * per + (threadIdx.x >> 3), r1 = min(rows, ((int)blockIdx.y + 1) * per);
+    const bool first = c0 < cols && r0 < r1;
+    float xv[8], rv[8];
+    if (first) {
+        load_vec(x + (int64_t)r0 * cols + c0, xv);
+        if (resid) load_vec(resid + (int64_t)r0 * cols + c0, rv);
+    }
     float p[BN_STRIP_MAX], a[BN_STRIP_MAX], b[BN_STRIP_MAX];
 #pragma unroll
     for (int j = 0; j < BN_STRIP_MAX; ++j) {
@@ -1173,16 +1192,50 @@ __global__ __launch_bounds__(BN_STRIP_WAVES * 64) void bn_finish_strips_kernel(i
     }
     red[1][wave][lane] = sq;
     __syncthreads();
-    if (wave != 0 || blockIdx.x * 64 + lane >= cols) return;
-    float q = 0.f;
+    if (wave == 0) {
+        float q = 0.f;
 #pragma unroll
-    for (int w = 0; w < BN_STRIP_WAVES; ++w) q += red[1][w][lane];
-    const float var = fmaxf(q / (float)rows, 0.f);
-    mean[c] = mu;
-    rstd[c] = 1.0f / sqrtf(var + eps);
-    if (run_mean) {  // nn.BatchNorm2d: running_var uses the unbiased estimate
-        run_mean[c] = (1.f - momentum) * run_mean[c] + momentum * mu;
-        run_var[c] = (1.f - momentum) * run_var[c] + momentum * var * (float)rows / (float)(rows - 1);
+        for (int w = 0; w < BN_STRIP_WAVES; ++w) q += red[1][w][lane];
+        const float var = fmaxf(q / (float)rows, 0.f);
+        const float rs = 1.0f / sqrtf(var + eps);
+        const float sc = Elem<bf16>::load(gamma + c) * rs;
+        fold[0][lane] = sc;
+        fold[1][lane] = Elem<bf16>::load(beta + c) - mu * sc;
+        if (blockIdx.y == 0 && blockIdx.x * 64 + lane < cols) {
+            mean[c] = mu;
+            rstd[c] = rs;
+            if (run_mean) {  // nn.BatchNorm2d: running_var uses the unbiased estimate
+                run_mean[c] = (1.f - momentum) * run_mean[c] + momentum * mu;
+                run_var[c] = (1.f - momentum) * run_var[c] + momentum * var * (float)rows / (float)(rows - 1);
+            }
+        }
+    }
+    __syncthreads();
+    // normalise the block's rows: thread = (row within a pass of 128, eight channels)
+    if (c0 >= cols) return;
+    float sc[8], sh[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+        sc[e] = fold[0][v8 + e];
+        sh[e] = fold[1][v8 + e];
+    }
+    for (int r = r0; r < r1; r += BN_STRIP_WAVES * 8) {
+        const int64_t off = (int64_t)r * cols + c0;
+        if (r != r0) {
+            load_vec(x + off, xv);
+            if (resid) load_vec(resid + off, rv);
+        }
+#pragma unroll
+        for (int e = 0; e < 8; ++e) xv[e] = fmaf(xv[e], sc[e], sh[e]);
+        if (resid) {
+#pragma unroll
+            for (int e = 0; e < 8; ++e) xv[e] += rv[e];
+        }
+        if (relu) {
+#pragma unroll
+            for (int e = 0; e < 8; ++e) xv[e] = fmaxf(xv[e], 0.f);
+        }
+        store_vec(y + off, xv);
     }
 }
 
@@ -1230,48 +1283,87 @@ __global__ __launch_bounds__(256) void bn_apply_kernel(int64_t nvec, int cols, i
     }
 }
 
-// backward apply: g = dy * (relu_out > 0); dx = gamma * rstd * (g - mean(g) - xhat * mean(g * xhat));
-// optionally also writes g itself (the gradient that flows into the residual branch)
+// Backward BatchNorm after the column reduction, finish and apply in ONE launch: a block owns 64 channels and one of
+// gridDim.y row ranges.  It first adds up the BN_SPLITS partial rows of its channels (sum g and sum g * xhat; sixteen
+// thread groups take four partial rows each, the sixteen sums are added in group order: the same bits in every
+// block), folds dx = k g + a x + b per channel (k = gamma rstd, a = -k mean(g xhat) rstd, b = -k mean(g) - a mean)
+// -- the block of the first row range also accumulates dgamma and dbeta -- and then applies it to its rows, whose
+// first pass was fetched before the reduction.
 template <typename T>
-__global__ __launch_bounds__(256) void bn_bwd_apply_kernel(int64_t nvec, int cols, const T* __restrict__ x,
-                                                           const float* __restrict__ mean, const float* __restrict__ rstd,
-                                                           const T* __restrict__ gamma, const float* __restrict__ sums,
-                                                           const T* __restrict__ dy, const T* __restrict__ relu_out,
-                                                           T* __restrict__ dx, T* __restrict__ g_out) {
-    constexpr int VEC = Elem<T>::VEC;
-    // dx = k (g - mean(g) - xhat mean(g xhat)), k = gamma rstd, folded per channel into
-    // dx = k g + a x + b; a thread keeps its channels when the grid stride is a multiple of a row
-    const int64_t stride = (int64_t)gridDim.x * 256;
-    const bool fixed = stride % (cols / VEC) == 0;
+__global__ __launch_bounds__(1024) void bn_bwd_finish_apply_kernel(int rows, int cols, const float* __restrict__ partial,
+                                                                   const T* __restrict__ x, const float* __restrict__ mean,
+                                                                   const float* __restrict__ rstd, const T* __restrict__ gamma,
+                                                                   const T* __restrict__ dy, const T* __restrict__ relu_out,
+                                                                   T* __restrict__ dx, T* __restrict__ g_out,
+                                                                   float* __restrict__ dgamma, float* __restrict__ dbeta) {
+    constexpr int VEC = Elem<T>::VEC, LPR = 64 / VEC, RPP = 1024 / LPR;   // lanes per row of the slab, rows per pass
+    static_assert(BN_SPLITS == 64, "sixteen groups of four partial rows");
+    __shared__ float red[2][16][64];
+    __shared__ float fold[3][64];
+    const int lane = threadIdx.x & 63, grp = threadIdx.x >> 6;
+    const int c = min(blockIdx.x * 64 + lane, cols - 1);
+    const int vc = (threadIdx.x % LPR) * VEC, c0 = blockIdx.x * 64 + vc;
+    const int per = (rows + gridDim.y - 1) / gridDim.y;
+    const int r0 = blockIdx.y * per + threadIdx.x / LPR, r1 = min(rows, ((int)blockIdx.y + 1) * per);
+    const bool first = c0 < cols && r0 < r1;
+    float xv[VEC], gv[VEC], ov[VEC];
+    if (first) {
+        const int64_t off = (int64_t)r0 * cols + c0;
+        load_vec(x + off, xv);
+        load_vec(dy + off, gv);
+        if (relu_out) load_vec(relu_out + off, ov);
+    }
+    float t0[4], t1[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        t0[j] = partial[((int64_t)(grp * 4 + j) * 2) * cols + c];
+        t1[j] = partial[((int64_t)(grp * 4 + j) * 2 + 1) * cols + c];
+    }
+    red[0][grp][lane] = (t0[0] + t0[1]) + (t0[2] + t0[3]);
+    red[1][grp][lane] = (t1[0] + t1[1]) + (t1[2] + t1[3]);
+    __syncthreads();
+    if (grp == 0) {
+        float s0 = 0.f, s1 = 0.f;
+#pragma unroll
+        for (int q = 0; q < 16; ++q) {
+            s0 += red[0][q][lane];
+            s1 += red[1][q][lane];
+        }
+        const float rs = rstd[c], k = Elem<T>::load(gamma + c) * rs;
+        const float ka = -k * (s1 / (float)rows) * rs;
+        fold[0][lane] = k;
+        fold[1][lane] = ka;
+        fold[2][lane] = -k * (s0 / (float)rows) - ka * mean[c];
+        if (blockIdx.y == 0 && blockIdx.x * 64 + lane < cols) {
+            dbeta[c] += s0;
+            dgamma[c] += s1;
+        }
+    }
+    __syncthreads();
+    if (c0 >= cols) return;
     float k[VEC], ka[VEC], kb[VEC];
-    auto fold = [&](int c0) {
-        float gm[VEC];
-        load_vec(gamma + c0, gm);
 #pragma unroll
-        for (int e = 0; e < VEC; ++e) {
-            const float rs = rstd[c0 + e];
-            k[e] = gm[e] * rs;
-            ka[e] = -k[e] * sums[cols + c0 + e] * rs;
-            kb[e] = -k[e] * sums[c0 + e] - ka[e] * mean[c0 + e];
+    for (int e = 0; e < VEC; ++e) {
+        k[e] = fold[0][vc + e];
+        ka[e] = fold[1][vc + e];
+        kb[e] = fold[2][vc + e];
+    }
+    for (int r = r0; r < r1; r += RPP) {
+        const int64_t off = (int64_t)r * cols + c0;
+        if (r != r0) {
+            load_vec(x + off, xv);
+            load_vec(dy + off, gv);
+            if (relu_out) load_vec(relu_out + off, ov);
         }
-    };
-    const int64_t first = (int64_t)blockIdx.x * 256 + threadIdx.x;
-    if (fixed && first < nvec) fold((int)((first * VEC) % cols));
-    for (int64_t i = first; i < nvec; i += stride) {
-        if (!fixed) fold((int)((i * VEC) % cols));
-        float v[VEC], g[VEC], o[VEC];
-        load_vec(x + i * VEC, v);
-        load_vec(dy + i * VEC, g);
         if (relu_out) {
-            float ro[VEC];
-            load_vec(relu_out + i * VEC, ro);
 #pragma unroll
-            for (int e = 0; e < VEC; ++e) g[e] = ro[e] > 0.f ? g[e] : 0.f;
+            for (int e = 0; e < VEC; ++e) gv[e] = ov[e] > 0.f ? gv[e] : 0.f;
         }
+        float o[VEC];
 #pragma unroll
-        for (int e = 0; e < VEC; ++e) o[e] = fmaf(k[e], g[e], fmaf(ka[e], v[e], kb[e]));
-        store_vec(dx + i * VEC, o);
-        if (g_out) store_vec(g_out + i * VEC, g);
+        for (int e = 0; e < VEC; ++e) o[e] = fmaf(k[e], gv[e], fmaf(ka[e], xv[e], kb[e]));
+        store_vec(dx + off, o);
+        if (g_out) store_vec(g_out + off, gv);
     }
 }
 
@@ -1320,11 +1412,12 @@ extern "C" int bb_batchnorm_fwd_strips(int dtype, int rows, int cols, float eps,
     BB_REQUIRE(rows <= 32 * BN_STRIP_WAVES * BN_STRIP_MAX, "bb_batchnorm_fwd_strips: at most %d rows", 32 * BN_STRIP_WAVES * BN_STRIP_MAX);
     BB_REQUIRE((running_mean == nullptr) == (running_var == nullptr), "bb_batchnorm_fwd_strips: give both running buffers or none");
     hipStream_t st = (hipStream_t)stream;
-    const int64_t nvec = (int64_t)rows * cols / 8;
-    hipLaunchKernelGGL(bn_finish_strips_kernel, dim3((cols + 63) / 64), dim3(BN_STRIP_WAVES * 64), 0, st, rows, cols, eps, momentum, strip_stats,
-                       mean, rstd, running_mean, running_var);
-    hipLaunchKernelGGL(bn_apply_kernel<bf16>, dim3(grid_for(nvec)), dim3(256), 0, st, nvec, cols, relu, (const bf16*)x, mean, rstd,
-                       (const bf16*)gamma, (const bf16*)beta, (const bf16*)resid, (bf16*)y);
+    // about one block per CU; wide tensors get fewer row ranges (each repeats the strip reduction of its channels)
+    const int slabs = (cols + 63) / 64;
+    const int ranges = max(4, min(BN_FWD_ROW_RANGES, 256 / slabs));
+    hipLaunchKernelGGL(bn_fwd_strips_kernel, dim3(slabs, ranges), dim3(BN_STRIP_WAVES * 64), 0, st, rows, cols, eps, momentum, relu,
+                       strip_stats, (const bf16*)x, (const bf16*)gamma, (const bf16*)beta, (const bf16*)resid, (bf16*)y, mean, rstd,
+                       running_mean, running_var);
     BB_LAUNCH_CHECK();
     return BB_OK;
 }
@@ -1337,18 +1430,16 @@ extern "C" int bb_batchnorm_bwd(int dtype, int rows, int cols, const void* x, co
     BB_REQUIRE(x && gamma && mean && rstd && dy && dx && dgamma && dbeta && workspace, "bb_batchnorm_bwd: null pointer");
     hipStream_t st = (hipStream_t)stream;
     const int vec = dtype == BB_BF16 ? 8 : 4;
-    dim3 grid((cols + 64 * vec - 1) / (64 * vec), BN_SPLITS), fgrid((cols + 31) / 32);
-    const int64_t nvec = (int64_t)rows * cols / vec;
-    float* sums = workspace + (int64_t)BN_SPLITS * 2 * cols;
+    dim3 grid((cols + 64 * vec - 1) / (64 * vec), BN_SPLITS);
+    const int slabs = (cols + 63) / 64;
+    dim3 agrid(slabs, max(4, min(64, 256 / slabs)));   // about one block per CU
     const dim3 block(BN_WAVES * 64);
     if (dtype == BB_BF16) {
         hipLaunchKernelGGL((bn_colred_kernel<bf16, 2>), grid, block, 0, st, rows, cols, (const bf16*)x, mean, rstd, (const bf16*)dy, (const bf16*)relu_out, workspace);
-        hipLaunchKernelGGL(bn_finish_kernel<bf16>, fgrid, dim3(256), 0, st, 2, rows, cols, 0.f, 0.f, workspace, (const bf16*)x, nullptr, nullptr, nullptr, nullptr, dgamma, dbeta, sums);
-        hipLaunchKernelGGL(bn_bwd_apply_kernel<bf16>, dim3(grid_for(nvec)), dim3(256), 0, st, nvec, cols, (const bf16*)x, mean, rstd, (const bf16*)gamma, sums, (const bf16*)dy, (const bf16*)relu_out, (bf16*)dx, (bf16*)g_out);
+        hipLaunchKernelGGL(bn_bwd_finish_apply_kernel<bf16>, agrid, dim3(1024), 0, st, rows, cols, workspace, (const bf16*)x, mean, rstd, (const bf16*)gamma, (const bf16*)dy, (const bf16*)relu_out, (bf16*)dx, (bf16*)g_out, dgamma, dbeta);
     } else {
         hipLaunchKernelGGL((bn_colred_kernel<float, 2>), grid, block, 0, st, rows, cols, (const float*)x, mean, rstd, (const float*)dy, (const float*)relu_out, workspace);
-        hipLaunchKernelGGL(bn_finish_kernel<float>, fgrid, dim3(256), 0, st, 2, rows, cols, 0.f, 0.f, workspace, (const float*)x, nullptr, nullptr, nullptr, nullptr, dgamma, dbeta, sums);
-        hipLaunchKernelGGL(bn_bwd_apply_kernel<float>, dim3(grid_for(nvec)), dim3(256), 0, st, nvec, cols, (const float*)x, mean, rstd, (const float*)gamma, sums, (const float*)dy, (const float*)relu_out, (float*)dx, (float*)g_out);
+        hipLaunchKernelGGL(bn_bwd_finish_apply_kernel<float>, agrid, dim3(1024), 0, st, rows, cols, workspace, (const float*)x, mean, rstd, (const float*)gamma, (const float*)dy, (const float*)relu_out, (float*)dx, (float*)g_out, dgamma, dbeta);
     }
     BB_LAUNCH_CHECK();
     return BB_OK;
