@@ -372,7 +372,8 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dkv_kernel(const AttnArgs a) 
 
     // query range that can see keys of this block
     const int q_begin = a.mask == BB_MASK_CAUSAL ? (kb * 128) / 64 : 0;  // first 64-query tile
-    const int ntiles = (a.seq + 63) / 64;
+    // a block whose 128 keys are all padding has nothing to accumulate: it only stores its zeros
+    const int ntiles = kb * 128 >= pad_limit ? 0 : (a.seq + 63) / 64;
 
     bf16x8 kf[4], vf[4];
     {
