@@ -304,9 +304,36 @@ def gemm_batched(layout, dtype, M, N, K, A_ptr, lda, sA, B_ptr, ldb, sB, C_ptr, 
     check(lib().bb_gemm(byref(d), stream_ptr(stream)), "bb_gemm(batched)")
 
 
+
+# ---- operand checks: the C ABI takes raw pointers, so what a kernel and its grid assume about its operands is
+# ---- verified here, before anything is launched (a tensor that is too small would be an out-of-bounds access on
+# ---- the GPU)
+def _like(what, ref, **tensors):
+    """Every given tensor (None allowed) is contiguous and has the shape and dtype of ``ref``."""
+    if not ref.is_contiguous():
+        raise HipKernelError(f"{what}: operands must be contiguous, got strides {ref.stride()} for {tuple(ref.shape)}")
+    for name, t in tensors.items():
+        if t is None:
+            continue
+        if tuple(t.shape) != tuple(ref.shape) or t.dtype != ref.dtype or not t.is_contiguous():
+            raise HipKernelError(f"{what}: {name} must be a contiguous {tuple(ref.shape)} tensor of {ref.dtype}, got "
+                                 f"{tuple(t.shape)} {t.dtype} strides {t.stride()}")
+
+
+def _vector(what, n, dtype, **tensors):
+    """Every given tensor (None allowed) holds exactly ``n`` contiguous elements of ``dtype``."""
+    for name, t in tensors.items():
+        if t is None:
+            continue
+        if t.numel() != n or t.dtype != dtype or not t.is_contiguous():
+            raise HipKernelError(f"{what}: {name} must hold {n} contiguous elements of {dtype}, got {tuple(t.shape)} {t.dtype}")
+
 # ------------------------------------------------------------------------- row-wise kernels
 def layernorm_fwd(x, gain, shift, y, mean, rinv, kind, eps, stream=None):
     rows, cols = x.shape
+    _like("layernorm_fwd", x, y=y)
+    _vector("layernorm_fwd", cols, x.dtype, gain=gain, shift=shift)
+    _vector("layernorm_fwd", rows, torch.float32, mean=mean, rinv=rinv)
     check(lib().bb_layernorm_fwd(dtype_code(x.dtype), kind, rows, cols, eps, _ptr(x), _ptr(gain), _ptr(shift),
                                  _ptr(y), _ptr(mean), _ptr(rinv), stream_ptr(stream)), "bb_layernorm_fwd")
 
@@ -315,8 +342,17 @@ def layernorm_bwd_workspace(cols):
     return int(lib().bb_layernorm_bwd_workspace(cols))
 
 
+def _check_ln_bwd(what, x, gain, mean, rinv, dy, dres, dx, dgain, dshift):
+    rows, cols = x.shape
+    _like(what, x, dy=dy, dres=dres, dx=dx)
+    _vector(what, cols, x.dtype, gain=gain)
+    _vector(what, rows, torch.float32, mean=mean, rinv=rinv)
+    _vector(what, cols, torch.float32, dgain=dgain, dshift=dshift)
+
+
 def layernorm_bwd(x, gain, mean, rinv, dy, dres, dx, dgain, dshift, workspace, kind, eps, stream=None):
     rows, cols = x.shape
+    _check_ln_bwd("layernorm_bwd", x, gain, mean, rinv, dy, dres, dx, dgain, dshift)
     if workspace.numel() < layernorm_bwd_workspace(cols) or workspace.dtype != torch.float32:
         raise HipKernelError("layernorm_bwd: workspace too small")
     check(lib().bb_layernorm_bwd(dtype_code(x.dtype), kind, rows, cols, eps, _ptr(x), _ptr(gain), _ptr(mean),
@@ -328,6 +364,7 @@ def layernorm_bwd_static(x, gain, mean, rinv, dy, dres, dx, dgain, dshift, kind,
     """:func:`layernorm_bwd` on the library's built-in scratch array: allocates nothing, cols <= 2048, calls that
     overlap on one GPU race."""
     rows, cols = x.shape
+    _check_ln_bwd("layernorm_bwd_static", x, gain, mean, rinv, dy, dres, dx, dgain, dshift)
     check(lib().bb_layernorm_bwd_static(dtype_code(x.dtype), kind, rows, cols, eps, _ptr(x), _ptr(gain), _ptr(mean),
                                         _ptr(rinv), _ptr(dy), _ptr(dres), _ptr(dx), _ptr(dgain), _ptr(dshift),
                                         stream_ptr(stream)), "bb_layernorm_bwd_static")
@@ -366,14 +403,14 @@ def softmax_fwd(s, mask, key_len=None, stream=None):
     b, h, sq, sk = s.shape
     if not s.is_contiguous():
         raise HipKernelError("softmax_fwd: scores must be contiguous")
+    _vector("softmax_fwd", b, torch.int32, key_len=key_len)
     check(lib().bb_softmax_fwd(dtype_code(s.dtype), mask, b, h, sq, sk, _ptr(s), _ptr(key_len),
                                stream_ptr(stream)), "bb_softmax_fwd")
 
 
 def softmax_bwd(p, dp, stream=None):
     b, h, sq, sk = p.shape
-    if not (p.is_contiguous() and dp.is_contiguous()):
-        raise HipKernelError("softmax_bwd: tensors must be contiguous")
+    _like("softmax_bwd", p, dp=dp)
     check(lib().bb_softmax_bwd(dtype_code(p.dtype), b, h, sq, sk, _ptr(p), _ptr(dp), stream_ptr(stream)),
           "bb_softmax_bwd")
 
@@ -384,9 +421,24 @@ def _drop_args(dropout):
     return float(dropout[0]), int(dropout[1][0]), int(dropout[1][1])
 
 
+def _check_attention(what, qkv, batch, heads, seq, key_len, lse, out=None, d_out=None, delta=None, d_qkv=None):
+    """qkv / d_qkv: [batch*seq, 3*heads*64], out / d_out: [batch*seq, heads*64] (rows may be strided views with a unit
+    inner stride), lse / delta: fp32 with batch*heads*seq contiguous elements, key_len: int32 [batch]."""
+    rows, h = batch * seq, heads * 64
+    for name, t, width in (("qkv", qkv, 3 * h), ("d_qkv", d_qkv, 3 * h), ("out", out, h), ("d_out", d_out, h)):
+        if t is None:
+            continue
+        if t.dim() != 2 or tuple(t.shape) != (rows, width) or t.stride(1) != 1 or t.stride(0) < width or t.dtype != qkv.dtype:
+            raise HipKernelError(f"{what}: {name} must be [{rows}, {width}] of {qkv.dtype} with unit inner stride for batch={batch} "
+                                 f"heads={heads} seq={seq}, got {tuple(t.shape)} {t.dtype} strides {t.stride()}")
+    _vector(what, batch * heads * seq, torch.float32, lse=lse, delta=delta)
+    _vector(what, batch, torch.int32, key_len=key_len)
+
+
 def attention_fwd(qkv, out, lse, batch, heads, seq, mask, key_len=None, stream=None, dropout=None):
     """qkv: [batch*seq, 3*heads*64] (Q | K | V thirds), out: [batch*seq, heads*64], lse: fp32 [batch, heads, seq].
     ``dropout=(p, (k0, k1))``: dropout on the probabilities with the decisions of that key."""
+    _check_attention("attention_fwd", qkv, batch, heads, seq, key_len, lse, out=out)
     h = heads * 64
     es = qkv.element_size()
     q = qkv.data_ptr()
@@ -397,6 +449,9 @@ def attention_fwd(qkv, out, lse, batch, heads, seq, mask, key_len=None, stream=N
 
 
 def attention_bwd(qkv, out, d_out, lse, delta, d_qkv, batch, heads, seq, mask, key_len=None, stream=None, dropout=None):
+    _check_attention("attention_bwd", qkv, batch, heads, seq, key_len, lse, out=out, d_out=d_out, delta=delta, d_qkv=d_qkv)
+    if d_out.stride(0) != out.stride(0):
+        raise HipKernelError("attention_bwd: out and d_out must share one leading dimension")
     h = heads * 64
     es = qkv.element_size()
     q, dq = qkv.data_ptr(), d_qkv.data_ptr()
@@ -436,12 +491,14 @@ def dropout_key(base_seed, step, micro_batch, layer_idx, site):
 
 
 def residual_add(a, b, out, stream=None):
+    _like("residual_add", a, b=b, out=out)
     check(lib().bb_residual_add(dtype_code(a.dtype), a.numel(), _ptr(a), _ptr(b), _ptr(out), stream_ptr(stream)),
           "bb_residual_add")
 
 
 def act_fwd(x, out, act, dact=None, stream=None):
     """out = act(x); dact (optional, may be x itself) receives act'(x)."""
+    _like("act_fwd", x, out=out, dact=dact)
     check(lib().bb_act_fwd(dtype_code(x.dtype), act, x.numel(), _ptr(x), _ptr(out), _ptr(dact), stream_ptr(stream)),
           "bb_act_fwd")
 
@@ -494,6 +551,9 @@ def batchnorm_fwd(x, gamma, beta, resid, y, mean, rstd, run_mean, run_var, works
     """``strip_stats``: the statistics the kernel that produced ``x`` left (``gemm(..., strip_stats=)``,
     ``conv3x3(..., strip_stats=)``); the statistics pass over ``x`` is then skipped."""
     rows, cols = x.shape
+    _like("batchnorm_fwd", x, resid=resid, y=y)
+    _vector("batchnorm_fwd", cols, x.dtype, gamma=gamma, beta=beta)
+    _vector("batchnorm_fwd", cols, torch.float32, mean=mean, rstd=rstd, run_mean=run_mean, run_var=run_var)
     if strip_stats is not None:
         _check_strip_stats(strip_stats, rows, cols)
         check(lib().bb_batchnorm_fwd_strips(dtype_code(x.dtype), rows, cols, eps, momentum, int(relu), _ptr(x), _ptr(gamma),
@@ -509,6 +569,9 @@ def batchnorm_fwd(x, gamma, beta, resid, y, mean, rstd, run_mean, run_var, works
 
 def batchnorm_bwd(x, gamma, mean, rstd, dy, relu_out, dx, g_out, dgamma, dbeta, workspace, stream=None):
     rows, cols = x.shape
+    _like("batchnorm_bwd", x, dy=dy, relu_out=relu_out, dx=dx, g_out=g_out)
+    _vector("batchnorm_bwd", cols, x.dtype, gamma=gamma)
+    _vector("batchnorm_bwd", cols, torch.float32, mean=mean, rstd=rstd, dgamma=dgamma, dbeta=dbeta)
     if workspace.numel() < bn_workspace(cols):
         raise HipKernelError("batchnorm_bwd: workspace too small")
     check(lib().bb_batchnorm_bwd(dtype_code(x.dtype), rows, cols, _ptr(x), _ptr(gamma), _ptr(mean), _ptr(rstd),
@@ -589,6 +652,11 @@ def mse_workspace():
 
 
 def mse_fwd_bwd(y, target, dy, grad_scale, loss_out, accumulate, workspace, stream=None):
+    if not y.is_contiguous():
+        raise HipKernelError("mse_fwd_bwd: operands must be contiguous")
+    _vector("mse_fwd_bwd", y.numel(), y.dtype, target=target, dy=dy)
+    if loss_out.dtype != torch.float32 or loss_out.numel() < 1 or workspace.dtype != torch.float32 or workspace.numel() < mse_workspace():
+        raise HipKernelError("mse_fwd_bwd: loss_out / workspace must be fp32 (1 resp. mse_workspace() elements)")
     check(lib().bb_mse_fwd_bwd(dtype_code(y.dtype), y.numel(), _ptr(y), _ptr(target), _ptr(dy), grad_scale,
                                _ptr(loss_out), int(accumulate), _ptr(workspace), stream_ptr(stream)),
           "bb_mse_fwd_bwd")
@@ -612,6 +680,8 @@ def adam_multi(g, p, m, v, lowp, *, lr, beta1, beta2, eps, step, adam_w_mode=Tru
 
 
 def cast(src, dst, stream=None):
+    if src.numel() != dst.numel() or not (src.is_contiguous() and dst.is_contiguous()):
+        raise HipKernelError(f"cast: contiguous tensors of one size expected, got {tuple(src.shape)} -> {tuple(dst.shape)}")
     check(lib().bb_cast(dtype_code(src.dtype), dtype_code(dst.dtype), src.numel(), _ptr(src), _ptr(dst),
                         stream_ptr(stream)), "bb_cast")
 

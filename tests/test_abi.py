@@ -153,3 +153,41 @@ def test_engine_flag_errors_without_gpu():
     from bamboo_amd.utils import get_redundant_stage_ids
     assert get_redundant_stage_ids(1, 1, 4) == [2]
     assert get_redundant_stage_ids(0, 1, 4) == []
+
+
+def test_wrappers_refuse_operands_that_do_not_fit_before_any_launch():
+    """The C ABI takes raw pointers; the ctypes layer checks what a kernel and its grid assume about its operands
+    (shapes, dtypes, contiguity) and raises before anything is launched -- here on CPU tensors, without a GPU."""
+    import pytest
+    import torch
+
+    from bamboo_amd import hip
+    bf, f32 = torch.bfloat16, torch.float32
+    batch, heads, seq = 2, 2, 64
+    h = heads * 64
+    qkv, out = torch.zeros(batch * seq, 3 * h, dtype=bf), torch.zeros(batch * seq, h, dtype=bf)
+    lse = torch.zeros(batch, heads, seq)
+    with pytest.raises(hip.HipKernelError, match="qkv must be"):
+        hip.attention_fwd(qkv, out, lse, batch + 1, heads, seq, 0)              # more samples than the tensor holds
+    with pytest.raises(hip.HipKernelError, match="lse"):
+        hip.attention_fwd(qkv, out, lse[:, :1], batch, heads, seq, 0)
+    with pytest.raises(hip.HipKernelError, match="key_len"):
+        hip.attention_fwd(qkv, out, lse, batch, heads, seq, 2, key_len=torch.zeros(batch + 1, dtype=torch.int32))
+    with pytest.raises(hip.HipKernelError, match="d_qkv"):
+        hip.attention_bwd(qkv, out, out.clone(), lse, lse.clone(), qkv[:-1], batch, heads, seq, 0)
+    x = torch.zeros(16, 32, dtype=bf)
+    with pytest.raises(hip.HipKernelError, match="mean"):
+        hip.layernorm_fwd(x, torch.zeros(32, dtype=bf), torch.zeros(32, dtype=bf), torch.zeros_like(x), torch.zeros(15), torch.zeros(16), 0, 1e-5)
+    with pytest.raises(hip.HipKernelError, match="gain"):
+        hip.layernorm_fwd(x, torch.zeros(32), torch.zeros(32, dtype=bf), torch.zeros_like(x), torch.zeros(16), torch.zeros(16), 0, 1e-5)
+    with pytest.raises(hip.HipKernelError, match="contiguous"):
+        hip.layernorm_fwd(x.t(), torch.zeros(16, dtype=bf), torch.zeros(16, dtype=bf), torch.zeros(32, 16, dtype=bf), torch.zeros(32), torch.zeros(32), 0, 1e-5)
+    with pytest.raises(hip.HipKernelError, match="dy"):
+        hip.batchnorm_bwd(x, torch.zeros(32, dtype=bf), torch.zeros(32), torch.zeros(32), x[:8], None, torch.zeros_like(x), None,
+                          torch.zeros(32), torch.zeros(32), torch.zeros(1))
+    with pytest.raises(hip.HipKernelError, match="out"):
+        hip.residual_add(x, x, torch.zeros(16, 32))
+    with pytest.raises(hip.HipKernelError, match="target"):
+        hip.mse_fwd_bwd(x, x[:8], torch.zeros_like(x), 1.0, torch.zeros(1), False, torch.zeros(4096))
+    with pytest.raises(hip.HipKernelError, match="cast"):
+        hip.cast(x, torch.zeros(8, 32))
