@@ -321,31 +321,6 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const AttnArgs a) {
 }
 
 // =========================================================================================
-// backward, preparation: delta[b, head, q] = sum_d dO[q, d] * O[q, d]
-// =========================================================================================
-__global__ __launch_bounds__(256) void attn_delta_kernel(const AttnArgs a) {
-    // Eight lanes per (row, head): each takes 16 bytes of the head's 128-byte slice of O and of dO (one cache line per
-    // group and tensor), products summed over the group by three shuffles.  A block covers 32 consecutive rows of one
-    // head, so the results leave as one run of 32 floats.
-    const int lane8 = threadIdx.x & 7, g = threadIdx.x >> 3;
-    const int head = blockIdx.y;
-    const int64_t rows = (int64_t)a.batch * a.seq;
-    const int64_t row = min((int64_t)blockIdx.x * 32 + g, rows - 1);   // rows past the end repeat the last one, store nothing
-    float x[8], y[8];
-    load_vec(a.o + row * a.ld_o + head * 64 + lane8 * 8, x);
-    load_vec(a.d_o + row * a.ld_o + head * 64 + lane8 * 8, y);
-    float s = 0.f;
-#pragma unroll
-    for (int e = 0; e < 8; ++e) s += x[e] * y[e];
-#pragma unroll
-    for (int o = 1; o < 8; o <<= 1) s += __shfl_xor(s, o, 64);
-    if (lane8 == 0 && (int64_t)blockIdx.x * 32 + g < rows) {
-        const int b = (int)(row / a.seq), q = (int)(row % a.seq);
-        a.delta[((int64_t)b * a.heads + head) * a.seq + q] = s;
-    }
-}
-
-// =========================================================================================
 // backward dK, dV: block = 128 keys (4 waves x 32), loop over 64-query tiles
 // =========================================================================================
 template <bool DROP>
@@ -564,7 +539,22 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dq_kernel(const AttnArgs a) {
         }
     }
     const int64_t stat = ((int64_t)b * a.heads + head) * a.seq + min(myq, last);
-    const float my_lse = a.lse[stat], my_delta = a.delta[stat];
+    const float my_lse = a.lse[stat];
+    // delta[q] = rowsum(dO o O): the lane and its partner (lane ^ 32) hold the two halves of the query's dO row; the
+    // matching halves of O are fetched once.  Written out for the dK / dV kernel, which runs after this one.
+    float my_delta = 0.f;
+    {
+        const bf16* O = a.o + row_base * a.ld_o + head * 64;
+        const int64_t r = min(myq, last);
+#pragma unroll
+        for (int ks = 0; ks < 4; ++ks) {
+            const bf16x8 of = *(const bf16x8*)(O + r * a.ld_o + (lane >> 5) * 8 + ks * 16);
+#pragma unroll
+            for (int e = 0; e < 8; ++e) my_delta = fmaf((float)dof[ks][e], (float)of[e], my_delta);
+        }
+        my_delta += __shfl_xor(my_delta, 32, 64);
+        if (lane < 32 && myq < a.seq) a.delta[stat] = my_delta;
+    }
     f32x16 dq[2];
 #pragma unroll
     for (int t = 0; t < 2; ++t)
@@ -706,14 +696,14 @@ extern "C" int bb_attention_bwd(int dtype, int mask, int batch, int heads, int s
     a.scale = 1.0f / sqrtf((float)head_dim);
     a.scale_log2 = a.scale * 1.4426950408889634f;
     hipStream_t st = (hipStream_t)stream;
-    hipLaunchKernelGGL(attn_delta_kernel, dim3((unsigned)(((int64_t)batch * seq + 31) / 32), (unsigned)heads), dim3(256), 0, st, a);
+    // the dQ kernel first: it also leaves delta = rowsum(dO o O) of its queries for the dK / dV kernel
     dim3 grid(attn_grid(seq, batch * heads));
     if (a.drop.thresh) {
-        hipLaunchKernelGGL(attn_bwd_dkv_kernel<true>, grid, dim3(256), 0, st, a);
         hipLaunchKernelGGL(attn_bwd_dq_kernel<true>, grid, dim3(256), 0, st, a);
+        hipLaunchKernelGGL(attn_bwd_dkv_kernel<true>, grid, dim3(256), 0, st, a);
     } else {
-        hipLaunchKernelGGL(attn_bwd_dkv_kernel<false>, grid, dim3(256), 0, st, a);
         hipLaunchKernelGGL(attn_bwd_dq_kernel<false>, grid, dim3(256), 0, st, a);
+        hipLaunchKernelGGL(attn_bwd_dkv_kernel<false>, grid, dim3(256), 0, st, a);
     }
     BB_LAUNCH_CHECK();
     return BB_OK;
