@@ -200,7 +200,7 @@ static int fill_args(const bb_gemm_desc* d, GemmArgs& g, int64_t& batches, bool&
     BB_REQUIRE(d->layout >= BB_NT && d->layout <= BB_TN, "bb_gemm: bad layout %d", d->layout);
     BB_REQUIRE(d->M >= 0 && d->N >= 0 && d->K >= 0, "bb_gemm: negative dimension");
     BB_REQUIRE(!d->accumulate || d->c_dtype == BB_F32, "bb_gemm: accumulate needs an fp32 C");
-    BB_REQUIRE(d->epilogue >= BB_EPI_NONE && d->epilogue <= BB_EPI_ACT_DACT, "bb_gemm: bad epilogue");
+    BB_REQUIRE(d->epilogue >= BB_EPI_NONE && d->epilogue <= BB_EPI_MUL_POS, "bb_gemm: bad epilogue");
     const int nb1 = d->nb1 > 0 ? d->nb1 : 1, nb2 = d->nb2 > 0 ? d->nb2 : 1;
     batches = (int64_t)nb1 * nb2;
     ta = d->layout == BB_TN;
@@ -208,7 +208,8 @@ static int fill_args(const bb_gemm_desc* d, GemmArgs& g, int64_t& batches, bool&
     g.M = d->M; g.N = d->N; g.K = d->K; g.nb2 = nb2;
     if (d->M == 0 || d->N == 0) return BB_OK;
     BB_REQUIRE(d->A && d->B && d->C, "bb_gemm: null operand");
-    BB_REQUIRE((d->epilogue != BB_EPI_DACT && d->epilogue != BB_EPI_MUL) || d->aux_in, "bb_gemm: DACT/MUL epilogue needs aux_in");
+    BB_REQUIRE((d->epilogue != BB_EPI_DACT && d->epilogue != BB_EPI_MUL && d->epilogue != BB_EPI_MUL_POS && d->epilogue != BB_EPI_MUL_POS) || d->aux_in,
+               "bb_gemm: DACT / MUL / MUL_POS epilogue needs aux_in");
     BB_REQUIRE(d->epilogue != BB_EPI_RESIDUAL || d->resid, "bb_gemm: RESIDUAL epilogue needs resid");
     BB_REQUIRE(d->epilogue != BB_EPI_ACT_DACT || d->aux_out, "bb_gemm: ACT_DACT epilogue needs aux_out");
     BB_REQUIRE(batches <= 65535, "bb_gemm: too many batches (%lld)", (long long)batches);
@@ -246,9 +247,9 @@ static int fill_args(const bb_gemm_desc* d, GemmArgs& g, int64_t& batches, bool&
     g.epilogue = d->epilogue; g.act = d->act; g.accumulate = d->accumulate;
     g.c_f32 = (d->c_dtype == BB_F32);
     BB_REQUIRE(d->dropout_p >= 0.f && d->dropout_p < 1.f, "bb_gemm: dropout_p must be in [0, 1)");
-    BB_REQUIRE(d->dropout_p == 0.f || (batches == 1 && d->layout == BB_NT && d->epilogue != BB_EPI_DACT && d->epilogue != BB_EPI_MUL &&
+    BB_REQUIRE(d->dropout_p == 0.f || (batches == 1 && d->layout == BB_NT && d->epilogue != BB_EPI_DACT && d->epilogue != BB_EPI_MUL && d->epilogue != BB_EPI_MUL_POS &&
                                        !d->accumulate),
-               "bb_gemm: dropout goes with an unbatched, non-accumulating NT problem and not with the DACT / MUL epilogues");
+               "bb_gemm: dropout goes with an unbatched, non-accumulating NT problem and not with the DACT / MUL / MUL_POS epilogues");
     g.drop = bb_drop_key(d->dropout_p, d->dropout_k0, d->dropout_k1, (uint64_t)d->M * (uint64_t)d->N);
     g.tiles_m = g.tiles_n = 0;
     return BB_OK;

@@ -65,6 +65,8 @@ __device__ __forceinline__ void epilogue_elem(const GemmArgs& g, int64_t coff, i
         v = v * keep + Elem<T>::load((const T*)g.resid + xi);
     } else if (g.epilogue == BB_EPI_MUL) {
         v *= Elem<T>::load((const T*)g.aux_in + xi);
+    } else if (g.epilogue == BB_EPI_MUL_POS) {
+        v = Elem<T>::load((const T*)g.aux_in + xi) > 0.f ? v : 0.f;
     } else if (g.epilogue == BB_EPI_ACT_DACT) {
         float a, d;
         act_dact_f(v, g.act, a, d);
@@ -134,6 +136,11 @@ __device__ __forceinline__ void epilogue_vec8(const GemmArgs& g, int64_t coff, i
         load_vec((const bf16*)g.aux_in + xi, d);
 #pragma unroll
         for (int e = 0; e < 8; ++e) v[e] *= d[e];
+    } else if (g.epilogue == BB_EPI_MUL_POS) {
+        float d[8];
+        load_vec((const bf16*)g.aux_in + xi, d);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) v[e] = d[e] > 0.f ? v[e] : 0.f;
     } else if (g.epilogue == BB_EPI_ACT_DACT) {
         float d[8];
 #pragma unroll

@@ -13,7 +13,7 @@ import torch
 
 F32, BF16 = 0, 1
 NT, NN, TN = 0, 1, 2
-EPI_NONE, EPI_ACT, EPI_DACT, EPI_RESIDUAL, EPI_MUL, EPI_ACT_DACT = 0, 1, 2, 3, 4, 5
+EPI_NONE, EPI_ACT, EPI_DACT, EPI_RESIDUAL, EPI_MUL, EPI_ACT_DACT, EPI_MUL_POS = 0, 1, 2, 3, 4, 5, 6
 ACT_RELU, ACT_GELU_TANH = 0, 1
 MASK_NONE, MASK_CAUSAL, MASK_KEY_PADDING = 0, 1, 2
 LN_STANDARD, LN_ANNOTATED = 0, 1

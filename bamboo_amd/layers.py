@@ -176,10 +176,12 @@ class TransformerLayer:
         dt, f32 = ctx.dtype, torch.float32
         attn = ("lse", (ctx.batch, self.heads, ctx.seq), f32) if self.fused_attention(ctx) else \
             ("prob", (ctx.batch, self.heads, ctx.seq, ctx.seq), dt)
+        # ReLU's derivative is read off its kept output (relu'(u) = [relu(u) > 0]); other activations keep act'
+        dact = [] if self.activation == "relu" else [("dact", (R, f), dt)]
         return [
             ("n1", (R, h), dt), ("qkv", (R, 3 * h), dt), attn,
             ("ctx", (R, h), dt), ("x1", (R, h), dt), ("n2", (R, h), dt),
-            ("dact", (R, f), dt), ("act", (R, f), dt), ("out", (R, h), dt),
+            *dact, ("act", (R, f), dt), ("out", (R, h), dt),
             ("mean1", (R,), f32), ("rinv1", (R,), f32), ("mean2", (R,), f32), ("rinv2", (R,), f32),
         ]
 
@@ -300,8 +302,9 @@ class TransformerLayer:
         # evaluating act') both leave the GEMM epilogue: on the power-limited stage the saved pass over the
         # pre-activation (read 64 MB, write 64 MB at the GPT-2-medium shapes) outweighs the epilogue's
         # transcendental work (measured inside the stage, not on the kernel alone)
-        if ctx.defer:
-            # act' is read by the backward pass only: a forward that most likely has none writes act alone
+        if ctx.defer or self.activation == "relu":
+            # act' is read by the backward pass only: a forward that most likely has none writes act alone (and a
+            # ReLU layer never writes it: its backward pass reads the derivative off act)
             hip.gemm(hip.NT, st["n2"], w["feed_forward.w_1.weight"], st["act"], bias=w["feed_forward.w_1.bias"],
                      epilogue=hip.EPI_ACT, act=act, dropout=self._drop(ctx, self.SITE_FFN), stream=sm)
         else:
@@ -332,7 +335,7 @@ class TransformerLayer:
         # ... and each carries its bias gradient (column sums of dy) in the same kernel
         wgrad = lambda dy, x, name: wgrads.append(hip.gemm_desc(
             hip.TN, dy, x, g[name], accumulate=True, colsum_out=g[name[:-len("weight")] + "bias"], colsum_ws=ws))
-        if ctx.deferred:
+        if ctx.deferred and self.activation != "relu":
             self._ffn1(st, ctx)   # the forward of this stash left act' out: same kernel, same bits as a normal forward
         # the gradient behind a sublayer's dropout feeds the sublayer; the residual branch takes the one in front of it
         d_ff2, d_proj = d_out, None
@@ -341,7 +344,12 @@ class TransformerLayer:
             hip.dropout_apply(d_out, d_ff2, *self._drop(ctx, self.SITE_SUBLAYER1), stream=sm)
         # feed-forward
         wgrad(d_ff2, st["act"], "feed_forward.w_2.weight")
-        hip.gemm(hip.NN, d_ff2, w["feed_forward.w_2.weight"], d_ffn, epilogue=hip.EPI_MUL, aux_in=st["dact"], stream=sm)
+        if self.activation == "relu":
+            # act = relu(u) * keep / (1 - p): positive exactly where the gradient passes, and then with factor 1 / (1 - p)
+            hip.gemm(hip.NN, d_ff2, w["feed_forward.w_2.weight"], d_ffn, epilogue=hip.EPI_MUL_POS, aux_in=st["act"],
+                     alpha=1.0 / (1.0 - self.dropout) if self.dropout > 0 else 1.0, stream=sm)
+        else:
+            hip.gemm(hip.NN, d_ff2, w["feed_forward.w_2.weight"], d_ffn, epilogue=hip.EPI_MUL, aux_in=st["dact"], stream=sm)
         wgrad(d_ffn, st["n2"], "feed_forward.w_1.weight")
         hip.gemm(hip.NN, d_ffn, w["feed_forward.w_1.weight"], d_h0, stream=sm)
         # d_x1 = d_out + LN2'(d_n2)

@@ -331,6 +331,9 @@ def main():
     ap.add_argument("--dropout", type=float, default=0.0,
                     help="dropout probability of the transformer layers (the reference scripts run 0.1; the benchmark "
                          "line is quoted at 0, the configuration names none)")
+    ap.add_argument("--script-layers", action="store_true",
+                    help="the layer variant of the reference's transformer script (ReLU, annotated LayerNorm, no mask) "
+                         "at the configuration's sizes, instead of its GPT-2 / BERT variant")
     ap.add_argument("--no-paced", action="store_true",
                     help="skip the legs that run the stage inside the closed-loop model of a 4-stage 1F1B pipeline")
     ap.add_argument("--paced-timeline", default=None, metavar="FILE",
@@ -346,6 +349,13 @@ def main():
 
     from bamboo_amd import hip
     cfg = CONFIGS[args.config]
+    if args.script_layers:
+        if "variant" not in cfg:
+            print("bench.py: --script-layers goes with the transformer configurations", file=sys.stderr)
+            sys.exit(2)
+        cfg = dict(cfg, variant=dict(activation="relu", ln="annotated", mask="none"),
+                   label=cfg["label"] + " (script layers: relu, annotated LayerNorm, no mask)")
+        cfg.pop("key_len_range", None)
     if args.dropout > 0.0:
         # keys change every batch, so no HIP graphs, and the paced legs (which replay graphs) are left out
         if args.graphs or cfg.get("kind") == "resnet":

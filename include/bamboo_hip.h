@@ -54,6 +54,9 @@ extern "C" {
  *   BB_EPI_MUL       C = v * aux_in[m,n]  (e.g. aux_in = act'(u) kept by BB_EPI_ACT_DACT or bb_act_fwd)
  *   BB_EPI_ACT_DACT  aux_out = act'(v);  C = act(v)   (forward of an FFN whose backward then needs no
  *                    transcendental: its input gradient is a BB_EPI_MUL product with aux_out)
+ *   BB_EPI_MUL_POS   C = v where aux_in[m,n] > 0, else 0  (input gradient through a ReLU whose OUTPUT was kept:
+ *                    relu'(u) = [relu(u) > 0], so the forward stores nothing beside its output; a dropout
+ *                    factor 1/(1-p) on that output goes into alpha)
  * `accumulate` != 0 adds the result to the existing contents of C (C must be fp32).       */
 #define BB_EPI_NONE 0
 #define BB_EPI_ACT 1
@@ -61,6 +64,7 @@ extern "C" {
 #define BB_EPI_RESIDUAL 3
 #define BB_EPI_MUL 4
 #define BB_EPI_ACT_DACT 5
+#define BB_EPI_MUL_POS 6
 
 #define BB_ACT_RELU 0
 #define BB_ACT_GELU_TANH 1
@@ -120,7 +124,7 @@ typedef struct bb_gemm_desc {
      * (nn.Dropout of SublayerConnection and PositionwiseFeedForward, transformer.py:98-103,154-158):
      * element (m, n) is kept and scaled by 1 / (1 - dropout_p) when bb_dropout_keep(key, m * N + n) says so
      * (the decision function of bb_dropout_apply), else zero; with BB_EPI_ACT_DACT the stored derivative gets
-     * the same factor.  dropout_p = 0: none.  Not with BB_EPI_DACT / BB_EPI_MUL, not batched.            */
+     * the same factor.  dropout_p = 0: none.  Not with BB_EPI_DACT / BB_EPI_MUL / BB_EPI_MUL_POS, not batched.            */
     float dropout_p;
     uint32_t dropout_k0, dropout_k1;
 } bb_gemm_desc;

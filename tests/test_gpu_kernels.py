@@ -99,6 +99,16 @@ def test_gemm_epilogues(hiplib, dtype):
     # mul: C = (A W^T) * R
     hiplib.gemm(hiplib.NT, A, W, C, epilogue=hiplib.EPI_MUL, aux_in=R)
     assert rel_err(C, (Af @ Wf.t()) * Rf) < tol(dtype)
+    # mul_pos: C = alpha (A W^T) where R > 0, else 0 -- the gradient through a ReLU whose output R was kept; exactly
+    # the alpha-product where it passes, exactly zero elsewhere, and equal to MUL with the 0 / 1 mask
+    Rz = torch.where(R.abs() < 0.3, torch.zeros_like(R), R)     # zeros of its own, like a ReLU output
+    hiplib.gemm(hiplib.NT, A, W, C, epilogue=hiplib.EPI_MUL_POS, aux_in=Rz, alpha=1.25)
+    pos = (Rz > 0)
+    assert rel_err(C, 1.25 * (Af @ Wf.t()) * pos.double().cpu()) < tol(dtype)
+    assert not C[~pos].any()
+    Cm = torch.empty_like(C)
+    hiplib.gemm(hiplib.NT, A, W, Cm, epilogue=hiplib.EPI_MUL, aux_in=pos.to(dtype), alpha=1.25)
+    assert torch.equal(C, Cm)
     # fp32 accumulate (weight-gradient form): G += A^T B
     G0 = randn(K, N, dtype=torch.float32, seed=7)
     G = G0.clone()
