@@ -708,9 +708,10 @@ __device__ __forceinline__ void gemm_bf16_dma_body(const GemmArgs& g, const int 
     // reads ride on the first FM MFMAs so that the last ones cover their latency), each group fenced:
     // the DMA instructions are inline assembly, opaque to the scheduler's group hints, and unfenced
     // they end up bunched behind the barrier.
+    // (KOFF: the step issues DMA instructions KOFF .. KOFF + ND - 1 of the k-tile)
     auto placed_step = [&](const Frags& f, auto ks_c, auto nd_c, unsigned char* dst, auto reads_c, Frags& nf,
-                           const unsigned char* src, int h) {
-        constexpr int ks = decltype(ks_c)::value, ND = decltype(nd_c)::value;
+                           const unsigned char* src, int h, auto koff_c) {
+        constexpr int ks = decltype(ks_c)::value, ND = decltype(nd_c)::value, KOFF = decltype(koff_c)::value;
         constexpr bool READS = decltype(reads_c)::value;
         constexpr int NM = TM * TN, NF = 2 * (TM + TN), FM = NM > 2 ? NM - 2 : NM;
         static_for(
@@ -727,7 +728,7 @@ __device__ __forceinline__ void gemm_bf16_dma_body(const GemmArgs& g, const int 
                 }
                 static_for(
                     [&](auto d) {
-                        constexpr int k = (ND * m) / NM + decltype(d)::value;
+                        constexpr int k = KOFF + (ND * m) / NM + decltype(d)::value;
                         if constexpr (k < OpA::ROUNDS) opa.template issue_one<k>(dst, wave);
                         else opb.template issue_one<k - OpA::ROUNDS>(dst + OpA::BYTES, wave);
                     },
@@ -795,14 +796,26 @@ __device__ __forceinline__ void gemm_bf16_dma_body(const GemmArgs& g, const int 
             rs = rs + 1 == STAGES ? 0 : rs + 1;
             const unsigned char* nxt = smem + rs * STAGE_BYTES;
             if constexpr (STAGES >= 3) {
+                // the DMA instructions of tile kt+STAGES-1 a third each between the MFMAs of the first three quarters
+                // (issued in one burst at the top they queue up in front of the texture path and the waves behind
+                // them: 2-5 % slower), the second half's fragment reads between the first MFMAs
                 stop_at_end(kt + STAGES);
-                issue_tile();
+                unsigned char* into = smem + issue_stage * STAGE_BYTES;
+                issue_stage = issue_stage + 1 == STAGES ? 0 : issue_stage + 1;
+                constexpr int THIRD = LOADS / 3;
+                placed_step(f0, std::integral_constant<int, 0>{}, std::integral_constant<int, THIRD>{}, into, std::true_type{}, f1,
+                            cur, 1, std::integral_constant<int, 0>{});
+                placed_step(f0, std::integral_constant<int, 1>{}, std::integral_constant<int, THIRD>{}, into, std::false_type{}, f1,
+                            cur, 1, std::integral_constant<int, THIRD>{});
+                placed_step(f1, std::integral_constant<int, 0>{}, std::integral_constant<int, LOADS - 2 * THIRD>{}, into,
+                            std::false_type{}, f1, cur, 1, std::integral_constant<int, 2 * THIRD>{});
+            } else {
+                load_half(f1, cur, 1);
+                mfma_step(f0, 0);
+                mfma_step(f0, 1);
+                interleave_mfma_with<2 * TM * TN, FRAG_READS, 0x100>();
+                mfma_step(f1, 0);
             }
-            load_half(f1, cur, 1);
-            mfma_step(f0, 0);
-            mfma_step(f0, 1);
-            interleave_mfma_with<2 * TM * TN, FRAG_READS, 0x100>();
-            mfma_step(f1, 0);
             // scheduling fences: without them the compiler sinks this third quarter below the barrier
             // and bunches the next tile's fragment reads at the end of the iteration, right in front
             // of the wait for them
@@ -819,7 +832,7 @@ __device__ __forceinline__ void gemm_bf16_dma_body(const GemmArgs& g, const int 
                 issue_stage = issue_stage + 1 == STAGES ? 0 : issue_stage + 1;
             }
             placed_step(f1, std::integral_constant<int, 1>{}, std::integral_constant<int, STAGES == 2 ? LOADS : 0>{}, dst,
-                        std::true_type{}, f0, nxt, 0);
+                        std::true_type{}, f0, nxt, 0, std::integral_constant<int, 0>{});
             __builtin_amdgcn_sched_barrier(0);
         }
     } else {
@@ -845,12 +858,12 @@ __device__ __forceinline__ void gemm_bf16_dma_body(const GemmArgs& g, const int 
             unsigned char* dst = smem + issue_stage * STAGE_BYTES;
             issue_stage = issue_stage + 1 == STAGES ? 0 : issue_stage + 1;
             placed_step(cur, std::integral_constant<int, 0>{}, std::integral_constant<int, LOADS>{}, dst, std::false_type{},
-                        nxt, smem, 0);
+                        nxt, smem, 0, std::integral_constant<int, 0>{});
             sync_tile();
             const unsigned char* st = smem + read_stage * STAGE_BYTES;
             read_stage = read_stage + 1 == STAGES ? 0 : read_stage + 1;
             placed_step(cur, std::integral_constant<int, 1>{}, std::integral_constant<int, 0>{}, dst, std::true_type{}, nxt,
-                        st, 0);
+                        st, 0, std::integral_constant<int, 0>{});
           } else {
             constexpr int FRAG_READS = 2 * (TM * (AKM ? 2 : 1) + TN * (BKM ? 2 : 1));
             stop_at_end(kt + STAGES);
