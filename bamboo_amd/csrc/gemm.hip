@@ -57,6 +57,23 @@ static int launch_bf16_dma(GemmArgs& g, int batches, hipStream_t st) {
     return BB_OK;
 }
 
+// persistent kernels: one block per CU walks the tiles
+static constexpr int kPersistBlocks = 256;
+template <int BM, int BN, int WM, int WN, bool TB> static int launch_bf16_dma_persist(GemmArgs& g, hipStream_t st) {
+    constexpr int smem = 3 * (BM + BN) * 32 * 2 + WM * WN * 32 * 64 * 4;
+    auto kern = gemm_bf16_dma_persist_kernel<BM, BN, WM, WN, TB, false>;
+    if constexpr (!TB) {
+        if (g.drop.thresh) kern = gemm_bf16_dma_persist_kernel<BM, BN, WM, WN, TB, true>;
+    }
+    BB_HIP_CHECK(bb_allow_dynamic_lds((const void*)kern, smem));
+    g.tiles_m = (g.M + BM - 1) / BM;
+    g.tiles_n = (g.N + BN - 1) / BN;
+    const int total = g.tiles_m * g.tiles_n;
+    hipLaunchKernelGGL(kern, dim3(total < kPersistBlocks ? (total + 7) / 8 * 8 : kPersistBlocks), dim3(WM * WN * 64), smem, st, g);
+    BB_LAUNCH_CHECK();
+    return BB_OK;
+}
+
 template <int BM, int BN, int WM, int WN>
 static int launch_bf16_dma_stats(GemmArgs& g, hipStream_t st) {
     constexpr int smem = 3 * (BM + BN) * 64 * 2;
@@ -71,12 +88,13 @@ static int launch_bf16_dma_stats(GemmArgs& g, hipStream_t st) {
 
 // DMA kernels need K % 32 == 0 and at least one full vector of rows; tile by problem size
 enum DmaTile { D_NONE = 0, D256x256w8db, D256x128w8db, D128x128s3, D256x256k64, D256x128k64s3, D128x128k64, D128x64k64s3, D128x64s3,
-               D64x128k64s3, D64x128s3, D256x192k64 };
+               D64x128k64s3, D64x128s3, D256x192k64, D256x256p };
 static const char* const kDmaTileNames[] = {"", "dma256x256w8db", "dma256x128w8db", "dma128x128s3", "dma256x256k64", "dma256x128k64s3",
                                             "dma128x128k64", "dma128x64k64s3", "dma128x64s3", "dma64x128k64s3", "dma64x128s3",
-                                            "dma256x192k64"};
-// The tile of a problem depends on its shape and layout only (never on the stream, the environment or what ran
-// before): a redundant forward and a normal forward of the same layer run the same kernel and give the same bits.
+                                            "dma256x192k64", "dma256x256p"};
+// The tile of a problem depends on its shape, layout and epilogue kind only (never on the stream, the environment or
+// what ran before), and every kernel adds up a contraction in the same order: a redundant forward and a normal forward
+// of the same layer give the same bits.
 static DmaTile pick_dma_tile(int M, int N, int K, int64_t batches, int layout) {
     if (K % 32 != 0 || K < 64 || M < 128 || N < 128 || N % 8 != 0) return D_NONE;
     // Rules read off sweeps of M 2048..16384 x N 768..6400 x K 1024/4096 (NT and NN) on MI355X (256 CUs,
@@ -143,8 +161,22 @@ static DmaTile pick_dma_tile(int M, int N, int K, int64_t batches, int layout) {
     return small;
 }
 
+// The tile of a (shape, layout, epilogue kind): NT / NN problems of more than one round of 256x256 tiles take the
+// persistent kernel (blocks walk their tiles with the DMA ring running through the tile boundaries) unless the epilogue
+// evaluates the activation: that work keeps the vector ALUs busy for about as long as the tile's matrix work does, the
+// boundary is not what such a launch waits for (FFN1 with act + act': 114 us on the plain kernel, 118 persistent;
+// the plain product 95 against 77).  All kernels add up a contraction in the same order: which one runs changes no bit.
+static DmaTile pick_dma_tile_for(int M, int N, int K, int64_t batches, int layout, int epilogue) {
+    const DmaTile t = pick_dma_tile(M, N, K, batches, layout);
+    const bool light = epilogue != BB_EPI_ACT && epilogue != BB_EPI_ACT_DACT && epilogue != BB_EPI_DACT;
+    const int64_t t256 = (int64_t)((M + 255) / 256) * ((N + 255) / 256);
+    if ((t == D256x256k64 || t == D256x256w8db) && light && batches == 1 && layout != BB_TN && K % 64 == 0 && t256 > kPersistBlocks)
+        return D256x256p;
+    return t;
+}
+
 template <bool TA, bool TB> static int dispatch_bf16(GemmArgs& g, int batches, hipStream_t st) {
-    switch (pick_dma_tile(g.M, g.N, g.K, batches, TA ? BB_TN : TB ? BB_NN : BB_NT)) {
+    switch (pick_dma_tile_for(g.M, g.N, g.K, batches, TA ? BB_TN : TB ? BB_NN : BB_NT, g.epilogue)) {
         case D256x256w8db: return launch_bf16_dma<256, 256, 2, 4, TA, TB, true>(g, batches, st);
         case D256x128w8db: return launch_bf16_dma<256, 128, 4, 2, TA, TB, true>(g, batches, st);
         case D128x128s3: return launch_bf16_dma<128, 128, 2, 2, TA, TB, true, 3>(g, batches, st);
@@ -155,6 +187,9 @@ template <bool TA, bool TB> static int dispatch_bf16(GemmArgs& g, int batches, h
         case D128x64s3: return launch_bf16_dma<128, 64, 4, 1, TA, TB, true, 3>(g, batches, st);
         case D64x128k64s3: return launch_bf16_dma<64, 128, 2, 2, TA, TB, true, 3, 64>(g, batches, st);
         case D64x128s3: return launch_bf16_dma<64, 128, 2, 2, TA, TB, true, 3>(g, batches, st);
+        case D256x256p:
+            if constexpr (!TA) return launch_bf16_dma_persist<256, 256, 2, 4, TB>(g, st);
+            else break;
         case D256x192k64:
             // k-contiguous operands only (192 rows do not divide into the k-major loader's instructions)
             if constexpr (!TA && !TB) return launch_bf16_dma<256, 192, 4, 2, TA, TB, true, 2, 64>(g, batches, st);
@@ -184,7 +219,7 @@ extern "C" int bb_gemm_variant(const bb_gemm_desc* d, char* out, int out_len) {
     BB_REQUIRE(d->layout >= BB_NT && d->layout <= BB_TN, "bb_gemm_variant: bad layout %d", d->layout);
     const int64_t batches = (int64_t)(d->nb1 > 0 ? d->nb1 : 1) * (d->nb2 > 0 ? d->nb2 : 1);
     if (d->dtype == BB_BF16) {
-        const DmaTile dt = pick_dma_tile(d->M, d->N, d->K, batches, d->layout);
+        const DmaTile dt = pick_dma_tile_for(d->M, d->N, d->K, batches, d->layout, d->epilogue);
         snprintf(out, out_len, "bf16_%s_%s", layouts[d->layout],
                  dt != D_NONE ? kDmaTileNames[dt] : kBf16TileNames[pick_bf16_tile(d->M, d->N, batches)]);
     }

@@ -984,6 +984,205 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_bf16_dma_stats_kernel(const 
     gemm_bf16_dma_body<BM, BN, WM, WN, false, false, true, 3, 64, false, 0, true>(g, blockIdx.x, blockIdx.z);
 }
 
+// Persistent variant for problems of more than one round of 256x256 tiles (NT and NN, 32-wide k-tiles, three stages,
+// eight waves): a block walks the output tiles b, b + gridDim, ... and treats their k-tiles as ONE stream, so the DMA
+// ring never drains - while the last k-tiles of a tile are multiplied, the first ones of the block's next tile are
+// already landing, and the epilogue's stores go out behind them.  What a tile boundary costs a block of the plain
+// kernel (retiring, the next block's launch, its pipeline prologue) is gone: 95 -> 77 us on the plain product
+// 8192 x 4096 x 1024.  The waits of the first k-tiles after a boundary count the epilogue's stores in (completion is in
+// order): exact counts that spare them changed nothing, the stores are acknowledged quickly.  The epilogue patch
+// cannot share the ring's LDS any more (the ring is live during the epilogue): it has 64 KB of its own behind the
+// three stages, [32][64] floats per wave with the 16-byte chunks of a row swizzled by the row instead of padded.
+// Results are bit-equal to the plain kernels' (same k order, same epilogue function).  Needs K % 64 == 0 (the two
+// fragment sets alternate, a tile takes an even number of k-tiles), unbatched operands, a grid that is a multiple of 8
+// (the tile order's XCD mapping).  Instantiated for 256x256 tiles only: 256x128 tiles on this loop load their 32-wide
+// k-tiles as half lines and lose more than the boundaries give (90 against 71 us on 8192 x 3072 x 1024).
+template <int BM, int BN, int WM, int WN, bool BKM, bool DROP>
+__global__ __launch_bounds__(WM* WN * 64) void gemm_bf16_dma_persist_kernel(const GemmArgs g) {
+    constexpr int NW = WM * WN, BK = 32, STAGES = 3;
+    constexpr int WTM = BM / WM, WTN = BN / WN, TM = WTM / 32, TN = WTN / 32;
+    static_assert(TN == 2 && TM * TN > 2, "the epilogue patch holds two accumulator tiles side by side");
+    using OpA = DmaOperand<BM, false, NW, BK>;
+    using OpB = DmaOperand<BN, BKM, NW, BK>;
+    constexpr int STAGE_BYTES = OpA::BYTES + OpB::BYTES;
+    constexpr int LOADS = OpA::ROUNDS + OpB::ROUNDS;
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wm = wave / WN, wn = wave % WN;
+    const int total = g.tiles_m * g.tiles_n, G = gridDim.x;
+    const bf16* A = (const bf16*)g.A;
+    const bf16* B = (const bf16*)g.B;
+    const int KT = g.K / BK;
+
+    OpA opa;
+    OpB opb;
+    FragReader<BM, TM, false, BK> fa;
+    FragReader<BN, TN, BKM, BK> fb;
+    fa.init(wm * WTM, lane);
+    fb.init(wn * WTN, lane);
+    struct Frags {
+        bf16x8 a[2][TM], b[2][TN];
+    };
+    Frags f0, f1;
+    f32x16 acc[TM][TN];
+
+    // the stream: ki = index of the next k-tile to issue inside output tile issue_tile
+    int issue_stage = 0, read_stage = 0, ki = 0, issue_tile = blockIdx.x;
+    auto point_at = [&](int t) {
+        int tm, tn;
+        tile_coords(t, g.tiles_m, g.tiles_n, tm, tn);
+        opa.init(A, g.lda, tm * BM, g.M, tid);
+        opb.init(B, g.ldb, tn * BN, g.N, tid);
+    };
+    point_at(issue_tile);
+    // before a k-tile is issued: move on to the block's next output tile, or (no tile left) stay on the last k-tile,
+    // which is then fetched again and again into stages nobody reads
+    auto prep_issue = [&]() {
+        if (ki == KT) {
+            if (issue_tile + G < total) {
+                issue_tile += G;
+                ki = 0;
+                point_at(issue_tile);
+            } else {
+                ki = KT - 1;
+            }
+        }
+        if (ki == KT - 1 && issue_tile + G >= total) {
+            opa.stop();
+            opb.stop();
+        }
+    };
+    // MFMA m of step ks, then its share of ND DMA instructions into `dst` and of the fragment reads of `src` into
+    // nf, each group fenced (see gemm_bf16_dma_body)
+    auto placed_step = [&](const Frags& f, auto ks_c, auto nd_c, unsigned char* dst, auto reads_c, Frags& nf,
+                           const unsigned char* src) {
+        constexpr int ks = decltype(ks_c)::value, ND = decltype(nd_c)::value;
+        constexpr bool READS = decltype(reads_c)::value;
+        constexpr int NM = TM * TN, NF = 2 * (TM + TN), FM = NM - 2;
+        static_for(
+            [&](auto idx) {
+                constexpr int m = decltype(idx)::value, i = m / TN, j = m % TN;
+                acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(f.a[ks][i], f.b[ks][j], acc[i][j], 0, 0, 0);
+                static_for(
+                    [&](auto d) {
+                        constexpr int k = (ND * m) / NM + decltype(d)::value;
+                        if constexpr (k < OpA::ROUNDS) opa.template issue_one<k>(dst, wave);
+                        else opb.template issue_one<k - OpA::ROUNDS>(dst + OpA::BYTES, wave);
+                    },
+                    std::make_integer_sequence<int, (ND * (m + 1)) / NM - (ND * m) / NM>{});
+                if constexpr (READS && m < FM) {
+                    static_for(
+                        [&](auto r) {
+                            constexpr int q = (NF * m) / FM + decltype(r)::value, fk = q / (TM + TN), t = q % (TM + TN);
+                            if constexpr (t < TM) nf.a[fk][t] = fa.load(src, t, fk);
+                            else nf.b[fk][t - TM] = fb.load(src + OpA::BYTES, t - TM, fk);
+                        },
+                        std::make_integer_sequence<int, (NF * (m + 1)) / FM - (NF * m) / FM>{});
+                }
+                __builtin_amdgcn_sched_barrier(0);
+            },
+            std::make_integer_sequence<int, NM>{});
+    };
+    // one k-tile: first half with the DMA instructions of the stream's k-tile two ahead, the wait for the k-tile
+    // one ahead (in-order completion: whatever the epilogue stored before is acknowledged by then too), second half
+    // with that k-tile's fragment reads
+    auto body = [&](Frags& cur, Frags& nxt, auto reads_c) {
+        prep_issue();
+        unsigned char* dst = smem + issue_stage * STAGE_BYTES;
+        issue_stage = issue_stage + 1 == STAGES ? 0 : issue_stage + 1;
+        placed_step(cur, std::integral_constant<int, 0>{}, std::integral_constant<int, LOADS>{}, dst, std::false_type{}, nxt, smem);
+        ++ki;
+        asm volatile("" ::: "memory");
+        wait_vmcnt_lgkm0<(STAGES - 2) * LOADS>();
+        __builtin_amdgcn_s_barrier();
+        asm volatile("" ::: "memory");
+        const unsigned char* st = smem + read_stage * STAGE_BYTES;
+        read_stage = read_stage + 1 == STAGES ? 0 : read_stage + 1;
+        placed_step(cur, std::integral_constant<int, 1>{}, std::integral_constant<int, 0>{}, dst, reads_c, nxt, st);
+    };
+    auto load_frags = [&](Frags& f, const unsigned char* st) {
+#pragma unroll
+        for (int ks = 0; ks < 2; ++ks) {
+#pragma unroll
+            for (int i = 0; i < TM; ++i) f.a[ks][i] = fa.load(st, i, ks);
+#pragma unroll
+            for (int j = 0; j < TN; ++j) f.b[ks][j] = fb.load(st + OpA::BYTES, j, ks);
+        }
+    };
+
+    // prologue of the stream
+#pragma unroll
+    for (int t = 0; t < STAGES - 1; ++t) {
+        prep_issue();
+        unsigned char* st = smem + issue_stage * STAGE_BYTES;
+        opa.issue(st, wave);
+        opb.issue(st + OpA::BYTES, wave);
+        issue_stage = issue_stage + 1 == STAGES ? 0 : issue_stage + 1;
+        ++ki;
+    }
+    asm volatile("" ::: "memory");
+    wait_vmcnt_lgkm0<(STAGES - 2) * LOADS>();
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+
+    float* patch = (float*)(smem + STAGES * STAGE_BYTES) + wave * (32 * 64);
+    const int prow = lane >> 3, pchunk = lane & 7;
+    // the two 16-byte chunks of a lane's eight columns, read in an order that keeps the eight lanes of a row on
+    // eight different bank groups: lanes 0..3 of the row take their even chunk first, lanes 4..7 their odd one
+    const int first_chunk = 2 * pchunk + (pchunk >> 2), second_chunk = 2 * pchunk + 1 - (pchunk >> 2);
+    for (int tile = blockIdx.x; tile < total; tile += G) {
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+            for (int j = 0; j < TN; ++j)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+        // the tile's first fragments (the k-tile landed and was made visible by the last barrier before this point);
+        // a tile's last k-tile does not fetch the next tile's, so that no fragment registers live through the epilogue
+        load_frags(f0, smem + read_stage * STAGE_BYTES);
+        read_stage = read_stage + 1 == STAGES ? 0 : read_stage + 1;
+        for (int kt = 0; kt + 2 < KT; kt += 2) {
+            body(f0, f1, std::true_type{});
+            body(f1, f0, std::true_type{});
+        }
+        body(f0, f1, std::true_type{});
+        body(f1, f0, std::false_type{});
+        read_stage = read_stage == 0 ? STAGES - 1 : read_stage - 1;   // that k-tile is still to be read
+        int tm, tn;
+        tile_coords(tile, g.tiles_m, g.tiles_n, tm, tn);
+        const int m0 = tm * BM + wm * WTM, n = tn * BN + wn * WTN + pchunk * 8;
+        // (static_for: a loop the compiler declines to unroll would index the accumulators dynamically, i.e. from scratch)
+        static_for(
+            [&](auto idx) {
+                constexpr int i = decltype(idx)::value;
+#pragma unroll
+                for (int h = 0; h < 2; ++h)
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) {
+                        const int row = 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3), col = h * 32 + (lane & 31);
+                        patch[row * 64 + ((((col >> 2) ^ (row & 15)) << 2) | (col & 3))] = acc[i][h][r] * g.alpha;
+                    }
+                asm volatile("" ::: "memory");
+                static_for(
+                    [&](auto it_c) {
+                    constexpr int it = decltype(it_c)::value;
+                    const int row = it * 8 + prow, m = m0 + i * 32 + row;
+                    const f32x4 c1 = *(const f32x4*)(patch + row * 64 + ((first_chunk ^ (row & 15)) << 2));
+                    const f32x4 c2 = *(const f32x4*)(patch + row * 64 + ((second_chunk ^ (row & 15)) << 2));
+                    const f32x4 lo = pchunk < 4 ? c1 : c2, hi = pchunk < 4 ? c2 : c1;
+                    float v[8] = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+                    if (m < g.M && n < g.N) {
+                        epilogue_vec8<DROP>(g, 0, m, n, v);
+                    }
+                    },
+                    std::make_integer_sequence<int, 4>{});
+                asm volatile("" ::: "memory");
+            },
+            std::make_integer_sequence<int, TM>{});
+    }
+    wait_vmcnt_lgkm0<0>();   // the k-tiles issued past the end of the stream land before the block leaves
+}
+
 // 3x3 convolution as an implicit GEMM: forward (BKM = false: y = patches(x) W^T) and input gradient
 // (BKM = true: dx = patches(dy) W_flipped) on the same main loop, operands gathered by the loaders.
 template <int BM, int BN, int WM, int WN, bool BKM, int STAGES, bool STATS = false>

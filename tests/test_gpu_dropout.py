@@ -39,8 +39,9 @@ def test_dropout_kernel_makes_the_oracle_decisions(hiplib, dtype):
     assert torch.equal(z, y)
 
 
-@pytest.mark.parametrize("dtype,M,N,K", [(torch.bfloat16, 512, 384, 256), (torch.bfloat16, 200, 72, 96), (torch.float32, 130, 68, 40)],
-                         ids=["bf16-dma", "bf16-fallback", "fp32"])
+@pytest.mark.parametrize("dtype,M,N,K", [(torch.bfloat16, 512, 384, 256), (torch.bfloat16, 200, 72, 96), (torch.float32, 130, 68, 40),
+                                         (torch.bfloat16, 7168, 4096, 576)],
+                         ids=["bf16-dma", "bf16-fallback", "fp32", "bf16-persistent"])
 @pytest.mark.parametrize("epi", ["none", "act", "act_dact", "residual"])
 def test_gemm_epilogue_dropout(hiplib, dtype, M, N, K, epi):
     p = 0.25

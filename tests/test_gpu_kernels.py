@@ -120,6 +120,58 @@ def test_gemm_epilogues(hiplib, dtype):
     assert rel_err(C, 0.125 * (Af @ Wf.t())) < tol(dtype)
 
 
+@pytest.mark.parametrize("layout", ["nt", "nn"])
+@pytest.mark.parametrize("M,N,K", [(7168, 4096, 576), (7100, 4104, 640), (8192, 4096, 1024)])
+def test_gemm_persistent_blocks(hiplib, layout, M, N, K):
+    """More than one round of 256x256 tiles: the blocks of the persistent kernel walk several tiles each with the
+    k-tile stream running through the tile boundaries.  Every epilogue kind against fp64 (ragged edges included), and
+    bit for bit against the same product cut into row slabs small enough for the one-tile-per-block kernels: the
+    order of the contraction is the same in all of them."""
+    dtype = torch.bfloat16
+    lay = hiplib.NT if layout == "nt" else hiplib.NN
+    A = randn(M, K, dtype=dtype, seed=11)
+    W = randn(N, K, dtype=dtype, seed=12, scale=0.1) if layout == "nt" else randn(K, N, dtype=dtype, seed=12, scale=0.1)
+    bias, X = randn(N, dtype=dtype, seed=13), randn(M, N, dtype=dtype, seed=14)
+    C, D = torch.empty(M, N, dtype=dtype, device=DEV), torch.empty(M, N, dtype=dtype, device=DEV)
+    assert hiplib.gemm_variant(hiplib.gemm_desc(lay, A, W, C)).endswith("dma256x256p")
+    Af, Wf = A.double().cpu(), (W.double().cpu().t() if layout == "nt" else W.double().cpu())
+    lin = Af @ Wf
+    cases = {
+        "plain": (dict(), lambda: lin),
+        "bias": (dict(bias=bias), lambda: lin + bias.double().cpu()),
+        "residual": (dict(bias=bias, epilogue=hiplib.EPI_RESIDUAL, resid=X), lambda: lin + bias.double().cpu() + X.double().cpu()),
+        "mul": (dict(epilogue=hiplib.EPI_MUL, aux_in=X), lambda: lin * X.double().cpu()),
+        "act_dact": (dict(bias=bias, epilogue=hiplib.EPI_ACT_DACT, act=hiplib.ACT_GELU_TANH, aux_out=D),
+                     lambda: ol.activation(lin + bias.double().cpu(), "gelu_tanh")),
+    }
+    slab = 1024
+    for name, (kw, ref) in cases.items():
+        C.fill_(float("nan"))
+        hiplib.gemm(lay, A, W, C, **kw)
+        assert rel_err(C, ref()) < tol(dtype), name
+        if name == "act_dact":
+            u = (lin + bias.double().cpu()).requires_grad_(True)
+            ol.activation(u, "gelu_tanh").sum().backward()
+            assert rel_err(D, u.grad) < tol(dtype)
+        # row slabs: at most 4 x 17 tiles, far below a round, so another kernel runs them
+        Cs, Ds = torch.empty_like(C), torch.empty_like(D)
+        for r0 in range(0, M, slab):
+            r1 = min(M, r0 + slab)
+            kws = {k: (v[r0:r1] if k in ("resid", "aux_in") else v) for k, v in kw.items()}
+            if "aux_out" in kws:
+                kws["aux_out"] = Ds[r0:r1]
+            assert not hiplib.gemm_variant(hiplib.gemm_desc(lay, A[r0:r1], W, Cs[r0:r1])).endswith("p")
+            hiplib.gemm(lay, A[r0:r1], W, Cs[r0:r1], **kws)
+        assert torch.equal(C, Cs), name
+        if name == "act_dact":
+            assert torch.equal(D, Ds)
+    # fp32 output, accumulated into
+    G0 = randn(M, N, dtype=torch.float32, seed=15)
+    G = G0.clone()
+    hiplib.gemm(lay, A, W, G, accumulate=True)
+    assert rel_err(G, G0.double().cpu() + lin) < tol(dtype)
+
+
 @pytest.mark.parametrize("layout", ["tn", "nt"])
 def test_gemm_grouped_splitk(hiplib, layout):
     """Few output tiles, long contraction: chunks of the contraction into fp32 partials, added to C
