@@ -119,19 +119,29 @@ __device__ __forceinline__ float wave_max(float v) {
 }
 
 // ---- activations ------------------------------------------------------------------------
-// tanh-GELU: 0.5 x (1 + tanh z) = x * sigmoid(2z), z = k0 (x + k1 x^3); one v_exp_f32 and one
-// v_rcp_f32 per element (both accurate to 1 ulp), so the epilogue stays far below the MFMA time.
-__device__ __forceinline__ float sigmoid2z_f(float x) {
-    const float k0 = 0.7978845608028654f, k1 = 0.044715f;
-    const float z2 = 2.0f * k0 * (x + k1 * x * x * x);
-    return __frcp_rn(1.0f + __expf(-z2));
+// tanh-GELU: 0.5 x (1 + tanh z) = x * sigmoid(2z), z = k0 (x + k1 x^3).  sigmoid(2z) = 1 / (1 + 2^(x (c0 + c1 x^2))) with
+// c0 = -2 k0 log2(e), c1 = c0 k1: three multiply-adds, one v_exp_f32 and one v_rcp_f32 per element (both instructions
+// accurate to 1 ulp).  Bare instructions on purpose: a correctly rounded 1 / x expands into a ten-instruction division
+// sequence per element, which in a GEMM epilogue that evaluates GELU and its derivative for 128 elements per lane and
+// tile is a third of the epilogue's vector work (the matrix cores idle meanwhile).
+// GELU'(x) = s + x s (1 - s) dz, dz = d(2z)/dx = 2 k0 (1 + 3 k1 x^2) = d0 + d1 x^2.
+#define BB_GELU_C0 (-2.3022081983f)    /* -2 * 0.7978845608 * 1.4426950409 */
+#define BB_GELU_C1 (-0.10294323957f)   /* c0 * 0.044715 */
+#define BB_GELU_D0 (1.5957691216f)     /* 2 * 0.7978845608 */
+#define BB_GELU_D1 (0.21406444882f)    /* 6 * 0.7978845608 * 0.044715 */
+__device__ __forceinline__ float sigmoid2z_f(float x, float x2) {
+    return __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(x * fmaf(BB_GELU_C1, x2, BB_GELU_C0)));
 }
-__device__ __forceinline__ float gelu_tanh_f(float x) { return x * sigmoid2z_f(x); }
+__device__ __forceinline__ float gelu_tanh_f(float x) { return x * sigmoid2z_f(x, x * x); }
+__device__ __forceinline__ void gelu_dgelu_f(float x, float& a, float& d) {
+    const float x2 = x * x, s = sigmoid2z_f(x, x2);
+    a = x * s;
+    d = fmaf(a * (1.0f - s), fmaf(BB_GELU_D1, x2, BB_GELU_D0), s);
+}
 __device__ __forceinline__ float dgelu_tanh_f(float x) {
-    const float k0 = 0.7978845608028654f, k1 = 0.044715f;
-    const float s = sigmoid2z_f(x);
-    const float dz2 = 2.0f * k0 * (1.0f + 3.0f * k1 * x * x);
-    return s + x * s * (1.0f - s) * dz2;
+    float a, d;
+    gelu_dgelu_f(x, a, d);
+    return d;
 }
 // act(x) and act'(x) together (one sigmoid for both)
 __device__ __forceinline__ void act_dact_f(float x, int kind, float& a, float& d) {
@@ -139,11 +149,7 @@ __device__ __forceinline__ void act_dact_f(float x, int kind, float& a, float& d
         a = fmaxf(x, 0.0f);
         d = x > 0.0f ? 1.0f : 0.0f;
     } else {
-        const float k0 = 0.7978845608028654f, k1 = 0.044715f;
-        const float s = sigmoid2z_f(x);
-        const float dz2 = 2.0f * k0 * (1.0f + 3.0f * k1 * x * x);
-        a = x * s;
-        d = s + x * s * (1.0f - s) * dz2;
+        gelu_dgelu_f(x, a, d);
     }
 }
 __device__ __forceinline__ float act_f(float x, int kind) {

@@ -111,8 +111,15 @@ __device__ __forceinline__ void epilogue_vec8(const GemmArgs& g, int64_t coff, i
     }
     if (g.epilogue == BB_EPI_ACT) {
         if (g.aux_out) store_vec((bf16*)g.aux_out + xi, v);
+        // one branch over the kind for the eight elements (inside the element loop the compiler turns it into
+        // both evaluations and a select per element)
+        if (g.act == BB_ACT_RELU) {
 #pragma unroll
-        for (int e = 0; e < 8; ++e) v[e] = act_f(v[e], g.act);
+            for (int e = 0; e < 8; ++e) v[e] = fmaxf(v[e], 0.0f);
+        } else {
+#pragma unroll
+            for (int e = 0; e < 8; ++e) v[e] = gelu_tanh_f(v[e]);
+        }
         if (drop) {
 #pragma unroll
             for (int e = 0; e < 8; ++e) v[e] *= keep[e];
@@ -120,8 +127,13 @@ __device__ __forceinline__ void epilogue_vec8(const GemmArgs& g, int64_t coff, i
     } else if (g.epilogue == BB_EPI_DACT) {
         float u[8];
         load_vec((const bf16*)g.aux_in + xi, u);
+        if (g.act == BB_ACT_RELU) {
 #pragma unroll
-        for (int e = 0; e < 8; ++e) v[e] *= dact_f(u[e], g.act);
+            for (int e = 0; e < 8; ++e) v[e] *= u[e] > 0.0f ? 1.0f : 0.0f;
+        } else {
+#pragma unroll
+            for (int e = 0; e < 8; ++e) v[e] *= dgelu_tanh_f(u[e]);
+        }
     } else if (g.epilogue == BB_EPI_RESIDUAL) {
         float r[8];
         load_vec((const bf16*)g.resid + xi, r);
@@ -143,8 +155,16 @@ __device__ __forceinline__ void epilogue_vec8(const GemmArgs& g, int64_t coff, i
         for (int e = 0; e < 8; ++e) v[e] = d[e] > 0.f ? v[e] : 0.f;
     } else if (g.epilogue == BB_EPI_ACT_DACT) {
         float d[8];
+        if (g.act == BB_ACT_RELU) {
 #pragma unroll
-        for (int e = 0; e < 8; ++e) act_dact_f(v[e], g.act, v[e], d[e]);
+            for (int e = 0; e < 8; ++e) {
+                d[e] = v[e] > 0.0f ? 1.0f : 0.0f;
+                v[e] = fmaxf(v[e], 0.0f);
+            }
+        } else {
+#pragma unroll
+            for (int e = 0; e < 8; ++e) gelu_dgelu_f(v[e], v[e], d[e]);
+        }
         if (drop) {
 #pragma unroll
             for (int e = 0; e < 8; ++e) {
