@@ -120,8 +120,8 @@ def test_gemm_epilogues(hiplib, dtype):
     assert rel_err(C, 0.125 * (Af @ Wf.t())) < tol(dtype)
 
 
-@pytest.mark.parametrize("layout", ["nt", "nn"])
-@pytest.mark.parametrize("M,N,K", [(7168, 4096, 576), (7100, 4104, 640), (8192, 4096, 1024), (7168, 4096, 128)])
+@pytest.mark.parametrize("layout,M,N,K", [(lay, *shape) for shape in [(7168, 4096, 576), (7100, 4104, 640), (8192, 4096, 1024)]
+                                          for lay in ("nt", "nn")] + [("nn", 7168, 4096, 128)])
 def test_gemm_persistent_blocks(hiplib, layout, M, N, K):
     """More than one round of 256x256 tiles: the blocks of the persistent kernel walk several tiles each with the
     k-tile stream running through the tile boundaries.  Every epilogue kind against fp64 (ragged edges included), and
@@ -129,8 +129,6 @@ def test_gemm_persistent_blocks(hiplib, layout, M, N, K):
     order of the contraction is the same in all of them."""
     dtype = torch.bfloat16
     lay = hiplib.NT if layout == "nt" else hiplib.NN
-    if layout == "nt" and K <= 512:
-        pytest.skip("short forward contractions take the 128x64 tiles")
     A = randn(M, K, dtype=dtype, seed=11)
     W = randn(N, K, dtype=dtype, seed=12, scale=0.1) if layout == "nt" else randn(K, N, dtype=dtype, seed=12, scale=0.1)
     bias, X = randn(N, dtype=dtype, seed=13), randn(M, N, dtype=dtype, seed=14)
