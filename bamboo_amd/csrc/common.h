@@ -66,8 +66,13 @@ __device__ __forceinline__ float bf2f(uint16_t b) { return __uint_as_float(((uin
 __device__ __forceinline__ uint16_t f2bf(float f) {
     return __builtin_bit_cast(uint16_t, (__bf16)f);  // round-to-nearest-even (v_cvt_pk_bf16_f32)
 }
+// two floats -> two bf16 in one register: a vector conversion, so that it is ONE v_cvt_pk_bf16_f32 (two scalar
+// conversions and an OR take three instructions; the rounding is the same)
 __device__ __forceinline__ uint32_t pack2bf(float lo, float hi) {
-    return (uint32_t)f2bf(lo) | ((uint32_t)f2bf(hi) << 16);
+    typedef __attribute__((ext_vector_type(2))) float f32x2_t;
+    typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2_t;
+    const f32x2_t f = {lo, hi};
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(f, bf16x2_t));
 }
 
 template <typename T> struct Elem;
