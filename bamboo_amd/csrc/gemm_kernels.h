@@ -84,13 +84,12 @@ __device__ __forceinline__ void epilogue_elem(const GemmArgs& g, int64_t coff, i
 }
 
 // Vector epilogue for bf16 operands: 8 consecutive columns of one row (n % 8 == 0, n + 8 <= N).
+// (ci, xi: element offsets of (m, n) in C and in the epilogue's operand / second output; b: the bias of the eight
+// columns, read by the caller once for all the rows it stores in them)
 template <bool DROP>
-__device__ __forceinline__ void epilogue_vec8(const GemmArgs& g, int64_t coff, int m, int n, float (&v)[8]) {
-    const int64_t ci = coff + (int64_t)m * g.ldc + n;
-    const int64_t xi = coff + (int64_t)m * g.ldaux + n;
+__device__ __forceinline__ void epilogue_vec8_at(const GemmArgs& g, int64_t ci, int64_t xi, int m, int n, float (&v)[8],
+                                                 const float (&b)[8]) {
     if (g.bias) {
-        float b[8];
-        load_vec((const bf16*)g.bias + n, b);
 #pragma unroll
         for (int e = 0; e < 8; ++e) v[e] += b[e];
     }
@@ -189,6 +188,12 @@ __device__ __forceinline__ void epilogue_vec8(const GemmArgs& g, int64_t coff, i
     } else {
         store_vec((bf16*)g.C + ci, v);
     }
+}
+template <bool DROP>
+__device__ __forceinline__ void epilogue_vec8(const GemmArgs& g, int64_t coff, int m, int n, float (&v)[8]) {
+    float b[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    if (g.bias) load_vec((const bf16*)g.bias + n, b);
+    epilogue_vec8_at<DROP>(g, coff + (int64_t)m * g.ldc + n, coff + (int64_t)m * g.ldaux + n, m, n, v, b);
 }
 
 template <typename F, int... Is> __device__ __forceinline__ void static_for(F&& f, std::integer_sequence<int, Is...>) {
@@ -950,10 +955,16 @@ __device__ __forceinline__ void gemm_bf16_dma_body(const GemmArgs& g, const int 
                     patch[(8 * (r >> 2) + 4 * (lane >> 5) + (r & 3)) * PLD + h * 32 + (lane & 31)] = acc[i][jp * 2 + h][r] * g.alpha;
             asm volatile("" ::: "memory");
             const int n = n0 + wn * WTN + jp * 64 + pcol;
-            const bool live = NH == 2 || pcol < 32;
+            const bool live = (NH == 2 || pcol < 32) && n < g.N;
+            // per patch: the bias of the lane's eight columns once, the offsets of its first row by multiplication
+            // and of the other three by addition (a 64-bit multiply is several quarter-rate instructions)
+            float b8[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+            if (g.bias && live) load_vec((const bf16*)g.bias + n, b8);
+            const int m_first = m0 + wm * WTM + i * 32 + prow;
+            int64_t ci = coff + (int64_t)m_first * g.ldc + n, xi = coff + (int64_t)m_first * g.ldaux + n;
 #pragma unroll
             for (int it = 0; it < 4; ++it) {
-                const int m = m0 + wm * WTM + i * 32 + it * 8 + prow;
+                const int m = m_first + it * 8;
                 float v[8];
                 const f32x4 lo = *(const f32x4*)(patch + (it * 8 + prow) * PLD + pcol);
                 const f32x4 hi = *(const f32x4*)(patch + (it * 8 + prow) * PLD + pcol + 4);
@@ -962,7 +973,9 @@ __device__ __forceinline__ void gemm_bf16_dma_body(const GemmArgs& g, const int 
                     v[e] = lo[e];
                     v[4 + e] = hi[e];
                 }
-                if (live && m < g.M && n < g.N) epilogue_vec8<DROP>(g, coff, m, n, v);
+                if (live && m < g.M) epilogue_vec8_at<DROP>(g, ci, xi, m, n, v, b8);
+                ci += 8 * (int64_t)g.ldc;
+                xi += 8 * (int64_t)g.ldaux;
             }
             if constexpr (STATS) {
                 // Column statistics of this 32-row strip straight from the patch: lane = column, 32 conflict-free LDS
