@@ -1184,6 +1184,10 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_bf16_dma_persist_kernel(cons
         int tm, tn;
         tile_coords(tile, g.tiles_m, g.tiles_n, tm, tn);
         const int m0 = tm * BM + wm * WTM, n = tn * BN + wn * WTN + pchunk * 8;
+        // the bias of the lane's eight columns once per tile; row offsets by addition (see gemm_bf16_dma_body)
+        float b8[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+        if (g.bias && n < g.N) load_vec((const bf16*)g.bias + n, b8);
+        int64_t ci = (int64_t)(m0 + prow) * g.ldc + n, xi = (int64_t)(m0 + prow) * g.ldaux + n;
         // (static_for: a loop the compiler declines to unroll would index the accumulators dynamically, i.e. from scratch)
         static_for(
             [&](auto idx) {
@@ -1204,9 +1208,9 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_bf16_dma_persist_kernel(cons
                     const f32x4 c2 = *(const f32x4*)(patch + row * 64 + ((second_chunk ^ (row & 15)) << 2));
                     const f32x4 lo = pchunk < 4 ? c1 : c2, hi = pchunk < 4 ? c2 : c1;
                     float v[8] = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
-                    if (m < g.M && n < g.N) {
-                        epilogue_vec8<DROP>(g, 0, m, n, v);
-                    }
+                    if (m < g.M && n < g.N) epilogue_vec8_at<DROP>(g, ci, xi, m, n, v, b8);
+                    ci += 8 * (int64_t)g.ldc;
+                    xi += 8 * (int64_t)g.ldaux;
                     },
                     std::make_integer_sequence<int, 4>{});
                 asm volatile("" ::: "memory");
