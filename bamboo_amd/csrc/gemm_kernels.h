@@ -28,8 +28,8 @@ __device__ __forceinline__ float drop_factor(const GemmArgs& g, int m, int n) {
 // round-robin over the 8 XCDs, each with a private L2), and walk the output in column
 // panels of GROUP_M row-tiles so that an XCD's resident tiles share A rows and B columns.
 // logical tile -> (row tile, column tile): column panels of GROUP_M row-tiles
+template <int GROUP_M = 8>
 __device__ __forceinline__ void panel_coords(int lid, int tiles_m, int tiles_n, int& tm, int& tn) {
-    constexpr int GROUP_M = 8;
     const int width = GROUP_M * tiles_n;
     const int group = lid / width;
     const int first_m = group * GROUP_M;
@@ -43,8 +43,9 @@ __device__ __forceinline__ int xcd_contiguous(int bid, int total) {
     const int per = total / 8;
     return (per > 0 && bid < per * 8) ? (bid % 8) * per + bid / 8 : bid;
 }
+template <int GROUP_M = 8>
 __device__ __forceinline__ void tile_coords(int bid, int tiles_m, int tiles_n, int& tm, int& tn) {
-    panel_coords(xcd_contiguous(bid, tiles_m * tiles_n), tiles_m, tiles_n, tm, tn);
+    panel_coords<GROUP_M>(xcd_contiguous(bid, tiles_m * tiles_n), tiles_m, tiles_n, tm, tn);
 }
 
 // Generic scalar epilogue.  T = operand dtype (bias/aux/resid), output fp32 or T.
@@ -651,8 +652,11 @@ __device__ __forceinline__ void gemm_bf16_dma_body(const GemmArgs& g, const int 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wm = wave / WN, wn = wave % WN;
     int tile_m, tile_n;
-    if (logical_id) panel_coords(block_id, g.tiles_m, g.tiles_n, tile_m, tile_n);
-    else tile_coords(block_id, g.tiles_m, g.tiles_n, tile_m, tile_n);
+    // the 32 tiles an XCD holds at a time read BM * rows + BN * columns operand rows: 4 x 8 tiles of 256 x 128 read
+    // 2048, 8 x 4 read 2560
+    constexpr int GROUP_M = (BM == 256 && BN == 128 && CONV == 0) ? 4 : 8;
+    if (logical_id) panel_coords<8>(block_id, g.tiles_m, g.tiles_n, tile_m, tile_n);
+    else tile_coords<GROUP_M>(block_id, g.tiles_m, g.tiles_n, tile_m, tile_n);
     const int m0 = tile_m * BM, n0 = tile_n * BN;
     const int b1 = batch_id / g.nb2, b2 = batch_id % g.nb2;
     const bf16* A = (const bf16*)g.A + b1 * g.sA1 + b2 * g.sA2;
