@@ -8,6 +8,8 @@
 
 #include <stdarg.h>
 
+#include <atomic>
+
 // ---- error string ------------------------------------------------------------------------
 static thread_local char g_err[512] = "";
 void bb_set_error(const char* fmt, ...) {
@@ -421,7 +423,9 @@ extern "C" int bb_layernorm_bwd(int dtype, int kind, int rows, int cols, float e
 // hipGetSymbolAddress returns with that device current -- the array's name is no device address on the host.
 static __device__ __align__(256) float ln_bwd_static_scratch[LN_BWD_BLOCKS * 2 * BB_LN_BWD_STATIC_MAX_COLS];
 constexpr int LN_STATIC_MAX_DEVICES = 64;
-static float* g_ln_static_ptr[LN_STATIC_MAX_DEVICES];   // per device: address of its copy, null until set up
+// per device: address of its copy, null until set up.  Written once under the mutex (release), read by the entry
+// point without it (acquire): a reader that sees the address also sees the set-up that preceded its store.
+static std::atomic<float*> g_ln_static_ptr[LN_STATIC_MAX_DEVICES];
 static std::mutex g_ln_static_mu;
 
 template <typename T, int IT> static hipError_t ln_bwd_allow_one_pass() {
@@ -433,7 +437,7 @@ template <typename T, int IT> static hipError_t ln_bwd_allow_one_pass() {
 static int ln_bwd_static_setup(int dev) {
     BB_REQUIRE(dev >= 0 && dev < LN_STATIC_MAX_DEVICES, "bb_layernorm_bwd_static: device ordinal %d out of range", dev);
     std::lock_guard<std::mutex> lock(g_ln_static_mu);
-    if (g_ln_static_ptr[dev]) return BB_OK;
+    if (g_ln_static_ptr[dev].load(std::memory_order_acquire)) return BB_OK;
     float* ptr = nullptr;
     BB_HIP_CHECK(hipGetSymbolAddress((void**)&ptr, HIP_SYMBOL(ln_bwd_static_scratch)));
     BB_REQUIRE(ptr != nullptr, "bb_layernorm_bwd_static: no address for the scratch array on device %d", dev);
@@ -445,7 +449,7 @@ static int ln_bwd_static_setup(int dev) {
     BB_HIP_CHECK((ln_bwd_allow_one_pass<float, 4>()));
     BB_HIP_CHECK((ln_bwd_allow_one_pass<float, 8>()));
     BB_HIP_CHECK((ln_bwd_allow_one_pass<float, 16>()));
-    g_ln_static_ptr[dev] = ptr;
+    g_ln_static_ptr[dev].store(ptr, std::memory_order_release);
     return BB_OK;
 }
 
@@ -457,14 +461,16 @@ extern "C" int bb_layernorm_bwd_static(int dtype, int kind, int rows, int cols, 
     int dev = 0;
     BB_HIP_CHECK(hipGetDevice(&dev));
     BB_REQUIRE(dev >= 0 && dev < LN_STATIC_MAX_DEVICES, "bb_layernorm_bwd_static: device ordinal %d out of range", dev);
-    if (!g_ln_static_ptr[dev]) {    // bb_init was not called on this device: set up now (not under stream capture)
+    float* scratch = g_ln_static_ptr[dev].load(std::memory_order_acquire);
+    if (!scratch) {    // bb_init was not called on this device: set up now (not under stream capture)
         int rc = ln_bwd_static_setup(dev);
         if (rc) return rc;
+        scratch = g_ln_static_ptr[dev].load(std::memory_order_acquire);
     }
     // every block of the kernel writes its whole partial row (zeros where it had no rows) before the reduction
     // reads it: nothing of the previous call's contents is read, so nothing has to be cleared
     return ln_bwd_run("bb_layernorm_bwd_static", dtype, kind, rows, cols, eps, x, gain, mean, rinv, dy, dres, dx, dgain, dshift,
-                      g_ln_static_ptr[dev], (hipStream_t)stream);
+                      scratch, (hipStream_t)stream);
 }
 
 // =========================================================================================

@@ -440,8 +440,9 @@ extern "C" int bb_gemm_grouped(const bb_gemm_desc* descs, int count, void* strea
     bool fuse = count >= (has_conv ? 1 : 2) && count <= GROUP_MAX;
     for (int i = 0; i < count && fuse; ++i) {
         const bb_gemm_desc& d = descs[i];
+        // the grouped kernel is built without dropout decisions in its epilogue: such a problem runs by itself
         fuse = d.dtype == BB_BF16 && d.layout == descs[0].layout && d.nb1 <= 1 && d.nb2 <= 1 && d.M > 0 && d.N > 0 &&
-               pick_dma_tile(d.M, d.N, d.K, 1, d.layout) != D_NONE;
+               d.dropout_p == 0.f && pick_dma_tile(d.M, d.N, d.K, 1, d.layout) != D_NONE;
     }
     // a patch-matrix B exists only inside the grouped kernel: no one-by-one route for it
     BB_REQUIRE(fuse || !has_conv, "bb_gemm_grouped: a problem with a patch-matrix B must share a launch of bf16 BB_TN "

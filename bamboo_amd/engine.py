@@ -33,15 +33,6 @@ from .optim import FusedAdam
 from .p2p import AllReduceException, NextStageException, PrevStageException, SeededActivationQueue  # noqa: F401
 from .utils import get_redundant_stage_ids, get_redundant_user_stage_ids
 
-should_stop = False
-
-
-def sig_handler(signum, frame):
-    global should_stop
-    print("[Engine] Signal handler called with signal", signum)
-    should_stop = True
-
-
 class PipelineEngine:
     def __init__(self, args=None, model=None, optimizer=None, model_parameters=None, training_data=None,
                  lr_scheduler=None, mpu=None, dist_init_required=None, collate_fn=None, config=None,
@@ -58,8 +49,12 @@ class PipelineEngine:
         self.config = cfg if isinstance(cfg, BambooConfig) else BambooConfig(cfg)
         if self.config.compute_dtype != model.dtype:
             raise PipelineError(f"config asks for {self.config.compute_dtype} but the module was built for {model.dtype}")
+        # SIGTERM (the spot instance's preemption notice) makes the next train_batch exit with code 13
+        # (reference engine.py:98-111, 1077-1079).  The flag lives on the engine; a process has one handler slot, so
+        # with several engines in one process (one per thread) the last one built with the handler owns it.
+        self.should_stop = False
         if install_signal_handler:
-            signal.signal(signal.SIGTERM, sig_handler)
+            signal.signal(signal.SIGTERM, self.sig_handler)
 
         self.device = model.device
         self.micro_batch_size = self.config.train_micro_batch_size_per_gpu
@@ -101,7 +96,7 @@ class PipelineEngine:
         # of (stage, micro-batch) touches the same static buffers in every batch, so its ~100
         # launches are captured the second time they occur and launched as one graph afterwards.
         self.use_graphs = bool(use_graphs)
-        if self.use_graphs and any(getattr(l, "dropout", 0) > 0 for ls in model.func_buckets.values() for l in ls):
+        if self.use_graphs and self._has_dropout(model.func_buckets):
             raise PipelineError("use_graphs with dropout: the dropout keys change with every batch and are kernel "
                                 "arguments, a replayed graph would repeat the first batch's masks")
         if self.use_graphs and self.main_stream.cuda_stream == 0:
@@ -168,6 +163,19 @@ class PipelineEngine:
         self._install_sched_generator()
         self.tput_t0 = None
         self.timers = {}
+
+    def _has_dropout(self, stage_ids):
+        return any(getattr(layer, "dropout", 0) > 0 for sid in stage_ids for layer in self.module.func_buckets.get(sid, []))
+
+    def sig_handler(self, signum, frame):
+        print("[Engine] Signal handler called with signal", signum)
+        self.should_stop = True
+
+    def set_gemm_hook(self, hook):
+        """Observer of every GEMM launch of THIS engine's lanes (``hook(desc, launch, stream)``, see ``hip.gemm``), or
+        None.  While one is set the engine launches eagerly (a captured graph would replay the launches past it)."""
+        self.ctx.gemm_hook = hook
+        self.rc_ctx.gemm_hook = hook
 
     # ------------------------------------------------------------------ redundancy
     def _inc(self, stage_id):
@@ -302,8 +310,7 @@ class PipelineEngine:
         """Run one batch (``micro_batches`` micro-batches) through the stage's schedule, including
         the redundant forwards and, if the successor is lost, the failover; returns the mean
         micro-batch loss where this process sees one (loss-head peer or last stage), else 0."""
-        global should_stop
-        if should_stop:
+        if self.should_stop:
             raise SystemExit(13)
         if data_iter is not None:
             self.set_dataiterator(data_iter)
@@ -404,6 +411,11 @@ class PipelineEngine:
         if not self.eager_recovery:
             # lazy mode keeps CPU mirrors only: materialise the layers from them now
             self.module.build_layers(absorbed, self.param_buffers[absorbed])
+            if self.use_graphs and self._has_dropout([absorbed]):
+                # the layers that arrive only now carry dropout (the constructor's check saw the own stage alone):
+                # from here on every kernel is launched with this batch's keys, nothing is replayed
+                self.use_graphs = False
+                self._graphs.clear()
             sp = self.module.stage_params[absorbed]
             flats = getattr(self.state_buffers[absorbed], "flat", None)
             if flats is not None and flats["exp_avg"].numel() == sp.numel:
@@ -413,7 +425,9 @@ class PipelineEngine:
                 for i, name in enumerate(sp.index):
                     sp.view(sp.exp_avg, name).copy_(self.state_buffers[absorbed][f"{i}.exp_avg"])
                     sp.view(sp.exp_avg_sq, name).copy_(self.state_buffers[absorbed][f"{i}.exp_avg_sq"])
+            hook = self.ctx.gemm_hook
             self.ctx = self.module.prepare_context(self.stage_ids + [absorbed], self.batch, self.seq, stream=self.main_stream)
+            self.ctx.gemm_hook = hook
             self.stash_bytes += self.module.allocate_stash(absorbed, self.ctx, self.micro_batches)
             act_shape = self.module.stage_io_shapes(absorbed, self.batch)[0]
             self._input_grad_store[absorbed] = [torch.empty(act_shape, dtype=self.module.dtype, device=self.device)
@@ -437,7 +451,7 @@ class PipelineEngine:
         """Run ``issue()`` (which only launches kernels of this library on ``stream`` and returns a
         value that does not change between batches): eagerly the first time ``key`` occurs, captured
         and launched the second time, replayed from then on."""
-        if not self.use_graphs or hip.gemm_hook is not None:
+        if not self.use_graphs or self.ctx.gemm_hook is not None:
             return issue()
         state = self._graphs.get(key)
         if state is None:

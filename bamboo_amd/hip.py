@@ -244,11 +244,14 @@ def gemm_strip_stats_supported(layout, A, B, C):
     return bool(lib().bb_gemm_strip_stats_supported(byref(gemm_desc(layout, A, B, C))))
 
 
-def gemm(layout, A, B, C, *, stream=None, **kw):
-    """C = epilogue(alpha * op(A) op(B) [+ bias]) on 2-D row-major views (inner stride 1)."""
+def gemm(layout, A, B, C, *, stream=None, hook=None, **kw):
+    """C = epilogue(alpha * op(A) op(B) [+ bias]) on 2-D row-major views (inner stride 1).
+    ``hook``: optional observer called as ``hook(desc, launch, stream)`` instead of the launch; ``launch()`` performs
+    the call on ``stream`` (the benchmark brackets launches with events this way).  It belongs to the caller (an
+    execution context of one engine), never to the module."""
     d = gemm_desc(layout, A, B, C, **kw)
-    if gemm_hook is not None:
-        gemm_hook(d, lambda: check(lib().bb_gemm(byref(d), stream_ptr(stream)), "bb_gemm"), stream)
+    if hook is not None:
+        hook(d, lambda: check(lib().bb_gemm(byref(d), stream_ptr(stream)), "bb_gemm"), stream)
     else:
         check(lib().bb_gemm(byref(d), stream_ptr(stream)), "bb_gemm")
     return C
@@ -259,7 +262,7 @@ def gemm_splitk_workspace(descs):
     return int(lib().bb_gemm_splitk_workspace(arr, len(descs)))
 
 
-def gemm_grouped(descs, stream=None, splitk_ws=None):
+def gemm_grouped(descs, stream=None, splitk_ws=None, hook=None):
     """Independent GEMMs of one layout in one launch (falls back to one launch each inside the
     library when they cannot share a kernel).  With ``splitk_ws`` (a tensor of at least
     ``gemm_splitk_workspace(descs)`` bytes) problems with few output tiles and a long contraction
@@ -271,8 +274,8 @@ def gemm_grouped(descs, stream=None, splitk_ws=None):
                              "bb_gemm_grouped_splitk")
     else:
         call = lambda: check(lib().bb_gemm_grouped(arr, len(descs), stream_ptr(stream)), "bb_gemm_grouped")
-    if gemm_hook is not None:
-        gemm_hook(descs, call, stream)
+    if hook is not None:
+        hook(descs, call, stream)
     else:
         call()
 
@@ -281,11 +284,6 @@ def gemm_variant(desc):
     buf = ctypes.create_string_buffer(64)
     check(lib().bb_gemm_variant(byref(desc), buf, 64), "bb_gemm_variant")
     return buf.value.decode()
-
-
-# Optional observer called as hook(desc, launch, stream) around every dense GEMM; `launch()`
-# performs the call on `stream` (None = the current stream).  Used by the benchmark to bracket launches with events; None in normal operation.
-gemm_hook = None
 
 
 def gemm_batched(layout, dtype, M, N, K, A_ptr, lda, sA, B_ptr, ldb, sB, C_ptr, ldc, sC, nb1, nb2, *,
@@ -616,7 +614,7 @@ def conv3x3_supported(dtype, mode, n, h, w, cin, cout):
     return bool(lib().bb_conv3x3_supported(dtype_code(dtype), mode, n, h, w, cin, cout))
 
 
-def conv3x3(mode, src, weight, dst, n, h, w, cin, cout, strip_stats=None, stream=None):
+def conv3x3(mode, src, weight, dst, n, h, w, cin, cout, strip_stats=None, stream=None, hook=None):
     """``CONV_FWD``: dst[n*h*w, cout] = conv3x3(src[n*h*w, cin]); ``CONV_DGRAD``: dst[n*h*w, cin] = the input
     gradient for src = dy[n*h*w, cout]; weight [cout, 3, 3, cin]."""
     rows = n * h * w
@@ -632,14 +630,14 @@ def conv3x3(mode, src, weight, dst, n, h, w, cin, cout, strip_stats=None, stream
         _check_strip_stats(strip_stats, rows, cout)
     call = lambda: check(lib().bb_conv3x3(dtype_code(src.dtype), mode, n, h, w, cin, cout, _ptr(src), _ptr(weight),
                                           _ptr(dst), _ptr(strip_stats), stream_ptr(stream)), "bb_conv3x3")
-    if gemm_hook is not None:
-        gemm_hook(ConvLaunch(mode, rows, cin, cout), call, stream)
+    if hook is not None:
+        hook(ConvLaunch(mode, rows, cin, cout), call, stream)
     else:
         call()
 
 
 class ConvLaunch:
-    """What ``gemm_hook`` is handed for an implicit-GEMM convolution: the GEMM it amounts to."""
+    """What a launch observer (``hook=``) is handed for an implicit-GEMM convolution: the GEMM it amounts to."""
 
     def __init__(self, mode, rows, cin, cout):
         self.variant_name = "bf16_conv3x3_fwd_igemm128x64w8k64s3" if mode == CONV_FWD else "bf16_conv3x3_dgrad_igemm64x128w8k64s3"

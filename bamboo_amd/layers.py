@@ -41,6 +41,18 @@ class StageContext:
         # by a backward pass only after a failover); ``deferred`` tells that backward pass to produce it first
         self.defer = False
         self.deferred = False
+        # optional observer of this lane's GEMM launches (``hip.gemm(..., hook=)``); set through the engine that owns
+        # the context, so a probe on one engine sees and changes nothing of another
+        self.gemm_hook = None
+
+    def gemm(self, *a, **kw):
+        return hip.gemm(*a, hook=self.gemm_hook, **kw)
+
+    def gemm_grouped(self, *a, **kw):
+        return hip.gemm_grouped(*a, hook=self.gemm_hook, **kw)
+
+    def conv3x3(self, *a, **kw):
+        return hip.conv3x3(*a, hook=self.gemm_hook, **kw)
 
     @property
     def rows(self):
@@ -292,9 +304,9 @@ class TransformerLayer:
         st["x0"] = x
         hip.layernorm_fwd(x, w["sublayer.0.norm.a_2"], w["sublayer.0.norm.b_2"], st["n1"], st["mean1"],
                           st["rinv1"], kind, self.eps, stream=sm)
-        hip.gemm(hip.NT, st["n1"], w["qkv.weight"], st["qkv"], bias=w["qkv.bias"], stream=sm)
+        ctx.gemm(hip.NT, st["n1"], w["qkv.weight"], st["qkv"], bias=w["qkv.bias"], stream=sm)
         self._attention_fwd(st, ctx)
-        hip.gemm(hip.NT, st["ctx"], w["self_attn.linears.3.weight"], st["x1"], bias=w["self_attn.linears.3.bias"],
+        ctx.gemm(hip.NT, st["ctx"], w["self_attn.linears.3.weight"], st["x1"], bias=w["self_attn.linears.3.bias"],
                  epilogue=hip.EPI_RESIDUAL, resid=x, dropout=self._drop(ctx, self.SITE_SUBLAYER0), stream=sm)
         hip.layernorm_fwd(st["x1"], w["sublayer.1.norm.a_2"], w["sublayer.1.norm.b_2"], st["n2"], st["mean2"],
                           st["rinv2"], kind, self.eps, stream=sm)
@@ -305,11 +317,11 @@ class TransformerLayer:
         if ctx.defer or self.activation == "relu":
             # act' is read by the backward pass only: a forward that most likely has none writes act alone (and a
             # ReLU layer never writes it: its backward pass reads the derivative off act)
-            hip.gemm(hip.NT, st["n2"], w["feed_forward.w_1.weight"], st["act"], bias=w["feed_forward.w_1.bias"],
+            ctx.gemm(hip.NT, st["n2"], w["feed_forward.w_1.weight"], st["act"], bias=w["feed_forward.w_1.bias"],
                      epilogue=hip.EPI_ACT, act=act, dropout=self._drop(ctx, self.SITE_FFN), stream=sm)
         else:
             self._ffn1(st, ctx)
-        hip.gemm(hip.NT, st["act"], w["feed_forward.w_2.weight"], st["out"], bias=w["feed_forward.w_2.bias"],
+        ctx.gemm(hip.NT, st["act"], w["feed_forward.w_2.weight"], st["out"], bias=w["feed_forward.w_2.bias"],
                  epilogue=hip.EPI_RESIDUAL, resid=st["x1"], dropout=self._drop(ctx, self.SITE_SUBLAYER1), stream=sm)
         return st["out"]
 
@@ -317,7 +329,7 @@ class TransformerLayer:
         """act and act' of the feed-forward's hidden layer; under dropout both carry the keep factor, so the backward
         pass multiplies by the stored derivative as before."""
         w = self.w
-        hip.gemm(hip.NT, st["n2"], w["feed_forward.w_1.weight"], st["act"], bias=w["feed_forward.w_1.bias"],
+        ctx.gemm(hip.NT, st["n2"], w["feed_forward.w_1.weight"], st["act"], bias=w["feed_forward.w_1.bias"],
                  epilogue=hip.EPI_ACT_DACT, act=hip.ACT_CODES[self.activation], aux_out=st["dact"],
                  dropout=self._drop(ctx, self.SITE_FFN), stream=ctx.stream)
 
@@ -346,12 +358,12 @@ class TransformerLayer:
         wgrad(d_ff2, st["act"], "feed_forward.w_2.weight")
         if self.activation == "relu":
             # act = relu(u) * keep / (1 - p): positive exactly where the gradient passes, and then with factor 1 / (1 - p)
-            hip.gemm(hip.NN, d_ff2, w["feed_forward.w_2.weight"], d_ffn, epilogue=hip.EPI_MUL_POS, aux_in=st["act"],
+            ctx.gemm(hip.NN, d_ff2, w["feed_forward.w_2.weight"], d_ffn, epilogue=hip.EPI_MUL_POS, aux_in=st["act"],
                      alpha=1.0 / (1.0 - self.dropout) if self.dropout > 0 else 1.0, stream=sm)
         else:
-            hip.gemm(hip.NN, d_ff2, w["feed_forward.w_2.weight"], d_ffn, epilogue=hip.EPI_MUL, aux_in=st["dact"], stream=sm)
+            ctx.gemm(hip.NN, d_ff2, w["feed_forward.w_2.weight"], d_ffn, epilogue=hip.EPI_MUL, aux_in=st["dact"], stream=sm)
         wgrad(d_ffn, st["n2"], "feed_forward.w_1.weight")
-        hip.gemm(hip.NN, d_ffn, w["feed_forward.w_1.weight"], d_h0, stream=sm)
+        ctx.gemm(hip.NN, d_ffn, w["feed_forward.w_1.weight"], d_h0, stream=sm)
         # d_x1 = d_out + LN2'(d_n2)
         hip.layernorm_bwd(st["x1"], w["sublayer.1.norm.a_2"], st["mean2"], st["rinv2"], d_h0, d_out, d_h1,
                           g["sublayer.1.norm.a_2"], g["sublayer.1.norm.b_2"], ws, kind, self.eps, stream=sm)
@@ -361,16 +373,16 @@ class TransformerLayer:
             d_proj = ctx.buf("d_drop0", (R, h))
             hip.dropout_apply(d_h1, d_proj, *self._drop(ctx, self.SITE_SUBLAYER0), stream=sm)
         wgrad(d_proj, st["ctx"], "self_attn.linears.3.weight")
-        hip.gemm(hip.NN, d_proj, w["self_attn.linears.3.weight"], d_h0, stream=sm)
+        ctx.gemm(hip.NN, d_proj, w["self_attn.linears.3.weight"], d_h0, stream=sm)
         self._attention_bwd(d_h0, d_qkv, st, ctx)
         # QKV projection
         wgrad(d_qkv, st["n1"], "qkv.weight")
-        hip.gemm(hip.NN, d_qkv, w["qkv.weight"], d_h0, stream=sm)
+        ctx.gemm(hip.NN, d_qkv, w["qkv.weight"], d_h0, stream=sm)
         # d_x0 = d_x1 + LN1'(d_n1)
         hip.layernorm_bwd(st["x0"], w["sublayer.0.norm.a_2"], st["mean1"], st["rinv1"], d_h0, d_h1, d_x,
                           g["sublayer.0.norm.a_2"], g["sublayer.0.norm.b_2"], ws, kind, self.eps, stream=sm)
         # d_out (d_drop1), d_ffn, d_h1 (d_drop0) and d_qkv still hold the four output gradients here
-        hip.gemm_grouped(wgrads, stream=sm)
+        ctx.gemm_grouped(wgrads, stream=sm)
         return d_x
 
 
@@ -682,7 +694,7 @@ class BottleNeck:
             self._stats_ok[key] = x.shape[0] <= 8192 and hip.gemm_strip_stats_supported(hip.NT, x, weight, y)
         if self._stats_ok[key]:
             strips = ctx.buf("strips", (hip.strip_stats_workspace(x.shape[0], y.shape[1]),))
-        hip.gemm(hip.NT, x, weight, y, stream=ctx.stream, strip_stats=strips)
+        ctx.gemm(hip.NT, x, weight, y, stream=ctx.stream, strip_stats=strips)
         return strips
 
     def _implicit(self, ctx, mode):
@@ -704,7 +716,7 @@ class BottleNeck:
         self._bn_fwd(1, st["y1"], None, st["a1"], st["mean1"], st["rstd1"], True, ctx, strips)
         if self._implicit(ctx, hip.CONV_FWD):
             strips = ctx.buf("strips", (hip.strip_stats_workspace(R, cm),)) if R <= 8192 else None
-            hip.conv3x3(hip.CONV_FWD, st["a1"], w["residual_function.3.weight"], st["y2"], ctx.batch, self.h, self.w,
+            ctx.conv3x3(hip.CONV_FWD, st["a1"], w["residual_function.3.weight"], st["y2"], ctx.batch, self.h, self.w,
                         cm, cm, strip_stats=strips, stream=sm)
         else:
             col = ctx.buf("col", (R2, 9 * cm))
@@ -740,9 +752,9 @@ class BottleNeck:
         if self.projection:
             d_ys, d_xs = ctx.buf("d_ys", (R2, co)), ctx.buf("d_xs", (R2, ci))
             bn("shortcut", "ys", "mean_s", "rstd_s", d_res, None, d_ys, None)
-            hip.gemm(hip.NN, d_ys, w["shortcut.0.weight"], d_xs, stream=sm)
+            ctx.gemm(hip.NN, d_ys, w["shortcut.0.weight"], d_xs, stream=sm)
             xs = self._shortcut_input(st["x0"], ctx, R2)
-        hip.gemm(hip.NN, d_y3, w["residual_function.6.weight"], d_m0, stream=sm)          # d_a2
+        ctx.gemm(hip.NN, d_y3, w["residual_function.6.weight"], d_m0, stream=sm)          # d_a2
         bn(4, "y2", "mean2", "rstd2", d_m0, st["a2"], d_m1, None)                          # d_y2
         # weight gradient of the 3x3 convolution: patch matrix gathered inside the GEMM, else built again here
         # (cheaper than stashing it)
@@ -751,18 +763,18 @@ class BottleNeck:
             hip.patch3x3(st["a1"], col, ctx.batch, self.h, self.w, cm, stride=self.stride, stream=sm)
         d_a1, d_m2 = ctx.buf("d_m0", (R, cm)), ctx.buf("d_m2", (R, cm))
         if self._implicit(ctx, hip.CONV_DGRAD):
-            hip.conv3x3(hip.CONV_DGRAD, d_m1, w["residual_function.3.weight"], d_a1, ctx.batch, self.h, self.w, cm, cm,
+            ctx.conv3x3(hip.CONV_DGRAD, d_m1, w["residual_function.3.weight"], d_a1, ctx.batch, self.h, self.w, cm, cm,
                         stream=sm)
         else:
             d_col = ctx.buf("d_col", (R2, 9 * cm))
-            hip.gemm(hip.NN, d_m1, w["conv2"], d_col, stream=sm)
+            ctx.gemm(hip.NN, d_m1, w["conv2"], d_col, stream=sm)
             hip.patch3x3(d_col, d_a1, ctx.batch, self.h, self.w, cm, adjoint=True, stride=self.stride, stream=sm)
         bn(1, "y1", "mean1", "rstd1", d_a1, st["a1"], d_m2, None)                          # d_y1
         if self.projection and self.stride > 1:
-            hip.gemm(hip.NN, d_m2, w["residual_function.0.weight"], d_x, stream=sm)
+            ctx.gemm(hip.NN, d_m2, w["residual_function.0.weight"], d_x, stream=sm)
             hip.subsample(d_xs, d_x, ctx.batch, self.h, self.w, ci, self.stride, adjoint=True, stream=sm)
         else:
-            hip.gemm(hip.NN, d_m2, w["residual_function.0.weight"], d_x, epilogue=hip.EPI_RESIDUAL,
+            ctx.gemm(hip.NN, d_m2, w["residual_function.0.weight"], d_x, epilogue=hip.EPI_RESIDUAL,
                      resid=d_xs if self.projection else d_res, stream=sm)
         # the weight gradients in one launch: few output tiles over thousands of rows, cut along the rows
         descs = [hip.gemm_desc(hip.TN, d_y3, st["a2"], g["residual_function.6.weight"], accumulate=True),
@@ -771,7 +783,7 @@ class BottleNeck:
                  hip.gemm_desc(hip.TN, d_m2, st["x0"], g["residual_function.0.weight"], accumulate=True)]
         if self.projection:
             descs.append(hip.gemm_desc(hip.TN, d_ys, xs, g["shortcut.0.weight"], accumulate=True))
-        hip.gemm_grouped(descs, stream=sm, splitk_ws=ctx.buf("splitk", (8 * self._wgrad_elems(),)))
+        ctx.gemm_grouped(descs, stream=sm, splitk_ws=ctx.buf("splitk", (8 * self._wgrad_elems(),)))
         return d_x
 
 

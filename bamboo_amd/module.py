@@ -186,12 +186,50 @@ class PipelineModule:
             return int(first[1])  # (dp_id, stage_id)
         return 0
 
+    # ------------------------------------------------------------------ seeding
+    def _seed_layer(self, layer_idx):
+        """``seed_layers``: every layer is built under the seed ``base_seed + layer_idx`` (reference module.py:270-274;
+        ``seed_fn`` if given, else random / numpy / torch as ``set_random_seed``, runtime/utils.py:51-61), so the
+        process that owns a stage and the one that shadows it build the same weights from a ``LayerSpec``."""
+        if not self.seed_layers:
+            return
+        seed = self.base_seed + layer_idx
+        if self.seed_fn:
+            self.seed_fn(seed)
+        else:
+            import random
+
+            import numpy
+            random.seed(seed)
+            numpy.random.seed(seed)
+            torch.manual_seed(seed)
+
+    def _build_spec(self, layer_idx, auxiliary=False):
+        """The layer object of ``_layer_specs[layer_idx]``.  ``auxiliary``: a build whose only purpose is to look at
+        the layer (parameter count, width): the random generators are left as they were found."""
+        spec = self._layer_specs[layer_idx]
+        if not isinstance(spec, LayerSpec):
+            return spec
+        if not auxiliary:
+            self._seed_layer(layer_idx)
+            return spec.build()
+        import random
+
+        import numpy
+        saved = (random.getstate(), numpy.random.get_state(), torch.get_rng_state())
+        try:
+            return spec.build()
+        finally:
+            random.setstate(saved[0])
+            numpy.random.set_state(saved[1])
+            torch.set_rng_state(saved[2])
+
     # ------------------------------------------------------------------ partitioning
     def _count_layer_params(self):
         """Trainable parameters per layer (reference module.py:337-360: modules count theirs, bare callables 0)."""
         counts = []
-        for spec in self._layer_specs:
-            layer = spec.build() if isinstance(spec, LayerSpec) else spec
+        for idx in range(len(self._layer_specs)):
+            layer = self._build_spec(idx, auxiliary=True)
             if hasattr(layer, "num_params"):
                 counts.append(layer.num_params())
             elif isinstance(layer, torch.nn.Module):
@@ -230,7 +268,7 @@ class PipelineModule:
         self._local_start, self._local_stop = self.parts[self.stage_id], self.parts[self.stage_id + 1]
 
     # ------------------------------------------------------------------ building
-    def _instantiate(self, stage_id):
+    def _instantiate(self, stage_id, auxiliary=False):
         """Layer objects of a stage.  Layers of the reference's scripts (``nn.Module`` instances, ``LayerSpec`` of
         module classes, the ``x.sum(-1)`` callable; reference module.py:281-318) are replaced by the native layer
         that computes the same function; their weights are kept to be loaded into the arenas."""
@@ -240,7 +278,7 @@ class PipelineModule:
         for li, spec in enumerate(self._layer_specs[self.parts[stage_id]: self.parts[stage_id + 1]]):
             if isinstance(spec, TiedLayerSpec):
                 raise NotImplementedError("tied layers are not supported on the accelerated stage path")
-            layer = spec.build() if isinstance(spec, LayerSpec) else spec
+            layer = self._build_spec(self.parts[stage_id] + li, auxiliary=auxiliary)
             try:
                 layer, taken = adopt_layer(layer)
             except AdoptionError as e:
@@ -262,8 +300,7 @@ class PipelineModule:
         from .adopt import adopt_layer
         if layer_idx == 0:
             raise PipelineError("the first layer of the model must state its width")
-        spec = self._layer_specs[layer_idx - 1]
-        layer, _ = adopt_layer(spec.build() if isinstance(spec, LayerSpec) else spec)
+        layer, _ = adopt_layer(self._build_spec(layer_idx - 1, auxiliary=True))
         return layer.out_features
 
     def build_layers(self, stage_id, buffer=None):
@@ -298,7 +335,10 @@ class PipelineModule:
         ``param_buffer`` that are views of ONE flat tensor in the arena's order (``param_buffer.flat`` where the
         buffer is a :class:`MirrorBuffer`), page-locked when it lives on the host of a GPU process, so that a
         refresh and a promotion move it in a single transfer."""
-        layers = self.func_buckets.get(stage_id) or self._instantiate(stage_id)
+        layers = self.func_buckets.get(stage_id)
+        if not layers:
+            layers = self._instantiate(stage_id, auxiliary=True)
+            self._adopted_weights = {}           # only the shapes were wanted
         specs = [(f"{self.parts[stage_id] + li}.{name}", shape) for li, layer in enumerate(layers)
                  for name, shape in layer.param_specs().items()]
         flat = flat_mirror(sum(math.prod(shape) for _, shape in specs), device)

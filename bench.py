@@ -400,11 +400,11 @@ def main():
     if not args.no_probe:
         # the same steps again with every GEMM launch bracketed (costs ~10 % of the rate: not what is reported)
         probe = GemmProbe()
-        hip.gemm_hook = probe
+        engine.set_gemm_hook(probe)
         for _ in range(args.steps):
             engine.train_batch()
         torch.cuda.synchronize()
-        hip.gemm_hook = None
+        engine.set_gemm_hook(None)
     t_on = t_on_serial
 
     # leg 3 (default): RC on with the redundant forwards on a second HIP stream; this is the

@@ -88,13 +88,27 @@ def layer_norm(x, gain, shift, kind, eps):
     return F.layer_norm(x, x.shape[-1:], gain, shift, eps)
 
 
+# Set to a list by a test that hands a low-precision run's ReLU decisions to the oracle: every ReLU evaluated with
+# such decisions appends (elements, elements whose decision differs from the oracle's own x > 0, the largest |x|
+# among those, the largest |x| of the tensor).  Decisions may differ only where x is within rounding of zero.
+RELU_AUDIT = None
+
+
 def activation(x, kind, mask=None):
     """``mask`` (relu only): use this 0/1 tensor as the ReLU's decision instead of ``x > 0``.  A low-precision
     run decides ``x > 0`` on its own rounded ``x``; for the few pre-activations closer to zero than the
     rounding error the decision differs from the exact one and the derivative jumps.  Feeding the run's own
     decisions makes the comparison one of arithmetic, not of tie-breaking at the kink."""
     if kind == "relu":
-        return F.relu(x) if mask is None else x * mask.to(x.dtype)
+        if mask is None:
+            return F.relu(x)
+        if RELU_AUDIT is not None:
+            # what the handed-in decisions differ in from the oracle's own ``x > 0``, for the caller to bound
+            xd = x.detach()
+            differ = (xd > 0) != mask.to(torch.bool).view_as(xd)
+            worst = float(xd.abs()[differ].max()) if bool(differ.any()) else 0.0
+            RELU_AUDIT.append((xd.numel(), int(differ.sum()), worst, float(xd.abs().max())))
+        return x * mask.to(x.dtype)
     if kind == "gelu_tanh":
         return F.gelu(x, approximate="tanh")
     raise ValueError(kind)

@@ -131,3 +131,44 @@ def test_bottleneck_whose_shortcut_contradicts_its_shape_is_refused():
     ref.residual_function[3].stride = (2, 2)         # ... but a stride: the reference would have built a projection
     with pytest.raises(PipelineError, match="projection shortcut"):
         PipelineModule([ref], num_stages=1, stage_id=0, dtype=torch.float32, device="cpu")
+
+
+def test_seed_layers_gives_the_owner_and_the_shadow_the_same_weights():
+    """``seed_layers=True`` (reference module.py:270-274): every LayerSpec is built under ``base_seed + layer_idx``, so the
+    process that owns stage 2 and the one that shadows it start from equal weights whatever the ambient generator
+    holds; auxiliary builds (parameter counting for the partition, widths, host mirrors) leave the generators alone;
+    a ``seed_fn`` is called with the same seeds."""
+    specs = lambda: [LayerSpec(RefEncoderLayer, 32, 4, 64, 0.0) for _ in range(6)] + [LayerSpec(RefLayerNorm, 32), lambda x: x.sum(-1)]
+    kw = dict(num_stages=4, partition_method="parameters", dtype=torch.float32, device="cpu", seed_layers=True, base_seed=77)
+    torch.manual_seed(5)
+    owner = PipelineModule(specs(), stage_id=2, **kw)
+    torch.manual_seed(6)                                     # another process: another ambient state
+    torch.randn(17)
+    pred = PipelineModule(specs(), stage_id=1, **kw)
+    state = torch.get_rng_state()
+    pred.allocate_param(2, {})                               # host mirrors: shapes only
+    pred._count_layer_params()
+    assert torch.equal(torch.get_rng_state(), state)
+    pred.build_layers(2)                                     # the shadow stage
+    a, b = owner.stage_params[2], pred.stage_params[2]
+    assert list(a.index) == list(b.index) and a.numel > 0
+    assert torch.equal(a.master, b.master)
+    # the weights are those of a module built under that seed
+    first = owner.parts[2]
+    torch.manual_seed(77 + first)
+    ref = RefEncoderLayer(32, 4, 64, 0.0)
+    named = a.named(a.master)
+    for name, prm in ref.named_parameters():
+        assert torch.equal(named[f"{first}.{name}"], prm.detach()), name
+    # without seed_layers the ambient generator decides (the reference's behaviour too)
+    kw2 = dict(kw, seed_layers=False)
+    torch.manual_seed(5)
+    o2 = PipelineModule(specs(), stage_id=2, **kw2)
+    torch.manual_seed(6)
+    p2 = PipelineModule(specs(), stage_id=1, **kw2)
+    p2.build_layers(2)
+    assert not torch.equal(o2.stage_params[2].master, p2.stage_params[2].master)
+    # seed_fn sees base_seed + layer_idx of every layer it builds for real, in order
+    seen = []
+    PipelineModule(specs(), stage_id=3, seed_fn=lambda s: (seen.append(s), torch.manual_seed(s)), **kw)
+    assert seen == [77 + i for i in range(owner.parts[3], owner.parts[4]) if i < 7]

@@ -259,3 +259,79 @@ def test_failover_at_the_gpt2_1p5b_layer_shape(hiplib):
             err = float((g.double().cpu() - r).norm() / r.norm().clamp_min(floor * r.numel() ** 0.5))
             assert err < 2e-2, (s_, name, err)
     assert abs(float(loss) - float(peer.loss) / M) < 2e-2 * float(peer.loss) / M
+
+
+# ---------------------------------------------------------------- GPT-2-small stage (fp32) at its own shapes
+MB1, SEQ1, HID1, HEADS1, FFN1 = 4, 512, 768, 12, 3072
+
+
+def test_gpt2_small_stage_full_shape_fp32_matches_oracle(hiplib):
+    """The fp32 configuration at its own sizes (hidden 768, 12 heads, ffn 3072, seq 512, micro-batch 4, causal,
+    MSE to seeded N(0,1) targets): one own and one shadow layer, two micro-batches, redundant forwards on; stage
+    outputs (own and redundant) within 1e-5 and every gradient within 1e-4 of the fp64 CPU oracle, largest error
+    over the tensor's largest magnitude.  This is the only place where the fp32 path -- `gemm_f32_kernel` with
+    K = 768 / 3072 and the unfused attention (batched head products + softmax over 4 x 12 x 512 x 512
+    probabilities) -- meets the oracle at the sizes it is benchmarked on."""
+    from tests.test_gpu_stage import GPT_VARIANT, NoStep, build, grad_floor, oracle_for, rel_err
+    L, S, sid, M = 1, 4, 1, 2
+    engine, q = build(HID1, HEADS1, FFN1, L, S, sid, MB1, M, SEQ1, torch.float32, GPT_VARIANT, 1, True, grad_mode="mse")
+    assert not engine.module.func_buckets[sid][0].fused_attention(engine.ctx)
+    st, peer = oracle_for(engine, q, GPT_VARIANT, HID1, HEADS1, FFN1, L, S, sid, M, 1, True)
+    keep = {}
+    with NoStep(engine):
+        engine._clean_pipe_buffers = lambda: keep.update({k: list(v) for k, v in engine.pipe_buffers.items()})
+        loss = engine.train_batch()
+    torch.cuda.synchronize()
+    bufs, _ = st.run_batch(peer, optimizer_step=False)
+    rel_err.lowp = False
+    rows = MB1 * SEQ1
+    for k in range(M):
+        assert rel_err(keep[f"output_{sid}"][k], bufs["out"][(sid, k)].detach().view(rows, HID1)) < 1e-5, k
+        assert rel_err(keep[f"output_{sid + 1}"][k], bufs["out"][(sid + 1, k)].detach().view(rows, HID1)) < 1e-5, k
+        assert rel_err(keep[f"input_grad_{sid}"][k], bufs["sent_grad"][(sid, k)].view(rows, HID1)) < 1e-4, k
+    ref = st.named_grads(sid)
+    for name, g in engine.module.get_named_grad(sid):
+        assert rel_err(g, ref[name], grad_floor(ref)) < 1e-4, name
+    assert abs(float(loss) - float(peer.loss) / M) < 1e-5 * float(peer.loss) / M
+
+
+@pytest.mark.parametrize("mask", ["causal", "key_padding"])
+def test_unfused_attention_fp32_at_12_heads_512_positions(hiplib, mask):
+    """The fp32 attention core by itself at the GPT-2-small stage's size (4 x 12 heads x 512 positions, head
+    dimension 64): scores, masked softmax, context and the three input gradients against fp64 autograd on
+    ``softmax(Q K^T / sqrt(d) [masked]) V``, 1e-5 forward / 1e-4 backward of each tensor's largest magnitude."""
+    from bamboo_amd.layers import StageContext
+    b, a, s, d = MB1, HEADS1, SEQ1, 64
+    h = a * d
+    layer = TransformerLayer(h, a, 4 * h, activation="gelu_tanh", ln="standard", mask=mask)
+    ctx = StageContext(b, s, torch.float32, torch.device(DEV))
+    lens = None
+    if mask == "key_padding":
+        lens = torch.randint(128, s + 1, (b,), generator=torch.Generator().manual_seed(8), dtype=torch.int32).to(DEV)
+        lens[0] = s
+    ctx.key_len = lens
+    qkv = randn(b * s, 3 * h, seed=41, scale=0.7, dtype=torch.float32)
+    d_ctx = randn(b * s, h, seed=42, dtype=torch.float32)
+    st = {"qkv": qkv, "ctx": torch.empty(b * s, h, device=DEV), "prob": torch.empty(b, a, s, s, device=DEV)}
+    ctx.ensure_scratch([("d_prob", (b, a, s, s), torch.float32)])
+    assert not layer.fused_attention(ctx)
+    layer._attention_fwd(st, ctx)
+    d_qkv = torch.empty_like(qkv)
+    layer._attention_bwd(d_ctx, d_qkv, st, ctx)
+    torch.cuda.synchronize()
+    # fp64 autograd on the CPU
+    x = qkv.double().cpu().requires_grad_(True)
+    qq, kk, vv = [x[:, i * h:(i + 1) * h].view(b, s, a, d).transpose(1, 2) for i in range(3)]
+    scores = qq @ kk.transpose(-2, -1) / math.sqrt(d)
+    if mask == "causal":
+        keep_ = torch.tril(torch.ones(s, s, dtype=torch.bool)).view(1, 1, s, s)
+    else:
+        keep_ = torch.arange(s).view(1, 1, 1, s) < lens.cpu().view(b, 1, 1, 1)
+    prob = torch.softmax(scores.masked_fill(~keep_, -1e9), dim=-1)
+    out = (prob @ vv).transpose(1, 2).reshape(b * s, h)
+    out.backward(d_ctx.double().cpu())
+    err = lambda got, want: float((got.double().cpu() - want).abs().max() / want.abs().max())
+    assert err(st["prob"], prob.detach()) < 1e-5
+    assert err(st["ctx"], out.detach()) < 1e-5
+    for i, name in enumerate("qkv"):
+        assert err(d_qkv[:, i * h:(i + 1) * h], x.grad[:, i * h:(i + 1) * h]) < 1e-4, f"d{name}"

@@ -42,9 +42,9 @@ def build(hidden, heads, ffn, layers_per_stage, stages, stage_id, mb, M, seq, dt
                               grad_mode=grad_mode, device=DEV, key_len_range=key_len_range)
     cfg = {"train_micro_batch_size_per_gpu": mb, "gradient_accumulation_steps": M,
            "optimizer": {"type": "Adam", "params": {"lr": 1e-3}}, "bf16": {"enabled": dtype == torch.bfloat16}}
+    engine_kwargs.setdefault("install_signal_handler", False)
     engine, _, _, _ = bamboo_amd.initialize(model=model, config=cfg, redundancy_level=rl, eager_recovery=eager,
-                                            activation_queue=q, rc_stream=rc_stream, install_signal_handler=False,
-                                            **engine_kwargs)
+                                            activation_queue=q, rc_stream=rc_stream, **engine_kwargs)
     return engine, q
 
 
@@ -85,6 +85,51 @@ def relu_decisions(engine, stage_ids, M, mb):
     return out
 
 
+class ReluHandover:
+    """Guard of the hand-over of the GPU's ReLU decisions to the oracle (bf16 ReLU layers and bottleneck blocks).
+
+    The masked oracle run measures the kernels' arithmetic at the 2e-2 bar, but would also follow a kernel that
+    zeroed (or passed) activations it should not.  So every ReLU evaluated with handed-in decisions is audited
+    (``oracle.layers.RELU_AUDIT``): the decisions may differ from the oracle's own ``u > 0`` on under 1 % of the
+    elements, and only where the oracle's |u| is below 2e-2 of the tensor's largest |u|: a decision can flip only
+    where the low-precision pre-activation is off by more than |u|, and 2e-2 of the tensor's scale is the largest
+    element-wise error the bf16 bar grants any tensor (bf16 storage of the operands upstream: 8 bits of mantissa,
+    2^-9 relative per stored value, a few stored values deep, amplified by 1/sigma in a BatchNorm).  For scale: a
+    ReLU that decided at random would differ on half of the elements, one that was off by a tenth of the tensor's
+    spread on a few per cent, with |u| up to that tenth.  And a second oracle run that makes its OWN decisions must
+    still agree with the GPU at the looser bars ``LOOSE_ACT`` / ``LOOSE_GRAD`` (a flipped decision moves an
+    activation by less than its rounding error, but switches that element's gradient on or off)."""
+
+    def __init__(self, st, peer):
+        import copy
+        self.own_st, self.own_peer = copy.deepcopy(st), copy.deepcopy(peer)      # before any run: clean gradients
+        ol.RELU_AUDIT = self.audit = []
+
+    def check(self, max_fraction=0.01, max_rel=2e-2):
+        ol.RELU_AUDIT = None
+        assert self.audit, "no ReLU was evaluated with handed-in decisions"
+        total, differ = sum(a[0] for a in self.audit), sum(a[1] for a in self.audit)
+        assert differ < max_fraction * total, (differ, total)
+        for numel, n_diff, worst, top in self.audit:
+            assert n_diff < max_fraction * numel, (n_diff, numel)
+            assert worst <= max_rel * top, (worst, top, n_diff, numel)
+        print(f"relu hand-over: {differ} of {total} decisions differ ({100.0 * differ / total:.3f} %), largest |u| among "
+              f"them {max(a[2] / a[3] for a in self.audit):.5f} of its tensor's largest")
+        return differ / total
+
+    def own_run(self):
+        """The oracle with its own decisions: (buffers, info, stage)."""
+        assert not self.own_peer.relu_masks
+        bufs, info = self.own_st.run_batch(self.own_peer, optimizer_step=False)
+        return bufs, info, self.own_st
+
+
+def max_err(got, ref):
+    """Largest element-wise error over the reference's largest magnitude."""
+    got, ref = got.double().cpu(), ref.double().cpu()
+    return float((got - ref).abs().max() / ref.abs().max().clamp_min(1e-30))
+
+
 def snapshot_grads(engine, sid):
     return {k: v.clone() for k, v in engine.module.get_named_grad(sid)}
 
@@ -107,6 +152,12 @@ class NoStep:
 
 
 REFERENCE_VARIANT = dict(activation="relu", ln="annotated", mask="none")
+# bars of the comparison with an oracle that makes its own ReLU decisions (see ReluHandover): activations stay at the
+# bf16 bar; gradients get room for the elements whose decision differs -- 0.1-0.26 % of the decisions per ReLU, each
+# switching a whole gradient element on or off, six ReLUs deep in a two-block stage and spread over the batch by the
+# BatchNorm backward: relative L2 up to sqrt(6 x 0.0025) = 0.12 (measured 0.10-0.11 on the bottleneck stages, 0.03
+# on the transformer's single ReLU per layer)
+LOOSE_ACT, LOOSE_GRAD = 2e-2, 2e-1
 GPT_VARIANT = dict(activation="gelu_tanh", ln="standard", mask="causal")
 BERT_VARIANT = dict(activation="gelu_tanh", ln="standard", mask="key_padding")
 
@@ -130,7 +181,10 @@ def test_stage_matches_oracle_with_rc(hiplib, variant, klr, dtype):
         # ReLU'(u) is discontinuous: the ~0.2 % of pre-activations closer to zero than their bf16 rounding
         # error would take the other branch in an fp64 run.  The oracle is handed the decisions the GPU made,
         # so that the 2e-2 below measures the kernels' arithmetic
+        handover = ReluHandover(st, peer)
         peer.relu_masks = relu_decisions(engine, [sid, sid + 1], M, mb)
+    else:
+        handover = None
     bufs, _ = st.run_batch(peer, optimizer_step=False)
     t_act = 1e-5 if dtype == torch.float32 else 2e-2
     t_grad = 1e-4 if dtype == torch.float32 else 2e-2
@@ -139,9 +193,21 @@ def test_stage_matches_oracle_with_rc(hiplib, variant, klr, dtype):
         assert rel_err(keep[f"output_{sid}"][k], bufs["out"][(sid, k)].detach().view(mb * seq, hid)) < t_act
         assert rel_err(keep[f"output_{sid + 1}"][k], bufs["out"][(sid + 1, k)].detach().view(mb * seq, hid)) < t_act
         assert rel_err(keep[f"input_grad_{sid}"][k], bufs["sent_grad"][(sid, k)].view(mb * seq, hid)) < t_grad
+        if dtype == torch.bfloat16:     # beside the L2 bars: no single element off by more than 5e-2 of the tensor's scale
+            assert max_err(keep[f"output_{sid}"][k], bufs["out"][(sid, k)].detach().view(mb * seq, hid)) < 5e-2
+            assert max_err(keep[f"output_{sid + 1}"][k], bufs["out"][(sid + 1, k)].detach().view(mb * seq, hid)) < 5e-2
     ref_grads = st.named_grads(sid)
     for name, g in engine.module.get_named_grad(sid):
         assert rel_err(g, ref_grads[name], grad_floor(ref_grads)) < t_grad, name
+    if handover is not None:
+        handover.check()
+        own_bufs, _, own_st = handover.own_run()
+        for k in range(M):
+            assert rel_err(keep[f"output_{sid}"][k], own_bufs["out"][(sid, k)].detach().view(mb * seq, hid)) < LOOSE_ACT
+            assert rel_err(keep[f"input_grad_{sid}"][k], own_bufs["sent_grad"][(sid, k)].view(mb * seq, hid)) < LOOSE_GRAD
+        own_grads = own_st.named_grads(sid)
+        for name, g in engine.module.get_named_grad(sid):
+            assert rel_err(g, own_grads[name], grad_floor(own_grads)) < LOOSE_GRAD, name
     # shadow parameters receive no gradient from redundant forwards
     for name, g in engine.module.get_named_grad(sid + 1):
         assert float(g.abs().max()) == 0.0
@@ -326,20 +392,32 @@ def test_resnet_stage_matches_oracle_with_rc(hiplib, dtype, cin, cmid):
     if dtype == torch.bfloat16:
         # every block has three ReLUs; the oracle takes the decisions the GPU made at each of them (see the
         # transformer ReLU case), so the bf16 bar stays at 2e-2
+        handover = ReluHandover(st, peer)
         peer.relu_masks = relu_decisions(engine, [sid, sid + 1], M, mb)
     bufs, _ = st.run_batch(peer, optimizer_step=False)
     t_act = 1e-5 if dtype == torch.float32 else 2e-2
     t_grad = 1e-4 if dtype == torch.float32 else 2e-2
-    for k in range(M):
-        assert rel_err(keep[f"output_{sid}"][k], bufs["out"][(sid, k)].detach().reshape(mb * side * side, cin)) < t_act
-        assert rel_err(keep[f"output_{sid + 1}"][k], bufs["out"][(sid + 1, k)].detach().reshape(mb * side * side, cin)) < t_act
-        assert rel_err(keep[f"input_grad_{sid}"][k], bufs["sent_grad"][(sid, k)].reshape(mb * side * side, cin)) < t_grad
-    ref = st.named_grads(sid)
-    for name, g in engine.module.get_named_grad(sid):
-        r = ref[name]
-        if r.dim() == 4:
-            r = r.permute(0, 2, 3, 1)
-        assert rel_err(g, r.reshape(g.shape), grad_floor(ref)) < t_grad, name
+    rows = mb * side * side
+
+    def compare(bufs, stage, t_act, t_grad, elementwise):
+        for k in range(M):
+            assert rel_err(keep[f"output_{sid}"][k], bufs["out"][(sid, k)].detach().reshape(rows, cin)) < t_act
+            assert rel_err(keep[f"output_{sid + 1}"][k], bufs["out"][(sid + 1, k)].detach().reshape(rows, cin)) < t_act
+            assert rel_err(keep[f"input_grad_{sid}"][k], bufs["sent_grad"][(sid, k)].reshape(rows, cin)) < t_grad
+            if elementwise:
+                assert max_err(keep[f"output_{sid}"][k], bufs["out"][(sid, k)].detach().reshape(rows, cin)) < 5e-2
+                assert max_err(keep[f"output_{sid + 1}"][k], bufs["out"][(sid + 1, k)].detach().reshape(rows, cin)) < 5e-2
+        ref = stage.named_grads(sid)
+        for name, g in engine.module.get_named_grad(sid):
+            r = ref[name]
+            if r.dim() == 4:
+                r = r.permute(0, 2, 3, 1)
+            assert rel_err(g, r.reshape(g.shape), grad_floor(ref)) < t_grad, name
+    compare(bufs, st, t_act, t_grad, dtype == torch.bfloat16)
+    if dtype == torch.bfloat16:
+        handover.check()
+        own_bufs, _, own_st = handover.own_run()
+        compare(own_bufs, own_st, LOOSE_ACT, LOOSE_GRAD, False)
     # redundant forwards left the shadow blocks' running statistics alone; own blocks updated theirs M times
     for layer in engine.module.func_buckets[sid + 1]:
         assert layer.running is None
@@ -407,25 +485,36 @@ def test_resnet_stage_with_projection_shortcuts_matches_oracle(hiplib, dtype, ne
         engine.train_batch()
     torch.cuda.synchronize()
     if dtype == torch.bfloat16:
+        handover = ReluHandover(st, peer)
         peer.relu_masks = relu_decisions(engine, [sid, sid + 1], M, mb)
     bufs, info = st.run_batch(peer, optimizer_step=False)
     assert (info["failed_step"] is not None) == (dead_from is not None)
     assert engine.stage_ids == ([sid, sid + 1] if dead_from is not None else [sid])
     t_act = 1e-5 if dtype == torch.float32 else 2e-2
     t_grad = 1e-4 if dtype == torch.float32 else 2e-2
-    for k in range(M):
-        for s_ in (sid, sid + 1):
-            want = bufs["out"][(s_, k)].detach()
-            assert rel_err(keep[f"output_{s_}"][k], want.reshape(-1, want.shape[-1])) < t_act, (s_, k)
-        want = bufs["sent_grad"][(sid, k)]
-        assert rel_err(keep[f"input_grad_{sid}"][k], want.reshape(-1, want.shape[-1])) < t_grad, k
-    for s_ in engine.stage_ids:
-        ref = st.named_grads(s_)
-        for name, g in engine.module.get_named_grad(s_):
-            r = ref[name]
-            if r.dim() == 4:
-                r = r.permute(0, 2, 3, 1)
-            assert rel_err(g, r.reshape(g.shape), grad_floor(ref)) < t_grad, (s_, name)
+
+    def compare(bufs, stage, t_act, t_grad, elementwise):
+        for k in range(M):
+            for s_ in (sid, sid + 1):
+                want = bufs["out"][(s_, k)].detach()
+                assert rel_err(keep[f"output_{s_}"][k], want.reshape(-1, want.shape[-1])) < t_act, (s_, k)
+                if elementwise:
+                    assert max_err(keep[f"output_{s_}"][k], want.reshape(-1, want.shape[-1])) < 5e-2, (s_, k)
+            want = bufs["sent_grad"][(sid, k)]
+            assert rel_err(keep[f"input_grad_{sid}"][k], want.reshape(-1, want.shape[-1])) < t_grad, k
+        for s_ in engine.stage_ids:
+            ref = stage.named_grads(s_)
+            for name, g in engine.module.get_named_grad(s_):
+                r = ref[name]
+                if r.dim() == 4:
+                    r = r.permute(0, 2, 3, 1)
+                assert rel_err(g, r.reshape(g.shape), grad_floor(ref)) < t_grad, (s_, name)
+    compare(bufs, st, t_act, t_grad, dtype == torch.bfloat16)
+    if dtype == torch.bfloat16:
+        handover.check()
+        own_bufs, own_info, own_st = handover.own_run()
+        assert (own_info["failed_step"] is not None) == (dead_from is not None)
+        compare(own_bufs, own_st, LOOSE_ACT, LOOSE_GRAD, False)
     # the shortcut's BatchNorm keeps running statistics like the others
     own = engine.module.func_buckets[sid][0]
     assert float(own.running["shortcut"][0].abs().max()) > 0
@@ -784,3 +873,33 @@ def test_engine_surface(hiplib):
     loss = engine.train_batch()
     assert loss.shape == (1,) and engine.global_steps == 1
     assert all(b is None for b in engine.pipe_buffers[f"output_{sid}"])
+
+
+def test_sigterm_and_launch_observer_belong_to_one_engine(hiplib):
+    """SIGTERM (the preemption notice) stops the engine that installed the handler at its next batch with exit code
+    13 (reference engine.py:98-111, 1096-1097) and leaves another engine of the process alone; a GEMM launch observer
+    set on one engine sees that engine's launches only and does not switch the other's graph replay off."""
+    import os
+    import signal
+    hid, heads, ffn, L, S, sid, mb, M, seq = 128, 2, 256, 1, 4, 1, 2, 4, 64
+    prev = signal.getsignal(signal.SIGTERM)
+    try:
+        a, _ = build(hid, heads, ffn, L, S, sid, mb, M, seq, torch.bfloat16, GPT_VARIANT, 1, True, install_signal_handler=True)
+        b, _ = build(hid, heads, ffn, L, S, sid, mb, M, seq, torch.bfloat16, GPT_VARIANT, 1, True)
+        seen = []
+        a.set_gemm_hook(lambda desc, launch, stream: (seen.append(desc), launch()))
+        b.train_batch()
+        assert not seen
+        a.train_batch()
+        # per layer and micro-batch: own forward and redundant forward 4 products each, own backward 4 input
+        # gradients and the grouped weight-gradient launch
+        assert len(seen) == M * L * (4 + 4 + 5)
+        a.set_gemm_hook(None)
+        os.kill(os.getpid(), signal.SIGTERM)
+        assert a.should_stop and not b.should_stop
+        b.train_batch()
+        with pytest.raises(SystemExit) as e:
+            a.train_batch()
+        assert e.value.code == 13
+    finally:
+        signal.signal(signal.SIGTERM, prev)
