@@ -389,11 +389,17 @@ class PipelineEngine:
             # it, so the replay keeps the successor's sends (the second replay case of the
             # reference, schedule.py:349-353)
             failed_step = 0
+        # micro-batches whose own forward has run but whose redundant forward has not (held back for a bubble, issued
+        # in part, or simply not due yet where the schedule places it): the replay computes these first
+        own_out, rc_out = self.pipe_buffers[f"output_{self.stage_id}"], self.pipe_buffers.get(f"output_{nxt}", [])
+        partial = self._rc_partial[0] if self._rc_partial is not None else None
+        missing = sum(1 for k, o in enumerate(own_out)
+                      if o is not None and (k >= len(rc_out) or rc_out[k] is None or k == partial))
         self._promote(nxt, failed_step=failed_step, curr_step=step_i)
         if hasattr(self.queue, "adopt"):
             self.queue.adopt(nxt)
         self.last_failover = {"step": step_i, "failed_step": failed_step, "t_detect": t0,
-                              "promote_s": time.perf_counter() - t0}
+                              "promote_s": time.perf_counter() - t0, "rc_missing": missing}
         self._replay_until = step_i
 
     def _handle_prev_stage_failure(self, step_i):

@@ -58,13 +58,17 @@ def measured_traffic_bytes(config, kernel):
     return None
 
 
-def build_engine(cfg, rc, rc_stream, seed=1138, use_graphs=False, paced=None, rc_issue="reference", eager=True):
+def build_engine(cfg, rc, rc_stream, seed=1138, use_graphs=False, paced=None, rc_issue="reference", eager=True,
+                 stage_id=STAGE_ID):
     """``paced=(t_fwd, t_bwd)``: the neighbours are a closed-loop model of the other stages of a 1F1B pipeline whose
-    forward / backward passes take that long, so the stage waits for its inputs as in a real pipeline."""
+    forward / backward passes take that long, so the stage waits for its inputs as in a real pipeline.
+    ``stage_id``: which stage of the ``STAGES`` is the real one (all stages have the same layers)."""
+    import itertools
+
     import torch
 
     import bamboo_amd
-    from bamboo_amd import BottleNeck, LayerSpec, PipelineModule, SeededActivationQueue, TransformerLayer
+    from bamboo_amd import BottleNeck, LayerSpec, MSELoss, PipelineModule, SeededActivationQueue, TransformerLayer
     from bamboo_amd.p2p import PacedActivationQueue
     dtype = torch.bfloat16 if cfg["dtype"] == "bf16" else torch.float32
     if cfg.get("kind") == "resnet":
@@ -74,12 +78,14 @@ def build_engine(cfg, rc, rc_stream, seed=1138, use_graphs=False, paced=None, rc
         specs = [LayerSpec(TransformerLayer, cfg["hidden"], cfg["heads"], cfg["ffn"], dropout=cfg.get("dropout", 0.0),
                            **cfg["variant"])
                  for _ in range(cfg["layers"] * STAGES)]
-    model = PipelineModule(specs, num_stages=STAGES, partition_method="uniform", stage_id=STAGE_ID, dtype=dtype,
-                           device="cuda:0")
-    qargs = dict(stage_ids=[STAGE_ID, STAGE_ID + 1], seed=seed, grad_mode=cfg["grad_mode"], device="cuda:0",
+    # a stage that shadows the last one must be able to run it after a failover: the last stage carries the loss
+    loss_fn = MSELoss() if stage_id + 1 == STAGES - 1 else None
+    model = PipelineModule(specs, num_stages=STAGES, partition_method="uniform", stage_id=stage_id, dtype=dtype,
+                           device="cuda:0", loss_fn=loss_fn)
+    qargs = dict(stage_ids=[stage_id, stage_id + 1], seed=seed, grad_mode=cfg["grad_mode"], device="cuda:0",
                  key_len_range=cfg.get("key_len_range"))
     if paced is not None:
-        q = PacedActivationQueue((cfg["mb"], cfg["seq"], cfg["hidden"]), dtype, cfg["M"], stages=STAGES, stage_id=STAGE_ID,
+        q = PacedActivationQueue((cfg["mb"], cfg["seq"], cfg["hidden"]), dtype, cfg["M"], stages=STAGES, stage_id=stage_id,
                                  t_fwd=paced[0], t_bwd=paced[1], **qargs)
     else:
         q = SeededActivationQueue((cfg["mb"], cfg["seq"], cfg["hidden"]), dtype, cfg["M"], **qargs)
@@ -89,6 +95,10 @@ def build_engine(cfg, rc, rc_stream, seed=1138, use_graphs=False, paced=None, rc
     engine, _, _, _ = bamboo_amd.initialize(model=model, config=ds, redundancy_level=1 if rc else 0,
                                             eager_recovery=rc and eager, activation_queue=q, rc_stream=rc_stream,
                                             install_signal_handler=False, use_graphs=use_graphs, rc_issue=rc_issue)
+    if stage_id == 0 or stage_id + 1 == STAGES - 1:
+        # the first stage loads its input itself (LoadMicroBatch), and a stage that shadows the last one loads that
+        # stage's labels: both come from the resident seeded tensors, micro-batch k of every batch the same
+        engine.set_dataiterator(itertools.cycle([(a, a) for a in q.activations]))
     return engine, q
 
 
@@ -159,14 +169,29 @@ def paced_timeline(q, t_start):
     return "\n".join(lines)
 
 
-def paced_leg(cfg, rc, rc_issue, t_fwd, t_bwd, steps, warmup, timeline=None):
+def own_pass_means(q):
+    """Mean GPU duration (seconds) of the real stage's forward and backward passes in the batch the queue's clock
+    holds: a pass runs from the later of its input's arrival and the previous pass's end to its own end, so time
+    it shared with redundant work on the other stream is in it."""
+    c, sid = q.clock, q.stage_id
+    durs, prev = {"F": [], "B": []}, c.t0
+    for kind, k in c.order[sid]:
+        arrive = c.activation_at(k) if kind == "F" else c.grad_at(k)
+        end = c.end_of(sid, kind, k)
+        durs[kind].append(end - max(arrive, prev))
+        prev = end
+    return sum(durs["F"]) / len(durs["F"]), sum(durs["B"]) / len(durs["B"])
+
+
+def paced_leg(cfg, rc, rc_issue, t_fwd, t_bwd, steps, warmup, timeline=None, stage_id=STAGE_ID):
     """Batch time (seconds, mean of ``steps`` batches) of the stage inside the closed-loop pipeline model, graphs on
     (one launch per pass: the host never holds the GPU back after a receive has returned)."""
     import torch
     work = torch.cuda.Stream()
     work.wait_stream(torch.cuda.current_stream())
     with torch.cuda.stream(work):
-        engine, q = build_engine(cfg, rc=rc, rc_stream=rc, use_graphs=True, paced=(t_fwd, t_bwd), rc_issue=rc_issue)
+        engine, q = build_engine(cfg, rc=rc, rc_stream=rc, use_graphs=True, paced=(t_fwd, t_bwd), rc_issue=rc_issue,
+                                 stage_id=stage_id)
         for _ in range(max(warmup, 3)):      # eager batch, capturing batch, first replay
             engine.train_batch()
         q.reset()
@@ -179,6 +204,7 @@ def paced_leg(cfg, rc, rc_issue, t_fwd, t_bwd, steps, warmup, timeline=None):
             waits.append(q.waited)
             per_batch.append(q.batch_seconds)
         total = q.finish()
+        own_f, own_b = own_pass_means(q)
         if timeline is not None:
             with open(timeline, "w") as f:
                 f.write(paced_timeline(q, t_start) + "\n")
@@ -186,7 +212,58 @@ def paced_leg(cfg, rc, rc_issue, t_fwd, t_bwd, steps, warmup, timeline=None):
     gc.collect()
     torch.cuda.empty_cache()
     mean = lambda v: sum(v) / len(v)
-    return {"batch_s": total / steps, "host_wait_s": mean(waits), "first_batch_s": per_batch[0], "later_batches_s": mean(per_batch[1:] or per_batch)}
+    return {"batch_s": total / steps, "host_wait_s": mean(waits), "first_batch_s": per_batch[0],
+            "later_batches_s": mean(per_batch[1:] or per_batch), "own_fwd_s": own_f, "own_bwd_s": own_b}
+
+
+def paced_failure(cfg, rc_issue, t_fwd, t_bwd, at, stage_id):
+    """The successor is lost at micro-batch ``at`` of a batch inside the pipeline model, redundant forwards issued
+    as ``rc_issue`` says: how many shadow stashes the promoted stage finds missing (redundant forwards still held
+    back, or issued in part) and has to compute first, and the pause (failure detected with the GPU drained ->
+    the lost stage's work up to that point replayed)."""
+    import torch
+    engine, q = build_engine(cfg, rc=True, rc_stream=True, paced=(t_fwd, t_bwd), rc_issue=rc_issue, stage_id=stage_id)
+    for _ in range(2):
+        engine.train_batch()
+    q.preempt_successor(at, stage_id)
+    engine.train_batch()
+    torch.cuda.synchronize()
+    fo = engine.last_failover
+    out = {"shadow_stashes_missing": fo["rc_missing"], "pause_ms": round(fo["pause_s"] * 1e3, 3),
+           "detected_at_step": fo["step"]}
+    del engine, q
+    gc.collect()
+    torch.cuda.empty_cache()
+    return out
+
+
+def paced_per_stage(cfg, t_fwd, t_bwd, steps, warmup, fail_at, known=None):
+    """RC overhead inside the pipeline model with stage 0, 1, 2, ... of ``STAGES`` as the real one (the last stage
+    shadows nobody in this build: redundancy ids are not wrapped round to stage 0's layers on another device).
+    Every Bamboo stage runs redundant forwards, so for the RC-on legs the modelled neighbours get the pass times
+    the real stage's own passes measure WITH its redundant work beside them (second leg, fed from the first);
+    the RC-off leg uses the plain pass times for everybody.  The pipeline's figure is the worst stage's."""
+    stages = {}
+    for sid in range(STAGES - 1):
+        off = (known or {}).get((sid, "off")) or paced_leg(cfg, False, "reference", t_fwd, t_bwd, steps, warmup, stage_id=sid)
+        on1 = (known or {}).get((sid, "bubble")) or paced_leg(cfg, True, "bubble", t_fwd, t_bwd, steps, warmup, stage_id=sid)
+        on2 = paced_leg(cfg, True, "bubble", on1["own_fwd_s"], on1["own_bwd_s"], steps, warmup, stage_id=sid)
+        pct = lambda leg: round(100.0 * (leg["batch_s"] - off["batch_s"]) / off["batch_s"], 2)
+        stages[str(sid)] = {
+            "rc_off_batch_ms": round(off["batch_s"] * 1e3, 3),
+            "rc_on_batch_ms_neighbours_plain": round(on1["batch_s"] * 1e3, 3),
+            "rc_on_batch_ms_neighbours_with_rc": round(on2["batch_s"] * 1e3, 3),
+            "own_pass_ms_with_rc": [round(on1["own_fwd_s"] * 1e3, 3), round(on1["own_bwd_s"] * 1e3, 3)],
+            "rc_overhead_paced_pct_neighbours_plain": pct(on1),
+            "rc_overhead_paced_pct": pct(on2),
+            "failure_at_micro_batch": fail_at,
+            "failure_bubble": paced_failure(cfg, "bubble", t_fwd, t_bwd, fail_at, sid),
+            "failure_reference": paced_failure(cfg, "reference", t_fwd, t_bwd, fail_at, sid)}
+    worst = max(stages, key=lambda k: stages[k]["rc_overhead_paced_pct"])
+    return {"rc_issue": "bubble", "stages": stages, "pipeline_rc_overhead_paced_pct": stages[worst]["rc_overhead_paced_pct"],
+            "worst_stage": int(worst),
+            "note": "neighbours' passes in the RC-on figure take the real stage's mean pass times measured with its "
+                    "redundant forwards beside them; pipeline figure = worst stage"}
 
 
 def time_steps(engine, steps, warmup):
@@ -310,6 +387,107 @@ def cpu_baseline(cfg, threads):
                       f"mean extrapolated x{M} micro-batches; optimizer step not included"}
 
 
+def failover_legs(cfg, engine, q, at, steps, warmup):
+    """The successor is preempted at micro-batch ``at`` (reference path: the NextStageException branch of
+    train_batch, engine.py:1190-1264).  ``engine`` has run warm-up and timed batches with redundant forwards (eager
+    recovery); afterwards the same failure in lazy recovery (host mirrors of the shadow parameters, nothing computed
+    ahead: promotion materialises the layers and the replay recomputes the successor's forwards)."""
+    import torch
+    samples = cfg["mb"] * cfg["M"]
+    q.preempt_successor(at, STAGE_ID)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    engine.train_batch()
+    torch.cuda.synchronize()
+    t_fail_batch = time.perf_counter() - t0
+    q.revive()
+    t_post = time_steps(engine, steps, 1)       # merged own+promoted stream from step 0
+    fo = engine.last_failover
+    failover = {"preempted_at_micro_batch": at, "detected_at_step": fo["step"],
+                "promote_ms": round(fo["promote_s"] * 1e3, 3), "pause_ms": round(fo["pause_s"] * 1e3, 3),
+                "shadow_stashes_missing": fo["rc_missing"],
+                "failover_batch_ms": round(t_fail_batch * 1e3, 3),
+                "post_failover_samples_per_s": round(samples / t_post, 3),
+                "post_failover_ms_per_step": round(t_post * 1e3, 3),
+                "note": "pause = failure detected (GPU drained) -> successor's lost work replayed from the RC stash; "
+                        "post-failover = own + promoted layers as two local stages"}
+    del engine, q
+    gc.collect()
+    torch.cuda.empty_cache()
+    engine, q = build_engine(cfg, rc=True, rc_stream=False, eager=False)
+    t_lazy = time_steps(engine, steps, warmup)
+    q.preempt_successor(at, STAGE_ID)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    engine.train_batch()
+    torch.cuda.synchronize()
+    t_fail_lazy = time.perf_counter() - t0
+    q.revive()
+    fo = engine.last_failover
+    failover["lazy"] = {"samples_per_s_before": round(samples / t_lazy, 3), "promote_ms": round(fo["promote_s"] * 1e3, 3),
+                        "pause_ms": round(fo["pause_s"] * 1e3, 3), "failover_batch_ms": round(t_fail_lazy * 1e3, 3),
+                        "note": "redundancy_level=1 without eager recovery: no RC overhead before the failure, the "
+                                "pause pays for building the layers from host mirrors and for the lost forwards"}
+    del engine, q
+    gc.collect()
+    torch.cuda.empty_cache()
+    return failover
+
+
+def dominant_gemm(probe, dtype):
+    """(name, launches, flops, seconds, all variants) of the GEMM variant with the largest total time."""
+    overhead_s = probe.bracket_overhead()
+    agg = probe.summary(overhead_s)
+    name, (count, flops, secs) = max(agg.items(), key=lambda kv: kv[1][2])
+    return name, count, flops, secs, agg, overhead_s
+
+
+def quick_config(name, steps, warmup, failover_at=None, dropout=None):
+    """A bounded run of another configuration with the same code: RC off, RC on (second stream), the dominant GEMM
+    variant's rate from event brackets on a single-stream RC-on leg, optionally the failover figures."""
+    import torch
+    cfg = CONFIGS[name]
+    if dropout:
+        cfg = dict(cfg, dropout=dropout)
+    samples = cfg["mb"] * cfg["M"]
+    peak = PEAK_BF16_TFLOPS if cfg["dtype"] == "bf16" else PEAK_F32_TFLOPS
+
+    def drop(engine, q):
+        del engine, q
+        gc.collect()
+        torch.cuda.empty_cache()
+    engine, q = build_engine(cfg, rc=False, rc_stream=False)
+    t_off = time_steps(engine, steps, warmup)
+    drop(engine, q)
+    out = {"workload": cfg["label"], "dtype": cfg["dtype"], "steps": steps, "warmup": warmup, "samples_per_step": samples,
+           "dropout": cfg.get("dropout", 0.0)}
+    if dropout is None:
+        engine, q = build_engine(cfg, rc=True, rc_stream=False)
+        for _ in range(warmup):
+            engine.train_batch()
+        probe = GemmProbe()
+        engine.set_gemm_hook(probe)
+        for _ in range(steps):
+            engine.train_batch()
+        torch.cuda.synchronize()
+        engine.set_gemm_hook(None)
+        drop(engine, q)
+        kname, count, flops, secs, _, _ = dominant_gemm(probe, cfg["dtype"])
+        out["dominant_kernel"] = {"kernel": f"gemm_{kname}", "launches": count, "avg_launch_us": round(secs / count * 1e6, 2),
+                                  "achieved_tflops": round(flops / secs / 1e12, 2), "peak_tflops": peak,
+                                  "frac": round(flops / secs / 1e12 / peak, 4)}
+    engine, q = build_engine(cfg, rc=True, rc_stream=True)
+    t_on = time_steps(engine, steps, warmup)
+    out.update({"rc_on_samples_per_s": round(samples / t_on, 3), "rc_off_samples_per_s": round(samples / t_off, 3),
+                "rc_overhead_pct": round(100.0 * (t_on - t_off) / t_off, 2), "ms_per_step_rc_on": round(t_on * 1e3, 3)})
+    if failover_at is not None:
+        out["failover"] = failover_legs(cfg, engine, q, failover_at, steps, warmup)
+        engine = q = None
+    else:
+        drop(engine, q)
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -340,6 +518,10 @@ def main():
                     help="write the last batch of the paced 'bubble' leg as a table: own passes and pieces of redundant work")
     ap.add_argument("--failover-at", type=int, default=None,
                     help="also measure a failover: the successor is preempted at this micro-batch (config c5: 7)")
+    ap.add_argument("--no-other-configs", action="store_true",
+                    help="only the configuration --config names: leave out the bounded runs of the other configurations "
+                         "(3 batches each; GPT-2-1.5B with a failover at micro-batch 7), the per-stage legs of the "
+                         "pipeline model and the dropout 0.1 rates that the default run appends")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures ONE pipeline stage on ONE GPU; --gpus N>1 is not part of this build", file=sys.stderr)
@@ -416,59 +598,25 @@ def main():
         engine, q = build_engine(cfg, rc=True, rc_stream=True, use_graphs=graphs)
         t_on = time_steps(engine, args.steps, args.warmup)
 
+    n_graphs = sum(1 for v in engine._graphs.values() if isinstance(v, tuple))
+    fwd_flops_layer = engine.module.func_buckets[STAGE_ID][0].flops_fwd(cfg["mb"], cfg["seq"])
     failover = None
     if args.failover_at is not None:
-        # the engine of the last leg has run warm-up + timed batches with RC; now lose the successor
-        q.preempt_successor(args.failover_at, STAGE_ID)
-        torch.cuda.synchronize()
-        t0 = time.perf_counter()
-        engine.train_batch()
-        torch.cuda.synchronize()
-        t_fail_batch = time.perf_counter() - t0
-        q.revive()
-        t_post = time_steps(engine, args.steps, 1)       # merged own+promoted stream from step 0
-        fo = engine.last_failover
-        failover = {"preempted_at_micro_batch": args.failover_at, "detected_at_step": fo["step"],
-                    "promote_ms": round(fo["promote_s"] * 1e3, 3), "pause_ms": round(fo["pause_s"] * 1e3, 3),
-                    "failover_batch_ms": round(t_fail_batch * 1e3, 3),
-                    "post_failover_samples_per_s": round(samples / t_post, 3),
-                    "post_failover_ms_per_step": round(t_post * 1e3, 3),
-                    "note": "pause = failure detected (GPU drained) -> successor's lost work replayed from the RC stash; "
-                            "post-failover = own + promoted layers as two local stages"}
-        # the same failure without redundant forwards (lazy recovery: host mirrors of the shadow parameters, nothing
-        # computed ahead): promotion materialises the layers and the replay recomputes the successor's forwards
-        del engine, q
-        gc.collect()
-        torch.cuda.empty_cache()
-        engine, q = build_engine(cfg, rc=True, rc_stream=False, eager=False)
-        t_lazy = time_steps(engine, args.steps, args.warmup)
-        q.preempt_successor(args.failover_at, STAGE_ID)
-        torch.cuda.synchronize()
-        t0 = time.perf_counter()
-        engine.train_batch()
-        torch.cuda.synchronize()
-        t_fail_lazy = time.perf_counter() - t0
-        q.revive()
-        fo = engine.last_failover
-        failover["lazy"] = {"samples_per_s_before": round(samples / t_lazy, 3), "promote_ms": round(fo["promote_s"] * 1e3, 3),
-                            "pause_ms": round(fo["pause_s"] * 1e3, 3), "failover_batch_ms": round(t_fail_lazy * 1e3, 3),
-                            "note": "redundancy_level=1 without eager recovery: no RC overhead before the failure, the "
-                                    "pause pays for building the layers from host mirrors and for the lost forwards"}
+        failover = failover_legs(cfg, engine, q, args.failover_at, args.steps, args.warmup)
+    engine = q = None
+    gc.collect()
+    torch.cuda.empty_cache()
 
-    n_graphs = sum(1 for v in engine._graphs.values() if isinstance(v, tuple))
-    layer = engine.module.func_buckets[STAGE_ID][0]
-    fwd_flops = layer.flops_fwd(cfg["mb"], cfg["seq"]) * cfg["layers"]
+    fwd_flops = fwd_flops_layer * cfg["layers"]
     own_flops, rc_flops = 3 * fwd_flops * cfg["M"], fwd_flops * cfg["M"]
 
     roofline = None
     if probe is not None:
-        overhead_s = probe.bracket_overhead()
-        agg = probe.summary(overhead_s)
+        name, count, flops, secs, agg, overhead_s = dominant_gemm(probe, cfg["dtype"])
         if args.gemm_shapes:
-            for (name, shape), (n, fl, sec) in sorted(probe.by_shape().items(), key=lambda kv: -kv[1][2]):
-                print(f"{name:34s} {shape:40s} n={n:5d} {sec / n * 1e6:8.1f} us {fl / sec / 1e12:7.1f} TF {sec * 1e3:8.2f} ms",
+            for (vname, shape), (n, fl, sec) in sorted(probe.by_shape().items(), key=lambda kv: -kv[1][2]):
+                print(f"{vname:34s} {shape:40s} n={n:5d} {sec / n * 1e6:8.1f} us {fl / sec / 1e12:7.1f} TF {sec * 1e3:8.2f} ms",
                       file=sys.stderr)
-        name, (count, flops, secs) = max(agg.items(), key=lambda kv: kv[1][2])
         peak = PEAK_BF16_TFLOPS if cfg["dtype"] == "bf16" else PEAK_F32_TFLOPS
         achieved = flops / secs / 1e12
         roofline = {"bound": "mfma", "achieved": round(achieved, 2), "peak": peak, "unit": "TFLOP/s",
@@ -540,6 +688,19 @@ def main():
             "rc_on_samples_per_s": round(samples / legs[best]["batch_s"], 3)}
     if failover is not None:
         out["failover"] = failover
+    extras = not args.no_other_configs and args.config == "c2" and args.dropout == 0.0 and not args.script_layers
+    if extras and pass_times is not None:
+        # every stage of the pipeline runs redundant forwards: the pipeline's overhead is the worst stage's
+        known = {(STAGE_ID, "off"): off, (STAGE_ID, "bubble"): legs["bubble"]}
+        out["paced_per_stage"] = paced_per_stage(cfg, t_fwd, t_bwd, args.steps, args.warmup, fail_at=7, known=known)
+    if extras:
+        # the configuration the reference's scripts train with (dropout 0.1 at all four sites of a layer)
+        d = quick_config("c2", 3, 1, dropout=0.1)
+        out["dropout_0p1"] = {k: d[k] for k in ("rc_on_samples_per_s", "rc_off_samples_per_s", "rc_overhead_pct", "steps")}
+        other = {}
+        for name in ("c1", "c3", "c4", "c5"):
+            other[name] = quick_config(name, 3, 1, failover_at=7 if name == "c5" else None)
+        out["other_configs"] = other
     if not args.no_cpu_baseline:
         # all host cores this process may run on (the affinity mask is what the box really grants; os.cpu_count()
         # reports the machine's)
