@@ -2,7 +2,7 @@
 
 Batch triad ``train_batch_size = micro_batch * gradient_accumulation_steps * dp_world``
 as in ``deepspeed/runtime/config.py:862-932`` (any two determine the third; dp_world is 1
-here), ``optimizer{type, params{lr, betas, eps, weight_decay}}``, ``steps_per_print``,
+here), ``optimizer{type, params{lr, betas, eps, weight_decay}}``, ``gradient_clipping``, ``steps_per_print``,
 ``wall_clock_breakdown`` (``DeepSpeedExamples/pipeline_parallelism/transformer.json:1-17``).
 ``bf16.enabled`` selects bf16 compute with fp32 master weights (this build's analogue of the
 reference's fp16 wrapper, ``deepspeed/runtime/fp16/fused_optimizer.py:24-122``).
@@ -51,6 +51,11 @@ class BambooConfig:
         self.bias_correction = bool(p.get("bias_correction", True))
         # reference default: Adam type => adam_w_mode unless torch_adam (deepspeed/runtime/engine.py:985-1008)
         self.adam_w_mode = bool(p.get("adam_w_mode", True))
+        # clip the global gradient norm to this value before the optimizer step; 0 = off
+        # (deepspeed/runtime/config.py "gradient_clipping", used in _take_model_step, deepspeed/runtime/engine.py:1526-1531)
+        self.gradient_clipping = float(config.get("gradient_clipping", 0.0))
+        if self.gradient_clipping < 0:
+            raise ValueError("gradient_clipping must be >= 0")
         self.steps_per_print = int(config.get("steps_per_print", 10))
         self.wall_clock_breakdown = bool(config.get("wall_clock_breakdown", False))
         self.bf16 = bool(config.get("bf16", {}).get("enabled", False))

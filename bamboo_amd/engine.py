@@ -718,7 +718,13 @@ class PipelineEngine:
         return
 
     def _exec_optimizer_step(self):
-        self.optimizer.step(stream=self.main_stream)
+        if self.config.gradient_clipping > 0.0 and hasattr(self.optimizer, "clip_coef"):
+            # clip_fp32_gradients of the reference (deepspeed/runtime/engine.py:1521-1531): the norm and the
+            # coefficient stay on the device, the Adam kernel scales the gradients as it reads them
+            self.grad_norm = self.optimizer.clip_coef(self.config.gradient_clipping, stream=self.main_stream)
+            self.optimizer.step(stream=self.main_stream, grad_scale=self.grad_norm[1:])
+        else:
+            self.optimizer.step(stream=self.main_stream)
         if self.lr_scheduler is not None:
             self.lr_scheduler.step()
         self.global_steps += 1

@@ -26,7 +26,7 @@ EXPORTS = (
     "bb_version", "bb_last_error", "bb_init", "bb_gemm", "bb_gemm_grouped", "bb_gemm_splitk_workspace", "bb_gemm_grouped_splitk", "bb_gemm_variant", "bb_layernorm_fwd",
     "bb_layernorm_bwd_workspace", "bb_layernorm_bwd", "bb_layernorm_bwd_static", "bb_colsum_workspace", "bb_colsum_acc", "bb_rowsum_fwd", "bb_rowsum_bwd", "bb_dropout_apply", "bb_dropout_keep_host",
     "bb_softmax_fwd", "bb_softmax_bwd", "bb_attention_fwd", "bb_attention_bwd", "bb_residual_add", "bb_act_fwd", "bb_bn_workspace", "bb_batchnorm_fwd", "bb_batchnorm_bwd", "bb_patch3x3", "bb_patch3x3_strided", "bb_subsample", "bb_conv3x3_supported", "bb_conv3x3", "bb_gemm_strip_stats_supported", "bb_strip_stats_workspace", "bb_batchnorm_fwd_strips", "bb_mse_workspace", "bb_mse_fwd_bwd", "bb_graph_begin", "bb_graph_end", "bb_graph_launch", "bb_graph_destroy",
-    "bb_adam_multi", "bb_cast", "bb_fill_f32",
+    "bb_adam_multi", "bb_adam_multi_scaled", "bb_grad_clip_workspace", "bb_grad_clip_coef", "bb_cast", "bb_fill_f32",
 )
 
 
@@ -125,6 +125,10 @@ def lib():
     L.bb_adam_multi.argtypes = [c_int, POINTER(c_void_p), POINTER(c_void_p), POINTER(c_void_p),
                                 POINTER(c_void_p), POINTER(c_void_p), POINTER(c_int64), c_float, c_float,
                                 c_float, c_float, c_int, c_int, c_int, c_float, c_int, c_void_p]
+    L.bb_adam_multi_scaled.argtypes = L.bb_adam_multi.argtypes[:-1] + [c_void_p, c_void_p]
+    L.bb_grad_clip_workspace.argtypes = [c_int, POINTER(c_int64)]
+    L.bb_grad_clip_workspace.restype = c_int64
+    L.bb_grad_clip_coef.argtypes = [c_int, POINTER(c_void_p), POINTER(c_int64), c_float, c_void_p, c_void_p, c_void_p]
     L.bb_cast.argtypes = [c_int, c_int, c_int64, c_void_p, c_void_p, c_void_p]
     L.bb_fill_f32.argtypes = [c_void_p, c_int64, c_float, c_void_p]
     _lib = L
@@ -660,9 +664,29 @@ def mse_fwd_bwd(y, target, dy, grad_scale, loss_out, accumulate, workspace, stre
           "bb_mse_fwd_bwd")
 
 
+def grad_clip_workspace(grads):
+    """Floats of workspace :func:`grad_clip_coef` needs for these gradient tensors."""
+    n = len(grads)
+    return int(lib().bb_grad_clip_workspace(n, (c_int64 * n)(*[t.numel() for t in grads])))
+
+
+def grad_clip_coef(grads, max_norm, out, workspace, stream=None):
+    """out[0] = global L2 norm of the fp32 tensors ``grads``, out[1] = min(1, max_norm / (norm + 1e-6)) (both stay on the
+    device: :func:`adam_multi` takes ``out[1:]`` as its ``grad_scale``)."""
+    n = len(grads)
+    if any(t.dtype != torch.float32 or not t.is_contiguous() for t in grads):
+        raise HipKernelError("grad_clip_coef: contiguous float32 gradients expected")
+    if out.dtype != torch.float32 or out.numel() < 2 or workspace.dtype != torch.float32 or \
+            workspace.numel() < grad_clip_workspace(grads):
+        raise HipKernelError("grad_clip_coef: out needs 2 floats, workspace grad_clip_workspace(grads) floats")
+    check(lib().bb_grad_clip_coef(n, (c_void_p * n)(*[t.data_ptr() for t in grads]), (c_int64 * n)(*[t.numel() for t in grads]),
+                                  float(max_norm), _ptr(out), _ptr(workspace), stream_ptr(stream)), "bb_grad_clip_coef")
+
+
 def adam_multi(g, p, m, v, lowp, *, lr, beta1, beta2, eps, step, adam_w_mode=True, bias_correction=True,
-               weight_decay=0.0, zero_grad=False, stream=None):
-    """Lists of fp32 tensors g/p/m/v (same lengths); lowp: list of bf16 tensors or None entries, or None."""
+               weight_decay=0.0, zero_grad=False, grad_scale=None, stream=None):
+    """Lists of fp32 tensors g/p/m/v (same lengths); lowp: list of bf16 tensors or None entries, or None.
+    ``grad_scale``: one-element fp32 device tensor every gradient is multiplied by before the update (clipping)."""
     n = len(p)
     arr = lambda ts: (c_void_p * n)(*[None if t is None else t.data_ptr() for t in ts])
     sizes = (c_int64 * n)(*[t.numel() for t in p])
@@ -672,6 +696,13 @@ def adam_multi(g, p, m, v, lowp, *, lr, beta1, beta2, eps, step, adam_w_mode=Tru
         if not (a.numel() == b_.numel() == c.numel() == d.numel()):
             raise HipKernelError("adam_multi: size mismatch")
     lp = arr(lowp) if lowp is not None else None
+    if grad_scale is not None:
+        if grad_scale.dtype != torch.float32 or grad_scale.numel() < 1 or not grad_scale.is_cuda:
+            raise HipKernelError("adam_multi: grad_scale must be a float32 device tensor")
+        check(lib().bb_adam_multi_scaled(n, arr(g), arr(p), arr(m), arr(v), lp, sizes, lr, beta1, beta2, eps, step,
+                                         1 if adam_w_mode else 0, 1 if bias_correction else 0, weight_decay,
+                                         int(zero_grad), _ptr(grad_scale), stream_ptr(stream)), "bb_adam_multi_scaled")
+        return
     check(lib().bb_adam_multi(n, arr(g), arr(p), arr(m), arr(v), lp, sizes, lr, beta1, beta2, eps, step,
                               1 if adam_w_mode else 0, 1 if bias_correction else 0, weight_decay,
                               int(zero_grad), stream_ptr(stream)), "bb_adam_multi")

@@ -43,7 +43,21 @@ class FusedAdam:
         for sp in self.stages.values():
             sp.grad.zero_()
 
-    def step(self, closure=None, stream=None):
+    def clip_coef(self, max_norm, stream=None):
+        """Global-norm clipping over the gradients of every stage under this optimizer (the reference clips what
+        ``module.parameters()`` yields with a gradient: own stage, and an absorbed one after a failover;
+        deepspeed/runtime/engine.py:1521-1531): returns a device tensor ``[norm, coefficient]``; hand
+        ``[1:]`` to :meth:`step` as ``grad_scale``."""
+        grads = [sp.grad for sp in self.stages.values()]
+        need = hip.grad_clip_workspace(grads)
+        if getattr(self, "_clip_ws", None) is None or self._clip_ws.numel() < need:
+            import torch
+            self._clip_ws = torch.empty(need, dtype=torch.float32, device=grads[0].device)
+            self._clip_out = torch.zeros(2, dtype=torch.float32, device=grads[0].device)
+        hip.grad_clip_coef(grads, max_norm, self._clip_out, self._clip_ws, stream=stream)
+        return self._clip_out
+
+    def step(self, closure=None, stream=None, grad_scale=None):
         group = self.param_groups[0]
         group["step"] = group.get("step", 0) + 1
         sps = list(self.stages.values())
@@ -53,5 +67,5 @@ class FusedAdam:
                        lr=group["lr"], beta1=group["betas"][0], beta2=group["betas"][1], eps=group["eps"],
                        step=group["step"], adam_w_mode=bool(self.adam_w_mode),
                        bias_correction=group["bias_correction"], weight_decay=group["weight_decay"],
-                       zero_grad=True, stream=stream)
+                       zero_grad=True, grad_scale=grad_scale, stream=stream)
         return None

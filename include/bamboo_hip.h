@@ -320,6 +320,23 @@ int bb_adam_multi(int n_tensors, void* const* g, void* const* p, void* const* m,
                   float beta1, float beta2, float eps, int step, int mode,
                   int bias_correction, float weight_decay, int zero_grad, void* stream);
 
+/* Gradient clipping by the global norm: clip_grad_norm_ (deepspeed/runtime/utils.py:259-326) as
+ * _take_model_step calls it before optimizer.step() (deepspeed/runtime/engine.py:1526-1531,
+ * clip_fp32_gradients :1521-1524).  bb_grad_clip_coef leaves out[0] = sqrt(sum of squares of all
+ * the listed fp32 gradient tensors) and out[1] = min(1, max_norm / (out[0] + 1e-6)) in device
+ * memory (fixed summation order, no atomics); bb_adam_multi_scaled is bb_adam_multi with every
+ * gradient multiplied by the device scalar *grad_scale (NULL: by nothing) before the update, so
+ * the clipped gradients never make a pass of their own through memory and the host never waits
+ * for the norm.  workspace: bb_grad_clip_workspace(n_tensors, sizes) floats, 8-byte aligned.   */
+int64_t bb_grad_clip_workspace(int n_tensors, const int64_t* sizes);
+int bb_grad_clip_coef(int n_tensors, void* const* g, const int64_t* sizes, float max_norm,
+                      float* out, float* workspace, void* stream);
+int bb_adam_multi_scaled(int n_tensors, void* const* g, void* const* p, void* const* m,
+                         void* const* v, void* const* lowp, const int64_t* sizes, float lr,
+                         float beta1, float beta2, float eps, int step, int mode,
+                         int bias_correction, float weight_decay, int zero_grad,
+                         const float* grad_scale, void* stream);
+
 /* dtype conversion / fill helpers used when (re)materialising compute weights.            */
 int bb_cast(int src_dtype, int dst_dtype, int64_t n, const void* src, void* dst, void* stream);
 int bb_fill_f32(float* dst, int64_t n, float value, void* stream);

@@ -25,3 +25,21 @@ def adam_step(p, g, m, v, step, lr=1e-3, beta1=0.9, beta2=0.999, eps=1e-8,
         update = update + wd * p32
     p[...] = p32 - lr * update
     return p, m, v
+
+
+def clip_grad_norm(grads, max_norm):
+    """Global-norm clipping of a list of fp32 gradient arrays, in place; returns (total_norm, clip_coef).
+
+    Follows clip_grad_norm_ (deepspeed/runtime/utils.py:295-326) as _take_model_step calls it for fp32
+    gradients (deepspeed/runtime/engine.py:1521-1531), norm_type 2, one process: total_norm = (sum over the
+    tensors of ||g||_2 ** 2) ** 0.5, summed in Python floats; clip_coef = max_norm / (total_norm + 1e-6); the
+    gradients are multiplied by it (in fp32) only when it is below 1."""
+    total = 0.0
+    for g in grads:
+        total += float(np.sqrt(np.sum(g.astype(np.float64) ** 2))) ** 2
+    total_norm = total ** 0.5
+    clip_coef = float(max_norm) / (total_norm + 1e-6)
+    if clip_coef < 1:
+        for g in grads:
+            g *= np.float32(clip_coef)
+    return total_norm, clip_coef

@@ -335,3 +335,43 @@ def test_unfused_attention_fp32_at_12_heads_512_positions(hiplib, mask):
     assert err(st["ctx"], out.detach()) < 1e-5
     for i, name in enumerate("qkv"):
         assert err(d_qkv[:, i * h:(i + 1) * h], x.grad[:, i * h:(i + 1) * h]) < 1e-4, f"d{name}"
+
+
+@pytest.mark.parametrize("mask", ["none", "causal", "key_padding"])
+@pytest.mark.parametrize("d", [32, 128])
+def test_bf16_attention_with_other_head_widths(hiplib, mask, d):
+    """bf16 heads that are not 64 wide (the reference's GPT-2 script defaults to 512 / 16 = 32, gpt2.py:212-214) take
+    the path that materialises the probabilities: context and the three input gradients against fp64 autograd on
+    ``softmax(Q K^T / sqrt(d) [masked]) V``, 2e-2 of each tensor's largest magnitude, for the three masks."""
+    from bamboo_amd.layers import StageContext
+    b, a, s = 2, 4, 256
+    h = a * d
+    layer = TransformerLayer(h, a, 4 * h, activation="gelu_tanh", ln="standard", mask=mask)
+    ctx = StageContext(b, s, torch.bfloat16, torch.device(DEV))
+    lens = None
+    if mask == "key_padding":
+        lens = torch.tensor([s, 77], dtype=torch.int32, device=DEV)
+    ctx.key_len = lens
+    qkv = randn(b * s, 3 * h, seed=51, scale=0.7)
+    d_ctx = randn(b * s, h, seed=52)
+    st = {"qkv": qkv, "ctx": torch.empty(b * s, h, dtype=torch.bfloat16, device=DEV),
+          "prob": torch.empty(b, a, s, s, dtype=torch.bfloat16, device=DEV)}
+    ctx.ensure_scratch([("d_prob", (b, a, s, s), torch.bfloat16)])
+    assert not layer.fused_attention(ctx)
+    layer._attention_fwd(st, ctx)
+    d_qkv = torch.empty_like(qkv)
+    layer._attention_bwd(d_ctx, d_qkv, st, ctx)
+    torch.cuda.synchronize()
+    x = qkv.double().cpu().requires_grad_(True)
+    qq, kk, vv = [x[:, i * h:(i + 1) * h].view(b, s, a, d).transpose(1, 2) for i in range(3)]
+    scores = qq @ kk.transpose(-2, -1) / math.sqrt(d)
+    if mask == "causal":
+        scores = scores.masked_fill(~torch.tril(torch.ones(s, s, dtype=torch.bool)).view(1, 1, s, s), -1e9)
+    elif mask == "key_padding":
+        scores = scores.masked_fill(~(torch.arange(s).view(1, 1, 1, s) < lens.cpu().view(b, 1, 1, 1)), -1e9)
+    out = (torch.softmax(scores, dim=-1) @ vv).transpose(1, 2).reshape(b * s, h)
+    out.backward(d_ctx.double().cpu())
+    err = lambda got, want: float((got.double().cpu() - want).abs().max() / want.abs().max())
+    assert err(st["ctx"], out.detach()) < 2e-2
+    for i, name in enumerate("qkv"):
+        assert err(d_qkv[:, i * h:(i + 1) * h], x.grad[:, i * h:(i + 1) * h]) < 2e-2, f"d{name}"

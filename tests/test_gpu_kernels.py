@@ -764,6 +764,42 @@ def test_adam_bit_exact_with_oracle(hiplib, adam_w, wd):
     # agreement with torch.optim (the reference's own check, atol 1e-2) follows from the oracle test
 
 
+@pytest.mark.parametrize("max_norm", [1.0, 1e9])
+def test_gradient_clipping_coefficient_and_scaled_adam(hiplib, max_norm):
+    """Global gradient norm over several tensors (ragged sizes, more tensors than one launch's table holds) and the
+    clipping coefficient against the oracle's restatement of clip_grad_norm_; the Adam step that reads the
+    coefficient from device memory equals, bit for bit, the oracle's Adam step on gradients multiplied by that
+    coefficient in fp32; a bound above the norm changes nothing."""
+    sizes = [(n + 3) // 4 * 4 for n in [22, 4097, 1048576, 8192 + 3, 64] + [128] * 24]
+    total = sum(sizes)
+    offs = np.cumsum([0] + sizes)
+    split = lambda t: [t[offs[i]: offs[i + 1]] for i in range(len(sizes))]
+    G, P = randn(total, seed=61), randn(total, seed=62)
+    M_, V = torch.zeros(total, device=DEV), torch.zeros(total, device=DEV)
+    out = torch.full((2,), -1.0, device=DEV)
+    ws = torch.full((hiplib.grad_clip_workspace(split(G)),), float("nan"), device=DEV)
+    hiplib.grad_clip_coef(split(G), max_norm, out, ws)
+    hiplib.grad_clip_coef(split(G), max_norm, out, ws)       # the carried sum starts over with every call
+    g_ref = [g.cpu().numpy().copy() for g in split(G)]
+    norm, coef = oadam.clip_grad_norm(g_ref, max_norm)
+    assert abs(float(out[0]) - norm) < 2e-6 * norm
+    assert abs(float(out[1]) - min(coef, 1.0)) < 2e-6 * min(coef, 1.0)
+    assert (float(out[1]) == 1.0) == (max_norm > 1e6)
+    # the reference multiplies by the coefficient in fp32 (p.grad.data.mul_), then steps
+    c = np.float32(float(out[1]))
+    g_clipped = np.concatenate([g.cpu().numpy() for g in split(G)])
+    if c < 1:
+        g_clipped = g_clipped * c
+    p_ref, m_ref, v_ref = P.cpu().numpy().copy(), np.zeros(total, np.float32), np.zeros(total, np.float32)
+    oadam.adam_step(p_ref, g_clipped, m_ref, v_ref, 1)
+    hiplib.adam_multi(split(G), split(P), split(M_), split(V), None, lr=1e-3, beta1=0.9, beta2=0.999, eps=1e-8, step=1,
+                      grad_scale=out[1:])
+    assert np.array_equal(P.cpu().numpy(), p_ref) and np.array_equal(M_.cpu().numpy(), m_ref) and np.array_equal(V.cpu().numpy(), v_ref)
+    # no tensors at all: norm 0, coefficient 1
+    hiplib.grad_clip_coef([], 1.0, out, ws)
+    assert out.tolist() == [0.0, 1.0]
+
+
 def test_adam_rejects_bad_arguments(hiplib):
     t = torch.zeros(16, device=DEV)
     with pytest.raises(hiplib.HipKernelError):

@@ -4,6 +4,7 @@ bit-exactness of redundant forwards, failover promotion and the optimizer step.
 
 Tolerances (of the tensor's own scale): fp32 1e-5 on activations / 1e-4 on accumulated
 gradients (different summation order over 2048 rows x 8 micro-batches), bf16 2e-2."""
+import numpy as np
 import pytest
 import torch
 
@@ -903,3 +904,87 @@ def test_sigterm_and_launch_observer_belong_to_one_engine(hiplib):
         assert e.value.code == 13
     finally:
         signal.signal(signal.SIGTERM, prev)
+
+
+@pytest.mark.parametrize("heads", [4, 1], ids=["head-width-32", "head-width-128"])
+def test_bf16_stage_with_other_head_widths_matches_oracle(hiplib, heads):
+    """A bf16 stage whose heads are 32 (the reference GPT-2 script's default, gpt2.py:212-214) or 128 wide, with
+    redundant forwards: outputs, input gradients and parameter gradients against the fp64 oracle at the bf16 bars,
+    and the redundant forward's output bit-equal to the own forward of the same layers on the same input."""
+    hid, ffn, L, S, sid, mb, M, seq = 128, 256, 2, 4, 1, 2, 4, 64
+    dtype = torch.bfloat16
+    engine, q = build(hid, heads, ffn, L, S, sid, mb, M, seq, dtype, GPT_VARIANT, 1, True)
+    assert not engine.module.func_buckets[sid][0].fused_attention(engine.ctx)
+    st, peer = oracle_for(engine, q, GPT_VARIANT, hid, heads, ffn, L, S, sid, M, 1, True)
+    keep = {}
+    with NoStep(engine):
+        engine._clean_pipe_buffers = lambda: keep.update({k: list(v) for k, v in engine.pipe_buffers.items()})
+        engine.train_batch()
+    torch.cuda.synchronize()
+    bufs, _ = st.run_batch(peer, optimizer_step=False)
+    rel_err.lowp = True
+    for k in range(M):
+        for s_ in (sid, sid + 1):
+            want = bufs["out"][(s_, k)].detach().view(mb * seq, hid)
+            assert rel_err(keep[f"output_{s_}"][k], want) < 2e-2 and max_err(keep[f"output_{s_}"][k], want) < 5e-2
+        assert rel_err(keep[f"input_grad_{sid}"][k], bufs["sent_grad"][(sid, k)].view(mb * seq, hid)) < 2e-2
+    ref = st.named_grads(sid)
+    for name, g in engine.module.get_named_grad(sid):
+        assert rel_err(g, ref[name], grad_floor(ref)) < 2e-2, name
+    # the shadow layers run as a stage of their own on the own outputs: same bits as the redundant forward
+    specs = [LayerSpec(TransformerLayer, hid, heads, ffn, **GPT_VARIANT) for _ in range(L * S)]
+    model2 = PipelineModule(specs, num_stages=S, partition_method="uniform", stage_id=sid + 1, dtype=dtype, device=DEV)
+    ctx2 = model2.prepare_context([sid + 1], mb, seq)
+    model2.allocate_stash(sid + 1, ctx2, 1)
+    for k in range(M):
+        normal = model2.forward(keep[f"output_{sid}"][k], sid + 1, slot=0, ctx=ctx2)
+        torch.cuda.synchronize()
+        assert torch.equal(normal, keep[f"output_{sid + 1}"][k]), k
+
+
+def test_gradient_clipping_in_the_optimizer_step(hiplib):
+    """``gradient_clipping`` of the DeepSpeed JSON (deepspeed/runtime/engine.py:1526-1531): with a bound far below the
+    gradient norm the step equals the oracle stage's Adam step on gradients scaled by max_norm / (norm + 1e-6); the
+    reported norm is the oracle's; with a bound far above it the weights equal the unclipped run bit for bit."""
+    from oracle import adam as oadam
+    rel_err.lowp = False
+    hid, heads, ffn, L, S, sid, mb, M, seq = 128, 2, 256, 2, 4, 1, 2, 4, 64
+
+    def run(clip):
+        specs = [LayerSpec(TransformerLayer, hid, heads, ffn, **GPT_VARIANT) for _ in range(L * S)]
+        model = PipelineModule(specs, num_stages=S, partition_method="uniform", stage_id=sid, dtype=torch.float32, device=DEV)
+        q = SeededActivationQueue((mb, seq, hid), torch.float32, M, stage_ids=[sid, sid + 1], seed=7, device=DEV)
+        cfg = {"train_micro_batch_size_per_gpu": mb, "gradient_accumulation_steps": M, "gradient_clipping": clip,
+               "optimizer": {"type": "Adam", "params": {"lr": 1e-3}}}
+        engine, _, _, _ = bamboo_amd.initialize(model=model, config=cfg, activation_queue=q, install_signal_handler=False)
+        return engine, q
+    plain, _ = run(0.0)
+    loose, _ = run(1e9)
+    tight, q = run(1e-3)
+    st, peer = oracle_for(tight, q, GPT_VARIANT, hid, heads, ffn, L, S, sid, M, 0, False, dtype=torch.float32)
+    before = {k: v.clone() for k, v in tight.module.get_named_param(sid)}
+    for e in (plain, loose, tight):
+        e.train_batch()
+    torch.cuda.synchronize()
+    assert torch.equal(plain.module.stage_params[sid].master, loose.module.stage_params[sid].master)
+    assert float(loose.grad_norm[1]) == 1.0
+    # oracle: gradients of the batch, clipped, then the Adam step
+    st.run_batch(peer, optimizer_step=False)
+    names = list(st.named_grads(sid))
+    grads = [st.named_grads(sid)[n].detach().numpy().astype(np.float32).copy() for n in names]
+    norm, coef = oadam.clip_grad_norm(grads, 1e-3)
+    assert coef < 0.1 and abs(float(tight.grad_norm[0]) - norm) < 1e-4 * norm
+    got = dict(tight.module.get_named_param(sid))
+    for n, g in zip(names, grads):
+        if n.endswith("linears.1.bias"):
+            continue    # key bias: the exact gradient is zero, Adam normalises rounding noise
+        p0 = before[n].cpu().numpy().copy()
+        ref, m_ref = p0.copy(), np.zeros_like(p0)
+        oadam.adam_step(ref, g, m_ref, np.zeros_like(ref), 1)
+        d, dr = got[n].cpu().numpy() - p0, ref - p0
+        assert float(np.abs(d - dr).max()) < 2e-4, n       # movement against lr = 1e-3, as in the unclipped test
+        # the first moment is (1 - beta1) x the CLIPPED gradient: the first step's movement alone would not tell
+        sp = tight.module.stage_params[sid]
+        m_got = sp.view(sp.exp_avg, n).cpu().numpy()
+        assert float(np.abs(m_got - m_ref).max()) < 1e-4 * float(np.abs(m_ref).max()) + 1e-12, n
+    assert not torch.equal(plain.module.stage_params[sid].exp_avg, tight.module.stage_params[sid].exp_avg)

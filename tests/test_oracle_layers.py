@@ -253,6 +253,30 @@ def test_adam_matches_torch(adam_w, wd):
         np.testing.assert_allclose(p, p_t.detach().numpy(), rtol=2e-6, atol=2e-7)
 
 
+@pytest.mark.parametrize("max_norm", [0.5, 1e6])
+def test_clip_grad_norm_matches_torch(max_norm):
+    """The restated global-norm clipping against torch.nn.utils.clip_grad_norm_ (the routine the reference's
+    clip_grad_norm_ is adapted from: same coefficient max_norm / (norm + 1e-6), applied only below 1), on tensors of
+    different sizes; a bound far above the norm leaves the gradients untouched bit for bit."""
+    torch.manual_seed(4)
+    params = [torch.nn.Parameter(torch.zeros(n)) for n in (7, 1024, 33)]
+    for prm in params:
+        prm.grad = torch.randn_like(prm) * 3
+    grads = [prm.grad.numpy().copy() for prm in params]
+    before = [g.copy() for g in grads]
+    norm_t = float(torch.nn.utils.clip_grad_norm_(params, max_norm))
+    norm, coef = oadam.clip_grad_norm(grads, max_norm)
+    assert abs(norm - norm_t) < 1e-5 * norm_t
+    want = (sum(float((b.astype(np.float64) ** 2).sum()) for b in before)) ** 0.5      # the closed form
+    assert abs(norm - want) < 1e-12 * want and abs(coef - max_norm / (want + 1e-6)) < 1e-12
+    for g, prm, b in zip(grads, params, before):
+        np.testing.assert_allclose(g, prm.grad.numpy(), rtol=1e-6, atol=0)
+        if max_norm > 1e5:
+            assert np.array_equal(g, b)
+        else:
+            assert abs(float(np.abs(g).max()) / float(np.abs(b).max()) - coef) < 1e-6
+
+
 def test_adam_first_step_closed_form():
     # step 1 with zero moments: update = g / (|g| + eps*sqrt(1-b2)) ~ sign(g): p1 = p0 - lr*sign(g)
     p = np.array([1.0, -2.0, 3.0], np.float32)
