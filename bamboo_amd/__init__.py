@@ -7,7 +7,7 @@ successor's shadow layers, failover promotion) on a single MI355X, behind the re
 """
 from . import hip, schedule
 from .config import BambooConfig
-from .layers import BottleNeck, FinalLayerNorm, MSELoss, SumLast, TransformerLayer
+from .layers import BottleNeck, DecoderLayer, FinalLayerNorm, MSELoss, SumLast, TransformerLayer
 from .module import LayerSpec, PipelineError, PipelineModule, TiedLayerSpec
 from .optim import FusedAdam
 from .p2p import (AllReduceException, LocalFabric, NextStageException, PrevStageException, SeededActivationQueue,

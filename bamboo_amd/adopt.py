@@ -9,6 +9,7 @@ take the module's weights into the stage's arenas:
 
   ``EncoderLayer``   (DeepSpeedExamples/pipeline_parallelism/transformer.py:161-172;
                      ``EncoderLayerSimple``, bert.py:20-31: same parameters, same function)   -> :class:`TransformerLayer`
+  ``DecoderLayerSimple`` (DeepSpeedExamples/pipeline_parallelism/gpt2.py:20-34)        -> :class:`DecoderLayer`
   ``LayerNorm``      (transformer.py:77-88, the ``encoder.norm`` of :181,250)          -> :class:`FinalLayerNorm`
   ``lambda x: x.sum(-1)`` (transformer.py:250)                                        -> :class:`SumLast`
   ``BottleNeck``     (DeepSpeedExamples/pipeline_parallelism/resnet.py:49-75)          -> :class:`BottleNeck`
@@ -18,7 +19,7 @@ Anything else is refused with an error that says what was found: there is no aut
 """
 import torch
 
-from .layers import BottleNeck, FinalLayerNorm, MSELoss, SumLast, TransformerLayer
+from .layers import BottleNeck, DecoderLayer, FinalLayerNorm, MSELoss, SumLast, TransformerLayer
 
 
 class AdoptionError(Exception):
@@ -69,6 +70,19 @@ def adopt_layer(obj, training=True):
         layer = TransformerLayer(hidden, int(heads), ffn, activation="relu", ln="annotated", mask="none", ln_eps=eps,
                                  dropout=drops[0] if drops else 0.0)
         return layer, params
+    if names == set(DecoderLayer.REFERENCE_ORDER):
+        hidden = params["sublayer.0.norm.a_2"].numel()
+        ffn = params["feed_forward.w_1.weight"].shape[0]
+        heads = getattr(getattr(obj, "self_attn", None), "h", None)
+        if heads is None or getattr(getattr(obj, "src_attn", None), "h", None) != heads:
+            raise AdoptionError("DecoderLayerSimple-shaped module whose two attention modules do not state one number of heads (.h)")
+        if len(drops) > 1:
+            raise AdoptionError(f"DecoderLayerSimple-shaped module with different dropout probabilities {drops}: the layer "
+                                "takes one probability for its six dropout sites")
+        eps = float(getattr(obj.sublayer[0].norm, "eps", 1e-6))
+        layer = DecoderLayer(hidden, int(heads), ffn, activation="relu", ln="annotated", mask="none", ln_eps=eps,
+                             dropout=drops[0] if drops else 0.0)
+        return layer, params
     if names in (set(BottleNeck.RESIDUAL_ORDER), set(BottleNeck.RESIDUAL_ORDER + BottleNeck.SHORTCUT_ORDER)):
         w0, conv3 = params["residual_function.0.weight"], obj.residual_function[3]
         stride = conv3.stride[0] if isinstance(conv3.stride, tuple) else int(conv3.stride)
@@ -91,7 +105,7 @@ def adopt_layer(obj, training=True):
     if names == {"a_2", "b_2"}:
         return FinalLayerNorm(params["a_2"].numel(), ln="annotated", ln_eps=float(getattr(obj, "eps", 1e-6))), params
     raise AdoptionError(f"module {type(obj).__name__} with parameters {sorted(names)[:6]}... is not one of the layers this "
-                        "engine accelerates (EncoderLayer, LayerNorm, BottleNeck of the reference's pipeline_parallelism scripts)")
+                        "engine accelerates (EncoderLayer, DecoderLayerSimple, LayerNorm, BottleNeck of the reference's pipeline_parallelism scripts)")
 
 
 def adopt_loss(loss_fn):

@@ -713,6 +713,69 @@ extern "C" int bb_residual_add(int dtype, int64_t n, const void* a, const void* 
     return BB_OK;
 }
 
+// m = sqrt(1 - x): the stand-in "memory" of the reference's DecoderLayerSimple (gpt2.py:31), and its backward
+// dx (+)= dm * (-1 / (2 m)).  NaN where x > 1 and an infinite derivative at x = 1, as torch gives them.
+template <typename T>
+__global__ __launch_bounds__(256) void sqrt1m_fwd_kernel(int64_t nvec, const T* __restrict__ x, T* __restrict__ m) {
+    constexpr int VEC = Elem<T>::VEC;
+    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < nvec; i += (int64_t)gridDim.x * 256) {
+        float v[VEC];
+        load_vec(x + i * VEC, v);
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) v[e] = sqrtf(1.0f - v[e]);
+        store_vec(m + i * VEC, v);
+    }
+}
+template <typename T>
+__global__ __launch_bounds__(256) void sqrt1m_bwd_kernel(int64_t nvec, const T* __restrict__ dm, const T* __restrict__ m,
+                                                         T* __restrict__ dx, int accumulate) {
+    constexpr int VEC = Elem<T>::VEC;
+    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < nvec; i += (int64_t)gridDim.x * 256) {
+        float g[VEC], mv[VEC], acc[VEC];
+        load_vec(dm + i * VEC, g);
+        load_vec(m + i * VEC, mv);
+        if (accumulate) load_vec(dx + i * VEC, acc);
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) {
+            const float d = g[e] * (-0.5f / mv[e]);
+            acc[e] = accumulate ? acc[e] + d : d;
+        }
+        store_vec(dx + i * VEC, acc);
+    }
+}
+extern "C" int bb_sqrt_one_minus_fwd(int dtype, int64_t n, const void* x, void* m, void* stream) {
+    BB_REQUIRE(dtype == BB_F32 || dtype == BB_BF16, "bb_sqrt_one_minus_fwd: bad dtype %d", dtype);
+    const int vec = dtype == BB_BF16 ? 8 : 4;
+    BB_REQUIRE(n >= 0 && n % vec == 0, "bb_sqrt_one_minus_fwd: n (%lld) must be a multiple of %d", (long long)n, vec);
+    BB_REQUIRE(x && m, "bb_sqrt_one_minus_fwd: null pointer");
+    if (n == 0) return BB_OK;
+    hipStream_t st = (hipStream_t)stream;
+    const int64_t nvec = n / vec;
+    if (dtype == BB_BF16)
+        hipLaunchKernelGGL(sqrt1m_fwd_kernel<bf16>, dim3(grid_for(nvec)), dim3(256), 0, st, nvec, (const bf16*)x, (bf16*)m);
+    else
+        hipLaunchKernelGGL(sqrt1m_fwd_kernel<float>, dim3(grid_for(nvec)), dim3(256), 0, st, nvec, (const float*)x, (float*)m);
+    BB_LAUNCH_CHECK();
+    return BB_OK;
+}
+extern "C" int bb_sqrt_one_minus_bwd(int dtype, int64_t n, const void* dm, const void* m, void* dx, int accumulate, void* stream) {
+    BB_REQUIRE(dtype == BB_F32 || dtype == BB_BF16, "bb_sqrt_one_minus_bwd: bad dtype %d", dtype);
+    const int vec = dtype == BB_BF16 ? 8 : 4;
+    BB_REQUIRE(n >= 0 && n % vec == 0, "bb_sqrt_one_minus_bwd: n (%lld) must be a multiple of %d", (long long)n, vec);
+    BB_REQUIRE(dm && m && dx, "bb_sqrt_one_minus_bwd: null pointer");
+    if (n == 0) return BB_OK;
+    hipStream_t st = (hipStream_t)stream;
+    const int64_t nvec = n / vec;
+    if (dtype == BB_BF16)
+        hipLaunchKernelGGL(sqrt1m_bwd_kernel<bf16>, dim3(grid_for(nvec)), dim3(256), 0, st, nvec, (const bf16*)dm, (const bf16*)m,
+                           (bf16*)dx, accumulate);
+    else
+        hipLaunchKernelGGL(sqrt1m_bwd_kernel<float>, dim3(grid_for(nvec)), dim3(256), 0, st, nvec, (const float*)dm, (const float*)m,
+                           (float*)dx, accumulate);
+    BB_LAUNCH_CHECK();
+    return BB_OK;
+}
+
 // dst = dropout(src) with the decisions of key (k0, k1): element i of the contiguous tensor is kept (and scaled by
 // 1 / (1 - p)) when bb_dropout_keep says so.  nn.Dropout in training mode (transformer.py:98-103,125-126,154-158)
 // with a mask that is a pure function of (key, i); the same call on a gradient is its backward.

@@ -25,7 +25,7 @@ LN_CODES = {"standard": LN_STANDARD, "annotated": LN_ANNOTATED}
 EXPORTS = (
     "bb_version", "bb_last_error", "bb_init", "bb_gemm", "bb_gemm_grouped", "bb_gemm_splitk_workspace", "bb_gemm_grouped_splitk", "bb_gemm_variant", "bb_layernorm_fwd",
     "bb_layernorm_bwd_workspace", "bb_layernorm_bwd", "bb_layernorm_bwd_static", "bb_colsum_workspace", "bb_colsum_acc", "bb_rowsum_fwd", "bb_rowsum_bwd", "bb_dropout_apply", "bb_dropout_keep_host",
-    "bb_softmax_fwd", "bb_softmax_bwd", "bb_attention_fwd", "bb_attention_bwd", "bb_residual_add", "bb_act_fwd", "bb_bn_workspace", "bb_batchnorm_fwd", "bb_batchnorm_bwd", "bb_patch3x3", "bb_patch3x3_strided", "bb_subsample", "bb_conv3x3_supported", "bb_conv3x3", "bb_gemm_strip_stats_supported", "bb_strip_stats_workspace", "bb_batchnorm_fwd_strips", "bb_mse_workspace", "bb_mse_fwd_bwd", "bb_graph_begin", "bb_graph_end", "bb_graph_launch", "bb_graph_destroy",
+    "bb_softmax_fwd", "bb_softmax_bwd", "bb_attention_fwd", "bb_attention_bwd", "bb_residual_add", "bb_sqrt_one_minus_fwd", "bb_sqrt_one_minus_bwd", "bb_act_fwd", "bb_bn_workspace", "bb_batchnorm_fwd", "bb_batchnorm_bwd", "bb_patch3x3", "bb_patch3x3_strided", "bb_subsample", "bb_conv3x3_supported", "bb_conv3x3", "bb_gemm_strip_stats_supported", "bb_strip_stats_workspace", "bb_batchnorm_fwd_strips", "bb_mse_workspace", "bb_mse_fwd_bwd", "bb_graph_begin", "bb_graph_end", "bb_graph_launch", "bb_graph_destroy",
     "bb_adam_multi", "bb_adam_multi_scaled", "bb_grad_clip_workspace", "bb_grad_clip_coef", "bb_cast", "bb_fill_f32",
 )
 
@@ -101,6 +101,8 @@ def lib():
     L.bb_dropout_apply.argtypes = [c_int, c_int64, c_void_p, c_void_p, c_float, c_uint32, c_uint32, c_void_p]
     L.bb_dropout_keep_host.argtypes = [c_float, c_uint32, c_uint32, c_uint64]
     L.bb_residual_add.argtypes = [c_int, c_int64, c_void_p, c_void_p, c_void_p, c_void_p]
+    L.bb_sqrt_one_minus_fwd.argtypes = [c_int, c_int64, c_void_p, c_void_p, c_void_p]
+    L.bb_sqrt_one_minus_bwd.argtypes = [c_int, c_int64, c_void_p, c_void_p, c_void_p, c_int, c_void_p]
     L.bb_graph_begin.argtypes = [c_void_p]
     L.bb_graph_end.argtypes = [c_void_p, POINTER(c_void_p)]
     L.bb_graph_launch.argtypes = [c_void_p, c_void_p]
@@ -496,6 +498,19 @@ def residual_add(a, b, out, stream=None):
     _like("residual_add", a, b=b, out=out)
     check(lib().bb_residual_add(dtype_code(a.dtype), a.numel(), _ptr(a), _ptr(b), _ptr(out), stream_ptr(stream)),
           "bb_residual_add")
+
+
+def sqrt_one_minus_fwd(x, m, stream=None):
+    """m = sqrt(1 - x)."""
+    _like("sqrt_one_minus_fwd", x, m=m)
+    check(lib().bb_sqrt_one_minus_fwd(dtype_code(x.dtype), x.numel(), _ptr(x), _ptr(m), stream_ptr(stream)), "bb_sqrt_one_minus_fwd")
+
+
+def sqrt_one_minus_bwd(dm, m, dx, accumulate=True, stream=None):
+    """dx (+)= dm * (-1 / (2 m)) for m = sqrt(1 - x)."""
+    _like("sqrt_one_minus_bwd", dm, m=m, dx=dx)
+    check(lib().bb_sqrt_one_minus_bwd(dtype_code(dm.dtype), dm.numel(), _ptr(dm), _ptr(m), _ptr(dx), int(accumulate),
+                                      stream_ptr(stream)), "bb_sqrt_one_minus_bwd")
 
 
 def act_fwd(x, out, act, dact=None, stream=None):

@@ -233,12 +233,15 @@ class TransformerLayer:
         hip.gemm_batched(layout, hip.dtype_code(ctx.dtype), M, N, K, A, lda, sA, B, ldb, sB, C, ldc, sC,
                          ctx.batch, self.heads, alpha=alpha, stream=ctx.stream)
 
-    def _attention_fwd(self, st, ctx):
+    def _attention_fwd(self, st, ctx, site=0, mask=None):
+        """``st``: the entries ``qkv`` ([rows, 3h]: queries, keys, values side by side), ``ctx`` and ``lse`` / ``prob``;
+        ``site``: the dropout site of the probabilities; ``mask``: the layer's own unless given."""
         h, d, s = self.hidden, self.head_dim, ctx.seq
-        drop = self._drop(ctx, self.SITE_ATTENTION)
+        mask = self.mask if mask is None else mask
+        drop = self._drop(ctx, site)
         if self.fused_attention(ctx):
-            hip.attention_fwd(st["qkv"], st["ctx"], st["lse"], ctx.batch, self.heads, s, hip.MASK_CODES[self.mask],
-                              ctx.key_len, stream=ctx.stream, dropout=drop)
+            hip.attention_fwd(st["qkv"], st["ctx"], st["lse"], ctx.batch, self.heads, s, hip.MASK_CODES[mask],
+                              ctx.key_len if mask == "key_padding" else None, stream=ctx.stream, dropout=drop)
             return
         es = st["qkv"].element_size()
         q = st["qkv"].data_ptr()
@@ -248,7 +251,7 @@ class TransformerLayer:
         # scores = Q K^T / sqrt(d)
         self._heads_gemm(ctx, hip.NT, s, s, d, q, 3 * h, head_in, k, 3 * h, head_in,
                          prob.data_ptr(), s, (self.heads * s * s, s * s), alpha=1.0 / math.sqrt(d))
-        hip.softmax_fwd(prob, hip.MASK_CODES[self.mask], ctx.key_len, stream=ctx.stream)
+        hip.softmax_fwd(prob, hip.MASK_CODES[mask], ctx.key_len if mask == "key_padding" else None, stream=ctx.stream)
         if drop is not None:
             # the stash keeps the probabilities themselves (the softmax backward needs them); V meets the dropped-out copy
             kept = ctx.buf("prob_drop", tuple(prob.shape))
@@ -258,13 +261,15 @@ class TransformerLayer:
         self._heads_gemm(ctx, hip.NN, s, d, s, prob.data_ptr(), s, (self.heads * s * s, s * s), v, 3 * h, head_in,
                          st["ctx"].data_ptr(), h, (s * h, d))
 
-    def _attention_bwd(self, d_ctx, d_qkv, st, ctx):
+    def _attention_bwd(self, d_ctx, d_qkv, st, ctx, site=0, mask=None):
         h, d, s = self.hidden, self.head_dim, ctx.seq
-        drop = self._drop(ctx, self.SITE_ATTENTION)
+        mask = self.mask if mask is None else mask
+        drop = self._drop(ctx, site)
         if self.fused_attention(ctx):
             delta = ctx.buf("attn_delta", (ctx.batch, self.heads, s))
             hip.attention_bwd(st["qkv"], st["ctx"], d_ctx, st["lse"], delta, d_qkv, ctx.batch, self.heads, s,
-                              hip.MASK_CODES[self.mask], ctx.key_len, stream=ctx.stream, dropout=drop)
+                              hip.MASK_CODES[mask], ctx.key_len if mask == "key_padding" else None, stream=ctx.stream,
+                              dropout=drop)
             return
         es = st["qkv"].element_size()
         q = st["qkv"].data_ptr()
@@ -381,6 +386,198 @@ class TransformerLayer:
                           g["sublayer.0.norm.a_2"], g["sublayer.0.norm.b_2"], ws, kind, self.eps, stream=sm)
         # d_out (d_drop1), d_ffn, d_h1 (d_drop0) and d_qkv still hold the four output gradients here
         ctx.gemm_grouped(wgrads, stream=sm)
+        return d_x
+
+
+class DecoderLayer(TransformerLayer):
+    """The layer of the reference's GPT-2 script, ``DecoderLayerSimple`` (DeepSpeedExamples/pipeline_parallelism/
+    gpt2.py:20-34): three pre-LN residual sublayers -- self-attention, attention over a "memory" (queries from the
+    normalised stream, keys and values from ``m = sqrt(1 - x)`` of the layer's own INPUT ``x``: the script has no second
+    input, gpt2.py:31), feed-forward.  ``m`` is defined for inputs below 1; beyond, its NaN enters the attention as
+    in the reference (what becomes of NaN scores inside the attention kernels is not specified here).
+
+    Parameters carry the reference module's names: ``self_attn.linears.{0..3}``, ``src_attn.linears.{0..3}``,
+    ``feed_forward.w_{1,2}``, ``sublayer.{0,1,2}.norm.{a_2,b_2}``.  The memory attention reuses the kernels of
+    the self-attention: its queries (one product on the normalised stream) and its keys / values (one product on
+    ``m``, the two weights being neighbours in the arena) are written side by side into one ``[rows, 3h]`` buffer.
+    Dropout sites: the four of :class:`TransformerLayer` (0 self-attention probabilities, 1 first sublayer, 2
+    feed-forward hidden, 3 last sublayer) plus 4 (memory-attention probabilities) and 5 (second sublayer).
+    ``mask`` applies to the self-attention only (the script passes none)."""
+
+    SITE_SRC_ATTENTION, SITE_SUBLAYER_SRC = 4, 5
+
+    REFERENCE_ORDER = tuple(
+        [f"self_attn.linears.{i}.{k}" for i in range(4) for k in ("weight", "bias")] +
+        [f"src_attn.linears.{i}.{k}" for i in range(4) for k in ("weight", "bias")] +
+        ["feed_forward.w_1.weight", "feed_forward.w_1.bias", "feed_forward.w_2.weight", "feed_forward.w_2.bias"] +
+        [f"sublayer.{i}.norm.{k}" for i in range(3) for k in ("a_2", "b_2")])
+
+    def param_specs(self):
+        h, f = self.hidden, self.ffn
+        return OrderedDict([
+            ("sublayer.0.norm.a_2", (h,)), ("sublayer.0.norm.b_2", (h,)),
+            ("self_attn.linears.0.weight", (h, h)), ("self_attn.linears.1.weight", (h, h)), ("self_attn.linears.2.weight", (h, h)),
+            ("self_attn.linears.0.bias", (h,)), ("self_attn.linears.1.bias", (h,)), ("self_attn.linears.2.bias", (h,)),
+            ("self_attn.linears.3.weight", (h, h)), ("self_attn.linears.3.bias", (h,)),
+            ("sublayer.1.norm.a_2", (h,)), ("sublayer.1.norm.b_2", (h,)),
+            ("src_attn.linears.0.weight", (h, h)), ("src_attn.linears.0.bias", (h,)),
+            ("src_attn.linears.1.weight", (h, h)), ("src_attn.linears.2.weight", (h, h)),      # keys, values: one [2h, h] product
+            ("src_attn.linears.1.bias", (h,)), ("src_attn.linears.2.bias", (h,)),
+            ("src_attn.linears.3.weight", (h, h)), ("src_attn.linears.3.bias", (h,)),
+            ("sublayer.2.norm.a_2", (h,)), ("sublayer.2.norm.b_2", (h,)),
+            ("feed_forward.w_1.weight", (f, h)), ("feed_forward.w_1.bias", (f,)),
+            ("feed_forward.w_2.weight", (h, f)), ("feed_forward.w_2.bias", (h,)),
+        ])
+
+    def init_params(self, master, seed):
+        """Weights N(0, init_std) from per-tensor seeded generators (index = position in the reference module's
+        parameter order), biases 0, LayerNorm gain 1."""
+        for i, name in enumerate(self.REFERENCE_ORDER):
+            t = master[name]
+            if name.endswith("a_2"):
+                t.fill_(1.0)
+            elif name.endswith("weight"):
+                g = torch.Generator().manual_seed(seed * 1000 + i)
+                t.copy_(torch.randn(t.shape, generator=g, dtype=torch.float32) * self.init_std)
+            else:
+                t.zero_()
+
+    def bind(self, compute, grads):
+        super().bind(compute, grads)
+        h = self.hidden
+        for d, src in ((self.w, compute), (self.g, grads)):
+            d["kv.weight"] = torch.as_strided(src["src_attn.linears.1.weight"], (2 * h, h), (h, 1))
+            d["kv.bias"] = torch.as_strided(src["src_attn.linears.1.bias"], (2 * h,), (1,))
+
+    def stash_specs(self, ctx):
+        R, h, f = ctx.rows, self.hidden, self.ffn
+        dt, f32 = ctx.dtype, torch.float32
+        fused = self.fused_attention(ctx)
+        attn = lambda tag: (f"lse{tag}", (ctx.batch, self.heads, ctx.seq), f32) if fused else \
+            (f"prob{tag}", (ctx.batch, self.heads, ctx.seq, ctx.seq), dt)
+        dact = [] if self.activation == "relu" else [("dact", (R, f), dt)]
+        return [
+            ("n1", (R, h), dt), ("qkv", (R, 3 * h), dt), attn(""), ("ctx", (R, h), dt), ("x1", (R, h), dt),
+            ("mem", (R, h), dt), ("n_src", (R, h), dt), ("qkv_src", (R, 3 * h), dt), attn("_src"), ("ctx_src", (R, h), dt),
+            ("x2", (R, h), dt), ("n2", (R, h), dt), *dact, ("act", (R, f), dt), ("out", (R, h), dt),
+            ("mean1", (R,), f32), ("rinv1", (R,), f32), ("mean_src", (R,), f32), ("rinv_src", (R,), f32),
+            ("mean2", (R,), f32), ("rinv2", (R,), f32),
+        ]
+
+    def scratch_specs(self, ctx):
+        R, h = ctx.rows, self.hidden
+        specs = super().scratch_specs(ctx) + [("d_mem", (R, h), ctx.dtype), ("d_h2", (R, h), ctx.dtype)]
+        if self.dropout > 0:
+            specs.append(("d_drop_src", (R, h), ctx.dtype))
+        return specs
+
+    def flops_fwd(self, batch, seq):
+        h, f = self.hidden, self.ffn
+        return batch * seq * (16 * h * h + 4 * h * f) + 8 * batch * seq * seq * h
+
+    def _src_views(self, st):
+        return {"qkv": st["qkv_src"], "ctx": st["ctx_src"], "lse": st.get("lse_src"), "prob": st.get("prob_src")}
+
+    def forward(self, x, st, ctx):
+        w, sm = self.w, ctx.stream
+        kind, act = hip.LN_CODES[self.ln], hip.ACT_CODES[self.activation]
+        h = self.hidden
+        st["x0"] = x
+        hip.sqrt_one_minus_fwd(x, st["mem"], stream=sm)                                      # gpt2.py:31
+        # sublayer 0: self-attention
+        hip.layernorm_fwd(x, w["sublayer.0.norm.a_2"], w["sublayer.0.norm.b_2"], st["n1"], st["mean1"], st["rinv1"],
+                          kind, self.eps, stream=sm)
+        ctx.gemm(hip.NT, st["n1"], w["qkv.weight"], st["qkv"], bias=w["qkv.bias"], stream=sm)
+        self._attention_fwd(st, ctx, site=self.SITE_ATTENTION)
+        ctx.gemm(hip.NT, st["ctx"], w["self_attn.linears.3.weight"], st["x1"], bias=w["self_attn.linears.3.bias"],
+                 epilogue=hip.EPI_RESIDUAL, resid=x, dropout=self._drop(ctx, self.SITE_SUBLAYER0), stream=sm)
+        # sublayer 1: queries from the stream, keys and values from the memory
+        hip.layernorm_fwd(st["x1"], w["sublayer.1.norm.a_2"], w["sublayer.1.norm.b_2"], st["n_src"], st["mean_src"],
+                          st["rinv_src"], kind, self.eps, stream=sm)
+        qs = st["qkv_src"]
+        ctx.gemm(hip.NT, st["n_src"], w["src_attn.linears.0.weight"], qs[:, :h], bias=w["src_attn.linears.0.bias"], stream=sm)
+        ctx.gemm(hip.NT, st["mem"], w["kv.weight"], qs[:, h:], bias=w["kv.bias"], stream=sm)
+        self._attention_fwd(self._src_views(st), ctx, site=self.SITE_SRC_ATTENTION, mask="none")
+        ctx.gemm(hip.NT, st["ctx_src"], w["src_attn.linears.3.weight"], st["x2"], bias=w["src_attn.linears.3.bias"],
+                 epilogue=hip.EPI_RESIDUAL, resid=st["x1"], dropout=self._drop(ctx, self.SITE_SUBLAYER_SRC), stream=sm)
+        # sublayer 2: feed-forward
+        hip.layernorm_fwd(st["x2"], w["sublayer.2.norm.a_2"], w["sublayer.2.norm.b_2"], st["n2"], st["mean2"],
+                          st["rinv2"], kind, self.eps, stream=sm)
+        if ctx.defer or self.activation == "relu":
+            ctx.gemm(hip.NT, st["n2"], w["feed_forward.w_1.weight"], st["act"], bias=w["feed_forward.w_1.bias"],
+                     epilogue=hip.EPI_ACT, act=act, dropout=self._drop(ctx, self.SITE_FFN), stream=sm)
+        else:
+            self._ffn1(st, ctx)
+        ctx.gemm(hip.NT, st["act"], w["feed_forward.w_2.weight"], st["out"], bias=w["feed_forward.w_2.bias"],
+                 epilogue=hip.EPI_RESIDUAL, resid=st["x2"], dropout=self._drop(ctx, self.SITE_SUBLAYER1), stream=sm)
+        return st["out"]
+
+    def backward(self, d_out, d_x, st, ctx):
+        w, g, sm, ws = self.w, self.g, ctx.stream, ctx.workspace
+        R, h, f = ctx.rows, self.hidden, self.ffn
+        kind = hip.LN_CODES[self.ln]
+        d_ffn, d_h0, d_h1, d_h2 = (ctx.buf("d_ffn", (R, f)), ctx.buf("d_h0", (R, h)), ctx.buf("d_h1", (R, h)),
+                                   ctx.buf("d_h2", (R, h)))
+        d_qkv, d_mem = ctx.buf("d_qkv", (R, 3 * h)), ctx.buf("d_mem", (R, h))
+        wgrads = []
+        wgrad = lambda dy, x, name, bias=None: wgrads.append(hip.gemm_desc(
+            hip.TN, dy, x, g[name], accumulate=True, colsum_out=g[bias or (name[:-len("weight")] + "bias")], colsum_ws=ws))
+
+        def flush():
+            # the weight gradients collected so far, before a scratch buffer they read is written again
+            if wgrads:
+                ctx.gemm_grouped(list(wgrads), stream=sm)
+                wgrads.clear()
+        if ctx.deferred and self.activation != "relu":
+            self._ffn1(st, ctx)
+        # ---- sublayer 2: feed-forward (as in TransformerLayer.backward)
+        d_ff2 = d_out
+        if self.dropout > 0:
+            d_ff2 = ctx.buf("d_drop1", (R, h))
+            hip.dropout_apply(d_out, d_ff2, *self._drop(ctx, self.SITE_SUBLAYER1), stream=sm)
+        wgrad(d_ff2, st["act"], "feed_forward.w_2.weight")
+        if self.activation == "relu":
+            ctx.gemm(hip.NN, d_ff2, w["feed_forward.w_2.weight"], d_ffn, epilogue=hip.EPI_MUL_POS, aux_in=st["act"],
+                     alpha=1.0 / (1.0 - self.dropout) if self.dropout > 0 else 1.0, stream=sm)
+        else:
+            ctx.gemm(hip.NN, d_ff2, w["feed_forward.w_2.weight"], d_ffn, epilogue=hip.EPI_MUL, aux_in=st["dact"], stream=sm)
+        wgrad(d_ffn, st["n2"], "feed_forward.w_1.weight")
+        ctx.gemm(hip.NN, d_ffn, w["feed_forward.w_1.weight"], d_h0, stream=sm)
+        # d_x2 = d_out + LN2'(d_n2)  -> d_h2
+        hip.layernorm_bwd(st["x2"], w["sublayer.2.norm.a_2"], st["mean2"], st["rinv2"], d_h0, d_out, d_h2,
+                          g["sublayer.2.norm.a_2"], g["sublayer.2.norm.b_2"], ws, kind, self.eps, stream=sm)
+        # ---- sublayer 1: attention over the memory
+        d_proj = d_h2
+        if self.dropout > 0:
+            d_proj = ctx.buf("d_drop_src", (R, h))
+            hip.dropout_apply(d_h2, d_proj, *self._drop(ctx, self.SITE_SUBLAYER_SRC), stream=sm)
+        wgrad(d_proj, st["ctx_src"], "src_attn.linears.3.weight")
+        ctx.gemm(hip.NN, d_proj, w["src_attn.linears.3.weight"], d_h0, stream=sm)
+        self._attention_bwd(d_h0, d_qkv, self._src_views(st), ctx, site=self.SITE_SRC_ATTENTION, mask="none")
+        wgrad(d_qkv[:, :h], st["n_src"], "src_attn.linears.0.weight")
+        wgrads.append(hip.gemm_desc(hip.TN, d_qkv[:, h:], st["mem"], g["kv.weight"], accumulate=True,
+                                    colsum_out=g["kv.bias"], colsum_ws=ws))
+        ctx.gemm(hip.NN, d_qkv[:, :h], w["src_attn.linears.0.weight"], d_h0, stream=sm)        # d_n_src
+        ctx.gemm(hip.NN, d_qkv[:, h:], w["kv.weight"], d_mem, stream=sm)                       # gradient of the memory
+        # d_x1 = d_x2 + LN_src'(d_n_src)  -> d_h1
+        hip.layernorm_bwd(st["x1"], w["sublayer.1.norm.a_2"], st["mean_src"], st["rinv_src"], d_h0, d_h2, d_h1,
+                          g["sublayer.1.norm.a_2"], g["sublayer.1.norm.b_2"], ws, kind, self.eps, stream=sm)
+        flush()      # d_qkv, d_ffn and the first sublayers' gradient buffers are free again
+        # ---- sublayer 0: self-attention
+        d_proj0 = d_h1
+        if self.dropout > 0:
+            d_proj0 = ctx.buf("d_drop0", (R, h))
+            hip.dropout_apply(d_h1, d_proj0, *self._drop(ctx, self.SITE_SUBLAYER0), stream=sm)
+        wgrad(d_proj0, st["ctx"], "self_attn.linears.3.weight")
+        ctx.gemm(hip.NN, d_proj0, w["self_attn.linears.3.weight"], d_h0, stream=sm)
+        self._attention_bwd(d_h0, d_qkv, st, ctx, site=self.SITE_ATTENTION)
+        wgrad(d_qkv, st["n1"], "qkv.weight")
+        ctx.gemm(hip.NN, d_qkv, w["qkv.weight"], d_h0, stream=sm)
+        # d_x = d_x1 + LN0'(d_n1) + d_mem * dm/dx
+        hip.layernorm_bwd(st["x0"], w["sublayer.0.norm.a_2"], st["mean1"], st["rinv1"], d_h0, d_h1, d_x,
+                          g["sublayer.0.norm.a_2"], g["sublayer.0.norm.b_2"], ws, kind, self.eps, stream=sm)
+        hip.sqrt_one_minus_bwd(d_mem, st["mem"], d_x, accumulate=True, stream=sm)
+        flush()
         return d_x
 
 

@@ -243,6 +243,13 @@ int bb_attention_bwd(int dtype, int mask, int batch, int heads, int seq, int hea
 int bb_residual_add(int dtype, int64_t n, const void* a, const void* b, void* out,
                     void* stream);
 
+/* m = sqrt(1 - x), elementwise: the stand-in memory of DecoderLayerSimple.forward
+ * (DeepSpeedExamples/pipeline_parallelism/gpt2.py:31), and its backward dx (+)= dm * (-1 / (2 m))
+ * (accumulate != 0 adds to dx).  n a multiple of 8 (bf16) / 4 (fp32).                       */
+int bb_sqrt_one_minus_fwd(int dtype, int64_t n, const void* x, void* m, void* stream);
+int bb_sqrt_one_minus_bwd(int dtype, int64_t n, const void* dm, const void* m, void* dx,
+                          int accumulate, void* stream);
+
 /* out = act(x), elementwise: the activation of PositionwiseFeedForward (transformer.py:158) as a
  * bandwidth-bound pass of its own.  If dact != NULL it also receives act'(x), the factor autograd
  * applies in the backward pass; dact may be x itself (each element is read before it is

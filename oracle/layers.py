@@ -5,6 +5,8 @@ Follows DeepSpeedExamples/pipeline_parallelism/transformer.py of the reference:
   attention           transformer.py:106-146 (MultiHeadedAttention, masked_fill(mask==0,-1e9))
   feed_forward        transformer.py:149-158 (PositionwiseFeedForward)
   transformer_layer   transformer.py:91-103,161-172 (SublayerConnection + EncoderLayer, pre-LN)
+  decoder_layer       gpt2.py:20-34          (DecoderLayerSimple: self-attention, attention over
+                      m = sqrt(1 - x) of the layer's input, feed-forward; three pre-LN residual sublayers)
   script_tail         transformer.py:181,250 (final LayerNorm, then sum over the hidden dimension)
   bottleneck          resnet.py:49-75        (BottleNeck, bias-free convs, train-mode BN)
   batch_stats_from_strips  resnet.py:56,59,62 (nn.BatchNorm2d batch statistics, restated over
@@ -43,6 +45,7 @@ class TransformerCfg:
     mask: str = "none"            # none | causal | key_padding
     ln_eps: float = None
     dropout: float = 0.0          # the reference scripts run 0.1 (transformer.py:196); masks are handed in explicitly
+    decoder: bool = False         # the GPT-2 script's DecoderLayerSimple (gpt2.py:20-34) instead of EncoderLayer
 
     @property
     def eps(self):
@@ -51,8 +54,20 @@ class TransformerCfg:
         return 1e-6 if self.ln == "annotated" else 1e-5
 
 
+# registration order of DecoderLayerSimple's parameters (self_attn, src_attn, feed_forward, sublayer: gpt2.py:22-27)
+DECODER_PARAM_ORDER = tuple(
+    [f"self_attn.linears.{i}.{k}" for i in range(4) for k in ("weight", "bias")] +
+    [f"src_attn.linears.{i}.{k}" for i in range(4) for k in ("weight", "bias")] +
+    ["feed_forward.w_1.weight", "feed_forward.w_1.bias", "feed_forward.w_2.weight", "feed_forward.w_2.bias"] +
+    [f"sublayer.{i}.norm.{k}" for i in range(3) for k in ("a_2", "b_2")])
+
+
 def param_shapes(cfg):
     h, f = cfg.hidden, cfg.ffn
+    if cfg.decoder:
+        shape = lambda n: (f, h) if n == "feed_forward.w_1.weight" else (h, f) if n == "feed_forward.w_2.weight" else \
+            (f,) if n == "feed_forward.w_1.bias" else (h, h) if n.endswith("weight") else (h,)
+        return {n: shape(n) for n in DECODER_PARAM_ORDER}
     return {
         "sublayer.0.norm.a_2": (h,), "sublayer.0.norm.b_2": (h,),
         "self_attn.linears.0.weight": (h, h), "self_attn.linears.0.bias": (h,),
@@ -133,13 +148,16 @@ def drop(x, mask, p_drop):
     return x * mask.to(x.dtype).view_as(x) / (1.0 - p_drop)
 
 
-def attention(x, p, cfg, key_lens=None, prob_mask=None):
+def attention(x, p, cfg, key_lens=None, prob_mask=None, memory=None, prefix="self_attn"):
+    """``memory``: keys and values are projected from it instead of from ``x`` (MultiHeadedAttention(query, key, value)
+    with key = value = memory, gpt2.py:33), and no mask applies."""
     b, s, h = x.shape
     a, d = cfg.heads, cfg.hidden // cfg.heads
-    lin = lambda i, t: F.linear(t, p[f"self_attn.linears.{i}.weight"], p[f"self_attn.linears.{i}.bias"])
-    q, k, v = [lin(i, x).view(b, s, a, d).transpose(1, 2) for i in range(3)]
+    lin = lambda i, t: F.linear(t, p[f"{prefix}.linears.{i}.weight"], p[f"{prefix}.linears.{i}.bias"])
+    kv_in = x if memory is None else memory
+    q, k, v = [lin(i, t).view(b, s, a, d).transpose(1, 2) for i, t in ((0, x), (1, kv_in), (2, kv_in))]
     scores = torch.matmul(q, k.transpose(-2, -1)) / math.sqrt(d)
-    mask = build_mask(cfg, b, s, key_lens)
+    mask = build_mask(cfg, b, s, key_lens) if memory is None else None
     if mask is not None:
         scores = scores.masked_fill(~mask, -1e9)
     prob = drop(F.softmax(scores, dim=-1), prob_mask, cfg.dropout)          # transformer.py:125-126
@@ -153,9 +171,22 @@ def feed_forward(x, p, cfg, relu_mask=None, hidden_mask=None):
     return F.linear(a, p["feed_forward.w_2.weight"], p["feed_forward.w_2.bias"])
 
 
+def decoder_layer(x, p, cfg, key_lens=None, relu_mask=None, drop_masks=None):
+    """DecoderLayerSimple.forward (gpt2.py:29-34).  Dropout sites: 0 self-attention probabilities, 1 first sublayer,
+    4 memory-attention probabilities, 5 second sublayer, 2 feed-forward hidden, 3 last sublayer."""
+    dm = drop_masks or {}
+    norm = lambda t, i: layer_norm(t, p[f"sublayer.{i}.norm.a_2"], p[f"sublayer.{i}.norm.b_2"], cfg.ln, cfg.eps)
+    m = torch.sqrt(1 - x)                                                                              # gpt2.py:31
+    x = x + drop(attention(norm(x, 0), p, cfg, key_lens, dm.get(0)), dm.get(1), cfg.dropout)          # :32
+    x = x + drop(attention(norm(x, 1), p, cfg, None, dm.get(4), memory=m, prefix="src_attn"), dm.get(5), cfg.dropout)   # :33
+    return x + drop(feed_forward(norm(x, 2), p, cfg, relu_mask, dm.get(2)), dm.get(3), cfg.dropout)  # :34
+
+
 def transformer_layer(x, p, cfg, key_lens=None, relu_mask=None, drop_masks=None):
     """``drop_masks``: {site: 0/1 tensor} for the layer's four dropout sites (oracle.dropout.SITE_*): attention
     probabilities [b, heads, s, s], sublayer outputs [b, s, h], feed-forward hidden [b, s, ffn]."""
+    if cfg.decoder:
+        return decoder_layer(x, p, cfg, key_lens, relu_mask, drop_masks)
     dm = drop_masks or {}
     n1 = layer_norm(x, p["sublayer.0.norm.a_2"], p["sublayer.0.norm.b_2"], cfg.ln, cfg.eps)
     x = x + drop(attention(n1, p, cfg, key_lens, dm.get(0)), dm.get(1), cfg.dropout)      # transformer.py:103
@@ -168,6 +199,8 @@ def layer_drop_masks(cfg, base_seed, step, micro_batch, layer_idx, batch, seq):
     from . import dropout as od
     shapes = {od.SITE_ATTENTION: (batch, cfg.heads, seq, seq), od.SITE_SUBLAYER0: (batch, seq, cfg.hidden),
               od.SITE_FFN: (batch, seq, cfg.ffn), od.SITE_SUBLAYER1: (batch, seq, cfg.hidden)}
+    if cfg.decoder:
+        shapes.update({4: (batch, cfg.heads, seq, seq), 5: (batch, seq, cfg.hidden)})
     return {site: torch.from_numpy(od.mask(cfg.dropout, od.key(base_seed, step, micro_batch, layer_idx, site), shape))
             for site, shape in shapes.items()}
 

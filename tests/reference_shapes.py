@@ -3,7 +3,7 @@
 The reference's scripts cannot be imported here (``transformer.py`` imports ``deepspeed`` at module scope), so
 these small modules rebuild the *structure* those scripts give their layers -- attribute names, registration order
 and forward arithmetic of ``EncoderLayer`` / ``LayerNorm`` (DeepSpeedExamples/pipeline_parallelism/
-transformer.py:77-172) and ``BottleNeck`` (resnet.py:49-75) -- so that ``state_dict()`` keys, their order and the
+transformer.py:77-172), ``DecoderLayerSimple`` (gpt2.py:20-34) and ``BottleNeck`` (resnet.py:49-75) -- so that ``state_dict()`` keys, their order and the
 forward results are the reference's.  They are torch-autograd modules: the parity oracle for what this package
 takes over from such modules."""
 import math
@@ -72,6 +72,25 @@ class RefEncoderLayer(nn.Module):
     def forward(self, x, mask=None):
         x = self.sublayer[0](x, lambda t: self.self_attn(t, t, t, mask))
         return self.sublayer[1](x, self.feed_forward)
+
+
+class RefDecoderLayer(nn.Module):
+    """Structure of ``DecoderLayerSimple`` (gpt2.py:20-34): attribute names and registration order self_attn, src_attn,
+    feed_forward, sublayer[0..2]; the memory of the second attention is sqrt(1 - x) of the layer's input."""
+
+    def __init__(self, size, heads, d_ff, dropout):
+        super().__init__()
+        self.size = size
+        self.self_attn = RefAttention(heads, size, dropout)
+        self.src_attn = RefAttention(heads, size, dropout)
+        self.feed_forward = RefFeedForward(size, d_ff, dropout)
+        self.sublayer = nn.ModuleList([RefSublayer(size, dropout) for _ in range(3)])
+
+    def forward(self, x):
+        m = torch.sqrt(1 - x)
+        x = self.sublayer[0](x, lambda t: self.self_attn(t, t, t))
+        x = self.sublayer[1](x, lambda t: self.src_attn(t, m, m))
+        return self.sublayer[2](x, self.feed_forward)
 
 
 class RefBottleNeck(nn.Module):

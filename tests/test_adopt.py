@@ -5,9 +5,9 @@ the arenas runs no kernel in fp32."""
 import pytest
 import torch
 
-from bamboo_amd import (BottleNeck, FinalLayerNorm, LayerSpec, MSELoss, PipelineError, PipelineModule, SumLast,
+from bamboo_amd import (BottleNeck, DecoderLayer, FinalLayerNorm, LayerSpec, MSELoss, PipelineError, PipelineModule, SumLast,
                         TransformerLayer)
-from tests.reference_shapes import RefBottleNeck, RefEncoderLayer, RefLayerNorm
+from tests.reference_shapes import RefBottleNeck, RefDecoderLayer, RefEncoderLayer, RefLayerNorm
 
 
 def encoder_script_layers(n=4, d=32, h=4, ff=64, p=0.0):
@@ -172,3 +172,34 @@ def test_seed_layers_gives_the_owner_and_the_shadow_the_same_weights():
     seen = []
     PipelineModule(specs(), stage_id=3, seed_fn=lambda s: (seen.append(s), torch.manual_seed(s)), **kw)
     assert seen == [77 + i for i in range(owner.parts[3], owner.parts[4]) if i < 7]
+
+
+def test_gpt2_script_layer_list_is_taken_over():
+    """The layer list of the reference's GPT-2 script (``GPT2Simple.join_layers``, gpt2.py:149-150: decoder layers, the
+    final norm, the sum over the hidden dimension): every ``DecoderLayerSimple`` becomes a :class:`DecoderLayer` with
+    the module's 26 parameters under the reference's keys, its state travels in the module's ``state_dict`` order,
+    and the keys / values weights of the memory attention sit side by side in the arena (one product)."""
+    torch.manual_seed(8)
+    layers = [RefDecoderLayer(32, 4, 64, 0.1) for _ in range(4)] + [RefLayerNorm(32), lambda x: x.sum(-1)]
+    model = PipelineModule(layers, num_stages=2, loss_fn=torch.nn.MSELoss(), partition_method="uniform", stage_id=0,
+                           dtype=torch.float32, device="cpu")
+    built = model.func_buckets[0]
+    assert [type(b) for b in built] == [DecoderLayer] * 3
+    assert (built[0].hidden, built[0].heads, built[0].ffn, built[0].activation, built[0].ln, built[0].mask) == (32, 4, 64, "relu", "annotated", "none")
+    assert abs(built[0].dropout - 0.1) < 1e-7
+    sp = model.stage_params[0]
+    named = sp.named(sp.master)
+    for li in range(3):
+        want = dict(layers[li].named_parameters())
+        assert len(want) == 26
+        for name, prm in want.items():
+            assert torch.equal(named[f"{li}.{name}"], prm.detach()), (li, name)
+        assert list(model.layer_state_dict(li)) == list(layers[li].state_dict())
+    kv = built[1].w["kv.weight"]
+    assert kv.shape == (64, 32) and torch.equal(kv[:32], named["1.src_attn.linears.1.weight"]) and torch.equal(kv[32:], named["1.src_attn.linears.2.weight"])
+    assert built[0].num_params() == sum(p.numel() for p in layers[0].parameters())
+    # two attention modules that disagree on the heads are refused
+    odd = RefDecoderLayer(32, 4, 64, 0.0)
+    odd.src_attn.h = 2
+    with pytest.raises(PipelineError, match="number of heads"):
+        PipelineModule([odd], num_stages=1, stage_id=0, dtype=torch.float32, device="cpu")

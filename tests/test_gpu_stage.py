@@ -988,3 +988,159 @@ def test_gradient_clipping_in_the_optimizer_step(hiplib):
         m_got = sp.view(sp.exp_avg, n).cpu().numpy()
         assert float(np.abs(m_got - m_ref).max()) < 1e-4 * float(np.abs(m_ref).max()) + 1e-12, n
     assert not torch.equal(plain.module.stage_params[sid].exp_avg, tight.module.stage_params[sid].exp_avg)
+
+
+def _decoder_stage(dtype, variant, dropout=0.0, dead_from=None, grad_mode="queue"):
+    """Engine (stage 1 of 4, one DecoderLayer per stage, redundant forwards on) and oracle on the same weights and
+    inputs drawn from U(0, 0.4): the memory sqrt(1 - x) of every layer stays real (the sublayers move the stream by
+    a few hundredths at these weight scales)."""
+    from bamboo_amd import DecoderLayer
+    hid, heads, ffn, S, sid, mb, M, seq = 128, 2, 256, 4, 1, 2, 4, 64
+    specs = [LayerSpec(DecoderLayer, hid, heads, ffn, dropout=dropout, **variant) for _ in range(S)]
+    model = PipelineModule(specs, num_stages=S, partition_method="uniform", stage_id=sid, dtype=dtype, device=DEV)
+    q = SeededActivationQueue((mb, seq, hid), dtype, M, stage_ids=[sid, sid + 1], seed=7, grad_mode=grad_mode, device=DEV)
+    g = torch.Generator().manual_seed(77)
+    q.activations = [(0.4 * torch.rand(mb, seq, hid, generator=g)).to(dtype).to(DEV) for _ in range(M)]
+    cfg = {"train_micro_batch_size_per_gpu": mb, "gradient_accumulation_steps": M, "bf16": {"enabled": dtype == torch.bfloat16}}
+    engine, _, _, _ = bamboo_amd.initialize(model=model, config=cfg, redundancy_level=1, eager_recovery=True,
+                                            activation_queue=q, install_signal_handler=False)
+    ocfg = ol.TransformerCfg(hidden=hid, heads=heads, ffn=ffn, decoder=True, dropout=dropout, **variant)
+    st = OracleStage(ocfg, list(range(S + 1)), sid, M, dtype=torch.float64, redundancy_level=1, eager=True)
+    for s_ in list(st.params):
+        sp = engine.module.stage_params[s_]
+        named = sp.named(sp.compute)
+        assert set(named) == set(st.named_params(s_))
+        for key, t in st.named_params(s_).items():
+            with torch.no_grad():
+                t.copy_(named[key].double().cpu())
+    acts = [a.double().cpu() for a in q.activations]
+    if grad_mode == "queue":
+        peer = OraclePeer(acts, M, grads={s_: [t.double().cpu() for t in gs] for s_, gs in q.grads.items()})
+    else:
+        peer = OraclePeer(acts, M, targets={s_: [t.double().cpu() for t in ts] for s_, ts in q.targets.items()})
+    return engine, q, st, peer, (hid, mb, M, seq, sid)
+
+
+@pytest.mark.parametrize("dtype,variant", [(torch.float32, REFERENCE_VARIANT), (torch.float32, GPT_VARIANT), (torch.bfloat16, GPT_VARIANT)],
+                         ids=["fp32-script-variant", "fp32-gpt", "bf16-gpt"])
+def test_decoder_stage_matches_oracle_with_rc(hiplib, dtype, variant):
+    """A stage of the GPT-2 script's layers (DecoderLayerSimple, gpt2.py:20-34: self-attention, attention over
+    sqrt(1 - x) of the layer input, feed-forward) with redundant forwards: own and redundant outputs, the gradient
+    sent upstream (which also flows through the memory) and all 26 parameter gradients of the own layer against
+    the fp64 oracle; the shadow layer's gradients stay zero."""
+    engine, q, st, peer, (hid, mb, M, seq, sid) = _decoder_stage(dtype, variant)
+    keep = {}
+    with NoStep(engine):
+        engine._clean_pipe_buffers = lambda: keep.update({k: list(v) for k, v in engine.pipe_buffers.items()})
+        engine.train_batch()
+    torch.cuda.synchronize()
+    bufs, _ = st.run_batch(peer, optimizer_step=False)
+    t_act, t_grad = (1e-5, 1e-4) if dtype == torch.float32 else (2e-2, 2e-2)
+    rel_err.lowp = dtype == torch.bfloat16
+    for k in range(M):
+        for s_ in (sid, sid + 1):
+            want = bufs["out"][(s_, k)].detach().view(mb * seq, hid)
+            assert not torch.isnan(want).any()
+            assert rel_err(keep[f"output_{s_}"][k], want) < t_act, (s_, k)
+        assert rel_err(keep[f"input_grad_{sid}"][k], bufs["sent_grad"][(sid, k)].view(mb * seq, hid)) < t_grad, k
+    ref = st.named_grads(sid)
+    assert len(ref) == 26
+    for name, g in engine.module.get_named_grad(sid):
+        assert rel_err(g, ref[name], grad_floor(ref)) < t_grad, name
+    for name, g in engine.module.get_named_grad(sid + 1):
+        assert float(g.abs().max()) == 0.0
+    # the redundant forward is bit-equal to the same layer run as a stage of its own on the same input
+    from bamboo_amd import DecoderLayer
+    heads, ffn, S = engine.module.func_buckets[sid][0].heads, engine.module.func_buckets[sid][0].ffn, engine.num_stages
+    specs = [LayerSpec(DecoderLayer, hid, heads, ffn, **variant) for _ in range(S)]
+    model2 = PipelineModule(specs, num_stages=S, partition_method="uniform", stage_id=sid + 1, dtype=dtype, device=DEV)
+    ctx2 = model2.prepare_context([sid + 1], mb, seq)
+    model2.allocate_stash(sid + 1, ctx2, 1)
+    for k in range(M):
+        normal = model2.forward(keep[f"output_{sid}"][k], sid + 1, slot=0, ctx=ctx2)
+        torch.cuda.synchronize()
+        assert torch.equal(normal, keep[f"output_{sid + 1}"][k]), k
+
+
+@pytest.mark.parametrize("dtype,dropout", [(torch.float32, 0.0), (torch.bfloat16, 0.0), (torch.float32, 0.1)], ids=["fp32", "bf16", "fp32-dropout"])
+def test_decoder_stage_failover_matches_oracle(hiplib, dtype, dropout):
+    """The successor is lost at micro-batch 2: the promoted decoder layer's backward passes run from the stash of the
+    redundant forwards (which left the activation derivative out: it is produced first), with dropout at the layer's
+    six sites making the redundant forward's decisions again; gradients of both stages and the loss against the
+    oracle's run of the same stream."""
+    variant = dict(GPT_VARIANT)
+    engine, q, st, peer, (hid, mb, M, seq, sid) = _decoder_stage(dtype, variant, dropout=dropout, dead_from=2, grad_mode="mse")
+    true_grads = []
+    for k in range(M):
+        o1 = st.forward(peer.activations[k], sid, drop_id=(0, k)).detach().requires_grad_(True)
+        o2 = st.forward(o1, sid + 1, drop_id=(0, k))
+        (torch.nn.functional.mse_loss(o2, peer.targets[sid + 1][k]) / M).backward()
+        true_grads.append(o1.grad)
+    for s_ in st.params.values():
+        for p in s_:
+            for t in p.values():
+                t.grad = None
+    peer.targets = {sid + 1: peer.targets[sid + 1]}
+    peer.grads = {sid: true_grads}
+    peer.dead_from, peer.dead_stage = 2, sid
+    st.run_batch(peer, optimizer_step=False)
+    q.set_grads(sid, [g.view(mb, seq, hid) for g in true_grads])
+    q.targets.pop(sid)
+    orig_send = q.send_activation
+    q.send_activation = lambda k, t, stage_id, stream=None: (q._check_alive(k, stage_id) if stage_id == sid
+                                                              else orig_send(k, t, stage_id, stream=stream))
+    q.preempt_successor(2, sid)
+    with NoStep(engine):
+        loss = engine.train_batch()
+    assert engine.stage_ids == [sid, sid + 1]
+    tg = 1e-4 if dtype == torch.float32 else 2e-2
+    rel_err.lowp = dtype == torch.bfloat16
+    for s_ in (sid, sid + 1):
+        ref = st.named_grads(s_)
+        for name, g in engine.module.get_named_grad(s_):
+            assert rel_err(g, ref[name], grad_floor(ref)) < tg, (s_, name)
+    assert abs(float(loss) - float(peer.loss) / M) < tg * max(1.0, float(peer.loss) / M)
+
+
+def test_gpt2_script_layers_taken_over_run_as_the_last_stage(hiplib):
+    """The GPT-2 script's own layer list (``GPT2Simple.join_layers``, gpt2.py:149-150: DecoderLayerSimple modules, the
+    final LayerNorm, ``x.sum(-1)``) with ``nn.MSELoss()``, handed over as it is: the last stage (one decoder layer,
+    norm, sum) on the HIP kernels against torch autograd on the modules themselves (fp32), inputs in (0, 0.4)."""
+    from tests.reference_shapes import RefDecoderLayer, RefLayerNorm
+    hid, heads, ffn, mb, M, seq = 128, 2, 256, 2, 4, 64
+    torch.manual_seed(13)
+    mods = [RefDecoderLayer(hid, heads, ffn, 0.0) for _ in range(2)] + [RefLayerNorm(hid)]
+    with torch.no_grad():
+        for m in mods:
+            for prm in m.parameters():
+                prm.add_(0.02 * torch.randn_like(prm))
+    layers = mods + [lambda x: x.sum(-1)]
+    g = torch.Generator().manual_seed(14)
+    labels = [torch.randn(mb, seq, generator=g) for _ in range(M)]
+    model = PipelineModule(layers, num_stages=2, partition_method="custom", custom_partitions=[0, 1, 4], stage_id=1,
+                           loss_fn=torch.nn.MSELoss(), dtype=torch.float32, device=DEV)
+    q = SeededActivationQueue((mb, seq, hid), torch.float32, M, stage_ids=[1], seed=5, device=DEV)
+    q.activations = [(0.4 * torch.rand(mb, seq, hid, generator=g)).to(DEV) for _ in range(M)]
+    cfg = {"train_micro_batch_size_per_gpu": mb, "gradient_accumulation_steps": M}
+    engine, _, _, _ = bamboo_amd.initialize(model=model, config=cfg, activation_queue=q, install_signal_handler=False,
+                                            training_data=[(torch.zeros(1), y) for y in labels])
+    with NoStep(engine):
+        loss = engine.train_batch()
+    torch.cuda.synchronize()
+    total, xgrads = 0.0, []
+    for k in range(M):
+        x = q.activations[k].cpu().clone().requires_grad_(True)
+        l = torch.nn.functional.mse_loss(layers[3](mods[2](mods[1](x))), labels[k])
+        (l / M).backward()
+        total += float(l)
+        xgrads.append(x.grad)
+    rel_err.lowp = False
+    assert abs(float(loss) - total / M) < 1e-5 * total / M
+    ref = {f"{li}.{n}": p.grad for li in (1, 2) for n, p in mods[li].named_parameters()}
+    got = dict(engine.module.get_named_grad(1))
+    assert set(got) == set(ref)
+    floor = grad_floor(ref)
+    for name, gr in got.items():
+        assert rel_err(gr, ref[name], floor) < 1e-4, name
+    for k in range(M):
+        assert rel_err(q.sent_grads[(1, k)], xgrads[k].view(mb * seq, hid)) < 1e-4

@@ -79,6 +79,60 @@ def test_layer_matches_torch_encoder_layer():
     torch.testing.assert_close(ol.transformer_layer(x, p, cfg_c), ref(x, src_mask=cm, is_causal=True), rtol=1e-9, atol=1e-9)
 
 
+@pytest.mark.parametrize("mistake", [None, "memory_from_stream", "unnormalised_queries", "memory_normalised", "wrong_sign"])
+def test_decoder_layer_against_library_attention(mistake):
+    """``oracle.layers.decoder_layer`` (gpt2.py:20-34) against a composition of library routines: both attentions by
+    ``nn.MultiheadAttention`` (self: query = key = value = the normalised stream; memory: query = the normalised
+    stream, key = value = sqrt(1 - x) of the layer's INPUT, un-normalised), LayerNorm by the closed form, the
+    feed-forward by ``F.linear``; output and every gradient in fp64.  Four plausible mistakes in the composition
+    (memory taken from the running stream instead of the layer input, queries not normalised, memory normalised,
+    sqrt(1 + x)) each break the agreement."""
+    torch.manual_seed(6)
+    h, a, f, b, s = 32, 4, 64, 2, 9
+    cfg = ol.TransformerCfg(hidden=h, heads=a, ffn=f, decoder=True)
+    p = {k: (v.double() + 0.1 * torch.randn(v.shape, dtype=torch.float64)).requires_grad_(True)
+         for k, v in ol.init_params(cfg, 3, std=0.3).items()}
+    assert list(p) == list(ol.DECODER_PARAM_ORDER) and len(p) == 26
+    x = (0.9 * torch.rand(b, s, h, dtype=torch.float64)).requires_grad_(True)
+    dy = torch.randn(b, s, h, dtype=torch.float64)
+    out = ol.decoder_layer(x, p, cfg)
+    grads = torch.autograd.grad(out, [x] + list(p.values()), dy)
+
+    def mha(prefix, q_in, kv_in):
+        m = torch.nn.MultiheadAttention(h, a, batch_first=True, dtype=torch.float64)
+        with torch.no_grad():
+            m.in_proj_weight.copy_(torch.cat([p[f"{prefix}.linears.{i}.weight"] for i in range(3)]))
+            m.in_proj_bias.copy_(torch.cat([p[f"{prefix}.linears.{i}.bias"] for i in range(3)]))
+            m.out_proj.weight.copy_(p[f"{prefix}.linears.3.weight"])
+            m.out_proj.bias.copy_(p[f"{prefix}.linears.3.bias"])
+        return m, m(q_in, kv_in, kv_in, need_weights=False)[0]
+    ln = lambda t, i: p[f"sublayer.{i}.norm.a_2"] * (t - t.mean(-1, keepdim=True)) / (t.std(-1, keepdim=True) + 1e-6) + p[f"sublayer.{i}.norm.b_2"]
+    x2 = x.detach().clone().requires_grad_(True)
+    mem = torch.sqrt(1 + x2) if mistake == "wrong_sign" else torch.sqrt(1 - x2)
+    m0, y0 = mha("self_attn", ln(x2, 0), ln(x2, 0))
+    x_1 = x2 + y0
+    if mistake == "memory_from_stream":
+        mem = torch.sqrt(1 - x_1.clamp(max=0.99))
+    if mistake == "memory_normalised":
+        mem = ln(mem, 1)
+    m1, y1 = mha("src_attn", x_1 if mistake == "unnormalised_queries" else ln(x_1, 1), mem)
+    x_2 = x_1 + y1
+    ref = x_2 + F.linear(torch.relu(F.linear(ln(x_2, 2), p["feed_forward.w_1.weight"], p["feed_forward.w_1.bias"])),
+                         p["feed_forward.w_2.weight"], p["feed_forward.w_2.bias"])
+    ok = bool(torch.allclose(out, ref, rtol=1e-9, atol=1e-10))
+    assert ok == (mistake is None)
+    if mistake is None:
+        gx, = torch.autograd.grad(ref, [x2], dy, retain_graph=True)
+        assert torch.allclose(grads[0], gx, rtol=1e-8, atol=1e-10)
+        # parameter gradients: the library modules hold copies, so compare through them
+        ref.backward(dy)
+        names = list(p)
+        for prefix, mod in (("self_attn", m0), ("src_attn", m1)):
+            gw = torch.cat([grads[1 + names.index(f"{prefix}.linears.{i}.weight")] for i in range(3)])
+            assert torch.allclose(gw, mod.in_proj_weight.grad, rtol=1e-8, atol=1e-10)
+            assert torch.allclose(grads[1 + names.index(f"{prefix}.linears.3.weight")], mod.out_proj.weight.grad, rtol=1e-8, atol=1e-10)
+
+
 def test_script_tail_equals_the_module_form():
     """final LayerNorm + sum over the hidden dimension against the stand-in of the reference's LayerNorm module
     followed by the script's lambda, values and gradients."""
