@@ -1436,6 +1436,90 @@ __global__ __launch_bounds__(1024) void bn_bwd_finish_apply_kernel(int rows, int
     }
 }
 
+// The same after a kernel that left the sums per 32-row strip (the GEMM or convolution that produced the gradient,
+// which has the ReLU mask applied already): a block adds up the strips of its 64 channels -- sixteen thread groups
+// take the strips q, q + 16, ... in that order, the sixteen sums are added in group order: the same bits in every
+// block -- and applies the folded dx = k g + a x + b to its rows.
+template <typename T>
+__global__ __launch_bounds__(1024) void bn_bwd_strips_apply_kernel(int rows, int cols, const float* __restrict__ strips,
+                                                                   const T* __restrict__ x, const float* __restrict__ mean,
+                                                                   const float* __restrict__ rstd, const T* __restrict__ gamma,
+                                                                   const T* __restrict__ gin, T* __restrict__ dx,
+                                                                   float* __restrict__ dgamma, float* __restrict__ dbeta) {
+    constexpr int VEC = Elem<T>::VEC, LPR = 64 / VEC, RPP = 1024 / LPR;
+    __shared__ float red[2][16][64];
+    __shared__ float fold[3][64];
+    const int lane = threadIdx.x & 63, grp = threadIdx.x >> 6;
+    const int c = min(blockIdx.x * 64 + lane, cols - 1);
+    const int vc = (threadIdx.x % LPR) * VEC, c0 = blockIdx.x * 64 + vc;
+    const int per = (rows + gridDim.y - 1) / gridDim.y;
+    const int r0 = blockIdx.y * per + threadIdx.x / LPR, r1 = min(rows, ((int)blockIdx.y + 1) * per);
+    const bool first = c0 < cols && r0 < r1;
+    float xv[VEC], gv[VEC];
+    if (first) {
+        const int64_t off = (int64_t)r0 * cols + c0;
+        load_vec(x + off, xv);
+        load_vec(gin + off, gv);
+    }
+    const int nstrips = (rows + 31) / 32;
+    float s0 = 0.f, s1 = 0.f;
+    for (int q0 = grp; q0 < nstrips; q0 += 16 * 4) {
+        // four strips' loads go out together
+        float t0[4], t1[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int q = q0 + 16 * j;
+            t0[j] = q < nstrips ? strips[((int64_t)q * 2) * cols + c] : 0.f;
+            t1[j] = q < nstrips ? strips[((int64_t)q * 2 + 1) * cols + c] : 0.f;
+        }
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            s0 += t0[j];
+            s1 += t1[j];
+        }
+    }
+    red[0][grp][lane] = s0;
+    red[1][grp][lane] = s1;
+    __syncthreads();
+    if (grp == 0) {
+        float a0 = 0.f, a1 = 0.f;
+#pragma unroll
+        for (int q = 0; q < 16; ++q) {
+            a0 += red[0][q][lane];
+            a1 += red[1][q][lane];
+        }
+        const float rs = rstd[c], k = Elem<T>::load(gamma + c) * rs;
+        const float ka = -k * (a1 / (float)rows) * rs;
+        fold[0][lane] = k;
+        fold[1][lane] = ka;
+        fold[2][lane] = -k * (a0 / (float)rows) - ka * mean[c];
+        if (blockIdx.y == 0 && blockIdx.x * 64 + lane < cols) {
+            dbeta[c] += a0;
+            dgamma[c] += a1;
+        }
+    }
+    __syncthreads();
+    if (c0 >= cols) return;
+    float k[VEC], ka[VEC], kb[VEC];
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) {
+        k[e] = fold[0][vc + e];
+        ka[e] = fold[1][vc + e];
+        kb[e] = fold[2][vc + e];
+    }
+    for (int r = r0; r < r1; r += RPP) {
+        const int64_t off = (int64_t)r * cols + c0;
+        if (r != r0) {
+            load_vec(x + off, xv);
+            load_vec(gin + off, gv);
+        }
+        float o[VEC];
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) o[e] = fmaf(k[e], gv[e], fmaf(ka[e], xv[e], kb[e]));
+        store_vec(dx + off, o);
+    }
+}
+
 extern "C" int64_t bb_bn_workspace(int cols) { return (int64_t)BN_SPLITS * 2 * cols + 2 * cols; }
 
 static int check_bn(const char* name, int dtype, int rows, int cols) {
@@ -1510,6 +1594,21 @@ extern "C" int bb_batchnorm_bwd(int dtype, int rows, int cols, const void* x, co
         hipLaunchKernelGGL((bn_colred_kernel<float, 2>), grid, block, 0, st, rows, cols, (const float*)x, mean, rstd, (const float*)dy, (const float*)relu_out, workspace);
         hipLaunchKernelGGL(bn_bwd_finish_apply_kernel<float>, agrid, dim3(1024), 0, st, rows, cols, workspace, (const float*)x, mean, rstd, (const float*)gamma, (const float*)dy, (const float*)relu_out, (float*)dx, (float*)g_out, dgamma, dbeta);
     }
+    BB_LAUNCH_CHECK();
+    return BB_OK;
+}
+
+extern "C" int bb_batchnorm_bwd_strips(int dtype, int rows, int cols, const void* x, const void* gamma, const float* mean,
+                                       const float* rstd, const void* g, const float* strips, void* dx, float* dgamma,
+                                       float* dbeta, void* stream) {
+    int rc = check_bn("bb_batchnorm_bwd_strips", dtype, rows, cols);
+    if (rc) return rc;
+    BB_REQUIRE(dtype == BB_BF16, "bb_batchnorm_bwd_strips: bf16 only (the kernels that leave the strip sums are)");
+    BB_REQUIRE(x && gamma && mean && rstd && g && strips && dx && dgamma && dbeta, "bb_batchnorm_bwd_strips: null pointer");
+    const int slabs = (cols + 63) / 64;
+    dim3 agrid(slabs, max(4, min(64, 256 / slabs)));   // about one block per CU
+    hipLaunchKernelGGL(bn_bwd_strips_apply_kernel<bf16>, agrid, dim3(1024), 0, (hipStream_t)stream, rows, cols, strips, (const bf16*)x,
+                       mean, rstd, (const bf16*)gamma, (const bf16*)g, (bf16*)dx, dgamma, dbeta);
     BB_LAUNCH_CHECK();
     return BB_OK;
 }

@@ -86,6 +86,18 @@ static int launch_bf16_dma_stats(GemmArgs& g, hipStream_t st) {
     return BB_OK;
 }
 
+template <int BM, int BN, int WM, int WN>
+static int launch_bf16_dma_bnbwd(GemmArgs& g, const BnBwdArgs& bn, hipStream_t st) {
+    constexpr int smem = 3 * (BM + BN) * 64 * 2;
+    auto kern = gemm_bf16_dma_bnbwd_kernel<BM, BN, WM, WN>;
+    BB_HIP_CHECK(bb_allow_dynamic_lds((const void*)kern, smem));
+    g.tiles_m = (g.M + BM - 1) / BM;
+    g.tiles_n = (g.N + BN - 1) / BN;
+    hipLaunchKernelGGL(kern, dim3(g.tiles_m * g.tiles_n), dim3(WM * WN * 64), smem, st, g, bn);
+    BB_LAUNCH_CHECK();
+    return BB_OK;
+}
+
 // DMA kernels need K % 32 == 0 and at least one full vector of rows; tile by problem size
 enum DmaTile { D_NONE = 0, D256x256w8db, D256x128w8db, D128x128s3, D256x256k64, D256x128k64s3, D128x128k64, D128x64k64s3, D128x64s3,
                D64x128k64s3, D64x128s3, D256x192k64, D256x256p };
@@ -307,6 +319,39 @@ extern "C" int bb_gemm_strip_stats_supported(const bb_gemm_desc* d) {
 }
 extern "C" int64_t bb_strip_stats_workspace(int rows, int cols) { return (int64_t)((rows + 31) / 32) * 3 * cols; }
 
+extern "C" int64_t bb_bn_bwd_strips_workspace(int rows, int cols) { return (int64_t)((rows + 31) / 32) * 2 * cols; }
+
+static int check_bn_bwd_stats(const char* name, const bb_bn_bwd_stats* bn) {
+    BB_REQUIRE(bn && bn->x && bn->mean && bn->rstd && bn->strips, "%s: null pointer in bb_bn_bwd_stats", name);
+    BB_REQUIRE(((uintptr_t)bn->x % 16) == 0 && ((uintptr_t)bn->mean % 16) == 0 && ((uintptr_t)bn->rstd % 16) == 0 &&
+               ((uintptr_t)bn->strips % 16) == 0, "%s: the bb_bn_bwd_stats operands must be 16-byte aligned", name);
+    return BB_OK;
+}
+
+extern "C" int bb_gemm_bn_bwd_supported(const bb_gemm_desc* d) {
+    return d && d->dtype == BB_BF16 && d->c_dtype == BB_BF16 && d->layout == BB_NN && d->nb1 <= 1 && d->nb2 <= 1 &&
+           d->M >= 128 && d->N >= 128 && d->N % 8 == 0 && d->K >= 128 && d->K % 64 == 0 && d->conv_c == 0 && !d->colsum_out &&
+           !d->strip_stats && !d->bias && !d->accumulate && d->alpha == 1.0f && d->dropout_p == 0.f && d->ldc == d->N &&
+           (d->ldaux == 0 || d->ldaux == d->N) &&
+           (d->epilogue == BB_EPI_NONE || (d->epilogue == BB_EPI_RESIDUAL && d->resid) || (d->epilogue == BB_EPI_MUL_POS && d->aux_in));
+}
+
+extern "C" int bb_gemm_bn_bwd(const bb_gemm_desc* d, const bb_bn_bwd_stats* bn, void* stream) {
+    BB_REQUIRE(bb_gemm_bn_bwd_supported(d), "bb_gemm_bn_bwd: needs an unbatched bf16 BB_NN problem with a contiguous bf16 C, M >= 128, "
+               "N >= 128, N %% 8 == 0, K >= 128, K %% 64 == 0, alpha = 1, no bias, epilogue BB_EPI_NONE, BB_EPI_RESIDUAL or BB_EPI_MUL_POS");
+    int rc = check_bn_bwd_stats("bb_gemm_bn_bwd", bn);
+    if (rc) return rc;
+    GemmArgs g;
+    int64_t batches;
+    bool ta, tb;
+    rc = fill_args(d, g, batches, ta, tb);
+    if (rc) return rc;
+    const BnBwdArgs b = {bn->x, bn->mean, bn->rstd, bn->strips};
+    // the tile the plain product of this shape would take, where it is one of the two built with the sums
+    if (pick_dma_tile(d->M, d->N, d->K, 1, BB_NN) == D256x128k64s3) return launch_bf16_dma_bnbwd<256, 128, 4, 2>(g, b, (hipStream_t)stream);
+    return launch_bf16_dma_bnbwd<64, 128, 2, 2>(g, b, (hipStream_t)stream);
+}
+
 extern "C" int bb_gemm(const bb_gemm_desc* d, void* stream) {
     if (d && d->conv_c != 0) return bb_gemm_grouped(d, 1, stream);   // only the grouped kernel gathers a patch-matrix B
     if (d && d->strip_stats) {
@@ -409,6 +454,45 @@ extern "C" int bb_conv3x3(int dtype, int mode, int n, int h, int w, int cin, int
     cv.b_every = cout / 64;
     cv.b_wrap = -(int64_t)cout * g.ldb - cin;
     return launch_conv3x3<64, 128, 2, 4, true, 3>(g, cv, st);
+}
+
+extern "C" int bb_conv3x3_dgrad_bn(int dtype, int n, int h, int w, int cin, int cout, const void* src, const void* weight, void* dst,
+                                   const void* relu_out, const bb_bn_bwd_stats* bn, void* stream) {
+    BB_REQUIRE(src && weight && dst, "bb_conv3x3_dgrad_bn: null operand");
+    BB_REQUIRE(bb_conv3x3_supported(dtype, BB_CONV_DGRAD, n, h, w, cin, cout),
+               "bb_conv3x3_dgrad_bn: unsupported problem (see bb_conv3x3): dtype %d n %d h %d w %d cin %d cout %d", dtype, n, h, w, cin, cout);
+    BB_REQUIRE(((uintptr_t)src % 16) == 0 && ((uintptr_t)weight % 16) == 0 && ((uintptr_t)dst % 16) == 0 && ((uintptr_t)relu_out % 16) == 0,
+               "bb_conv3x3_dgrad_bn: operands must be 16-byte aligned");
+    int rc = check_bn_bwd_stats("bb_conv3x3_dgrad_bn", bn);
+    if (rc) return rc;
+    GemmArgs g = {};
+    ConvArgs cv = {};
+    g.M = n * h * w;
+    g.N = cin;
+    g.K = 9 * cout;
+    g.nb2 = 1;
+    g.A = src;
+    g.C = dst;
+    g.lda = cout;
+    g.ldc = g.ldaux = g.N;
+    g.alpha = 1.f;
+    g.epilogue = relu_out ? BB_EPI_MUL_POS : BB_EPI_NONE;
+    g.aux_in = relu_out;
+    cv.h = h; cv.w = w; cv.c = cout;
+    // the flipped filter read in place, as in bb_conv3x3
+    g.B = (const bf16*)weight + 8 * (int64_t)cin;
+    g.ldb = 9 * (int64_t)cin;
+    cv.b_every = cout / 64;
+    cv.b_wrap = -(int64_t)cout * g.ldb - cin;
+    constexpr int BM = 64, BN = 128, STAGES = 3, smem = STAGES * (BM + BN) * 64 * 2;
+    auto kern = conv3x3_bf16_igemm_bnbwd_kernel<BM, BN, 2, 4, STAGES>;
+    BB_HIP_CHECK(bb_allow_dynamic_lds((const void*)kern, smem));
+    g.tiles_m = (g.M + BM - 1) / BM;
+    g.tiles_n = (g.N + BN - 1) / BN;
+    const BnBwdArgs b = {bn->x, bn->mean, bn->rstd, bn->strips};
+    hipLaunchKernelGGL(kern, dim3(g.tiles_m * g.tiles_n), dim3(2 * 4 * 64), smem, (hipStream_t)stream, g, cv, b);
+    BB_LAUNCH_CHECK();
+    return BB_OK;
 }
 
 template <bool TA, bool TB, bool CONVB = false> static int launch_grouped(GroupedArgs& G, hipStream_t st) {

@@ -19,6 +19,15 @@ struct GemmArgs {
     float* strip_stats;  // [ceil(M / 32)][3][N]: per 32-row strip and output column (pivot, sum (c - pivot), sum (c - pivot)^2)
     DropKey drop;        // dropout on the product after bias and activation, before the residual (thresh 0: none)
 };
+// Backward statistics of the batch normalisation whose (ReLU'd) output the product is the gradient of: the kernels
+// built with STATS = 2 leave, per 32-row strip and column, sum g and sum g * xhat of the stored (masked, bf16-rounded)
+// gradient g, with xhat = (x - mean) * rstd of the normalisation's input x ([M, N], rows ldc apart like C).
+struct BnBwdArgs {
+    const void* x;
+    const float* mean;
+    const float* rstd;
+    float* strips;   // [ceil(M / 32)][2][N]
+};
 // keep-and-scale factor of element (m, n) of the [M, N] product
 __device__ __forceinline__ float drop_factor(const GemmArgs& g, int m, int n) {
     return bb_dropout_keep(g.drop.k0, g.drop.k1, g.drop.thresh, (uint64_t)m * (uint64_t)g.N + (uint64_t)n) ? g.drop.scale : 0.f;
@@ -67,6 +76,7 @@ __device__ __forceinline__ void epilogue_elem(const GemmArgs& g, int64_t coff, i
     } else if (g.epilogue == BB_EPI_MUL) {
         v *= Elem<T>::load((const T*)g.aux_in + xi);
     } else if (g.epilogue == BB_EPI_MUL_POS) {
+        if (g.resid) v += Elem<T>::load((const T*)g.resid + xi);
         v = Elem<T>::load((const T*)g.aux_in + xi) > 0.f ? v : 0.f;
     } else if (g.epilogue == BB_EPI_ACT_DACT) {
         float a, d;
@@ -151,6 +161,12 @@ __device__ __forceinline__ void epilogue_vec8_at(const GemmArgs& g, int64_t ci, 
     } else if (g.epilogue == BB_EPI_MUL_POS) {
         float d[8];
         load_vec((const bf16*)g.aux_in + xi, d);
+        if (g.resid) {
+            float r[8];
+            load_vec((const bf16*)g.resid + xi, r);
+#pragma unroll
+            for (int e = 0; e < 8; ++e) v[e] += r[e];
+        }
 #pragma unroll
         for (int e = 0; e < 8; ++e) v[e] = d[e] > 0.f ? v[e] : 0.f;
     } else if (g.epilogue == BB_EPI_ACT_DACT) {
@@ -628,12 +644,16 @@ template <int BR, int T, bool KM, int BK = 32> struct FragReader {
     }
 };
 
-// STATS: the epilogue also leaves the column statistics of the stored (bf16-rounded) output per 32-row strip, for the
+// STATS 1: the epilogue also leaves the column statistics of the stored (bf16-rounded) output per 32-row strip, for the
 // batch normalisation that follows a convolution (its statistics pass then has nothing left to read).
+// STATS 2: the product is the gradient that arrives at a batch normalisation (+ ReLU, applied by the epilogue kind);
+// the epilogue also leaves that normalisation's backward sums per strip (BnBwdArgs), so that its backward pass has no
+// reduction over the tensor left.
 template <int BM, int BN, int WM, int WN, bool AKM, bool BKM, bool DB, int STAGES, int BK = 32, bool VIS = false, int CONV = 0,
-          bool STATS = false, bool DROP = false>
+          int STATS = 0, bool DROP = false>
 __device__ __forceinline__ void gemm_bf16_dma_body(const GemmArgs& g, const int block_id, const int batch_id,
-                                                   const bool logical_id = false, const ConvArgs& cv = ConvArgs{}) {
+                                                   const bool logical_id = false, const ConvArgs& cv = ConvArgs{},
+                                                   const BnBwdArgs& bn = BnBwdArgs{}) {
     constexpr int NW = WM * WN;
     static_assert(BK == 64 ? (STAGES >= 2 && DB) : STAGES >= 3,
                   "32-wide k-tiles: the ring needs one stage being read, one landing, one in flight; "
@@ -966,6 +986,23 @@ __device__ __forceinline__ void gemm_bf16_dma_body(const GemmArgs& g, const int 
             if (g.bias && live) load_vec((const bf16*)g.bias + n, b8);
             const int m_first = m0 + wm * WTM + i * 32 + prow;
             int64_t ci = coff + (int64_t)m_first * g.ldc + n, xi = coff + (int64_t)m_first * g.ldaux + n;
+            // STATS 2: the lane's sums over its four rows, for its eight columns
+            float mu8[8], rs8[8], sg[8], sgx[8];
+            if constexpr (STATS == 2) {
+#pragma unroll
+                for (int e = 0; e < 8; ++e) mu8[e] = rs8[e] = sg[e] = sgx[e] = 0.f;
+                if (live) {
+                    const f32x4 m_lo = *(const f32x4*)(bn.mean + n), m_hi = *(const f32x4*)(bn.mean + n + 4);
+                    const f32x4 r_lo = *(const f32x4*)(bn.rstd + n), r_hi = *(const f32x4*)(bn.rstd + n + 4);
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        mu8[e] = m_lo[e];
+                        mu8[4 + e] = m_hi[e];
+                        rs8[e] = r_lo[e];
+                        rs8[4 + e] = r_hi[e];
+                    }
+                }
+            }
 #pragma unroll
             for (int it = 0; it < 4; ++it) {
                 const int m = m_first + it * 8;
@@ -977,11 +1014,46 @@ __device__ __forceinline__ void gemm_bf16_dma_body(const GemmArgs& g, const int 
                     v[e] = lo[e];
                     v[4 + e] = hi[e];
                 }
-                if (live && m < g.M) epilogue_vec8_at<DROP>(g, ci, xi, m, n, v, b8);
+                if (live && m < g.M) {
+                    epilogue_vec8_at<DROP>(g, ci, xi, m, n, v, b8);
+                    if constexpr (STATS == 2) {
+                        float xv[8];
+                        load_vec((const bf16*)bn.x + ci, xv);
+#pragma unroll
+                        for (int e = 0; e < 8; ++e) {
+                            const float gr = bf2f(f2bf(v[e]));   // what was stored
+                            sg[e] += gr;
+                            sgx[e] += gr * (xv[e] - mu8[e]) * rs8[e];
+                        }
+                    }
+                }
                 ci += 8 * (int64_t)g.ldc;
                 xi += 8 * (int64_t)g.ldaux;
             }
-            if constexpr (STATS) {
+            if constexpr (STATS == 2) {
+                // the eight row groups' sums through the patch (all of it has been read): rows 0..7 sum g, rows 8..15
+                // sum g xhat, then lane = column adds the eight up in row order
+                asm volatile("" ::: "memory");
+                *(f32x4*)(patch + prow * PLD + pcol) = f32x4{sg[0], sg[1], sg[2], sg[3]};
+                *(f32x4*)(patch + prow * PLD + pcol + 4) = f32x4{sg[4], sg[5], sg[6], sg[7]};
+                *(f32x4*)(patch + (8 + prow) * PLD + pcol) = f32x4{sgx[0], sgx[1], sgx[2], sgx[3]};
+                *(f32x4*)(patch + (8 + prow) * PLD + pcol + 4) = f32x4{sgx[4], sgx[5], sgx[6], sgx[7]};
+                asm volatile("" ::: "memory");
+                float t0 = 0.f, t1 = 0.f;
+#pragma unroll
+                for (int r = 0; r < 8; ++r) {
+                    t0 += patch[r * PLD + lane];
+                    t1 += patch[(8 + r) * PLD + lane];
+                }
+                const int strip_row = m0 + wm * WTM + i * 32;
+                const int nc = n0 + wn * WTN + jp * 64 + lane;
+                if (strip_row < g.M && nc < g.N && (NH == 2 || lane < 32)) {
+                    float* o = bn.strips + ((int64_t)(strip_row >> 5) * 2) * g.N + nc;
+                    o[0] = t0;
+                    o[g.N] = t1;
+                }
+            }
+            if constexpr (STATS == 1) {
                 // Column statistics of this 32-row strip straight from the patch: lane = column, 32 conflict-free LDS
                 // reads.  The patch holds what is stored (alpha = 1, no bias, no epilogue), rounded here as the
                 // store rounds it; the pivot is the strip's first row.
@@ -1013,12 +1085,18 @@ __device__ __forceinline__ void gemm_bf16_dma_body(const GemmArgs& g, const int 
 // kernels without dropout nothing (they decide how many blocks of the small tiles a CU holds).
 template <int BM, int BN, int WM, int WN, bool AKM, bool BKM, bool DB, int STAGES, int BK, bool DROP = false>
 __global__ __launch_bounds__(WM* WN * 64) void gemm_bf16_dma_kernel(const GemmArgs g) {
-    gemm_bf16_dma_body<BM, BN, WM, WN, AKM, BKM, DB, STAGES, BK, false, 0, false, DROP>(g, blockIdx.x, blockIdx.z);
+    gemm_bf16_dma_body<BM, BN, WM, WN, AKM, BKM, DB, STAGES, BK, false, 0, 0, DROP>(g, blockIdx.x, blockIdx.z);
 }
 // the same with the strip statistics of the output (NT, 64-wide k-tiles, three stages)
 template <int BM, int BN, int WM, int WN>
 __global__ __launch_bounds__(WM* WN * 64) void gemm_bf16_dma_stats_kernel(const GemmArgs g) {
-    gemm_bf16_dma_body<BM, BN, WM, WN, false, false, true, 3, 64, false, 0, true>(g, blockIdx.x, blockIdx.z);
+    gemm_bf16_dma_body<BM, BN, WM, WN, false, false, true, 3, 64, false, 0, 1>(g, blockIdx.x, blockIdx.z);
+}
+// input gradient of a 1x1 convolution (NN, 64-wide k-tiles, three stages) with the backward sums of the batch
+// normalisation in front of it
+template <int BM, int BN, int WM, int WN>
+__global__ __launch_bounds__(WM* WN * 64) void gemm_bf16_dma_bnbwd_kernel(const GemmArgs g, const BnBwdArgs bn) {
+    gemm_bf16_dma_body<BM, BN, WM, WN, false, true, true, 3, 64, false, 0, 2>(g, blockIdx.x, 0, false, ConvArgs{}, bn);
 }
 
 // Persistent variant for problems of more than one round of 256x256 tiles (NT and NN, 32-wide k-tiles, three stages,
@@ -1228,7 +1306,12 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_bf16_dma_persist_kernel(cons
 // (BKM = true: dx = patches(dy) W_flipped) on the same main loop, operands gathered by the loaders.
 template <int BM, int BN, int WM, int WN, bool BKM, int STAGES, bool STATS = false>
 __global__ __launch_bounds__(WM* WN * 64) void conv3x3_bf16_igemm_kernel(const GemmArgs g, const ConvArgs cv) {
-    gemm_bf16_dma_body<BM, BN, WM, WN, false, BKM, true, STAGES, 64, false, BKM ? 2 : 1, STATS>(g, blockIdx.x, 0, false, cv);
+    gemm_bf16_dma_body<BM, BN, WM, WN, false, BKM, true, STAGES, 64, false, BKM ? 2 : 1, STATS ? 1 : 0>(g, blockIdx.x, 0, false, cv);
+}
+// the input gradient with the backward sums of the batch normalisation in front of the convolution
+template <int BM, int BN, int WM, int WN, int STAGES>
+__global__ __launch_bounds__(WM* WN * 64) void conv3x3_bf16_igemm_bnbwd_kernel(const GemmArgs g, const ConvArgs cv, const BnBwdArgs bn) {
+    gemm_bf16_dma_body<BM, BN, WM, WN, false, true, true, STAGES, 64, false, 2, 2>(g, blockIdx.x, 0, false, cv, bn);
 }
 
 // Several independent problems of one kind in a single launch (the four weight-gradient GEMMs

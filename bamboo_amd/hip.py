@@ -25,7 +25,7 @@ LN_CODES = {"standard": LN_STANDARD, "annotated": LN_ANNOTATED}
 EXPORTS = (
     "bb_version", "bb_last_error", "bb_init", "bb_gemm", "bb_gemm_grouped", "bb_gemm_splitk_workspace", "bb_gemm_grouped_splitk", "bb_gemm_variant", "bb_layernorm_fwd",
     "bb_layernorm_bwd_workspace", "bb_layernorm_bwd", "bb_layernorm_bwd_static", "bb_colsum_workspace", "bb_colsum_acc", "bb_rowsum_fwd", "bb_rowsum_bwd", "bb_dropout_apply", "bb_dropout_keep_host",
-    "bb_softmax_fwd", "bb_softmax_bwd", "bb_attention_fwd", "bb_attention_bwd", "bb_residual_add", "bb_sqrt_one_minus_fwd", "bb_sqrt_one_minus_bwd", "bb_act_fwd", "bb_bn_workspace", "bb_batchnorm_fwd", "bb_batchnorm_bwd", "bb_patch3x3", "bb_patch3x3_strided", "bb_subsample", "bb_conv3x3_supported", "bb_conv3x3", "bb_gemm_strip_stats_supported", "bb_strip_stats_workspace", "bb_batchnorm_fwd_strips", "bb_mse_workspace", "bb_mse_fwd_bwd", "bb_graph_begin", "bb_graph_end", "bb_graph_launch", "bb_graph_destroy",
+    "bb_softmax_fwd", "bb_softmax_bwd", "bb_attention_fwd", "bb_attention_bwd", "bb_residual_add", "bb_sqrt_one_minus_fwd", "bb_sqrt_one_minus_bwd", "bb_act_fwd", "bb_bn_workspace", "bb_batchnorm_fwd", "bb_batchnorm_bwd", "bb_patch3x3", "bb_patch3x3_strided", "bb_subsample", "bb_conv3x3_supported", "bb_conv3x3", "bb_gemm_strip_stats_supported", "bb_strip_stats_workspace", "bb_batchnorm_fwd_strips", "bb_bn_bwd_strips_workspace", "bb_gemm_bn_bwd_supported", "bb_gemm_bn_bwd", "bb_conv3x3_dgrad_bn", "bb_batchnorm_bwd_strips", "bb_mse_workspace", "bb_mse_fwd_bwd", "bb_graph_begin", "bb_graph_end", "bb_graph_launch", "bb_graph_destroy",
     "bb_adam_multi", "bb_adam_multi_scaled", "bb_grad_clip_workspace", "bb_grad_clip_coef", "bb_cast", "bb_fill_f32",
 )
 
@@ -51,6 +51,10 @@ class GemmDesc(Structure):
         ("strip_stats", c_void_p),
         ("dropout_p", c_float), ("dropout_k0", c_uint32), ("dropout_k1", c_uint32),
     ]
+
+
+class BnBwdStats(Structure):
+    _fields_ = [("x", c_void_p), ("mean", c_void_p), ("rstd", c_void_p), ("strips", c_void_p)]
 
 
 def library_path():
@@ -121,6 +125,12 @@ def lib():
     L.bb_strip_stats_workspace.argtypes = [c_int, c_int]
     L.bb_strip_stats_workspace.restype = c_int64
     L.bb_batchnorm_fwd_strips.argtypes = [c_int, c_int, c_int, c_float, c_float, c_int] + [c_void_p] * 11
+    L.bb_bn_bwd_strips_workspace.argtypes = [c_int, c_int]
+    L.bb_bn_bwd_strips_workspace.restype = c_int64
+    L.bb_gemm_bn_bwd_supported.argtypes = [POINTER(GemmDesc)]
+    L.bb_gemm_bn_bwd.argtypes = [POINTER(GemmDesc), POINTER(BnBwdStats), c_void_p]
+    L.bb_conv3x3_dgrad_bn.argtypes = [c_int] * 6 + [c_void_p] * 4 + [POINTER(BnBwdStats), c_void_p]
+    L.bb_batchnorm_bwd_strips.argtypes = [c_int, c_int, c_int] + [c_void_p] * 10
     L.bb_mse_workspace.restype = c_int64
     L.bb_mse_fwd_bwd.argtypes = [c_int, c_int64, c_void_p, c_void_p, c_void_p, c_float, c_void_p, c_int,
                                  c_void_p, c_void_p]
@@ -596,6 +606,20 @@ def batchnorm_bwd(x, gamma, mean, rstd, dy, relu_out, dx, g_out, dgamma, dbeta, 
                                  _ptr(workspace), stream_ptr(stream)), "bb_batchnorm_bwd")
 
 
+def batchnorm_bwd_strips(x, gamma, mean, rstd, g, strips, dx, dgamma, dbeta, stream=None):
+    """``batchnorm_bwd`` for a gradient ``g`` that is masked already and whose sums per strip the kernel that produced
+    it left in ``strips`` (``gemm_bn_bwd`` / ``conv3x3_dgrad_bn``)."""
+    rows, cols = x.shape
+    _like("batchnorm_bwd_strips", x, g=g, dx=dx)
+    _vector("batchnorm_bwd_strips", cols, x.dtype, gamma=gamma)
+    _vector("batchnorm_bwd_strips", cols, torch.float32, mean=mean, rstd=rstd, dgamma=dgamma, dbeta=dbeta)
+    if strips.dtype != torch.float32 or not strips.is_contiguous() or strips.numel() < bn_bwd_strips_workspace(rows, cols):
+        raise HipKernelError("batchnorm_bwd_strips: strips too small")
+    check(lib().bb_batchnorm_bwd_strips(dtype_code(x.dtype), rows, cols, _ptr(x), _ptr(gamma), _ptr(mean), _ptr(rstd),
+                                        _ptr(g), _ptr(strips), _ptr(dx), _ptr(dgamma), _ptr(dbeta), stream_ptr(stream)),
+          "bb_batchnorm_bwd_strips")
+
+
 def _out_side(side, stride):
     return (side - 1) // stride + 1
 
@@ -651,6 +675,71 @@ def conv3x3(mode, src, weight, dst, n, h, w, cin, cout, strip_stats=None, stream
                                           _ptr(dst), _ptr(strip_stats), stream_ptr(stream)), "bb_conv3x3")
     if hook is not None:
         hook(ConvLaunch(mode, rows, cin, cout), call, stream)
+    else:
+        call()
+
+
+def bn_bwd_strips_workspace(rows, cols):
+    """fp32 elements of the per-32-row-strip backward sums a GEMM / convolution leaves for batchnorm_bwd_strips."""
+    return int(lib().bb_bn_bwd_strips_workspace(rows, cols))
+
+
+def _bn_bwd_stats(what, rows, cols, dtype, x, mean, rstd, strips):
+    """The checked ``bb_bn_bwd_stats`` of a [rows, cols] gradient: the kernel reads x, mean and rstd at the product's
+    indices and writes one pair of sums per 32-row strip and column."""
+    if tuple(x.shape) != (rows, cols) or x.dtype != dtype or not x.is_contiguous():
+        raise HipKernelError(f"{what}: x must be a contiguous {(rows, cols)} tensor of {dtype}, got {tuple(x.shape)} {x.dtype}")
+    _vector(what, cols, torch.float32, mean=mean, rstd=rstd)
+    if strips.dtype != torch.float32 or not strips.is_contiguous() or strips.numel() < bn_bwd_strips_workspace(rows, cols):
+        raise HipKernelError(f"{what}: strips must be a contiguous fp32 tensor of >= {bn_bwd_strips_workspace(rows, cols)} elements")
+    return BnBwdStats(_ptr(x), _ptr(mean), _ptr(rstd), _ptr(strips))
+
+
+def _bn_bwd_epilogue(relu_out, resid):
+    if relu_out is not None:
+        return dict(epilogue=EPI_MUL_POS, aux_in=relu_out, resid=resid)
+    return dict(epilogue=EPI_RESIDUAL, resid=resid) if resid is not None else {}
+
+
+def gemm_bn_bwd_supported(A, B, C, relu_out=None, resid=None):
+    """Whether ``gemm_bn_bwd(A, B, C, ...)`` is taken (bf16 NN problems of the convolution shapes)."""
+    return bool(lib().bb_gemm_bn_bwd_supported(byref(gemm_desc(NN, A, B, C, **_bn_bwd_epilogue(relu_out, resid)))))
+
+
+def gemm_bn_bwd(A, B, C, relu_out, x, mean, rstd, strips, resid=None, stream=None, hook=None):
+    """C = (A B [+ resid]) * (relu_out > 0): the input gradient of a 1x1 convolution (plus the gradient of a skip
+    connection that joins it), masked by the ReLU in front of it, with the backward sums of the batch normalisation
+    in front of that ReLU (input x, statistics mean / rstd) left in ``strips`` for ``batchnorm_bwd_strips``.
+    ``relu_out`` None: no ReLU."""
+    d = gemm_desc(NN, A, B, C, **_bn_bwd_epilogue(relu_out, resid))
+    _like("gemm_bn_bwd", C, relu_out=relu_out, resid=resid)
+    bn = _bn_bwd_stats("gemm_bn_bwd", C.shape[0], C.shape[1], C.dtype, x, mean, rstd, strips)
+    call = lambda: check(lib().bb_gemm_bn_bwd(byref(d), byref(bn), stream_ptr(stream)), "bb_gemm_bn_bwd")
+    if hook is not None:
+        hook(d, call, stream)
+    else:
+        call()
+    return C
+
+
+def conv3x3_dgrad_bn(src, weight, dst, n, h, w, cin, cout, relu_out, x, mean, rstd, strips, stream=None, hook=None):
+    """``conv3x3(CONV_DGRAD, ...)`` with the result masked by ``relu_out > 0`` (None: no ReLU) and the backward sums of
+    the batch normalisation in front of it left in ``strips``, as ``gemm_bn_bwd``."""
+    rows = n * h * w
+    if tuple(src.shape) != (rows, cout) or tuple(dst.shape) != (rows, cin) or weight.numel() != 9 * cin * cout:
+        raise HipKernelError(f"conv3x3_dgrad_bn: shapes {tuple(src.shape)} {tuple(weight.shape)} {tuple(dst.shape)} do not fit "
+                             f"n={n} h={h} w={w} cin={cin} cout={cout}")
+    if not (src.is_contiguous() and dst.is_contiguous() and weight.is_contiguous()):
+        raise HipKernelError("conv3x3_dgrad_bn: operands must be contiguous")
+    if not (src.dtype == weight.dtype == dst.dtype):
+        raise HipKernelError("conv3x3_dgrad_bn: operands must share one dtype")
+    if relu_out is not None:
+        _like("conv3x3_dgrad_bn", dst, relu_out=relu_out)
+    bn = _bn_bwd_stats("conv3x3_dgrad_bn", rows, cin, dst.dtype, x, mean, rstd, strips)
+    call = lambda: check(lib().bb_conv3x3_dgrad_bn(dtype_code(src.dtype), n, h, w, cin, cout, _ptr(src), _ptr(weight), _ptr(dst),
+                                                   _ptr(relu_out), byref(bn), stream_ptr(stream)), "bb_conv3x3_dgrad_bn")
+    if hook is not None:
+        hook(ConvLaunch(CONV_DGRAD, rows, cin, cout), call, stream)
     else:
         call()
 

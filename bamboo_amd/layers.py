@@ -44,6 +44,13 @@ class StageContext:
         # optional observer of this lane's GEMM launches (``hip.gemm(..., hook=)``); set through the engine that owns
         # the context, so a probe on one engine sees and changes nothing of another
         self.gemm_hook = None
+        # hand-over between two neighbouring layers of a backward pass: what the layer that receives this layer's
+        # input gradient wants done to it on the way (``grad_sink``, offered by ``PipelineModule.backward``), whether
+        # this layer did it (``grad_sink_used``), and whether the gradient this layer receives had it done
+        # (``grad_presummed``)
+        self.grad_sink = None
+        self.grad_sink_used = False
+        self.grad_presummed = False
 
     def gemm(self, *a, **kw):
         return hip.gemm(*a, hook=self.gemm_hook, **kw)
@@ -53,6 +60,12 @@ class StageContext:
 
     def conv3x3(self, *a, **kw):
         return hip.conv3x3(*a, hook=self.gemm_hook, **kw)
+
+    def gemm_bn_bwd(self, *a, **kw):
+        return hip.gemm_bn_bwd(*a, hook=self.gemm_hook, **kw)
+
+    def conv3x3_dgrad_bn(self, *a, **kw):
+        return hip.conv3x3_dgrad_bn(*a, hook=self.gemm_hook, **kw)
 
     @property
     def rows(self):
@@ -838,7 +851,11 @@ class BottleNeck:
         specs = [("d_col", (R2, 9 * cm), dt), ("d_y3", (R2, co), dt), ("d_res", (R2, co), dt),
                  ("d_m0", (R, cm), dt), ("d_m1", (R2, cm), dt), ("d_m2", (R, cm), dt),
                  # split-K partial products of the weight gradients (8 chunks of each, fp32)
-                 ("splitk", (8 * self._wgrad_elems(),), torch.float32)]
+                 ("splitk", (8 * self._wgrad_elems(),), torch.float32),
+                 # backward sums of an inner BatchNorm per 32-row strip, left by the kernel that produces its gradient
+                 ("bn_strips", (hip.bn_bwd_strips_workspace(R, cm),), torch.float32),
+                 # the same for the last BatchNorm, left by the block behind this one (grad_sink)
+                 ("bn_strips_in", (hip.bn_bwd_strips_workspace(R2, co),), torch.float32)]
         if self.projection:
             specs += [("d_ys", (R2, co), dt), ("d_xs", (R2, ci), dt)]
         return specs + self.forward_scratch_specs(ctx)
@@ -929,6 +946,17 @@ class BottleNeck:
         self._bn_fwd(7, st["y3"], sc, st["out"], st["mean3"], st["rstd3"], True, ctx, strips)
         return st["out"]
 
+    def grad_sink(self, st, ctx):
+        """What the layer behind this one may do to the gradient it hands over (``ctx.seq`` is this block's): mask it
+        with the block's last ReLU and leave the backward sums of the last BatchNorm per strip -- the kernel that
+        writes that gradient does both in its epilogue, this block's backward then starts without a reduction pass
+        over its widest tensor.  None where the kernels for it do not exist (fp32)."""
+        if ctx.dtype != torch.bfloat16:
+            return None
+        _, R2, _, _ = self._rows(ctx)
+        return {"rows": R2, "cols": self.cout, "relu_out": st["out"], "x": st["y3"], "mean": st["mean3"], "rstd": st["rstd3"],
+                "strips": ctx.buf("bn_strips_in", (hip.bn_bwd_strips_workspace(R2, self.cout),))}
+
     def backward(self, d_out, d_x, st, ctx):
         w, g, sm, ws = self.w_, self.g_, ctx.stream, ctx.workspace
         R, R2, _, _ = self._rows(ctx)
@@ -941,16 +969,38 @@ class BottleNeck:
             name = self._BN_NAMES[idx]
             hip.batchnorm_bwd(st[xk], w[f"{name}.weight"], st[mk], st[rk], dy, relu_out, dx, g_out,
                               g[f"{name}.weight"], g[f"{name}.bias"], ws, stream=sm)
+
+        def bn_strips(idx, xk, mk, rk, gk, strips, dx):
+            name = self._BN_NAMES[idx]
+            hip.batchnorm_bwd_strips(st[xk], w[f"{name}.weight"], st[mk], st[rk], gk, strips, dx,
+                                     g[f"{name}.weight"], g[f"{name}.bias"], stream=sm)
         # final ReLU + BN3; d_res keeps the masked gradient for the shortcut
-        bn(7, "y3", "mean3", "rstd3", d_out, st["out"], d_y3, d_res)
+        if ctx.grad_presummed:
+            # the block behind this one has masked d_out and left the sums (grad_sink)
+            d_res = d_out
+            bn_strips(7, "y3", "mean3", "rstd3", d_out, ctx.buf("bn_strips_in", (hip.bn_bwd_strips_workspace(R2, co),)), d_y3)
+        else:
+            bn(7, "y3", "mean3", "rstd3", d_out, st["out"], d_y3, d_res)
         d_ys = d_xs = xs = None
         if self.projection:
             d_ys, d_xs = ctx.buf("d_ys", (R2, co)), ctx.buf("d_xs", (R2, ci))
             bn("shortcut", "ys", "mean_s", "rstd_s", d_res, None, d_ys, None)
             ctx.gemm(hip.NN, d_ys, w["shortcut.0.weight"], d_xs, stream=sm)
             xs = self._shortcut_input(st["x0"], ctx, R2)
-        ctx.gemm(hip.NN, d_y3, w["residual_function.6.weight"], d_m0, stream=sm)          # d_a2
-        bn(4, "y2", "mean2", "rstd2", d_m0, st["a2"], d_m1, None)                          # d_y2
+        # The two inner BatchNorms receive their gradient from a convolution's input gradient: where the kernel can,
+        # it masks the gradient with the ReLU and leaves the normalisation's backward sums per strip, so that no
+        # pass over the tensor is needed for them.
+        key = ("bn_bwd", R2, cm, co, ctx.dtype)
+        if key not in self._stats_ok:
+            self._stats_ok[key] = hip.gemm_bn_bwd_supported(d_y3, w["residual_function.6.weight"], d_m0, st["a2"])
+        if self._stats_ok[key]:
+            strips = ctx.buf("bn_strips", (hip.bn_bwd_strips_workspace(R2, cm),))
+            ctx.gemm_bn_bwd(d_y3, w["residual_function.6.weight"], d_m0, st["a2"], st["y2"], st["mean2"], st["rstd2"],
+                            strips, stream=sm)                                             # d_a2, masked
+            bn_strips(4, "y2", "mean2", "rstd2", d_m0, strips, d_m1)                       # d_y2
+        else:
+            ctx.gemm(hip.NN, d_y3, w["residual_function.6.weight"], d_m0, stream=sm)      # d_a2
+            bn(4, "y2", "mean2", "rstd2", d_m0, st["a2"], d_m1, None)                      # d_y2
         # weight gradient of the 3x3 convolution: patch matrix gathered inside the GEMM, else built again here
         # (cheaper than stashing it)
         wgrad_implicit = (self._implicit(ctx, hip.CONV_DGRAD) and cm % 128 == 0 and R % 32 == 0 and 32 // self.w + 1 <= self.h)
@@ -958,19 +1008,35 @@ class BottleNeck:
             hip.patch3x3(st["a1"], col, ctx.batch, self.h, self.w, cm, stride=self.stride, stream=sm)
         d_a1, d_m2 = ctx.buf("d_m0", (R, cm)), ctx.buf("d_m2", (R, cm))
         if self._implicit(ctx, hip.CONV_DGRAD):
-            ctx.conv3x3(hip.CONV_DGRAD, d_m1, w["residual_function.3.weight"], d_a1, ctx.batch, self.h, self.w, cm, cm,
-                        stream=sm)
+            strips = ctx.buf("bn_strips", (hip.bn_bwd_strips_workspace(R, cm),))
+            ctx.conv3x3_dgrad_bn(d_m1, w["residual_function.3.weight"], d_a1, ctx.batch, self.h, self.w, cm, cm,
+                                 st["a1"], st["y1"], st["mean1"], st["rstd1"], strips, stream=sm)
+            bn_strips(1, "y1", "mean1", "rstd1", d_a1, strips, d_m2)                       # d_y1
         else:
             d_col = ctx.buf("d_col", (R2, 9 * cm))
             ctx.gemm(hip.NN, d_m1, w["conv2"], d_col, stream=sm)
             hip.patch3x3(d_col, d_a1, ctx.batch, self.h, self.w, cm, adjoint=True, stride=self.stride, stream=sm)
-        bn(1, "y1", "mean1", "rstd1", d_a1, st["a1"], d_m2, None)                          # d_y1
+            bn(1, "y1", "mean1", "rstd1", d_a1, st["a1"], d_m2, None)                      # d_y1
         if self.projection and self.stride > 1:
             ctx.gemm(hip.NN, d_m2, w["residual_function.0.weight"], d_x, stream=sm)
             hip.subsample(d_xs, d_x, ctx.batch, self.h, self.w, ci, self.stride, adjoint=True, stream=sm)
         else:
-            ctx.gemm(hip.NN, d_m2, w["residual_function.0.weight"], d_x, epilogue=hip.EPI_RESIDUAL,
-                     resid=d_xs if self.projection else d_res, stream=sm)
+            resid = d_xs if self.projection else d_res
+            sink = ctx.grad_sink
+            if sink is not None and (sink["rows"], sink["cols"]) == (R, ci):
+                key = ("sink", R, ci, cm, ctx.dtype)
+                if key not in self._stats_ok:
+                    self._stats_ok[key] = hip.gemm_bn_bwd_supported(d_m2, w["residual_function.0.weight"], d_x, sink["relu_out"], resid)
+                if not self._stats_ok[key]:
+                    sink = None
+            else:
+                sink = None
+            if sink is not None:
+                ctx.gemm_bn_bwd(d_m2, w["residual_function.0.weight"], d_x, sink["relu_out"], sink["x"], sink["mean"],
+                                sink["rstd"], sink["strips"], resid=resid, stream=sm)
+                ctx.grad_sink_used = True
+            else:
+                ctx.gemm(hip.NN, d_m2, w["residual_function.0.weight"], d_x, epilogue=hip.EPI_RESIDUAL, resid=resid, stream=sm)
         # the weight gradients in one launch: few output tiles over thousands of rows, cut along the rows
         descs = [hip.gemm_desc(hip.TN, d_y3, st["a2"], g["residual_function.6.weight"], accumulate=True),
                  hip.gemm_desc(hip.TN, d_m1, st["a1"], g["conv2"], accumulate=True, conv=(self.h, self.w))

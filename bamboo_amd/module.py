@@ -578,11 +578,22 @@ class PipelineModule:
                     ctx.seq = seqs[i]
                     x = layers[i].forward(x, stash[i], ctx)
                 ctx.redundant = was
+            presummed = False
             for i in range(b - 1, a - 1, -1):
                 dst = grad_input if i == 0 else ctx.buf(f"d_layer{i % 2}", (ctx.batch * seqs[i], layers[i].feature_dim))
+                # Inside a group the layer in front (whose stash is there) may ask for its incoming gradient to be
+                # prepared by the kernel that writes it (a bottleneck: masked by its last ReLU, with the sums of its
+                # last BatchNorm); a layer that does so says so, and the receiver is told.
+                sink = None
+                if i > a and hasattr(layers[i - 1], "grad_sink"):
+                    ctx.seq = seqs[i - 1]
+                    sink = layers[i - 1].grad_sink(stash[i - 1], ctx)
                 ctx.seq = seqs[i]
+                ctx.grad_sink, ctx.grad_sink_used, ctx.grad_presummed = sink, False, presummed
                 layers[i].backward(d, dst, stash[i], ctx)
+                presummed = ctx.grad_sink_used
                 d = dst
+            ctx.grad_sink, ctx.grad_sink_used, ctx.grad_presummed = None, False, False
         ctx.deferred = False
         return grad_input
 

@@ -54,9 +54,10 @@ extern "C" {
  *   BB_EPI_MUL       C = v * aux_in[m,n]  (e.g. aux_in = act'(u) kept by BB_EPI_ACT_DACT or bb_act_fwd)
  *   BB_EPI_ACT_DACT  aux_out = act'(v);  C = act(v)   (forward of an FFN whose backward then needs no
  *                    transcendental: its input gradient is a BB_EPI_MUL product with aux_out)
- *   BB_EPI_MUL_POS   C = v where aux_in[m,n] > 0, else 0  (input gradient through a ReLU whose OUTPUT was kept:
- *                    relu'(u) = [relu(u) > 0], so the forward stores nothing beside its output; a dropout
- *                    factor 1/(1-p) on that output goes into alpha)
+ *   BB_EPI_MUL_POS   C = v (+ resid[m,n] if resid != NULL) where aux_in[m,n] > 0, else 0  (input gradient through a
+ *                    ReLU whose OUTPUT was kept: relu'(u) = [relu(u) > 0], so the forward stores nothing beside
+ *                    its output; a dropout factor 1/(1-p) on that output goes into alpha; with resid: the
+ *                    gradient that meets a skip connection's before it passes the ReLU of the block in front)
  * `accumulate` != 0 adds the result to the existing contents of C (C must be fp32).       */
 #define BB_EPI_NONE 0
 #define BB_EPI_ACT 1
@@ -306,6 +307,37 @@ int bb_subsample(int dtype, int adjoint, int n, int h, int w, int c, int stride,
 int bb_conv3x3_supported(int dtype, int mode, int n, int h, int w, int cin, int cout);
 int bb_conv3x3(int dtype, int mode, int n, int h, int w, int cin, int cout, const void* src, const void* weight,
                void* dst, float* strip_stats /* BB_CONV_FWD: as bb_gemm_desc.strip_stats, or NULL */, void* stream);
+
+/* The backward pass of "BatchNorm2d, ReLU, Conv2d" (resnet.py:56-61: each of the two inner normalisations of a
+ * bottleneck feeds a ReLU and a convolution; autograd's backward of that chain, engine.py:1701-1709) without a
+ * reduction pass over the tensor: the kernel that computes the convolution's input gradient dy also masks it with
+ * the ReLU (g = dy * (relu_out > 0), stored as C / dst) and leaves, per strip of 32 consecutive rows and per
+ * column, sum g and sum g * xhat of the stored bf16 values, xhat = (x - mean) * rstd of the normalisation's input
+ * x ([M, N] contiguous like C): strips[(strip * 2 + j) * N + n], fp32, >= bb_bn_bwd_strips_workspace(M, N) floats.
+ * bb_batchnorm_bwd_strips adds the strips up in a fixed order and applies
+ * dx = gamma * rstd * (g - mean(g) - xhat * mean(g * xhat)); dgamma += sum g * xhat; dbeta += sum g
+ * (bb_batchnorm_bwd's result up to the fp32 summation order).  bf16 only.
+ *   bb_gemm_bn_bwd       the input gradient of a 1x1 convolution: a BB_NN problem (C = dy_next W) with epilogue
+ *                        BB_EPI_MUL_POS and aux_in = relu_out (or BB_EPI_NONE / BB_EPI_RESIDUAL: no ReLU);
+ *                        bb_gemm_bn_bwd_supported() says (1 / 0) whether the problem is taken.  With resid this
+ *                        is also the gradient a bottleneck hands to the block in front of it (resnet.py:75: the
+ *                        sum of the residual function's and the shortcut's, then that block's last ReLU and
+ *                        BatchNorm): x, mean, rstd, relu_out are then that block's
+ *   bb_conv3x3_dgrad_bn  bb_conv3x3(BB_CONV_DGRAD) with the same additions (relu_out may be NULL)               */
+typedef struct bb_bn_bwd_stats {
+    const void* x;      /* [M, N] input of the normalisation */
+    const float* mean;  /* [N] */
+    const float* rstd;  /* [N] */
+    float* strips;      /* out */
+} bb_bn_bwd_stats;
+int64_t bb_bn_bwd_strips_workspace(int rows, int cols);
+int bb_gemm_bn_bwd_supported(const bb_gemm_desc* desc);
+int bb_gemm_bn_bwd(const bb_gemm_desc* desc, const bb_bn_bwd_stats* bn, void* stream);
+int bb_conv3x3_dgrad_bn(int dtype, int n, int h, int w, int cin, int cout, const void* src, const void* weight,
+                        void* dst, const void* relu_out, const bb_bn_bwd_stats* bn, void* stream);
+int bb_batchnorm_bwd_strips(int dtype, int rows, int cols, const void* x, const void* gamma, const float* mean,
+                            const float* rstd, const void* g, const float* strips, void* dx, float* dgamma,
+                            float* dbeta, void* stream);
 
 /* Mean-squared-error head (nn.MSELoss, transformer.py:264) fused with its gradient:
  * loss_out[0] (+)= mean((y-t)^2);  dy = grad_scale * 2 (y-t) / n.  Deterministic two-pass

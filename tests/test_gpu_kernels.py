@@ -496,6 +496,80 @@ def test_batchnorm_fwd_bwd(hiplib, dtype, rows, cols, relu, with_resid):
     assert torch.equal(y, y2) and torch.equal(rm, rm2)
 
 
+@pytest.mark.parametrize("kind", ["conv1x1", "conv1x1+skip", "conv3x3"])
+@pytest.mark.parametrize("n,h,w,cm,co,relu", [(32, 14, 14, 256, 1024, True), (32, 14, 14, 1024, 256, True), (3, 10, 10, 128, 256, True),
+                                              (5, 9, 7, 192, 128, False)])
+def test_bn_bwd_sums_from_the_input_gradient(hiplib, kind, n, h, w, cm, co, relu):
+    """The backward pass of BatchNorm -> ReLU -> convolution with the normalisation's sums taken from the epilogue of
+    the convolution's input gradient: against the separate kernels (input gradient, then ``batchnorm_bwd`` with its own
+    reduction pass), and against fp64.  The ResNet-152 conv4_x shape (6272 rows: 196 strips over 98 row tiles) and two
+    with a ragged last strip, one of them with a column count that leaves half a pair of accumulator tiles."""
+    dt, R = torch.bfloat16, n * h * w
+    x = randn(R, cm, dtype=dt, seed=71, scale=2.0) + 0.5             # the normalisation's input
+    gamma = (1 + 0.1 * randn(cm, seed=72)).to(dt)
+    beta = (0.1 * randn(cm, seed=73)).to(dt)
+    a = torch.empty_like(x)                                          # its (ReLU'd) output
+    mean, rstd = torch.empty(cm, device=DEV), torch.empty(cm, device=DEV)
+    ws = torch.empty(hiplib.bn_workspace(max(cm, co)), device=DEV)
+    hiplib.batchnorm_fwd(x, gamma, beta, None, a, mean, rstd, None, None, ws, 1e-5, 0.1, relu)
+    relu_out = a if relu else None
+    if kind.startswith("conv1x1"):
+        # "+skip": the gradient of a skip connection joins the product before the ReLU (what a bottleneck hands to
+        # the block in front of it)
+        skip = randn(R, cm, dtype=dt, seed=78) if kind.endswith("skip") else None
+        dy_next = randn(R, co, dtype=dt, seed=74)
+        wt = randn(co, cm, dtype=dt, seed=75, scale=co ** -0.5)
+        plain = lambda dst: hiplib.gemm(hiplib.NN, dy_next, wt, dst, **(dict(epilogue=hiplib.EPI_RESIDUAL, resid=skip) if skip is not None else {}))
+        fused = lambda dst, strips: hiplib.gemm_bn_bwd(dy_next, wt, dst, relu_out, x, mean, rstd, strips, resid=skip)
+        assert hiplib.gemm_bn_bwd_supported(dy_next, wt, torch.empty_like(x), relu_out, skip)
+        full = dy_next.double().cpu() @ wt.double().cpu() + (skip.double().cpu() if skip is not None else 0)
+    else:
+        dy_next = randn(R, co, dtype=dt, seed=74)
+        if not hiplib.conv3x3_supported(dt, hiplib.CONV_DGRAD, n, h, w, cm, co):
+            pytest.skip("the implicit input gradient does not take this shape")
+        wt = randn(co, 3, 3, cm, dtype=dt, seed=75, scale=(9 * co) ** -0.5)
+        plain = lambda dst: hiplib.conv3x3(hiplib.CONV_DGRAD, dy_next, wt, dst, n, h, w, cm, co)
+        fused = lambda dst, strips: hiplib.conv3x3_dgrad_bn(dy_next, wt, dst, n, h, w, cm, co, relu_out, x, mean, rstd, strips)
+        F = torch.nn.functional
+        dn = dy_next.double().cpu().view(n, h, w, co).permute(0, 3, 1, 2)
+        full = F.conv_transpose2d(dn, wt.double().cpu().permute(0, 3, 1, 2), padding=1).permute(0, 2, 3, 1).reshape(R, cm)
+    # separate kernels
+    d_a, dx0, g0 = torch.empty_like(x), torch.empty_like(x), torch.empty_like(x)
+    dg_init, db_init = randn(cm, seed=76), randn(cm, seed=77)
+    dg0, db0 = dg_init.clone(), db_init.clone()
+    plain(d_a)
+    hiplib.batchnorm_bwd(x, gamma, mean, rstd, d_a, relu_out, dx0, g0, dg0, db0, ws)
+    # sums from the epilogue
+    g1 = torch.full_like(x, 3.0)
+    dx1 = torch.full_like(x, 5.0)
+    strips = torch.full((hiplib.bn_bwd_strips_workspace(R, cm) + 8,), float("nan"), device=DEV)
+    dg1, db1 = dg_init.clone(), db_init.clone()
+    fused(g1, strips)
+    hiplib.batchnorm_bwd_strips(x, gamma, mean, rstd, g1, strips, dx1, dg1, db1)
+    torch.cuda.synchronize()
+    assert torch.equal(g1, g0)                                  # the masked gradient: same products, same rounding
+    assert bool(torch.isnan(strips[-8:]).all()) and not bool(torch.isnan(strips[:-8]).any())
+    # fp64 from the stored gradient
+    gd, xd = g1.double().cpu(), x.double().cpu()
+    mask = (a.double().cpu() > 0) if relu else torch.ones_like(gd, dtype=torch.bool)
+    assert rel_err(g1, full * mask) < 1e-2
+    xhat = (xd - mean.double().cpu()) * rstd.double().cpu()
+    sg, sgx = gd.sum(0), (gd * xhat).sum(0)
+    scale_g, scale_gx = gd.abs().sum(0).max(), (gd * xhat).abs().sum(0).max()
+    assert float(((db1 - db_init).double().cpu() - sg).abs().max() / scale_g) < 1e-5
+    assert float(((dg1 - dg_init).double().cpu() - sgx).abs().max() / scale_gx) < 1e-5
+    dx_ref = gamma.double().cpu() * rstd.double().cpu() * (gd - sg / R - xhat * sgx / R)
+    assert rel_err(dx1, dx_ref) < 1e-2
+    # and against the separate kernels: sums equal up to the fp32 order of addition, dx up to an ulp of bf16
+    assert float((db1 - db0).abs().max() / scale_g) < 1e-5 and float((dg1 - dg0).abs().max() / scale_gx) < 1e-5
+    assert float((dx1.float() - dx0.float()).abs().max() / dx0.float().abs().max()) < 2 ** -7
+    # what does not fit is refused before anything is launched
+    with pytest.raises(hiplib.HipKernelError):
+        fused(g1, strips[: hiplib.bn_bwd_strips_workspace(R, cm) - 1])
+    with pytest.raises(hiplib.HipKernelError):
+        hiplib.batchnorm_bwd_strips(x, gamma, mean[:-1], rstd, g1, strips, dx1, dg1, db1)
+
+
 @pytest.mark.parametrize("stride", [1, 2, 3])
 @pytest.mark.parametrize("dtype", DTYPES)
 def test_patch3x3_and_adjoint(hiplib, dtype, stride):
