@@ -97,9 +97,25 @@ __device__ __forceinline__ void epilogue_elem(const GemmArgs& g, int64_t coff, i
 // Vector epilogue for bf16 operands: 8 consecutive columns of one row (n % 8 == 0, n + 8 <= N).
 // (ci, xi: element offsets of (m, n) in C and in the epilogue's operand / second output; b: the bias of the eight
 // columns, read by the caller once for all the rows it stores in them)
-template <bool DROP>
+// The operand the epilogue kind reads beside the product (nullptr: none): the kernels fetch its 16 bytes per lane a
+// patch ahead of their use (epilogue_vec8_at<DROP, true>), so that the loads' latency passes under the previous
+// patch's work instead of in front of every patch's stores.
+__device__ __forceinline__ const bf16* epilogue_operand(const GemmArgs& g) {
+    if (g.epilogue == BB_EPI_DACT || g.epilogue == BB_EPI_MUL || g.epilogue == BB_EPI_MUL_POS) return (const bf16*)g.aux_in;
+    if (g.epilogue == BB_EPI_RESIDUAL) return (const bf16*)g.resid;
+    return nullptr;
+}
+__device__ __forceinline__ void unpack_bf16x8(const u32x4& t, float (&v)[8]) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        v[2 * i] = __uint_as_float(t[i] << 16);
+        v[2 * i + 1] = __uint_as_float(t[i] & 0xffff0000u);
+    }
+}
+// PRE: `pre` holds the 16 bytes of epilogue_operand(g) at xi (fetched earlier)
+template <bool DROP, bool PRE = false>
 __device__ __forceinline__ void epilogue_vec8_at(const GemmArgs& g, int64_t ci, int64_t xi, int m, int n, float (&v)[8],
-                                                 const float (&b)[8]) {
+                                                 const float (&b)[8], const u32x4& pre = u32x4{0u, 0u, 0u, 0u}) {
     if (g.bias) {
 #pragma unroll
         for (int e = 0; e < 8; ++e) v[e] += b[e];
@@ -136,7 +152,8 @@ __device__ __forceinline__ void epilogue_vec8_at(const GemmArgs& g, int64_t ci, 
         }
     } else if (g.epilogue == BB_EPI_DACT) {
         float u[8];
-        load_vec((const bf16*)g.aux_in + xi, u);
+        if constexpr (PRE) unpack_bf16x8(pre, u);
+        else load_vec((const bf16*)g.aux_in + xi, u);
         if (g.act == BB_ACT_RELU) {
 #pragma unroll
             for (int e = 0; e < 8; ++e) v[e] *= u[e] > 0.0f ? 1.0f : 0.0f;
@@ -146,7 +163,8 @@ __device__ __forceinline__ void epilogue_vec8_at(const GemmArgs& g, int64_t ci, 
         }
     } else if (g.epilogue == BB_EPI_RESIDUAL) {
         float r[8];
-        load_vec((const bf16*)g.resid + xi, r);
+        if constexpr (PRE) unpack_bf16x8(pre, r);
+        else load_vec((const bf16*)g.resid + xi, r);
         if (drop) {
 #pragma unroll
             for (int e = 0; e < 8; ++e) v[e] *= keep[e];
@@ -155,12 +173,14 @@ __device__ __forceinline__ void epilogue_vec8_at(const GemmArgs& g, int64_t ci, 
         for (int e = 0; e < 8; ++e) v[e] += r[e];
     } else if (g.epilogue == BB_EPI_MUL) {
         float d[8];
-        load_vec((const bf16*)g.aux_in + xi, d);
+        if constexpr (PRE) unpack_bf16x8(pre, d);
+        else load_vec((const bf16*)g.aux_in + xi, d);
 #pragma unroll
         for (int e = 0; e < 8; ++e) v[e] *= d[e];
     } else if (g.epilogue == BB_EPI_MUL_POS) {
         float d[8];
-        load_vec((const bf16*)g.aux_in + xi, d);
+        if constexpr (PRE) unpack_bf16x8(pre, d);
+        else load_vec((const bf16*)g.aux_in + xi, d);
         if (g.resid) {
             float r[8];
             load_vec((const bf16*)g.resid + xi, r);
@@ -811,6 +831,31 @@ __device__ __forceinline__ void gemm_bf16_dma_body(const GemmArgs& g, const int 
         }
     };
 
+    // the operand of the epilogue kinds that read one, fetched a patch ahead of its use: the four 16-byte pieces of
+    // patch q; patch 0's go out at the top of the last k-tile
+    constexpr int PLD = 68;
+    constexpr int NP = (TN + 1) / 2;   // pairs per row of accumulator tiles, the last one possibly a single
+    const int prow = lane >> 3, pcol = (lane & 7) * 8;
+    // Only on the large tiles (one block per CU, two waves per SIMD whatever the kernel's register count): on the
+    // small ones the 32 registers would cost a resident block.
+    constexpr bool PREF = BM * BN >= 256 * 128 && !VIS && CONV == 0 && STATS == 0;
+    const bf16* opnd = PREF ? epilogue_operand(g) : nullptr;
+    u32x4 opc[PREF ? 4 : 1], opn[PREF ? 4 : 1];
+    auto fetch = [&](auto q_c, u32x4 (&dst)[PREF ? 4 : 1]) {
+        if constexpr (!PREF) return;
+        constexpr int q = decltype(q_c)::value, i = q / NP, jp = q % NP;
+        constexpr int NH = (jp * 2 + 1 < TN) ? 2 : 1;
+        const int n = n0 + wn * WTN + jp * 64 + pcol;
+        const bool live = (NH == 2 || pcol < 32) && n < g.N;
+        const int m_first = m0 + wm * WTM + i * 32 + prow;
+#pragma unroll
+        for (int it = 0; it < (PREF ? 4 : 1); ++it) {
+            const int m = m_first + it * 8;
+            dst[it] = u32x4{0u, 0u, 0u, 0u};
+            if (opnd && live && m < g.M) dst[it] = *(const u32x4*)(opnd + coff + (int64_t)m * g.ldaux + n);
+        }
+    };
+
     if constexpr (BK == 64) {
         // Two stages of 64-wide k-tiles, each multiplied as two 32-wide halves from the two fragment
         // sets.  Per tile one barrier, in the middle of its second half: by then every wave has read
@@ -845,6 +890,7 @@ __device__ __forceinline__ void gemm_bf16_dma_body(const GemmArgs& g, const int 
             rs = rs + 1 == STAGES ? 0 : rs + 1;
             const unsigned char* nxt = smem + rs * STAGE_BYTES;
             if constexpr (STAGES >= 3) {
+                if (kt == KT - 1) fetch(std::integral_constant<int, 0>{}, opc);
                 // the DMA instructions of tile kt+STAGES-1 a third each between the MFMAs of the first three quarters
                 // (issued in one burst at the top they queue up in front of the texture path and the waves behind
                 // them: 2-5 % slower), the second half's fragment reads between the first MFMAs
@@ -962,12 +1008,10 @@ __device__ __forceinline__ void gemm_bf16_dma_body(const GemmArgs& g, const int 
     // 128-byte row segments (256 bytes for fp32 outputs).
     // An odd tile count per row ends with a single tile: its 32 columns use half of the patch and half of
     // the lanes of the row pass.
+    if constexpr (!(BK == 64 && STAGES >= 3)) fetch(std::integral_constant<int, 0>{}, opc);
     wait_vmcnt_lgkm0<0>();  // the tiles issued past the end of K have to land before their stages become the patch
     __syncthreads();
-    constexpr int PLD = 68;
-    constexpr int NP = (TN + 1) / 2;   // pairs per row of accumulator tiles, the last one possibly a single
     float* patch = (float*)smem + wave * (32 * PLD);
-    const int prow = lane >> 3, pcol = (lane & 7) * 8;
     static_for(
         [&](auto idx) {
             constexpr int i = decltype(idx)::value / NP, jp = decltype(idx)::value % NP;
@@ -978,6 +1022,7 @@ __device__ __forceinline__ void gemm_bf16_dma_body(const GemmArgs& g, const int 
                 for (int r = 0; r < 16; ++r)
                     patch[(8 * (r >> 2) + 4 * (lane >> 5) + (r & 3)) * PLD + h * 32 + (lane & 31)] = acc[i][jp * 2 + h][r] * g.alpha;
             asm volatile("" ::: "memory");
+            if constexpr (decltype(idx)::value + 1 < TM * NP) fetch(std::integral_constant<int, decltype(idx)::value + 1>{}, opn);
             const int n = n0 + wn * WTN + jp * 64 + pcol;
             const bool live = (NH == 2 || pcol < 32) && n < g.N;
             // per patch: the bias of the lane's eight columns once, the offsets of its first row by multiplication
@@ -1015,7 +1060,7 @@ __device__ __forceinline__ void gemm_bf16_dma_body(const GemmArgs& g, const int 
                     v[4 + e] = hi[e];
                 }
                 if (live && m < g.M) {
-                    epilogue_vec8_at<DROP>(g, ci, xi, m, n, v, b8);
+                    epilogue_vec8_at<DROP, PREF>(g, ci, xi, m, n, v, b8, opc[PREF ? it : 0]);
                     if constexpr (STATS == 2) {
                         float xv[8];
                         load_vec((const bf16*)bn.x + ci, xv);
@@ -1077,6 +1122,8 @@ __device__ __forceinline__ void gemm_bf16_dma_body(const GemmArgs& g, const int 
                 }
             }
             asm volatile("" ::: "memory");
+#pragma unroll
+            for (int it = 0; it < (PREF ? 4 : 1); ++it) opc[it] = opn[it];
         },
         std::make_integer_sequence<int, TM * NP>{});
 }
@@ -1270,6 +1317,19 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_bf16_dma_persist_kernel(cons
         float b8[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
         if (g.bias && n < g.N) load_vec((const bf16*)g.bias + n, b8);
         int64_t ci = (int64_t)(m0 + prow) * g.ldc + n, xi = (int64_t)(m0 + prow) * g.ldaux + n;
+        // the operand of the epilogue kinds that read one, fetched a patch ahead of its use (inside the epilogue only:
+        // the main loop has no register to spare for it)
+        const bf16* opnd = epilogue_operand(g);
+        u32x4 opc[4], opn[4];
+        auto fetch = [&](int i, u32x4 (&dst)[4]) {
+#pragma unroll
+            for (int it = 0; it < 4; ++it) {
+                const int m = m0 + i * 32 + it * 8 + prow;
+                dst[it] = u32x4{0u, 0u, 0u, 0u};
+                if (opnd && m < g.M && n < g.N) dst[it] = *(const u32x4*)(opnd + (int64_t)m * g.ldaux + n);
+            }
+        };
+        fetch(0, opc);
         // (static_for: a loop the compiler declines to unroll would index the accumulators dynamically, i.e. from scratch)
         static_for(
             [&](auto idx) {
@@ -1282,6 +1342,7 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_bf16_dma_persist_kernel(cons
                         patch[row * 64 + ((((col >> 2) ^ (row & 15)) << 2) | (col & 3))] = acc[i][h][r] * g.alpha;
                     }
                 asm volatile("" ::: "memory");
+                if constexpr (i + 1 < TM) fetch(i + 1, opn);
                 static_for(
                     [&](auto it_c) {
                     constexpr int it = decltype(it_c)::value;
@@ -1290,12 +1351,14 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_bf16_dma_persist_kernel(cons
                     const f32x4 c2 = *(const f32x4*)(patch + row * 64 + ((second_chunk ^ (row & 15)) << 2));
                     const f32x4 lo = pchunk < 4 ? c1 : c2, hi = pchunk < 4 ? c2 : c1;
                     float v[8] = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
-                    if (m < g.M && n < g.N) epilogue_vec8_at<DROP>(g, ci, xi, m, n, v, b8);
+                    if (m < g.M && n < g.N) epilogue_vec8_at<DROP, true>(g, ci, xi, m, n, v, b8, opc[it]);
                     ci += 8 * (int64_t)g.ldc;
                     xi += 8 * (int64_t)g.ldaux;
                     },
                     std::make_integer_sequence<int, 4>{});
                 asm volatile("" ::: "memory");
+#pragma unroll
+                for (int it = 0; it < 4; ++it) opc[it] = opn[it];
             },
             std::make_integer_sequence<int, TM>{});
     }
