@@ -419,6 +419,14 @@ def test_resnet_stage_matches_oracle_with_rc(hiplib, dtype, cin, cmid):
         handover.check()
         own_bufs, _, own_st = handover.own_run()
         compare(own_bufs, own_st, LOOSE_ACT, LOOSE_GRAD, False)
+    # where the kernels exist (bf16, whole 64-channel k-tiles) the BatchNorm backward sums came out of the epilogues of
+    # the kernels that write the gradients, also across the boundary between the stage's two blocks; elsewhere from
+    # the reduction pass
+    fused = {k[0]: v for layer in engine.module.func_buckets[sid] for k, v in layer._stats_ok.items() if k[0] in ("bn_bwd", "sink")}
+    if cmid == 128:
+        assert fused == {"bn_bwd": True, "sink": True}
+    elif cmid == 16:
+        assert not any(fused.values())
     # redundant forwards left the shadow blocks' running statistics alone; own blocks updated theirs M times
     for layer in engine.module.func_buckets[sid + 1]:
         assert layer.running is None
