@@ -112,10 +112,12 @@ __device__ __forceinline__ void unpack_bf16x8(const u32x4& t, float (&v)[8]) {
         v[2 * i + 1] = __uint_as_float(t[i] & 0xffff0000u);
     }
 }
-// PRE: `pre` holds the 16 bytes of epilogue_operand(g) at xi (fetched earlier)
-template <bool DROP, bool PRE = false>
+// PRE: `pre` holds the 16 bytes of epilogue_operand(g) at xi (fetched earlier); PRE2: `pre2` those of g.resid at xi where
+// BB_EPI_MUL_POS has one
+template <bool DROP, bool PRE = false, bool PRE2 = false>
 __device__ __forceinline__ void epilogue_vec8_at(const GemmArgs& g, int64_t ci, int64_t xi, int m, int n, float (&v)[8],
-                                                 const float (&b)[8], const u32x4& pre = u32x4{0u, 0u, 0u, 0u}) {
+                                                 const float (&b)[8], const u32x4& pre = u32x4{0u, 0u, 0u, 0u},
+                                                 const u32x4& pre2 = u32x4{0u, 0u, 0u, 0u}) {
     if (g.bias) {
 #pragma unroll
         for (int e = 0; e < 8; ++e) v[e] += b[e];
@@ -183,7 +185,8 @@ __device__ __forceinline__ void epilogue_vec8_at(const GemmArgs& g, int64_t ci, 
         else load_vec((const bf16*)g.aux_in + xi, d);
         if (g.resid) {
             float r[8];
-            load_vec((const bf16*)g.resid + xi, r);
+            if constexpr (PRE2) unpack_bf16x8(pre2, r);
+            else load_vec((const bf16*)g.resid + xi, r);
 #pragma unroll
             for (int e = 0; e < 8; ++e) v[e] += r[e];
         }
@@ -838,21 +841,35 @@ __device__ __forceinline__ void gemm_bf16_dma_body(const GemmArgs& g, const int 
     const int prow = lane >> 3, pcol = (lane & 7) * 8;
     // Only on the large tiles (one block per CU, two waves per SIMD whatever the kernel's register count): on the
     // small ones the 32 registers would cost a resident block.
+    // Some of the other kernels fetch a patch's operand(s) in one go at the top of that patch: the pointers of GemmArgs
+    // may alias as far as the compiler knows, so left inside the row loop every load waits behind the previous row's
+    // store (four round trips in a row per patch instead of one).
+    // (HOIST: where that does not cost a resident block -- the kernels with the BatchNorm backward sums, whose three
+    // operand reads per row are most of their epilogue)
     constexpr bool PREF = BM * BN >= 256 * 128 && !VIS && CONV == 0 && STATS == 0;
-    const bf16* opnd = PREF ? epilogue_operand(g) : nullptr;
-    u32x4 opc[PREF ? 4 : 1], opn[PREF ? 4 : 1];
-    auto fetch = [&](auto q_c, u32x4 (&dst)[PREF ? 4 : 1]) {
-        if constexpr (!PREF) return;
+    constexpr bool HOIST = STATS == 2;
+    const bf16* opnd = PREF || HOIST ? epilogue_operand(g) : nullptr;
+    u32x4 opc[PREF || HOIST ? 4 : 1], opn[PREF ? 4 : 1];
+    u32x4 xw[STATS == 2 ? 4 : 1], rw[STATS == 2 ? 4 : 1];   // STATS 2: the normalisation's input and the skip gradient
+    auto fetch = [&](auto q_c, u32x4 (&dst)[PREF || HOIST ? 4 : 1]) {
+        if constexpr (!(PREF || HOIST)) return;
         constexpr int q = decltype(q_c)::value, i = q / NP, jp = q % NP;
         constexpr int NH = (jp * 2 + 1 < TN) ? 2 : 1;
         const int n = n0 + wn * WTN + jp * 64 + pcol;
         const bool live = (NH == 2 || pcol < 32) && n < g.N;
         const int m_first = m0 + wm * WTM + i * 32 + prow;
 #pragma unroll
-        for (int it = 0; it < (PREF ? 4 : 1); ++it) {
+        for (int it = 0; it < (PREF || HOIST ? 4 : 1); ++it) {
             const int m = m_first + it * 8;
             dst[it] = u32x4{0u, 0u, 0u, 0u};
             if (opnd && live && m < g.M) dst[it] = *(const u32x4*)(opnd + coff + (int64_t)m * g.ldaux + n);
+            if constexpr (STATS == 2) {
+                xw[it] = rw[it] = u32x4{0u, 0u, 0u, 0u};
+                if (live && m < g.M) {
+                    xw[it] = *(const u32x4*)((const bf16*)bn.x + coff + (int64_t)m * g.ldc + n);
+                    if (g.epilogue == BB_EPI_MUL_POS && g.resid) rw[it] = *(const u32x4*)((const bf16*)g.resid + coff + (int64_t)m * g.ldaux + n);
+                }
+            }
         }
     };
 
@@ -890,7 +907,9 @@ __device__ __forceinline__ void gemm_bf16_dma_body(const GemmArgs& g, const int 
             rs = rs + 1 == STAGES ? 0 : rs + 1;
             const unsigned char* nxt = smem + rs * STAGE_BYTES;
             if constexpr (STAGES >= 3) {
-                if (kt == KT - 1) fetch(std::integral_constant<int, 0>{}, opc);
+                if constexpr (PREF) {
+                    if (kt == KT - 1) fetch(std::integral_constant<int, 0>{}, opc);
+                }
                 // the DMA instructions of tile kt+STAGES-1 a third each between the MFMAs of the first three quarters
                 // (issued in one burst at the top they queue up in front of the texture path and the waves behind
                 // them: 2-5 % slower), the second half's fragment reads between the first MFMAs
@@ -1008,7 +1027,7 @@ __device__ __forceinline__ void gemm_bf16_dma_body(const GemmArgs& g, const int 
     // 128-byte row segments (256 bytes for fp32 outputs).
     // An odd tile count per row ends with a single tile: its 32 columns use half of the patch and half of
     // the lanes of the row pass.
-    if constexpr (!(BK == 64 && STAGES >= 3)) fetch(std::integral_constant<int, 0>{}, opc);
+    if constexpr (PREF && !(BK == 64 && STAGES >= 3)) fetch(std::integral_constant<int, 0>{}, opc);
     wait_vmcnt_lgkm0<0>();  // the tiles issued past the end of K have to land before their stages become the patch
     __syncthreads();
     float* patch = (float*)smem + wave * (32 * PLD);
@@ -1022,7 +1041,8 @@ __device__ __forceinline__ void gemm_bf16_dma_body(const GemmArgs& g, const int 
                 for (int r = 0; r < 16; ++r)
                     patch[(8 * (r >> 2) + 4 * (lane >> 5) + (r & 3)) * PLD + h * 32 + (lane & 31)] = acc[i][jp * 2 + h][r] * g.alpha;
             asm volatile("" ::: "memory");
-            if constexpr (decltype(idx)::value + 1 < TM * NP) fetch(std::integral_constant<int, decltype(idx)::value + 1>{}, opn);
+            if constexpr (HOIST) fetch(idx, opc);
+            else if constexpr (decltype(idx)::value + 1 < TM * NP) fetch(std::integral_constant<int, decltype(idx)::value + 1>{}, opn);
             const int n = n0 + wn * WTN + jp * 64 + pcol;
             const bool live = (NH == 2 || pcol < 32) && n < g.N;
             // per patch: the bias of the lane's eight columns once, the offsets of its first row by multiplication
@@ -1060,10 +1080,10 @@ __device__ __forceinline__ void gemm_bf16_dma_body(const GemmArgs& g, const int 
                     v[4 + e] = hi[e];
                 }
                 if (live && m < g.M) {
-                    epilogue_vec8_at<DROP, PREF>(g, ci, xi, m, n, v, b8, opc[PREF ? it : 0]);
+                    epilogue_vec8_at<DROP, PREF || HOIST, HOIST>(g, ci, xi, m, n, v, b8, opc[PREF || HOIST ? it : 0], rw[HOIST ? it : 0]);
                     if constexpr (STATS == 2) {
                         float xv[8];
-                        load_vec((const bf16*)bn.x + ci, xv);
+                        unpack_bf16x8(xw[it], xv);
 #pragma unroll
                         for (int e = 0; e < 8; ++e) {
                             const float gr = bf2f(f2bf(v[e]));   // what was stored
@@ -1122,8 +1142,10 @@ __device__ __forceinline__ void gemm_bf16_dma_body(const GemmArgs& g, const int 
                 }
             }
             asm volatile("" ::: "memory");
+            if constexpr (PREF) {
 #pragma unroll
-            for (int it = 0; it < (PREF ? 4 : 1); ++it) opc[it] = opn[it];
+                for (int it = 0; it < 4; ++it) opc[it] = opn[it];
+            }
         },
         std::make_integer_sequence<int, TM * NP>{});
 }
