@@ -1,4 +1,4 @@
-// Fused masked softmax-attention for gfx950, bf16, head dimension 64: forward and the two
+// Fused masked softmax-attention for gfx950, bf16, head dimension 64 or 32: forward and the two
 // backward kernels (dK/dV and dQ).  No [batch, heads, seq, seq] tensor ever reaches HBM; the
 // forward keeps one fp32 log-sum-exp per (batch, head, query) for the backward.
 //
@@ -11,7 +11,11 @@
 // buffer.  Each wave owns 32 rows (queries in forward / dQ, keys in dK/dV) and keeps one score
 // COLUMN per lane: scores are produced transposed (S^T = K Q^T), so the softmax reductions over
 // keys are in-lane plus one cross-half shuffle, and P^T comes out of the accumulators already
-// in the register layout the next MFMA wants as its B operand.  Operands that are contracted
+// in the register layout the next MFMA wants as its B operand.  With 32-wide heads (HP = 2) a block
+// owns a PAIR of neighbouring heads, whose columns together are one 64-wide slice: the tiles in LDS,
+// their loads and the fragment layout are those of one 64-wide head, every product takes the k-steps
+// (scores) or the output tile (context, gradients) of its head, the softmax runs once per head.
+// Operands that are contracted
 // over their row index (V in O = PV, Q and dO in dK/dV, K in dQ) are read from LDS with
 // ds_read_b64_tr_b16.  Tiles travel global -> LDS by DMA (global_load_lds_dwordx4),
 // double-buffered.  All reductions have a fixed order: results are reproducible bit for bit.
@@ -179,18 +183,22 @@ static unsigned attn_grid(int seq, int nbh) { return (unsigned)(8 * ((nbh + 7) /
 // =========================================================================================
 // forward: block = 128 queries (4 waves x 32), loop over 64-key tiles
 // =========================================================================================
-template <bool DROP>
+// HP: heads per block (1: 64-wide heads, 2: a pair of 32-wide heads); KS k-steps of a head's scores, DT 32-wide output
+// tiles of a head
+template <bool DROP, int HP>
 __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const AttnArgs a) {
+    constexpr int KS = 4 / HP, DT = 2 / HP;
     __shared__ __attribute__((aligned(16))) unsigned char smem[2 * 2 * 8192];  // 2 stages x (K, V)
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const BlockMap bm = map_block(a.batch * a.heads);
-    if (bm.bh >= a.batch * a.heads) return;
+    const int groups = a.heads / HP;
+    const BlockMap bm = map_block(a.batch * groups);
+    if (bm.bh >= a.batch * groups) return;
     const int qb = (a.seq + 127) / 128 - 1 - bm.rank;  // long (late) query blocks first
-    const int b = bm.bh / a.heads, head = bm.bh % a.heads;
+    const int b = bm.bh / groups, hg = bm.bh % groups, head0 = hg * HP;
     const int64_t row_base = (int64_t)b * a.seq;
-    const bf16* Q = a.q + row_base * a.ld_qkv + head * 64;
-    const bf16* K = a.k + row_base * a.ld_qkv + head * 64;
-    const bf16* V = a.v + row_base * a.ld_qkv + head * 64;
+    const bf16* Q = a.q + row_base * a.ld_qkv + hg * 64;
+    const bf16* K = a.k + row_base * a.ld_qkv + hg * 64;
+    const bf16* V = a.v + row_base * a.ld_qkv + hg * 64;
     const int q0 = qb * 128 + wave * 32;
     const int myq = q0 + (lane & 31);
     const int last = a.seq - 1;
@@ -214,7 +222,12 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const AttnArgs a) {
     for (int t = 0; t < 2; ++t)
 #pragma unroll
         for (int r = 0; r < 16; ++r) o[t][r] = 0.f;
-    float m = -INFINITY, lsum = 0.f;
+    float m[HP], lsum[HP];
+#pragma unroll
+    for (int hh = 0; hh < HP; ++hh) {
+        m[hh] = -INFINITY;
+        lsum[hh] = 0.f;
+    }
 
     const LaneOff lo = lane_off(a.ld_qkv, wave, lane);
     auto issue = [&](int t) {
@@ -240,14 +253,16 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const AttnArgs a) {
         // waves whose queries all precede this tile have nothing to add (causal)
         const bool active = !(a.mask == BB_MASK_CAUSAL && kv0 > q0 + 31);
         if (active) {
+#pragma unroll
+          for (int hh = 0; hh < HP; ++hh) {
             f32x16 s[2];
 #pragma unroll
             for (int u = 0; u < 2; ++u) {
 #pragma unroll
                 for (int r = 0; r < 16; ++r) s[u][r] = 0.f;
 #pragma unroll
-                for (int ks = 0; ks < 4; ++ks)
-                    s[u] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frag_kc(kt, u * 32, ks, lane), qf[ks], s[u], 0, 0, 0);
+                for (int k = 0; k < KS; ++k)
+                    s[u] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frag_kc(kt, u * 32, hh * KS + k, lane), qf[hh * KS + k], s[u], 0, 0, 0);
             }
             // running max on the raw scores (the scale is positive), masking only on tiles that
             // reach past the first key some query of this wave may not see
@@ -267,9 +282,9 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const AttnArgs a) {
 #pragma unroll
                 for (int r = 0; r < 16; ++r) tmax = fmaxf(tmax, s[u][r]);
             tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64)) * a.scale_log2;
-            const float mnew = fmaxf(m, tmax);
+            const float mnew = fmaxf(m[hh], tmax);
             const float msafe = mnew == -INFINITY ? 0.f : mnew;
-            const float alpha = __builtin_amdgcn_exp2f(m - msafe);  // m = -inf -> 0
+            const float alpha = __builtin_amdgcn_exp2f(m[hh] - msafe);  // m = -inf -> 0
             float psum = 0.f;
 #pragma unroll
             for (int u = 0; u < 2; ++u)
@@ -279,67 +294,79 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const AttnArgs a) {
                     s[u][r] = p;
                     psum += p;
                 }
-            lsum = lsum * alpha + psum;
-            m = mnew;
+            lsum[hh] = lsum[hh] * alpha + psum;
+            m[hh] = mnew;
             if (DROP && a.drop.thresh) {   // the normaliser takes every probability, the context only the kept ones
-                const uint64_t base = prob_index(a, b, head, min(myq, last)) + kv0;
+                const uint64_t base = prob_index(a, b, head0 + hh, min(myq, last)) + kv0;
 #pragma unroll
                 for (int u = 0; u < 2; ++u) drop_acc_rows(a.drop, base + u * 32, lane, s[u]);
             }
             if (__any(alpha != 1.0f)) {  // wave-uniform: once the maxima have settled nothing is rescaled
 #pragma unroll
-                for (int t2 = 0; t2 < 2; ++t2)
+                for (int d = 0; d < DT; ++d)
 #pragma unroll
-                    for (int r = 0; r < 16; ++r) o[t2][r] *= alpha;
+                    for (int r = 0; r < 16; ++r) o[hh * DT + d][r] *= alpha;
             }
             // O^T += V^T P^T
 #pragma unroll
             for (int kk = 0; kk < 4; ++kk) {
                 const bf16x8 pf = pack_acc(s[kk >> 1], kk & 1);
 #pragma unroll
-                for (int dt = 0; dt < 2; ++dt)
-                    o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frag_tr(vt, kk * 16, dt * 32, lane), pf, o[dt], 0, 0, 0);
+                for (int d = 0; d < DT; ++d)
+                    o[hh * DT + d] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frag_tr(vt, kk * 16, (hh * DT + d) * 32, lane), pf,
+                                                                             o[hh * DT + d], 0, 0, 0);
             }
+          }
         }
         block_sync();
     }
-    lsum += __shfl_xor(lsum, 32, 64);
-    const float inv = lsum > 0.f ? 1.0f / lsum : 0.f;
+    float inv[HP];
+#pragma unroll
+    for (int hh = 0; hh < HP; ++hh) {
+        lsum[hh] += __shfl_xor(lsum[hh], 32, 64);
+        inv[hh] = lsum[hh] > 0.f ? 1.0f / lsum[hh] : 0.f;
+    }
     if (myq < a.seq) {
-        bf16* op = a.out + (row_base + myq) * a.ld_o + head * 64;
+        bf16* op = a.out + (row_base + myq) * a.ld_o + hg * 64;
 #pragma unroll
         for (int dt = 0; dt < 2; ++dt)
 #pragma unroll
             for (int g4 = 0; g4 < 4; ++g4) {
                 const int d = dt * 32 + 8 * g4 + 4 * (lane >> 5);
-                u32x2 w = {pack2bf(o[dt][g4 * 4] * inv, o[dt][g4 * 4 + 1] * inv),
-                           pack2bf(o[dt][g4 * 4 + 2] * inv, o[dt][g4 * 4 + 3] * inv)};
+                const float iv = inv[dt / DT];
+                u32x2 w = {pack2bf(o[dt][g4 * 4] * iv, o[dt][g4 * 4 + 1] * iv),
+                           pack2bf(o[dt][g4 * 4 + 2] * iv, o[dt][g4 * 4 + 3] * iv)};
                 *(u32x2*)(op + d) = w;
             }
-        if (lane < 32) a.lse[((int64_t)b * a.heads + head) * a.seq + myq] = m + log2f(lsum);
+#pragma unroll
+        for (int hh = 0; hh < HP; ++hh)
+            if (lane < 32) a.lse[((int64_t)b * a.heads + head0 + hh) * a.seq + myq] = m[hh] + log2f(lsum[hh]);
     }
 }
 
 // =========================================================================================
 // backward dK, dV: block = 128 keys (4 waves x 32), loop over 64-query tiles
 // =========================================================================================
-template <bool DROP>
+template <bool DROP, int HP>
 __global__ __launch_bounds__(256, 2) void attn_bwd_dkv_kernel(const AttnArgs a) {
-    // 2 stages x (Q tile 8 KiB, dO tile 8 KiB, lse 256 B, delta 256 B)
-    constexpr int STAGE = 2 * 8192 + 512;
+    constexpr int KS = 4 / HP, DT = 2 / HP;
+    // 2 stages x (Q tile 8 KiB, dO tile 8 KiB, lse 256 B per head, delta 256 B per head)
+    constexpr int STAGE = 2 * 8192 + 512 * HP;
     __shared__ __attribute__((aligned(16))) unsigned char smem[2 * STAGE];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const BlockMap bm = map_block(a.batch * a.heads);
-    if (bm.bh >= a.batch * a.heads) return;
+    const int groups = a.heads / HP;
+    const BlockMap bm = map_block(a.batch * groups);
+    if (bm.bh >= a.batch * groups) return;
     const int kb = bm.rank;  // early key blocks are seen by the most queries
-    const int b = bm.bh / a.heads, head = bm.bh % a.heads;
+    const int b = bm.bh / groups, hg = bm.bh % groups, head0 = hg * HP;
     const int64_t row_base = (int64_t)b * a.seq;
-    const bf16* Q = a.q + row_base * a.ld_qkv + head * 64;
-    const bf16* K = a.k + row_base * a.ld_qkv + head * 64;
-    const bf16* V = a.v + row_base * a.ld_qkv + head * 64;
-    const bf16* DO = a.d_o + row_base * a.ld_o + head * 64;
-    const float* LSE = a.lse + ((int64_t)b * a.heads + head) * a.seq;
-    const float* DELTA = a.delta + ((int64_t)b * a.heads + head) * a.seq;
+    const bf16* Q = a.q + row_base * a.ld_qkv + hg * 64;
+    const bf16* K = a.k + row_base * a.ld_qkv + hg * 64;
+    const bf16* V = a.v + row_base * a.ld_qkv + hg * 64;
+    const bf16* DO = a.d_o + row_base * a.ld_o + hg * 64;
+    // the statistics of the block's heads lie behind each other: [batch, heads, seq]
+    const float* LSE = a.lse + ((int64_t)b * a.heads + head0) * a.seq;
+    const float* DELTA = a.delta + ((int64_t)b * a.heads + head0) * a.seq;
     const int kv0 = kb * 128 + wave * 32;
     const int mykv = kv0 + (lane & 31);
     const int last = a.seq - 1;
@@ -371,8 +398,14 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dkv_kernel(const AttnArgs a) 
         const int qs = t * 64;
         dma_tile64(Q, a.ld_qkv, qs, last, st, wave, lane, lo);
         dma_tile64(DO, a.ld_o, qs, last, st + 8192, wave, lane, lo_o);
-        if (wave == 0) dma_f32x64(LSE, qs, last, st + 16384, lane);
-        if (wave == 1) dma_f32x64(DELTA, qs, last, st + 16384 + 256, lane);
+        // one extra load for waves 0 and 1 (one head), for all four waves (a pair): lse of the heads, then delta
+        if constexpr (HP == 1) {
+            if (wave == 0) dma_f32x64(LSE, qs, last, st + 16384, lane);
+            if (wave == 1) dma_f32x64(DELTA, qs, last, st + 16384 + 256, lane);
+        } else {
+            const float* src = (wave >> 1 ? DELTA : LSE) + (int64_t)(wave & 1) * a.seq;
+            dma_f32x64(src, qs, last, st + 16384 + (wave >> 1) * 512 + (wave & 1) * 256, lane);
+        }
     };
 
     if (q_begin < ntiles) issue(q_begin, 0);
@@ -381,27 +414,33 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dkv_kernel(const AttnArgs a) 
         asm volatile("" ::: "memory");
         if (t + 1 < ntiles) {
             issue(t + 1, slot ^ 1);
-            // waves 0 and 1 carry one extra load each; waiting for <= 5 newer loads covers both cases
-            if (wave < 2) wait_vm<5>(); else wait_vm<4>();
+            // the waves with an extra load wait for <= 5 newer loads, the others for <= 4
+            if (HP == 2 || wave < 2) wait_vm<5>(); else wait_vm<4>();
         } else {
             wait_vm<0>();
         }
         block_sync();
         const unsigned char* qt = smem + slot * STAGE;
         const unsigned char* dot = qt + 8192;
-        const float* lse_t = (const float*)(qt + 16384);
-        const float* del_t = lse_t + 64;
+        const float* lse_all = (const float*)(qt + 16384);
+        const float* del_all = lse_all + 64 * HP;
 #pragma unroll
         for (int u = 0; u < 2; ++u) {
             const int qs = t * 64 + u * 32;
             if (a.mask == BB_MASK_CAUSAL && qs + 31 < kv0) continue;  // all queries precede this wave's keys
             if (qs >= a.seq) continue;
+#pragma unroll
+          for (int hh = 0; hh < HP; ++hh) {
+            const float* lse_t = lse_all + 64 * hh;
+            const float* del_t = del_all + 64 * hh;
+            const int head = head0 + hh;
             // S[q][kv] and dP[q][kv]
             f32x16 s, dp;
 #pragma unroll
             for (int r = 0; r < 16; ++r) s[r] = dp[r] = 0.f;
 #pragma unroll
-            for (int ks = 0; ks < 4; ++ks) {
+            for (int k = 0; k < KS; ++k) {
+                const int ks = hh * KS + k;
                 s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frag_kc(qt, u * 32, ks, lane), kf[ks], s, 0, 0, 0);
                 dp = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frag_kc(dot, u * 32, ks, lane), vf[ks], dp, 0, 0, 0);
             }
@@ -471,11 +510,13 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dkv_kernel(const AttnArgs a) 
             for (int kk = 0; kk < 2; ++kk) {
                 const bf16x8 pf = pack_acc(s, kk), dsf = pack_acc(dp, kk);
 #pragma unroll
-                for (int dt = 0; dt < 2; ++dt) {
+                for (int d = 0; d < DT; ++d) {
+                    const int dt = hh * DT + d;
                     dv[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frag_tr(dot, u * 32 + kk * 16, dt * 32, lane), pf, dv[dt], 0, 0, 0);
                     dk[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frag_tr(qt, u * 32 + kk * 16, dt * 32, lane), dsf, dk[dt], 0, 0, 0);
                 }
             }
+          }
         }
         block_sync();
     }
@@ -486,8 +527,8 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dkv_kernel(const AttnArgs a) 
             for (int r = 0; r < 16; ++r) dk[t][r] = dv[t][r] = 0.f;
     }
     if (mykv < a.seq) {
-        bf16* dkp = a.dk + (row_base + mykv) * a.ld_dqkv + head * 64;
-        bf16* dvp = a.dv + (row_base + mykv) * a.ld_dqkv + head * 64;
+        bf16* dkp = a.dk + (row_base + mykv) * a.ld_dqkv + hg * 64;
+        bf16* dvp = a.dv + (row_base + mykv) * a.ld_dqkv + hg * 64;
 #pragma unroll
         for (int dt = 0; dt < 2; ++dt)
 #pragma unroll
@@ -505,19 +546,21 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dkv_kernel(const AttnArgs a) 
 // =========================================================================================
 // backward dQ: block = 128 queries (4 waves x 32), loop over 64-key tiles
 // =========================================================================================
-template <bool DROP>
+template <bool DROP, int HP>
 __global__ __launch_bounds__(256, 2) void attn_bwd_dq_kernel(const AttnArgs a) {
+    constexpr int KS = 4 / HP, DT = 2 / HP;
     __shared__ __attribute__((aligned(16))) unsigned char smem[2 * 2 * 8192];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const BlockMap bm = map_block(a.batch * a.heads);
-    if (bm.bh >= a.batch * a.heads) return;
+    const int groups = a.heads / HP;
+    const BlockMap bm = map_block(a.batch * groups);
+    if (bm.bh >= a.batch * groups) return;
     const int qb = (a.seq + 127) / 128 - 1 - bm.rank;
-    const int b = bm.bh / a.heads, head = bm.bh % a.heads;
+    const int b = bm.bh / groups, hg = bm.bh % groups, head0 = hg * HP;
     const int64_t row_base = (int64_t)b * a.seq;
-    const bf16* Q = a.q + row_base * a.ld_qkv + head * 64;
-    const bf16* K = a.k + row_base * a.ld_qkv + head * 64;
-    const bf16* V = a.v + row_base * a.ld_qkv + head * 64;
-    const bf16* DO = a.d_o + row_base * a.ld_o + head * 64;
+    const bf16* Q = a.q + row_base * a.ld_qkv + hg * 64;
+    const bf16* K = a.k + row_base * a.ld_qkv + hg * 64;
+    const bf16* V = a.v + row_base * a.ld_qkv + hg * 64;
+    const bf16* DO = a.d_o + row_base * a.ld_o + hg * 64;
     const int q0 = qb * 128 + wave * 32;
     const int myq = q0 + (lane & 31);
     const int last = a.seq - 1;
@@ -538,22 +581,29 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dq_kernel(const AttnArgs a) {
             dof[ks] = *(const bf16x8*)(DO + r * a.ld_o + (lane >> 5) * 8 + ks * 16);
         }
     }
-    const int64_t stat = ((int64_t)b * a.heads + head) * a.seq + min(myq, last);
-    const float my_lse = a.lse[stat];
-    // delta[q] = rowsum(dO o O): the lane and its partner (lane ^ 32) hold the two halves of the query's dO row; the
-    // matching halves of O are fetched once.  Written out for the dK / dV kernel, which runs after this one.
-    float my_delta = 0.f;
+    // delta[q] = rowsum(dO o O) over the head's columns: the lane and its partner (lane ^ 32) hold the two halves of
+    // each 16-column step of the query's dO row; the matching halves of O are fetched once.  Written out for the
+    // dK / dV kernel, which runs after this one.
+    float my_lse[HP], my_delta[HP];
     {
-        const bf16* O = a.o + row_base * a.ld_o + head * 64;
+        const bf16* O = a.o + row_base * a.ld_o + hg * 64;
         const int64_t r = min(myq, last);
 #pragma unroll
-        for (int ks = 0; ks < 4; ++ks) {
-            const bf16x8 of = *(const bf16x8*)(O + r * a.ld_o + (lane >> 5) * 8 + ks * 16);
+        for (int hh = 0; hh < HP; ++hh) {
+            const int64_t stat = ((int64_t)b * a.heads + head0 + hh) * a.seq + min(myq, last);
+            my_lse[hh] = a.lse[stat];
+            float dl = 0.f;
 #pragma unroll
-            for (int e = 0; e < 8; ++e) my_delta = fmaf((float)dof[ks][e], (float)of[e], my_delta);
+            for (int k = 0; k < KS; ++k) {
+                const int ks = hh * KS + k;
+                const bf16x8 of = *(const bf16x8*)(O + r * a.ld_o + (lane >> 5) * 8 + ks * 16);
+#pragma unroll
+                for (int e = 0; e < 8; ++e) dl = fmaf((float)dof[ks][e], (float)of[e], dl);
+            }
+            dl += __shfl_xor(dl, 32, 64);
+            if (lane < 32 && myq < a.seq) a.delta[stat] = dl;
+            my_delta[hh] = dl;
         }
-        my_delta += __shfl_xor(my_delta, 32, 64);
-        if (lane < 32 && myq < a.seq) a.delta[stat] = my_delta;
     }
     f32x16 dq[2];
 #pragma unroll
@@ -585,16 +635,20 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dq_kernel(const AttnArgs a) {
         if (active) {
 #pragma unroll
             for (int u = 0; u < 2; ++u) {
+#pragma unroll
+              for (int hh = 0; hh < HP; ++hh) {
+                const int head = head0 + hh;
                 f32x16 s, dp;
 #pragma unroll
                 for (int r = 0; r < 16; ++r) s[r] = dp[r] = 0.f;
 #pragma unroll
-                for (int ks = 0; ks < 4; ++ks) {
+                for (int k = 0; k < KS; ++k) {
+                    const int ks = hh * KS + k;
                     s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frag_kc(kt, u * 32, ks, lane), qf[ks], s, 0, 0, 0);
                     dp = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frag_kc(vt, u * 32, ks, lane), dof[ks], dp, 0, 0, 0);
                 }
 #pragma unroll
-                for (int r = 0; r < 16; ++r) s[r] = __builtin_amdgcn_exp2f(fmaf(s[r], a.scale_log2, -my_lse));
+                for (int r = 0; r < 16; ++r) s[r] = __builtin_amdgcn_exp2f(fmaf(s[r], a.scale_log2, -my_lse[hh]));
                 if (kv0 + u * 32 + 32 > wave_min_limit) {
                     asm volatile("" ::: "memory");  // a real branch: only tiles on the mask boundary pay for it
                     const int lim = my_limit - kv0 - u * 32 - 4 * (lane >> 5);
@@ -607,21 +661,24 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dq_kernel(const AttnArgs a) {
                     drop_acc_rows(a.drop, base, lane, dp);
                 }
 #pragma unroll
-                for (int r = 0; r < 16; ++r) dp[r] = s[r] * (dp[r] - my_delta);
+                for (int r = 0; r < 16; ++r) dp[r] = s[r] * (dp[r] - my_delta[hh]);
                 // dQ^T += K^T dS^T (contraction over the 32 keys of this sub-tile)
 #pragma unroll
                 for (int kk = 0; kk < 2; ++kk) {
                     const bf16x8 dsf = pack_acc(dp, kk);
 #pragma unroll
-                    for (int dt = 0; dt < 2; ++dt)
+                    for (int d = 0; d < DT; ++d) {
+                        const int dt = hh * DT + d;
                         dq[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frag_tr(kt, u * 32 + kk * 16, dt * 32, lane), dsf, dq[dt], 0, 0, 0);
+                    }
                 }
+              }
             }
         }
         block_sync();
     }
     if (myq < a.seq) {
-        bf16* dqp = a.dq + (row_base + myq) * a.ld_dqkv + head * 64;
+        bf16* dqp = a.dq + (row_base + myq) * a.ld_dqkv + hg * 64;
 #pragma unroll
         for (int dt = 0; dt < 2; ++dt)
 #pragma unroll
@@ -640,11 +697,12 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dq_kernel(const AttnArgs a) {
 static int check_attn(const char* name, int dtype, int mask, int batch, int heads, int seq, int head_dim, int64_t ld_qkv,
                       int64_t ld_o, const int32_t* key_len) {
     BB_REQUIRE(dtype == BB_BF16, "%s: the fused attention kernels are bf16 only (got dtype %d)", name, dtype);
-    BB_REQUIRE(head_dim == 64, "%s: head dimension must be 64 (got %d)", name, head_dim);
+    BB_REQUIRE(head_dim == 64 || (head_dim == 32 && heads % 2 == 0),
+               "%s: head dimension must be 64, or 32 with an even number of heads (got %d, %d heads)", name, head_dim, heads);
     BB_REQUIRE(mask >= BB_MASK_NONE && mask <= BB_MASK_KEY_PADDING, "%s: bad mask %d", name, mask);
     BB_REQUIRE(mask != BB_MASK_KEY_PADDING || key_len, "%s: key_padding mask needs key_len", name);
     BB_REQUIRE(batch >= 0 && heads > 0 && seq >= 0, "%s: bad shape", name);
-    BB_REQUIRE(ld_qkv % 8 == 0 && ld_o % 8 == 0 && ld_qkv >= heads * 64 && ld_o >= heads * 64, "%s: bad leading dimension", name);
+    BB_REQUIRE(ld_qkv % 8 == 0 && ld_o % 8 == 0 && ld_qkv >= heads * head_dim && ld_o >= heads * head_dim, "%s: bad leading dimension", name);
     BB_REQUIRE(ld_qkv < (1 << 24) && ld_o < (1 << 24), "%s: leading dimension too large", name);
     BB_REQUIRE(((int64_t)batch * heads + 8) * ((seq + 127) / 128) < (1ll << 31), "%s: batch * heads * seq exceeds the grid limit", name);
     return BB_OK;
@@ -668,8 +726,16 @@ extern "C" int bb_attention_fwd(int dtype, int mask, int batch, int heads, int s
     a.scale = 1.0f / sqrtf((float)head_dim);
     a.scale_log2 = a.scale * 1.4426950408889634f;
     // dropout is a kernel of its own: its keep decisions cost registers that decide how many blocks a CU holds
-    if (a.drop.thresh) hipLaunchKernelGGL(attn_fwd_kernel<true>, dim3(attn_grid(seq, batch * heads)), dim3(256), 0, (hipStream_t)stream, a);
-    else hipLaunchKernelGGL(attn_fwd_kernel<false>, dim3(attn_grid(seq, batch * heads)), dim3(256), 0, (hipStream_t)stream, a);
+    const int hp = 64 / head_dim;   // heads per block
+    const dim3 grid(attn_grid(seq, batch * (heads / hp)));
+    hipStream_t st = (hipStream_t)stream;
+    if (hp == 1) {
+        if (a.drop.thresh) hipLaunchKernelGGL((attn_fwd_kernel<true, 1>), grid, dim3(256), 0, st, a);
+        else hipLaunchKernelGGL((attn_fwd_kernel<false, 1>), grid, dim3(256), 0, st, a);
+    } else {
+        if (a.drop.thresh) hipLaunchKernelGGL((attn_fwd_kernel<true, 2>), grid, dim3(256), 0, st, a);
+        else hipLaunchKernelGGL((attn_fwd_kernel<false, 2>), grid, dim3(256), 0, st, a);
+    }
     BB_LAUNCH_CHECK();
     return BB_OK;
 }
@@ -683,7 +749,7 @@ extern "C" int bb_attention_bwd(int dtype, int mask, int batch, int heads, int s
     if (rc) return rc;
     if (batch == 0 || seq == 0) return BB_OK;
     BB_REQUIRE(q && k && v && out && d_out && lse && delta && dq && dk && dv, "bb_attention_bwd: null pointer");
-    BB_REQUIRE(ld_dqkv % 4 == 0 && ld_dqkv >= heads * 64, "bb_attention_bwd: bad gradient leading dimension");
+    BB_REQUIRE(ld_dqkv % 4 == 0 && ld_dqkv >= heads * head_dim, "bb_attention_bwd: bad gradient leading dimension");
     BB_REQUIRE(dropout_p >= 0.f && dropout_p < 1.f, "bb_attention_bwd: dropout_p must be in [0, 1)");
     AttnArgs a = {};
     a.drop = bb_drop_key(dropout_p, dropout_k0, dropout_k1, (uint64_t)batch * heads * (uint64_t)seq * (uint64_t)seq);
@@ -697,13 +763,24 @@ extern "C" int bb_attention_bwd(int dtype, int mask, int batch, int heads, int s
     a.scale_log2 = a.scale * 1.4426950408889634f;
     hipStream_t st = (hipStream_t)stream;
     // the dQ kernel first: it also leaves delta = rowsum(dO o O) of its queries for the dK / dV kernel
-    dim3 grid(attn_grid(seq, batch * heads));
-    if (a.drop.thresh) {
-        hipLaunchKernelGGL(attn_bwd_dq_kernel<true>, grid, dim3(256), 0, st, a);
-        hipLaunchKernelGGL(attn_bwd_dkv_kernel<true>, grid, dim3(256), 0, st, a);
+    const int hp = 64 / head_dim;   // heads per block
+    dim3 grid(attn_grid(seq, batch * (heads / hp)));
+    if (hp == 1) {
+        if (a.drop.thresh) {
+            hipLaunchKernelGGL((attn_bwd_dq_kernel<true, 1>), grid, dim3(256), 0, st, a);
+            hipLaunchKernelGGL((attn_bwd_dkv_kernel<true, 1>), grid, dim3(256), 0, st, a);
+        } else {
+            hipLaunchKernelGGL((attn_bwd_dq_kernel<false, 1>), grid, dim3(256), 0, st, a);
+            hipLaunchKernelGGL((attn_bwd_dkv_kernel<false, 1>), grid, dim3(256), 0, st, a);
+        }
     } else {
-        hipLaunchKernelGGL(attn_bwd_dq_kernel<false>, grid, dim3(256), 0, st, a);
-        hipLaunchKernelGGL(attn_bwd_dkv_kernel<false>, grid, dim3(256), 0, st, a);
+        if (a.drop.thresh) {
+            hipLaunchKernelGGL((attn_bwd_dq_kernel<true, 2>), grid, dim3(256), 0, st, a);
+            hipLaunchKernelGGL((attn_bwd_dkv_kernel<true, 2>), grid, dim3(256), 0, st, a);
+        } else {
+            hipLaunchKernelGGL((attn_bwd_dq_kernel<false, 2>), grid, dim3(256), 0, st, a);
+            hipLaunchKernelGGL((attn_bwd_dkv_kernel<false, 2>), grid, dim3(256), 0, st, a);
+        }
     }
     BB_LAUNCH_CHECK();
     return BB_OK;

@@ -435,10 +435,17 @@ def _drop_args(dropout):
     return float(dropout[0]), int(dropout[1][0]), int(dropout[1][1])
 
 
+FUSED_HEAD_DIMS = (64, 32)   # the fused attention kernels: 64-wide heads, or pairs of 32-wide heads
+
+
 def _check_attention(what, qkv, batch, heads, seq, key_len, lse, out=None, d_out=None, delta=None, d_qkv=None):
-    """qkv / d_qkv: [batch*seq, 3*heads*64], out / d_out: [batch*seq, heads*64] (rows may be strided views with a unit
+    """qkv / d_qkv: [batch*seq, 3*heads*d], out / d_out: [batch*seq, heads*d] (rows may be strided views with a unit
     inner stride), lse / delta: fp32 with batch*heads*seq contiguous elements, key_len: int32 [batch]."""
-    rows, h = batch * seq, heads * 64
+    if qkv.dim() != 2 or qkv.shape[1] % (3 * heads) != 0 or qkv.shape[1] // (3 * heads) not in FUSED_HEAD_DIMS or \
+            (qkv.shape[1] // (3 * heads) == 32 and heads % 2 != 0):
+        raise HipKernelError(f"{what}: qkv must be [rows, 3 * heads * d] with d = 64, or d = 32 and an even number of heads; "
+                             f"got {tuple(qkv.shape)} for {heads} heads")
+    rows, h = batch * seq, qkv.shape[1] // 3
     for name, t, width in (("qkv", qkv, 3 * h), ("d_qkv", d_qkv, 3 * h), ("out", out, h), ("d_out", d_out, h)):
         if t is None:
             continue
@@ -450,10 +457,11 @@ def _check_attention(what, qkv, batch, heads, seq, key_len, lse, out=None, d_out
 
 
 def attention_fwd(qkv, out, lse, batch, heads, seq, mask, key_len=None, stream=None, dropout=None):
-    """qkv: [batch*seq, 3*heads*64] (Q | K | V thirds), out: [batch*seq, heads*64], lse: fp32 [batch, heads, seq].
+    """qkv: [batch*seq, 3*heads*d] (Q | K | V thirds), out: [batch*seq, heads*d], lse: fp32 [batch, heads, seq]; head
+    dimension d = 64, or 32 with an even number of heads.
     ``dropout=(p, (k0, k1))``: dropout on the probabilities with the decisions of that key."""
     _check_attention("attention_fwd", qkv, batch, heads, seq, key_len, lse, out=out)
-    h = heads * 64
+    h = qkv.shape[1] // 3
     es = qkv.element_size()
     q = qkv.data_ptr()
     check(lib().bb_attention_fwd(dtype_code(qkv.dtype), mask, batch, heads, seq, qkv.shape[1] // (3 * heads),
@@ -466,7 +474,7 @@ def attention_bwd(qkv, out, d_out, lse, delta, d_qkv, batch, heads, seq, mask, k
     _check_attention("attention_bwd", qkv, batch, heads, seq, key_len, lse, out=out, d_out=d_out, delta=delta, d_qkv=d_qkv)
     if d_out.stride(0) != out.stride(0):
         raise HipKernelError("attention_bwd: out and d_out must share one leading dimension")
-    h = heads * 64
+    h = qkv.shape[1] // 3
     es = qkv.element_size()
     q, dq = qkv.data_ptr(), d_qkv.data_ptr()
     check(lib().bb_attention_bwd(dtype_code(qkv.dtype), mask, batch, heads, seq, qkv.shape[1] // (3 * heads),

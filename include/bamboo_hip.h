@@ -220,11 +220,13 @@ int bb_softmax_fwd(int dtype, int mask, int batch, int heads, int sq, int sk, vo
 int bb_softmax_bwd(int dtype, int batch, int heads, int sq, int sk, const void* p, void* dp,
                    void* stream);
 
-/* Fused masked softmax-attention (bf16, head_dim 64): out = softmax(Q K^T / sqrt(d), mask) V for
- * every (batch, head), without materialising the score matrix (transformer.py:117-127).
+/* Fused masked softmax-attention (bf16; head_dim d = 64, or d = 32 with an even number of heads -- the kernels
+ * then take two neighbouring heads per block; gpt2.py:212-214 defaults to 512 / 16 = 32):
+ * out = softmax(Q K^T / sqrt(d), mask) V for every (batch, head), without materialising the score matrix
+ * (transformer.py:117-127).
  * q, k, v point at head 0 of batch 0; rows are tokens (batch-major), head j occupies columns
- * j*64.. of each pointer, row stride ld_qkv (the three pointers may alias one [rows, 3h] buffer).
- * out: [rows, heads*64] with row stride ld_out.  lse: fp32 [batch, heads, seq] log-sum-exp (base 2,
+ * j*d.. of each pointer, row stride ld_qkv (the three pointers may alias one [rows, 3h] buffer).
+ * out: [rows, heads*d] with row stride ld_out.  lse: fp32 [batch, heads, seq] log-sum-exp (base 2,
  * scaled scores) kept for the backward.
  * dropout_p > 0: dropout on the probabilities (transformer.py:125-126), out = (P o mask / (1 - p)) V with the
  * decisions of key (dropout_k0, dropout_k1) at element ((batch * heads + head) * seq + query) * seq + key;

@@ -82,11 +82,12 @@ def test_gemm_epilogue_dropout(hiplib, dtype, M, N, K, epi):
 
 
 @pytest.mark.parametrize("mask", ["none", "causal", "key_padding"])
-@pytest.mark.parametrize("batch,heads,seq", [(2, 2, 128), (1, 3, 200)])
-def test_fused_attention_dropout_fwd_bwd(hiplib, mask, batch, heads, seq):
+@pytest.mark.parametrize("batch,heads,seq,d", [(2, 2, 128, 64), (1, 3, 200, 64), (2, 4, 128, 32), (1, 2, 200, 32)])
+def test_fused_attention_dropout_fwd_bwd(hiplib, mask, batch, heads, seq, d):
     """softmax(QK^T / sqrt(d), mask) -> dropout -> V with the oracle's explicit mask through torch autograd in fp64,
-    against the fused kernels that evaluate the decisions themselves: context, dQ, dK, dV."""
-    p, h = 0.2, heads * 64
+    against the fused kernels that evaluate the decisions themselves: context, dQ, dK, dV (64-wide heads, and 32-wide
+    heads in pairs: every head keeps its own decisions)."""
+    p, h = 0.2, heads * d
     g = torch.Generator(device=DEV).manual_seed(9)
     qkv = (torch.randn(batch * seq, 3 * h, generator=g, device=DEV) * 0.7).to(torch.bfloat16)
     d_out = torch.randn(batch * seq, h, generator=g, device=DEV).to(torch.bfloat16)
@@ -99,9 +100,9 @@ def test_fused_attention_dropout_fwd_bwd(hiplib, mask, batch, heads, seq):
     delta, d_qkv = torch.empty(batch, heads, seq, device=DEV), torch.empty_like(qkv)
     hiplib.attention_bwd(qkv, out, d_out, lse, delta, d_qkv, batch, heads, seq, code, lens, dropout=(p, KEY))
     # reference
-    x = qkv.double().cpu().view(batch, seq, 3, heads, 64).requires_grad_(True)
+    x = qkv.double().cpu().view(batch, seq, 3, heads, d).requires_grad_(True)
     q, k, v = [x[:, :, i].transpose(1, 2) for i in range(3)]
-    sc = q @ k.transpose(-2, -1) / 8.0
+    sc = q @ k.transpose(-2, -1) / d ** 0.5
     if mask == "causal":
         sc = sc.masked_fill(~torch.tril(torch.ones(seq, seq, dtype=torch.bool)), -1e9)
     elif mask == "key_padding":

@@ -338,13 +338,15 @@ def test_unfused_attention_fp32_at_12_heads_512_positions(hiplib, mask):
 
 
 @pytest.mark.parametrize("mask", ["none", "causal", "key_padding"])
-@pytest.mark.parametrize("d", [32, 128])
-def test_bf16_attention_with_other_head_widths(hiplib, mask, d):
-    """bf16 heads that are not 64 wide (the reference's GPT-2 script defaults to 512 / 16 = 32, gpt2.py:212-214) take
-    the path that materialises the probabilities: context and the three input gradients against fp64 autograd on
-    ``softmax(Q K^T / sqrt(d) [masked]) V``, 2e-2 of each tensor's largest magnitude, for the three masks."""
+@pytest.mark.parametrize("d,a,fused", [(32, 4, True), (32, 3, False), (128, 4, False)], ids=["d32-pairs-fused", "d32-odd-heads", "d128"])
+def test_bf16_attention_with_other_head_widths(hiplib, mask, d, a, fused):
+    """bf16 heads that are not 64 wide, through the layer's attention calls.  An even number of 32-wide heads (the
+    reference's GPT-2 script defaults to 512 / 16 = 32, gpt2.py:212-214) runs on the fused kernels, which take the
+    heads in pairs; an odd number of them and 128-wide heads take the path that materialises the probabilities.
+    Context and the three input gradients against fp64 autograd on ``softmax(Q K^T / sqrt(d) [masked]) V``, 2e-2 of
+    each tensor's largest magnitude, for the three masks."""
     from bamboo_amd.layers import StageContext
-    b, a, s = 2, 4, 256
+    b, s = 2, 256
     h = a * d
     layer = TransformerLayer(h, a, 4 * h, activation="gelu_tanh", ln="standard", mask=mask)
     ctx = StageContext(b, s, torch.bfloat16, torch.device(DEV))
@@ -355,9 +357,9 @@ def test_bf16_attention_with_other_head_widths(hiplib, mask, d):
     qkv = randn(b * s, 3 * h, seed=51, scale=0.7)
     d_ctx = randn(b * s, h, seed=52)
     st = {"qkv": qkv, "ctx": torch.empty(b * s, h, dtype=torch.bfloat16, device=DEV),
-          "prob": torch.empty(b, a, s, s, dtype=torch.bfloat16, device=DEV)}
-    ctx.ensure_scratch([("d_prob", (b, a, s, s), torch.bfloat16)])
-    assert not layer.fused_attention(ctx)
+          "prob": torch.empty(b, a, s, s, dtype=torch.bfloat16, device=DEV), "lse": torch.empty(b, a, s, device=DEV)}
+    ctx.ensure_scratch([("d_prob", (b, a, s, s), torch.bfloat16), ("attn_delta", (b, a, s), torch.float32)])
+    assert layer.fused_attention(ctx) == fused
     layer._attention_fwd(st, ctx)
     d_qkv = torch.empty_like(qkv)
     layer._attention_bwd(d_ctx, d_qkv, st, ctx)

@@ -345,11 +345,12 @@ def test_softmax(hiplib, dtype, mask):
 
 
 @pytest.mark.parametrize("mask", ["none", "causal", "key_padding"])
-@pytest.mark.parametrize("b,a,s", [(2, 3, 128), (1, 2, 64), (2, 2, 96), (1, 4, 384), (3, 1, 32), (1, 16, 1024)])
-def test_fused_attention_fwd_bwd(hiplib, mask, b, a, s):
-    """Fused attention (bf16, d = 64) against softmax(QK^T/sqrt(d), mask) V and its autograd gradients,
-    computed in fp64 from the same bf16 inputs."""
-    d, h = 64, a * 64
+@pytest.mark.parametrize("b,a,s,d", [(2, 3, 128, 64), (1, 2, 64, 64), (2, 2, 96, 64), (1, 4, 384, 64), (3, 1, 32, 64), (1, 16, 1024, 64),
+                                     (2, 6, 128, 32), (1, 2, 64, 32), (2, 4, 96, 32), (3, 2, 32, 32), (1, 16, 1024, 32)])
+def test_fused_attention_fwd_bwd(hiplib, mask, b, a, s, d):
+    """Fused attention (bf16, d = 64, and d = 32 with the heads taken in pairs) against softmax(QK^T/sqrt(d), mask) V and
+    its autograd gradients, computed in fp64 from the same bf16 inputs."""
+    h = a * d
     qkv = randn(b * s, 3 * h, dtype=torch.bfloat16, seed=70, scale=1.0)
     d_out = randn(b * s, h, dtype=torch.bfloat16, seed=71)
     lens = None
@@ -391,6 +392,18 @@ def test_fused_attention_rejects(hiplib):
     qkv = torch.zeros(64, 3 * 64, device=DEV)
     with pytest.raises(hiplib.HipKernelError):
         hiplib.attention_fwd(qkv, torch.zeros(64, 64, device=DEV), torch.zeros(1, 1, 64, device=DEV), 1, 1, 64, 0)  # fp32
+    # 32-wide heads go in pairs: an odd number of them is refused (by the wrapper, and by the library itself)
+    q3 = torch.zeros(64, 3 * 96, dtype=torch.bfloat16, device=DEV)
+    o3, l3 = torch.zeros(64, 96, dtype=torch.bfloat16, device=DEV), torch.zeros(1, 3, 64, device=DEV)
+    with pytest.raises(hiplib.HipKernelError):
+        hiplib.attention_fwd(q3, o3, l3, 1, 3, 64, 0)
+    L = hiplib.lib()
+    rc = L.bb_attention_fwd(hiplib.BF16, 0, 1, 3, 64, 32, q3.data_ptr(), q3.data_ptr() + 192, q3.data_ptr() + 384, 288, o3.data_ptr(), 96,
+                            l3.data_ptr(), None, 0.0, 0, 0, None)
+    assert rc != 0 and b"even number of heads" in L.bb_last_error()
+    rc = L.bb_attention_fwd(hiplib.BF16, 0, 1, 1, 64, 128, q3.data_ptr(), q3.data_ptr(), q3.data_ptr(), 384, o3.data_ptr(), 128,
+                            l3.data_ptr(), None, 0.0, 0, 0, None)
+    assert rc != 0 and b"head dimension" in L.bb_last_error()
 
 
 @pytest.mark.parametrize("dtype", DTYPES)

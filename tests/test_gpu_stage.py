@@ -914,15 +914,17 @@ def test_sigterm_and_launch_observer_belong_to_one_engine(hiplib):
         signal.signal(signal.SIGTERM, prev)
 
 
-@pytest.mark.parametrize("heads", [4, 1], ids=["head-width-32", "head-width-128"])
-def test_bf16_stage_with_other_head_widths_matches_oracle(hiplib, heads):
-    """A bf16 stage whose heads are 32 (the reference GPT-2 script's default, gpt2.py:212-214) or 128 wide, with
-    redundant forwards: outputs, input gradients and parameter gradients against the fp64 oracle at the bf16 bars,
-    and the redundant forward's output bit-equal to the own forward of the same layers on the same input."""
-    hid, ffn, L, S, sid, mb, M, seq = 128, 256, 2, 4, 1, 2, 4, 64
+@pytest.mark.parametrize("hid,heads,fused", [(128, 4, True), (96, 3, False), (128, 1, False)],
+                         ids=["head-width-32-pairs", "head-width-32-odd-heads", "head-width-128"])
+def test_bf16_stage_with_other_head_widths_matches_oracle(hiplib, hid, heads, fused):
+    """A bf16 stage whose heads are 32 (the reference GPT-2 script's default, gpt2.py:212-214: the fused kernels take
+    an even number of them in pairs, an odd number materialises the probabilities) or 128 wide, with redundant
+    forwards: outputs, input gradients and parameter gradients against the fp64 oracle at the bf16 bars, and the
+    redundant forward's output bit-equal to the own forward of the same layers on the same input."""
+    ffn, L, S, sid, mb, M, seq = 256, 2, 4, 1, 2, 4, 64
     dtype = torch.bfloat16
     engine, q = build(hid, heads, ffn, L, S, sid, mb, M, seq, dtype, GPT_VARIANT, 1, True)
-    assert not engine.module.func_buckets[sid][0].fused_attention(engine.ctx)
+    assert engine.module.func_buckets[sid][0].fused_attention(engine.ctx) == fused
     st, peer = oracle_for(engine, q, GPT_VARIANT, hid, heads, ffn, L, S, sid, M, 1, True)
     keep = {}
     with NoStep(engine):
