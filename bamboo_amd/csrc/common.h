@@ -88,6 +88,13 @@ template <> struct Elem<bf16> {
 };
 
 // 16-byte vector load/store of VEC elements <-> float registers
+// One element's share of the backward sums of a batch normalisation (sum g, sum g * xhat with xhat = (x - mean) * rstd),
+// in explicitly rounded steps: whichever kernel adds the sums up -- the epilogue of the GEMM that writes g, or the
+// stand-alone pass -- the compiler contracts nothing, and with the same order of additions the bits are the same.
+__device__ __forceinline__ void bn_bwd_sums_add(float g, float x, float mu, float rs, float& sg, float& sgx) {
+    sg = __fadd_rn(sg, g);
+    sgx = __fadd_rn(sgx, __fmul_rn(__fmul_rn(g, __fsub_rn(x, mu)), rs));
+}
 __device__ __forceinline__ void load_vec(const float* p, float (&v)[4]) {
     f32x4 t = *(const f32x4*)p;
     v[0] = t.x; v[1] = t.y; v[2] = t.z; v[3] = t.w;

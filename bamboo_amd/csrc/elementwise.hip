@@ -1598,6 +1598,94 @@ extern "C" int bb_batchnorm_bwd(int dtype, int rows, int cols, const void* x, co
     return BB_OK;
 }
 
+// The strip sums where no GEMM epilogue left them (the gradient arrived from another stage, or the shape is not one
+// the kernels with the sums take): a wave owns one 32-row strip x 64 columns and adds up exactly as those epilogues
+// do -- lane (row group l / 8, eight columns) over its four rows in row order, then the eight row groups in order
+// through LDS -- so both ways give the same bits.  Also writes the masked gradient g = dy * (relu_out > 0) (g_out may
+// be dy itself).
+__global__ __launch_bounds__(256) void bn_bwd_strip_sums_kernel(int rows, int cols, const bf16* x, const float* __restrict__ mean,
+                                                                const float* __restrict__ rstd, const bf16* dy, const bf16* relu_out,
+                                                                bf16* g_out, float* __restrict__ strips) {
+    constexpr int PLD = 68;
+    __shared__ float patches[4][16 * PLD];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int strip = blockIdx.y * 4 + wave;
+    if (strip * 32 >= rows) return;   // no block-wide barrier below
+    float* patch = patches[wave];
+    const int prow = lane >> 3, pcol = (lane & 7) * 8;
+    const int n = blockIdx.x * 64 + pcol;
+    const bool live = n < cols;
+    float mu8[8], rs8[8], sg[8], sgx[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) mu8[e] = rs8[e] = sg[e] = sgx[e] = 0.f;
+    if (live) {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            mu8[e] = mean[n + e];
+            rs8[e] = rstd[n + e];
+        }
+    }
+    u32x4 gw[4], xw[4], ow[4];
+#pragma unroll
+    for (int it = 0; it < 4; ++it) {
+        const int m = strip * 32 + it * 8 + prow;
+        gw[it] = xw[it] = ow[it] = u32x4{0u, 0u, 0u, 0u};
+        if (live && m < rows) {
+            const int64_t off = (int64_t)m * cols + n;
+            gw[it] = *(const u32x4*)(dy + off);
+            xw[it] = *(const u32x4*)(x + off);
+            if (relu_out) ow[it] = *(const u32x4*)(relu_out + off);
+        }
+    }
+#pragma unroll
+    for (int it = 0; it < 4; ++it) {
+        const int m = strip * 32 + it * 8 + prow;
+        if (live && m < rows) {
+            float g[8], xv[8], o[8];
+            unpack16(gw[it], g);
+            unpack16(xw[it], xv);
+            if (relu_out) {
+                unpack16(ow[it], o);
+#pragma unroll
+                for (int e = 0; e < 8; ++e) g[e] = o[e] > 0.f ? g[e] : 0.f;
+            }
+            if (g_out) store_vec(g_out + (int64_t)m * cols + n, g);
+#pragma unroll
+            for (int e = 0; e < 8; ++e) bn_bwd_sums_add(g[e], xv[e], mu8[e], rs8[e], sg[e], sgx[e]);
+        }
+    }
+    *(f32x4*)(patch + prow * PLD + pcol) = f32x4{sg[0], sg[1], sg[2], sg[3]};
+    *(f32x4*)(patch + prow * PLD + pcol + 4) = f32x4{sg[4], sg[5], sg[6], sg[7]};
+    *(f32x4*)(patch + (8 + prow) * PLD + pcol) = f32x4{sgx[0], sgx[1], sgx[2], sgx[3]};
+    *(f32x4*)(patch + (8 + prow) * PLD + pcol + 4) = f32x4{sgx[4], sgx[5], sgx[6], sgx[7]};
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");   // the wave's own writes, then its reads: no other wave is involved
+    float t0 = 0.f, t1 = 0.f;
+#pragma unroll
+    for (int r = 0; r < 8; ++r) {
+        t0 = __fadd_rn(t0, patch[r * PLD + lane]);
+        t1 = __fadd_rn(t1, patch[(8 + r) * PLD + lane]);
+    }
+    const int nc = blockIdx.x * 64 + lane;
+    if (nc < cols) {
+        strips[((int64_t)strip * 2) * cols + nc] = t0;
+        strips[((int64_t)strip * 2 + 1) * cols + nc] = t1;
+    }
+}
+
+extern "C" int bb_batchnorm_bwd_strip_sums(int dtype, int rows, int cols, const void* x, const float* mean, const float* rstd,
+                                           const void* dy, const void* relu_out, void* g_out, float* strips, void* stream) {
+    int rc = check_bn("bb_batchnorm_bwd_strip_sums", dtype, rows, cols);
+    if (rc) return rc;
+    BB_REQUIRE(dtype == BB_BF16, "bb_batchnorm_bwd_strip_sums: bf16 only");
+    BB_REQUIRE(x && mean && rstd && dy && strips, "bb_batchnorm_bwd_strip_sums: null pointer");
+    BB_REQUIRE(!relu_out || g_out, "bb_batchnorm_bwd_strip_sums: with relu_out the masked gradient needs a place (g_out, may be dy)");
+    const int nstrips = (rows + 31) / 32;
+    hipLaunchKernelGGL(bn_bwd_strip_sums_kernel, dim3((cols + 63) / 64, (nstrips + 3) / 4), dim3(256), 0, (hipStream_t)stream, rows, cols,
+                       (const bf16*)x, mean, rstd, (const bf16*)dy, (const bf16*)relu_out, (bf16*)g_out, strips);
+    BB_LAUNCH_CHECK();
+    return BB_OK;
+}
+
 extern "C" int bb_batchnorm_bwd_strips(int dtype, int rows, int cols, const void* x, const void* gamma, const float* mean,
                                        const float* rstd, const void* g, const float* strips, void* dx, float* dgamma,
                                        float* dbeta, void* stream) {

@@ -1085,11 +1085,7 @@ __device__ __forceinline__ void gemm_bf16_dma_body(const GemmArgs& g, const int 
                         float xv[8];
                         unpack_bf16x8(xw[it], xv);
 #pragma unroll
-                        for (int e = 0; e < 8; ++e) {
-                            const float gr = bf2f(f2bf(v[e]));   // what was stored
-                            sg[e] += gr;
-                            sgx[e] += gr * (xv[e] - mu8[e]) * rs8[e];
-                        }
+                        for (int e = 0; e < 8; ++e) bn_bwd_sums_add(bf2f(f2bf(v[e])) /* what was stored */, xv[e], mu8[e], rs8[e], sg[e], sgx[e]);
                     }
                 }
                 ci += 8 * (int64_t)g.ldc;
@@ -1107,8 +1103,8 @@ __device__ __forceinline__ void gemm_bf16_dma_body(const GemmArgs& g, const int 
                 float t0 = 0.f, t1 = 0.f;
 #pragma unroll
                 for (int r = 0; r < 8; ++r) {
-                    t0 += patch[r * PLD + lane];
-                    t1 += patch[(8 + r) * PLD + lane];
+                    t0 = __fadd_rn(t0, patch[r * PLD + lane]);
+                    t1 = __fadd_rn(t1, patch[(8 + r) * PLD + lane]);
                 }
                 const int strip_row = m0 + wm * WTM + i * 32;
                 const int nc = n0 + wn * WTN + jp * 64 + lane;

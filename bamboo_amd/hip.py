@@ -25,7 +25,7 @@ LN_CODES = {"standard": LN_STANDARD, "annotated": LN_ANNOTATED}
 EXPORTS = (
     "bb_version", "bb_last_error", "bb_init", "bb_gemm", "bb_gemm_grouped", "bb_gemm_splitk_workspace", "bb_gemm_grouped_splitk", "bb_gemm_variant", "bb_layernorm_fwd",
     "bb_layernorm_bwd_workspace", "bb_layernorm_bwd", "bb_layernorm_bwd_static", "bb_colsum_workspace", "bb_colsum_acc", "bb_rowsum_fwd", "bb_rowsum_bwd", "bb_dropout_apply", "bb_dropout_keep_host",
-    "bb_softmax_fwd", "bb_softmax_bwd", "bb_attention_fwd", "bb_attention_bwd", "bb_residual_add", "bb_sqrt_one_minus_fwd", "bb_sqrt_one_minus_bwd", "bb_act_fwd", "bb_bn_workspace", "bb_batchnorm_fwd", "bb_batchnorm_bwd", "bb_patch3x3", "bb_patch3x3_strided", "bb_subsample", "bb_conv3x3_supported", "bb_conv3x3", "bb_gemm_strip_stats_supported", "bb_strip_stats_workspace", "bb_batchnorm_fwd_strips", "bb_bn_bwd_strips_workspace", "bb_gemm_bn_bwd_supported", "bb_gemm_bn_bwd", "bb_conv3x3_dgrad_bn", "bb_batchnorm_bwd_strips", "bb_mse_workspace", "bb_mse_fwd_bwd", "bb_graph_begin", "bb_graph_end", "bb_graph_launch", "bb_graph_destroy",
+    "bb_softmax_fwd", "bb_softmax_bwd", "bb_attention_fwd", "bb_attention_bwd", "bb_residual_add", "bb_sqrt_one_minus_fwd", "bb_sqrt_one_minus_bwd", "bb_act_fwd", "bb_bn_workspace", "bb_batchnorm_fwd", "bb_batchnorm_bwd", "bb_patch3x3", "bb_patch3x3_strided", "bb_subsample", "bb_conv3x3_supported", "bb_conv3x3", "bb_gemm_strip_stats_supported", "bb_strip_stats_workspace", "bb_batchnorm_fwd_strips", "bb_bn_bwd_strips_workspace", "bb_gemm_bn_bwd_supported", "bb_gemm_bn_bwd", "bb_conv3x3_dgrad_bn", "bb_batchnorm_bwd_strips", "bb_batchnorm_bwd_strip_sums", "bb_mse_workspace", "bb_mse_fwd_bwd", "bb_graph_begin", "bb_graph_end", "bb_graph_launch", "bb_graph_destroy",
     "bb_adam_multi", "bb_adam_multi_scaled", "bb_grad_clip_workspace", "bb_grad_clip_coef", "bb_cast", "bb_fill_f32",
 )
 
@@ -131,6 +131,7 @@ def lib():
     L.bb_gemm_bn_bwd.argtypes = [POINTER(GemmDesc), POINTER(BnBwdStats), c_void_p]
     L.bb_conv3x3_dgrad_bn.argtypes = [c_int] * 6 + [c_void_p] * 4 + [POINTER(BnBwdStats), c_void_p]
     L.bb_batchnorm_bwd_strips.argtypes = [c_int, c_int, c_int] + [c_void_p] * 10
+    L.bb_batchnorm_bwd_strip_sums.argtypes = [c_int, c_int, c_int] + [c_void_p] * 8
     L.bb_mse_workspace.restype = c_int64
     L.bb_mse_fwd_bwd.argtypes = [c_int, c_int64, c_void_p, c_void_p, c_void_p, c_float, c_void_p, c_int,
                                  c_void_p, c_void_p]
@@ -612,6 +613,21 @@ def batchnorm_bwd(x, gamma, mean, rstd, dy, relu_out, dx, g_out, dgamma, dbeta, 
     check(lib().bb_batchnorm_bwd(dtype_code(x.dtype), rows, cols, _ptr(x), _ptr(gamma), _ptr(mean), _ptr(rstd),
                                  _ptr(dy), _ptr(relu_out), _ptr(dx), _ptr(g_out), _ptr(dgamma), _ptr(dbeta),
                                  _ptr(workspace), stream_ptr(stream)), "bb_batchnorm_bwd")
+
+
+def batchnorm_bwd_strip_sums(x, mean, rstd, dy, relu_out, g_out, strips, stream=None):
+    """The strip sums of ``batchnorm_bwd_strips`` by a pass of their own (bf16), in the order the GEMM epilogues add them
+    up: ``g_out`` (may be ``dy``) receives ``dy * (relu_out > 0)``; without a ReLU ``g`` is ``dy`` and ``g_out`` may be None."""
+    rows, cols = x.shape
+    _like("batchnorm_bwd_strip_sums", x, dy=dy, relu_out=relu_out, g_out=g_out)
+    _vector("batchnorm_bwd_strip_sums", cols, torch.float32, mean=mean, rstd=rstd)
+    if relu_out is not None and g_out is None:
+        raise HipKernelError("batchnorm_bwd_strip_sums: with relu_out the masked gradient needs g_out (may be dy)")
+    if strips.dtype != torch.float32 or not strips.is_contiguous() or strips.numel() < bn_bwd_strips_workspace(rows, cols):
+        raise HipKernelError("batchnorm_bwd_strip_sums: strips too small")
+    check(lib().bb_batchnorm_bwd_strip_sums(dtype_code(x.dtype), rows, cols, _ptr(x), _ptr(mean), _ptr(rstd), _ptr(dy),
+                                            _ptr(relu_out), _ptr(g_out), _ptr(strips), stream_ptr(stream)),
+          "bb_batchnorm_bwd_strip_sums")
 
 
 def batchnorm_bwd_strips(x, gamma, mean, rstd, g, strips, dx, dgamma, dbeta, stream=None):

@@ -966,26 +966,37 @@ class BottleNeck:
         d_y3, d_res = ctx.buf("d_y3", (R2, co)), ctx.buf("d_res", (R2, co))
         d_m0, d_m1 = ctx.buf("d_m0", (R2, cm)), ctx.buf("d_m1", (R2, cm))
 
-        def bn(idx, xk, mk, rk, dy, relu_out, dx, g_out):
-            name = self._BN_NAMES[idx]
-            hip.batchnorm_bwd(st[xk], w[f"{name}.weight"], st[mk], st[rk], dy, relu_out, dx, g_out,
-                              g[f"{name}.weight"], g[f"{name}.bias"], ws, stream=sm)
-
         def bn_strips(idx, xk, mk, rk, gk, strips, dx):
             name = self._BN_NAMES[idx]
             hip.batchnorm_bwd_strips(st[xk], w[f"{name}.weight"], st[mk], st[rk], gk, strips, dx,
                                      g[f"{name}.weight"], g[f"{name}.bias"], stream=sm)
+
+        def bn(idx, xk, mk, rk, dy, relu_out, dx, g_out, strips_name):
+            """BatchNorm backward with a reduction pass of its own.  bf16: the pass adds the sums up in the order of the
+            GEMM epilogues that leave them elsewhere, so a gradient gives the same bits whichever kernel made its
+            sums (a block at a stage or checkpoint-group boundary, a promoted stage, a shape the fused kernels do
+            not take); the masked gradient goes to ``g_out``, else in place into ``dy``."""
+            name = self._BN_NAMES[idx]
+            if ctx.dtype != torch.bfloat16:
+                hip.batchnorm_bwd(st[xk], w[f"{name}.weight"], st[mk], st[rk], dy, relu_out, dx, g_out,
+                                  g[f"{name}.weight"], g[f"{name}.bias"], ws, stream=sm)
+                return
+            strips = ctx.buf(strips_name, (hip.bn_bwd_strips_workspace(*st[xk].shape),))
+            masked = dy if relu_out is None else (g_out if g_out is not None else dy)
+            hip.batchnorm_bwd_strip_sums(st[xk], st[mk], st[rk], dy, relu_out, masked if relu_out is not None else None, strips,
+                                         stream=sm)
+            bn_strips(idx, xk, mk, rk, masked, strips, dx)
         # final ReLU + BN3; d_res keeps the masked gradient for the shortcut
         if ctx.grad_presummed:
             # the block behind this one has masked d_out and left the sums (grad_sink)
             d_res = d_out
             bn_strips(7, "y3", "mean3", "rstd3", d_out, ctx.buf("bn_strips_in", (hip.bn_bwd_strips_workspace(R2, co),)), d_y3)
         else:
-            bn(7, "y3", "mean3", "rstd3", d_out, st["out"], d_y3, d_res)
+            bn(7, "y3", "mean3", "rstd3", d_out, st["out"], d_y3, d_res, "bn_strips_in")
         d_ys = d_xs = xs = None
         if self.projection:
             d_ys, d_xs = ctx.buf("d_ys", (R2, co)), ctx.buf("d_xs", (R2, ci))
-            bn("shortcut", "ys", "mean_s", "rstd_s", d_res, None, d_ys, None)
+            bn("shortcut", "ys", "mean_s", "rstd_s", d_res, None, d_ys, None, "bn_strips_in")
             ctx.gemm(hip.NN, d_ys, w["shortcut.0.weight"], d_xs, stream=sm)
             xs = self._shortcut_input(st["x0"], ctx, R2)
         # The two inner BatchNorms receive their gradient from a convolution's input gradient: where the kernel can,
@@ -1001,7 +1012,7 @@ class BottleNeck:
             bn_strips(4, "y2", "mean2", "rstd2", d_m0, strips, d_m1)                       # d_y2
         else:
             ctx.gemm(hip.NN, d_y3, w["residual_function.6.weight"], d_m0, stream=sm)      # d_a2
-            bn(4, "y2", "mean2", "rstd2", d_m0, st["a2"], d_m1, None)                      # d_y2
+            bn(4, "y2", "mean2", "rstd2", d_m0, st["a2"], d_m1, None, "bn_strips")         # d_y2
         # weight gradient of the 3x3 convolution: patch matrix gathered inside the GEMM, else built again here
         # (cheaper than stashing it)
         wgrad_implicit = (self._implicit(ctx, hip.CONV_DGRAD) and cm % 128 == 0 and R % 32 == 0 and 32 // self.w + 1 <= self.h)
@@ -1017,7 +1028,7 @@ class BottleNeck:
             d_col = ctx.buf("d_col", (R2, 9 * cm))
             ctx.gemm(hip.NN, d_m1, w["conv2"], d_col, stream=sm)
             hip.patch3x3(d_col, d_a1, ctx.batch, self.h, self.w, cm, adjoint=True, stride=self.stride, stream=sm)
-            bn(1, "y1", "mean1", "rstd1", d_a1, st["a1"], d_m2, None)                      # d_y1
+            bn(1, "y1", "mean1", "rstd1", d_a1, st["a1"], d_m2, None, "bn_strips")         # d_y1
         if self.projection and self.stride > 1:
             ctx.gemm(hip.NN, d_m2, w["residual_function.0.weight"], d_x, stream=sm)
             hip.subsample(d_xs, d_x, ctx.batch, self.h, self.w, ci, self.stride, adjoint=True, stream=sm)

@@ -337,6 +337,12 @@ int bb_gemm_bn_bwd_supported(const bb_gemm_desc* desc);
 int bb_gemm_bn_bwd(const bb_gemm_desc* desc, const bb_bn_bwd_stats* bn, void* stream);
 int bb_conv3x3_dgrad_bn(int dtype, int n, int h, int w, int cin, int cout, const void* src, const void* weight,
                         void* dst, const void* relu_out, const bb_bn_bwd_stats* bn, void* stream);
+/* The same strip sums where no such kernel wrote the gradient (it arrived from another stage, or the shape is not
+ * one they take): one pass over x, dy and relu_out (NULL: no ReLU) that writes g = dy * (relu_out > 0) to g_out (may be
+ * dy itself; may be NULL without a ReLU) and the sums to strips, added up in the order of those epilogues: whichever
+ * way the sums were made, bb_batchnorm_bwd_strips gives the same bits.                                             */
+int bb_batchnorm_bwd_strip_sums(int dtype, int rows, int cols, const void* x, const float* mean, const float* rstd,
+                                const void* dy, const void* relu_out, void* g_out, float* strips, void* stream);
 int bb_batchnorm_bwd_strips(int dtype, int rows, int cols, const void* x, const void* gamma, const float* mean,
                             const float* rstd, const void* g, const float* strips, void* dx, float* dgamma,
                             float* dbeta, void* stream);

@@ -576,6 +576,18 @@ def test_bn_bwd_sums_from_the_input_gradient(hiplib, kind, n, h, w, cm, co, relu
     # and against the separate kernels: sums equal up to the fp32 order of addition, dx up to an ulp of bf16
     assert float((db1 - db0).abs().max() / scale_g) < 1e-5 and float((dg1 - dg0).abs().max() / scale_gx) < 1e-5
     assert float((dx1.float() - dx0.float()).abs().max() / dx0.float().abs().max()) < 2 ** -7
+    # The pass that makes the strip sums where no epilogue left them adds up in the epilogues' order: from the
+    # unmasked gradient of the plain kernel it gives the same strips, hence the same dx, dgamma and dbeta, bit for bit
+    # (masked gradient in place).
+    d_a2 = torch.empty_like(x)
+    plain(d_a2)
+    strips2 = torch.full_like(strips, float("nan"))
+    dx2, dg2, db2 = torch.full_like(x, 7.0), dg_init.clone(), db_init.clone()
+    hiplib.batchnorm_bwd_strip_sums(x, mean, rstd, d_a2, relu_out, d_a2 if relu else None, strips2)
+    hiplib.batchnorm_bwd_strips(x, gamma, mean, rstd, d_a2, strips2, dx2, dg2, db2)
+    torch.cuda.synchronize()
+    assert torch.equal(d_a2, g1) and torch.equal(strips2[:-8], strips[:-8])
+    assert torch.equal(dx2, dx1) and torch.equal(dg2, dg1) and torch.equal(db2, db1)
     # what does not fit is refused before anything is launched
     with pytest.raises(hiplib.HipKernelError):
         fused(g1, strips[: hiplib.bn_bwd_strips_workspace(R, cm) - 1])

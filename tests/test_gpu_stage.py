@@ -641,15 +641,19 @@ def test_activation_checkpointing_equals_full_stash(hiplib, interval, rc_stream)
         assert torch.equal(a.exp_avg, b.exp_avg) and torch.equal(a.exp_avg_sq, b.exp_avg_sq)
 
 
-@pytest.mark.parametrize("net", ["identity", "down-sampling"])
+@pytest.mark.parametrize("net", ["identity", "identity-wide", "down-sampling"])
 def test_activation_checkpointing_resnet_keeps_running_statistics(hiplib, net):
     """Bottleneck stage with checkpoint groups of one block: gradients, outputs and the BatchNorm running
     statistics (updated once per forward, not again by the recomputation) equal the full stash bit for bit; also
-    where the kept group inputs differ in rows and channels (blocks with a stride and a projection shortcut)."""
+    where the kept group inputs differ in rows and channels (blocks with a stride and a projection shortcut), and
+    ("wide") where the full stash takes the last BatchNorm's backward sums of the stage's first block from the
+    epilogue of the second block's last GEMM while a group of one block makes them in a pass of its own."""
     from bamboo_amd import BottleNeck
     cin, cmid, side, L, S, sid, mb, M = 64, 16, 6, 2, 4, 1, 4, 4
-    blocks = [(cin, cmid, 1)] * (L * S) if net == "identity" else DOWNSAMPLING_NET
-    if net != "identity":
+    if net == "identity-wide":
+        cin, cmid, mb = 512, 128, 8
+    blocks = [(cin, cmid, 1)] * (L * S) if net != "down-sampling" else DOWNSAMPLING_NET
+    if net == "down-sampling":
         side = 16
     out_shapes = {s_: (mb, side * side // 4 ** sum(st_ == 2 for _, _, st_ in blocks[:(s_ + 1) * L]), 4 * blocks[(s_ + 1) * L - 1][1])
                   for s_ in (sid, sid + 1)}
@@ -669,6 +673,9 @@ def test_activation_checkpointing_resnet_keeps_running_statistics(hiplib, net):
         torch.cuda.synchronize()
         runs.append(engine)
     a, b = runs
+    if net == "identity-wide":
+        sunk = lambda e: [any(k[0] == "sink" and v for k, v in layer._stats_ok.items()) for layer in e.module.func_buckets[sid]]
+        assert sunk(a) == [False, True] and sunk(b) == [False, False]
     for s_ in (sid, sid + 1):
         pa, pb = a.module.stage_params[s_], b.module.stage_params[s_]
         assert torch.equal(pa.master, pb.master) and torch.equal(pa.exp_avg_sq, pb.exp_avg_sq)
