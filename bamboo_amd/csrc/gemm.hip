@@ -216,11 +216,19 @@ template <bool TA, bool TB> static int dispatch_bf16(GemmArgs& g, int batches, h
     }
 }
 
+static int pick_f32_tile(int M, int N, int64_t batches) {
+    const int64_t t128 = (int64_t)((M + 127) / 128) * ((N + 127) / 128) * batches;
+    return t128 < 2 * 256 ? 64 : 128;
+}
 template <bool TA, bool TB> static int dispatch_f32(GemmArgs& g, int batches, hipStream_t st) {
-    g.tiles_m = (g.M + 127) / 128;
-    g.tiles_n = (g.N + 127) / 128;
+    // 64x64 tiles while 128x128 ones would leave most CUs with a single block (one wave per SIMD): shape only, and the
+    // same order of additions on both, so which one runs changes no bit
+    const int tile = pick_f32_tile(g.M, g.N, batches);
+    g.tiles_m = (g.M + tile - 1) / tile;
+    g.tiles_n = (g.N + tile - 1) / tile;
     dim3 grid(g.tiles_m * g.tiles_n, 1, batches);
-    hipLaunchKernelGGL((gemm_f32_kernel<TA, TB>), grid, dim3(256), 0, st, g);
+    if (tile == 64) hipLaunchKernelGGL((gemm_f32_kernel<TA, TB, 64>), grid, dim3(256), 0, st, g);
+    else hipLaunchKernelGGL((gemm_f32_kernel<TA, TB, 128>), grid, dim3(256), 0, st, g);
     BB_LAUNCH_CHECK();
     return BB_OK;
 }
@@ -236,7 +244,10 @@ extern "C" int bb_gemm_variant(const bb_gemm_desc* d, char* out, int out_len) {
                  dt != D_NONE ? kDmaTileNames[dt] : kBf16TileNames[pick_bf16_tile(d->M, d->N, batches)]);
     }
     else
-        snprintf(out, out_len, "f32_%s_128x128", layouts[d->layout]);
+    {
+        const int tile = pick_f32_tile(d->M, d->N, batches);
+        snprintf(out, out_len, "f32_%s_%dx%d", layouts[d->layout], tile, tile);
+    }
     return BB_OK;
 }
 

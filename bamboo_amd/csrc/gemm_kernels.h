@@ -1427,9 +1427,15 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_bf16_dma_grouped_kernel(cons
 // =========================================================================================
 // fp32 kernel: 128x128x16 tiles, 4 waves (2x2), LDS k-major with padded rows.
 // =========================================================================================
-template <bool TA, bool TB>
+// TILE = BM = BN: 128 (wave tile 64x64), or 64 (wave tile 32x32) for problems with so few 128x128 tiles that most CUs
+// would hold one block, i.e. one wave per SIMD with nobody to cover its waits for the next k-tile.  Every element adds
+// up its contraction in the same order on both.
+template <bool TA, bool TB, int TILE = 128>
 __global__ __launch_bounds__(256) void gemm_f32_kernel(const GemmArgs g) {
-    constexpr int BM = 128, BN = 128, BK = 16, LDS_LD = 132, NT = 256;
+    constexpr int BM = TILE, BN = TILE, BK = 16, LDS_LD = TILE + 4, NT = 256;
+    constexpr int WT = TILE / 2, TF = WT / 32;          // wave tile side, 32x32 accumulator tiles along it
+    constexpr int CH = TILE * BK / 4 / NT;              // 16-byte chunks of an operand tile per thread
+    constexpr int RQ = TILE / 4;                        // chunks along a row-contiguous (transposed) tile row
     __shared__ __attribute__((aligned(16))) float As[2][BK * LDS_LD];
     __shared__ __attribute__((aligned(16))) float Bs[2][BK * LDS_LD];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -1442,10 +1448,10 @@ __global__ __launch_bounds__(256) void gemm_f32_kernel(const GemmArgs g) {
     const float* B = (const float*)g.B + b1 * g.sB1 + b2 * g.sB2;
     const int64_t coff = b1 * g.sC1 + b2 * g.sC2;
 
-    f32x4 ra[2], rb[2];
-    auto gload = [&](const float* base, int64_t ld, int row0, int rows, int k0, bool tr, f32x4 (&r)[2]) {
+    f32x4 ra[CH], rb[CH];
+    auto gload = [&](const float* base, int64_t ld, int row0, int rows, int k0, bool tr, f32x4 (&r)[CH]) {
 #pragma unroll
-        for (int i = 0; i < 2; ++i) {
+        for (int i = 0; i < CH; ++i) {
             const int c = tid + i * NT;
             f32x4 v = {0.f, 0.f, 0.f, 0.f};
             if (!tr) {
@@ -1453,33 +1459,33 @@ __global__ __launch_bounds__(256) void gemm_f32_kernel(const GemmArgs g) {
                 if (row0 + row < rows && k0 + kq * 4 < g.K)
                     v = *(const f32x4*)(base + (int64_t)(row0 + row) * ld + k0 + kq * 4);
             } else {
-                const int k = c >> 5, rq = c & 31;
+                const int k = c / RQ, rq = c % RQ;
                 if (row0 + rq * 4 < rows && k0 + k < g.K)
                     v = *(const f32x4*)(base + (int64_t)(k0 + k) * ld + row0 + rq * 4);
             }
             r[i] = v;
         }
     };
-    auto sstore = [&](float* lds, bool tr, const f32x4 (&r)[2]) {
+    auto sstore = [&](float* lds, bool tr, const f32x4 (&r)[CH]) {
 #pragma unroll
-        for (int i = 0; i < 2; ++i) {
+        for (int i = 0; i < CH; ++i) {
             const int c = tid + i * NT;
             if (!tr) {
                 const int row = c >> 2, kq = c & 3;
 #pragma unroll
                 for (int e = 0; e < 4; ++e) lds[(kq * 4 + e) * LDS_LD + row] = r[i][e];
             } else {
-                const int k = c >> 5, rq = c & 31;
+                const int k = c / RQ, rq = c % RQ;
                 *(f32x4*)(lds + k * LDS_LD + rq * 4) = r[i];
             }
         }
     };
 
-    f32x16 acc[2][2];
+    f32x16 acc[TF][TF];
 #pragma unroll
-    for (int i = 0; i < 2; ++i)
+    for (int i = 0; i < TF; ++i)
 #pragma unroll
-        for (int j = 0; j < 2; ++j)
+        for (int j = 0; j < TF; ++j)
 #pragma unroll
             for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
 
@@ -1498,16 +1504,16 @@ __global__ __launch_bounds__(256) void gemm_f32_kernel(const GemmArgs g) {
         }
 #pragma unroll
         for (int ks = 0; ks < BK / 2; ++ks) {
-            float af[2], bfr[2];
+            float af[TF], bfr[TF];
             const int kk = ks * 2 + (lane >> 5);
 #pragma unroll
-            for (int i = 0; i < 2; ++i) af[i] = As[cur][kk * LDS_LD + wm * 64 + i * 32 + (lane & 31)];
+            for (int i = 0; i < TF; ++i) af[i] = As[cur][kk * LDS_LD + wm * WT + i * 32 + (lane & 31)];
 #pragma unroll
-            for (int j = 0; j < 2; ++j) bfr[j] = Bs[cur][kk * LDS_LD + wn * 64 + j * 32 + (lane & 31)];
+            for (int j = 0; j < TF; ++j) bfr[j] = Bs[cur][kk * LDS_LD + wn * WT + j * 32 + (lane & 31)];
 #pragma unroll
-            for (int i = 0; i < 2; ++i)
+            for (int i = 0; i < TF; ++i)
 #pragma unroll
-                for (int j = 0; j < 2; ++j)
+                for (int j = 0; j < TF; ++j)
                     acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(af[i], bfr[j], acc[i][j], 0, 0, 0);
         }
         if (more) {
@@ -1517,14 +1523,14 @@ __global__ __launch_bounds__(256) void gemm_f32_kernel(const GemmArgs g) {
         __syncthreads();
     }
 #pragma unroll
-    for (int i = 0; i < 2; ++i)
+    for (int i = 0; i < TF; ++i)
 #pragma unroll
-        for (int j = 0; j < 2; ++j) {
-            const int n = n0 + wn * 64 + j * 32 + (lane & 31);
+        for (int j = 0; j < TF; ++j) {
+            const int n = n0 + wn * WT + j * 32 + (lane & 31);
             if (n >= g.N) continue;
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
-                const int m = m0 + wm * 64 + i * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
+                const int m = m0 + wm * WT + i * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
                 if (m < g.M) epilogue_elem<float>(g, coff, coff, m, n, acc[i][j][r]);
             }
         }
