@@ -191,3 +191,40 @@ def test_wrappers_refuse_operands_that_do_not_fit_before_any_launch():
         hip.mse_fwd_bwd(x, x[:8], torch.zeros_like(x), 1.0, torch.zeros(1), False, torch.zeros(4096))
     with pytest.raises(hip.HipKernelError, match="cast"):
         hip.cast(x, torch.zeros(8, 32))
+
+
+def test_batchnorm_backward_sums_and_head_pairs_validate_on_the_host():
+    """The entry points of the BatchNorm backward sums and the fused attention's head widths: refused on the host,
+    before any HIP call, when the problem is not one the kernels take."""
+    from bamboo_amd import hip
+    L = hip.lib()
+    BF16, F32 = hip.BF16, hip.F32
+    one = ctypes.c_void_p(16)
+    assert L.bb_bn_bwd_strips_workspace(6272, 256) == 196 * 2 * 256 and L.bb_bn_bwd_strips_workspace(33, 8) == 2 * 2 * 8
+    # fp32 has no strip-sum kernels
+    assert L.bb_batchnorm_bwd_strip_sums(F32, 64, 64, one, one, one, one, None, None, one, None) == -1
+    assert b"bf16 only" in L.bb_last_error()
+    # a ReLU needs a place for the masked gradient
+    assert L.bb_batchnorm_bwd_strip_sums(BF16, 64, 64, one, one, one, one, one, None, one, None) == -1
+    assert b"masked gradient" in L.bb_last_error()
+    assert L.bb_batchnorm_bwd_strips(BF16, 64, 64, one, one, one, one, one, None, one, one, one, None) == -1
+    assert b"null pointer" in L.bb_last_error()
+    # the GEMM with the sums: an NN product whose C is contiguous, no bias, no accumulation
+    d = hip.GemmDesc()
+    d.layout, d.dtype, d.c_dtype, d.M, d.N, d.K = hip.NN, BF16, BF16, 6272, 256, 1024
+    d.A, d.B, d.C, d.lda, d.ldb, d.ldc, d.alpha = 16, 16, 16, 1024, 256, 256, 1.0
+    assert L.bb_gemm_bn_bwd_supported(ctypes.byref(d)) == 1
+    d.ldc = 512
+    assert L.bb_gemm_bn_bwd_supported(ctypes.byref(d)) == 0
+    d.ldc, d.layout = 256, hip.NT
+    assert L.bb_gemm_bn_bwd_supported(ctypes.byref(d)) == 0
+    d.layout, d.K = hip.NN, 96
+    assert L.bb_gemm_bn_bwd_supported(ctypes.byref(d)) == 0
+    assert L.bb_gemm_bn_bwd(ctypes.byref(d), None, None) == -1 and b"bb_gemm_bn_bwd: needs" in L.bb_last_error()
+    d.K = 1024
+    bn = hip.BnBwdStats(16, 16, 16, None)
+    assert L.bb_gemm_bn_bwd(ctypes.byref(d), ctypes.byref(bn), None) == -1 and b"null pointer in bb_bn_bwd_stats" in L.bb_last_error()
+    # attention: 64-wide heads, or an even number of 32-wide ones
+    args = lambda heads, dim: (BF16, 0, 1, heads, 64, dim, one, one, one, 3 * heads * dim, one, heads * dim, one, None, 0.0, 0, 0, None)
+    assert L.bb_attention_fwd(*args(3, 32)) == -1 and b"even number of heads" in L.bb_last_error()
+    assert L.bb_attention_fwd(*args(2, 128)) == -1 and b"head dimension" in L.bb_last_error()
