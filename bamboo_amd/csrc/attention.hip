@@ -1,4 +1,4 @@
-// Fused masked softmax-attention for gfx950, bf16, head dimension 64 or 32: forward and the two
+// Fused masked softmax-attention for gfx950, bf16, head dimension 64, 32 or 128: forward and the two
 // backward kernels (dK/dV and dQ).  No [batch, heads, seq, seq] tensor ever reaches HBM; the
 // forward keeps one fp32 log-sum-exp per (batch, head, query) for the backward.
 //
@@ -183,12 +183,14 @@ static unsigned attn_grid(int seq, int nbh) { return (unsigned)(8 * ((nbh + 7) /
 // =========================================================================================
 // forward: block = 128 queries (4 waves x 32), loop over 64-key tiles
 // =========================================================================================
-// HP: heads per block (1: 64-wide heads, 2: a pair of 32-wide heads); KS k-steps of a head's scores, DT 32-wide output
-// tiles of a head
-template <bool DROP, int HP>
+// HP: heads per block (1: one head, 2: a pair of 32-wide heads); NPAN: 64-wide column panels of a head (1; 2 for
+// 128-wide heads, HP = 1: a tile in LDS is then two [64][64] panels behind each other, each in the format above);
+// KS k-steps of a head's scores, DT 32-wide output tiles of a head
+template <bool DROP, int HP, int NPAN = 1>
 __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const AttnArgs a) {
-    constexpr int KS = 4 / HP, DT = 2 / HP;
-    __shared__ __attribute__((aligned(16))) unsigned char smem[2 * 2 * 8192];  // 2 stages x (K, V)
+    static_assert(HP == 1 || NPAN == 1, "pairs of heads are 32 wide");
+    constexpr int KS = 4 * NPAN / HP, DT = 2 * NPAN / HP, TILE = NPAN * 8192;
+    __shared__ __attribute__((aligned(16))) unsigned char smem[2 * 2 * TILE];  // 2 stages x (K, V)
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int groups = a.heads / HP;
     const BlockMap bm = map_block(a.batch * groups);
@@ -196,9 +198,9 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const AttnArgs a) {
     const int qb = (a.seq + 127) / 128 - 1 - bm.rank;  // long (late) query blocks first
     const int b = bm.bh / groups, hg = bm.bh % groups, head0 = hg * HP;
     const int64_t row_base = (int64_t)b * a.seq;
-    const bf16* Q = a.q + row_base * a.ld_qkv + hg * 64;
-    const bf16* K = a.k + row_base * a.ld_qkv + hg * 64;
-    const bf16* V = a.v + row_base * a.ld_qkv + hg * 64;
+    const bf16* Q = a.q + row_base * a.ld_qkv + hg * (64 * NPAN);
+    const bf16* K = a.k + row_base * a.ld_qkv + hg * (64 * NPAN);
+    const bf16* V = a.v + row_base * a.ld_qkv + hg * (64 * NPAN);
     const int q0 = qb * 128 + wave * 32;
     const int myq = q0 + (lane & 31);
     const int last = a.seq - 1;
@@ -211,15 +213,15 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const AttnArgs a) {
     const int my_limit = kv_limit(a, b, myq);
     const int wave_min_limit = kv_limit(a, b, q0);  // limits grow with the query index
 
-    bf16x8 qf[4];
+    bf16x8 qf[4 * NPAN];
     {
         const bf16* qp = Q + (int64_t)min(myq, last) * a.ld_qkv + (lane >> 5) * 8;
 #pragma unroll
-        for (int ks = 0; ks < 4; ++ks) qf[ks] = *(const bf16x8*)(qp + ks * 16);
+        for (int ks = 0; ks < 4 * NPAN; ++ks) qf[ks] = *(const bf16x8*)(qp + ks * 16);
     }
-    f32x16 o[2];
+    f32x16 o[2 * NPAN];
 #pragma unroll
-    for (int t = 0; t < 2; ++t)
+    for (int t = 0; t < 2 * NPAN; ++t)
 #pragma unroll
         for (int r = 0; r < 16; ++r) o[t][r] = 0.f;
     float m[HP], lsum[HP];
@@ -231,10 +233,13 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const AttnArgs a) {
 
     const LaneOff lo = lane_off(a.ld_qkv, wave, lane);
     auto issue = [&](int t) {
-        unsigned char* st = smem + (t & 1) * 16384;
+        unsigned char* st = smem + (t & 1) * (2 * TILE);
         const int kv0 = t * 64;
-        dma_tile64(K, a.ld_qkv, kv0, last, st, wave, lane, lo);
-        dma_tile64(V, a.ld_qkv, kv0, last, st + 8192, wave, lane, lo);
+#pragma unroll
+        for (int p = 0; p < NPAN; ++p) {
+            dma_tile64(K + p * 64, a.ld_qkv, kv0, last, st + p * 8192, wave, lane, lo);
+            dma_tile64(V + p * 64, a.ld_qkv, kv0, last, st + TILE + p * 8192, wave, lane, lo);
+        }
     };
 
     if (ntiles > 0) issue(0);
@@ -242,13 +247,13 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const AttnArgs a) {
         asm volatile("" ::: "memory");
         if (t + 1 < ntiles) {
             issue(t + 1);
-            wait_vm<4>();
+            wait_vm<4 * NPAN>();
         } else {
             wait_vm<0>();
         }
         block_sync();
-        const unsigned char* kt = smem + (t & 1) * 16384;
-        const unsigned char* vt = kt + 8192;
+        const unsigned char* kt = smem + (t & 1) * (2 * TILE);
+        const unsigned char* vt = kt + TILE;
         const int kv0 = t * 64;
         // waves whose queries all precede this tile have nothing to add (causal)
         const bool active = !(a.mask == BB_MASK_CAUSAL && kv0 > q0 + 31);
@@ -261,8 +266,10 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const AttnArgs a) {
 #pragma unroll
                 for (int r = 0; r < 16; ++r) s[u][r] = 0.f;
 #pragma unroll
-                for (int k = 0; k < KS; ++k)
-                    s[u] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frag_kc(kt, u * 32, hh * KS + k, lane), qf[hh * KS + k], s[u], 0, 0, 0);
+                for (int k = 0; k < KS; ++k) {
+                    const int ks = hh * KS + k;   // k-step ks: panel ks / 4, step ks % 4 inside it
+                    s[u] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frag_kc(kt + (ks >> 2) * 8192, u * 32, ks & 3, lane), qf[ks], s[u], 0, 0, 0);
+                }
             }
             // running max on the raw scores (the scale is positive), masking only on tiles that
             // reach past the first key some query of this wave may not see
@@ -312,9 +319,10 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const AttnArgs a) {
             for (int kk = 0; kk < 4; ++kk) {
                 const bf16x8 pf = pack_acc(s[kk >> 1], kk & 1);
 #pragma unroll
-                for (int d = 0; d < DT; ++d)
-                    o[hh * DT + d] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frag_tr(vt, kk * 16, (hh * DT + d) * 32, lane), pf,
-                                                                             o[hh * DT + d], 0, 0, 0);
+                for (int d = 0; d < DT; ++d) {
+                    const int dt = hh * DT + d;   // output tile dt: panel dt / 2, columns (dt % 2) * 32 inside it
+                    o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frag_tr(vt + (dt >> 1) * 8192, kk * 16, (dt & 1) * 32, lane), pf, o[dt], 0, 0, 0);
+                }
             }
           }
         }
@@ -327,9 +335,9 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const AttnArgs a) {
         inv[hh] = lsum[hh] > 0.f ? 1.0f / lsum[hh] : 0.f;
     }
     if (myq < a.seq) {
-        bf16* op = a.out + (row_base + myq) * a.ld_o + hg * 64;
+        bf16* op = a.out + (row_base + myq) * a.ld_o + hg * (64 * NPAN);
 #pragma unroll
-        for (int dt = 0; dt < 2; ++dt)
+        for (int dt = 0; dt < 2 * NPAN; ++dt)
 #pragma unroll
             for (int g4 = 0; g4 < 4; ++g4) {
                 const int d = dt * 32 + 8 * g4 + 4 * (lane >> 5);
@@ -347,23 +355,31 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const AttnArgs a) {
 // =========================================================================================
 // backward dK, dV: block = 128 keys (4 waves x 32), loop over 64-query tiles
 // =========================================================================================
-template <bool DROP, int HP>
+// NPAN = 2 (128-wide heads): a block accumulates dK and dV for ONE 64-wide half `fh` of the head's columns (the grid
+// has two blocks per head and key block); scores and dP take the full 128 columns in both, i.e. are made twice -- a wave
+// that held all four output tiles of dK and of dV next to K, V, S and dP would need more registers than it has.
+template <bool DROP, int HP, int NPAN = 1>
 __global__ __launch_bounds__(256, 2) void attn_bwd_dkv_kernel(const AttnArgs a) {
-    constexpr int KS = 4 / HP, DT = 2 / HP;
-    // 2 stages x (Q tile 8 KiB, dO tile 8 KiB, lse 256 B per head, delta 256 B per head)
-    constexpr int STAGE = 2 * 8192 + 512 * HP;
-    __shared__ __attribute__((aligned(16))) unsigned char smem[2 * STAGE];
+    static_assert(HP == 1 || NPAN == 1, "pairs of heads are 32 wide");
+    constexpr int KS = 4 * NPAN / HP, DT = 2 / HP, TILE = NPAN * 8192;
+    // 2 stages x (Q tile, dO tile: 8 KiB per panel, lse 256 B per head, delta 256 B per head); two panels: more than the
+    // 64 KiB a kernel may declare, so the launch brings it
+    constexpr int STAGE = 2 * TILE + 512 * HP;
+    __shared__ __attribute__((aligned(16))) unsigned char smem_fixed[NPAN == 1 ? 2 * STAGE : 16];
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem_launch[];
+    unsigned char* smem = NPAN == 1 ? smem_fixed : smem_launch;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int groups = a.heads / HP;
-    const BlockMap bm = map_block(a.batch * groups);
-    if (bm.bh >= a.batch * groups) return;
+    const BlockMap bm = map_block(a.batch * groups * NPAN);
+    if (bm.bh >= a.batch * groups * NPAN) return;
     const int kb = bm.rank;  // early key blocks are seen by the most queries
-    const int b = bm.bh / groups, hg = bm.bh % groups, head0 = hg * HP;
+    const int fh = bm.bh % NPAN, bg = bm.bh / NPAN;
+    const int b = bg / groups, hg = bg % groups, head0 = hg * HP;
     const int64_t row_base = (int64_t)b * a.seq;
-    const bf16* Q = a.q + row_base * a.ld_qkv + hg * 64;
-    const bf16* K = a.k + row_base * a.ld_qkv + hg * 64;
-    const bf16* V = a.v + row_base * a.ld_qkv + hg * 64;
-    const bf16* DO = a.d_o + row_base * a.ld_o + hg * 64;
+    const bf16* Q = a.q + row_base * a.ld_qkv + hg * (64 * NPAN);
+    const bf16* K = a.k + row_base * a.ld_qkv + hg * (64 * NPAN);
+    const bf16* V = a.v + row_base * a.ld_qkv + hg * (64 * NPAN);
+    const bf16* DO = a.d_o + row_base * a.ld_o + hg * (64 * NPAN);
     // the statistics of the block's heads lie behind each other: [batch, heads, seq]
     const float* LSE = a.lse + ((int64_t)b * a.heads + head0) * a.seq;
     const float* DELTA = a.delta + ((int64_t)b * a.heads + head0) * a.seq;
@@ -377,11 +393,11 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dkv_kernel(const AttnArgs a) 
     // a block whose 128 keys are all padding has nothing to accumulate: it only stores its zeros
     const int ntiles = kb * 128 >= pad_limit ? 0 : (a.seq + 63) / 64;
 
-    bf16x8 kf[4], vf[4];
+    bf16x8 kf[4 * NPAN], vf[4 * NPAN];
     {
         const int64_t off = (int64_t)min(mykv, last) * a.ld_qkv + (lane >> 5) * 8;
 #pragma unroll
-        for (int ks = 0; ks < 4; ++ks) {
+        for (int ks = 0; ks < 4 * NPAN; ++ks) {
             kf[ks] = *(const bf16x8*)(K + off + ks * 16);
             vf[ks] = *(const bf16x8*)(V + off + ks * 16);
         }
@@ -396,15 +412,18 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dkv_kernel(const AttnArgs a) 
     auto issue = [&](int t, int slot) {
         unsigned char* st = smem + slot * STAGE;
         const int qs = t * 64;
-        dma_tile64(Q, a.ld_qkv, qs, last, st, wave, lane, lo);
-        dma_tile64(DO, a.ld_o, qs, last, st + 8192, wave, lane, lo_o);
+#pragma unroll
+        for (int p = 0; p < NPAN; ++p) {
+            dma_tile64(Q + p * 64, a.ld_qkv, qs, last, st + p * 8192, wave, lane, lo);
+            dma_tile64(DO + p * 64, a.ld_o, qs, last, st + TILE + p * 8192, wave, lane, lo_o);
+        }
         // one extra load for waves 0 and 1 (one head), for all four waves (a pair): lse of the heads, then delta
         if constexpr (HP == 1) {
-            if (wave == 0) dma_f32x64(LSE, qs, last, st + 16384, lane);
-            if (wave == 1) dma_f32x64(DELTA, qs, last, st + 16384 + 256, lane);
+            if (wave == 0) dma_f32x64(LSE, qs, last, st + 2 * TILE, lane);
+            if (wave == 1) dma_f32x64(DELTA, qs, last, st + 2 * TILE + 256, lane);
         } else {
             const float* src = (wave >> 1 ? DELTA : LSE) + (int64_t)(wave & 1) * a.seq;
-            dma_f32x64(src, qs, last, st + 16384 + (wave >> 1) * 512 + (wave & 1) * 256, lane);
+            dma_f32x64(src, qs, last, st + 2 * TILE + (wave >> 1) * 512 + (wave & 1) * 256, lane);
         }
     };
 
@@ -414,15 +433,15 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dkv_kernel(const AttnArgs a) 
         asm volatile("" ::: "memory");
         if (t + 1 < ntiles) {
             issue(t + 1, slot ^ 1);
-            // the waves with an extra load wait for <= 5 newer loads, the others for <= 4
-            if (HP == 2 || wave < 2) wait_vm<5>(); else wait_vm<4>();
+            // the waves with an extra load wait for one more newer load than the others
+            if (HP == 2 || wave < 2) wait_vm<4 * NPAN + 1>(); else wait_vm<4 * NPAN>();
         } else {
             wait_vm<0>();
         }
         block_sync();
         const unsigned char* qt = smem + slot * STAGE;
-        const unsigned char* dot = qt + 8192;
-        const float* lse_all = (const float*)(qt + 16384);
+        const unsigned char* dot = qt + TILE;
+        const float* lse_all = (const float*)(qt + 2 * TILE);
         const float* del_all = lse_all + 64 * HP;
 #pragma unroll
         for (int u = 0; u < 2; ++u) {
@@ -441,8 +460,8 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dkv_kernel(const AttnArgs a) 
 #pragma unroll
             for (int k = 0; k < KS; ++k) {
                 const int ks = hh * KS + k;
-                s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frag_kc(qt, u * 32, ks, lane), kf[ks], s, 0, 0, 0);
-                dp = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frag_kc(dot, u * 32, ks, lane), vf[ks], dp, 0, 0, 0);
+                s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frag_kc(qt + (ks >> 2) * 8192, u * 32, ks & 3, lane), kf[ks], s, 0, 0, 0);
+                dp = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frag_kc(dot + (ks >> 2) * 8192, u * 32, ks & 3, lane), vf[ks], dp, 0, 0, 0);
             }
             // P = exp2(S * c - lse[q]); dS = P * (dP - delta[q]); rows q = acc_row(r), column kv = lane.
             // Only sub-tiles on the causal diagonal or past the last query mask per element; keys
@@ -512,8 +531,8 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dkv_kernel(const AttnArgs a) 
 #pragma unroll
                 for (int d = 0; d < DT; ++d) {
                     const int dt = hh * DT + d;
-                    dv[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frag_tr(dot, u * 32 + kk * 16, dt * 32, lane), pf, dv[dt], 0, 0, 0);
-                    dk[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frag_tr(qt, u * 32 + kk * 16, dt * 32, lane), dsf, dk[dt], 0, 0, 0);
+                    dv[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frag_tr(dot + fh * 8192, u * 32 + kk * 16, dt * 32, lane), pf, dv[dt], 0, 0, 0);
+                    dk[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frag_tr(qt + fh * 8192, u * 32 + kk * 16, dt * 32, lane), dsf, dk[dt], 0, 0, 0);
                 }
             }
           }
@@ -527,8 +546,8 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dkv_kernel(const AttnArgs a) 
             for (int r = 0; r < 16; ++r) dk[t][r] = dv[t][r] = 0.f;
     }
     if (mykv < a.seq) {
-        bf16* dkp = a.dk + (row_base + mykv) * a.ld_dqkv + hg * 64;
-        bf16* dvp = a.dv + (row_base + mykv) * a.ld_dqkv + hg * 64;
+        bf16* dkp = a.dk + (row_base + mykv) * a.ld_dqkv + hg * (64 * NPAN) + fh * 64;
+        bf16* dvp = a.dv + (row_base + mykv) * a.ld_dqkv + hg * (64 * NPAN) + fh * 64;
 #pragma unroll
         for (int dt = 0; dt < 2; ++dt)
 #pragma unroll
@@ -546,10 +565,11 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dkv_kernel(const AttnArgs a) 
 // =========================================================================================
 // backward dQ: block = 128 queries (4 waves x 32), loop over 64-key tiles
 // =========================================================================================
-template <bool DROP, int HP>
+template <bool DROP, int HP, int NPAN = 1>
 __global__ __launch_bounds__(256, 2) void attn_bwd_dq_kernel(const AttnArgs a) {
-    constexpr int KS = 4 / HP, DT = 2 / HP;
-    __shared__ __attribute__((aligned(16))) unsigned char smem[2 * 2 * 8192];
+    static_assert(HP == 1 || NPAN == 1, "pairs of heads are 32 wide");
+    constexpr int KS = 4 * NPAN / HP, DT = 2 * NPAN / HP, TILE = NPAN * 8192;
+    __shared__ __attribute__((aligned(16))) unsigned char smem[2 * 2 * TILE];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int groups = a.heads / HP;
     const BlockMap bm = map_block(a.batch * groups);
@@ -557,10 +577,10 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dq_kernel(const AttnArgs a) {
     const int qb = (a.seq + 127) / 128 - 1 - bm.rank;
     const int b = bm.bh / groups, hg = bm.bh % groups, head0 = hg * HP;
     const int64_t row_base = (int64_t)b * a.seq;
-    const bf16* Q = a.q + row_base * a.ld_qkv + hg * 64;
-    const bf16* K = a.k + row_base * a.ld_qkv + hg * 64;
-    const bf16* V = a.v + row_base * a.ld_qkv + hg * 64;
-    const bf16* DO = a.d_o + row_base * a.ld_o + hg * 64;
+    const bf16* Q = a.q + row_base * a.ld_qkv + hg * (64 * NPAN);
+    const bf16* K = a.k + row_base * a.ld_qkv + hg * (64 * NPAN);
+    const bf16* V = a.v + row_base * a.ld_qkv + hg * (64 * NPAN);
+    const bf16* DO = a.d_o + row_base * a.ld_o + hg * (64 * NPAN);
     const int q0 = qb * 128 + wave * 32;
     const int myq = q0 + (lane & 31);
     const int last = a.seq - 1;
@@ -572,11 +592,11 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dq_kernel(const AttnArgs a) {
     const int my_limit = kv_limit(a, b, myq);
     const int wave_min_limit = kv_limit(a, b, q0);  // limits grow with the query index
 
-    bf16x8 qf[4], dof[4];
+    bf16x8 qf[4 * NPAN], dof[4 * NPAN];
     {
         const int64_t r = min(myq, last);
 #pragma unroll
-        for (int ks = 0; ks < 4; ++ks) {
+        for (int ks = 0; ks < 4 * NPAN; ++ks) {
             qf[ks] = *(const bf16x8*)(Q + r * a.ld_qkv + (lane >> 5) * 8 + ks * 16);
             dof[ks] = *(const bf16x8*)(DO + r * a.ld_o + (lane >> 5) * 8 + ks * 16);
         }
@@ -586,7 +606,7 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dq_kernel(const AttnArgs a) {
     // dK / dV kernel, which runs after this one.
     float my_lse[HP], my_delta[HP];
     {
-        const bf16* O = a.o + row_base * a.ld_o + hg * 64;
+        const bf16* O = a.o + row_base * a.ld_o + hg * (64 * NPAN);
         const int64_t r = min(myq, last);
 #pragma unroll
         for (int hh = 0; hh < HP; ++hh) {
@@ -605,31 +625,34 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dq_kernel(const AttnArgs a) {
             my_delta[hh] = dl;
         }
     }
-    f32x16 dq[2];
+    f32x16 dq[2 * NPAN];
 #pragma unroll
-    for (int t = 0; t < 2; ++t)
+    for (int t = 0; t < 2 * NPAN; ++t)
 #pragma unroll
         for (int r = 0; r < 16; ++r) dq[t][r] = 0.f;
 
     const LaneOff lo = lane_off(a.ld_qkv, wave, lane);
     auto issue = [&](int t) {
-        unsigned char* st = smem + (t & 1) * 16384;
+        unsigned char* st = smem + (t & 1) * (2 * TILE);
         const int kv0 = t * 64;
-        dma_tile64(K, a.ld_qkv, kv0, last, st, wave, lane, lo);
-        dma_tile64(V, a.ld_qkv, kv0, last, st + 8192, wave, lane, lo);
+#pragma unroll
+        for (int p = 0; p < NPAN; ++p) {
+            dma_tile64(K + p * 64, a.ld_qkv, kv0, last, st + p * 8192, wave, lane, lo);
+            dma_tile64(V + p * 64, a.ld_qkv, kv0, last, st + TILE + p * 8192, wave, lane, lo);
+        }
     };
     if (ntiles > 0) issue(0);
     for (int t = 0; t < ntiles; ++t) {
         asm volatile("" ::: "memory");
         if (t + 1 < ntiles) {
             issue(t + 1);
-            wait_vm<4>();
+            wait_vm<4 * NPAN>();
         } else {
             wait_vm<0>();
         }
         block_sync();
-        const unsigned char* kt = smem + (t & 1) * 16384;
-        const unsigned char* vt = kt + 8192;
+        const unsigned char* kt = smem + (t & 1) * (2 * TILE);
+        const unsigned char* vt = kt + TILE;
         const int kv0 = t * 64;
         const bool active = !(a.mask == BB_MASK_CAUSAL && kv0 > q0 + 31);
         if (active) {
@@ -644,8 +667,8 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dq_kernel(const AttnArgs a) {
 #pragma unroll
                 for (int k = 0; k < KS; ++k) {
                     const int ks = hh * KS + k;
-                    s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frag_kc(kt, u * 32, ks, lane), qf[ks], s, 0, 0, 0);
-                    dp = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frag_kc(vt, u * 32, ks, lane), dof[ks], dp, 0, 0, 0);
+                    s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frag_kc(kt + (ks >> 2) * 8192, u * 32, ks & 3, lane), qf[ks], s, 0, 0, 0);
+                    dp = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frag_kc(vt + (ks >> 2) * 8192, u * 32, ks & 3, lane), dof[ks], dp, 0, 0, 0);
                 }
 #pragma unroll
                 for (int r = 0; r < 16; ++r) s[r] = __builtin_amdgcn_exp2f(fmaf(s[r], a.scale_log2, -my_lse[hh]));
@@ -669,7 +692,7 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dq_kernel(const AttnArgs a) {
 #pragma unroll
                     for (int d = 0; d < DT; ++d) {
                         const int dt = hh * DT + d;
-                        dq[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frag_tr(kt, u * 32 + kk * 16, dt * 32, lane), dsf, dq[dt], 0, 0, 0);
+                        dq[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frag_tr(kt + (dt >> 1) * 8192, u * 32 + kk * 16, (dt & 1) * 32, lane), dsf, dq[dt], 0, 0, 0);
                     }
                 }
               }
@@ -678,9 +701,9 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dq_kernel(const AttnArgs a) {
         block_sync();
     }
     if (myq < a.seq) {
-        bf16* dqp = a.dq + (row_base + myq) * a.ld_dqkv + hg * 64;
+        bf16* dqp = a.dq + (row_base + myq) * a.ld_dqkv + hg * (64 * NPAN);
 #pragma unroll
-        for (int dt = 0; dt < 2; ++dt)
+        for (int dt = 0; dt < 2 * NPAN; ++dt)
 #pragma unroll
             for (int g4 = 0; g4 < 4; ++g4) {
                 const int d = dt * 32 + 8 * g4 + 4 * (lane >> 5);
@@ -697,14 +720,14 @@ __global__ __launch_bounds__(256, 2) void attn_bwd_dq_kernel(const AttnArgs a) {
 static int check_attn(const char* name, int dtype, int mask, int batch, int heads, int seq, int head_dim, int64_t ld_qkv,
                       int64_t ld_o, const int32_t* key_len) {
     BB_REQUIRE(dtype == BB_BF16, "%s: the fused attention kernels are bf16 only (got dtype %d)", name, dtype);
-    BB_REQUIRE(head_dim == 64 || (head_dim == 32 && heads % 2 == 0),
-               "%s: head dimension must be 64, or 32 with an even number of heads (got %d, %d heads)", name, head_dim, heads);
+    BB_REQUIRE(head_dim == 64 || head_dim == 128 || (head_dim == 32 && heads % 2 == 0),
+               "%s: head dimension must be 64, 128, or 32 with an even number of heads (got %d, %d heads)", name, head_dim, heads);
     BB_REQUIRE(mask >= BB_MASK_NONE && mask <= BB_MASK_KEY_PADDING, "%s: bad mask %d", name, mask);
     BB_REQUIRE(mask != BB_MASK_KEY_PADDING || key_len, "%s: key_padding mask needs key_len", name);
     BB_REQUIRE(batch >= 0 && heads > 0 && seq >= 0, "%s: bad shape", name);
     BB_REQUIRE(ld_qkv % 8 == 0 && ld_o % 8 == 0 && ld_qkv >= heads * head_dim && ld_o >= heads * head_dim, "%s: bad leading dimension", name);
     BB_REQUIRE(ld_qkv < (1 << 24) && ld_o < (1 << 24), "%s: leading dimension too large", name);
-    BB_REQUIRE(((int64_t)batch * heads + 8) * ((seq + 127) / 128) < (1ll << 31), "%s: batch * heads * seq exceeds the grid limit", name);
+    BB_REQUIRE(((int64_t)batch * heads * 2 + 8) * ((seq + 127) / 128) < (1ll << 31), "%s: batch * heads * seq exceeds the grid limit", name);
     return BB_OK;
 }
 
@@ -726,10 +749,13 @@ extern "C" int bb_attention_fwd(int dtype, int mask, int batch, int heads, int s
     a.scale = 1.0f / sqrtf((float)head_dim);
     a.scale_log2 = a.scale * 1.4426950408889634f;
     // dropout is a kernel of its own: its keep decisions cost registers that decide how many blocks a CU holds
-    const int hp = 64 / head_dim;   // heads per block
+    const int hp = head_dim == 32 ? 2 : 1;   // heads per block
     const dim3 grid(attn_grid(seq, batch * (heads / hp)));
     hipStream_t st = (hipStream_t)stream;
-    if (hp == 1) {
+    if (head_dim == 128) {
+        if (a.drop.thresh) hipLaunchKernelGGL((attn_fwd_kernel<true, 1, 2>), grid, dim3(256), 0, st, a);
+        else hipLaunchKernelGGL((attn_fwd_kernel<false, 1, 2>), grid, dim3(256), 0, st, a);
+    } else if (hp == 1) {
         if (a.drop.thresh) hipLaunchKernelGGL((attn_fwd_kernel<true, 1>), grid, dim3(256), 0, st, a);
         else hipLaunchKernelGGL((attn_fwd_kernel<false, 1>), grid, dim3(256), 0, st, a);
     } else {
@@ -763,9 +789,22 @@ extern "C" int bb_attention_bwd(int dtype, int mask, int batch, int heads, int s
     a.scale_log2 = a.scale * 1.4426950408889634f;
     hipStream_t st = (hipStream_t)stream;
     // the dQ kernel first: it also leaves delta = rowsum(dO o O) of its queries for the dK / dV kernel
-    const int hp = 64 / head_dim;   // heads per block
+    const int hp = head_dim == 32 ? 2 : 1;   // heads per block
     dim3 grid(attn_grid(seq, batch * (heads / hp)));
-    if (hp == 1) {
+    if (head_dim == 128) {
+        // two dK / dV blocks per head and key block (one per 64-wide half of the columns), their LDS from the launch
+        constexpr int smem = 2 * (2 * 2 * 8192 + 512);
+        const dim3 grid2(attn_grid(seq, batch * heads * 2));
+        if (a.drop.thresh) {
+            BB_HIP_CHECK(bb_allow_dynamic_lds((const void*)attn_bwd_dkv_kernel<true, 1, 2>, smem));
+            hipLaunchKernelGGL((attn_bwd_dq_kernel<true, 1, 2>), grid, dim3(256), 0, st, a);
+            hipLaunchKernelGGL((attn_bwd_dkv_kernel<true, 1, 2>), grid2, dim3(256), smem, st, a);
+        } else {
+            BB_HIP_CHECK(bb_allow_dynamic_lds((const void*)attn_bwd_dkv_kernel<false, 1, 2>, smem));
+            hipLaunchKernelGGL((attn_bwd_dq_kernel<false, 1, 2>), grid, dim3(256), 0, st, a);
+            hipLaunchKernelGGL((attn_bwd_dkv_kernel<false, 1, 2>), grid2, dim3(256), smem, st, a);
+        }
+    } else if (hp == 1) {
         if (a.drop.thresh) {
             hipLaunchKernelGGL((attn_bwd_dq_kernel<true, 1>), grid, dim3(256), 0, st, a);
             hipLaunchKernelGGL((attn_bwd_dkv_kernel<true, 1>), grid, dim3(256), 0, st, a);

@@ -436,7 +436,7 @@ def _drop_args(dropout):
     return float(dropout[0]), int(dropout[1][0]), int(dropout[1][1])
 
 
-FUSED_HEAD_DIMS = (64, 32)   # the fused attention kernels: 64-wide heads, or pairs of 32-wide heads
+FUSED_HEAD_DIMS = (64, 32, 128)   # the fused attention kernels: 64- and 128-wide heads, or pairs of 32-wide heads
 
 
 def _check_attention(what, qkv, batch, heads, seq, key_len, lse, out=None, d_out=None, delta=None, d_qkv=None):
@@ -444,7 +444,7 @@ def _check_attention(what, qkv, batch, heads, seq, key_len, lse, out=None, d_out
     inner stride), lse / delta: fp32 with batch*heads*seq contiguous elements, key_len: int32 [batch]."""
     if qkv.dim() != 2 or qkv.shape[1] % (3 * heads) != 0 or qkv.shape[1] // (3 * heads) not in FUSED_HEAD_DIMS or \
             (qkv.shape[1] // (3 * heads) == 32 and heads % 2 != 0):
-        raise HipKernelError(f"{what}: qkv must be [rows, 3 * heads * d] with d = 64, or d = 32 and an even number of heads; "
+        raise HipKernelError(f"{what}: qkv must be [rows, 3 * heads * d] with d = 64 or 128, or d = 32 and an even number of heads; "
                              f"got {tuple(qkv.shape)} for {heads} heads")
     rows, h = batch * seq, qkv.shape[1] // 3
     for name, t, width in (("qkv", qkv, 3 * h), ("d_qkv", d_qkv, 3 * h), ("out", out, h), ("d_out", d_out, h)):
@@ -459,7 +459,7 @@ def _check_attention(what, qkv, batch, heads, seq, key_len, lse, out=None, d_out
 
 def attention_fwd(qkv, out, lse, batch, heads, seq, mask, key_len=None, stream=None, dropout=None):
     """qkv: [batch*seq, 3*heads*d] (Q | K | V thirds), out: [batch*seq, heads*d], lse: fp32 [batch, heads, seq]; head
-    dimension d = 64, or 32 with an even number of heads.
+    dimension d = 64 or 128, or 32 with an even number of heads.
     ``dropout=(p, (k0, k1))``: dropout on the probabilities with the decisions of that key."""
     _check_attention("attention_fwd", qkv, batch, heads, seq, key_len, lse, out=out)
     h = qkv.shape[1] // 3

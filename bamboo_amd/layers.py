@@ -188,12 +188,12 @@ class TransformerLayer:
         return self.hidden
 
     def fused_attention(self, ctx):
-        """bf16 with 64-wide heads, or with an even number of 32-wide heads (the reference's GPT-2 script defaults to
-        512 / 16 = 32, gpt2.py:212-214: the kernels then take the heads in pairs), runs the fused attention kernels
-        (no score matrix in HBM).  Everything else -- fp32, the correctness configuration, and bf16 with another head
-        width -- materialises the probabilities like the reference does: batched head products and the masked softmax
-        kernels."""
-        return ctx.dtype == torch.bfloat16 and (self.head_dim == 64 or (self.head_dim == 32 and self.heads % 2 == 0))
+        """bf16 with 64- or 128-wide heads, or with an even number of 32-wide heads (the reference's GPT-2 script
+        defaults to 512 / 16 = 32, gpt2.py:212-214: the kernels then take the heads in pairs), runs the fused attention
+        kernels (no score matrix in HBM).  Everything else -- fp32, the correctness configuration, and bf16 with another
+        head width -- materialises the probabilities like the reference does: batched head products and the masked
+        softmax kernels."""
+        return ctx.dtype == torch.bfloat16 and (self.head_dim in (64, 128) or (self.head_dim == 32 and self.heads % 2 == 0))
 
     def stash_specs(self, ctx):
         R, h, f = ctx.rows, self.hidden, self.ffn

@@ -220,7 +220,7 @@ int bb_softmax_fwd(int dtype, int mask, int batch, int heads, int sq, int sk, vo
 int bb_softmax_bwd(int dtype, int batch, int heads, int sq, int sk, const void* p, void* dp,
                    void* stream);
 
-/* Fused masked softmax-attention (bf16; head_dim d = 64, or d = 32 with an even number of heads -- the kernels
+/* Fused masked softmax-attention (bf16; head_dim d = 64 or 128, or d = 32 with an even number of heads -- the kernels
  * then take two neighbouring heads per block; gpt2.py:212-214 defaults to 512 / 16 = 32):
  * out = softmax(Q K^T / sqrt(d), mask) V for every (batch, head), without materialising the score matrix
  * (transformer.py:117-127).

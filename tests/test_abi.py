@@ -227,4 +227,4 @@ def test_batchnorm_backward_sums_and_head_pairs_validate_on_the_host():
     # attention: 64-wide heads, or an even number of 32-wide ones
     args = lambda heads, dim: (BF16, 0, 1, heads, 64, dim, one, one, one, 3 * heads * dim, one, heads * dim, one, None, 0.0, 0, 0, None)
     assert L.bb_attention_fwd(*args(3, 32)) == -1 and b"even number of heads" in L.bb_last_error()
-    assert L.bb_attention_fwd(*args(2, 128)) == -1 and b"head dimension" in L.bb_last_error()
+    assert L.bb_attention_fwd(*args(2, 96)) == -1 and b"head dimension" in L.bb_last_error()

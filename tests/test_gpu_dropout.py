@@ -82,7 +82,8 @@ def test_gemm_epilogue_dropout(hiplib, dtype, M, N, K, epi):
 
 
 @pytest.mark.parametrize("mask", ["none", "causal", "key_padding"])
-@pytest.mark.parametrize("batch,heads,seq,d", [(2, 2, 128, 64), (1, 3, 200, 64), (2, 4, 128, 32), (1, 2, 200, 32)])
+@pytest.mark.parametrize("batch,heads,seq,d", [(2, 2, 128, 64), (1, 3, 200, 64), (2, 4, 128, 32), (1, 2, 200, 32), (2, 2, 128, 128),
+                                               (1, 1, 200, 128)])
 def test_fused_attention_dropout_fwd_bwd(hiplib, mask, batch, heads, seq, d):
     """softmax(QK^T / sqrt(d), mask) -> dropout -> V with the oracle's explicit mask through torch autograd in fp64,
     against the fused kernels that evaluate the decisions themselves: context, dQ, dK, dV (64-wide heads, and 32-wide

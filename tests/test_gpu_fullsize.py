@@ -338,11 +338,13 @@ def test_unfused_attention_fp32_at_12_heads_512_positions(hiplib, mask):
 
 
 @pytest.mark.parametrize("mask", ["none", "causal", "key_padding"])
-@pytest.mark.parametrize("d,a,fused", [(32, 4, True), (32, 3, False), (128, 4, False)], ids=["d32-pairs-fused", "d32-odd-heads", "d128"])
+@pytest.mark.parametrize("d,a,fused", [(32, 4, True), (32, 3, False), (128, 4, True), (96, 2, False)],
+                         ids=["d32-pairs-fused", "d32-odd-heads", "d128-fused", "d96"])
 def test_bf16_attention_with_other_head_widths(hiplib, mask, d, a, fused):
     """bf16 heads that are not 64 wide, through the layer's attention calls.  An even number of 32-wide heads (the
     reference's GPT-2 script defaults to 512 / 16 = 32, gpt2.py:212-214) runs on the fused kernels, which take the
-    heads in pairs; an odd number of them and 128-wide heads take the path that materialises the probabilities.
+    heads in pairs, and so do 128-wide heads (two column panels); an odd number of 32-wide heads and other widths take
+    the path that materialises the probabilities.
     Context and the three input gradients against fp64 autograd on ``softmax(Q K^T / sqrt(d) [masked]) V``, 2e-2 of
     each tensor's largest magnitude, for the three masks."""
     from bamboo_amd.layers import StageContext

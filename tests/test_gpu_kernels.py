@@ -346,10 +346,11 @@ def test_softmax(hiplib, dtype, mask):
 
 @pytest.mark.parametrize("mask", ["none", "causal", "key_padding"])
 @pytest.mark.parametrize("b,a,s,d", [(2, 3, 128, 64), (1, 2, 64, 64), (2, 2, 96, 64), (1, 4, 384, 64), (3, 1, 32, 64), (1, 16, 1024, 64),
-                                     (2, 6, 128, 32), (1, 2, 64, 32), (2, 4, 96, 32), (3, 2, 32, 32), (1, 16, 1024, 32)])
+                                     (2, 6, 128, 32), (1, 2, 64, 32), (2, 4, 96, 32), (3, 2, 32, 32), (1, 16, 1024, 32),
+                                     (2, 3, 128, 128), (1, 2, 64, 128), (2, 1, 96, 128), (3, 1, 32, 128), (1, 8, 1024, 128)])
 def test_fused_attention_fwd_bwd(hiplib, mask, b, a, s, d):
-    """Fused attention (bf16, d = 64, and d = 32 with the heads taken in pairs) against softmax(QK^T/sqrt(d), mask) V and
-    its autograd gradients, computed in fp64 from the same bf16 inputs."""
+    """Fused attention (bf16, d = 64, d = 32 with the heads taken in pairs, d = 128 as two 64-wide column panels) against
+    softmax(QK^T/sqrt(d), mask) V and its autograd gradients, computed in fp64 from the same bf16 inputs."""
     h = a * d
     qkv = randn(b * s, 3 * h, dtype=torch.bfloat16, seed=70, scale=1.0)
     d_out = randn(b * s, h, dtype=torch.bfloat16, seed=71)
@@ -401,7 +402,7 @@ def test_fused_attention_rejects(hiplib):
     rc = L.bb_attention_fwd(hiplib.BF16, 0, 1, 3, 64, 32, q3.data_ptr(), q3.data_ptr() + 192, q3.data_ptr() + 384, 288, o3.data_ptr(), 96,
                             l3.data_ptr(), None, 0.0, 0, 0, None)
     assert rc != 0 and b"even number of heads" in L.bb_last_error()
-    rc = L.bb_attention_fwd(hiplib.BF16, 0, 1, 1, 64, 128, q3.data_ptr(), q3.data_ptr(), q3.data_ptr(), 384, o3.data_ptr(), 128,
+    rc = L.bb_attention_fwd(hiplib.BF16, 0, 1, 1, 64, 96, q3.data_ptr(), q3.data_ptr(), q3.data_ptr(), 288, o3.data_ptr(), 96,
                             l3.data_ptr(), None, 0.0, 0, 0, None)
     assert rc != 0 and b"head dimension" in L.bb_last_error()
 

@@ -921,12 +921,12 @@ def test_sigterm_and_launch_observer_belong_to_one_engine(hiplib):
         signal.signal(signal.SIGTERM, prev)
 
 
-@pytest.mark.parametrize("hid,heads,fused", [(128, 4, True), (96, 3, False), (128, 1, False)],
-                         ids=["head-width-32-pairs", "head-width-32-odd-heads", "head-width-128"])
+@pytest.mark.parametrize("hid,heads,fused", [(128, 4, True), (96, 3, False), (128, 1, True), (192, 2, False)],
+                         ids=["head-width-32-pairs", "head-width-32-odd-heads", "head-width-128", "head-width-96"])
 def test_bf16_stage_with_other_head_widths_matches_oracle(hiplib, hid, heads, fused):
     """A bf16 stage whose heads are 32 (the reference GPT-2 script's default, gpt2.py:212-214: the fused kernels take
-    an even number of them in pairs, an odd number materialises the probabilities) or 128 wide, with redundant
-    forwards: outputs, input gradients and parameter gradients against the fp64 oracle at the bf16 bars, and the
+    an even number of them in pairs, an odd number materialises the probabilities), 128 (fused) or 96 wide (not),
+    with redundant forwards: outputs, input gradients and parameter gradients against the fp64 oracle at the bf16 bars, and the
     redundant forward's output bit-equal to the own forward of the same layers on the same input."""
     ffn, L, S, sid, mb, M, seq = 256, 2, 4, 1, 2, 4, 64
     dtype = torch.bfloat16
