@@ -1007,12 +1007,12 @@ def test_gradient_clipping_in_the_optimizer_step(hiplib):
     assert not torch.equal(plain.module.stage_params[sid].exp_avg, tight.module.stage_params[sid].exp_avg)
 
 
-def _decoder_stage(dtype, variant, dropout=0.0, dead_from=None, grad_mode="queue"):
+def _decoder_stage(dtype, variant, dropout=0.0, dead_from=None, grad_mode="queue", heads=2):
     """Engine (stage 1 of 4, one DecoderLayer per stage, redundant forwards on) and oracle on the same weights and
     inputs drawn from U(0, 0.4): the memory sqrt(1 - x) of every layer stays real (the sublayers move the stream by
     a few hundredths at these weight scales)."""
     from bamboo_amd import DecoderLayer
-    hid, heads, ffn, S, sid, mb, M, seq = 128, 2, 256, 4, 1, 2, 4, 64
+    hid, ffn, S, sid, mb, M, seq = 128, 256, 4, 1, 2, 4, 64
     specs = [LayerSpec(DecoderLayer, hid, heads, ffn, dropout=dropout, **variant) for _ in range(S)]
     model = PipelineModule(specs, num_stages=S, partition_method="uniform", stage_id=sid, dtype=dtype, device=DEV)
     q = SeededActivationQueue((mb, seq, hid), dtype, M, stage_ids=[sid, sid + 1], seed=7, grad_mode=grad_mode, device=DEV)
@@ -1038,14 +1038,18 @@ def _decoder_stage(dtype, variant, dropout=0.0, dead_from=None, grad_mode="queue
     return engine, q, st, peer, (hid, mb, M, seq, sid)
 
 
-@pytest.mark.parametrize("dtype,variant", [(torch.float32, REFERENCE_VARIANT), (torch.float32, GPT_VARIANT), (torch.bfloat16, GPT_VARIANT)],
-                         ids=["fp32-script-variant", "fp32-gpt", "bf16-gpt"])
-def test_decoder_stage_matches_oracle_with_rc(hiplib, dtype, variant):
+@pytest.mark.parametrize("dtype,variant,heads", [(torch.float32, REFERENCE_VARIANT, 2), (torch.float32, GPT_VARIANT, 2),
+                                                 (torch.bfloat16, GPT_VARIANT, 2), (torch.bfloat16, GPT_VARIANT, 4)],
+                         ids=["fp32-script-variant", "fp32-gpt", "bf16-gpt", "bf16-gpt-head-width-32"])
+def test_decoder_stage_matches_oracle_with_rc(hiplib, dtype, variant, heads):
     """A stage of the GPT-2 script's layers (DecoderLayerSimple, gpt2.py:20-34: self-attention, attention over
     sqrt(1 - x) of the layer input, feed-forward) with redundant forwards: own and redundant outputs, the gradient
     sent upstream (which also flows through the memory) and all 26 parameter gradients of the own layer against
-    the fp64 oracle; the shadow layer's gradients stay zero."""
-    engine, q, st, peer, (hid, mb, M, seq, sid) = _decoder_stage(dtype, variant)
+    the fp64 oracle; the shadow layer's gradients stay zero.  The last case has the script's own head width (512 / 16 =
+    32, gpt2.py:212-214): both attentions of the layer on the fused kernels, heads in pairs."""
+    engine, q, st, peer, (hid, mb, M, seq, sid) = _decoder_stage(dtype, variant, heads=heads)
+    if dtype == torch.bfloat16:
+        assert engine.module.func_buckets[sid][0].fused_attention(engine.ctx)
     keep = {}
     with NoStep(engine):
         engine._clean_pipe_buffers = lambda: keep.update({k: list(v) for k, v in engine.pipe_buffers.items()})
