@@ -613,6 +613,40 @@ def test_graph_replay_equals_eager(hiplib, variant, klr, rc_stream, ckpt):
     assert losses[4] != losses[0]
 
 
+def test_graph_replay_equals_eager_on_a_resnet_stage(hiplib):
+    """The same for a bottleneck stage of the widths whose backward takes the BatchNorm sums from GEMM epilogues and
+    hands a gradient from block to block with the next block's mask and sums: four batches with optimizer steps,
+    weights, Adam moments and BatchNorm running statistics bit-equal between launching every kernel and replaying
+    the captured passes."""
+    from bamboo_amd import BottleNeck
+    cin, cmid, side, L, S, sid, mb, M = 512, 128, 6, 2, 4, 1, 8, 4
+    def make(use_graphs):
+        specs = [LayerSpec(BottleNeck, cin, cmid, height=side, width=side) for _ in range(L * S)]
+        model = PipelineModule(specs, num_stages=S, partition_method="uniform", stage_id=sid, dtype=torch.bfloat16, device=DEV)
+        q = SeededActivationQueue((mb, side * side, cin), torch.bfloat16, M, stage_ids=[sid, sid + 1], seed=9, device=DEV)
+        cfg = {"train_micro_batch_size_per_gpu": mb, "gradient_accumulation_steps": M, "bf16": {"enabled": True},
+               "optimizer": {"type": "Adam", "params": {"lr": 1e-3}}}
+        engine, _, _, _ = bamboo_amd.initialize(model=model, config=cfg, redundancy_level=1, eager_recovery=True,
+                                                activation_queue=q, install_signal_handler=False, use_graphs=use_graphs)
+        for _ in range(4):
+            engine.train_batch()
+            torch.cuda.synchronize()
+        return engine
+    eager = make(False)
+    side_stream = torch.cuda.Stream()
+    with torch.cuda.stream(side_stream):
+        graphed = make(True)
+    torch.cuda.synchronize()
+    assert graphed._graphs and all(isinstance(v, tuple) for v in graphed._graphs.values())
+    assert any(k[0] == "sink" and v for layer in graphed.module.func_buckets[sid] for k, v in layer._stats_ok.items())
+    a, b = graphed.module.stage_params[sid], eager.module.stage_params[sid]
+    assert torch.equal(a.master, b.master) and torch.equal(a.exp_avg_sq, b.exp_avg_sq)
+    for la, lb in zip(graphed.module.func_buckets[sid], eager.module.func_buckets[sid]):
+        ra, rb = la._running(DEV), lb._running(DEV)
+        for idx in ra:
+            assert torch.equal(ra[idx][0], rb[idx][0]) and torch.equal(ra[idx][1], rb[idx][1])
+
+
 @pytest.mark.parametrize("interval", [1, 2, 3])
 @pytest.mark.parametrize("rc_stream", [False, True], ids=["one-stream", "rc-stream"])
 def test_activation_checkpointing_equals_full_stash(hiplib, interval, rc_stream):
