@@ -539,6 +539,37 @@ extern "C" int bb_gemm_grouped(const bb_gemm_desc* descs, int count, void* strea
         fuse = d.dtype == BB_BF16 && d.layout == descs[0].layout && d.nb1 <= 1 && d.nb2 <= 1 && d.M > 0 && d.N > 0 &&
                d.dropout_p == 0.f && pick_dma_tile(d.M, d.N, d.K, 1, d.layout) != D_NONE;
     }
+    // fp32: unbatched problems of one layout that all take the small tile (each alone would leave CUs idle) share a launch
+    bool fuse32 = !fuse && !has_conv && count >= 2 && count <= GROUP_MAX;
+    for (int i = 0; i < count && fuse32; ++i) {
+        const bb_gemm_desc& d = descs[i];
+        fuse32 = d.dtype == BB_F32 && d.layout == descs[0].layout && d.nb1 <= 1 && d.nb2 <= 1 && d.M > 0 && d.N > 0 &&
+                 d.dropout_p == 0.f && pick_f32_tile(d.M, d.N, 1) == 64;
+    }
+    if (fuse32) {
+        GroupedArgs G;
+        G.count = count;
+        int blocks = 0;
+        for (int i = 0; i < count; ++i) {
+            int64_t batches;
+            bool ta, tb;
+            int rc = fill_args(&descs[i], G.p[i], batches, ta, tb);
+            if (rc) return rc;
+            // the bias gradient that rides on a weight gradient: its own kernel, as on the one-by-one route
+            if (descs[i].colsum_out && (rc = colsum_standalone(&descs[i], stream)) != BB_OK) return rc;
+            G.p[i].tiles_m = (G.p[i].M + 63) / 64;
+            G.p[i].tiles_n = (G.p[i].N + 63) / 64;
+            G.first_block[i] = blocks;
+            blocks += G.p[i].tiles_m * G.p[i].tiles_n;
+        }
+        G.first_block[count] = blocks;
+        const int layout = descs[0].layout;
+        if (layout == BB_NT) hipLaunchKernelGGL((gemm_f32_grouped_kernel<false, false, 64>), dim3(blocks), dim3(256), 0, st, G);
+        else if (layout == BB_NN) hipLaunchKernelGGL((gemm_f32_grouped_kernel<false, true, 64>), dim3(blocks), dim3(256), 0, st, G);
+        else hipLaunchKernelGGL((gemm_f32_grouped_kernel<true, true, 64>), dim3(blocks), dim3(256), 0, st, G);
+        BB_LAUNCH_CHECK();
+        return BB_OK;
+    }
     // a patch-matrix B exists only inside the grouped kernel: no one-by-one route for it
     BB_REQUIRE(fuse || !has_conv, "bb_gemm_grouped: a problem with a patch-matrix B must share a launch of bf16 BB_TN "
                                   "problems the DMA kernel takes (M, N >= 128, K %% 32 == 0)");

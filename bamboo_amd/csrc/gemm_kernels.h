@@ -1430,8 +1430,10 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_bf16_dma_grouped_kernel(cons
 // TILE = BM = BN: 128 (wave tile 64x64), or 64 (wave tile 32x32) for problems with so few 128x128 tiles that most CUs
 // would hold one block, i.e. one wave per SIMD with nobody to cover its waits for the next k-tile.  Every element adds
 // up its contraction in the same order on both.
-template <bool TA, bool TB, int TILE = 128>
-__global__ __launch_bounds__(256) void gemm_f32_kernel(const GemmArgs g) {
+// (block_id: the block's index among the problem's tiles; logical_id: it is not a hardware block id, so the tile order
+// takes it as it is instead of undoing the round-robin over the XCDs)
+template <bool TA, bool TB, int TILE>
+__device__ __forceinline__ void gemm_f32_body(const GemmArgs& g, const int block_id, const int batch_id, const bool logical_id) {
     constexpr int BM = TILE, BN = TILE, BK = 16, LDS_LD = TILE + 4, NT = 256;
     constexpr int WT = TILE / 2, TF = WT / 32;          // wave tile side, 32x32 accumulator tiles along it
     constexpr int CH = TILE * BK / 4 / NT;              // 16-byte chunks of an operand tile per thread
@@ -1441,9 +1443,10 @@ __global__ __launch_bounds__(256) void gemm_f32_kernel(const GemmArgs g) {
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wm = wave >> 1, wn = wave & 1;
     int tile_m, tile_n;
-    tile_coords(blockIdx.x, g.tiles_m, g.tiles_n, tile_m, tile_n);
+    if (logical_id) panel_coords(block_id, g.tiles_m, g.tiles_n, tile_m, tile_n);
+    else tile_coords(block_id, g.tiles_m, g.tiles_n, tile_m, tile_n);
     const int m0 = tile_m * BM, n0 = tile_n * BN;
-    const int b1 = blockIdx.z / g.nb2, b2 = blockIdx.z % g.nb2;
+    const int b1 = batch_id / g.nb2, b2 = batch_id % g.nb2;
     const float* A = (const float*)g.A + b1 * g.sA1 + b2 * g.sA2;
     const float* B = (const float*)g.B + b1 * g.sB1 + b2 * g.sB2;
     const int64_t coff = b1 * g.sC1 + b2 * g.sC2;
@@ -1534,5 +1537,18 @@ __global__ __launch_bounds__(256) void gemm_f32_kernel(const GemmArgs g) {
                 if (m < g.M) epilogue_elem<float>(g, coff, coff, m, n, acc[i][j][r]);
             }
         }
+}
+
+template <bool TA, bool TB, int TILE = 128>
+__global__ __launch_bounds__(256) void gemm_f32_kernel(const GemmArgs g) {
+    gemm_f32_body<TA, TB, TILE>(g, blockIdx.x, blockIdx.z, false);
+}
+// several unbatched problems in one launch (the weight gradients of an fp32 layer: the smallest has 144 tiles of 64x64)
+template <bool TA, bool TB, int TILE>
+__global__ __launch_bounds__(256) void gemm_f32_grouped_kernel(const GroupedArgs G) {
+    const int lid = xcd_contiguous(blockIdx.x, G.first_block[G.count]);
+    int pi = 0;
+    while (pi + 1 < G.count && lid >= G.first_block[pi + 1]) ++pi;
+    gemm_f32_body<TA, TB, TILE>(G.p[pi], lid - G.first_block[pi], 0, true);
 }
 
