@@ -279,6 +279,47 @@ def test_gemm_grouped_weight_gradients(hiplib, dtype):
         assert rel_err(a, b.double().cpu()) < 1e-6
 
 
+@pytest.mark.parametrize("layout", ["tn", "nt", "nn"])
+def test_gemm_grouped_fp32_shares_a_launch_bit_equal(hiplib, layout):
+    """fp32 problems that take the small tile share one launch: ragged shapes (rows, columns and contraction that are
+    no multiples of the tile or the k-step), bias-gradient column sums on the weight-gradient layout, an accumulating
+    and a plain problem side by side -- every output bit-equal to the calls made one by one."""
+    K = 200
+    shapes = [(100, 72), (260, 132), (64, 64), (36, 300)]
+    lay = {"tn": hiplib.TN, "nt": hiplib.NT, "nn": hiplib.NN}[layout]
+    mk = lambda *sh, seed: randn(*sh, seed=seed)
+    ops = []
+    for i, (M, N) in enumerate(shapes):
+        A = mk(K, M, seed=80 + i) if layout == "tn" else mk(M, K, seed=80 + i)
+        B = mk(N, K, seed=90 + i) if layout == "nt" else mk(K, N, seed=90 + i)
+        ops.append((A, B, mk(M, N, seed=100 + i), mk(M, seed=110 + i)))
+    ws = torch.empty(hiplib.colsum_workspace(max(m for m, _ in shapes)), device=DEV)
+    def run(grouped):
+        Cs, sums, descs = [c.clone() for _, _, c, _ in ops], [b.clone() for _, _, _, b in ops], []
+        for i, ((A, B, _, _), C, bsum) in enumerate(zip(ops, Cs, sums)):
+            kw = dict(accumulate=i % 2 == 0)
+            if layout == "tn":
+                kw.update(colsum_out=bsum, colsum_ws=ws)
+            descs.append(hiplib.gemm_desc(lay, A, B, C, **kw))
+        if grouped:
+            hiplib.gemm_grouped(descs)
+        else:
+            for d in descs:
+                hiplib.gemm_grouped([d])
+        torch.cuda.synchronize()
+        return Cs, sums
+    c1, s1 = run(False)
+    c2, s2 = run(True)
+    for i, ((A, B, C0, b0), a, b) in enumerate(zip(ops, c1, c2)):
+        assert torch.equal(a, b), i
+        Ad, Bd = A.double().cpu(), B.double().cpu()
+        ref = (Ad.t() if layout == "tn" else Ad) @ (Bd.t() if layout == "nt" else Bd) + (C0.double().cpu() if i % 2 == 0 else 0)
+        assert rel_err(b, ref) < 1e-5, i
+    if layout == "tn":
+        for i, ((A, _, _, b0), x, y) in enumerate(zip(ops, s1, s2)):
+            assert torch.equal(x, y) and rel_err(y, b0.double().cpu() + A.double().cpu().sum(0)) < 1e-5, i
+
+
 def test_gemm_rejects_bad_arguments(hiplib):
     A = torch.zeros(16, 12, dtype=torch.bfloat16, device=DEV)   # K = 12 is not a multiple of 8
     B = torch.zeros(16, 12, dtype=torch.bfloat16, device=DEV)
