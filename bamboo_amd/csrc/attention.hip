@@ -187,7 +187,7 @@ static unsigned attn_grid(int seq, int nbh) { return (unsigned)(8 * ((nbh + 7) /
 // 128-wide heads, HP = 1: a tile in LDS is then two [64][64] panels behind each other, each in the format above);
 // KS k-steps of a head's scores, DT 32-wide output tiles of a head
 template <bool DROP, int HP, int NPAN = 1>
-__global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const AttnArgs a) {
+__global__ __launch_bounds__(256, (!DROP && NPAN == 1 && HP == 1) ? 4 : 2) void attn_fwd_kernel(const AttnArgs a) {
     static_assert(HP == 1 || NPAN == 1, "pairs of heads are 32 wide");
     constexpr int KS = 4 * NPAN / HP, DT = 2 * NPAN / HP, TILE = NPAN * 8192;
     __shared__ __attribute__((aligned(16))) unsigned char smem[2 * 2 * TILE];  // 2 stages x (K, V)
