@@ -120,18 +120,24 @@ __device__ __forceinline__ void unpack16(const u32x4& t, float (&v)[8]) {
 }
 
 constexpr int LN_BWD_BLOCKS = 256;
-constexpr int LN_BWD_WAVES = 16;  // one block per CU, four waves per SIMD to cover the load latency
+// One block per CU.  A lane keeps five fp32 values per element it owns (gain, two running sums, the normalised input and
+// the scaled gradient of the row in flight): up to 16 elements per lane that fits the 128 registers of sixteen waves
+// (four per SIMD, to cover the load latency); wider rows take eight or four waves with more registers each instead of
+// spilling.
+template <typename T, int IT> constexpr int ln_bwd_waves() {
+    return IT * Elem<T>::VEC <= 16 ? 16 : IT * Elem<T>::VEC <= 32 ? 8 : 4;
+}
 
 // dx per row, dgain/dshift partial sums per block (fixed row->block assignment).
 template <typename T, int IT>
-__global__ __launch_bounds__(LN_BWD_WAVES * 64) void layernorm_bwd_kernel(int kind, int rows, int cols, float eps,
+__global__ __launch_bounds__((ln_bwd_waves<T, IT>() * 64)) void layernorm_bwd_kernel(int kind, int rows, int cols, float eps,
                                                             const T* __restrict__ x, const T* __restrict__ gain,
                                                             const float* __restrict__ mean_in,
                                                             const float* __restrict__ rinv_in, const T* __restrict__ dy,
                                                             const T* __restrict__ dres, T* __restrict__ dx,
                                                             float* __restrict__ partial, int one_pass) {
-    constexpr int VEC = Elem<T>::VEC;
-    extern __shared__ float red[];  // [16 waves][2][cols] (one pass) or [3 waves][2][cols] for the cross-wave sum
+    constexpr int VEC = Elem<T>::VEC, LN_BWD_WAVES = ln_bwd_waves<T, IT>();
+    extern __shared__ float red[];  // [all waves][2][cols] (one pass) or [3 waves][2][cols] for the cross-wave sum
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int nvec = cols / VEC;
     float gv[IT][VEC], dg[IT][VEC], db[IT][VEC];
@@ -202,7 +208,7 @@ __global__ __launch_bounds__(LN_BWD_WAVES * 64) void layernorm_bwd_kernel(int ki
             }
         }
     }
-    // cross-wave sum.  Where the LDS holds all sixteen waves' sums (2 * cols floats each): one barrier, then every
+    // cross-wave sum.  Where the LDS holds all waves' sums (2 * cols floats each): one barrier, then every
     // thread adds up its share of the 2 * cols outputs over the waves in wave order, and the block's partial row is
     // written by all threads.  Wider rows go three waves per round through three slots (fixed order as well).
     if (one_pass) {
@@ -335,6 +341,7 @@ static int ln_fwd_launch(int kind, int rows, int cols, float eps, const void* x,
 template <typename T, int IT>
 static int ln_bwd_launch(int kind, int rows, int cols, float eps, const void* x, const void* gain, const float* mean,
                          const float* rinv, const void* dy, const void* dres, void* dx, float* ws, hipStream_t st) {
+    constexpr int LN_BWD_WAVES = ln_bwd_waves<T, IT>();
     const size_t all = (size_t)LN_BWD_WAVES * 2 * cols * sizeof(float);
     const int one_pass = all <= 128 * 1024;
     const size_t smem = one_pass ? all : (size_t)3 * 2 * cols * sizeof(float);
