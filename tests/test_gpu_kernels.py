@@ -335,8 +335,13 @@ def test_gemm_rejects_bad_arguments(hiplib):
 
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("kind", ["standard", "annotated"])
-@pytest.mark.parametrize("rows,cols", [(64, 768), (37, 1024), (16, 1600), (5, 64), (3, 4096)])
+@pytest.mark.parametrize("rows,cols", [(64, 768), (37, 1024), (16, 1600), (5, 64), (3, 4096),
+                                       (2100, 1600),   # every wave of every block owns rows, some two (8 waves in bf16)
+                                       (300, 2048),    # fp32: 8 waves, bf16: 8 waves at their widest row
+                                       (130, 6144)])   # bf16 only: 4 waves, sums through the three LDS slots
 def test_layernorm_fwd_bwd(hiplib, dtype, kind, rows, cols):
+    if cols > 4096 and dtype == torch.float32:
+        pytest.skip("fp32 rows hold at most 4096 columns")
     eps = 1e-6 if kind == "annotated" else 1e-5
     x, dy, dres = randn(rows, cols, dtype=dtype, seed=10), randn(rows, cols, dtype=dtype, seed=11), randn(rows, cols, dtype=dtype, seed=12)
     g = (1 + 0.1 * randn(cols, seed=13)).to(dtype)
