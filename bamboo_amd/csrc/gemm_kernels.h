@@ -1430,17 +1430,24 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_bf16_dma_grouped_kernel(cons
 // TILE = BM = BN: 128 (wave tile 64x64), or 64 (wave tile 32x32) for problems with so few 128x128 tiles that most CUs
 // would hold one block, i.e. one wave per SIMD with nobody to cover its waits for the next k-tile.  Every element adds
 // up its contraction in the same order on both.
+// KG > 1: KG groups of four waves share a 64x64 tile; group j takes the k-tiles j, j + KG, ... through LDS buffers of
+// its own and the groups' partial tiles are added in group order at the end -- for problems that have fewer than two
+// 64x64 tiles per CU and a long contraction (a different, equally fixed order of additions: the shape alone decides).
 // (block_id: the block's index among the problem's tiles; logical_id: it is not a hardware block id, so the tile order
 // takes it as it is instead of undoing the round-robin over the XCDs)
-template <bool TA, bool TB, int TILE>
+template <bool TA, bool TB, int TILE, int KG = 1>
 __device__ __forceinline__ void gemm_f32_body(const GemmArgs& g, const int block_id, const int batch_id, const bool logical_id) {
     constexpr int BM = TILE, BN = TILE, BK = 16, LDS_LD = TILE + 4, NT = 256;
     constexpr int WT = TILE / 2, TF = WT / 32;          // wave tile side, 32x32 accumulator tiles along it
     constexpr int CH = TILE * BK / 4 / NT;              // 16-byte chunks of an operand tile per thread
     constexpr int RQ = TILE / 4;                        // chunks along a row-contiguous (transposed) tile row
-    __shared__ __attribute__((aligned(16))) float As[2][BK * LDS_LD];
-    __shared__ __attribute__((aligned(16))) float Bs[2][BK * LDS_LD];
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    static_assert(KG == 1 || TILE == 64, "the contraction is split over wave groups on the small tile only");
+    __shared__ __attribute__((aligned(16))) float As_all[KG][2][BK * LDS_LD];
+    __shared__ __attribute__((aligned(16))) float Bs_all[KG][2][BK * LDS_LD];
+    const int grp = KG == 1 ? 0 : threadIdx.x >> 8;
+    const int tid = threadIdx.x & 255, lane = tid & 63, wave = tid >> 6;
+    float (*As)[BK * LDS_LD] = As_all[grp];
+    float (*Bs)[BK * LDS_LD] = Bs_all[grp];
     const int wm = wave >> 1, wn = wave & 1;
     int tile_m, tile_n;
     if (logical_id) panel_coords(block_id, g.tiles_m, g.tiles_n, tile_m, tile_n);
@@ -1452,6 +1459,7 @@ __device__ __forceinline__ void gemm_f32_body(const GemmArgs& g, const int block
     const int64_t coff = b1 * g.sC1 + b2 * g.sC2;
 
     f32x4 ra[CH], rb[CH];
+    // a k-tile past the end of the contraction loads zeros (a group whose share is one k-tile shorter adds nothing)
     auto gload = [&](const float* base, int64_t ld, int row0, int rows, int k0, bool tr, f32x4 (&r)[CH]) {
 #pragma unroll
         for (int i = 0; i < CH; ++i) {
@@ -1492,9 +1500,11 @@ __device__ __forceinline__ void gemm_f32_body(const GemmArgs& g, const int block
 #pragma unroll
             for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
 
-    const int KT = (g.K + BK - 1) / BK;
-    gload(A, g.lda, m0, g.M, 0, TA, ra);
-    gload(B, g.ldb, n0, g.N, 0, TB, rb);
+    // every group runs the same number of rounds (the barriers are the block's); round it of group grp is k-tile
+    // it * KG + grp
+    const int KT = ((g.K + BK - 1) / BK + KG - 1) / KG;
+    gload(A, g.lda, m0, g.M, grp * BK, TA, ra);
+    gload(B, g.ldb, n0, g.N, grp * BK, TB, rb);
     sstore(As[0], TA, ra);
     sstore(Bs[0], TB, rb);
     __syncthreads();
@@ -1502,8 +1512,8 @@ __device__ __forceinline__ void gemm_f32_body(const GemmArgs& g, const int block
         const int cur = kt & 1;
         const bool more = kt + 1 < KT;
         if (more) {
-            gload(A, g.lda, m0, g.M, (kt + 1) * BK, TA, ra);
-            gload(B, g.ldb, n0, g.N, (kt + 1) * BK, TB, rb);
+            gload(A, g.lda, m0, g.M, ((kt + 1) * KG + grp) * BK, TA, ra);
+            gload(B, g.ldb, n0, g.N, ((kt + 1) * KG + grp) * BK, TB, rb);
         }
 #pragma unroll
         for (int ks = 0; ks < BK / 2; ++ks) {
@@ -1525,6 +1535,27 @@ __device__ __forceinline__ void gemm_f32_body(const GemmArgs& g, const int block
         }
         __syncthreads();
     }
+    if constexpr (KG > 1) {
+        // partial tiles of groups 1 .. KG-1 go through the groups' own (now idle) operand buffers, eight of a thread's
+        // sixteen values through each of A's and B's; group 0 adds them up in group order
+        static_assert(TF == 1 && 2 * BK * LDS_LD >= 8 * NT, "a group's operand buffers hold its partial tile");
+        if (grp > 0) {
+#pragma unroll
+            for (int r = 0; r < 8; ++r) {
+                (&As_all[grp][0][0])[r * NT + tid] = acc[0][0][r];
+                (&Bs_all[grp][0][0])[r * NT + tid] = acc[0][0][8 + r];
+            }
+        }
+        __syncthreads();
+        if (grp > 0) return;
+#pragma unroll
+        for (int j = 1; j < KG; ++j)
+#pragma unroll
+            for (int r = 0; r < 8; ++r) {
+                acc[0][0][r] += (&As_all[j][0][0])[r * NT + tid];
+                acc[0][0][8 + r] += (&Bs_all[j][0][0])[r * NT + tid];
+            }
+    }
 #pragma unroll
     for (int i = 0; i < TF; ++i)
 #pragma unroll
@@ -1542,6 +1573,11 @@ __device__ __forceinline__ void gemm_f32_body(const GemmArgs& g, const int block
 template <bool TA, bool TB, int TILE = 128>
 __global__ __launch_bounds__(256) void gemm_f32_kernel(const GemmArgs g) {
     gemm_f32_body<TA, TB, TILE>(g, blockIdx.x, blockIdx.z, false);
+}
+// 64x64 tiles, the contraction dealt to KG groups of four waves
+template <bool TA, bool TB, int KG>
+__global__ __launch_bounds__(256 * KG) void gemm_f32_ksplit_kernel(const GemmArgs g) {
+    gemm_f32_body<TA, TB, 64, KG>(g, blockIdx.x, blockIdx.z, false);
 }
 // several unbatched problems in one launch (the weight gradients of an fp32 layer: the smallest has 144 tiles of 64x64)
 template <bool TA, bool TB, int TILE>

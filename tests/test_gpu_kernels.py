@@ -279,6 +279,37 @@ def test_gemm_grouped_weight_gradients(hiplib, dtype):
         assert rel_err(a, b.double().cpu()) < 1e-6
 
 
+@pytest.mark.parametrize("layout", ["nt", "nn"])
+@pytest.mark.parametrize("M,N,K", [(256, 192, 520),     # 33 k-tiles: the second wave group's share is one shorter
+                                   (2048, 768, 768),    # C1's attention output projection
+                                   (100, 72, 1036)])    # ragged rows, columns and contraction
+def test_gemm_fp32_contraction_shared_by_wave_groups(hiplib, layout, M, N, K):
+    """fp32 problems with fewer than two 64x64 tiles per CU and a long contraction deal the k-tiles of a tile to two
+    groups of waves (partial tiles added in group order): against fp64 with bias, residual and accumulation, the same
+    bits on a second call, and problems outside the rule keep the plain kernel."""
+    lay = {"nt": hiplib.NT, "nn": hiplib.NN}[layout]
+    A = randn(M, K, seed=120)
+    B = randn(N, K, seed=121) if layout == "nt" else randn(K, N, seed=121)
+    bias, resid, C0 = randn(N, seed=122), randn(M, N, seed=123), randn(M, N, seed=124)
+    prod = A.double().cpu() @ (B.double().cpu().t() if layout == "nt" else B.double().cpu())
+    C = torch.empty(M, N, device=DEV)
+    assert hiplib.gemm_variant(hiplib.gemm_desc(lay, A, B, C)).endswith("64x64k2")
+    hiplib.gemm(lay, A, B, C, bias=bias, epilogue=hiplib.EPI_RESIDUAL, resid=resid)
+    assert rel_err(C, prod + bias.double().cpu() + resid.double().cpu()) < 1e-5
+    C2 = torch.zeros_like(C)
+    hiplib.gemm(lay, A, B, C2, bias=bias, epilogue=hiplib.EPI_RESIDUAL, resid=resid)
+    assert torch.equal(C, C2)
+    Ca = C0.clone()
+    hiplib.gemm(lay, A, B, Ca, accumulate=True, alpha=0.5)
+    assert rel_err(Ca, C0.double().cpu() + 0.5 * prod) < 1e-5
+    # a short contraction, many tiles, or the weight-gradient layout: the plain kernels
+    assert hiplib.gemm_variant(hiplib.gemm_desc(lay, A[:, :256], B[:, :256] if layout == "nt" else B[:256], C)).endswith("64x64")
+    big = torch.empty(2048, 3072, device=DEV)
+    Bb = torch.empty(3072, K, device=DEV) if layout == "nt" else torch.empty(K, 3072, device=DEV)
+    assert hiplib.gemm_variant(hiplib.gemm_desc(lay, torch.empty(2048, K, device=DEV), Bb, big)).endswith("64x64")
+    assert hiplib.gemm_variant(hiplib.gemm_desc(hiplib.TN, torch.empty(K, M, device=DEV), torch.empty(K, N, device=DEV), C)).endswith("64x64")
+
+
 @pytest.mark.parametrize("layout", ["tn", "nt", "nn"])
 def test_gemm_grouped_fp32_shares_a_launch_bit_equal(hiplib, layout):
     """fp32 problems that take the small tile share one launch: ragged shapes (rows, columns and contraction that are
