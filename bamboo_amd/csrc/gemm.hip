@@ -216,20 +216,19 @@ template <bool TA, bool TB> static int dispatch_bf16(GemmArgs& g, int batches, h
     }
 }
 
-#ifndef F32_KGROUPS
-#define F32_KGROUPS 2
-#endif
 static int pick_f32_tile(int M, int N, int64_t batches) {
     const int64_t t128 = (int64_t)((M + 127) / 128) * ((N + 127) / 128) * batches;
     return t128 < 2 * 256 ? 64 : 128;
 }
-// Wave groups that share the contraction of a 64x64 tile: problems with fewer than two such tiles per CU (one or two
-// waves per SIMD) and at least 32 k-tiles wait for operands most of the time; two groups halve each wave's chain of
-// k-tiles and double the waves.  NT and NN only: the weight gradients (TN) of a layer share a grouped launch.
-static int pick_f32_kgroups(int M, int N, int K, int64_t batches, int layout) {
-    if (layout == BB_TN || pick_f32_tile(M, N, batches) != 64) return 1;
+// Problems with fewer than two 64x64 tiles per CU (one or two waves per SIMD, and some CUs with twice the tiles of
+// others) and at least 32 k-tiles wait for operands most of the time: they take 64x32 tiles whose contraction two
+// groups of two waves share (kF32SplitGroups; twice the tiles, each wave's chain of k-tiles halved).  NT and NN only:
+// the weight gradients (TN) of a layer share a grouped launch.
+static constexpr int kF32SplitGroups = 2, kF32SplitBN = 32;
+static bool pick_f32_split(int M, int N, int K, int64_t batches, int layout) {
+    if (layout == BB_TN || pick_f32_tile(M, N, batches) != 64) return false;
     const int64_t t64 = (int64_t)((M + 63) / 64) * ((N + 63) / 64) * batches;
-    return t64 < 2 * 256 && K >= 512 ? F32_KGROUPS : 1;
+    return t64 < 2 * 256 && K >= 512;
 }
 template <bool TA, bool TB> static int dispatch_f32(GemmArgs& g, int batches, hipStream_t st) {
     // 64x64 tiles while 128x128 ones would leave most CUs with a single block (one wave per SIMD): shape only, and the
@@ -238,8 +237,11 @@ template <bool TA, bool TB> static int dispatch_f32(GemmArgs& g, int batches, hi
     g.tiles_m = (g.M + tile - 1) / tile;
     g.tiles_n = (g.N + tile - 1) / tile;
     dim3 grid(g.tiles_m * g.tiles_n, 1, batches);
-    const int kg = pick_f32_kgroups(g.M, g.N, g.K, batches, TA ? BB_TN : TB ? BB_NN : BB_NT);
-    if (kg > 1) hipLaunchKernelGGL((gemm_f32_ksplit_kernel<TA, TB, F32_KGROUPS>), grid, dim3(256 * F32_KGROUPS), 0, st, g);
+    if (pick_f32_split(g.M, g.N, g.K, batches, TA ? BB_TN : TB ? BB_NN : BB_NT)) {
+        g.tiles_n = (g.N + kF32SplitBN - 1) / kF32SplitBN;
+        grid.x = g.tiles_m * g.tiles_n;
+        hipLaunchKernelGGL((gemm_f32_ksplit_kernel<TA, TB, kF32SplitGroups, kF32SplitBN>), grid, dim3(4 * kF32SplitBN * kF32SplitGroups), 0, st, g);
+    }
     else if (tile == 64) hipLaunchKernelGGL((gemm_f32_kernel<TA, TB, 64>), grid, dim3(256), 0, st, g);
     else hipLaunchKernelGGL((gemm_f32_kernel<TA, TB, 128>), grid, dim3(256), 0, st, g);
     BB_LAUNCH_CHECK();
@@ -259,8 +261,8 @@ extern "C" int bb_gemm_variant(const bb_gemm_desc* d, char* out, int out_len) {
     else
     {
         const int tile = pick_f32_tile(d->M, d->N, batches);
-        const int kg = pick_f32_kgroups(d->M, d->N, d->K, batches, d->layout);
-        if (kg > 1) snprintf(out, out_len, "f32_%s_%dx%dk%d", layouts[d->layout], tile, tile, kg);
+        if (pick_f32_split(d->M, d->N, d->K, batches, d->layout))
+            snprintf(out, out_len, "f32_%s_64x%dk%d", layouts[d->layout], kF32SplitBN, kF32SplitGroups);
         else snprintf(out, out_len, "f32_%s_%dx%d", layouts[d->layout], tile, tile);
     }
     return BB_OK;

@@ -1430,25 +1430,66 @@ __global__ __launch_bounds__(WM* WN * 64) void gemm_bf16_dma_grouped_kernel(cons
 // TILE = BM = BN: 128 (wave tile 64x64), or 64 (wave tile 32x32) for problems with so few 128x128 tiles that most CUs
 // would hold one block, i.e. one wave per SIMD with nobody to cover its waits for the next k-tile.  Every element adds
 // up its contraction in the same order on both.
-// KG > 1: KG groups of four waves share a 64x64 tile; group j takes the k-tiles j, j + KG, ... through LDS buffers of
-// its own and the groups' partial tiles are added in group order at the end -- for problems that have fewer than two
-// 64x64 tiles per CU and a long contraction (a different, equally fixed order of additions: the shape alone decides).
+// BN = 32 (TILE 64): 64x32 tiles of two waves, and KG > 1: KG groups of waves share a tile; group j takes the k-tiles
+// j, j + KG, ... through LDS buffers of its own and the groups' partial tiles are added in group order at the end --
+// for problems that have fewer than two 64x64 tiles per CU and a long contraction (a different, equally fixed order of
+// additions: the shape alone decides).
 // (block_id: the block's index among the problem's tiles; logical_id: it is not a hardware block id, so the tile order
 // takes it as it is instead of undoing the round-robin over the XCDs)
-template <bool TA, bool TB, int TILE, int KG = 1>
+
+// one k-tile of an operand, ROWS x BK: global -> registers (zeros past the operand's rows and past the contraction, so
+// a group whose share is one k-tile shorter adds nothing), registers -> LDS [k][row]
+template <int ROWS, int BK, int NT, int CH>
+__device__ __forceinline__ void f32_gload(const float* base, int64_t ld, int row0, int rows, int k0, int K, bool tr, int tid,
+                                          f32x4 (&r)[CH]) {
+    constexpr int RQ = ROWS / 4;   // chunks along a row-contiguous (transposed) tile row
+#pragma unroll
+    for (int i = 0; i < CH; ++i) {
+        const int c = tid + i * NT;
+        f32x4 v = {0.f, 0.f, 0.f, 0.f};
+        if (!tr) {
+            const int row = c >> 2, kq = c & 3;
+            if (row0 + row < rows && k0 + kq * 4 < K) v = *(const f32x4*)(base + (int64_t)(row0 + row) * ld + k0 + kq * 4);
+        } else {
+            const int k = c / RQ, rq = c % RQ;
+            if (row0 + rq * 4 < rows && k0 + k < K) v = *(const f32x4*)(base + (int64_t)(k0 + k) * ld + row0 + rq * 4);
+        }
+        r[i] = v;
+    }
+}
+template <int ROWS, int LD, int NT, int CH>
+__device__ __forceinline__ void f32_sstore(float* lds, bool tr, int tid, const f32x4 (&r)[CH]) {
+    constexpr int RQ = ROWS / 4;
+#pragma unroll
+    for (int i = 0; i < CH; ++i) {
+        const int c = tid + i * NT;
+        if (!tr) {
+            const int row = c >> 2, kq = c & 3;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) lds[(kq * 4 + e) * LD + row] = r[i][e];
+        } else {
+            const int k = c / RQ, rq = c % RQ;
+            *(f32x4*)(lds + k * LD + rq * 4) = r[i];
+        }
+    }
+}
+
+template <bool TA, bool TB, int TILE, int KG = 1, int BN = TILE>
 __device__ __forceinline__ void gemm_f32_body(const GemmArgs& g, const int block_id, const int batch_id, const bool logical_id) {
-    constexpr int BM = TILE, BN = TILE, BK = 16, LDS_LD = TILE + 4, NT = 256;
-    constexpr int WT = TILE / 2, TF = WT / 32;          // wave tile side, 32x32 accumulator tiles along it
-    constexpr int CH = TILE * BK / 4 / NT;              // 16-byte chunks of an operand tile per thread
-    constexpr int RQ = TILE / 4;                        // chunks along a row-contiguous (transposed) tile row
-    static_assert(KG == 1 || TILE == 64, "the contraction is split over wave groups on the small tile only");
-    __shared__ __attribute__((aligned(16))) float As_all[KG][2][BK * LDS_LD];
-    __shared__ __attribute__((aligned(16))) float Bs_all[KG][2][BK * LDS_LD];
-    const int grp = KG == 1 ? 0 : threadIdx.x >> 8;
-    const int tid = threadIdx.x & 255, lane = tid & 63, wave = tid >> 6;
-    float (*As)[BK * LDS_LD] = As_all[grp];
-    float (*Bs)[BK * LDS_LD] = Bs_all[grp];
-    const int wm = wave >> 1, wn = wave & 1;
+    static_assert(BN == TILE || (TILE == 64 && BN == 32), "tiles: 128x128, 64x64, 64x32");
+    static_assert(KG == 1 || TILE == 64, "the contraction is split over wave groups on the small tiles only");
+    constexpr int BM = TILE, BK = 16, LDA = BM + 4, LDB = BN + 4;
+    constexpr int WTM = TILE / 2, WTN = BN == TILE ? TILE / 2 : BN;   // wave tile
+    constexpr int WN = BN / WTN, NT = 64 * (BM / WTM) * WN;           // waves along N, threads of a group
+    constexpr int TFM = WTM / 32, TFN = WTN / 32;                     // 32x32 accumulator tiles of a wave
+    constexpr int CHA = BM * BK / 4 / NT, CHB = BN * BK / 4 / NT;     // 16-byte chunks of an operand tile per thread
+    constexpr int GROUP_LDS = 2 * BK * (LDA + LDB);                   // two stages of A, then two of B
+    __shared__ __attribute__((aligned(16))) float lds_all[KG][GROUP_LDS];
+    const int grp = KG == 1 ? 0 : threadIdx.x / NT;
+    const int tid = threadIdx.x % NT, lane = tid & 63, wave = tid >> 6;
+    float* const As = lds_all[grp];
+    float* const Bs = lds_all[grp] + 2 * BK * LDA;
+    const int wm = WN == 2 ? wave >> 1 : wave, wn = WN == 2 ? wave & 1 : 0;
     int tile_m, tile_n;
     if (logical_id) panel_coords(block_id, g.tiles_m, g.tiles_n, tile_m, tile_n);
     else tile_coords(block_id, g.tiles_m, g.tiles_n, tile_m, tile_n);
@@ -1458,113 +1499,76 @@ __device__ __forceinline__ void gemm_f32_body(const GemmArgs& g, const int block
     const float* B = (const float*)g.B + b1 * g.sB1 + b2 * g.sB2;
     const int64_t coff = b1 * g.sC1 + b2 * g.sC2;
 
-    f32x4 ra[CH], rb[CH];
-    // a k-tile past the end of the contraction loads zeros (a group whose share is one k-tile shorter adds nothing)
-    auto gload = [&](const float* base, int64_t ld, int row0, int rows, int k0, bool tr, f32x4 (&r)[CH]) {
+    f32x4 ra[CHA], rb[CHB];
+    f32x16 acc[TFM][TFN];
 #pragma unroll
-        for (int i = 0; i < CH; ++i) {
-            const int c = tid + i * NT;
-            f32x4 v = {0.f, 0.f, 0.f, 0.f};
-            if (!tr) {
-                const int row = c >> 2, kq = c & 3;
-                if (row0 + row < rows && k0 + kq * 4 < g.K)
-                    v = *(const f32x4*)(base + (int64_t)(row0 + row) * ld + k0 + kq * 4);
-            } else {
-                const int k = c / RQ, rq = c % RQ;
-                if (row0 + rq * 4 < rows && k0 + k < g.K)
-                    v = *(const f32x4*)(base + (int64_t)(k0 + k) * ld + row0 + rq * 4);
-            }
-            r[i] = v;
-        }
-    };
-    auto sstore = [&](float* lds, bool tr, const f32x4 (&r)[CH]) {
+    for (int i = 0; i < TFM; ++i)
 #pragma unroll
-        for (int i = 0; i < CH; ++i) {
-            const int c = tid + i * NT;
-            if (!tr) {
-                const int row = c >> 2, kq = c & 3;
-#pragma unroll
-                for (int e = 0; e < 4; ++e) lds[(kq * 4 + e) * LDS_LD + row] = r[i][e];
-            } else {
-                const int k = c / RQ, rq = c % RQ;
-                *(f32x4*)(lds + k * LDS_LD + rq * 4) = r[i];
-            }
-        }
-    };
-
-    f32x16 acc[TF][TF];
-#pragma unroll
-    for (int i = 0; i < TF; ++i)
-#pragma unroll
-        for (int j = 0; j < TF; ++j)
+        for (int j = 0; j < TFN; ++j)
 #pragma unroll
             for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
 
-    // every group runs the same number of rounds (the barriers are the block's); round it of group grp is k-tile
-    // it * KG + grp
+    // every group runs the same number of rounds (the barriers are the block's); round kt of group grp is k-tile
+    // kt * KG + grp
     const int KT = ((g.K + BK - 1) / BK + KG - 1) / KG;
-    gload(A, g.lda, m0, g.M, grp * BK, TA, ra);
-    gload(B, g.ldb, n0, g.N, grp * BK, TB, rb);
-    sstore(As[0], TA, ra);
-    sstore(Bs[0], TB, rb);
+    f32_gload<BM, BK, NT, CHA>(A, g.lda, m0, g.M, grp * BK, g.K, TA, tid, ra);
+    f32_gload<BN, BK, NT, CHB>(B, g.ldb, n0, g.N, grp * BK, g.K, TB, tid, rb);
+    f32_sstore<BM, LDA, NT, CHA>(As, TA, tid, ra);
+    f32_sstore<BN, LDB, NT, CHB>(Bs, TB, tid, rb);
     __syncthreads();
     for (int kt = 0; kt < KT; ++kt) {
         const int cur = kt & 1;
         const bool more = kt + 1 < KT;
         if (more) {
-            gload(A, g.lda, m0, g.M, ((kt + 1) * KG + grp) * BK, TA, ra);
-            gload(B, g.ldb, n0, g.N, ((kt + 1) * KG + grp) * BK, TB, rb);
+            f32_gload<BM, BK, NT, CHA>(A, g.lda, m0, g.M, ((kt + 1) * KG + grp) * BK, g.K, TA, tid, ra);
+            f32_gload<BN, BK, NT, CHB>(B, g.ldb, n0, g.N, ((kt + 1) * KG + grp) * BK, g.K, TB, tid, rb);
         }
+        const float* as = As + cur * BK * LDA;
+        const float* bs = Bs + cur * BK * LDB;
 #pragma unroll
         for (int ks = 0; ks < BK / 2; ++ks) {
-            float af[TF], bfr[TF];
+            float af[TFM], bfr[TFN];
             const int kk = ks * 2 + (lane >> 5);
 #pragma unroll
-            for (int i = 0; i < TF; ++i) af[i] = As[cur][kk * LDS_LD + wm * WT + i * 32 + (lane & 31)];
+            for (int i = 0; i < TFM; ++i) af[i] = as[kk * LDA + wm * WTM + i * 32 + (lane & 31)];
 #pragma unroll
-            for (int j = 0; j < TF; ++j) bfr[j] = Bs[cur][kk * LDS_LD + wn * WT + j * 32 + (lane & 31)];
+            for (int j = 0; j < TFN; ++j) bfr[j] = bs[kk * LDB + wn * WTN + j * 32 + (lane & 31)];
 #pragma unroll
-            for (int i = 0; i < TF; ++i)
+            for (int i = 0; i < TFM; ++i)
 #pragma unroll
-                for (int j = 0; j < TF; ++j)
+                for (int j = 0; j < TFN; ++j)
                     acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(af[i], bfr[j], acc[i][j], 0, 0, 0);
         }
         if (more) {
-            sstore(As[cur ^ 1], TA, ra);
-            sstore(Bs[cur ^ 1], TB, rb);
+            f32_sstore<BM, LDA, NT, CHA>(As + (cur ^ 1) * BK * LDA, TA, tid, ra);
+            f32_sstore<BN, LDB, NT, CHB>(Bs + (cur ^ 1) * BK * LDB, TB, tid, rb);
         }
         __syncthreads();
     }
     if constexpr (KG > 1) {
-        // partial tiles of groups 1 .. KG-1 go through the groups' own (now idle) operand buffers, eight of a thread's
-        // sixteen values through each of A's and B's; group 0 adds them up in group order
-        static_assert(TF == 1 && 2 * BK * LDS_LD >= 8 * NT, "a group's operand buffers hold its partial tile");
+        // partial tiles of groups 1 .. KG-1 go through the groups' own (now idle) operand buffers; group 0 adds them up
+        // in group order
+        static_assert(TFM == 1 && TFN == 1 && GROUP_LDS >= 16 * NT, "a group's operand buffers hold its partial tile");
         if (grp > 0) {
 #pragma unroll
-            for (int r = 0; r < 8; ++r) {
-                (&As_all[grp][0][0])[r * NT + tid] = acc[0][0][r];
-                (&Bs_all[grp][0][0])[r * NT + tid] = acc[0][0][8 + r];
-            }
+            for (int r = 0; r < 16; ++r) lds_all[grp][r * NT + tid] = acc[0][0][r];
         }
         __syncthreads();
         if (grp > 0) return;
 #pragma unroll
         for (int j = 1; j < KG; ++j)
 #pragma unroll
-            for (int r = 0; r < 8; ++r) {
-                acc[0][0][r] += (&As_all[j][0][0])[r * NT + tid];
-                acc[0][0][8 + r] += (&Bs_all[j][0][0])[r * NT + tid];
-            }
+            for (int r = 0; r < 16; ++r) acc[0][0][r] += lds_all[j][r * NT + tid];
     }
 #pragma unroll
-    for (int i = 0; i < TF; ++i)
+    for (int i = 0; i < TFM; ++i)
 #pragma unroll
-        for (int j = 0; j < TF; ++j) {
-            const int n = n0 + wn * WT + j * 32 + (lane & 31);
+        for (int j = 0; j < TFN; ++j) {
+            const int n = n0 + wn * WTN + j * 32 + (lane & 31);
             if (n >= g.N) continue;
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
-                const int m = m0 + wm * WT + i * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
+                const int m = m0 + wm * WTM + i * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
                 if (m < g.M) epilogue_elem<float>(g, coff, coff, m, n, acc[i][j][r]);
             }
         }
@@ -1574,10 +1578,10 @@ template <bool TA, bool TB, int TILE = 128>
 __global__ __launch_bounds__(256) void gemm_f32_kernel(const GemmArgs g) {
     gemm_f32_body<TA, TB, TILE>(g, blockIdx.x, blockIdx.z, false);
 }
-// 64x64 tiles, the contraction dealt to KG groups of four waves
-template <bool TA, bool TB, int KG>
-__global__ __launch_bounds__(256 * KG) void gemm_f32_ksplit_kernel(const GemmArgs g) {
-    gemm_f32_body<TA, TB, 64, KG>(g, blockIdx.x, blockIdx.z, false);
+// small tiles (64 x BN), the contraction dealt to KG groups of waves
+template <bool TA, bool TB, int KG, int BN>
+__global__ __launch_bounds__(4 * BN * KG) void gemm_f32_ksplit_kernel(const GemmArgs g) {
+    gemm_f32_body<TA, TB, 64, KG, BN>(g, blockIdx.x, blockIdx.z, false);
 }
 // several unbatched problems in one launch (the weight gradients of an fp32 layer: the smallest has 144 tiles of 64x64)
 template <bool TA, bool TB, int TILE>

@@ -284,8 +284,8 @@ def test_gemm_grouped_weight_gradients(hiplib, dtype):
                                    (2048, 768, 768),    # C1's attention output projection
                                    (100, 72, 1036)])    # ragged rows, columns and contraction
 def test_gemm_fp32_contraction_shared_by_wave_groups(hiplib, layout, M, N, K):
-    """fp32 problems with fewer than two 64x64 tiles per CU and a long contraction deal the k-tiles of a tile to two
-    groups of waves (partial tiles added in group order): against fp64 with bias, residual and accumulation, the same
+    """fp32 problems with fewer than two 64x64 tiles per CU and a long contraction take 64x32 tiles and deal the k-tiles
+    of a tile to two groups of waves (partial tiles added in group order): against fp64 with bias, residual and accumulation, the same
     bits on a second call, and problems outside the rule keep the plain kernel."""
     lay = {"nt": hiplib.NT, "nn": hiplib.NN}[layout]
     A = randn(M, K, seed=120)
@@ -293,7 +293,7 @@ def test_gemm_fp32_contraction_shared_by_wave_groups(hiplib, layout, M, N, K):
     bias, resid, C0 = randn(N, seed=122), randn(M, N, seed=123), randn(M, N, seed=124)
     prod = A.double().cpu() @ (B.double().cpu().t() if layout == "nt" else B.double().cpu())
     C = torch.empty(M, N, device=DEV)
-    assert hiplib.gemm_variant(hiplib.gemm_desc(lay, A, B, C)).endswith("64x64k2")
+    assert hiplib.gemm_variant(hiplib.gemm_desc(lay, A, B, C)).endswith("64x32k2")
     hiplib.gemm(lay, A, B, C, bias=bias, epilogue=hiplib.EPI_RESIDUAL, resid=resid)
     assert rel_err(C, prod + bias.double().cpu() + resid.double().cpu()) < 1e-5
     C2 = torch.zeros_like(C)
